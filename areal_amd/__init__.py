@@ -1,0 +1,30 @@
+"""MI355X-native kernels for AReaL's PPO/GRPO log-prob, entropy and actor-loss path.
+
+Importing the package does not load the HIP library; the first op call does, and
+raises ``NativeLibraryError`` if ``libareal_amd.so`` has not been built.
+"""
+from .config import RejectionSamplingConfig
+from .functional import (
+    RejectionSamplingResult,
+    apply_rejection_sampling,
+    fused_logprobs_ppo_loss,
+    gather_logprobs,
+    gather_logprobs_entropy,
+    gather_logprobs_entropy_stats,
+    ppo_actor_loss_fn,
+)
+from ._native import NativeLibraryError
+
+__version__ = "0.1.0"
+
+__all__ = [
+    "NativeLibraryError",
+    "RejectionSamplingConfig",
+    "RejectionSamplingResult",
+    "apply_rejection_sampling",
+    "fused_logprobs_ppo_loss",
+    "gather_logprobs",
+    "gather_logprobs_entropy",
+    "gather_logprobs_entropy_stats",
+    "ppo_actor_loss_fn",
+]

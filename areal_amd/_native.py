@@ -1,0 +1,101 @@
+"""ctypes binding of ``libareal_amd.so`` (the C ABI declared in ``include/areal_amd.h``).
+
+The library is loaded from the package directory.  There is no fallback: if it
+is missing or a call returns a non-zero status, an exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import threading
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "libareal_amd.so"
+
+AA_OK = 0
+AA_BF16, AA_F16, AA_F32 = 0, 1, 2
+
+RS_LEVEL = {"token": 0, "sequence": 1}
+RS_ACTION = {"mask": 0, "clamp": 1}
+RS_METRIC = {"ratio": 0, "kl_k1": 1, "kl_k2": 2, "kl_k3": 3}
+RS_AGG = {"sum": 0, "mean": 1, "max": 2}
+
+
+class NativeLibraryError(RuntimeError):
+    """The HIP library is missing, incomplete, or a call into it failed."""
+
+
+class PpoParams(C.Structure):
+    """``aa_ppo_params``"""
+
+    _fields_ = [
+        ("clip_lo", C.c_float),
+        ("clip_hi", C.c_float),
+        ("c_clip", C.c_float),
+        ("has_c_clip", C.c_int32),
+        ("has_behave_weight", C.c_int32),
+    ]
+
+
+_p = C.c_void_p
+_i64 = C.c_int64
+_f = C.c_float
+_i = C.c_int
+
+# name -> (restype, argtypes); must list every function of include/areal_amd.h
+SIGNATURES = {
+    "aa_version": (_i, []),
+    "aa_status_string": (C.c_char_p, [_i]),
+    "aa_logits_fwd": (_i, [_p, _i, _i64, _i64, _i64, _p, _f, _p, _p, _p, _p, _p, _p, _p]),
+    "aa_logits_bwd": (_i, [_p, _i, _i64, _i64, _i64, _p, _f, _p, _p, _p, _p, _i64, _p, _p]),
+    "aa_logits_ppo_fused": (
+        _i,
+        [_p, _i, _i64, _i64, _i64, _p, _f, _i64, _p, _p, _p, _p, C.POINTER(PpoParams), _p, _p,
+         _p, _p, _p, _p, _p, _p, _p, _p, _p],
+    ),
+    "aa_rejection_sampling": (_i, [_p, _p, _p, _i64, _p, _i64, _i, _i, _i, _i, _f, _f, _i, _p, _p, _p, _p]),
+    "aa_count_nonzero_u8": (_i, [_p, _i64, _p, _p]),
+    "aa_ppo_loss": (_i, [_p, _p, _p, _p, _p, _i64, _p, _i64, _i, C.POINTER(PpoParams), _p, _p, _p, _p, _p, _p]),
+    "aa_masked_sum": (_i, [_p, _p, _i64, _p, _p, _p, _p]),
+    "aa_scale_inplace": (_i, [_p, _i, _i64, _p, _p]),
+    "aa_lmhead_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "aa_lmhead_fwd": (_i, [_p, _p, _i64, _i64, _i64, _p, _f, _p, _p, _p, _p, _p, _i64, _p]),
+    "aa_lmhead_bwd": (_i, [_p, _p, _i64, _i64, _i64, _p, _f, _p, _p, _p, _p, _p, _p, _p, _i64, _p]),
+    "aa_copy_bytes": (_i, [_p, _p, _i64, _p]),
+}
+
+_lib = None
+_lock = threading.Lock()
+
+
+def load() -> C.CDLL:
+    """Load the shared library once and bind the signatures."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not LIB_PATH.exists():
+            raise NativeLibraryError(
+                f"{LIB_PATH} not found: build it with `python -m areal_amd.build` "
+                "(there is no CPU or PyTorch fallback for these ops)"
+            )
+        try:
+            lib = C.CDLL(str(LIB_PATH))
+        except OSError as e:  # missing ROCm runtime etc.
+            raise NativeLibraryError(f"cannot load {LIB_PATH}: {e}") from e
+        for name, (res, args) in SIGNATURES.items():
+            try:
+                fn = getattr(lib, name)
+            except AttributeError as e:
+                raise NativeLibraryError(f"{LIB_PATH} does not export {name}") from e
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def check(status: int, what: str) -> None:
+    if status != AA_OK:
+        msg = load().aa_status_string(status).decode()
+        raise NativeLibraryError(f"{what} failed: {msg} (status {status})")

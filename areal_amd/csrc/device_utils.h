@@ -1,0 +1,141 @@
+// Device helpers shared by the gfx950 kernels: 16-bit float packing, wave64 and
+// workgroup reductions, and the (max, sum-exp, sum x*exp) softmax partials.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <float.h>
+
+#include "../../include/areal_amd.h"
+
+namespace aa {
+
+constexpr int kWave = 64;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+// Finite stand-in for "no element seen yet": exp2((kNegBig - m) * c) is 0 for
+// every finite m, and 0 * kNegBig stays finite (no NaN from inf * 0).
+constexpr float kNegBig = -3.0e38f;
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// ---- 16-bit element access: DT is an aa_dtype value -------------------------
+template <int DT>
+struct Elem;
+
+template <>
+struct Elem<AA_BF16> {
+  typedef uint16_t storage;
+  static constexpr int kBytes = 2;
+  __device__ static __forceinline__ float lo(uint32_t w) { return __uint_as_float(w << 16); }
+  __device__ static __forceinline__ float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+  __device__ static __forceinline__ float load1(const void* p, int64_t i) {
+    return __uint_as_float(((uint32_t)((const uint16_t*)p)[i]) << 16);
+  }
+  __device__ static __forceinline__ uint32_t pack(float a, float b) {
+    f32x2_t v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+  }
+  __device__ static __forceinline__ void store1(void* p, int64_t i, float v) {
+    ((uint16_t*)p)[i] = (uint16_t)(pack(v, 0.f) & 0xffffu);
+  }
+};
+
+template <>
+struct Elem<AA_F16> {
+  typedef uint16_t storage;
+  static constexpr int kBytes = 2;
+  __device__ static __forceinline__ float lo(uint32_t w) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu));
+  }
+  __device__ static __forceinline__ float hi(uint32_t w) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
+  }
+  __device__ static __forceinline__ float load1(const void* p, int64_t i) {
+    return (float)((const _Float16*)p)[i];
+  }
+  __device__ static __forceinline__ uint32_t pack(float a, float b) {
+    f32x2_t v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+  }
+  __device__ static __forceinline__ void store1(void* p, int64_t i, float v) {
+    ((_Float16*)p)[i] = (_Float16)v;
+  }
+};
+
+template <>
+struct Elem<AA_F32> {
+  typedef float storage;
+  static constexpr int kBytes = 4;
+  __device__ static __forceinline__ float load1(const void* p, int64_t i) { return ((const float*)p)[i]; }
+  __device__ static __forceinline__ void store1(void* p, int64_t i, float v) { ((float*)p)[i] = v; }
+};
+
+// Eight consecutive elements starting at element index i (i * kBytes must be
+// 16-byte aligned relative to an aligned base).
+template <int DT>
+__device__ __forceinline__ void load8(const void* base, int64_t i, float (&x)[8]) {
+  if constexpr (DT == AA_F32) {
+    const float4* p = (const float4*)((const float*)base + i);
+    float4 a = p[0], b = p[1];
+    x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w;
+    x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
+  } else {
+    uint4 q = *(const uint4*)((const uint16_t*)base + i);
+    x[0] = Elem<DT>::lo(q.x); x[1] = Elem<DT>::hi(q.x);
+    x[2] = Elem<DT>::lo(q.y); x[3] = Elem<DT>::hi(q.y);
+    x[4] = Elem<DT>::lo(q.z); x[5] = Elem<DT>::hi(q.z);
+    x[6] = Elem<DT>::lo(q.w); x[7] = Elem<DT>::hi(q.w);
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ void store8(void* base, int64_t i, const float (&x)[8]) {
+  if constexpr (DT == AA_F32) {
+    float4* p = (float4*)((float*)base + i);
+    p[0] = make_float4(x[0], x[1], x[2], x[3]);
+    p[1] = make_float4(x[4], x[5], x[6], x[7]);
+  } else {
+    uint4 q;
+    q.x = Elem<DT>::pack(x[0], x[1]);
+    q.y = Elem<DT>::pack(x[2], x[3]);
+    q.z = Elem<DT>::pack(x[4], x[5]);
+    q.w = Elem<DT>::pack(x[6], x[7]);
+    *(uint4*)((uint16_t*)base + i) = q;
+  }
+}
+
+// ---- wave64 reductions -------------------------------------------------------
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+  return v;
+}
+__device__ __forceinline__ float wave_min(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, kWave));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+__device__ __forceinline__ int wave_sum(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+
+inline int launch_status() { return hipGetLastError() == hipSuccess ? AA_OK : AA_ERR_LAUNCH; }
+
+}  // namespace aa

@@ -1,0 +1,629 @@
+// Logits path for gfx950: per-token log-prob / entropy over the full vocabulary,
+// its backward, and the fused forward + token-level PPO loss + backward.
+//
+// Replaces, for one GPU, the PyTorch sequence
+//   log_softmax(logits.float() / T) -> gather -> (entropy) -> ppo_actor_loss_fn -> autograd
+// (areal/utils/functional/vocab_parallel.py:15-29,
+//  areal/utils/functional/functional.py:429-559).
+//
+// All kernels are HBM-streaming kernels: one workgroup owns one row of the
+// [T, V] logits.  Exponentials are taken in base 2 with c = log2(e) / T folded
+// into one fma per element; row statistics are carried as
+//   k = max_j x_j * c,   s = sum_j 2^(x_j c - k),   u = sum_j x_j 2^(x_j c - k)
+// so that  log2-sum-exp = k + log2 s  exactly reuses the rounded k.
+#include "device_utils.h"
+#include "ppo_math.h"
+
+namespace aa {
+
+// -----------------------------------------------------------------------------
+// Generic row traversal (any V, any row alignment): a scalar head up to the
+// first 16-byte boundary, 8-element vectors, a scalar tail.
+// -----------------------------------------------------------------------------
+struct RowSplit {
+  int head;   // scalar elements before the vector body
+  int nvec;   // 8-element vectors
+  int tail0;  // first element of the scalar tail
+};
+
+template <int DT>
+__device__ __forceinline__ RowSplit split_row(const void* row, int V, bool vec_ok) {
+  RowSplit r;
+  if (!vec_ok) {
+    r.head = V; r.nvec = 0; r.tail0 = V;
+    return r;
+  }
+  const int mis = (int)((uintptr_t)row & 15);
+  int head = mis ? (16 - mis) / Elem<DT>::kBytes : 0;
+  if (head > V) head = V;
+  r.head = head;
+  r.nvec = (V - head) >> 3;
+  r.tail0 = head + (r.nvec << 3);
+  return r;
+}
+
+struct ThreadStats {
+  float k, s, u, mx, mn;
+};
+
+__device__ __forceinline__ void stats_add1(ThreadStats& a, float x, float c) {
+  const float xc = x * c;
+  if (xc > a.k) {
+    const float f = fast_exp2(a.k - xc);
+    a.s *= f; a.u *= f; a.k = xc;
+  }
+  const float e = fast_exp2(fmaf(x, c, -a.k));
+  a.s += e;
+  a.u = fmaf(x, e, a.u);
+  a.mx = fmaxf(a.mx, x);
+  a.mn = fminf(a.mn, x);
+}
+
+__device__ __forceinline__ void stats_add8(ThreadStats& a, const float (&x)[8], float c) {
+  float m8 = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+  float n8 = fminf(fminf(fminf(x[0], x[1]), fminf(x[2], x[3])), fminf(fminf(x[4], x[5]), fminf(x[6], x[7])));
+  const float kc = m8 * c;
+  if (kc > a.k) {
+    const float f = fast_exp2(a.k - kc);
+    a.s *= f; a.u *= f; a.k = kc;
+  }
+  a.mx = fmaxf(a.mx, m8);
+  a.mn = fminf(a.mn, n8);
+  float s = 0.f, u = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float e = fast_exp2(fmaf(x[i], c, -a.k));
+    s += e;
+    u = fmaf(x[i], e, u);
+  }
+  a.s += s;
+  a.u += u;
+}
+
+struct RowStats {
+  float k, s, u, mx, mn;  // merged over the workgroup, same value in every thread
+};
+
+// Merge in a fixed order: lane butterflies inside each wave, then a butterfly
+// over the per-wave entries (each lane reads entry lane % NWAVES, so every
+// thread ends with the same value without a second barrier).
+template <int NWAVES>
+__device__ __forceinline__ RowStats block_stats(const ThreadStats& t, float* smem) {
+  static_assert(NWAVES >= 1 && NWAVES <= 16 && (NWAVES & (NWAVES - 1)) == 0, "power-of-two wave count");
+  const float wk = wave_max(t.k);
+  const float f = fast_exp2(t.k - wk);
+  const float ws = wave_sum(t.s * f);
+  const float wu = wave_sum(t.u * f);
+  const float wmx = wave_max(t.mx);
+  const float wmn = wave_min(t.mn);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  __syncthreads();  // smem may still be read from a previous use
+  if (lane == 0) {
+    smem[wave * 5 + 0] = wk; smem[wave * 5 + 1] = ws; smem[wave * 5 + 2] = wu;
+    smem[wave * 5 + 3] = wmx; smem[wave * 5 + 4] = wmn;
+  }
+  __syncthreads();
+  const int e = lane & (NWAVES - 1);
+  RowStats r{smem[e * 5 + 0], smem[e * 5 + 1], smem[e * 5 + 2], smem[e * 5 + 3], smem[e * 5 + 4]};
+#pragma unroll
+  for (int o = NWAVES / 2; o > 0; o >>= 1) {
+    const float qk = __shfl_xor(r.k, o, kWave);
+    const float qs = __shfl_xor(r.s, o, kWave);
+    const float qu = __shfl_xor(r.u, o, kWave);
+    const float nk = fmaxf(r.k, qk);
+    const float fa = fast_exp2(r.k - nk), fb = fast_exp2(qk - nk);
+    // symmetric in (r, q): both partners compute bit-identical sums
+    r.s = r.s * fa + qs * fb;
+    r.u = r.u * fa + qu * fb;
+    r.k = nk;
+    r.mx = fmaxf(r.mx, __shfl_xor(r.mx, o, kWave));
+    r.mn = fminf(r.mn, __shfl_xor(r.mn, o, kWave));
+  }
+  return r;
+}
+
+template <int DT, int NT>
+__device__ __forceinline__ RowStats row_stats_generic(const void* row, int V, bool vec_ok, float c, float* smem) {
+  ThreadStats a{kNegBig, 0.f, 0.f, -FLT_MAX, FLT_MAX};
+  const RowSplit sp = split_row<DT>(row, V, vec_ok);
+  const int tid = threadIdx.x;
+  for (int j = tid; j < sp.head; j += NT) stats_add1(a, Elem<DT>::load1(row, j), c);
+  for (int v = tid; v < sp.nvec; v += NT) {
+    float x[8];
+    load8<DT>(row, sp.head + ((int64_t)v << 3), x);
+    stats_add8(a, x, c);
+  }
+  for (int j = sp.tail0 + tid; j < V; j += NT) stats_add1(a, Elem<DT>::load1(row, j), c);
+  return block_stats<NT / kWave>(a, smem);
+}
+
+// Row-level quantities derived from the merged statistics.
+struct RowOut {
+  float lse2;  // log2 sum_j 2^(x_j c)
+  float lse;   // natural-log logsumexp of z = x / T
+  float ez;    // sum_j p_j z_j
+};
+
+__device__ __forceinline__ RowOut finish_row(const RowStats& r, float inv_t) {
+  RowOut o;
+  o.lse2 = r.k + fast_log2(r.s);
+  o.lse = o.lse2 * kLn2;
+  o.ez = (r.u / r.s) * inv_t;
+  return o;
+}
+
+// out_j = p_j * (A + B x_j), p_j = 2^(x_j c - lse2); the label gets + lab_add.
+struct GradCoef {
+  float c, lse2, A, B, lab_add;
+  int label;  // -1 = none
+};
+
+template <int DT, int NT>
+__device__ __forceinline__ void row_grad_generic(const void* row, void* out, int V, bool vec_ok, const GradCoef& g) {
+  const RowSplit sp = split_row<DT>(row, V, vec_ok);
+  const int tid = threadIdx.x;
+  auto one = [&](int j) {
+    const float x = Elem<DT>::load1(row, j);
+    float o = fast_exp2(fmaf(x, g.c, -g.lse2)) * fmaf(g.B, x, g.A);
+    if (j == g.label) o += g.lab_add;
+    Elem<DT>::store1(out, j, o);
+  };
+  for (int j = tid; j < sp.head; j += NT) one(j);
+  for (int v = tid; v < sp.nvec; v += NT) {
+    const int e0 = sp.head + (v << 3);
+    float x[8], o[8];
+    load8<DT>(row, e0, x);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = fast_exp2(fmaf(x[i], g.c, -g.lse2)) * fmaf(g.B, x[i], g.A);
+    if ((unsigned)(g.label - e0) < 8u) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (e0 + i == g.label) o[i] += g.lab_add;
+    }
+    store8<DT>(out, e0, o);
+  }
+  for (int j = sp.tail0 + tid; j < V; j += NT) one(j);
+}
+
+template <int DT, int NT>
+__device__ __forceinline__ void row_zero_generic(const void* row_like, void* out, int V, bool vec_ok) {
+  const RowSplit sp = split_row<DT>(row_like, V, vec_ok);
+  const int tid = threadIdx.x;
+  const float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int j = tid; j < sp.head; j += NT) Elem<DT>::store1(out, j, 0.f);
+  for (int v = tid; v < sp.nvec; v += NT) store8<DT>(out, sp.head + (v << 3), z);
+  for (int j = sp.tail0 + tid; j < V; j += NT) Elem<DT>::store1(out, j, 0.f);
+}
+
+__device__ __forceinline__ const void* row_ptr(const void* base, int64_t t, int64_t stride, int bytes) {
+  return (const char*)base + t * stride * bytes;
+}
+
+// -----------------------------------------------------------------------------
+// Forward: logp, entropy, row statistics.  grid = T rows, NT threads.
+// -----------------------------------------------------------------------------
+template <int DT, int NT>
+__global__ __launch_bounds__(NT) void k_logits_fwd(const void* __restrict__ logits, int V, int64_t stride,
+                                                   const int64_t* __restrict__ labels, float inv_t, int vec_ok,
+                                                   float* __restrict__ logp, float* __restrict__ entropy,
+                                                   float* __restrict__ row_lse, float* __restrict__ row_ez,
+                                                   float* __restrict__ vmax, float* __restrict__ vmin) {
+  __shared__ float smem[(NT / kWave) * 5];
+  const int64_t t = blockIdx.x;
+  const void* row = row_ptr(logits, t, stride, Elem<DT>::kBytes);
+  const float c = kLog2e * inv_t;
+  const int64_t y = labels[t];
+  const bool y_ok = (y >= 0) && (y < V);
+  const float xy = y_ok ? Elem<DT>::load1(row, y) : 0.f;
+  const RowStats rs = row_stats_generic<DT, NT>(row, V, vec_ok != 0, c, smem);
+  if (threadIdx.x == 0) {
+    const RowOut ro = finish_row(rs, inv_t);
+    logp[t] = y_ok ? fmaf(xy, c, -ro.lse2) * kLn2 : __builtin_nanf("");
+    if (entropy) entropy[t] = ro.lse - ro.ez;
+    if (row_lse) row_lse[t] = ro.lse;
+    if (row_ez) row_ez[t] = ro.ez;
+    if (vmax) vmax[t] = rs.mx;
+    if (vmin) vmin[t] = rs.mn;
+  }
+}
+
+// -----------------------------------------------------------------------------
+// Backward: dlogits from g_logp / g_entropy and the saved row statistics.
+// -----------------------------------------------------------------------------
+template <int DT, int NT>
+__global__ __launch_bounds__(NT) void k_logits_bwd(const void* __restrict__ logits, int V, int64_t stride,
+                                                   const int64_t* __restrict__ labels, float inv_t, int vec_ok,
+                                                   const float* __restrict__ row_lse,
+                                                   const float* __restrict__ row_ez,
+                                                   const float* __restrict__ g_logp,
+                                                   const float* __restrict__ g_entropy, int64_t T_active,
+                                                   void* __restrict__ dlogits) {
+  const int64_t t = blockIdx.x;
+  const void* row = row_ptr(logits, t, stride, Elem<DT>::kBytes);
+  void* out = (void*)row_ptr(dlogits, t, stride, Elem<DT>::kBytes);
+  const float gl = (t < T_active) ? g_logp[t] : 0.f;
+  const float gh = (t < T_active && g_entropy) ? g_entropy[t] : 0.f;
+  if (gl == 0.f && gh == 0.f) {
+    row_zero_generic<DT, NT>(row, out, V, vec_ok != 0);
+    return;
+  }
+  const int64_t y = labels[t];
+  GradCoef g;
+  g.c = kLog2e * inv_t;
+  g.lse2 = row_lse[t] * kLog2e;
+  const float ez = (gh != 0.f) ? row_ez[t] : 0.f;
+  g.A = inv_t * (gh * ez - gl);
+  g.B = -gh * inv_t * inv_t;
+  g.lab_add = gl * inv_t;
+  g.label = (y >= 0 && y < V) ? (int)y : -1;
+  row_grad_generic<DT, NT>(row, out, V, vec_ok != 0, g);
+}
+
+// -----------------------------------------------------------------------------
+// Per-token tail of the fused kernels: PPO surrogate from the row's log-prob,
+// per-token outputs, and the coefficient of the gradient row.
+// -----------------------------------------------------------------------------
+struct FusedTokenArgs {
+  const float* prox_logp;
+  const float* adv;
+  const uint8_t* mask_eff;
+  const float* behave_w;
+  const int32_t* n_valid;
+  const float* grad_scale;
+  float* logp;
+  float* entropy;
+  float* vmax;
+  float* vmin;
+  float* stat_loss;
+  float* ratio;
+  uint8_t* flags;
+  aa_ppo_params P;
+  int64_t T_active;
+};
+
+// Returns g = d(scaled loss)/d(logp_t); writes the per-token outputs from one thread.
+__device__ __forceinline__ float fused_token_tail(const FusedTokenArgs& a, int64_t t, float lp, const RowStats& rs,
+                                                  const RowOut& ro, bool writer) {
+  if (writer) {
+    a.logp[t] = lp;
+    if (a.entropy) a.entropy[t] = ro.lse - ro.ez;
+    if (a.vmax) a.vmax[t] = rs.mx;
+    if (a.vmin) a.vmin[t] = rs.mn;
+  }
+  if (t >= a.T_active) return 0.f;
+  const bool m = a.mask_eff[t] != 0;
+  const float prox = a.prox_logp[t];
+  const float r = m ? expf(lp - prox) : 0.f;
+  const float w = a.P.has_behave_weight ? a.behave_w[t] : 1.f;
+  const Surrogate s = surrogate(r, a.adv[t], w, a.P);
+  if (writer) {
+    a.stat_loss[t] = s.loss;
+    a.ratio[t] = r;
+    a.flags[t] = (uint8_t)(((s.clip && m) ? 1 : 0) | ((s.dual && m) ? 2 : 0));
+  }
+  if (!m) return 0.f;
+  int n = *a.n_valid;
+  if (n < 1) n = 1;
+  float g = s.dloss_dr * r / (float)n;
+  if (a.grad_scale) g *= *a.grad_scale;
+  return g;
+}
+
+template <int DT, int NT>
+__global__ __launch_bounds__(NT) void k_fused_generic(const void* __restrict__ logits, int V, int64_t stride,
+                                                      const int64_t* __restrict__ labels, float inv_t, int vec_ok,
+                                                      FusedTokenArgs a, void* __restrict__ dlogits) {
+  __shared__ float smem[(NT / kWave) * 5];
+  const int64_t t = blockIdx.x;
+  const void* row = row_ptr(logits, t, stride, Elem<DT>::kBytes);
+  void* out = (void*)row_ptr(dlogits, t, stride, Elem<DT>::kBytes);
+  const float c = kLog2e * inv_t;
+  const int64_t y = labels[t];
+  const bool y_ok = (y >= 0) && (y < V);
+  const float xy = y_ok ? Elem<DT>::load1(row, y) : 0.f;
+  const RowStats rs = row_stats_generic<DT, NT>(row, V, vec_ok != 0, c, smem);
+  const RowOut ro = finish_row(rs, inv_t);
+  const float lp = y_ok ? fmaf(xy, c, -ro.lse2) * kLn2 : __builtin_nanf("");
+  const float g = fused_token_tail(a, t, lp, rs, ro, threadIdx.x == 0);
+  if (g == 0.f) {
+    row_zero_generic<DT, NT>(row, out, V, vec_ok != 0);
+    return;
+  }
+  GradCoef gc;
+  gc.c = c; gc.lse2 = ro.lse2; gc.A = -g * inv_t; gc.B = 0.f; gc.lab_add = g * inv_t;
+  gc.label = y_ok ? (int)y : -1;
+  row_grad_generic<DT, NT>(row, out, V, vec_ok != 0, gc);
+}
+
+// -----------------------------------------------------------------------------
+// Fused kernel, register-resident row: 1024 threads hold one row of 16-bit
+// logits as NCH 16-byte chunks per thread, so HBM sees exactly one read of the
+// row and one write of its gradient.  Requires V % 8 == 0, 16-byte aligned
+// rows and 8192 * (NCH - 1) < V <= 8192 * NCH, so that only the last chunk can
+// be partly out of range.  Rows are addressed through buffer descriptors: one
+// VGPR offset per thread, the chunk offset in an SGPR, and the hardware drops
+// out-of-range lanes (loads return 0, stores are ignored).
+// -----------------------------------------------------------------------------
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+constexpr int kBufferFlags = 0x00020000;  // raw buffer, 32-bit data format
+
+// Marks the packed row as modified (no instruction is emitted) so that the
+// unpacked floats of one pass are not kept alive for the next: the row stays
+// at 4 registers per chunk instead of 12.
+template <int NCH>
+__device__ __forceinline__ void keep_packed(u32x4_t (&d)[NCH]) {
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    uint32_t a = d[i][0], b = d[i][1], c = d[i][2], e = d[i][3];
+    asm volatile("" : "+v"(a), "+v"(b), "+v"(c), "+v"(e));
+    d[i][0] = a; d[i][1] = b; d[i][2] = c; d[i][3] = e;
+  }
+}
+
+template <int DT, int NCH>
+__global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ logits, int V, int64_t stride_vec,
+                                                     const int64_t* __restrict__ labels, float inv_t,
+                                                     FusedTokenArgs a, uint4* __restrict__ dlogits) {
+  constexpr int NT = 1024;
+  constexpr int kChunkBytes = NT * 16;
+  __shared__ float smem[(NT / kWave) * 5];
+  const int64_t t = blockIdx.x;
+  const uint4* src = logits + t * stride_vec;
+  uint4* dst = dlogits + t * stride_vec;
+  const int nvec = V >> 3;
+  const int tid = threadIdx.x;
+  const float c = kLog2e * inv_t;
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, V * 2, kBufferFlags);
+  const __amdgpu_buffer_rsrc_t wsrc = __builtin_amdgcn_make_buffer_rsrc((void*)dst, 0, V * 2, kBufferFlags);
+  const int voff = tid * 16;
+  const bool last_ok = (NCH - 1) * NT + tid < nvec;
+
+  u32x4_t d[NCH];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) d[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, i * kChunkBytes, 0);
+  const int64_t y = labels[t];
+  const bool y_ok = (y >= 0) && (y < V);
+  const float xy = y_ok ? Elem<DT>::load1(src, y) : 0.f;
+
+  // pass 1 over registers: thread maximum / minimum
+  float mx = -FLT_MAX, mn = FLT_MAX;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    float cmx = -FLT_MAX, cmn = FLT_MAX;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float lo = Elem<DT>::lo(d[i][q]), hi = Elem<DT>::hi(d[i][q]);
+      cmx = fmaxf(cmx, fmaxf(lo, hi));
+      cmn = fminf(cmn, fminf(lo, hi));
+    }
+    if (i == NCH - 1 && !last_ok) { cmx = -FLT_MAX; cmn = FLT_MAX; }
+    mx = fmaxf(mx, cmx);
+    mn = fminf(mn, cmn);
+  }
+  keep_packed(d);
+  // one maximum per wave keeps the second pass free of rescaling
+  ThreadStats ts;
+  ts.k = fmaxf(wave_max(mx) * c, kNegBig);
+  ts.mx = mx; ts.mn = mn;
+  float s = 0.f, u = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    float cs = 0.f, cu = 0.f;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float lo = Elem<DT>::lo(d[i][q]), hi = Elem<DT>::hi(d[i][q]);
+      const float e0 = fast_exp2(fmaf(lo, c, -ts.k));
+      const float e1 = fast_exp2(fmaf(hi, c, -ts.k));
+      cs += e0 + e1;
+      cu = fmaf(lo, e0, cu);
+      cu = fmaf(hi, e1, cu);
+    }
+    if (i == NCH - 1 && !last_ok) { cs = 0.f; cu = 0.f; }
+    s += cs;
+    u += cu;
+  }
+  ts.s = s; ts.u = u;
+  keep_packed(d);
+  const RowStats rs = block_stats<NT / kWave>(ts, smem);
+  const RowOut ro = finish_row(rs, inv_t);
+  const float lp = y_ok ? fmaf(xy, c, -ro.lse2) * kLn2 : __builtin_nanf("");
+  const float g = fused_token_tail(a, t, lp, rs, ro, tid == 0);
+
+  if (g == 0.f) {
+    const u32x4_t z = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, voff, i * kChunkBytes, 0);
+    return;
+  }
+  const float A = -g * inv_t;
+  const float lab_add = g * inv_t;
+  const int yv = y_ok ? (int)(y >> 3) : -1;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    float o[8];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      o[2 * q] = A * fast_exp2(fmaf(Elem<DT>::lo(d[i][q]), c, -ro.lse2));
+      o[2 * q + 1] = A * fast_exp2(fmaf(Elem<DT>::hi(d[i][q]), c, -ro.lse2));
+    }
+    if (i * NT + tid == yv) {
+      const int e = (int)(y & 7);
+#pragma unroll
+      for (int q = 0; q < 8; ++q)
+        if (q == e) o[q] += lab_add;
+    }
+    u32x4_t r;
+    r[0] = Elem<DT>::pack(o[0], o[1]);
+    r[1] = Elem<DT>::pack(o[2], o[3]);
+    r[2] = Elem<DT>::pack(o[4], o[5]);
+    r[3] = Elem<DT>::pack(o[6], o[7]);
+    __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff, i * kChunkBytes, 0);
+  }
+}
+
+// -----------------------------------------------------------------------------
+// Plain copy (calibration of the HBM counters) and in-place scaling.
+// -----------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_copy16(const uint4* __restrict__ src, uint4* __restrict__ dst, int64_t n) {
+  const int64_t step = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += step) dst[i] = src[i];
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void k_scale(void* __restrict__ data, int64_t n, const float* __restrict__ factor) {
+  const float f = *factor;
+  if (f == 1.0f) return;
+  const int64_t step = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += step)
+    Elem<DT>::store1(data, i, Elem<DT>::load1(data, i) * f);
+}
+
+// -----------------------------------------------------------------------------
+// Host-side dispatch
+// -----------------------------------------------------------------------------
+static bool common_args_ok(const void* logits, int dtype, int64_t T, int64_t V, int64_t stride,
+                           const int64_t* labels) {
+  if (!logits || !labels) return false;
+  if (dtype != AA_BF16 && dtype != AA_F16 && dtype != AA_F32) return false;
+  if (T <= 0 || V <= 0 || V > 0x7fffffff || stride < V) return false;
+  if (T > 0x7fffffff) return false;  // one workgroup per row, grid.x limit
+  return true;
+}
+
+static bool rows_vec_ok(const void* a, const void* b, int dtype) {
+  // element alignment is guaranteed by the element type; vector access needs
+  // both buffers to reach a 16-byte boundary after the same number of elements
+  const int eb = dtype == AA_F32 ? 4 : 2;
+  if (((uintptr_t)a % eb) != 0) return false;
+  if (b && ((((uintptr_t)a) ^ ((uintptr_t)b)) & 15)) return false;
+  return true;
+}
+
+template <int DT, int NCH>
+static void launch_regs(const void* logits, int64_t T, int V, int64_t stride, const int64_t* labels, float inv_t,
+                        const FusedTokenArgs& a, void* dlogits, hipStream_t st) {
+  hipLaunchKernelGGL((k_fused_regs<DT, NCH>), dim3((unsigned)T), dim3(1024), 0, st, (const uint4*)logits, V,
+                     stride >> 3, labels, inv_t, a, (uint4*)dlogits);
+}
+
+template <int DT>
+static bool dispatch_regs(int nch, const void* logits, int64_t T, int V, int64_t stride, const int64_t* labels,
+                          float inv_t, const FusedTokenArgs& a, void* dlogits, hipStream_t st) {
+  switch (nch) {
+#define AA_CASE(N) \
+  case N: launch_regs<DT, N>(logits, T, V, stride, labels, inv_t, a, dlogits, st); return true;
+    AA_CASE(1) AA_CASE(2) AA_CASE(3) AA_CASE(4) AA_CASE(5) AA_CASE(6) AA_CASE(7) AA_CASE(8)
+    AA_CASE(9) AA_CASE(10) AA_CASE(11) AA_CASE(12) AA_CASE(13) AA_CASE(14) AA_CASE(15) AA_CASE(16)
+    AA_CASE(17) AA_CASE(18) AA_CASE(19) AA_CASE(20) AA_CASE(21) AA_CASE(22) AA_CASE(23) AA_CASE(24)
+#undef AA_CASE
+    default: return false;
+  }
+}
+
+}  // namespace aa
+
+using namespace aa;
+
+extern "C" int aa_logits_fwd(const void* logits, int dtype, int64_t T, int64_t V, int64_t row_stride,
+                             const int64_t* labels, float inv_temperature, float* logp, float* entropy,
+                             float* row_lse, float* row_ez, float* vmax, float* vmin, void* stream) {
+  if (!common_args_ok(logits, dtype, T, V, row_stride, labels) || !logp) return AA_ERR_INVALID_ARGUMENT;
+  if (!(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
+  hipStream_t st = (hipStream_t)stream;
+  const int vec_ok = rows_vec_ok(logits, nullptr, dtype) ? 1 : 0;
+  constexpr int NT = 256;
+#define AA_LAUNCH(DT)                                                                                        \
+  hipLaunchKernelGGL((k_logits_fwd<DT, NT>), dim3((unsigned)T), dim3(NT), 0, st, logits, (int)V, row_stride, \
+                     labels, inv_temperature, vec_ok, logp, entropy, row_lse, row_ez, vmax, vmin)
+  if (dtype == AA_BF16) AA_LAUNCH(AA_BF16);
+  else if (dtype == AA_F16) AA_LAUNCH(AA_F16);
+  else AA_LAUNCH(AA_F32);
+#undef AA_LAUNCH
+  return launch_status();
+}
+
+extern "C" int aa_logits_bwd(const void* logits, int dtype, int64_t T, int64_t V, int64_t row_stride,
+                             const int64_t* labels, float inv_temperature, const float* row_lse,
+                             const float* row_ez, const float* g_logp, const float* g_entropy, int64_t T_active,
+                             void* dlogits, void* stream) {
+  if (!common_args_ok(logits, dtype, T, V, row_stride, labels)) return AA_ERR_INVALID_ARGUMENT;
+  if (!row_lse || !g_logp || !dlogits || (g_entropy && !row_ez)) return AA_ERR_INVALID_ARGUMENT;
+  if (T_active < 0 || T_active > T || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
+  hipStream_t st = (hipStream_t)stream;
+  const int vec_ok = rows_vec_ok(logits, dlogits, dtype) ? 1 : 0;
+  constexpr int NT = 256;
+#define AA_LAUNCH(DT)                                                                                        \
+  hipLaunchKernelGGL((k_logits_bwd<DT, NT>), dim3((unsigned)T), dim3(NT), 0, st, logits, (int)V, row_stride, \
+                     labels, inv_temperature, vec_ok, row_lse, row_ez, g_logp, g_entropy, T_active, dlogits)
+  if (dtype == AA_BF16) AA_LAUNCH(AA_BF16);
+  else if (dtype == AA_F16) AA_LAUNCH(AA_F16);
+  else AA_LAUNCH(AA_F32);
+#undef AA_LAUNCH
+  return launch_status();
+}
+
+extern "C" int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int64_t V, int64_t row_stride,
+                                   const int64_t* labels, float inv_temperature, int64_t T_active,
+                                   const float* prox_logp, const float* adv, const uint8_t* mask_eff,
+                                   const float* behave_w, const aa_ppo_params* params, const int32_t* n_valid,
+                                   const float* grad_scale, float* logp, float* entropy, float* vmax, float* vmin,
+                                   float* stat_loss, float* ratio, uint8_t* flags, void* dlogits, void* stream) {
+  if (!common_args_ok(logits, dtype, T, V, row_stride, labels)) return AA_ERR_INVALID_ARGUMENT;
+  if (!params || !prox_logp || !adv || !mask_eff || !n_valid || !logp || !stat_loss || !ratio || !flags || !dlogits)
+    return AA_ERR_INVALID_ARGUMENT;
+  if (params->has_behave_weight && !behave_w) return AA_ERR_INVALID_ARGUMENT;
+  if (T_active < 0 || T_active > T || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
+  hipStream_t st = (hipStream_t)stream;
+  FusedTokenArgs a;
+  a.prox_logp = prox_logp; a.adv = adv; a.mask_eff = mask_eff; a.behave_w = behave_w;
+  a.n_valid = n_valid; a.grad_scale = grad_scale;
+  a.logp = logp; a.entropy = entropy; a.vmax = vmax; a.vmin = vmin;
+  a.stat_loss = stat_loss; a.ratio = ratio; a.flags = flags;
+  a.P = *params; a.T_active = T_active;
+
+  const bool fast = (dtype != AA_F32) && (V % 8 == 0) && (row_stride % 8 == 0) && (((uintptr_t)logits & 15) == 0) &&
+                    (((uintptr_t)dlogits & 15) == 0) && (V >= 8 * 1024) && (V <= 24 * 8192);
+  if (fast) {
+    const int nch = (int)((V / 8 + 1023) / 1024);
+    bool ok = (dtype == AA_BF16)
+                  ? dispatch_regs<AA_BF16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, st)
+                  : dispatch_regs<AA_F16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, st);
+    if (ok) return launch_status();
+  }
+  const int vec_ok = rows_vec_ok(logits, dlogits, dtype) ? 1 : 0;
+  constexpr int NT = 256;
+#define AA_LAUNCH(DT)                                                                                           \
+  hipLaunchKernelGGL((k_fused_generic<DT, NT>), dim3((unsigned)T), dim3(NT), 0, st, logits, (int)V, row_stride, \
+                     labels, inv_temperature, vec_ok, a, dlogits)
+  if (dtype == AA_BF16) AA_LAUNCH(AA_BF16);
+  else if (dtype == AA_F16) AA_LAUNCH(AA_F16);
+  else AA_LAUNCH(AA_F32);
+#undef AA_LAUNCH
+  return launch_status();
+}
+
+extern "C" int aa_copy_bytes(const void* src, void* dst, int64_t nbytes, void* stream) {
+  if (!src || !dst || nbytes < 0 || (nbytes & 15) || ((uintptr_t)src & 15) || ((uintptr_t)dst & 15))
+    return AA_ERR_INVALID_ARGUMENT;
+  if (nbytes == 0) return AA_OK;
+  const int64_t n = nbytes >> 4;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 256 * 32) blocks = 256 * 32;
+  hipLaunchKernelGGL(k_copy16, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const uint4*)src,
+                     (uint4*)dst, n);
+  return launch_status();
+}
+
+extern "C" int aa_scale_inplace(void* data, int dtype, int64_t n, const float* factor, void* stream) {
+  if (!data || !factor || n < 0) return AA_ERR_INVALID_ARGUMENT;
+  if (n == 0) return AA_OK;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == AA_BF16) hipLaunchKernelGGL(k_scale<AA_BF16>, dim3((unsigned)blocks), dim3(256), 0, st, data, n, factor);
+  else if (dtype == AA_F16) hipLaunchKernelGGL(k_scale<AA_F16>, dim3((unsigned)blocks), dim3(256), 0, st, data, n, factor);
+  else if (dtype == AA_F32) hipLaunchKernelGGL(k_scale<AA_F32>, dim3((unsigned)blocks), dim3(256), 0, st, data, n, factor);
+  else return AA_ERR_INVALID_ARGUMENT;
+  return launch_status();
+}

@@ -1,0 +1,56 @@
+// Per-token arithmetic of the clipped PPO surrogate and of its derivative,
+// shared by the fused logits kernel and the stand-alone loss kernel.
+//
+// Follows areal/utils/functional/functional.py:516-539.  The derivative is the
+// one PyTorch autograd produces for that sequence of ops: torch.max/torch.min
+// of two tensors send half of the gradient to each operand where they are
+// equal, and torch.clamp passes gradient on the closed interval [lo, hi].
+#pragma once
+#include "device_utils.h"
+
+namespace aa {
+
+struct Surrogate {
+  float loss;      // pg_loss after the optional dual clip and behave weight
+  float dloss_dr;  // d(loss) / d(ratio)
+  bool clip;       // pg_loss1 < pg_loss2
+  bool dual;       // pg_loss3 < max(pg_loss1, pg_loss2)
+};
+
+// max/min that return NaN if either side is NaN (torch.max / torch.min do)
+__device__ __forceinline__ float nan_max(float a, float b) { return (a != a || b != b) ? (a + b) : fmaxf(a, b); }
+__device__ __forceinline__ float nan_min(float a, float b) { return (a != a || b != b) ? (a + b) : fminf(a, b); }
+
+__device__ __forceinline__ Surrogate surrogate(float r, float adv, float behave_w, const aa_ppo_params& P) {
+  // torch.clamp(r, lo, hi) = min(max(r, lo), hi), NaN stays NaN
+  float rc = nan_min(nan_max(r, P.clip_lo), P.clip_hi);
+  const bool in_range = (r >= P.clip_lo) && (r <= P.clip_hi);
+  const float na = -adv;
+  const float l1 = na * r;
+  const float l2 = na * rc;
+  Surrogate o;
+  o.clip = l1 < l2;
+  float l = nan_max(l1, l2);
+  // share of d(max)/d(l1); the rest goes to l2
+  const float w1 = (l1 == l2) ? 0.5f : ((l1 < l2) ? 0.f : 1.f);
+  const float w2 = (l1 == l2) ? 0.5f : ((l1 > l2) ? 0.f : 1.f);
+  float d = na * w1 + (in_range ? na * w2 : 0.f);
+  o.dual = false;
+  if (P.has_c_clip) {
+    const float sg = (adv > 0.f) ? 1.f : ((adv < 0.f) ? -1.f : adv);  // torch.sign, sign(0)=0, sign(NaN)=NaN
+    const float l3 = (sg * P.c_clip) * adv;
+    o.dual = l3 < l;
+    const float wl = (l == l3) ? 0.5f : ((l > l3) ? 0.f : 1.f);  // share of d(min)/d(l)
+    l = nan_min(l, l3);
+    d *= wl;
+  }
+  if (P.has_behave_weight) {
+    l *= behave_w;
+    d *= behave_w;
+  }
+  o.loss = l;
+  o.dloss_dr = d;
+  return o;
+}
+
+}  // namespace aa

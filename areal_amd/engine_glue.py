@@ -1,0 +1,82 @@
+"""The engine-side call contract of the path, as a small harness.
+
+Mirrors what FSDPEngine does around the functional ops for one packed
+micro-batch (areal/engine/fsdp_engine.py:1908-1964, 1977-2046) and the part of
+``grpo_loss_fn`` that feeds ``ppo_actor_loss_fn`` (areal/trainer/ppo/actor.py:408-480):
+labels are the packed ``input_ids`` rolled by one over the WHOLE packed tensor,
+the batch padding is trimmed after the log-prob op, entropy is detached, and the
+loss is scaled by ``local_weight / total_loss_weight * loss_multiplier``.
+"""
+from __future__ import annotations
+
+from typing import Any
+
+import torch
+
+from .functional import fused_logprobs_ppo_loss, gather_logprobs, gather_logprobs_entropy_stats, ppo_actor_loss_fn
+
+
+def rolled_labels(model_inputs: dict[str, Any]) -> torch.Tensor:
+    """``rolled_input_ids`` if present, else ``roll(input_ids, -1)``; a leading batch dim of 1 is dropped
+    (fsdp_engine.py:1915-1921).  The roll is over the packed tensor, not per sequence: the last token of a
+    sequence is labelled with the first token of the next one and is expected to be masked out."""
+    labels = model_inputs.get("rolled_input_ids")
+    if labels is None:
+        labels = torch.roll(model_inputs["input_ids"], shifts=-1, dims=-1)
+    if labels.ndim == 2 and labels.shape[0] == 1:
+        labels = labels.squeeze(0)
+    return labels
+
+
+def compute_logprobs(logits: torch.Tensor, model_inputs: dict[str, Any], temperature: float = 1.0) -> torch.Tensor:
+    """Forward-only log-probs of a micro-batch (fsdp_engine.py:1938-1964)."""
+    return gather_logprobs(logits, rolled_labels(model_inputs), temperature=temperature)
+
+
+def compute_logprobs_and_loss(
+    logits: torch.Tensor,
+    model_inputs: dict[str, Any],
+    mb_input: dict[str, Any],
+    pad_length: int,
+    total_loss_weight: torch.Tensor | float,
+    eps_clip: float,
+    eps_clip_higher: float | None = None,
+    c_clip: float | None = None,
+    rejection_sampling: Any | None = None,
+    importance_sampling_level: str = "token",
+    temperature: float = 1.0,
+    loss_multiplier: float = 1.0,
+    fused: bool = True,
+) -> tuple[torch.Tensor, dict]:
+    """Scaled PPO loss of one micro-batch and its stat dict (fsdp_engine.py:1977-2046 with
+    ``loss_fn = grpo_loss_fn`` and ``loss_weight_fn = loss_mask.count_nonzero``, actor.py:345-364).
+
+    ``logits`` is ``[T_pad, V]``; ``mb_input`` holds the un-padded ``[T]`` tensors ``loss_mask``, ``logprobs``
+    (behaviour policy), ``prox_logp``, ``advantages`` and ``cu_seqlens``.  An all-masked micro-batch returns
+    ``logits.mean() * 0`` like the reference (fsdp_engine.py:1988-1989).
+    """
+    loss_mask = mb_input["loss_mask"].bool()
+    local_weight = loss_mask.count_nonzero()
+    if local_weight == 0:
+        return logits.mean() * 0.0, {}
+    labels = rolled_labels(model_inputs)
+    old_logp = mb_input["logprobs"]
+    prox_logp = mb_input.get("prox_logp")
+    if prox_logp is None:
+        raise ValueError("prox_logp is None: only the recomputed proximal log-probs are supported here")
+    scale = local_weight / total_loss_weight * loss_multiplier
+    kw = dict(
+        eps_clip=eps_clip, eps_clip_higher=eps_clip_higher, c_clip=c_clip, rejection_sampling=rejection_sampling,
+        importance_sampling_level=importance_sampling_level, cu_seqlens=mb_input.get("cu_seqlens"),
+    )
+    if fused:
+        return fused_logprobs_ppo_loss(
+            logits, labels, prox_logp, old_logp, mb_input["advantages"], loss_mask=loss_mask,
+            temperature=temperature, loss_scale=scale, **kw,
+        )
+    logp, entropy, vmin, vmax = gather_logprobs_entropy_stats(logits, labels, temperature)
+    if pad_length > 0:
+        logp, entropy, vmin, vmax = (t[:-pad_length] for t in (logp, entropy, vmin, vmax))
+    loss, stat = ppo_actor_loss_fn(logp, prox_logp, old_logp, mb_input["advantages"], loss_mask=loss_mask, **kw)
+    stat.update(logprobs=logp.detach(), entropy=entropy.detach(), vocab_min_logits=vmin, vocab_max_logits=vmax)
+    return loss * scale, stat

@@ -1,0 +1,607 @@
+"""Drop-in functional API of the PPO/GRPO log-prob / entropy / actor-loss path.
+
+Same names, argument meaning and error behaviour as the reference's
+``areal.utils.functional`` (vocab_parallel.py:401-469, functional.py:185-559);
+the arithmetic runs in hand-written gfx950 kernels reached through the C ABI of
+``libareal_amd.so``.  PyTorch is used for device memory, streams and autograd
+bookkeeping only.  Tensors must live on a ROCm device: there is no CPU path.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Any
+
+import torch
+
+from . import _native as N
+
+__all__ = [
+    "RejectionSamplingResult",
+    "gather_logprobs",
+    "gather_logprobs_entropy",
+    "gather_logprobs_entropy_stats",
+    "apply_rejection_sampling",
+    "ppo_actor_loss_fn",
+    "fused_logprobs_ppo_loss",
+]
+
+_DTYPES = {torch.bfloat16: N.AA_BF16, torch.float16: N.AA_F16, torch.float32: N.AA_F32}
+
+
+# ----------------------------------------------------------------------------
+# helpers
+# ----------------------------------------------------------------------------
+def _ptr(t: torch.Tensor | None) -> C.c_void_p:
+    return C.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream(device: torch.device) -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _require_gpu(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise N.NativeLibraryError(
+            f"{name} is on {t.device}: areal_amd ops run on a ROCm GPU only (no CPU fallback)"
+        )
+
+
+def _f32(t: torch.Tensor) -> torch.Tensor:
+    return t.to(torch.float32).contiguous()
+
+
+def _mask_u8(mask: torch.Tensor) -> torch.Tensor:
+    """One byte per token, non-zero = valid, without a copy for bool masks."""
+    m = mask.contiguous()
+    if m.dtype == torch.bool:
+        return m.view(torch.uint8)
+    return (m != 0).view(torch.uint8)
+
+
+def _rows(logits: torch.Tensor) -> tuple[torch.Tensor, int, int, int]:
+    """View logits as [T, V] rows with unit inner stride; returns (2-D tensor, T, V, row stride)."""
+    V = logits.shape[-1]
+    x = logits.reshape(-1, V)
+    if x.dtype not in _DTYPES:
+        x = x.float()
+    if x.stride(-1) != 1 or (x.shape[0] > 1 and x.stride(0) < V):
+        x = x.contiguous()
+    T = x.shape[0]
+    stride = x.stride(0) if T > 1 else V
+    return x, T, V, stride
+
+
+def _check_tp(tp_group: Any) -> None:
+    if tp_group is not None:
+        import torch.distributed as dist
+
+        if dist.get_world_size(tp_group) > 1:
+            raise NotImplementedError(
+                "vocab-parallel log-probs (tp_group with more than one rank) are not part of the "
+                "single-GPU build; pass tp_group=None"
+            )
+
+
+def _ppo_params(eps_clip, eps_clip_higher, c_clip, has_w) -> N.PpoParams:
+    if c_clip is not None:
+        assert c_clip > 1.0, c_clip
+    hi = eps_clip if eps_clip_higher is None else eps_clip_higher
+    return N.PpoParams(
+        clip_lo=1.0 - eps_clip,
+        clip_hi=1.0 + hi,
+        c_clip=0.0 if c_clip is None else float(c_clip),
+        has_c_clip=0 if c_clip is None else 1,
+        has_behave_weight=1 if has_w else 0,
+    )
+
+
+# ----------------------------------------------------------------------------
+# log-probs / entropy
+# ----------------------------------------------------------------------------
+class _LogprobsEntropy(torch.autograd.Function):
+    """logp, entropy, vocab max, vocab min of each row; differentiable in logits."""
+
+    @staticmethod
+    def forward(ctx, logits2d, labels1d, temperature, stride, want_entropy, want_minmax):
+        lib = N.load()
+        T, V = logits2d.shape
+        dev = logits2d.device
+        kw = dict(dtype=torch.float32, device=dev)
+        logp = torch.empty(T, **kw)
+        entropy = torch.empty(T, **kw) if want_entropy else None
+        need_bwd = ctx.needs_input_grad[0]
+        row_lse = torch.empty(T, **kw) if need_bwd else None
+        row_ez = torch.empty(T, **kw) if (need_bwd and want_entropy) else None
+        vmax = torch.empty(T, **kw) if want_minmax else None
+        vmin = torch.empty(T, **kw) if want_minmax else None
+        with torch.cuda.device(dev):
+            N.check(
+                lib.aa_logits_fwd(
+                    _ptr(logits2d), _DTYPES[logits2d.dtype], T, V, stride, _ptr(labels1d),
+                    1.0 / float(temperature), _ptr(logp), _ptr(entropy), _ptr(row_lse), _ptr(row_ez),
+                    _ptr(vmax), _ptr(vmin), _stream(dev),
+                ),
+                "aa_logits_fwd",
+            )
+        ctx.save_for_backward(logits2d, labels1d, row_lse, row_ez)
+        ctx.temperature = float(temperature)
+        ctx.stride = stride
+        outs = (logp, entropy, vmax, vmin)
+        ctx.mark_non_differentiable(*[o for o in (vmax, vmin) if o is not None])
+        return outs
+
+    @staticmethod
+    def backward(ctx, g_logp, g_entropy, _g_vmax, _g_vmin):
+        lib = N.load()
+        logits2d, labels1d, row_lse, row_ez = ctx.saved_tensors
+        T, V = logits2d.shape
+        dev = logits2d.device
+        if g_logp is None:
+            g_logp = torch.zeros(T, dtype=torch.float32, device=dev)
+        g_logp = _f32(g_logp)
+        g_entropy = _f32(g_entropy) if (g_entropy is not None and row_ez is not None) else None
+        if ctx.stride == V:
+            dlogits = torch.empty_like(logits2d, memory_format=torch.contiguous_format)
+        else:  # keep the row stride of the input so that both buffers are walked alike
+            dlogits = torch.empty_strided((T, V), (ctx.stride, 1), dtype=logits2d.dtype, device=dev)
+        with torch.cuda.device(dev):
+            N.check(
+                lib.aa_logits_bwd(
+                    _ptr(logits2d), _DTYPES[logits2d.dtype], T, V, ctx.stride, _ptr(labels1d),
+                    1.0 / ctx.temperature, _ptr(row_lse), _ptr(row_ez), _ptr(g_logp), _ptr(g_entropy),
+                    T, _ptr(dlogits), _stream(dev),
+                ),
+                "aa_logits_bwd",
+            )
+        return dlogits, None, None, None, None, None
+
+
+def _logprobs_impl(logits, labels, temperature, tp_group, want_entropy, want_minmax):
+    _check_tp(tp_group)
+    _require_gpu(logits, "logits")
+    assert logits.shape[0] > 0, "Input logits must have at least one element"
+    if tuple(labels.shape) != tuple(logits.shape[:-1]):
+        raise ValueError(f"labels shape {tuple(labels.shape)} != logits shape[:-1] {tuple(logits.shape[:-1])}")
+    x, T, V, stride = _rows(logits)
+    y = labels.reshape(-1).to(device=x.device, dtype=torch.int64).contiguous()
+    logp, entropy, vmax, vmin = _LogprobsEntropy.apply(x, y, float(temperature), stride, want_entropy, want_minmax)
+    shp = labels.shape
+    return (
+        logp.view(shp),
+        entropy.view(shp) if entropy is not None else None,
+        vmax.view(shp) if vmax is not None else None,
+        vmin.view(shp) if vmin is not None else None,
+    )
+
+
+def gather_logprobs(
+    logits: torch.Tensor,
+    labels: torch.Tensor,
+    temperature: float = 1.0,
+    tp_group: Any | None = None,
+    chunk_size: int = 1024,
+) -> torch.Tensor:
+    """``log_softmax(logits.float() / temperature)[..., labels]`` as fp32, shaped like ``labels``.
+
+    Same contract as vocab_parallel.py:401-431.  ``chunk_size`` is accepted and
+    ignored: the kernel never materialises an fp32 copy of the logits, and the
+    result does not depend on chunking.
+    """
+    del chunk_size
+    return _logprobs_impl(logits, labels, temperature, tp_group, False, False)[0]
+
+
+def gather_logprobs_entropy(
+    logits: torch.Tensor,
+    labels: torch.Tensor,
+    temperature: float = 1.0,
+    tp_group: Any | None = None,
+    chunk_size: int = 1024,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """(log-probs at ``labels``, entropy of each row); vocab_parallel.py:434-469."""
+    del chunk_size
+    logp, entropy, _, _ = _logprobs_impl(logits, labels, temperature, tp_group, True, False)
+    return logp, entropy
+
+
+def gather_logprobs_entropy_stats(
+    logits: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(logp, entropy, vocab_min_logits, vocab_max_logits) from the same single pass.
+
+    The last two are what FSDPEngine._get_vocab_min_max_logits
+    (fsdp_engine.py:1893-1906) computes with two more passes over the logits.
+    """
+    logp, entropy, vmax, vmin = _logprobs_impl(logits, labels, temperature, None, True, True)
+    return logp, entropy, vmin, vmax
+
+
+# ----------------------------------------------------------------------------
+# rejection sampling
+# ----------------------------------------------------------------------------
+@dataclass
+class RejectionSamplingResult:
+    """functional.py:152-164"""
+
+    loss_mask: torch.Tensor
+    behave_imp_weight: torch.Tensor
+    filtered_fraction: float
+
+
+def _segments(shape, cu_seqlens, what: str):
+    """(cu_seqlens int32 tensor or None, number of segments) for a 1-D packed or 2-D padded layout."""
+    if len(shape) == 1:
+        if cu_seqlens is None:
+            raise ValueError(what)
+        cu = cu_seqlens.to(dtype=torch.int32).contiguous()
+        return cu, cu.shape[0] - 1
+    return None, shape[0]
+
+
+def _rejection_sampling_device(prox, old, mask_u8, shape, cu_seqlens, cfg):
+    """Runs the kernel; returns (mask_out u8 [n], weight f32 [n], counts i32 [3]) without syncing."""
+    lib = N.load()
+    dev = prox.device
+    n = prox.numel()
+    cu, B = (None, 0)
+    if cfg.level == "sequence":
+        cu, B = _segments(
+            shape, cu_seqlens, "cu_seqlens is required for 1D packed tensors in sequence-level filtering."
+        )
+        if cu is not None:
+            cu = cu.to(dev)
+    mask_out = torch.empty(n, dtype=torch.uint8, device=dev)
+    w = torch.empty(n, dtype=torch.float32, device=dev)
+    counts = torch.empty(3, dtype=torch.int32, device=dev)
+    lower = cfg.lower
+    with torch.cuda.device(dev):
+        N.check(
+            lib.aa_rejection_sampling(
+                _ptr(prox), _ptr(old), _ptr(mask_u8), n, _ptr(cu), B,
+                N.RS_LEVEL[cfg.level], N.RS_ACTION[cfg.action], N.RS_METRIC[cfg.metric], N.RS_AGG[cfg.agg],
+                float(cfg.upper), 0.0 if lower is None else float(lower), 0 if lower is None else 1,
+                _ptr(mask_out), _ptr(w), _ptr(counts), _stream(dev),
+            ),
+            "aa_rejection_sampling",
+        )
+    return mask_out, w, counts
+
+
+def _validate_rs(cfg) -> None:
+    for field, table in (("level", N.RS_LEVEL), ("action", N.RS_ACTION), ("agg", N.RS_AGG)):
+        if getattr(cfg, field) not in table:
+            raise ValueError(f"Unknown {field}: {getattr(cfg, field)}")
+    if cfg.metric not in N.RS_METRIC:
+        raise ValueError(f"Unknown metric: {cfg.metric}")
+
+
+def apply_rejection_sampling(
+    proximal_logprobs: torch.Tensor,
+    old_logprobs: torch.Tensor,
+    loss_mask: torch.Tensor,
+    cu_seqlens: torch.Tensor | None,
+    config: Any,
+) -> RejectionSamplingResult:
+    """Filter or clamp tokens / sequences by the divergence between the proximal
+    and the behaviour policy; functional.py:185-426.
+
+    ``config`` is any object with the attributes of ``RejectionSamplingConfig``.
+    """
+    if proximal_logprobs.shape != old_logprobs.shape:
+        raise ValueError(
+            f"proximal_logprobs shape {proximal_logprobs.shape} != old_logprobs shape {old_logprobs.shape}"
+        )
+    if proximal_logprobs.shape != loss_mask.shape:
+        raise ValueError(
+            f"proximal_logprobs shape {proximal_logprobs.shape} != loss_mask shape {loss_mask.shape}"
+        )
+    if proximal_logprobs.ndim not in (1, 2):
+        raise ValueError(f"Expected 1D (packed) or 2D (padded) tensors, got ndim={proximal_logprobs.ndim}")
+    _validate_rs(config)
+    _require_gpu(proximal_logprobs, "proximal_logprobs")
+    shape = proximal_logprobs.shape
+    prox = _f32(proximal_logprobs.detach()).reshape(-1)
+    old = _f32(old_logprobs.detach()).reshape(-1)
+    m8 = _mask_u8(loss_mask).reshape(-1)
+    mask_out, w, counts = _rejection_sampling_device(prox, old, m8, shape, cu_seqlens, config)
+    total, hit, _ = counts.tolist()  # the reference returns a Python float here too
+    if config.action == "mask":
+        new_mask = mask_out.view(shape).to(loss_mask.dtype)
+    else:
+        new_mask = loss_mask
+    return RejectionSamplingResult(
+        loss_mask=new_mask,
+        behave_imp_weight=w.view(shape),
+        filtered_fraction=hit / max(total, 1),
+    )
+
+
+# ----------------------------------------------------------------------------
+# PPO actor loss on log-probs
+# ----------------------------------------------------------------------------
+class _PpoLoss(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logp, prox, adv, mask_eff, behave_w, cu, B, seq_level, params, n_valid):
+        lib = N.load()
+        dev = logp.device
+        n = logp.numel()
+        stat_loss = torch.empty(n, dtype=torch.float32, device=dev)
+        ratio = torch.empty(n, dtype=torch.float32, device=dev)
+        flags = torch.empty(n, dtype=torch.uint8, device=dev)
+        g_logp = torch.empty(n, dtype=torch.float32, device=dev)
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            st = _stream(dev)
+            N.check(
+                lib.aa_ppo_loss(
+                    _ptr(logp), _ptr(prox), _ptr(adv), _ptr(mask_eff), _ptr(behave_w), n, _ptr(cu), B,
+                    1 if seq_level else 0, C.byref(params), _ptr(n_valid), _ptr(stat_loss), _ptr(ratio),
+                    _ptr(flags), _ptr(g_logp), st,
+                ),
+                "aa_ppo_loss",
+            )
+            N.check(
+                lib.aa_masked_sum(_ptr(stat_loss), _ptr(mask_eff), n, _ptr(n_valid), None, _ptr(loss), st),
+                "aa_masked_sum",
+            )
+        ctx.save_for_backward(g_logp)
+        ctx.mark_non_differentiable(stat_loss, ratio, flags)
+        return loss, stat_loss, ratio, flags
+
+    @staticmethod
+    def backward(ctx, g_loss, *_unused):
+        (g_logp,) = ctx.saved_tensors
+        return (g_logp * g_loss,) + (None,) * 9
+
+
+def _count_nonzero(mask_u8: torch.Tensor) -> torch.Tensor:
+    lib = N.load()
+    dev = mask_u8.device
+    out = torch.empty(1, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        N.check(lib.aa_count_nonzero_u8(_ptr(mask_u8), mask_u8.numel(), _ptr(out), _stream(dev)), "aa_count_nonzero_u8")
+    return out
+
+
+def _rs_stats(stat, prox, old, mask_eff_u8, w, counts, shape):
+    behave_mask = (w > 0) & mask_eff_u8.bool()
+    total, hit, _ = counts.tolist()
+    stat.update(
+        behave_approx_kl=torch.where(behave_mask, prox - old, 0.0).view(shape),
+        behave_imp_weight=w.view(shape),
+        behave_mask=behave_mask.view(shape),
+        filtered_fraction=hit / max(total, 1),
+    )
+
+
+def ppo_actor_loss_fn(
+    logprobs: torch.Tensor,
+    proximal_logprobs: torch.Tensor,
+    old_logprobs: torch.Tensor,
+    advantages: torch.Tensor,
+    eps_clip: float,
+    loss_mask: torch.Tensor,
+    eps_clip_higher: float | None = None,
+    c_clip: float | None = None,
+    rejection_sampling: Any | None = None,
+    importance_sampling_level: str = "token",
+    cu_seqlens: torch.Tensor | None = None,
+) -> tuple[torch.Tensor, dict]:
+    """Decoupled-proximal clipped PPO actor loss; functional.py:429-559.
+
+    Returns ``(loss, stat)`` with the reference's stat keys: ``loss``,
+    ``importance_weight``, ``approx_kl``, ``clip_mask``, ``dual_clip_mask`` and,
+    with rejection sampling, ``behave_approx_kl``, ``behave_imp_weight``,
+    ``behave_mask``, ``filtered_fraction``.  The loss is differentiable in
+    ``logprobs`` (closed-form gradient computed with the forward).
+    """
+    if importance_sampling_level not in ("token", "sequence"):
+        raise ValueError(
+            f"Invalid importance_sampling_level: {importance_sampling_level}. Must be 'token' or 'sequence'."
+        )
+    _require_gpu(logprobs, "logprobs")
+    shape = logprobs.shape
+    seq_level = importance_sampling_level == "sequence"
+    cu, B = None, 0
+    if seq_level:
+        cu, B = _segments(
+            shape,
+            cu_seqlens,
+            "cu_seqlens is required for 1D tensors (packed format). For a single sequence, use "
+            "cu_seqlens=torch.tensor([0, seq_len], dtype=torch.int32).",
+        )
+        if cu is not None:
+            cu = cu.to(logprobs.device)
+    params = _ppo_params(eps_clip, eps_clip_higher, c_clip, rejection_sampling is not None)
+
+    lp = _f32(logprobs).reshape(-1)
+    prox = _f32(proximal_logprobs.detach()).reshape(-1)
+    old = _f32(old_logprobs.detach()).reshape(-1)
+    adv = _f32(advantages.detach()).reshape(-1)
+    m8 = _mask_u8(loss_mask).reshape(-1)
+
+    w = counts = None
+    mask_eff = m8
+    if rejection_sampling is not None:
+        _validate_rs(rejection_sampling)
+        mask_eff, w, counts = _rejection_sampling_device(prox, old, m8, shape, cu_seqlens, rejection_sampling)
+        if rejection_sampling.action != "mask":
+            mask_eff = m8
+        n_valid = counts  # counts[0] is the non-zero count of the original mask
+    else:
+        n_valid = _count_nonzero(m8)
+
+    loss, stat_loss, ratio, flags = _PpoLoss.apply(lp, prox, adv, mask_eff, w, cu, B, seq_level, params, n_valid)
+    stat = dict(
+        loss=stat_loss.view(shape),
+        importance_weight=ratio.view(shape),
+        approx_kl=(lp.detach() - prox).view(shape),
+        clip_mask=(flags & 1).bool().view(shape),
+        dual_clip_mask=(flags & 2).bool().view(shape),
+    )
+    if rejection_sampling is not None:
+        _rs_stats(stat, prox, old, mask_eff, w, counts, shape)
+    return loss, stat
+
+
+# ----------------------------------------------------------------------------
+# fused: logits -> logp/entropy -> token-level PPO loss -> d(logits), one pass
+# ----------------------------------------------------------------------------
+class _FusedLogitsPpo(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits2d, labels1d, stride, temperature, T_active, prox, adv, mask_eff, behave_w, params,
+                n_valid, grad_scale, want_minmax):
+        lib = N.load()
+        T, V = logits2d.shape
+        dev = logits2d.device
+        f32 = dict(dtype=torch.float32, device=dev)
+        logp = torch.empty(T, **f32)
+        entropy = torch.empty(T, **f32)
+        vmax = torch.empty(T, **f32) if want_minmax else None
+        vmin = torch.empty(T, **f32) if want_minmax else None
+        stat_loss = torch.empty(T_active, **f32)
+        ratio = torch.empty(T_active, **f32)
+        flags = torch.empty(T_active, dtype=torch.uint8, device=dev)
+        loss = torch.empty((), **f32)
+        if stride == V:
+            dlogits = torch.empty_like(logits2d, memory_format=torch.contiguous_format)
+        else:
+            dlogits = torch.empty_strided((T, V), (stride, 1), dtype=logits2d.dtype, device=dev)
+        with torch.cuda.device(dev):
+            st = _stream(dev)
+            N.check(
+                lib.aa_logits_ppo_fused(
+                    _ptr(logits2d), _DTYPES[logits2d.dtype], T, V, stride, _ptr(labels1d), 1.0 / float(temperature),
+                    T_active, _ptr(prox), _ptr(adv), _ptr(mask_eff), _ptr(behave_w), C.byref(params),
+                    _ptr(n_valid), _ptr(grad_scale), _ptr(logp), _ptr(entropy), _ptr(vmax), _ptr(vmin),
+                    _ptr(stat_loss), _ptr(ratio), _ptr(flags), _ptr(dlogits), st,
+                ),
+                "aa_logits_ppo_fused",
+            )
+            N.check(
+                lib.aa_masked_sum(
+                    _ptr(stat_loss), _ptr(mask_eff), T_active, _ptr(n_valid), _ptr(grad_scale), _ptr(loss), st
+                ),
+                "aa_masked_sum",
+            )
+        ctx.save_for_backward(dlogits)
+        others = [logp, entropy, stat_loss, ratio, flags] + [t for t in (vmax, vmin) if t is not None]
+        ctx.mark_non_differentiable(*others)
+        return loss, logp, entropy, vmax, vmin, stat_loss, ratio, flags
+
+    @staticmethod
+    def backward(ctx, g_loss, *_unused):
+        lib = N.load()
+        (dlogits,) = ctx.saved_tensors
+        dev = dlogits.device
+        g = _f32(g_loss).reshape(1)
+        # d(logits) was written with the loss; an upstream factor other than 1 is
+        # applied in place (the kernel returns at once when the factor is 1).
+        n = (dlogits.shape[0] - 1) * dlogits.stride(0) + dlogits.shape[1]
+        with torch.cuda.device(dev):
+            N.check(
+                lib.aa_scale_inplace(_ptr(dlogits), _DTYPES[dlogits.dtype], n, _ptr(g), _stream(dev)),
+                "aa_scale_inplace",
+            )
+        return (dlogits,) + (None,) * 12
+
+
+def fused_logprobs_ppo_loss(
+    logits: torch.Tensor,
+    labels: torch.Tensor,
+    proximal_logprobs: torch.Tensor,
+    old_logprobs: torch.Tensor,
+    advantages: torch.Tensor,
+    eps_clip: float,
+    loss_mask: torch.Tensor,
+    eps_clip_higher: float | None = None,
+    c_clip: float | None = None,
+    rejection_sampling: Any | None = None,
+    importance_sampling_level: str = "token",
+    cu_seqlens: torch.Tensor | None = None,
+    temperature: float = 1.0,
+    loss_scale: torch.Tensor | float | None = None,
+) -> tuple[torch.Tensor, dict]:
+    """``gather_logprobs_entropy`` + ``ppo_actor_loss_fn`` (+ backward) in one pass over the logits.
+
+    ``logits`` is ``[T_pad, V]`` and ``labels`` ``[T_pad]`` (the batch-padded
+    micro-batch, fsdp_engine.py:1908-1936); the per-token tensors are the
+    un-padded ``[T]`` ones with ``T <= T_pad``: rows past ``T`` are the padding
+    the engine trims after the log-prob op (fsdp_engine.py:2027-2031) and get a
+    zero gradient.  ``loss_scale`` is the factor the engine multiplies the loss
+    with (fsdp_engine.py:2045); the returned loss already includes it, and
+    ``loss.backward()`` hands back a gradient that was written during the
+    forward pass.
+
+    The stat dict has the keys of ``ppo_actor_loss_fn`` plus ``logprobs``,
+    ``entropy``, ``vocab_min_logits`` and ``vocab_max_logits`` (all ``[T]``).
+    With ``importance_sampling_level="sequence"`` the loss of a token depends on
+    its whole sequence, so the call runs the unfused kernels instead.
+    """
+    if importance_sampling_level not in ("token", "sequence"):
+        raise ValueError(
+            f"Invalid importance_sampling_level: {importance_sampling_level}. Must be 'token' or 'sequence'."
+        )
+    _require_gpu(logits, "logits")
+    if logits.ndim != 2 or labels.ndim != 1 or labels.shape[0] != logits.shape[0]:
+        raise ValueError(f"expected logits [T, V] and labels [T], got {tuple(logits.shape)} and {tuple(labels.shape)}")
+    assert logits.shape[0] > 0, "Input logits must have at least one element"
+    T_active = loss_mask.shape[0]
+    if loss_mask.ndim != 1 or T_active > logits.shape[0]:
+        raise ValueError(f"loss_mask shape {tuple(loss_mask.shape)} does not fit logits {tuple(logits.shape)}")
+    for name, t in (("proximal_logprobs", proximal_logprobs), ("old_logprobs", old_logprobs), ("advantages", advantages)):
+        if t.shape != loss_mask.shape:
+            raise ValueError(f"{name} shape {tuple(t.shape)} != loss_mask shape {tuple(loss_mask.shape)}")
+    dev = logits.device
+    scale_t = None
+    if loss_scale is not None:
+        scale_t = torch.as_tensor(loss_scale, dtype=torch.float32, device=dev).reshape(1)
+
+    if importance_sampling_level == "sequence":
+        logp, entropy, vmin, vmax = gather_logprobs_entropy_stats(logits, labels, temperature)
+        logp, entropy, vmin, vmax = (t[:T_active] for t in (logp, entropy, vmin, vmax))
+        loss, stat = ppo_actor_loss_fn(
+            logp, proximal_logprobs, old_logprobs, advantages, eps_clip, loss_mask, eps_clip_higher, c_clip,
+            rejection_sampling, importance_sampling_level, cu_seqlens,
+        )
+        if scale_t is not None:
+            loss = loss * scale_t.squeeze(0)
+        stat.update(logprobs=logp.detach(), entropy=entropy.detach(), vocab_min_logits=vmin, vocab_max_logits=vmax)
+        return loss, stat
+
+    x, T, V, stride = _rows(logits)
+    y = labels.to(device=dev, dtype=torch.int64).contiguous()
+    prox = _f32(proximal_logprobs.detach())
+    old = _f32(old_logprobs.detach())
+    adv = _f32(advantages.detach())
+    m8 = _mask_u8(loss_mask)
+    params = _ppo_params(eps_clip, eps_clip_higher, c_clip, rejection_sampling is not None)
+    w = counts = None
+    mask_eff = m8
+    if rejection_sampling is not None:
+        _validate_rs(rejection_sampling)
+        mask_eff, w, counts = _rejection_sampling_device(prox, old, m8, loss_mask.shape, cu_seqlens, rejection_sampling)
+        if rejection_sampling.action != "mask":
+            mask_eff = m8
+        n_valid = counts
+    else:
+        n_valid = _count_nonzero(m8)
+    loss, logp, entropy, vmax, vmin, stat_loss, ratio, flags = _FusedLogitsPpo.apply(
+        x, y, stride, float(temperature), T_active, prox, adv, mask_eff, w, params, n_valid, scale_t, True
+    )
+    logp_a = logp[:T_active]
+    stat = dict(
+        loss=stat_loss,
+        importance_weight=ratio,
+        approx_kl=logp_a - prox,
+        clip_mask=(flags & 1).bool(),
+        dual_clip_mask=(flags & 2).bool(),
+        logprobs=logp_a,
+        entropy=entropy[:T_active],
+        vocab_min_logits=vmin[:T_active],
+        vocab_max_logits=vmax[:T_active],
+    )
+    if rejection_sampling is not None:
+        _rs_stats(stat, prox, old, mask_eff, w, counts, loss_mask.shape)
+    return loss, stat

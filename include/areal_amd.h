@@ -1,0 +1,226 @@
+/*
+ * areal_amd.h -- C ABI of the MI355X (gfx950) kernels behind AReaL's PPO/GRPO
+ * log-prob / entropy / actor-loss path.
+ *
+ * Every entry point takes plain device pointers and sizes, enqueues its work on
+ * the HIP stream it is given (hipStream_t passed as void*; NULL = the default
+ * stream), allocates nothing, and never synchronises the device.  The return
+ * value is an aa_status; a non-zero value means nothing was enqueued.
+ *
+ * Layout conventions (the reference's "packed 1-D" layout):
+ *   logits      [T, V]  row-major, element (t, j) at logits[t * row_stride + j]
+ *   labels      [T]     int64, already rolled by the caller
+ *   cu_seqlens  [B+1]   int32, cu_seqlens[i] = first token of sequence i
+ *   per-token   [T]     float32 unless stated, masks are one byte per token
+ *
+ * Reference citations are relative to the AReaL source tree.
+ */
+#ifndef AREAL_AMD_H
+#define AREAL_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  AA_OK = 0,
+  AA_ERR_INVALID_ARGUMENT = 1,
+  AA_ERR_UNSUPPORTED = 2,
+  AA_ERR_LAUNCH = 3
+} aa_status;
+
+/* element type of logits / hidden / weight buffers */
+typedef enum { AA_BF16 = 0, AA_F16 = 1, AA_F32 = 2 } aa_dtype;
+
+/* rejection-sampling switches; mirror RejectionSamplingConfig
+ * (areal/api/cli_args.py:1223-1385) */
+typedef enum { AA_RS_LEVEL_TOKEN = 0, AA_RS_LEVEL_SEQUENCE = 1 } aa_rs_level;
+typedef enum { AA_RS_ACTION_MASK = 0, AA_RS_ACTION_CLAMP = 1 } aa_rs_action;
+typedef enum { AA_RS_RATIO = 0, AA_RS_KL_K1 = 1, AA_RS_KL_K2 = 2, AA_RS_KL_K3 = 3 } aa_rs_metric;
+typedef enum { AA_RS_AGG_SUM = 0, AA_RS_AGG_MEAN = 1, AA_RS_AGG_MAX = 2 } aa_rs_agg;
+
+/* Clipped-surrogate parameters of ppo_actor_loss_fn
+ * (areal/utils/functional/functional.py:516-532). */
+typedef struct {
+  float clip_lo;       /* 1 - eps_clip                                   */
+  float clip_hi;       /* 1 + (eps_clip_higher or eps_clip)              */
+  float c_clip;        /* dual-clip factor, used only if has_c_clip != 0 */
+  int32_t has_c_clip;
+  int32_t has_behave_weight; /* multiply the loss by behave_w (rejection sampling on) */
+} aa_ppo_params;
+
+/* Library version (major * 10000 + minor * 100 + patch). */
+int aa_version(void);
+
+/* Text for an aa_status value (static storage). */
+const char* aa_status_string(int status);
+
+/* ------------------------------------------------------------------ */
+/* Logits path                                                         */
+/* ------------------------------------------------------------------ */
+
+/*
+ * Forward of gather_logprobs / gather_logprobs_entropy
+ * (areal/utils/functional/vocab_parallel.py:15-29, 401-469): one streaming
+ * pass per row, fp32 online softmax.
+ *   logp[t]    = z[label] - logsumexp(z),  z = logits[t, :] / temperature
+ *   entropy[t] = logsumexp(z) - sum_j softmax(z)_j * z_j          (nullable)
+ *   row_lse[t] = logsumexp(z)     row_ez[t] = sum_j softmax(z)_j z_j
+ *                (nullable; what aa_logits_bwd needs)
+ *   vmax / vmin = max / min of the raw row (nullable; replaces the two extra
+ *                passes of FSDPEngine._get_vocab_min_max_logits,
+ *                areal/engine/fsdp_engine.py:1893-1906)
+ * A label outside [0, V) yields logp = NaN and never faults.
+ */
+int aa_logits_fwd(const void* logits, int dtype, int64_t T, int64_t V,
+                  int64_t row_stride, const int64_t* labels,
+                  float inv_temperature, float* logp, float* entropy,
+                  float* row_lse, float* row_ez, float* vmax, float* vmin,
+                  void* stream);
+
+/*
+ * Backward of the same op (autograd of vocab_parallel.py:15-29; closed form
+ * as in vocab_parallel.py:339-370):
+ *   dlogits[t, j] = inv_temperature * ( g_logp[t] * (1[j == label] - p_j)
+ *                                     + g_entropy[t] * p_j * (row_ez[t] - z_j) )
+ * g_entropy may be NULL (treated as zero).  dlogits has the dtype and row
+ * stride of logits.  Rows with t >= T_active (the batch padding the caller
+ * trims after the op, fsdp_engine.py:2027-2031) are written as zeros.
+ */
+int aa_logits_bwd(const void* logits, int dtype, int64_t T, int64_t V,
+                  int64_t row_stride, const int64_t* labels,
+                  float inv_temperature, const float* row_lse,
+                  const float* row_ez, const float* g_logp,
+                  const float* g_entropy, int64_t T_active, void* dlogits,
+                  void* stream);
+
+/*
+ * Fused forward + token-level PPO loss + backward for one micro-batch
+ * (vocab_parallel.py:23-29 -> functional.py:429-559 with
+ * importance_sampling_level="token" -> autograd), one launch:
+ * each row is read once, and d(loss)/d(logits) is written once.
+ *
+ * Per-token inputs [T_active]: prox_logp, adv, mask_eff (uint8, the mask after
+ * rejection sampling), behave_w (nullable unless params->has_behave_weight).
+ * n_valid: device pointer to the int32 count of non-zero entries of the
+ *   ORIGINAL loss mask (functional.py:483); the loss is divided by
+ *   max(*n_valid, 1).
+ * grad_scale: device pointer to a float the gradient is multiplied by (the
+ *   engine's local_weight / total_loss_weight * multiplier,
+ *   fsdp_engine.py:2045); NULL = 1.
+ * Outputs [T]: logp, entropy (nullable), vmax, vmin (nullable);
+ * outputs [T_active]: stat_loss (per-token surrogate times behave_w, before
+ *   masking), ratio, flags (bit0 = clip_mask & mask_eff, bit1 =
+ *   dual_clip_mask & mask_eff); dlogits [T, V] in the dtype of logits (rows
+ *   >= T_active are zeros).  The scalar loss is finished by aa_masked_sum.
+ */
+int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int64_t V,
+                        int64_t row_stride, const int64_t* labels,
+                        float inv_temperature, int64_t T_active,
+                        const float* prox_logp, const float* adv,
+                        const uint8_t* mask_eff, const float* behave_w,
+                        const aa_ppo_params* params, const int32_t* n_valid,
+                        const float* grad_scale, float* logp, float* entropy,
+                        float* vmax, float* vmin, float* stat_loss,
+                        float* ratio, uint8_t* flags, void* dlogits,
+                        void* stream);
+
+/* ------------------------------------------------------------------ */
+/* Per-token PPO pieces                                                */
+/* ------------------------------------------------------------------ */
+
+/*
+ * apply_rejection_sampling (functional.py:185-426) on packed tokens.
+ * Segments come from cu_seqlens [B+1], or, when cu_seqlens is NULL, are B
+ * equal-length rows of n / B tokens (the reference's 2-D padded layout).
+ *   mask_in  uint8 [n]  (non-zero = valid)
+ *   mask_out uint8 [n]  updated mask (action mask) or a copy (action clamp)
+ *   behave_w float [n]  importance weight, zero where mask_out is zero
+ *   counts   int32 [3]  {non-zero entries of mask_in, filtered-or-clamped
+ *                        valid tokens, unused}; written, not accumulated
+ * lower is ignored unless has_lower != 0.
+ */
+int aa_rejection_sampling(const float* prox_logp, const float* old_logp,
+                          const uint8_t* mask_in, int64_t n,
+                          const int32_t* cu_seqlens, int64_t B, int level,
+                          int action, int metric, int agg, float upper,
+                          float lower, int has_lower, uint8_t* mask_out,
+                          float* behave_w, int32_t* counts, void* stream);
+
+/* counts[0] = number of non-zero bytes of mask[0..n) (functional.py:483). */
+int aa_count_nonzero_u8(const uint8_t* mask, int64_t n, int32_t* count,
+                        void* stream);
+
+/*
+ * ppo_actor_loss_fn given log-probs (functional.py:429-559), both
+ * importance-sampling levels, forward and closed-form backward in one call.
+ *   sequence_level != 0 selects the GSPO branch (functional.py:56-149), which
+ *   needs segments (cu_seqlens / B as in aa_rejection_sampling).
+ * Outputs [n]: stat_loss, ratio, flags (as in aa_logits_ppo_fused),
+ *   g_logp = d(loss)/d(logp) with loss = sum(mask_eff ? stat_loss : 0) /
+ *   max(*n_valid, 1).  The scalar loss is finished by aa_masked_sum.
+ */
+int aa_ppo_loss(const float* logp, const float* prox_logp, const float* adv,
+                const uint8_t* mask_eff, const float* behave_w, int64_t n,
+                const int32_t* cu_seqlens, int64_t B, int sequence_level,
+                const aa_ppo_params* params, const int32_t* n_valid,
+                float* stat_loss, float* ratio, uint8_t* flags, float* g_logp,
+                void* stream);
+
+/*
+ * out[0] = scale * sum_{i<n, mask[i] != 0} values[i] / max(*n_valid, 1)
+ * (functional.py:542), accumulated in a fixed order so that repeated calls are
+ * bit-identical.  n_valid may be NULL (divide by 1); scale may be NULL (1).
+ */
+int aa_masked_sum(const float* values, const uint8_t* mask, int64_t n,
+                  const int32_t* n_valid, const float* scale, float* out,
+                  void* stream);
+
+/* data[i] *= *factor for i < n (dtype as aa_dtype); a no-op when *factor == 1. */
+int aa_scale_inplace(void* data, int dtype, int64_t n, const float* factor,
+                     void* stream);
+
+/* ------------------------------------------------------------------ */
+/* Fused lm_head path (no counterpart in the reference: its equivalent is  */
+/* logits = hidden @ weight.T followed by the logits path above)           */
+/* ------------------------------------------------------------------ */
+
+/* Bytes of workspace aa_lmhead_fwd / aa_lmhead_bwd need for these sizes. */
+int64_t aa_lmhead_workspace_bytes(int64_t T, int64_t H, int64_t V);
+
+/*
+ * logp / entropy of softmax(hidden @ weight.T / temperature) without writing
+ * the [T, V] logits: bf16 MFMA tiles with an online-softmax epilogue.
+ * hidden [T, H] bf16 row-major, weight [V, H] bf16 row-major.
+ * row_lse / row_ez as in aa_logits_fwd (needed by aa_lmhead_bwd).
+ */
+int aa_lmhead_fwd(const void* hidden, const void* weight, int64_t T, int64_t H,
+                  int64_t V, const int64_t* labels, float inv_temperature,
+                  float* logp, float* entropy, float* row_lse, float* row_ez,
+                  void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
+ * Backward of aa_lmhead_fwd: d_hidden [T, H] bf16 and d_weight [V, H] fp32
+ * (overwritten, fp32 accumulation), given g_logp and optional g_entropy.
+ */
+int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, int64_t H,
+                  int64_t V, const int64_t* labels, float inv_temperature,
+                  const float* row_lse, const float* row_ez,
+                  const float* g_logp, const float* g_entropy, void* d_hidden,
+                  float* d_weight, void* workspace, int64_t workspace_bytes,
+                  void* stream);
+
+/* ------------------------------------------------------------------ */
+/* Measurement helper                                                  */
+/* ------------------------------------------------------------------ */
+
+/* dst[0..nbytes) = src[0..nbytes), 16-byte aligned, nbytes % 16 == 0: the
+ * plain copy the HBM counters of the other kernels are calibrated against. */
+int aa_copy_bytes(const void* src, void* dst, int64_t nbytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AREAL_AMD_H */

@@ -1,0 +1,173 @@
+"""GPU parity of gather_logprobs / gather_logprobs_entropy (forward and backward) against the CPU oracle.
+
+Tolerances are the ones the task states: log-probs within 2e-3 absolute of an fp32/fp64 reference, gradient
+cosine similarity above 0.9999; integer indexing (labels) bit-exact, which shows as exact agreement of the
+gathered element."""
+import math
+
+import pytest
+import torch
+
+import areal_amd
+import oracle
+from helpers import cosine
+
+pytestmark = pytest.mark.gpu
+
+LOGP_ATOL = 2e-3   # stated tolerance
+TIGHT = 2e-5       # what fp32 accumulation actually delivers
+
+
+def _case(T, V, dtype, seed, std=3.0):
+    g = torch.Generator().manual_seed(seed)
+    x = (std * torch.randn(T, V, generator=g)).to(dtype)
+    y = torch.randint(0, V, (T,), generator=g)
+    return x, y
+
+
+@pytest.mark.parametrize(
+    "T,V,dtype",
+    [
+        (37, 128, torch.float32),       # the reference's determinism-test shape class
+        (33, 1000, torch.bfloat16),
+        (5, 50257, torch.bfloat16),     # odd V: rows are not 16-byte aligned
+        (19, 32003, torch.float16),
+        (3, 151936, torch.bfloat16),    # the benchmark vocabulary
+        (2, 262144, torch.float32),
+        (1, 7, torch.bfloat16),         # shorter than one vector
+    ],
+)
+@pytest.mark.parametrize("temperature", [1.0, 0.7])
+def test_forward_matches_oracle(device, T, V, dtype, temperature):
+    x, y = _case(T, V, dtype, seed=T + V)
+    lp, ent = areal_amd.gather_logprobs_entropy(x.to(device), y.to(device), temperature)
+    lp_only = areal_amd.gather_logprobs(x.to(device), y.to(device), temperature)
+    ref_lp, ref_ent = oracle.logprobs_entropy_f64(x, y, temperature)
+    assert lp.dtype == torch.float32 and lp.shape == y.shape
+    assert float((lp.cpu().double() - ref_lp).abs().max()) < min(LOGP_ATOL, TIGHT * max(1.0, math.log(V)))
+    assert float((ent.cpu().double() - ref_ent).abs().max()) < 1e-4
+    assert torch.equal(lp_only, lp)
+    # fp32 restatement of the reference path agrees as well
+    o_lp, o_ent = oracle.logprobs_entropy(x, y, temperature)
+    assert float((lp.cpu() - o_lp).abs().max()) < 1e-4
+
+
+def test_vocab_min_max_by_products_are_exact(device):
+    x, y = _case(9, 4099, torch.bfloat16, seed=3)
+    lp, ent, vmin, vmax = areal_amd.gather_logprobs_entropy_stats(x.to(device), y.to(device))
+    assert torch.equal(vmin.cpu(), x.min(-1).values.float())
+    assert torch.equal(vmax.cpu(), x.max(-1).values.float())
+
+
+def test_leading_dims_strides_and_label_dtypes(device):
+    x, y = _case(24, 515, torch.bfloat16, seed=5)
+    ref, _ = oracle.logprobs_entropy_f64(x, y)
+    # [B, S, V] input, int32 labels
+    lp3 = areal_amd.gather_logprobs(x.view(4, 6, 515).to(device), y.view(4, 6).int().to(device))
+    assert lp3.shape == (4, 6)
+    assert float((lp3.cpu().double().view(-1) - ref).abs().max()) < TIGHT * 10
+    # rows of a wider buffer (row stride > V)
+    wide = torch.zeros(24, 640, dtype=torch.bfloat16, device=device)
+    wide[:, :515] = x.to(device)
+    lp_s = areal_amd.gather_logprobs(wide[:, :515], y.to(device))
+    assert torch.equal(lp_s, lp3.view(-1))
+    # offset view: base pointer not 16-byte aligned
+    flat = torch.zeros(24 * 515 + 3, dtype=torch.bfloat16, device=device)
+    flat[3:] = x.to(device).reshape(-1)
+    lp_o = areal_amd.gather_logprobs(flat[3:].view(24, 515), y.to(device))
+    assert float((lp_o - lp_s).abs().max()) < 1e-5
+
+
+def test_closed_forms_and_stability(device):
+    V = 4096
+    x = torch.full((2, V), 0.75, dtype=torch.bfloat16, device=device)
+    y = torch.tensor([0, V - 1], device=device)
+    lp, ent = areal_amd.gather_logprobs_entropy(x, y)
+    assert float((lp + math.log(V)).abs().max()) < 1e-5 and float((ent - math.log(V)).abs().max()) < 1e-4
+    x = torch.zeros(1, V, device=device)
+    x[0, 9] = 80.0
+    lp, ent = areal_amd.gather_logprobs_entropy(x, torch.tensor([9], device=device))
+    assert abs(float(lp)) < 1e-6 and abs(float(ent)) < 1e-6
+    # logits scaled by 100 stay finite and match (run_vocab_parallel.py:169-215 of the reference)
+    g = torch.Generator().manual_seed(7)
+    big = torch.randn(6, 333, generator=g) * 100
+    yy = torch.randint(0, 333, (6,), generator=g)
+    lp, ent = areal_amd.gather_logprobs_entropy(big.to(device), yy.to(device))
+    r_lp, r_ent = oracle.logprobs_entropy_f64(big, yy)
+    assert torch.isfinite(lp).all() and float((lp.cpu().double() - r_lp).abs().max()) < 1e-3
+    assert float((ent.cpu().double() - r_ent).abs().max()) < 1e-3
+    # shift invariance
+    a = areal_amd.gather_logprobs(big.to(device) / 100, yy.to(device))
+    b = areal_amd.gather_logprobs(big.to(device) / 100 + 5.0, yy.to(device))
+    assert float((a - b).abs().max()) < 1e-5
+
+
+def test_two_calls_are_bit_identical(device):
+    # tests/test_cuda_deterministic.py:199-225 of the reference asks rtol=0, atol=0 of its compiled op
+    torch.manual_seed(42)
+    x = torch.randn(32, 128, device=device)
+    y = torch.randint(0, 128, (32,), device=device)
+    a = areal_amd.gather_logprobs_entropy(x, y)
+    b = areal_amd.gather_logprobs_entropy(x, y)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    xb = (3 * torch.randn(16, 151936, device=device)).bfloat16()
+    yb = torch.randint(0, 151936, (16,), device=device)
+    a = areal_amd.gather_logprobs_entropy(xb, yb)
+    b = areal_amd.gather_logprobs_entropy(xb, yb)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+def test_errors_and_out_of_range_labels(device):
+    with pytest.raises(AssertionError):
+        areal_amd.gather_logprobs(torch.zeros(0, 8, device=device), torch.zeros(0, dtype=torch.long, device=device))
+    with pytest.raises(ValueError, match="shape"):
+        areal_amd.gather_logprobs(torch.zeros(2, 8, device=device), torch.zeros(3, dtype=torch.long, device=device))
+    x = torch.randn(3, 64, device=device)
+    y = torch.tensor([5, 64, -1], device=device)  # only the first is valid
+    lp = areal_amd.gather_logprobs(x, y)
+    assert torch.isfinite(lp[0]) and torch.isnan(lp[1]) and torch.isnan(lp[2])
+
+
+@pytest.mark.parametrize(
+    "T,V,dtype,temperature,with_entropy",
+    [
+        (11, 257, torch.float32, 1.0, True),
+        (11, 257, torch.float32, 0.6, True),
+        (7, 4104, torch.bfloat16, 1.0, False),
+        (7, 4104, torch.bfloat16, 0.7, True),
+        (4, 50257, torch.bfloat16, 1.0, True),
+        (5, 1031, torch.float16, 1.3, True),
+        (2, 151936, torch.bfloat16, 1.0, False),
+    ],
+)
+def test_backward_matches_autograd_of_oracle(device, T, V, dtype, temperature, with_entropy):
+    x, y = _case(T, V, dtype, seed=11 * T + V, std=2.0)
+    g = torch.Generator().manual_seed(1)
+    gl = torch.randn(T, generator=g)
+    gh = torch.randn(T, generator=g) if with_entropy else None
+    gl[0] = 0.0  # a row without log-prob gradient
+    xd = x.to(device).requires_grad_(True)
+    if with_entropy:
+        lp, ent = areal_amd.gather_logprobs_entropy(xd, y.to(device), temperature)
+        ((lp * gl.to(device)).sum() + (ent * gh.to(device)).sum()).backward()
+    else:
+        lp = areal_amd.gather_logprobs(xd, y.to(device), temperature)
+        (lp * gl.to(device)).sum().backward()
+    got = xd.grad
+    assert got.dtype == dtype and got.shape == x.shape
+    want64 = oracle.logprobs_entropy_grad_closed_form(x, y, gl, gh, temperature)
+    # autograd of the fp32 restatement (what the reference itself would return in this dtype)
+    xo = x.clone().requires_grad_(True)
+    o_lp, o_ent = oracle.logprobs_entropy(xo, y, temperature)
+    ((o_lp * gl).sum() + ((o_ent * gh).sum() if with_entropy else 0.0)).backward()
+    assert cosine(got.cpu(), want64) > 0.9999
+    assert cosine(got.cpu(), xo.grad) > 0.9999
+    if dtype == torch.float32:
+        assert float((got.cpu().double() - want64).abs().max()) < 1e-5  # atol of run_vocab_parallel.py:257-317
+    else:
+        # no worse than one rounding of the exact value to the storage type
+        err = (got.cpu().double() - want64).abs()
+        assert bool((err <= want64.abs() * 2 ** -7 + 1e-6).all())
+    if not with_entropy:
+        assert float(got[0].float().abs().max()) == 0.0
+        assert float(got.float().sum(-1).abs().max()) < 5e-2  # each row of (onehot - p) sums to zero
