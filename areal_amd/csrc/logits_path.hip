@@ -8,9 +8,10 @@
 //
 // All kernels are HBM-streaming kernels: one workgroup owns one row of the
 // [T, V] logits.  Exponentials are taken in base 2 with c = log2(e) / T folded
-// into one fma per element; row statistics are carried as
-//   k = max_j x_j * c,   s = sum_j 2^(x_j c - k),   u = sum_j x_j 2^(x_j c - k)
-// so that  log2-sum-exp = k + log2 s  exactly reuses the rounded k.
+// into one fma per element; with t_j = x_j c - k row statistics are carried as
+//   k = max_j x_j * c,   s = sum_j 2^t_j,   u = sum_j t_j 2^t_j
+// so that  logp = ln2 (t_label - log2 s)  and  entropy = ln2 (log2 s - u / s)
+// are differences of small numbers whatever the magnitude of the logits.
 #include "device_utils.h"
 #include "ppo_math.h"
 
@@ -46,15 +47,22 @@ struct ThreadStats {
   float k, s, u, mx, mn;
 };
 
+// move the partial sums to a larger reference exponent k_new >= a.k
+__device__ __forceinline__ void rebase(ThreadStats& a, float k_new) {
+  const float d = a.k - k_new;
+  const float f = fast_exp2(d);
+  a.u = f * fmaf(d, a.s, a.u);
+  a.s *= f;
+  a.k = k_new;
+}
+
 __device__ __forceinline__ void stats_add1(ThreadStats& a, float x, float c) {
   const float xc = x * c;
-  if (xc > a.k) {
-    const float f = fast_exp2(a.k - xc);
-    a.s *= f; a.u *= f; a.k = xc;
-  }
-  const float e = fast_exp2(fmaf(x, c, -a.k));
+  if (xc > a.k) rebase(a, xc);
+  const float t = fmaf(x, c, -a.k);
+  const float e = fast_exp2(t);
   a.s += e;
-  a.u = fmaf(x, e, a.u);
+  a.u = fmaf(t, e, a.u);
   a.mx = fmaxf(a.mx, x);
   a.mn = fminf(a.mn, x);
 }
@@ -63,18 +71,16 @@ __device__ __forceinline__ void stats_add8(ThreadStats& a, const float (&x)[8], 
   float m8 = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
   float n8 = fminf(fminf(fminf(x[0], x[1]), fminf(x[2], x[3])), fminf(fminf(x[4], x[5]), fminf(x[6], x[7])));
   const float kc = m8 * c;
-  if (kc > a.k) {
-    const float f = fast_exp2(a.k - kc);
-    a.s *= f; a.u *= f; a.k = kc;
-  }
+  if (kc > a.k) rebase(a, kc);
   a.mx = fmaxf(a.mx, m8);
   a.mn = fminf(a.mn, n8);
   float s = 0.f, u = 0.f;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const float e = fast_exp2(fmaf(x[i], c, -a.k));
+    const float t = fmaf(x[i], c, -a.k);
+    const float e = fast_exp2(t);
     s += e;
-    u = fmaf(x[i], e, u);
+    u = fmaf(t, e, u);
   }
   a.s += s;
   a.u += u;
@@ -91,9 +97,10 @@ template <int NWAVES>
 __device__ __forceinline__ RowStats block_stats(const ThreadStats& t, float* smem) {
   static_assert(NWAVES >= 1 && NWAVES <= 16 && (NWAVES & (NWAVES - 1)) == 0, "power-of-two wave count");
   const float wk = wave_max(t.k);
-  const float f = fast_exp2(t.k - wk);
+  const float dk = t.k - wk;
+  const float f = fast_exp2(dk);
   const float ws = wave_sum(t.s * f);
-  const float wu = wave_sum(t.u * f);
+  const float wu = wave_sum(f * fmaf(dk, t.s, t.u));
   const float wmx = wave_max(t.mx);
   const float wmn = wave_min(t.mn);
   const int lane = threadIdx.x & (kWave - 1);
@@ -112,10 +119,11 @@ __device__ __forceinline__ RowStats block_stats(const ThreadStats& t, float* sme
     const float qs = __shfl_xor(r.s, o, kWave);
     const float qu = __shfl_xor(r.u, o, kWave);
     const float nk = fmaxf(r.k, qk);
-    const float fa = fast_exp2(r.k - nk), fb = fast_exp2(qk - nk);
+    const float da = r.k - nk, db = qk - nk;
+    const float fa = fast_exp2(da), fb = fast_exp2(db);
     // symmetric in (r, q): both partners compute bit-identical sums
+    r.u = fa * fmaf(da, r.s, r.u) + fb * fmaf(db, qs, qu);
     r.s = r.s * fa + qs * fb;
-    r.u = r.u * fa + qu * fb;
     r.k = nk;
     r.mx = fmaxf(r.mx, __shfl_xor(r.mx, o, kWave));
     r.mn = fminf(r.mn, __shfl_xor(r.mn, o, kWave));
@@ -140,17 +148,27 @@ __device__ __forceinline__ RowStats row_stats_generic(const void* row, int V, bo
 
 // Row-level quantities derived from the merged statistics.
 struct RowOut {
-  float lse2;  // log2 sum_j 2^(x_j c)
-  float lse;   // natural-log logsumexp of z = x / T
-  float ez;    // sum_j p_j z_j
+  float log2s;    // log2 s
+  float lse2;     // log2 sum_j 2^(x_j c) = k + log2 s
+  float lse;      // natural-log logsumexp of z = x / T
+  float ez;       // sum_j p_j z_j
+  float entropy;  // lse - ez, formed without cancellation
 };
 
-__device__ __forceinline__ RowOut finish_row(const RowStats& r, float inv_t) {
+__device__ __forceinline__ RowOut finish_row(const RowStats& r) {
   RowOut o;
-  o.lse2 = r.k + fast_log2(r.s);
+  const float mean_t = r.u / r.s;  // sum_j p_j t_j  (<= 0)
+  o.log2s = fast_log2(r.s);
+  o.lse2 = r.k + o.log2s;
   o.lse = o.lse2 * kLn2;
-  o.ez = (r.u / r.s) * inv_t;
+  o.ez = (r.k + mean_t) * kLn2;
+  o.entropy = (o.log2s - mean_t) * kLn2;
   return o;
+}
+
+// log-prob of the label from its raw logit
+__device__ __forceinline__ float label_logp(float xy, float c, const RowStats& r, const RowOut& o) {
+  return (fmaf(xy, c, -r.k) - o.log2s) * kLn2;
 }
 
 // out_j = p_j * (A + B x_j), p_j = 2^(x_j c - lse2); the label gets + lab_add.
@@ -218,9 +236,9 @@ __global__ __launch_bounds__(NT) void k_logits_fwd(const void* __restrict__ logi
   const float xy = y_ok ? Elem<DT>::load1(row, y) : 0.f;
   const RowStats rs = row_stats_generic<DT, NT>(row, V, vec_ok != 0, c, smem);
   if (threadIdx.x == 0) {
-    const RowOut ro = finish_row(rs, inv_t);
-    logp[t] = y_ok ? fmaf(xy, c, -ro.lse2) * kLn2 : __builtin_nanf("");
-    if (entropy) entropy[t] = ro.lse - ro.ez;
+    const RowOut ro = finish_row(rs);
+    logp[t] = y_ok ? label_logp(xy, c, rs, ro) : __builtin_nanf("");
+    if (entropy) entropy[t] = ro.entropy;
     if (row_lse) row_lse[t] = ro.lse;
     if (row_ez) row_ez[t] = ro.ez;
     if (vmax) vmax[t] = rs.mx;
@@ -287,7 +305,7 @@ __device__ __forceinline__ float fused_token_tail(const FusedTokenArgs& a, int64
                                                   const RowOut& ro, bool writer) {
   if (writer) {
     a.logp[t] = lp;
-    if (a.entropy) a.entropy[t] = ro.lse - ro.ez;
+    if (a.entropy) a.entropy[t] = ro.entropy;
     if (a.vmax) a.vmax[t] = rs.mx;
     if (a.vmin) a.vmin[t] = rs.mn;
   }
@@ -323,8 +341,8 @@ __global__ __launch_bounds__(NT) void k_fused_generic(const void* __restrict__ l
   const bool y_ok = (y >= 0) && (y < V);
   const float xy = y_ok ? Elem<DT>::load1(row, y) : 0.f;
   const RowStats rs = row_stats_generic<DT, NT>(row, V, vec_ok != 0, c, smem);
-  const RowOut ro = finish_row(rs, inv_t);
-  const float lp = y_ok ? fmaf(xy, c, -ro.lse2) * kLn2 : __builtin_nanf("");
+  const RowOut ro = finish_row(rs);
+  const float lp = y_ok ? label_logp(xy, c, rs, ro) : __builtin_nanf("");
   const float g = fused_token_tail(a, t, lp, rs, ro, threadIdx.x == 0);
   if (g == 0.f) {
     row_zero_generic<DT, NT>(row, out, V, vec_ok != 0);
@@ -342,8 +360,13 @@ __global__ __launch_bounds__(NT) void k_fused_generic(const void* __restrict__ l
 // row and one write of its gradient.  Requires V % 8 == 0, 16-byte aligned
 // rows and 8192 * (NCH - 1) < V <= 8192 * NCH, so that only the last chunk can
 // be partly out of range.  Rows are addressed through buffer descriptors: one
-// VGPR offset per thread, the chunk offset in an SGPR, and the hardware drops
-// out-of-range lanes (loads return 0, stores are ignored).
+// VGPR offset per thread, and the hardware drops out-of-range lanes (loads
+// return 0, stores are ignored).  Loads take the chunk offset in the scalar
+// offset operand.  Stores must NOT: with a register in the scalar-offset operand
+// the compiler leaves out the wait states between a 16-byte buffer store and
+// the next write of its data registers, and on gfx950 the store then picks up
+// the overwritten value in some lanes.  The chunk offset of a store is added to
+// the VGPR offset instead.
 // -----------------------------------------------------------------------------
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 constexpr int kBufferFlags = 0x00020000;  // raw buffer, 32-bit data format
@@ -413,11 +436,11 @@ __global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ l
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const float lo = Elem<DT>::lo(d[i][q]), hi = Elem<DT>::hi(d[i][q]);
-      const float e0 = fast_exp2(fmaf(lo, c, -ts.k));
-      const float e1 = fast_exp2(fmaf(hi, c, -ts.k));
+      const float t0 = fmaf(lo, c, -ts.k), t1 = fmaf(hi, c, -ts.k);
+      const float e0 = fast_exp2(t0), e1 = fast_exp2(t1);
       cs += e0 + e1;
-      cu = fmaf(lo, e0, cu);
-      cu = fmaf(hi, e1, cu);
+      cu = fmaf(t0, e0, cu);
+      cu = fmaf(t1, e1, cu);
     }
     if (i == NCH - 1 && !last_ok) { cs = 0.f; cu = 0.f; }
     s += cs;
@@ -426,14 +449,14 @@ __global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ l
   ts.s = s; ts.u = u;
   keep_packed(d);
   const RowStats rs = block_stats<NT / kWave>(ts, smem);
-  const RowOut ro = finish_row(rs, inv_t);
-  const float lp = y_ok ? fmaf(xy, c, -ro.lse2) * kLn2 : __builtin_nanf("");
+  const RowOut ro = finish_row(rs);
+  const float lp = y_ok ? label_logp(xy, c, rs, ro) : __builtin_nanf("");
   const float g = fused_token_tail(a, t, lp, rs, ro, tid == 0);
 
   if (g == 0.f) {
     const u32x4_t z = {0u, 0u, 0u, 0u};
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, voff, i * kChunkBytes, 0);
+    for (int i = 0; i < NCH; ++i) __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, voff + i * kChunkBytes, 0, 0);
     return;
   }
   const float A = -g * inv_t;
@@ -458,7 +481,7 @@ __global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ l
     r[1] = Elem<DT>::pack(o[2], o[3]);
     r[2] = Elem<DT>::pack(o[4], o[5]);
     r[3] = Elem<DT>::pack(o[6], o[7]);
-    __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff, i * kChunkBytes, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + i * kChunkBytes, 0, 0);
   }
 }
 

@@ -20,8 +20,8 @@ def _finish_case(case, seed=0):
 
 def _oracle_step(case, pad=0, **over):
     kw = dict(case.ppo)
-    rs = kw.pop("rejection_sampling", None)
     kw.update(over)
+    rs = kw.pop("rejection_sampling", None)
     cfg = RejectionSamplingConfig(**rs) if isinstance(rs, dict) else rs
     n = case.n_tokens - pad
     return oracle.logits_ppo_step(
@@ -33,8 +33,8 @@ def _oracle_step(case, pad=0, **over):
 
 def _fused_step(case, pad=0, **over):
     kw = dict(case.ppo)
-    rs = kw.pop("rejection_sampling", None)
     kw.update(over)
+    rs = kw.pop("rejection_sampling", None)
     cfg = RejectionSamplingConfig(**rs) if isinstance(rs, dict) else rs
     n = case.n_tokens - pad
     x = case.logits.clone().requires_grad_(True)
@@ -117,7 +117,7 @@ def test_fused_equals_unfused_kernels_and_sequence_level_falls_back(device):
     lp, ent = areal_amd.gather_logprobs_entropy(x, case.labels)
     loss, stat = areal_amd.ppo_actor_loss_fn(lp, case.prox_logp, case.old_logp, case.advantages, 0.2, case.loss_mask)
     loss.backward()
-    assert float(f_loss) == pytest.approx(float(loss), rel=1e-6)
+    assert float(f_loss) == pytest.approx(float(loss.detach()), rel=1e-6)
     assert float((f_stat["logprobs"] - lp.detach()).abs().max()) < 1e-5
     assert cosine(f_grad, x.grad) > 0.999999
     # GSPO: per-token loss depends on the whole sequence -> unfused kernels, same API

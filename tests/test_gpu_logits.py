@@ -70,7 +70,7 @@ def test_leading_dims_strides_and_label_dtypes(device):
     wide = torch.zeros(24, 640, dtype=torch.bfloat16, device=device)
     wide[:, :515] = x.to(device)
     lp_s = areal_amd.gather_logprobs(wide[:, :515], y.to(device))
-    assert torch.equal(lp_s, lp3.view(-1))
+    assert float((lp_s - lp3.view(-1)).abs().max()) < 1e-5  # other alignment, other summation order
     # offset view: base pointer not 16-byte aligned
     flat = torch.zeros(24 * 515 + 3, dtype=torch.bfloat16, device=device)
     flat[3:] = x.to(device).reshape(-1)
