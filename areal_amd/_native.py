@@ -50,7 +50,7 @@ SIGNATURES = {
     "aa_logits_ppo_fused": (
         _i,
         [_p, _i, _i64, _i64, _i64, _p, _f, _i64, _p, _p, _p, _p, C.POINTER(PpoParams), _p, _p,
-         _p, _p, _p, _p, _p, _p, _p, _p, _p],
+         _p, _p, _p, _p, _p, _p, _p, _p, _p, _p],
     ),
     "aa_rejection_sampling": (_i, [_p, _p, _p, _i64, _p, _i64, _i, _i, _i, _i, _f, _f, _i, _p, _p, _p, _p]),
     "aa_count_nonzero_u8": (_i, [_p, _i64, _p, _p]),

@@ -300,32 +300,90 @@ struct FusedTokenArgs {
   int64_t T_active;
 };
 
+// Per-token inputs of the loss, fetched ahead of the row statistics so that
+// their latency hides behind the streaming passes.  The loads are
+// unconditional (index clamped into [0, T_active)) and nothing is converted
+// here, so no wait is forced at the point of issue.  Needs T_active > 0.
+struct TokenIn {
+  float prox, adv, w;
+  uint8_t mask_raw;
+  bool active;
+  __device__ __forceinline__ bool mask() const { return active && mask_raw != 0; }
+};
+
+__device__ __forceinline__ TokenIn load_token_in(const FusedTokenArgs& a, int64_t t) {
+  TokenIn in;
+  in.active = t < a.T_active;
+  const int64_t tc = in.active ? t : a.T_active - 1;
+  in.mask_raw = a.mask_eff[tc];
+  in.prox = a.prox_logp[tc];
+  in.adv = a.adv[tc];
+  in.w = a.P.has_behave_weight ? a.behave_w[tc] : 1.f;
+  return in;
+}
+
+// Same, for the persistent kernel: the arrays come in as separate read-only
+// kernel arguments and every access is an aligned 32-bit load at a
+// workgroup-uniform address, so that the values can travel through scalar
+// loads into scalar registers instead of occupying vector registers for the
+// length of a row.
+// mask byte i of an array whose enclosing aligned words start at mask32 (the
+// host passes the byte pointer rounded down to 4 bytes, and the remainder)
+__device__ __forceinline__ uint32_t load_byte_uniform(const uint32_t* __restrict__ mask32, unsigned mis, int64_t i) {
+  const int64_t j = i + mis;
+  return (mask32[j >> 2] >> ((unsigned)(j & 3) * 8)) & 0xffu;
+}
+
+__device__ __forceinline__ TokenIn load_token_in_ro(const float* __restrict__ prox, const float* __restrict__ adv,
+                                                    const uint32_t* __restrict__ mask32, unsigned mask_mis,
+                                                    const float* __restrict__ bw, bool has_w, int64_t T_active,
+                                                    int64_t t) {
+  TokenIn in;
+  in.active = t < T_active;
+  const int64_t tc = in.active ? t : T_active - 1;
+  in.mask_raw = (uint8_t)load_byte_uniform(mask32, mask_mis, tc);
+  in.prox = prox[tc];
+  in.adv = adv[tc];
+  in.w = has_w ? bw[tc] : 1.f;
+  return in;
+}
+
+// raw 16-bit pattern of element i of a row of 16-bit values (row 4-byte aligned)
+__device__ __forceinline__ uint32_t load_u16_uniform(const void* __restrict__ row, int64_t i) {
+  const uint32_t w = ((const uint32_t*)row)[i >> 1];
+  return (i & 1) ? (w >> 16) : (w & 0xffffu);
+}
+
+// 1 / max(n_valid, 1) times the optional gradient scale: the factor between
+// d(surrogate)/d(logp) and d(scaled loss)/d(logp).
+__device__ __forceinline__ void load_loss_scale(const FusedTokenArgs& a, float& fn, float& gscale) {
+  int n = *a.n_valid;
+  if (n < 1) n = 1;
+  fn = (float)n;
+  gscale = a.grad_scale ? *a.grad_scale : 1.f;
+}
+
 // Returns g = d(scaled loss)/d(logp_t); writes the per-token outputs from one thread.
-__device__ __forceinline__ float fused_token_tail(const FusedTokenArgs& a, int64_t t, float lp, const RowStats& rs,
-                                                  const RowOut& ro, bool writer) {
+__device__ __forceinline__ float fused_token_tail(const FusedTokenArgs& a, int64_t t, const TokenIn& in, float fn,
+                                                  float gscale, float lp, const RowStats& rs, const RowOut& ro,
+                                                  bool writer) {
   if (writer) {
     a.logp[t] = lp;
     if (a.entropy) a.entropy[t] = ro.entropy;
     if (a.vmax) a.vmax[t] = rs.mx;
     if (a.vmin) a.vmin[t] = rs.mn;
   }
-  if (t >= a.T_active) return 0.f;
-  const bool m = a.mask_eff[t] != 0;
-  const float prox = a.prox_logp[t];
-  const float r = m ? expf(lp - prox) : 0.f;
-  const float w = a.P.has_behave_weight ? a.behave_w[t] : 1.f;
-  const Surrogate s = surrogate(r, a.adv[t], w, a.P);
+  if (!in.active) return 0.f;
+  const bool m = in.mask();
+  const float r = m ? expf(lp - in.prox) : 0.f;
+  const Surrogate s = surrogate(r, in.adv, in.w, a.P);
   if (writer) {
     a.stat_loss[t] = s.loss;
     a.ratio[t] = r;
     a.flags[t] = (uint8_t)(((s.clip && m) ? 1 : 0) | ((s.dual && m) ? 2 : 0));
   }
   if (!m) return 0.f;
-  int n = *a.n_valid;
-  if (n < 1) n = 1;
-  float g = s.dloss_dr * r / (float)n;
-  if (a.grad_scale) g *= *a.grad_scale;
-  return g;
+  return (s.dloss_dr * r / fn) * gscale;
 }
 
 template <int DT, int NT>
@@ -340,10 +398,14 @@ __global__ __launch_bounds__(NT) void k_fused_generic(const void* __restrict__ l
   const int64_t y = labels[t];
   const bool y_ok = (y >= 0) && (y < V);
   const float xy = y_ok ? Elem<DT>::load1(row, y) : 0.f;
+  TokenIn tin{0.f, 0.f, 1.f, 0, false};
+  if (a.T_active > 0) tin = load_token_in(a, t);
+  float fn, gscale;
+  load_loss_scale(a, fn, gscale);
   const RowStats rs = row_stats_generic<DT, NT>(row, V, vec_ok != 0, c, smem);
   const RowOut ro = finish_row(rs);
   const float lp = y_ok ? label_logp(xy, c, rs, ro) : __builtin_nanf("");
-  const float g = fused_token_tail(a, t, lp, rs, ro, threadIdx.x == 0);
+  const float g = fused_token_tail(a, t, tin, fn, gscale, lp, rs, ro, threadIdx.x == 0);
   if (g == 0.f) {
     row_zero_generic<DT, NT>(row, out, V, vec_ok != 0);
     return;
@@ -369,7 +431,10 @@ __global__ __launch_bounds__(NT) void k_fused_generic(const void* __restrict__ l
 // the VGPR offset instead.
 // -----------------------------------------------------------------------------
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef short s16x2_t __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
 constexpr int kBufferFlags = 0x00020000;  // raw buffer, 32-bit data format
+constexpr int kAuxStream = 2;  // cache-policy bit 'nt': data is touched once, do not keep it in the caches
 
 // Marks the packed row as modified (no instruction is emitted) so that the
 // unpacked floats of one pass are not kept alive for the next: the row stays
@@ -384,93 +449,30 @@ __device__ __forceinline__ void keep_packed(u32x4_t (&d)[NCH]) {
   }
 }
 
-template <int DT, int NCH>
-__global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ logits, int V, int64_t stride_vec,
-                                                     const int64_t* __restrict__ labels, float inv_t,
-                                                     FusedTokenArgs a, uint4* __restrict__ dlogits) {
+// Gradient of one register-resident row, chunk by chunk:
+//   out_j = -(g / T) p_j  (+ g / T at the label),  p_j = 2^(x_j c - lse2).
+// The factor g / T is folded into the exponent, 2^(x_j c - lse2 + log2|g / T|),
+// and its sign is applied in the conversion to 16 bits, so an element costs
+// one fma and one exponential.
+template <int DT, int NCH, bool G_POSITIVE>
+__device__ __forceinline__ void grad_pass(const u32x4_t (&d)[NCH], float g, float inv_t, float c, float lse2,
+                                          int64_t y, int tid, int voff, __amdgpu_buffer_rsrc_t wsrc) {
   constexpr int NT = 1024;
   constexpr int kChunkBytes = NT * 16;
-  __shared__ float smem[(NT / kWave) * 5];
-  const int64_t t = blockIdx.x;
-  const uint4* src = logits + t * stride_vec;
-  uint4* dst = dlogits + t * stride_vec;
-  const int nvec = V >> 3;
-  const int tid = threadIdx.x;
-  const float c = kLog2e * inv_t;
-  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, V * 2, kBufferFlags);
-  const __amdgpu_buffer_rsrc_t wsrc = __builtin_amdgcn_make_buffer_rsrc((void*)dst, 0, V * 2, kBufferFlags);
-  const int voff = tid * 16;
-  const bool last_ok = (NCH - 1) * NT + tid < nvec;
-
-  u32x4_t d[NCH];
-#pragma unroll
-  for (int i = 0; i < NCH; ++i) d[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, i * kChunkBytes, 0);
-  const int64_t y = labels[t];
-  const bool y_ok = (y >= 0) && (y < V);
-  const float xy = y_ok ? Elem<DT>::load1(src, y) : 0.f;
-
-  // pass 1 over registers: thread maximum / minimum
-  float mx = -FLT_MAX, mn = FLT_MAX;
-#pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    float cmx = -FLT_MAX, cmn = FLT_MAX;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const float lo = Elem<DT>::lo(d[i][q]), hi = Elem<DT>::hi(d[i][q]);
-      cmx = fmaxf(cmx, fmaxf(lo, hi));
-      cmn = fminf(cmn, fminf(lo, hi));
-    }
-    if (i == NCH - 1 && !last_ok) { cmx = -FLT_MAX; cmn = FLT_MAX; }
-    mx = fmaxf(mx, cmx);
-    mn = fminf(mn, cmn);
-  }
-  keep_packed(d);
-  // one maximum per wave keeps the second pass free of rescaling
-  ThreadStats ts;
-  ts.k = fmaxf(wave_max(mx) * c, kNegBig);
-  ts.mx = mx; ts.mn = mn;
-  float s = 0.f, u = 0.f;
-#pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    float cs = 0.f, cu = 0.f;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const float lo = Elem<DT>::lo(d[i][q]), hi = Elem<DT>::hi(d[i][q]);
-      const float t0 = fmaf(lo, c, -ts.k), t1 = fmaf(hi, c, -ts.k);
-      const float e0 = fast_exp2(t0), e1 = fast_exp2(t1);
-      cs += e0 + e1;
-      cu = fmaf(t0, e0, cu);
-      cu = fmaf(t1, e1, cu);
-    }
-    if (i == NCH - 1 && !last_ok) { cs = 0.f; cu = 0.f; }
-    s += cs;
-    u += cu;
-  }
-  ts.s = s; ts.u = u;
-  keep_packed(d);
-  const RowStats rs = block_stats<NT / kWave>(ts, smem);
-  const RowOut ro = finish_row(rs);
-  const float lp = y_ok ? label_logp(xy, c, rs, ro) : __builtin_nanf("");
-  const float g = fused_token_tail(a, t, lp, rs, ro, tid == 0);
-
-  if (g == 0.f) {
-    const u32x4_t z = {0u, 0u, 0u, 0u};
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, voff + i * kChunkBytes, 0, 0);
-    return;
-  }
-  const float A = -g * inv_t;
   const float lab_add = g * inv_t;
-  const int yv = y_ok ? (int)(y >> 3) : -1;
+  const float kk = fast_log2(fabsf(lab_add)) - lse2;
+  const int yv = y >= 0 ? (int)(y >> 3) : -1;
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     float o[8];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      o[2 * q] = A * fast_exp2(fmaf(Elem<DT>::lo(d[i][q]), c, -ro.lse2));
-      o[2 * q + 1] = A * fast_exp2(fmaf(Elem<DT>::hi(d[i][q]), c, -ro.lse2));
+      const float e0 = fast_exp2(fmaf(Elem<DT>::lo(d[i][q]), c, kk));
+      const float e1 = fast_exp2(fmaf(Elem<DT>::hi(d[i][q]), c, kk));
+      o[2 * q] = G_POSITIVE ? -e0 : e0;
+      o[2 * q + 1] = G_POSITIVE ? -e1 : e1;
     }
-    if (i * NT + tid == yv) {
+    if (yv - i * NT == tid) {  // uniform left side: no per-chunk index registers
       const int e = (int)(y & 7);
 #pragma unroll
       for (int q = 0; q < 8; ++q)
@@ -481,7 +483,152 @@ __global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ l
     r[1] = Elem<DT>::pack(o[2], o[3]);
     r[2] = Elem<DT>::pack(o[4], o[5]);
     r[3] = Elem<DT>::pack(o[6], o[7]);
-    __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + i * kChunkBytes, 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + i * kChunkBytes, 0, kAuxStream);
+  }
+}
+
+// Rows are handed out through a device counter (work[0]) so that compute
+// units that get through their rows faster take more of them; work[1] counts
+// finished workgroups, and the last one puts both words back to zero, which is
+// the state the next launch expects.  With work == nullptr the rows are dealt
+// round-robin (t, t + gridDim.x, ...).
+template <int DT, int NCH>
+__global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ logits, int V, int64_t stride_vec,
+                                                     const int64_t* __restrict__ labels, float inv_t,
+                                                     const float* __restrict__ in_prox,
+                                                     const float* __restrict__ in_adv,
+                                                     const uint32_t* __restrict__ in_mask32, unsigned mask_mis,
+                                                     const float* __restrict__ in_bw, FusedTokenArgs a,
+                                                     uint4* __restrict__ dlogits, int64_t T, int32_t* work) {
+  constexpr int NT = 1024;
+  constexpr int kChunkBytes = NT * 16;
+  const bool has_w = a.P.has_behave_weight != 0;
+  __shared__ float smem[(NT / kWave) * 5];
+  __shared__ int64_t next_row[2];  // written at the top of a row, read behind its barriers: two slots, no reuse race
+  int slot = 0;
+  const int nvec = V >> 3;
+  const int tid = threadIdx.x;
+  const float c = kLog2e * inv_t;
+  const int voff = tid * 16;
+  const bool last_ok = (NCH - 1) * NT + tid < nvec;
+  float fn, gscale;
+  load_loss_scale(a, fn, gscale);
+
+  int64_t t = blockIdx.x;  // the host launches at most T workgroups
+  const uint4* src = logits + t * stride_vec;
+  u32x4_t d[NCH];
+  {
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, V * 2, kBufferFlags);
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) d[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, i * kChunkBytes, kAuxStream);
+  }
+  int64_t y = labels[t];
+  bool y_ok = (y >= 0) && (y < V);
+  uint32_t xy_raw = load_u16_uniform(src, y_ok ? y : 0);
+  TokenIn tin = load_token_in_ro(in_prox, in_adv, in_mask32, mask_mis, in_bw, has_w, a.T_active, t);
+
+  for (;;) {
+    // claim the row after this one; the answer is picked up behind the barriers of block_stats
+    if (tid == 0) next_row[slot] = work ? (int64_t)atomicAdd(&work[0], 1) + gridDim.x : t + gridDim.x;
+
+    // pass 1 over registers: thread maximum / minimum, taken on the raw 16-bit
+    // patterns with packed integer min/max (two elements per instruction, no
+    // unpacking).  For sign-magnitude floats: if any value is non-negative the
+    // largest signed pattern is the maximum, otherwise the smallest signed
+    // pattern is; if any value is negative the largest unsigned pattern is the
+    // minimum, otherwise the smallest unsigned pattern is.
+    s16x2_t smax = {-32768, -32768}, smin = {32767, 32767};
+    u16x2_t umax = {0, 0}, umin = {65535, 65535};
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      if (i < NCH - 1 || last_ok) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const uint32_t w = d[i][q];  // a scalar copy: bit_cast of a vector element expression reads element 0
+          const s16x2_t ws = __builtin_bit_cast(s16x2_t, w);
+          const u16x2_t wu = __builtin_bit_cast(u16x2_t, w);
+          smax = __builtin_elementwise_max(smax, ws);
+          smin = __builtin_elementwise_min(smin, ws);
+          umax = __builtin_elementwise_max(umax, wu);
+          umin = __builtin_elementwise_min(umin, wu);
+        }
+      }
+    }
+    const int hi_s = smax[0] > smax[1] ? smax[0] : smax[1];
+    const int lo_s = smin[0] < smin[1] ? smin[0] : smin[1];
+    const unsigned hi_u = umax[0] > umax[1] ? umax[0] : umax[1];
+    const unsigned lo_u = umin[0] < umin[1] ? umin[0] : umin[1];
+    const float mx = Elem<DT>::lo((uint32_t)((hi_s >= 0 ? hi_s : lo_s) & 0xffff));
+    const float mn = Elem<DT>::lo(lo_s < 0 ? hi_u : lo_u);
+    keep_packed(d);
+    // one maximum per wave keeps the second pass free of rescaling
+    ThreadStats ts;
+    ts.k = fmaxf(wave_max(mx) * c, kNegBig);
+    ts.mx = mx; ts.mn = mn;
+    float s = 0.f, u = 0.f;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      float cs = 0.f, cu = 0.f;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float lo = Elem<DT>::lo(d[i][q]), hi = Elem<DT>::hi(d[i][q]);
+        const float t0 = fmaf(lo, c, -ts.k), t1 = fmaf(hi, c, -ts.k);
+        const float e0 = fast_exp2(t0), e1 = fast_exp2(t1);
+        cs += e0 + e1;
+        cu = fmaf(t0, e0, cu);
+        cu = fmaf(t1, e1, cu);
+      }
+      if (i == NCH - 1 && !last_ok) { cs = 0.f; cu = 0.f; }
+      s += cs;
+      u += cu;
+    }
+    ts.s = s; ts.u = u;
+    keep_packed(d);
+    const RowStats rs = block_stats<NT / kWave>(ts, smem);
+    const int64_t tn = next_row[slot];
+    slot ^= 1;
+    const RowOut ro = finish_row(rs);
+    const float xy = Elem<DT>::lo(xy_raw);
+    const float lp = y_ok ? label_logp(xy, c, rs, ro) : __builtin_nanf("");
+    const float g = fused_token_tail(a, t, tin, fn, gscale, lp, rs, ro, tid == 0);
+
+    // scalars of the next row, fetched ahead of the gradient pass
+    const bool more = tn < T;
+    const uint4* src_n = logits + (more ? tn : t) * stride_vec;
+    const int64_t y_n = more ? labels[tn] : -1;
+    const bool y_ok_n = (y_n >= 0) && (y_n < V);
+    const uint32_t xy_raw_n = load_u16_uniform(src_n, y_ok_n ? y_n : 0);
+    const TokenIn tin_n = load_token_in_ro(in_prox, in_adv, in_mask32, mask_mis, in_bw, has_w, a.T_active, more ? tn : t);
+
+    const __amdgpu_buffer_rsrc_t wsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void*)(dlogits + t * stride_vec), 0, V * 2, kBufferFlags);
+    if (g == 0.f) {
+      const u32x4_t z = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, voff + i * kChunkBytes, 0, kAuxStream);
+    } else if (g > 0.f) {
+      grad_pass<DT, NCH, true>(d, g, inv_t, c, ro.lse2, y_ok ? y : -1, tid, voff, wsrc);
+    } else {
+      grad_pass<DT, NCH, false>(d, g, inv_t, c, ro.lse2, y_ok ? y : -1, tid, voff, wsrc);
+    }
+    if (!more) break;
+    // All stores of this row are issued before the loads of the next one:
+    // alternating them chunk by chunk costs bandwidth on this memory system.
+    {
+      const __amdgpu_buffer_rsrc_t rsrc_n = __builtin_amdgcn_make_buffer_rsrc((void*)src_n, 0, V * 2, kBufferFlags);
+#pragma unroll
+      for (int i = 0; i < NCH; ++i)
+        d[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_n, voff, i * kChunkBytes, kAuxStream);
+    }
+    t = tn; y = y_n; y_ok = y_ok_n; xy_raw = xy_raw_n; tin = tin_n;
+  }
+  if (work && tid == 0) {
+    __threadfence();
+    if (atomicAdd(&work[1], 1) == (int)gridDim.x - 1) {
+      work[0] = 0;
+      work[1] = 0;
+      __threadfence();
+    }
   }
 }
 
@@ -523,22 +670,41 @@ static bool rows_vec_ok(const void* a, const void* b, int dtype) {
   return true;
 }
 
+// Largest row (in 16 KiB chunks) that still fits the register file without spills.
+constexpr int kMaxRegChunks = 21;
+
+// One 1024-thread workgroup per compute unit (its row fills the register file).
+static int persistent_workgroups() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    n = cus;
+  }
+  return n;
+}
+
 template <int DT, int NCH>
 static void launch_regs(const void* logits, int64_t T, int V, int64_t stride, const int64_t* labels, float inv_t,
-                        const FusedTokenArgs& a, void* dlogits, hipStream_t st) {
-  hipLaunchKernelGGL((k_fused_regs<DT, NCH>), dim3((unsigned)T), dim3(1024), 0, st, (const uint4*)logits, V,
-                     stride >> 3, labels, inv_t, a, (uint4*)dlogits);
+                        const FusedTokenArgs& a, void* dlogits, int32_t* work, hipStream_t st) {
+  const int64_t wgs = T < persistent_workgroups() ? T : persistent_workgroups();
+  const uintptr_t mask_addr = (uintptr_t)a.mask_eff;
+  hipLaunchKernelGGL((k_fused_regs<DT, NCH>), dim3((unsigned)wgs), dim3(1024), 0, st, (const uint4*)logits, V,
+                     stride >> 3, labels, inv_t, a.prox_logp, a.adv, (const uint32_t*)(mask_addr & ~(uintptr_t)3),
+                     (unsigned)(mask_addr & 3), a.behave_w, a, (uint4*)dlogits, T, work);
 }
 
 template <int DT>
 static bool dispatch_regs(int nch, const void* logits, int64_t T, int V, int64_t stride, const int64_t* labels,
-                          float inv_t, const FusedTokenArgs& a, void* dlogits, hipStream_t st) {
+                          float inv_t, const FusedTokenArgs& a, void* dlogits, int32_t* work, hipStream_t st) {
   switch (nch) {
 #define AA_CASE(N) \
-  case N: launch_regs<DT, N>(logits, T, V, stride, labels, inv_t, a, dlogits, st); return true;
+  case N: launch_regs<DT, N>(logits, T, V, stride, labels, inv_t, a, dlogits, work, st); return true;
     AA_CASE(1) AA_CASE(2) AA_CASE(3) AA_CASE(4) AA_CASE(5) AA_CASE(6) AA_CASE(7) AA_CASE(8)
     AA_CASE(9) AA_CASE(10) AA_CASE(11) AA_CASE(12) AA_CASE(13) AA_CASE(14) AA_CASE(15) AA_CASE(16)
-    AA_CASE(17) AA_CASE(18) AA_CASE(19) AA_CASE(20) AA_CASE(21) AA_CASE(22) AA_CASE(23) AA_CASE(24)
+    AA_CASE(17) AA_CASE(18) AA_CASE(19) AA_CASE(20) AA_CASE(21)
 #undef AA_CASE
     default: return false;
   }
@@ -591,7 +757,8 @@ extern "C" int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int
                                    const float* prox_logp, const float* adv, const uint8_t* mask_eff,
                                    const float* behave_w, const aa_ppo_params* params, const int32_t* n_valid,
                                    const float* grad_scale, float* logp, float* entropy, float* vmax, float* vmin,
-                                   float* stat_loss, float* ratio, uint8_t* flags, void* dlogits, void* stream) {
+                                   float* stat_loss, float* ratio, uint8_t* flags, void* dlogits, int32_t* work,
+                                   void* stream) {
   if (!common_args_ok(logits, dtype, T, V, row_stride, labels)) return AA_ERR_INVALID_ARGUMENT;
   if (!params || !prox_logp || !adv || !mask_eff || !n_valid || !logp || !stat_loss || !ratio || !flags || !dlogits)
     return AA_ERR_INVALID_ARGUMENT;
@@ -606,12 +773,12 @@ extern "C" int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int
   a.P = *params; a.T_active = T_active;
 
   const bool fast = (dtype != AA_F32) && (V % 8 == 0) && (row_stride % 8 == 0) && (((uintptr_t)logits & 15) == 0) &&
-                    (((uintptr_t)dlogits & 15) == 0) && (V >= 8 * 1024) && (V <= 24 * 8192);
+                    (((uintptr_t)dlogits & 15) == 0) && (V >= 8 * 1024) && (V <= kMaxRegChunks * 8192) && (T_active > 0);
   if (fast) {
     const int nch = (int)((V / 8 + 1023) / 1024);
     bool ok = (dtype == AA_BF16)
-                  ? dispatch_regs<AA_BF16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, st)
-                  : dispatch_regs<AA_F16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, st);
+                  ? dispatch_regs<AA_BF16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st)
+                  : dispatch_regs<AA_F16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st);
     if (ok) return launch_status();
   }
   const int vec_ok = rows_vec_ok(logits, dlogits, dtype) ? 1 : 0;

@@ -83,6 +83,19 @@ def _check_tp(tp_group: Any) -> None:
             )
 
 
+_WORK: dict = {}
+
+
+def _work_words(dev: torch.device) -> torch.Tensor:
+    """Two zeroed int32 words per (device, stream) for the row hand-out of the fused kernel, which returns
+    them to zero at the end of every launch."""
+    key = (dev.index, torch.cuda.current_stream(dev).cuda_stream)
+    buf = _WORK.get(key)
+    if buf is None:
+        buf = _WORK[key] = torch.zeros(2, dtype=torch.int32, device=dev)
+    return buf
+
+
 def _ppo_params(eps_clip, eps_clip_higher, c_clip, has_w) -> N.PpoParams:
     if c_clip is not None:
         assert c_clip > 1.0, c_clip
@@ -475,7 +488,7 @@ class _FusedLogitsPpo(torch.autograd.Function):
                     _ptr(logits2d), _DTYPES[logits2d.dtype], T, V, stride, _ptr(labels1d), 1.0 / float(temperature),
                     T_active, _ptr(prox), _ptr(adv), _ptr(mask_eff), _ptr(behave_w), C.byref(params),
                     _ptr(n_valid), _ptr(grad_scale), _ptr(logp), _ptr(entropy), _ptr(vmax), _ptr(vmin),
-                    _ptr(stat_loss), _ptr(ratio), _ptr(flags), _ptr(dlogits), st,
+                    _ptr(stat_loss), _ptr(ratio), _ptr(flags), _ptr(dlogits), _ptr(_work_words(dev)), st,
                 ),
                 "aa_logits_ppo_fused",
             )

@@ -117,7 +117,7 @@ def time_dominant_kernel(case, kw, cfg, iters: int):
                 F._ptr(case.logits), N.AA_BF16, T, V, V, F._ptr(case.labels), 1.0 / case.temperature, T,
                 F._ptr(prox), F._ptr(adv), F._ptr(mask_eff), F._ptr(w), C.byref(params), F._ptr(counts), None,
                 F._ptr(logp), F._ptr(ent), None, None, F._ptr(sl), F._ptr(ratio), F._ptr(flags), F._ptr(dlogits),
-                C.c_void_p(stream.cuda_stream),
+                F._ptr(F._work_words(dev)), C.c_void_p(stream.cuda_stream),
             ),
             "aa_logits_ppo_fused",
         )

@@ -115,6 +115,11 @@ int aa_logits_bwd(const void* logits, int dtype, int64_t T, int64_t V,
  *   masking), ratio, flags (bit0 = clip_mask & mask_eff, bit1 =
  *   dual_clip_mask & mask_eff); dlogits [T, V] in the dtype of logits (rows
  *   >= T_active are zeros).  The scalar loss is finished by aa_masked_sum.
+ * work: NULL, or two int32 words of device memory that are zero on entry; the
+ *   kernel hands rows to compute units through them (faster than a fixed
+ *   assignment) and leaves them zero on exit, so one zeroed buffer serves
+ *   every launch on a stream.  Launches that may run concurrently need
+ *   separate buffers.
  */
 int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int64_t V,
                         int64_t row_stride, const int64_t* labels,
@@ -125,7 +130,7 @@ int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int64_t V,
                         const float* grad_scale, float* logp, float* entropy,
                         float* vmax, float* vmin, float* stat_loss,
                         float* ratio, uint8_t* flags, void* dlogits,
-                        void* stream);
+                        int32_t* work, void* stream);
 
 /* ------------------------------------------------------------------ */
 /* Per-token PPO pieces                                                */
