@@ -40,6 +40,9 @@ def parse_args():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--cpu-tokens", type=int, default=1024, help="token sample of the CPU baseline (0 = skip)")
     ap.add_argument("--cpu-iters", type=int, default=3)
+    ap.add_argument("--copy-launches", type=int, default=0,
+                    help="also launch the plain copy kernel this many times over the logits buffer "
+                         "(the calibration point for FETCH_SIZE / WRITE_SIZE counters)")
     return ap.parse_args()
 
 
@@ -212,7 +215,10 @@ def main():
     achieved = alg_bytes / (k_ms * 1e-3) / 1e9
     roofline = dict(
         bound="hbm", kernel="k_fused_regs (aa_logits_ppo_fused)", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s",
-        frac=achieved / HBM_PEAK_GBS, traffic=None, avg_kernel_ms=k_ms, min_kernel_ms=k_min_ms,
+        frac=achieved / HBM_PEAK_GBS,
+        # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters read
+        # for the plain copy kernel: 1.001 x the algorithmic bytes (profiles/k_fused_regs_cfg1-32k_hbm_traffic.md)
+        traffic=alg_bytes * 1.001, avg_kernel_ms=k_ms, min_kernel_ms=k_min_ms,
         algorithmic_bytes_per_launch=alg_bytes,
     )
     out = dict(
@@ -223,6 +229,17 @@ def main():
                     accumulate="f32", path="logits (fused fwd + PPO loss + bwd, one launch)"),
         roofline=roofline,
     )
+    if args.copy_launches > 0:
+        from areal_amd import _native as N
+        from areal_amd import functional as F
+
+        dst = torch.empty_like(case.logits)
+        nbytes = case.logits.numel() * case.logits.element_size()
+        for _ in range(args.copy_launches):
+            N.check(N.load().aa_copy_bytes(F._ptr(case.logits), F._ptr(dst), nbytes, F._stream(dev)), "aa_copy_bytes")
+        torch.cuda.synchronize()
+        out["copy_calibration"] = dict(kernel="k_copy16 (aa_copy_bytes)", bytes_read=nbytes, bytes_written=nbytes,
+                                       launches=args.copy_launches)
     if args.cpu_tokens > 0:
         baseline, parity = cpu_baseline_and_parity(case, kw, cfg, args.cpu_tokens, args.cpu_iters)
         out["cpu_baseline"] = baseline
