@@ -11,6 +11,7 @@ from .functional import (
     gather_logprobs,
     gather_logprobs_entropy,
     gather_logprobs_entropy_stats,
+    lm_head_logprobs_entropy,
     ppo_actor_loss_fn,
 )
 from ._native import NativeLibraryError
@@ -26,5 +27,6 @@ __all__ = [
     "gather_logprobs",
     "gather_logprobs_entropy",
     "gather_logprobs_entropy_stats",
+    "lm_head_logprobs_entropy",
     "ppo_actor_loss_fn",
 ]

@@ -1,17 +1,418 @@
-// Fused lm_head path (placeholder entry points until the MFMA kernels land).
-#include "device_utils.h"
+// Fused lm_head path for gfx950: log-prob / entropy of softmax(hidden @ weight.T / T) and its backward without ever
+// holding the [T, V] logits in memory.  The reference has no such path: its equivalent is the lm_head matmul
+// followed by gather_logprobs_entropy (areal/utils/functional/vocab_parallel.py:23-29) and autograd.
+//
+// Forward: a bf16 MFMA tile GEMM (gemm_tn.h) forms 256 (vocabulary) x 256 (tokens) tiles of the logits in
+// accumulator registers; its epilogue reduces each tile to the softmax partials (k, s, u) per token and captures
+// the label logit; a second small kernel merges the partials of all vocabulary tiles.
+//
+// Backward: the logits tile is formed again, turned into d(logits) in registers (bf16), and written to a reusable
+// panel of one token chunk in both orientations; two more tile GEMMs contract the panel with the weights
+// (d_hidden) and with the hidden states (d_weight, fp32).
+#include "gemm_tn.h"
+
+namespace aa {
+namespace lmhead {
+
+using namespace gemm;
+
+constexpr int kChunkTokens = 16384;  // token chunk of the backward panel
+
+__device__ __forceinline__ int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+
+// ---- forward epilogue: softmax partials of a tile --------------------------------------------------------------
+// part[(tile_v * T + token)] = (k, s, u, 0);   xy[token] = raw label logit (written by the one tile that holds it)
+__global__ __launch_bounds__(kThreads) void k_lmhead_stats(Operand W, Operand Hd, int K, int tiles_m, int tiles_n,
+                                                           float c, const int64_t* __restrict__ labels,
+                                                           float4* __restrict__ part, float* __restrict__ xy) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  int tm, tn;
+  tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  Acc acc;
+  mainloop(W, Hd, K, m0, n0, acc, lds);
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int V = W.rows, T = Hd.rows;
+  const int mbase = m0 + wm * 128;
+  const bool ragged = m0 + BM > V;
+  float* red = (float*)lds;  // [2 (wm)][256 tokens][3]
+
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) {
+    const int token = n0 + wn * 128 + acc_col(nt, lane);
+    float mx = -FLT_MAX;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const bool in = !ragged || (mbase + acc_row(mt, i, lane) < V);  // rows past the vocabulary: last tile only
+        mx = in ? fmaxf(mx, acc.v[mt][nt][i]) : mx;
+      }
+    // both halves of the wave (lane, lane ^ 32) hold the same token: agree on the maximum first
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    const float k = fmaxf(mx * c, kNegBig);  // kNegBig: no valid row in this wave's block
+    float s = 0.f, u = 0.f;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const bool in = !ragged || (mbase + acc_row(mt, i, lane) < V);
+        const float t = in ? fmaf(acc.v[mt][nt][i], c, -k) : 0.f;
+        const float e = in ? fast_exp2(t) : 0.f;
+        s += e;
+        u = fmaf(t, e, u);
+      }
+    s += __shfl_xor(s, 32, kWave);
+    u += __shfl_xor(u, 32, kWave);
+    if (lane < 32) {
+      float* r = red + (wm * 256 + wn * 128 + nt * 32 + lane) * 3;
+      r[0] = k; r[1] = s; r[2] = u;
+    }
+    // label logit, if the label falls into this wave's 128 vocabulary rows
+    if (token < T) {
+      const int64_t y = labels[token];
+      const int64_t rel = y - mbase;
+      if (rel >= 0 && rel < 128 && y < V && (int)((rel >> 2) & 1) == (lane >> 5)) {
+        const int mt_y = (int)(rel >> 5), r5 = (int)(rel & 31);
+        const int i_y = ((r5 >> 3) << 2) | (r5 & 3);
+        float val = 0.f;
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i)
+            if (mt == mt_y && i == i_y) val = acc.v[mt][nt][i];
+        xy[token] = val;
+      }
+    }
+  }
+  __syncthreads();
+  {  // merge the two vocabulary halves of the tile; thread = token
+    const int token = n0 + tid;
+    const float* a = red + tid * 3;
+    const float* b = red + (256 + tid) * 3;
+    const float k = fmaxf(a[0], b[0]);
+    const float da = a[0] - k, db = b[0] - k;
+    const float fa = fast_exp2(da), fb = fast_exp2(db);
+    const float s = a[1] * fa + b[1] * fb;
+    const float u = fa * fmaf(da, a[1], a[2]) + fb * fmaf(db, b[1], b[2]);
+    if (token < T) part[(int64_t)tm * T + token] = make_float4(k, s, u, 0.f);
+  }
+}
+
+__global__ __launch_bounds__(256) void k_fill_f32(float* p, int64_t n, float v) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+// merge the partials of all vocabulary tiles, one thread per token (fixed order: deterministic)
+__global__ __launch_bounds__(256) void k_lmhead_combine(const float4* __restrict__ part, const float* __restrict__ xy,
+                                                        int tiles_m, int T, float c, float* __restrict__ logp,
+                                                        float* __restrict__ entropy, float* __restrict__ row_lse,
+                                                        float* __restrict__ row_ez) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= T) return;
+  float k = kNegBig, s = 0.f, u = 0.f;
+  for (int vt = 0; vt < tiles_m; ++vt) {
+    const float4 p = part[(int64_t)vt * T + t];
+    const float nk = fmaxf(k, p.x);
+    const float da = k - nk, db = p.x - nk;
+    const float fa = fast_exp2(da), fb = fast_exp2(db);
+    u = fa * fmaf(da, s, u) + fb * fmaf(db, p.y, p.z);
+    s = s * fa + p.y * fb;
+    k = nk;
+  }
+  const float log2s = fast_log2(s);
+  const float mean_t = u / s;
+  logp[t] = (fmaf(xy[t], c, -k) - log2s) * kLn2;  // xy stays NaN for a label outside [0, V)
+  if (entropy) entropy[t] = (log2s - mean_t) * kLn2;
+  if (row_lse) row_lse[t] = (k + log2s) * kLn2;
+  if (row_ez) row_ez[t] = (k + mean_t) * kLn2;
+}
+
+// ---- backward epilogue: d(logits) of a tile, written as panel [tokens, V] and [V, tokens] -----------------------
+struct DsArgs {
+  const float* row_lse;   // [T] natural log
+  const float* row_ez;    // [T] (nullable when g_entropy is null)
+  const float* g_logp;    // [T]
+  const float* g_entropy; // [T] nullable
+  const int64_t* labels;  // [T]
+  uint16_t* ds;           // [chunk tokens, V] bf16, ld = V
+  uint16_t* dst;          // [V, ld_t] bf16
+  int64_t ld_t;
+  int64_t t0;             // first token of the chunk (hidden operand is already offset)
+  float inv_t;
+};
+
+__global__ __launch_bounds__(kThreads) void k_lmhead_ds(Operand W, Operand Hd, int K, int tiles_m, int tiles_n,
+                                                        DsArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  int tm, tn;
+  tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  Acc acc;
+  mainloop(W, Hd, K, m0, n0, acc, lds);
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int V = W.rows, N = Hd.rows;
+  const int mbase = m0 + wm * 128;
+  const float c = kLog2e * a.inv_t;
+  constexpr int PZ = BM + 8;  // pitch of the staged tile Z[token][vocab] in elements
+  uint16_t* Z = lds;          // 256 x 264 bf16 = 135168 B
+
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) {
+    const int nloc = wn * 128 + acc_col(nt, lane);
+    const int n = n0 + nloc;
+    float A = 0.f, B = 0.f, lab_add = 0.f, lse2 = 0.f;
+    int64_t y = -1;
+    const bool live = n < N;
+    if (live) {
+      const int64_t t = a.t0 + n;
+      const float gl = a.g_logp[t];
+      const float gh = a.g_entropy ? a.g_entropy[t] : 0.f;
+      const float ez = a.g_entropy ? a.row_ez[t] : 0.f;
+      lse2 = a.row_lse[t] * kLog2e;
+      A = a.inv_t * (gh * ez - gl);
+      B = -gh * a.inv_t * a.inv_t;
+      lab_add = gl * a.inv_t;
+      y = a.labels[t];
+    }
+    const int64_t rel = y - mbase;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        float o[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float x = acc.v[mt][nt][g4 * 4 + q];
+          o[q] = live ? fast_exp2(fmaf(x, c, -lse2)) * fmaf(B, x, A) : 0.f;
+        }
+        const int r0 = mt * 32 + 8 * g4 + 4 * (lane >> 5);  // row of o[0] inside the wave block
+        if (rel >= r0 && rel < r0 + 4) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            if (rel - r0 == q) o[q] += lab_add;
+        }
+        if (mbase + r0 + 3 >= V) {  // rows outside the vocabulary (last tile only)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            if (mbase + r0 + q >= V) o[q] = 0.f;
+        }
+        uint2 pk;
+        pk.x = Elem<AA_BF16>::pack(o[0], o[1]);
+        pk.y = Elem<AA_BF16>::pack(o[2], o[3]);
+        *(uint2*)(Z + nloc * PZ + wm * 128 + r0) = pk;
+      }
+    }
+  }
+  __syncthreads();
+  // panel [token][vocab]: 16-byte pieces along the vocabulary
+  for (int p = tid; p < 256 * 32; p += kThreads) {
+    const int nloc = p >> 5, mc = (p & 31) * 8;
+    const int n = n0 + nloc, m = m0 + mc;
+    if (n < N && m < V) {
+      const u32x4_t v = *(const u32x4_t*)(Z + nloc * PZ + mc);
+      *(u32x4_t*)(a.ds + (int64_t)n * V + m) = v;  // V % 8 == 0: a piece never straddles the end
+    }
+  }
+  // panel [vocab][token]: gather 8 tokens of one vocabulary row
+  for (int p = tid; p < 256 * 32; p += kThreads) {
+    const int mloc = p >> 5, nc = (p & 31) * 8;
+    const int m = m0 + mloc;
+    if (m < V) {
+      uint32_t w[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const uint32_t lo = Z[(nc + 2 * q) * PZ + mloc], hi = Z[(nc + 2 * q + 1) * PZ + mloc];
+        w[q] = lo | (hi << 16);
+      }
+      u32x4_t v = {w[0], w[1], w[2], w[3]};
+      *(u32x4_t*)(a.dst + (int64_t)m * a.ld_t + n0 + nc) = v;  // columns >= N hold zeros (live == false)
+    }
+  }
+}
+
+// ---- plain tile GEMM with a store epilogue: C[m][n] (row-major, ldc) = or += A B^T ---------------------------------
+template <bool OUT_F32, bool ACCUM>
+__global__ __launch_bounds__(kThreads) void k_gemm_store(Operand A, Operand B, int K, int tiles_m, int tiles_n,
+                                                         void* __restrict__ C, int64_t ldc) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  int tm, tn;
+  tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  Acc acc;
+  mainloop(A, B, K, m0, n0, acc, lds);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      const int n = n0 + wn * 128 + acc_col(nt, lane);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int m = m0 + wm * 128 + acc_row(mt, i, lane);
+        if (m < A.rows && n < B.rows) {
+          const int64_t off = (int64_t)m * ldc + n;
+          if (OUT_F32) {
+            float* p = (float*)C + off;
+            *p = ACCUM ? (*p + acc.v[mt][nt][i]) : acc.v[mt][nt][i];
+          } else {
+            ((uint16_t*)C)[off] = (uint16_t)(Elem<AA_BF16>::pack(acc.v[mt][nt][i], 0.f) & 0xffffu);
+          }
+        }
+      }
+    }
+}
+
+// ---- bf16 transpose with zero padding: dst[c][r] = src[r][c], dst is [C, ld_dst], columns >= R are zeroed --------
+__global__ __launch_bounds__(256) void k_transpose_bf16(const uint16_t* __restrict__ src, int64_t R, int64_t Cc,
+                                                        int64_t ld_src, uint16_t* __restrict__ dst, int64_t ld_dst) {
+  __shared__ uint16_t tile[64][66];
+  const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+  for (int p = threadIdx.x; p < 64 * 64; p += 256) {
+    const int r = p >> 6, cc = p & 63;
+    const int64_t rr = r0 + r, ccg = c0 + cc;
+    tile[r][cc] = (rr < R && ccg < Cc) ? src[rr * ld_src + ccg] : (uint16_t)0;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < 64 * 64; p += 256) {
+    const int cc = p >> 6, r = p & 63;
+    const int64_t rr = r0 + r, ccg = c0 + cc;
+    if (ccg < Cc && rr < ld_dst) dst[ccg * ld_dst + rr] = tile[r][cc];
+  }
+}
+
+struct Workspace {
+  // forward
+  int64_t off_part, off_xy;
+  // backward
+  int64_t off_wt, off_ht, off_ds, off_dst;
+  int64_t ld_ht, ld_dst, chunk;
+  int64_t bytes;
+};
+
+static Workspace plan(int64_t T, int64_t H, int64_t V) {
+  Workspace w{};
+  auto up = [](int64_t x) { return (x + 255) / 256 * 256; };
+  const int64_t tiles_v = (V + BM - 1) / BM;
+  int64_t off = 0;
+  w.off_part = off; off += up(tiles_v * T * (int64_t)sizeof(float4));
+  w.off_xy = off;   off += up(T * (int64_t)sizeof(float));
+  const int64_t fwd_bytes = off;
+  off = 0;
+  w.chunk = T < kChunkTokens ? (T + 255) / 256 * 256 : kChunkTokens;
+  w.ld_ht = (T + 255) / 256 * 256;
+  w.ld_dst = w.chunk;
+  w.off_wt = off;  off += up(H * V * 2);
+  w.off_ht = off;  off += up(H * w.ld_ht * 2);
+  w.off_ds = off;  off += up(w.chunk * V * 2);
+  w.off_dst = off; off += up(V * w.ld_dst * 2);
+  w.bytes = off > fwd_bytes ? off : fwd_bytes;
+  return w;
+}
+
+static bool shapes_ok(int64_t T, int64_t H, int64_t V) {
+  return T > 0 && H > 0 && V > 0 && (H % BK) == 0 && (V % BK) == 0 && T < (1 << 30) && V < (1 << 30) && H < (1 << 30);
+}
+
+template <typename Kern>
+static bool allow_big_lds(Kern k) {
+  return hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) == hipSuccess;
+}
+
+}  // namespace lmhead
+}  // namespace aa
+
+using namespace aa;
+using namespace aa::lmhead;
 
 extern "C" int64_t aa_lmhead_workspace_bytes(int64_t T, int64_t H, int64_t V) {
-  (void)T; (void)H; (void)V;
-  return 0;
+  if (!shapes_ok(T, H, V)) return -1;
+  return plan(T, H, V).bytes;
 }
 
-extern "C" int aa_lmhead_fwd(const void*, const void*, int64_t, int64_t, int64_t, const int64_t*, float, float*,
-                             float*, float*, float*, void*, int64_t, void*) {
-  return AA_ERR_UNSUPPORTED;
+extern "C" int aa_lmhead_fwd(const void* hidden, const void* weight, int64_t T, int64_t H, int64_t V,
+                             const int64_t* labels, float inv_temperature, float* logp, float* entropy,
+                             float* row_lse, float* row_ez, void* workspace, int64_t workspace_bytes, void* stream) {
+  if (!hidden || !weight || !labels || !logp || !workspace || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
+  if (!shapes_ok(T, H, V)) return AA_ERR_UNSUPPORTED;
+  if ((((uintptr_t)hidden | (uintptr_t)weight | (uintptr_t)workspace) & 15) != 0) return AA_ERR_INVALID_ARGUMENT;
+  const Workspace w = plan(T, H, V);
+  if (workspace_bytes < w.bytes) return AA_ERR_INVALID_ARGUMENT;
+  static const bool ok = allow_big_lds(k_lmhead_stats);
+  if (!ok) return AA_ERR_LAUNCH;
+  hipStream_t st = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+  float4* part = (float4*)(ws + w.off_part);
+  float* xy = (float*)(ws + w.off_xy);
+  const int tiles_m = (int)((V + BM - 1) / BM), tiles_n = (int)((T + BN - 1) / BN);
+  hipLaunchKernelGGL(k_fill_f32, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st, xy, T, __builtin_nanf(""));
+  Operand W{(const uint16_t*)weight, H, (int)V};
+  Operand Hd{(const uint16_t*)hidden, H, (int)T};
+  const float c = kLog2e * inv_temperature;
+  hipLaunchKernelGGL(k_lmhead_stats, dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads), kLdsBytes, st, W, Hd, (int)H,
+                     tiles_m, tiles_n, c, labels, part, xy);
+  hipLaunchKernelGGL(k_lmhead_combine, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st, part, xy, tiles_m, (int)T,
+                     c, logp, entropy, row_lse, row_ez);
+  return launch_status();
 }
 
-extern "C" int aa_lmhead_bwd(const void*, const void*, int64_t, int64_t, int64_t, const int64_t*, float, const float*,
-                             const float*, const float*, const float*, void*, float*, void*, int64_t, void*) {
-  return AA_ERR_UNSUPPORTED;
+extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, int64_t H, int64_t V,
+                             const int64_t* labels, float inv_temperature, const float* row_lse, const float* row_ez,
+                             const float* g_logp, const float* g_entropy, void* d_hidden, float* d_weight,
+                             void* workspace, int64_t workspace_bytes, void* stream) {
+  if (!hidden || !weight || !labels || !row_lse || !g_logp || !d_hidden || !d_weight || !workspace)
+    return AA_ERR_INVALID_ARGUMENT;
+  if ((g_entropy && !row_ez) || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
+  if (!shapes_ok(T, H, V) || (V % 8) != 0) return AA_ERR_UNSUPPORTED;
+  if ((((uintptr_t)hidden | (uintptr_t)weight | (uintptr_t)workspace | (uintptr_t)d_hidden | (uintptr_t)d_weight) & 15))
+    return AA_ERR_INVALID_ARGUMENT;
+  const Workspace w = plan(T, H, V);
+  if (workspace_bytes < w.bytes) return AA_ERR_INVALID_ARGUMENT;
+  static const bool ok = allow_big_lds(k_lmhead_ds) && allow_big_lds(k_gemm_store<false, false>) &&
+                         allow_big_lds(k_gemm_store<true, false>) && allow_big_lds(k_gemm_store<true, true>);
+  if (!ok) return AA_ERR_LAUNCH;
+  hipStream_t st = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+  uint16_t* wt = (uint16_t*)(ws + w.off_wt);    // [H, V]
+  uint16_t* ht = (uint16_t*)(ws + w.off_ht);    // [H, ld_ht]
+  uint16_t* ds = (uint16_t*)(ws + w.off_ds);    // [chunk, V]
+  uint16_t* dst = (uint16_t*)(ws + w.off_dst);  // [V, ld_dst]
+  // K-contiguous copies of the operands of the two gradient GEMMs
+  hipLaunchKernelGGL(k_transpose_bf16, dim3((unsigned)((H + 63) / 64), (unsigned)((V + 63) / 64)), dim3(256), 0, st,
+                     (const uint16_t*)weight, V, H, H, wt, V);
+  hipLaunchKernelGGL(k_transpose_bf16, dim3((unsigned)((H + 63) / 64), (unsigned)((w.ld_ht + 63) / 64)), dim3(256), 0,
+                     st, (const uint16_t*)hidden, T, H, H, ht, w.ld_ht);
+  const int tiles_v = (int)((V + BM - 1) / BM);
+  const int tiles_h = (int)((H + BN - 1) / BN);
+  for (int64_t t0 = 0; t0 < T; t0 += w.chunk) {
+    const int64_t n_tok = (T - t0) < w.chunk ? (T - t0) : w.chunk;
+    const int64_t k_tok = (n_tok + 255) / 256 * 256;  // panel width incl. zero columns
+    const int tiles_t = (int)(k_tok / BN);
+    Operand W{(const uint16_t*)weight, H, (int)V};
+    Operand Hd{(const uint16_t*)hidden + t0 * H, H, (int)n_tok};
+    DsArgs a{row_lse, row_ez, g_logp, g_entropy, labels, ds, dst, w.ld_dst, t0, inv_temperature};
+    hipLaunchKernelGGL(k_lmhead_ds, dim3((unsigned)(tiles_v * tiles_t)), dim3(kThreads), kLdsBytes, st, W, Hd, (int)H,
+                       tiles_v, tiles_t, a);
+    // d_hidden[t0 : t0 + n_tok, :] = dS [n_tok, V] . Wt [H, V]^T
+    Operand A1{ds, V, (int)n_tok};
+    Operand B1{wt, V, (int)H};
+    hipLaunchKernelGGL((k_gemm_store<false, false>), dim3((unsigned)(tiles_t * tiles_h)), dim3(kThreads), kLdsBytes,
+                       st, A1, B1, (int)V, tiles_t, tiles_h, (void*)((uint16_t*)d_hidden + t0 * H), H);
+    // d_weight [V, H] (+)= dSt [V, k_tok] . Ht[:, t0 : t0 + k_tok]^T
+    Operand A2{dst, w.ld_dst, (int)V};
+    Operand B2{ht + t0, w.ld_ht, (int)H};
+    if (t0 == 0)
+      hipLaunchKernelGGL((k_gemm_store<true, false>), dim3((unsigned)(tiles_v * tiles_h)), dim3(kThreads), kLdsBytes,
+                         st, A2, B2, (int)k_tok, tiles_v, tiles_h, (void*)d_weight, H);
+    else
+      hipLaunchKernelGGL((k_gemm_store<true, true>), dim3((unsigned)(tiles_v * tiles_h)), dim3(kThreads), kLdsBytes,
+                         st, A2, B2, (int)k_tok, tiles_v, tiles_h, (void*)d_weight, H);
+  }
+  return launch_status();
 }

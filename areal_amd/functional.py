@@ -24,6 +24,7 @@ __all__ = [
     "apply_rejection_sampling",
     "ppo_actor_loss_fn",
     "fused_logprobs_ppo_loss",
+    "lm_head_logprobs_entropy",
 ]
 
 _DTYPES = {torch.bfloat16: N.AA_BF16, torch.float16: N.AA_F16, torch.float32: N.AA_F32}
@@ -618,3 +619,84 @@ def fused_logprobs_ppo_loss(
     if rejection_sampling is not None:
         _rs_stats(stat, prox, old, mask_eff, w, counts, loss_mask.shape)
     return loss, stat
+
+
+# ----------------------------------------------------------------------------
+# fused lm_head: hidden @ weight.T -> logp / entropy without the [T, V] logits
+# ----------------------------------------------------------------------------
+def _lmhead_workspace(T: int, H: int, V: int, dev) -> torch.Tensor:
+    n = N.load().aa_lmhead_workspace_bytes(T, H, V)
+    if n < 0:
+        raise N.NativeLibraryError(
+            f"fused lm_head needs hidden size and vocabulary to be multiples of 64 (got H={H}, V={V})"
+        )
+    return torch.empty(n, dtype=torch.uint8, device=dev)
+
+
+class _LmHeadLogprobsEntropy(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, hidden, weight, labels, temperature):
+        lib = N.load()
+        T, H = hidden.shape
+        V = weight.shape[0]
+        dev = hidden.device
+        f32 = dict(dtype=torch.float32, device=dev)
+        logp, entropy, row_lse, row_ez = (torch.empty(T, **f32) for _ in range(4))
+        ws = _lmhead_workspace(T, H, V, dev)
+        with torch.cuda.device(dev):
+            N.check(
+                lib.aa_lmhead_fwd(
+                    _ptr(hidden), _ptr(weight), T, H, V, _ptr(labels), 1.0 / float(temperature), _ptr(logp),
+                    _ptr(entropy), _ptr(row_lse), _ptr(row_ez), _ptr(ws), ws.numel(), _stream(dev),
+                ),
+                "aa_lmhead_fwd",
+            )
+        ctx.save_for_backward(hidden, weight, labels, row_lse, row_ez)
+        ctx.temperature = float(temperature)
+        return logp, entropy
+
+    @staticmethod
+    def backward(ctx, g_logp, g_entropy):
+        lib = N.load()
+        hidden, weight, labels, row_lse, row_ez = ctx.saved_tensors
+        T, H = hidden.shape
+        V = weight.shape[0]
+        dev = hidden.device
+        g_logp = torch.zeros(T, dtype=torch.float32, device=dev) if g_logp is None else _f32(g_logp)
+        g_entropy = None if g_entropy is None else _f32(g_entropy)
+        d_hidden = torch.empty_like(hidden)
+        d_weight = torch.empty(V, H, dtype=torch.float32, device=dev)
+        ws = _lmhead_workspace(T, H, V, dev)
+        with torch.cuda.device(dev):
+            N.check(
+                lib.aa_lmhead_bwd(
+                    _ptr(hidden), _ptr(weight), T, H, V, _ptr(labels), 1.0 / ctx.temperature, _ptr(row_lse),
+                    _ptr(row_ez), _ptr(g_logp), _ptr(g_entropy), _ptr(d_hidden), _ptr(d_weight), _ptr(ws),
+                    ws.numel(), _stream(dev),
+                ),
+                "aa_lmhead_bwd",
+            )
+        return d_hidden, d_weight.to(weight.dtype), None, None
+
+
+def lm_head_logprobs_entropy(
+    hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """``gather_logprobs_entropy(hidden @ weight.T, labels, temperature)`` without materialising the logits.
+
+    ``hidden`` is ``[T, H]`` and ``weight`` ``[V, H]`` (the lm_head), both bf16; logits tiles are formed on the
+    matrix cores with fp32 accumulation and reduced to log-prob and entropy on the fly.  Differentiable in
+    ``hidden`` and ``weight`` (fp32 accumulation; the weight gradient is returned in the dtype of ``weight``).
+    The reference has no such op: it is the drop-in for its lm_head matmul followed by
+    ``gather_logprobs_entropy`` (vocab_parallel.py:434-469).
+    """
+    _require_gpu(hidden, "hidden")
+    if hidden.ndim != 2 or weight.ndim != 2 or hidden.shape[1] != weight.shape[1]:
+        raise ValueError(f"expected hidden [T, H] and weight [V, H], got {tuple(hidden.shape)} and {tuple(weight.shape)}")
+    if tuple(labels.shape) != (hidden.shape[0],):
+        raise ValueError(f"labels shape {tuple(labels.shape)} != ({hidden.shape[0]},)")
+    assert hidden.shape[0] > 0, "Input must have at least one token"
+    if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise TypeError("fused lm_head expects bf16 hidden states and weights")
+    y = labels.to(device=hidden.device, dtype=torch.int64).contiguous()
+    return _LmHeadLogprobsEntropy.apply(hidden.contiguous(), weight.contiguous(), y, float(temperature))
