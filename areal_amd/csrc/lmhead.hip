@@ -17,6 +17,8 @@ namespace lmhead {
 using namespace gemm;
 
 constexpr int kChunkTokens = 16384;  // token chunk of the backward panel
+constexpr int kPanelPitch = BM + 8;   // pitch (elements) of the d(logits) tile staged in LDS as [token][vocab]
+constexpr int kLdsBytesDs = 256 * kPanelPitch * 2 > kLdsBytes ? 256 * kPanelPitch * 2 : kLdsBytes;  // 135168 B
 
 __device__ __forceinline__ int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
@@ -159,8 +161,8 @@ __global__ __launch_bounds__(kThreads) void k_lmhead_ds(Operand W, Operand Hd, i
   const int V = W.rows, N = Hd.rows;
   const int mbase = m0 + wm * 128;
   const float c = kLog2e * a.inv_t;
-  constexpr int PZ = BM + 8;  // pitch of the staged tile Z[token][vocab] in elements
-  uint16_t* Z = lds;          // 256 x 264 bf16 = 135168 B
+  constexpr int PZ = kPanelPitch;
+  uint16_t* Z = lds;  // 256 x 264 bf16 = 135168 B, over the operand stages (the main loop is done with them)
 
 #pragma unroll
   for (int nt = 0; nt < 4; ++nt) {
@@ -321,8 +323,8 @@ static bool shapes_ok(int64_t T, int64_t H, int64_t V) {
 }
 
 template <typename Kern>
-static bool allow_big_lds(Kern k) {
-  return hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) == hipSuccess;
+static bool allow_big_lds(Kern k, int bytes = kLdsBytes) {
+  return hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess;
 }
 
 }  // namespace lmhead
@@ -374,7 +376,7 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
     return AA_ERR_INVALID_ARGUMENT;
   const Workspace w = plan(T, H, V);
   if (workspace_bytes < w.bytes) return AA_ERR_INVALID_ARGUMENT;
-  static const bool ok = allow_big_lds(k_lmhead_ds) && allow_big_lds(k_gemm_store<false, false>) &&
+  static const bool ok = allow_big_lds(k_lmhead_ds, kLdsBytesDs) && allow_big_lds(k_gemm_store<false, false>) &&
                          allow_big_lds(k_gemm_store<true, false>) && allow_big_lds(k_gemm_store<true, true>);
   if (!ok) return AA_ERR_LAUNCH;
   hipStream_t st = (hipStream_t)stream;
@@ -397,7 +399,7 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
     Operand W{(const uint16_t*)weight, H, (int)V};
     Operand Hd{(const uint16_t*)hidden + t0 * H, H, (int)n_tok};
     DsArgs a{row_lse, row_ez, g_logp, g_entropy, labels, ds, dst, w.ld_dst, t0, inv_temperature};
-    hipLaunchKernelGGL(k_lmhead_ds, dim3((unsigned)(tiles_v * tiles_t)), dim3(kThreads), kLdsBytes, st, W, Hd, (int)H,
+    hipLaunchKernelGGL(k_lmhead_ds, dim3((unsigned)(tiles_v * tiles_t)), dim3(kThreads), kLdsBytesDs, st, W, Hd, (int)H,
                        tiles_v, tiles_t, a);
     // d_hidden[t0 : t0 + n_tok, :] = dS [n_tok, V] . Wt [H, V]^T
     Operand A1{ds, V, (int)n_tok};
