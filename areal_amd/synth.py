@@ -181,3 +181,85 @@ def config1(device, seed: int = 0, V: int = V_QWEN, n_seqs: int = 64, total_toke
     adv = grpo_advantages(lengths, 16, 0.4, seed + 3)
     ppo = dict(eps_clip=0.2, rejection_sampling=dict(level="token", action="mask", metric="ratio", upper=5.0))
     return make_logits_case(name, lengths, V, seed, device, adv, ppo=ppo)
+
+
+# ----------------------------------------------------------------------------
+# fused lm_head configurations: hidden states and lm_head weights instead of logits
+# ----------------------------------------------------------------------------
+def random_matrix(rows: int, cols: int, std: float, seed: int, device, rows_per_chunk: int = 8192) -> torch.Tensor:
+    """``std * N(0,1)`` bf16 matrix generated chunk by chunk on ``device``."""
+    out = torch.empty(rows, cols, dtype=torch.bfloat16, device=device)
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    for a in range(0, rows, rows_per_chunk):
+        b = min(a + rows_per_chunk, rows)
+        out[a:b] = (torch.randn(b - a, cols, generator=g, device=device, dtype=torch.float32) * std).to(torch.bfloat16)
+    return out
+
+
+def lengths_until_total(lo: int, hi: int, total: int, seed: int) -> list[int]:
+    """Uniform lengths in [lo, hi], drawn until they add up to ``total`` (the last one is shortened)."""
+    out, acc, g = [], 0, _gen(seed)
+    while acc < total:
+        n = int(torch.randint(lo, hi + 1, (1,), generator=g))
+        n = min(n, total - acc)
+        out.append(n)
+        acc += n
+    return out
+
+
+def make_hidden_case(name, lengths, H, V, seed, device, advantages, loss_mask=None, temperature=1.0, ppo=None,
+                     labels=None) -> PackedCase:
+    T = sum(lengths)
+    if labels is None:
+        labels = torch.randint(0, V, (T,), generator=_gen(seed + 1), dtype=torch.int64)
+    mask = prefix_mask(lengths, 0.3) if loss_mask is None else loss_mask
+    return PackedCase(
+        name=name,
+        cu_seqlens=cu_from_lengths(lengths).to(device),
+        labels=labels.to(device),
+        loss_mask=mask.to(device),
+        advantages=advantages.float().to(device),
+        hidden=random_matrix(T, H, 1.0, seed + 2, device),
+        weight=random_matrix(V, H, 0.02, seed + 4, device),
+        temperature=temperature,
+        ppo=dict(ppo or {}),
+    )
+
+
+def config2(device, seed: int = 0, T: int = 16384, H: int = 4096, V: int = V_QWEN) -> PackedCase:
+    """Fused lm_head path at the 8B shape: hidden [16384, 4096] ~ N(0,1), W [151936, 4096] ~ N(0, 0.02^2), labels
+    and masks as in configuration 0 on sequences of 64..512 tokens covering T tokens."""
+    lengths = lengths_until_total(64, 512, T, seed)
+    return make_hidden_case("cfg2", lengths, H, V, seed, device, per_sequence_normal_advantages(lengths, seed + 3),
+                            ppo=dict(eps_clip=0.2))
+
+
+def config3(device, seed: int = 0, n_seqs: int = 8, seq_len: int = 32768, H: int = 4096, V: int = V_QWEN) -> PackedCase:
+    """Long-context agentic rollout: 8 packed sequences of 32768 tokens, multi-turn mask (alternating 512-token
+    masked / unmasked spans), dual clip c = 3, importance-weight cap 5, eps_clip 0.2 low / 0.28 high."""
+    lengths = [seq_len] * n_seqs
+    ppo = dict(eps_clip=0.2, eps_clip_higher=0.28, c_clip=3.0,
+               rejection_sampling=dict(level="token", action="mask", metric="ratio", upper=5.0))
+    return make_hidden_case("cfg3", lengths, H, V, seed, device, per_sequence_normal_advantages(lengths, seed + 3),
+                            loss_mask=alternating_mask(lengths, 512), ppo=ppo)
+
+
+def config4(device, seed: int = 0, T: int = 32768, H: int = 5376, V: int = 262144, argmax_fraction: float = 0.2,
+            lo: int = 32, hi: int = 256) -> PackedCase:
+    """Large vocabulary, wide hidden: hidden [32768, 5376], W [262144, 5376], temperature 0.7, sequences of
+    32..256 tokens, 20 % of the labels are the argmax token of their row, 80 % uniform."""
+    lengths = lengths_until_total(lo, hi, T, seed)
+    case = make_hidden_case("cfg4", lengths, H, V, seed, device, per_sequence_normal_advantages(lengths, seed + 3),
+                            temperature=0.7, ppo=dict(eps_clip=0.2))
+    pick = (torch.rand(T, generator=_gen(seed + 5)) < argmax_fraction).to(device)
+    labels = case.labels.clone()
+    rows = 64 if torch.device(device).type == "cpu" else 1024
+    on_cpu = torch.device(device).type == "cpu"
+    for a in range(0, T, rows):  # tiled argmax of hidden @ W.T (input generation only)
+        b = min(a + rows, T)
+        h, w = case.hidden[a:b], case.weight
+        scores = h.float() @ w.float().t() if on_cpu else torch.matmul(h, w.t())
+        labels[a:b] = torch.where(pick[a:b], scores.argmax(-1), labels[a:b])
+    case.labels = labels
+    return case

@@ -1,18 +1,25 @@
 #!/usr/bin/env python3
 """Benchmark of the PPO/GRPO log-prob + entropy + actor-loss path (forward and backward) on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg1|cfg1-32k|cfg0]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg1|cfg1-32k|cfg0|cfg2|cfg3|cfg4]
 
-One "step" is one pass of the hot path over one synthetic packed micro-batch that is already resident in HBM:
-rejection sampling (importance-weight cap) -> fused log-prob / entropy / clipped PPO loss / d(logits) -> scalar
-loss, i.e. ``fused_logprobs_ppo_loss(...)`` followed by ``loss.backward()``.  Prints ONE JSON line.
+One "step" is one pass of the hot path over one synthetic packed micro-batch that is already resident in HBM.
 
-Besides the whole-step throughput the line carries
-  roofline      achieved HBM bandwidth of the dominant kernel (algorithmic bytes = 4 * V per token: the bf16
-                logits read once, their gradient written once) from HIP events around each launch;
-  cpu_baseline  the CPU oracle (a PyTorch restatement of the reference path) timed on this machine's host
-                cores on a bounded token sample of the same workload;
-  parity        the GPU result checked against that oracle on the same sample.
+* logits workloads (cfg0, cfg1, cfg1-32k; cfg1 is the default, the configuration the metric is quoted on):
+  rejection sampling (importance-weight cap) -> fused log-prob / entropy / clipped PPO loss / d(logits) -> scalar
+  loss, i.e. ``fused_logprobs_ppo_loss(...)`` followed by ``loss.backward()``.  Roofline: HBM, algorithmic bytes
+  4 * V per token (the bf16 logits read once, their gradient written once).
+* fused lm_head workloads (cfg2, cfg3, cfg4): ``lm_head_logprobs_entropy(hidden, W, labels)`` ->
+  ``ppo_actor_loss_fn`` -> ``loss.backward()`` down to d(hidden) and d(W), logits never materialised.  Roofline:
+  bf16 MFMA, algorithmic flops 6 * T * V * H (forward 2TVH, backward 4TVH; the backward's recompute of the logits
+  tiles is overhead and is not counted).
+
+Prints ONE JSON line.  Besides the whole-step throughput it carries
+  roofline      of the dominant kernel(s), timed with HIP events on the launch stream;
+  cpu_baseline  the CPU oracle (a PyTorch restatement of the reference path) timed on this machine's host cores on a
+                bounded token sample of the same workload;
+  parity        the GPU result checked against that oracle on the same sample;
+  fused_lm_head (default run only) the same figures for the cfg2 workload, so that one run reports both paths.
 """
 from __future__ import annotations
 
@@ -28,7 +35,11 @@ ROOT = Path(__file__).resolve().parent
 if str(ROOT) not in sys.path:
     sys.path.insert(0, str(ROOT))
 
-HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published peak
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published peak
+METRIC = "tokens/sec for logprob+entropy+PPO loss fwd+bwd"
+LOGITS_WORKLOADS = ("cfg0", "cfg1", "cfg1-32k")
+FUSED_WORKLOADS = ("cfg2", "cfg3", "cfg4")
 
 
 def parse_args():
@@ -36,17 +47,54 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg1-32k"])
+    ap.add_argument("--workload", default="cfg1", choices=LOGITS_WORKLOADS + FUSED_WORKLOADS)
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--cpu-tokens", type=int, default=1024, help="token sample of the CPU baseline (0 = skip)")
+    ap.add_argument("--cpu-tokens", type=int, default=1024,
+                    help="token sample of the CPU baseline (0 = skip); fused lm_head workloads use at most 128")
     ap.add_argument("--cpu-iters", type=int, default=3)
+    ap.add_argument("--no-fused-extra", action="store_true",
+                    help="default workload only: do not append the cfg2 fused lm_head figures")
     ap.add_argument("--copy-launches", type=int, default=0,
                     help="also launch the plain copy kernel this many times over the logits buffer "
                          "(the calibration point for FETCH_SIZE / WRITE_SIZE counters)")
     return ap.parse_args()
 
 
-def build_case(name: str, seed: int, device):
+def ppo_kwargs(case):
+    from areal_amd import RejectionSamplingConfig
+
+    kw = dict(case.ppo)
+    rs = kw.pop("rejection_sampling", None)
+    cfg = RejectionSamplingConfig(**rs) if rs else None
+    return kw, cfg
+
+
+def cosine(a, b) -> float:
+    a, b = a.double().reshape(-1), b.double().reshape(-1)
+    return float(a @ b / (a.norm() * b.norm()))
+
+
+def time_events(launch, iters: int, stream):
+    """(mean, min) milliseconds of ``launch()`` between HIP events recorded on ``stream``."""
+    import torch
+
+    for _ in range(3):
+        launch()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    for a, b in evs:
+        a.record(stream)
+        launch()
+        b.record(stream)
+    torch.cuda.synchronize()
+    times = sorted(a.elapsed_time(b) for a, b in evs)
+    return sum(times) / len(times), times[0]
+
+
+# ----------------------------------------------------------------------------------------------------------------
+# logits path
+# ----------------------------------------------------------------------------------------------------------------
+def build_logits_case(name: str, seed: int, device):
     import areal_amd
     from areal_amd import synth
 
@@ -65,16 +113,7 @@ def build_case(name: str, seed: int, device):
     return case, desc
 
 
-def ppo_kwargs(case):
-    from areal_amd import RejectionSamplingConfig
-
-    kw = dict(case.ppo)
-    rs = kw.pop("rejection_sampling", None)
-    cfg = RejectionSamplingConfig(**rs) if rs else None
-    return kw, cfg
-
-
-def run_steps(case, n, kw, cfg):
+def run_logits_steps(case, n, kw, cfg):
     import areal_amd
 
     x = case.logits
@@ -89,8 +128,8 @@ def run_steps(case, n, kw, cfg):
     return loss
 
 
-def time_dominant_kernel(case, kw, cfg, iters: int):
-    """Average duration of aa_logits_ppo_fused alone, HIP events on the launch stream, outputs pre-allocated."""
+def time_fused_logits_kernel(case, kw, cfg, iters: int):
+    """Duration of aa_logits_ppo_fused alone, HIP events on the launch stream, outputs pre-allocated."""
     import torch
 
     from areal_amd import _native as N
@@ -125,20 +164,10 @@ def time_dominant_kernel(case, kw, cfg, iters: int):
             "aa_logits_ppo_fused",
         )
 
-    for _ in range(3):
-        launch()
-    torch.cuda.synchronize()
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
-    for a, b in evs:
-        a.record(stream)
-        launch()
-        b.record(stream)
-    torch.cuda.synchronize()
-    times = sorted(a.elapsed_time(b) for a, b in evs)
-    return sum(times) / len(times), times[0]
+    return time_events(launch, iters, stream)
 
 
-def cpu_baseline_and_parity(case, kw, cfg, n_tokens: int, iters: int):
+def logits_cpu_baseline_and_parity(case, kw, cfg, n_tokens: int, iters: int):
     """Oracle fwd+bwd on the first ``n_tokens`` tokens (host cores), and the GPU path checked on the same slice."""
     import torch
 
@@ -166,12 +195,11 @@ def cpu_baseline_and_parity(case, kw, cfg, n_tokens: int, iters: int):
     )
     loss.backward()
     torch.cuda.synchronize()
-    a, b = x.grad.cpu().double().reshape(-1), w_grad.double().reshape(-1)
     parity = dict(
         tokens=n,
         logp_max_abs_err=float((stat["logprobs"].cpu() - w_stat["logprobs"]).abs().max()),
         loss_rel_err=abs(float(loss.detach()) - float(w_loss)) / max(abs(float(w_loss)), 1e-12),
-        grad_cosine=float(a @ b / (a.norm() * b.norm())),
+        grad_cosine=cosine(x.grad.cpu(), w_grad),
         masks_equal=bool(torch.equal(stat["clip_mask"].cpu(), w_stat["clip_mask"])),
     )
     baseline = dict(
@@ -182,35 +210,24 @@ def cpu_baseline_and_parity(case, kw, cfg, n_tokens: int, iters: int):
     return baseline, parity
 
 
-def main():
-    args = parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build measures one GPU; run it with --gpus 1 (no multi-GPU path exists)", file=sys.stderr)
-        sys.exit(2)
+def bench_logits(args, dev):
     import torch
 
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(2)
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    case, desc = build_case(args.workload, args.seed, dev)
+    case, desc = build_logits_case(args.workload, args.seed, dev)
     kw, cfg = ppo_kwargs(case)
     T, V = case.logits.shape
     case.logits.requires_grad_(True)
-
-    run_steps(case, args.warmup, kw, cfg)
+    run_logits_steps(case, args.warmup, kw, cfg)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    loss = run_steps(case, args.steps, kw, cfg)
+    loss = run_logits_steps(case, args.steps, kw, cfg)
     torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    ms_per_step = dt / args.steps * 1e3
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
     assert bool(torch.isfinite(loss)), "loss is not finite"
 
     case.logits.grad = None
     case.logits.requires_grad_(False)
-    k_ms, k_min_ms = time_dominant_kernel(case, kw, cfg, max(args.steps, 10))
+    k_ms, k_min_ms = time_fused_logits_kernel(case, kw, cfg, max(args.steps, 10))
     alg_bytes = 4.0 * T * V
     achieved = alg_bytes / (k_ms * 1e-3) / 1e9
     roofline = dict(
@@ -222,7 +239,7 @@ def main():
         algorithmic_bytes_per_launch=alg_bytes,
     )
     out = dict(
-        metric="tokens/sec for logprob+entropy+PPO loss fwd+bwd", value=T / (ms_per_step * 1e-3), unit="tokens/s",
+        metric=METRIC, value=T / (ms_per_step * 1e-3), unit="tokens/s",
         n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=ms_per_step, higher_is_better=True,
         scaling="weak", vs_baseline=None, dtype="bf16", data="synthetic",
         config=dict(workload=f"{case.name}: {desc}", tokens=T, vocab=V, sequences=int(case.cu_seqlens.numel() - 1),
@@ -241,9 +258,215 @@ def main():
         out["copy_calibration"] = dict(kernel="k_copy16 (aa_copy_bytes)", bytes_read=nbytes, bytes_written=nbytes,
                                        launches=args.copy_launches)
     if args.cpu_tokens > 0:
-        baseline, parity = cpu_baseline_and_parity(case, kw, cfg, args.cpu_tokens, args.cpu_iters)
+        baseline, parity = logits_cpu_baseline_and_parity(case, kw, cfg, args.cpu_tokens, args.cpu_iters)
         out["cpu_baseline"] = baseline
         out["parity"] = parity
+    return out
+
+
+# ----------------------------------------------------------------------------------------------------------------
+# fused lm_head path
+# ----------------------------------------------------------------------------------------------------------------
+def build_fused_case(name: str, seed: int, device):
+    import torch
+
+    import areal_amd
+    from areal_amd import synth
+
+    if name == "cfg2":
+        case = synth.config2(device, seed)
+        desc = "configs[2]: hidden [16384,4096], W [151936,4096], masks as configs[0], eps_clip=0.2"
+    elif name == "cfg3":
+        case = synth.config3(device, seed)
+        desc = ("configs[3]: 8 packed seqs of 32768 tokens, hidden [262144,4096], W [151936,4096], alternating "
+                "512-token mask, dual clip c=3, importance-weight cap 5, eps_clip 0.2 / 0.28")
+    else:
+        case = synth.config4(device, seed)
+        desc = "configs[4]: hidden [32768,5376], W [262144,5376], temperature 0.7, 20% argmax labels"
+    with torch.no_grad():
+        ref, _ = areal_amd.lm_head_logprobs_entropy(case.hidden, case.weight, case.labels, case.temperature)
+    synth.attach_old_and_prox(case, ref, 0.05, seed + 9)
+    return case, desc
+
+
+def run_fused_steps(case, n, kw, cfg):
+    import areal_amd
+
+    h, w = case.hidden, case.weight
+    loss = None
+    for _ in range(n):
+        h.grad = None
+        w.grad = None
+        lp, _ent = areal_amd.lm_head_logprobs_entropy(h, w, case.labels, case.temperature)
+        loss, _ = areal_amd.ppo_actor_loss_fn(
+            lp, case.prox_logp, case.old_logp, case.advantages, loss_mask=case.loss_mask, rejection_sampling=cfg,
+            cu_seqlens=case.cu_seqlens, **kw,
+        )
+        loss.backward()
+    return loss
+
+
+def time_lmhead_kernels(case, iters: int):
+    """Durations of aa_lmhead_fwd and aa_lmhead_bwd (all the kernels each enqueues), HIP events on the launch stream."""
+    import torch
+
+    from areal_amd import _native as N
+    from areal_amd import functional as F
+
+    lib = N.load()
+    dev = case.hidden.device
+    T, H = case.hidden.shape
+    V = case.weight.shape[0]
+    f32 = dict(dtype=torch.float32, device=dev)
+    logp, ent, lse, ez = (torch.empty(T, **f32) for _ in range(4))
+    ws = F._lmhead_workspace(T, H, V, dev)
+    g = torch.randn(T, **f32) * case.loss_mask.float() / T
+    dh = torch.empty_like(case.hidden)
+    dw = torch.empty(V, H, **f32)
+    stream = torch.cuda.current_stream(dev)
+    st = C.c_void_p(stream.cuda_stream)
+    inv_t = 1.0 / case.temperature
+
+    def fwd():
+        N.check(lib.aa_lmhead_fwd(F._ptr(case.hidden), F._ptr(case.weight), T, H, V, F._ptr(case.labels), inv_t,
+                                  F._ptr(logp), F._ptr(ent), F._ptr(lse), F._ptr(ez), F._ptr(ws), ws.numel(), st),
+                "aa_lmhead_fwd")
+
+    def bwd():
+        N.check(lib.aa_lmhead_bwd(F._ptr(case.hidden), F._ptr(case.weight), T, H, V, F._ptr(case.labels), inv_t,
+                                  F._ptr(lse), F._ptr(ez), F._ptr(g), None, F._ptr(dh), F._ptr(dw), F._ptr(ws),
+                                  ws.numel(), st), "aa_lmhead_bwd")
+
+    f_ms, _ = time_events(fwd, iters, stream)
+    b_ms, _ = time_events(bwd, iters, stream)
+    return f_ms, b_ms
+
+
+def fused_cpu_baseline_and_parity(case, kw, cfg, n_tokens: int, iters: int):
+    """Oracle (fp32 matmul + logits path + PPO loss + autograd) on the first ``n_tokens`` tokens against the full
+    weight matrix, and the GPU path checked on the same slice."""
+    import torch
+
+    import areal_amd
+    import oracle
+
+    n = min(n_tokens, case.n_tokens)
+    sl = slice(0, n)
+    cpu = lambda t: t[sl].cpu()
+    hid, lab = cpu(case.hidden).float(), cpu(case.labels)
+    w_cpu = case.weight.cpu().float()
+    prox, old, adv, mask = cpu(case.prox_logp), cpu(case.old_logp), cpu(case.advantages), cpu(case.loss_mask)
+    cu = torch.tensor([0, n], dtype=torch.int32)
+    threads = torch.get_num_threads()
+
+    def oracle_step():
+        h = hid.clone().requires_grad_(True)
+        w = w_cpu.clone().requires_grad_(True)
+        lp, _ent = oracle.logprobs_entropy(h @ w.t(), lab, case.temperature)
+        loss, _stat = oracle.ppo_actor_loss(lp, prox, old, adv, loss_mask=mask.bool(), rejection_sampling_cfg=cfg,
+                                            cu_seqlens=cu, **kw)
+        loss.backward()
+        return loss.detach(), lp.detach(), h.grad, w.grad
+
+    oracle_step()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        w_loss, w_lp, w_dh, w_dw = oracle_step()
+    dt = (time.perf_counter() - t0) / iters
+
+    h = case.hidden[sl].detach().clone().requires_grad_(True)
+    w = case.weight.detach().clone().requires_grad_(True)
+    lp, _ent = areal_amd.lm_head_logprobs_entropy(h, w, case.labels[sl], case.temperature)
+    loss, _stat = areal_amd.ppo_actor_loss_fn(lp, case.prox_logp[sl], case.old_logp[sl], case.advantages[sl],
+                                              loss_mask=case.loss_mask[sl], rejection_sampling=cfg,
+                                              cu_seqlens=cu.to(h.device), **kw)
+    loss.backward()
+    torch.cuda.synchronize()
+    parity = dict(
+        tokens=n,
+        logp_max_abs_err=float((lp.detach().cpu() - w_lp).abs().max()),
+        loss_rel_err=abs(float(loss.detach()) - float(w_loss)) / max(abs(float(w_loss)), 1e-12),
+        d_hidden_cosine=cosine(h.grad.cpu(), w_dh),
+        d_weight_cosine=cosine(w.grad.cpu(), w_dw),
+    )
+    baseline = dict(
+        value=n / dt, unit="tokens/s", cores=threads, kind="port",
+        sample=f"first {n} tokens of the workload against the full weight matrix, {iters} timed fwd+bwd passes of the "
+               f"PyTorch CPU oracle (fp32 hidden @ W.T, log_softmax + gather + entropy, PPO loss, autograd to "
+               f"d(hidden) and d(W))",
+    )
+    return baseline, parity
+
+
+def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: int):
+    import torch
+
+    case, desc = build_fused_case(workload, args.seed, dev)
+    kw, cfg = ppo_kwargs(case)
+    T, H = case.hidden.shape
+    V = case.weight.shape[0]
+    case.hidden.requires_grad_(True)
+    case.weight.requires_grad_(True)
+    run_fused_steps(case, warmup, kw, cfg)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    loss = run_fused_steps(case, steps, kw, cfg)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / steps * 1e3
+    assert bool(torch.isfinite(loss)), "loss is not finite"
+    case.hidden.grad = None
+    case.weight.grad = None
+    case.hidden.requires_grad_(False)
+    case.weight.requires_grad_(False)
+
+    f_ms, b_ms = time_lmhead_kernels(case, max(min(steps, 10), 3))
+    alg_flops = 6.0 * T * V * H
+    achieved = alg_flops / ((f_ms + b_ms) * 1e-3) / 1e12
+    roofline = dict(
+        bound="mfma", kernel="aa_lmhead_fwd + aa_lmhead_bwd (k_lmhead_stats, k_lmhead_ds, k_gemm_store x 2)",
+        achieved=achieved, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s", frac=achieved / MFMA_BF16_PEAK_TFLOPS,
+        traffic=None, fwd_ms=f_ms, bwd_ms=b_ms,
+        fwd_tflops=2.0 * T * V * H / (f_ms * 1e-3) / 1e12, bwd_tflops=4.0 * T * V * H / (b_ms * 1e-3) / 1e12,
+        algorithmic_flops_per_step=alg_flops, executed_flops_per_step=8.0 * T * V * H,
+    )
+    out = dict(
+        metric=METRIC, value=T / (ms_per_step * 1e-3), unit="tokens/s",
+        n_gpus=1, steps=steps, warmup=warmup, ms_per_step=ms_per_step, higher_is_better=True,
+        scaling="weak", vs_baseline=None, dtype="bf16", data="synthetic",
+        config=dict(workload=f"{case.name}: {desc}", tokens=T, hidden=H, vocab=V,
+                    sequences=int(case.cu_seqlens.numel() - 1), accumulate="f32",
+                    path="fused lm_head (logits never materialised) + PPO loss, fwd + bwd"),
+        roofline=roofline,
+    )
+    if cpu_tokens > 0:
+        baseline, parity = fused_cpu_baseline_and_parity(case, kw, cfg, cpu_tokens, args.cpu_iters)
+        out["cpu_baseline"] = baseline
+        out["parity"] = parity
+    return out
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU; run it with --gpus 1 (no multi-GPU path exists)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    if args.workload in LOGITS_WORKLOADS:
+        out = bench_logits(args, dev)
+        if args.workload == "cfg1" and not args.no_fused_extra and args.copy_launches == 0:
+            torch.cuda.empty_cache()
+            extra = bench_fused(args, dev, "cfg2", steps=min(args.steps, 5), warmup=min(args.warmup, 2),
+                                cpu_tokens=min(args.cpu_tokens, 128))
+            keys = ("value", "unit", "ms_per_step", "steps", "warmup", "config", "roofline", "cpu_baseline", "parity")
+            out["fused_lm_head"] = {k: extra[k] for k in keys if k in extra}
+    else:
+        out = bench_fused(args, dev, args.workload, args.steps, args.warmup, min(args.cpu_tokens, 128))
     print(json.dumps(out))
 
 

@@ -108,3 +108,66 @@ def test_lm_head_into_ppo_loss_end_to_end(device):
     o_loss.backward()
     assert float(loss.detach()) == pytest.approx(float(o_loss), rel=1e-3, abs=1e-7)
     assert cosine(h_d.grad.cpu(), h_o.grad) > 0.9999 and cosine(w_d.grad.cpu(), w_o.grad) > 0.9999
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Full-size configurations.  The oracle cannot run these whole, so they are checked on token slices (every token's
+# log-prob, entropy and d(hidden) row depend only on that token's hidden state and the full weight matrix) and
+# through properties that hold at any size: determinism, log-prob <= 0, 0 <= entropy <= log V, and linearity of
+# d(W) in the upstream gradient, which ties the full-size weight gradient to a slice the oracle can compute.
+# ---------------------------------------------------------------------------------------------------------------
+def _cos_dev(a, b, device):
+    a, b = a.to(device).double().reshape(-1), b.to(device).double().reshape(-1)
+    return float(a @ b / (a.norm() * b.norm()))
+
+
+def _oracle_slice(case, idx, g_slice):
+    h = case.hidden[idx].cpu().float().requires_grad_(True)
+    w = case.weight.cpu().float().requires_grad_(True)
+    lp, ent = oracle.logprobs_entropy(h @ w.t(), case.labels[idx].cpu(), case.temperature)
+    (lp * g_slice).sum().backward()
+    return lp.detach(), ent.detach(), h.grad, w.grad
+
+
+@pytest.mark.parametrize("name", ["cfg2", "cfg4", "cfg3"])
+def test_full_size_configuration(device, name):
+    from areal_amd import synth
+
+    case = getattr(synth, {"cfg2": "config2", "cfg3": "config3", "cfg4": "config4"}[name])(device, seed=0)
+    T, H = case.hidden.shape
+    V = case.weight.shape[0]
+    print(f"full-size {name}: T={T} H={H} V={V}", flush=True)
+    n_s = 48
+    idx = torch.cat([torch.arange(0, 16), torch.arange(T // 2 - 8, T // 2 + 8), torch.arange(T - 16, T)]).to(device)
+    g = torch.Generator().manual_seed(11)
+    g_slice = torch.randn(n_s, generator=g)
+    g_rest = (torch.randn(T, generator=g) * case.loss_mask.cpu().float()).to(device)
+    g_rest[idx] = 0.0
+    g_only = torch.zeros(T, device=device)
+    g_only[idx] = g_slice.to(device)
+
+    def run(gvec):
+        h = case.hidden.detach().requires_grad_(True)
+        w = case.weight.detach().requires_grad_(True)
+        lp, ent = areal_amd.lm_head_logprobs_entropy(h, w, case.labels, case.temperature)
+        (lp * gvec).sum().backward()
+        return lp.detach(), ent.detach(), h.grad, w.grad
+
+    lp, ent, dh_only, dw_only = run(g_only)
+    assert bool((lp <= 1e-6).all()) and bool((ent >= -1e-4).all()) and bool((ent <= math.log(V) + 1e-4).all())
+    o_lp, o_ent, o_dh, o_dw = _oracle_slice(case, idx, g_slice)
+    assert float((lp[idx].cpu() - o_lp).abs().max()) < 2e-3  # stated tolerance
+    assert float((ent[idx].cpu() - o_ent).abs().max()) < 2e-3
+    assert cosine(dh_only[idx].cpu().float(), o_dh) > 0.9999
+    assert float(dh_only.float().abs().sum()) == pytest.approx(float(dh_only[idx].float().abs().sum()), rel=1e-6)
+    # the full-size weight gradient with only the slice's tokens switched on is the oracle's slice gradient
+    assert _cos_dev(dw_only, o_dw, device) > 0.9999
+    del o_dw
+    # determinism and linearity of d(W), d(hidden) in the upstream gradient
+    lp2, ent2, dh_rest, dw_rest = run(g_rest)
+    assert torch.equal(lp, lp2) and torch.equal(ent, ent2)
+    _, _, dh_all, dw_all = run(g_rest + g_only)
+    assert _cos_dev(dw_rest.float() + dw_only.float(), dw_all, device) > 0.9999
+    assert _cos_dev(dh_rest.float() + dh_only.float(), dh_all, device) > 0.9999
+    _, _, dh_again, dw_again = run(g_rest + g_only)
+    assert torch.equal(dh_all, dh_again) and torch.equal(dw_all, dw_again)

@@ -79,3 +79,21 @@ def test_synthetic_layouts():
     case = synth.config0("cpu", seed=0, V=64, n_seqs=3, lo=4, hi=9)
     assert case.logits.shape == (case.n_tokens, 64) and case.logits.dtype == torch.bfloat16
     assert case.labels.dtype == torch.int64 and case.loss_mask.dtype == torch.bool
+
+
+def test_synthetic_hidden_state_configurations():
+    lengths = synth.lengths_until_total(4, 9, 50, seed=1)
+    assert sum(lengths) == 50 and all(1 <= n <= 9 for n in lengths)
+    c2 = synth.config2("cpu", seed=0, T=300, H=64, V=640)
+    assert c2.hidden.shape == (300, 64) and c2.weight.shape == (640, 64) and c2.logits is None
+    assert c2.hidden.dtype == torch.bfloat16 and int(c2.cu_seqlens[-1]) == 300
+    assert 0.015 < float(c2.weight.float().std()) < 0.025 and 0.9 < float(c2.hidden.float().std()) < 1.1
+    c3 = synth.config3("cpu", seed=0, n_seqs=2, seq_len=2048, H=64, V=128)
+    assert c3.ppo["c_clip"] == 3.0 and c3.ppo["eps_clip_higher"] == 0.28
+    assert c3.ppo["rejection_sampling"]["upper"] == 5.0
+    assert not c3.loss_mask[:512].any() and c3.loss_mask[512:1024].all() and not c3.loss_mask[2048 : 2048 + 512].any()
+    c4 = synth.config4("cpu", seed=0, T=400, H=64, V=256, lo=8, hi=32)
+    assert c4.temperature == 0.7
+    best = (c4.hidden.float() @ c4.weight.float().t()).argmax(-1)
+    frac = float((best == c4.labels).float().mean())
+    assert 0.12 < frac < 0.30  # 20 % argmax labels (+ chance hits)
