@@ -7,6 +7,7 @@ from .config import RejectionSamplingConfig
 from .functional import (
     RejectionSamplingResult,
     apply_rejection_sampling,
+    fused_lm_head_ppo_loss,
     fused_logprobs_ppo_loss,
     gather_logprobs,
     gather_logprobs_entropy,
@@ -23,6 +24,7 @@ __all__ = [
     "RejectionSamplingConfig",
     "RejectionSamplingResult",
     "apply_rejection_sampling",
+    "fused_lm_head_ppo_loss",
     "fused_logprobs_ppo_loss",
     "gather_logprobs",
     "gather_logprobs_entropy",

@@ -272,20 +272,38 @@ __global__ __launch_bounds__(kThreads) void k_gemm_store(Operand A, Operand B, i
 }
 
 // ---- bf16 transpose with zero padding: dst[c][r] = src[r][c], dst is [C, ld_dst], columns >= R are zeroed --------
+// 64 x 64 tiles, 16-byte global loads and stores; the tile is turned in LDS (pitch 33 words, so the eight 2-byte reads
+// that gather one output chunk fall in different banks).  Needs Cc, ld_src, ld_dst multiples of 8 and 16-byte bases.
 __global__ __launch_bounds__(256) void k_transpose_bf16(const uint16_t* __restrict__ src, int64_t R, int64_t Cc,
                                                         int64_t ld_src, uint16_t* __restrict__ dst, int64_t ld_dst) {
-  __shared__ uint16_t tile[64][66];
+  __shared__ uint32_t tile[64 * 33];
   const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
-  for (int p = threadIdx.x; p < 64 * 64; p += 256) {
-    const int r = p >> 6, cc = p & 63;
-    const int64_t rr = r0 + r, ccg = c0 + cc;
-    tile[r][cc] = (rr < R && ccg < Cc) ? src[rr * ld_src + ccg] : (uint16_t)0;
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    const int p = threadIdx.x + 256 * s;
+    const int r = p >> 3, ch = p & 7;
+    const int64_t rr = r0 + r, cg = c0 + ch * 8;
+    uint4 v = make_uint4(0u, 0u, 0u, 0u);
+    if (rr < R && cg < Cc) v = *(const uint4*)(src + rr * ld_src + cg);
+    uint32_t* t = tile + r * 33 + ch * 4;
+    t[0] = v.x; t[1] = v.y; t[2] = v.z; t[3] = v.w;
   }
   __syncthreads();
-  for (int p = threadIdx.x; p < 64 * 64; p += 256) {
-    const int cc = p >> 6, r = p & 63;
-    const int64_t rr = r0 + r, ccg = c0 + cc;
-    if (ccg < Cc && rr < ld_dst) dst[ccg * ld_dst + rr] = tile[r][cc];
+  const uint16_t* t16 = (const uint16_t*)tile;
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    const int p = threadIdx.x + 256 * s;
+    const int c = p >> 3, j = p & 7;
+    const int64_t cg = c0 + c, rg = r0 + j * 8;
+    if (cg < Cc && rg < ld_dst) {
+      uint32_t w[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const uint32_t lo = t16[(j * 8 + 2 * q) * 66 + c], hi = t16[(j * 8 + 2 * q + 1) * 66 + c];
+        w[q] = lo | (hi << 16);
+      }
+      *(uint4*)(dst + cg * ld_dst + rg) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
   }
 }
 
@@ -407,6 +425,73 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
     hipLaunchKernelGGL((k_gemm_store<false, false>), dim3((unsigned)(tiles_t * tiles_h)), dim3(kThreads), kLdsBytes,
                        st, A1, B1, (int)V, tiles_t, tiles_h, (void*)((uint16_t*)d_hidden + t0 * H), H);
     // d_weight [V, H] (+)= dSt [V, k_tok] . Ht[:, t0 : t0 + k_tok]^T
+    Operand A2{dst, w.ld_dst, (int)V};
+    Operand B2{ht + t0, w.ld_ht, (int)H};
+    if (t0 == 0)
+      hipLaunchKernelGGL((k_gemm_store<true, false>), dim3((unsigned)(tiles_v * tiles_h)), dim3(kThreads), kLdsBytes,
+                         st, A2, B2, (int)k_tok, tiles_v, tiles_h, (void*)d_weight, H);
+    else
+      hipLaunchKernelGGL((k_gemm_store<true, true>), dim3((unsigned)(tiles_v * tiles_h)), dim3(kThreads), kLdsBytes,
+                         st, A2, B2, (int)k_tok, tiles_v, tiles_h, (void*)d_weight, H);
+  }
+  return launch_status();
+}
+
+extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64_t T, int64_t H, int64_t V,
+                                   const int64_t* labels, float inv_temperature, int64_t T_active,
+                                   const float* prox_logp, const float* adv, const uint8_t* mask_eff,
+                                   const float* behave_w, const aa_ppo_params* params, const int32_t* n_valid,
+                                   const float* grad_scale, float* logp, float* entropy, float* stat_loss, float* ratio,
+                                   uint8_t* flags, void* d_hidden, float* d_weight, int32_t* work, void* workspace,
+                                   int64_t workspace_bytes, void* stream) {
+  if (!hidden || !weight || !labels || !d_hidden || !d_weight || !workspace) return AA_ERR_INVALID_ARGUMENT;
+  if (!params || !prox_logp || !adv || !mask_eff || !n_valid || !logp || !stat_loss || !ratio || !flags)
+    return AA_ERR_INVALID_ARGUMENT;
+  if (params->has_behave_weight && !behave_w) return AA_ERR_INVALID_ARGUMENT;
+  if (T_active < 0 || T_active > T || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
+  if (!shapes_ok(T, H, V) || (V % 8) != 0) return AA_ERR_UNSUPPORTED;
+  if ((((uintptr_t)hidden | (uintptr_t)weight | (uintptr_t)workspace | (uintptr_t)d_hidden | (uintptr_t)d_weight) & 15))
+    return AA_ERR_INVALID_ARGUMENT;
+  const Workspace w = plan(T, H, V);
+  if (workspace_bytes < w.bytes) return AA_ERR_INVALID_ARGUMENT;
+  static const bool ok = allow_big_lds(k_gemm_store<false, false>) && allow_big_lds(k_gemm_store<true, false>) &&
+                         allow_big_lds(k_gemm_store<true, true>);
+  if (!ok) return AA_ERR_LAUNCH;
+  hipStream_t st = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+  uint16_t* wt = (uint16_t*)(ws + w.off_wt);    // [H, V]
+  uint16_t* ht = (uint16_t*)(ws + w.off_ht);    // [H, ld_ht]
+  uint16_t* ds = (uint16_t*)(ws + w.off_ds);    // [chunk, V]: logits of the chunk, then their gradient in place
+  uint16_t* dst = (uint16_t*)(ws + w.off_dst);  // [V, ld_dst]: the gradient panel transposed
+  hipLaunchKernelGGL(k_transpose_bf16, dim3((unsigned)((H + 63) / 64), (unsigned)((V + 63) / 64)), dim3(256), 0, st,
+                     (const uint16_t*)weight, V, H, H, wt, V);
+  hipLaunchKernelGGL(k_transpose_bf16, dim3((unsigned)((H + 63) / 64), (unsigned)((w.ld_ht + 63) / 64)), dim3(256), 0,
+                     st, (const uint16_t*)hidden, T, H, H, ht, w.ld_ht);
+  const int tiles_v = (int)((V + BM - 1) / BM);
+  const int tiles_h = (int)((H + BN - 1) / BN);
+  for (int64_t t0 = 0; t0 < T; t0 += w.chunk) {
+    const int64_t n_tok = (T - t0) < w.chunk ? (T - t0) : w.chunk;
+    const int64_t k_tok = (n_tok + 255) / 256 * 256;
+    const int tiles_t = (int)(k_tok / BM);
+    int64_t act = T_active - t0;
+    act = act < 0 ? 0 : (act > n_tok ? n_tok : act);
+    // logits[t0 : t0 + n_tok, :] = hidden . W^T, rounded to bf16 as the reference's lm_head output is
+    Operand Hd{(const uint16_t*)hidden + t0 * H, H, (int)n_tok};
+    Operand W{(const uint16_t*)weight, H, (int)V};
+    hipLaunchKernelGGL((k_gemm_store<false, false>), dim3((unsigned)(tiles_t * tiles_v)), dim3(kThreads), kLdsBytes,
+                       st, Hd, W, (int)H, tiles_t, tiles_v, (void*)ds, V);
+    // log-prob, entropy, PPO loss and d(loss)/d(logits) in place: one streaming pass over the panel
+    const int rc = aa_logits_ppo_fused(ds, AA_BF16, n_tok, V, V, labels + t0, inv_temperature, act, prox_logp + t0,
+                                       adv + t0, mask_eff + t0, behave_w ? behave_w + t0 : nullptr, params, n_valid,
+                                       grad_scale, logp + t0, entropy ? entropy + t0 : nullptr, nullptr, nullptr,
+                                       stat_loss + t0, ratio + t0, flags + t0, ds, work, stream);
+    if (rc != AA_OK) return rc;
+    hipLaunchKernelGGL(k_transpose_bf16, dim3((unsigned)((V + 63) / 64), (unsigned)(w.ld_dst / 64)), dim3(256), 0, st,
+                       (const uint16_t*)ds, n_tok, V, V, dst, w.ld_dst);
+    Operand A1{ds, V, (int)n_tok};
+    Operand B1{wt, V, (int)H};
+    hipLaunchKernelGGL((k_gemm_store<false, false>), dim3((unsigned)(tiles_t * tiles_h)), dim3(kThreads), kLdsBytes,
+                       st, A1, B1, (int)V, tiles_t, tiles_h, (void*)((uint16_t*)d_hidden + t0 * H), H);
     Operand A2{dst, w.ld_dst, (int)V};
     Operand B2{ht + t0, w.ld_ht, (int)H};
     if (t0 == 0)

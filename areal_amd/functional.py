@@ -700,3 +700,151 @@ def lm_head_logprobs_entropy(
         raise TypeError("fused lm_head expects bf16 hidden states and weights")
     y = labels.to(device=hidden.device, dtype=torch.int64).contiguous()
     return _LmHeadLogprobsEntropy.apply(hidden.contiguous(), weight.contiguous(), y, float(temperature))
+
+
+class _FusedLmHeadPpo(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, hidden, weight, labels, temperature, T_active, prox, adv, mask_eff, behave_w, params, n_valid,
+                grad_scale):
+        lib = N.load()
+        T, H = hidden.shape
+        V = weight.shape[0]
+        dev = hidden.device
+        f32 = dict(dtype=torch.float32, device=dev)
+        logp = torch.empty(T, **f32)
+        entropy = torch.empty(T, **f32)
+        stat_loss = torch.empty(T_active, **f32)
+        ratio = torch.empty(T_active, **f32)
+        flags = torch.empty(T_active, dtype=torch.uint8, device=dev)
+        loss = torch.empty((), **f32)
+        d_hidden = torch.empty_like(hidden)
+        d_weight = torch.empty(V, H, **f32)
+        ws = _lmhead_workspace(T, H, V, dev)
+        with torch.cuda.device(dev):
+            st = _stream(dev)
+            N.check(
+                lib.aa_lmhead_ppo_fused(
+                    _ptr(hidden), _ptr(weight), T, H, V, _ptr(labels), 1.0 / float(temperature), T_active, _ptr(prox),
+                    _ptr(adv), _ptr(mask_eff), _ptr(behave_w), C.byref(params), _ptr(n_valid), _ptr(grad_scale),
+                    _ptr(logp), _ptr(entropy), _ptr(stat_loss), _ptr(ratio), _ptr(flags), _ptr(d_hidden),
+                    _ptr(d_weight), _ptr(_work_words(dev)), _ptr(ws), ws.numel(), st,
+                ),
+                "aa_lmhead_ppo_fused",
+            )
+            N.check(
+                lib.aa_masked_sum(
+                    _ptr(stat_loss), _ptr(mask_eff), T_active, _ptr(n_valid), _ptr(grad_scale), _ptr(loss), st
+                ),
+                "aa_masked_sum",
+            )
+        ctx.save_for_backward(d_hidden, d_weight.to(weight.dtype))
+        ctx.mark_non_differentiable(logp, entropy, stat_loss, ratio, flags)
+        return loss, logp, entropy, stat_loss, ratio, flags
+
+    @staticmethod
+    def backward(ctx, g_loss, *_unused):
+        lib = N.load()
+        d_hidden, d_weight = ctx.saved_tensors
+        dev = d_hidden.device
+        g = _f32(g_loss).reshape(1)
+        with torch.cuda.device(dev):  # both gradients were written with the loss; a factor of 1 is a no-op
+            for t in (d_hidden, d_weight):
+                N.check(lib.aa_scale_inplace(_ptr(t), _DTYPES[t.dtype], t.numel(), _ptr(g), _stream(dev)),
+                        "aa_scale_inplace")
+        return (d_hidden, d_weight) + (None,) * 10
+
+
+def fused_lm_head_ppo_loss(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    proximal_logprobs: torch.Tensor,
+    old_logprobs: torch.Tensor,
+    advantages: torch.Tensor,
+    eps_clip: float,
+    loss_mask: torch.Tensor,
+    eps_clip_higher: float | None = None,
+    c_clip: float | None = None,
+    rejection_sampling: Any | None = None,
+    importance_sampling_level: str = "token",
+    cu_seqlens: torch.Tensor | None = None,
+    temperature: float = 1.0,
+    loss_scale: torch.Tensor | float | None = None,
+) -> tuple[torch.Tensor, dict]:
+    """lm_head + ``gather_logprobs_entropy`` + ``ppo_actor_loss_fn`` (+ backward) for one micro-batch.
+
+    ``hidden`` is ``[T_pad, H]`` (the final hidden states of the batch-padded micro-batch), ``weight`` the ``[V, H]``
+    lm_head, both bf16; the other arguments are those of ``fused_logprobs_ppo_loss``.  Tokens are processed in chunks
+    of at most 16384: a chunk's logits are rounded to bf16 into a workspace, exactly as the reference's lm_head
+    output is, and turned in place into their gradient, so the full ``[T, V]`` logits never exist and nothing is
+    recomputed.  ``loss.backward()`` hands back ``d(hidden)`` and ``d(weight)`` written during the forward pass.
+    With ``importance_sampling_level="sequence"`` the call runs ``lm_head_logprobs_entropy`` and the unfused loss.
+    """
+    if importance_sampling_level not in ("token", "sequence"):
+        raise ValueError(
+            f"Invalid importance_sampling_level: {importance_sampling_level}. Must be 'token' or 'sequence'."
+        )
+    _require_gpu(hidden, "hidden")
+    if hidden.ndim != 2 or weight.ndim != 2 or hidden.shape[1] != weight.shape[1]:
+        raise ValueError(f"expected hidden [T, H] and weight [V, H], got {tuple(hidden.shape)} and {tuple(weight.shape)}")
+    if tuple(labels.shape) != (hidden.shape[0],):
+        raise ValueError(f"labels shape {tuple(labels.shape)} != ({hidden.shape[0]},)")
+    assert hidden.shape[0] > 0, "Input must have at least one token"
+    if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise TypeError("fused lm_head expects bf16 hidden states and weights")
+    T_active = loss_mask.shape[0]
+    if loss_mask.ndim != 1 or T_active > hidden.shape[0]:
+        raise ValueError(f"loss_mask shape {tuple(loss_mask.shape)} does not fit hidden {tuple(hidden.shape)}")
+    for name, t in (("proximal_logprobs", proximal_logprobs), ("old_logprobs", old_logprobs), ("advantages", advantages)):
+        if t.shape != loss_mask.shape:
+            raise ValueError(f"{name} shape {tuple(t.shape)} != loss_mask shape {tuple(loss_mask.shape)}")
+    dev = hidden.device
+    scale_t = None
+    if loss_scale is not None:
+        scale_t = torch.as_tensor(loss_scale, dtype=torch.float32, device=dev).reshape(1)
+    y = labels.to(device=dev, dtype=torch.int64).contiguous()
+
+    if importance_sampling_level == "sequence":
+        logp, entropy = lm_head_logprobs_entropy(hidden, weight, y, temperature)
+        logp, entropy = logp[:T_active], entropy[:T_active]
+        loss, stat = ppo_actor_loss_fn(
+            logp, proximal_logprobs, old_logprobs, advantages, eps_clip, loss_mask, eps_clip_higher, c_clip,
+            rejection_sampling, importance_sampling_level, cu_seqlens,
+        )
+        if scale_t is not None:
+            loss = loss * scale_t.squeeze(0)
+        stat.update(logprobs=logp.detach(), entropy=entropy.detach())
+        return loss, stat
+
+    prox = _f32(proximal_logprobs.detach())
+    old = _f32(old_logprobs.detach())
+    adv = _f32(advantages.detach())
+    m8 = _mask_u8(loss_mask)
+    params = _ppo_params(eps_clip, eps_clip_higher, c_clip, rejection_sampling is not None)
+    w = counts = None
+    mask_eff = m8
+    if rejection_sampling is not None:
+        _validate_rs(rejection_sampling)
+        mask_eff, w, counts = _rejection_sampling_device(prox, old, m8, loss_mask.shape, cu_seqlens, rejection_sampling)
+        if rejection_sampling.action != "mask":
+            mask_eff = m8
+        n_valid = counts
+    else:
+        n_valid = _count_nonzero(m8)
+    loss, logp, entropy, stat_loss, ratio, flags = _FusedLmHeadPpo.apply(
+        hidden.contiguous(), weight.contiguous(), y, float(temperature), T_active, prox, adv, mask_eff, w, params,
+        n_valid, scale_t,
+    )
+    logp_a = logp[:T_active]
+    stat = dict(
+        loss=stat_loss,
+        importance_weight=ratio,
+        approx_kl=logp_a - prox,
+        clip_mask=(flags & 1).bool(),
+        dual_clip_mask=(flags & 2).bool(),
+        logprobs=logp_a,
+        entropy=entropy[:T_active],
+    )
+    if rejection_sampling is not None:
+        _rs_stats(stat, prox, old, mask_eff, w, counts, loss_mask.shape)
+    return loss, stat

@@ -9,10 +9,10 @@ One "step" is one pass of the hot path over one synthetic packed micro-batch tha
   rejection sampling (importance-weight cap) -> fused log-prob / entropy / clipped PPO loss / d(logits) -> scalar
   loss, i.e. ``fused_logprobs_ppo_loss(...)`` followed by ``loss.backward()``.  Roofline: HBM, algorithmic bytes
   4 * V per token (the bf16 logits read once, their gradient written once).
-* fused lm_head workloads (cfg2, cfg3, cfg4): ``lm_head_logprobs_entropy(hidden, W, labels)`` ->
-  ``ppo_actor_loss_fn`` -> ``loss.backward()`` down to d(hidden) and d(W), logits never materialised.  Roofline:
-  bf16 MFMA, algorithmic flops 6 * T * V * H (forward 2TVH, backward 4TVH; the backward's recompute of the logits
-  tiles is overhead and is not counted).
+* fused lm_head workloads (cfg2, cfg3, cfg4): ``fused_lm_head_ppo_loss(hidden, W, labels, ...)`` followed by
+  ``loss.backward()``: lm_head, log-prob / entropy, PPO loss and the gradients d(hidden), d(W), token chunk by
+  token chunk, the full [T, V] logits never in memory.  Roofline: bf16 MFMA, algorithmic flops 6 * T * V * H
+  (logits 2TVH, the two gradient GEMMs 4TVH).
 
 Prints ONE JSON line.  Besides the whole-step throughput it carries
   roofline      of the dominant kernel(s), timed with HIP events on the launch stream;
@@ -297,17 +297,59 @@ def run_fused_steps(case, n, kw, cfg):
     for _ in range(n):
         h.grad = None
         w.grad = None
-        lp, _ent = areal_amd.lm_head_logprobs_entropy(h, w, case.labels, case.temperature)
-        loss, _ = areal_amd.ppo_actor_loss_fn(
-            lp, case.prox_logp, case.old_logp, case.advantages, loss_mask=case.loss_mask, rejection_sampling=cfg,
-            cu_seqlens=case.cu_seqlens, **kw,
+        loss, _ = areal_amd.fused_lm_head_ppo_loss(
+            h, w, case.labels, case.prox_logp, case.old_logp, case.advantages, loss_mask=case.loss_mask,
+            rejection_sampling=cfg, cu_seqlens=case.cu_seqlens, temperature=case.temperature, **kw,
         )
         loss.backward()
     return loss
 
 
-def time_lmhead_kernels(case, iters: int):
-    """Durations of aa_lmhead_fwd and aa_lmhead_bwd (all the kernels each enqueues), HIP events on the launch stream."""
+def time_lmhead_step(case, kw, cfg, iters: int):
+    """Duration of aa_lmhead_ppo_fused (every kernel it enqueues), HIP events on the launch stream."""
+    import torch
+
+    from areal_amd import _native as N
+    from areal_amd import functional as F
+
+    lib = N.load()
+    dev = case.hidden.device
+    T, H = case.hidden.shape
+    V = case.weight.shape[0]
+    f32 = dict(dtype=torch.float32, device=dev)
+    m8 = F._mask_u8(case.loss_mask)
+    prox, old, adv = (F._f32(t) for t in (case.prox_logp, case.old_logp, case.advantages))
+    params = F._ppo_params(kw["eps_clip"], kw.get("eps_clip_higher"), kw.get("c_clip"), cfg is not None)
+    if cfg is not None:
+        mask_eff, w, counts = F._rejection_sampling_device(prox, old, m8, m8.shape, case.cu_seqlens, cfg)
+        if cfg.action != "mask":
+            mask_eff = m8
+    else:
+        mask_eff, w, counts = m8, None, F._count_nonzero(m8)
+    logp, ent, sl, ratio = (torch.empty(T, **f32) for _ in range(4))
+    flags = torch.empty(T, dtype=torch.uint8, device=dev)
+    dh = torch.empty_like(case.hidden)
+    dw = torch.empty(V, H, **f32)
+    ws = F._lmhead_workspace(T, H, V, dev)
+    stream = torch.cuda.current_stream(dev)
+
+    def launch():
+        N.check(
+            lib.aa_lmhead_ppo_fused(
+                F._ptr(case.hidden), F._ptr(case.weight), T, H, V, F._ptr(case.labels), 1.0 / case.temperature, T,
+                F._ptr(prox), F._ptr(adv), F._ptr(mask_eff), F._ptr(w), C.byref(params), F._ptr(counts), None,
+                F._ptr(logp), F._ptr(ent), F._ptr(sl), F._ptr(ratio), F._ptr(flags), F._ptr(dh), F._ptr(dw),
+                F._ptr(F._work_words(dev)), F._ptr(ws), ws.numel(), C.c_void_p(stream.cuda_stream),
+            ),
+            "aa_lmhead_ppo_fused",
+        )
+
+    return time_events(launch, iters, stream)
+
+
+def time_lmhead_op(case, iters: int):
+    """Durations of aa_lmhead_fwd and aa_lmhead_bwd, the stand-alone differentiable op (its backward recomputes the
+    logits tiles), HIP events on the launch stream."""
     import torch
 
     from areal_amd import _native as N
@@ -362,7 +404,8 @@ def fused_cpu_baseline_and_parity(case, kw, cfg, n_tokens: int, iters: int):
     def oracle_step():
         h = hid.clone().requires_grad_(True)
         w = w_cpu.clone().requires_grad_(True)
-        lp, _ent = oracle.logprobs_entropy(h @ w.t(), lab, case.temperature)
+        logits = (h @ w.t()).to(torch.bfloat16)  # the lm_head output dtype of the reference
+        lp, _ent = oracle.logprobs_entropy(logits, lab, case.temperature)
         loss, _stat = oracle.ppo_actor_loss(lp, prox, old, adv, loss_mask=mask.bool(), rejection_sampling_cfg=cfg,
                                             cu_seqlens=cu, **kw)
         loss.backward()
@@ -376,10 +419,11 @@ def fused_cpu_baseline_and_parity(case, kw, cfg, n_tokens: int, iters: int):
 
     h = case.hidden[sl].detach().clone().requires_grad_(True)
     w = case.weight.detach().clone().requires_grad_(True)
-    lp, _ent = areal_amd.lm_head_logprobs_entropy(h, w, case.labels[sl], case.temperature)
-    loss, _stat = areal_amd.ppo_actor_loss_fn(lp, case.prox_logp[sl], case.old_logp[sl], case.advantages[sl],
-                                              loss_mask=case.loss_mask[sl], rejection_sampling=cfg,
-                                              cu_seqlens=cu.to(h.device), **kw)
+    loss, stat = areal_amd.fused_lm_head_ppo_loss(
+        h, w, case.labels[sl], case.prox_logp[sl], case.old_logp[sl], case.advantages[sl],
+        loss_mask=case.loss_mask[sl], rejection_sampling=cfg, cu_seqlens=cu.to(h.device),
+        temperature=case.temperature, **kw)
+    lp = stat["logprobs"]
     loss.backward()
     torch.cuda.synchronize()
     parity = dict(
@@ -392,8 +436,8 @@ def fused_cpu_baseline_and_parity(case, kw, cfg, n_tokens: int, iters: int):
     baseline = dict(
         value=n / dt, unit="tokens/s", cores=threads, kind="port",
         sample=f"first {n} tokens of the workload against the full weight matrix, {iters} timed fwd+bwd passes of the "
-               f"PyTorch CPU oracle (fp32 hidden @ W.T, log_softmax + gather + entropy, PPO loss, autograd to "
-               f"d(hidden) and d(W))",
+               f"PyTorch CPU oracle (fp32 hidden @ W.T rounded to bf16, log_softmax + gather + entropy, PPO loss, "
+               f"autograd to d(hidden) and d(W))",
     )
     return baseline, parity
 
@@ -419,15 +463,17 @@ def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: i
     case.hidden.requires_grad_(False)
     case.weight.requires_grad_(False)
 
-    f_ms, b_ms = time_lmhead_kernels(case, max(min(steps, 10), 3))
+    k_ms, k_min_ms = time_lmhead_step(case, kw, cfg, max(min(steps, 10), 3))
+    f_ms, b_ms = time_lmhead_op(case, 3)
     alg_flops = 6.0 * T * V * H
-    achieved = alg_flops / ((f_ms + b_ms) * 1e-3) / 1e12
+    achieved = alg_flops / (k_ms * 1e-3) / 1e12
     roofline = dict(
-        bound="mfma", kernel="aa_lmhead_fwd + aa_lmhead_bwd (k_lmhead_stats, k_lmhead_ds, k_gemm_store x 2)",
+        bound="mfma", kernel="aa_lmhead_ppo_fused (k_gemm_store x 3, k_fused_regs, k_transpose_bf16 per token chunk)",
         achieved=achieved, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s", frac=achieved / MFMA_BF16_PEAK_TFLOPS,
-        traffic=None, fwd_ms=f_ms, bwd_ms=b_ms,
-        fwd_tflops=2.0 * T * V * H / (f_ms * 1e-3) / 1e12, bwd_tflops=4.0 * T * V * H / (b_ms * 1e-3) / 1e12,
-        algorithmic_flops_per_step=alg_flops, executed_flops_per_step=8.0 * T * V * H,
+        traffic=None, avg_call_ms=k_ms, min_call_ms=k_min_ms, algorithmic_flops_per_step=alg_flops,
+        # the stand-alone differentiable op lm_head_logprobs_entropy, whose backward recomputes the logits tiles
+        standalone_op=dict(fwd_ms=f_ms, bwd_ms=b_ms, fwd_tflops=2.0 * T * V * H / (f_ms * 1e-3) / 1e12,
+                           bwd_tflops=4.0 * T * V * H / (b_ms * 1e-3) / 1e12),
     )
     out = dict(
         metric=METRIC, value=T / (ms_per_step * 1e-3), unit="tokens/s",
@@ -435,7 +481,7 @@ def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: i
         scaling="weak", vs_baseline=None, dtype="bf16", data="synthetic",
         config=dict(workload=f"{case.name}: {desc}", tokens=T, hidden=H, vocab=V,
                     sequences=int(case.cu_seqlens.numel() - 1), accumulate="f32",
-                    path="fused lm_head (logits never materialised) + PPO loss, fwd + bwd"),
+                    path="lm_head + PPO loss step in token chunks (at most one chunk of logits in memory), fwd + bwd"),
         roofline=roofline,
     )
     if cpu_tokens > 0:

@@ -217,6 +217,34 @@ int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, int64_t H,
                   float* d_weight, void* workspace, int64_t workspace_bytes,
                   void* stream);
 
+/*
+ * Whole training step of the lm_head + PPO actor loss for one micro-batch,
+ * token-level importance sampling: what the reference runs as lm_head matmul
+ * (bf16 logits) -> gather_logprobs_entropy (vocab_parallel.py:434-469) ->
+ * ppo_actor_loss_fn (functional.py:429-559) -> autograd back to the hidden
+ * states and the lm_head weight.  Tokens are processed in chunks of at most
+ * 16384: the chunk's logits are formed on the matrix cores and rounded to
+ * bf16 into the workspace (as the reference's lm_head output is), one
+ * streaming pass turns them in place into d(loss)/d(logits) while emitting
+ * the per-token outputs (the kernel of aa_logits_ppo_fused), and two GEMMs
+ * accumulate the gradients.  No recompute: 6 T V H flops in all, and never
+ * more than one chunk of logits in memory.
+ *
+ * Per-token arguments, params, n_valid, grad_scale, work: as in
+ * aa_logits_ppo_fused.  d_hidden [T, H] bf16 and d_weight [V, H] fp32 are
+ * overwritten.  workspace: aa_lmhead_workspace_bytes(T, H, V) bytes.
+ */
+int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64_t T,
+                        int64_t H, int64_t V, const int64_t* labels,
+                        float inv_temperature, int64_t T_active,
+                        const float* prox_logp, const float* adv,
+                        const uint8_t* mask_eff, const float* behave_w,
+                        const aa_ppo_params* params, const int32_t* n_valid,
+                        const float* grad_scale, float* logp, float* entropy,
+                        float* stat_loss, float* ratio, uint8_t* flags,
+                        void* d_hidden, float* d_weight, int32_t* work,
+                        void* workspace, int64_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------ */
 /* Measurement helper                                                  */
 /* ------------------------------------------------------------------ */

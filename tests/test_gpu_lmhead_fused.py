@@ -1,0 +1,146 @@
+"""GPU parity of the whole lm_head + PPO-loss training step (``fused_lm_head_ppo_loss``).
+
+Oracle: the reference pipeline on materialised logits -- lm_head matmul with the output rounded to bf16, chunked
+log-softmax / gather / entropy, ``ppo_actor_loss_fn`` with rejection sampling, autograd back to the hidden states and
+the lm_head weight."""
+import pytest
+import torch
+
+import areal_amd
+import oracle
+from areal_amd import RejectionSamplingConfig
+from helpers import cosine
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(T_pad, T, H, V, seed, w_std=0.3):
+    g = torch.Generator().manual_seed(seed)
+    hidden = torch.randn(T_pad, H, generator=g).bfloat16()
+    weight = (w_std * torch.randn(V, H, generator=g)).bfloat16()
+    labels = torch.randint(0, V, (T_pad,), generator=g)
+    logits = (hidden.float() @ weight.float().t()).bfloat16()
+    ref_lp = oracle.logprobs(logits, labels)[:T]
+    prox = ref_lp + 0.05 * torch.randn(T, generator=g)
+    old = ref_lp + 0.3 * torch.randn(T, generator=g)
+    adv = torch.randn(T, generator=g)
+    mask = torch.rand(T, generator=g) < 0.7
+    return hidden, weight, labels, prox, old, adv, mask
+
+
+def _oracle_step(hidden, weight, labels, prox, old, adv, mask, temperature, loss_scale, **kw):
+    h = hidden.float().requires_grad_(True)
+    w = weight.float().requires_grad_(True)
+    logits = (h @ w.t()).to(torch.bfloat16)                                   # the lm_head output dtype
+    lp, ent = oracle.logprobs_entropy(logits, labels, temperature)
+    n = mask.shape[0]
+    loss, stat = oracle.ppo_actor_loss(lp[:n], prox, old, adv, loss_mask=mask, **kw)
+    (loss * loss_scale).backward()
+    return float(loss.detach()) * loss_scale, stat, lp.detach(), ent.detach(), h.grad, w.grad
+
+
+CASES = [
+    # T_pad, T, H, V, temperature, loss_scale, options
+    (300, 300, 128, 1088, 1.0, 1.0, dict(eps_clip=0.2)),                                    # row kernel for any V
+    (520, 500, 64, 8256, 0.8, 0.37, dict(eps_clip=0.2, eps_clip_higher=0.28, c_clip=3.0)),  # register-resident kernel
+    (16384 + 200, 16384 + 130, 64, 640, 1.0, 1.0, dict(eps_clip=0.2, rs=True)),             # two token chunks
+]
+
+
+@pytest.mark.parametrize("T_pad,T,H,V,temperature,loss_scale,opts", CASES)
+def test_step_matches_reference_pipeline(device, T_pad, T, H, V, temperature, loss_scale, opts):
+    opts = dict(opts)
+    rs = RejectionSamplingConfig(level="token", action="mask", metric="ratio", upper=1.3) if opts.pop("rs", False) else None
+    hidden, weight, labels, prox, old, adv, mask = _inputs(T_pad, T, H, V, seed=T + V)
+    cu = torch.tensor([0, T], dtype=torch.int32)
+    h_d = hidden.to(device).requires_grad_(True)
+    w_d = weight.to(device).requires_grad_(True)
+    loss, stat = areal_amd.fused_lm_head_ppo_loss(
+        h_d, w_d, labels.to(device), prox.to(device), old.to(device), adv.to(device), loss_mask=mask.to(device),
+        rejection_sampling=rs, cu_seqlens=cu.to(device), temperature=temperature, loss_scale=loss_scale, **opts)
+    loss.backward()
+    o_loss, o_stat, o_lp, o_ent, o_dh, o_dw = _oracle_step(
+        hidden, weight, labels, prox, old, adv, mask, temperature, loss_scale, rejection_sampling_cfg=rs,
+        cu_seqlens=cu, **opts)
+    assert float(loss.detach()) == pytest.approx(o_loss, rel=1e-3, abs=1e-7)
+    assert float((stat["logprobs"].cpu() - o_lp[:T]).abs().max()) < 2e-3
+    assert float((stat["entropy"].cpu() - o_ent[:T]).abs().max()) < 2e-3
+    assert torch.equal(stat["clip_mask"].cpu(), o_stat["clip_mask"])
+    assert torch.equal(stat["dual_clip_mask"].cpu(), o_stat["dual_clip_mask"])
+    assert cosine(h_d.grad.cpu().float(), o_dh) > 0.9999
+    assert cosine(w_d.grad.cpu().float(), o_dw) > 0.9999
+    assert float(h_d.grad[T:].abs().sum()) == 0.0  # batch padding gets no gradient
+    if rs is not None:
+        assert float(stat["filtered_fraction"]) == pytest.approx(float(o_stat["filtered_fraction"]), abs=1e-6)
+
+
+def test_upstream_gradient_scales_both_gradients(device):
+    hidden, weight, labels, prox, old, adv, mask = _inputs(260, 260, 64, 704, seed=3)
+    args = [t.to(device) for t in (labels, prox, old, adv)]
+
+    def grads(factor):
+        h = hidden.to(device).requires_grad_(True)
+        w = weight.to(device).requires_grad_(True)
+        loss, _ = areal_amd.fused_lm_head_ppo_loss(h, w, *args, eps_clip=0.2, loss_mask=mask.to(device))
+        (loss * factor).backward()
+        return h.grad.float(), w.grad.float()
+
+    h1, w1 = grads(1.0)
+    h2, w2 = grads(-2.0)
+    assert torch.allclose(h2, -2.0 * h1, rtol=1e-2, atol=1e-12) and torch.allclose(w2, -2.0 * w1, rtol=1e-2, atol=1e-12)
+
+
+def test_sequence_level_runs_the_unfused_kernels(device):
+    hidden, weight, labels, prox, old, adv, mask = _inputs(300, 300, 64, 704, seed=5)
+    cu = torch.tensor([0, 100, 180, 300], dtype=torch.int32)
+    h_d = hidden.to(device).requires_grad_(True)
+    w_d = weight.to(device).requires_grad_(True)
+    loss, stat = areal_amd.fused_lm_head_ppo_loss(
+        h_d, w_d, labels.to(device), prox.to(device), old.to(device), adv.to(device), eps_clip=0.2,
+        loss_mask=mask.to(device), importance_sampling_level="sequence", cu_seqlens=cu.to(device))
+    loss.backward()
+    h = hidden.float().requires_grad_(True)
+    w = weight.float().requires_grad_(True)
+    lp, _ = oracle.logprobs_entropy(h @ w.t(), labels)
+    o_loss, _ = oracle.ppo_actor_loss(lp, prox, old, adv, 0.2, mask, importance_sampling_level="sequence", cu_seqlens=cu)
+    o_loss.backward()
+    assert float(loss.detach()) == pytest.approx(float(o_loss), rel=1e-3, abs=1e-7)
+    assert cosine(h_d.grad.cpu().float(), h.grad) > 0.9999 and cosine(w_d.grad.cpu().float(), w.grad) > 0.9999
+    with pytest.raises(ValueError, match="Invalid importance_sampling_level"):
+        areal_amd.fused_lm_head_ppo_loss(h_d, w_d, labels.to(device), prox.to(device), old.to(device), adv.to(device),
+                                         eps_clip=0.2, loss_mask=mask.to(device), importance_sampling_level="bad")
+
+
+def test_full_size_step_agrees_with_unfused_path(device):
+    """8B shape: the chunked step against lm_head_logprobs_entropy -> ppo_actor_loss_fn -> autograd (which the slice
+    tests tie to the oracle); also bit-identical when repeated."""
+    from areal_amd import synth
+
+    case = synth.config2(device, seed=0)
+    with torch.no_grad():
+        ref, _ = areal_amd.lm_head_logprobs_entropy(case.hidden, case.weight, case.labels)
+    synth.attach_old_and_prox(case, ref, 0.05, 9)
+
+    def fused():
+        h = case.hidden.detach().requires_grad_(True)
+        w = case.weight.detach().requires_grad_(True)
+        loss, stat = areal_amd.fused_lm_head_ppo_loss(h, w, case.labels, case.prox_logp, case.old_logp,
+                                                      case.advantages, eps_clip=0.2, loss_mask=case.loss_mask)
+        loss.backward()
+        return loss.detach(), stat, h.grad, w.grad
+
+    l1, s1, dh1, dw1 = fused()
+    l2, s2, dh2, dw2 = fused()
+    assert torch.equal(l1, l2) and torch.equal(dh1, dh2) and torch.equal(dw1, dw2)
+    h = case.hidden.detach().requires_grad_(True)
+    w = case.weight.detach().requires_grad_(True)
+    lp, ent = areal_amd.lm_head_logprobs_entropy(h, w, case.labels)
+    loss, stat = areal_amd.ppo_actor_loss_fn(lp, case.prox_logp, case.old_logp, case.advantages, 0.2, case.loss_mask)
+    loss.backward()
+    assert float(l1) == pytest.approx(float(loss.detach()), rel=1e-3)
+    # the chunked step rounds logits to bf16 as the reference does, the recomputing path keeps fp32 tiles
+    assert float((s1["logprobs"] - lp.detach()).abs().max()) < 0.02
+    a, b = dh1.double().reshape(-1), h.grad.double().reshape(-1)
+    assert float(a @ b / (a.norm() * b.norm())) > 0.9999
+    a, b = dw1.double().reshape(-1), w.grad.double().reshape(-1)
+    assert float(a @ b / (a.norm() * b.norm())) > 0.9999
