@@ -393,7 +393,9 @@ def fused_cpu_baseline_and_parity(case, kw, cfg, n_tokens: int, iters: int):
     import oracle
 
     n = min(n_tokens, case.n_tokens)
-    sl = slice(0, n)
+    first = int(torch.nonzero(case.loss_mask)[0]) if bool(case.loss_mask.any()) else 0
+    start = max(0, min(first - n // 4, case.n_tokens - n))  # a window that holds masked and unmasked tokens
+    sl = slice(start, start + n)
     cpu = lambda t: t[sl].cpu()
     hid, lab = cpu(case.hidden).float(), cpu(case.labels)
     w_cpu = case.weight.cpu().float()
@@ -427,7 +429,7 @@ def fused_cpu_baseline_and_parity(case, kw, cfg, n_tokens: int, iters: int):
     loss.backward()
     torch.cuda.synchronize()
     parity = dict(
-        tokens=n,
+        tokens=n, first_token=start,
         logp_max_abs_err=float((lp.detach().cpu() - w_lp).abs().max()),
         loss_rel_err=abs(float(loss.detach()) - float(w_loss)) / max(abs(float(w_loss)), 1e-12),
         d_hidden_cosine=cosine(h.grad.cpu(), w_dh),
@@ -435,7 +437,7 @@ def fused_cpu_baseline_and_parity(case, kw, cfg, n_tokens: int, iters: int):
     )
     baseline = dict(
         value=n / dt, unit="tokens/s", cores=threads, kind="port",
-        sample=f"first {n} tokens of the workload against the full weight matrix, {iters} timed fwd+bwd passes of the "
+        sample=f"tokens {start}..{start + n - 1} of the workload against the full weight matrix, {iters} timed fwd+bwd passes of the "
                f"PyTorch CPU oracle (fp32 hidden @ W.T rounded to bf16, log_softmax + gather + entropy, PPO loss, "
                f"autograd to d(hidden) and d(W))",
     )

@@ -172,7 +172,7 @@ def test_engine_contract_roll_pad_and_scale(device):
             x, {"input_ids": input_ids.to(device)}, mb_d, pad, total_w, eps_clip=0.2, fused=fused
         )
         loss.backward()
-        results.append((float(loss), x.grad.clone(), stat))
+        results.append((float(loss.detach()), x.grad.clone(), stat))
     w_loss, _, w_grad = oracle.logits_ppo_step(
         logits, labels.cpu(), mb["prox_logp"], mb["logprobs"], mb["advantages"], 0.2, mb["loss_mask"],
         loss_scale=float(mb["loss_mask"].sum()) / 40.0,
