@@ -27,6 +27,10 @@ HIPCC_FLAGS = [
 ]
 
 
+# hipBLASLt serves the plain GEMMs of the lm_head path
+LINK_LIBS = ["-L/opt/rocm/lib", "-lhipblaslt"]
+
+
 def _hipcc() -> str:
     for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
         if cand and (os.path.isabs(cand) and os.path.exists(cand) or not os.path.isabs(cand)):
@@ -61,7 +65,7 @@ def build_library(verbose: bool = True, jobs: int = 4) -> Path:
     with ThreadPoolExecutor(max_workers=max(1, jobs)) as pool:
         list(pool.map(compile_one, zip(srcs, objs)))
     tmp = LIB_PATH.with_suffix(".so.tmp")
-    _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)])
+    _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs), *LINK_LIBS])
     os.replace(tmp, LIB_PATH)
     if verbose:
         print(f"[areal_amd.build] wrote {LIB_PATH}", flush=True)

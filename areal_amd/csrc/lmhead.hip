@@ -1,15 +1,20 @@
-// Fused lm_head path for gfx950: log-prob / entropy of softmax(hidden @ weight.T / T) and its backward without ever
-// holding the [T, V] logits in memory.  The reference has no such path: its equivalent is the lm_head matmul
-// followed by gather_logprobs_entropy (areal/utils/functional/vocab_parallel.py:23-29) and autograd.
+// lm_head path for gfx950: log-prob / entropy of softmax(hidden @ weight.T / T), their backward, and the whole
+// lm_head + PPO-loss training step, without ever holding the [T, V] logits in memory.  The reference has no such
+// path: its equivalent is the lm_head matmul followed by gather_logprobs_entropy
+// (areal/utils/functional/vocab_parallel.py:23-29), ppo_actor_loss_fn and autograd.
 //
-// Forward: a bf16 MFMA tile GEMM (gemm_tn.h) forms 256 (vocabulary) x 256 (tokens) tiles of the logits in
-// accumulator registers; its epilogue reduces each tile to the softmax partials (k, s, u) per token and captures
-// the label logit; a second small kernel merges the partials of all vocabulary tiles.
+// Stand-alone op, forward: a bf16 MFMA tile GEMM (gemm_tn.h) forms 256 (vocabulary) x 256 (tokens) tiles of the
+// logits in accumulator registers; its epilogue reduces each tile to the softmax partials (k, s, u) per token and
+// captures the label logit; a second small kernel merges the partials of all vocabulary tiles.
 //
-// Backward: the logits tile is formed again, turned into d(logits) in registers (bf16), and written to a reusable
-// panel of one token chunk in both orientations; two more tile GEMMs contract the panel with the weights
-// (d_hidden) and with the hidden states (d_weight, fp32).
+// Stand-alone op, backward: the logits tile is formed again, turned into d(logits) in registers (bf16) and written
+// to a reusable panel [token chunk, V]; the two plain GEMMs that contract the panel with the weights (d_hidden)
+// and with the hidden states (d_weight, fp32) go to hipBLASLt (lt_gemm.h).
+//
+// Training step (aa_lmhead_ppo_fused): per token chunk, a library GEMM writes the bf16 logits panel, the fused
+// row kernel of the logits path turns it in place into d(loss)/d(logits), and the same two library GEMMs follow.
 #include "gemm_tn.h"
+#include "lt_gemm.h"
 
 namespace aa {
 namespace lmhead {
@@ -133,7 +138,7 @@ __global__ __launch_bounds__(256) void k_lmhead_combine(const float4* __restrict
   if (row_ez) row_ez[t] = (k + mean_t) * kLn2;
 }
 
-// ---- backward epilogue: d(logits) of a tile, written as panel [tokens, V] and [V, tokens] -----------------------
+// ---- backward epilogue: d(logits) of a tile, written into the panel [tokens, V] -------------------------------------
 struct DsArgs {
   const float* row_lse;   // [T] natural log
   const float* row_ez;    // [T] (nullable when g_entropy is null)
@@ -141,8 +146,6 @@ struct DsArgs {
   const float* g_entropy; // [T] nullable
   const int64_t* labels;  // [T]
   uint16_t* ds;           // [chunk tokens, V] bf16, ld = V
-  uint16_t* dst;          // [V, ld_t] bf16
-  int64_t ld_t;
   int64_t t0;             // first token of the chunk (hidden operand is already offset)
   float inv_t;
 };
@@ -221,98 +224,12 @@ __global__ __launch_bounds__(kThreads) void k_lmhead_ds(Operand W, Operand Hd, i
       *(u32x4_t*)(a.ds + (int64_t)n * V + m) = v;  // V % 8 == 0: a piece never straddles the end
     }
   }
-  // panel [vocab][token]: gather 8 tokens of one vocabulary row
-  for (int p = tid; p < 256 * 32; p += kThreads) {
-    const int mloc = p >> 5, nc = (p & 31) * 8;
-    const int m = m0 + mloc;
-    if (m < V) {
-      uint32_t w[4];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const uint32_t lo = Z[(nc + 2 * q) * PZ + mloc], hi = Z[(nc + 2 * q + 1) * PZ + mloc];
-        w[q] = lo | (hi << 16);
-      }
-      u32x4_t v = {w[0], w[1], w[2], w[3]};
-      *(u32x4_t*)(a.dst + (int64_t)m * a.ld_t + n0 + nc) = v;  // columns >= N hold zeros (live == false)
-    }
-  }
-}
-
-// ---- plain tile GEMM with a store epilogue: C[m][n] (row-major, ldc) = or += A B^T ---------------------------------
-template <bool OUT_F32, bool ACCUM>
-__global__ __launch_bounds__(kThreads) void k_gemm_store(Operand A, Operand B, int K, int tiles_m, int tiles_n,
-                                                         void* __restrict__ C, int64_t ldc) {
-  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
-  int tm, tn;
-  tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
-  const int m0 = tm * BM, n0 = tn * BN;
-  Acc acc;
-  mainloop(A, B, K, m0, n0, acc, lds);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-#pragma unroll
-  for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt) {
-      const int n = n0 + wn * 128 + acc_col(nt, lane);
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int m = m0 + wm * 128 + acc_row(mt, i, lane);
-        if (m < A.rows && n < B.rows) {
-          const int64_t off = (int64_t)m * ldc + n;
-          if (OUT_F32) {
-            float* p = (float*)C + off;
-            *p = ACCUM ? (*p + acc.v[mt][nt][i]) : acc.v[mt][nt][i];
-          } else {
-            ((uint16_t*)C)[off] = (uint16_t)(Elem<AA_BF16>::pack(acc.v[mt][nt][i], 0.f) & 0xffffu);
-          }
-        }
-      }
-    }
-}
-
-// ---- bf16 transpose with zero padding: dst[c][r] = src[r][c], dst is [C, ld_dst], columns >= R are zeroed --------
-// 64 x 64 tiles, 16-byte global loads and stores; the tile is turned in LDS (pitch 33 words, so the eight 2-byte reads
-// that gather one output chunk fall in different banks).  Needs Cc, ld_src, ld_dst multiples of 8 and 16-byte bases.
-__global__ __launch_bounds__(256) void k_transpose_bf16(const uint16_t* __restrict__ src, int64_t R, int64_t Cc,
-                                                        int64_t ld_src, uint16_t* __restrict__ dst, int64_t ld_dst) {
-  __shared__ uint32_t tile[64 * 33];
-  const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
-#pragma unroll
-  for (int s = 0; s < 2; ++s) {
-    const int p = threadIdx.x + 256 * s;
-    const int r = p >> 3, ch = p & 7;
-    const int64_t rr = r0 + r, cg = c0 + ch * 8;
-    uint4 v = make_uint4(0u, 0u, 0u, 0u);
-    if (rr < R && cg < Cc) v = *(const uint4*)(src + rr * ld_src + cg);
-    uint32_t* t = tile + r * 33 + ch * 4;
-    t[0] = v.x; t[1] = v.y; t[2] = v.z; t[3] = v.w;
-  }
-  __syncthreads();
-  const uint16_t* t16 = (const uint16_t*)tile;
-#pragma unroll
-  for (int s = 0; s < 2; ++s) {
-    const int p = threadIdx.x + 256 * s;
-    const int c = p >> 3, j = p & 7;
-    const int64_t cg = c0 + c, rg = r0 + j * 8;
-    if (cg < Cc && rg < ld_dst) {
-      uint32_t w[4];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const uint32_t lo = t16[(j * 8 + 2 * q) * 66 + c], hi = t16[(j * 8 + 2 * q + 1) * 66 + c];
-        w[q] = lo | (hi << 16);
-      }
-      *(uint4*)(dst + cg * ld_dst + rg) = make_uint4(w[0], w[1], w[2], w[3]);
-    }
-  }
 }
 
 struct Workspace {
-  // forward
-  int64_t off_part, off_xy;
-  // backward
-  int64_t off_wt, off_ht, off_ds, off_dst;
-  int64_t ld_ht, ld_dst, chunk;
+  int64_t off_part, off_xy;  // forward: per-tile partials, label logits
+  int64_t off_ds, off_lt;    // backward / step: the [chunk, V] panel, scratch of the GEMM library
+  int64_t chunk;
   int64_t bytes;
 };
 
@@ -326,13 +243,10 @@ static Workspace plan(int64_t T, int64_t H, int64_t V) {
   const int64_t fwd_bytes = off;
   off = 0;
   w.chunk = T < kChunkTokens ? (T + 255) / 256 * 256 : kChunkTokens;
-  w.ld_ht = (T + 255) / 256 * 256;
-  w.ld_dst = w.chunk;
-  w.off_wt = off;  off += up(H * V * 2);
-  w.off_ht = off;  off += up(H * w.ld_ht * 2);
   w.off_ds = off;  off += up(w.chunk * V * 2);
-  w.off_dst = off; off += up(V * w.ld_dst * 2);
+  w.off_lt = off;  off += lt::kWorkspaceBytes;
   w.bytes = off > fwd_bytes ? off : fwd_bytes;
+  (void)H;
   return w;
 }
 
@@ -394,45 +308,30 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
     return AA_ERR_INVALID_ARGUMENT;
   const Workspace w = plan(T, H, V);
   if (workspace_bytes < w.bytes) return AA_ERR_INVALID_ARGUMENT;
-  static const bool ok = allow_big_lds(k_lmhead_ds, kLdsBytesDs) && allow_big_lds(k_gemm_store<false, false>) &&
-                         allow_big_lds(k_gemm_store<true, false>) && allow_big_lds(k_gemm_store<true, true>);
+  static const bool ok = allow_big_lds(k_lmhead_ds, kLdsBytesDs);
   if (!ok) return AA_ERR_LAUNCH;
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
-  uint16_t* wt = (uint16_t*)(ws + w.off_wt);    // [H, V]
-  uint16_t* ht = (uint16_t*)(ws + w.off_ht);    // [H, ld_ht]
-  uint16_t* ds = (uint16_t*)(ws + w.off_ds);    // [chunk, V]
-  uint16_t* dst = (uint16_t*)(ws + w.off_dst);  // [V, ld_dst]
-  // K-contiguous copies of the operands of the two gradient GEMMs
-  hipLaunchKernelGGL(k_transpose_bf16, dim3((unsigned)((H + 63) / 64), (unsigned)((V + 63) / 64)), dim3(256), 0, st,
-                     (const uint16_t*)weight, V, H, H, wt, V);
-  hipLaunchKernelGGL(k_transpose_bf16, dim3((unsigned)((H + 63) / 64), (unsigned)((w.ld_ht + 63) / 64)), dim3(256), 0,
-                     st, (const uint16_t*)hidden, T, H, H, ht, w.ld_ht);
+  uint16_t* ds = (uint16_t*)(ws + w.off_ds);  // [chunk, V]
+  void* lt_ws = ws + w.off_lt;
   const int tiles_v = (int)((V + BM - 1) / BM);
-  const int tiles_h = (int)((H + BN - 1) / BN);
   for (int64_t t0 = 0; t0 < T; t0 += w.chunk) {
     const int64_t n_tok = (T - t0) < w.chunk ? (T - t0) : w.chunk;
-    const int64_t k_tok = (n_tok + 255) / 256 * 256;  // panel width incl. zero columns
-    const int tiles_t = (int)(k_tok / BN);
+    const int tiles_t = (int)((n_tok + BN - 1) / BN);
+    const uint16_t* hid = (const uint16_t*)hidden + t0 * H;
     Operand W{(const uint16_t*)weight, H, (int)V};
-    Operand Hd{(const uint16_t*)hidden + t0 * H, H, (int)n_tok};
-    DsArgs a{row_lse, row_ez, g_logp, g_entropy, labels, ds, dst, w.ld_dst, t0, inv_temperature};
+    Operand Hd{hid, H, (int)n_tok};
+    DsArgs a{row_lse, row_ez, g_logp, g_entropy, labels, ds, t0, inv_temperature};
     hipLaunchKernelGGL(k_lmhead_ds, dim3((unsigned)(tiles_v * tiles_t)), dim3(kThreads), kLdsBytesDs, st, W, Hd, (int)H,
                        tiles_v, tiles_t, a);
-    // d_hidden[t0 : t0 + n_tok, :] = dS [n_tok, V] . Wt [H, V]^T
-    Operand A1{ds, V, (int)n_tok};
-    Operand B1{wt, V, (int)H};
-    hipLaunchKernelGGL((k_gemm_store<false, false>), dim3((unsigned)(tiles_t * tiles_h)), dim3(kThreads), kLdsBytes,
-                       st, A1, B1, (int)V, tiles_t, tiles_h, (void*)((uint16_t*)d_hidden + t0 * H), H);
-    // d_weight [V, H] (+)= dSt [V, k_tok] . Ht[:, t0 : t0 + k_tok]^T
-    Operand A2{dst, w.ld_dst, (int)V};
-    Operand B2{ht + t0, w.ld_ht, (int)H};
-    if (t0 == 0)
-      hipLaunchKernelGGL((k_gemm_store<true, false>), dim3((unsigned)(tiles_v * tiles_h)), dim3(kThreads), kLdsBytes,
-                         st, A2, B2, (int)k_tok, tiles_v, tiles_h, (void*)d_weight, H);
-    else
-      hipLaunchKernelGGL((k_gemm_store<true, true>), dim3((unsigned)(tiles_v * tiles_h)), dim3(kThreads), kLdsBytes,
-                         st, A2, B2, (int)k_tok, tiles_v, tiles_h, (void*)d_weight, H);
+    // d_hidden[t0 : t0 + n_tok, :] = dS . W: column-major [H, n_tok] = W' [H, V] . dS' [V, n_tok]
+    if (!lt::gemm(st, false, false, H, n_tok, V, weight, H, ds, V, (uint16_t*)d_hidden + t0 * H, H, false, 0.f, lt_ws,
+                  lt::kWorkspaceBytes))
+      return AA_ERR_LAUNCH;
+    // d_weight (+)= dS^T . hidden: column-major [H, V] = hidden' [H, n_tok] . dS'^T [n_tok, V], fp32
+    if (!lt::gemm(st, false, true, H, V, n_tok, hid, H, ds, V, d_weight, H, true, t0 == 0 ? 0.f : 1.f, lt_ws,
+                  lt::kWorkspaceBytes))
+      return AA_ERR_LAUNCH;
   }
   return launch_status();
 }
@@ -454,52 +353,33 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
     return AA_ERR_INVALID_ARGUMENT;
   const Workspace w = plan(T, H, V);
   if (workspace_bytes < w.bytes) return AA_ERR_INVALID_ARGUMENT;
-  static const bool ok = allow_big_lds(k_gemm_store<false, false>) && allow_big_lds(k_gemm_store<true, false>) &&
-                         allow_big_lds(k_gemm_store<true, true>);
-  if (!ok) return AA_ERR_LAUNCH;
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
-  uint16_t* wt = (uint16_t*)(ws + w.off_wt);    // [H, V]
-  uint16_t* ht = (uint16_t*)(ws + w.off_ht);    // [H, ld_ht]
-  uint16_t* ds = (uint16_t*)(ws + w.off_ds);    // [chunk, V]: logits of the chunk, then their gradient in place
-  uint16_t* dst = (uint16_t*)(ws + w.off_dst);  // [V, ld_dst]: the gradient panel transposed
-  hipLaunchKernelGGL(k_transpose_bf16, dim3((unsigned)((H + 63) / 64), (unsigned)((V + 63) / 64)), dim3(256), 0, st,
-                     (const uint16_t*)weight, V, H, H, wt, V);
-  hipLaunchKernelGGL(k_transpose_bf16, dim3((unsigned)((H + 63) / 64), (unsigned)((w.ld_ht + 63) / 64)), dim3(256), 0,
-                     st, (const uint16_t*)hidden, T, H, H, ht, w.ld_ht);
-  const int tiles_v = (int)((V + BM - 1) / BM);
-  const int tiles_h = (int)((H + BN - 1) / BN);
+  uint16_t* ds = (uint16_t*)(ws + w.off_ds);  // [chunk, V]: logits of the chunk, then their gradient in place
+  void* lt_ws = ws + w.off_lt;
   for (int64_t t0 = 0; t0 < T; t0 += w.chunk) {
     const int64_t n_tok = (T - t0) < w.chunk ? (T - t0) : w.chunk;
-    const int64_t k_tok = (n_tok + 255) / 256 * 256;
-    const int tiles_t = (int)(k_tok / BM);
     int64_t act = T_active - t0;
     act = act < 0 ? 0 : (act > n_tok ? n_tok : act);
-    // logits[t0 : t0 + n_tok, :] = hidden . W^T, rounded to bf16 as the reference's lm_head output is
-    Operand Hd{(const uint16_t*)hidden + t0 * H, H, (int)n_tok};
-    Operand W{(const uint16_t*)weight, H, (int)V};
-    hipLaunchKernelGGL((k_gemm_store<false, false>), dim3((unsigned)(tiles_t * tiles_v)), dim3(kThreads), kLdsBytes,
-                       st, Hd, W, (int)H, tiles_t, tiles_v, (void*)ds, V);
+    const uint16_t* hid = (const uint16_t*)hidden + t0 * H;
+    // logits[t0 : t0 + n_tok, :] = hidden . W^T, rounded to bf16 as the reference's lm_head output is.
+    // Row-major [n_tok, V] is column-major [V, n_tok]: W'^T [V, H] . hidden' [H, n_tok].
+    if (!lt::gemm(st, true, false, V, n_tok, H, weight, H, hid, H, ds, V, false, 0.f, lt_ws, lt::kWorkspaceBytes))
+      return AA_ERR_LAUNCH;
     // log-prob, entropy, PPO loss and d(loss)/d(logits) in place: one streaming pass over the panel
     const int rc = aa_logits_ppo_fused(ds, AA_BF16, n_tok, V, V, labels + t0, inv_temperature, act, prox_logp + t0,
                                        adv + t0, mask_eff + t0, behave_w ? behave_w + t0 : nullptr, params, n_valid,
                                        grad_scale, logp + t0, entropy ? entropy + t0 : nullptr, nullptr, nullptr,
                                        stat_loss + t0, ratio + t0, flags + t0, ds, work, stream);
     if (rc != AA_OK) return rc;
-    hipLaunchKernelGGL(k_transpose_bf16, dim3((unsigned)((V + 63) / 64), (unsigned)(w.ld_dst / 64)), dim3(256), 0, st,
-                       (const uint16_t*)ds, n_tok, V, V, dst, w.ld_dst);
-    Operand A1{ds, V, (int)n_tok};
-    Operand B1{wt, V, (int)H};
-    hipLaunchKernelGGL((k_gemm_store<false, false>), dim3((unsigned)(tiles_t * tiles_h)), dim3(kThreads), kLdsBytes,
-                       st, A1, B1, (int)V, tiles_t, tiles_h, (void*)((uint16_t*)d_hidden + t0 * H), H);
-    Operand A2{dst, w.ld_dst, (int)V};
-    Operand B2{ht + t0, w.ld_ht, (int)H};
-    if (t0 == 0)
-      hipLaunchKernelGGL((k_gemm_store<true, false>), dim3((unsigned)(tiles_v * tiles_h)), dim3(kThreads), kLdsBytes,
-                         st, A2, B2, (int)k_tok, tiles_v, tiles_h, (void*)d_weight, H);
-    else
-      hipLaunchKernelGGL((k_gemm_store<true, true>), dim3((unsigned)(tiles_v * tiles_h)), dim3(kThreads), kLdsBytes,
-                         st, A2, B2, (int)k_tok, tiles_v, tiles_h, (void*)d_weight, H);
+    // d_hidden[t0 : t0 + n_tok, :] = dS . W: column-major [H, n_tok] = W' [H, V] . dS' [V, n_tok]
+    if (!lt::gemm(st, false, false, H, n_tok, V, weight, H, ds, V, (uint16_t*)d_hidden + t0 * H, H, false, 0.f, lt_ws,
+                  lt::kWorkspaceBytes))
+      return AA_ERR_LAUNCH;
+    // d_weight (+)= dS^T . hidden: column-major [H, V] = hidden' [H, n_tok] . dS'^T [n_tok, V], fp32
+    if (!lt::gemm(st, false, true, H, V, n_tok, hid, H, ds, V, d_weight, H, true, t0 == 0 ? 0.f : 1.f, lt_ws,
+                  lt::kWorkspaceBytes))
+      return AA_ERR_LAUNCH;
   }
   return launch_status();
 }
