@@ -3,7 +3,8 @@
 Importing the package does not load the HIP library; the first op call does, and
 raises ``NativeLibraryError`` if ``libareal_amd.so`` has not been built.
 """
-from .config import RejectionSamplingConfig
+from .advantages import Normalization, gae_advantages, masked_moments
+from .config import NormConfig, RejectionSamplingConfig
 from .functional import (
     RejectionSamplingResult,
     apply_rejection_sampling,
@@ -21,14 +22,18 @@ __version__ = "0.1.0"
 
 __all__ = [
     "NativeLibraryError",
+    "NormConfig",
+    "Normalization",
     "RejectionSamplingConfig",
     "RejectionSamplingResult",
     "apply_rejection_sampling",
     "fused_lm_head_ppo_loss",
     "fused_logprobs_ppo_loss",
+    "gae_advantages",
     "gather_logprobs",
     "gather_logprobs_entropy",
     "gather_logprobs_entropy_stats",
     "lm_head_logprobs_entropy",
+    "masked_moments",
     "ppo_actor_loss_fn",
 ]

@@ -36,6 +36,19 @@ class PpoParams(C.Structure):
     ]
 
 
+class NormParams(C.Structure):
+    """``aa_norm_params``"""
+
+    _fields_ = [
+        ("mean_level", C.c_int32),
+        ("mean_leave1out", C.c_int32),
+        ("std_level", C.c_int32),
+        ("std_unbiased", C.c_int32),
+        ("eps", C.c_float),
+        ("group_size", C.c_int64),
+    ]
+
+
 _p = C.c_void_p
 _i64 = C.c_int64
 _f = C.c_float
@@ -65,6 +78,10 @@ SIGNATURES = {
         [_p, _p, _i64, _i64, _i64, _p, _f, _i64, _p, _p, _p, _p, C.POINTER(PpoParams), _p, _p,
          _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _p],
     ),
+    "aa_gae": (_i, [_p, _p, _p, _p, _i64, _i64, _f, _f, _p, _p, _p]),
+    "aa_normalize_scratch_bytes": (_i64, [_i64, _i64]),
+    "aa_normalize": (_i, [_p, _p, _i64, _i64, C.POINTER(NormParams), _p, _p, _i64, _p]),
+    "aa_masked_moments": (_i, [C.POINTER(C.c_void_p), _i, _p, _i64, _p, _p]),
     "aa_copy_bytes": (_i, [_p, _p, _i64, _p]),
 }
 

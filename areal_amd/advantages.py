@@ -1,0 +1,145 @@
+"""Advantage pipeline of the PPO actor on the GPU: GAE, reward / advantage normalisation, masked moments.
+
+Host-side mirror of ``Normalization`` (areal/utils/data.py:1378-1596), of the GAE loop of
+``PPOActor._compute_advantages`` (areal/trainer/ppo/actor.py:209-236) and of the masked reductions the statistics
+tracker performs per tensor (areal/utils/stats_tracker.py:227-285).  Everything runs in the HIP library; CPU tensors
+are refused.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Any, Mapping
+
+import torch
+
+from . import _native as N
+from .functional import _f32, _mask_u8, _ptr, _require_gpu, _stream
+
+_LEVELS = {None: 0, "none": 0, "batch": 1, "group": 2}
+
+
+class Normalization:
+    """``Normalization(config)(x, loss_mask)`` with the reference's semantics (data.py:1378-1504).
+
+    ``config`` is any object with the attributes of ``NormConfig``.  Sums are accumulated in float64 whatever
+    ``high_precision`` says.  One process only: with ``torch.distributed`` initialised on more than one rank the
+    batch-level statistics would need an all-reduce, which this build does not have.
+    """
+
+    def __init__(self, config: Any):
+        self.mean_level = config.mean_level
+        self.mean_leave1out = config.mean_leave1out
+        self.std_level = config.std_level
+        self.std_unbiased = config.std_unbiased
+        self.group_size = config.group_size
+        self.eps = config.eps
+        for name, level in (("mean_level", self.mean_level), ("std_level", self.std_level)):
+            if level not in _LEVELS:
+                raise ValueError(f"{name} must be 'batch', 'group' or None, got {level}")
+        if (self.mean_level == "group" or self.std_level == "group") and self.group_size < 1:
+            raise ValueError(
+                f"group_size must be a positive integer when using group normalization, got {self.group_size}"
+            )
+
+    @torch.no_grad()
+    def __call__(self, x: torch.Tensor, loss_mask: torch.Tensor | None = None, high_precision: bool = True,
+                 reduce_group=None) -> torch.Tensor:
+        _require_gpu(x, "x")
+        if torch.distributed.is_available() and torch.distributed.is_initialized():
+            if torch.distributed.get_world_size(reduce_group) > 1:
+                raise NotImplementedError("Normalization across ranks is not part of this build (one GPU)")
+        if loss_mask is not None and loss_mask.shape != x.shape:
+            raise ValueError(f"loss_mask shape {tuple(loss_mask.shape)} != x shape {tuple(x.shape)}")
+        if x.ndim == 0:
+            raise ValueError("x must have a batch dimension")
+        bs = x.shape[0]
+        if x.numel() == 0:
+            return x.float()
+        xf = _f32(x)
+        mf = None if loss_mask is None else _f32(loss_mask)
+        inner = xf.numel() // bs
+        params = N.NormParams(_LEVELS[self.mean_level], int(bool(self.mean_leave1out)), _LEVELS[self.std_level],
+                              int(bool(self.std_unbiased)), float(self.eps), int(self.group_size))
+        lib = N.load()
+        dev = xf.device
+        grouped = params.mean_level == 2 or params.std_level == 2
+        n_bytes = lib.aa_normalize_scratch_bytes(bs, int(self.group_size) if grouped else max(bs, 1))
+        scratch = torch.empty(max(n_bytes, 32) // 8, dtype=torch.float64, device=dev)
+        out = torch.empty_like(xf)
+        with torch.cuda.device(dev):
+            N.check(
+                lib.aa_normalize(_ptr(xf), _ptr(mf), bs, inner, C.byref(params), _ptr(out), _ptr(scratch),
+                                 scratch.numel() * 8, _stream(dev)),
+                "aa_normalize",
+            )
+        return out
+
+
+@torch.no_grad()
+def gae_advantages(rewards: torch.Tensor, values: torch.Tensor | None, loss_mask: torch.Tensor,
+                   seq_no_eos_mask: torch.Tensor | None, discount: float, gae_lambda: float
+                   ) -> tuple[torch.Tensor, torch.Tensor]:
+    """``(advantages, returns)`` of the GAE loop in ``PPOActor._compute_advantages`` (actor.py:209-232).
+
+    ``rewards``, ``values``, ``loss_mask`` are the padded ``[bs, max_seqlen]`` tensors of that function (the mask
+    already rolled by -1), ``seq_no_eos_mask`` is ``[bs]``; ``values=None`` stands for zeros (actor.py:210-211).
+    """
+    _require_gpu(rewards, "rewards")
+    if rewards.ndim != 2:
+        raise ValueError(f"expected rewards [bs, max_seqlen], got {tuple(rewards.shape)}")
+    if loss_mask.shape != rewards.shape or (values is not None and values.shape != rewards.shape):
+        raise ValueError("rewards, values and loss_mask must have the same shape")
+    bs, L = rewards.shape
+    if seq_no_eos_mask is not None and tuple(seq_no_eos_mask.shape) != (bs,):
+        raise ValueError(f"seq_no_eos_mask shape {tuple(seq_no_eos_mask.shape)} != ({bs},)")
+    assert L > 0, "max_seqlen must be positive"
+    dev = rewards.device
+    r, m = _f32(rewards), _f32(loss_mask)
+    v = None if values is None else _f32(values)
+    ne = None if seq_no_eos_mask is None else _mask_u8(seq_no_eos_mask.to(dev) != 0)
+    adv = torch.empty_like(r)
+    ret = torch.empty_like(r)
+    lib = N.load()
+    with torch.cuda.device(dev):
+        N.check(
+            lib.aa_gae(_ptr(r), _ptr(v), _ptr(m), _ptr(ne), bs, L, float(discount), float(gae_lambda), _ptr(adv),
+                       _ptr(ret), _stream(dev)),
+            "aa_gae",
+        )
+    return adv, ret
+
+
+@torch.no_grad()
+def masked_moments(values: Mapping[str, torch.Tensor], mask: torch.Tensor) -> dict[str, dict[str, torch.Tensor]]:
+    """Sum, mean, min, max and count of every tensor in ``values`` over ``mask``, in one launch.
+
+    These are the quantities ``stats_tracker.stat(..., denominator=mask)`` reduces one tensor at a time
+    (stats_tracker.py:227-285).  Returns ``{name: {"sum", "avg", "min", "max", "count"}}`` of 0-d device tensors;
+    ``avg`` is NaN and ``min`` / ``max`` are +/-inf when the mask selects nothing.
+    """
+    names = list(values)
+    if not names:
+        return {}
+    if len(names) > 16:
+        raise ValueError("at most 16 tensors per call")
+    _require_gpu(mask, "mask")
+    m8 = _mask_u8(mask.reshape(-1))
+    n = m8.numel()
+    tensors = []
+    for k in names:
+        t = values[k]
+        _require_gpu(t, k)
+        if t.numel() != n:
+            raise ValueError(f"{k} has {t.numel()} elements, the mask has {n}")
+        tensors.append(_f32(t.detach()).reshape(-1))
+    dev = m8.device
+    out = torch.empty(len(names), 4, dtype=torch.float32, device=dev)
+    ptrs = (C.c_void_p * len(names))(*[t.data_ptr() for t in tensors])
+    lib = N.load()
+    with torch.cuda.device(dev):
+        N.check(lib.aa_masked_moments(ptrs, len(names), _ptr(m8), n, _ptr(out), _stream(dev)), "aa_masked_moments")
+    res = {}
+    for i, k in enumerate(names):
+        s, lo, hi, c = out[i, 0], out[i, 1], out[i, 2], out[i, 3]
+        res[k] = dict(sum=s, avg=s / c, min=lo, max=hi, count=c)
+    return res

@@ -55,3 +55,27 @@ class RejectionSamplingConfig:
                 UserWarning,
                 stacklevel=2,
             )
+
+
+@dataclass
+class NormConfig:
+    """Reward / advantage normalisation options; fields, defaults and validation texts of ``NormConfig`` in
+    areal/api/cli_args.py:42-95."""
+
+    mean_level: str | None = "batch"
+    mean_leave1out: bool = False
+    std_level: str | None = "batch"
+    std_unbiased: bool = True
+    eps: float = 1e-5
+    group_size: int = 1
+
+    def __post_init__(self) -> None:
+        valid_levels = {"batch", "group", None}
+        if self.mean_level not in valid_levels:
+            raise ValueError(f"mean_level must be 'batch', 'group' or None, got {self.mean_level}")
+        if self.std_level not in valid_levels:
+            raise ValueError(f"std_level must be 'batch', 'group', or None, got {self.std_level}")
+        if (self.mean_level == "group" or self.std_level == "group") and self.group_size < 1:
+            raise ValueError(
+                f"group_size must be a positive integer when using group normalization, got {self.group_size}"
+            )

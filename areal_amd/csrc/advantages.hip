@@ -1,0 +1,363 @@
+// Advantage pipeline of the PPO actor on gfx950: the GAE reverse scan, reward / advantage normalisation, and the
+// masked moments the statistics logger asks for.  Reference: areal/trainer/ppo/actor.py:209-236 (GAE, a Python
+// loop over max_seqlen), areal/utils/data.py:1378-1596 (Normalization), areal/utils/stats_tracker.py:227-285.
+#include "device_utils.h"
+
+namespace aa {
+namespace adv {
+
+constexpr int kThreads = 1024;
+
+template <typename T>
+__device__ __forceinline__ T block_sum(T v, T* smem) {
+  v = wave_sum(v);
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  __syncthreads();
+  if (lane == 0) smem[wave] = v;
+  __syncthreads();
+  T r = smem[0];
+  for (int w = 1; w < (int)(blockDim.x / kWave); ++w) r += smem[w];
+  return r;
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// GAE.  Going backwards over t = L-2 .. 0 the reference carries (nv, lg) = (next value, last advantage):
+//     delta = r_t + gamma * nv - v_t;  new = delta + gamma * lambda * lg
+//     nv <- nv (1 - m_t) + v_t m_t;    lg <- lg (1 - m_t) + new m_t;    adv_t = lg
+// which is the affine map  nv' = a nv + e,  lg' = c nv + d lg + f  with
+//     a = 1 - m, e = m v, c = m gamma, d = 1 - m + m gamma lambda, f = m (r - v).
+// Affine maps compose, so one wave handles one row in blocks of 64 positions: each lane builds the map of its
+// position, an inclusive wave scan composes them in processing order, and the carry of the block is applied last.
+// ------------------------------------------------------------------------------------------------------------------
+struct Affine {
+  float a, c, d, e, f;
+};
+
+// `first` is applied before `second`
+__device__ __forceinline__ Affine compose(const Affine& first, const Affine& second) {
+  Affine r;
+  r.a = second.a * first.a;
+  r.c = fmaf(second.c, first.a, second.d * first.c);
+  r.d = second.d * first.d;
+  r.e = fmaf(second.a, first.e, second.e);
+  r.f = fmaf(second.c, first.e, fmaf(second.d, first.f, second.f));
+  return r;
+}
+
+__device__ __forceinline__ Affine shfl_up(const Affine& x, int delta) {
+  Affine r;
+  r.a = __shfl_up(x.a, delta, kWave);
+  r.c = __shfl_up(x.c, delta, kWave);
+  r.d = __shfl_up(x.d, delta, kWave);
+  r.e = __shfl_up(x.e, delta, kWave);
+  r.f = __shfl_up(x.f, delta, kWave);
+  return r;
+}
+
+__global__ __launch_bounds__(256) void k_gae(const float* __restrict__ rewards, const float* __restrict__ values,
+                                             const float* __restrict__ mask, const uint8_t* __restrict__ no_eos,
+                                             int64_t bs, int64_t L, float gamma, float lam,
+                                             float* __restrict__ adv, float* __restrict__ returns) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t row = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (row >= bs) return;  // whole waves leave together: no barrier below
+  const float* r = rewards + row * L;
+  const float* v = values ? values + row * L : nullptr;
+  const float* m = mask + row * L;
+  float* out_a = adv + row * L;
+  float* out_r = returns ? returns + row * L : nullptr;
+  const float v_last = v ? v[L - 1] : 0.f;
+  if (lane == 0) {
+    out_a[L - 1] = 0.f;
+    if (out_r) out_r[L - 1] = v_last;
+  }
+  float nv = (no_eos && no_eos[row]) ? v_last : 0.f;  // values[:, L-1] * seq_no_eos_mask
+  float lg = 0.f;
+  const float gl = gamma * lam;
+  for (int64_t hi = L - 2; hi >= 0; hi -= kWave) {  // lane j handles t = hi - j: processing order = lane order
+    const int64_t t = hi - lane;
+    const bool live = t >= 0;
+    float rt = 0.f, vt = 0.f, mt = 0.f;
+    if (live) {
+      rt = r[t];
+      vt = v ? v[t] : 0.f;
+      mt = m[t];
+    }
+    Affine x;  // identity where the row has ended (mt = 0)
+    x.a = 1.f - mt;
+    x.e = mt * vt;
+    x.c = mt * gamma;
+    x.d = (1.f - mt) + mt * gl;
+    x.f = mt * (rt - vt);
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+      const Affine prev = shfl_up(x, o);
+      if (lane >= o) x = compose(prev, x);
+    }
+    const float lg_t = fmaf(x.c, nv, fmaf(x.d, lg, x.f));
+    const float nv_t = fmaf(x.a, nv, x.e);
+    if (live) {
+      out_a[t] = lg_t;
+      if (out_r) out_r[t] = lg_t + vt;
+    }
+    nv = __shfl(nv_t, kWave - 1, kWave);
+    lg = __shfl(lg_t, kWave - 1, kWave);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// Normalization.  Segment 0 is the whole batch, segment 1 + g is group g (group_size rows of `inner` elements);
+// rows past the last full group belong to no group (the reference leaves their mean and std at zero).
+// stats[seg] = {sum(x m), sum(m), sum((x m - mean m)^2), -}
+// ------------------------------------------------------------------------------------------------------------------
+struct NormArgs {
+  const float* x;
+  const float* mask;  // nullable
+  int64_t n;          // bs * inner
+  int64_t seg_elems;  // group_size * inner
+  int64_t n_groups;   // bs / group_size
+  int64_t group_size;
+  int mean_level, mean_leave1out, std_level, std_unbiased;  // levels: 0 none, 1 batch, 2 group
+  float eps;
+};
+
+__device__ __forceinline__ void seg_range(const NormArgs& a, int seg, int64_t& beg, int64_t& end) {
+  if (seg == 0) {
+    beg = 0;
+    end = a.n;
+  } else {
+    beg = (int64_t)(seg - 1) * a.seg_elems;
+    end = beg + a.seg_elems;
+  }
+}
+
+// mean of Normalization._compute_mean for one element, from the (sum, count) of its segment
+__device__ __forceinline__ double level_mean(double S, double F, bool loo, bool has_mask, double xi, double mi) {
+  if (loo) {
+    if (F <= 1.0) return 0.0;
+    if (!has_mask) return (S - xi) / (F - 1.0);
+    if (mi > 0.0) {
+      double den = F - mi;
+      if (den < 1.0) den = 1.0;
+      return (S - xi * mi) / den;
+    }
+    return S / F;
+  }
+  return F == 0.0 ? 0.0 : S / F;
+}
+
+// The mean the reference subtracts from element i.  `as_float`: the reference keeps group-level (and absent) means
+// in a tensor of the dtype of x, batch-level means in float64.
+__device__ __forceinline__ double mean_at(const NormArgs& a, const double4* stats, int64_t i, float xi, float mi,
+                                          bool& as_float) {
+  as_float = true;
+  if (a.mean_level == 0) return 0.0;
+  const bool has_mask = a.mask != nullptr;
+  if (a.mean_level == 1) {
+    as_float = false;
+    return level_mean(stats[0].x, stats[0].y, a.mean_leave1out != 0, has_mask, xi, mi);
+  }
+  const int64_t g = i / a.seg_elems;
+  if (g >= a.n_groups) return 0.0;
+  if (a.group_size == 1 && a.mean_leave1out) return 0.0;
+  const double4 s = stats[1 + g];
+  return (double)(float)level_mean(s.x, s.y, a.mean_leave1out != 0, has_mask, xi, mi);
+}
+
+__global__ __launch_bounds__(kThreads) void k_norm_sums(NormArgs a, double4* __restrict__ stats) {
+  __shared__ double smem[kThreads / kWave];
+  int64_t beg, end;
+  seg_range(a, blockIdx.x, beg, end);
+  double s = 0.0, f = 0.0;
+  for (int64_t i = beg + threadIdx.x; i < end; i += kThreads) {
+    const double mi = a.mask ? (double)a.mask[i] : 1.0;
+    s += (double)a.x[i] * mi;
+    f += mi;
+  }
+  s = block_sum<double>(s, smem);
+  f = block_sum<double>(f, smem);
+  if (threadIdx.x == 0) stats[blockIdx.x] = make_double4(s, f, 0.0, 0.0);
+}
+
+__global__ __launch_bounds__(kThreads) void k_norm_sumsq(NormArgs a, double4* __restrict__ stats) {
+  __shared__ double smem[kThreads / kWave];
+  int64_t beg, end;
+  seg_range(a, blockIdx.x, beg, end);
+  double q = 0.0;
+  for (int64_t i = beg + threadIdx.x; i < end; i += kThreads) {
+    const float xi = a.x[i];
+    const float mi = a.mask ? a.mask[i] : 1.f;
+    bool as_float;
+    const double mean = mean_at(a, stats, i, xi, mi, as_float);
+    const double d = (double)xi * (double)mi - mean * (double)mi;  // x_masked - mean * mask
+    q += d * d;
+  }
+  q = block_sum<double>(q, smem);
+  if (threadIdx.x == 0) stats[blockIdx.x].z = q;
+}
+
+__device__ __forceinline__ double level_std(double Q, double F, bool unbiased) {
+  if (unbiased) return F <= 1.0 ? 1.0 : sqrt(Q / (F - 1.0));
+  return F == 0.0 ? 1.0 : sqrt(Q / F);
+}
+
+__global__ __launch_bounds__(256) void k_norm_apply(NormArgs a, const double4* __restrict__ stats,
+                                                    float* __restrict__ out) {
+  const bool has_mask = a.mask != nullptr;
+  const bool passthrough = has_mask && stats[0].y == 0.0;  // nothing active: the input comes back unchanged
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.n; i += (int64_t)gridDim.x * blockDim.x) {
+    const float xi = a.x[i];
+    if (passthrough) {
+      out[i] = xi;
+      continue;
+    }
+    const float mi = has_mask ? a.mask[i] : 1.f;
+    bool mean_f;
+    const double mean = mean_at(a, stats, i, xi, mi, mean_f);
+    // x - mean, then * mask, in the precision the reference's tensors have at that point
+    double cen;
+    if (mean_f) {
+      float c = xi - (float)mean;
+      if (has_mask) c *= mi;
+      cen = (double)c;
+    } else {
+      cen = (double)xi - mean;
+      if (has_mask) cen *= (double)mi;
+    }
+    double sd;
+    bool std_f = true;
+    float eps = a.eps;
+    if (a.std_level == 0) {
+      sd = 1.0;
+      eps = 0.f;
+    } else if (a.std_level == 1) {
+      sd = level_std(stats[0].z, stats[0].y, a.std_unbiased != 0);
+      std_f = false;
+    } else {
+      const int64_t g = i / a.seg_elems;
+      if (g >= a.n_groups) sd = 0.0;
+      else if (a.group_size == 1 && a.std_unbiased) sd = 1.0;
+      else sd = (double)(float)level_std(stats[1 + g].z, stats[1 + g].y, a.std_unbiased != 0);
+    }
+    float r;
+    if (std_f && mean_f) {
+      r = (float)cen / ((float)sd + eps);
+    } else if (std_f) {
+      r = (float)(cen / (double)((float)sd + eps));
+    } else {
+      r = (float)(cen / (sd + (double)eps));
+    }
+    out[i] = r;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// Masked moments of up to kMaxTensors per-token tensors under one mask: out[k] = {sum, min, max, count}
+// (min = +inf, max = -inf when nothing is selected).  One workgroup per tensor, fixed summation order.
+// ------------------------------------------------------------------------------------------------------------------
+constexpr int kMaxTensors = 16;
+struct MomentArgs {
+  const float* v[kMaxTensors];
+};
+
+__global__ __launch_bounds__(kThreads) void k_masked_moments(MomentArgs a, const uint8_t* __restrict__ mask, int64_t n,
+                                                             float* __restrict__ out) {
+  __shared__ double smem_d[kThreads / kWave];
+  __shared__ float smem_lo[kThreads / kWave], smem_hi[kThreads / kWave];
+  const float* v = a.v[blockIdx.x];
+  double s = 0.0, c = 0.0;
+  float lo = __builtin_inff(), hi = -__builtin_inff();
+  for (int64_t i = threadIdx.x; i < n; i += kThreads) {
+    if (mask[i] != 0) {
+      const float x = v[i];
+      s += (double)x;
+      c += 1.0;
+      lo = fminf(lo, x);
+      hi = fmaxf(hi, x);
+    }
+  }
+  s = block_sum<double>(s, smem_d);
+  c = block_sum<double>(c, smem_d);
+  lo = wave_min(lo);
+  hi = wave_max(hi);
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  if (lane == 0) {
+    smem_lo[wave] = lo;
+    smem_hi[wave] = hi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kThreads / kWave; ++w) {
+      lo = fminf(lo, smem_lo[w]);
+      hi = fmaxf(hi, smem_hi[w]);
+    }
+    float* o = out + 4 * blockIdx.x;
+    o[0] = (float)s;
+    o[1] = lo;
+    o[2] = hi;
+    o[3] = (float)c;
+  }
+}
+
+}  // namespace adv
+}  // namespace aa
+
+using namespace aa;
+using namespace aa::adv;
+
+extern "C" int aa_gae(const float* rewards, const float* values, const float* loss_mask, const uint8_t* seq_no_eos,
+                      int64_t bs, int64_t L, float discount, float gae_lambda, float* advantages, float* returns,
+                      void* stream) {
+  if (!rewards || !loss_mask || !advantages || bs < 0 || L < 1) return AA_ERR_INVALID_ARGUMENT;
+  if (bs == 0) return AA_OK;
+  const int rows_per_wg = 256 / kWave;
+  hipLaunchKernelGGL(k_gae, dim3((unsigned)((bs + rows_per_wg - 1) / rows_per_wg)), dim3(256), 0, (hipStream_t)stream,
+                     rewards, values, loss_mask, seq_no_eos, bs, L, discount, gae_lambda, advantages, returns);
+  return launch_status();
+}
+
+extern "C" int64_t aa_normalize_scratch_bytes(int64_t bs, int64_t group_size) {
+  if (bs < 0 || group_size < 1) return -1;
+  return (int64_t)sizeof(double4) * (1 + bs / group_size);
+}
+
+extern "C" int aa_normalize(const float* x, const float* loss_mask, int64_t bs, int64_t inner,
+                            const aa_norm_params* params, float* out, void* scratch, int64_t scratch_bytes,
+                            void* stream) {
+  if (!x || !out || !params || !scratch || bs < 0 || inner < 1) return AA_ERR_INVALID_ARGUMENT;
+  const aa_norm_params& p = *params;
+  if (p.mean_level < 0 || p.mean_level > 2 || p.std_level < 0 || p.std_level > 2) return AA_ERR_INVALID_ARGUMENT;
+  const bool grouped = p.mean_level == 2 || p.std_level == 2;
+  if (grouped && p.group_size < 1) return AA_ERR_INVALID_ARGUMENT;
+  if (bs == 0) return AA_OK;
+  const int64_t gs = grouped ? p.group_size : bs;
+  const int64_t n_groups = grouped ? bs / gs : 0;
+  if (scratch_bytes < (int64_t)sizeof(double4) * (1 + n_groups) || (((uintptr_t)scratch) & 31))
+    return AA_ERR_INVALID_ARGUMENT;
+  NormArgs a{x, loss_mask, bs * inner, gs * inner, n_groups, gs, p.mean_level, p.mean_leave1out, p.std_level,
+             p.std_unbiased, p.eps};
+  hipStream_t st = (hipStream_t)stream;
+  double4* stats = (double4*)scratch;
+  const unsigned segs = (unsigned)(1 + n_groups);
+  hipLaunchKernelGGL(k_norm_sums, dim3(segs), dim3(kThreads), 0, st, a, stats);
+  if (p.std_level != 0) hipLaunchKernelGGL(k_norm_sumsq, dim3(segs), dim3(kThreads), 0, st, a, stats);
+  int64_t blocks = (a.n + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(k_norm_apply, dim3((unsigned)blocks), dim3(256), 0, st, a, stats, out);
+  return launch_status();
+}
+
+extern "C" int aa_masked_moments(const float* const* values, int n_tensors, const uint8_t* mask, int64_t n,
+                                 float* out, void* stream) {
+  if (!values || !out || n_tensors < 0 || n_tensors > kMaxTensors || n < 0 || (n > 0 && !mask))
+    return AA_ERR_INVALID_ARGUMENT;
+  if (n_tensors == 0) return AA_OK;
+  MomentArgs a{};
+  for (int k = 0; k < n_tensors; ++k) {
+    if (!values[k] && n > 0) return AA_ERR_INVALID_ARGUMENT;
+    a.v[k] = values[k];
+  }
+  hipLaunchKernelGGL(k_masked_moments, dim3((unsigned)n_tensors), dim3(kThreads), 0, (hipStream_t)stream, a, mask, n,
+                     out);
+  return launch_status();
+}

@@ -188,6 +188,66 @@ int aa_scale_inplace(void* data, int dtype, int64_t n, const float* factor,
                      void* stream);
 
 /* ------------------------------------------------------------------ */
+/* Advantage pipeline (rows are sequences of a padded [bs, L] batch)      */
+/* ------------------------------------------------------------------ */
+
+/*
+ * GAE reverse scan of PPOActor._compute_advantages
+ * (areal/trainer/ppo/actor.py:209-236), which the reference runs as a Python
+ * loop over max_seqlen.  For t = L-2 .. 0, with nv = values[:, L-1] *
+ * seq_no_eos and lg = 0 to start:
+ *   delta = rewards[t] + discount * nv - values[t]
+ *   new   = delta + discount * gae_lambda * lg
+ *   nv    = nv * (1 - m[t]) + values[t] * m[t]
+ *   lg    = lg * (1 - m[t]) + new * m[t];   advantages[t] = lg
+ * advantages[:, L-1] = 0; returns = advantages + values (nullable).
+ * rewards, loss_mask [bs, L] float32 contiguous; values nullable (zeros);
+ * seq_no_eos [bs] bytes, nullable (zeros).  One wave per row: the
+ * recurrence is an affine map per token, composed by a wave-level scan.
+ */
+int aa_gae(const float* rewards, const float* values, const float* loss_mask,
+           const uint8_t* seq_no_eos, int64_t bs, int64_t L, float discount,
+           float gae_lambda, float* advantages, float* returns, void* stream);
+
+/* Normalization (areal/utils/data.py:1378-1596); levels: 0 none, 1 batch,
+ * 2 group; mirrors NormConfig (areal/api/cli_args.py:42-95). */
+typedef struct {
+  int32_t mean_level;
+  int32_t mean_leave1out;
+  int32_t std_level;
+  int32_t std_unbiased;
+  float eps;
+  int64_t group_size; /* rows per group, used when a level is 2 */
+} aa_norm_params;
+
+/* Bytes of scratch aa_normalize needs (32-byte aligned device memory). */
+int64_t aa_normalize_scratch_bytes(int64_t bs, int64_t group_size);
+
+/*
+ * out = Normalization(params)(x, loss_mask) for x [bs, inner] float32
+ * contiguous and an optional float32 mask of the same shape: centring by the
+ * batch / group mean (optionally leave-one-out), masking, division by the
+ * batch / group standard deviation (+ eps).  Sums are accumulated in float64
+ * in a fixed order; group-level means and deviations are rounded to float32
+ * where the reference stores them in float32 tensors.  Rows past the last
+ * full group keep mean = std = 0, and an all-zero mask returns x, both as in
+ * the reference.
+ */
+int aa_normalize(const float* x, const float* loss_mask, int64_t bs,
+                 int64_t inner, const aa_norm_params* params, float* out,
+                 void* scratch, int64_t scratch_bytes, void* stream);
+
+/*
+ * Masked moments of up to 16 per-token float32 tensors under one byte mask,
+ * the reductions the statistics logger performs one tensor at a time
+ * (areal/utils/stats_tracker.py:227-285): out[k] = {sum, min, max, count}
+ * over mask != 0 (min = +inf, max = -inf when the mask is empty).
+ * values is a HOST array of n_tensors device pointers.
+ */
+int aa_masked_moments(const float* const* values, int n_tensors,
+                      const uint8_t* mask, int64_t n, float* out, void* stream);
+
+/* ------------------------------------------------------------------ */
 /* Fused lm_head path (no counterpart in the reference: its equivalent is  */
 /* logits = hidden @ weight.T followed by the logits path above)           */
 /* ------------------------------------------------------------------ */

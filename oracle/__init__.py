@@ -24,6 +24,7 @@ from .ppo import (
     rejection_sampling,
     sequence_level_ratio_and_advantages,
 )
+from .advantages import gae, masked_moments, normalization
 from .pipeline import lmhead_logits, logits_ppo_step
 
 __all__ = [
@@ -36,6 +37,9 @@ __all__ = [
     "ppo_actor_loss",
     "rejection_sampling",
     "sequence_level_ratio_and_advantages",
+    "gae",
+    "masked_moments",
+    "normalization",
     "lmhead_logits",
     "logits_ppo_step",
 ]

@@ -1,0 +1,135 @@
+"""CPU oracle of the advantage pipeline: GAE, Normalization, masked moments.  TEST INFRASTRUCTURE ONLY.
+
+Restates, in plain PyTorch on the CPU,
+  * the GAE loop of ``PPOActor._compute_advantages`` (areal/trainer/ppo/actor.py:209-236),
+  * ``Normalization`` (areal/utils/data.py:1378-1596) for one process (no all-reduce),
+  * the masked reductions of the statistics tracker (areal/utils/stats_tracker.py:227-285).
+How each function is pinned is listed in ``oracle/PINNING.md``.
+"""
+from __future__ import annotations
+
+import torch
+
+
+def gae(rewards, values, loss_mask, seq_no_eos_mask, discount: float, gae_lambda: float):
+    """(advantages, returns) for padded ``[bs, L]`` float tensors; actor.py:209-236, statement by statement."""
+    bs, max_seqlen = rewards.shape
+    advantages_reversed = [torch.zeros(bs, dtype=torch.float32)]          # :216-218
+    lastgaelam = 0                                                        # :219
+    nextvalues = values[:, max_seqlen - 1] * seq_no_eos_mask              # :220
+    for t in reversed(range(max_seqlen - 1)):                             # :221
+        delta = rewards[:, t] + discount * nextvalues - values[:, t]      # :222
+        newgaelam = delta + discount * gae_lambda * lastgaelam            # :223
+        mask = loss_mask[:, t]                                            # :226
+        nextvalues = nextvalues * (1 - mask) + values[:, t] * mask        # :227
+        lastgaelam = lastgaelam * (1 - mask) + newgaelam * mask           # :228
+        advantages_reversed.append(lastgaelam)                            # :229
+    advantages = torch.stack(advantages_reversed[::-1], dim=1)            # :231
+    return advantages, advantages + values                                # :232
+
+
+def _compute_mean(x, mask, high_precision: bool, leave_one_out: bool):
+    """data.py:1506-1557 without the all-reduce."""
+    dtype = torch.float64 if high_precision else torch.float32
+    x = x.to(dtype)
+    dim = tuple(range(x.dim()))
+    if mask is None:
+        factor = torch.tensor(float(x.numel()), dtype=dtype)
+        x_masked = x
+        x_sum = x.sum(dim=dim, keepdim=True)
+    else:
+        mask = mask.to(dtype)
+        x_masked = x * mask
+        factor = mask.sum(dim, keepdim=True)
+        x_sum = x_masked.sum(dim=dim, keepdim=True)
+    if leave_one_out:
+        if factor.item() <= 1:
+            return torch.zeros_like(x_sum)
+        if mask is None:
+            return (x_sum.expand_as(x) - x) / (factor - 1)
+        regular = x_sum / factor
+        loo = (x_sum.expand_as(x) - x_masked) / torch.clamp(factor - mask, min=1.0)
+        return torch.where(mask > 0, loo, regular.expand_as(x))
+    if factor.item() == 0:
+        return torch.zeros_like(x_sum)
+    return x_sum / factor
+
+
+def _compute_std(x, mask, mean, unbiased: bool, high_precision: bool):
+    """data.py:1559-1596 without the all-reduce."""
+    dtype = torch.float64 if high_precision else torch.float32
+    x = x.to(dtype)
+    mean = mean.to(dtype)
+    dim = tuple(range(x.dim()))
+    if mask is None:
+        factor = torch.tensor(float(x.numel()), dtype=dtype)
+        x_sum_sq = ((x - mean) ** 2).sum(dim=dim, keepdim=True)
+    else:
+        mask = mask.to(dtype)
+        factor = mask.sum(dim, keepdim=True)
+        x_sum_sq = ((x * mask - mean * mask) ** 2).sum(dim=dim, keepdim=True)
+    if unbiased:
+        if factor.item() <= 1:
+            return torch.ones_like(x_sum_sq)
+        return (x_sum_sq / (factor - 1)).sqrt()
+    if factor.item() == 0:
+        return torch.ones_like(x_sum_sq)
+    return (x_sum_sq / factor).sqrt()
+
+
+def normalization(x, loss_mask=None, mean_level="batch", mean_leave1out=False, std_level="batch", std_unbiased=True,
+                  eps: float = 1e-5, group_size: int = 1, high_precision: bool = True):
+    """``Normalization(NormConfig(...))(x, loss_mask)``; data.py:1395-1504."""
+    bs = x.size(0)
+    if loss_mask is not None and loss_mask.sum().item() == 0:             # :1407-1408
+        return x.float()
+    if mean_level == "batch":                                             # :1411-1420
+        mean = _compute_mean(x, loss_mask, high_precision, mean_leave1out).expand_as(x)
+    elif mean_level == "group":                                           # :1421-1444
+        mean = torch.zeros_like(x)
+        for i in range(0, bs // group_size):
+            s = slice(i * group_size, (i + 1) * group_size)
+            xx = x[s]
+            m = loss_mask[s] if loss_mask is not None else None
+            if group_size == 1 and mean_leave1out:
+                group_mean = torch.zeros((1, *xx.shape[1:]), dtype=torch.float64 if high_precision else torch.float32)
+            else:
+                group_mean = _compute_mean(xx, m, high_precision, mean_leave1out)
+            mean[s] = group_mean.expand_as(xx)
+    else:
+        mean = torch.zeros_like(x)                                        # :1446
+    x_centered = x - mean                                                 # :1449
+    if loss_mask is not None:
+        x_centered = x_centered * loss_mask                               # :1452
+    if std_level == "batch":                                              # :1455-1465
+        std = _compute_std(x, loss_mask, mean, std_unbiased, high_precision).expand_as(x)
+    elif std_level == "group":                                            # :1466-1492
+        std = torch.zeros_like(x)
+        for i in range(0, bs // group_size):
+            s = slice(i * group_size, (i + 1) * group_size)
+            xx = x[s]
+            m = loss_mask[s] if loss_mask is not None else None
+            if group_size == 1 and std_unbiased:
+                group_std = torch.ones((1, *xx.shape[1:]), dtype=torch.float64 if high_precision else torch.float32)
+            else:
+                group_std = _compute_std(xx, m, mean[s], std_unbiased, high_precision)
+            std[s] = group_std.expand_as(xx)
+    else:
+        std = torch.ones_like(x)                                          # :1494-1495
+        eps = 0.0
+    return (x_centered / (std + eps)).float()                             # :1498
+
+
+def masked_moments(values, mask):
+    """``[K, 4]`` (sum, min, max, count) of each tensor under ``mask``; stats_tracker.py:238, 252-253, 270, 285."""
+    d = mask.bool()
+    rows = []
+    for v in values:
+        v = v.float()
+        rows.append(torch.stack([
+            torch.where(d, v, 0.0).double().sum().float(),
+            torch.where(d, v, float("inf")).min() if v.numel() else torch.tensor(float("inf")),
+            torch.where(d, v, -float("inf")).max() if v.numel() else torch.tensor(-float("inf")),
+            d.sum().float(),
+        ]))
+    return torch.stack(rows) if rows else torch.zeros(0, 4)

@@ -1,0 +1,148 @@
+"""GPU parity of the advantage pipeline (GAE scan, Normalization, masked moments) against the CPU oracle and the
+reference's own known-answer cases."""
+import itertools
+import json
+from pathlib import Path
+
+import pytest
+import torch
+
+import areal_amd
+from areal_amd import NormConfig, Normalization
+from oracle import advantages as O
+
+pytestmark = pytest.mark.gpu
+
+GOLD = json.loads((Path(__file__).parent / "golden" / "reference_norm_known_answers.json").read_text())
+
+
+@pytest.mark.parametrize("c", GOLD["cases"], ids=[c["name"] for c in GOLD["cases"]])
+def test_normalization_reference_known_answers(device, c):
+    x = torch.tensor(c["x"], dtype=torch.float32)
+    mask = torch.ones_like(x) if c["mask"] == "ones" else torch.tensor(c["mask"], dtype=torch.float32)
+    out = Normalization(NormConfig(**c["cfg"]))(x.to(device), mask.to(device)).cpu()
+    assert out.dtype == torch.float32 and out.shape == x.shape
+    atol = c.get("atol", 1e-6)
+    if "expected" in c:
+        assert torch.allclose(out, torch.tensor(c["expected"], dtype=torch.float32), atol=atol)
+    for key, val in c.get("expected_at", {}).items():
+        i, j = (int(t) for t in key.split(","))
+        assert abs(float(out[i, j]) - val) <= atol
+    p = c.get("properties", {})
+    if "mean_abs_below" in p:
+        assert abs(float(out.mean())) < p["mean_abs_below"]
+    if "nonmasked_mean_abs_below" in p:
+        nm = out[mask.bool()]
+        assert abs(float(nm.mean())) < p["nonmasked_mean_abs_below"]
+        assert abs(float(nm.std()) - 1.0) < p["nonmasked_unbiased_std_minus_one_abs_below"]
+
+
+LEVELS = [None, "batch", "group"]
+
+
+@pytest.mark.parametrize("mean_level,std_level", list(itertools.product(LEVELS, LEVELS)))
+@pytest.mark.parametrize("loo,unbiased", [(False, True), (True, False), (True, True)])
+def test_normalization_matches_oracle(device, mean_level, std_level, loo, unbiased):
+    g = torch.Generator().manual_seed(hash((str(mean_level), str(std_level), loo, unbiased)) % 1000)
+    for shape, gs, with_mask in [((14, 37), 4, True), ((12, 5), 3, False), ((9,), 2, False), ((6, 3, 4), 1, True),
+                                 ((5, 8), 8, True)]:
+        x = torch.randn(*shape, generator=g) * 2.0 + 0.5
+        mask = (torch.rand(*shape, generator=g) < 0.6).float() if with_mask else None
+        cfg = dict(mean_level=mean_level, mean_leave1out=loo, std_level=std_level, std_unbiased=unbiased, eps=1e-5,
+                   group_size=gs)
+        want = O.normalization(x, mask, **cfg)
+        got = Normalization(NormConfig(**cfg))(x.to(device), None if mask is None else mask.to(device)).cpu()
+        assert got.shape == want.shape and got.dtype == torch.float32
+        scale = float(want.abs().max()) + 1.0
+        assert float((got - want).abs().max()) <= 2e-6 * scale, (shape, gs, cfg)
+
+
+def test_normalization_edge_cases(device):
+    x = torch.randn(4, 6)
+    zero = torch.zeros_like(x)
+    out = Normalization(NormConfig())(x.to(device), zero.to(device))
+    assert torch.equal(out.cpu(), x)  # nothing active: the input comes back
+    with pytest.raises(ValueError, match="group_size must be a positive integer"):
+        NormConfig(mean_level="group", std_level="batch", group_size=0)
+    with pytest.raises(ValueError, match="mean_level must be"):
+        NormConfig(mean_level="bad")
+    with pytest.raises(areal_amd.NativeLibraryError):
+        Normalization(NormConfig())(x)  # CPU tensors are refused
+    # bf16 input is accepted and comes back float32
+    out = Normalization(NormConfig())(x.bfloat16().to(device))
+    assert out.dtype == torch.float32
+    assert torch.allclose(out.cpu(), O.normalization(x.bfloat16().float()), atol=1e-5)
+
+
+def test_normalization_full_size(device):
+    bs, L = 512, 4096
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(bs, L, generator=g)
+    mask = (torch.rand(bs, L, generator=g) < 0.7).float()
+    for cfg in (dict(), dict(mean_level="group", std_level="group", group_size=16),
+                dict(mean_level="batch", std_level="group", group_size=8, mean_leave1out=True)):
+        want = O.normalization(x, mask, **cfg)
+        norm = Normalization(NormConfig(**cfg))
+        got = norm(x.to(device), mask.to(device))
+        assert float((got.cpu() - want).abs().max()) < 1e-5
+        assert torch.equal(got, norm(x.to(device), mask.to(device)))  # fixed summation order
+
+
+@pytest.mark.parametrize("bs,L", [(1, 1), (3, 2), (5, 63), (4, 64), (7, 65), (6, 66), (9, 129), (2, 1000)])
+@pytest.mark.parametrize("gamma,lam", [(1.0, 1.0), (0.99, 0.95)])
+def test_gae_matches_oracle(device, bs, L, gamma, lam):
+    g = torch.Generator().manual_seed(bs * 1000 + L)
+    r = torch.randn(bs, L, generator=g)
+    v = torch.randn(bs, L, generator=g)
+    m = (torch.rand(bs, L, generator=g) < 0.6).float()
+    ne = torch.rand(bs, generator=g) < 0.5
+    want_a, want_r = O.gae(r.double(), v.double(), m.double(), ne.double(), gamma, lam)
+    adv, ret = areal_amd.gae_advantages(r.to(device), v.to(device), m.to(device), ne.to(device), gamma, lam)
+    scale = float(want_a.abs().max()) + 1.0
+    assert float((adv.cpu().double() - want_a).abs().max()) < 2e-5 * scale
+    assert float((ret.cpu().double() - want_r).abs().max()) < 2e-5 * scale
+    # the fp32 loop of the reference agrees to the same bar
+    ref_a, _ = O.gae(r, v, m, ne.float(), gamma, lam)
+    assert float((adv.cpu() - ref_a).abs().max()) < 4e-5 * scale
+    # no critic: values = None stands for zeros
+    adv0, ret0 = areal_amd.gae_advantages(r.to(device), None, m.to(device), None, gamma, lam)
+    want0, _ = O.gae(r.double(), torch.zeros(bs, L).double(), m.double(), torch.zeros(bs).double(), gamma, lam)
+    assert float((adv0.cpu().double() - want0).abs().max()) < 2e-5 * (float(want0.abs().max()) + 1.0)
+    assert torch.equal(adv0, ret0)
+
+
+def test_gae_full_size_and_grpo_shape(device):
+    bs, L = 512, 4096
+    g = torch.Generator().manual_seed(1)
+    lens = torch.randint(L // 4, L + 1, (bs,), generator=g)
+    pos = torch.arange(L)[None, :]
+    m = ((pos >= (lens[:, None] * 0.3).long()) & (pos < lens[:, None] - 1)).float()
+    r = torch.zeros(bs, L)
+    r[torch.arange(bs), (lens - 2).clamp(min=0)] = torch.randn(bs, generator=g)   # one terminal reward per sequence
+    r = r - 0.01 * torch.rand(bs, L, generator=g) * m                             # plus KL penalties
+    v = torch.randn(bs, L, generator=g) * 0.1
+    ne = lens == L
+    want_a, want_r = O.gae(r, v, m, ne.float(), 1.0, 1.0)
+    adv, ret = areal_amd.gae_advantages(r.to(device), v.to(device), m.to(device), ne.to(device), 1.0, 1.0)
+    assert float((adv.cpu() - want_a).abs().max()) < 1e-4 and float((ret.cpu() - want_r).abs().max()) < 1e-4
+    adv2, _ = areal_amd.gae_advantages(r.to(device), v.to(device), m.to(device), ne.to(device), 1.0, 1.0)
+    assert torch.equal(adv, adv2)
+
+
+def test_masked_moments(device):
+    g = torch.Generator().manual_seed(2)
+    n = 10007
+    vals = {f"s{k}": torch.randn(n, generator=g) * (k + 1) for k in range(5)}
+    vals["flag"] = (torch.rand(n, generator=g) < 0.3).float()
+    mask = torch.rand(n, generator=g) < 0.4
+    got = areal_amd.masked_moments({k: v.to(device) for k, v in vals.items()}, mask.to(device))
+    want = O.masked_moments(list(vals.values()), mask)
+    for i, k in enumerate(vals):
+        assert float(got[k]["sum"]) == pytest.approx(float(want[i, 0]), rel=1e-5, abs=1e-4)
+        assert float(got[k]["min"]) == float(want[i, 1]) and float(got[k]["max"]) == float(want[i, 2])
+        assert float(got[k]["count"]) == float(want[i, 3])
+        assert float(got[k]["avg"]) == pytest.approx(float(want[i, 0] / want[i, 3]), rel=1e-5, abs=1e-6)
+    empty = areal_amd.masked_moments({"a": vals["s0"].to(device)}, torch.zeros(n, dtype=torch.bool, device=device))
+    assert float(empty["a"]["count"]) == 0.0 and float(empty["a"]["min"]) == float("inf")
+    with pytest.raises(ValueError):
+        areal_amd.masked_moments({"a": vals["s0"][:5].to(device)}, mask.to(device))
