@@ -63,7 +63,7 @@ class Normalization:
         lib = N.load()
         dev = xf.device
         grouped = params.mean_level == 2 or params.std_level == 2
-        n_bytes = lib.aa_normalize_scratch_bytes(bs, int(self.group_size) if grouped else max(bs, 1))
+        n_bytes = lib.aa_normalize_scratch_bytes(bs, inner, int(self.group_size) if grouped else max(bs, 1))
         scratch = torch.empty(max(n_bytes, 32) // 8, dtype=torch.float64, device=dev)
         out = torch.empty_like(xf)
         with torch.cuda.device(dev):

@@ -74,15 +74,24 @@ __global__ __launch_bounds__(256) void k_gae(const float* __restrict__ rewards, 
   float nv = (no_eos && no_eos[row]) ? v_last : 0.f;  // values[:, L-1] * seq_no_eos_mask
   float lg = 0.f;
   const float gl = gamma * lam;
-  for (int64_t hi = L - 2; hi >= 0; hi -= kWave) {  // lane j handles t = hi - j: processing order = lane order
+  // lane j handles t = hi - j: processing order = lane order.  The next block's loads are issued before this
+  // block's scan, so that memory latency hides behind the shuffles.
+  auto fetch = [&](int64_t hi, float& rt, float& vt, float& mt) {
     const int64_t t = hi - lane;
-    const bool live = t >= 0;
-    float rt = 0.f, vt = 0.f, mt = 0.f;
-    if (live) {
+    rt = 0.f; vt = 0.f; mt = 0.f;
+    if (t >= 0 && hi >= 0) {
       rt = r[t];
       vt = v ? v[t] : 0.f;
       mt = m[t];
     }
+  };
+  float rt, vt, mt;
+  fetch(L - 2, rt, vt, mt);
+  for (int64_t hi = L - 2; hi >= 0; hi -= kWave) {
+    float rn, vn, mn;
+    fetch(hi - kWave, rn, vn, mn);
+    const int64_t t = hi - lane;
+    const bool live = t >= 0;
     Affine x;  // identity where the row has ended (mt = 0)
     x.a = 1.f - mt;
     x.e = mt * vt;
@@ -102,6 +111,7 @@ __global__ __launch_bounds__(256) void k_gae(const float* __restrict__ rewards, 
     }
     nv = __shfl(nv_t, kWave - 1, kWave);
     lg = __shfl(lg_t, kWave - 1, kWave);
+    rt = rn; vt = vn; mt = mn;
   }
 }
 
@@ -164,36 +174,49 @@ __device__ __forceinline__ double mean_at(const NormArgs& a, const double4* stat
   return (double)(float)level_mean(s.x, s.y, a.mean_leave1out != 0, has_mask, xi, mi);
 }
 
-__global__ __launch_bounds__(kThreads) void k_norm_sums(NormArgs a, double4* __restrict__ stats) {
+// Pass 0 accumulates (sum x m, sum m), pass 1 sum (x m - mean m)^2.  A segment is cut into `parts` equal slices, one
+// workgroup each, so that the batch-wide segment fills the chip; k_norm_finish adds the slices in index order.
+template <int PASS>
+__global__ __launch_bounds__(kThreads) void k_norm_partial(NormArgs a, const double4* __restrict__ stats, int parts,
+                                                           double2* __restrict__ partial) {
   __shared__ double smem[kThreads / kWave];
+  const int seg = blockIdx.x / parts, part = blockIdx.x % parts;
   int64_t beg, end;
-  seg_range(a, blockIdx.x, beg, end);
+  seg_range(a, seg, beg, end);
+  const int64_t per = (end - beg + parts - 1) / parts;
+  const int64_t pb = beg + part * per;
+  const int64_t pe = pb + per < end ? pb + per : end;
   double s = 0.0, f = 0.0;
-  for (int64_t i = beg + threadIdx.x; i < end; i += kThreads) {
-    const double mi = a.mask ? (double)a.mask[i] : 1.0;
-    s += (double)a.x[i] * mi;
-    f += mi;
-  }
-  s = block_sum<double>(s, smem);
-  f = block_sum<double>(f, smem);
-  if (threadIdx.x == 0) stats[blockIdx.x] = make_double4(s, f, 0.0, 0.0);
-}
-
-__global__ __launch_bounds__(kThreads) void k_norm_sumsq(NormArgs a, double4* __restrict__ stats) {
-  __shared__ double smem[kThreads / kWave];
-  int64_t beg, end;
-  seg_range(a, blockIdx.x, beg, end);
-  double q = 0.0;
-  for (int64_t i = beg + threadIdx.x; i < end; i += kThreads) {
+  for (int64_t i = pb + threadIdx.x; i < pe; i += kThreads) {
     const float xi = a.x[i];
     const float mi = a.mask ? a.mask[i] : 1.f;
-    bool as_float;
-    const double mean = mean_at(a, stats, i, xi, mi, as_float);
-    const double d = (double)xi * (double)mi - mean * (double)mi;  // x_masked - mean * mask
-    q += d * d;
+    if (PASS == 0) {
+      s += (double)xi * (double)mi;
+      f += (double)mi;
+    } else {
+      bool as_float;
+      const double mean = mean_at(a, stats, i, xi, mi, as_float);
+      const double d = (double)xi * (double)mi - mean * (double)mi;  // x_masked - mean * mask
+      s += d * d;
+    }
   }
-  q = block_sum<double>(q, smem);
-  if (threadIdx.x == 0) stats[blockIdx.x].z = q;
+  s = block_sum<double>(s, smem);
+  if (PASS == 0) f = block_sum<double>(f, smem);
+  if (threadIdx.x == 0) partial[blockIdx.x] = make_double2(s, f);
+}
+
+template <int PASS>
+__global__ __launch_bounds__(kWave) void k_norm_finish(const double2* __restrict__ partial, int parts, int segs,
+                                                       double4* __restrict__ stats) {
+  const int seg = blockIdx.x * kWave + threadIdx.x;
+  if (seg >= segs) return;
+  double s = 0.0, f = 0.0;
+  for (int p = 0; p < parts; ++p) {
+    s += partial[seg * parts + p].x;
+    f += partial[seg * parts + p].y;
+  }
+  if (PASS == 0) stats[seg] = make_double4(s, f, 0.0, 0.0);
+  else stats[seg].z = s;
 }
 
 __device__ __forceinline__ double level_std(double Q, double F, bool unbiased) {
@@ -316,9 +339,15 @@ extern "C" int aa_gae(const float* rewards, const float* values, const float* lo
   return launch_status();
 }
 
-extern "C" int64_t aa_normalize_scratch_bytes(int64_t bs, int64_t group_size) {
-  if (bs < 0 || group_size < 1) return -1;
-  return (int64_t)sizeof(double4) * (1 + bs / group_size);
+static int norm_parts(int64_t n) {
+  int64_t p = (n + 8191) / 8192;
+  return (int)(p < 1 ? 1 : (p > 256 ? 256 : p));
+}
+
+extern "C" int64_t aa_normalize_scratch_bytes(int64_t bs, int64_t inner, int64_t group_size) {
+  if (bs < 0 || inner < 1 || group_size < 1) return -1;
+  const int64_t segs = 1 + bs / group_size;
+  return segs * (int64_t)sizeof(double4) + segs * norm_parts(bs * inner) * (int64_t)sizeof(double2);
 }
 
 extern "C" int aa_normalize(const float* x, const float* loss_mask, int64_t bs, int64_t inner,
@@ -332,15 +361,24 @@ extern "C" int aa_normalize(const float* x, const float* loss_mask, int64_t bs, 
   if (bs == 0) return AA_OK;
   const int64_t gs = grouped ? p.group_size : bs;
   const int64_t n_groups = grouped ? bs / gs : 0;
-  if (scratch_bytes < (int64_t)sizeof(double4) * (1 + n_groups) || (((uintptr_t)scratch) & 31))
-    return AA_ERR_INVALID_ARGUMENT;
+  const int64_t segs = 1 + n_groups;
+  const int parts = norm_parts(bs * inner);
+  if (segs * parts > (int64_t)0x7fffffff) return AA_ERR_UNSUPPORTED;
+  const int64_t need = segs * (int64_t)sizeof(double4) + segs * parts * (int64_t)sizeof(double2);
+  if (scratch_bytes < need || (((uintptr_t)scratch) & 31)) return AA_ERR_INVALID_ARGUMENT;
   NormArgs a{x, loss_mask, bs * inner, gs * inner, n_groups, gs, p.mean_level, p.mean_leave1out, p.std_level,
              p.std_unbiased, p.eps};
   hipStream_t st = (hipStream_t)stream;
   double4* stats = (double4*)scratch;
-  const unsigned segs = (unsigned)(1 + n_groups);
-  hipLaunchKernelGGL(k_norm_sums, dim3(segs), dim3(kThreads), 0, st, a, stats);
-  if (p.std_level != 0) hipLaunchKernelGGL(k_norm_sumsq, dim3(segs), dim3(kThreads), 0, st, a, stats);
+  double2* partial = (double2*)(stats + segs);
+  const unsigned fin = (unsigned)((segs + kWave - 1) / kWave);
+  hipLaunchKernelGGL(k_norm_partial<0>, dim3((unsigned)(segs * parts)), dim3(kThreads), 0, st, a, stats, parts, partial);
+  hipLaunchKernelGGL(k_norm_finish<0>, dim3(fin), dim3(kWave), 0, st, partial, parts, (int)segs, stats);
+  if (p.std_level != 0) {
+    hipLaunchKernelGGL(k_norm_partial<1>, dim3((unsigned)(segs * parts)), dim3(kThreads), 0, st, a, stats, parts,
+                       partial);
+    hipLaunchKernelGGL(k_norm_finish<1>, dim3(fin), dim3(kWave), 0, st, partial, parts, (int)segs, stats);
+  }
   int64_t blocks = (a.n + 255) / 256;
   if (blocks > 4096) blocks = 4096;
   hipLaunchKernelGGL(k_norm_apply, dim3((unsigned)blocks), dim3(256), 0, st, a, stats, out);

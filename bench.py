@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the PPO/GRPO log-prob + entropy + actor-loss path (forward and backward) on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg1|cfg1-32k|cfg0|cfg2|cfg3|cfg4]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg1|cfg1-32k|cfg0|cfg2|cfg3|cfg4|adv]
 
 One "step" is one pass of the hot path over one synthetic packed micro-batch that is already resident in HBM.
 
@@ -13,6 +13,10 @@ One "step" is one pass of the hot path over one synthetic packed micro-batch tha
   ``loss.backward()``: lm_head, log-prob / entropy, PPO loss and the gradients d(hidden), d(W), token chunk by
   token chunk, the full [T, V] logits never in memory.  Roofline: bf16 MFMA, algorithmic flops 6 * T * V * H
   (logits 2TVH, the two gradient GEMMs 4TVH).
+
+* adv: the advantage pipeline that precedes the loss (not a BASELINE configuration): GAE reverse scan plus batch
+  normalisation over a padded [512, 4096] batch.  Roofline: HBM, 20 bytes per token for the scan (rewards, values,
+  mask read; advantages, returns written).
 
 Prints ONE JSON line.  Besides the whole-step throughput it carries
   roofline      of the dominant kernel(s), timed with HIP events on the launch stream;
@@ -40,6 +44,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published peak
 METRIC = "tokens/sec for logprob+entropy+PPO loss fwd+bwd"
 LOGITS_WORKLOADS = ("cfg0", "cfg1", "cfg1-32k")
 FUSED_WORKLOADS = ("cfg2", "cfg3", "cfg4")
+ADV_WORKLOADS = ("adv",)
 
 
 def parse_args():
@@ -47,7 +52,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="cfg1", choices=LOGITS_WORKLOADS + FUSED_WORKLOADS)
+    ap.add_argument("--workload", default="cfg1", choices=LOGITS_WORKLOADS + FUSED_WORKLOADS + ADV_WORKLOADS)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--cpu-tokens", type=int, default=1024,
                     help="token sample of the CPU baseline (0 = skip); fused lm_head workloads use at most 128")
@@ -492,6 +497,79 @@ def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: i
         out["parity"] = parity
     return out
 
+# ----------------------------------------------------------------------------------------------------------------
+# advantage pipeline
+# ----------------------------------------------------------------------------------------------------------------
+def bench_adv(args, dev):
+    import torch
+
+    import areal_amd
+    from areal_amd import NormConfig, Normalization
+    from oracle import advantages as O
+
+    bs, L = 512, 4096
+    g = torch.Generator().manual_seed(args.seed)
+    lens = torch.randint(L // 4, L + 1, (bs,), generator=g)
+    pos = torch.arange(L)[None, :]
+    mask = ((pos >= (lens[:, None] * 0.3).long()) & (pos < lens[:, None] - 1)).float()
+    rewards = torch.zeros(bs, L)
+    rewards[torch.arange(bs), (lens - 2).clamp(min=0)] = torch.randn(bs, generator=g)
+    rewards = rewards - 0.01 * torch.rand(bs, L, generator=g) * mask
+    values = torch.randn(bs, L, generator=g) * 0.1
+    no_eos = lens == L
+    d = [t.to(dev) for t in (rewards, values, mask, no_eos)]
+    norm = Normalization(NormConfig(mean_level="batch", std_level="batch"))
+
+    def step():
+        adv, ret = areal_amd.gae_advantages(d[0], d[1], d[2], d[3], 1.0, 0.95)
+        return norm(adv, d[2]), ret
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out, ret = step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+
+    from areal_amd import _native as N
+    from areal_amd import functional as F
+
+    lib = N.load()
+    adv = torch.empty_like(d[0])
+    ret = torch.empty_like(d[0])
+    ne8 = F._mask_u8(d[3])
+    stream = torch.cuda.current_stream(dev)
+
+    def launch():
+        N.check(lib.aa_gae(F._ptr(d[0]), F._ptr(d[1]), F._ptr(d[2]), F._ptr(ne8), bs, L, 1.0, 0.95, F._ptr(adv),
+                           F._ptr(ret), C.c_void_p(stream.cuda_stream)), "aa_gae")
+
+    k_ms, k_min = time_events(launch, max(args.steps, 10), stream)
+    alg_bytes = 20.0 * bs * L
+    achieved = alg_bytes / (k_ms * 1e-3) / 1e9
+    t0 = time.perf_counter()
+    w_adv, _ = O.gae(rewards, values, mask, no_eos.float(), 1.0, 0.95)
+    w_out = O.normalization(w_adv, mask)
+    cpu_s = time.perf_counter() - t0
+    return dict(
+        metric="tokens/sec for GAE + advantage normalisation", value=bs * L / (ms_per_step * 1e-3), unit="tokens/s",
+        n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=ms_per_step, higher_is_better=True,
+        scaling="weak", vs_baseline=None, dtype="f32", data="synthetic",
+        config=dict(workload="adv: padded batch [512, 4096], one terminal reward per sequence plus KL penalties, "
+                             "critic values, gamma 1, lambda 0.95, batch-level mean / std normalisation",
+                    sequences=bs, max_seqlen=L),
+        roofline=dict(bound="hbm", kernel="k_gae (aa_gae)", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s",
+                      frac=achieved / HBM_PEAK_GBS, traffic=None, avg_kernel_ms=k_ms, min_kernel_ms=k_min,
+                      algorithmic_bytes_per_launch=alg_bytes),
+        cpu_baseline=dict(value=bs * L / cpu_s, unit="tokens/s", cores=torch.get_num_threads(), kind="port",
+                          sample="the whole workload once: the reference's Python loop over max_seqlen (4095 steps "
+                                 "of [512]-wide tensor ops) and Normalization, restated in the CPU oracle"),
+        parity=dict(adv_max_abs_err=float((out.cpu() - w_out).abs().max()),
+                    returns_max_abs_err=float((ret.cpu() - (w_adv + values)).abs().max())),
+    )
+
 
 def main():
     args = parse_args()
@@ -505,7 +583,9 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    if args.workload in LOGITS_WORKLOADS:
+    if args.workload in ADV_WORKLOADS:
+        out = bench_adv(args, dev)
+    elif args.workload in LOGITS_WORKLOADS:
         out = bench_logits(args, dev)
         if args.workload == "cfg1" and not args.no_fused_extra and args.copy_launches == 0:
             torch.cuda.empty_cache()

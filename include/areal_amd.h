@@ -221,7 +221,8 @@ typedef struct {
 } aa_norm_params;
 
 /* Bytes of scratch aa_normalize needs (32-byte aligned device memory). */
-int64_t aa_normalize_scratch_bytes(int64_t bs, int64_t group_size);
+int64_t aa_normalize_scratch_bytes(int64_t bs, int64_t inner,
+                                   int64_t group_size);
 
 /*
  * out = Normalization(params)(x, loss_mask) for x [bs, inner] float32
