@@ -3,6 +3,7 @@
 Importing the package does not load the HIP library; the first op call does, and
 raises ``NativeLibraryError`` if ``libareal_amd.so`` has not been built.
 """
+from .actor_ops import apply_m2po_masking, compute_prox_logp_approximations
 from .advantages import Normalization, gae_advantages, masked_moments
 from .config import NormConfig, RejectionSamplingConfig
 from .functional import (
@@ -15,6 +16,8 @@ from .functional import (
     gather_logprobs_entropy_stats,
     lm_head_logprobs_entropy,
     ppo_actor_loss_fn,
+    ppo_critic_loss_fn,
+    sapo_loss_fn,
 )
 from ._native import NativeLibraryError
 
@@ -26,7 +29,9 @@ __all__ = [
     "Normalization",
     "RejectionSamplingConfig",
     "RejectionSamplingResult",
+    "apply_m2po_masking",
     "apply_rejection_sampling",
+    "compute_prox_logp_approximations",
     "fused_lm_head_ppo_loss",
     "fused_logprobs_ppo_loss",
     "gae_advantages",
@@ -36,4 +41,6 @@ __all__ = [
     "lm_head_logprobs_entropy",
     "masked_moments",
     "ppo_actor_loss_fn",
+    "ppo_critic_loss_fn",
+    "sapo_loss_fn",
 ]

@@ -284,7 +284,7 @@ __global__ __launch_bounds__(1024) void k_masked_sum(const float* __restrict__ v
   __shared__ double smem[1024 / kWave];
   double acc = 0.0;
   for (int64_t i = threadIdx.x; i < n; i += 1024)
-    if (mask[i] != 0) acc += (double)values[i];
+    if (!mask || mask[i] != 0) acc += (double)values[i];
   acc = block_sum<double>(acc, smem);
   if (threadIdx.x == 0) {
     int nv = n_valid ? *n_valid : 1;
@@ -292,6 +292,162 @@ __global__ __launch_bounds__(1024) void k_masked_sum(const float* __restrict__ v
     float r = (float)acc / (float)nv;
     if (scale) r *= *scale;
     out[0] = r;
+  }
+}
+
+// ---- SAPO: soft sigmoid gates instead of clipping (functional.py:562-638) ---------------------------------------
+struct SapoTerm {
+  float loss, dloss_dr, soft, gate_pos, gate_neg;
+};
+
+__device__ __forceinline__ float sigmoidf(float z) { return 1.f / (1.f + expf(-z)); }
+
+__device__ __forceinline__ SapoTerm sapo_term(float r, float adv, float tau_pos, float tau_neg) {
+  const float gp = sigmoidf(tau_pos * (r - 1.f)), gn = sigmoidf(tau_neg * (r - 1.f));
+  SapoTerm o;
+  o.gate_pos = gp * (4.f / tau_pos);
+  o.gate_neg = gn * (4.f / tau_neg);
+  const bool pos = adv > 0.f;
+  o.soft = pos ? o.gate_pos : o.gate_neg;
+  o.loss = -o.soft * adv;
+  const float g = pos ? gp : gn;
+  o.dloss_dr = -4.f * adv * g * (1.f - g);  // (4 / tau) * sigmoid'(tau (r - 1)) * tau
+  return o;
+}
+
+__global__ __launch_bounds__(256) void k_sapo_token(const float* __restrict__ logp, const float* __restrict__ old,
+                                                    const float* __restrict__ adv, const uint8_t* __restrict__ mask,
+                                                    int64_t n, float tau_pos, float tau_neg,
+                                                    const int32_t* __restrict__ n_valid, float* __restrict__ stat_loss,
+                                                    float* __restrict__ ratio, float* __restrict__ gates,
+                                                    float* __restrict__ g_logp) {
+  int nv = *n_valid;
+  if (nv < 1) nv = 1;
+  const float fn = (float)nv;
+  const int64_t step = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += step) {
+    const float r = expf(logp[i] - old[i]);  // not masked: functional.py:600
+    const SapoTerm t = sapo_term(r, adv[i], tau_pos, tau_neg);
+    stat_loss[i] = t.loss;
+    ratio[i] = r;
+    gates[i] = t.soft;
+    gates[n + i] = t.gate_pos;
+    gates[2 * n + i] = t.gate_neg;
+    g_logp[i] = mask[i] != 0 ? t.dloss_dr * r / fn : 0.f;
+  }
+}
+
+__global__ __launch_bounds__(kSegThreads) void k_sapo_sequence(const float* __restrict__ logp,
+                                                               const float* __restrict__ old,
+                                                               const float* __restrict__ adv,
+                                                               const uint8_t* __restrict__ mask, Segments seg,
+                                                               float tau_pos, float tau_neg,
+                                                               const int32_t* __restrict__ n_valid,
+                                                               float* __restrict__ stat_loss,
+                                                               float* __restrict__ ratio, float* __restrict__ gates,
+                                                               float* __restrict__ g_logp) {
+  __shared__ double smem_d[kSegThreads / kWave];
+  __shared__ int smem_i[kSegThreads / kWave];
+  const int64_t b = blockIdx.x, n = seg.n;
+  int64_t beg, end;
+  seg.range(b, beg, end);
+  double slr = 0.0, sadv = 0.0;
+  int cnt = 0;
+  const bool tail = b == seg.B;  // tokens no sequence covers: ratio 0, advantage 0
+  if (!tail) {
+    for (int64_t i = beg + threadIdx.x; i < end; i += kSegThreads) {
+      if (mask[i] != 0) {
+        slr += (double)(logp[i] - old[i]);
+        sadv += (double)adv[i];
+        cnt += 1;
+      }
+    }
+  }
+  const float f_slr = (float)block_sum<double>(slr, smem_d);
+  const float f_sadv = (float)block_sum<double>(sadv, smem_d);
+  const int raw = block_sum<int>(cnt, smem_i);
+  const float fcnt = (float)(raw < 1 ? 1 : raw);
+  const float r_seq = expf(f_slr / fcnt);
+  const float a_seq = f_sadv / fcnt;
+  double gsum = 0.0;
+  for (int64_t i = beg + threadIdx.x; i < end; i += kSegThreads) {
+    const bool m = !tail && mask[i] != 0;
+    const SapoTerm t = sapo_term(m ? r_seq : 0.f, m ? a_seq : 0.f, tau_pos, tau_neg);
+    stat_loss[i] = t.loss;
+    ratio[i] = m ? r_seq : 0.f;
+    gates[i] = t.soft;
+    gates[n + i] = t.gate_pos;
+    gates[2 * n + i] = t.gate_neg;
+    if (m) gsum += (double)t.dloss_dr;
+  }
+  const float G = (float)block_sum<double>(gsum, smem_d);
+  int nv = *n_valid;
+  if (nv < 1) nv = 1;
+  const float gk = G * r_seq / fcnt / (float)nv;
+  for (int64_t i = beg + threadIdx.x; i < end; i += kSegThreads) g_logp[i] = (!tail && mask[i] != 0) ? gk : 0.f;
+}
+
+// ---- clipped value loss of the critic (functional.py:704-778) ---------------------------------------------------
+__device__ __forceinline__ void value_loss_term(int huber, float x, float y, float& loss, float& dx) {
+  const float e = x - y;
+  if (!huber) {
+    loss = 0.5f * e * e;
+    dx = e;
+    return;
+  }
+  const float delta = 10.f, diff = fabsf(e);
+  if (diff < delta) {
+    loss = 0.5f * diff * diff;
+    dx = e;
+  } else {
+    loss = delta * (diff - 0.5f * delta);
+    dx = e > 0.f ? delta : -delta;
+  }
+}
+
+__global__ __launch_bounds__(256) void k_critic_loss(const float* __restrict__ value, const float* __restrict__ old,
+                                                     const float* __restrict__ target,
+                                                     const uint8_t* __restrict__ mask, int64_t n, float eps,
+                                                     int huber, const int32_t* __restrict__ n_valid,
+                                                     float* __restrict__ stat_loss, uint8_t* __restrict__ clip,
+                                                     float* __restrict__ g_value) {
+  // the reference divides by count_nonzero (or by n without a mask) with no floor: an empty mask gives 0 / 0
+  const float fn = (float)(*n_valid);
+  const int64_t step = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += step) {
+    const float v = value[i], o = old[i], y = target[i];
+    const float d = v - o;
+    const float dc = nan_min(nan_max(d, -eps), eps);
+    const bool in_range = (d >= -eps) && (d <= eps);
+    float l1, g1, l2, g2;
+    value_loss_term(huber, v, y, l1, g1);
+    value_loss_term(huber, o + dc, y, l2, g2);
+    const bool m = mask ? mask[i] != 0 : true;
+    const float w1 = (l1 == l2) ? 0.5f : ((l1 > l2) ? 1.f : 0.f);
+    stat_loss[i] = nan_max(l1, l2);
+    clip[i] = (uint8_t)((l2 > l1 && m) ? 1 : 0);
+    g_value[i] = m ? (w1 * g1 + (in_range ? (1.f - w1) * g2 : 0.f)) / fn : 0.f;
+  }
+}
+
+// ---- proximal log-prob approximations from per-token policy versions (actor.py:604-684) --------------------------
+__global__ __launch_bounds__(256) void k_prox_approx(const float* __restrict__ old, const float* __restrict__ logp,
+                                                     const int32_t* __restrict__ versions, int64_t n,
+                                                     int current_version, int method, float* __restrict__ out) {
+  const float v_theta = (float)current_version, v_prox = (float)(current_version - 1);
+  const int64_t step = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += step) {
+    const int ver = versions[i];
+    const float vb = (float)ver;
+    const float diff = v_theta - vb, gap = v_prox - vb;
+    float alpha = (diff > 0.f && ver >= 0) ? gap / diff : 0.f;
+    alpha = fminf(fmaxf(alpha, 0.f), 1.f);
+    const float lo = old[i], ln = logp[i];
+    float r;
+    if (method == 0) r = lo + alpha * (ln - lo);
+    else if (method == 1) r = logf((1.f - alpha) * expf(lo) + alpha * expf(ln) + 1e-10f);
+    else r = lo;
+    out[i] = r;
   }
 }
 
@@ -363,7 +519,50 @@ extern "C" int aa_ppo_loss(const float* logp, const float* prox_logp, const floa
 
 extern "C" int aa_masked_sum(const float* values, const uint8_t* mask, int64_t n, const int32_t* n_valid,
                              const float* scale, float* out, void* stream) {
-  if (!out || n < 0 || (n > 0 && (!values || !mask))) return AA_ERR_INVALID_ARGUMENT;
+  if (!out || n < 0 || (n > 0 && !values)) return AA_ERR_INVALID_ARGUMENT;
   hipLaunchKernelGGL(k_masked_sum, dim3(1), dim3(1024), 0, (hipStream_t)stream, values, mask, n, n_valid, scale, out);
+  return launch_status();
+}
+
+extern "C" int aa_sapo_loss(const float* logp, const float* old_logp, const float* adv, const uint8_t* mask, int64_t n,
+                            const int32_t* cu_seqlens, int64_t B, int sequence_level, float tau_pos, float tau_neg,
+                            const int32_t* n_valid, float* stat_loss, float* ratio, float* gates, float* g_logp,
+                            void* stream) {
+  if (!n_valid || n < 0 || !(tau_pos > 0.f) || !(tau_neg > 0.f)) return AA_ERR_INVALID_ARGUMENT;
+  if (n == 0) return AA_OK;
+  if (!logp || !old_logp || !adv || !mask || !stat_loss || !ratio || !gates || !g_logp) return AA_ERR_INVALID_ARGUMENT;
+  hipStream_t st = (hipStream_t)stream;
+  if (!sequence_level) {
+    hipLaunchKernelGGL(k_sapo_token, dim3(grid_for(n)), dim3(256), 0, st, logp, old_logp, adv, mask, n, tau_pos,
+                       tau_neg, n_valid, stat_loss, ratio, gates, g_logp);
+  } else {
+    if (B <= 0 || B > 0x7ffffffe) return AA_ERR_INVALID_ARGUMENT;
+    if (!cu_seqlens && (n % B) != 0) return AA_ERR_INVALID_ARGUMENT;
+    Segments seg{cu_seqlens, B, n};
+    hipLaunchKernelGGL(k_sapo_sequence, dim3((unsigned)(B + 1)), dim3(kSegThreads), 0, st, logp, old_logp, adv, mask,
+                       seg, tau_pos, tau_neg, n_valid, stat_loss, ratio, gates, g_logp);
+  }
+  return launch_status();
+}
+
+extern "C" int aa_critic_loss(const float* value, const float* old_value, const float* target_value,
+                              const uint8_t* mask, int64_t n, float value_eps_clip, int loss_type,
+                              const int32_t* n_valid, float* stat_loss, uint8_t* clip_mask, float* g_value,
+                              void* stream) {
+  if (!n_valid || n < 0 || loss_type < 0 || loss_type > 1) return AA_ERR_INVALID_ARGUMENT;
+  if (n == 0) return AA_OK;
+  if (!value || !old_value || !target_value || !stat_loss || !clip_mask || !g_value) return AA_ERR_INVALID_ARGUMENT;
+  hipLaunchKernelGGL(k_critic_loss, dim3(grid_for(n)), dim3(256), 0, (hipStream_t)stream, value, old_value,
+                     target_value, mask, n, value_eps_clip, loss_type, n_valid, stat_loss, clip_mask, g_value);
+  return launch_status();
+}
+
+extern "C" int aa_prox_logp_approx(const float* old_logp, const float* logp, const int32_t* versions, int64_t n,
+                                   int current_version, int method, float* out, void* stream) {
+  if (n < 0 || method < 0 || method > 2) return AA_ERR_INVALID_ARGUMENT;
+  if (n == 0) return AA_OK;
+  if (!old_logp || !logp || !versions || !out) return AA_ERR_INVALID_ARGUMENT;
+  hipLaunchKernelGGL(k_prox_approx, dim3(grid_for(n)), dim3(256), 0, (hipStream_t)stream, old_logp, logp, versions, n,
+                     current_version, method, out);
   return launch_status();
 }

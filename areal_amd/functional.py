@@ -848,3 +848,144 @@ def fused_lm_head_ppo_loss(
     if rejection_sampling is not None:
         _rs_stats(stat, prox, old, mask_eff, w, counts, loss_mask.shape)
     return loss, stat
+
+
+# ----------------------------------------------------------------------------
+# sibling losses: SAPO, clipped value loss of the critic
+# ----------------------------------------------------------------------------
+class _SapoLoss(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logp, old, adv, mask, cu, B, seq_level, tau_pos, tau_neg, n_valid):
+        lib = N.load()
+        dev = logp.device
+        n = logp.numel()
+        f32 = dict(dtype=torch.float32, device=dev)
+        stat_loss, ratio, g_logp = (torch.empty(n, **f32) for _ in range(3))
+        gates = torch.empty(3, n, **f32)
+        loss = torch.empty((), **f32)
+        with torch.cuda.device(dev):
+            st = _stream(dev)
+            N.check(
+                lib.aa_sapo_loss(_ptr(logp), _ptr(old), _ptr(adv), _ptr(mask), n, _ptr(cu), B, 1 if seq_level else 0,
+                                 float(tau_pos), float(tau_neg), _ptr(n_valid), _ptr(stat_loss), _ptr(ratio),
+                                 _ptr(gates), _ptr(g_logp), st),
+                "aa_sapo_loss",
+            )
+            N.check(lib.aa_masked_sum(_ptr(stat_loss), _ptr(mask), n, _ptr(n_valid), None, _ptr(loss), st),
+                    "aa_masked_sum")
+        ctx.save_for_backward(g_logp)
+        ctx.mark_non_differentiable(stat_loss, ratio, gates)
+        return loss, stat_loss, ratio, gates
+
+    @staticmethod
+    def backward(ctx, g_loss, *_unused):
+        (g_logp,) = ctx.saved_tensors
+        return (g_logp * g_loss,) + (None,) * 9
+
+
+def sapo_loss_fn(
+    logprobs: torch.Tensor,
+    old_logprobs: torch.Tensor,
+    advantages: torch.Tensor,
+    tau_pos: float,
+    tau_neg: float,
+    loss_mask: torch.Tensor,
+    importance_sampling_level: str = "token",
+    cu_seqlens: torch.Tensor | None = None,
+) -> tuple[torch.Tensor, dict]:
+    """SAPO loss with asymmetric sigmoid gates; functional.py:562-638, same stat keys."""
+    if tau_pos <= 0 or tau_neg <= 0:
+        raise ValueError("SAPO temperatures (tau_pos, tau_neg) must be positive.")
+    if importance_sampling_level not in ("token", "sequence"):
+        raise ValueError(
+            f"Invalid importance_sampling_level: {importance_sampling_level}. Must be 'token' or 'sequence'."
+        )
+    _require_gpu(logprobs, "logprobs")
+    shape = logprobs.shape
+    seq_level = importance_sampling_level == "sequence"
+    cu, B = None, 0
+    if seq_level:
+        cu, B = _segments(
+            shape,
+            cu_seqlens,
+            "cu_seqlens is required for 1D tensors (packed format). For a single sequence, use "
+            "cu_seqlens=torch.tensor([0, seq_len], dtype=torch.int32).",
+        )
+        if cu is not None:
+            cu = cu.to(logprobs.device)
+    lp = _f32(logprobs).reshape(-1)
+    old = _f32(old_logprobs.detach()).reshape(-1)
+    adv = _f32(advantages.detach()).reshape(-1)
+    m8 = _mask_u8(loss_mask).reshape(-1)
+    n_valid = _count_nonzero(m8)
+    loss, stat_loss, ratio, gates = _SapoLoss.apply(lp, old, adv, m8, cu, B, seq_level, tau_pos, tau_neg, n_valid)
+    zeros = torch.zeros(shape, dtype=torch.bool, device=lp.device)
+    stat = dict(
+        loss=stat_loss.view(shape),
+        importance_weight=ratio.view(shape),
+        approx_kl=(lp.detach() - old).view(shape),
+        clip_mask=zeros,
+        dual_clip_mask=zeros.clone(),
+        sapo_soft_gate=gates[0].view(shape),
+        sapo_scaled_gate_pos=gates[1].view(shape),
+        sapo_scaled_gate_neg=gates[2].view(shape),
+    )
+    return loss, stat
+
+
+class _CriticLoss(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, value, old, target, mask, eps, loss_type, n_valid):
+        lib = N.load()
+        dev = value.device
+        n = value.numel()
+        f32 = dict(dtype=torch.float32, device=dev)
+        stat_loss, g_value = torch.empty(n, **f32), torch.empty(n, **f32)
+        clip = torch.empty(n, dtype=torch.uint8, device=dev)
+        total = torch.empty((), **f32)
+        with torch.cuda.device(dev):
+            st = _stream(dev)
+            N.check(
+                lib.aa_critic_loss(_ptr(value), _ptr(old), _ptr(target), _ptr(mask), n, float(eps), loss_type,
+                                   _ptr(n_valid), _ptr(stat_loss), _ptr(clip), _ptr(g_value), st),
+                "aa_critic_loss",
+            )
+            N.check(lib.aa_masked_sum(_ptr(stat_loss), _ptr(mask), n, None, None, _ptr(total), st), "aa_masked_sum")
+        loss = total / n_valid[0].to(torch.float32)  # no floor: an empty mask gives NaN, as in the reference
+        ctx.save_for_backward(g_value)
+        ctx.mark_non_differentiable(stat_loss, clip)
+        return loss, stat_loss, clip
+
+    @staticmethod
+    def backward(ctx, g_loss, *_unused):
+        (g_value,) = ctx.saved_tensors
+        return (g_value * g_loss,) + (None,) * 6
+
+
+def ppo_critic_loss_fn(
+    value: torch.Tensor,
+    old_value: torch.Tensor,
+    target_value: torch.Tensor,
+    value_eps_clip: float,
+    loss_mask: torch.Tensor | None = None,
+    loss_fn_type: str = "mse",
+) -> tuple[torch.Tensor, dict]:
+    """Clipped value loss of the PPO critic; functional.py:704-778 (stat keys ``clip_mask``, ``loss``)."""
+    assert value.dtype == torch.float32
+    assert old_value.dtype == torch.float32
+    assert target_value.dtype == torch.float32
+    if loss_fn_type not in ("mse", "huber"):
+        raise NotImplementedError(f"Unknown loss fn type: {loss_fn_type}")
+    _require_gpu(value, "value")
+    shape = value.shape
+    v = value.contiguous().reshape(-1)
+    o = old_value.detach().contiguous().reshape(-1)
+    t = target_value.detach().contiguous().reshape(-1)
+    if loss_mask is not None:
+        m8 = _mask_u8(loss_mask).reshape(-1)
+        n_valid = _count_nonzero(m8)
+    else:
+        m8 = None
+        n_valid = torch.full((1,), v.numel(), dtype=torch.int32, device=v.device)
+    loss, stat_loss, clip = _CriticLoss.apply(v, o, t, m8, value_eps_clip, 0 if loss_fn_type == "mse" else 1, n_valid)
+    return loss, dict(clip_mask=clip.bool().view(shape), loss=stat_loss.view(shape))

@@ -177,7 +177,8 @@ int aa_ppo_loss(const float* logp, const float* prox_logp, const float* adv,
 /*
  * out[0] = scale * sum_{i<n, mask[i] != 0} values[i] / max(*n_valid, 1)
  * (functional.py:542), accumulated in a fixed order so that repeated calls are
- * bit-identical.  n_valid may be NULL (divide by 1); scale may be NULL (1).
+ * bit-identical.  n_valid may be NULL (divide by 1); scale may be NULL (1);
+ * mask may be NULL (every element counts).
  */
 int aa_masked_sum(const float* values, const uint8_t* mask, int64_t n,
                   const int32_t* n_valid, const float* scale, float* out,
@@ -186,6 +187,64 @@ int aa_masked_sum(const float* values, const uint8_t* mask, int64_t n,
 /* data[i] *= *factor for i < n (dtype as aa_dtype); a no-op when *factor == 1. */
 int aa_scale_inplace(void* data, int dtype, int64_t n, const float* factor,
                      void* stream);
+
+/* ------------------------------------------------------------------ */
+/* Sibling losses and actor-side token filters                            */
+/* ------------------------------------------------------------------ */
+
+/*
+ * sapo_loss_fn (functional.py:562-638): asymmetric sigmoid gates in place of
+ * clipping, forward and closed-form backward.  ratio = exp(logp - old_logp)
+ * (token level, unmasked) or the per-sequence geometric mean
+ * (sequence_level != 0, segments as in aa_ppo_loss).
+ * Outputs [n]: stat_loss = -soft_gate * adv, ratio, g_logp; gates [3, n] =
+ * {soft gate, scaled positive gate, scaled negative gate}.  The scalar loss
+ * is aa_masked_sum(stat_loss, mask, n_valid).
+ */
+int aa_sapo_loss(const float* logp, const float* old_logp, const float* adv,
+                 const uint8_t* mask, int64_t n, const int32_t* cu_seqlens,
+                 int64_t B, int sequence_level, float tau_pos, float tau_neg,
+                 const int32_t* n_valid, float* stat_loss, float* ratio,
+                 float* gates, float* g_logp, void* stream);
+
+/*
+ * ppo_critic_loss_fn (functional.py:704-778): clipped value loss, forward and
+ * closed-form backward (torch.max ties split in half, clamp passes gradient
+ * on the closed interval).  loss_type 0 = mse, 1 = huber (delta 10).
+ * mask may be NULL (plain mean); *n_valid is the divisor (count of non-zero
+ * mask bytes, or n) and is NOT floored at 1, as in the reference.
+ * Outputs [n]: stat_loss = max(original, clipped), clip_mask bytes, g_value.
+ */
+int aa_critic_loss(const float* value, const float* old_value,
+                   const float* target_value, const uint8_t* mask, int64_t n,
+                   float value_eps_clip, int loss_type, const int32_t* n_valid,
+                   float* stat_loss, uint8_t* clip_mask, float* g_value,
+                   void* stream);
+
+/*
+ * compute_prox_logp_approximations (areal/trainer/ppo/actor.py:604-684):
+ * method 0 = loglinear, 1 = linear (probability space), 2 = rollout.
+ * versions: per-token policy version, int32, negative for prompt tokens.
+ */
+int aa_prox_logp_approx(const float* old_logp, const float* logp,
+                        const int32_t* versions, int64_t n,
+                        int current_version, int method, float* out,
+                        void* stream);
+
+/* Bytes of 256-byte aligned workspace aa_m2po_mask needs for n tokens. */
+int64_t aa_m2po_workspace_bytes(int64_t n);
+
+/*
+ * _apply_m2po_masking (areal/trainer/ppo/actor.py:769-850): among the tokens
+ * with mask_in != 0, clear those with the largest (old_logp - prox_logp)^2
+ * until the mean of the rest is below m2_threshold (at least one token is
+ * kept).  mask_out [n] bytes; info[0] = selected tokens, info[1] = tokens
+ * cleared.  Equal values are cleared in index order.
+ */
+int aa_m2po_mask(const float* old_logp, const float* prox_logp,
+                 const uint8_t* mask_in, int64_t n, float m2_threshold,
+                 uint8_t* mask_out, int32_t* info, void* workspace,
+                 int64_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------ */
 /* Advantage pipeline (rows are sequences of a padded [bs, L] batch)      */

@@ -25,6 +25,7 @@ from .ppo import (
     sequence_level_ratio_and_advantages,
 )
 from .advantages import gae, masked_moments, normalization
+from .siblings import critic_loss, m2po_mask, prox_logp_approximations, sapo_loss
 from .pipeline import lmhead_logits, logits_ppo_step
 
 __all__ = [
@@ -40,6 +41,10 @@ __all__ = [
     "gae",
     "masked_moments",
     "normalization",
+    "critic_loss",
+    "m2po_mask",
+    "prox_logp_approximations",
+    "sapo_loss",
     "lmhead_logits",
     "logits_ppo_step",
 ]

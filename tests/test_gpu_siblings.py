@@ -1,0 +1,143 @@
+"""GPU parity of the sibling losses (SAPO, clipped value loss) and the actor-side filters (proximal log-prob
+approximations, M2PO masking) against the CPU oracle and the reference's known answers."""
+import pytest
+import torch
+
+import areal_amd
+from helpers import cosine
+from oracle import siblings as S
+
+pytestmark = pytest.mark.gpu
+
+
+def _tok(n, seed):
+    g = torch.Generator().manual_seed(seed)
+    lp = -torch.rand(n, generator=g) * 3
+    old = lp + 0.3 * torch.randn(n, generator=g)
+    adv = torch.randn(n, generator=g)
+    mask = torch.rand(n, generator=g) < 0.7
+    return lp, old, adv, mask
+
+
+@pytest.mark.parametrize("level", ["token", "sequence"])
+@pytest.mark.parametrize("tau_pos,tau_neg", [(1.0, 1.05), (2.5, 0.7)])
+def test_sapo_matches_oracle(device, level, tau_pos, tau_neg):
+    n = 777
+    lp, old, adv, mask = _tok(n, 3)
+    adv[5] = 0.0
+    cu = torch.tensor([0, 100, 101, 400, 777], dtype=torch.int32)
+    mask[100:101] = False  # a sequence with no valid token
+    x = lp.clone().requires_grad_(True)
+    w_loss, w_stat = S.sapo_loss(x, old, adv, tau_pos, tau_neg, mask, level, cu)
+    w_loss.backward()
+    y = lp.to(device).requires_grad_(True)
+    loss, stat = areal_amd.sapo_loss_fn(y, old.to(device), adv.to(device), tau_pos, tau_neg, mask.to(device), level,
+                                        cu.to(device))
+    loss.backward()
+    assert float(loss.detach()) == pytest.approx(float(w_loss.detach()), rel=1e-5, abs=1e-7)
+    for k in ("loss", "importance_weight", "approx_kl", "sapo_soft_gate", "sapo_scaled_gate_pos",
+              "sapo_scaled_gate_neg"):
+        assert torch.allclose(stat[k].cpu(), w_stat[k], rtol=2e-5, atol=2e-6), k
+    assert not stat["clip_mask"].any() and stat["clip_mask"].dtype == torch.bool
+    assert torch.allclose(y.grad.cpu(), x.grad, rtol=1e-4, atol=1e-8) and cosine(y.grad.cpu(), x.grad) > 0.999999
+
+
+def test_sapo_known_value_2d_and_errors(device):
+    one = torch.ones(1, 2, device=device)
+    loss, stat = areal_amd.sapo_loss_fn(one, one, one, 1.0, 1.0, torch.ones(1, 2, dtype=torch.bool, device=device))
+    assert abs(float(loss) + 2.0) < 1e-5 and stat["sapo_soft_gate"].shape == (1, 2)
+    assert torch.allclose(stat["sapo_soft_gate"].cpu(), torch.full((1, 2), 2.0), atol=1e-5)
+    with pytest.raises(ValueError, match="must be positive"):
+        areal_amd.sapo_loss_fn(one, one, one, 1.0, -1.0, one.bool())
+    with pytest.raises(ValueError, match="Invalid importance_sampling_level"):
+        areal_amd.sapo_loss_fn(one, one, one, 1.0, 1.0, one.bool(), importance_sampling_level="x")
+    # 2-D sequence level: rows are the sequences
+    g = torch.Generator().manual_seed(1)
+    lp, old, adv = torch.randn(4, 8, generator=g), torch.randn(4, 8, generator=g), torch.randn(4, 8, generator=g)
+    mask = torch.rand(4, 8, generator=g) < 0.8
+    w_loss, _ = S.sapo_loss(lp, old, adv, 1.0, 1.05, mask, "sequence")
+    loss, _ = areal_amd.sapo_loss_fn(lp.to(device), old.to(device), adv.to(device), 1.0, 1.05, mask.to(device),
+                                     "sequence")
+    assert float(loss) == pytest.approx(float(w_loss), rel=1e-5, abs=1e-7)
+
+
+@pytest.mark.parametrize("kind", ["mse", "huber"])
+@pytest.mark.parametrize("with_mask", [True, False])
+def test_critic_loss_matches_oracle(device, kind, with_mask):
+    g = torch.Generator().manual_seed(9)
+    shape = (6, 50)
+    old = torch.randn(*shape, generator=g) * (8.0 if kind == "huber" else 1.0)
+    value = old + 0.3 * torch.randn(*shape, generator=g)
+    target = old + torch.randn(*shape, generator=g) * (12.0 if kind == "huber" else 1.0)
+    value[0, :5] = old[0, :5]                 # ties: original == clipped
+    value[1, :3] = old[1, :3] + 0.2           # exactly on the clip boundary
+    mask = torch.rand(*shape, generator=g) < 0.6 if with_mask else None
+    x = value.clone().requires_grad_(True)
+    w_loss, w_stat = S.critic_loss(x, old, target, 0.2, mask, kind)
+    w_loss.backward()
+    y = value.to(device).requires_grad_(True)
+    loss, stat = areal_amd.ppo_critic_loss_fn(y, old.to(device), target.to(device), 0.2,
+                                              None if mask is None else mask.to(device), kind)
+    loss.backward()
+    assert float(loss.detach()) == pytest.approx(float(w_loss.detach()), rel=1e-5)
+    assert torch.allclose(stat["loss"].cpu(), w_stat["loss"], rtol=1e-6, atol=1e-7)
+    assert torch.equal(stat["clip_mask"].cpu(), w_stat["clip_mask"])
+    assert torch.allclose(y.grad.cpu(), x.grad, rtol=1e-5, atol=1e-9)
+
+
+def test_critic_loss_edge_cases(device):
+    v = torch.randn(8, device=device)
+    loss, _ = areal_amd.ppo_critic_loss_fn(v, v.clone(), v + 1, 0.2, torch.zeros(8, dtype=torch.bool, device=device))
+    assert torch.isnan(loss)  # 0 / 0, as in the reference
+    with pytest.raises(NotImplementedError):
+        areal_amd.ppo_critic_loss_fn(v, v, v, 0.2, None, "l1")
+    with pytest.raises(AssertionError):
+        areal_amd.ppo_critic_loss_fn(v.double(), v, v, 0.2)
+
+
+def test_prox_approx_matches_oracle_and_known_answers(device):
+    f = lambda v: torch.tensor(v, dtype=torch.float32)
+    a = areal_amd.compute_prox_logp_approximations(f([[-1.0], [-2.0]]).to(device), f([[-1.5], [-2.2]]).to(device),
+                                                   torch.tensor([[0], [2]], dtype=torch.int32).to(device), 4)
+    assert torch.allclose(a["loglinear"].cpu(), f([[-1.375], [-2.1]]), atol=1e-4)   # tests/test_prox_approx.py:84-106
+    assert set(a) == {"loglinear", "linear", "rollout"} and a["linear"].shape == (2, 1)
+    g = torch.Generator().manual_seed(2)
+    old, new = -torch.rand(5, 40, generator=g) * 4, -torch.rand(5, 40, generator=g) * 4
+    ver = torch.randint(-1, 12, (5, 40), generator=g)
+    for cur in (0, 3, 10, 12):
+        want = S.prox_logp_approximations(old, new, ver, cur)
+        got = areal_amd.compute_prox_logp_approximations(old.to(device), new.to(device), ver.to(device), cur)
+        for k in want:
+            assert torch.allclose(got[k].cpu(), want[k], rtol=1e-5, atol=1e-6), (cur, k)
+    only = areal_amd.compute_prox_logp_approximations(old.to(device), new.to(device), ver.to(device), 5, "loglinear")
+    assert list(only) == ["loglinear"]
+
+
+@pytest.mark.parametrize("n,thr", [(1, 0.1), (77, 0.05), (5000, 0.02), (5000, 1e-9), (5000, 50.0), (200000, 0.04)])
+def test_m2po_matches_oracle(device, n, thr):
+    g = torch.Generator().manual_seed(n)
+    old = torch.randn(n, generator=g) * 0.5
+    prox = old + torch.randn(n, generator=g) * 0.3
+    mask = torch.rand(n, generator=g) < 0.7
+    if n > 10:
+        prox[3] = old[3] + 0.7
+        prox[7] = old[7] + 0.7  # a tie
+    want = S.m2po_mask(old, prox, mask, thr)
+    got = areal_amd.apply_m2po_masking(old.to(device), prox.to(device), mask.to(device), thr).cpu()
+    assert got.dtype == torch.bool and got.shape == mask.shape
+    diff = int((got != want).sum())
+    # float32 suffix sums in another order may move the cut by a token or two on long inputs
+    assert diff <= (0 if n <= 5000 else 2), diff
+    assert not (got & ~mask).any() and (int(got.sum()) >= 1 or not mask.any())
+    # the mean second momentum of what is kept is below the threshold (or a single token is left)
+    d = (old - prox)[got]
+    assert int(got.sum()) <= 1 or float((d * d).double().mean()) < thr * (1 + 1e-5)
+
+
+def test_m2po_2d_and_empty(device):
+    old, prox = torch.zeros(2, 5), torch.tensor([[0.0, 1.0, 2.0, 3.0, 4.0]] * 2)
+    allm = torch.ones(2, 5, dtype=torch.bool)
+    got = areal_amd.apply_m2po_masking(old.to(device), prox.to(device), allm.to(device), 2.0).cpu()
+    assert torch.equal(got, S.m2po_mask(old, prox, allm, 2.0)) and got.shape == (2, 5)
+    none = torch.zeros(2, 5, dtype=torch.bool)
+    assert not areal_amd.apply_m2po_masking(old.to(device), prox.to(device), none.to(device), 2.0).any()
