@@ -19,6 +19,7 @@ from .functional import (
     ppo_critic_loss_fn,
     sapo_loss_fn,
 )
+from .packing import pack_tensor_dict, pad_packed_tensor_dict, segment_copy, unpad_logits
 from ._native import NativeLibraryError
 
 __version__ = "0.1.0"
@@ -40,7 +41,11 @@ __all__ = [
     "gather_logprobs_entropy_stats",
     "lm_head_logprobs_entropy",
     "masked_moments",
+    "pack_tensor_dict",
+    "pad_packed_tensor_dict",
     "ppo_actor_loss_fn",
     "ppo_critic_loss_fn",
     "sapo_loss_fn",
+    "segment_copy",
+    "unpad_logits",
 ]

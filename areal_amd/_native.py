@@ -87,6 +87,7 @@ SIGNATURES = {
     "aa_normalize_scratch_bytes": (_i64, [_i64, _i64, _i64]),
     "aa_normalize": (_i, [_p, _p, _i64, _i64, C.POINTER(NormParams), _p, _p, _i64, _p]),
     "aa_masked_moments": (_i, [C.POINTER(C.c_void_p), _i, _p, _i64, _p, _p]),
+    "aa_segment_copy": (_i, [_p, _p, _i64, _p, _p, _p, _i64, _i64, _p]),
     "aa_copy_bytes": (_i, [_p, _p, _i64, _p]),
 }
 

@@ -366,6 +366,25 @@ int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64_t T,
                         void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------ */
+/* Packing                                                                 */
+/* ------------------------------------------------------------------ */
+
+/*
+ * Segmented row copy, the data movement of pack_tensor_dict,
+ * pad_packed_tensor_dict and unpad_logits (areal/utils/data.py:492-541,
+ * 818-978, 1046-1074), which the reference does with one slice assignment
+ * per sequence.  Rows (tokens) have row_bytes bytes.  seg_cu [B+1] int32:
+ * seg_cu[i] = rows in segments before i (seg_cu[B] = total_rows); row o of
+ * segment i is copied from src row src_starts[i] + o to dst row
+ * dst_starts[i] + o.  All index arrays live on the device.  Rows of dst that
+ * no segment covers are left untouched.
+ */
+int aa_segment_copy(const void* src, void* dst, int64_t row_bytes,
+                    const int64_t* src_starts, const int64_t* dst_starts,
+                    const int32_t* seg_cu, int64_t B, int64_t total_rows,
+                    void* stream);
+
+/* ------------------------------------------------------------------ */
 /* Measurement helper                                                  */
 /* ------------------------------------------------------------------ */
 
