@@ -48,7 +48,17 @@ __global__ __launch_bounds__(256) void k_copy_rows(const W* __restrict__ src, W*
     const int64_t o = r - seg_cu[s];
     const W* p = src + (src_starts[s] + o) * n_words;
     W* q = dst + (dst_starts[s] + o) * n_words;
-    for (int64_t i = threadIdx.x; i < n_words; i += 256) q[i] = __builtin_nontemporal_load(p + i);
+    // four independent loads in flight per thread before the first store
+    int64_t i = threadIdx.x;
+    for (; i + 3 * 256 < n_words; i += 4 * 256) {
+      const W a = __builtin_nontemporal_load(p + i), b = __builtin_nontemporal_load(p + i + 256);
+      const W c = __builtin_nontemporal_load(p + i + 512), d = __builtin_nontemporal_load(p + i + 768);
+      __builtin_nontemporal_store(a, q + i);
+      __builtin_nontemporal_store(b, q + i + 256);
+      __builtin_nontemporal_store(c, q + i + 512);
+      __builtin_nontemporal_store(d, q + i + 768);
+    }
+    for (; i < n_words; i += 256) __builtin_nontemporal_store(__builtin_nontemporal_load(p + i), q + i);
   }
 }
 

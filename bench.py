@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the PPO/GRPO log-prob + entropy + actor-loss path (forward and backward) on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg1|cfg1-32k|cfg0|cfg2|cfg3|cfg4|adv]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg1|cfg1-32k|cfg0|cfg2|cfg3|cfg4|adv|aux]
 
 One "step" is one pass of the hot path over one synthetic packed micro-batch that is already resident in HBM.
 
@@ -17,6 +17,10 @@ One "step" is one pass of the hot path over one synthetic packed micro-batch tha
 * adv: the advantage pipeline that precedes the loss (not a BASELINE configuration): GAE reverse scan plus batch
   normalisation over a padded [512, 4096] batch.  Roofline: HBM, 20 bytes per token for the scan (rewards, values,
   mask read; advantages, returns written).
+
+* aux: the other per-token pieces around the loss at the configs[1] token count (SAPO loss, clipped value loss, M2PO
+  masking, proximal log-prob approximation) and the packing helpers (pack of a [512, 4096] batch, un-padding of
+  [32768 + pad, 151936] bf16 logits).  Roofline: HBM, on the logits un-padding copy (4 * V bytes per token).
 
 Prints ONE JSON line.  Besides the whole-step throughput it carries
   roofline      of the dominant kernel(s), timed with HIP events on the launch stream;
@@ -44,7 +48,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published peak
 METRIC = "tokens/sec for logprob+entropy+PPO loss fwd+bwd"
 LOGITS_WORKLOADS = ("cfg0", "cfg1", "cfg1-32k")
 FUSED_WORKLOADS = ("cfg2", "cfg3", "cfg4")
-ADV_WORKLOADS = ("adv",)
+ADV_WORKLOADS = ("adv", "aux")
 
 
 def parse_args():
@@ -570,6 +574,106 @@ def bench_adv(args, dev):
                     returns_max_abs_err=float((ret.cpu() - (w_adv + values)).abs().max())),
     )
 
+def bench_aux(args, dev):
+    import torch
+
+    import areal_amd
+    from oracle import packing as OP
+    from oracle import siblings as OS
+
+    g = torch.Generator().manual_seed(args.seed)
+    T = 122433
+    lp = -torch.rand(T, generator=g) * 3
+    old = lp + 0.05 * torch.randn(T, generator=g)
+    prox = lp + 0.05 * torch.randn(T, generator=g)
+    adv = torch.randn(T, generator=g)
+    mask = torch.rand(T, generator=g) < 0.7
+    ver = torch.randint(-1, 6, (T,), generator=g)
+    val, tgt = torch.randn(T, generator=g), torch.randn(T, generator=g)
+    d = {k: v.to(dev) for k, v in dict(lp=lp, old=old, prox=prox, adv=adv, mask=mask, ver=ver, val=val, tgt=tgt).items()}
+    stream = torch.cuda.current_stream(dev)
+
+    def sapo():
+        x = d["lp"].detach().requires_grad_(True)
+        loss, _ = areal_amd.sapo_loss_fn(x, d["old"], d["adv"], 1.0, 1.05, d["mask"])
+        loss.backward()
+
+    def critic():
+        x = d["val"].detach().requires_grad_(True)
+        loss, _ = areal_amd.ppo_critic_loss_fn(x, d["val"] * 0.9, d["tgt"], 0.2, d["mask"])
+        loss.backward()
+
+    pieces = dict(
+        sapo_loss_fwd_bwd=sapo, critic_loss_fwd_bwd=critic,
+        m2po_masking=lambda: areal_amd.apply_m2po_masking(d["old"], d["prox"], d["mask"], 0.002),
+        prox_logp_loglinear=lambda: areal_amd.compute_prox_logp_approximations(d["old"], d["lp"], d["ver"], 6, "loglinear"),
+    )
+    out_pieces = {}
+    for name, fn in pieces.items():
+        ms, _ = time_events(fn, max(args.steps, 10), stream)
+        out_pieces[name] = dict(ms=ms, tokens_per_s=T / (ms * 1e-3))
+    t0 = time.perf_counter()
+    x = lp.clone().requires_grad_(True)
+    w_loss, _ = OS.sapo_loss(x, old, adv, 1.0, 1.05, mask)
+    w_loss.backward()
+    OS.m2po_mask(old, prox, mask, 0.002)
+    cpu_sib_s = time.perf_counter() - t0
+    y = d["lp"].detach().requires_grad_(True)
+    g_loss, _ = areal_amd.sapo_loss_fn(y, d["old"], d["adv"], 1.0, 1.05, d["mask"])
+    g_loss.backward()
+    m2_gpu = areal_amd.apply_m2po_masking(d["old"], d["prox"], d["mask"], 0.002).cpu()
+    m2_cpu = OS.m2po_mask(old, prox, mask, 0.002)
+
+    # packing: a padded batch, and the logits of an aligned + page-padded micro-batch
+    bs, S, V = 512, 4096, 151936
+    lens = torch.randint(S // 8, S + 1, (bs,), generator=g)
+    am = (torch.arange(S)[None, :] < lens[:, None])
+    batch = dict(attention_mask=am.to(dev), input_ids=torch.randint(0, V, (bs, S), generator=g).to(dev),
+                 logprobs=torch.randn(bs, S, generator=g).to(dev), loss_mask=(torch.rand(bs, S, generator=g) < 0.5).to(dev))
+    pack_ms, _ = time_events(lambda: areal_amd.pack_tensor_dict(batch), max(args.steps, 10), stream)
+    mb_lens = synth_lengths(32768, args.seed)
+    cu = torch.tensor([0] + list(torch.tensor(mb_lens).cumsum(0)), dtype=torch.int32)
+    mb = dict(cu_seqlens=cu, max_seqlen=max(mb_lens), rows=torch.arange(int(cu[-1])))
+    padded, pad_len, old_cu, _ = OP.pad_packed_tensor_dict(mb, int(cu[-1]), seq_align_to=64)
+    T_pad = padded["rows"].shape[0]
+    logits = torch.randn(T_pad, V, device=dev, dtype=torch.bfloat16)
+    new_cu_d, old_cu_d = padded["cu_seqlens"].to(dev), old_cu.to(dev)
+    un_ms, un_min = time_events(lambda: areal_amd.unpad_logits(logits, pad_len, new_cu_d, old_cu_d),
+                                max(args.steps, 10), stream)
+    n_tok = int(old_cu[-1])
+    alg_bytes = 4.0 * n_tok * V
+    achieved = alg_bytes / (un_ms * 1e-3) / 1e9
+    sample = 2048
+    t0 = time.perf_counter()
+    cpu_rows = OP.unpad_logits(logits[: int(padded["cu_seqlens"][8])].cpu(), 0, padded["cu_seqlens"][:9], old_cu[:9])
+    cpu_un_s = time.perf_counter() - t0
+    got_rows = areal_amd.unpad_logits(logits, pad_len, new_cu_d, old_cu_d)[: cpu_rows.shape[0]].cpu()
+    return dict(
+        metric="tokens/sec for logits un-padding (packed, sequence-aligned micro-batch)",
+        value=n_tok / (un_ms * 1e-3), unit="tokens/s", n_gpus=1, steps=args.steps, warmup=args.warmup,
+        ms_per_step=un_ms, higher_is_better=True, scaling="weak", vs_baseline=None, dtype="bytes", data="synthetic",
+        config=dict(workload=f"aux: per-token pieces at T={T}; pack of a [{bs}, {S}] batch; un-padding of bf16 logits "
+                             f"[{T_pad}, {V}] (sequences aligned to 64 tokens, page padding {pad_len}) to [{n_tok}, {V}]"),
+        roofline=dict(bound="hbm", kernel="k_copy_rows (aa_segment_copy)", achieved=achieved, peak=HBM_PEAK_GBS,
+                      unit="GB/s", frac=achieved / HBM_PEAK_GBS, traffic=None, avg_kernel_ms=un_ms,
+                      min_kernel_ms=un_min, algorithmic_bytes_per_launch=alg_bytes),
+        cpu_baseline=dict(value=cpu_rows.shape[0] / cpu_un_s, unit="tokens/s", cores=torch.get_num_threads(), kind="port",
+                          sample=f"un-padding of the first 8 sequences ({cpu_rows.shape[0]} tokens) with the per-sequence "
+                                 f"slice loop of the CPU oracle"),
+        per_token_pieces=out_pieces, pack_tensor_dict_ms=pack_ms,
+        cpu_sapo_plus_m2po_s=cpu_sib_s,
+        parity=dict(unpad_rows_equal=bool(torch.equal(got_rows, cpu_rows)),
+                    sapo_loss_rel_err=abs(float(g_loss.detach()) - float(w_loss.detach())) / abs(float(w_loss.detach())),
+                    sapo_grad_cosine=cosine(y.grad.cpu(), x.grad),
+                    m2po_mask_mismatches=int((m2_gpu != m2_cpu).sum())),
+    )
+
+
+def synth_lengths(total, seed):
+    from areal_amd import synth
+
+    return synth.truncate_to_total(synth.lengths_lognormal(64, 7.5, 0.6, 128, 4096, seed), total)
+
 
 def main():
     args = parse_args()
@@ -583,7 +687,9 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    if args.workload in ADV_WORKLOADS:
+    if args.workload == "aux":
+        out = bench_aux(args, dev)
+    elif args.workload in ADV_WORKLOADS:
         out = bench_adv(args, dev)
     elif args.workload in LOGITS_WORKLOADS:
         out = bench_logits(args, dev)
