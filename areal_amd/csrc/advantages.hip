@@ -205,18 +205,23 @@ __global__ __launch_bounds__(kThreads) void k_norm_partial(NormArgs a, const dou
   if (threadIdx.x == 0) partial[blockIdx.x] = make_double2(s, f);
 }
 
+// one wave per segment: lane l adds slices l, l + 64, ... in order, then a fixed butterfly adds the lanes
 template <int PASS>
 __global__ __launch_bounds__(kWave) void k_norm_finish(const double2* __restrict__ partial, int parts, int segs,
                                                        double4* __restrict__ stats) {
-  const int seg = blockIdx.x * kWave + threadIdx.x;
-  if (seg >= segs) return;
+  const int seg = blockIdx.x;
   double s = 0.0, f = 0.0;
-  for (int p = 0; p < parts; ++p) {
-    s += partial[seg * parts + p].x;
-    f += partial[seg * parts + p].y;
+  for (int p = threadIdx.x; p < parts; p += kWave) {
+    const double2 v = partial[seg * parts + p];
+    s += v.x;
+    f += v.y;
   }
-  if (PASS == 0) stats[seg] = make_double4(s, f, 0.0, 0.0);
-  else stats[seg].z = s;
+  s = wave_sum(s);
+  f = wave_sum(f);
+  if (threadIdx.x == 0) {
+    if (PASS == 0) stats[seg] = make_double4(s, f, 0.0, 0.0);
+    else stats[seg].z = s;
+  }
 }
 
 __device__ __forceinline__ double level_std(double Q, double F, bool unbiased) {
@@ -371,7 +376,7 @@ extern "C" int aa_normalize(const float* x, const float* loss_mask, int64_t bs, 
   hipStream_t st = (hipStream_t)stream;
   double4* stats = (double4*)scratch;
   double2* partial = (double2*)(stats + segs);
-  const unsigned fin = (unsigned)((segs + kWave - 1) / kWave);
+  const unsigned fin = (unsigned)segs;
   hipLaunchKernelGGL(k_norm_partial<0>, dim3((unsigned)(segs * parts)), dim3(kThreads), 0, st, a, stats, parts, partial);
   hipLaunchKernelGGL(k_norm_finish<0>, dim3(fin), dim3(kWave), 0, st, partial, parts, (int)segs, stats);
   if (p.std_level != 0) {

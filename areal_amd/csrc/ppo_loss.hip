@@ -195,7 +195,13 @@ __global__ __launch_bounds__(1024) void k_count_nonzero(const uint8_t* __restric
                                                         int32_t* __restrict__ count) {
   __shared__ int smem[1024 / kWave];
   int c = 0;
-  for (int64_t i = threadIdx.x; i < n; i += 1024) c += mask[i] != 0 ? 1 : 0;
+  const int64_t n4 = ((((uintptr_t)mask) & 3) == 0) ? (n >> 2) : 0;  // four mask bytes per load
+  for (int64_t q = threadIdx.x; q < n4; q += 1024) {
+    const uint32_t m = ((const uint32_t*)mask)[q];
+    c += ((m & 0x000000ffu) ? 1 : 0) + ((m & 0x0000ff00u) ? 1 : 0) + ((m & 0x00ff0000u) ? 1 : 0) +
+         ((m & 0xff000000u) ? 1 : 0);
+  }
+  for (int64_t i = (n4 << 2) + threadIdx.x; i < n; i += 1024) c += mask[i] != 0 ? 1 : 0;
   c = block_sum<int>(c, smem);
   if (threadIdx.x == 0) count[0] = c;
 }
@@ -283,7 +289,20 @@ __global__ __launch_bounds__(1024) void k_masked_sum(const float* __restrict__ v
                                                      const float* __restrict__ scale, float* __restrict__ out) {
   __shared__ double smem[1024 / kWave];
   double acc = 0.0;
-  for (int64_t i = threadIdx.x; i < n; i += 1024)
+  // four elements per thread and trip (16-byte value loads when the base allows), always in the same order
+  const bool vec = (((uintptr_t)values) & 15) == 0 && (!mask || (((uintptr_t)mask) & 3) == 0);
+  const int64_t n4 = vec ? (n >> 2) : 0;
+  for (int64_t q = threadIdx.x; q < n4; q += 1024) {
+    const float4 v = ((const float4*)values)[q];
+    const uint32_t m = mask ? ((const uint32_t*)mask)[q] : 0x01010101u;
+    double part = 0.0;
+    if (m & 0x000000ffu) part += (double)v.x;
+    if (m & 0x0000ff00u) part += (double)v.y;
+    if (m & 0x00ff0000u) part += (double)v.z;
+    if (m & 0xff000000u) part += (double)v.w;
+    acc += part;
+  }
+  for (int64_t i = (n4 << 2) + threadIdx.x; i < n; i += 1024)
     if (!mask || mask[i] != 0) acc += (double)values[i];
   acc = block_sum<double>(acc, smem);
   if (threadIdx.x == 0) {
