@@ -44,7 +44,7 @@ __device__ __forceinline__ int acc_col(int nt, int lane) { return nt * 32 + (lan
 // turn.  Ids are first regrouped so that each XCD gets a contiguous range, and
 // that range then walks the tile grid in bands of `kGroupM` tile rows, so that
 // tiles that run at the same time on one XCD share A and B slices in its L2.
-constexpr int kGroupM = 8;
+constexpr int kGroupM = 4;
 // The XCD regrouping above is a bijection only when the tile count is a multiple of 8; otherwise use the plain order.
 __device__ __forceinline__ void tile_of(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
   const int total = tiles_m * tiles_n;
