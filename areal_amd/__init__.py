@@ -20,6 +20,12 @@ from .functional import (
     sapo_loss_fn,
 )
 from .packing import pack_tensor_dict, pad_packed_tensor_dict, segment_copy, unpad_logits
+from .tree import (
+    gather_logprobs_entropy_pairs,
+    gather_packed_tree_logprobs,
+    gather_packed_tree_logprobs_entropy,
+    tree_sequence_pairs,
+)
 from ._native import NativeLibraryError
 
 __version__ = "0.1.0"
@@ -38,7 +44,10 @@ __all__ = [
     "gae_advantages",
     "gather_logprobs",
     "gather_logprobs_entropy",
+    "gather_logprobs_entropy_pairs",
     "gather_logprobs_entropy_stats",
+    "gather_packed_tree_logprobs",
+    "gather_packed_tree_logprobs_entropy",
     "lm_head_logprobs_entropy",
     "masked_moments",
     "pack_tensor_dict",
@@ -47,5 +56,6 @@ __all__ = [
     "ppo_critic_loss_fn",
     "sapo_loss_fn",
     "segment_copy",
+    "tree_sequence_pairs",
     "unpad_logits",
 ]

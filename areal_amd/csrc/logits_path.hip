@@ -793,6 +793,87 @@ extern "C" int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int
   return launch_status();
 }
 
+// -----------------------------------------------------------------------------
+// (row, label) pairs that are not "the next token of the same row": the transitions of a packed prefix tree
+// (areal/models/tree_attn/functional.py:160-203), where the row that predicts and the token it predicts sit at
+// unrelated positions and one row may predict several tokens.
+// -----------------------------------------------------------------------------
+namespace aa {
+template <int DT>
+__global__ __launch_bounds__(256) void k_pairs_fwd(const void* __restrict__ logits, int64_t T, int V, int64_t stride,
+                                                   const int64_t* __restrict__ rows, const int64_t* __restrict__ labels,
+                                                   int64_t K, float inv_t, const float* __restrict__ row_lse,
+                                                   const float* __restrict__ row_entropy, float* __restrict__ logp,
+                                                   float* __restrict__ entropy) {
+  const int64_t step = (int64_t)gridDim.x * 256;
+  for (int64_t k = (int64_t)blockIdx.x * 256 + threadIdx.x; k < K; k += step) {
+    const int64_t r = rows[k], y = labels[k];
+    const bool ok = r >= 0 && r < T && y >= 0 && y < V;
+    float lp = __builtin_nanf("");
+    if (ok) lp = Elem<DT>::load1(row_ptr(logits, r, stride, Elem<DT>::kBytes), y) * inv_t - row_lse[r];
+    logp[k] = lp;
+    if (entropy) entropy[k] = (r >= 0 && r < T) ? row_entropy[r] : __builtin_nanf("");
+  }
+}
+
+// dlogits[rows[k], labels[k]] += g[k] * inv_t; pairs must be distinct (read-modify-write without atomics)
+template <int DT>
+__global__ __launch_bounds__(256) void k_pairs_scatter(void* __restrict__ dlogits, int64_t T, int V, int64_t stride,
+                                                       const int64_t* __restrict__ rows,
+                                                       const int64_t* __restrict__ labels, int64_t K,
+                                                       const float* __restrict__ g, float inv_t) {
+  const int64_t step = (int64_t)gridDim.x * 256;
+  for (int64_t k = (int64_t)blockIdx.x * 256 + threadIdx.x; k < K; k += step) {
+    const int64_t r = rows[k], y = labels[k];
+    if (r < 0 || r >= T || y < 0 || y >= V) continue;
+    void* row = (void*)row_ptr(dlogits, r, stride, Elem<DT>::kBytes);
+    Elem<DT>::store1(row, y, Elem<DT>::load1(row, y) + g[k] * inv_t);
+  }
+}
+}  // namespace aa
+
+extern "C" int aa_logits_pairs_fwd(const void* logits, int dtype, int64_t T, int64_t V, int64_t row_stride,
+                                   const int64_t* rows, const int64_t* labels, int64_t K, float inv_temperature,
+                                   const float* row_lse, const float* row_entropy, float* logp, float* entropy,
+                                   void* stream) {
+  if (K < 0 || T < 0 || V < 1 || V > 0x7fffffff || row_stride < V || !(inv_temperature > 0.f))
+    return AA_ERR_INVALID_ARGUMENT;
+  if (K == 0) return AA_OK;
+  if (!logits || !rows || !labels || !row_lse || !logp || (entropy && !row_entropy)) return AA_ERR_INVALID_ARGUMENT;
+  int64_t blocks = (K + 255) / 256;
+  if (blocks > 2048) blocks = 2048;
+  hipStream_t st = (hipStream_t)stream;
+#define AA_LAUNCH(DT)                                                                                              \
+  hipLaunchKernelGGL((k_pairs_fwd<DT>), dim3((unsigned)blocks), dim3(256), 0, st, logits, T, (int)V, row_stride, rows, \
+                     labels, K, inv_temperature, row_lse, row_entropy, logp, entropy)
+  if (dtype == AA_BF16) AA_LAUNCH(AA_BF16);
+  else if (dtype == AA_F16) AA_LAUNCH(AA_F16);
+  else if (dtype == AA_F32) AA_LAUNCH(AA_F32);
+  else return AA_ERR_INVALID_ARGUMENT;
+#undef AA_LAUNCH
+  return launch_status();
+}
+
+extern "C" int aa_logits_pairs_scatter(void* dlogits, int dtype, int64_t T, int64_t V, int64_t row_stride,
+                                       const int64_t* rows, const int64_t* labels, int64_t K, const float* g,
+                                       float inv_temperature, void* stream) {
+  if (K < 0 || T < 0 || V < 1 || V > 0x7fffffff || row_stride < V) return AA_ERR_INVALID_ARGUMENT;
+  if (K == 0) return AA_OK;
+  if (!dlogits || !rows || !labels || !g) return AA_ERR_INVALID_ARGUMENT;
+  int64_t blocks = (K + 255) / 256;
+  if (blocks > 2048) blocks = 2048;
+  hipStream_t st = (hipStream_t)stream;
+#define AA_LAUNCH(DT)                                                                                                \
+  hipLaunchKernelGGL((k_pairs_scatter<DT>), dim3((unsigned)blocks), dim3(256), 0, st, dlogits, T, (int)V, row_stride, \
+                     rows, labels, K, g, inv_temperature)
+  if (dtype == AA_BF16) AA_LAUNCH(AA_BF16);
+  else if (dtype == AA_F16) AA_LAUNCH(AA_F16);
+  else if (dtype == AA_F32) AA_LAUNCH(AA_F32);
+  else return AA_ERR_INVALID_ARGUMENT;
+#undef AA_LAUNCH
+  return launch_status();
+}
+
 extern "C" int aa_copy_bytes(const void* src, void* dst, int64_t nbytes, void* stream) {
   if (!src || !dst || nbytes < 0 || (nbytes & 15) || ((uintptr_t)src & 15) || ((uintptr_t)dst & 15))
     return AA_ERR_INVALID_ARGUMENT;

@@ -132,6 +132,33 @@ int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int64_t V,
                         float* ratio, uint8_t* flags, void* dlogits,
                         int32_t* work, void* stream);
 
+/*
+ * Log-probs for arbitrary (row, label) pairs, the transitions of a packed
+ * prefix tree (areal/models/tree_attn/functional.py:160-203, 206-316), where a
+ * row may predict several tokens that sit elsewhere in the packed tensor:
+ *   logp[k] = logits[rows[k], labels[k]] * inv_temperature - row_lse[rows[k]]
+ *   entropy[k] = row_entropy[rows[k]]                               (nullable)
+ * row_lse / row_entropy come from one aa_logits_fwd pass over the rows.
+ * A row or label out of range gives NaN.
+ */
+int aa_logits_pairs_fwd(const void* logits, int dtype, int64_t T, int64_t V,
+                        int64_t row_stride, const int64_t* rows,
+                        const int64_t* labels, int64_t K,
+                        float inv_temperature, const float* row_lse,
+                        const float* row_entropy, float* logp, float* entropy,
+                        void* stream);
+
+/*
+ * The one-hot part of the backward of aa_logits_pairs_fwd:
+ *   dlogits[rows[k], labels[k]] += g[k] * inv_temperature
+ * (the softmax part is aa_logits_bwd with the per-row sums of g and a label of
+ * -1).  The pairs must be distinct: the update is a plain read-modify-write.
+ */
+int aa_logits_pairs_scatter(void* dlogits, int dtype, int64_t T, int64_t V,
+                            int64_t row_stride, const int64_t* rows,
+                            const int64_t* labels, int64_t K, const float* g,
+                            float inv_temperature, void* stream);
+
 /* ------------------------------------------------------------------ */
 /* Per-token PPO pieces                                                */
 /* ------------------------------------------------------------------ */
