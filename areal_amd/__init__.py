@@ -4,7 +4,7 @@ Importing the package does not load the HIP library; the first op call does, and
 raises ``NativeLibraryError`` if ``libareal_amd.so`` has not been built.
 """
 from .actor_ops import apply_m2po_masking, compute_prox_logp_approximations
-from .advantages import Normalization, gae_advantages, masked_moments
+from .advantages import Normalization, gae_advantages, kl_regularized_rewards, masked_moments
 from .config import NormConfig, RejectionSamplingConfig
 from .functional import (
     RejectionSamplingResult,
@@ -48,6 +48,7 @@ __all__ = [
     "gather_logprobs_entropy_stats",
     "gather_packed_tree_logprobs",
     "gather_packed_tree_logprobs_entropy",
+    "kl_regularized_rewards",
     "lm_head_logprobs_entropy",
     "masked_moments",
     "pack_tensor_dict",

@@ -143,3 +143,38 @@ def masked_moments(values: Mapping[str, torch.Tensor], mask: torch.Tensor) -> di
         s, lo, hi, c = out[i, 0], out[i, 1], out[i, 2], out[i, 3]
         res[k] = dict(sum=s, avg=s / c, min=lo, max=hi, count=c)
     return res
+
+
+_KL_IDS = {"k1": 0, "k2": 1, "k3": 2}
+
+
+@torch.no_grad()
+def kl_regularized_rewards(old_logp: torch.Tensor, ref_logp: torch.Tensor | None, loss_mask: torch.Tensor,
+                           seqlens: torch.Tensor, reward_score: torch.Tensor, kl_ctl: float,
+                           kl_estimator: str = "k1", mask_no_eos_with_zero: bool = False
+                           ) -> tuple[torch.Tensor, torch.Tensor]:
+    """``(rewards, kl_rewards)`` of ``PPOActor._compute_advantages`` (actor.py:182-207) for padded ``[bs, L]`` inputs:
+    the token-level KL penalty against the reference policy, the reward at each sequence's last position cleared
+    and its scalar reward added one position earlier."""
+    if kl_estimator not in _KL_IDS:
+        raise ValueError(f"Invalid KL estimator: {kl_estimator}. Valid choices: k1, k2, k3")
+    _require_gpu(old_logp, "old_logp")
+    if old_logp.ndim != 2 or loss_mask.shape != old_logp.shape:
+        raise ValueError("old_logp and loss_mask must be [bs, max_seqlen] tensors of the same shape")
+    bs, L = old_logp.shape
+    dev = old_logp.device
+    lo, m = _f32(old_logp), _f32(loss_mask)
+    lr = None if ref_logp is None else _f32(ref_logp)
+    sl = seqlens.to(device=dev, dtype=torch.int64).contiguous()
+    sc = _f32(reward_score.to(dev)).reshape(-1)
+    if sl.numel() != bs or sc.numel() != bs:
+        raise ValueError("seqlens and reward_score must have one entry per sequence")
+    rewards, kl_rewards = torch.empty_like(lo), torch.empty_like(lo)
+    with torch.cuda.device(dev):
+        N.check(
+            N.load().aa_kl_rewards(_ptr(lo), _ptr(lr), _ptr(m), _ptr(sl), _ptr(sc), bs, L, float(kl_ctl),
+                                   _KL_IDS[kl_estimator], int(bool(mask_no_eos_with_zero)), _ptr(rewards),
+                                   _ptr(kl_rewards), _stream(dev)),
+            "aa_kl_rewards",
+        )
+    return rewards, kl_rewards

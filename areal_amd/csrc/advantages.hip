@@ -280,6 +280,42 @@ __global__ __launch_bounds__(256) void k_norm_apply(NormArgs a, const double4* _
 }
 
 // ------------------------------------------------------------------------------------------------------------------
+// KL-regularised token rewards (actor.py:182-207): kl_rewards = -kl_ctl * KL(old_logp * m, ref_logp * m) with the
+// k1 / k2 / k3 estimators clamped to [-10, 10] (data.py:1620-1656), then per sequence the reward at position
+// seqlen - 1 is cleared and the sequence's scalar reward is added at position max(seqlen - 2, 0).
+// ------------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_kl_rewards(const float* __restrict__ old_logp, const float* __restrict__ ref_logp,
+                                                    const float* __restrict__ mask, const int64_t* __restrict__ seqlens,
+                                                    const float* __restrict__ score, int64_t bs, int64_t L,
+                                                    float kl_ctl, int estimator, int mask_no_eos_with_zero,
+                                                    float* __restrict__ rewards, float* __restrict__ kl_rewards) {
+  const int64_t n = bs * L;
+  const int64_t step = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += step) {
+    const int64_t b = i / L, t = i - b * L;
+    const float m = mask[i];
+    const float lo = old_logp[i] * m, lr = (ref_logp ? ref_logp[i] : 0.f) * m;
+    float d = lo - lr;
+    if (estimator == 1) d = d * d / 2.0f;
+    else if (estimator == 2) { d = -d; d = expf(d) - 1.f - d; }
+    d = (d != d) ? d : fminf(fmaxf(d, -10.f), 10.f);  // torch.clamp keeps NaN
+    const float kr = -kl_ctl * d;
+    kl_rewards[i] = kr;
+    const int64_t sl = seqlens[b];
+    int64_t last = sl - 1;
+    if (last < 0) last += L;  // Python's negative index, as the reference's fancy indexing does
+    int64_t put = sl - 2;
+    if (put < 0) put = 0;
+    float r = (t == last) ? 0.f : kr;
+    if (t == put) {
+      const bool no_eos = sl == L;
+      r += (mask_no_eos_with_zero && no_eos) ? 0.f : score[b];
+    }
+    rewards[i] = r;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------------------------
 // Masked moments of up to kMaxTensors per-token tensors under one mask: out[k] = {sum, min, max, count}
 // (min = +inf, max = -inf when nothing is selected).  One workgroup per tensor, fixed summation order.
 // ------------------------------------------------------------------------------------------------------------------
@@ -402,5 +438,20 @@ extern "C" int aa_masked_moments(const float* const* values, int n_tensors, cons
   }
   hipLaunchKernelGGL(k_masked_moments, dim3((unsigned)n_tensors), dim3(kThreads), 0, (hipStream_t)stream, a, mask, n,
                      out);
+  return launch_status();
+}
+
+extern "C" int aa_kl_rewards(const float* old_logp, const float* ref_logp, const float* loss_mask,
+                             const int64_t* seqlens, const float* reward_score, int64_t bs, int64_t L, float kl_ctl,
+                             int estimator, int mask_no_eos_with_zero, float* rewards, float* kl_rewards,
+                             void* stream) {
+  if (bs < 0 || L < 1 || estimator < 0 || estimator > 2) return AA_ERR_INVALID_ARGUMENT;
+  if (bs == 0) return AA_OK;
+  if (!old_logp || !loss_mask || !seqlens || !reward_score || !rewards || !kl_rewards) return AA_ERR_INVALID_ARGUMENT;
+  int64_t blocks = (bs * L + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(k_kl_rewards, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, old_logp, ref_logp,
+                     loss_mask, seqlens, reward_score, bs, L, kl_ctl, estimator, mask_no_eos_with_zero, rewards,
+                     kl_rewards);
   return launch_status();
 }

@@ -13,6 +13,7 @@ from typing import Any
 
 import torch
 
+from .advantages import gae_advantages, kl_regularized_rewards
 from .functional import fused_logprobs_ppo_loss, gather_logprobs, gather_logprobs_entropy_stats, ppo_actor_loss_fn
 
 
@@ -80,3 +81,64 @@ def compute_logprobs_and_loss(
     loss, stat = ppo_actor_loss_fn(logp, prox_logp, old_logp, mb_input["advantages"], loss_mask=loss_mask, **kw)
     stat.update(logprobs=logp.detach(), entropy=entropy.detach(), vocab_min_logits=vmin, vocab_max_logits=vmax)
     return loss * scale, stat
+
+
+def compute_advantages(
+    data: dict[str, Any],
+    *,
+    kl_ctl: float = 0.0,
+    kl_estimator: str = "k1",
+    discount: float = 1.0,
+    gae_lambda: float = 1.0,
+    reward_bias: float = 0.0,
+    reward_scaling: float = 1.0,
+    reward_clip: float = 20.0,
+    reward_norm: Any | None = None,
+    adv_norm: Any | None = None,
+    mask_no_eos_with_zero: bool = False,
+    use_decoupled_loss: bool = False,
+    recompute_logprob: bool = False,
+) -> dict[str, Any]:
+    """``PPOActor._compute_advantages`` (areal/trainer/ppo/actor.py:145-250) on the GPU for one padded batch.
+
+    ``data`` holds ``input_ids``, ``attention_mask``, ``loss_mask``, ``logprobs``, ``rewards`` as ``[bs, max_seqlen]``
+    (``rewards`` is ``[bs]``) and optionally ``ref_logp``, ``values``, ``prox_logp``.  ``reward_norm`` / ``adv_norm``
+    are ``Normalization`` objects or None.  Writes ``advantages``, ``returns``, ``kl_rewards``, ``tot_rewards``,
+    the rolled ``loss_mask`` and ``logprobs`` back into ``data`` and returns it, as the reference does.  The
+    overlong-reward penalty (a per-sample Python loop over scalars, functional.py:782-804) is left to the caller.
+    """
+    reward_score = (data["rewards"] + reward_bias) * reward_scaling          # actor.py:166-170
+    reward_score = torch.clip(reward_score, max=reward_clip, min=-reward_clip)
+    if reward_norm is not None:
+        reward_score = reward_norm(reward_score)
+    loss_mask = torch.roll(data["loss_mask"].float(), shifts=-1, dims=-1)    # :174-175
+    if not use_decoupled_loss and recompute_logprob:                          # :177-186
+        prox = data["prox_logp"]
+        if prox is None:
+            raise ValueError(
+                "prox_logp is None but recompute_logprob=True. This indicates compute_logp() was skipped incorrectly."
+            )
+        old_logp = data["logprobs"] = prox
+    else:
+        old_logp = torch.roll(data["logprobs"], shifts=-1, dims=-1)          # :188
+        if not use_decoupled_loss:
+            data["prox_logp"] = old_logp
+    old_logp = old_logp * loss_mask                                           # :195-196
+    ref_logp = data.get("ref_logp")
+    if ref_logp is not None:
+        ref_logp = ref_logp * loss_mask
+    seqlens = data["attention_mask"].sum(-1).long()                           # :199-201
+    rewards, kl_rewards = kl_regularized_rewards(old_logp, ref_logp, loss_mask, seqlens, reward_score, kl_ctl,
+                                                 kl_estimator, mask_no_eos_with_zero)
+    values = data.get("values")
+    no_eos = seqlens == data["attention_mask"].shape[1]
+    advantages, returns = gae_advantages(rewards, values, loss_mask, no_eos, discount, gae_lambda)   # :209-232
+    data["returns"] = returns
+    if adv_norm is not None:
+        advantages = adv_norm(advantages, loss_mask)                          # :235-236
+    data["advantages"] = advantages
+    data["kl_rewards"] = kl_rewards
+    data["tot_rewards"] = rewards
+    data["loss_mask"] = loss_mask
+    data["logprobs"] = old_logp
+    return data

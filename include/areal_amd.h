@@ -295,6 +295,22 @@ int aa_gae(const float* rewards, const float* values, const float* loss_mask,
            const uint8_t* seq_no_eos, int64_t bs, int64_t L, float discount,
            float gae_lambda, float* advantages, float* returns, void* stream);
 
+/*
+ * KL-regularised token rewards of PPOActor._compute_advantages
+ * (areal/trainer/ppo/actor.py:182-207) for a padded [bs, L] batch:
+ *   kl_rewards = -kl_ctl * KL(old_logp * m, ref_logp * m), estimator 0 = k1,
+ *                1 = k2, 2 = k3, clamped to [-10, 10] (areal/utils/data.py:1620-1656)
+ *   rewards    = kl_rewards, with position seqlens[b] - 1 cleared and
+ *                reward_score[b] added at position max(seqlens[b] - 2, 0)
+ *                (not added when mask_no_eos_with_zero and seqlens[b] == L).
+ * ref_logp may be NULL (zeros).  loss_mask is the float mask already rolled.
+ */
+int aa_kl_rewards(const float* old_logp, const float* ref_logp,
+                  const float* loss_mask, const int64_t* seqlens,
+                  const float* reward_score, int64_t bs, int64_t L,
+                  float kl_ctl, int estimator, int mask_no_eos_with_zero,
+                  float* rewards, float* kl_rewards, void* stream);
+
 /* Normalization (areal/utils/data.py:1378-1596); levels: 0 none, 1 batch,
  * 2 group; mirrors NormConfig (areal/api/cli_args.py:42-95). */
 typedef struct {

@@ -133,3 +133,59 @@ def masked_moments(values, mask):
             d.sum().float(),
         ]))
     return torch.stack(rows) if rows else torch.zeros(0, 4)
+
+
+def kl_rewards(old_logp, ref_logp, loss_mask, seqlens, reward_score, kl_ctl, kl_estimator="k1",
+               mask_no_eos_with_zero=False):
+    """(rewards, kl_rewards); actor.py:198-207 with KLEstimator(apply_clamp=True) (data.py:1620-1656)."""
+    from .ppo import kl_estimate
+
+    bs, L = old_logp.shape
+    batch_indices = torch.arange(bs)
+    kl = kl_estimate(old_logp, ref_logp, kl_estimator).clamp(min=-10, max=10)
+    rewards = -kl_ctl * kl
+    kl_rew = rewards.clone()
+    rewards[batch_indices, seqlens - 1] = 0                                # :203
+    indices = torch.clip(seqlens - 2, min=0)                               # :204
+    seq_no_eos_mask = seqlens == L
+    if mask_no_eos_with_zero:
+        rewards[batch_indices, indices] += torch.where(seq_no_eos_mask, 0, reward_score)
+    else:
+        rewards[batch_indices, indices] += reward_score
+    return rewards, kl_rew
+
+
+def compute_advantages(data, kl_ctl=0.0, kl_estimator="k1", discount=1.0, gae_lambda=1.0, reward_bias=0.0,
+                       reward_scaling=1.0, reward_clip=20.0, reward_norm=None, adv_norm=None,
+                       mask_no_eos_with_zero=False, use_decoupled_loss=False, recompute_logprob=False):
+    """PPOActor._compute_advantages, actor.py:145-250; ``reward_norm`` / ``adv_norm`` are kwargs dicts of
+    ``normalization`` or None."""
+    data = dict(data)
+    reward_score = (data["rewards"] + reward_bias) * reward_scaling
+    reward_score = torch.clip(reward_score, max=reward_clip, min=-reward_clip)
+    if reward_norm is not None:
+        reward_score = normalization(reward_score, **reward_norm)
+    loss_mask = torch.roll(data["loss_mask"].float(), shifts=-1, dims=-1)
+    if not use_decoupled_loss and recompute_logprob:
+        old_logp = data["logprobs"] = data["prox_logp"]
+    else:
+        old_logp = torch.roll(data["logprobs"], shifts=-1, dims=-1)
+        if not use_decoupled_loss:
+            data["prox_logp"] = old_logp
+    ref_logp = data.get("ref_logp")
+    if ref_logp is None:
+        ref_logp = torch.zeros_like(old_logp)
+    ref_logp = ref_logp * loss_mask
+    old_logp = old_logp * loss_mask
+    attn_mask = data["attention_mask"]
+    seqlens = attn_mask.sum(-1).long()
+    seq_no_eos_mask = seqlens == attn_mask.shape[1]
+    rewards, kl_rew = kl_rewards(old_logp, ref_logp, loss_mask, seqlens, reward_score, kl_ctl, kl_estimator,
+                                 mask_no_eos_with_zero)
+    values = data["values"] if "values" in data else torch.zeros_like(rewards)
+    advantages, returns = gae(rewards, values, loss_mask, seq_no_eos_mask.float(), discount, gae_lambda)
+    data["returns"] = returns
+    if adv_norm is not None:
+        advantages = normalization(advantages, loss_mask, **adv_norm)
+    data.update(advantages=advantages, kl_rewards=kl_rew, tot_rewards=rewards, loss_mask=loss_mask, logprobs=old_logp)
+    return data

@@ -146,3 +146,62 @@ def test_masked_moments(device):
     assert float(empty["a"]["count"]) == 0.0 and float(empty["a"]["min"]) == float("inf")
     with pytest.raises(ValueError):
         areal_amd.masked_moments({"a": vals["s0"][:5].to(device)}, mask.to(device))
+
+
+@pytest.mark.parametrize("est", ["k1", "k2", "k3"])
+@pytest.mark.parametrize("no_eos_zero", [False, True])
+def test_kl_rewards_match_oracle(device, est, no_eos_zero):
+    g = torch.Generator().manual_seed(11)
+    bs, L = 9, 40
+    seqlens = torch.tensor([40, 1, 2, 17, 40, 5, 39, 3, 40])
+    old, ref = -torch.rand(bs, L, generator=g) * 12, -torch.rand(bs, L, generator=g) * 3
+    mask = (torch.rand(bs, L, generator=g) < 0.6).float()
+    score = torch.randn(bs, generator=g)
+    want_r, want_k = O.kl_rewards(old * mask, ref * mask, mask, seqlens, score, 0.2, est, no_eos_zero)
+    r, k = areal_amd.kl_regularized_rewards((old * mask).to(device), (ref * mask).to(device), mask.to(device),
+                                            seqlens.to(device), score.to(device), 0.2, est, no_eos_zero)
+    assert torch.allclose(k.cpu(), want_k, rtol=1e-5, atol=1e-6) and torch.allclose(r.cpu(), want_r, rtol=1e-5, atol=1e-6)
+    r0, _ = areal_amd.kl_regularized_rewards((old * mask).to(device), None, mask.to(device), seqlens.to(device),
+                                             score.to(device), 0.2, est, no_eos_zero)
+    w0, _ = O.kl_rewards(old * mask, torch.zeros(bs, L), mask, seqlens, score, 0.2, est, no_eos_zero)
+    assert torch.allclose(r0.cpu(), w0, rtol=1e-5, atol=1e-6)
+    with pytest.raises(ValueError, match="Invalid KL estimator"):
+        areal_amd.kl_regularized_rewards(old.to(device), None, mask.to(device), seqlens.to(device), score.to(device), 0.1, "k9")
+
+
+@pytest.mark.parametrize("case", ["grpo", "critic_kl", "recompute"])
+def test_compute_advantages_matches_oracle(device, case):
+    from areal_amd.engine_glue import compute_advantages
+
+    g = torch.Generator().manual_seed(21)
+    bs, L = 16, 96
+    lens = torch.randint(4, L + 1, (bs,), generator=g)
+    lens[0] = L
+    pos = torch.arange(L)[None, :]
+    am = (pos < lens[:, None]).long()
+    lm = ((pos >= (lens[:, None] * 0.4).long()) & (pos < lens[:, None])).long()
+    data = dict(input_ids=torch.randint(0, 100, (bs, L), generator=g), attention_mask=am, loss_mask=lm,
+                logprobs=-torch.rand(bs, L, generator=g) * 2, rewards=torch.randn(bs, generator=g) * 3)
+    if case == "grpo":
+        kw = dict(reward_scaling=2.0, reward_bias=-0.5, reward_clip=4.0,
+                  reward_norm=dict(mean_level="group", std_level="group", group_size=4),
+                  adv_norm=dict(mean_level="batch", std_level="batch"))
+    elif case == "critic_kl":
+        data["values"] = torch.randn(bs, L, generator=g) * 0.3
+        data["ref_logp"] = -torch.rand(bs, L, generator=g) * 2
+        kw = dict(kl_ctl=0.1, kl_estimator="k3", discount=0.99, gae_lambda=0.95, mask_no_eos_with_zero=True,
+                  use_decoupled_loss=True, adv_norm=dict(mean_level="batch", std_level=None, mean_leave1out=True))
+    else:
+        data["prox_logp"] = -torch.rand(bs, L, generator=g) * 2
+        kw = dict(recompute_logprob=True, use_decoupled_loss=False)
+    want = O.compute_advantages({k: (v.clone() if torch.is_tensor(v) else v) for k, v in data.items()}, **kw)
+    gkw = dict(kw)
+    for name in ("reward_norm", "adv_norm"):
+        if gkw.get(name) is not None:
+            gkw[name] = Normalization(NormConfig(**gkw[name]))
+    got = compute_advantages({k: (v.to(device) if torch.is_tensor(v) else v) for k, v in data.items()}, **gkw)
+    for key in ("advantages", "returns", "kl_rewards", "tot_rewards", "loss_mask", "logprobs"):
+        scale = float(want[key].abs().max()) + 1.0
+        assert float((got[key].cpu() - want[key]).abs().max()) < 2e-5 * scale, key
+    if case != "critic_kl":
+        assert torch.allclose(got["prox_logp"].cpu(), want["prox_logp"])

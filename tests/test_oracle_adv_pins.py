@@ -161,3 +161,45 @@ def test_masked_moments_against_numpy():
         assert np.allclose(out[k].numpy(), [sel.sum(), sel.min(), sel.max(), len(sel)], rtol=1e-6)
     empty = O.masked_moments(vals[:1], torch.zeros(50, dtype=torch.bool))
     assert float(empty[0, 0]) == 0.0 and math.isinf(float(empty[0, 1])) and float(empty[0, 3]) == 0.0
+
+
+def test_kl_rewards_hand_case():
+    # two sequences of a padded [2, 5] batch: lengths 4 and 5 (the second fills the row: no EOS seen)
+    old = torch.tensor([[-1.0, -2.0, -3.0, -4.0, 0.0], [-1.0, -1.0, -1.0, -1.0, -1.0]])
+    ref = torch.tensor([[-1.5, -2.0, -2.0, -4.0, 0.0], [-1.0, -2.0, -1.0, -1.0, -3.0]])
+    mask = torch.ones(2, 5)
+    seqlens = torch.tensor([4, 5])
+    score = torch.tensor([2.0, -1.0])
+    rewards, kl = O.kl_rewards(old, ref, mask, seqlens, score, kl_ctl=0.1)
+    assert torch.allclose(kl, -0.1 * (old - ref))                                  # k1: the plain difference
+    want = kl.clone()
+    want[0, 3] = 0.0
+    want[0, 2] += 2.0          # score one step before the last token
+    want[1, 4] = 0.0
+    want[1, 3] += -1.0
+    assert torch.allclose(rewards, want)
+    rewards, _ = O.kl_rewards(old, ref, mask, seqlens, score, kl_ctl=0.1, mask_no_eos_with_zero=True)
+    want[1, 3] -= -1.0         # the sequence that fills the row gets no score
+    assert torch.allclose(rewards, want)
+    # k2 and the clamp at 10
+    _, kl2 = O.kl_rewards(old * 10, ref, mask, seqlens, score, kl_ctl=1.0, kl_estimator="k2")
+    d = old * 10 - ref
+    assert torch.allclose(kl2, -(d * d / 2).clamp(max=10.0))
+
+
+def test_compute_advantages_grpo_shape_by_hand():
+    # no critic, no KL, gamma = lambda = 1: every unmasked token before the score gets the (clipped, scaled) score
+    bs, L = 2, 6
+    am = torch.tensor([[1, 1, 1, 1, 1, 0], [1, 1, 1, 0, 0, 0]])
+    lm = torch.tensor([[0, 0, 1, 1, 1, 0], [0, 1, 1, 0, 0, 0]])
+    data = dict(input_ids=torch.zeros(bs, L, dtype=torch.long), attention_mask=am, loss_mask=lm,
+                logprobs=-torch.rand(bs, L), rewards=torch.tensor([30.0, -0.5]))
+    out = O.compute_advantages(data, reward_scaling=0.5, reward_clip=5.0)
+    rolled = torch.roll(lm.float(), -1, -1)
+    assert torch.equal(out["loss_mask"], rolled)
+    # sequence 0: score min(30 * 0.5, 5) = 5 placed at position 3; rolled mask = positions 1, 2, 3
+    assert out["advantages"][0].tolist() == [5.0, 5.0, 5.0, 5.0, 0.0, 0.0]
+    # sequence 1: score -0.25 at position 1; rolled mask = positions 0, 1
+    assert out["advantages"][1].tolist() == [-0.25, -0.25, 0.0, 0.0, 0.0, 0.0]
+    assert torch.equal(out["returns"], out["advantages"]) and torch.equal(out["tot_rewards"][0, 3], torch.tensor(5.0))
+    assert torch.equal(out["prox_logp"], torch.roll(data["logprobs"], -1, -1))
