@@ -142,3 +142,117 @@ def compute_advantages(
     data["loss_mask"] = loss_mask
     data["logprobs"] = old_logp
     return data
+
+
+PROX_LOGP_METHOD_RECOMPUTE = "recompute"
+PROX_LOGP_METHOD_LOGLINEAR = "loglinear"
+PROX_LOGP_METHOD_METRICS = "metrics"
+
+
+def resolve_proximal_logp(prox_logp_gt, prox_logp_method: str, old_logp, logprobs, versions, current_version):
+    """``_resolve_proximal_logp`` (areal/trainer/ppo/actor.py:687-765): the recomputed proximal log-probs when
+    they are there, the log-linear approximation from per-token versions when the forward pass was skipped."""
+    from .actor_ops import compute_prox_logp_approximations
+
+    if prox_logp_method not in (PROX_LOGP_METHOD_RECOMPUTE, PROX_LOGP_METHOD_LOGLINEAR, PROX_LOGP_METHOD_METRICS):
+        raise ValueError(f"'{prox_logp_method}' is not a valid ProxLogpMethod")
+    if prox_logp_gt is None:
+        if prox_logp_method != PROX_LOGP_METHOD_LOGLINEAR:  # the only method that skips the forward pass
+            raise ValueError(
+                f"prox_logp is None but prox_logp_method='{prox_logp_method}'. "
+                "This indicates compute_logp() was skipped incorrectly."
+            )
+        if versions is None:
+            raise ValueError(
+                f"prox_logp is None with prox_logp_method='{prox_logp_method}' but versions not available. "
+                "Cannot proceed without either ground truth or approximation."
+            )
+    prox_logp = prox_logp_gt
+    if prox_logp_method == PROX_LOGP_METHOD_LOGLINEAR:
+        if prox_logp_gt is None and versions is not None and current_version is not None:
+            prox_logp = compute_prox_logp_approximations(old_logp, logprobs, versions, current_version,
+                                                         method="loglinear")["loglinear"]
+    if prox_logp is None:
+        raise RuntimeError(
+            f"prox_logp is None after handling prox_logp_method='{prox_logp_method}'. "
+            "This indicates configuration or computation error."
+        )
+    return prox_logp
+
+
+def grpo_loss_fn(
+    logprobs: torch.Tensor,
+    entropy: torch.Tensor,
+    input_data: dict,
+    eps_clip: float,
+    eps_clip_higher: float | None,
+    c_clip: float | None,
+    rejection_sampling: Any | None = None,
+    m2_threshold: float | None = None,
+    importance_sampling_level: str = "token",
+    current_version: int | None = None,
+    prox_logp_method: str = PROX_LOGP_METHOD_RECOMPUTE,
+    use_sapo_loss: bool = False,
+    sapo_tau_pos: float = 1.0,
+    sapo_tau_neg: float = 1.05,
+    use_decoupled_loss: bool = False,
+    vocab_min_logits: torch.Tensor | None = None,
+    vocab_max_logits: torch.Tensor | None = None,
+) -> tuple[torch.Tensor, dict]:
+    """The actor's loss function for one micro-batch (areal/trainer/ppo/actor.py:408-480) on the GPU ops: proximal
+    log-probs resolved, optional M2PO masking, SAPO or clipped PPO loss.  The knowledge-distillation branch
+    (``teacher_logp``, actor.py:482-511) is not part of this build and raises.
+
+    Returns ``(loss, stat)``.  ``stat`` is the per-token dict of the loss function plus ``"reduced"``: what the
+    reference hands to its statistics tracker tensor by tensor (actor.py:513-573) as sums / averages / extrema
+    under the same denominators, computed in one launch per denominator.
+    """
+    from .actor_ops import apply_m2po_masking
+    from .advantages import masked_moments
+    from .functional import sapo_loss_fn
+
+    if input_data.get("teacher_logp") is not None:
+        raise NotImplementedError("joint distillation (teacher_logp) is outside the scope of this build")
+    old_logp = input_data["logprobs"]
+    advantages = input_data["advantages"]
+    loss_mask = input_data["loss_mask"].bool()
+    entropy = entropy.detach()
+    prox_logp = resolve_proximal_logp(input_data.get("prox_logp"), prox_logp_method, old_logp, logprobs.detach(),
+                                      input_data.get("versions"), current_version)
+    if m2_threshold is not None:
+        loss_mask = apply_m2po_masking(old_logp, prox_logp, loss_mask, m2_threshold)
+    if use_sapo_loss:
+        if use_decoupled_loss:
+            raise ValueError(
+                "SAPO is not compatible with `use_decoupled_loss=True`. "
+                "Please set `actor.use_decoupled_loss=false` in your configuration."
+            )
+        loss, stat = sapo_loss_fn(logprobs, old_logp, advantages, sapo_tau_pos, sapo_tau_neg, loss_mask,
+                                  importance_sampling_level, input_data.get("cu_seqlens"))
+    else:
+        loss, stat = ppo_actor_loss_fn(logprobs, prox_logp, old_logp, advantages, eps_clip, loss_mask, eps_clip_higher,
+                                       c_clip, rejection_sampling, importance_sampling_level,
+                                       input_data.get("cu_seqlens"))
+    per_valid = dict(
+        importance_weight=stat["importance_weight"], approx_kl=stat["approx_kl"], new_logp=logprobs.detach(),
+        old_logp=old_logp, entropy=entropy.float(), actor_loss=stat["loss"], clip_ratio=stat["clip_mask"].float(),
+        dual_clip_ratio=stat["dual_clip_mask"].float(),
+    )
+    if use_sapo_loss:
+        per_valid.update(sapo_soft_gate=stat["sapo_soft_gate"], sapo_scaled_gate_pos=stat["sapo_scaled_gate_pos"],
+                         sapo_scaled_gate_neg=stat["sapo_scaled_gate_neg"])
+    reduced = masked_moments(per_valid, loss_mask)
+    if not use_sapo_loss:
+        clip_mask = stat["clip_mask"]
+        reduced.update(masked_moments(dict(clipped_new_logp=logprobs.detach(), clipped_old_logp=old_logp), clip_mask))
+    if "behave_imp_weight" in stat:
+        reduced.update(masked_moments(dict(behave_imp_weight=stat["behave_imp_weight"],
+                                           behave_approx_kl=stat["behave_approx_kl"]), stat["behave_mask"]))
+    if "filtered_fraction" in stat:
+        reduced["rs_filtered_fraction"] = stat["filtered_fraction"]
+    if vocab_min_logits is not None and vocab_max_logits is not None:
+        everything = torch.ones_like(loss_mask)
+        reduced.update(masked_moments(dict(vocab_min_logits=vocab_min_logits, vocab_max_logits=vocab_max_logits),
+                                      everything))
+    stat = dict(stat, loss_mask=loss_mask, reduced=reduced)
+    return loss, stat

@@ -141,3 +141,60 @@ def test_m2po_2d_and_empty(device):
     assert torch.equal(got, S.m2po_mask(old, prox, allm, 2.0)) and got.shape == (2, 5)
     none = torch.zeros(2, 5, dtype=torch.bool)
     assert not areal_amd.apply_m2po_masking(old.to(device), prox.to(device), none.to(device), 2.0).any()
+
+
+@pytest.mark.parametrize("variant", ["ppo_rs", "sapo", "loglinear_m2po"])
+def test_grpo_loss_fn_matches_composed_oracle(device, variant):
+    """The actor's loss function (actor.py:408-480) against the same composition of oracle pieces."""
+    from areal_amd import RejectionSamplingConfig
+    from areal_amd.engine_glue import grpo_loss_fn
+    from oracle import ppo as OP
+
+    n = 600
+    lp, old, adv, mask = _tok(n, 13)
+    g = torch.Generator().manual_seed(14)
+    prox = lp + 0.1 * torch.randn(n, generator=g)
+    ent = torch.rand(n, generator=g)
+    ver = torch.randint(-1, 4, (n,), generator=g)
+    cu = torch.tensor([0, 200, 600], dtype=torch.int32)
+    data = dict(logprobs=old, advantages=adv, loss_mask=mask, prox_logp=prox, cu_seqlens=cu, versions=ver)
+    kw = dict(eps_clip=0.2, eps_clip_higher=0.28, c_clip=3.0)
+    x = lp.clone().requires_grad_(True)
+    if variant == "ppo_rs":
+        rs = RejectionSamplingConfig(level="token", action="mask", metric="ratio", upper=1.25)
+        kw.update(rejection_sampling=rs, use_decoupled_loss=True)
+        w_loss, w_stat = OP.ppo_actor_loss(x, prox, old, adv, 0.2, mask, 0.28, 3.0, rs, "token", cu)
+        w_mask = mask
+    elif variant == "sapo":
+        kw.update(use_sapo_loss=True, sapo_tau_pos=1.0, sapo_tau_neg=1.05)
+        w_loss, w_stat = S.sapo_loss(x, old, adv, 1.0, 1.05, mask)
+        w_mask = mask
+    else:
+        data["prox_logp"] = None
+        kw.update(prox_logp_method="loglinear", current_version=4, m2_threshold=0.05, use_decoupled_loss=True)
+        w_prox = S.prox_logp_approximations(old, lp, ver, 4, "loglinear")["loglinear"]
+        w_mask = S.m2po_mask(old, w_prox, mask, 0.05)
+        w_loss, w_stat = OP.ppo_actor_loss(x, w_prox, old, adv, 0.2, w_mask, 0.28, 3.0, None, "token", cu)
+    w_loss.backward()
+    y = lp.to(device).requires_grad_(True)
+    d_dev = {k: (v.to(device) if torch.is_tensor(v) else v) for k, v in data.items()}
+    loss, stat = grpo_loss_fn(y, ent.to(device), d_dev, **kw)
+    loss.backward()
+    assert float(loss.detach()) == pytest.approx(float(w_loss.detach()), rel=1e-4, abs=1e-7)
+    assert torch.allclose(y.grad.cpu(), x.grad, rtol=1e-4, atol=1e-8)
+    assert torch.equal(stat["loss_mask"].cpu(), w_mask)
+    red = stat["reduced"]
+    sel = w_mask
+    assert float(red["importance_weight"]["avg"]) == pytest.approx(float(w_stat["importance_weight"][sel].mean()), rel=1e-4)
+    assert float(red["actor_loss"]["sum"]) == pytest.approx(float(w_stat["loss"][sel].sum()), rel=1e-4, abs=1e-5)
+    assert float(red["entropy"]["max"]) == float(ent[sel].max()) and float(red["new_logp"]["count"]) == float(sel.sum())
+    if variant == "ppo_rs":
+        assert float(red["rs_filtered_fraction"]) == pytest.approx(float(w_stat["filtered_fraction"]), abs=1e-6)
+        assert float(red["behave_imp_weight"]["count"]) == float(w_stat["behave_mask"].sum())
+        assert float(red["clipped_new_logp"]["count"]) == float(w_stat["clip_mask"].sum())
+    if variant == "sapo":
+        assert "sapo_soft_gate" in red and "clipped_new_logp" not in red
+        with pytest.raises(ValueError, match="SAPO is not compatible"):
+            grpo_loss_fn(y, ent.to(device), d_dev, **dict(kw, use_decoupled_loss=True))
+    with pytest.raises(ValueError, match="compute_logp\\(\\) was skipped incorrectly"):
+        grpo_loss_fn(y, ent.to(device), dict(d_dev, prox_logp=None), 0.2, None, None)
