@@ -26,8 +26,7 @@ __device__ __forceinline__ T block_sum(T v, T* smem) {
 //     nv <- nv (1 - m_t) + v_t m_t;    lg <- lg (1 - m_t) + new m_t;    adv_t = lg
 // which is the affine map  nv' = a nv + e,  lg' = c nv + d lg + f  with
 //     a = 1 - m, e = m v, c = m gamma, d = 1 - m + m gamma lambda, f = m (r - v).
-// Affine maps compose, so one wave handles one row in blocks of 64 positions: each lane builds the map of its
-// position, an inclusive wave scan composes them in processing order, and the carry of the block is applied last.
+// Affine maps compose, so a row can be cut into chunks whose composite maps are scanned in parallel.
 // ------------------------------------------------------------------------------------------------------------------
 struct Affine {
   float a, c, d, e, f;
@@ -54,64 +53,105 @@ __device__ __forceinline__ Affine shfl_up(const Affine& x, int delta) {
   return r;
 }
 
-__global__ __launch_bounds__(256) void k_gae(const float* __restrict__ rewards, const float* __restrict__ values,
-                                             const float* __restrict__ mask, const uint8_t* __restrict__ no_eos,
-                                             int64_t bs, int64_t L, float gamma, float lam,
-                                             float* __restrict__ adv, float* __restrict__ returns) {
-  const int lane = threadIdx.x & (kWave - 1);
-  const int64_t row = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
-  if (row >= bs) return;  // whole waves leave together: no barrier below
+// One workgroup per row, walking the row from its end in super-blocks of 256 x 16 positions.  A super-block is
+// copied into LDS with coalesced loads; thread k then owns the k-th chunk of 16 consecutive positions counted from
+// the end of the super-block (thread order = processing order), composes the maps of its chunk, an exclusive scan
+// over the 256 threads (wave scan + wave totals through LDS) gives the state entering the chunk, the thread walks
+// its chunk with the recurrence as written, and the results leave through LDS with coalesced stores.  Chunks are
+// padded by one word in LDS so that the 64 lanes of a wave, 16 positions apart, hit different banks.
+constexpr int kGaeThreads = 256;
+constexpr int kGaeChunk = 16;
+constexpr int kGaeBlock = kGaeThreads * kGaeChunk;                 // positions per super-block
+constexpr int kGaeLds = kGaeBlock + kGaeThreads;                   // + one pad word per chunk
+
+__device__ __forceinline__ int gae_slot(int i) { return i + i / kGaeChunk; }
+
+__global__ __launch_bounds__(kGaeThreads) void k_gae(const float* __restrict__ rewards, const float* __restrict__ values,
+                                                     const float* __restrict__ mask, const uint8_t* __restrict__ no_eos,
+                                                     int64_t bs, int64_t L, float gamma, float lam,
+                                                     float* __restrict__ adv, float* __restrict__ returns) {
+  __shared__ float sr[kGaeLds], sv[kGaeLds], sm[kGaeLds];
+  __shared__ Affine wave_tot[kGaeThreads / kWave];
+  __shared__ float carry[2];
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int64_t row = blockIdx.x;
   const float* r = rewards + row * L;
   const float* v = values ? values + row * L : nullptr;
   const float* m = mask + row * L;
   float* out_a = adv + row * L;
   float* out_r = returns ? returns + row * L : nullptr;
   const float v_last = v ? v[L - 1] : 0.f;
-  if (lane == 0) {
+  if (tid == 0) {
     out_a[L - 1] = 0.f;
     if (out_r) out_r[L - 1] = v_last;
+    carry[0] = (no_eos && no_eos[row]) ? v_last : 0.f;   // nextvalues = values[:, L-1] * seq_no_eos_mask
+    carry[1] = 0.f;                                       // lastgaelam
   }
-  float nv = (no_eos && no_eos[row]) ? v_last : 0.f;  // values[:, L-1] * seq_no_eos_mask
-  float lg = 0.f;
   const float gl = gamma * lam;
-  // lane j handles t = hi - j: processing order = lane order.  The next block's loads are issued before this
-  // block's scan, so that memory latency hides behind the shuffles.
-  auto fetch = [&](int64_t hi, float& rt, float& vt, float& mt) {
-    const int64_t t = hi - lane;
-    rt = 0.f; vt = 0.f; mt = 0.f;
-    if (t >= 0 && hi >= 0) {
-      rt = r[t];
-      vt = v ? v[t] : 0.f;
-      mt = m[t];
+  const Affine ident{1.f, 0.f, 1.f, 0.f, 0.f};
+  // positions 0 .. L-2, super-blocks aligned to the end: [base, base + cnt)
+  for (int64_t end = L - 1; end > 0; end -= kGaeBlock) {
+    const int64_t base = end > kGaeBlock ? end - kGaeBlock : 0;
+    const int cnt = (int)(end - base);
+    __syncthreads();  // the previous super-block has been written out; carry is visible
+    for (int i = tid; i < cnt; i += kGaeThreads) {
+      const int sl = gae_slot(i);
+      sr[sl] = r[base + i];
+      sv[sl] = v ? v[base + i] : 0.f;
+      sm[sl] = m[base + i];
     }
-  };
-  float rt, vt, mt;
-  fetch(L - 2, rt, vt, mt);
-  for (int64_t hi = L - 2; hi >= 0; hi -= kWave) {
-    float rn, vn, mn;
-    fetch(hi - kWave, rn, vn, mn);
-    const int64_t t = hi - lane;
-    const bool live = t >= 0;
-    Affine x;  // identity where the row has ended (mt = 0)
-    x.a = 1.f - mt;
-    x.e = mt * vt;
-    x.c = mt * gamma;
-    x.d = (1.f - mt) + mt * gl;
-    x.f = mt * (rt - vt);
+    __syncthreads();
+    // local index i = position - base; thread k owns [hi - 15, hi] with hi = cnt - 1 - 16 k (clipped at 0)
+    const int hi = cnt - 1 - tid * kGaeChunk;
+    const int lo = hi - kGaeChunk + 1 > 0 ? hi - kGaeChunk + 1 : 0;
+    Affine x = ident;
+    for (int i = hi; i >= lo; --i) {
+      const int sl = gae_slot(i);
+      const float mt = sm[sl], vt = sv[sl], rt = sr[sl];
+      Affine e;
+      e.a = 1.f - mt;
+      e.e = mt * vt;
+      e.c = mt * gamma;
+      e.d = (1.f - mt) + mt * gl;
+      e.f = mt * (rt - vt);
+      x = compose(x, e);
+    }
+    Affine inc = x;
 #pragma unroll
     for (int o = 1; o < kWave; o <<= 1) {
-      const Affine prev = shfl_up(x, o);
-      if (lane >= o) x = compose(prev, x);
+      const Affine prev = shfl_up(inc, o);
+      if (lane >= o) inc = compose(prev, inc);
     }
-    const float lg_t = fmaf(x.c, nv, fmaf(x.d, lg, x.f));
-    const float nv_t = fmaf(x.a, nv, x.e);
-    if (live) {
-      out_a[t] = lg_t;
-      if (out_r) out_r[t] = lg_t + vt;
+    if (lane == kWave - 1) wave_tot[wave] = inc;
+    const float nv0 = carry[0], lg0 = carry[1];
+    __syncthreads();
+    Affine before = ident;  // everything processed in this super-block before this thread's chunk
+    for (int w = 0; w < wave; ++w) before = compose(before, wave_tot[w]);
+    Affine excl = shfl_up(inc, 1);
+    if (lane == 0) excl = ident;
+    before = compose(before, excl);
+    float nv = fmaf(before.a, nv0, before.e);
+    float lg = fmaf(before.c, nv0, fmaf(before.d, lg0, before.f));
+    for (int i = hi; i >= lo; --i) {
+      const int sl = gae_slot(i);
+      const float mt = sm[sl], vt = sv[sl], rt = sr[sl];
+      const float delta = rt + gamma * nv - vt;
+      const float newlg = delta + gl * lg;
+      nv = nv * (1.f - mt) + vt * mt;
+      lg = lg * (1.f - mt) + newlg * mt;
+      sr[sl] = lg;        // advantages
+      sv[sl] = lg + vt;   // returns
     }
-    nv = __shfl(nv_t, kWave - 1, kWave);
-    lg = __shfl(lg_t, kWave - 1, kWave);
-    rt = rn; vt = vn; mt = mn;
+    if (tid == kGaeThreads - 1) {  // the last thread ends at the front of the super-block: its state carries on
+      carry[0] = nv;
+      carry[1] = lg;
+    }
+    __syncthreads();
+    for (int i = tid; i < cnt; i += kGaeThreads) {
+      const int sl = gae_slot(i);
+      out_a[base + i] = sr[sl];
+      if (out_r) out_r[base + i] = sv[sl];
+    }
   }
 }
 
@@ -374,9 +414,8 @@ extern "C" int aa_gae(const float* rewards, const float* values, const float* lo
                       void* stream) {
   if (!rewards || !loss_mask || !advantages || bs < 0 || L < 1) return AA_ERR_INVALID_ARGUMENT;
   if (bs == 0) return AA_OK;
-  const int rows_per_wg = 256 / kWave;
-  hipLaunchKernelGGL(k_gae, dim3((unsigned)((bs + rows_per_wg - 1) / rows_per_wg)), dim3(256), 0, (hipStream_t)stream,
-                     rewards, values, loss_mask, seq_no_eos, bs, L, discount, gae_lambda, advantages, returns);
+  hipLaunchKernelGGL(k_gae, dim3((unsigned)bs), dim3(kGaeThreads), 0, (hipStream_t)stream, rewards, values, loss_mask,
+                     seq_no_eos, bs, L, discount, gae_lambda, advantages, returns);
   return launch_status();
 }
 
