@@ -14,7 +14,7 @@ One "step" is one pass of the hot path over one synthetic packed micro-batch tha
   token chunk, the full [T, V] logits never in memory.  Roofline: bf16 MFMA, algorithmic flops 6 * T * V * H
   (logits 2TVH, the two gradient GEMMs 4TVH).
 
-* adv: the advantage pipeline that precedes the loss (not a BASELINE configuration): GAE reverse scan plus batch
+* adv: the advantage pipeline that precedes the loss (not one of the headline configurations): GAE reverse scan plus batch
   normalisation over a padded [512, 4096] batch.  Roofline: HBM, 20 bytes per token for the scan (rewards, values,
   mask read; advantages, returns written).
 
