@@ -344,10 +344,10 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
                                    uint8_t* flags, void* d_hidden, float* d_weight, int32_t* work, void* workspace,
                                    int64_t workspace_bytes, void* stream) {
   if (!hidden || !weight || !labels || !d_hidden || !d_weight || !workspace) return AA_ERR_INVALID_ARGUMENT;
-  if (!params || !prox_logp || !adv || !mask_eff || !n_valid || !logp || !stat_loss || !ratio || !flags)
-    return AA_ERR_INVALID_ARGUMENT;
-  if (params->has_behave_weight && !behave_w) return AA_ERR_INVALID_ARGUMENT;
+  if (!params || !n_valid || !logp) return AA_ERR_INVALID_ARGUMENT;
   if (T_active < 0 || T_active > T || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
+  if (T_active > 0 && (!prox_logp || !adv || !mask_eff || !stat_loss || !ratio || !flags)) return AA_ERR_INVALID_ARGUMENT;
+  if (T_active > 0 && params->has_behave_weight && !behave_w) return AA_ERR_INVALID_ARGUMENT;
   if (!shapes_ok(T, H, V) || (V % 8) != 0) return AA_ERR_UNSUPPORTED;
   if ((((uintptr_t)hidden | (uintptr_t)weight | (uintptr_t)workspace | (uintptr_t)d_hidden | (uintptr_t)d_weight) & 15))
     return AA_ERR_INVALID_ARGUMENT;
@@ -367,10 +367,10 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
     if (!lt::gemm(st, true, false, V, n_tok, H, weight, H, hid, H, ds, V, false, 0.f, lt_ws, lt::kWorkspaceBytes))
       return AA_ERR_LAUNCH;
     // log-prob, entropy, PPO loss and d(loss)/d(logits) in place: one streaming pass over the panel
-    const int rc = aa_logits_ppo_fused(ds, AA_BF16, n_tok, V, V, labels + t0, inv_temperature, act, prox_logp + t0,
-                                       adv + t0, mask_eff + t0, behave_w ? behave_w + t0 : nullptr, params, n_valid,
-                                       grad_scale, logp + t0, entropy ? entropy + t0 : nullptr, nullptr, nullptr,
-                                       stat_loss + t0, ratio + t0, flags + t0, ds, work, stream);
+    auto at = [t0](auto* p) { return p ? p + t0 : nullptr; };
+    const int rc = aa_logits_ppo_fused(ds, AA_BF16, n_tok, V, V, labels + t0, inv_temperature, act, at(prox_logp), at(adv),
+                                       at(mask_eff), at(behave_w), params, n_valid, grad_scale, logp + t0, at(entropy),
+                                       nullptr, nullptr, at(stat_loss), at(ratio), at(flags), ds, work, stream);
     if (rc != AA_OK) return rc;
     // d_hidden[t0 : t0 + n_tok, :] = dS . W: column-major [H, n_tok] = W' [H, V] . dS' [V, n_tok]
     if (!lt::gemm(st, false, false, H, n_tok, V, weight, H, ds, V, (uint16_t*)d_hidden + t0 * H, H, false, 0.f, lt_ws,

@@ -760,10 +760,11 @@ extern "C" int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int
                                    float* stat_loss, float* ratio, uint8_t* flags, void* dlogits, int32_t* work,
                                    void* stream) {
   if (!common_args_ok(logits, dtype, T, V, row_stride, labels)) return AA_ERR_INVALID_ARGUMENT;
-  if (!params || !prox_logp || !adv || !mask_eff || !n_valid || !logp || !stat_loss || !ratio || !flags || !dlogits)
-    return AA_ERR_INVALID_ARGUMENT;
-  if (params->has_behave_weight && !behave_w) return AA_ERR_INVALID_ARGUMENT;
+  if (!params || !n_valid || !logp || !dlogits) return AA_ERR_INVALID_ARGUMENT;
   if (T_active < 0 || T_active > T || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
+  // the per-token arrays have T_active entries: with no active token they may be absent
+  if (T_active > 0 && (!prox_logp || !adv || !mask_eff || !stat_loss || !ratio || !flags)) return AA_ERR_INVALID_ARGUMENT;
+  if (T_active > 0 && params->has_behave_weight && !behave_w) return AA_ERR_INVALID_ARGUMENT;
   hipStream_t st = (hipStream_t)stream;
   FusedTokenArgs a;
   a.prox_logp = prox_logp; a.adv = adv; a.mask_eff = mask_eff; a.behave_w = behave_w;

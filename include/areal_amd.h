@@ -103,7 +103,8 @@ int aa_logits_bwd(const void* logits, int dtype, int64_t T, int64_t V,
  * each row is read once, and d(loss)/d(logits) is written once.
  *
  * Per-token inputs [T_active]: prox_logp, adv, mask_eff (uint8, the mask after
- * rejection sampling), behave_w (nullable unless params->has_behave_weight).
+ * rejection sampling), behave_w (nullable unless params->has_behave_weight);
+ * with T_active == 0 they and the [T_active] outputs may all be NULL.
  * n_valid: device pointer to the int32 count of non-zero entries of the
  *   ORIGINAL loss mask (functional.py:483); the loss is divided by
  *   max(*n_valid, 1).

@@ -104,7 +104,7 @@ def test_sequence_level_runs_the_unfused_kernels(device):
     lp, _ = oracle.logprobs_entropy(h @ w.t(), labels)
     o_loss, _ = oracle.ppo_actor_loss(lp, prox, old, adv, 0.2, mask, importance_sampling_level="sequence", cu_seqlens=cu)
     o_loss.backward()
-    assert float(loss.detach()) == pytest.approx(float(o_loss), rel=1e-3, abs=1e-7)
+    assert float(loss.detach()) == pytest.approx(float(o_loss.detach()), rel=1e-3, abs=1e-7)
     assert cosine(h_d.grad.cpu().float(), h.grad) > 0.9999 and cosine(w_d.grad.cpu().float(), w.grad) > 0.9999
     with pytest.raises(ValueError, match="Invalid importance_sampling_level"):
         areal_amd.fused_lm_head_ppo_loss(h_d, w_d, labels.to(device), prox.to(device), old.to(device), adv.to(device),
@@ -144,3 +144,28 @@ def test_full_size_step_agrees_with_unfused_path(device):
     assert float(a @ b / (a.norm() * b.norm())) > 0.9999
     a, b = dw1.double().reshape(-1), w.grad.double().reshape(-1)
     assert float(a @ b / (a.norm() * b.norm())) > 0.9999
+
+
+def test_padding_only_chunk_and_no_active_token(device):
+    g = torch.Generator().manual_seed(0)
+    T_pad, T, H, V = 16384 + 300, 16384, 64, 640           # the second token chunk is batch padding only
+    hidden = torch.randn(T_pad, H, generator=g).bfloat16().to(device).requires_grad_(True)
+    weight = (0.3 * torch.randn(V, H, generator=g)).bfloat16().to(device).requires_grad_(True)
+    labels = torch.randint(0, V, (T_pad,), generator=g).to(device)
+    z = torch.zeros(T, device=device)
+    mask = (torch.rand(T, generator=g) < 0.7).to(device)
+    loss, _ = areal_amd.fused_lm_head_ppo_loss(hidden, weight, labels, z - 6.0, z - 6.0,
+                                               torch.randn(T, generator=g).to(device), 0.2, mask)
+    loss.backward()
+    assert float(hidden.grad[T:].abs().sum()) == 0.0 and bool(torch.isfinite(weight.grad).all())
+    # no active token at all: zero loss, zero gradients (both the lm_head step and the logits path)
+    e = torch.zeros(0, device=device)
+    none = torch.zeros(0, dtype=torch.bool, device=device)
+    h2 = hidden.detach()[:50].clone().requires_grad_(True)
+    loss, stat = areal_amd.fused_lm_head_ppo_loss(h2, weight, labels[:50], e, e, e, 0.2, none)
+    loss.backward()
+    assert float(loss.detach()) == 0.0 and float(h2.grad.abs().sum()) == 0.0 and stat["logprobs"].numel() == 0
+    x = torch.randn(30, 9000, device=device).bfloat16().requires_grad_(True)
+    loss, _ = areal_amd.fused_logprobs_ppo_loss(x, labels[:30] % 9000, e, e, e, 0.2, none)
+    loss.backward()
+    assert float(loss.detach()) == 0.0 and float(x.grad.float().abs().sum()) == 0.0
