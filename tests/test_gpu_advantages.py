@@ -88,7 +88,8 @@ def test_normalization_full_size(device):
         assert torch.equal(got, norm(x.to(device), mask.to(device)))  # fixed summation order
 
 
-@pytest.mark.parametrize("bs,L", [(1, 1), (3, 2), (5, 63), (4, 64), (7, 65), (6, 66), (9, 129), (2, 1000)])
+@pytest.mark.parametrize("bs,L", [(1, 1), (3, 2), (5, 63), (4, 64), (7, 65), (6, 66), (9, 129), (2, 1000), (3, 4096),
+                                   (2, 4097), (2, 4098), (2, 9001), (1, 20000)])
 @pytest.mark.parametrize("gamma,lam", [(1.0, 1.0), (0.99, 0.95)])
 def test_gae_matches_oracle(device, bs, L, gamma, lam):
     g = torch.Generator().manual_seed(bs * 1000 + L)
