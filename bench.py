@@ -479,7 +479,7 @@ def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: i
     alg_flops = 6.0 * T * V * H
     achieved = alg_flops / (k_ms * 1e-3) / 1e12
     roofline = dict(
-        bound="mfma", kernel="aa_lmhead_ppo_fused (per token chunk: hipBLASLt logits GEMM, k_fused_regs in place, hipBLASLt d_hidden and d_weight GEMMs)",
+        bound="mfma", kernel="aa_lmhead_ppo_fused (per token chunk: hipBLASLt logits GEMM, k_fused_regs in place, k_transpose_bf16 copies, hipBLASLt d_hidden and d_weight GEMMs)",
         achieved=achieved, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s", frac=achieved / MFMA_BF16_PEAK_TFLOPS,
         traffic=None, avg_call_ms=k_ms, min_call_ms=k_min_ms, algorithmic_flops_per_step=alg_flops,
         # the stand-alone differentiable op lm_head_logprobs_entropy, whose backward recomputes the logits tiles

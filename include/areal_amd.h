@@ -356,7 +356,10 @@ int aa_masked_moments(const float* const* values, int n_tensors,
 /* logits = hidden @ weight.T followed by the logits path above)           */
 /* ------------------------------------------------------------------ */
 
-/* Bytes of workspace aa_lmhead_fwd / aa_lmhead_bwd need for these sizes. */
+/* Bytes of workspace aa_lmhead_fwd / aa_lmhead_bwd / aa_lmhead_ppo_fused need
+ * for these sizes: about 4 * min(T, 16384) * V + 2 * H * V bytes (one chunk of
+ * bf16 logits and its transposed copy, a transposed copy of the weight) plus
+ * 128 MiB for the GEMM library. */
 int64_t aa_lmhead_workspace_bytes(int64_t T, int64_t H, int64_t V);
 
 /*
