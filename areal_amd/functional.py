@@ -682,11 +682,14 @@ class _LmHeadLogprobsEntropy(torch.autograd.Function):
 def lm_head_logprobs_entropy(
     hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0
 ) -> tuple[torch.Tensor, torch.Tensor]:
-    """``gather_logprobs_entropy(hidden @ weight.T, labels, temperature)`` without materialising the logits.
+    """``gather_logprobs_entropy(hidden @ weight.T, labels, temperature)`` without materialising the ``[T, V]`` logits.
 
-    ``hidden`` is ``[T, H]`` and ``weight`` ``[V, H]`` (the lm_head), both bf16; logits tiles are formed on the
-    matrix cores with fp32 accumulation and reduced to log-prob and entropy on the fly.  Differentiable in
-    ``hidden`` and ``weight`` (fp32 accumulation; the weight gradient is returned in the dtype of ``weight``).
+    ``hidden`` is ``[T, H]`` and ``weight`` ``[V, H]`` (the lm_head), both bf16.  Tokens go through in chunks of at
+    most 16384: the chunk's logits are formed on the matrix cores (fp32 accumulation, rounded to bf16 as the model's
+    lm_head output is) and reduced to log-prob and entropy by the streaming kernel of ``gather_logprobs_entropy``.
+    Differentiable in ``hidden`` and ``weight`` (the backward forms each chunk's logits again, turns them in place
+    into their gradient and contracts that with the weight and the hidden states; fp32 accumulation, the weight
+    gradient is returned in the dtype of ``weight``).
     The reference has no such op: it is the drop-in for its lm_head matmul followed by
     ``gather_logprobs_entropy`` (vocab_parallel.py:434-469).
     """

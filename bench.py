@@ -357,8 +357,8 @@ def time_lmhead_step(case, kw, cfg, iters: int):
 
 
 def time_lmhead_op(case, iters: int):
-    """Durations of aa_lmhead_fwd and aa_lmhead_bwd, the stand-alone differentiable op (its backward recomputes the
-    logits tiles), HIP events on the launch stream."""
+    """Durations of aa_lmhead_fwd and aa_lmhead_bwd, the stand-alone differentiable op (its backward forms the
+    logits of each chunk again), HIP events on the launch stream."""
     import torch
 
     from areal_amd import _native as N
@@ -482,7 +482,7 @@ def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: i
         bound="mfma", kernel="aa_lmhead_ppo_fused (per token chunk: hipBLASLt logits GEMM, k_fused_regs in place, k_transpose_bf16 copies, hipBLASLt d_hidden and d_weight GEMMs)",
         achieved=achieved, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s", frac=achieved / MFMA_BF16_PEAK_TFLOPS,
         traffic=None, avg_call_ms=k_ms, min_call_ms=k_min_ms, algorithmic_flops_per_step=alg_flops,
-        # the stand-alone differentiable op lm_head_logprobs_entropy, whose backward recomputes the logits tiles
+        # the stand-alone differentiable op lm_head_logprobs_entropy, whose backward forms the logits again
         standalone_op=dict(fwd_ms=f_ms, bwd_ms=b_ms, fwd_tflops=2.0 * T * V * H / (f_ms * 1e-3) / 1e12,
                            bwd_tflops=4.0 * T * V * H / (b_ms * 1e-3) / 1e12),
     )

@@ -363,10 +363,12 @@ int aa_masked_moments(const float* const* values, int n_tensors,
 int64_t aa_lmhead_workspace_bytes(int64_t T, int64_t H, int64_t V);
 
 /*
- * logp / entropy of softmax(hidden @ weight.T / temperature) without writing
- * the [T, V] logits: bf16 MFMA tiles with an online-softmax epilogue.
- * hidden [T, H] bf16 row-major, weight [V, H] bf16 row-major.
- * row_lse / row_ez as in aa_logits_fwd (needed by aa_lmhead_bwd).
+ * logp / entropy of softmax(hidden @ weight.T / temperature), holding at most
+ * one chunk of 16384 tokens of logits (bf16, as the reference's lm_head output
+ * is) in the workspace: a GEMM per chunk, then the kernel of aa_logits_fwd.
+ * hidden [T, H] bf16 row-major, weight [V, H] bf16 row-major; H and V
+ * multiples of 8.  entropy, row_lse, row_ez may be NULL; row_lse / row_ez as
+ * in aa_logits_fwd (needed by aa_lmhead_bwd).
  */
 int aa_lmhead_fwd(const void* hidden, const void* weight, int64_t T, int64_t H,
                   int64_t V, const int64_t* labels, float inv_temperature,
@@ -376,6 +378,8 @@ int aa_lmhead_fwd(const void* hidden, const void* weight, int64_t T, int64_t H,
 /*
  * Backward of aa_lmhead_fwd: d_hidden [T, H] bf16 and d_weight [V, H] fp32
  * (overwritten, fp32 accumulation), given g_logp and optional g_entropy.
+ * Per chunk: the logits GEMM again, the kernel of aa_logits_bwd in place, and
+ * the two gradient GEMMs (6 T V H flops for the 4 T V H of the backward).
  */
 int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, int64_t H,
                   int64_t V, const int64_t* labels, float inv_temperature,

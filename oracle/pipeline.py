@@ -16,8 +16,10 @@ from .ppo import ppo_actor_loss
 
 
 def lmhead_logits(hidden: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-    """fp32 logits of the lm_head, ``hidden @ weight.T`` with fp32 accumulation."""
-    return hidden.float() @ weight.float().t()
+    """Logits as the reference's bf16 lm_head hands them to ``gather_logprobs_entropy``: ``hidden @ weight.T`` with
+    fp32 accumulation, rounded to bf16.  Differentiable (the rounding passes gradients through, as autograd's
+    ``.to(torch.bfloat16)`` does)."""
+    return (hidden.float() @ weight.float().t()).to(torch.bfloat16)
 
 
 def logits_ppo_step(

@@ -1,5 +1,6 @@
-"""GPU parity of the fused lm_head path.  The reference has no fused path, so the oracle is its equivalent:
-logits = hidden @ weight.T in fp32, then the log-prob / entropy oracle, with autograd for the gradients."""
+"""GPU parity of the lm_head path.  The reference has no such path, so the oracle is its equivalent: bf16 logits
+= hidden @ weight.T (fp32 accumulation, rounded as the model's lm_head output is), then the log-prob / entropy
+oracle, with autograd for the gradients."""
 import math
 
 import pytest
@@ -23,10 +24,11 @@ def _case(T, H, V, seed, w_std=0.02):
 @pytest.mark.parametrize(
     "T,H,V,temperature",
     [
-        (256, 128, 1024, 1.0),    # exactly one tile column, four tile rows
-        (300, 192, 1088, 1.0),    # ragged in tokens and in vocabulary
-        (37, 64, 576, 0.7),       # smaller than a tile
+        (256, 128, 1024, 1.0),
+        (300, 192, 1088, 1.0),    # token count not a multiple of 8: the transposed copies pad it
+        (37, 64, 576, 0.7),
         (700, 256, 4160, 1.3),
+        (203, 200, 1096, 1.0),    # H and V multiples of 8 only
     ],
 )
 def test_forward_matches_oracle(device, T, H, V, temperature):
@@ -35,9 +37,11 @@ def test_forward_matches_oracle(device, T, H, V, temperature):
     logits = oracle.lmhead_logits(hidden, weight)
     r_lp, r_ent = oracle.logprobs_entropy_f64(logits, labels, temperature)
     assert lp.dtype == torch.float32 and lp.shape == (T,)
-    assert float((lp.cpu().double() - r_lp).abs().max()) < 2e-3     # stated tolerance
-    assert float((lp.cpu().double() - r_lp).abs().max()) < 2e-4
-    assert float((ent.cpu().double() - r_ent).abs().max()) < 2e-4
+    # stated tolerance; a logit whose fp32 sum lies next to a bf16 rounding boundary may round the other way than the
+    # oracle's (different summation order), which moves a row by up to one bf16 step of that logit, hence the medians
+    e_lp, e_ent = (lp.cpu().double() - r_lp).abs(), (ent.cpu().double() - r_ent).abs()
+    assert float(e_lp.max()) < 2e-3 and float(e_ent.max()) < 2e-3
+    assert float(e_lp.median()) < 2e-5 and float(e_ent.median()) < 2e-5
     # deterministic
     lp2, ent2 = areal_amd.lm_head_logprobs_entropy(hidden.to(device), weight.to(device), labels.to(device), temperature)
     assert torch.equal(lp, lp2) and torch.equal(ent, ent2)
@@ -56,10 +60,11 @@ def test_closed_form_and_bad_label(device):
     assert float((lp[ok] + math.log(V)).abs().max()) < 1e-5 and float((ent - math.log(V)).abs().max()) < 1e-4
     assert torch.isnan(lp[3])
     with pytest.raises(areal_amd.NativeLibraryError):
-        areal_amd.lm_head_logprobs_entropy(hidden[:, :40].contiguous(), weight[:, :40].contiguous(), labels)  # H % 64
+        areal_amd.lm_head_logprobs_entropy(hidden[:, :44].contiguous(), weight[:, :44].contiguous(), labels)  # H % 8
 
 
-@pytest.mark.parametrize("T,H,V,temperature,with_entropy", [(300, 128, 1088, 1.0, False), (520, 192, 832, 0.8, True)])
+@pytest.mark.parametrize("T,H,V,temperature,with_entropy",
+                         [(300, 128, 1088, 1.0, False), (520, 192, 832, 0.8, True), (203, 200, 1096, 1.0, True)])
 def test_backward_matches_autograd_of_oracle(device, T, H, V, temperature, with_entropy):
     hidden, weight, labels = _case(T, H, V, seed=7 * T + V, w_std=0.3)
     g = torch.Generator().manual_seed(3)
@@ -75,7 +80,7 @@ def test_backward_matches_autograd_of_oracle(device, T, H, V, temperature, with_
     obj.backward()
     h_o = hidden.float().requires_grad_(True)
     w_o = weight.float().requires_grad_(True)
-    o_lp, o_ent = oracle.logprobs_entropy(h_o @ w_o.t(), labels, temperature)
+    o_lp, o_ent = oracle.logprobs_entropy(oracle.lmhead_logits(h_o, w_o), labels, temperature)
     ref = (o_lp * gl).sum() + ((o_ent * gh).sum() if with_entropy else 0.0)
     ref.backward()
     assert h_d.grad.dtype == torch.bfloat16 and w_d.grad.dtype == torch.bfloat16
@@ -103,10 +108,10 @@ def test_lm_head_into_ppo_loss_end_to_end(device):
     loss.backward()
     h_o = hidden.float().requires_grad_(True)
     w_o = weight.float().requires_grad_(True)
-    o_lp, _ = oracle.logprobs_entropy(h_o @ w_o.t(), labels)
+    o_lp, _ = oracle.logprobs_entropy(oracle.lmhead_logits(h_o, w_o), labels)
     o_loss, _ = oracle.ppo_actor_loss(o_lp, prox, old, adv, 0.2, mask, 0.28, 3.0)
     o_loss.backward()
-    assert float(loss.detach()) == pytest.approx(float(o_loss), rel=1e-3, abs=1e-7)
+    assert float(loss.detach()) == pytest.approx(float(o_loss.detach()), rel=1e-3, abs=1e-7)
     assert cosine(h_d.grad.cpu(), h_o.grad) > 0.9999 and cosine(w_d.grad.cpu(), w_o.grad) > 0.9999
 
 
@@ -124,7 +129,7 @@ def _cos_dev(a, b, device):
 def _oracle_slice(case, idx, g_slice):
     h = case.hidden[idx].cpu().float().requires_grad_(True)
     w = case.weight.cpu().float().requires_grad_(True)
-    lp, ent = oracle.logprobs_entropy(h @ w.t(), case.labels[idx].cpu(), case.temperature)
+    lp, ent = oracle.logprobs_entropy(oracle.lmhead_logits(h, w), case.labels[idx].cpu(), case.temperature)
     (lp * g_slice).sum().backward()
     return lp.detach(), ent.detach(), h.grad, w.grad
 
