@@ -63,10 +63,16 @@ def parse_args():
     ap.add_argument("--cpu-iters", type=int, default=3)
     ap.add_argument("--no-fused-extra", action="store_true",
                     help="default workload only: do not append the cfg2 fused lm_head figures")
+    ap.add_argument("--rs-action", choices=["mask", "clamp"], default=None,
+                    help="override the action of the workload's importance-weight cap (cfg1 is quoted with 'mask', "
+                         "the documented equivalent of behave_imp_weight_cap; 'clamp' keeps every token)")
     ap.add_argument("--copy-launches", type=int, default=0,
                     help="also launch the plain copy kernel this many times over the logits buffer "
                          "(the calibration point for FETCH_SIZE / WRITE_SIZE counters)")
     return ap.parse_args()
+
+
+RS_ACTION = None  # set from --rs-action
 
 
 def ppo_kwargs(case):
@@ -74,6 +80,8 @@ def ppo_kwargs(case):
 
     kw = dict(case.ppo)
     rs = kw.pop("rejection_sampling", None)
+    if rs and RS_ACTION:
+        rs = dict(rs, action=RS_ACTION)
     cfg = RejectionSamplingConfig(**rs) if rs else None
     return kw, cfg
 
@@ -255,6 +263,8 @@ def bench_logits(args, dev):
                     accumulate="f32", path="logits (fused fwd + PPO loss + bwd, one launch)"),
         roofline=roofline,
     )
+    if cfg is not None:
+        out["config"]["importance_weight_cap"] = f"{cfg.level} {cfg.metric} <= {cfg.upper}, action={cfg.action}"
     if args.copy_launches > 0:
         from areal_amd import _native as N
         from areal_amd import functional as F
@@ -676,7 +686,9 @@ def synth_lengths(total, seed):
 
 
 def main():
+    global RS_ACTION
     args = parse_args()
+    RS_ACTION = args.rs_action
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU; run it with --gpus 1 (no multi-GPU path exists)", file=sys.stderr)
         sys.exit(2)
