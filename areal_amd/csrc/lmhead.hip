@@ -77,9 +77,26 @@ static void launch_transpose(hipStream_t st, const uint16_t* src, int64_t R, int
                      ldd, (int)tiles_c, (int)tiles_r);
 }
 
+// fp32 -> bf16 (round to nearest even), 8 elements per thread; n % 8 == 0
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void k_f32_to_bf16(const f32x4_t* __restrict__ src, u32x4_t* __restrict__ dst,
+                                                     int64_t n8) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n8) return;
+  const f32x4_t a = __builtin_nontemporal_load(src + 2 * i), b = __builtin_nontemporal_load(src + 2 * i + 1);
+  u32x4_t o;
+  o[0] = Elem<AA_BF16>::pack(a[0], a[1]);
+  o[1] = Elem<AA_BF16>::pack(a[2], a[3]);
+  o[2] = Elem<AA_BF16>::pack(b[0], b[1]);
+  o[3] = Elem<AA_BF16>::pack(b[2], b[3]);
+  __builtin_nontemporal_store(o, dst + i);
+}
+
 struct Workspace {
   int64_t off_ds, off_lt;           // the [chunk, V] panel, scratch of the GEMM library
   int64_t off_dst, off_wt, off_ht;  // transposed copies: panel [V, chunk], weight [H, V], hidden chunk [H, chunk]
+  int64_t off_dw;                   // fp32 accumulator of a bf16 d_weight when there is more than one chunk
   int64_t chunk;
   int64_t bytes;
 };
@@ -94,6 +111,7 @@ static Workspace plan(int64_t T, int64_t H, int64_t V) {
   w.off_dst = off; off += up(w.chunk * V * 2);
   w.off_wt = off;  off += up(H * V * 2);
   w.off_ht = off;  off += up(w.chunk * H * 2);
+  w.off_dw = off;  off += T > w.chunk ? up(V * H * 4) : 0;
   w.bytes = off;
   return w;
 }
@@ -107,11 +125,11 @@ static bool panel_logits(hipStream_t st, const Workspace& w, char* ws, const uin
 }
 
 // The two GEMMs that contract the d(logits) panel ds [n_tok, V] of one token chunk:
-//   d_hidden[chunk] = ds . W          (bf16)          d_weight (+)= ds^T . hidden[chunk]   (fp32)
+//   d_hidden[chunk] = ds . W          (bf16)          d_weight (+)= ds^T . hidden[chunk]   (fp32, or bf16 when first)
 // with transposed copies of the panel and of the hidden chunk (made here) and of the weight (made once per call, by
 // the caller, at ws + off_wt).  The copies pad the token count to a multiple of 8 with zeros.
 static bool panel_gradients(hipStream_t st, const Workspace& w, char* ws, const uint16_t* hid, int64_t n_tok, int64_t H,
-                            int64_t V, uint16_t* d_hidden_chunk, float* d_weight, bool first) {
+                            int64_t V, uint16_t* d_hidden_chunk, void* d_weight, bool dw_f32, bool first) {
   const uint16_t* ds = (const uint16_t*)(ws + w.off_ds);
   uint16_t* ds_t = (uint16_t*)(ws + w.off_dst);
   const uint16_t* w_t = (const uint16_t*)(ws + w.off_wt);
@@ -124,8 +142,29 @@ static bool panel_gradients(hipStream_t st, const Workspace& w, char* ws, const 
   launch_transpose(st, ds, n_tok, V, V, ds_t);
   launch_transpose(st, hid, n_tok, H, H, hid_t);
   // column-major [H, V] = (hidden^T)'^T [H, kp] . (ds^T)' [kp, V], fp32, accumulated over the chunks
-  return lt::gemm(st, true, false, H, V, kp, hid_t, kp, ds_t, kp, d_weight, H, true, first ? 0.f : 1.f, lt_ws,
+  return lt::gemm(st, true, false, H, V, kp, hid_t, kp, ds_t, kp, d_weight, H, dw_f32, first ? 0.f : 1.f, lt_ws,
                   lt::kWorkspaceBytes);
+}
+
+// d_weight of dtype AA_F32 is accumulated in place.  A bf16 d_weight is written by the GEMM itself when there is one
+// chunk, and otherwise accumulated in fp32 in the workspace and rounded once at the end.
+struct WeightGrad {
+  void* acc;    // what the GEMMs write
+  bool acc_f32;
+  bool convert; // acc is the workspace buffer: round it into the caller's bf16 array at the end
+};
+
+static WeightGrad weight_grad(const Workspace& w, char* ws, void* d_weight, int dtype, int64_t T) {
+  if (dtype == AA_F32) return {d_weight, true, false};
+  if (T <= w.chunk) return {d_weight, false, false};
+  return {ws + w.off_dw, true, true};
+}
+
+static void finish_weight_grad(hipStream_t st, const WeightGrad& g, void* d_weight, int64_t V, int64_t H) {
+  if (!g.convert) return;
+  const int64_t n8 = V * H / 8;
+  hipLaunchKernelGGL(k_f32_to_bf16, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, st, (const f32x4_t*)g.acc,
+                     (u32x4_t*)d_weight, n8);
 }
 
 static bool shapes_ok(int64_t T, int64_t H, int64_t V) {
@@ -167,12 +206,12 @@ extern "C" int aa_lmhead_fwd(const void* hidden, const void* weight, int64_t T, 
 
 extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, int64_t H, int64_t V,
                              const int64_t* labels, float inv_temperature, const float* row_lse, const float* row_ez,
-                             const float* g_logp, const float* g_entropy, void* d_hidden, float* d_weight,
-                             void* workspace, int64_t workspace_bytes, void* stream) {
+                             const float* g_logp, const float* g_entropy, void* d_hidden, void* d_weight,
+                             int d_weight_dtype, void* workspace, int64_t workspace_bytes, void* stream) {
   if (!hidden || !weight || !labels || !row_lse || !g_logp || !d_hidden || !d_weight || !workspace)
     return AA_ERR_INVALID_ARGUMENT;
   if ((g_entropy && !row_ez) || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
-  if (!shapes_ok(T, H, V)) return AA_ERR_UNSUPPORTED;
+  if (!shapes_ok(T, H, V) || (d_weight_dtype != AA_F32 && d_weight_dtype != AA_BF16)) return AA_ERR_UNSUPPORTED;
   if ((((uintptr_t)hidden | (uintptr_t)weight | (uintptr_t)workspace | (uintptr_t)d_hidden | (uintptr_t)d_weight) & 15))
     return AA_ERR_INVALID_ARGUMENT;
   const Workspace w = plan(T, H, V);
@@ -181,6 +220,7 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
   char* ws = (char*)workspace;
   void* ds = ws + w.off_ds;  // [chunk, V]: logits of the chunk, then their gradient in place
   launch_transpose(st, (const uint16_t*)weight, V, H, H, (uint16_t*)(ws + w.off_wt));
+  const WeightGrad dw = weight_grad(w, ws, d_weight, d_weight_dtype, T);
   for (int64_t t0 = 0; t0 < T; t0 += w.chunk) {
     const int64_t n_tok = (T - t0) < w.chunk ? (T - t0) : w.chunk;
     const uint16_t* hid = (const uint16_t*)hidden + t0 * H;
@@ -189,9 +229,10 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
                                  row_ez ? row_ez + t0 : nullptr, g_logp + t0, g_entropy ? g_entropy + t0 : nullptr, n_tok,
                                  ds, stream);
     if (rc != AA_OK) return rc;
-    if (!panel_gradients(st, w, ws, hid, n_tok, H, V, (uint16_t*)d_hidden + t0 * H, d_weight, t0 == 0))
+    if (!panel_gradients(st, w, ws, hid, n_tok, H, V, (uint16_t*)d_hidden + t0 * H, dw.acc, dw.acc_f32, t0 == 0))
       return AA_ERR_LAUNCH;
   }
+  finish_weight_grad(st, dw, d_weight, V, H);
   return launch_status();
 }
 
@@ -200,14 +241,14 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
                                    const float* prox_logp, const float* adv, const uint8_t* mask_eff,
                                    const float* behave_w, const aa_ppo_params* params, const int32_t* n_valid,
                                    const float* grad_scale, float* logp, float* entropy, float* stat_loss, float* ratio,
-                                   uint8_t* flags, void* d_hidden, float* d_weight, int32_t* work, void* workspace,
-                                   int64_t workspace_bytes, void* stream) {
+                                   uint8_t* flags, void* d_hidden, void* d_weight, int d_weight_dtype, int32_t* work,
+                                   void* workspace, int64_t workspace_bytes, void* stream) {
   if (!hidden || !weight || !labels || !d_hidden || !d_weight || !workspace) return AA_ERR_INVALID_ARGUMENT;
   if (!params || !n_valid || !logp) return AA_ERR_INVALID_ARGUMENT;
   if (T_active < 0 || T_active > T || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
   if (T_active > 0 && (!prox_logp || !adv || !mask_eff || !stat_loss || !ratio || !flags)) return AA_ERR_INVALID_ARGUMENT;
   if (T_active > 0 && params->has_behave_weight && !behave_w) return AA_ERR_INVALID_ARGUMENT;
-  if (!shapes_ok(T, H, V)) return AA_ERR_UNSUPPORTED;
+  if (!shapes_ok(T, H, V) || (d_weight_dtype != AA_F32 && d_weight_dtype != AA_BF16)) return AA_ERR_UNSUPPORTED;
   if ((((uintptr_t)hidden | (uintptr_t)weight | (uintptr_t)workspace | (uintptr_t)d_hidden | (uintptr_t)d_weight) & 15))
     return AA_ERR_INVALID_ARGUMENT;
   const Workspace w = plan(T, H, V);
@@ -216,6 +257,7 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
   char* ws = (char*)workspace;
   uint16_t* ds = (uint16_t*)(ws + w.off_ds);  // [chunk, V]: logits of the chunk, then their gradient in place
   launch_transpose(st, (const uint16_t*)weight, V, H, H, (uint16_t*)(ws + w.off_wt));
+  const WeightGrad dw = weight_grad(w, ws, d_weight, d_weight_dtype, T);
   for (int64_t t0 = 0; t0 < T; t0 += w.chunk) {
     const int64_t n_tok = (T - t0) < w.chunk ? (T - t0) : w.chunk;
     int64_t act = T_active - t0;
@@ -228,8 +270,9 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
                                        at(mask_eff), at(behave_w), params, n_valid, grad_scale, logp + t0, at(entropy),
                                        nullptr, nullptr, at(stat_loss), at(ratio), at(flags), ds, work, stream);
     if (rc != AA_OK) return rc;
-    if (!panel_gradients(st, w, ws, hid, n_tok, H, V, (uint16_t*)d_hidden + t0 * H, d_weight, t0 == 0))
+    if (!panel_gradients(st, w, ws, hid, n_tok, H, V, (uint16_t*)d_hidden + t0 * H, dw.acc, dw.acc_f32, t0 == 0))
       return AA_ERR_LAUNCH;
   }
+  finish_weight_grad(st, dw, d_weight, V, H);
   return launch_status();
 }

@@ -665,18 +665,18 @@ class _LmHeadLogprobsEntropy(torch.autograd.Function):
         g_logp = torch.zeros(T, dtype=torch.float32, device=dev) if g_logp is None else _f32(g_logp)
         g_entropy = None if g_entropy is None else _f32(g_entropy)
         d_hidden = torch.empty_like(hidden)
-        d_weight = torch.empty(V, H, dtype=torch.float32, device=dev)
+        d_weight = torch.empty_like(weight)  # bf16: rounded once, after fp32 accumulation over the chunks
         ws = _lmhead_workspace(T, H, V, dev)
         with torch.cuda.device(dev):
             N.check(
                 lib.aa_lmhead_bwd(
                     _ptr(hidden), _ptr(weight), T, H, V, _ptr(labels), 1.0 / ctx.temperature, _ptr(row_lse),
-                    _ptr(row_ez), _ptr(g_logp), _ptr(g_entropy), _ptr(d_hidden), _ptr(d_weight), _ptr(ws),
-                    ws.numel(), _stream(dev),
+                    _ptr(row_ez), _ptr(g_logp), _ptr(g_entropy), _ptr(d_hidden), _ptr(d_weight),
+                    _DTYPES[d_weight.dtype], _ptr(ws), ws.numel(), _stream(dev),
                 ),
                 "aa_lmhead_bwd",
             )
-        return d_hidden, d_weight.to(weight.dtype), None, None
+        return d_hidden, d_weight, None, None
 
 
 def lm_head_logprobs_entropy(
@@ -721,7 +721,7 @@ class _FusedLmHeadPpo(torch.autograd.Function):
         flags = torch.empty(T_active, dtype=torch.uint8, device=dev)
         loss = torch.empty((), **f32)
         d_hidden = torch.empty_like(hidden)
-        d_weight = torch.empty(V, H, **f32)
+        d_weight = torch.empty_like(weight)  # bf16: rounded once, after fp32 accumulation over the chunks
         ws = _lmhead_workspace(T, H, V, dev)
         with torch.cuda.device(dev):
             st = _stream(dev)
@@ -730,7 +730,7 @@ class _FusedLmHeadPpo(torch.autograd.Function):
                     _ptr(hidden), _ptr(weight), T, H, V, _ptr(labels), 1.0 / float(temperature), T_active, _ptr(prox),
                     _ptr(adv), _ptr(mask_eff), _ptr(behave_w), C.byref(params), _ptr(n_valid), _ptr(grad_scale),
                     _ptr(logp), _ptr(entropy), _ptr(stat_loss), _ptr(ratio), _ptr(flags), _ptr(d_hidden),
-                    _ptr(d_weight), _ptr(_work_words(dev)), _ptr(ws), ws.numel(), st,
+                    _ptr(d_weight), _DTYPES[d_weight.dtype], _ptr(_work_words(dev)), _ptr(ws), ws.numel(), st,
                 ),
                 "aa_lmhead_ppo_fused",
             )
@@ -740,7 +740,7 @@ class _FusedLmHeadPpo(torch.autograd.Function):
                 ),
                 "aa_masked_sum",
             )
-        ctx.save_for_backward(d_hidden, d_weight.to(weight.dtype))
+        ctx.save_for_backward(d_hidden, d_weight)
         ctx.mark_non_differentiable(logp, entropy, stat_loss, ratio, flags)
         return loss, logp, entropy, stat_loss, ratio, flags
 

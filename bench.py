@@ -348,7 +348,7 @@ def time_lmhead_step(case, kw, cfg, iters: int):
     logp, ent, sl, ratio = (torch.empty(T, **f32) for _ in range(4))
     flags = torch.empty(T, dtype=torch.uint8, device=dev)
     dh = torch.empty_like(case.hidden)
-    dw = torch.empty(V, H, **f32)
+    dw = torch.empty_like(case.weight)  # bf16, as the Python wrapper asks for
     ws = F._lmhead_workspace(T, H, V, dev)
     stream = torch.cuda.current_stream(dev)
 
@@ -358,7 +358,7 @@ def time_lmhead_step(case, kw, cfg, iters: int):
                 F._ptr(case.hidden), F._ptr(case.weight), T, H, V, F._ptr(case.labels), 1.0 / case.temperature, T,
                 F._ptr(prox), F._ptr(adv), F._ptr(mask_eff), F._ptr(w), C.byref(params), F._ptr(counts), None,
                 F._ptr(logp), F._ptr(ent), F._ptr(sl), F._ptr(ratio), F._ptr(flags), F._ptr(dh), F._ptr(dw),
-                F._ptr(F._work_words(dev)), F._ptr(ws), ws.numel(), C.c_void_p(stream.cuda_stream),
+                N.AA_BF16, F._ptr(F._work_words(dev)), F._ptr(ws), ws.numel(), C.c_void_p(stream.cuda_stream),
             ),
             "aa_lmhead_ppo_fused",
         )
@@ -383,7 +383,7 @@ def time_lmhead_op(case, iters: int):
     ws = F._lmhead_workspace(T, H, V, dev)
     g = torch.randn(T, **f32) * case.loss_mask.float() / T
     dh = torch.empty_like(case.hidden)
-    dw = torch.empty(V, H, **f32)
+    dw = torch.empty_like(case.weight)  # bf16, as the Python wrapper asks for
     stream = torch.cuda.current_stream(dev)
     st = C.c_void_p(stream.cuda_stream)
     inv_t = 1.0 / case.temperature
@@ -395,8 +395,8 @@ def time_lmhead_op(case, iters: int):
 
     def bwd():
         N.check(lib.aa_lmhead_bwd(F._ptr(case.hidden), F._ptr(case.weight), T, H, V, F._ptr(case.labels), inv_t,
-                                  F._ptr(lse), F._ptr(ez), F._ptr(g), None, F._ptr(dh), F._ptr(dw), F._ptr(ws),
-                                  ws.numel(), st), "aa_lmhead_bwd")
+                                  F._ptr(lse), F._ptr(ez), F._ptr(g), None, F._ptr(dh), F._ptr(dw), N.AA_BF16,
+                                  F._ptr(ws), ws.numel(), st), "aa_lmhead_bwd")
 
     f_ms, _ = time_events(fwd, iters, stream)
     b_ms, _ = time_events(bwd, iters, stream)

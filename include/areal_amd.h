@@ -359,7 +359,8 @@ int aa_masked_moments(const float* const* values, int n_tensors,
 /* Bytes of workspace aa_lmhead_fwd / aa_lmhead_bwd / aa_lmhead_ppo_fused need
  * for these sizes: about 4 * min(T, 16384) * V + 2 * H * V bytes (one chunk of
  * bf16 logits and its transposed copy, a transposed copy of the weight) plus
- * 128 MiB for the GEMM library. */
+ * 128 MiB for the GEMM library, plus 4 * H * V (an fp32 accumulator for a bf16
+ * d_weight) when T > 16384. */
 int64_t aa_lmhead_workspace_bytes(int64_t T, int64_t H, int64_t V);
 
 /*
@@ -376,8 +377,10 @@ int aa_lmhead_fwd(const void* hidden, const void* weight, int64_t T, int64_t H,
                   void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
- * Backward of aa_lmhead_fwd: d_hidden [T, H] bf16 and d_weight [V, H] fp32
- * (overwritten, fp32 accumulation), given g_logp and optional g_entropy.
+ * Backward of aa_lmhead_fwd: d_hidden [T, H] bf16 and d_weight [V, H]
+ * (overwritten), given g_logp and optional g_entropy.  d_weight_dtype is
+ * AA_F32 or AA_BF16; either way the sum over tokens is accumulated in fp32
+ * (bf16: rounded once at the end).
  * Per chunk: the logits GEMM again, the kernel of aa_logits_bwd in place, and
  * the two gradient GEMMs (6 T V H flops for the 4 T V H of the backward).
  */
@@ -385,8 +388,8 @@ int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, int64_t H,
                   int64_t V, const int64_t* labels, float inv_temperature,
                   const float* row_lse, const float* row_ez,
                   const float* g_logp, const float* g_entropy, void* d_hidden,
-                  float* d_weight, void* workspace, int64_t workspace_bytes,
-                  void* stream);
+                  void* d_weight, int d_weight_dtype, void* workspace,
+                  int64_t workspace_bytes, void* stream);
 
 /*
  * Whole training step of the lm_head + PPO actor loss for one micro-batch,
@@ -402,7 +405,8 @@ int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, int64_t H,
  * more than one chunk of logits in memory.
  *
  * Per-token arguments, params, n_valid, grad_scale, work: as in
- * aa_logits_ppo_fused.  d_hidden [T, H] bf16 and d_weight [V, H] fp32 are
+ * aa_logits_ppo_fused.  d_hidden [T, H] bf16 and d_weight [V, H] (AA_F32 or
+ * AA_BF16, fp32 accumulation either way, as in aa_lmhead_bwd) are
  * overwritten.  workspace: aa_lmhead_workspace_bytes(T, H, V) bytes.
  */
 int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64_t T,
@@ -413,8 +417,9 @@ int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64_t T,
                         const aa_ppo_params* params, const int32_t* n_valid,
                         const float* grad_scale, float* logp, float* entropy,
                         float* stat_loss, float* ratio, uint8_t* flags,
-                        void* d_hidden, float* d_weight, int32_t* work,
-                        void* workspace, int64_t workspace_bytes, void* stream);
+                        void* d_hidden, void* d_weight, int d_weight_dtype,
+                        int32_t* work, void* workspace, int64_t workspace_bytes,
+                        void* stream);
 
 /* ------------------------------------------------------------------ */
 /* Packing                                                                 */

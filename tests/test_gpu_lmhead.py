@@ -176,3 +176,48 @@ def test_full_size_configuration(device, name):
     assert _cos_dev(dh_rest.float() + dh_only.float(), dh_all, device) > 0.9999
     _, _, dh_again, dw_again = run(g_rest + g_only)
     assert torch.equal(dh_all, dh_again) and torch.equal(dw_all, dw_again)
+
+
+@pytest.mark.parametrize("T,H,V", [(300, 128, 1088), (16384 + 72, 64, 640)])  # one chunk; two chunks
+def test_weight_gradient_dtypes_through_the_c_abi(device, T, H, V):
+    """aa_lmhead_bwd with d_weight as fp32 and as bf16: the fp32 result against autograd of the oracle, and the bf16
+    result equal to it up to one rounding (the sum over tokens is kept in fp32 in both)."""
+    import ctypes as C
+
+    from areal_amd import _native as N
+    from areal_amd import functional as F
+
+    lib = N.load()
+    hidden, weight, labels = _case(T, H, V, seed=T + H, w_std=0.3)
+    g = torch.Generator().manual_seed(1)
+    gl = torch.randn(T, generator=g) / T
+    h_o = hidden.float().requires_grad_(True)
+    w_o = weight.float().requires_grad_(True)
+    o_lp, _ = oracle.logprobs_entropy(oracle.lmhead_logits(h_o, w_o), labels)
+    (o_lp * gl).sum().backward()
+
+    hd, wd, ld, gd = hidden.to(device), weight.to(device), labels.to(device), gl.to(device)
+    f32 = dict(dtype=torch.float32, device=device)
+    logp, ent, lse, ez = (torch.empty(T, **f32) for _ in range(4))
+    ws = F._lmhead_workspace(T, H, V, device)
+    st = C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    N.check(lib.aa_lmhead_fwd(F._ptr(hd), F._ptr(wd), T, H, V, F._ptr(ld), 1.0, F._ptr(logp), F._ptr(ent), F._ptr(lse),
+                              F._ptr(ez), F._ptr(ws), ws.numel(), st), "aa_lmhead_fwd")
+    out = {}
+    for dt, code in ((torch.float32, N.AA_F32), (torch.bfloat16, N.AA_BF16)):
+        dh = torch.empty_like(hd)
+        dw = torch.full((V, H), float("nan"), dtype=dt, device=device)
+        N.check(lib.aa_lmhead_bwd(F._ptr(hd), F._ptr(wd), T, H, V, F._ptr(ld), 1.0, F._ptr(lse), F._ptr(ez), F._ptr(gd),
+                                  None, F._ptr(dh), F._ptr(dw), code, F._ptr(ws), ws.numel(), st), "aa_lmhead_bwd")
+        out[dt] = (dh.cpu().float(), dw.cpu().float())
+    dh32, dw32 = out[torch.float32]
+    dh16, dw16 = out[torch.bfloat16]
+    assert cosine(dw32, w_o.grad) > 0.9999 and cosine(dh32, h_o.grad) > 0.9999
+    assert torch.equal(dh32, dh16)
+    scale = float(dw32.abs().max())
+    assert float((dw16 - dw32).abs().max()) <= scale * 2.0 ** -8 * 1.01     # half a bf16 step at the largest magnitude
+    assert cosine(dw16, dw32) > 0.99999
+    # an unknown dtype code is refused
+    rc = lib.aa_lmhead_bwd(F._ptr(hd), F._ptr(wd), T, H, V, F._ptr(ld), 1.0, F._ptr(lse), F._ptr(ez), F._ptr(gd), None,
+                           F._ptr(dh), F._ptr(dw), N.AA_F16, F._ptr(ws), ws.numel(), st)
+    assert rc == 2  # AA_ERR_UNSUPPORTED
