@@ -421,7 +421,8 @@ __global__ __launch_bounds__(NT) void k_fused_generic(const void* __restrict__ l
 // logits as NCH 16-byte chunks per thread, so HBM sees exactly one read of the
 // row and one write of its gradient.  Requires V % 8 == 0, 16-byte aligned
 // rows and 8192 * (NCH - 1) < V <= 8192 * NCH, so that only the last chunk can
-// be partly out of range.  Rows are addressed through buffer descriptors: one
+// be partly out of range (longer rows: the EXT variant below, which adds chunks
+// held in LDS and chunks streamed once per pass).  Rows are addressed through buffer descriptors: one
 // VGPR offset per thread, and the hardware drops out-of-range lanes (loads
 // return 0, stores are ignored).  Loads take the chunk offset in the scalar
 // offset operand.  Stores must NOT: with a register in the scalar-offset operand
@@ -487,22 +488,94 @@ __device__ __forceinline__ void grad_pass(const u32x4_t (&d)[NCH], float g, floa
   }
 }
 
+// ---- rows longer than the register file --------------------------------------
+// The extended variant of k_fused_regs (EXT) keeps kExtRegChunks chunks of the row in registers, up to
+// kExtLdsChunks more in LDS (brought in by direct-to-LDS loads, each thread reads back only the 16 bytes its own
+// lane deposited) and streams up to kExtTailChunks last chunks from memory once per pass.  These helpers are the
+// per-chunk bodies of the three passes for a chunk that is not in registers.
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+constexpr int kExtRegChunks = 21;
+constexpr int kExtLdsChunks = 9;
+constexpr int kExtTailChunks = 2;
+
+struct MinMax16 {
+  s16x2_t smax, smin;
+  u16x2_t umax, umin;
+};
+
+__device__ __forceinline__ void minmax_chunk(MinMax16& m, const u32x4_t v) {
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const uint32_t w = v[q];
+    const s16x2_t ws = __builtin_bit_cast(s16x2_t, w);
+    const u16x2_t wu = __builtin_bit_cast(u16x2_t, w);
+    m.smax = __builtin_elementwise_max(m.smax, ws);
+    m.smin = __builtin_elementwise_min(m.smin, ws);
+    m.umax = __builtin_elementwise_max(m.umax, wu);
+    m.umin = __builtin_elementwise_min(m.umin, wu);
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ void sum_chunk(const u32x4_t v, float c, float k, float& s, float& u) {
+  float cs = 0.f, cu = 0.f;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const float lo = Elem<DT>::lo(v[q]), hi = Elem<DT>::hi(v[q]);
+    const float t0 = fmaf(lo, c, -k), t1 = fmaf(hi, c, -k);
+    const float e0 = fast_exp2(t0), e1 = fast_exp2(t1);
+    cs += e0 + e1;
+    cu = fmaf(t0, e0, cu);
+    cu = fmaf(t1, e1, cu);
+  }
+  s += cs;
+  u += cu;
+}
+
+// gradient of chunk `ci` (any chunk index), as grad_pass does it for the register chunks
+template <int DT>
+__device__ __forceinline__ u32x4_t grad_chunk(const u32x4_t v, float c, float kk, float lab_add, bool g_positive,
+                                              int yv, int y_elem, int ci, int tid) {
+  float o[8];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const float e0 = fast_exp2(fmaf(Elem<DT>::lo(v[q]), c, kk));
+    const float e1 = fast_exp2(fmaf(Elem<DT>::hi(v[q]), c, kk));
+    o[2 * q] = g_positive ? -e0 : e0;
+    o[2 * q + 1] = g_positive ? -e1 : e1;
+  }
+  if (yv - ci * 1024 == tid) {
+#pragma unroll
+    for (int q = 0; q < 8; ++q)
+      if (q == y_elem) o[q] += lab_add;
+  }
+  u32x4_t r;
+  r[0] = Elem<DT>::pack(o[0], o[1]);
+  r[1] = Elem<DT>::pack(o[2], o[3]);
+  r[2] = Elem<DT>::pack(o[4], o[5]);
+  r[3] = Elem<DT>::pack(o[6], o[7]);
+  return r;
+}
+
 // Rows are handed out through a device counter (work[0]) so that compute
 // units that get through their rows faster take more of them; work[1] counts
 // finished workgroups, and the last one puts both words back to zero, which is
 // the state the next launch expects.  With work == nullptr the rows are dealt
 // round-robin (t, t + gridDim.x, ...).
-template <int DT, int NCH>
+// With EXT the row continues past the NCH register chunks: n_lds chunks in dynamic LDS, then the tail chunks.
+template <int DT, int NCH, bool EXT = false>
 __global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ logits, int V, int64_t stride_vec,
                                                      const int64_t* __restrict__ labels, float inv_t,
                                                      const float* __restrict__ in_prox,
                                                      const float* __restrict__ in_adv,
                                                      const uint32_t* __restrict__ in_mask32, unsigned mask_mis,
                                                      const float* __restrict__ in_bw, FusedTokenArgs a,
-                                                     uint4* __restrict__ dlogits, int64_t T, int32_t* work) {
+                                                     uint4* __restrict__ dlogits, int64_t T, int32_t* work,
+                                                     int n_lds) {
   constexpr int NT = 1024;
   constexpr int kChunkBytes = NT * 16;
   const bool has_w = a.P.has_behave_weight != 0;
+  extern __shared__ __align__(16) unsigned char ext_lds[];  // EXT: n_lds chunks of 16 KiB
   __shared__ float smem[(NT / kWave) * 5];
   __shared__ int64_t next_row[2];  // written at the top of a row, read behind its barriers: two slots, no reuse race
   int slot = 0;
@@ -510,9 +583,18 @@ __global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ l
   const int tid = threadIdx.x;
   const float c = kLog2e * inv_t;
   const int voff = tid * 16;
-  const bool last_ok = (NCH - 1) * NT + tid < nvec;
+  const bool last_ok = EXT || (NCH - 1) * NT + tid < nvec;  // EXT: every register chunk is full
   float fn, gscale;
   load_loss_scale(a, fn, gscale);
+  // EXT: chunk NCH + j goes to LDS for j < n_lds; each wave deposits its 1 KiB piece, lane by lane
+  const u32x4_t* my_lds = (const u32x4_t*)ext_lds + tid;
+  const int lds_wave_off = (tid >> 6) * 1024;
+  const int tail0 = NCH + n_lds;  // first chunk that is neither in registers nor in LDS
+  auto load_lds_chunks = [&](const __amdgpu_buffer_rsrc_t rsrc) {
+    for (int j = 0; j < n_lds; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(ext_lds + j * kChunkBytes + lds_wave_off), 16, voff,
+                                               (NCH + j) * kChunkBytes, 0, kAuxStream);
+  };
 
   int64_t t = blockIdx.x;  // the host launches at most T workgroups
   const uint4* src = logits + t * stride_vec;
@@ -521,6 +603,7 @@ __global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ l
     const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, V * 2, kBufferFlags);
 #pragma unroll
     for (int i = 0; i < NCH; ++i) d[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, i * kChunkBytes, kAuxStream);
+    if constexpr (EXT) load_lds_chunks(rsrc);
   }
   int64_t y = labels[t];
   bool y_ok = (y >= 0) && (y < V);
@@ -539,6 +622,18 @@ __global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ l
     // minimum, otherwise the smallest unsigned pattern is.
     s16x2_t smax = {-32768, -32768}, smin = {32767, 32767};
     u16x2_t umax = {0, 0}, umin = {65535, 65535};
+    // EXT: the tail chunks of this row, fetched again at the top of every pass (lanes past the row read zeros)
+    __amdgpu_buffer_rsrc_t rsrc_t;
+    u32x4_t tv[kExtTailChunks];
+    bool tail_ok[kExtTailChunks];
+    if constexpr (EXT) {
+      rsrc_t = __builtin_amdgcn_make_buffer_rsrc((void*)(logits + t * stride_vec), 0, V * 2, kBufferFlags);
+#pragma unroll
+      for (int q = 0; q < kExtTailChunks; ++q) {
+        tv[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_t, voff, (tail0 + q) * kChunkBytes, kAuxStream);
+        tail_ok[q] = (tail0 + q) * NT + tid < nvec;
+      }
+    }
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       if (i < NCH - 1 || last_ok) {
@@ -554,6 +649,16 @@ __global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ l
         }
       }
     }
+    if constexpr (EXT) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the direct-to-LDS loads of this row have landed
+      MinMax16 m{smax, smin, umax, umin};
+      for (int j = 0; j < n_lds; ++j)
+        if ((NCH + j) * NT + tid < nvec) minmax_chunk(m, my_lds[j * NT]);
+#pragma unroll
+      for (int q = 0; q < kExtTailChunks; ++q)
+        if (tail_ok[q]) minmax_chunk(m, tv[q]);
+      smax = m.smax; smin = m.smin; umax = m.umax; umin = m.umin;
+    }
     const int hi_s = smax[0] > smax[1] ? smax[0] : smax[1];
     const int lo_s = smin[0] < smin[1] ? smin[0] : smin[1];
     const unsigned hi_u = umax[0] > umax[1] ? umax[0] : umax[1];
@@ -566,6 +671,11 @@ __global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ l
     ts.k = fmaxf(wave_max(mx) * c, kNegBig);
     ts.mx = mx; ts.mn = mn;
     float s = 0.f, u = 0.f;
+    if constexpr (EXT) {
+#pragma unroll
+      for (int q = 0; q < kExtTailChunks; ++q)
+        tv[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_t, voff, (tail0 + q) * kChunkBytes, kAuxStream);
+    }
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       float cs = 0.f, cu = 0.f;
@@ -581,6 +691,13 @@ __global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ l
       if (i == NCH - 1 && !last_ok) { cs = 0.f; cu = 0.f; }
       s += cs;
       u += cu;
+    }
+    if constexpr (EXT) {
+      for (int j = 0; j < n_lds; ++j)
+        if ((NCH + j) * NT + tid < nvec) sum_chunk<DT>(my_lds[j * NT], c, ts.k, s, u);
+#pragma unroll
+      for (int q = 0; q < kExtTailChunks; ++q)
+        if (tail_ok[q]) sum_chunk<DT>(tv[q], c, ts.k, s, u);
     }
     ts.s = s; ts.u = u;
     keep_packed(d);
@@ -602,14 +719,42 @@ __global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ l
 
     const __amdgpu_buffer_rsrc_t wsrc =
         __builtin_amdgcn_make_buffer_rsrc((void*)(dlogits + t * stride_vec), 0, V * 2, kBufferFlags);
+    if constexpr (EXT) {
+      if (g != 0.f) {
+#pragma unroll
+        for (int q = 0; q < kExtTailChunks; ++q)
+          tv[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_t, voff, (tail0 + q) * kChunkBytes, kAuxStream);
+      }
+    }
     if (g == 0.f) {
       const u32x4_t z = {0u, 0u, 0u, 0u};
 #pragma unroll
       for (int i = 0; i < NCH; ++i) __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, voff + i * kChunkBytes, 0, kAuxStream);
+      if constexpr (EXT) {
+        for (int j = 0; j < n_lds + kExtTailChunks; ++j)  // chunks past the row are dropped by the descriptor
+          __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, voff + (NCH + j) * kChunkBytes, 0, kAuxStream);
+      }
     } else if (g > 0.f) {
       grad_pass<DT, NCH, true>(d, g, inv_t, c, ro.lse2, y_ok ? y : -1, tid, voff, wsrc);
     } else {
       grad_pass<DT, NCH, false>(d, g, inv_t, c, ro.lse2, y_ok ? y : -1, tid, voff, wsrc);
+    }
+    if constexpr (EXT) {
+      if (g != 0.f) {
+        const float lab_add = g * inv_t;
+        const float kk = fast_log2(fabsf(lab_add)) - ro.lse2;
+        const int yv = y_ok ? (int)(y >> 3) : -1;
+        const int y_elem = (int)(y & 7);
+        for (int j = 0; j < n_lds; ++j) {
+          const u32x4_t r = grad_chunk<DT>(my_lds[j * NT], c, kk, lab_add, g > 0.f, yv, y_elem, NCH + j, tid);
+          __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + (NCH + j) * kChunkBytes, 0, kAuxStream);
+        }
+#pragma unroll
+        for (int q = 0; q < kExtTailChunks; ++q) {
+          const u32x4_t r = grad_chunk<DT>(tv[q], c, kk, lab_add, g > 0.f, yv, y_elem, tail0 + q, tid);
+          __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + (tail0 + q) * kChunkBytes, 0, kAuxStream);
+        }
+      }
     }
     if (!more) break;
     // All stores of this row are issued before the loads of the next one:
@@ -619,6 +764,10 @@ __global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ l
 #pragma unroll
       for (int i = 0; i < NCH; ++i)
         d[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_n, voff, i * kChunkBytes, kAuxStream);
+      if constexpr (EXT) {
+        asm volatile("" ::: "memory");  // the LDS reads of the gradient pass stay ahead of the next row's deposits
+        load_lds_chunks(rsrc_n);
+      }
     }
     t = tn; y = y_n; y_ok = y_ok_n; xy_raw = xy_raw_n; tin = tin_n;
   }
@@ -693,7 +842,27 @@ static void launch_regs(const void* logits, int64_t T, int V, int64_t stride, co
   const uintptr_t mask_addr = (uintptr_t)a.mask_eff;
   hipLaunchKernelGGL((k_fused_regs<DT, NCH>), dim3((unsigned)wgs), dim3(1024), 0, st, (const uint4*)logits, V,
                      stride >> 3, labels, inv_t, a.prox_logp, a.adv, (const uint32_t*)(mask_addr & ~(uintptr_t)3),
-                     (unsigned)(mask_addr & 3), a.behave_w, a, (uint4*)dlogits, T, work);
+                     (unsigned)(mask_addr & 3), a.behave_w, a, (uint4*)dlogits, T, work, 0);
+}
+
+// Rows of more than kMaxRegChunks chunks: registers + LDS + streamed tail (see k_fused_regs, EXT).
+constexpr int kMaxExtChunks = kExtRegChunks + kExtLdsChunks + kExtTailChunks;
+
+template <int DT>
+static bool launch_regs_ext(int nch, const void* logits, int64_t T, int V, int64_t stride, const int64_t* labels,
+                            float inv_t, const FusedTokenArgs& a, void* dlogits, int32_t* work, hipStream_t st) {
+  static const bool ok =
+      hipFuncSetAttribute((const void*)k_fused_regs<DT, kExtRegChunks, true>,
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kExtLdsChunks * 16384) == hipSuccess;
+  if (!ok || nch <= kExtRegChunks || nch > kMaxExtChunks) return false;
+  const int n_lds = nch - kExtRegChunks < kExtLdsChunks ? nch - kExtRegChunks : kExtLdsChunks;
+  const int64_t wgs = T < persistent_workgroups() ? T : persistent_workgroups();
+  const uintptr_t mask_addr = (uintptr_t)a.mask_eff;
+  hipLaunchKernelGGL((k_fused_regs<DT, kExtRegChunks, true>), dim3((unsigned)wgs), dim3(1024), n_lds * 16384, st,
+                     (const uint4*)logits, V, stride >> 3, labels, inv_t, a.prox_logp, a.adv,
+                     (const uint32_t*)(mask_addr & ~(uintptr_t)3), (unsigned)(mask_addr & 3), a.behave_w, a,
+                     (uint4*)dlogits, T, work, n_lds);
+  return true;
 }
 
 template <int DT>
@@ -774,12 +943,18 @@ extern "C" int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int
   a.P = *params; a.T_active = T_active;
 
   const bool fast = (dtype != AA_F32) && (V % 8 == 0) && (row_stride % 8 == 0) && (((uintptr_t)logits & 15) == 0) &&
-                    (((uintptr_t)dlogits & 15) == 0) && (V >= 8 * 1024) && (V <= kMaxRegChunks * 8192) && (T_active > 0);
+                    (((uintptr_t)dlogits & 15) == 0) && (V >= 8 * 1024) && (V <= kMaxExtChunks * 8192) && (T_active > 0);
   if (fast) {
     const int nch = (int)((V / 8 + 1023) / 1024);
-    bool ok = (dtype == AA_BF16)
-                  ? dispatch_regs<AA_BF16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st)
-                  : dispatch_regs<AA_F16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st);
+    bool ok;
+    if (nch <= kMaxRegChunks)
+      ok = (dtype == AA_BF16)
+               ? dispatch_regs<AA_BF16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st)
+               : dispatch_regs<AA_F16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st);
+    else
+      ok = (dtype == AA_BF16)
+               ? launch_regs_ext<AA_BF16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st)
+               : launch_regs_ext<AA_F16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st);
     if (ok) return launch_status();
   }
   const int vec_ok = rows_vec_ok(logits, dlogits, dtype) ? 1 : 0;

@@ -78,6 +78,11 @@ def _compare(case, got, want, pad=0):
         (8200, torch.float16, 8, 40),      # 2 chunks, the second almost empty
         (50257, torch.bfloat16, 4, 20),    # generic rows (V % 8 != 0)
         (4099, torch.float32, 4, 20),      # generic rows, fp32 logits
+        (172040, torch.bfloat16, 4, 12),   # 22 chunks: 21 in registers, one (a single 16-byte piece of it) in LDS
+        (245760, torch.bfloat16, 4, 12),   # 30 chunks: registers and LDS full, no tail
+        (250008, torch.float16, 4, 12),    # 31 chunks: a partial streamed tail chunk
+        (262144, torch.bfloat16, 4, 12),   # 32 chunks: the largest row of the register / LDS / tail kernel
+        (262152, torch.bfloat16, 4, 12),   # one vector more: generic rows again
     ],
 )
 def test_fused_config0_shape_matches_oracle(device, V, dtype, lo, hi):
@@ -85,6 +90,25 @@ def test_fused_config0_shape_matches_oracle(device, V, dtype, lo, hi):
     case = synth.make_logits_case("t", lengths, V, V, device, synth.per_sequence_normal_advantages(lengths, 3),
                                   dtype=dtype, ppo=dict(eps_clip=0.2))
     _finish_case(case)
+    _compare(case, _fused_step(case), _oracle_step(case))
+
+
+def test_long_rows_labels_and_extrema_in_every_region(device):
+    """V = 262144: labels and the row maximum / minimum placed in the register, LDS and streamed parts of the row."""
+    V = 262144
+    spots = [0, 8191, 21 * 8192 - 1, 21 * 8192, 25 * 8192 + 77, 30 * 8192 - 1, 30 * 8192, 31 * 8192 + 5, V - 1]
+    lengths = [len(spots), len(spots)]
+    case = synth.make_logits_case("t", lengths, V, 11, device, synth.per_sequence_normal_advantages(lengths, 4),
+                                  ppo=dict(eps_clip=0.2, eps_clip_higher=0.28, c_clip=3.0), temperature=0.9)
+    n = len(spots)
+    with torch.no_grad():
+        for r, j in enumerate(spots):
+            case.labels[r] = j                      # first sequence: the label sits at the spot
+            case.logits[n + r, j] = 30.0            # second sequence: the maximum does ...
+            case.logits[n + r, spots[-1 - r]] = -40.0   # ... and the minimum at the mirrored spot
+    _finish_case(case)
+    case.loss_mask[:] = True
+    case.loss_mask[4] = False                      # one masked row: its gradient must be exactly zero
     _compare(case, _fused_step(case), _oracle_step(case))
 
 
