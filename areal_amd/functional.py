@@ -282,6 +282,25 @@ def _rejection_sampling_device(prox, old, mask_u8, shape, cu_seqlens, cfg):
     return mask_out, w, counts
 
 
+class _HostCounts:
+    """The counters of the rejection-sampling kernel on their way to the host.
+
+    The copy into pinned memory is queued right behind the kernel and gets an event of its own, so reading the
+    counters later (``filtered_fraction`` is a Python float, as in the reference) waits for that copy only and not
+    for the long kernels queued after it: the host keeps running ahead of the GPU."""
+
+    def __init__(self, counts: torch.Tensor):
+        self._host = torch.empty(counts.shape, dtype=counts.dtype, pin_memory=True)
+        with torch.cuda.device(counts.device):
+            self._host.copy_(counts, non_blocking=True)
+            self._event = torch.cuda.Event()
+            self._event.record()
+
+    def tolist(self):
+        self._event.synchronize()
+        return self._host.tolist()
+
+
 def _validate_rs(cfg) -> None:
     for field, table in (("level", N.RS_LEVEL), ("action", N.RS_ACTION), ("agg", N.RS_AGG)):
         if getattr(cfg, field) not in table:
@@ -440,6 +459,7 @@ def ppo_actor_loss_fn(
     if rejection_sampling is not None:
         _validate_rs(rejection_sampling)
         mask_eff, w, counts = _rejection_sampling_device(prox, old, m8, shape, cu_seqlens, rejection_sampling)
+        host_counts = _HostCounts(counts)
         if rejection_sampling.action != "mask":
             mask_eff = m8
         n_valid = counts  # counts[0] is the non-zero count of the original mask
@@ -455,7 +475,7 @@ def ppo_actor_loss_fn(
         dual_clip_mask=(flags & 2).bool().view(shape),
     )
     if rejection_sampling is not None:
-        _rs_stats(stat, prox, old, mask_eff, w, counts, shape)
+        _rs_stats(stat, prox, old, mask_eff, w, host_counts, shape)
     return loss, stat
 
 
@@ -596,6 +616,7 @@ def fused_logprobs_ppo_loss(
     if rejection_sampling is not None:
         _validate_rs(rejection_sampling)
         mask_eff, w, counts = _rejection_sampling_device(prox, old, m8, loss_mask.shape, cu_seqlens, rejection_sampling)
+        host_counts = _HostCounts(counts)
         if rejection_sampling.action != "mask":
             mask_eff = m8
         n_valid = counts
@@ -617,7 +638,7 @@ def fused_logprobs_ppo_loss(
         vocab_max_logits=vmax[:T_active],
     )
     if rejection_sampling is not None:
-        _rs_stats(stat, prox, old, mask_eff, w, counts, loss_mask.shape)
+        _rs_stats(stat, prox, old, mask_eff, w, host_counts, loss_mask.shape)
     return loss, stat
 
 
@@ -829,6 +850,7 @@ def fused_lm_head_ppo_loss(
     if rejection_sampling is not None:
         _validate_rs(rejection_sampling)
         mask_eff, w, counts = _rejection_sampling_device(prox, old, m8, loss_mask.shape, cu_seqlens, rejection_sampling)
+        host_counts = _HostCounts(counts)
         if rejection_sampling.action != "mask":
             mask_eff = m8
         n_valid = counts
@@ -849,7 +871,7 @@ def fused_lm_head_ppo_loss(
         entropy=entropy[:T_active],
     )
     if rejection_sampling is not None:
-        _rs_stats(stat, prox, old, mask_eff, w, counts, loss_mask.shape)
+        _rs_stats(stat, prox, old, mask_eff, w, host_counts, loss_mask.shape)
     return loss, stat
 
 
