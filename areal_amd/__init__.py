@@ -3,7 +3,7 @@
 Importing the package does not load the HIP library; the first op call does, and
 raises ``NativeLibraryError`` if ``libareal_amd.so`` has not been built.
 """
-from .actor_ops import apply_m2po_masking, compute_prox_logp_approximations
+from .actor_ops import apply_m2po_masking, compute_prox_logp_approximations, distillation_terms
 from .advantages import Normalization, gae_advantages, kl_regularized_rewards, masked_moments
 from .config import NormConfig, RejectionSamplingConfig
 from .functional import (
@@ -39,6 +39,7 @@ __all__ = [
     "apply_m2po_masking",
     "apply_rejection_sampling",
     "compute_prox_logp_approximations",
+    "distillation_terms",
     "fused_lm_head_ppo_loss",
     "fused_logprobs_ppo_loss",
     "gae_advantages",

@@ -73,3 +73,53 @@ def apply_m2po_masking(old_logp: torch.Tensor, prox_logp: torch.Tensor, loss_mas
         N.check(lib.aa_m2po_mask(_ptr(lo), _ptr(lp), _ptr(m8), n, float(m2_threshold), _ptr(out), _ptr(info), _ptr(ws),
                                  ws.numel(), _stream(dev)), "aa_m2po_mask")
     return out.view(shape)
+
+
+class _KdTerms(torch.autograd.Function):
+    """sum(term) / max(sum(mask), 1) of ``aa_kd_terms`` and the per-token terms; differentiable in ``logp``."""
+
+    @staticmethod
+    def forward(ctx, logp, old, teacher, mask_u8, pure):
+        from .functional import _count_nonzero
+
+        lib = N.load()
+        dev = logp.device
+        n = logp.numel()
+        term = torch.empty(n, dtype=torch.float32, device=dev)
+        dterm = torch.empty(n, dtype=torch.float32, device=dev)
+        mean = torch.empty((), dtype=torch.float32, device=dev)
+        n_valid = _count_nonzero(mask_u8)
+        with torch.cuda.device(dev):
+            st = _stream(dev)
+            N.check(lib.aa_kd_terms(_ptr(logp), _ptr(old), _ptr(teacher), _ptr(mask_u8), n, 1 if pure else 0, _ptr(term),
+                                    _ptr(dterm), st), "aa_kd_terms")
+            N.check(lib.aa_masked_sum(_ptr(term), None, n, _ptr(n_valid), None, _ptr(mean), st), "aa_masked_sum")
+        ctx.save_for_backward(dterm, n_valid)
+        ctx.mark_non_differentiable(term)
+        return mean, term
+
+    @staticmethod
+    def backward(ctx, g_mean, _g_term):
+        dterm, n_valid = ctx.saved_tensors
+        return dterm * (g_mean / n_valid.clamp(min=1).float()), None, None, None, None
+
+
+def distillation_terms(logprobs: torch.Tensor, old_logp: torch.Tensor | None, teacher_logp: torch.Tensor,
+                       loss_mask: torch.Tensor, pure: bool) -> tuple[torch.Tensor, torch.Tensor]:
+    """The reverse-KL terms of the joint-distillation branch of the actor loss; actor.py:482-511.
+
+    ``pure`` (``rl_loss_weight == 0``): per token ``exp(logp - old) * (teacher - logp.detach()) * mask``
+    (actor.py:494-498); otherwise ``(logp - teacher) * mask`` (actor.py:505).  Returns
+    ``(sum(term) / max(sum(mask), 1), term)``: the first is differentiable in ``logprobs``, the second is detached.
+    """
+    _require_gpu(logprobs, "logprobs")
+    shape = logprobs.shape
+    if teacher_logp.shape != shape or loss_mask.shape != shape or (pure and old_logp.shape != shape):
+        raise ValueError("logprobs, old_logp, teacher_logp and loss_mask must have the same shape")
+    lp = logprobs.reshape(-1)
+    if lp.dtype != torch.float32 or not lp.is_contiguous():
+        lp = lp.float().contiguous()
+    old = _f32(old_logp.detach()).reshape(-1) if pure else None
+    mean, term = _KdTerms.apply(lp, old, _f32(teacher_logp.detach()).reshape(-1), _mask_u8(loss_mask).reshape(-1),
+                                bool(pure))
+    return mean, term.view(shape)

@@ -470,6 +470,31 @@ __global__ __launch_bounds__(256) void k_prox_approx(const float* __restrict__ o
   }
 }
 
+// ---- joint-distillation terms of the actor loss (actor.py:482-511) ------------------------------------------------
+// pure (rl_loss_weight == 0):  term = exp(logp - old) * (teacher - logp) * mask,  d term / d logp = term
+//                              (the reward teacher - logp is detached; the importance weight carries the gradient)
+// joint:                       term = (logp - teacher) * mask,                     d term / d logp = mask
+__global__ __launch_bounds__(256) void k_kd_terms(const float* __restrict__ logp, const float* __restrict__ old,
+                                                  const float* __restrict__ teacher, const uint8_t* __restrict__ mask,
+                                                  int64_t n, int pure, float* __restrict__ term,
+                                                  float* __restrict__ dterm) {
+  const int64_t step = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += step) {
+    const float m = mask[i] ? 1.f : 0.f;
+    const float lp = logp[i], tl = teacher[i];
+    float t, d;
+    if (pure) {
+      t = expf(lp - old[i]) * (tl - lp) * m;  // (x * y) * mask as the reference orders it: NaN/inf propagate alike
+      d = t;
+    } else {
+      t = (lp - tl) * m;
+      d = m;
+    }
+    term[i] = t;
+    dterm[i] = d;
+  }
+}
+
 static unsigned grid_for(int64_t n) {
   int64_t b = (n + 255) / 256;
   if (b > 2048) b = 2048;
@@ -583,5 +608,16 @@ extern "C" int aa_prox_logp_approx(const float* old_logp, const float* logp, con
   if (!old_logp || !logp || !versions || !out) return AA_ERR_INVALID_ARGUMENT;
   hipLaunchKernelGGL(k_prox_approx, dim3(grid_for(n)), dim3(256), 0, (hipStream_t)stream, old_logp, logp, versions, n,
                      current_version, method, out);
+  return launch_status();
+}
+
+extern "C" int aa_kd_terms(const float* logp, const float* old_logp, const float* teacher_logp, const uint8_t* mask,
+                           int64_t n, int pure_distillation, float* term, float* dterm, void* stream) {
+  if (n < 0) return AA_ERR_INVALID_ARGUMENT;
+  if (n == 0) return AA_OK;
+  if (!logp || !teacher_logp || !mask || !term || !dterm || (pure_distillation && !old_logp))
+    return AA_ERR_INVALID_ARGUMENT;
+  hipLaunchKernelGGL(k_kd_terms, dim3(grid_for(n)), dim3(256), 0, (hipStream_t)stream, logp, old_logp, teacher_logp, mask,
+                     n, pure_distillation ? 1 : 0, term, dterm);
   return launch_status();
 }

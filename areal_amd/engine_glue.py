@@ -200,19 +200,17 @@ def grpo_loss_fn(
     vocab_max_logits: torch.Tensor | None = None,
 ) -> tuple[torch.Tensor, dict]:
     """The actor's loss function for one micro-batch (areal/trainer/ppo/actor.py:408-480) on the GPU ops: proximal
-    log-probs resolved, optional M2PO masking, SAPO or clipped PPO loss.  The knowledge-distillation branch
-    (``teacher_logp``, actor.py:482-511) is not part of this build and raises.
+    log-probs resolved, optional M2PO masking, SAPO or clipped PPO loss, and the joint-distillation terms
+    (``teacher_logp`` with ``rl_loss_weight`` / ``distill_loss_weight``, actor.py:482-511).
 
     Returns ``(loss, stat)``.  ``stat`` is the per-token dict of the loss function plus ``"reduced"``: what the
     reference hands to its statistics tracker tensor by tensor (actor.py:513-573) as sums / averages / extrema
     under the same denominators, computed in one launch per denominator.
     """
-    from .actor_ops import apply_m2po_masking
+    from .actor_ops import apply_m2po_masking, distillation_terms
     from .advantages import masked_moments
     from .functional import sapo_loss_fn
 
-    if input_data.get("teacher_logp") is not None:
-        raise NotImplementedError("joint distillation (teacher_logp) is outside the scope of this build")
     old_logp = input_data["logprobs"]
     advantages = input_data["advantages"]
     loss_mask = input_data["loss_mask"].bool()
@@ -233,6 +231,19 @@ def grpo_loss_fn(
         loss, stat = ppo_actor_loss_fn(logprobs, prox_logp, old_logp, advantages, eps_clip, loss_mask, eps_clip_higher,
                                        c_clip, rejection_sampling, importance_sampling_level,
                                        input_data.get("cu_seqlens"))
+    rkl_stat = None
+    teacher_logp = input_data.get("teacher_logp")
+    if teacher_logp is not None:
+        rl_loss_weight = input_data.get("rl_loss_weight", 1.0)
+        distill_loss_weight = input_data.get("distill_loss_weight", 0.005)
+        if rl_loss_weight == 0:  # pure distillation with the reverse KL as an importance-weighted reward
+            mean, term = distillation_terms(logprobs, old_logp, teacher_logp, loss_mask, pure=True)
+            loss = -distill_loss_weight * mean
+            rkl_stat = -term
+        else:                    # the RL loss plus a reverse-KL penalty
+            mean, term = distillation_terms(logprobs, None, teacher_logp, loss_mask, pure=False)
+            loss = rl_loss_weight * loss + distill_loss_weight * mean
+            rkl_stat = term
     per_valid = dict(
         importance_weight=stat["importance_weight"], approx_kl=stat["approx_kl"], new_logp=logprobs.detach(),
         old_logp=old_logp, entropy=entropy.float(), actor_loss=stat["loss"], clip_ratio=stat["clip_mask"].float(),
@@ -241,6 +252,8 @@ def grpo_loss_fn(
     if use_sapo_loss:
         per_valid.update(sapo_soft_gate=stat["sapo_soft_gate"], sapo_scaled_gate_pos=stat["sapo_scaled_gate_pos"],
                          sapo_scaled_gate_neg=stat["sapo_scaled_gate_neg"])
+    if rkl_stat is not None:
+        per_valid.update(rkl_loss=rkl_stat)
     reduced = masked_moments(per_valid, loss_mask)
     if not use_sapo_loss:
         clip_mask = stat["clip_mask"]

@@ -259,6 +259,25 @@ int aa_prox_logp_approx(const float* old_logp, const float* logp,
                         int current_version, int method, float* out,
                         void* stream);
 
+/*
+ * Per-token terms of the joint-distillation branch of grpo_loss_fn
+ * (trainer/ppo/actor.py:482-511), with mask the bool loss mask as bytes:
+ *   pure_distillation != 0 (rl_loss_weight == 0, :493-503):
+ *     term = exp(logp - old_logp) * (teacher_logp - logp) * mask, the reward
+ *     (teacher_logp - logp) detached, so dterm = d term / d logp = term;
+ *     loss = -distill_loss_weight * sum(term) / max(sum(mask), 1),
+ *     rkl statistic = -term.
+ *   otherwise (:504-511): term = (logp - teacher_logp) * mask, dterm = mask;
+ *     loss = rl_loss_weight * loss + distill_loss_weight * sum(term) /
+ *     max(sum(mask), 1), rkl statistic = term.
+ * The sums are finished by aa_masked_sum.  old_logp may be NULL in the second
+ * form.
+ */
+int aa_kd_terms(const float* logp, const float* old_logp,
+                const float* teacher_logp, const uint8_t* mask, int64_t n,
+                int pure_distillation, float* term, float* dterm,
+                void* stream);
+
 /* Bytes of 256-byte aligned workspace aa_m2po_mask needs for n tokens. */
 int64_t aa_m2po_workspace_bytes(int64_t n);
 

@@ -25,7 +25,7 @@ from .ppo import (
     sequence_level_ratio_and_advantages,
 )
 from .advantages import gae, masked_moments, normalization
-from .siblings import critic_loss, m2po_mask, prox_logp_approximations, sapo_loss
+from .siblings import critic_loss, distillation_loss, m2po_mask, prox_logp_approximations, sapo_loss
 from .pipeline import lmhead_logits, logits_ppo_step
 
 __all__ = [
@@ -42,6 +42,7 @@ __all__ = [
     "masked_moments",
     "normalization",
     "critic_loss",
+    "distillation_loss",
     "m2po_mask",
     "prox_logp_approximations",
     "sapo_loss",

@@ -128,3 +128,19 @@ def m2po_mask(old_logp, prox_logp, loss_mask, m2_threshold):
     full = torch.zeros_like(mask_flat, dtype=torch.bool)
     full[mask_flat] = sel_mask
     return full.view_as(loss_mask)
+
+
+def distillation_loss(loss, logprobs, old_logp, teacher_logp, loss_mask, rl_loss_weight=1.0, distill_loss_weight=0.005):
+    """``(loss, rkl_stat)`` after the joint-distillation branch of ``grpo_loss_fn``; actor.py:482-511."""
+    teacher_logp = teacher_logp.detach()                                          # :489-491
+    if rl_loss_weight == 0:                                                       # :493
+        rkl_reward = teacher_logp - logprobs.detach()                             # :495
+        importance_weight = torch.exp(logprobs - old_logp)                        # :496
+        rkl_weighted_term = importance_weight * rkl_reward * loss_mask            # :498
+        kd_coef = -1 * distill_loss_weight                                        # :500
+        loss = kd_coef * rkl_weighted_term.sum() / loss_mask.sum().clamp(min=1)   # :501
+        return loss, -1 * rkl_weighted_term                                       # :503
+    rkl_penalty_per_token = (logprobs - teacher_logp) * loss_mask                 # :506
+    rkl_penalty = rkl_penalty_per_token.sum() / loss_mask.sum().clamp(min=1)      # :507
+    loss = rl_loss_weight * loss + distill_loss_weight * rkl_penalty              # :509
+    return loss, rkl_penalty_per_token                                            # :511

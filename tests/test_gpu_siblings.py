@@ -198,3 +198,47 @@ def test_grpo_loss_fn_matches_composed_oracle(device, variant):
             grpo_loss_fn(y, ent.to(device), d_dev, **dict(kw, use_decoupled_loss=True))
     with pytest.raises(ValueError, match="compute_logp\\(\\) was skipped incorrectly"):
         grpo_loss_fn(y, ent.to(device), dict(d_dev, prox_logp=None), 0.2, None, None)
+
+
+@pytest.mark.parametrize("rl_weight", [0, 0.8])
+def test_grpo_loss_fn_joint_distillation(device, rl_weight):
+    """teacher_logp in the micro-batch (actor.py:482-511): pure reverse-KL distillation and the joint RL + KD loss."""
+    from areal_amd.engine_glue import grpo_loss_fn
+    from oracle import ppo as OP
+
+    n = 500
+    lp, old, adv, mask = _tok(n, 21)
+    g = torch.Generator().manual_seed(22)
+    prox = lp + 0.1 * torch.randn(n, generator=g)
+    teacher = lp + 0.4 * torch.randn(n, generator=g)
+    ent = torch.rand(n, generator=g)
+    cu = torch.tensor([0, 150, 500], dtype=torch.int32)
+    data = dict(logprobs=old, advantages=adv, loss_mask=mask, prox_logp=prox, cu_seqlens=cu, teacher_logp=teacher,
+                rl_loss_weight=rl_weight, distill_loss_weight=0.02)
+    x = lp.clone().requires_grad_(True)
+    w_loss, _ = OP.ppo_actor_loss(x, prox, old, adv, 0.2, mask, None, None, None, "token", cu)
+    w_loss, w_rkl = S.distillation_loss(w_loss, x, old, teacher, mask, rl_weight, 0.02)
+    w_loss.backward()
+    y = lp.to(device).requires_grad_(True)
+    d_dev = {k: (v.to(device) if torch.is_tensor(v) else v) for k, v in data.items()}
+    loss, stat = grpo_loss_fn(y, ent.to(device), d_dev, 0.2, None, None, use_decoupled_loss=True)
+    loss.backward()
+    assert float(loss.detach()) == pytest.approx(float(w_loss.detach()), rel=1e-4, abs=1e-7)
+    assert torch.allclose(y.grad.cpu(), x.grad, rtol=1e-4, atol=1e-9)
+    assert float(stat["reduced"]["rkl_loss"]["sum"]) == pytest.approx(float(w_rkl.detach()[mask].sum()), rel=1e-4, abs=1e-6)
+
+
+def test_distillation_terms_shapes_and_empty_mask(device):
+    lp = torch.randn(3, 7, device=device) - 2
+    teacher = lp + 0.1
+    none = torch.zeros(3, 7, dtype=torch.bool, device=device)
+    x = lp.clone().requires_grad_(True)
+    mean, term = areal_amd.distillation_terms(x, lp, teacher, none, pure=True)
+    mean.backward()
+    assert float(mean.detach()) == 0.0 and term.shape == (3, 7) and float(term.abs().max()) == 0.0
+    assert float(x.grad.abs().max()) == 0.0
+    allm = ~none
+    mean, term = areal_amd.distillation_terms(lp, None, teacher, allm, pure=False)
+    assert float(mean) == pytest.approx(-0.1, rel=1e-5) and torch.allclose(term, lp - teacher)
+    with pytest.raises(ValueError, match="same shape"):
+        areal_amd.distillation_terms(lp, None, teacher[:2], allm, pure=False)

@@ -129,3 +129,51 @@ def test_m2po_edge_cases():
     assert S.m2po_mask(old, prox, allm, 2.0).tolist() == [True, True, True, False, False]
     # nothing qualifies: one token (the smallest) survives
     assert S.m2po_mask(old + 5, prox, allm, 0.0).tolist() == [False, False, False, False, True]
+
+
+def test_distillation_loss_against_scalar_definitions():
+    """No test of the reference covers actor.py:482-511, so the restatement is pinned by what the formulas fix:
+    scalar Python loops over the definitions, special cases with a closed form, and central differences for the
+    gradients (with the reward of the pure form held fixed, as `.detach()` there prescribes)."""
+    rng = np.random.default_rng(3)
+    n = 23
+    lp = rng.normal(-1.5, 0.7, n)
+    old = lp + rng.normal(0, 0.2, n)
+    teacher = lp + rng.normal(0, 0.5, n)
+    mask = rng.random(n) < 0.6
+    cnt = max(int(mask.sum()), 1)
+    t = lambda a: torch.tensor(a, dtype=torch.float64)
+    base = torch.tensor(0.37, dtype=torch.float64)
+
+    # joint form: rl_w * loss + kd_w * mean over valid tokens of (logp - teacher)
+    want = 0.8 * 0.37 + 0.01 * sum((lp[i] - teacher[i]) for i in range(n) if mask[i]) / cnt
+    x = t(lp).requires_grad_(True)
+    loss, stat = S.distillation_loss(base, x, t(old), t(teacher), torch.tensor(mask), 0.8, 0.01)
+    assert abs(float(loss.detach()) - want) < 1e-12
+    loss.backward()
+    assert torch.allclose(x.grad, t(np.where(mask, 0.01 / cnt, 0.0)), atol=1e-15)   # constant gradient per valid token
+    assert torch.allclose(stat.detach(), t(np.where(mask, lp - teacher, 0.0)))
+    # student == teacher: the penalty vanishes
+    loss0, _ = S.distillation_loss(base, t(teacher), t(old), t(teacher), torch.tensor(mask), 0.8, 0.01)
+    assert abs(float(loss0) - 0.8 * 0.37) < 1e-15
+
+    # pure form: -kd_w * mean over valid tokens of exp(logp - old) * (teacher - logp), the RL loss dropped
+    def pure(lp_w, lp_r):  # importance weight from lp_w, reward from lp_r
+        return -0.01 * sum(math.exp(lp_w[i] - old[i]) * (teacher[i] - lp_r[i]) for i in range(n) if mask[i]) / cnt
+    x = t(lp).requires_grad_(True)
+    loss, stat = S.distillation_loss(base, x, t(old), t(teacher), torch.tensor(mask), 0, 0.01)
+    assert abs(float(loss.detach()) - pure(lp, lp)) < 1e-12
+    loss.backward()
+    for i in range(n):
+        up, dn = lp.copy(), lp.copy()
+        up[i] += 1e-6
+        dn[i] -= 1e-6
+        fd = (pure(up, lp) - pure(dn, lp)) / 2e-6            # the reward does not move
+        assert abs(float(x.grad[i]) - fd) < 1e-8
+    assert torch.allclose(stat.detach(), t(np.where(mask, -np.exp(lp - old) * (teacher - lp), 0.0)))
+    # on-policy (logp == old): importance weights are 1, the loss is -kd_w * mean(teacher - logp)
+    loss1, _ = S.distillation_loss(base, t(old), t(old), t(teacher), torch.tensor(mask), 0, 0.01)
+    assert abs(float(loss1) + 0.01 * float((teacher - old)[mask].sum()) / cnt) < 1e-12
+    # an all-masked batch divides by 1
+    lossm, _ = S.distillation_loss(base, t(lp), t(old), t(teacher), torch.zeros(n, dtype=torch.bool), 0, 0.01)
+    assert float(lossm) == 0.0
