@@ -649,7 +649,7 @@ def _lmhead_workspace(T: int, H: int, V: int, dev) -> torch.Tensor:
     n = N.load().aa_lmhead_workspace_bytes(T, H, V)
     if n < 0:
         raise N.NativeLibraryError(
-            f"fused lm_head needs hidden size and vocabulary to be multiples of 64 (got H={H}, V={V})"
+            f"the lm_head path needs hidden size and vocabulary to be multiples of 8 (got H={H}, V={V})"
         )
     return torch.empty(n, dtype=torch.uint8, device=dev)
 
