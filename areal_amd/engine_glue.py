@@ -149,6 +149,24 @@ PROX_LOGP_METHOD_LOGLINEAR = "loglinear"
 PROX_LOGP_METHOD_METRICS = "metrics"
 
 
+def infer_token_denominator(input_data: dict[str, Any], fallback: torch.Tensor) -> torch.Tensor:
+    """All-true mask whose size is the number of logical tokens of the micro-batch, for the ``n_tokens``
+    denominator of the logged statistics (areal/trainer/ppo/stats.py:10-40): the shape of ``attention_mask`` if
+    that is a tensor, else ``cu_seqlens[-1]`` tokens, else the shape of ``input_ids`` when it matches ``fallback``,
+    else the shape of ``fallback``."""
+    common = dict(dtype=torch.bool, device=fallback.device)
+    attention_mask = input_data.get("attention_mask")
+    if isinstance(attention_mask, torch.Tensor):
+        return torch.ones_like(attention_mask, **common)
+    cu_seqlens = input_data.get("cu_seqlens")
+    if isinstance(cu_seqlens, torch.Tensor) and cu_seqlens.numel() > 0:
+        return torch.ones(int(cu_seqlens[-1].item()), **common)
+    input_ids = input_data.get("input_ids")
+    if isinstance(input_ids, torch.Tensor) and input_ids.shape == fallback.shape:
+        return torch.ones_like(input_ids, **common)
+    return torch.ones_like(fallback, **common)
+
+
 def resolve_proximal_logp(prox_logp_gt, prox_logp_method: str, old_logp, logprobs, versions, current_version):
     """``_resolve_proximal_logp`` (areal/trainer/ppo/actor.py:687-765): the recomputed proximal log-probs when
     they are there, the log-linear approximation from per-token versions when the forward pass was skipped."""
@@ -267,5 +285,27 @@ def grpo_loss_fn(
         everything = torch.ones_like(loss_mask)
         reduced.update(masked_moments(dict(vocab_min_logits=vocab_min_logits, vocab_max_logits=vocab_max_logits),
                                       everything))
+    reduced["n_tokens"] = infer_token_denominator(input_data, loss_mask).numel()
     stat = dict(stat, loss_mask=loss_mask, reduced=reduced)
     return loss, stat
+
+
+def critic_loss_fn(value: torch.Tensor, input_data: dict[str, Any], eps_clip: float) -> tuple[torch.Tensor, dict]:
+    """The critic's loss function for one micro-batch (areal/trainer/ppo/critic.py:105-149) on the GPU ops.
+
+    Returns ``(loss, stat)`` with ``stat["reduced"]`` holding what the reference logs tensor by tensor (sums,
+    averages, extrema under ``n_valid_tokens`` and ``clipped_tokens``) and ``n_tokens``."""
+    from .advantages import masked_moments
+    from .functional import ppo_critic_loss_fn
+
+    value = value.squeeze(-1).float()
+    old_value = input_data["values"].float()
+    target_value = input_data["returns"].float()
+    loss_mask = input_data["loss_mask"].bool()
+    loss, stat = ppo_critic_loss_fn(value, old_value, target_value, eps_clip, loss_mask)
+    clip_mask = stat["clip_mask"]
+    reduced = masked_moments(dict(new_value=value.detach(), old_value=old_value, target_value=target_value,
+                                  critic_loss=stat["loss"], clip_ratio=clip_mask.float()), loss_mask)
+    reduced.update(masked_moments(dict(clipped_new_value=value.detach(), clipped_old_value=old_value), clip_mask))
+    reduced["n_tokens"] = infer_token_denominator(input_data, value).numel()
+    return loss, dict(stat, loss_mask=loss_mask, reduced=reduced)

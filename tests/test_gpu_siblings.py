@@ -242,3 +242,36 @@ def test_distillation_terms_shapes_and_empty_mask(device):
     assert float(mean) == pytest.approx(-0.1, rel=1e-5) and torch.allclose(term, lp - teacher)
     with pytest.raises(ValueError, match="same shape"):
         areal_amd.distillation_terms(lp, None, teacher[:2], allm, pure=False)
+
+
+def test_loss_adapters_count_logical_tokens(device):
+    """tests/test_ppo_stats.py:54-111: with cu_seqlens = [0, 4] and two local tokens, n_tokens is 4 for the actor's
+    and the critic's loss function; the critic adapter against the oracle's value loss."""
+    from areal_amd.engine_glue import critic_loss_fn, grpo_loss_fn
+
+    cu = torch.tensor([0, 4], dtype=torch.int32, device=device)
+    z2 = torch.zeros(2, device=device)
+    data = dict(input_ids=torch.tensor([11, 12], device=device), cu_seqlens=cu, logprobs=z2, advantages=z2 + 1,
+                loss_mask=torch.ones(2, dtype=torch.bool, device=device), prox_logp=z2,
+                versions=torch.zeros(2, dtype=torch.int32, device=device))
+    _, stat = grpo_loss_fn(z2.clone().requires_grad_(True), z2, data, 0.2, None, None)
+    assert stat["reduced"]["n_tokens"] == 4
+    g = torch.Generator().manual_seed(2)
+    n = 300
+    value, old, target = (torch.randn(n, generator=g) for _ in range(3))
+    mask = torch.rand(n, generator=g) < 0.7
+    cdata = dict(input_ids=torch.zeros(n, dtype=torch.long, device=device), values=old.to(device),
+                 returns=target.to(device), loss_mask=mask.to(device),
+                 cu_seqlens=torch.tensor([0, 2 * n], dtype=torch.int32, device=device))
+    v = value.to(device).unsqueeze(-1).requires_grad_(True)
+    loss, cstat = critic_loss_fn(v, cdata, 0.3)
+    loss.backward()
+    x = value.clone().requires_grad_(True)
+    w_loss, w_stat = S.critic_loss(x, old, target, 0.3, mask)
+    w_loss.backward()
+    assert float(loss.detach()) == pytest.approx(float(w_loss.detach()), rel=1e-5)
+    assert torch.allclose(v.grad.squeeze(-1).cpu(), x.grad, rtol=1e-4, atol=1e-9)
+    red = cstat["reduced"]
+    assert red["n_tokens"] == 2 * n and float(red["new_value"]["count"]) == float(mask.sum())
+    assert float(red["clipped_new_value"]["count"]) == float(w_stat["clip_mask"].sum())
+    assert float(red["critic_loss"]["sum"]) == pytest.approx(float(w_stat["loss"][mask].sum()), rel=1e-4)

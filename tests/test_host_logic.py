@@ -97,3 +97,21 @@ def test_synthetic_hidden_state_configurations():
     best = (c4.hidden.float() @ c4.weight.float().t()).argmax(-1)
     frac = float((best == c4.labels).float().mean())
     assert 0.12 < frac < 0.30  # 20 % argmax labels (+ chance hits)
+
+
+def test_infer_token_denominator_cases_of_the_reference():
+    """The four cases of tests/test_ppo_stats.py:11-51, inputs and expected shapes transcribed."""
+    from areal_amd.engine_glue import infer_token_denominator
+
+    cases = [
+        (dict(attention_mask=torch.tensor([[1, 1, 0], [1, 1, 1]]), input_ids=torch.tensor([[11, 12], [13, 14]])),
+         torch.zeros(5), (2, 3)),                                               # attention_mask wins
+        (dict(input_ids=torch.tensor([[11, 12, 13], [14, 15, 16]])), torch.zeros(2, 3), (2, 3)),   # input_ids
+        (dict(input_ids=torch.tensor([11, 12, 13, 0])), torch.zeros(3), (3,)),  # padded tree input_ids: fallback
+        (dict(logprobs=torch.zeros(2)), torch.zeros(4), (4,)),                  # no metadata: fallback
+        (dict(input_ids=torch.tensor([11, 12]), cu_seqlens=torch.tensor([0, 4], dtype=torch.int32)), torch.zeros(2),
+         (4,)),                                                                 # tests/test_ppo_stats.py:54-87
+    ]
+    for data, fallback, shape in cases:
+        n_tokens = infer_token_denominator(data, fallback)
+        assert tuple(n_tokens.shape) == shape and n_tokens.dtype == torch.bool and bool(n_tokens.all())
