@@ -13,6 +13,7 @@
 // so that  logp = ln2 (t_label - log2 s)  and  entropy = ln2 (log2 s - u / s)
 // are differences of small numbers whatever the magnitude of the logits.
 #include "device_utils.h"
+#include "logits_path.h"
 #include "ppo_math.h"
 
 namespace aa {
@@ -298,6 +299,9 @@ struct FusedTokenArgs {
   uint8_t* flags;
   aa_ppo_params P;
   int64_t T_active;
+  // Optional row map of the gradient: row t is written to dlogits row out_rows[t]; a negative entry means the row
+  // is not written at all (its token has no gradient).  Null: row t goes to row t.
+  const int32_t* out_rows;
 };
 
 // Per-token inputs of the loss, fetched ahead of the row statistics so that
@@ -392,8 +396,9 @@ __global__ __launch_bounds__(NT) void k_fused_generic(const void* __restrict__ l
                                                       FusedTokenArgs a, void* __restrict__ dlogits) {
   __shared__ float smem[(NT / kWave) * 5];
   const int64_t t = blockIdx.x;
+  const int64_t orow = a.out_rows ? (int64_t)a.out_rows[t] : t;
   const void* row = row_ptr(logits, t, stride, Elem<DT>::kBytes);
-  void* out = (void*)row_ptr(dlogits, t, stride, Elem<DT>::kBytes);
+  void* out = (void*)row_ptr(dlogits, orow < 0 ? 0 : orow, stride, Elem<DT>::kBytes);
   const float c = kLog2e * inv_t;
   const int64_t y = labels[t];
   const bool y_ok = (y >= 0) && (y < V);
@@ -406,6 +411,7 @@ __global__ __launch_bounds__(NT) void k_fused_generic(const void* __restrict__ l
   const RowOut ro = finish_row(rs);
   const float lp = y_ok ? label_logp(xy, c, rs, ro) : __builtin_nanf("");
   const float g = fused_token_tail(a, t, tin, fn, gscale, lp, rs, ro, threadIdx.x == 0);
+  if (orow < 0) return;  // uniform over the workgroup
   if (g == 0.f) {
     row_zero_generic<DT, NT>(row, out, V, vec_ok != 0);
     return;
@@ -609,6 +615,7 @@ __global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ l
   bool y_ok = (y >= 0) && (y < V);
   uint32_t xy_raw = load_u16_uniform(src, y_ok ? y : 0);
   TokenIn tin = load_token_in_ro(in_prox, in_adv, in_mask32, mask_mis, in_bw, has_w, a.T_active, t);
+  int64_t orow = a.out_rows ? (int64_t)a.out_rows[t] : t;  // where the gradient of this row goes; < 0: nowhere
 
   for (;;) {
     // claim the row after this one; the answer is picked up behind the barriers of block_stats
@@ -716,9 +723,11 @@ __global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ l
     const bool y_ok_n = (y_n >= 0) && (y_n < V);
     const uint32_t xy_raw_n = load_u16_uniform(src_n, y_ok_n ? y_n : 0);
     const TokenIn tin_n = load_token_in_ro(in_prox, in_adv, in_mask32, mask_mis, in_bw, has_w, a.T_active, more ? tn : t);
+    const int64_t orow_n = a.out_rows ? (int64_t)a.out_rows[more ? tn : t] : tn;
 
-    const __amdgpu_buffer_rsrc_t wsrc =
-        __builtin_amdgcn_make_buffer_rsrc((void*)(dlogits + t * stride_vec), 0, V * 2, kBufferFlags);
+    // a row that is not to be written gets an empty descriptor: the hardware drops every store
+    const __amdgpu_buffer_rsrc_t wsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(dlogits + (orow < 0 ? 0 : orow) * stride_vec), 0, orow < 0 ? 0 : V * 2, kBufferFlags);
     if constexpr (EXT) {
       if (g != 0.f) {
 #pragma unroll
@@ -769,7 +778,7 @@ __global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ l
         load_lds_chunks(rsrc_n);
       }
     }
-    t = tn; y = y_n; y_ok = y_ok_n; xy_raw = xy_raw_n; tin = tin_n;
+    t = tn; y = y_n; y_ok = y_ok_n; xy_raw = xy_raw_n; tin = tin_n; orow = orow_n;
   }
   if (work && tid == 0) {
     __threadfence();
@@ -928,6 +937,17 @@ extern "C" int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int
                                    const float* grad_scale, float* logp, float* entropy, float* vmax, float* vmin,
                                    float* stat_loss, float* ratio, uint8_t* flags, void* dlogits, int32_t* work,
                                    void* stream) {
+  return aa::logits_ppo_fused_rows(logits, dtype, T, V, row_stride, labels, inv_temperature, T_active, prox_logp, adv,
+                                   mask_eff, behave_w, params, n_valid, grad_scale, logp, entropy, vmax, vmin, stat_loss,
+                                   ratio, flags, dlogits, nullptr, work, stream);
+}
+
+int aa::logits_ppo_fused_rows(const void* logits, int dtype, int64_t T, int64_t V, int64_t row_stride,
+                              const int64_t* labels, float inv_temperature, int64_t T_active, const float* prox_logp,
+                              const float* adv, const uint8_t* mask_eff, const float* behave_w,
+                              const aa_ppo_params* params, const int32_t* n_valid, const float* grad_scale, float* logp,
+                              float* entropy, float* vmax, float* vmin, float* stat_loss, float* ratio, uint8_t* flags,
+                              void* dlogits, const int32_t* out_rows, int32_t* work, void* stream) {
   if (!common_args_ok(logits, dtype, T, V, row_stride, labels)) return AA_ERR_INVALID_ARGUMENT;
   if (!params || !n_valid || !logp || !dlogits) return AA_ERR_INVALID_ARGUMENT;
   if (T_active < 0 || T_active > T || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
@@ -941,6 +961,7 @@ extern "C" int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int
   a.logp = logp; a.entropy = entropy; a.vmax = vmax; a.vmin = vmin;
   a.stat_loss = stat_loss; a.ratio = ratio; a.flags = flags;
   a.P = *params; a.T_active = T_active;
+  a.out_rows = out_rows;
 
   const bool fast = (dtype != AA_F32) && (V % 8 == 0) && (row_stride % 8 == 0) && (((uintptr_t)logits & 15) == 0) &&
                     (((uintptr_t)dlogits & 15) == 0) && (V >= 8 * 1024) && (V <= kMaxExtChunks * 8192) && (T_active > 0);

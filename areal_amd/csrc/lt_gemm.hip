@@ -1,9 +1,15 @@
-// hipBLASLt front end for the plain GEMMs of the lm_head path: one handle per device, the heuristic's first
-// algorithm per problem shape, cached.
+// hipBLASLt front end for the plain GEMMs of the lm_head path: one handle per device, one algorithm per problem
+// shape, cached.  The library's heuristic ranks its kernels without running them, and its first choice is up to
+// 30 % slower than its second for some row counts (e.g. m = 4096, k = 151936: n = 11520 runs at 1 258 TFLOP/s with
+// the first and 1 560 with the second, n = 12288 the other way round).  So the first time a shape is seen with
+// beta == 0 (the output is overwritten, a trial run does no harm) the leading candidates are timed on the caller's
+// stream with the caller's operands and the fastest is kept.  That blocks the host for a few GEMM durations, once
+// per shape; AREAL_AMD_GEMM_TUNE=0 turns it off, and a capturing stream is never timed.
 #include "lt_gemm.h"
 
 #include <hipblaslt/hipblaslt.h>
 
+#include <cstdlib>
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -18,6 +24,21 @@ hipblasLtHandle_t g_handle[kMaxDevices] = {};
 
 using Key = std::tuple<int, bool, bool, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, bool, bool>;
 std::map<Key, hipblasLtMatmulAlgo_t> g_algos;
+
+constexpr int kCandidates = 4;
+
+bool tuning_enabled() {
+  static const bool on = [] {
+    const char* v = std::getenv("AREAL_AMD_GEMM_TUNE");
+    return !(v && v[0] == '0');
+  }();
+  return on;
+}
+
+bool stream_is_capturing(hipStream_t st) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  return hipStreamIsCapturing(st, &status) != hipSuccess || status != hipStreamCaptureStatusNone;
+}
 
 struct Problem {
   hipblasLtMatmulDesc_t desc = nullptr;
@@ -60,13 +81,38 @@ bool gemm(hipStream_t st, bool transA, bool transB, int64_t m, int64_t n, int64_
     if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return false;
     const uint64_t max_ws = workspace ? (uint64_t)workspace_bytes : 0;
     hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &max_ws, sizeof(max_ws));
-    hipblasLtMatmulHeuristicResult_t result[1];
+    hipblasLtMatmulHeuristicResult_t result[kCandidates];
     int found = 0;
-    const hipblasStatus_t hs =
-        hipblasLtMatmulAlgoGetHeuristic(handle, p.desc, p.a, p.b, p.d, p.d, pref, 1, result, &found);
+    const bool tune = beta == 0.f && tuning_enabled() && !stream_is_capturing(st);
+    const hipblasStatus_t hs = hipblasLtMatmulAlgoGetHeuristic(handle, p.desc, p.a, p.b, p.d, p.d, pref,
+                                                               tune ? kCandidates : 1, result, &found);
     hipblasLtMatmulPreferenceDestroy(pref);
     if (hs != HIPBLAS_STATUS_SUCCESS || found < 1) return false;
-    it = g_algos.emplace(key, result[0].algo).first;
+    int best = 0;
+    if (tune && found > 1) {
+      hipEvent_t e0 = nullptr, e1 = nullptr;
+      if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
+        const float one = 1.f, zero = 0.f;
+        float best_ms = -1.f;
+        for (int c = 0; c < found; ++c) {
+          auto run = [&] {
+            return hipblasLtMatmul(handle, p.desc, &one, A, p.a, B, p.b, &zero, D, p.d, D, p.d, &result[c].algo, workspace,
+                                   workspace ? (size_t)workspace_bytes : 0, st) == HIPBLAS_STATUS_SUCCESS;
+          };
+          float ms = 0.f;
+          if (!run() || hipEventRecord(e0, st) != hipSuccess || !run() || hipEventRecord(e1, st) != hipSuccess ||
+              hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(&ms, e0, e1) != hipSuccess)
+            continue;
+          if (best_ms < 0.f || ms < best_ms) {
+            best_ms = ms;
+            best = c;
+          }
+        }
+      }
+      if (e0) hipEventDestroy(e0);
+      if (e1) hipEventDestroy(e1);
+    }
+    it = g_algos.emplace(key, result[best].algo).first;
   }
   const float alpha = 1.f;
   return hipblasLtMatmul(handle, p.desc, &alpha, A, p.a, B, p.b, &beta, D, p.d, D, p.d, &it->second, workspace,

@@ -729,8 +729,9 @@ def lm_head_logprobs_entropy(
 class _FusedLmHeadPpo(torch.autograd.Function):
     @staticmethod
     def forward(ctx, hidden, weight, labels, temperature, T_active, prox, adv, mask_eff, behave_w, params, n_valid,
-                grad_scale):
+                grad_scale, kept_per_chunk):
         lib = N.load()
+        kept = None if kept_per_chunk is None else (C.c_int64 * len(kept_per_chunk))(*kept_per_chunk)
         T, H = hidden.shape
         V = weight.shape[0]
         dev = hidden.device
@@ -749,7 +750,7 @@ class _FusedLmHeadPpo(torch.autograd.Function):
             N.check(
                 lib.aa_lmhead_ppo_fused(
                     _ptr(hidden), _ptr(weight), T, H, V, _ptr(labels), 1.0 / float(temperature), T_active, _ptr(prox),
-                    _ptr(adv), _ptr(mask_eff), _ptr(behave_w), C.byref(params), _ptr(n_valid), _ptr(grad_scale),
+                    _ptr(adv), _ptr(mask_eff), _ptr(behave_w), C.byref(params), _ptr(n_valid), _ptr(grad_scale), kept,
                     _ptr(logp), _ptr(entropy), _ptr(stat_loss), _ptr(ratio), _ptr(flags), _ptr(d_hidden),
                     _ptr(d_weight), _DTYPES[d_weight.dtype], _ptr(_work_words(dev)), _ptr(ws), ws.numel(), st,
                 ),
@@ -775,7 +776,7 @@ class _FusedLmHeadPpo(torch.autograd.Function):
             for t in (d_hidden, d_weight):
                 N.check(lib.aa_scale_inplace(_ptr(t), _DTYPES[t.dtype], t.numel(), _ptr(g), _stream(dev)),
                         "aa_scale_inplace")
-        return (d_hidden, d_weight) + (None,) * 10
+        return (d_hidden, d_weight) + (None,) * 11
 
 
 def fused_lm_head_ppo_loss(
@@ -794,6 +795,7 @@ def fused_lm_head_ppo_loss(
     cu_seqlens: torch.Tensor | None = None,
     temperature: float = 1.0,
     loss_scale: torch.Tensor | float | None = None,
+    skip_masked_tokens: bool = True,
 ) -> tuple[torch.Tensor, dict]:
     """lm_head + ``gather_logprobs_entropy`` + ``ppo_actor_loss_fn`` (+ backward) for one micro-batch.
 
@@ -803,6 +805,12 @@ def fused_lm_head_ppo_loss(
     output is, and turned in place into their gradient, so the full ``[T, V]`` logits never exist and nothing is
     recomputed.  ``loss.backward()`` hands back ``d(hidden)`` and ``d(weight)`` written during the forward pass.
     With ``importance_sampling_level="sequence"`` the call runs ``lm_head_logprobs_entropy`` and the unfused loss.
+
+    ``skip_masked_tokens``: a token whose (effective) loss mask is zero has a zero gradient row, so the two gradient
+    GEMMs run on the other tokens only; the results are those of the dense computation.  The per-chunk token counts
+    size the GEMMs, so the host reads them (one small device-to-host copy that waits for the mask only) before it
+    queues the chunk.  ``False`` multiplies the zero rows through, as the reference's autograd does, without that
+    read.
     """
     if importance_sampling_level not in ("token", "sequence"):
         raise ValueError(
@@ -856,9 +864,17 @@ def fused_lm_head_ppo_loss(
         n_valid = counts
     else:
         n_valid = _count_nonzero(m8)
+    kept = None
+    if skip_masked_tokens:
+        chunk = int(N.load().aa_lmhead_chunk_tokens())
+        n_chunks = (hidden.shape[0] + chunk - 1) // chunk
+        on = mask_eff.ne(0)
+        if n_chunks * chunk != T_active:
+            on = torch.nn.functional.pad(on, (0, n_chunks * chunk - T_active))
+        kept = _HostCounts(on.view(n_chunks, chunk).sum(1)).tolist()
     loss, logp, entropy, stat_loss, ratio, flags = _FusedLmHeadPpo.apply(
         hidden.contiguous(), weight.contiguous(), y, float(temperature), T_active, prox, adv, mask_eff, w, params,
-        n_valid, scale_t,
+        n_valid, scale_t, kept,
     )
     logp_a = logp[:T_active]
     stat = dict(

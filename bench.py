@@ -66,6 +66,9 @@ def parse_args():
     ap.add_argument("--rs-action", choices=["mask", "clamp"], default=None,
                     help="override the action of the workload's importance-weight cap (cfg1 is quoted with 'mask', "
                          "the documented equivalent of behave_imp_weight_cap; 'clamp' keeps every token)")
+    ap.add_argument("--dense-backward", action="store_true",
+                    help="lm_head workloads: run masked tokens through the gradient GEMMs too (as the reference's "
+                         "autograd does) instead of leaving their zero rows out")
     ap.add_argument("--copy-launches", type=int, default=0,
                     help="also launch the plain copy kernel this many times over the logits buffer "
                          "(the calibration point for FETCH_SIZE / WRITE_SIZE counters)")
@@ -308,6 +311,9 @@ def build_fused_case(name: str, seed: int, device):
     return case, desc
 
 
+DENSE_BACKWARD = False  # set from --dense-backward
+
+
 def run_fused_steps(case, n, kw, cfg):
     import areal_amd
 
@@ -318,14 +324,16 @@ def run_fused_steps(case, n, kw, cfg):
         w.grad = None
         loss, _ = areal_amd.fused_lm_head_ppo_loss(
             h, w, case.labels, case.prox_logp, case.old_logp, case.advantages, loss_mask=case.loss_mask,
-            rejection_sampling=cfg, cu_seqlens=case.cu_seqlens, temperature=case.temperature, **kw,
+            rejection_sampling=cfg, cu_seqlens=case.cu_seqlens, temperature=case.temperature,
+            skip_masked_tokens=not DENSE_BACKWARD, **kw,
         )
         loss.backward()
     return loss
 
 
-def time_lmhead_step(case, kw, cfg, iters: int):
-    """Duration of aa_lmhead_ppo_fused (every kernel it enqueues), HIP events on the launch stream."""
+def time_lmhead_step(case, kw, cfg, iters: int, skip_masked: bool):
+    """Duration of aa_lmhead_ppo_fused (every kernel it enqueues), HIP events on the launch stream, and the number
+    of tokens that go through the gradient GEMMs."""
     import torch
 
     from areal_amd import _native as N
@@ -351,19 +359,24 @@ def time_lmhead_step(case, kw, cfg, iters: int):
     dw = torch.empty_like(case.weight)  # bf16, as the Python wrapper asks for
     ws = F._lmhead_workspace(T, H, V, dev)
     stream = torch.cuda.current_stream(dev)
+    kept, kept_tokens = None, T
+    if skip_masked:  # per-chunk counts of tokens with a mask, read once here (the Python wrapper reads them per step)
+        chunk = int(lib.aa_lmhead_chunk_tokens())
+        per_chunk = [int(mask_eff[i:i + chunk].ne(0).sum()) for i in range(0, T, chunk)]
+        kept, kept_tokens = (C.c_int64 * len(per_chunk))(*per_chunk), sum(per_chunk)
 
     def launch():
         N.check(
             lib.aa_lmhead_ppo_fused(
                 F._ptr(case.hidden), F._ptr(case.weight), T, H, V, F._ptr(case.labels), 1.0 / case.temperature, T,
-                F._ptr(prox), F._ptr(adv), F._ptr(mask_eff), F._ptr(w), C.byref(params), F._ptr(counts), None,
+                F._ptr(prox), F._ptr(adv), F._ptr(mask_eff), F._ptr(w), C.byref(params), F._ptr(counts), None, kept,
                 F._ptr(logp), F._ptr(ent), F._ptr(sl), F._ptr(ratio), F._ptr(flags), F._ptr(dh), F._ptr(dw),
                 N.AA_BF16, F._ptr(F._work_words(dev)), F._ptr(ws), ws.numel(), C.c_void_p(stream.cuda_stream),
             ),
             "aa_lmhead_ppo_fused",
         )
 
-    return time_events(launch, iters, stream)
+    return time_events(launch, iters, stream) + (kept_tokens,)
 
 
 def time_lmhead_op(case, iters: int):
@@ -484,14 +497,19 @@ def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: i
     case.hidden.requires_grad_(False)
     case.weight.requires_grad_(False)
 
-    k_ms, k_min_ms = time_lmhead_step(case, kw, cfg, max(min(steps, 10), 3))
+    k_ms, k_min_ms, kept_tokens = time_lmhead_step(case, kw, cfg, max(min(steps, 10), 3), not args.dense_backward)
     f_ms, b_ms = time_lmhead_op(case, 3)
-    alg_flops = 6.0 * T * V * H
+    # Flops the step needs: logits of every token (2 T V H) and the two gradient GEMMs over the tokens that have a
+    # gradient (4 T_kept V H).  The reference's autograd runs them over all T tokens: 6 T V H.
+    dense_flops = 6.0 * T * V * H
+    alg_flops = 2.0 * T * V * H + 4.0 * kept_tokens * V * H
     achieved = alg_flops / (k_ms * 1e-3) / 1e12
     roofline = dict(
-        bound="mfma", kernel="aa_lmhead_ppo_fused (per token chunk: hipBLASLt logits GEMM, k_fused_regs in place, k_transpose_bf16 copies, hipBLASLt d_hidden and d_weight GEMMs)",
+        bound="mfma", kernel="aa_lmhead_ppo_fused (per token chunk: hipBLASLt logits GEMM, k_fused_regs, k_transpose_bf16 copies, hipBLASLt d_hidden and d_weight GEMMs over the tokens with a gradient)",
         achieved=achieved, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s", frac=achieved / MFMA_BF16_PEAK_TFLOPS,
         traffic=None, avg_call_ms=k_ms, min_call_ms=k_min_ms, algorithmic_flops_per_step=alg_flops,
+        tokens_with_gradient=kept_tokens, dense_flops_per_step=dense_flops,
+        dense_equivalent_tflops=dense_flops / (k_ms * 1e-3) / 1e12,
         # the stand-alone differentiable op lm_head_logprobs_entropy, whose backward forms the logits again
         standalone_op=dict(fwd_ms=f_ms, bwd_ms=b_ms, fwd_tflops=2.0 * T * V * H / (f_ms * 1e-3) / 1e12,
                            bwd_tflops=4.0 * T * V * H / (b_ms * 1e-3) / 1e12),
@@ -686,9 +704,10 @@ def synth_lengths(total, seed):
 
 
 def main():
-    global RS_ACTION
+    global RS_ACTION, DENSE_BACKWARD
     args = parse_args()
     RS_ACTION = args.rs_action
+    DENSE_BACKWARD = args.dense_backward
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU; run it with --gpus 1 (no multi-GPU path exists)", file=sys.stderr)
         sys.exit(2)

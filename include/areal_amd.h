@@ -6,6 +6,11 @@
  * the HIP stream it is given (hipStream_t passed as void*; NULL = the default
  * stream), allocates nothing, and never synchronises the device.  The return
  * value is an aa_status; a non-zero value means nothing was enqueued.
+ * One exception, for the aa_lmhead_* entry points only: the first time they
+ * meet a GEMM shape they time a few candidate algorithms of the GEMM library
+ * on the given stream (the host waits for those runs; the GEMM library keeps a
+ * handle and its kernels per device).  AREAL_AMD_GEMM_TUNE=0 in the environment
+ * turns the timing off; a stream that is being captured is never timed.
  *
  * Layout conventions (the reference's "packed 1-D" layout):
  *   logits      [T, V]  row-major, element (t, j) at logits[t * row_stride + j]
@@ -382,6 +387,9 @@ int aa_masked_moments(const float* const* values, int n_tensors,
  * d_weight) when T > 16384. */
 int64_t aa_lmhead_workspace_bytes(int64_t T, int64_t H, int64_t V);
 
+/* Tokens per chunk of the lm_head entry points (16384). */
+int64_t aa_lmhead_chunk_tokens(void);
+
 /*
  * logp / entropy of softmax(hidden @ weight.T / temperature), holding at most
  * one chunk of 16384 tokens of logits (bf16, as the reference's lm_head output
@@ -427,6 +435,15 @@ int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, int64_t H,
  * aa_logits_ppo_fused.  d_hidden [T, H] bf16 and d_weight [V, H] (AA_F32 or
  * AA_BF16, fp32 accumulation either way, as in aa_lmhead_bwd) are
  * overwritten.  workspace: aa_lmhead_workspace_bytes(T, H, V) bytes.
+ *
+ * kept_per_chunk (HOST memory, nullable): a token whose mask_eff is zero has
+ * a zero gradient row, so it adds nothing to d_weight and its d_hidden row is
+ * zero.  Given, for every chunk of aa_lmhead_chunk_tokens() tokens, the number
+ * of non-zero mask_eff bytes among the chunk's first min(T_active - t0, chunk)
+ * tokens, the two gradient GEMMs of the chunk run on those tokens only (the
+ * reference's autograd multiplies the zero rows through).  The counts size the
+ * GEMMs, which is why they come from the host; tokens beyond a count that is
+ * too small are treated as masked.  NULL: every row goes through the GEMMs.
  */
 int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64_t T,
                         int64_t H, int64_t V, const int64_t* labels,
@@ -434,7 +451,8 @@ int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64_t T,
                         const float* prox_logp, const float* adv,
                         const uint8_t* mask_eff, const float* behave_w,
                         const aa_ppo_params* params, const int32_t* n_valid,
-                        const float* grad_scale, float* logp, float* entropy,
+                        const float* grad_scale, const int64_t* kept_per_chunk,
+                        float* logp, float* entropy,
                         float* stat_loss, float* ratio, uint8_t* flags,
                         void* d_hidden, void* d_weight, int d_weight_dtype,
                         int32_t* work, void* workspace, int64_t workspace_bytes,

@@ -211,7 +211,7 @@ def test_engine_contract_roll_pad_and_scale(device):
     x = logits.to(device).requires_grad_(True)
     loss, _ = engine_glue.compute_logprobs_and_loss(x, {"input_ids": input_ids.to(device)}, mb_d, pad, total_w, 0.2)
     loss.backward()
-    assert float(loss) == 0.0 and float(x.grad.float().abs().max()) == 0.0
+    assert float(loss.detach()) == 0.0 and float(x.grad.float().abs().max()) == 0.0
 
 
 def test_full_size_properties_config1(device):

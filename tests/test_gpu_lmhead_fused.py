@@ -169,3 +169,56 @@ def test_padding_only_chunk_and_no_active_token(device):
     loss, _ = areal_amd.fused_logprobs_ppo_loss(x, labels[:30] % 9000, e, e, e, 0.2, none)
     loss.backward()
     assert float(loss.detach()) == 0.0 and float(x.grad.float().abs().sum()) == 0.0
+
+
+@pytest.mark.parametrize("pattern", ["random", "second_chunk_masked", "first_chunk_masked", "all_masked", "one_token"])
+def test_skipping_masked_tokens_equals_the_dense_backward(device, pattern):
+    """Tokens with a zero mask are left out of the gradient GEMMs: same loss and statistics, same gradients as when
+    their zero rows are multiplied through (two token chunks, batch padding at the end)."""
+    g = torch.Generator().manual_seed(5)
+    T_pad, T, H, V = 16384 + 300, 16384 + 200, 64, 8200       # the register-resident row kernel writes the closed-up rows
+    hidden = torch.randn(T_pad, H, generator=g).bfloat16().to(device)
+    weight = (0.3 * torch.randn(V, H, generator=g)).bfloat16().to(device)
+    labels = torch.randint(0, V, (T_pad,), generator=g).to(device)
+    with torch.no_grad():
+        ref, _ = areal_amd.lm_head_logprobs_entropy(hidden, weight, labels)
+    ref = ref[:T]
+    prox = ref + 0.05 * torch.randn(T, generator=g).to(device)
+    old = ref + 0.2 * torch.randn(T, generator=g).to(device)
+    adv = torch.randn(T, generator=g).to(device)
+    mask = (torch.rand(T, generator=g) < 0.5).to(device)
+    if pattern == "second_chunk_masked":
+        mask[16384:] = False
+    elif pattern == "first_chunk_masked":
+        mask[:16384] = False
+    elif pattern == "all_masked":
+        mask[:] = False
+    elif pattern == "one_token":
+        mask[:] = False
+        mask[16384 + 7] = True
+    rs = RejectionSamplingConfig(level="token", action="mask", metric="ratio", upper=1.3)
+
+    def run(skip):
+        h = hidden.clone().requires_grad_(True)
+        w = weight.clone().requires_grad_(True)
+        loss, stat = areal_amd.fused_lm_head_ppo_loss(h, w, labels, prox, old, adv, 0.2, mask, eps_clip_higher=0.28,
+                                                      c_clip=3.0, rejection_sampling=rs, skip_masked_tokens=skip)
+        loss.backward()
+        return loss.detach(), stat, h.grad.float(), w.grad.float()
+
+    l1, s1, dh1, dw1 = run(True)
+    l0, s0, dh0, dw0 = run(False)
+    assert torch.equal(l1, l0)
+    for k in ("logprobs", "entropy", "loss", "importance_weight", "clip_mask", "dual_clip_mask", "behave_mask"):
+        assert torch.equal(s1[k], s0[k]), k
+    rows_off = torch.ones(T_pad, dtype=torch.bool, device=device)
+    rows_off[:T] = ~s1["behave_mask"]
+    assert float(dh1[rows_off].abs().max()) == 0.0
+    if pattern == "all_masked":
+        assert float(dh1.abs().max()) == 0.0 and float(dw1.abs().max()) == 0.0 and float(dw0.abs().max()) == 0.0
+        return
+    # different GEMM shapes may sum in a different order: equal up to the bf16 rounding of the outputs
+    for a, b in ((dh1, dh0), (dw1, dw0)):
+        scale = float(b.abs().max())
+        assert float((a - b).abs().max()) <= scale * 2.0 ** -7
+        assert cosine(a.cpu(), b.cpu()) > 0.99999
