@@ -270,11 +270,13 @@ extern "C" int aa_lmhead_fwd(const void* hidden, const void* weight, int64_t T, 
 
 extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, int64_t H, int64_t V,
                              const int64_t* labels, float inv_temperature, const float* row_lse, const float* row_ez,
-                             const float* g_logp, const float* g_entropy, void* d_hidden, void* d_weight,
-                             int d_weight_dtype, void* workspace, int64_t workspace_bytes, void* stream) {
+                             const float* g_logp, const float* g_entropy, const uint8_t* row_has_gradient,
+                             const int64_t* kept_per_chunk, void* d_hidden, void* d_weight, int d_weight_dtype,
+                             void* workspace, int64_t workspace_bytes, void* stream) {
   if (!hidden || !weight || !labels || !row_lse || !g_logp || !d_hidden || !d_weight || !workspace)
     return AA_ERR_INVALID_ARGUMENT;
   if ((g_entropy && !row_ez) || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
+  if ((kept_per_chunk != nullptr) != (row_has_gradient != nullptr)) return AA_ERR_INVALID_ARGUMENT;
   if (!shapes_ok(T, H, V) || (d_weight_dtype != AA_F32 && d_weight_dtype != AA_BF16)) return AA_ERR_UNSUPPORTED;
   if ((((uintptr_t)hidden | (uintptr_t)weight | (uintptr_t)workspace | (uintptr_t)d_hidden | (uintptr_t)d_weight) & 15))
     return AA_ERR_INVALID_ARGUMENT;
@@ -282,21 +284,53 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
   if (workspace_bytes < w.bytes) return AA_ERR_INVALID_ARGUMENT;
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
-  void* ds = ws + w.off_ds;  // [chunk, V]: logits of the chunk, then their gradient in place
   launch_transpose(st, (const uint16_t*)weight, V, H, H, (uint16_t*)(ws + w.off_wt), V);
   const WeightGrad dw = weight_grad(w, ws, d_weight, d_weight_dtype, T);
-  for (int64_t t0 = 0; t0 < T; t0 += w.chunk) {
+  int32_t* out_rows = (int32_t*)(ws + w.off_rows);
+  int32_t* act_rows = out_rows + w.chunk;
+  bool first = true;  // no GEMM has written d_weight yet
+  int64_t chunk_index = 0;
+  for (int64_t t0 = 0; t0 < T; t0 += w.chunk, ++chunk_index) {
     const int64_t n_tok = (T - t0) < w.chunk ? (T - t0) : w.chunk;
     const uint16_t* hid = (const uint16_t*)hidden + t0 * H;
+    uint16_t* dh = (uint16_t*)d_hidden + t0 * H;
+    const float* ez = row_ez ? row_ez + t0 : nullptr;
+    const float* gh = g_entropy ? g_entropy + t0 : nullptr;
+    if (!kept_per_chunk) {
+      void* ds = ws + w.off_ds;  // [chunk, V]: logits of the chunk, then their gradient in place
+      if (!panel_logits(st, w, ws, hid, weight, n_tok, H, V)) return AA_ERR_LAUNCH;
+      const int rc = aa_logits_bwd(ds, AA_BF16, n_tok, V, V, labels + t0, inv_temperature, row_lse + t0, ez, g_logp + t0,
+                                   gh, n_tok, ds, stream);
+      if (rc != AA_OK) return rc;
+      if (!panel_gradients(st, w, ws, w.off_ds, w.off_dst, hid, nullptr, n_tok, round_up(n_tok, 8), n_tok, H, V, dh,
+                           dw.acc, dw.acc_f32, first))
+        return AA_ERR_LAUNCH;
+      first = false;
+      continue;
+    }
+    // rows whose upstream gradients are all zero are left out, as in aa_lmhead_ppo_fused
+    int64_t kept = kept_per_chunk[chunk_index];
+    kept = kept < 0 ? 0 : (kept > n_tok ? n_tok : kept);
+    if (kept == 0) {
+      launch_zero(st, dh, n_tok * H * 2);
+      continue;
+    }
+    hipLaunchKernelGGL(k_compact_map, dim3(1), dim3(1024), 0, st, row_has_gradient + t0, (int)n_tok, (int)n_tok, (int)kept,
+                       out_rows, act_rows);
     if (!panel_logits(st, w, ws, hid, weight, n_tok, H, V)) return AA_ERR_LAUNCH;
-    const int rc = aa_logits_bwd(ds, AA_BF16, n_tok, V, V, labels + t0, inv_temperature, row_lse + t0,
-                                 row_ez ? row_ez + t0 : nullptr, g_logp + t0, g_entropy ? g_entropy + t0 : nullptr, n_tok,
-                                 ds, stream);
+    const int rc = logits_bwd_rows(ws + w.off_ds, AA_BF16, n_tok, V, V, labels + t0, inv_temperature, row_lse + t0, ez,
+                                   g_logp + t0, gh, n_tok, ws + w.off_dst, out_rows, stream);
     if (rc != AA_OK) return rc;
-    if (!panel_gradients(st, w, ws, w.off_ds, w.off_dst, hid, nullptr, n_tok, round_up(n_tok, 8), n_tok, H, V,
-                         (uint16_t*)d_hidden + t0 * H, dw.acc, dw.acc_f32, t0 == 0))
+    uint16_t* dh_kept = (uint16_t*)(ws + w.off_dhc);
+    const int64_t n_gemm = round_up(kept, 256);
+    if (!panel_gradients(st, w, ws, w.off_dst, w.off_ds, hid, act_rows, kept, n_gemm, n_gemm, H, V, dh_kept, dw.acc,
+                         dw.acc_f32, first))
       return AA_ERR_LAUNCH;
+    first = false;
+    hipLaunchKernelGGL(k_scatter_rows, dim3((unsigned)n_tok), dim3(256), 0, st, (const u32x4_t*)dh_kept, out_rows,
+                       (u32x4_t*)dh, (int)(H / 8));
   }
+  if (first) launch_zero(st, dw.acc, V * H * (dw.acc_f32 ? 4 : 2));  // no row of the batch has a gradient
   finish_weight_grad(st, dw, d_weight, V, H);
   return launch_status();
 }

@@ -16,4 +16,9 @@ int logits_ppo_fused_rows(const void* logits, int dtype, int64_t T, int64_t V, i
                           float* vmin, float* stat_loss, float* ratio, uint8_t* flags, void* dlogits,
                           const int32_t* out_rows, int32_t* work, void* stream);
 
+// aa_logits_bwd with the same kind of row map.
+int logits_bwd_rows(const void* logits, int dtype, int64_t T, int64_t V, int64_t row_stride, const int64_t* labels,
+                    float inv_temperature, const float* row_lse, const float* row_ez, const float* g_logp,
+                    const float* g_entropy, int64_t T_active, void* dlogits, const int32_t* out_rows, void* stream);
+
 }  // namespace aa

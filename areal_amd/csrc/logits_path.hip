@@ -257,10 +257,12 @@ __global__ __launch_bounds__(NT) void k_logits_bwd(const void* __restrict__ logi
                                                    const float* __restrict__ row_ez,
                                                    const float* __restrict__ g_logp,
                                                    const float* __restrict__ g_entropy, int64_t T_active,
-                                                   void* __restrict__ dlogits) {
+                                                   void* __restrict__ dlogits, const int32_t* __restrict__ out_rows) {
   const int64_t t = blockIdx.x;
+  const int64_t orow = out_rows ? (int64_t)out_rows[t] : t;  // row map of the gradient, as in the fused kernels
+  if (orow < 0) return;
   const void* row = row_ptr(logits, t, stride, Elem<DT>::kBytes);
-  void* out = (void*)row_ptr(dlogits, t, stride, Elem<DT>::kBytes);
+  void* out = (void*)row_ptr(dlogits, orow, stride, Elem<DT>::kBytes);
   const float gl = (t < T_active) ? g_logp[t] : 0.f;
   const float gh = (t < T_active && g_entropy) ? g_entropy[t] : 0.f;
   if (gl == 0.f && gh == 0.f) {
@@ -914,6 +916,13 @@ extern "C" int aa_logits_bwd(const void* logits, int dtype, int64_t T, int64_t V
                              const int64_t* labels, float inv_temperature, const float* row_lse,
                              const float* row_ez, const float* g_logp, const float* g_entropy, int64_t T_active,
                              void* dlogits, void* stream) {
+  return aa::logits_bwd_rows(logits, dtype, T, V, row_stride, labels, inv_temperature, row_lse, row_ez, g_logp, g_entropy,
+                             T_active, dlogits, nullptr, stream);
+}
+
+int aa::logits_bwd_rows(const void* logits, int dtype, int64_t T, int64_t V, int64_t row_stride, const int64_t* labels,
+                        float inv_temperature, const float* row_lse, const float* row_ez, const float* g_logp,
+                        const float* g_entropy, int64_t T_active, void* dlogits, const int32_t* out_rows, void* stream) {
   if (!common_args_ok(logits, dtype, T, V, row_stride, labels)) return AA_ERR_INVALID_ARGUMENT;
   if (!row_lse || !g_logp || !dlogits || (g_entropy && !row_ez)) return AA_ERR_INVALID_ARGUMENT;
   if (T_active < 0 || T_active > T || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
@@ -922,7 +931,7 @@ extern "C" int aa_logits_bwd(const void* logits, int dtype, int64_t T, int64_t V
   constexpr int NT = 256;
 #define AA_LAUNCH(DT)                                                                                        \
   hipLaunchKernelGGL((k_logits_bwd<DT, NT>), dim3((unsigned)T), dim3(NT), 0, st, logits, (int)V, row_stride, \
-                     labels, inv_temperature, vec_ok, row_lse, row_ez, g_logp, g_entropy, T_active, dlogits)
+                     labels, inv_temperature, vec_ok, row_lse, row_ez, g_logp, g_entropy, T_active, dlogits, out_rows)
   if (dtype == AA_BF16) AA_LAUNCH(AA_BF16);
   else if (dtype == AA_F16) AA_LAUNCH(AA_F16);
   else AA_LAUNCH(AA_F32);

@@ -688,12 +688,20 @@ class _LmHeadLogprobsEntropy(torch.autograd.Function):
         d_hidden = torch.empty_like(hidden)
         d_weight = torch.empty_like(weight)  # bf16: rounded once, after fp32 accumulation over the chunks
         ws = _lmhead_workspace(T, H, V, dev)
+        # Rows whose upstream gradients are all zero (masked tokens) are left out of the gradient GEMMs; their
+        # count per chunk sizes the GEMMs, so the host reads it here.
+        has_grad = g_logp != 0 if g_entropy is None else (g_logp != 0) | (g_entropy != 0)
+        chunk = int(lib.aa_lmhead_chunk_tokens())
+        n_chunks = (T + chunk - 1) // chunk
+        padded = has_grad if n_chunks * chunk == T else torch.nn.functional.pad(has_grad, (0, n_chunks * chunk - T))
+        per_chunk = _HostCounts(padded.view(n_chunks, chunk).sum(1)).tolist()
+        kept = (C.c_int64 * n_chunks)(*per_chunk)
         with torch.cuda.device(dev):
             N.check(
                 lib.aa_lmhead_bwd(
                     _ptr(hidden), _ptr(weight), T, H, V, _ptr(labels), 1.0 / ctx.temperature, _ptr(row_lse),
-                    _ptr(row_ez), _ptr(g_logp), _ptr(g_entropy), _ptr(d_hidden), _ptr(d_weight),
-                    _DTYPES[d_weight.dtype], _ptr(ws), ws.numel(), _stream(dev),
+                    _ptr(row_ez), _ptr(g_logp), _ptr(g_entropy), _ptr(has_grad.view(torch.uint8)), kept,
+                    _ptr(d_hidden), _ptr(d_weight), _DTYPES[d_weight.dtype], _ptr(ws), ws.numel(), _stream(dev),
                 ),
                 "aa_lmhead_bwd",
             )

@@ -410,11 +410,18 @@ int aa_lmhead_fwd(const void* hidden, const void* weight, int64_t T, int64_t H,
  * (bf16: rounded once at the end).
  * Per chunk: the logits GEMM again, the kernel of aa_logits_bwd in place, and
  * the two gradient GEMMs (6 T V H flops for the 4 T V H of the backward).
+ * row_has_gradient [T] (device, one byte per token) with kept_per_chunk (HOST,
+ * its non-zero count per chunk of aa_lmhead_chunk_tokens() tokens), both or
+ * neither: rows whose byte is zero must have g_logp == 0 and g_entropy == 0;
+ * they are left out of the gradient GEMMs (see aa_lmhead_ppo_fused), and a
+ * chunk without any such row skips its logits GEMM as well.
  */
 int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, int64_t H,
                   int64_t V, const int64_t* labels, float inv_temperature,
                   const float* row_lse, const float* row_ez,
-                  const float* g_logp, const float* g_entropy, void* d_hidden,
+                  const float* g_logp, const float* g_entropy,
+                  const uint8_t* row_has_gradient,
+                  const int64_t* kept_per_chunk, void* d_hidden,
                   void* d_weight, int d_weight_dtype, void* workspace,
                   int64_t workspace_bytes, void* stream);
 

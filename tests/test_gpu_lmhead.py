@@ -208,7 +208,7 @@ def test_weight_gradient_dtypes_through_the_c_abi(device, T, H, V):
         dh = torch.empty_like(hd)
         dw = torch.full((V, H), float("nan"), dtype=dt, device=device)
         N.check(lib.aa_lmhead_bwd(F._ptr(hd), F._ptr(wd), T, H, V, F._ptr(ld), 1.0, F._ptr(lse), F._ptr(ez), F._ptr(gd),
-                                  None, F._ptr(dh), F._ptr(dw), code, F._ptr(ws), ws.numel(), st), "aa_lmhead_bwd")
+                                  None, None, None, F._ptr(dh), F._ptr(dw), code, F._ptr(ws), ws.numel(), st), "aa_lmhead_bwd")
         out[dt] = (dh.cpu().float(), dw.cpu().float())
     dh32, dw32 = out[torch.float32]
     dh16, dw16 = out[torch.bfloat16]
@@ -219,5 +219,50 @@ def test_weight_gradient_dtypes_through_the_c_abi(device, T, H, V):
     assert cosine(dw16, dw32) > 0.99999
     # an unknown dtype code is refused
     rc = lib.aa_lmhead_bwd(F._ptr(hd), F._ptr(wd), T, H, V, F._ptr(ld), 1.0, F._ptr(lse), F._ptr(ez), F._ptr(gd), None,
-                           F._ptr(dh), F._ptr(dw), N.AA_F16, F._ptr(ws), ws.numel(), st)
+                           None, None, F._ptr(dh), F._ptr(dw), N.AA_F16, F._ptr(ws), ws.numel(), st)
     assert rc == 2  # AA_ERR_UNSUPPORTED
+
+
+def test_backward_leaves_out_rows_without_gradient(device):
+    """lm_head_logprobs_entropy backward with many zero upstream gradients (two chunks, one of them all zero) against
+    the same call through the C ABI with every row multiplied through."""
+    import ctypes as C
+
+    from areal_amd import _native as N
+    from areal_amd import functional as F
+
+    T, H, V = 16384 + 520, 64, 1088
+    hidden, weight, labels = _case(T, H, V, seed=77, w_std=0.3)
+    g = torch.Generator().manual_seed(78)
+    gl = torch.randn(T, generator=g) * (torch.rand(T, generator=g) < 0.4)
+    gh = 0.2 * torch.randn(T, generator=g) * (torch.rand(T, generator=g) < 0.1)
+    gl[16384:] = 0.0
+    gh[16384:] = 0.0                                   # the second chunk has no gradient at all
+    h_d = hidden.to(device).requires_grad_(True)
+    w_d = weight.to(device).requires_grad_(True)
+    lp, ent = areal_amd.lm_head_logprobs_entropy(h_d, w_d, labels.to(device))
+    ((lp * gl.to(device)).sum() + (ent * gh.to(device)).sum()).backward()
+    # dense reference through the C ABI
+    lib = N.load()
+    hd, wd, ld = hidden.to(device), weight.to(device), labels.to(device)
+    f32 = dict(dtype=torch.float32, device=device)
+    logp, e, lse, ez = (torch.empty(T, **f32) for _ in range(4))
+    ws = F._lmhead_workspace(T, H, V, device)
+    st = C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    N.check(lib.aa_lmhead_fwd(F._ptr(hd), F._ptr(wd), T, H, V, F._ptr(ld), 1.0, F._ptr(logp), F._ptr(e), F._ptr(lse),
+                              F._ptr(ez), F._ptr(ws), ws.numel(), st), "aa_lmhead_fwd")
+    dh, dw = torch.empty_like(hd), torch.empty_like(wd)
+    gld, ghd = gl.to(device), gh.to(device)
+    N.check(lib.aa_lmhead_bwd(F._ptr(hd), F._ptr(wd), T, H, V, F._ptr(ld), 1.0, F._ptr(lse), F._ptr(ez), F._ptr(gld),
+                              F._ptr(ghd), None, None, F._ptr(dh), F._ptr(dw), N.AA_BF16, F._ptr(ws), ws.numel(), st),
+            "aa_lmhead_bwd")
+    off = ((gl == 0) & (gh == 0)).to(device)
+    assert float(h_d.grad[off].float().abs().max()) == 0.0 and float(dh[off].float().abs().max()) == 0.0
+    for a, b in ((h_d.grad.float(), dh.float()), (w_d.grad.float(), dw.float())):
+        assert float((a - b).abs().max()) <= float(b.abs().max()) * 2.0 ** -7
+        assert cosine(a.cpu(), b.cpu()) > 0.99999
+    # mismatched pair of arguments
+    rc = lib.aa_lmhead_bwd(F._ptr(hd), F._ptr(wd), T, H, V, F._ptr(ld), 1.0, F._ptr(lse), F._ptr(ez), F._ptr(gld),
+                           F._ptr(ghd), F._ptr(off.view(torch.uint8)), None, F._ptr(dh), F._ptr(dw), N.AA_BF16, F._ptr(ws),
+                           ws.numel(), st)
+    assert rc == 1  # AA_ERR_INVALID_ARGUMENT
