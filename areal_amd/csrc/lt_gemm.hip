@@ -4,11 +4,14 @@
 // the first and 1 560 with the second, n = 12288 the other way round).  So the first time a shape is seen with
 // beta == 0 (the output is overwritten, a trial run does no harm) the leading candidates are timed on the caller's
 // stream with the caller's operands and the fastest is kept.  That blocks the host for a few GEMM durations, once
-// per shape; AREAL_AMD_GEMM_TUNE=0 turns it off, and a capturing stream is never timed.
+// per shape; AREAL_AMD_GEMM_TUNE=0 turns it off, and a capturing stream is never timed.  AREAL_AMD_GEMM_TUNE_LOG=1
+// prints the timings.  Which candidate wins depends on the operands too (the matrix cores clock down on data with
+// many bit flips), which is one more reason to time with the caller's own data.
 #include "lt_gemm.h"
 
 #include <hipblaslt/hipblaslt.h>
 
+#include <cstdio>
 #include <cstdlib>
 #include <map>
 #include <mutex>
@@ -103,6 +106,9 @@ bool gemm(hipStream_t st, bool transA, bool transB, int64_t m, int64_t n, int64_
           if (!run() || hipEventRecord(e0, st) != hipSuccess || !run() || hipEventRecord(e1, st) != hipSuccess ||
               hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(&ms, e0, e1) != hipSuccess)
             continue;
+          if (std::getenv("AREAL_AMD_GEMM_TUNE_LOG"))
+            fprintf(stderr, "[areal_amd] gemm m=%lld n=%lld k=%lld f32=%d: candidate %d %.3f ms\n", (long long)m,
+                    (long long)n, (long long)k, (int)out_f32, c, ms);
           if (best_ms < 0.f || ms < best_ms) {
             best_ms = ms;
             best = c;
