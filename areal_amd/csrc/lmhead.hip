@@ -231,6 +231,28 @@ static void finish_weight_grad(hipStream_t st, const WeightGrad& g, void* d_weig
                      (u32x4_t*)d_weight, n8);
 }
 
+// Row count of the d_hidden GEMM for `kept` rows with a gradient (its output is a scratch buffer with room for a whole
+// chunk, the extra rows are never read).  The library's kernels for a small output with a very long contraction
+// split the contraction over the compute units, and at H = 4096 (16 tiles of 256 across) they run 20 % slower when
+// the 256 x 256 output tiles do not come to a multiple of half the unit count (n = 11520: 720 tiles, 11.9 ms;
+// n = 12288: 768 tiles, 9.9 ms).  Where H allows such a multiple within 2048 rows the count is rounded up to it;
+// otherwise (H = 5376: 21 tiles across, no gain measured) to the tile size.  The d_weight GEMM, where the rows are
+// the contraction, always takes the count rounded up to 256.
+static int64_t d_hidden_gemm_rows(int64_t kept, int64_t chunk, int64_t H) {
+  static const int64_t half_units = [] {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 2)
+      cus = 256;
+    return (int64_t)cus / 2;
+  }();
+  const int64_t tiles_across = (H + 255) / 256;
+  int64_t step = 256;
+  if (half_units % tiles_across == 0 && half_units / tiles_across <= 8) step = 256 * (half_units / tiles_across);
+  const int64_t n = round_up(kept, step);
+  return n < chunk ? n : chunk;
+}
+
 static bool shapes_ok(int64_t T, int64_t H, int64_t V) {
   return T > 0 && H > 0 && V > 0 && (H % 8) == 0 && (V % 8) == 0 && T < (1 << 30) && V < (1 << 30) && H < (1 << 30) &&
          (V / 64 + 1) * ((H > kChunkTokens ? H : kChunkTokens) / 64 + 1) < (1LL << 31);  // transpose grids
@@ -322,8 +344,8 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
                                    g_logp + t0, gh, n_tok, ws + w.off_dst, out_rows, stream);
     if (rc != AA_OK) return rc;
     uint16_t* dh_kept = (uint16_t*)(ws + w.off_dhc);
-    const int64_t n_gemm = round_up(kept, 256);
-    if (!panel_gradients(st, w, ws, w.off_dst, w.off_ds, hid, act_rows, kept, n_gemm, n_gemm, H, V, dh_kept, dw.acc,
+    if (!panel_gradients(st, w, ws, w.off_dst, w.off_ds, hid, act_rows, kept, round_up(kept, 256),
+                         d_hidden_gemm_rows(kept, w.chunk, H), H, V, dh_kept, dw.acc,
                          dw.acc_f32, first))
       return AA_ERR_LAUNCH;
     first = false;
@@ -401,9 +423,8 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
       continue;
     }
     uint16_t* dh_kept = (uint16_t*)(ws + w.off_dhc);
-    // GEMM sizes rounded up to the library's tile (the buffers hold a whole chunk, a multiple of 256 rows)
-    const int64_t n_gemm = round_up(kept, 256);
-    if (!panel_gradients(st, w, ws, w.off_dst, w.off_ds, hid, act_rows, kept, n_gemm, n_gemm, H, V, dh_kept, dw.acc,
+    if (!panel_gradients(st, w, ws, w.off_dst, w.off_ds, hid, act_rows, kept, round_up(kept, 256),
+                         d_hidden_gemm_rows(kept, w.chunk, H), H, V, dh_kept, dw.acc,
                          dw.acc_f32, first))
       return AA_ERR_LAUNCH;
     first = false;
