@@ -11,8 +11,10 @@ One "step" is one pass of the hot path over one synthetic packed micro-batch tha
   4 * V per token (the bf16 logits read once, their gradient written once).
 * fused lm_head workloads (cfg2, cfg3, cfg4): ``fused_lm_head_ppo_loss(hidden, W, labels, ...)`` followed by
   ``loss.backward()``: lm_head, log-prob / entropy, PPO loss and the gradients d(hidden), d(W), token chunk by
-  token chunk, the full [T, V] logits never in memory.  Roofline: bf16 MFMA, algorithmic flops 6 * T * V * H
-  (logits 2TVH, the two gradient GEMMs 4TVH).
+  token chunk, the full [T, V] logits never in memory.  Roofline: bf16 MFMA.  Algorithmic flops: 2 T V H for the
+  logits of every token + 4 T_grad V H for the two gradient GEMMs over the tokens that have a gradient (masked
+  tokens have none and are left out; ``--dense-backward`` multiplies their zero rows through like the reference's
+  autograd, 6 T V H).  ``roofline.dense_equivalent_tflops`` quotes the same time against 6 T V H.
 
 * adv: the advantage pipeline that precedes the loss (not one of the headline configurations): GAE reverse scan plus batch
   normalisation over a padded [512, 4096] batch.  Roofline: HBM, 20 bytes per token for the scan (rewards, values,
