@@ -804,6 +804,7 @@ def fused_lm_head_ppo_loss(
     temperature: float = 1.0,
     loss_scale: torch.Tensor | float | None = None,
     skip_masked_tokens: bool = True,
+    forward_masked_tokens: bool = True,
 ) -> tuple[torch.Tensor, dict]:
     """lm_head + ``gather_logprobs_entropy`` + ``ppo_actor_loss_fn`` (+ backward) for one micro-batch.
 
@@ -819,6 +820,12 @@ def fused_lm_head_ppo_loss(
     size the GEMMs, so the host reads them (one small device-to-host copy that waits for the mask only) before it
     queues the chunk.  ``False`` multiplies the zero rows through, as the reference's autograd does, without that
     read.
+
+    ``forward_masked_tokens=False`` (token level only) goes one step further than the reference's semantics: tokens
+    whose effective mask is zero are not run through the lm_head at all, so their entries of ``stat["logprobs"]``,
+    ``stat["entropy"]``, ``stat["loss"]``, ``stat["importance_weight"]`` and ``stat["approx_kl"]`` are zero instead
+    of the values the reference computes there (and every consumer masks out).  Loss, gradients and the entries of
+    the other tokens are unchanged.
     """
     if importance_sampling_level not in ("token", "sequence"):
         raise ValueError(
@@ -872,6 +879,41 @@ def fused_lm_head_ppo_loss(
         n_valid = counts
     else:
         n_valid = _count_nonzero(m8)
+    if not forward_masked_tokens:
+        # only the tokens with a mask go through the lm_head: gather them (autograd scatters d(hidden) back), run the
+        # step on the closed-up batch with an all-true mask, and put the per-token results back at their tokens
+        idx = mask_eff.nonzero().squeeze(-1)
+        n_kept = idx.numel()
+        full = lambda v, dtype=torch.float32: torch.zeros(T_active, dtype=dtype, device=dev).index_copy_(0, idx, v)
+        if n_kept == 0:
+            loss = (hidden[:1].float().sum() + weight[:1].float().sum()) * 0.0
+            z = torch.zeros(T_active, dtype=torch.float32, device=dev)
+            zb = torch.zeros(T_active, dtype=torch.bool, device=dev)
+            stat = dict(loss=z, importance_weight=z.clone(), approx_kl=z.clone(), clip_mask=zb, dual_clip_mask=zb.clone(),
+                        logprobs=z.clone(), entropy=z.clone())
+        else:
+            # the closed-up batch is padded to a multiple of 256 rows (batch padding: no outputs, no gradient), which
+            # keeps the GEMM library on its fast kernels
+            ones = torch.ones(n_kept, dtype=torch.uint8, device=dev)
+            chunk = int(N.load().aa_lmhead_chunk_tokens())
+            n_rows = (n_kept + 255) // 256 * 256
+            pad = n_rows - n_kept
+            kept = [max(0, min(chunk, n_kept - c)) for c in range(0, n_rows, chunk)]
+            loss, logp, entropy, stat_loss, ratio, flags = _FusedLmHeadPpo.apply(
+                torch.nn.functional.pad(hidden.index_select(0, idx), (0, 0, 0, pad)), weight.contiguous(),
+                torch.nn.functional.pad(y.index_select(0, idx), (0, pad)), float(temperature), n_kept,
+                prox.index_select(0, idx), adv.index_select(0, idx), ones,
+                None if w is None else w.index_select(0, idx), params, n_valid, scale_t, kept,
+            )
+            logp, entropy = logp[:n_kept], entropy[:n_kept]
+            stat = dict(
+                loss=full(stat_loss), importance_weight=full(ratio), approx_kl=full(logp - prox.index_select(0, idx)),
+                clip_mask=full((flags & 1).bool(), torch.bool), dual_clip_mask=full((flags & 2).bool(), torch.bool),
+                logprobs=full(logp), entropy=full(entropy),
+            )
+        if rejection_sampling is not None:
+            _rs_stats(stat, prox, old, mask_eff, w, host_counts, loss_mask.shape)
+        return loss, stat
     kept = None
     if skip_masked_tokens:
         chunk = int(N.load().aa_lmhead_chunk_tokens())

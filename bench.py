@@ -71,6 +71,10 @@ def parse_args():
     ap.add_argument("--dense-backward", action="store_true",
                     help="lm_head workloads: run masked tokens through the gradient GEMMs too (as the reference's "
                          "autograd does) instead of leaving their zero rows out")
+    ap.add_argument("--no-forward-of-masked", action="store_true",
+                    help="lm_head workloads, outside the reference's semantics: masked tokens skip the lm_head "
+                         "altogether (fused_lm_head_ppo_loss(forward_masked_tokens=False)); only ms_per_step and value "
+                         "reflect it, and the line says so in config.path")
     ap.add_argument("--copy-launches", type=int, default=0,
                     help="also launch the plain copy kernel this many times over the logits buffer "
                          "(the calibration point for FETCH_SIZE / WRITE_SIZE counters)")
@@ -314,6 +318,7 @@ def build_fused_case(name: str, seed: int, device):
 
 
 DENSE_BACKWARD = False  # set from --dense-backward
+NO_FORWARD_OF_MASKED = False  # set from --no-forward-of-masked
 
 
 def run_fused_steps(case, n, kw, cfg):
@@ -327,7 +332,7 @@ def run_fused_steps(case, n, kw, cfg):
         loss, _ = areal_amd.fused_lm_head_ppo_loss(
             h, w, case.labels, case.prox_logp, case.old_logp, case.advantages, loss_mask=case.loss_mask,
             rejection_sampling=cfg, cu_seqlens=case.cu_seqlens, temperature=case.temperature,
-            skip_masked_tokens=not DENSE_BACKWARD, **kw,
+            skip_masked_tokens=not DENSE_BACKWARD, forward_masked_tokens=not NO_FORWARD_OF_MASKED, **kw,
         )
         loss.backward()
     return loss
@@ -533,6 +538,9 @@ def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: i
                     path="lm_head + PPO loss step in token chunks (at most one chunk of logits in memory), fwd + bwd"),
         roofline=roofline,
     )
+    if NO_FORWARD_OF_MASKED:
+        out["config"]["path"] += "; NOT the reference's semantics: masked tokens skip the lm_head (value and " \
+                                 "ms_per_step only; roofline figures are those of the default call)"
     if cpu_tokens > 0:
         baseline, parity = fused_cpu_baseline_and_parity(case, kw, cfg, cpu_tokens, args.cpu_iters)
         out["cpu_baseline"] = baseline
@@ -714,10 +722,11 @@ def synth_lengths(total, seed):
 
 
 def main():
-    global RS_ACTION, DENSE_BACKWARD
+    global RS_ACTION, DENSE_BACKWARD, NO_FORWARD_OF_MASKED
     args = parse_args()
     RS_ACTION = args.rs_action
     DENSE_BACKWARD = args.dense_backward
+    NO_FORWARD_OF_MASKED = args.no_forward_of_masked
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU; run it with --gpus 1 (no multi-GPU path exists)", file=sys.stderr)
         sys.exit(2)

@@ -222,3 +222,40 @@ def test_skipping_masked_tokens_equals_the_dense_backward(device, pattern):
         scale = float(b.abs().max())
         assert float((a - b).abs().max()) <= scale * 2.0 ** -7
         assert cosine(a.cpu(), b.cpu()) > 0.99999
+
+
+@pytest.mark.parametrize("with_rs", [False, True])
+def test_not_forwarding_masked_tokens_keeps_loss_and_gradients(device, with_rs):
+    """forward_masked_tokens=False: tokens without a mask never reach the lm_head; loss, gradients and the statistics
+    of the other tokens are those of the default call, the masked entries are zero."""
+    hidden, weight, labels, prox, old, adv, mask = _inputs(700, 650, 64, 8200, seed=31)
+    rs = RejectionSamplingConfig(level="token", action="mask", metric="ratio", upper=1.3) if with_rs else None
+    args = [t.to(device) for t in (labels, prox, old, adv)]
+
+    def run(forward_masked):
+        h = hidden.to(device).requires_grad_(True)
+        w = weight.to(device).requires_grad_(True)
+        loss, stat = areal_amd.fused_lm_head_ppo_loss(h, w, *args, eps_clip=0.2, loss_mask=mask.to(device), c_clip=3.0,
+                                                      rejection_sampling=rs, forward_masked_tokens=forward_masked)
+        loss.backward()
+        return loss.detach(), stat, h.grad.float(), w.grad.float()
+
+    l0, s0, dh0, dw0 = run(True)
+    l1, s1, dh1, dw1 = run(False)
+    assert float(l1) == pytest.approx(float(l0), rel=1e-5)
+    on = s0["behave_mask"] if with_rs else mask.to(device)
+    for k in ("logprobs", "entropy", "loss", "importance_weight", "approx_kl"):
+        assert torch.allclose(s1[k][on], s0[k][on], rtol=1e-5, atol=1e-6), k
+        assert float(s1[k][~on].abs().sum()) == 0.0, k
+    for k in ("clip_mask", "dual_clip_mask"):
+        assert torch.equal(s1[k], s0[k]), k
+    for a, b in ((dh1, dh0), (dw1, dw0)):
+        assert float((a - b).abs().max()) <= float(b.abs().max()) * 2.0 ** -7 and cosine(a.cpu(), b.cpu()) > 0.99999
+    # nothing valid at all
+    none = torch.zeros_like(mask).to(device)
+    h = hidden.to(device).requires_grad_(True)
+    w = weight.to(device).requires_grad_(True)
+    loss, stat = areal_amd.fused_lm_head_ppo_loss(h, w, *args, eps_clip=0.2, loss_mask=none, forward_masked_tokens=False)
+    loss.backward()
+    assert float(loss.detach()) == 0.0 and float(h.grad.abs().sum()) == 0.0 and float(w.grad.abs().sum()) == 0.0
+    assert float(stat["logprobs"].abs().sum()) == 0.0
