@@ -709,7 +709,8 @@ class _LmHeadLogprobsEntropy(torch.autograd.Function):
 
 
 def lm_head_logprobs_entropy(
-    hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0
+    hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0,
+    token_mask: torch.Tensor | None = None,
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """``gather_logprobs_entropy(hidden @ weight.T, labels, temperature)`` without materialising the ``[T, V]`` logits.
 
@@ -721,6 +722,10 @@ def lm_head_logprobs_entropy(
     gradient is returned in the dtype of ``weight``).
     The reference has no such op: it is the drop-in for its lm_head matmul followed by
     ``gather_logprobs_entropy`` (vocab_parallel.py:434-469).
+
+    ``token_mask`` (``[T]``, optional, beyond the reference's semantics): only tokens whose entry is non-zero go
+    through the lm_head; the others get log-prob 0 and entropy 0 (e.g. the forward-only ``compute_logp`` pass, whose
+    results are multiplied by the loss mask anyway).
     """
     _require_gpu(hidden, "hidden")
     if hidden.ndim != 2 or weight.ndim != 2 or hidden.shape[1] != weight.shape[1]:
@@ -731,6 +736,21 @@ def lm_head_logprobs_entropy(
     if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
         raise TypeError("fused lm_head expects bf16 hidden states and weights")
     y = labels.to(device=hidden.device, dtype=torch.int64).contiguous()
+    if token_mask is not None:
+        if tuple(token_mask.shape) != (hidden.shape[0],):
+            raise ValueError(f"token_mask shape {tuple(token_mask.shape)} != ({hidden.shape[0]},)")
+        T, dev = hidden.shape[0], hidden.device
+        idx = token_mask.to(dev).ne(0).nonzero().squeeze(-1)
+        n_kept = idx.numel()
+        if n_kept == 0:
+            zero = (hidden[:1].float().sum() + weight[:1].float().sum()) * 0.0
+            return zero.expand(T), zero.expand(T)
+        pad = (n_kept + 255) // 256 * 256 - n_kept  # round sizes keep the GEMM library on its fast kernels
+        lp, ent = _LmHeadLogprobsEntropy.apply(
+            torch.nn.functional.pad(hidden.index_select(0, idx), (0, 0, 0, pad)), weight.contiguous(),
+            torch.nn.functional.pad(y.index_select(0, idx), (0, pad)), float(temperature))
+        full = lambda v: torch.zeros(T, dtype=torch.float32, device=dev).index_copy(0, idx, v[:n_kept])
+        return full(lp), full(ent)
     return _LmHeadLogprobsEntropy.apply(hidden.contiguous(), weight.contiguous(), y, float(temperature))
 
 

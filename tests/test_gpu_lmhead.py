@@ -266,3 +266,26 @@ def test_backward_leaves_out_rows_without_gradient(device):
                            F._ptr(ghd), F._ptr(off.view(torch.uint8)), None, F._ptr(dh), F._ptr(dw), N.AA_BF16, F._ptr(ws),
                            ws.numel(), st)
     assert rc == 1  # AA_ERR_INVALID_ARGUMENT
+
+
+def test_token_mask_runs_only_the_selected_tokens(device):
+    T, H, V = 700, 128, 1088
+    hidden, weight, labels = _case(T, H, V, seed=91, w_std=0.3)
+    g = torch.Generator().manual_seed(92)
+    sel = torch.rand(T, generator=g) < 0.4
+    gl = torch.randn(T, generator=g)
+    hd, wd, ld = hidden.to(device), weight.to(device), labels.to(device)
+    h0, w0 = hd.clone().requires_grad_(True), wd.clone().requires_grad_(True)
+    lp0, ent0 = areal_amd.lm_head_logprobs_entropy(h0, w0, ld, 0.9)
+    ((lp0 * gl.to(device) + 0.1 * ent0) * sel.to(device)).sum().backward()
+    h1, w1 = hd.clone().requires_grad_(True), wd.clone().requires_grad_(True)
+    lp1, ent1 = areal_amd.lm_head_logprobs_entropy(h1, w1, ld, 0.9, token_mask=sel.to(device))
+    (lp1 * gl.to(device) + 0.1 * ent1).sum().backward()
+    s = sel.to(device)
+    assert torch.allclose(lp1[s], lp0[s].detach(), atol=1e-6) and torch.allclose(ent1[s], ent0[s].detach(), atol=1e-6)
+    assert float(lp1.detach()[~s].abs().sum()) == 0.0 and float(ent1.detach()[~s].abs().sum()) == 0.0
+    assert cosine(h1.grad.cpu(), h0.grad.cpu()) > 0.99999 and cosine(w1.grad.cpu(), w0.grad.cpu()) > 0.99999
+    assert float(h1.grad[~s].float().abs().sum()) == 0.0
+    none = torch.zeros(T, dtype=torch.bool, device=device)
+    lp2, ent2 = areal_amd.lm_head_logprobs_entropy(hd, wd, ld, token_mask=none)
+    assert float(lp2.abs().sum()) == 0.0 and lp2.shape == (T,)
