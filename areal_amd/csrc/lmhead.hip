@@ -110,6 +110,11 @@ __global__ __launch_bounds__(1024) void k_compact_map(const uint8_t* __restrict_
     if (on) act_rows[pos] = t;
     pos += (t < act && mask[t] != 0) ? 1 : 0;
   }
+  // a host count larger than what the mask holds leaves positions without a token: point them at row 0, so that the
+  // gathers that follow stay inside the chunk (their contribution is then meaningless, as the caller's count was)
+  int total = 0;
+  for (int w = 0; w < 16; ++w) total += wave_sum[w];
+  for (int p = total + tid; p < limit; p += 1024) act_rows[p] = 0;
 }
 
 // dst[t, :] = out_rows[t] >= 0 ? src[out_rows[t], :] : 0 for the n_tok rows of a chunk (H % 8 == 0)

@@ -289,3 +289,45 @@ def test_token_mask_runs_only_the_selected_tokens(device):
     none = torch.zeros(T, dtype=torch.bool, device=device)
     lp2, ent2 = areal_amd.lm_head_logprobs_entropy(hd, wd, ld, token_mask=none)
     assert float(lp2.abs().sum()) == 0.0 and lp2.shape == (T,)
+
+
+def test_row_counts_that_disagree_with_the_mask_stay_in_bounds(device):
+    """kept_per_chunk comes from the host.  Too small: the rows beyond it count as rows without gradient.  Too large:
+    the result is meaningless but every access stays inside the buffers (the call returns, the device stays usable)."""
+    import ctypes as C
+
+    from areal_amd import _native as N
+    from areal_amd import functional as F
+
+    lib = N.load()
+    T, H, V = 900, 64, 1088
+    hidden, weight, labels = _case(T, H, V, seed=5, w_std=0.3)
+    hd, wd, ld = hidden.to(device), weight.to(device), labels.to(device)
+    g = torch.Generator().manual_seed(6)
+    gl = (torch.randn(T, generator=g) * (torch.rand(T, generator=g) < 0.5)).to(device)
+    f32 = dict(dtype=torch.float32, device=device)
+    logp, e, lse, ez = (torch.empty(T, **f32) for _ in range(4))
+    ws = F._lmhead_workspace(T, H, V, device)
+    st = C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    N.check(lib.aa_lmhead_fwd(F._ptr(hd), F._ptr(wd), T, H, V, F._ptr(ld), 1.0, F._ptr(logp), F._ptr(e), F._ptr(lse),
+                              F._ptr(ez), F._ptr(ws), ws.numel(), st), "aa_lmhead_fwd")
+    has = (gl != 0)
+    n = int(has.sum())
+
+    def run(g_vec, rows, count):
+        dh, dw = torch.empty_like(hd), torch.empty_like(wd)
+        N.check(lib.aa_lmhead_bwd(F._ptr(hd), F._ptr(wd), T, H, V, F._ptr(ld), 1.0, F._ptr(lse), F._ptr(ez), F._ptr(g_vec),
+                                  None, F._ptr(rows.view(torch.uint8)), (C.c_int64 * 1)(count), F._ptr(dh), F._ptr(dw),
+                                  N.AA_BF16, F._ptr(ws), ws.numel(), st), "aa_lmhead_bwd")
+        torch.cuda.synchronize()
+        return dh.float(), dw.float()
+
+    dh_small, dw_small = run(gl, has, n - 5)
+    last5 = has.nonzero().squeeze(-1)[-5:]
+    gl_cut = gl.clone()
+    gl_cut[last5] = 0.0
+    dh_ref, dw_ref = run(gl_cut, gl_cut != 0, n - 5)
+    assert torch.equal(dh_small, dh_ref) and torch.equal(dw_small, dw_ref)
+    run(gl, has, n + 7)                                   # must simply come back
+    dh_ok, _ = run(gl, has, n)
+    assert bool(torch.isfinite(dh_ok).all()) and float(dh_ok[~has].abs().sum()) == 0.0
