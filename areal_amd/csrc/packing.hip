@@ -37,28 +37,36 @@ __global__ __launch_bounds__(256) void k_copy_small(const W* __restrict__ src, W
   }
 }
 
-// rows of n_words words of type W, one workgroup per row (grid-stride over rows)
+// Rows of n_words words of type W, cut into pieces of kPieceWords words (eight per thread): one workgroup per piece,
+// grid-stride, pieces numbered along the rows.  The workgroups in flight together then cover one contiguous stretch of
+// source and destination (a few dozen rows) instead of thousands of separate row streams, which the memory system
+// serves markedly faster.
+constexpr int kPieceWords = 2048;
+
 template <typename W>
 __global__ __launch_bounds__(256) void k_copy_rows(const W* __restrict__ src, W* __restrict__ dst, int64_t n_words,
                                                    const int64_t* __restrict__ src_starts,
                                                    const int64_t* __restrict__ dst_starts,
-                                                   const int32_t* __restrict__ seg_cu, int64_t B, int64_t total) {
-  for (int64_t r = blockIdx.x; r < total; r += gridDim.x) {
+                                                   const int32_t* __restrict__ seg_cu, int64_t B, int64_t total,
+                                                   int64_t pieces_per_row) {
+  const int64_t n_pieces = total * pieces_per_row;
+  for (int64_t id = blockIdx.x; id < n_pieces; id += gridDim.x) {
+    const int64_t r = id / pieces_per_row;
     const int64_t s = find_segment(seg_cu, B, r);
     const int64_t o = r - seg_cu[s];
     const W* p = src + (src_starts[s] + o) * n_words;
     W* q = dst + (dst_starts[s] + o) * n_words;
-    // four independent loads in flight per thread before the first store
-    int64_t i = threadIdx.x;
-    for (; i + 3 * 256 < n_words; i += 4 * 256) {
-      const W a = __builtin_nontemporal_load(p + i), b = __builtin_nontemporal_load(p + i + 256);
-      const W c = __builtin_nontemporal_load(p + i + 512), d = __builtin_nontemporal_load(p + i + 768);
-      __builtin_nontemporal_store(a, q + i);
-      __builtin_nontemporal_store(b, q + i + 256);
-      __builtin_nontemporal_store(c, q + i + 512);
-      __builtin_nontemporal_store(d, q + i + 768);
+    const int64_t i = (id - r * pieces_per_row) * kPieceWords + threadIdx.x;
+    if (i + 7 * 256 < n_words) {  // eight independent loads in flight per thread before the first store
+      W v[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = __builtin_nontemporal_load(p + i + k * 256);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) __builtin_nontemporal_store(v[k], q + i + k * 256);
+    } else {
+      for (int64_t j = i; j < n_words && j < i + kPieceWords; j += 256)
+        __builtin_nontemporal_store(__builtin_nontemporal_load(p + j), q + j);
     }
-    for (; i < n_words; i += 256) __builtin_nontemporal_store(__builtin_nontemporal_load(p + i), q + i);
   }
 }
 
@@ -72,9 +80,11 @@ static void launch(const void* src, void* dst, int64_t row_bytes, const int64_t*
     hipLaunchKernelGGL(k_copy_small<W>, dim3((unsigned)blocks), dim3(256), 0, st, (const W*)src, (W*)dst, ss, ds, cu, B,
                        total);
   } else {
-    const int64_t blocks = total < 65536 ? total : 65536;
+    const int64_t pieces_per_row = (n_words + kPieceWords - 1) / kPieceWords;
+    const int64_t n_pieces = total * pieces_per_row;
+    const int64_t blocks = n_pieces < (1 << 20) ? n_pieces : (1 << 20);
     hipLaunchKernelGGL(k_copy_rows<W>, dim3((unsigned)blocks), dim3(256), 0, st, (const W*)src, (W*)dst, n_words, ss,
-                       ds, cu, B, total);
+                       ds, cu, B, total, pieces_per_row);
   }
 }
 
