@@ -251,3 +251,53 @@ def test_full_size_properties_config1(device):
         loss_scale=0.5,
     )
     assert float(loss_h) == pytest.approx(0.5 * float(l1), rel=1e-6)
+
+
+def test_fused_step_replays_from_a_hip_graph(device):
+    """The logits step (no rejection sampling, hence no host read) captured into a HIP graph: three replays on new
+    inputs, with eager work and synchronisations in between, each equal to the eager result on the same inputs."""
+    T, V = 96, 16384
+    g = torch.Generator().manual_seed(12)
+    x = torch.zeros(T, V, dtype=torch.bfloat16, device=device, requires_grad=True)
+    labels = torch.randint(0, V, (T,), generator=g).to(device)
+    prox, old, adv = (torch.zeros(T, device=device) for _ in range(3))
+    mask = (torch.rand(T, generator=g) < 0.7).to(device)
+
+    def fill(seed):
+        gg = torch.Generator().manual_seed(seed)
+        with torch.no_grad():
+            x.copy_((3 * torch.randn(T, V, generator=gg)).bfloat16())
+            ref = areal_amd.gather_logprobs(x, labels)
+            prox.copy_(ref + 0.05 * torch.randn(T, generator=gg).to(device))
+            old.copy_(ref + 0.05 * torch.randn(T, generator=gg).to(device))
+            adv.copy_(torch.randn(T, generator=gg).to(device))
+
+    def step():
+        loss, stat = areal_amd.fused_logprobs_ppo_loss(x, labels, prox, old, adv, 0.2, mask, eps_clip_higher=0.28)
+        loss.backward()
+        return loss, stat["logprobs"]
+
+    fill(0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            x.grad = None
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    x.grad = None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        g_loss, g_logp = step()
+    g_grad = x.grad
+    for seed in (1, 2, 3):
+        fill(seed)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = (g_loss.detach().clone(), g_logp.clone(), g_grad.clone())
+        y = x.detach().clone().requires_grad_(True)                     # eager, same inputs
+        e_loss, e_stat = areal_amd.fused_logprobs_ppo_loss(y, labels, prox, old, adv, 0.2, mask, eps_clip_higher=0.28)
+        e_loss.backward()
+        torch.cuda.synchronize()
+        assert torch.equal(got[0], e_loss.detach()) and torch.equal(got[1], e_stat["logprobs"])
+        assert torch.equal(got[2], y.grad)
