@@ -825,6 +825,7 @@ def fused_lm_head_ppo_loss(
     loss_scale: torch.Tensor | float | None = None,
     skip_masked_tokens: bool = True,
     forward_masked_tokens: bool = True,
+    kept_per_chunk: list[int] | None = None,
 ) -> tuple[torch.Tensor, dict]:
     """lm_head + ``gather_logprobs_entropy`` + ``ppo_actor_loss_fn`` (+ backward) for one micro-batch.
 
@@ -839,7 +840,9 @@ def fused_lm_head_ppo_loss(
     GEMMs run on the other tokens only; the results are those of the dense computation.  The per-chunk token counts
     size the GEMMs, so the host reads them (one small device-to-host copy that waits for the mask only) before it
     queues the chunk.  ``False`` multiplies the zero rows through, as the reference's autograd does, without that
-    read.
+    read.  A caller that already knows the counts on the host (the number of tokens with a non-zero effective mask
+    in each chunk of 16384 tokens, e.g. from the CPU copy of ``loss_mask`` when there is no rejection sampling) can
+    pass them as ``kept_per_chunk``; nothing is read back then.
 
     ``forward_masked_tokens=False`` (token level only) goes one step further than the reference's semantics: tokens
     whose effective mask is zero are not run through the lm_head at all, so their entries of ``stat["logprobs"]``,
@@ -935,7 +938,12 @@ def fused_lm_head_ppo_loss(
             _rs_stats(stat, prox, old, mask_eff, w, host_counts, loss_mask.shape)
         return loss, stat
     kept = None
-    if skip_masked_tokens:
+    if skip_masked_tokens and kept_per_chunk is not None:
+        chunk = int(N.load().aa_lmhead_chunk_tokens())
+        kept = [int(v) for v in kept_per_chunk]
+        if len(kept) != (hidden.shape[0] + chunk - 1) // chunk:
+            raise ValueError(f"kept_per_chunk needs one count per chunk of {chunk} tokens")
+    elif skip_masked_tokens:
         chunk = int(N.load().aa_lmhead_chunk_tokens())
         n_chunks = (hidden.shape[0] + chunk - 1) // chunk
         on = mask_eff.ne(0)

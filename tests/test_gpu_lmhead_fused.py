@@ -259,3 +259,21 @@ def test_not_forwarding_masked_tokens_keeps_loss_and_gradients(device, with_rs):
     loss.backward()
     assert float(loss.detach()) == 0.0 and float(h.grad.abs().sum()) == 0.0 and float(w.grad.abs().sum()) == 0.0
     assert float(stat["logprobs"].abs().sum()) == 0.0
+
+
+def test_counts_from_the_caller_replace_the_read_back(device):
+    hidden, weight, labels, prox, old, adv, mask = _inputs(16384 + 256, 16384 + 200, 64, 640, seed=41)
+    args = [t.to(device) for t in (labels, prox, old, adv)]
+    counts = [int(mask[:16384].sum()), int(mask[16384:].sum())]            # known on the host
+
+    def run(**kw):
+        h = hidden.to(device).requires_grad_(True)
+        w = weight.to(device).requires_grad_(True)
+        loss, _ = areal_amd.fused_lm_head_ppo_loss(h, w, *args, eps_clip=0.2, loss_mask=mask.to(device), **kw)
+        loss.backward()
+        return loss.detach(), h.grad, w.grad
+
+    a, b = run(kept_per_chunk=counts), run()
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]) and torch.equal(a[2], b[2])
+    with pytest.raises(ValueError, match="one count per chunk"):
+        run(kept_per_chunk=[1])
