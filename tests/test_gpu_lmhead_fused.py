@@ -172,12 +172,15 @@ def test_padding_only_chunk_and_no_active_token(device):
     assert float(loss.detach()) == 0.0 and float(x.grad.float().abs().sum()) == 0.0
 
 
-@pytest.mark.parametrize("pattern", ["random", "second_chunk_masked", "first_chunk_masked", "all_masked", "one_token"])
+@pytest.mark.parametrize("pattern", ["random", "second_chunk_masked", "first_chunk_masked", "all_masked", "one_token",
+                                     "random_long_rows"])
 def test_skipping_masked_tokens_equals_the_dense_backward(device, pattern):
     """Tokens with a zero mask are left out of the gradient GEMMs: same loss and statistics, same gradients as when
     their zero rows are multiplied through (two token chunks, batch padding at the end)."""
     g = torch.Generator().manual_seed(5)
     T_pad, T, H, V = 16384 + 300, 16384 + 200, 64, 8200       # the register-resident row kernel writes the closed-up rows
+    if pattern == "random_long_rows":
+        V = 180224                                            # 22 chunks: its register + LDS form
     hidden = torch.randn(T_pad, H, generator=g).bfloat16().to(device)
     weight = (0.3 * torch.randn(V, H, generator=g)).bfloat16().to(device)
     labels = torch.randint(0, V, (T_pad,), generator=g).to(device)
