@@ -592,7 +592,10 @@ def fused_logprobs_ppo_loss(
     if loss_scale is not None:
         scale_t = torch.as_tensor(loss_scale, dtype=torch.float32, device=dev).reshape(1)
 
-    if importance_sampling_level == "sequence":
+    # Without a gradient to produce (evaluation, torch.no_grad) the step is the forward kernel (one read of the logits,
+    # no [T, V] gradient buffer) followed by the loss on log-probs.
+    forward_only = not (torch.is_grad_enabled() and logits.requires_grad)
+    if importance_sampling_level == "sequence" or forward_only:
         logp, entropy, vmin, vmax = gather_logprobs_entropy_stats(logits, labels, temperature)
         logp, entropy, vmin, vmax = (t[:T_active] for t in (logp, entropy, vmin, vmax))
         loss, stat = ppo_actor_loss_fn(
@@ -874,7 +877,8 @@ def fused_lm_head_ppo_loss(
         scale_t = torch.as_tensor(loss_scale, dtype=torch.float32, device=dev).reshape(1)
     y = labels.to(device=dev, dtype=torch.int64).contiguous()
 
-    if importance_sampling_level == "sequence":
+    forward_only = not (torch.is_grad_enabled() and (hidden.requires_grad or weight.requires_grad))
+    if importance_sampling_level == "sequence" or forward_only:  # no gradient to produce: forward GEMM + loss only
         logp, entropy = lm_head_logprobs_entropy(hidden, weight, y, temperature)
         logp, entropy = logp[:T_active], entropy[:T_active]
         loss, stat = ppo_actor_loss_fn(

@@ -250,7 +250,7 @@ def test_full_size_properties_config1(device):
         x, case.labels, case.prox_logp, case.old_logp, case.advantages, 0.2, case.loss_mask, rejection_sampling=rs,
         loss_scale=0.5,
     )
-    assert float(loss_h) == pytest.approx(0.5 * float(l1), rel=1e-6)
+    assert float(loss_h.detach()) == pytest.approx(0.5 * float(l1.detach()), rel=1e-6)
 
 
 def test_fused_step_replays_from_a_hip_graph(device):
@@ -301,3 +301,33 @@ def test_fused_step_replays_from_a_hip_graph(device):
         torch.cuda.synchronize()
         assert torch.equal(got[0], e_loss.detach()) and torch.equal(got[1], e_stat["logprobs"])
         assert torch.equal(got[2], y.grad)
+
+
+def test_forward_only_calls_skip_the_gradient(device):
+    """Under torch.no_grad (or with inputs that need no gradient) the fused entry points return the same loss and
+    statistics without producing a gradient buffer."""
+    lengths = [21, 30]
+    case = synth.make_logits_case("t", lengths, 16384, 5, device, synth.per_sequence_normal_advantages(lengths, 2),
+                                  ppo=dict(eps_clip=0.2))
+    _finish_case(case)
+    loss, stat, _ = _fused_step(case)
+    with torch.no_grad():
+        l2, s2 = areal_amd.fused_logprobs_ppo_loss(case.logits, case.labels, case.prox_logp, case.old_logp,
+                                                   case.advantages, 0.2, case.loss_mask, cu_seqlens=case.cu_seqlens)
+    assert not l2.requires_grad and float(l2) == pytest.approx(float(loss), rel=1e-6)
+    for k in ("logprobs", "entropy", "loss", "importance_weight", "vocab_max_logits"):
+        assert torch.allclose(s2[k], stat[k], rtol=1e-5, atol=1e-6), k
+    assert torch.equal(s2["clip_mask"], stat["clip_mask"])
+    # lm_head step
+    g = torch.Generator().manual_seed(3)
+    T, H, V = 300, 64, 1088
+    hidden = torch.randn(T, H, generator=g).bfloat16().to(device)
+    weight = (0.3 * torch.randn(V, H, generator=g)).bfloat16().to(device)
+    labels = torch.randint(0, V, (T,), generator=g).to(device)
+    z = torch.zeros(T, device=device) - 6.0
+    adv, mask = torch.randn(T, generator=g).to(device), (torch.rand(T, generator=g) < 0.7).to(device)
+    h = hidden.clone().requires_grad_(True)
+    la, sa = areal_amd.fused_lm_head_ppo_loss(h, weight, labels, z, z, adv, 0.2, mask)
+    lb, sb = areal_amd.fused_lm_head_ppo_loss(hidden, weight, labels, z, z, adv, 0.2, mask)   # nothing requires grad
+    assert not lb.requires_grad and float(lb) == pytest.approx(float(la.detach()), rel=1e-6)
+    assert torch.allclose(sb["logprobs"], sa["logprobs"], atol=1e-6)
