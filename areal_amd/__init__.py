@@ -4,7 +4,13 @@ Importing the package does not load the HIP library; the first op call does, and
 raises ``NativeLibraryError`` if ``libareal_amd.so`` has not been built.
 """
 from .actor_ops import apply_m2po_masking, compute_prox_logp_approximations, distillation_terms
-from .advantages import Normalization, gae_advantages, kl_regularized_rewards, masked_moments
+from .advantages import (
+    Normalization,
+    gae_advantages,
+    kl_regularized_rewards,
+    masked_moments,
+    reward_overlong_penalty,
+)
 from .config import NormConfig, RejectionSamplingConfig
 from .functional import (
     RejectionSamplingResult,
@@ -56,6 +62,7 @@ __all__ = [
     "pad_packed_tensor_dict",
     "ppo_actor_loss_fn",
     "ppo_critic_loss_fn",
+    "reward_overlong_penalty",
     "sapo_loss_fn",
     "segment_copy",
     "tree_sequence_pairs",

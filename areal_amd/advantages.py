@@ -178,3 +178,28 @@ def kl_regularized_rewards(old_logp: torch.Tensor, ref_logp: torch.Tensor | None
             "aa_kl_rewards",
         )
     return rewards, kl_rewards
+
+
+@torch.no_grad()
+def reward_overlong_penalty(data: dict, overlong_tokens: int, overlong_penalty_factor: float,
+                            max_response_length: int) -> dict:
+    """Length penalty on the sequence rewards, in place on ``data["rewards"]`` like the reference
+    (areal/utils/functional/functional.py:782-803): a response longer than ``max_response_length - overlong_tokens``
+    loses ``overlong_penalty_factor`` per ``overlong_tokens`` tokens of excess.  ``data["loss_mask"]`` is ``[bs, L]``."""
+    rewards, mask = data["rewards"], data["loss_mask"]
+    _require_gpu(rewards, "rewards")
+    if mask.ndim != 2 or rewards.numel() != mask.shape[0]:
+        raise ValueError("rewards must have one entry per row of the [bs, max_seqlen] loss_mask")
+    bs, L = mask.shape
+    dev = rewards.device
+    r = rewards if (rewards.dtype == torch.float32 and rewards.is_contiguous()) else _f32(rewards).contiguous()
+    with torch.cuda.device(dev):
+        N.check(
+            N.load().aa_overlong_penalty(_ptr(r), _ptr(_f32(mask.to(dev)).contiguous()), bs, L, int(overlong_tokens),
+                                         float(overlong_penalty_factor), int(max_response_length), _stream(dev)),
+            "aa_overlong_penalty",
+        )
+    if r is not rewards:
+        rewards.copy_(r.view_as(rewards))
+    data["rewards"] = rewards
+    return data

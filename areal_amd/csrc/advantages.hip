@@ -356,6 +356,30 @@ __global__ __launch_bounds__(256) void k_kl_rewards(const float* __restrict__ ol
 }
 
 // ------------------------------------------------------------------------------------------------------------------
+// Length penalty on the sequence rewards (reward_overlong_penalty, areal/utils/functional/functional.py:782-803):
+// with len_b = long(sum of the row's loss mask), rewards[b] += min(-(len_b - (max_len - overlong)) / overlong * factor, 0),
+// the quotient and the product in float32 as the reference's tensor arithmetic.  One workgroup per sequence.
+// ------------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_overlong_penalty(float* __restrict__ rewards, const float* __restrict__ mask,
+                                                          int64_t L, int overlong_tokens, float factor,
+                                                          int64_t max_response_length) {
+  __shared__ float part[4];
+  const int64_t b = blockIdx.x;
+  float s = 0.f;
+  for (int64_t t = threadIdx.x; t < L; t += 256) s += mask[b * L + t];
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, kWave);
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int64_t len = (int64_t)((part[0] + part[1]) + (part[2] + part[3]));
+    const int64_t exceed = len - (max_response_length - overlong_tokens);
+    const float pen = ((float)(-exceed) / (float)overlong_tokens) * factor;
+    if (pen < 0.f) rewards[b] += pen;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------------------------
 // Masked moments of up to kMaxTensors per-token tensors under one mask: out[k] = {sum, min, max, count}
 // (min = +inf, max = -inf when nothing is selected).  One workgroup per tensor, fixed summation order.
 // ------------------------------------------------------------------------------------------------------------------
@@ -492,5 +516,15 @@ extern "C" int aa_kl_rewards(const float* old_logp, const float* ref_logp, const
   hipLaunchKernelGGL(k_kl_rewards, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, old_logp, ref_logp,
                      loss_mask, seqlens, reward_score, bs, L, kl_ctl, estimator, mask_no_eos_with_zero, rewards,
                      kl_rewards);
+  return launch_status();
+}
+
+extern "C" int aa_overlong_penalty(float* rewards, const float* loss_mask, int64_t bs, int64_t L, int overlong_tokens,
+                                   float overlong_penalty_factor, int64_t max_response_length, void* stream) {
+  if (bs < 0 || L < 1 || overlong_tokens == 0) return AA_ERR_INVALID_ARGUMENT;
+  if (bs == 0) return AA_OK;
+  if (!rewards || !loss_mask) return AA_ERR_INVALID_ARGUMENT;
+  hipLaunchKernelGGL(k_overlong_penalty, dim3((unsigned)bs), dim3(256), 0, (hipStream_t)stream, rewards, loss_mask, L,
+                     overlong_tokens, overlong_penalty_factor, max_response_length);
   return launch_status();
 }

@@ -98,15 +98,24 @@ def compute_advantages(
     mask_no_eos_with_zero: bool = False,
     use_decoupled_loss: bool = False,
     recompute_logprob: bool = False,
+    overlong_tokens: int | None = None,
+    overlong_penalty_factor: float | None = None,
+    max_new_tokens: int | None = None,
 ) -> dict[str, Any]:
     """``PPOActor._compute_advantages`` (areal/trainer/ppo/actor.py:145-250) on the GPU for one padded batch.
 
     ``data`` holds ``input_ids``, ``attention_mask``, ``loss_mask``, ``logprobs``, ``rewards`` as ``[bs, max_seqlen]``
     (``rewards`` is ``[bs]``) and optionally ``ref_logp``, ``values``, ``prox_logp``.  ``reward_norm`` / ``adv_norm``
     are ``Normalization`` objects or None.  Writes ``advantages``, ``returns``, ``kl_rewards``, ``tot_rewards``,
-    the rolled ``loss_mask`` and ``logprobs`` back into ``data`` and returns it, as the reference does.  The
-    overlong-reward penalty (a per-sample Python loop over scalars, functional.py:782-804) is left to the caller.
+    the rolled ``loss_mask`` and ``logprobs`` back into ``data`` and returns it, as the reference does.  With
+    ``overlong_tokens`` set (the reference's ``overlong_reward_penalty``), the length penalty of
+    ``reward_overlong_penalty`` is applied to ``data["rewards"]`` first, in place (actor.py:152-164).
     """
+    if overlong_tokens is not None:                                          # actor.py:152-164
+        from .advantages import reward_overlong_penalty
+
+        assert overlong_penalty_factor is not None and max_new_tokens is not None
+        data = reward_overlong_penalty(data, overlong_tokens, overlong_penalty_factor, max_new_tokens)
     reward_score = (data["rewards"] + reward_bias) * reward_scaling          # actor.py:166-170
     reward_score = torch.clip(reward_score, max=reward_clip, min=-reward_clip)
     if reward_norm is not None:

@@ -265,6 +265,17 @@ int aa_prox_logp_approx(const float* old_logp, const float* logp,
                         void* stream);
 
 /*
+ * reward_overlong_penalty (functional.py:782-803), in place on rewards [bs]:
+ *   len_b = (long) sum(loss_mask[b, :])           loss_mask [bs, L] float32
+ *   rewards[b] += min(-(len_b - (max_response_length - overlong_tokens))
+ *                     / overlong_tokens * overlong_penalty_factor, 0)
+ */
+int aa_overlong_penalty(float* rewards, const float* loss_mask, int64_t bs,
+                        int64_t L, int overlong_tokens,
+                        float overlong_penalty_factor,
+                        int64_t max_response_length, void* stream);
+
+/*
  * Per-token terms of the joint-distillation branch of grpo_loss_fn
  * (trainer/ppo/actor.py:482-511), with mask the bool loss mask as bytes:
  *   pure_distillation != 0 (rl_loss_weight == 0, :493-503):

@@ -157,10 +157,14 @@ def kl_rewards(old_logp, ref_logp, loss_mask, seqlens, reward_score, kl_ctl, kl_
 
 def compute_advantages(data, kl_ctl=0.0, kl_estimator="k1", discount=1.0, gae_lambda=1.0, reward_bias=0.0,
                        reward_scaling=1.0, reward_clip=20.0, reward_norm=None, adv_norm=None,
-                       mask_no_eos_with_zero=False, use_decoupled_loss=False, recompute_logprob=False):
+                       mask_no_eos_with_zero=False, use_decoupled_loss=False, recompute_logprob=False,
+                       overlong_tokens=None, overlong_penalty_factor=None, max_new_tokens=None):
     """PPOActor._compute_advantages, actor.py:145-250; ``reward_norm`` / ``adv_norm`` are kwargs dicts of
     ``normalization`` or None."""
     data = dict(data)
+    if overlong_tokens is not None:                                       # :152-164
+        data["rewards"] = data["rewards"].clone()
+        data = overlong_penalty(data, overlong_tokens, overlong_penalty_factor, max_new_tokens)
     reward_score = (data["rewards"] + reward_bias) * reward_scaling
     reward_score = torch.clip(reward_score, max=reward_clip, min=-reward_clip)
     if reward_norm is not None:
@@ -188,4 +192,21 @@ def compute_advantages(data, kl_ctl=0.0, kl_estimator="k1", discount=1.0, gae_la
     if adv_norm is not None:
         advantages = normalization(advantages, loss_mask, **adv_norm)
     data.update(advantages=advantages, kl_rewards=kl_rew, tot_rewards=rewards, loss_mask=loss_mask, logprobs=old_logp)
+    return data
+
+
+def overlong_penalty(data, overlong_tokens: int, overlong_penalty_factor: float, max_response_length: int):
+    """``reward_overlong_penalty``; areal/utils/functional/functional.py:782-803, statement by statement."""
+    reward_score = data["rewards"]
+    response_lengths = (data["loss_mask"].sum(dim=-1)).long()                       # :790
+    batch_size = data["input_ids"].shape[0]                                        # :791
+    for sample_idx in range(batch_size):                                           # :792
+        reward_score_cur = reward_score[sample_idx]
+        response_length_cur = response_lengths[sample_idx]
+        expected_len = max_response_length - overlong_tokens                       # :795
+        exceed_len = response_length_cur - expected_len                            # :796
+        overlong_reward = min(-exceed_len / overlong_tokens * overlong_penalty_factor, 0)   # :797-799
+        reward_score_cur += overlong_reward                                        # :800
+        reward_score[sample_idx] = reward_score_cur                                # :801
+    data["rewards"] = reward_score
     return data

@@ -170,7 +170,7 @@ def test_kl_rewards_match_oracle(device, est, no_eos_zero):
         areal_amd.kl_regularized_rewards(old.to(device), None, mask.to(device), seqlens.to(device), score.to(device), 0.1, "k9")
 
 
-@pytest.mark.parametrize("case", ["grpo", "critic_kl", "recompute"])
+@pytest.mark.parametrize("case", ["grpo", "critic_kl", "recompute", "overlong"])
 def test_compute_advantages_matches_oracle(device, case):
     from areal_amd.engine_glue import compute_advantages
 
@@ -192,6 +192,9 @@ def test_compute_advantages_matches_oracle(device, case):
         data["ref_logp"] = -torch.rand(bs, L, generator=g) * 2
         kw = dict(kl_ctl=0.1, kl_estimator="k3", discount=0.99, gae_lambda=0.95, mask_no_eos_with_zero=True,
                   use_decoupled_loss=True, adv_norm=dict(mean_level="batch", std_level=None, mean_leave1out=True))
+    elif case == "overlong":
+        kw = dict(overlong_tokens=16, overlong_penalty_factor=0.7, max_new_tokens=48,
+                  adv_norm=dict(mean_level="batch", std_level="batch"))
     else:
         data["prox_logp"] = -torch.rand(bs, L, generator=g) * 2
         kw = dict(recompute_logprob=True, use_decoupled_loss=False)
@@ -206,3 +209,17 @@ def test_compute_advantages_matches_oracle(device, case):
         assert float((got[key].cpu() - want[key]).abs().max()) < 2e-5 * scale, key
     if case != "critic_kl":
         assert torch.allclose(got["prox_logp"].cpu(), want["prox_logp"])
+
+
+def test_overlong_penalty_matches_oracle_and_updates_in_place(device):
+    g = torch.Generator().manual_seed(8)
+    bs, L = 37, 300
+    lens = torch.randint(1, L + 1, (bs,), generator=g)
+    mask = (torch.arange(L)[None, :] < lens[:, None]).float()
+    rewards = torch.randn(bs, generator=g)
+    want = O.overlong_penalty(dict(rewards=rewards.clone(), loss_mask=mask, input_ids=torch.zeros(bs, L)), 40, 1.3, 200)
+    r_dev = rewards.to(device)
+    data = dict(rewards=r_dev, loss_mask=mask.to(device), input_ids=torch.zeros(bs, L, device=device))
+    got = areal_amd.reward_overlong_penalty(data, 40, 1.3, 200)
+    assert got["rewards"] is r_dev and torch.equal(r_dev.cpu(), want["rewards"])
+    assert bool((want["rewards"] <= rewards).all()) and bool((want["rewards"] < rewards).any())

@@ -203,3 +203,15 @@ def test_compute_advantages_grpo_shape_by_hand():
     assert out["advantages"][1].tolist() == [-0.25, -0.25, 0.0, 0.0, 0.0, 0.0]
     assert torch.equal(out["returns"], out["advantages"]) and torch.equal(out["tot_rewards"][0, 3], torch.tensor(5.0))
     assert torch.equal(out["prox_logp"], torch.roll(data["logprobs"], -1, -1))
+
+
+def test_overlong_penalty_hand_cases():
+    """functional.py:782-803 has no test in the reference; the restatement is pinned by hand-computed cases of the
+    DAPO length penalty: nothing up to max_len - overlong tokens, then a linear ramp of factor per overlong tokens."""
+    L = 12
+    lens = [3, 6, 7, 9, 12]                     # max_len 10, overlong 4: expected length 6
+    mask = torch.tensor([[1.0] * n + [0.0] * (L - n) for n in lens])
+    data = dict(rewards=torch.tensor([1.0, 1.0, 1.0, -2.0, 0.5]), loss_mask=mask, input_ids=torch.zeros(5, L))
+    out = O.overlong_penalty(data, overlong_tokens=4, overlong_penalty_factor=2.0, max_response_length=10)
+    # excess 0, 0, 1, 3, 6 tokens -> penalty 0, 0, 0.5, 1.5, 3.0
+    assert torch.allclose(out["rewards"], torch.tensor([1.0, 1.0, 0.5, -3.5, -2.5]))
