@@ -11,6 +11,7 @@ from .advantages import (
     masked_moments,
     reward_overlong_penalty,
 )
+from .dpo import dpo_loss, dpo_pair_logratios, dpo_preference_loss
 from .config import NormConfig, RejectionSamplingConfig
 from .functional import (
     RejectionSamplingResult,
@@ -38,6 +39,9 @@ __version__ = "0.1.0"
 
 __all__ = [
     "NativeLibraryError",
+    "dpo_loss",
+    "dpo_pair_logratios",
+    "dpo_preference_loss",
     "NormConfig",
     "Normalization",
     "RejectionSamplingConfig",

@@ -53,6 +53,7 @@ _p = C.c_void_p
 _i64 = C.c_int64
 _f = C.c_float
 _i = C.c_int
+_d = C.c_double
 
 # name -> (restype, argtypes); must list every function of include/areal_amd.h
 SIGNATURES = {
@@ -86,6 +87,10 @@ SIGNATURES = {
     "aa_prox_logp_approx": (_i, [_p, _p, _p, _i64, _i, _i, _p, _p]),
     "aa_overlong_penalty": (_i, [_p, _p, _i64, _i64, _i, _f, _i64, _p]),
     "aa_kd_terms": (_i, [_p, _p, _p, _p, _i64, _i, _p, _p, _p]),
+    "aa_dpo_seq_sums": (_i, [_p, _p, _p, _p, _i64, _i64, _p, _p, _p, _p]),
+    "aa_dpo_seq_sums_bwd": (_i, [_p, _p, _p, _p, _i64, _i64, _p, _p]),
+    "aa_dpo_preference_loss": (_i, [_p, _i64, _d, _i, _p, _p, _p]),
+    "aa_dpo_pair_loss": (_i, [_p, _p, _p, _p, _i64, _d, _i, _p, _p, _p, _p, _p, _p, _p, _p]),
     "aa_m2po_workspace_bytes": (_i64, [_i64]),
     "aa_m2po_mask": (_i, [_p, _p, _p, _i64, _f, _p, _p, _p, _i64, _p]),
     "aa_kl_rewards": (_i, [_p, _p, _p, _p, _p, _i64, _i64, _f, _i, _i, _p, _p, _p]),

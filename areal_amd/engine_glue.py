@@ -318,3 +318,34 @@ def critic_loss_fn(value: torch.Tensor, input_data: dict[str, Any], eps_clip: fl
     reduced.update(masked_moments(dict(clipped_new_value=value.detach(), clipped_old_value=old_value), clip_mask))
     reduced["n_tokens"] = infer_token_denominator(input_data, value).numel()
     return loss, dict(stat, loss_mask=loss_mask, reduced=reduced)
+
+
+def dpo_valid_pairs(x: dict[str, Any]) -> torch.Tensor:
+    """Pairs whose chosen and rejected sequences are both non-empty (areal/trainer/dpo/dpo_engine.py:22-24)."""
+    seqlens = x["cu_seqlens"][1:] - x["cu_seqlens"][:-1]
+    return seqlens.view(-1, 2).ne(0).all(dim=1)
+
+
+def dpo_loss_weight(x: dict[str, Any]) -> torch.Tensor:
+    """Number of valid pairs as a float, the weight of a micro-batch (dpo_engine.py:27-28)."""
+    return dpo_valid_pairs(x).count_nonzero().float()
+
+
+def compute_dpo_loss(logprobs: torch.Tensor, entropy: torch.Tensor | None, input_: dict[str, Any], *, beta: float,
+                     loss_type: str = "sigmoid", vocab_min_logits: torch.Tensor | None = None,
+                     vocab_max_logits: torch.Tensor | None = None) -> tuple[torch.Tensor, dict]:
+    """The DPO loss function of one packed micro-batch (dpo_engine.py:147-213) on the GPU ops.
+
+    ``input_`` holds ``cu_seqlens``, ``loss_mask`` and ``ref_logprobs`` (``KeyError`` if one is missing), sequences
+    interleaved chosen / rejected.  Returns ``(loss, stat)``: the mean over the valid pairs (0 when there are none,
+    found on the device, without a read-back) and what the reference records per pair under its ``n_pairs``
+    denominator: ``loss``, ``chosen_reward``, ``rejected_reward``, ``reward_accuracy``, ``reward_margin``, with
+    ``valid_pairs`` selecting the pairs that count and ``n_pairs`` their number."""
+    from .dpo import dpo_loss
+
+    loss, stat = dpo_loss(logprobs, input_["ref_logprobs"], input_["cu_seqlens"], input_["loss_mask"], beta=beta,
+                          loss_type=loss_type)
+    with torch.no_grad():
+        stat["reward_accuracy"] = (stat["chosen_reward"] > stat["rejected_reward"]).float()
+        stat["reward_margin"] = stat["chosen_reward"] - stat["rejected_reward"]
+    return loss, stat

@@ -20,8 +20,8 @@ One "step" is one pass of the hot path over one synthetic packed micro-batch tha
   normalisation over a padded [512, 4096] batch.  Roofline: HBM, 20 bytes per token for the scan (rewards, values,
   mask read; advantages, returns written).
 
-* aux: the other per-token pieces around the loss at the configs[1] token count (SAPO loss, clipped value loss, M2PO
-  masking, proximal log-prob approximation) and the packing helpers (pack of a [512, 4096] batch, un-padding of
+* aux: the other per-token pieces around the loss at the configs[1] token count (SAPO loss, clipped value loss, DPO
+  loss over 32 pairs, M2PO masking, proximal log-prob approximation) and the packing helpers (pack of a [512, 4096] batch, un-padding of
   [32768 + pad, 151936] bf16 logits).  Roofline: HBM, on the logits un-padding copy (4 * V bytes per token).
 
 Prints ONE JSON line.  Besides the whole-step throughput it carries
@@ -649,8 +649,19 @@ def bench_aux(args, dev):
         loss, _ = areal_amd.ppo_critic_loss_fn(x, d["val"] * 0.9, d["tgt"], 0.2, d["mask"])
         loss.backward()
 
+    # DPO: the same tokens as 32 interleaved (chosen, rejected) pairs of random lengths
+    cuts = torch.sort(torch.randperm(T - 1, generator=g)[:63] + 1).values
+    dpo_cu = torch.cat([torch.zeros(1, dtype=torch.long), cuts, torch.tensor([T])]).to(torch.int32)
+    dpo_cu_d = dpo_cu.to(dev)
+
+    def dpo():
+        x = d["lp"].detach().requires_grad_(True)
+        loss, _ = areal_amd.dpo_loss(x, d["old"], dpo_cu_d, d["mask"], beta=0.1)
+        loss.backward()
+        return x, loss
+
     pieces = dict(
-        sapo_loss_fwd_bwd=sapo, critic_loss_fwd_bwd=critic,
+        sapo_loss_fwd_bwd=sapo, critic_loss_fwd_bwd=critic, dpo_loss_fwd_bwd=dpo,
         m2po_masking=lambda: areal_amd.apply_m2po_masking(d["old"], d["prox"], d["mask"], 0.002),
         prox_logp_loglinear=lambda: areal_amd.compute_prox_logp_approximations(d["old"], d["lp"], d["ver"], 6, "loglinear"),
     )
@@ -669,6 +680,14 @@ def bench_aux(args, dev):
     g_loss.backward()
     m2_gpu = areal_amd.apply_m2po_masking(d["old"], d["prox"], d["mask"], 0.002).cpu()
     m2_cpu = OS.m2po_mask(old, prox, mask, 0.002)
+    from oracle import dpo as OD
+
+    xd = lp.clone().requires_grad_(True)
+    t0 = time.perf_counter()
+    wd_loss, _ = OD.compute_dpo_loss(xd, old, dpo_cu, mask, 0.1)
+    wd_loss.backward()
+    cpu_dpo_s = time.perf_counter() - t0
+    yd, gd_loss = dpo()
 
     # packing: a padded batch, and the logits of an aligned + page-padded micro-batch
     bs, S, V = 512, 4096, 151936
@@ -707,11 +726,13 @@ def bench_aux(args, dev):
                           sample=f"un-padding of the first 8 sequences ({cpu_rows.shape[0]} tokens) with the per-sequence "
                                  f"slice loop of the CPU oracle"),
         per_token_pieces=out_pieces, pack_tensor_dict_ms=pack_ms,
-        cpu_sapo_plus_m2po_s=cpu_sib_s,
+        cpu_sapo_plus_m2po_s=cpu_sib_s, cpu_dpo_loss_fwd_bwd_s=cpu_dpo_s,
         parity=dict(unpad_rows_equal=bool(torch.equal(got_rows, cpu_rows)),
                     sapo_loss_rel_err=abs(float(g_loss.detach()) - float(w_loss.detach())) / abs(float(w_loss.detach())),
                     sapo_grad_cosine=cosine(y.grad.cpu(), x.grad),
-                    m2po_mask_mismatches=int((m2_gpu != m2_cpu).sum())),
+                    m2po_mask_mismatches=int((m2_gpu != m2_cpu).sum()),
+                    dpo_loss_rel_err=abs(float(gd_loss.detach()) - float(wd_loss.detach())) / abs(float(wd_loss.detach())),
+                    dpo_grad_cosine=cosine(yd.grad.cpu(), xd.grad)),
     )
 
 

@@ -294,6 +294,65 @@ int aa_kd_terms(const float* logp, const float* old_logp,
                 int pure_distillation, float* term, float* dterm,
                 void* stream);
 
+/*
+ * Direct preference optimisation over a packed batch whose sequences are
+ * interleaved [chosen_0, rejected_0, chosen_1, rejected_1, ...].
+ *
+ * aa_dpo_seq_sums: the per-sequence aggregation of dpo_pair_logratios
+ * (areal/utils/functional/functional.py:641-687) before the pairing view.
+ * loss_mask [T] bytes, cu_seqlens [n_seqs + 1] int32 on the device.  With
+ * shifted[t] = loss_mask[t + 1] inside a sequence and 0 at its last position:
+ *   policy_sums[s]     = sum_t (double)(logp[t] * shifted[t])
+ *   ref_sums[s]        = sum_t (double)(ref_logp[t] * shifted[t])
+ *   completion_lens[s] = sum_t shifted[t]
+ * all fp64, each summed in a fixed order (the reference's index_add_ has
+ * none).  An empty sequence gives zeros.
+ */
+int aa_dpo_seq_sums(const float* logp, const float* ref_logp,
+                    const uint8_t* loss_mask, const int32_t* cu_seqlens,
+                    int64_t n_seqs, int64_t T, double* policy_sums,
+                    double* ref_sums, double* completion_lens, void* stream);
+
+/*
+ * Backward of aa_dpo_seq_sums in logp (what autograd derives for
+ * functional.py:671-673): d_logp[t] = (float)(g_policy_sums[s(t)] * scale[0])
+ * * shifted[t]; scale (device, one float) may be NULL for 1.  Tokens outside
+ * every sequence get 0.
+ */
+int aa_dpo_seq_sums_bwd(const double* g_policy_sums, const float* scale,
+                        const uint8_t* loss_mask, const int32_t* cu_seqlens,
+                        int64_t n_seqs, int64_t T, float* d_logp,
+                        void* stream);
+
+/*
+ * dpo_preference_loss (functional.py:689-703) on logits already cast to
+ * float32 (the reference's first step): loss_type 0 ("sigmoid")
+ * loss = -logsigmoid(beta * x); 1 ("ipo") loss = (x - 1 / (2 beta))^2.
+ * dloss = d loss / d x, may be NULL.
+ */
+int aa_dpo_preference_loss(const float* logits, int64_t n, double beta,
+                           int loss_type, float* loss, float* dloss,
+                           void* stream);
+
+/*
+ * The rest of compute_dpo_loss (areal/trainer/dpo/dpo_engine.py:147-213) from
+ * the per-sequence sums, for n_pairs = n_seqs / 2 pairs: a pair is valid when
+ * both of its sequences are non-empty (_dpo_valid_pairs, :22-24); its logit is
+ * (policy_c - policy_r) - (ref_c - ref_r) for loss_type 0 and the difference
+ * of the per-token averages (policy - ref) / max(len, 1) for loss_type 1, in
+ * fp64, then the loss above in float32.  loss_mean[0] = mean over the valid
+ * pairs (0 when there are none), n_valid[0] their number; per pair
+ * pair_loss, chosen_reward = beta * (policy_c - ref_c), rejected_reward, valid
+ * (zeros for an invalid pair); g_policy_sums [2 * n_pairs] =
+ * d loss_mean / d policy_sums.
+ */
+int aa_dpo_pair_loss(const double* policy_sums, const double* ref_sums,
+                     const double* completion_lens, const int32_t* cu_seqlens,
+                     int64_t n_pairs, double beta, int loss_type,
+                     float* loss_mean, int32_t* n_valid, float* pair_loss,
+                     float* chosen_reward, float* rejected_reward,
+                     uint8_t* valid, double* g_policy_sums, void* stream);
+
 /* Bytes of 256-byte aligned workspace aa_m2po_mask needs for n tokens. */
 int64_t aa_m2po_workspace_bytes(int64_t n);
 
