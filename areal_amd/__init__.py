@@ -9,6 +9,7 @@ from .advantages import (
     gae_advantages,
     kl_regularized_rewards,
     masked_moments,
+    masked_normalization,
     reward_overlong_penalty,
 )
 from .dpo import dpo_loss, dpo_pair_logratios, dpo_preference_loss
@@ -39,6 +40,7 @@ __version__ = "0.1.0"
 
 __all__ = [
     "NativeLibraryError",
+    "masked_normalization",
     "dpo_loss",
     "dpo_pair_logratios",
     "dpo_preference_loss",

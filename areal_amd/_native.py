@@ -85,6 +85,8 @@ SIGNATURES = {
     "aa_sapo_loss": (_i, [_p, _p, _p, _p, _i64, _p, _i64, _i, _f, _f, _p, _p, _p, _p, _p, _p]),
     "aa_critic_loss": (_i, [_p, _p, _p, _p, _i64, _f, _i, _p, _p, _p, _p, _p]),
     "aa_prox_logp_approx": (_i, [_p, _p, _p, _i64, _i, _i, _p, _p]),
+    "aa_masked_normalization_scratch_bytes": (_i64, [_i64, _i64]),
+    "aa_masked_normalization": (_i, [_p, _p, _i64, _i64, _i, _d, _p, _p, _i64, _p]),
     "aa_overlong_penalty": (_i, [_p, _p, _i64, _i64, _i, _f, _i64, _p]),
     "aa_kd_terms": (_i, [_p, _p, _p, _p, _i64, _i, _p, _p, _p]),
     "aa_dpo_seq_sums": (_i, [_p, _p, _p, _p, _i64, _i64, _p, _p, _p, _p]),

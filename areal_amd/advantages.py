@@ -203,3 +203,45 @@ def reward_overlong_penalty(data: dict, overlong_tokens: int, overlong_penalty_f
         rewards.copy_(r.view_as(rewards))
     data["rewards"] = rewards
     return data
+
+
+@torch.no_grad()
+def masked_normalization(x: torch.Tensor, mask: torch.Tensor | None = None, dim=None, unbiased: bool = False,
+                         eps: float = 1e-5, high_precision: bool = True, all_reduce: bool = True,
+                         reduce_group=None) -> torch.Tensor:
+    """Whitening by the masked mean and the ``E[x^2] - E[x]^2`` variance over ``dim`` (all axes when None);
+    areal/utils/functional/functional.py:16-53.  Masked positions enter as zeros and are whitened like the rest, as
+    in the reference.  Returns float32 of the shape of ``x``.
+
+    Sums are accumulated in float64 whatever ``high_precision`` says.  The sums are local: with an initialised
+    process group of more than one rank and ``all_reduce=True`` the call raises ``NotImplementedError``."""
+    import torch.distributed as dist
+
+    _require_gpu(x, "x")
+    if all_reduce and dist.is_available() and dist.is_initialized() and dist.get_world_size(reduce_group) > 1:
+        raise NotImplementedError("masked_normalization sums over one GPU only")
+    nd = x.dim()
+    dims = tuple(range(nd)) if dim is None else tuple(sorted(d % nd for d in ((dim,) if isinstance(dim, int) else dim)))
+    keep = [d for d in range(nd) if d not in dims]
+    perm = keep + list(dims)
+    xv = _f32(x).permute(perm).contiguous()
+    mv = None
+    if mask is not None:
+        mv = _f32(mask.to(x.device)).expand(x.shape).permute(perm).contiguous()
+    rows = 1
+    for d in keep:
+        rows *= x.shape[d]
+    cols = xv.numel() // rows if rows else 0
+    out = torch.empty_like(xv)
+    if xv.numel():
+        lib = N.load()
+        dev = x.device
+        scratch = torch.empty(lib.aa_masked_normalization_scratch_bytes(rows, cols), dtype=torch.uint8, device=dev)
+        with torch.cuda.device(dev):
+            N.check(lib.aa_masked_normalization(_ptr(xv), _ptr(mv), rows, cols, 1 if unbiased else 0, float(eps),
+                                                _ptr(out), _ptr(scratch), scratch.numel(), _stream(dev)),
+                    "aa_masked_normalization")
+    inv = [0] * nd
+    for i, d in enumerate(perm):
+        inv[d] = i
+    return out.permute(inv).contiguous()

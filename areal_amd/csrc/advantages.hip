@@ -427,6 +427,89 @@ __global__ __launch_bounds__(kThreads) void k_masked_moments(MomentArgs a, const
   }
 }
 
+// ------------------------------------------------------------------------------------------------------------------
+// masked_normalization (areal/utils/functional/functional.py:16-53): every row of an [R, C] view is whitened by
+// the mean and the E[x^2] - E[x]^2 variance of its masked values.  A row is cut into `parts` slices, one workgroup
+// each; the second launch adds the slices of its row in a fixed order and writes the result.
+// ------------------------------------------------------------------------------------------------------------------
+struct MnPartial {
+  double s, q, f;
+};
+
+__host__ __device__ inline int mn_parts(int64_t R, int64_t C) {
+  int64_t parts = (C + 8191) / 8192;                     // at least 8192 values per workgroup
+  const int64_t want = (1024 + R - 1) / (R > 0 ? R : 1); // about 1024 workgroups in all
+  if (parts > want) parts = want;
+  if (parts > 256) parts = 256;
+  return parts < 1 ? 1 : (int)parts;
+}
+
+__device__ __forceinline__ void mn_slice(int64_t C, int parts, int part, int64_t& b, int64_t& e) {
+  const int64_t per = (C + parts - 1) / parts;
+  b = (int64_t)part * per;
+  e = b + per < C ? b + per : C;
+  if (b > e) b = e;
+}
+
+__global__ __launch_bounds__(kThreads) void k_mn_partial(const float* __restrict__ x, const float* __restrict__ mask,
+                                                         int64_t C, int parts, MnPartial* __restrict__ partial) {
+  __shared__ double smem[kThreads / kWave];
+  const int64_t row = blockIdx.x / parts;
+  int64_t b, e;
+  mn_slice(C, parts, blockIdx.x % parts, b, e);
+  const float* xr = x + row * C;
+  const float* mr = mask ? mask + row * C : nullptr;
+  double s = 0.0, q = 0.0, f = 0.0;
+  for (int64_t i = b + threadIdx.x; i < e; i += kThreads) {
+    const double m = mr ? (double)mr[i] : 1.0;
+    const double v = (double)xr[i] * m;
+    s += v;
+    q += v * v;
+    f += m;
+  }
+  s = block_sum<double>(s, smem);
+  q = block_sum<double>(q, smem);
+  f = block_sum<double>(f, smem);
+  if (threadIdx.x == 0) partial[blockIdx.x] = MnPartial{s, q, f};
+}
+
+__global__ __launch_bounds__(kThreads) void k_mn_apply(const float* __restrict__ x, const float* __restrict__ mask,
+                                                       int64_t C, int parts, const MnPartial* __restrict__ partial,
+                                                       int unbiased, double eps, float* __restrict__ out) {
+  __shared__ double stat[2];
+  const int64_t row = blockIdx.x / parts;
+  if (threadIdx.x < kWave) {  // parts <= 256: lane l adds slices l, l + 64, ... in order, then a fixed butterfly
+    double s = 0.0, q = 0.0, f = 0.0;
+    for (int p = threadIdx.x; p < parts; p += kWave) {
+      const MnPartial v = partial[row * parts + p];
+      s += v.s;
+      q += v.q;
+      f += v.f;
+    }
+    s = wave_sum(s);
+    q = wave_sum(q);
+    f = wave_sum(f);
+    if (threadIdx.x == 0) {
+      const double mean = s / f;
+      double var = q / f - mean * mean;
+      if (unbiased) var *= f / (f - 1.0);
+      stat[0] = mean;
+      stat[1] = sqrt(var) + eps;
+    }
+  }
+  __syncthreads();
+  const double mean = stat[0], den = stat[1];
+  int64_t b, e;
+  mn_slice(C, parts, blockIdx.x % parts, b, e);
+  const float* xr = x + row * C;
+  const float* mr = mask ? mask + row * C : nullptr;
+  float* o = out + row * C;
+  for (int64_t i = b + threadIdx.x; i < e; i += kThreads) {
+    const double v = (double)xr[i] * (mr ? (double)mr[i] : 1.0);
+    o[i] = (float)((v - mean) / den);
+  }
+}
+
 }  // namespace adv
 }  // namespace aa
 
@@ -526,5 +609,26 @@ extern "C" int aa_overlong_penalty(float* rewards, const float* loss_mask, int64
   if (!rewards || !loss_mask) return AA_ERR_INVALID_ARGUMENT;
   hipLaunchKernelGGL(k_overlong_penalty, dim3((unsigned)bs), dim3(256), 0, (hipStream_t)stream, rewards, loss_mask, L,
                      overlong_tokens, overlong_penalty_factor, max_response_length);
+  return launch_status();
+}
+
+extern "C" int64_t aa_masked_normalization_scratch_bytes(int64_t rows, int64_t cols) {
+  if (rows < 0 || cols < 0) return -1;
+  return rows * mn_parts(rows, cols) * (int64_t)sizeof(MnPartial);
+}
+
+extern "C" int aa_masked_normalization(const float* x, const float* mask, int64_t rows, int64_t cols, int unbiased,
+                                       double eps, float* out, void* scratch, int64_t scratch_bytes, void* stream) {
+  if (rows < 0 || cols < 0) return AA_ERR_INVALID_ARGUMENT;
+  if (rows == 0 || cols == 0) return AA_OK;
+  const int parts = mn_parts(rows, cols);
+  if (!x || !out || !scratch || scratch_bytes < rows * parts * (int64_t)sizeof(MnPartial) ||
+      rows * parts > 0x7fffffff)
+    return AA_ERR_INVALID_ARGUMENT;
+  hipStream_t st = (hipStream_t)stream;
+  MnPartial* partial = (MnPartial*)scratch;
+  const unsigned grid = (unsigned)(rows * parts);
+  hipLaunchKernelGGL(k_mn_partial, dim3(grid), dim3(kThreads), 0, st, x, mask, cols, parts, partial);
+  hipLaunchKernelGGL(k_mn_apply, dim3(grid), dim3(kThreads), 0, st, x, mask, cols, parts, partial, unbiased, eps, out);
   return launch_status();
 }

@@ -603,6 +603,9 @@ def bench_adv(args, dev):
     w_adv, _ = O.gae(rewards, values, mask, no_eos.float(), 1.0, 0.95)
     w_out = O.normalization(w_adv, mask)
     cpu_s = time.perf_counter() - t0
+    # masked_normalization of the same batch over all axes: 12 bytes per value read twice + 4 written
+    mn_ms, _ = time_events(lambda: areal_amd.masked_normalization(d[0], d[2]), max(args.steps, 10), stream)
+    mn_err = float((areal_amd.masked_normalization(d[0], d[2]).cpu() - O.masked_normalization(rewards, mask)).abs().max())
     return dict(
         metric="tokens/sec for GAE + advantage normalisation", value=bs * L / (ms_per_step * 1e-3), unit="tokens/s",
         n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=ms_per_step, higher_is_better=True,
@@ -616,8 +619,10 @@ def bench_adv(args, dev):
         cpu_baseline=dict(value=bs * L / cpu_s, unit="tokens/s", cores=torch.get_num_threads(), kind="port",
                           sample="the whole workload once: the reference's Python loop over max_seqlen (4095 steps "
                                  "of [512]-wide tensor ops) and Normalization, restated in the CPU oracle"),
+        masked_normalization_ms=mn_ms,
         parity=dict(adv_max_abs_err=float((out.cpu() - w_out).abs().max()),
-                    returns_max_abs_err=float((ret.cpu() - (w_adv + values)).abs().max())),
+                    returns_max_abs_err=float((ret.cpu() - (w_adv + values)).abs().max()),
+                    masked_normalization_max_abs_err=mn_err),
     )
 
 def bench_aux(args, dev):

@@ -264,6 +264,24 @@ int aa_prox_logp_approx(const float* old_logp, const float* logp,
                         int current_version, int method, float* out,
                         void* stream);
 
+/* Bytes of 256-byte aligned scratch aa_masked_normalization needs. */
+int64_t aa_masked_normalization_scratch_bytes(int64_t rows, int64_t cols);
+
+/*
+ * masked_normalization (areal/utils/functional/functional.py:16-53) over the
+ * last axis of an [rows, cols] view (the reference's `dim` axes brought to the
+ * back; dim=None is rows = 1).  mask float32 of the same shape or NULL.  With
+ * v = x * mask, F = sum(mask) (cols when mask is NULL), per row in float64:
+ *   mean = sum(v) / F, var = sum(v^2) / F - mean^2, var *= F / (F - 1) when
+ *   unbiased != 0; out = (float)((v - mean) / (sqrt(var) + eps)).
+ * Masked positions are whitened as zeros, as in the reference.  Sums are
+ * always float64 (the reference's high_precision=True), in a fixed order.
+ * The reference's all-reduce over a process group is not part of this call.
+ */
+int aa_masked_normalization(const float* x, const float* mask, int64_t rows,
+                            int64_t cols, int unbiased, double eps, float* out,
+                            void* scratch, int64_t scratch_bytes, void* stream);
+
 /*
  * reward_overlong_penalty (functional.py:782-803), in place on rewards [bs]:
  *   len_b = (long) sum(loss_mask[b, :])           loss_mask [bs, L] float32

@@ -210,3 +210,28 @@ def overlong_penalty(data, overlong_tokens: int, overlong_penalty_factor: float,
         reward_score[sample_idx] = reward_score_cur                                # :801
     data["rewards"] = reward_score
     return data
+
+
+def masked_normalization(x, mask=None, dim=None, unbiased=False, eps=1e-5, high_precision=True):
+    """areal/utils/functional/functional.py:16-53 on one process (the all-reduce of the three sums left out)."""
+    dtype = torch.float64 if high_precision else torch.float32
+    x = x.to(dtype)
+    if dim is None:
+        dim = tuple(range(len(x.shape)))
+    if mask is None:
+        n = 1
+        for d in (dim if isinstance(dim, (tuple, list)) else (dim,)):
+            n *= x.shape[d]
+        factor = torch.tensor(n, dtype=dtype)                                      # :31-33
+    else:
+        mask = mask.to(dtype)
+        x = x * mask                                                               # :36
+        factor = mask.sum(dim, keepdim=True)                                       # :37
+    x_sum = x.sum(dim=dim, keepdim=True)
+    x_sum_sq = x.square().sum(dim=dim, keepdim=True)
+    mean = x_sum / factor                                                          # :48
+    meansq = x_sum_sq / factor
+    var = meansq - mean ** 2                                                       # :50
+    if unbiased:
+        var = var * (factor / (factor - 1))                                        # :51-52
+    return ((x - mean) / (var.sqrt() + eps)).float()                               # :53

@@ -223,3 +223,28 @@ def test_overlong_penalty_matches_oracle_and_updates_in_place(device):
     got = areal_amd.reward_overlong_penalty(data, 40, 1.3, 200)
     assert got["rewards"] is r_dev and torch.equal(r_dev.cpu(), want["rewards"])
     assert bool((want["rewards"] <= rewards).all()) and bool((want["rewards"] < rewards).any())
+
+
+@pytest.mark.parametrize("shape,dim", [((2_000_003,), None), ((64, 4096), None), ((64, 4096), 1), ((64, 4096), 0),
+                                       ((5, 7, 33), (0, 2)), ((3, 1), None), ((1,), None)])
+@pytest.mark.parametrize("masked,unbiased", [(False, False), (True, True), (True, False)])
+def test_masked_normalization_matches_oracle(device, shape, dim, masked, unbiased):
+    g = torch.Generator().manual_seed(13)
+    x = torch.randn(shape, generator=g) * 3 + 1.5
+    mask = (torch.rand(shape, generator=g) < 0.7) if masked else None
+    want = O.masked_normalization(x, mask, dim, unbiased, 1e-5)
+    got = areal_amd.masked_normalization(x.to(device), None if mask is None else mask.to(device), dim, unbiased, 1e-5)
+    assert got.dtype == torch.float32 and got.shape == x.shape
+    # a single value (or a single selected value with Bessel's correction) divides by zero in both
+    assert torch.allclose(got.cpu(), want, rtol=1e-5, atol=1e-6, equal_nan=True)
+
+
+def test_masked_normalization_weights_and_broadcast_mask(device):
+    g = torch.Generator().manual_seed(14)
+    x = torch.randn(16, 300, generator=g)
+    w = torch.rand(16, 1, generator=g)                      # a float mask that broadcasts over the row
+    want = O.masked_normalization(x, w.expand_as(x), 1, False, 1e-3)
+    got = areal_amd.masked_normalization(x.to(device), w.to(device), dim=1, eps=1e-3)
+    assert torch.allclose(got.cpu(), want, rtol=1e-5, atol=1e-6)
+    got16 = areal_amd.masked_normalization(x.to(device).bfloat16(), None, dim=-1)
+    assert torch.allclose(got16.cpu(), O.masked_normalization(x.bfloat16(), None, 1), rtol=1e-5, atol=1e-6)

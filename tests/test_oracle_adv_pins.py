@@ -215,3 +215,36 @@ def test_overlong_penalty_hand_cases():
     out = O.overlong_penalty(data, overlong_tokens=4, overlong_penalty_factor=2.0, max_response_length=10)
     # excess 0, 0, 1, 3, 6 tokens -> penalty 0, 0, 0.5, 1.5, 3.0
     assert torch.allclose(out["rewards"], torch.tensor([1.0, 1.0, 0.5, -3.5, -2.5]))
+
+
+def test_masked_normalization_against_numpy_moments():
+    """No test of the reference covers functional.py:16-53; pinned by numpy's mean / std (with and without Bessel's
+    correction) over the selection, by hand values, and by the fate of masked positions (whitened as zeros)."""
+    from oracle.advantages import masked_normalization
+
+    rng = np.random.default_rng(4)
+    x = rng.normal(2.0, 3.0, (6, 50))
+    t = torch.tensor(x)
+    # no mask, all axes: numpy mean and population / sample std
+    for unbiased, ddof in ((False, 0), (True, 1)):
+        got = masked_normalization(t, None, None, unbiased, 1e-5).numpy()
+        want = (x - x.mean()) / (x.std(ddof=ddof) + 1e-5)
+        assert got.dtype == np.float32 and np.allclose(got, want, rtol=1e-6, atol=1e-6)
+    # hand value: [1, 2, 3, 4] -> mean 2.5, population std sqrt(1.25)
+    got = masked_normalization(torch.tensor([1.0, 2.0, 3.0, 4.0]), eps=0.0).tolist()
+    assert np.allclose(got, [(v - 2.5) / math.sqrt(1.25) for v in (1, 2, 3, 4)], rtol=1e-6)
+    # mask, per row (dim=1): moments over the selected entries; masked entries are whitened as zeros
+    m = rng.random((6, 50)) < 0.6
+    got = masked_normalization(t, torch.tensor(m), 1, True, 1e-5).numpy()
+    for r in range(6):
+        sel = x[r][m[r]]
+        mean, std = sel.mean(), sel.std(ddof=1)
+        assert np.allclose(got[r][m[r]], (sel - mean) / (std + 1e-5), rtol=1e-5, atol=1e-6)
+        assert np.allclose(got[r][~m[r]], (0.0 - mean) / (std + 1e-5), rtol=1e-5, atol=1e-6)
+    # a float mask weighs the entries: v = x * w, F = sum(w)
+    w = rng.random(50)
+    got = masked_normalization(t[0], torch.tensor(w), None, False, 0.0).numpy()
+    v = x[0] * w
+    mean = v.sum() / w.sum()
+    var = (v * v).sum() / w.sum() - mean * mean
+    assert np.allclose(got, (v - mean) / math.sqrt(var), rtol=1e-5, atol=1e-6)
