@@ -3,7 +3,12 @@
 Importing the package does not load the HIP library; the first op call does, and
 raises ``NativeLibraryError`` if ``libareal_amd.so`` has not been built.
 """
-from .actor_ops import apply_m2po_masking, compute_prox_logp_approximations, distillation_terms
+from .actor_ops import (
+    apply_m2po_masking,
+    compute_prox_logp_approximations,
+    distillation_terms,
+    proximal_logging_stats,
+)
 from .advantages import (
     Normalization,
     gae_advantages,
@@ -40,6 +45,7 @@ __version__ = "0.1.0"
 
 __all__ = [
     "NativeLibraryError",
+    "proximal_logging_stats",
     "masked_normalization",
     "dpo_loss",
     "dpo_pair_logratios",

@@ -5,6 +5,8 @@ Host-side mirror of ``compute_prox_logp_approximations`` (areal/trainer/ppo/acto
 """
 from __future__ import annotations
 
+from typing import Any
+
 import torch
 
 from . import _native as N
@@ -123,3 +125,77 @@ def distillation_terms(logprobs: torch.Tensor, old_logp: torch.Tensor | None, te
     mean, term = _KdTerms.apply(lp, old, _f32(teacher_logp.detach()).reshape(-1), _mask_u8(loss_mask).reshape(-1),
                                 bool(pure))
     return mean, term.view(shape)
+
+
+_LOGSTAT_METHOD_KEYS = ("approx_logp", "behave_imp_weight", "importance_weight", "abs_error", "rel_error",
+                        "squared_error", "behave_imp_weight_abs_error", "behave_imp_weight_rel_error",
+                        "importance_weight_abs_error", "importance_weight_rel_error")
+
+
+def _moment_rows(table: torch.Tensor) -> list[dict[str, torch.Tensor]]:
+    """``[rows, 4]`` of {sum, min, max, count} -> one dict of 0-d tensors per row, with one division for all rows."""
+    cols = torch.cat([table, (table[:, 0] / table[:, 3])[:, None]], dim=1)
+    rows = []
+    for row in cols.unbind(0):
+        s, lo, hi, c, avg = row.unbind(0)
+        rows.append(dict(sum=s, avg=avg, min=lo, max=hi, count=c))
+    return rows
+
+
+@torch.no_grad()
+def proximal_logging_stats(old_logp: torch.Tensor, logprobs: torch.Tensor, prox_logp_gt: torch.Tensor | None,
+                           versions: torch.Tensor | None, current_version: int | None, mask: torch.Tensor,
+                           prox_logp_method: str = "recompute") -> dict[str, dict]:
+    """What ``grpo_loss_fn`` logs under its ``compute_logp`` and ``version_stats`` scopes (actor.py:573-594,
+    982-1110), already reduced over ``mask``: one pass over the tokens instead of one tensor and one reduction per
+    logged quantity.
+
+    Returns ``{"compute_logp": {name: moments}, "version_stats": {...}}`` with ``moments`` = ``{"sum", "avg", "min",
+    "max", "count"}`` of 0-d device tensors.  The names and the conditions under which each appears are the
+    reference's: ``prox_logp_gt`` whenever it is given; nothing more without ``versions`` / ``current_version``;
+    ``loglinear/{approx_logp, behave_imp_weight, importance_weight}`` for the ``"loglinear"`` method; all three
+    methods with their error metrics for ``"metrics"`` with ground truth; ``kl_div_direct / taylor / dual``.
+    ``version_stats`` holds ``sample_staleness_proximal``, ``sample_staleness_theta`` (moments over the selected
+    tokens with ``version >= 0``; ``count`` is ``n_valid_generated_tokens``), ``v_theta`` and ``v_proximal``; it
+    is empty without versions.  Nothing is read back: whether any generated token is selected is the ``count``.
+    """
+    _require_gpu(old_logp, "old_logp")
+    lo = _f32(old_logp.detach()).reshape(-1)
+    ln = _f32(logprobs.detach()).reshape(-1)
+    m8 = _mask_u8(mask.to(lo.device)).reshape(-1)
+    n = lo.numel()
+    if ln.numel() != n or m8.numel() != n:
+        raise ValueError("old_logp, logprobs and mask must have the same number of elements")
+    gt = _f32(prox_logp_gt.detach()).reshape(-1) if prox_logp_gt is not None else None
+    have_versions = versions is not None and current_version is not None
+    ver = versions.to(device=lo.device, dtype=torch.int32).contiguous().reshape(-1) if have_versions else None
+    methods, with_errors = 0, False
+    if have_versions and prox_logp_method == "loglinear":
+        methods = 1
+    elif have_versions and prox_logp_method == "metrics" and gt is not None:
+        methods, with_errors = 7, True
+    lib = N.load()
+    dev = lo.device
+    out = torch.empty(36, 4, dtype=torch.float32, device=dev)
+    scratch = torch.empty(lib.aa_logging_stats_scratch_bytes(n), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        N.check(lib.aa_logging_stats(_ptr(lo), _ptr(ln), _ptr(gt), _ptr(ver), _ptr(m8), n,
+                                     int(current_version) if have_versions else 0, methods, 1 if with_errors else 0,
+                                     _ptr(out), _ptr(scratch), scratch.numel(), _stream(dev)), "aa_logging_stats")
+    rows = _moment_rows(out)
+    compute_logp: dict[str, dict] = {}
+    if gt is not None:
+        compute_logp["prox_logp_gt"] = rows[0]
+    version_stats: dict[str, Any] = {}
+    if have_versions:
+        for m, name in enumerate(PROX_APPROX_METHODS_ALL):
+            if not (methods >> m) & 1:
+                continue
+            for j, key in enumerate(_LOGSTAT_METHOD_KEYS[: 10 if with_errors else 3]):
+                compute_logp[f"{name}/{key}"] = rows[4 + 10 * m + j]
+        for j, key in enumerate(("kl_div_direct", "kl_div_taylor", "kl_div_dual")):
+            compute_logp[key] = rows[1 + j]
+        version_stats = dict(sample_staleness_proximal=rows[34],
+                             sample_staleness_theta=rows[35],
+                             v_theta=int(current_version), v_proximal=int(current_version) - 1)
+    return dict(compute_logp=compute_logp, version_stats=version_stats)

@@ -453,21 +453,9 @@ __global__ __launch_bounds__(256) void k_critic_loss(const float* __restrict__ v
 __global__ __launch_bounds__(256) void k_prox_approx(const float* __restrict__ old, const float* __restrict__ logp,
                                                      const int32_t* __restrict__ versions, int64_t n,
                                                      int current_version, int method, float* __restrict__ out) {
-  const float v_theta = (float)current_version, v_prox = (float)(current_version - 1);
   const int64_t step = (int64_t)gridDim.x * 256;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += step) {
-    const int ver = versions[i];
-    const float vb = (float)ver;
-    const float diff = v_theta - vb, gap = v_prox - vb;
-    float alpha = (diff > 0.f && ver >= 0) ? gap / diff : 0.f;
-    alpha = fminf(fmaxf(alpha, 0.f), 1.f);
-    const float lo = old[i], ln = logp[i];
-    float r;
-    if (method == 0) r = lo + alpha * (ln - lo);
-    else if (method == 1) r = logf((1.f - alpha) * expf(lo) + alpha * expf(ln) + 1e-10f);
-    else r = lo;
-    out[i] = r;
-  }
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += step)
+    out[i] = prox_approx_value(old[i], logp[i], versions[i], current_version, method);
 }
 
 // ---- joint-distillation terms of the actor loss (actor.py:482-511) ------------------------------------------------

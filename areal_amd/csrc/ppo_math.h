@@ -21,6 +21,21 @@ struct Surrogate {
 __device__ __forceinline__ float nan_max(float a, float b) { return (a != a || b != b) ? (a + b) : fmaxf(a, b); }
 __device__ __forceinline__ float nan_min(float a, float b) { return (a != a || b != b) ? (a + b) : fminf(a, b); }
 
+// Proximal log-prob approximated from the behaviour and the current log-prob of a token sampled by policy version
+// `ver` (negative for prompt tokens), areal/trainer/ppo/actor.py:604-684: alpha = (v_prox - v_behave) /
+// (v_theta - v_behave) clamped to [0, 1], 0 for prompt tokens; method 0 interpolates the log-probs, 1 the
+// probabilities, 2 returns the behaviour log-prob.
+__device__ __forceinline__ float prox_approx_value(float lo, float ln, int ver, int current_version, int method) {
+  const float v_theta = (float)current_version, v_prox = (float)(current_version - 1);
+  const float vb = (float)ver;
+  const float diff = v_theta - vb, gap = v_prox - vb;
+  float alpha = (diff > 0.f && ver >= 0) ? gap / diff : 0.f;
+  alpha = fminf(fmaxf(alpha, 0.f), 1.f);
+  if (method == 0) return lo + alpha * (ln - lo);
+  if (method == 1) return logf((1.f - alpha) * expf(lo) + alpha * expf(ln) + 1e-10f);
+  return lo;
+}
+
 __device__ __forceinline__ Surrogate surrogate(float r, float adv, float behave_w, const aa_ppo_params& P) {
   // torch.clamp(r, lo, hi) = min(max(r, lo), hi), NaN stays NaN
   float rc = nan_min(nan_max(r, P.clip_lo), P.clip_hi);

@@ -232,9 +232,10 @@ def grpo_loss_fn(
 
     Returns ``(loss, stat)``.  ``stat`` is the per-token dict of the loss function plus ``"reduced"``: what the
     reference hands to its statistics tracker tensor by tensor (actor.py:513-573) as sums / averages / extrema
-    under the same denominators, computed in one launch per denominator.
+    under the same denominators, computed in one launch per denominator, and under ``"compute_logp"`` and
+    ``"version_stats"`` what it logs in those scopes (actor.py:573-594, 982-1110; ``proximal_logging_stats``).
     """
-    from .actor_ops import apply_m2po_masking, distillation_terms
+    from .actor_ops import apply_m2po_masking, distillation_terms, proximal_logging_stats
     from .advantages import masked_moments
     from .functional import sapo_loss_fn
 
@@ -295,6 +296,10 @@ def grpo_loss_fn(
         reduced.update(masked_moments(dict(vocab_min_logits=vocab_min_logits, vocab_max_logits=vocab_max_logits),
                                       everything))
     reduced["n_tokens"] = infer_token_denominator(input_data, loss_mask).numel()
+    # the compute_logp and version_stats scopes (actor.py:573-594) under the mask the loss kept
+    reduced.update(proximal_logging_stats(old_logp, logprobs.detach(), input_data.get("prox_logp"),
+                                          input_data.get("versions"), current_version,
+                                          stat.get("behave_mask", loss_mask), prox_logp_method))
     stat = dict(stat, loss_mask=loss_mask, reduced=reduced)
     return loss, stat
 

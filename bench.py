@@ -21,7 +21,8 @@ One "step" is one pass of the hot path over one synthetic packed micro-batch tha
   mask read; advantages, returns written).
 
 * aux: the other per-token pieces around the loss at the configs[1] token count (SAPO loss, clipped value loss, DPO
-  loss over 32 pairs, M2PO masking, proximal log-prob approximation) and the packing helpers (pack of a [512, 4096] batch, un-padding of
+  loss over 32 pairs, M2PO masking, proximal log-prob approximation, the 36 logged moments of the approximation
+  metrics) and the packing helpers (pack of a [512, 4096] batch, un-padding of
   [32768 + pad, 151936] bf16 logits).  Roofline: HBM, on the logits un-padding copy (4 * V bytes per token).
 
 Prints ONE JSON line.  Besides the whole-step throughput it carries
@@ -669,6 +670,8 @@ def bench_aux(args, dev):
         sapo_loss_fwd_bwd=sapo, critic_loss_fwd_bwd=critic, dpo_loss_fwd_bwd=dpo,
         m2po_masking=lambda: areal_amd.apply_m2po_masking(d["old"], d["prox"], d["mask"], 0.002),
         prox_logp_loglinear=lambda: areal_amd.compute_prox_logp_approximations(d["old"], d["lp"], d["ver"], 6, "loglinear"),
+        logging_stats_metrics_mode=lambda: areal_amd.proximal_logging_stats(d["old"], d["lp"], d["prox"], d["ver"], 6,
+                                                                            d["mask"], "metrics"),
     )
     out_pieces = {}
     for name, fn in pieces.items():

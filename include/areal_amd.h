@@ -371,6 +371,45 @@ int aa_dpo_pair_loss(const double* policy_sums, const double* ref_sums,
                      float* chosen_reward, float* rejected_reward,
                      uint8_t* valid, double* g_policy_sums, void* stream);
 
+/*
+ * Rows of the table aa_logging_stats writes; each row is {sum, min, max,
+ * count} over the selected tokens (min = +inf, max = -inf, count = 0 when
+ * nothing is selected or the quantity was not asked for).
+ *   0      prox_logp_gt
+ *   1..3   kl_div_direct = -(logp - old), kl_div_taylor = (logp - old)^2 / 2,
+ *          kl_div_dual = exp(logp - old) - 1 - (logp - old)
+ *   4 + 10 m + j, method m = 0 loglinear, 1 linear, 2 rollout:
+ *          j = 0 approx_logp, 1 behave_imp_weight = exp(approx - old),
+ *          2 importance_weight = exp(logp - approx), 3 abs_error,
+ *          4 rel_error, 5 squared_error (of approx against prox_logp_gt),
+ *          6 behave_imp_weight_abs_error, 7 behave_imp_weight_rel_error,
+ *          8 importance_weight_abs_error, 9 importance_weight_rel_error
+ *   34, 35 sample staleness (current_version - 1) - version and
+ *          current_version - version over the selected tokens with
+ *          version >= 0
+ */
+#define AA_LOGSTAT_SLOTS 36
+
+/* Bytes of 256-byte aligned scratch aa_logging_stats needs for n tokens. */
+int64_t aa_logging_stats_scratch_bytes(int64_t n);
+
+/*
+ * The per-token quantities _log_proximal_approximation_stats and
+ * _log_version_staleness_stats (areal/trainer/ppo/actor.py:982-1110, helpers
+ * :859-979) hand to the statistics tracker, reduced under mask in one pass.
+ * prox_logp_gt may be NULL (row 0 and the error rows stay empty; with_errors
+ * must be 0); versions (int32, negative for prompt tokens) may be NULL when
+ * methods == 0 (then rows 1..3 and 34, 35 stay empty, as the reference
+ * returns before logging them).  methods: bit m selects method m of
+ * aa_prox_logp_approx.  An error is |gt - a|, |(gt - a) / (|gt| + 1e-8)|,
+ * (gt - a)^2.  out [AA_LOGSTAT_SLOTS, 4] float32.
+ */
+int aa_logging_stats(const float* old_logp, const float* logp,
+                     const float* prox_logp_gt, const int32_t* versions,
+                     const uint8_t* mask, int64_t n, int current_version,
+                     int methods, int with_errors, float* out, void* scratch,
+                     int64_t scratch_bytes, void* stream);
+
 /* Bytes of 256-byte aligned workspace aa_m2po_mask needs for n tokens. */
 int64_t aa_m2po_workspace_bytes(int64_t n);
 

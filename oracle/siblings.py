@@ -144,3 +144,62 @@ def distillation_loss(loss, logprobs, old_logp, teacher_logp, loss_mask, rl_loss
     rkl_penalty = rkl_penalty_per_token.sum() / loss_mask.sum().clamp(min=1)      # :507
     loss = rl_loss_weight * loss + distill_loss_weight * rkl_penalty              # :509
     return loss, rkl_penalty_per_token                                            # :511
+
+
+_EPSILON = 1e-8   # actor.py:856
+
+
+def approximation_errors(ground_truth, approximation):
+    """abs / rel / squared error; actor.py:867-886."""
+    diff = ground_truth - approximation
+    return dict(abs_error=torch.abs(diff).float(),
+                rel_error=torch.abs(diff / (torch.abs(ground_truth) + _EPSILON)).float(),
+                squared_error=(diff * diff).float())
+
+
+def proximal_logging_tensors(old_logp, logprobs, prox_logp_gt, versions, current_version, mask,
+                             prox_logp_method="recompute"):
+    """The per-token tensors the reference hands to its statistics tracker in the ``compute_logp`` and
+    ``version_stats`` scopes, before any reduction; actor.py:908-979 (one method), :982-1064 (which methods, the KL
+    estimators), :1067-1110 (staleness).  Returns ``(compute_logp, staleness)``: ``{name: tensor}`` to be reduced
+    over ``mask``, and ``{name: 1-D tensor of the selected generated tokens}`` (empty dict when the reference logs
+    nothing)."""
+    out = {}
+    if prox_logp_gt is not None:                                                   # :1002-1006
+        out["prox_logp_gt"] = prox_logp_gt.float()
+    staleness = {}
+    if versions is None or current_version is None:                                # :1009-1010
+        return out, staleness
+
+    def one_method(name, approx, gt):
+        behave = torch.exp(approx - old_logp).float()                              # :924
+        imp = torch.exp(logprobs - approx).float()                                 # :925
+        out.update({f"{name}/approx_logp": approx.float(), f"{name}/behave_imp_weight": behave,
+                    f"{name}/importance_weight": imp})
+        if gt is not None:                                                         # :934-968
+            for k, v in approximation_errors(gt, approx).items():
+                out[f"{name}/{k}"] = v
+            b = approximation_errors(torch.exp(gt - old_logp).float(), behave)
+            i = approximation_errors(torch.exp(logprobs - gt).float(), imp)
+            out[f"{name}/behave_imp_weight_abs_error"] = b["abs_error"]
+            out[f"{name}/behave_imp_weight_rel_error"] = b["rel_error"]
+            out[f"{name}/importance_weight_abs_error"] = i["abs_error"]
+            out[f"{name}/importance_weight_rel_error"] = i["rel_error"]
+
+    if prox_logp_method == "loglinear":                                            # :1012-1028
+        for name, approx in prox_logp_approximations(old_logp, logprobs, versions, current_version,
+                                                     "loglinear").items():
+            one_method(name, approx, None)
+    elif prox_logp_method == "metrics" and prox_logp_gt is not None:               # :1030-1046
+        for name, approx in prox_logp_approximations(old_logp, logprobs, versions, current_version, None).items():
+            one_method(name, approx, prox_logp_gt)
+    log_ratio = (logprobs.float() - old_logp.float()).detach()                     # :1049
+    out["kl_div_direct"] = -log_ratio                                              # :1053-1055
+    out["kl_div_taylor"] = log_ratio ** 2 / 2.0
+    out["kl_div_dual"] = log_ratio.exp() - 1 - log_ratio
+    valid_generated = mask.bool() & (versions >= 0)                                # :1088
+    if valid_generated.any():
+        v_behave = versions.float()
+        staleness = dict(sample_staleness_proximal=((current_version - 1) - v_behave)[valid_generated],
+                         sample_staleness_theta=(current_version - v_behave)[valid_generated])
+    return out, staleness

@@ -275,3 +275,94 @@ def test_loss_adapters_count_logical_tokens(device):
     assert red["n_tokens"] == 2 * n and float(red["new_value"]["count"]) == float(mask.sum())
     assert float(red["clipped_new_value"]["count"]) == float(w_stat["clip_mask"].sum())
     assert float(red["critic_loss"]["sum"]) == pytest.approx(float(w_stat["loss"][mask].sum()), rel=1e-4)
+
+
+def _check_moments(got: dict, tensors: dict, mask, tag=""):
+    assert sorted(got) == sorted(tensors), (tag, sorted(got), sorted(tensors))
+    for name, t in tensors.items():
+        sel = t.double()[mask]
+        g = {k: float(v) for k, v in got[name].items()}
+        assert g["count"] == sel.numel(), (tag, name)
+        scale = float(sel.abs().max()) + 1e-12
+        assert abs(g["sum"] - float(sel.sum())) <= 2e-5 * scale * max(sel.numel() ** 0.5, 1.0), (tag, name, "sum")
+        assert abs(g["min"] - float(sel.min())) <= 1e-5 * scale + 1e-7, (tag, name, "min")
+        assert abs(g["max"] - float(sel.max())) <= 1e-5 * scale + 1e-7, (tag, name, "max")
+        assert abs(g["avg"] - float(sel.mean())) <= 2e-5 * scale, (tag, name, "avg")
+
+
+@pytest.mark.parametrize("method,with_gt", [("recompute", True), ("loglinear", False), ("loglinear", True),
+                                            ("metrics", True), ("metrics", False)])
+@pytest.mark.parametrize("n", [1, 777, 200_003])
+def test_proximal_logging_stats_match_oracle(device, method, with_gt, n):
+    g = torch.Generator().manual_seed(n + 17)
+    lp = -torch.rand(n, generator=g) * 3
+    old = lp + 0.3 * torch.randn(n, generator=g)
+    gt = lp + 0.1 * torch.randn(n, generator=g) if with_gt else None
+    ver = torch.randint(-1, 7, (n,), generator=g, dtype=torch.int32)
+    mask = torch.rand(n, generator=g) < 0.6
+    mask[0] = True
+    ver[0] = 2
+    tensors, stale = S.proximal_logging_tensors(old, lp, gt, ver, 6, mask, method)
+    got = areal_amd.proximal_logging_stats(old.to(device), lp.to(device), None if gt is None else gt.to(device),
+                                           ver.to(device), 6, mask.to(device), method)
+    _check_moments(got["compute_logp"], tensors, mask, method)
+    vs = got["version_stats"]
+    assert vs["v_theta"] == 6 and vs["v_proximal"] == 5
+    gen = mask & (ver >= 0)
+    for key in ("sample_staleness_proximal", "sample_staleness_theta"):
+        want = stale[key]
+        assert float(vs[key]["count"]) == int(gen.sum()) == want.numel()
+        assert float(vs[key]["min"]) == float(want.min()) and float(vs[key]["max"]) == float(want.max())
+        assert float(vs[key]["avg"]) == pytest.approx(float(want.double().mean()), rel=1e-6)
+
+
+def test_proximal_logging_stats_without_versions_or_tokens(device):
+    n = 100
+    lp, old, _, mask = _tok(n, 4)
+    gt = lp + 0.1
+    for kw in (dict(versions=None, current_version=3), dict(versions=torch.zeros(n, dtype=torch.int32), current_version=None)):
+        got = areal_amd.proximal_logging_stats(old.to(device), lp.to(device), gt.to(device),
+                                               None if kw["versions"] is None else kw["versions"].to(device),
+                                               kw["current_version"], mask.to(device), "metrics")
+        assert list(got["compute_logp"]) == ["prox_logp_gt"] and got["version_stats"] == {}
+        assert float(got["compute_logp"]["prox_logp_gt"]["sum"]) == pytest.approx(float(gt[mask].sum()), rel=1e-5)
+    # only prompt tokens selected: the staleness count is 0 where the reference logs nothing
+    ver = torch.full((n,), -1, dtype=torch.int32)
+    got = areal_amd.proximal_logging_stats(old.to(device), lp.to(device), None, ver.to(device), 3, mask.to(device))
+    assert float(got["version_stats"]["sample_staleness_theta"]["count"]) == 0
+    assert sorted(got["compute_logp"]) == ["kl_div_direct", "kl_div_dual", "kl_div_taylor"]
+    # nothing selected at all
+    got = areal_amd.proximal_logging_stats(old.to(device), lp.to(device), None, ver.to(device), 3,
+                                           torch.zeros(n, dtype=torch.bool, device=device))
+    assert float(got["compute_logp"]["kl_div_dual"]["count"]) == 0
+    assert float(got["compute_logp"]["kl_div_dual"]["min"]) == float("inf")
+
+
+def test_grpo_loss_fn_reports_the_logging_scopes(device):
+    """Which names appear in which mode follows tests/test_prox_approx.py:795-935."""
+    from areal_amd import engine_glue as G
+
+    n = 512
+    lp, old, adv, mask = _tok(n, 6)
+    g = torch.Generator().manual_seed(1)
+    data = dict(logprobs=old.to(device), advantages=adv.to(device), loss_mask=mask.to(device),
+                prox_logp=(lp + 0.05 * torch.randn(n, generator=g)).to(device),
+                versions=torch.randint(-1, 3, (n,), generator=g, dtype=torch.int32).to(device))
+    ent = torch.rand(n, device=device)
+    kw = dict(eps_clip=0.2, eps_clip_higher=None, c_clip=None, current_version=3, use_decoupled_loss=True)
+    _, st = G.grpo_loss_fn(lp.to(device).requires_grad_(True), ent, data, prox_logp_method="recompute", **kw)
+    names = st["reduced"]["compute_logp"]
+    assert "prox_logp_gt" in names and "kl_div_dual" in names and not any("/" in k for k in names)
+    assert float(st["reduced"]["version_stats"]["sample_staleness_theta"]["min"]) >= 1.0
+    _, st = G.grpo_loss_fn(lp.to(device).requires_grad_(True), ent, data, prox_logp_method="loglinear", **kw)
+    names = st["reduced"]["compute_logp"]
+    assert "loglinear/approx_logp" in names and "loglinear/abs_error" not in names and "linear/approx_logp" not in names
+    _, st = G.grpo_loss_fn(lp.to(device).requires_grad_(True), ent, data, prox_logp_method="metrics", **kw)
+    names = st["reduced"]["compute_logp"]
+    for method in ("loglinear", "linear", "rollout"):
+        assert f"{method}/abs_error" in names and f"{method}/importance_weight_rel_error" in names
+    tensors, _ = S.proximal_logging_tensors(old, lp, data["prox_logp"].cpu(), data["versions"].cpu(), 3, mask, "metrics")
+    _check_moments(names, tensors, mask, "glue")
+    data.pop("versions")
+    _, st = G.grpo_loss_fn(lp.to(device).requires_grad_(True), ent, data, prox_logp_method="recompute", **kw)
+    assert list(st["reduced"]["compute_logp"]) == ["prox_logp_gt"] and st["reduced"]["version_stats"] == {}

@@ -177,3 +177,58 @@ def test_distillation_loss_against_scalar_definitions():
     # an all-masked batch divides by 1
     lossm, _ = S.distillation_loss(base, t(lp), t(old), t(teacher), torch.zeros(n, dtype=torch.bool), 0, 0.01)
     assert float(lossm) == 0.0
+
+
+def test_proximal_logging_tensors_hand_cases():
+    """No test of the reference checks the values logged under compute_logp / version_stats (tests/test_prox_approx.py
+    :795-935 checks which names appear); the values are pinned by hand arithmetic and the names by those tests."""
+    ln2 = math.log(2.0)
+    old = torch.tensor([-1.0, -2.0, -1.0, -3.0])
+    new = torch.tensor([-1.0 + ln2, -2.0, -1.5, -3.0])
+    gt = torch.tensor([-1.0, -1.5, -1.25, -3.0])
+    ver = torch.tensor([3, 4, 2, -1], dtype=torch.int32)       # current 5: alpha = 1/2, 0, 2/3, 0 (prompt)
+    mask = torch.tensor([True, True, True, False])
+    # recompute: ground truth and the KL estimators only
+    out, stale = S.proximal_logging_tensors(old, new, gt, ver, 5, mask, "recompute")
+    assert sorted(out) == ["kl_div_direct", "kl_div_dual", "kl_div_taylor", "prox_logp_gt"]
+    assert torch.allclose(out["kl_div_direct"], torch.tensor([-ln2, 0.0, 0.5, 0.0]))
+    assert torch.allclose(out["kl_div_taylor"], torch.tensor([ln2 * ln2 / 2, 0.0, 0.125, 0.0]))
+    assert torch.allclose(out["kl_div_dual"], torch.tensor([2 - 1 - ln2, 0.0, math.exp(-0.5) - 1 + 0.5, 0.0]))
+    assert stale["sample_staleness_proximal"].tolist() == [1.0, 0.0, 2.0]
+    assert stale["sample_staleness_theta"].tolist() == [2.0, 1.0, 3.0]
+    # no versions: the reference returns before the estimators
+    out, stale = S.proximal_logging_tensors(old, new, gt, None, 5, mask, "metrics")
+    assert list(out) == ["prox_logp_gt"] and stale == {}
+    out, stale = S.proximal_logging_tensors(old, new, None, ver, None, mask, "loglinear")
+    assert out == {} and stale == {}
+    # loglinear: three tensors, no error metrics (tests/test_prox_approx.py:795-817)
+    out, _ = S.proximal_logging_tensors(old, new, None, ver, 5, mask, "loglinear")
+    assert sorted(k for k in out if "/" in k) == ["loglinear/approx_logp", "loglinear/behave_imp_weight",
+                                                  "loglinear/importance_weight"]
+    approx = torch.tensor([-1.0 + ln2 / 2, -2.0, -1.0 - 0.5 * 2 / 3, -3.0])
+    assert torch.allclose(out["loglinear/approx_logp"], approx)
+    assert torch.allclose(out["loglinear/behave_imp_weight"], torch.tensor([math.sqrt(2.0), 1.0, math.exp(-1 / 3), 1.0]))
+    assert torch.allclose(out["loglinear/importance_weight"], torch.tensor([math.sqrt(2.0), 1.0, math.exp(-1 / 6), 1.0]))
+    # metrics with ground truth: every method with all ten names (tests/test_prox_approx.py:905-935)
+    out, _ = S.proximal_logging_tensors(old, new, gt, ver, 5, mask, "metrics")
+    for method in ("loglinear", "linear", "rollout"):
+        for key in ("approx_logp", "behave_imp_weight", "importance_weight", "abs_error", "rel_error", "squared_error",
+                    "behave_imp_weight_abs_error", "behave_imp_weight_rel_error", "importance_weight_abs_error",
+                    "importance_weight_rel_error"):
+            assert f"{method}/{key}" in out
+    # rollout approximates by the behaviour log-prob: errors are those of old against the ground truth
+    assert torch.allclose(out["rollout/abs_error"], torch.tensor([0.0, 0.5, 0.25, 0.0]))
+    assert torch.allclose(out["rollout/rel_error"], torch.tensor([0.0, 0.5 / 1.5, 0.25 / 1.25, 0.0]), atol=1e-7)
+    assert torch.allclose(out["rollout/squared_error"], torch.tensor([0.0, 0.25, 0.0625, 0.0]))
+    # behave weight: truth exp(gt - old), approximation 1
+    want = torch.tensor([0.0, math.exp(0.5) - 1, 1 - math.exp(-0.25), 0.0])
+    assert torch.allclose(out["rollout/behave_imp_weight_abs_error"], want, atol=1e-7)
+    assert torch.allclose(out["rollout/behave_imp_weight_rel_error"],
+                          want / torch.tensor([1.0, math.exp(0.5), math.exp(-0.25), 1.0]), atol=1e-6)
+    # importance weight: truth exp(new - gt), approximation exp(new - old)
+    t = torch.tensor([2.0, math.exp(-0.5), math.exp(-0.25), 1.0])
+    a = torch.tensor([2.0, 1.0, math.exp(-0.5), 1.0])
+    assert torch.allclose(out["rollout/importance_weight_abs_error"], (t - a).abs(), atol=1e-6)
+    # nothing generated under the mask: no staleness
+    _, stale = S.proximal_logging_tensors(old, new, gt, ver, 5, torch.tensor([False, False, False, True]), "recompute")
+    assert stale == {}
