@@ -39,12 +39,16 @@ from .tree import (
     gather_packed_tree_logprobs_entropy,
     tree_sequence_pairs,
 )
+from .sft import fused_lm_head_sft_loss, fused_logprobs_sft_loss, sft_loss_fn
 from ._native import NativeLibraryError
 
 __version__ = "0.1.0"
 
 __all__ = [
     "NativeLibraryError",
+    "fused_lm_head_sft_loss",
+    "fused_logprobs_sft_loss",
+    "sft_loss_fn",
     "proximal_logging_stats",
     "masked_normalization",
     "dpo_loss",

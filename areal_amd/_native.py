@@ -33,6 +33,7 @@ class PpoParams(C.Structure):
         ("c_clip", C.c_float),
         ("has_c_clip", C.c_int32),
         ("has_behave_weight", C.c_int32),
+        ("loss_kind", C.c_int32),
     ]
 
 
@@ -89,6 +90,7 @@ SIGNATURES = {
     "aa_masked_normalization": (_i, [_p, _p, _i64, _i64, _i, _d, _p, _p, _i64, _p]),
     "aa_overlong_penalty": (_i, [_p, _p, _i64, _i64, _i, _f, _i64, _p]),
     "aa_kd_terms": (_i, [_p, _p, _p, _p, _i64, _i, _p, _p, _p]),
+    "aa_sft_loss": (_i, [_p, _p, _i64, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _p]),
     "aa_dpo_seq_sums": (_i, [_p, _p, _p, _p, _i64, _i64, _p, _p, _p, _p]),
     "aa_dpo_seq_sums_bwd": (_i, [_p, _p, _p, _p, _i64, _i64, _p, _p]),
     "aa_dpo_preference_loss": (_i, [_p, _i64, _d, _i, _p, _p, _p]),

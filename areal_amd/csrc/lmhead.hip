@@ -375,7 +375,9 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
   if (!hidden || !weight || !labels || !d_hidden || !d_weight || !workspace) return AA_ERR_INVALID_ARGUMENT;
   if (!params || !n_valid || !logp) return AA_ERR_INVALID_ARGUMENT;
   if (T_active < 0 || T_active > T || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
-  if (T_active > 0 && (!prox_logp || !adv || !mask_eff || !stat_loss || !ratio || !flags)) return AA_ERR_INVALID_ARGUMENT;
+  const bool nll = params->loss_kind == AA_LOSS_NLL;  // prox_logp and adv are not used by that loss
+  if (T_active > 0 && (!mask_eff || !stat_loss || !ratio || !flags)) return AA_ERR_INVALID_ARGUMENT;
+  if (T_active > 0 && !nll && (!prox_logp || !adv)) return AA_ERR_INVALID_ARGUMENT;
   if (T_active > 0 && params->has_behave_weight && !behave_w) return AA_ERR_INVALID_ARGUMENT;
   if (!shapes_ok(T, H, V) || (d_weight_dtype != AA_F32 && d_weight_dtype != AA_BF16)) return AA_ERR_UNSUPPORTED;
   if ((((uintptr_t)hidden | (uintptr_t)weight | (uintptr_t)workspace | (uintptr_t)d_hidden | (uintptr_t)d_weight) & 15))

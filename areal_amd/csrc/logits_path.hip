@@ -364,8 +364,12 @@ __device__ __forceinline__ uint32_t load_u16_uniform(const void* __restrict__ ro
 // d(surrogate)/d(logp) and d(scaled loss)/d(logp).
 __device__ __forceinline__ void load_loss_scale(const FusedTokenArgs& a, float& fn, float& gscale) {
   int n = *a.n_valid;
-  if (n < 1) n = 1;
-  fn = (float)n;
+  if (a.P.loss_kind == AA_LOSS_NLL) {
+    fn = (float)n + 1e-5f;  // the supervised loss divides by 1e-5 + count (areal/trainer/sft/lm_engine.py:96)
+  } else {
+    if (n < 1) n = 1;
+    fn = (float)n;
+  }
   gscale = a.grad_scale ? *a.grad_scale : 1.f;
 }
 
@@ -381,6 +385,14 @@ __device__ __forceinline__ float fused_token_tail(const FusedTokenArgs& a, int64
   }
   if (!in.active) return 0.f;
   const bool m = in.mask();
+  if (a.P.loss_kind == AA_LOSS_NLL) {  // loss = -logp of the label, d loss / d logp = -1 on the selected tokens
+    if (writer) {
+      a.stat_loss[t] = m ? -lp : 0.f;  // what the trainer logs per token: -where(mask, logp, 0)
+      a.ratio[t] = 0.f;
+      a.flags[t] = 0;
+    }
+    return m ? (-1.f / fn) * gscale : 0.f;
+  }
   const float r = m ? expf(lp - in.prox) : 0.f;
   const Surrogate s = surrogate(r, in.adv, in.w, a.P);
   if (writer) {
@@ -961,7 +973,16 @@ int aa::logits_ppo_fused_rows(const void* logits, int dtype, int64_t T, int64_t 
   if (!params || !n_valid || !logp || !dlogits) return AA_ERR_INVALID_ARGUMENT;
   if (T_active < 0 || T_active > T || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
   // the per-token arrays have T_active entries: with no active token they may be absent
-  if (T_active > 0 && (!prox_logp || !adv || !mask_eff || !stat_loss || !ratio || !flags)) return AA_ERR_INVALID_ARGUMENT;
+  if (params->loss_kind != AA_LOSS_PPO && params->loss_kind != AA_LOSS_NLL) return AA_ERR_INVALID_ARGUMENT;
+  if (T_active > 0 && (!mask_eff || !stat_loss || !ratio || !flags)) return AA_ERR_INVALID_ARGUMENT;
+  if (params->loss_kind == AA_LOSS_NLL) {
+    if (params->has_behave_weight) return AA_ERR_INVALID_ARGUMENT;
+    // The kernels fetch these arrays ahead of the row pass whatever the loss; in this mode the values are never
+    // used, so any readable array of T_active floats serves.
+    if (!prox_logp) prox_logp = stat_loss;
+    if (!adv) adv = stat_loss;
+  }
+  if (T_active > 0 && (!prox_logp || !adv)) return AA_ERR_INVALID_ARGUMENT;
   if (T_active > 0 && params->has_behave_weight && !behave_w) return AA_ERR_INVALID_ARGUMENT;
   hipStream_t st = (hipStream_t)stream;
   FusedTokenArgs a;

@@ -535,6 +535,7 @@ extern "C" int aa_ppo_loss(const float* logp, const float* prox_logp, const floa
   if (!logp || !prox_logp || !adv || !mask_eff || !stat_loss || !ratio || !flags || !g_logp)
     return AA_ERR_INVALID_ARGUMENT;
   if (params->has_behave_weight && !behave_w) return AA_ERR_INVALID_ARGUMENT;
+  if (params->loss_kind != AA_LOSS_PPO) return AA_ERR_UNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
   if (!sequence_level) {
     hipLaunchKernelGGL(k_ppo_token, dim3(grid_for(n)), dim3(256), 0, st, logp, prox_logp, adv, mask_eff, behave_w, n,

@@ -354,3 +354,25 @@ def compute_dpo_loss(logprobs: torch.Tensor, entropy: torch.Tensor | None, input
         stat["reward_accuracy"] = (stat["chosen_reward"] > stat["rejected_reward"]).float()
         stat["reward_margin"] = stat["chosen_reward"] - stat["rejected_reward"]
     return loss, stat
+
+
+def compute_packed_sft_loss(logprobs: torch.Tensor, entropy: torch.Tensor | None, input_: dict[str, Any],
+                            vocab_min_logits: torch.Tensor | None = None,
+                            vocab_max_logits: torch.Tensor | None = None) -> tuple[torch.Tensor, dict]:
+    """The SFT loss function of one packed micro-batch (areal/trainer/sft/lm_engine.py:81-131) on the GPU ops.
+
+    Returns ``(loss, stat)``; ``stat`` holds what the reference records: per token ``loss`` under ``n_valid_tokens``
+    (= ``loss_mask``), per sequence ``ppl`` under ``n_seqs`` (the sequences with a selected token), and in
+    ``stat["reduced"]`` the moments of ``loss`` and of the vocabulary extrema (under all tokens) when given."""
+    from .advantages import masked_moments
+    from .sft import sft_loss_fn
+
+    del entropy  # SFT does not use entropy
+    loss_mask = input_["loss_mask"].bool()
+    loss, stat = sft_loss_fn(logprobs, loss_mask, input_["cu_seqlens"])
+    reduced = masked_moments(dict(loss=stat["loss"]), loss_mask)
+    if vocab_min_logits is not None and vocab_max_logits is not None:
+        reduced.update(masked_moments(dict(vocab_min_logits=vocab_min_logits, vocab_max_logits=vocab_max_logits),
+                                      torch.ones_like(loss_mask)))
+    reduced["n_tokens"] = logprobs.shape[0]
+    return loss, dict(stat, loss_mask=loss_mask, reduced=reduced)

@@ -482,6 +482,19 @@ def ppo_actor_loss_fn(
 # ----------------------------------------------------------------------------
 # fused: logits -> logp/entropy -> token-level PPO loss -> d(logits), one pass
 # ----------------------------------------------------------------------------
+def _finish_fused_loss(lib, params, stat_loss, logp, mask_eff, T_active, n_valid, grad_scale, loss, st) -> None:
+    """The scalar the fused kernels' per-token losses add up to: the clipped surrogate over ``max(n, 1)``, or the
+    negative log-likelihood over ``n + 1e-5`` (areal/trainer/sft/lm_engine.py:96)."""
+    if params.loss_kind == 1:
+        scratch = torch.empty(1, dtype=torch.float64, device=logp.device)
+        cnt = torch.empty(1, dtype=torch.int32, device=logp.device)
+        N.check(lib.aa_sft_loss(_ptr(logp), _ptr(mask_eff), T_active, None, 0, _ptr(n_valid), _ptr(grad_scale),
+                                _ptr(loss), None, None, _ptr(scratch), _ptr(cnt), None, st), "aa_sft_loss")
+    else:
+        N.check(lib.aa_masked_sum(_ptr(stat_loss), _ptr(mask_eff), T_active, _ptr(n_valid), _ptr(grad_scale),
+                                  _ptr(loss), st), "aa_masked_sum")
+
+
 class _FusedLogitsPpo(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits2d, labels1d, stride, temperature, T_active, prox, adv, mask_eff, behave_w, params,
@@ -513,12 +526,7 @@ class _FusedLogitsPpo(torch.autograd.Function):
                 ),
                 "aa_logits_ppo_fused",
             )
-            N.check(
-                lib.aa_masked_sum(
-                    _ptr(stat_loss), _ptr(mask_eff), T_active, _ptr(n_valid), _ptr(grad_scale), _ptr(loss), st
-                ),
-                "aa_masked_sum",
-            )
+            _finish_fused_loss(lib, params, stat_loss, logp, mask_eff, T_active, n_valid, grad_scale, loss, st)
         ctx.save_for_backward(dlogits)
         others = [logp, entropy, stat_loss, ratio, flags] + [t for t in (vmax, vmin) if t is not None]
         ctx.mark_non_differentiable(*others)
@@ -787,12 +795,7 @@ class _FusedLmHeadPpo(torch.autograd.Function):
                 ),
                 "aa_lmhead_ppo_fused",
             )
-            N.check(
-                lib.aa_masked_sum(
-                    _ptr(stat_loss), _ptr(mask_eff), T_active, _ptr(n_valid), _ptr(grad_scale), _ptr(loss), st
-                ),
-                "aa_masked_sum",
-            )
+            _finish_fused_loss(lib, params, stat_loss, logp, mask_eff, T_active, n_valid, grad_scale, loss, st)
         ctx.save_for_backward(d_hidden, d_weight)
         ctx.mark_non_differentiable(logp, entropy, stat_loss, ratio, flags)
         return loss, logp, entropy, stat_loss, ratio, flags

@@ -237,6 +237,39 @@ def logits_cpu_baseline_and_parity(case, kw, cfg, n_tokens: int, iters: int):
     return baseline, parity
 
 
+def time_sft_steps(case, iters: int):
+    """The supervised loss on the same logits: fused (one pass, 4 V bytes per token) against the log-prob op followed
+    by the loss on log-probs (forward pass + backward pass, 6 V bytes per token)."""
+    import torch
+
+    import areal_amd
+
+    T = case.logits.shape[0]
+
+    def fused():
+        x = case.logits.detach().requires_grad_(True)
+        loss, _ = areal_amd.fused_logprobs_sft_loss(x, case.labels, case.loss_mask, case.cu_seqlens, case.temperature)
+        loss.backward()
+
+    def two_pass():
+        x = case.logits.detach().requires_grad_(True)
+        logp = areal_amd.gather_logprobs(x, case.labels, case.temperature)
+        loss, _ = areal_amd.sft_loss_fn(logp, case.loss_mask, case.cu_seqlens)
+        loss.backward()
+
+    out = {}
+    for name, fn in (("fused", fused), ("two_pass", two_pass)):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            fn()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / iters * 1e3
+        out[name] = dict(ms_per_step=ms, tokens_per_s=T / (ms * 1e-3))
+    return out
+
+
 def bench_logits(args, dev):
     import torch
 
@@ -275,6 +308,7 @@ def bench_logits(args, dev):
     )
     if cfg is not None:
         out["config"]["importance_weight_cap"] = f"{cfg.level} {cfg.metric} <= {cfg.upper}, action={cfg.action}"
+    out["sft_loss_same_logits"] = time_sft_steps(case, max(args.steps // 2, 3))
     if args.copy_launches > 0:
         from areal_amd import _native as N
         from areal_amd import functional as F

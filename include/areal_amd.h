@@ -46,6 +46,17 @@ typedef enum { AA_RS_ACTION_MASK = 0, AA_RS_ACTION_CLAMP = 1 } aa_rs_action;
 typedef enum { AA_RS_RATIO = 0, AA_RS_KL_K1 = 1, AA_RS_KL_K2 = 2, AA_RS_KL_K3 = 3 } aa_rs_metric;
 typedef enum { AA_RS_AGG_SUM = 0, AA_RS_AGG_MEAN = 1, AA_RS_AGG_MAX = 2 } aa_rs_agg;
 
+/* Which per-token loss the fused entry points put on the log-probs:
+ *   AA_LOSS_PPO  the clipped surrogate of ppo_actor_loss_fn
+ *                (areal/utils/functional/functional.py:516-542), divided by
+ *                max(*n_valid, 1);
+ *   AA_LOSS_NLL  the supervised loss of compute_packed_sft_loss
+ *                (areal/trainer/sft/lm_engine.py:93-96): -logp on the selected
+ *                tokens, divided by (*n_valid + 1e-5).  stat_loss = -logp on
+ *                the selected tokens and 0 elsewhere, ratio = 0, flags = 0; prox_logp, adv and behave_w are not
+ *                used and may be NULL. */
+typedef enum { AA_LOSS_PPO = 0, AA_LOSS_NLL = 1 } aa_loss_kind;
+
 /* Clipped-surrogate parameters of ppo_actor_loss_fn
  * (areal/utils/functional/functional.py:516-532). */
 typedef struct {
@@ -54,6 +65,7 @@ typedef struct {
   float c_clip;        /* dual-clip factor, used only if has_c_clip != 0 */
   int32_t has_c_clip;
   int32_t has_behave_weight; /* multiply the loss by behave_w (rejection sampling on) */
+  int32_t loss_kind;   /* aa_loss_kind; aa_ppo_loss accepts AA_LOSS_PPO only */
 } aa_ppo_params;
 
 /* Library version (major * 10000 + minor * 100 + patch). */
@@ -311,6 +323,30 @@ int aa_kd_terms(const float* logp, const float* old_logp,
                 const float* teacher_logp, const uint8_t* mask, int64_t n,
                 int pure_distillation, float* term, float* dterm,
                 void* stream);
+
+/*
+ * compute_packed_sft_loss (areal/trainer/sft/lm_engine.py:81-131) given
+ * log-probs: with m the loss mask as bytes and n = *n_valid (device, the
+ * number of non-zero mask bytes, aa_count_nonzero_u8),
+ *   loss[0]      = -scale * sum_t (m ? logp[t] : 0) / (n + 1e-5)
+ *   g_logp[t]    = d loss / d logp[t] = m ? -scale / (n + 1e-5) : 0  (nullable)
+ *   stat_loss[t] = -(m ? logp[t] : 0), what the reference logs per token
+ *                  (nullable)
+ * and per sequence b of cu_seqlens [n_seqs + 1] (int32, device; the Python
+ * loop with one read-back per sequence at :101-112):
+ *   seq_count[b] = selected tokens of the sequence,
+ *   seq_logp[b]  = mean of their log-probs in fp64, 0 when there is none,
+ *   seq_ppl[b]   = (float)exp(-seq_logp[b])                          (nullable)
+ * seq_logp and seq_count have n_seqs + 1 entries; the last holds the sum and
+ * the number of the selected tokens outside every sequence.  cu_seqlens may be
+ * NULL with n_seqs == 0.  scale: device float, NULL = 1.  Sums are fp64 in a
+ * fixed order.
+ */
+int aa_sft_loss(const float* logp, const uint8_t* mask, int64_t T,
+                const int32_t* cu_seqlens, int64_t n_seqs,
+                const int32_t* n_valid, const float* scale, float* loss,
+                float* g_logp, float* stat_loss, double* seq_logp,
+                int32_t* seq_count, float* seq_ppl, void* stream);
 
 /*
  * Direct preference optimisation over a packed batch whose sequences are
