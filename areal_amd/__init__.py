@@ -17,7 +17,7 @@ from .advantages import (
     masked_normalization,
     reward_overlong_penalty,
 )
-from .dpo import dpo_loss, dpo_pair_logratios, dpo_preference_loss
+from .dpo import dpo_loss, dpo_pair_logratios, dpo_preference_loss, rw_pair_loss
 from .config import NormConfig, RejectionSamplingConfig
 from .functional import (
     RejectionSamplingResult,
@@ -54,6 +54,7 @@ __all__ = [
     "dpo_loss",
     "dpo_pair_logratios",
     "dpo_preference_loss",
+    "rw_pair_loss",
     "NormConfig",
     "Normalization",
     "RejectionSamplingConfig",

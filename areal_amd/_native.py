@@ -97,6 +97,7 @@ SIGNATURES = {
     "aa_dpo_pair_loss": (_i, [_p, _p, _p, _p, _i64, _d, _i, _p, _p, _p, _p, _p, _p, _p, _p]),
     "aa_logging_stats_scratch_bytes": (_i64, [_i64]),
     "aa_logging_stats": (_i, [_p, _p, _p, _p, _p, _i64, _i, _i, _i, _p, _p, _i64, _p]),
+    "aa_rw_pair_loss": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _p]),
     "aa_m2po_workspace_bytes": (_i64, [_i64]),
     "aa_m2po_mask": (_i, [_p, _p, _p, _i64, _f, _p, _p, _p, _i64, _p]),
     "aa_kl_rewards": (_i, [_p, _p, _p, _p, _p, _i64, _i64, _f, _i, _i, _p, _p, _p]),

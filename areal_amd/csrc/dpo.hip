@@ -192,6 +192,62 @@ __global__ __launch_bounds__(kThreads) void k_pair_loss(const double* __restrict
   }
 }
 
+// both sequences of pair p are non-empty (rw_engine.py:20-22) and their last tokens lie inside the score array
+__device__ __forceinline__ bool rw_pair_ok(const int32_t* cu, int64_t p, int64_t T) {
+  const int64_t b = cu[2 * p], ec = cu[2 * p + 1], er = cu[2 * p + 2];
+  return ec != b && er != ec && ec >= 1 && er >= 1 && ec <= T && er <= T;
+}
+
+// Reward-model loss (areal/trainer/rw/rw_engine.py:115-146): the score of a sequence is the one at its last token;
+// per valid pair -logsigmoid(score_chosen - score_rejected), mean over the valid pairs.  One workgroup: it first
+// clears the gradient of every token, then writes the two entries of each valid pair.
+__global__ __launch_bounds__(kSeqThreads) void k_rw_pair_loss(const float* __restrict__ scores, int64_t T,
+                                                              const int32_t* __restrict__ cu, int64_t n_pairs,
+                                                              float* __restrict__ loss_mean,
+                                                              int32_t* __restrict__ n_valid,
+                                                              float* __restrict__ pair_loss,
+                                                              float* __restrict__ pos_score,
+                                                              float* __restrict__ neg_score,
+                                                              uint8_t* __restrict__ valid,
+                                                              float* __restrict__ g_scores) {
+  __shared__ double smem[kMaxWaves];
+  if (g_scores) {
+    for (int64_t t = threadIdx.x; t < T; t += kSeqThreads) g_scores[t] = 0.f;
+    __syncthreads();
+  }
+  // pass 1: the number of valid pairs (the gradient of a pair is 1 / that number times its own derivative)
+  double cnt = 0.0;
+  for (int64_t p = threadIdx.x; p < n_pairs; p += kSeqThreads) cnt += rw_pair_ok(cu, p, T) ? 1.0 : 0.0;
+  cnt = block_sum_f64(cnt, smem);
+  const float inv = cnt > 0.0 ? (float)(1.0 / cnt) : 0.f;
+  double acc = 0.0;
+  for (int64_t p = threadIdx.x; p < n_pairs; p += kSeqThreads) {
+    const int64_t ec = cu[2 * p + 1], er = cu[2 * p + 2];
+    const bool ok = rw_pair_ok(cu, p, T);
+    float l = 0.f, sc = 0.f, sr = 0.f;
+    if (ok) {
+      sc = scores[ec - 1];
+      sr = scores[er - 1];
+      float dl;
+      neg_logsigmoid(sc - sr, l, dl);
+      acc += (double)l;
+      if (g_scores) {
+        g_scores[ec - 1] = dl * inv;
+        g_scores[er - 1] = -dl * inv;
+      }
+    }
+    pair_loss[p] = l;
+    pos_score[p] = sc;
+    neg_score[p] = sr;
+    valid[p] = ok ? 1 : 0;
+  }
+  acc = block_sum_f64(acc, smem);
+  if (threadIdx.x == 0) {
+    loss_mean[0] = (float)(acc * (double)inv);
+    n_valid[0] = (int32_t)cnt;
+  }
+}
+
 }  // namespace dpo
 }  // namespace aa
 
@@ -244,5 +300,16 @@ extern "C" int aa_dpo_pair_loss(const double* policy_sums, const double* ref_sum
   hipLaunchKernelGGL(k_pair_loss, dim3(1), dim3(kThreads), 0, (hipStream_t)stream, policy_sums, ref_sums,
                      completion_lens, cu_seqlens, n_pairs, beta, loss_type, loss_mean, n_valid, pair_loss,
                      chosen_reward, rejected_reward, valid, g_policy_sums);
+  return hipGetLastError() == hipSuccess ? AA_OK : AA_ERR_LAUNCH;
+}
+
+extern "C" int aa_rw_pair_loss(const float* scores, int64_t T, const int32_t* cu_seqlens, int64_t n_pairs,
+                               float* loss_mean, int32_t* n_valid, float* pair_loss, float* pos_score,
+                               float* neg_score, uint8_t* valid, float* g_scores, void* stream) {
+  if (T < 0 || n_pairs < 0 || !loss_mean || !n_valid) return AA_ERR_INVALID_ARGUMENT;
+  if (n_pairs > 0 && (!cu_seqlens || !pair_loss || !pos_score || !neg_score || !valid)) return AA_ERR_INVALID_ARGUMENT;
+  if (T > 0 && !scores) return AA_ERR_INVALID_ARGUMENT;
+  hipLaunchKernelGGL(k_rw_pair_loss, dim3(1), dim3(kSeqThreads), 0, (hipStream_t)stream, scores, T, cu_seqlens, n_pairs,
+                     loss_mean, n_valid, pair_loss, pos_score, neg_score, valid, g_scores);
   return hipGetLastError() == hipSuccess ? AA_OK : AA_ERR_LAUNCH;
 }

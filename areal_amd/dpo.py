@@ -1,14 +1,16 @@
-"""Direct preference optimisation over a packed batch of interleaved (chosen, rejected) sequences.
+"""Pairwise preference losses over a packed batch of interleaved (chosen, rejected) sequences: DPO and the
+reward-model loss.
 
 Host-side mirror of ``dpo_pair_logratios`` / ``dpo_preference_loss`` (areal/utils/functional/functional.py:641-703)
-and of the loss assembled from them in ``compute_dpo_loss`` (areal/trainer/dpo/dpo_engine.py:147-213).
+and of the loss assembled from them in ``compute_dpo_loss`` (areal/trainer/dpo/dpo_engine.py:147-213); of
+``compute_rw_loss`` (areal/trainer/rw/rw_engine.py:115-146).
 """
 from __future__ import annotations
 
 import torch
 
 from . import _native as N
-from .functional import _f32, _mask_u8, _ptr, _require_gpu, _stream
+from .functional import _DTYPES, _f32, _mask_u8, _ptr, _require_gpu, _stream
 
 _LOSS_TYPES = {"sigmoid": 0, "ipo": 1}
 
@@ -167,3 +169,48 @@ def dpo_loss(logprobs: torch.Tensor, ref_logprobs: torch.Tensor, cu_seqlens: tor
     loss, pair_loss, chosen, rejected, valid, n_valid = _DpoLoss.apply(lp, ref, m8, cu, float(beta), lt)
     stat = dict(loss=pair_loss, chosen_reward=chosen, rejected_reward=rejected, valid_pairs=valid, n_pairs=n_valid)
     return loss, stat
+
+
+class _RwLoss(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, scores, cu):
+        lib = N.load()
+        dev = scores.device
+        T, n_pairs = scores.numel(), (cu.numel() - 1) // 2
+        pair_loss, pos, neg = torch.empty(3, n_pairs, dtype=torch.float32, device=dev).unbind(0)
+        valid = torch.empty(n_pairs, dtype=torch.bool, device=dev)
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        n_valid = torch.empty((), dtype=torch.int32, device=dev)
+        g = torch.empty(T, dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            N.check(lib.aa_rw_pair_loss(_ptr(scores), T, _ptr(cu), n_pairs, _ptr(loss), _ptr(n_valid), _ptr(pair_loss),
+                                        _ptr(pos), _ptr(neg), _ptr(valid), _ptr(g), _stream(dev)), "aa_rw_pair_loss")
+        ctx.save_for_backward(g)
+        outs = (pair_loss, pos, neg, valid, n_valid)
+        ctx.mark_non_differentiable(*outs)
+        return (loss,) + outs
+
+    @staticmethod
+    def backward(ctx, g_loss, *_):
+        (g,) = ctx.saved_tensors
+        dev = g.device
+        up = _f32(g_loss).reshape(1)
+        if g.numel():
+            with torch.cuda.device(dev):   # in place: a factor of 1 is a no-op
+                N.check(N.load().aa_scale_inplace(_ptr(g), _DTYPES[g.dtype], g.numel(), _ptr(up), _stream(dev)),
+                        "aa_scale_inplace")
+        return g, None
+
+
+def rw_pair_loss(scores: torch.Tensor, cu_seqlens: torch.Tensor) -> tuple[torch.Tensor, dict]:
+    """Mean of ``-logsigmoid(score_chosen - score_rejected)`` over the valid pairs of a packed batch, a sequence's
+    score being the one at its last token; rw_engine.py:115-146 without its logging.  With no valid pair the loss
+    is 0.  Nothing is read back.  Returns ``(loss, stat)`` with per pair (zeros where invalid) ``loss``,
+    ``pos_score``, ``neg_score``, the bool ``valid_pairs`` and ``n_pairs`` (int32 scalar on the device)."""
+    _require_gpu(scores, "scores")
+    if scores.dim() != 1 or cu_seqlens.dim() != 1 or cu_seqlens.numel() < 1 or (cu_seqlens.numel() - 1) % 2:
+        raise ValueError("expected 1-D scores and cu_seqlens over an even number of sequences")
+    s = scores if scores.dtype == torch.float32 and scores.is_contiguous() else scores.float().contiguous()
+    cu = cu_seqlens.to(device=s.device, dtype=torch.int32).contiguous()
+    loss, pair_loss, pos, neg, valid, n_valid = _RwLoss.apply(s, cu)
+    return loss, dict(loss=pair_loss, pos_score=pos, neg_score=neg, valid_pairs=valid, n_pairs=n_valid)

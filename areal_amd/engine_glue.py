@@ -376,3 +376,25 @@ def compute_packed_sft_loss(logprobs: torch.Tensor, entropy: torch.Tensor | None
                                       torch.ones_like(loss_mask)))
     reduced["n_tokens"] = logprobs.shape[0]
     return loss, dict(stat, loss_mask=loss_mask, reduced=reduced)
+
+
+def rw_valid_pairs(x: dict[str, Any]) -> torch.Tensor:
+    """Pairs whose chosen and rejected sequences are both non-empty (areal/trainer/rw/rw_engine.py:20-22)."""
+    return dpo_valid_pairs(x)
+
+
+def rw_loss_weight(x: dict[str, Any]) -> torch.Tensor:
+    """Number of valid pairs as a float (rw_engine.py:25-26)."""
+    return rw_valid_pairs(x).count_nonzero().float()
+
+
+def compute_rw_loss(scores: torch.Tensor, input_: dict[str, Any]) -> tuple[torch.Tensor, dict]:
+    """The reward-model loss function of one packed micro-batch (rw_engine.py:115-146) on the GPU ops.  Returns
+    ``(loss, stat)`` with what the reference records per pair under ``n_pairs``: ``loss``, ``pos_score``,
+    ``neg_score``, ``correct_ratio``, selected by ``valid_pairs``."""
+    from .dpo import rw_pair_loss
+
+    loss, stat = rw_pair_loss(scores, input_["cu_seqlens"])
+    with torch.no_grad():
+        stat["correct_ratio"] = (stat["pos_score"] > stat["neg_score"]).float()
+    return loss, stat

@@ -446,6 +446,20 @@ int aa_logging_stats(const float* old_logp, const float* logp,
                      int methods, int with_errors, float* out, void* scratch,
                      int64_t scratch_bytes, void* stream);
 
+/*
+ * compute_rw_loss (areal/trainer/rw/rw_engine.py:115-146) over a packed batch
+ * of interleaved (chosen, rejected) sequences: the score of a sequence is
+ * scores[cu_seqlens[s + 1] - 1]; a pair is valid when both sequences are
+ * non-empty (:20-22).  Per pair: pair_loss = -logsigmoid(pos - neg),
+ * pos_score, neg_score, valid (zeros for an invalid pair); loss_mean[0] = mean
+ * over the valid pairs (0 when there are none), n_valid[0] their number;
+ * g_scores [T] = d loss_mean / d scores (nullable).
+ */
+int aa_rw_pair_loss(const float* scores, int64_t T, const int32_t* cu_seqlens,
+                    int64_t n_pairs, float* loss_mean, int32_t* n_valid,
+                    float* pair_loss, float* pos_score, float* neg_score,
+                    uint8_t* valid, float* g_scores, void* stream);
+
 /* Bytes of 256-byte aligned workspace aa_m2po_mask needs for n tokens. */
 int64_t aa_m2po_workspace_bytes(int64_t n);
 

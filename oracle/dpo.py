@@ -73,3 +73,19 @@ def compute_dpo_loss(logprobs, ref_logprobs, cu_seqlens, loss_mask, beta, loss_t
         valid_pairs=valid,
     )
     return per_pair.mean(), stat
+
+
+def compute_rw_loss(scores, cu_seqlens):
+    """(loss, stat); areal/trainer/rw/rw_engine.py:115-146 with the logged tensors returned."""
+    seqlens = cu_seqlens[1:] - cu_seqlens[:-1]
+    valid = valid_pairs(cu_seqlens)                                                 # :20-22, 119
+    if not valid.any():                                                            # :120-122
+        z = torch.zeros(0, dtype=torch.float32)
+        return torch.zeros((), dtype=torch.float32), dict(loss=z, pos_score=z, neg_score=z, valid_pairs=valid)
+    terminal = seqlens.cumsum(0) - 1                                               # :125
+    assert scores.shape[0] == seqlens.sum()
+    s = scores[terminal].view(-1, 2)[valid].float()                                # :128
+    loss = -(torch.nn.functional.logsigmoid(s[:, 0] - s[:, 1]))                    # :130
+    stat = dict(loss=loss.detach(), pos_score=s[:, 0].detach(), neg_score=s[:, 1].detach(), valid_pairs=valid,
+                correct_ratio=(s[:, 0] > s[:, 1]).float())
+    return loss.mean(), stat

@@ -166,3 +166,44 @@ def test_long_sequences_keep_fp64_accuracy(device):
     exact = float(chosen[100].double() - base[100].double())
     assert stat["chosen_reward"].item() == pytest.approx(exact, rel=1e-6) and stat["rejected_reward"].item() == 0.0
     assert float(loss) == pytest.approx(float(w_loss), rel=1e-6) and float(loss) < LOG2
+
+
+@pytest.mark.parametrize("name", list(LENS))
+def test_reward_model_loss_matches_oracle(device, name):
+    lens = LENS[name]
+    g = torch.Generator().manual_seed(4)
+    cu = torch.tensor([0] + lens, dtype=torch.int64).cumsum(0)
+    T = int(cu[-1])
+    scores = torch.randn(T, generator=g) * 2
+    x = scores.clone().requires_grad_(True)
+    w_loss, w_stat = D.compute_rw_loss(x, cu)
+    (1.7 * w_loss).backward()
+    y = scores.to(device).requires_grad_(True)
+    loss, stat = G.compute_rw_loss(y, {"cu_seqlens": cu.to(torch.int32).to(device)})
+    (1.7 * loss).backward()
+    assert float(loss.detach()) == pytest.approx(float(w_loss.detach()), rel=2e-6)
+    valid = stat["valid_pairs"].cpu()
+    assert torch.equal(valid, w_stat["valid_pairs"]) and int(stat["n_pairs"]) == int(valid.sum())
+    for k in ("loss", "pos_score", "neg_score", "correct_ratio"):
+        assert torch.allclose(stat[k].cpu()[valid], w_stat[k], rtol=2e-6, atol=1e-7), k
+    assert torch.allclose(y.grad.cpu(), x.grad, rtol=1e-5, atol=1e-9)
+    assert int((y.grad != 0).sum()) == 2 * int(valid.sum())
+
+
+def test_reward_model_loss_reference_cases(device):
+    """tests/test_eval_dispatch.py:325-371."""
+    inp = {"cu_seqlens": torch.tensor([0, 5, 9, 9, 9], dtype=torch.int32, device=device)}
+    scores = torch.tensor([0.0, 0.0, 0.0, 0.0, 3.0, 0.0, 0.0, 0.0, 1.0], device=device)
+    loss, stat = G.compute_rw_loss(scores, inp)
+    assert float(loss) == pytest.approx(math.log1p(math.exp(-2.0)), rel=1e-5)
+    assert int(stat["n_pairs"]) == 1 and float(G.rw_loss_weight(inp)) == 1.0
+    assert stat["pos_score"].tolist() == [3.0, 0.0] and stat["neg_score"].tolist() == [1.0, 0.0]
+    assert stat["correct_ratio"].tolist() == [1.0, 0.0]
+    loss, stat = G.compute_rw_loss(torch.zeros(0, device=device),
+                                   {"cu_seqlens": torch.tensor([0, 0, 0], dtype=torch.int32, device=device)})
+    assert float(loss) == 0.0 and int(stat["n_pairs"]) == 0
+    # bf16 scores, as a value head emits them
+    s16 = torch.randn(9, device=device).bfloat16().requires_grad_(True)
+    loss, _ = G.compute_rw_loss(s16, inp)
+    loss.backward()
+    assert s16.grad.dtype == torch.bfloat16 and int((s16.grad != 0).sum()) == 2

@@ -150,3 +150,28 @@ def test_preference_loss_closed_forms():
     assert np.allclose(got.numpy(), want, rtol=1e-6, atol=1e-30)
     got = D.preference_loss(x, 0.25, "ipo")
     assert np.allclose(got.numpy(), [(v - 2.0) ** 2 for v in x.tolist()], rtol=1e-6)
+
+
+def test_reward_model_loss_reference_cases():
+    """tests/test_eval_dispatch.py:325-371: lengths [5, 4, 0, 0], scores 3 and 1 at the two last tokens -> the loss
+    is -logsigmoid(2) over the one valid pair; only empty pairs -> 0."""
+    cu = torch.tensor([0, 5, 9, 9, 9])
+    scores = torch.tensor([0.0, 0.0, 0.0, 0.0, 3.0, 0.0, 0.0, 0.0, 1.0])
+    loss, stat = D.compute_rw_loss(scores, cu)
+    want = math.log1p(math.exp(-2.0))
+    assert abs(float(loss) - want) < 1e-6
+    assert stat["valid_pairs"].tolist() == [True, False]
+    assert stat["pos_score"].tolist() == [3.0] and stat["neg_score"].tolist() == [1.0]
+    assert stat["correct_ratio"].tolist() == [1.0] and abs(float(stat["loss"][0]) - want) < 1e-6
+    loss, stat = D.compute_rw_loss(torch.tensor([], dtype=torch.float32), torch.tensor([0, 0, 0]))
+    assert float(loss) == 0.0 and stat["valid_pairs"].tolist() == [False]
+    # equal scores -> log 2; gradient of the mean: -sigmoid(-(pos - neg)) / K at the chosen token, + at the rejected
+    cu = torch.tensor([0, 2, 5, 6, 8])
+    s = torch.tensor([9.0, 0.5, 9.0, 9.0, 0.5, 1.0, 9.0, -1.0], requires_grad=True)
+    loss, _ = D.compute_rw_loss(s, cu)
+    want = (LOG2 + math.log1p(math.exp(-2.0))) / 2
+    assert abs(float(loss.detach()) - want) < 1e-6
+    loss.backward()
+    sig = lambda z: 1 / (1 + math.exp(-z))
+    g = [0.0, -0.5 * sig(0.0), 0.0, 0.0, 0.5 * sig(0.0), -0.5 * sig(-2.0), 0.0, 0.5 * sig(-2.0)]
+    assert np.allclose(s.grad.numpy(), g, atol=1e-7)
