@@ -27,6 +27,7 @@ from .ppo import (
 from .advantages import gae, masked_moments, normalization
 from .siblings import critic_loss, distillation_loss, m2po_mask, prox_logp_approximations, sapo_loss
 from . import dpo  # noqa: F401  (DPO pair sums and loss)
+from . import microbatch  # noqa: F401  (micro-batch allocation and split)
 from . import sft  # noqa: F401  (supervised loss over a packed batch)
 from .pipeline import lmhead_logits, logits_ppo_step
 

@@ -97,3 +97,41 @@ def test_pack_full_size_round_trip(device):
     p = areal_amd.pack_tensor_dict(dict(attention_mask=am, input_ids=ids, logprobs=lp))
     assert p["input_ids"].shape[0] == int(lens.sum()) and p["max_seqlen"] == int(lens.max())
     assert torch.equal(p["input_ids"], ids[am]) and torch.equal(p["logprobs"], lp[am])  # row-major boolean gather
+
+
+@pytest.mark.parametrize("algorithm,seq_align_to,pad_to_maximum", [("ffd", None, False), ("kk", 64, False),
+                                                                  ("ffd", None, True)])
+def test_packed_mb_list_matches_oracle_chain(device, algorithm, seq_align_to, pad_to_maximum):
+    """Padded batch -> balanced micro-batches -> packed -> page padded (fsdp_engine.py:1778-1786), against the
+    oracle's row-by-row split, pack and pad."""
+    from areal_amd import microbatch as M
+    from oracle import microbatch as OM
+
+    g = torch.Generator().manual_seed(12)
+    bs, L = 24, 300
+    lens = torch.randint(1, L + 1, (bs,), generator=g)
+    attn = (torch.arange(L)[None, :] < lens[:, None]).long()
+    data = dict(attention_mask=attn, input_ids=torch.randint(0, 999, (bs, L), generator=g),
+                logprobs=torch.randn(bs, L, generator=g), loss_mask=(torch.rand(bs, L, generator=g) < 0.5),
+                rewards=torch.randn(bs, generator=g))
+    cap = 2048
+    spec = M.MicroBatchSpec(n_mbs=2, max_tokens_per_mb=cap, packing_algorithm=algorithm)
+    got = M.packed_mb_list({k: v.to(device) for k, v in data.items()}, spec, seq_align_to=seq_align_to,
+                           pad_to_maximum=pad_to_maximum)
+    ref = M.amend_position_ids(dict(data))
+    mbs, group_lens, fwd, bwd = OM.split_padded_tensor_dict(ref, cap, 2, 1, 1, algorithm)
+    assert got.group_lens == group_lens and [int(i) for i in got.forward_indices] == fwd
+    assert len(got) == len(mbs) >= 2
+    for item, mb, n_tok in zip(got, mbs, group_lens):
+        packed = P.pack_tensor_dict(mb)
+        pad_to = cap if pad_to_maximum else (n_tok + 255) // 256 * 256
+        want, pad_len, old_cu, _ = P.pad_packed_tensor_dict(packed, pad_to, 0.0, seq_align_to=seq_align_to)
+        assert item.padding_length == pad_len and item.padded_to_length == pad_to
+        for key in ("input_ids", "logprobs", "loss_mask", "position_ids", "cu_seqlens"):
+            assert torch.equal(item.padded_mb[key].cpu(), want[key]), key
+            assert torch.equal(item.orig_mb[key].cpu(), packed[key]), key
+        assert int(item.padded_mb["max_seqlen"]) == int(want["max_seqlen"])
+        assert torch.equal(item.orig_mb["rewards"].cpu(), data["rewards"])          # not split: shared by every micro-batch
+        if seq_align_to is not None:
+            assert torch.equal(item.old_cu_seqlens.cpu(), old_cu)
+    assert got.max_seqlen == max(int(m["cu_seqlens"][-1]) for m in got.padded_mbs)
