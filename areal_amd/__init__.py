@@ -10,6 +10,7 @@ from .actor_ops import (
     proximal_logging_stats,
 )
 from .advantages import (
+    KLEstimator,
     Normalization,
     gae_advantages,
     kl_regularized_rewards,
@@ -46,6 +47,7 @@ __version__ = "0.1.0"
 
 __all__ = [
     "NativeLibraryError",
+    "KLEstimator",
     "fused_lm_head_sft_loss",
     "fused_logprobs_sft_loss",
     "sft_loss_fn",

@@ -88,6 +88,7 @@ SIGNATURES = {
     "aa_prox_logp_approx": (_i, [_p, _p, _p, _i64, _i, _i, _p, _p]),
     "aa_masked_normalization_scratch_bytes": (_i64, [_i64, _i64]),
     "aa_masked_normalization": (_i, [_p, _p, _i64, _i64, _i, _d, _p, _p, _i64, _p]),
+    "aa_kl_estimate": (_i, [_p, _p, _i64, _i, _i, _p, _p]),
     "aa_overlong_penalty": (_i, [_p, _p, _i64, _i64, _i, _f, _i64, _p]),
     "aa_kd_terms": (_i, [_p, _p, _p, _p, _i64, _i, _p, _p, _p]),
     "aa_sft_loss": (_i, [_p, _p, _i64, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _p]),

@@ -245,3 +245,33 @@ def masked_normalization(x: torch.Tensor, mask: torch.Tensor | None = None, dim=
     for i, d in enumerate(perm):
         inv[d] = i
     return out.permute(inv).contiguous()
+
+
+class KLEstimator:
+    """k1 / k2 / k3 estimator of the KL divergence per token, optionally clamped to [-10, 10];
+    areal/utils/data.py:1598-1656.  Forward only (the reference uses it on detached log-probs)."""
+
+    def __init__(self, kl_estimator: str = "k1", apply_clamp: bool = True):
+        if kl_estimator not in _KL_IDS:
+            raise ValueError(f"Invalid KL estimator: {kl_estimator}. Valid choices: k1, k2, k3")
+        self.kl_estimator = kl_estimator
+        self.apply_clamp = apply_clamp
+
+    def __call__(self, log_probs: torch.Tensor, log_probs_base: torch.Tensor) -> torch.Tensor:
+        return self._compute_approx_kl(log_probs, log_probs_base, self.kl_estimator, self.apply_clamp)
+
+    @staticmethod
+    @torch.no_grad()
+    def _compute_approx_kl(log_probs: torch.Tensor, log_probs_base: torch.Tensor, kl_estimator: str = "k1",
+                           apply_clamp: bool = True) -> torch.Tensor:
+        if kl_estimator not in _KL_IDS:
+            raise ValueError(f"Invalid KL estimator: {kl_estimator}. Valid choices: k1, k2, k3")
+        _require_gpu(log_probs, "log_probs")
+        if log_probs_base.shape != log_probs.shape:
+            raise ValueError("log_probs and log_probs_base must have the same shape")
+        a, b = _f32(log_probs), _f32(log_probs_base.to(log_probs.device))
+        out = torch.empty_like(a)
+        with torch.cuda.device(a.device):
+            N.check(N.load().aa_kl_estimate(_ptr(a), _ptr(b), a.numel(), _KL_IDS[kl_estimator], 1 if apply_clamp else 0,
+                                            _ptr(out), _stream(a.device)), "aa_kl_estimate")
+        return out

@@ -510,6 +510,19 @@ __global__ __launch_bounds__(kThreads) void k_mn_apply(const float* __restrict__
   }
 }
 
+// KLEstimator (areal/utils/data.py:1598-1656) per element: k1 = d, k2 = d^2 / 2, k3 = exp(-d) - 1 + d with
+// d = logp - logp_base, optionally clamped to [-10, 10].
+__global__ __launch_bounds__(256) void k_kl_estimate(const float* __restrict__ logp, const float* __restrict__ base,
+                                                     int64_t n, int estimator, int clamp, float* __restrict__ out) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    float d = logp[i] - base[i];
+    if (estimator == 1) d = d * d / 2.0f;
+    else if (estimator == 2) { d = -d; d = expf(d) - 1.f - d; }
+    if (clamp) d = (d != d) ? d : fminf(fmaxf(d, -10.f), 10.f);
+    out[i] = d;
+  }
+}
+
 }  // namespace adv
 }  // namespace aa
 
@@ -630,5 +643,17 @@ extern "C" int aa_masked_normalization(const float* x, const float* mask, int64_
   const unsigned grid = (unsigned)(rows * parts);
   hipLaunchKernelGGL(k_mn_partial, dim3(grid), dim3(kThreads), 0, st, x, mask, cols, parts, partial);
   hipLaunchKernelGGL(k_mn_apply, dim3(grid), dim3(kThreads), 0, st, x, mask, cols, parts, partial, unbiased, eps, out);
+  return launch_status();
+}
+
+extern "C" int aa_kl_estimate(const float* logp, const float* logp_base, int64_t n, int estimator, int apply_clamp,
+                              float* out, void* stream) {
+  if (n < 0 || estimator < 0 || estimator > 2) return AA_ERR_INVALID_ARGUMENT;
+  if (n == 0) return AA_OK;
+  if (!logp || !logp_base || !out) return AA_ERR_INVALID_ARGUMENT;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(k_kl_estimate, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, logp, logp_base, n,
+                     estimator, apply_clamp ? 1 : 0, out);
   return launch_status();
 }

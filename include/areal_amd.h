@@ -276,6 +276,14 @@ int aa_prox_logp_approx(const float* old_logp, const float* logp,
                         int current_version, int method, float* out,
                         void* stream);
 
+/*
+ * KLEstimator (areal/utils/data.py:1598-1656) per element, d = logp -
+ * logp_base: estimator 0 (k1) = d, 1 (k2) = d^2 / 2, 2 (k3) = exp(-d) - 1 + d;
+ * apply_clamp != 0 clamps the result to [-10, 10].
+ */
+int aa_kl_estimate(const float* logp, const float* logp_base, int64_t n,
+                   int estimator, int apply_clamp, float* out, void* stream);
+
 /* Bytes of 256-byte aligned scratch aa_masked_normalization needs. */
 int64_t aa_masked_normalization_scratch_bytes(int64_t rows, int64_t cols);
 

@@ -248,3 +248,26 @@ def test_masked_normalization_weights_and_broadcast_mask(device):
     assert torch.allclose(got.cpu(), want, rtol=1e-5, atol=1e-6)
     got16 = areal_amd.masked_normalization(x.to(device).bfloat16(), None, dim=-1)
     assert torch.allclose(got16.cpu(), O.masked_normalization(x.bfloat16(), None, 1), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("estimator", ["k1", "k2", "k3"])
+@pytest.mark.parametrize("clamp", [True, False])
+def test_kl_estimator_matches_oracle(device, estimator, clamp):
+    from oracle import kl_estimate
+
+    g = torch.Generator().manual_seed(2)
+    a = -torch.rand(4, 333, generator=g) * 5
+    b = a + torch.randn(4, 333, generator=g) * 3          # differences large enough for the clamp to bind
+    b[0, 0] = a[0, 0] - 40.0                              # k3 overflows the clamp by far
+    want = kl_estimate(a, b, estimator)
+    if clamp:
+        want = want.clamp(min=-10, max=10)                # data.py:1654-1655
+    got = areal_amd.KLEstimator(estimator, clamp)(a.to(device), b.to(device))
+    assert got.shape == a.shape and torch.allclose(got.cpu(), want, rtol=2e-6, atol=1e-6)
+    # the numbers the reference's tests quote (tests/test_rejection_sampling.py:507-546): log-ratios 0.5, -0.5, 2.0
+    d = torch.tensor([0.5, -0.5, 2.0], device=device)
+    val = areal_amd.KLEstimator(estimator, clamp)(d, torch.zeros(3, device=device)).tolist()
+    quoted = {"k1": [0.5, -0.5, 2.0], "k2": [0.125, 0.125, 2.0], "k3": [0.1065, 0.1487, 1.1353]}[estimator]
+    assert val == pytest.approx(quoted, abs=1e-4)
+    with pytest.raises(ValueError, match="Invalid KL estimator"):
+        areal_amd.KLEstimator("k4")
