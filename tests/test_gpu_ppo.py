@@ -123,7 +123,7 @@ def test_ppo_loss_and_gradient_match_oracle(device, kw, level):
         (got_loss * 1.0).backward()
         assert got_loss.ndim == 0 and got_loss.dtype == torch.float32
         assert float(got_loss.detach()) == pytest.approx(float(want_loss.detach()), rel=1e-3, abs=1e-6)   # stated tolerance
-        assert float(got_loss) == pytest.approx(float(want_loss), rel=2e-5, abs=1e-6)   # what it delivers
+        assert float(got_loss.detach()) == pytest.approx(float(want_loss.detach()), rel=2e-5, abs=1e-6)   # what it delivers
         assert set(got) == set(want)
         for k in ("clip_mask", "dual_clip_mask") + (("behave_mask",) if cfg else ()):
             assert got[k].dtype == torch.bool and torch.equal(got[k].cpu(), want[k]), k
