@@ -58,3 +58,44 @@ def test_argument_validation_without_gpu():
     assert lib.aa_logits_fwd(null, 0, 1, 8, 8, null, 1.0, null, null, null, null, null, null, null) == 1
     assert lib.aa_copy_bytes(null, null, 16, null) == 1
     assert lib.aa_masked_sum(null, null, -1, null, null, null, null) == 1
+
+
+def test_argument_validation_of_the_sibling_entry_points_without_gpu():
+    """The losses, reductions and layout entry points return AA_ERR_INVALID_ARGUMENT (or AA_OK for empty input) before
+    any launch: null outputs, negative sizes, enum values out of range."""
+    lib = _native.load()
+    z = ctypes.c_void_p(0)
+    p = ctypes.c_void_p(256)        # a non-null address that is never dereferenced on the host
+    bad, ok = 1, 0
+    assert lib.aa_kl_estimate(p, p, -1, 0, 0, p, z) == bad
+    assert lib.aa_kl_estimate(p, p, 4, 3, 0, p, z) == bad
+    assert lib.aa_kl_estimate(z, z, 0, 0, 0, z, z) == ok
+    assert lib.aa_dpo_seq_sums(p, p, p, p, -1, 4, p, p, p, z) == bad
+    assert lib.aa_dpo_seq_sums(p, p, p, z, 2, 4, p, p, p, z) == bad
+    assert lib.aa_dpo_seq_sums(z, z, z, z, 0, 0, z, z, z, z) == ok
+    assert lib.aa_dpo_seq_sums_bwd(z, z, p, p, 2, 4, p, z) == bad
+    assert lib.aa_dpo_preference_loss(p, 4, 0.1, 2, p, z, z) == bad
+    assert lib.aa_dpo_preference_loss(p, 4, 0.1, 0, z, z, z) == bad
+    assert lib.aa_dpo_preference_loss(z, 0, 0.1, 0, z, z, z) == ok
+    assert lib.aa_dpo_pair_loss(p, p, p, p, 2, 0.1, 0, z, p, p, p, p, p, p, z) == bad
+    assert lib.aa_dpo_pair_loss(p, p, p, p, 2, 0.1, 5, p, p, p, p, p, p, p, z) == bad
+    assert lib.aa_rw_pair_loss(p, 4, z, 1, p, p, p, p, p, p, z, z) == bad
+    assert lib.aa_rw_pair_loss(z, 4, p, 1, p, p, p, p, p, p, z, z) == bad
+    assert lib.aa_sft_loss(p, p, 4, z, 2, p, z, p, z, z, p, p, z, z) == bad       # sequences without cu_seqlens
+    assert lib.aa_sft_loss(p, p, 4, p, 2, z, z, p, z, z, p, p, z, z) == bad       # no token count
+    assert lib.aa_sft_loss(z, z, 4, p, 2, p, z, p, z, z, p, p, z, z) == bad
+    assert lib.aa_logging_stats(p, p, z, z, p, 4, 0, 1, 0, p, p, 1 << 20, z) == bad    # a method without versions
+    assert lib.aa_logging_stats(p, p, z, p, p, 4, 0, 7, 1, p, p, 1 << 20, z) == bad    # errors without ground truth
+    assert lib.aa_logging_stats(p, p, z, p, p, 4, 0, 8, 0, p, p, 1 << 20, z) == bad
+    assert lib.aa_logging_stats(p, p, z, p, p, 4, 0, 1, 0, p, p, 8, z) == bad          # scratch too small
+    assert lib.aa_logging_stats_scratch_bytes(-1) == -1 and lib.aa_logging_stats_scratch_bytes(100000) > 0
+    assert lib.aa_masked_normalization(p, z, 2, 8, 0, 1e-5, p, p, 8, z) == bad         # scratch too small
+    assert lib.aa_masked_normalization(z, z, 0, 8, 0, 1e-5, z, z, 0, z) == ok
+    assert lib.aa_masked_normalization_scratch_bytes(4, -1) == -1
+    assert lib.aa_overlong_penalty(p, p, 4, 8, 0, 1.0, 100, z) == bad                   # division by overlong_tokens
+    assert lib.aa_kd_terms(p, z, p, p, 4, 1, p, p, z) == bad                            # pure form without old log-probs
+    params = _native.PpoParams(clip_lo=0.8, clip_hi=1.2, loss_kind=2)
+    assert lib.aa_logits_ppo_fused(p, 0, 4, 4096, 4096, p, 1.0, 4, p, p, p, z, ctypes.byref(params), p, z, p, z, z, z,
+                                   p, p, p, p, z, z) == bad                             # unknown loss kind
+    params = _native.PpoParams(clip_lo=0.8, clip_hi=1.2, loss_kind=1)
+    assert lib.aa_ppo_loss(p, p, p, p, z, 4, z, 0, 0, ctypes.byref(params), p, p, p, p, p, z) == 2   # unsupported
