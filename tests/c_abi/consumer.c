@@ -1,0 +1,146 @@
+/*
+ * A consumer of the C ABI written in plain C, with nothing but the HIP runtime beside it: device buffers from
+ * hipMalloc, the library's entry points, and the expected values computed right here in double precision from the
+ * definitions (log-softmax, entropy, the supervised loss and its gradient).  Exit status 0 = every check passed.
+ *
+ * Build (done by __graft_entry__.build()):
+ *   gcc -std=c99 -D__HIP_PLATFORM_AMD__ -I/opt/rocm/include -Iinclude tests/c_abi/consumer.c \
+ *       -o tests/c_abi/consumer -Lareal_amd -lareal_amd -L/opt/rocm/lib -lamdhip64 -lm -Wl,-rpath,...
+ */
+#include <hip/hip_runtime_api.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "areal_amd.h"
+
+#define T 7
+#define V 1003
+
+#define HIP_OK(call)                                                                 \
+  do {                                                                               \
+    hipError_t e_ = (call);                                                          \
+    if (e_ != hipSuccess) {                                                          \
+      fprintf(stderr, "%s failed: %s\n", #call, hipGetErrorString(e_));              \
+      return 2;                                                                      \
+    }                                                                                \
+  } while (0)
+
+#define AA_CHECK(call)                                                               \
+  do {                                                                               \
+    int s_ = (call);                                                                 \
+    if (s_ != AA_OK) {                                                               \
+      fprintf(stderr, "%s failed: %s\n", #call, aa_status_string(s_));               \
+      return 3;                                                                      \
+    }                                                                                \
+  } while (0)
+
+static int close_to(double got, double want, double tol, const char* what, int t) {
+  if (fabs(got - want) <= tol * (1.0 + fabs(want))) return 1;
+  fprintf(stderr, "%s[%d]: got %.9g, expected %.9g\n", what, t, got, want);
+  return 0;
+}
+
+int main(void) {
+  static float logits[T * V];
+  int64_t labels[T];
+  uint8_t mask[T] = {0, 1, 1, 0, 1, 1, 1};
+  const float inv_temperature = 1.0f / 0.8f;
+  uint32_t state = 12345u;
+  for (int i = 0; i < T * V; ++i) {  /* a small linear congruential generator: values in [-4, 4) */
+    state = state * 1664525u + 1013904223u;
+    logits[i] = (float)(state >> 8) / (float)(1u << 24) * 8.0f - 4.0f;
+  }
+  for (int t = 0; t < T; ++t) labels[t] = (t * 131 + 7) % V;
+
+  /* expected values from the definitions, in double */
+  double want_logp[T], want_entropy[T];
+  int n_valid = 0;
+  for (int t = 0; t < T; ++t) {
+    double mx = -1e300, s = 0.0, u = 0.0;
+    for (int j = 0; j < V; ++j) mx = fmax(mx, (double)logits[t * V + j] * inv_temperature);
+    for (int j = 0; j < V; ++j) {
+      const double z = (double)logits[t * V + j] * inv_temperature;
+      s += exp(z - mx);
+      u += exp(z - mx) * z;
+    }
+    const double lse = mx + log(s);
+    want_logp[t] = (double)logits[t * V + labels[t]] * inv_temperature - lse;
+    want_entropy[t] = lse - u / s;
+    n_valid += mask[t] ? 1 : 0;
+  }
+  double want_loss = 0.0;
+  for (int t = 0; t < T; ++t) want_loss -= mask[t] ? want_logp[t] : 0.0;
+  want_loss /= (double)n_valid + 1e-5;
+
+  float *d_logits, *d_logp, *d_entropy, *d_loss, *d_g, *d_stat, *d_ppl;
+  int64_t* d_labels;
+  uint8_t* d_mask;
+  int32_t *d_count, *d_cu, *d_seq_count;
+  double* d_seq_logp;
+  const int32_t cu[3] = {0, 3, T};
+  HIP_OK(hipMalloc((void**)&d_logits, sizeof(logits)));
+  HIP_OK(hipMalloc((void**)&d_labels, sizeof(labels)));
+  HIP_OK(hipMalloc((void**)&d_mask, 256));
+  HIP_OK(hipMalloc((void**)&d_logp, T * sizeof(float)));
+  HIP_OK(hipMalloc((void**)&d_entropy, T * sizeof(float)));
+  HIP_OK(hipMalloc((void**)&d_g, T * sizeof(float)));
+  HIP_OK(hipMalloc((void**)&d_stat, T * sizeof(float)));
+  HIP_OK(hipMalloc((void**)&d_loss, 256));
+  HIP_OK(hipMalloc((void**)&d_ppl, 256));
+  HIP_OK(hipMalloc((void**)&d_count, 256));
+  HIP_OK(hipMalloc((void**)&d_cu, 256));
+  HIP_OK(hipMalloc((void**)&d_seq_count, 256));
+  HIP_OK(hipMalloc((void**)&d_seq_logp, 256));
+  HIP_OK(hipMemcpy(d_logits, logits, sizeof(logits), hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_labels, labels, sizeof(labels), hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_mask, mask, sizeof(mask), hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_cu, cu, sizeof(cu), hipMemcpyHostToDevice));
+
+  if (aa_version() < 100) return 4;
+  /* the log-prob op, the token count, the supervised loss on the log-probs: all on the default stream */
+  AA_CHECK(aa_logits_fwd(d_logits, AA_F32, T, V, V, d_labels, inv_temperature, d_logp, d_entropy, NULL, NULL, NULL,
+                         NULL, NULL));
+  AA_CHECK(aa_count_nonzero_u8(d_mask, T, d_count, NULL));
+  AA_CHECK(aa_sft_loss(d_logp, d_mask, T, d_cu, 2, d_count, NULL, d_loss, d_g, d_stat, d_seq_logp, d_seq_count, d_ppl,
+                       NULL));
+  HIP_OK(hipDeviceSynchronize());
+
+  float logp[T], entropy[T], g[T], loss, ppl[2];
+  int32_t count, seq_count[3];
+  double seq_logp[3];
+  HIP_OK(hipMemcpy(logp, d_logp, sizeof(logp), hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(entropy, d_entropy, sizeof(entropy), hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(g, d_g, sizeof(g), hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(&loss, d_loss, sizeof(loss), hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(&count, d_count, sizeof(count), hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(ppl, d_ppl, sizeof(ppl), hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(seq_count, d_seq_count, sizeof(seq_count), hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(seq_logp, d_seq_logp, sizeof(seq_logp), hipMemcpyDeviceToHost));
+
+  int ok = count == n_valid;
+  for (int t = 0; t < T; ++t) {
+    ok &= close_to(logp[t], want_logp[t], 2e-6, "logp", t);
+    ok &= close_to(entropy[t], want_entropy[t], 2e-6, "entropy", t);
+    ok &= close_to(g[t], mask[t] ? -1.0 / ((double)n_valid + 1e-5) : 0.0, 1e-6, "g_logp", t);
+  }
+  ok &= close_to(loss, want_loss, 2e-6, "loss", 0);
+  /* sequence 0 = tokens 0..2 (two selected), sequence 1 = tokens 3..6 (three selected) */
+  ok &= seq_count[0] == 2 && seq_count[1] == 3 && seq_count[2] == 0;
+  ok &= close_to(seq_logp[0], (want_logp[1] + want_logp[2]) / 2.0, 2e-6, "seq_logp", 0);
+  ok &= close_to(seq_logp[1], (want_logp[4] + want_logp[5] + want_logp[6]) / 3.0, 2e-6, "seq_logp", 1);
+  ok &= close_to(ppl[0], exp(-(want_logp[1] + want_logp[2]) / 2.0), 1e-5, "ppl", 0);
+
+  /* a bad argument is refused before anything is queued */
+  ok &= aa_logits_fwd(d_logits, AA_F32, T, V, V, d_labels, 0.0f, d_logp, NULL, NULL, NULL, NULL, NULL, NULL) ==
+        AA_ERR_INVALID_ARGUMENT;
+
+  hipFree(d_logits); hipFree(d_labels); hipFree(d_mask); hipFree(d_logp); hipFree(d_entropy); hipFree(d_g);
+  hipFree(d_stat); hipFree(d_loss); hipFree(d_ppl); hipFree(d_count); hipFree(d_cu); hipFree(d_seq_count);
+  hipFree(d_seq_logp);
+  if (!ok) return 1;
+  printf("c_abi consumer ok: %d tokens, loss %.6f\n", T, loss);
+  return 0;
+}

@@ -171,3 +171,16 @@ def test_backward_matches_autograd_of_oracle(device, T, V, dtype, temperature, w
     if not with_entropy:
         assert float(got[0].float().abs().max()) == 0.0
         assert float(got.float().sum(-1).abs().max()) < 5e-2  # each row of (onehot - p) sums to zero
+
+
+def test_plain_c_consumer_of_the_abi(device):
+    """tests/c_abi/consumer.c drives the library from C99 with hipMalloc'ed buffers and checks log-probs, entropy, the
+    supervised loss, its gradient and the per-sequence statistics against values it computes itself in double."""
+    import subprocess
+    from pathlib import Path
+
+    exe = Path(__file__).resolve().parent / "c_abi" / "consumer"
+    assert exe.exists(), "build it first: python -c 'import __graft_entry__ as g; g.build_c_abi_consumer()'"
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0, run.stdout + run.stderr
+    assert "c_abi consumer ok" in run.stdout
