@@ -404,36 +404,43 @@ __device__ __forceinline__ float fused_token_tail(const FusedTokenArgs& a, int64
   return (s.dloss_dr * r / fn) * gscale;
 }
 
+constexpr int64_t kWalkRowBytes = 256 * 1024;  // rows at least this long are walked by kWalkGroups workgroups
+constexpr int kWalkGroups = 512;               // two per compute unit
+
 template <int DT, int NT>
-__global__ __launch_bounds__(NT) void k_fused_generic(const void* __restrict__ logits, int V, int64_t stride,
-                                                      const int64_t* __restrict__ labels, float inv_t, int vec_ok,
-                                                      FusedTokenArgs a, void* __restrict__ dlogits) {
+__global__ __launch_bounds__(NT) void k_fused_generic(const void* __restrict__ logits, int64_t T_rows, int V,
+                                                      int64_t stride, const int64_t* __restrict__ labels, float inv_t,
+                                                      int vec_ok, FusedTokenArgs a, void* __restrict__ dlogits) {
   __shared__ float smem[(NT / kWave) * 5];
-  const int64_t t = blockIdx.x;
-  const int64_t orow = a.out_rows ? (int64_t)a.out_rows[t] : t;
-  const void* row = row_ptr(logits, t, stride, Elem<DT>::kBytes);
-  void* out = (void*)row_ptr(dlogits, orow < 0 ? 0 : orow, stride, Elem<DT>::kBytes);
   const float c = kLog2e * inv_t;
-  const int64_t y = labels[t];
-  const bool y_ok = (y >= 0) && (y < V);
-  const float xy = y_ok ? Elem<DT>::load1(row, y) : 0.f;
-  TokenIn tin{0.f, 0.f, 1.f, 0, false};
-  if (a.T_active > 0) tin = load_token_in(a, t);
   float fn, gscale;
   load_loss_scale(a, fn, gscale);
-  const RowStats rs = row_stats_generic<DT, NT>(row, V, vec_ok != 0, c, smem);
-  const RowOut ro = finish_row(rs);
-  const float lp = y_ok ? label_logp(xy, c, rs, ro) : __builtin_nanf("");
-  const float g = fused_token_tail(a, t, tin, fn, gscale, lp, rs, ro, threadIdx.x == 0);
-  if (orow < 0) return;  // uniform over the workgroup
-  if (g == 0.f) {
-    row_zero_generic<DT, NT>(row, out, V, vec_ok != 0);
-    return;
+  // one row per trip; with fewer workgroups than rows (T_rows > gridDim.x) a workgroup walks rows t, t + grid, ...
+  for (int64_t t = blockIdx.x; t < T_rows; t += gridDim.x) {
+    const int64_t orow = a.out_rows ? (int64_t)a.out_rows[t] : t;
+    const void* row = row_ptr(logits, t, stride, Elem<DT>::kBytes);
+    void* out = (void*)row_ptr(dlogits, orow < 0 ? 0 : orow, stride, Elem<DT>::kBytes);
+    const int64_t y = labels[t];
+    const bool y_ok = (y >= 0) && (y < V);
+    const float xy = y_ok ? Elem<DT>::load1(row, y) : 0.f;
+    TokenIn tin{0.f, 0.f, 1.f, 0, false};
+    if (a.T_active > 0) tin = load_token_in(a, t);
+    const RowStats rs = row_stats_generic<DT, NT>(row, V, vec_ok != 0, c, smem);
+    const RowOut ro = finish_row(rs);
+    const float lp = y_ok ? label_logp(xy, c, rs, ro) : __builtin_nanf("");
+    const float g = fused_token_tail(a, t, tin, fn, gscale, lp, rs, ro, threadIdx.x == 0);
+    if (orow >= 0) {  // uniform over the workgroup
+      if (g == 0.f) {
+        row_zero_generic<DT, NT>(row, out, V, vec_ok != 0);
+      } else {
+        GradCoef gc;
+        gc.c = c; gc.lse2 = ro.lse2; gc.A = -g * inv_t; gc.B = 0.f; gc.lab_add = g * inv_t;
+        gc.label = y_ok ? (int)y : -1;
+        row_grad_generic<DT, NT>(row, out, V, vec_ok != 0, gc);
+      }
+    }
+    __syncthreads();  // the statistics scratch is reused by the next row
   }
-  GradCoef gc;
-  gc.c = c; gc.lse2 = ro.lse2; gc.A = -g * inv_t; gc.B = 0.f; gc.lab_add = g * inv_t;
-  gc.label = y_ok ? (int)y : -1;
-  row_grad_generic<DT, NT>(row, out, V, vec_ok != 0, gc);
 }
 
 // -----------------------------------------------------------------------------
@@ -1009,10 +1016,19 @@ int aa::logits_ppo_fused_rows(const void* logits, int dtype, int64_t T, int64_t 
     if (ok) return launch_status();
   }
   const int vec_ok = rows_vec_ok(logits, dlogits, dtype) ? 1 : 0;
-  constexpr int NT = 256;
-#define AA_LAUNCH(DT)                                                                                           \
-  hipLaunchKernelGGL((k_fused_generic<DT, NT>), dim3((unsigned)T), dim3(NT), 0, st, logits, (int)V, row_stride, \
-                     labels, inv_temperature, vec_ok, a, dlogits)
+  // A row is read twice (statistics, then gradient).  Long rows: few, large workgroups that walk the rows, so that
+  // the rows in flight (one per workgroup) stay small enough for the second read to come from the caches.
+  const int64_t row_bytes = V * (dtype == AA_F32 ? 4 : 2);
+  const bool walk = row_bytes >= kWalkRowBytes && T > kWalkGroups;
+#define AA_LAUNCH(DT)                                                                                              \
+  do {                                                                                                             \
+    if (walk)                                                                                                      \
+      hipLaunchKernelGGL((k_fused_generic<DT, 1024>), dim3((unsigned)kWalkGroups), dim3(1024), 0, st, logits, T,   \
+                         (int)V, row_stride, labels, inv_temperature, vec_ok, a, dlogits);                         \
+    else                                                                                                           \
+      hipLaunchKernelGGL((k_fused_generic<DT, 256>), dim3((unsigned)T), dim3(256), 0, st, logits, T, (int)V,       \
+                         row_stride, labels, inv_temperature, vec_ok, a, dlogits);                                 \
+  } while (0)
   if (dtype == AA_BF16) AA_LAUNCH(AA_BF16);
   else if (dtype == AA_F16) AA_LAUNCH(AA_F16);
   else AA_LAUNCH(AA_F32);

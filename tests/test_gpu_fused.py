@@ -93,6 +93,17 @@ def test_fused_config0_shape_matches_oracle(device, V, dtype, lo, hi):
     _compare(case, _fused_step(case), _oracle_step(case))
 
 
+def test_fp32_long_rows_walked_by_large_workgroups(device):
+    """fp32 rows of 256 KB or more with more rows than walking workgroups: every workgroup handles several rows."""
+    lengths = synth.lengths_uniform(40, 8, 24, seed=5)            # about 640 tokens > 512 workgroups
+    V = 70000                                                     # 280 KB per fp32 row
+    case = synth.make_logits_case("t", lengths, V, V, device, synth.per_sequence_normal_advantages(lengths, 3),
+                                  dtype=torch.float32, ppo=dict(eps_clip=0.2))
+    assert case.n_tokens > 512
+    _finish_case(case)
+    _compare(case, _fused_step(case), _oracle_step(case))
+
+
 def test_long_rows_labels_and_extrema_in_every_region(device):
     """V = 262144: labels and the row maximum / minimum placed in the register, LDS and streamed parts of the row."""
     V = 262144

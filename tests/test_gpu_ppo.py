@@ -163,7 +163,7 @@ def test_edge_cases(device):
     z = torch.randn(2, 4, device=device)
     none = torch.zeros(2, 4, dtype=torch.bool, device=device)
     loss, stat = areal_amd.ppo_actor_loss_fn(z.clone().requires_grad_(True), z, z, z, 0.2, none)
-    assert float(loss) == 0.0 and float(stat["importance_weight"].abs().sum()) == 0.0
+    assert float(loss.detach()) == 0.0 and float(stat["importance_weight"].abs().sum()) == 0.0
     assert "behave_imp_weight" not in stat and "filtered_fraction" not in stat
     with pytest.raises(ValueError, match="cu_seqlens is required for 1D tensors"):
         areal_amd.ppo_actor_loss_fn(z[0], z[0], z[0], z[0], 0.2, ~none[0], importance_sampling_level="sequence")
