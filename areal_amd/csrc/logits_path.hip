@@ -444,6 +444,113 @@ __global__ __launch_bounds__(NT) void k_fused_generic(const void* __restrict__ l
 }
 
 // -----------------------------------------------------------------------------
+// Fused kernel for fp32 logits: a row is too long for the register file alone (608 KB at V = 151 936 against
+// 512 KB), so the first kHoldReg chunks of a row (8 floats per thread and chunk) stay in registers, the next
+// kHoldLds chunks in LDS, and only what is left is read a second time for the gradient.  At V = 151 936 that is
+// 22 % of the row: 8.9 bytes per element through the fabric instead of the 12 of the two-pass kernel (8 is the
+// floor); rows up to 81 920 elements are read once.  One workgroup of 1024 threads per compute unit (the LDS
+// share allows no second one), walking rows t, t + grid, ...  Needs V % 8 == 0 and 16-byte aligned rows.
+// -----------------------------------------------------------------------------
+constexpr int kHoldReg = 10;                        // 10 x 8192 floats in registers (80 VGPRs per thread)
+constexpr int kHoldLds = 4;                         // 4 x 8192 floats in LDS (128 KB)
+constexpr int kHoldChunk = 8 * 1024;                // floats per chunk: 8 per thread
+
+__global__ __launch_bounds__(1024) void k_fused_f32_hold(const float* __restrict__ logits, int64_t T_rows, int V,
+                                                         int64_t stride, const int64_t* __restrict__ labels,
+                                                         float inv_t, FusedTokenArgs a, float* __restrict__ dlogits) {
+  __shared__ float smem[16 * 5];
+  __shared__ float4 held[kHoldLds * 2 * 1024];      // [chunk][half][thread]: consecutive lanes, consecutive 16 bytes
+  const int tid = threadIdx.x;
+  const float c = kLog2e * inv_t;
+  float fn, gscale;
+  load_loss_scale(a, fn, gscale);
+  for (int64_t t = blockIdx.x; t < T_rows; t += gridDim.x) {
+    const int64_t orow = a.out_rows ? (int64_t)a.out_rows[t] : t;
+    const float* row = logits + t * stride;
+    float* out = dlogits + (orow < 0 ? 0 : orow) * stride;
+    const int64_t y = labels[t];
+    const bool y_ok = (y >= 0) && (y < V);
+    const float xy = y_ok ? row[y] : 0.f;
+    TokenIn tin{0.f, 0.f, 1.f, 0, false};
+    if (a.T_active > 0) tin = load_token_in(a, t);
+
+    // pass 1: statistics of the whole row; the head of the row stays on the chip
+    ThreadStats st{kNegBig, 0.f, 0.f, -FLT_MAX, FLT_MAX};
+    float xr[kHoldReg][8];
+#pragma unroll
+    for (int k = 0; k < kHoldReg; ++k) {
+      const int e0 = k * kHoldChunk + tid * 8;
+      if (e0 < V) {
+        load8<AA_F32>(row, e0, xr[k]);
+        stats_add8(st, xr[k], c);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kHoldLds; ++k) {
+      const int e0 = (kHoldReg + k) * kHoldChunk + tid * 8;
+      if (e0 < V) {
+        float x[8];
+        load8<AA_F32>(row, e0, x);
+        held[(k * 2 + 0) * 1024 + tid] = make_float4(x[0], x[1], x[2], x[3]);
+        held[(k * 2 + 1) * 1024 + tid] = make_float4(x[4], x[5], x[6], x[7]);
+        stats_add8(st, x, c);
+      }
+    }
+    for (int e0 = (kHoldReg + kHoldLds) * kHoldChunk + tid * 8; e0 < V; e0 += kHoldChunk) {
+      float x[8];
+      load8<AA_F32>(row, e0, x);
+      stats_add8(st, x, c);
+    }
+    const RowStats rs = block_stats<16>(st, smem);
+    const RowOut ro = finish_row(rs);
+    const float lp = y_ok ? label_logp(xy, c, rs, ro) : __builtin_nanf("");
+    const float g = fused_token_tail(a, t, tin, fn, gscale, lp, rs, ro, tid == 0);
+
+    // pass 2: the gradient row (every thread reads back only what it stored itself: no barrier needed)
+    if (orow >= 0) {  // uniform over the workgroup
+      if (g == 0.f) {
+        const float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int e0 = tid * 8; e0 < V; e0 += kHoldChunk) store8<AA_F32>(out, e0, z);
+      } else {
+        const float A = -g * inv_t, lab_add = g * inv_t, lse2 = ro.lse2;
+        const int label = y_ok ? (int)y : -1;
+        auto emit = [&](int e0, const float (&x)[8]) {
+          float o[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) o[i] = fast_exp2(fmaf(x[i], c, -lse2)) * A;
+          if ((unsigned)(label - e0) < 8u) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+              if (e0 + i == label) o[i] += lab_add;
+          }
+          store8<AA_F32>(out, e0, o);
+        };
+#pragma unroll
+        for (int k = 0; k < kHoldReg; ++k) {
+          const int e0 = k * kHoldChunk + tid * 8;
+          if (e0 < V) emit(e0, xr[k]);
+        }
+#pragma unroll
+        for (int k = 0; k < kHoldLds; ++k) {
+          const int e0 = (kHoldReg + k) * kHoldChunk + tid * 8;
+          if (e0 < V) {
+            const float4 lo = held[(k * 2 + 0) * 1024 + tid], hi = held[(k * 2 + 1) * 1024 + tid];
+            const float x[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            emit(e0, x);
+          }
+        }
+        for (int e0 = (kHoldReg + kHoldLds) * kHoldChunk + tid * 8; e0 < V; e0 += kHoldChunk) {
+          float x[8];
+          load8<AA_F32>(row, e0, x);
+          emit(e0, x);
+        }
+      }
+    }
+    __syncthreads();  // the statistics scratch is reused by the next row
+  }
+}
+
+// -----------------------------------------------------------------------------
 // Fused kernel, register-resident row: 1024 threads hold one row of 16-bit
 // logits as NCH 16-byte chunks per thread, so HBM sees exactly one read of the
 // row and one write of its gradient.  Requires V % 8 == 0, 16-byte aligned
@@ -1014,6 +1121,14 @@ int aa::logits_ppo_fused_rows(const void* logits, int dtype, int64_t T, int64_t 
                ? launch_regs_ext<AA_BF16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st)
                : launch_regs_ext<AA_F16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st);
     if (ok) return launch_status();
+  }
+  if (dtype == AA_F32 && (V % 8 == 0) && (row_stride % 4 == 0) && V >= kHoldChunk &&
+      ((((uintptr_t)logits | (uintptr_t)dlogits) & 15) == 0)) {
+    const int cus = persistent_workgroups();
+    const unsigned grid = (unsigned)(T < cus ? T : cus);
+    hipLaunchKernelGGL(k_fused_f32_hold, dim3(grid), dim3(1024), 0, st, (const float*)logits, T, (int)V, row_stride,
+                       labels, inv_temperature, a, (float*)dlogits);
+    return launch_status();
   }
   const int vec_ok = rows_vec_ok(logits, dlogits, dtype) ? 1 : 0;
   // A row is read twice (statistics, then gradient).  Long rows: few, large workgroups that walk the rows, so that

@@ -78,6 +78,10 @@ def _compare(case, got, want, pad=0):
         (8200, torch.float16, 8, 40),      # 2 chunks, the second almost empty
         (50257, torch.bfloat16, 4, 20),    # generic rows (V % 8 != 0)
         (4099, torch.float32, 4, 20),      # generic rows, fp32 logits
+        (8192, torch.float32, 4, 12),      # fp32 rows held on the chip: exactly one register chunk
+        (81928, torch.float32, 4, 12),     # registers full, one vector in LDS
+        (114696, torch.float32, 4, 12),    # registers and LDS full, one vector read twice
+        (151936, torch.float32, 4, 12),    # benchmark vocabulary in fp32: 22 % of the row read twice
         (172040, torch.bfloat16, 4, 12),   # 22 chunks: 21 in registers, one (a single 16-byte piece of it) in LDS
         (245760, torch.bfloat16, 4, 12),   # 30 chunks: registers and LDS full, no tail
         (250008, torch.float16, 4, 12),    # 31 chunks: a partial streamed tail chunk
@@ -93,10 +97,12 @@ def test_fused_config0_shape_matches_oracle(device, V, dtype, lo, hi):
     _compare(case, _fused_step(case), _oracle_step(case))
 
 
-def test_fp32_long_rows_walked_by_large_workgroups(device):
-    """fp32 rows of 256 KB or more with more rows than walking workgroups: every workgroup handles several rows."""
-    lengths = synth.lengths_uniform(40, 8, 24, seed=5)            # about 640 tokens > 512 workgroups
-    V = 70000                                                     # 280 KB per fp32 row
+@pytest.mark.parametrize("V", [70004, 90112])
+def test_fp32_long_rows_walked_by_large_workgroups(device, V):
+    """More fp32 rows than workgroups, so every workgroup handles several rows: V = 70004 (not a multiple of 8, rows
+    of 280 KB) takes the two-pass kernel with 512 walking workgroups, V = 90112 the kernel that holds the row on the
+    chip with one workgroup per compute unit."""
+    lengths = synth.lengths_uniform(40, 8, 24, seed=5)            # about 640 tokens
     case = synth.make_logits_case("t", lengths, V, V, device, synth.per_sequence_normal_advantages(lengths, 3),
                                   dtype=torch.float32, ppo=dict(eps_clip=0.2))
     assert case.n_tokens > 512
