@@ -76,6 +76,9 @@ def parse_args():
                     help="lm_head workloads, outside the reference's semantics: masked tokens skip the lm_head "
                          "altogether (fused_lm_head_ppo_loss(forward_masked_tokens=False)); only ms_per_step and value "
                          "reflect it, and the line says so in config.path")
+    ap.add_argument("--logits-dtype", choices=["bf16", "f32"], default="bf16",
+                    help="logits workloads: hand the kernels fp32 logits (what a Megatron-style head emits) instead of "
+                         "bf16; 8 bytes per element instead of 4")
     ap.add_argument("--copy-launches", type=int, default=0,
                     help="also launch the plain copy kernel this many times over the logits buffer "
                          "(the calibration point for FETCH_SIZE / WRITE_SIZE counters)")
@@ -183,7 +186,7 @@ def time_fused_logits_kernel(case, kw, cfg, iters: int):
     def launch():
         N.check(
             lib.aa_logits_ppo_fused(
-                F._ptr(case.logits), N.AA_BF16, T, V, V, F._ptr(case.labels), 1.0 / case.temperature, T,
+                F._ptr(case.logits), F._DTYPES[case.logits.dtype], T, V, V, F._ptr(case.labels), 1.0 / case.temperature, T,
                 F._ptr(prox), F._ptr(adv), F._ptr(mask_eff), F._ptr(w), C.byref(params), F._ptr(counts), None,
                 F._ptr(logp), F._ptr(ent), None, None, F._ptr(sl), F._ptr(ratio), F._ptr(flags), F._ptr(dlogits),
                 F._ptr(F._work_words(dev)), C.c_void_p(stream.cuda_stream),
@@ -276,6 +279,10 @@ def bench_logits(args, dev):
     case, desc = build_logits_case(args.workload, args.seed, dev)
     kw, cfg = ppo_kwargs(case)
     T, V = case.logits.shape
+    f32 = args.logits_dtype == "f32"
+    if f32:
+        case.logits = case.logits.float()
+        desc += "; logits cast to fp32"
     case.logits.requires_grad_(True)
     run_logits_steps(case, args.warmup, kw, cfg)
     torch.cuda.synchronize()
@@ -288,20 +295,21 @@ def bench_logits(args, dev):
     case.logits.grad = None
     case.logits.requires_grad_(False)
     k_ms, k_min_ms = time_fused_logits_kernel(case, kw, cfg, max(args.steps, 10))
-    alg_bytes = 4.0 * T * V
+    alg_bytes = (8.0 if f32 else 4.0) * T * V
     achieved = alg_bytes / (k_ms * 1e-3) / 1e9
     roofline = dict(
-        bound="hbm", kernel="k_fused_regs (aa_logits_ppo_fused)", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s",
-        frac=achieved / HBM_PEAK_GBS,
+        bound="hbm", kernel=("k_fused_f32_hold" if f32 else "k_fused_regs") + " (aa_logits_ppo_fused)",
+        achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
         # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters read
-        # for the plain copy kernel: 1.001 x the algorithmic bytes (profiles/k_fused_regs_cfg1-32k_hbm_traffic.md)
-        traffic=alg_bytes * 1.001, avg_kernel_ms=k_ms, min_kernel_ms=k_min_ms,
+        # for the plain copy kernel: 1.001 x the algorithmic bytes (profiles/k_fused_regs_cfg1-32k_hbm_traffic.md);
+        # not measured for fp32 logits
+        traffic=None if f32 else alg_bytes * 1.001, avg_kernel_ms=k_ms, min_kernel_ms=k_min_ms,
         algorithmic_bytes_per_launch=alg_bytes,
     )
     out = dict(
         metric=METRIC, value=T / (ms_per_step * 1e-3), unit="tokens/s",
         n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=ms_per_step, higher_is_better=True,
-        scaling="weak", vs_baseline=None, dtype="bf16", data="synthetic",
+        scaling="weak", vs_baseline=None, dtype="f32" if f32 else "bf16", data="synthetic",
         config=dict(workload=f"{case.name}: {desc}", tokens=T, vocab=V, sequences=int(case.cu_seqlens.numel() - 1),
                     accumulate="f32", path="logits (fused fwd + PPO loss + bwd, one launch)"),
         roofline=roofline,
