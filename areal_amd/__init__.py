@@ -38,6 +38,8 @@ from .tree import (
     gather_logprobs_entropy_pairs,
     gather_packed_tree_logprobs,
     gather_packed_tree_logprobs_entropy,
+    gather_packed_tree_vocab_stats,
+    merge_packed_tree_results,
     tree_sequence_pairs,
 )
 from .sft import fused_lm_head_sft_loss, fused_logprobs_sft_loss, sft_loss_fn
@@ -47,6 +49,8 @@ __version__ = "0.1.0"
 
 __all__ = [
     "NativeLibraryError",
+    "gather_packed_tree_vocab_stats",
+    "merge_packed_tree_results",
     "KLEstimator",
     "fused_lm_head_sft_loss",
     "fused_logprobs_sft_loss",

@@ -154,3 +154,70 @@ def gather_packed_tree_logprobs(logits: torch.Tensor, trie: Any, input_ids: torc
                                 chunk_size: int = 1024, tp_group=None) -> torch.Tensor:
     """Log-probs only; functional.py:403-427."""
     return gather_packed_tree_logprobs_entropy(logits, trie, input_ids, temperature, chunk_size, tp_group)[0]
+
+
+@torch.no_grad()
+def gather_packed_tree_vocab_stats(logits: torch.Tensor, trie: Any) -> tuple[torch.Tensor, torch.Tensor]:
+    """``(vocab_min_logits, vocab_max_logits)`` of all sequences of a packed tree, concatenated in
+    ``trie.all_sequence_ids`` order; functional.py:471-564.  Every position of every node on a sequence's path
+    contributes the minimum / maximum of its row of logits (inclusive ranges, no shift).  One streaming pass gives the
+    extrema of all rows; the per-sequence results are one index select."""
+    if not trie.all_sequence_ids:
+        empty = torch.empty(0, device=logits.device, dtype=torch.float)
+        return empty, empty
+    _require_gpu(logits, "logits")
+    x, T, V, stride = _rows(logits.reshape(-1, logits.shape[-1]))
+    dev = x.device
+    positions: list[int] = []
+    for seq_id in trie.all_sequence_ids:
+        for start, end in trie.get_sequence_tree_indices(seq_id):
+            positions.extend(range(start, end + 1))
+    f32 = dict(dtype=torch.float32, device=dev)
+    vmax, vmin, scratch = torch.empty(T, **f32), torch.empty(T, **f32), torch.empty(T, **f32)
+    none_label = torch.full((T,), -1, dtype=torch.int64, device=dev)
+    with torch.cuda.device(dev):
+        N.check(N.load().aa_logits_fwd(_ptr(x), _DTYPES[x.dtype], T, V, stride, _ptr(none_label), 1.0, _ptr(scratch),
+                                       None, None, None, _ptr(vmax), _ptr(vmin), _stream(dev)), "aa_logits_fwd")
+    sel = torch.tensor(positions, dtype=torch.int64, device=dev)
+    return vmin[sel], vmax[sel]
+
+
+def merge_packed_tree_results(results_list: list[dict[int, torch.Tensor]], batch_size: int,
+                              max_seq_len: int | None = None, padding_value: float = 0.0) -> torch.Tensor:
+    """Per-sequence results of several packed trees back into one ``[batch_size, max_seq_len]`` tensor, sequence
+    ``seq_id`` in row ``seq_id``, cut or padded to ``max_seq_len`` (the longest result when None);
+    functional.py:567-639.  The rows are placed by one segment copy instead of one slice assignment each."""
+    from .packing import segment_copy
+
+    combined: dict[int, torch.Tensor] = {}
+    for results in results_list:
+        for seq_id, tensor in results.items():
+            if seq_id in combined:
+                raise ValueError(f"Duplicate sequence_id {seq_id} found across microbatches")
+            combined[seq_id] = tensor
+    if not combined:
+        return torch.full((batch_size, max_seq_len or 0), padding_value, device=torch.device("cpu"))
+    first = next(iter(combined.values()))
+    if max_seq_len is None:
+        max_seq_len = max(t.shape[0] for t in combined.values())
+    output = torch.full((batch_size, max_seq_len), padding_value, dtype=first.dtype, device=first.device)
+    for seq_id in combined:
+        if seq_id >= batch_size:
+            raise ValueError(f"sequence_id {seq_id} exceeds batch_size {batch_size}")
+    ids = list(combined)
+    lens = [int(combined[i].shape[0]) for i in ids]
+    take = [min(n, max_seq_len) for n in lens]
+    total = sum(take)
+    if total == 0:
+        return output
+    flat = torch.cat([combined[i].reshape(-1) for i in ids]).contiguous()
+    src_starts, dst_starts, cu = [], [], [0]
+    off = 0
+    for i, n, k in zip(ids, lens, take):
+        src_starts.append(off)
+        dst_starts.append(i * max_seq_len)
+        cu.append(cu[-1] + k)
+        off += n
+    segment_copy(flat, output.view(-1), torch.tensor(src_starts), torch.tensor(dst_starts),
+                 torch.tensor(cu, dtype=torch.int32), total)
+    return output

@@ -62,3 +62,35 @@ def test_pair_op_backward_matches_autograd(device, with_entropy):
     assert torch.allclose(y.grad.cpu(), x.grad, atol=2e-6) and cosine(y.grad.cpu(), x.grad) > 0.999999
     bad = areal_amd.gather_logprobs_entropy_pairs(logits.to(device), torch.tensor([T, 0]), torch.tensor([0, V]))
     assert torch.isnan(bad[0]).all()                        # out of range: NaN, never a fault
+
+
+@pytest.mark.parametrize("V,dtype", [(97, torch.float32), (151936, torch.bfloat16)])
+def test_tree_vocab_stats_match_oracle(device, V, dtype):
+    trie, T = random_tree(9, seed=3)
+    g = torch.Generator().manual_seed(2)
+    logits = (torch.randn(T, V, generator=g) * 3).to(dtype)
+    w_min, w_max = OT.packed_tree_vocab_stats(logits, trie)
+    vmin, vmax = areal_amd.gather_packed_tree_vocab_stats(logits.to(device), trie)
+    assert vmin.dtype == torch.float32 and torch.equal(vmin.cpu(), w_min) and torch.equal(vmax.cpu(), w_max)
+    e0, e1 = areal_amd.gather_packed_tree_vocab_stats(logits.to(device), Trie({}))
+    assert e0.numel() == 0 and e1.numel() == 0 and e0.device.type == "cuda"
+
+
+def test_merge_packed_tree_results_matches_oracle(device):
+    g = torch.Generator().manual_seed(5)
+    lens = {7: 13, 0: 1, 3: 300, 4: 0, 9: 64}
+    cpu = {k: torch.randn(n, generator=g) for k, n in lens.items()}
+    parts_cpu = [{k: cpu[k] for k in (7, 0)}, {k: cpu[k] for k in (3, 4, 9)}]
+    parts = [{k: v.to(device) for k, v in d.items()} for d in parts_cpu]
+    for kw in (dict(), dict(max_seq_len=40, padding_value=-2.5), dict(max_seq_len=512)):
+        want = OT.merge_tree_results(parts_cpu, 10, **kw)
+        got = areal_amd.merge_packed_tree_results(parts, 10, **kw)
+        assert got.device.type == "cuda" and torch.equal(got.cpu(), want), kw
+    ints = [{1: torch.arange(5, device=device)}, {0: torch.arange(3, device=device)}]
+    got = areal_amd.merge_packed_tree_results(ints, 2)
+    assert got.dtype == torch.int64 and got.tolist() == [[0, 1, 2, 0, 0], [0, 1, 2, 3, 4]]
+    assert areal_amd.merge_packed_tree_results([], 3, 2).shape == (3, 2)
+    with pytest.raises(ValueError, match="Duplicate sequence_id"):
+        areal_amd.merge_packed_tree_results([parts[0], parts[0]], 10)
+    with pytest.raises(ValueError, match="exceeds batch_size"):
+        areal_amd.merge_packed_tree_results(parts, 8)
