@@ -691,14 +691,19 @@ __device__ __forceinline__ u32x4_t grad_chunk(const u32x4_t v, float c, float kk
   return r;
 }
 
+constexpr int kTwoPerUnitChunks = 7;  // rows this short run two workgroups per compute unit
+
 // Rows are handed out through a device counter (work[0]) so that compute
 // units that get through their rows faster take more of them; work[1] counts
 // finished workgroups, and the last one puts both words back to zero, which is
 // the state the next launch expects.  With work == nullptr the rows are dealt
 // round-robin (t, t + gridDim.x, ...).
 // With EXT the row continues past the NCH register chunks: n_lds chunks in dynamic LDS, then the tail chunks.
+// Up to kTwoPerUnitChunks chunks the kernel is compiled for 8 waves per SIMD, so that two workgroups fit on a
+// compute unit: without that request the scalar registers alone (106 per wave: 7 waves) keep the second one out.
 template <int DT, int NCH, bool EXT = false>
-__global__ __launch_bounds__(1024) void k_fused_regs(const uint4* __restrict__ logits, int V, int64_t stride_vec,
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu((!EXT && NCH <= kTwoPerUnitChunks) ? 8 : 1)))
+void k_fused_regs(const uint4* __restrict__ logits, int V, int64_t stride_vec,
                                                      const int64_t* __restrict__ labels, float inv_t,
                                                      const float* __restrict__ in_prox,
                                                      const float* __restrict__ in_adv,
@@ -975,7 +980,10 @@ static int persistent_workgroups() {
 template <int DT, int NCH>
 static void launch_regs(const void* logits, int64_t T, int V, int64_t stride, const int64_t* labels, float inv_t,
                         const FusedTokenArgs& a, void* dlogits, int32_t* work, hipStream_t st) {
-  const int64_t wgs = T < persistent_workgroups() ? T : persistent_workgroups();
+  // Short rows (up to 6 chunks: at most 64 VGPRs per thread) leave room for a second workgroup on every compute
+  // unit; with two rows in flight per unit the fixed cost per row (three passes, two reductions) overlaps.
+  const int64_t resident = (int64_t)persistent_workgroups() * (NCH <= kTwoPerUnitChunks ? 2 : 1);
+  const int64_t wgs = T < resident ? T : resident;
   const uintptr_t mask_addr = (uintptr_t)a.mask_eff;
   hipLaunchKernelGGL((k_fused_regs<DT, NCH>), dim3((unsigned)wgs), dim3(1024), 0, st, (const uint4*)logits, V,
                      stride >> 3, labels, inv_t, a.prox_logp, a.adv, (const uint32_t*)(mask_addr & ~(uintptr_t)3),

@@ -97,6 +97,21 @@ def test_fused_config0_shape_matches_oracle(device, V, dtype, lo, hi):
     _compare(case, _fused_step(case), _oracle_step(case))
 
 
+@pytest.mark.parametrize("V,dtype", [(8192, torch.bfloat16), (32000, torch.float16), (57344, torch.bfloat16)])
+def test_short_rows_with_two_workgroups_per_unit(device, V, dtype):
+    """Rows of up to 7 chunks run two workgroups per compute unit; more rows than workgroups, so the rows after
+    the first 512 are handed out through the counter."""
+    lengths = synth.lengths_uniform(48, 16, 48, seed=V)           # about 1500 tokens
+    case = synth.make_logits_case("t", lengths, V, V, device, synth.per_sequence_normal_advantages(lengths, 3),
+                                  dtype=dtype, ppo=dict(eps_clip=0.2))
+    assert case.n_tokens > 1100
+    _finish_case(case)
+    first = _fused_step(case)
+    _compare(case, first, _oracle_step(case))
+    again = _fused_step(case)                                     # another hand-out order, the same bits
+    assert torch.equal(first[2], again[2]) and float(first[0]) == float(again[0])
+
+
 @pytest.mark.parametrize("V", [70004, 90112])
 def test_fp32_long_rows_walked_by_large_workgroups(device, V):
     """More fp32 rows than workgroups, so every workgroup handles several rows: V = 70004 (not a multiple of 8, rows
