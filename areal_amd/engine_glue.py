@@ -398,3 +398,61 @@ def compute_rw_loss(scores: torch.Tensor, input_: dict[str, Any]) -> tuple[torch
     with torch.no_grad():
         stat["correct_ratio"] = (stat["pos_score"] > stat["neg_score"]).float()
     return loss, stat
+
+
+def compute_loss_with(logits: torch.Tensor, model_inputs: dict[str, Any], mb_input: dict[str, Any], pad_length: int,
+                      loss_fn, loss_weight_fn, total_loss_weight: torch.Tensor | float, temperature: float = 1.0,
+                      loss_multiplier: float = 1.0, is_critic: bool = False, trie_node: Any = None):
+    """``_compute_logprobs_and_loss`` for any loss function (areal/engine/fsdp_engine.py:1977-2046): log-probs,
+    entropy and the vocabulary extrema of the micro-batch in one pass over the logits (packed trees: through the
+    tree gather), the batch padding trimmed, ``loss_fn(logprobs, entropy, mb_input, vocab_min_logits=...,
+    vocab_max_logits=...)`` (a critic: ``loss_fn(values, mb_input)``), scaled by ``local_weight / total_loss_weight *
+    loss_multiplier``.  ``loss_fn`` may return the loss alone, like the reference's, or ``(loss, stat)`` like the
+    loss functions of this module; the return value has the same form.  A micro-batch of weight 0 returns
+    ``logits.mean() * 0``."""
+    local_weight = loss_weight_fn(mb_input)
+    if local_weight == 0:
+        return logits.mean() * 0.0
+    if is_critic:
+        if trie_node is not None:
+            raise NotImplementedError("Tree training with critic model is not supported yet.")
+        values = logits.squeeze(-1)
+        if pad_length > 0:
+            values = values[:-pad_length]
+        out = loss_fn(values, mb_input)
+    else:
+        if trie_node is not None:
+            from .tree import gather_packed_tree_logprobs_entropy, gather_packed_tree_vocab_stats
+
+            if not trie_node.all_sequence_ids:
+                return logits.mean() * 0.0
+            vmin, vmax = gather_packed_tree_vocab_stats(logits, trie_node)
+            logp, entropy = gather_packed_tree_logprobs_entropy(logits, trie_node, mb_input["input_ids"],
+                                                                temperature=temperature)
+        else:
+            logp, entropy, vmin, vmax = gather_logprobs_entropy_stats(logits, rolled_labels(model_inputs), temperature)
+            if pad_length > 0:
+                logp, entropy, vmin, vmax = (t[:-pad_length] for t in (logp, entropy, vmin, vmax))
+        out = loss_fn(logp, entropy, mb_input, vocab_min_logits=vmin, vocab_max_logits=vmax)
+    scale = local_weight / total_loss_weight * loss_multiplier
+    if isinstance(out, tuple):
+        return out[0] * scale, out[1]
+    return out * scale
+
+
+def compute_logprobs_and_sft_loss(logits: torch.Tensor, model_inputs: dict[str, Any], mb_input: dict[str, Any],
+                                  total_loss_weight: torch.Tensor | float, temperature: float = 1.0,
+                                  loss_multiplier: float = 1.0) -> tuple[torch.Tensor, dict]:
+    """The supervised step of one micro-batch in one pass over the logits: what ``compute_loss_with`` does with
+    ``loss_fn = compute_packed_sft_loss`` and ``loss_weight_fn = loss_mask.count_nonzero``
+    (areal/trainer/sft/lm_engine.py:28-35), fused with the log-prob op and its backward.  ``mb_input`` holds the
+    un-padded ``loss_mask`` and ``cu_seqlens``; the rows of ``logits`` past them are the batch padding."""
+    from .sft import fused_logprobs_sft_loss
+
+    loss_mask = mb_input["loss_mask"].bool()
+    local_weight = loss_mask.count_nonzero()
+    if local_weight == 0:
+        return logits.mean() * 0.0, {}
+    scale = local_weight / total_loss_weight * loss_multiplier
+    return fused_logprobs_sft_loss(logits, rolled_labels(model_inputs), loss_mask, mb_input["cu_seqlens"], temperature,
+                                   loss_scale=scale)

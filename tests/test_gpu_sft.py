@@ -126,3 +126,39 @@ def test_fused_lm_head_sft_matches_oracle(device, skip):
         loss_f, _ = areal_amd.fused_lm_head_sft_loss(hidden.to(device), weight.to(device), labels.to(device),
                                                      mask.to(device), cu.to(device))
     assert float(loss_f) == pytest.approx(float(loss.detach()), rel=1e-4)
+
+
+def test_engine_glue_generic_and_fused_sft_agree(device):
+    """fsdp_engine.py:1977-2046 with the supervised loss function: the generic glue (log-prob op, trim, loss function,
+    scale) and the fused step give the same loss and the same gradient of the logits."""
+    lens = [30, 11, 0, 25]
+    g, cu, T, mask = _packed(lens, 21)
+    pad = 8
+    V = 8200
+    ids = torch.randint(0, V, (T + pad,), generator=g)
+    logits = (2 * torch.randn(T + pad, V, generator=g)).bfloat16()
+    model_inputs = dict(input_ids=ids.to(device)[None])
+    mb = dict(loss_mask=mask.to(device), cu_seqlens=cu.to(device))
+    total = 3.0 * int(mask.sum())
+    x = logits.to(device).requires_grad_(True)
+    loss, stat = G.compute_loss_with(x, model_inputs, mb, pad, G.compute_packed_sft_loss,
+                                     lambda d: d["loss_mask"].count_nonzero(), total, loss_multiplier=2.0)
+    loss.backward()
+    y = logits.to(device).requires_grad_(True)
+    loss_f, stat_f = G.compute_logprobs_and_sft_loss(y, model_inputs, mb, total, loss_multiplier=2.0)
+    loss_f.backward()
+    assert float(loss_f.detach()) == pytest.approx(float(loss.detach()), rel=1e-5)
+    assert torch.equal(stat_f["n_seqs"], stat["n_seqs"]) and torch.allclose(stat_f["ppl"], stat["ppl"], rtol=1e-5)
+    assert cosine(x.grad.float().cpu(), y.grad.float().cpu()) > 0.99999 and not y.grad[T:].any()
+    # against the oracle: labels rolled over the whole padded tensor, loss scaled by local / total * multiplier
+    labels = torch.roll(ids, -1)
+    w_logp = oracle.logprobs(logits, labels, 1.0)[:T]
+    w_loss, _ = packed_sft_loss(w_logp, mask, cu.long())
+    assert float(loss.detach()) == pytest.approx(float(w_loss) * int(mask.sum()) / total * 2.0, rel=1e-3)
+    # a loss function that returns the loss alone, and a micro-batch without weight
+    only = G.compute_loss_with(logits.to(device), model_inputs, mb, pad, lambda lp, ent, d, **kw: lp.sum(),
+                               lambda d: d["loss_mask"].count_nonzero(), total)
+    assert only.ndim == 0
+    none = dict(mb, loss_mask=torch.zeros_like(mb["loss_mask"]))
+    assert float(G.compute_loss_with(logits.to(device), model_inputs, none, pad, G.compute_packed_sft_loss,
+                                     lambda d: d["loss_mask"].count_nonzero(), total)) == 0.0
