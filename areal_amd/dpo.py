@@ -193,13 +193,14 @@ class _RwLoss(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g_loss, *_):
         (g,) = ctx.saved_tensors
+        out = g.clone()   # [T] floats: keeps the saved gradient intact for a second backward (retain_graph)
         dev = g.device
         up = _f32(g_loss).reshape(1)
-        if g.numel():
-            with torch.cuda.device(dev):   # in place: a factor of 1 is a no-op
-                N.check(N.load().aa_scale_inplace(_ptr(g), _DTYPES[g.dtype], g.numel(), _ptr(up), _stream(dev)),
+        if out.numel():
+            with torch.cuda.device(dev):
+                N.check(N.load().aa_scale_inplace(_ptr(out), _DTYPES[out.dtype], out.numel(), _ptr(up), _stream(dev)),
                         "aa_scale_inplace")
-        return g, None
+        return out, None
 
 
 def rw_pair_loss(scores: torch.Tensor, cu_seqlens: torch.Tensor) -> tuple[torch.Tensor, dict]:

@@ -68,12 +68,15 @@ class _SftLoss(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g_loss, *_unused):
         (g,) = ctx.saved_tensors
+        # [T] floats: a copy is cheap and keeps the saved gradient intact for a second backward (retain_graph)
+        out = g.clone()
         dev = g.device
         up = _f32(g_loss).reshape(1)
-        with torch.cuda.device(dev):   # in place: a factor of 1 is a no-op
-            N.check(N.load().aa_scale_inplace(_ptr(g), _DTYPES[g.dtype], g.numel(), _ptr(up), _stream(dev)),
-                    "aa_scale_inplace")
-        return g, None, None, None, None, None
+        if out.numel():
+            with torch.cuda.device(dev):
+                N.check(N.load().aa_scale_inplace(_ptr(out), _DTYPES[out.dtype], out.numel(), _ptr(up), _stream(dev)),
+                        "aa_scale_inplace")
+        return out, None, None, None, None, None
 
 
 def _stat(stat_loss, seq_logp, seq_count, seq_ppl, n_seqs, extra=None):

@@ -162,3 +162,19 @@ def test_engine_glue_generic_and_fused_sft_agree(device):
     none = dict(mb, loss_mask=torch.zeros_like(mb["loss_mask"]))
     assert float(G.compute_loss_with(logits.to(device), model_inputs, none, pad, G.compute_packed_sft_loss,
                                      lambda d: d["loss_mask"].count_nonzero(), total)) == 0.0
+
+
+def test_second_backward_of_the_small_losses_is_not_rescaled(device):
+    """The per-token gradients of the losses on log-probs / scores are copied before the upstream factor is applied,
+    so a second backward through a retained graph gives the same gradient."""
+    lp = (-torch.rand(50)).to(device).requires_grad_(True)
+    mask = torch.rand(50, device=device) < 0.7
+    loss, _ = areal_amd.sft_loss_fn(lp, mask, torch.tensor([0, 20, 50], device=device))
+    (g1,) = torch.autograd.grad(3.0 * loss, lp, retain_graph=True)
+    (g2,) = torch.autograd.grad(3.0 * loss, lp)
+    assert torch.equal(g1, g2)
+    s = torch.randn(50, device=device, requires_grad=True)
+    loss, _ = areal_amd.rw_pair_loss(s, torch.tensor([0, 20, 50], device=device))
+    (g1,) = torch.autograd.grad(0.5 * loss, s, retain_graph=True)
+    (g2,) = torch.autograd.grad(0.5 * loss, s)
+    assert torch.equal(g1, g2) and int((g1 != 0).sum()) == 2
