@@ -482,6 +482,16 @@ def ppo_actor_loss_fn(
 # ----------------------------------------------------------------------------
 # fused: logits -> logp/entropy -> token-level PPO loss -> d(logits), one pass
 # ----------------------------------------------------------------------------
+def _hand_out_once(ctx) -> None:
+    """The fused steps keep their gradients in the buffers the forward pass wrote and scale them in place by the
+    upstream factor, so those buffers can be handed out once: a second backward through a retained graph would scale
+    them again."""
+    if getattr(ctx, "handed_out", False):
+        raise RuntimeError("the gradient of this fused step was already handed out; run the forward pass again "
+                           "instead of a second backward through a retained graph")
+    ctx.handed_out = True
+
+
 def _finish_fused_loss(lib, params, stat_loss, logp, mask_eff, T_active, n_valid, grad_scale, loss, st) -> None:
     """The scalar the fused kernels' per-token losses add up to: the clipped surrogate over ``max(n, 1)``, or the
     negative log-likelihood over ``n + 1e-5`` (areal/trainer/sft/lm_engine.py:96)."""
@@ -534,6 +544,7 @@ class _FusedLogitsPpo(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g_loss, *_unused):
+        _hand_out_once(ctx)
         lib = N.load()
         (dlogits,) = ctx.saved_tensors
         dev = dlogits.device
@@ -802,6 +813,7 @@ class _FusedLmHeadPpo(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g_loss, *_unused):
+        _hand_out_once(ctx)
         lib = N.load()
         d_hidden, d_weight = ctx.saved_tensors
         dev = d_hidden.device

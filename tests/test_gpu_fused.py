@@ -363,3 +363,16 @@ def test_forward_only_calls_skip_the_gradient(device):
     lb, sb = areal_amd.fused_lm_head_ppo_loss(hidden, weight, labels, z, z, adv, 0.2, mask)   # nothing requires grad
     assert not lb.requires_grad and float(lb) == pytest.approx(float(la.detach()), rel=1e-6)
     assert torch.allclose(sb["logprobs"], sa["logprobs"], atol=1e-6)
+
+
+def test_second_backward_of_the_fused_step_is_refused(device):
+    lengths = [9, 14]
+    case = synth.make_logits_case("t", lengths, 8192, 8192, device, synth.per_sequence_normal_advantages(lengths, 3),
+                                  ppo=dict(eps_clip=0.2))
+    _finish_case(case)
+    x = case.logits.clone().requires_grad_(True)
+    loss, _ = areal_amd.fused_logprobs_ppo_loss(x, case.labels, case.prox_logp, case.old_logp, case.advantages, 0.2,
+                                                case.loss_mask)
+    loss.backward(retain_graph=True)
+    with pytest.raises(RuntimeError, match="already handed out"):
+        loss.backward()
