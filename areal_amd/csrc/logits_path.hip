@@ -447,8 +447,8 @@ __global__ __launch_bounds__(NT) void k_fused_generic(const void* __restrict__ l
 // Fused kernel for fp32 logits: a row is too long for the register file alone (608 KB at V = 151 936 against
 // 512 KB), so the first kHoldReg chunks of a row (8 floats per thread and chunk) stay in registers, the next
 // kHoldLds chunks in LDS, and only what is left is read a second time for the gradient.  At V = 151 936 that is
-// 22 % of the row: 8.9 bytes per element through the fabric instead of the 12 of the two-pass kernel (8 is the
-// floor); rows up to 81 920 elements are read once.  One workgroup of 1024 threads per compute unit (the LDS
+// 24.5 % of the row: at most 9 bytes per element through the fabric instead of the 12 of the two-pass kernel (8 is
+// the floor); rows up to 114 688 elements are read once.  One workgroup of 1024 threads per compute unit (the LDS
 // share allows no second one), walking rows t, t + grid, ...  Needs V % 8 == 0 and 16-byte aligned rows.
 // -----------------------------------------------------------------------------
 constexpr int kHoldReg = 10;                        // 10 x 8192 floats in registers (80 VGPRs per thread)
