@@ -8,7 +8,9 @@ One "step" is one pass of the hot path over one synthetic packed micro-batch tha
 * logits workloads (cfg0, cfg1, cfg1-32k; cfg1 is the default, the configuration the metric is quoted on):
   rejection sampling (importance-weight cap) -> fused log-prob / entropy / clipped PPO loss / d(logits) -> scalar
   loss, i.e. ``fused_logprobs_ppo_loss(...)`` followed by ``loss.backward()``.  Roofline: HBM, algorithmic bytes
-  4 * V per token (the bf16 logits read once, their gradient written once).
+  4 * V per token (the bf16 logits read once, their gradient written once); ``--logits-dtype f32`` casts the logits
+  to fp32 first (8 * V per token).  The line also carries ``sft_loss_same_logits``: the supervised loss on the same
+  logits, fused in one pass against the log-prob op followed by the loss and a separate backward pass.
 * fused lm_head workloads (cfg2, cfg3, cfg4): ``fused_lm_head_ppo_loss(hidden, W, labels, ...)`` followed by
   ``loss.backward()``: lm_head, log-prob / entropy, PPO loss and the gradients d(hidden), d(W), token chunk by
   token chunk, the full [T, V] logits never in memory.  Roofline: bf16 MFMA.  Algorithmic flops: 2 T V H for the
