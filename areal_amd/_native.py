@@ -67,6 +67,7 @@ SIGNATURES = {
         [_p, _i, _i64, _i64, _i64, _p, _f, _i64, _p, _p, _p, _p, C.POINTER(PpoParams), _p, _p,
          _p, _p, _p, _p, _p, _p, _p, _p, _p, _p],
     ),
+    "aa_vocab_partials_combine": (_i, [_p, _p, _p, _i, _i64, _p, _p, _p, _p, _p]),
     "aa_logits_pairs_fwd": (_i, [_p, _i, _i64, _i64, _i64, _p, _p, _i64, _f, _p, _p, _p, _p, _p]),
     "aa_logits_pairs_scatter": (_i, [_p, _i, _i64, _i64, _i64, _p, _p, _i64, _p, _f, _p]),
     "aa_rejection_sampling": (_i, [_p, _p, _p, _i64, _p, _i64, _i, _i, _i, _i, _f, _f, _i, _p, _p, _p, _p]),

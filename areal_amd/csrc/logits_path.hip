@@ -924,6 +924,40 @@ void k_fused_regs(const uint4* __restrict__ logits, int V, int64_t stride_vec,
 }
 
 // -----------------------------------------------------------------------------
+// One GPU's share of the vocabulary-parallel log-prob op (areal/utils/functional/vocab_parallel.py:84-372): every
+// shard runs the streaming forward pass on its [T, V / tp] slice and ends with three numbers per row: its own
+// logsumexp, its own sum_j softmax_j z_j, and the label's log-prob where the label lies in the shard (NaN where
+// not).  This kernel is the reduction the ranks would do with one exchange of those numbers: the global
+// logsumexp, sum p z, log-prob and entropy.  Fixed order over the shards.
+// -----------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_vocab_partials_combine(const float* __restrict__ lse,
+                                                                const float* __restrict__ ez,
+                                                                const float* __restrict__ logp_local, int S,
+                                                                int64_t T, float* __restrict__ logp,
+                                                                float* __restrict__ entropy,
+                                                                float* __restrict__ lse_out,
+                                                                float* __restrict__ ez_out) {
+  for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < T; t += (int64_t)gridDim.x * 256) {
+    float m = -__builtin_inff();
+    for (int i = 0; i < S; ++i) m = fmaxf(m, lse[i * T + t]);
+    float sum = 0.f;
+    for (int i = 0; i < S; ++i) sum += expf(lse[i * T + t] - m);
+    const float L = m + logf(sum);
+    float e = 0.f, lp = __builtin_nanf("");
+    for (int i = 0; i < S; ++i) {
+      const float li = lse[i * T + t];
+      e = fmaf(expf(li - L), ez[i * T + t], e);
+      const float q = logp_local[i * T + t];
+      if (q == q) lp = q + li - L;  // the shard that holds the label: z_label = logp_local + lse_i
+    }
+    logp[t] = lp;
+    if (entropy) entropy[t] = L - e;
+    if (lse_out) lse_out[t] = L;
+    if (ez_out) ez_out[t] = e;
+  }
+}
+
+// -----------------------------------------------------------------------------
 // Plain copy (calibration of the HBM counters) and in-place scaling.
 // -----------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void k_copy16(const uint4* __restrict__ src, uint4* __restrict__ dst, int64_t n) {
@@ -1262,5 +1296,18 @@ extern "C" int aa_scale_inplace(void* data, int dtype, int64_t n, const float* f
   else if (dtype == AA_F16) hipLaunchKernelGGL(k_scale<AA_F16>, dim3((unsigned)blocks), dim3(256), 0, st, data, n, factor);
   else if (dtype == AA_F32) hipLaunchKernelGGL(k_scale<AA_F32>, dim3((unsigned)blocks), dim3(256), 0, st, data, n, factor);
   else return AA_ERR_INVALID_ARGUMENT;
+  return launch_status();
+}
+
+extern "C" int aa_vocab_partials_combine(const float* shard_lse, const float* shard_ez, const float* shard_logp,
+                                         int n_shards, int64_t T, float* logp, float* entropy, float* row_lse,
+                                         float* row_ez, void* stream) {
+  if (n_shards < 1 || T < 0 || !logp) return AA_ERR_INVALID_ARGUMENT;
+  if (T == 0) return AA_OK;
+  if (!shard_lse || !shard_ez || !shard_logp) return AA_ERR_INVALID_ARGUMENT;
+  int64_t blocks = (T + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(k_vocab_partials_combine, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, shard_lse,
+                     shard_ez, shard_logp, n_shards, T, logp, entropy, row_lse, row_ez);
   return launch_status();
 }

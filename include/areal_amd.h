@@ -151,6 +151,26 @@ int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int64_t V,
                         int32_t* work, void* stream);
 
 /*
+ * The reduction step of the vocabulary-parallel op
+ * (areal/utils/functional/vocab_parallel.py:84-372), for n_shards slices
+ * [T, V_i] of one [T, V] logits tensor that each went through aa_logits_fwd
+ * with the labels shifted into the slice (a label outside it gives NaN there):
+ *   shard_lse, shard_ez, shard_logp: [n_shards, T], the row_lse, row_ez and
+ *   logp outputs of those calls;
+ *   row_lse = logsumexp_i shard_lse_i,  row_ez = sum_i exp(shard_lse_i -
+ *   row_lse) * shard_ez_i,  logp = shard_logp_i + shard_lse_i - row_lse for the
+ *   shard that holds the label (NaN if none does),  entropy = row_lse - row_ez.
+ * entropy, row_lse, row_ez may be NULL.  The backward of a slice is
+ * aa_logits_bwd on that slice with the shifted labels and the combined
+ * row_lse / row_ez.  Across GPUs the three [T] vectors per rank are what one
+ * exchange carries; the exchange itself is not part of this library.
+ */
+int aa_vocab_partials_combine(const float* shard_lse, const float* shard_ez,
+                              const float* shard_logp, int n_shards, int64_t T,
+                              float* logp, float* entropy, float* row_lse,
+                              float* row_ez, void* stream);
+
+/*
  * Log-probs for arbitrary (row, label) pairs, the transitions of a packed
  * prefix tree (areal/models/tree_attn/functional.py:160-203, 206-316), where a
  * row may predict several tokens that sit elsewhere in the packed tensor:

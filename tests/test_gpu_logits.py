@@ -184,3 +184,42 @@ def test_plain_c_consumer_of_the_abi(device):
     run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
     assert run.returncode == 0, run.stdout + run.stderr
     assert "c_abi consumer ok" in run.stdout
+
+
+@pytest.mark.parametrize("cuts,dtype,temperature", [([0.5], torch.bfloat16, 1.0), ([0.1, 0.35, 0.8], torch.float32, 0.7),
+                                                    ([0.125 * i for i in range(1, 8)], torch.bfloat16, 1.3)])
+def test_vocab_shards_equal_the_unsharded_op(device, cuts, dtype, temperature):
+    """The vocabulary axis cut into 2 / 4 / 8 slices (uneven ones too): statistics per slice, one combine, backward
+    per slice from the combined statistics (vocab_parallel.py:84-372 without its collectives) against the oracle and
+    against the unsharded kernels."""
+    import oracle
+    from areal_amd import vocab_parallel as VP
+
+    T, V = 300, 24000
+    g = torch.Generator().manual_seed(3)
+    logits = (torch.randn(T, V, generator=g) * 3).to(dtype)
+    labels = torch.randint(0, V, (T,), generator=g)
+    labels[:4] = torch.tensor([0, V - 1, int(cuts[0] * V) // 8 * 8 - 1, int(cuts[0] * V) // 8 * 8])   # slice borders
+    bounds = [0] + [int(c * V) // 8 * 8 for c in cuts] + [V]
+    x = logits.clone().requires_grad_(True)
+    w_lp, w_ent = oracle.logprobs_entropy(x, labels, temperature)
+    gl, gh = torch.randn(T, generator=g), torch.randn(T, generator=g)
+    (w_lp * gl + w_ent * gh).sum().backward()
+    shards = [logits[:, a:b].contiguous().to(device).requires_grad_(True) for a, b in zip(bounds[:-1], bounds[1:])]
+    lp, ent = VP.gather_logprobs_entropy_vocab_shards(shards, labels.to(device), temperature)
+    (lp * gl.to(device) + ent * gh.to(device)).sum().backward()
+    assert float((lp.detach().cpu() - w_lp.detach()).abs().max()) < 2e-3
+    assert float((ent.detach().cpu() - w_ent.detach()).abs().max()) < 2e-3
+    grad = torch.cat([sh.grad for sh in shards], dim=1).float().cpu()
+    assert cosine(grad, x.grad.float()) > 0.9999
+    # against the unsharded kernels: the same numbers up to the order of the sums
+    y = logits.to(device).requires_grad_(True)
+    lp1, ent1 = areal_amd.gather_logprobs_entropy(y, labels.to(device), temperature)
+    (lp1 * gl.to(device) + ent1 * gh.to(device)).sum().backward()
+    assert torch.allclose(lp, lp1, atol=2e-5) and torch.allclose(ent, ent1, atol=2e-5)
+    tol = (1e-4 if dtype == torch.float32 else 2e-2) * float(y.grad.float().abs().max())   # bf16: one rounding step
+    assert float((grad - y.grad.float().cpu()).abs().max()) <= tol
+    # a label that lies in no slice gives NaN, as the unsharded op does for a label out of range
+    lse, ez, lpl, _ = VP.shard_statistics(shards[0], torch.full((T,), V + 5), 0, temperature)
+    out = VP.combine_shard_statistics(lse[None], ez[None], lpl[None])
+    assert bool(torch.isnan(out[0]).all()) and bool(torch.isfinite(out[1]).all())
