@@ -94,6 +94,9 @@ def test_argument_validation_of_the_sibling_entry_points_without_gpu():
     assert lib.aa_masked_normalization_scratch_bytes(4, -1) == -1
     assert lib.aa_overlong_penalty(p, p, 4, 8, 0, 1.0, 100, z) == bad                   # division by overlong_tokens
     assert lib.aa_kd_terms(p, z, p, p, 4, 1, p, p, z) == bad                            # pure form without old log-probs
+    assert lib.aa_vocab_partials_combine(p, p, p, 0, 4, p, z, z, z, z) == bad       # no slice
+    assert lib.aa_vocab_partials_combine(z, p, p, 2, 4, p, z, z, z, z) == bad
+    assert lib.aa_vocab_partials_combine(z, z, z, 2, 0, p, z, z, z, z) == ok
     params = _native.PpoParams(clip_lo=0.8, clip_hi=1.2, loss_kind=2)
     assert lib.aa_logits_ppo_fused(p, 0, 4, 4096, 4096, p, 1.0, 4, p, p, p, z, ctypes.byref(params), p, z, p, z, z, z,
                                    p, p, p, p, z, z) == bad                             # unknown loss kind
