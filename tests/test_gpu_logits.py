@@ -180,7 +180,14 @@ def test_plain_c_consumer_of_the_abi(device):
     from pathlib import Path
 
     exe = Path(__file__).resolve().parent / "c_abi" / "consumer"
-    assert exe.exists(), "build it first: python -c 'import __graft_entry__ as g; g.build_c_abi_consumer()'"
+    if not exe.exists():      # normally built beforehand by __graft_entry__.build(); built here only if it is missing
+        import sys
+
+        sys.path.insert(0, str(Path(__file__).resolve().parents[1]))
+        import __graft_entry__
+
+        __graft_entry__.build_c_abi_consumer()
+    assert exe.exists()
     run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
     assert run.returncode == 0, run.stdout + run.stderr
     assert "c_abi consumer ok" in run.stdout
