@@ -178,3 +178,33 @@ def test_second_backward_of_the_small_losses_is_not_rescaled(device):
     (g1,) = torch.autograd.grad(0.5 * loss, s, retain_graph=True)
     (g2,) = torch.autograd.grad(0.5 * loss, s)
     assert torch.equal(g1, g2) and int((g1 != 0).sum()) == 2
+
+
+def test_full_size_supervised_lm_head_step(device):
+    """configs[2] shape (hidden [16384, 4096], W [151936, 4096]): the chunked supervised step against the stand-alone
+    lm_head op followed by the loss on log-probs and autograd; bit-identical when repeated; prompt tokens (the masked
+    30 % of every sequence) get no gradient."""
+    from areal_amd import synth
+
+    case = synth.config2(device, seed=0)
+
+    def fused():
+        h = case.hidden.detach().requires_grad_(True)
+        w = case.weight.detach().requires_grad_(True)
+        loss, stat = areal_amd.fused_lm_head_sft_loss(h, w, case.labels, case.loss_mask, case.cu_seqlens, loss_scale=0.5)
+        loss.backward()
+        return loss.detach(), stat, h.grad, w.grad
+
+    l1, s1, dh1, dw1 = fused()
+    l2, _, dh2, dw2 = fused()
+    assert torch.equal(l1, l2) and torch.equal(dh1, dh2) and torch.equal(dw1, dw2)
+    h = case.hidden.detach().requires_grad_(True)
+    w = case.weight.detach().requires_grad_(True)
+    lp, _ = areal_amd.lm_head_logprobs_entropy(h, w, case.labels)
+    loss, stat = areal_amd.sft_loss_fn(lp, case.loss_mask, case.cu_seqlens, loss_scale=0.5)
+    loss.backward()
+    assert float(l1) == pytest.approx(float(loss.detach()), rel=1e-3)
+    assert torch.equal(s1["n_seqs"], stat["n_seqs"]) and torch.allclose(s1["ppl"], stat["ppl"], rtol=2e-3)
+    assert cosine(dh1.float().cpu(), h.grad.float().cpu()) > 0.9999
+    assert cosine(dw1.float().cpu(), w.grad.float().cpu()) > 0.9999
+    assert not dh1[~case.loss_mask.bool()].any()
