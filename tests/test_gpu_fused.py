@@ -75,7 +75,8 @@ def _compare(case, got, want, pad=0):
     [
         (151936, torch.bfloat16, 8, 40),   # register-resident rows, 19 chunks (benchmark vocabulary)
         (32768, torch.bfloat16, 8, 40),    # register-resident rows, exact multiple of the chunk size
-        (8200, torch.float16, 8, 40),      # 2 chunks, the second almost empty
+        (8200, torch.float16, 8, 40),      # up to two chunks: the two-pass kernel
+        (16392, torch.float16, 8, 40),     # 3 chunks in registers, the third almost empty
         (50257, torch.bfloat16, 4, 20),    # generic rows (V % 8 != 0)
         (4099, torch.float32, 4, 20),      # generic rows, fp32 logits
         (8192, torch.float32, 4, 12),      # fp32 rows held on the chip: exactly one register chunk
@@ -97,9 +98,9 @@ def test_fused_config0_shape_matches_oracle(device, V, dtype, lo, hi):
     _compare(case, _fused_step(case), _oracle_step(case))
 
 
-@pytest.mark.parametrize("V,dtype", [(8192, torch.bfloat16), (32000, torch.float16), (57344, torch.bfloat16)])
+@pytest.mark.parametrize("V,dtype", [(16392, torch.bfloat16), (32000, torch.float16), (57344, torch.bfloat16)])
 def test_short_rows_with_two_workgroups_per_unit(device, V, dtype):
-    """Rows of up to 7 chunks run two workgroups per compute unit; more rows than workgroups, so the rows after
+    """Rows of 3 to 7 chunks run two workgroups per compute unit; more rows than workgroups, so the rows after
     the first 512 are handed out through the counter."""
     lengths = synth.lengths_uniform(48, 16, 48, seed=V)           # about 1500 tokens
     case = synth.make_logits_case("t", lengths, V, V, device, synth.per_sequence_normal_advantages(lengths, 3),
