@@ -63,8 +63,8 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="cfg1", choices=LOGITS_WORKLOADS + FUSED_WORKLOADS + ADV_WORKLOADS)
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--cpu-tokens", type=int, default=1024,
-                    help="token sample of the CPU baseline (0 = skip); fused lm_head workloads use at most 128")
+    ap.add_argument("--cpu-tokens", type=int, default=6144,
+                    help="token sample of the CPU baseline (0 = skip); fused lm_head workloads use at most 384")
     ap.add_argument("--cpu-iters", type=int, default=3)
     ap.add_argument("--no-fused-extra", action="store_true",
                     help="default workload only: do not append the cfg2 fused lm_head figures")
@@ -820,11 +820,11 @@ def main():
         if args.workload == "cfg1" and not args.no_fused_extra and args.copy_launches == 0:
             torch.cuda.empty_cache()
             extra = bench_fused(args, dev, "cfg2", steps=min(args.steps, 5), warmup=min(args.warmup, 2),
-                                cpu_tokens=min(args.cpu_tokens, 128))
+                                cpu_tokens=min(args.cpu_tokens, 384))
             keys = ("value", "unit", "ms_per_step", "steps", "warmup", "config", "roofline", "cpu_baseline", "parity")
             out["fused_lm_head"] = {k: extra[k] for k in keys if k in extra}
     else:
-        out = bench_fused(args, dev, args.workload, args.steps, args.warmup, min(args.cpu_tokens, 128))
+        out = bench_fused(args, dev, args.workload, args.steps, args.warmup, min(args.cpu_tokens, 384))
     print(json.dumps(out))
 
 
