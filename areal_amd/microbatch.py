@@ -246,6 +246,38 @@ class MicroBatchList:
                 padded_to_length=self.padded_to_lengths[i] if self.padded_to_lengths else None,
             )
 
+    def to(self, *args, **kwargs) -> "MicroBatchList":
+        """A copy with every tensor moved / cast; data.py:661-690."""
+        return MicroBatchList(
+            data=tensor_container_to(self.data, *args, **kwargs),
+            mb_spec=self.mb_spec,
+            mbs=[tensor_container_to(mb, *args, **kwargs) for mb in self.mbs],
+            forward_indices=self.forward_indices,
+            backward_indices=self.backward_indices,
+            group_lens=self.group_lens,
+            padded_mbs=None if self.padded_mbs is None else [tensor_container_to(mb, *args, **kwargs)
+                                                             for mb in self.padded_mbs],
+            _max_seqlen=self._max_seqlen,
+            padding_lengths=self.padding_lengths,
+            padded_to_lengths=self.padded_to_lengths,
+            old_cu_seqlens_list=None if self.old_cu_seqlens_list is None else [t.to(*args, **kwargs)
+                                                                             for t in self.old_cu_seqlens_list],
+            align_to_lengths=self.align_to_lengths,
+        )
+
+
+def tensor_container_to(d: Any, *args, **kwargs) -> Any:
+    """``.to(...)`` applied to every tensor of a nested dict / list / tuple; data.py:558-583."""
+    if torch.is_tensor(d):
+        return d.to(*args, **kwargs)
+    if isinstance(d, list):
+        return [tensor_container_to(v, *args, **kwargs) for v in d]
+    if isinstance(d, tuple):
+        return tuple(tensor_container_to(v, *args, **kwargs) for v in d)
+    if isinstance(d, dict):
+        return {k: tensor_container_to(v, *args, **kwargs) for k, v in d.items()}
+    return d
+
 
 def is_multi_modal_key(key: str) -> bool:
     return key.startswith("multi_modal_input")

@@ -148,3 +148,13 @@ def test_split_equals_oracle_on_cpu_tensors(algorithm, granularity):
         M.split_padded_tensor_dict_into_mb_list(data, M.MicroBatchSpec(granularity=5))
     with pytest.raises(ValueError, match="Call pad_mb_list first"):
         iter(got).__next__()
+
+
+def test_mb_list_to_moves_every_tensor():
+    attn = (torch.arange(6)[None, :] < torch.tensor([[6], [3], [2], [5]])).long()
+    data = dict(attention_mask=attn, input_ids=torch.arange(24).view(4, 6), meta=dict(w=torch.ones(2)), tag="x")
+    mbl = M.split_padded_tensor_dict_into_mb_list(data, M.MicroBatchSpec(n_mbs=2))
+    moved = mbl.to(torch.float64)
+    assert moved.mbs[0]["input_ids"].dtype == torch.float64 and moved.data["meta"]["w"].dtype == torch.float64
+    assert moved.mbs[0]["tag"] == "x" and moved.forward_indices == mbl.forward_indices
+    assert mbl.mbs[0]["input_ids"].dtype == torch.int64          # the original is untouched
