@@ -378,6 +378,31 @@ def pad_mb_list(mb_list: MicroBatchList, pad_value: float = 0.0, pad_to_maximum:
     return mb_list
 
 
+def unsqueeze_packed_tensor_dict(data: dict[str, Any], total_length: int | None = None) -> dict[str, Any]:
+    """A leading batch dimension of 1 on every packed tensor (``position_ids`` and every tensor with as many elements
+    as there are tokens), the form the model's forward takes; data.py:1077-1096.  ``total_length`` saves the read-back
+    of ``cu_seqlens[-1]`` when the caller knows it."""
+    assert "cu_seqlens" in data, "Input data must contain 'cu_seqlens' key."
+    assert "max_seqlen" in data, "Input data must contain 'max_seqlen' key."
+    if total_length is None:
+        total_length = int(data["cu_seqlens"][-1].item())
+    out = {}
+    for key, value in data.items():
+        packed = key == "position_ids" or (key not in ("cu_seqlens", "max_seqlen") and torch.is_tensor(value)
+                                           and value.numel() == total_length)
+        out[key] = value.unsqueeze(dim=0) if packed else value
+    return out
+
+
+def unsqueeze_mb_list(mb_list: MicroBatchList) -> MicroBatchList:
+    """``unsqueeze_packed_tensor_dict`` on every padded micro-batch; data.py:1099-1108.  The padded lengths are
+    known on the host, so nothing is read back."""
+    if mb_list.padded_mbs is not None:
+        lengths = mb_list.padded_to_lengths or [None] * len(mb_list.padded_mbs)
+        mb_list.padded_mbs = [unsqueeze_packed_tensor_dict(mb, n) for mb, n in zip(mb_list.padded_mbs, lengths)]
+    return mb_list
+
+
 def packed_mb_list(data: dict[str, Any], mb_spec: MicroBatchSpec, pad_value: float = 0.0, pad_to_maximum: bool = False,
                    batch_align_to: int | None = None, seq_align_to: int | None = None) -> MicroBatchList:
     """The chain an engine runs before its forward passes (areal/engine/fsdp_engine.py:1778-1786): position ids,

@@ -135,3 +135,22 @@ def test_packed_mb_list_matches_oracle_chain(device, algorithm, seq_align_to, pa
         if seq_align_to is not None:
             assert torch.equal(item.old_cu_seqlens.cpu(), old_cu)
     assert got.max_seqlen == max(int(m["cu_seqlens"][-1]) for m in got.padded_mbs)
+
+
+def test_unsqueeze_mb_list_adds_the_batch_dimension(device):
+    from areal_amd import microbatch as M
+
+    g = torch.Generator().manual_seed(2)
+    bs, L = 6, 50
+    lens = torch.randint(1, L + 1, (bs,), generator=g)
+    attn = (torch.arange(L)[None, :] < lens[:, None]).long()
+    data = dict(attention_mask=attn.to(device), input_ids=torch.randint(0, 9, (bs, L), generator=g).to(device),
+                rewards=torch.randn(bs, generator=g).to(device))
+    mbl = M.unsqueeze_mb_list(M.packed_mb_list(data, M.MicroBatchSpec(n_mbs=2)))
+    for item in mbl:
+        n = item.padded_to_length
+        assert item.padded_mb["input_ids"].shape == (1, n) and item.padded_mb["position_ids"].shape == (1, n)
+        assert item.padded_mb["cu_seqlens"].ndim == 1 and item.padded_mb["rewards"].shape == (bs,)
+        assert item.orig_mb["input_ids"].ndim == 1                                  # only the padded ones change
+    one = M.unsqueeze_packed_tensor_dict(mbl.mbs[0])
+    assert one["input_ids"].ndim == 2 and one["input_ids"].shape[0] == 1
