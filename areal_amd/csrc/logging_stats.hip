@@ -186,8 +186,9 @@ extern "C" int aa_logging_stats(const float* old_logp, const float* logp, const 
                                 void* stream) {
   if (n < 0 || !out || !scratch || methods < 0 || methods > 7) return AA_ERR_INVALID_ARGUMENT;
   if (n > 0 && (!old_logp || !logp || !mask)) return AA_ERR_INVALID_ARGUMENT;
-  if (methods != 0 && !versions) return AA_ERR_INVALID_ARGUMENT;
-  if (with_errors && !prox_logp_gt) return AA_ERR_INVALID_ARGUMENT;
+  // an empty batch may come with null data pointers: nothing is dereferenced, every row comes out empty
+  if (n > 0 && methods != 0 && !versions) return AA_ERR_INVALID_ARGUMENT;
+  if (n > 0 && with_errors && !prox_logp_gt) return AA_ERR_INVALID_ARGUMENT;
   const int parts = parts_for(n);
   if (scratch_bytes < (int64_t)kGroups * parts * kPerGroup * (int64_t)sizeof(Partial)) return AA_ERR_INVALID_ARGUMENT;
   hipStream_t st = (hipStream_t)stream;

@@ -331,6 +331,11 @@ def test_proximal_logging_stats_without_versions_or_tokens(device):
     got = areal_amd.proximal_logging_stats(old.to(device), lp.to(device), None, ver.to(device), 3, mask.to(device))
     assert float(got["version_stats"]["sample_staleness_theta"]["count"]) == 0
     assert sorted(got["compute_logp"]) == ["kl_div_direct", "kl_div_dual", "kl_div_taylor"]
+    # an empty batch (no tokens at all)
+    e = torch.zeros(0, device=device)
+    got = areal_amd.proximal_logging_stats(e, e, None, torch.zeros(0, dtype=torch.int32, device=device), 3,
+                                           torch.zeros(0, dtype=torch.bool, device=device), "loglinear")
+    assert float(got["compute_logp"]["loglinear/approx_logp"]["count"]) == 0
     # nothing selected at all
     got = areal_amd.proximal_logging_stats(old.to(device), lp.to(device), None, ver.to(device), 3,
                                            torch.zeros(n, dtype=torch.bool, device=device))
