@@ -532,8 +532,9 @@ using namespace aa::adv;
 extern "C" int aa_gae(const float* rewards, const float* values, const float* loss_mask, const uint8_t* seq_no_eos,
                       int64_t bs, int64_t L, float discount, float gae_lambda, float* advantages, float* returns,
                       void* stream) {
-  if (!rewards || !loss_mask || !advantages || bs < 0 || L < 1) return AA_ERR_INVALID_ARGUMENT;
+  if (bs < 0 || L < 1) return AA_ERR_INVALID_ARGUMENT;
   if (bs == 0) return AA_OK;
+  if (!rewards || !loss_mask || !advantages) return AA_ERR_INVALID_ARGUMENT;
   hipLaunchKernelGGL(k_gae, dim3((unsigned)bs), dim3(kGaeThreads), 0, (hipStream_t)stream, rewards, values, loss_mask,
                      seq_no_eos, bs, L, discount, gae_lambda, advantages, returns);
   return launch_status();

@@ -498,8 +498,9 @@ extern "C" int aa_rejection_sampling(const float* prox_logp, const float* old_lo
                                      const int32_t* cu_seqlens, int64_t B, int level, int action, int metric, int agg,
                                      float upper, float lower, int has_lower, uint8_t* mask_out, float* behave_w,
                                      int32_t* counts, void* stream) {
-  if (!prox_logp || !old_logp || !mask_in || !mask_out || !behave_w || !counts || n < 0)
-    return AA_ERR_INVALID_ARGUMENT;
+  if (!counts || n < 0) return AA_ERR_INVALID_ARGUMENT;
+  // an empty batch may come with null data pointers: only the counters are written
+  if (n > 0 && (!prox_logp || !old_logp || !mask_in || !mask_out || !behave_w)) return AA_ERR_INVALID_ARGUMENT;
   if (level < 0 || level > 1 || action < 0 || action > 1 || metric < 0 || metric > 3 || agg < 0 || agg > 2)
     return AA_ERR_INVALID_ARGUMENT;
   if (action == AA_RS_ACTION_CLAMP && metric != AA_RS_RATIO) return AA_ERR_INVALID_ARGUMENT;

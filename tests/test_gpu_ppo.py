@@ -189,3 +189,21 @@ def test_masked_positions_and_denominator_keep_reference_semantics(device):
     manual = float(stat["loss"].cpu()[kept].double().sum()) / int(mask.sum())
     assert float(loss) == pytest.approx(manual, rel=1e-5)
     assert float(stat["importance_weight"].cpu()[~kept].abs().sum()) == 0.0
+
+
+def test_empty_batches_do_not_raise(device):
+    """Zero tokens (a data-parallel rank without work): empty results, zero counts, no launch over null pointers."""
+    from areal_amd import RejectionSamplingConfig
+
+    e = torch.zeros(0, device=device)
+    eb = torch.zeros(0, dtype=torch.bool, device=device)
+    cu0 = torch.zeros(1, dtype=torch.int32, device=device)
+    for level in ("token", "sequence"):
+        res = areal_amd.apply_rejection_sampling(e, e, eb, cu0, RejectionSamplingConfig(level=level, metric="ratio",
+                                                                                         upper=2.0))
+        assert res.loss_mask.numel() == 0 and res.filtered_fraction == 0.0
+    loss, stat = areal_amd.ppo_actor_loss_fn(e.clone().requires_grad_(True), e, e, e, 0.2, eb)
+    assert float(loss.detach()) == 0.0 and stat["importance_weight"].numel() == 0
+    adv, ret = areal_amd.gae_advantages(torch.zeros(0, 8, device=device), torch.zeros(0, 8, device=device),
+                                        torch.zeros(0, 8, device=device), eb, 1.0, 0.95)
+    assert adv.shape == (0, 8) and ret.shape == (0, 8)
