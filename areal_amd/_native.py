@@ -76,13 +76,14 @@ SIGNATURES = {
     "aa_masked_sum": (_i, [_p, _p, _i64, _p, _p, _p, _p]),
     "aa_scale_inplace": (_i, [_p, _i, _i64, _p, _p]),
     "aa_lmhead_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "aa_lmhead_fwd_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "aa_lmhead_fwd": (_i, [_p, _p, _i64, _i64, _i64, _p, _f, _p, _p, _p, _p, _p, _i64, _p]),
     "aa_lmhead_chunk_tokens": (_i64, []),
     "aa_lmhead_bwd": (_i, [_p, _p, _i64, _i64, _i64, _p, _f, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i64, _p]),
     "aa_lmhead_ppo_fused": (
         _i,
-        [_p, _p, _i64, _i64, _i64, _p, _f, _i64, _p, _p, _p, _p, C.POINTER(PpoParams), _p, _p, _p,
-         _p, _p, _p, _p, _p, _p, _p, _i, _p, _p, _i64, _p],
+        [_p, _p, _i64, _i64, _i64, _p, _f, _i64, _p, _p, _p, _p, C.POINTER(PpoParams), _p, _p, _p, _i,
+         _p, _p, _p, _p, _p, _p, _p, _i, _p, _i64, _p],
     ),
     "aa_sapo_loss": (_i, [_p, _p, _p, _p, _i64, _p, _i64, _i, _f, _f, _p, _p, _p, _p, _p, _p]),
     "aa_critic_loss": (_i, [_p, _p, _p, _p, _i64, _f, _i, _p, _p, _p, _p, _p]),

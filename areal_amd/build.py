@@ -27,8 +27,8 @@ HIPCC_FLAGS = [
 ]
 
 
-# hipBLASLt serves the plain GEMMs of the lm_head path
-LINK_LIBS = ["-L/opt/rocm/lib", "-lhipblaslt"]
+# the library links against the HIP runtime only
+LINK_LIBS: list[str] = []
 
 
 def _hipcc() -> str:

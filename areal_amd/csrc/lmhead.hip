@@ -1,36 +1,385 @@
 // lm_head path for gfx950: log-prob / entropy of softmax(hidden @ weight.T / T), their backward, and the whole
-// lm_head + PPO-loss training step, holding at most one token chunk of logits in memory.  The reference has no such
-// path: its equivalent is the lm_head matmul followed by gather_logprobs_entropy
-// (areal/utils/functional/vocab_parallel.py:23-29), ppo_actor_loss_fn and autograd.
+// lm_head + PPO-loss training step, on this library's own bf16 MFMA tile GEMM (gemm_tn.h), without ever writing the
+// [T, V] logits to memory.  The reference has no such path: its equivalent is the lm_head matmul followed by
+// gather_logprobs_entropy (areal/utils/functional/vocab_parallel.py:23-29), ppo_actor_loss_fn
+// (areal/utils/functional/functional.py:429-559) and autograd.
 //
-// Tokens go through in chunks of at most kChunkTokens.  Per chunk the plain GEMMs go to hipBLASLt (lt_gemm.h), always
-// in the form the library runs fastest on this chip (contraction index contiguous in both operands), and everything
-// else is one of this library's streaming kernels over the chunk's bf16 logits panel:
-//   forward        panel = hidden_c . W^T (bf16, as the reference's lm_head output is)  ->  k_logits_fwd
-//   backward       panel again  ->  k_logits_bwd in place  ->  d_hidden_c, d_weight
-//   training step  panel  ->  the fused log-prob / entropy / PPO-loss / gradient kernel in place  ->  d_hidden_c, d_weight
-// The gradient GEMMs take transposed copies of the panel, of the hidden chunk and of the weight (k_transpose_bf16).
+// Forward (aa_lmhead_fwd, and the first half of the training step): 256 (vocabulary) x 256 (tokens) tiles of the
+// logits are formed in accumulator registers; the epilogue reduces every 128-row block of a tile to the softmax
+// partials (k, s, u) per token and captures the label logit; a small kernel merges the partials of all blocks into
+// log-prob and entropy.  Nothing of size T x V is written.
+//
+// Backward needs d(logits) twice (for d_hidden and for d_weight), so a bf16 panel [tokens with gradient, V] of it is
+// written once per token chunk and contracted by two plain tile GEMMs.  Two ways to fill the panel:
+//   recompute   the logits tiles are formed again and turned into d(logits) in registers (2 T_grad V H extra flops);
+//               what aa_lmhead_bwd does, where the upstream gradients only exist after the forward has returned.
+//   carry       (training step only) the forward tiles also write 2^(x c - k_block), the unnormalised probabilities
+//               that their statistics are made of, for the tokens that will have a gradient; once the row statistics
+//               and the loss are known, a streaming pass scales each 128-wide block of a row by
+//               -(g / T) 2^(k_block - k_row) / s_row and adds g / T at the label: the same d(logits), no second GEMM.
+// Tokens whose loss mask is zero have a zero gradient row: they are left out of the panel and of both GEMMs.
 #include "device_utils.h"
-#include "logits_path.h"
-#include "lt_gemm.h"
+#include "gemm_tn.h"
+#include "ppo_math.h"
 
 namespace aa {
 namespace lmhead {
 
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+using namespace gemm;
 
-constexpr int kChunkTokens = 16384;  // token chunk of the logits panel
+constexpr int kChunkTokens = 16384;        // token chunk of the panel
+constexpr int kPanelPitch = BM + 8;        // pitch (elements) of the tile staged in LDS as [token][vocab]
+constexpr int kStageBytes = 256 * kPanelPitch * 2;  // 135168 B, inside the 160 KiB the main loop uses
+static_assert(kStageBytes <= wide::kLdsBytes, "the staged tile must fit the main loop's LDS");
 
 __host__ __device__ __forceinline__ int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
+enum { kModeStats = 0, kModeStatsCarry = 1, kModeRecompute = 2 };
+
+struct TileArgs {
+  // statistics per (128-row vocabulary block, token): planes [blocks][pitch_t]
+  float* pk;
+  float* ps;
+  float* pu;
+  float* xy;              // [tokens of the chunk] raw label logit, written by the block that holds the label
+  const int64_t* labels;  // labels of the chunk
+  int64_t pitch_t;
+  float c;                // log2(e) / temperature
+  // panel [rows, panel_ld] bf16: row out_rows[token] (or the token itself when out_rows is null); negative: no row
+  uint16_t* panel;
+  int64_t panel_ld;
+  const int32_t* out_rows;
+  // recompute: per token of the chunk; column n of the tile is token col_tokens[n] (or n when null)
+  const int32_t* col_tokens;
+  const float* row_lse;    // natural-log logsumexp of the row
+  const float* row_ez;     // sum_j p_j z_j (used with g_entropy)
+  const float* g_logp;
+  const float* g_entropy;  // nullable
+  float inv_t;
+};
+
+// One 256 x 256 tile: rows m = vocabulary (operand A = weight), columns n = tokens (operand B = hidden states), so
+// that everything a token needs from the tile sits in one lane and its partner lane ^ 32.
+template <int MODE>
+__global__ __launch_bounds__(wide::kThreads) void k_lmhead_tiles(Operand W, Operand Hd, int K, int tiles_m, int tiles_n,
+                                                                 TileArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  int tm, tn;
+  tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  Acc<wide::S> acc;
+  wide::mainloop<0>(W, Hd, K, m0, n0, acc, lds);  // ends with a barrier: LDS is free
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int V = W.rows, N = Hd.rows;
+  const int mbase = m0 + wm * 128;    // first vocabulary row of this wave's block
+  const bool ragged = m0 + BM > V;    // rows past the vocabulary: last tile row only
+  uint16_t* Z = (uint16_t*)lds;       // [256 tokens][kPanelPitch] bf16
+  constexpr int PZ = kPanelPitch;
+
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) {
+    const int nloc = wn * 128 + acc_col(nt, lane);
+    const int n = n0 + nloc;
+    const bool live = n < N;
+    if constexpr (MODE != kModeRecompute) {
+      float mx = -FLT_MAX;
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const bool in = !ragged || (mbase + acc_row(mt, i, lane) < V);
+          mx = in ? fmaxf(mx, acc.v[mt][nt][i]) : mx;
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));  // both halves of the wave hold the same token
+      const float k = fmaxf(mx * a.c, kNegBig);   // kNegBig: no valid row in this block
+      float s = 0.f, u = 0.f;
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          float e[4];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const bool in = !ragged || (mbase + acc_row(mt, g4 * 4 + q, lane) < V);
+            const float t = in ? fmaf(acc.v[mt][nt][g4 * 4 + q], a.c, -k) : 0.f;
+            e[q] = in ? fast_exp2(t) : 0.f;
+            s += e[q];
+            u = fmaf(t, e[q], u);
+          }
+          if constexpr (MODE == kModeStatsCarry) {
+            uint2 pk;
+            pk.x = Elem<AA_BF16>::pack(e[0], e[1]);
+            pk.y = Elem<AA_BF16>::pack(e[2], e[3]);
+            *(uint2*)(Z + nloc * PZ + wm * 128 + mt * 32 + 8 * g4 + 4 * (lane >> 5)) = pk;
+          }
+        }
+      s += __shfl_xor(s, 32, kWave);
+      u += __shfl_xor(u, 32, kWave);
+      if (lane < 32 && live) {
+        const int64_t at = (int64_t)(tm * 2 + wm) * a.pitch_t + n;
+        a.pk[at] = k;
+        a.ps[at] = s;
+        a.pu[at] = u;
+      }
+      // label logit, if the label falls into this wave's 128 vocabulary rows (one of the two partner lanes owns it)
+      if (live) {
+        const int64_t y = a.labels[n];
+        const int64_t rel = y - mbase;
+        if (rel >= 0 && rel < 128 && y < V && (int)((rel >> 2) & 1) == (lane >> 5)) {
+          const int mt_y = (int)(rel >> 5), r5 = (int)(rel & 31);
+          const int i_y = ((r5 >> 3) << 2) | (r5 & 3);
+          float val = 0.f;
+#pragma unroll
+          for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+              if (mt == mt_y && i == i_y) val = acc.v[mt][nt][i];
+          a.xy[n] = val;
+        }
+      }
+    } else {
+      float A = 0.f, B = 0.f, lab_add = 0.f, lse2 = 0.f;
+      int64_t y = -1;
+      if (live) {
+        const int t = a.col_tokens ? a.col_tokens[n] : n;
+        const float gl = a.g_logp[t];
+        const float gh = a.g_entropy ? a.g_entropy[t] : 0.f;
+        const float ez = a.g_entropy ? a.row_ez[t] : 0.f;
+        lse2 = a.row_lse[t] * kLog2e;
+        A = a.inv_t * (gh * ez - gl);
+        B = -gh * a.inv_t * a.inv_t;
+        lab_add = gl * a.inv_t;
+        y = a.labels[t];
+      }
+      const int64_t rel = y - mbase;
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          float o[4];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const float x = acc.v[mt][nt][g4 * 4 + q];
+            o[q] = live ? fast_exp2(fmaf(x, a.c, -lse2)) * fmaf(B, x, A) : 0.f;
+          }
+          const int r0 = mt * 32 + 8 * g4 + 4 * (lane >> 5);  // row of o[0] inside the wave's block
+          if (rel >= r0 && rel < r0 + 4) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              if (rel - r0 == q) o[q] += lab_add;
+          }
+          uint2 pk;
+          pk.x = Elem<AA_BF16>::pack(o[0], o[1]);
+          pk.y = Elem<AA_BF16>::pack(o[2], o[3]);
+          *(uint2*)(Z + nloc * PZ + wm * 128 + r0) = pk;
+        }
+    }
+  }
+  if constexpr (MODE != kModeStats) {
+    __syncthreads();
+    // panel rows: 16-byte pieces along the vocabulary (V % 8 == 0: a piece never straddles the end)
+    for (int p = tid; p < 256 * 32; p += wide::kThreads) {
+      const int nloc = p >> 5, mc = (p & 31) * 8;
+      const int n = n0 + nloc, m = m0 + mc;
+      if (n < N && m < V) {
+        const int r = a.out_rows ? a.out_rows[n] : n;
+        if (r >= 0) *(u32x4_t*)(a.panel + (int64_t)r * a.panel_ld + m) = *(const u32x4_t*)(Z + nloc * PZ + mc);
+      }
+    }
+  }
+}
+
+// Merge of the block partials of one token, in block order (fixed order: deterministic)
+struct Merged {
+  float k, s, u;
+};
+__device__ __forceinline__ Merged merge_blocks(const float* __restrict__ pk, const float* __restrict__ ps,
+                                               const float* __restrict__ pu, int blocks, int64_t pitch_t, int64_t t) {
+  float k = kNegBig, s = 0.f, u = 0.f;
+  for (int b = 0; b < blocks; ++b) {
+    const int64_t at = (int64_t)b * pitch_t + t;
+    const float bk = pk[at], bs = ps[at], bu = pu[at];
+    const float nk = fmaxf(k, bk);
+    const float da = k - nk, db = bk - nk;
+    const float fa = fast_exp2(da), fb = fast_exp2(db);
+    u = fa * fmaf(da, s, u) + fb * fmaf(db, bs, bu);
+    s = s * fa + bs * fb;
+    k = nk;
+  }
+  return {k, s, u};
+}
+
+__global__ __launch_bounds__(256) void k_fill_f32(float* p, int64_t n, float v) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+// forward of the stand-alone op: one thread per token
+__global__ __launch_bounds__(256) void k_combine(const float* __restrict__ pk, const float* __restrict__ ps,
+                                                 const float* __restrict__ pu, const float* __restrict__ xy, int blocks,
+                                                 int64_t pitch_t, int n_tok, float c, float* __restrict__ logp,
+                                                 float* __restrict__ entropy, float* __restrict__ row_lse,
+                                                 float* __restrict__ row_ez) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= n_tok) return;
+  const Merged m = merge_blocks(pk, ps, pu, blocks, pitch_t, t);
+  const float log2s = fast_log2(m.s);
+  const float mean_t = m.u / m.s;
+  logp[t] = (fmaf(xy[t], c, -m.k) - log2s) * kLn2;  // xy stays NaN for a label outside [0, V)
+  if (entropy) entropy[t] = (log2s - mean_t) * kLn2;
+  if (row_lse) row_lse[t] = (m.k + log2s) * kLn2;
+  if (row_ez) row_ez[t] = (m.k + mean_t) * kLn2;
+}
+
+// What the streaming pass of the carry mode needs per panel row
+struct RowCoef {
+  float k_row;    // row maximum of x c
+  float base;     // -(g / T) / s_row
+  float lab_add;  // g / T
+  int32_t label;  // label of the row's token (-1 when it lies outside the vocabulary)
+};
+
+struct TokenLossArgs {
+  const float* prox_logp;
+  const float* adv;
+  const uint8_t* mask_eff;
+  const float* behave_w;
+  const int32_t* n_valid;
+  const float* grad_scale;
+  float* logp;
+  float* entropy;
+  float* stat_loss;
+  float* ratio;
+  uint8_t* flags;
+  aa_ppo_params P;
+  int64_t act;  // tokens of the chunk that are inside T_active
+};
+
+// Training step, after the forward tiles of a chunk: log-prob, entropy, per-token loss outputs (as the fused logits
+// kernel writes them, areal/utils/functional/functional.py:505-558) and g = d(scaled loss) / d(logp); then what the
+// backward needs: g and the row's logsumexp per token (recompute), or the row coefficients per panel row (carry).
+__global__ __launch_bounds__(256) void k_token_loss(const float* __restrict__ pk, const float* __restrict__ ps,
+                                                    const float* __restrict__ pu, const float* __restrict__ xy, int blocks,
+                                                    int64_t pitch_t, int n_tok, int V, float c, float inv_t,
+                                                    const int64_t* __restrict__ labels, TokenLossArgs a,
+                                                    const int32_t* __restrict__ out_rows, float* __restrict__ g_tok,
+                                                    float* __restrict__ lse_tok, RowCoef* __restrict__ rowc) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= n_tok) return;
+  const Merged m = merge_blocks(pk, ps, pu, blocks, pitch_t, t);
+  const float log2s = fast_log2(m.s);
+  const float lp = (fmaf(xy[t], c, -m.k) - log2s) * kLn2;
+  a.logp[t] = lp;
+  if (a.entropy) a.entropy[t] = (log2s - m.u / m.s) * kLn2;
+  float g = 0.f;
+  if (t < a.act) {
+    int n = *a.n_valid;
+    float fn;
+    if (a.P.loss_kind == AA_LOSS_NLL) {
+      fn = (float)n + 1e-5f;  // the supervised loss divides by 1e-5 + count (areal/trainer/sft/lm_engine.py:96)
+    } else {
+      fn = (float)(n < 1 ? 1 : n);
+    }
+    const float gscale = a.grad_scale ? *a.grad_scale : 1.f;
+    const bool on = a.mask_eff[t] != 0;
+    if (a.P.loss_kind == AA_LOSS_NLL) {
+      a.stat_loss[t] = on ? -lp : 0.f;
+      a.ratio[t] = 0.f;
+      a.flags[t] = 0;
+      g = on ? (-1.f / fn) * gscale : 0.f;
+    } else {
+      const float r = on ? expf(lp - a.prox_logp[t]) : 0.f;
+      const Surrogate sg = surrogate(r, a.adv[t], a.P.has_behave_weight ? a.behave_w[t] : 1.f, a.P);
+      a.stat_loss[t] = sg.loss;
+      a.ratio[t] = r;
+      a.flags[t] = (uint8_t)(((sg.clip && on) ? 1 : 0) | ((sg.dual && on) ? 2 : 0));
+      g = on ? (sg.dloss_dr * r / fn) * gscale : 0.f;
+    }
+  }
+  if (g_tok) g_tok[t] = g;
+  if (lse_tok) lse_tok[t] = (m.k + log2s) * kLn2;
+  if (rowc) {
+    const int r = out_rows ? out_rows[t] : t;
+    if (r >= 0) {
+      const int64_t y = labels[t];
+      rowc[r] = {m.k, -(g * inv_t) / m.s, g * inv_t, (y >= 0 && y < V) ? (int32_t)y : -1};
+    }
+  }
+}
+
+// Carry mode: panel row r holds 2^(x c - k_block) of token act_rows[r] (or r); scale every 128-wide block to
+// d(loss)/d(logits) in place.  One workgroup per row, 16-byte pieces (all 8 elements of a piece lie in one block).
+__global__ __launch_bounds__(256) void k_panel_scale(uint16_t* __restrict__ panel, int64_t panel_ld, int V,
+                                                     const RowCoef* __restrict__ rowc, const int32_t* __restrict__ act_rows,
+                                                     const float* __restrict__ pk, int64_t pitch_t) {
+  const int r = blockIdx.x;
+  const RowCoef rc = rowc[r];
+  const int64_t t = act_rows ? act_rows[r] : r;
+  uint16_t* row = panel + (int64_t)r * panel_ld;
+  const int pieces = V >> 3;
+  for (int p = threadIdx.x; p < pieces; p += 256) {
+    const float f = rc.base * fast_exp2(pk[(int64_t)(p >> 4) * pitch_t + t] - rc.k_row);
+    float x[8];
+    load8<AA_BF16>(row, (int64_t)p * 8, x);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[j] *= f;
+    const int rel = rc.label - p * 8;
+    if (rel >= 0 && rel < 8) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (rel == j) x[j] += rc.lab_add;
+    }
+    store8<AA_BF16>(row, (int64_t)p * 8, x);
+  }
+}
+
+// ---- plain product D = A . B^T on the same main loop ---------------------------------------------------------------
+// D [M, N] row-major with leading dimension ldd, bf16 or fp32; ACCUM adds to what D holds (fp32 only).
+template <typename OutT, bool ACCUM>
+__global__ __launch_bounds__(wide::kThreads) void k_gemm_store(Operand A, Operand B, int K, int tiles_m, int tiles_n,
+                                                               OutT* __restrict__ D, int64_t ldd) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  int tm, tn;
+  tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  Acc<wide::S> acc;
+  wide::mainloop<0>(A, B, K, m0, n0, acc, lds);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int M = A.rows, N = B.rows;
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int m = m0 + wm * 128 + acc_row(mt, i, lane);
+      if (m >= M) continue;
+      OutT* row = D + (int64_t)m * ldd;
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        const int n = n0 + wn * 128 + acc_col(nt, lane);
+        if (n >= N) continue;
+        float v = acc.v[mt][nt][i];
+        if constexpr (sizeof(OutT) == 4) {
+          if (ACCUM) v += row[n];
+          row[n] = v;
+        } else {
+          row[n] = (uint16_t)(Elem<AA_BF16>::pack(v, 0.f) & 0xffffu);
+        }
+      }
+    }
+}
+
 // ---- bf16 transpose: dst[c, r] = src[r, c] ----------------------------------------------------------------------
-// src is [R, C] with row pitch lds (elements), dst is [C, ldd] with ldd = R rounded up to 8; columns R .. ldd - 1 of dst
-// are written as zeros; with src_rows, row r of the source is row src_rows[r] of the array.  One workgroup moves a 64 x 64 tile through LDS: each thread loads 8 elements of two
-// adjacent rows (16 B each), pairs them into 32-bit words (two consecutive dst columns) and stores the words
-// transposed; the second half reads 16 B per thread and writes 128 B contiguous per dst row.  The word index is
-// XOR-ed with a key of the row so that both halves run without bank conflicts.  Requires C % 8 == 0, lds % 8 == 0.
-// Tiles are numbered along r first, in bands of kTransposeBand tile rows, so that the workgroups in flight together
-// write long contiguous pieces of the dst rows (measured: 5.2 TB/s against 3.9 with c first).
+// src is [R, C] with row pitch lds (elements), dst is [C, ldd] with ldd >= R a multiple of 8; columns R .. ldd - 1 of dst
+// are written as zeros; with src_rows, row r of the source is row src_rows[r] of the array.  One workgroup moves a
+// 64 x 64 tile through LDS: each thread loads 8 elements of two adjacent rows (16 B each), pairs them into 32-bit
+// words (two consecutive dst columns) and stores the words transposed; the second half reads 16 B per thread and
+// writes 128 B contiguous per dst row.  The word index is XOR-ed with a key of the row so that both halves run
+// without bank conflicts.  Requires C % 8 == 0, lds % 8 == 0.  Tiles are numbered along r first, in bands of
+// kTransposeBand tile rows, so that the workgroups in flight together write long contiguous pieces of the dst rows
+// (measured: 5.2 TB/s against 3.9 with c first).
 constexpr int kTransposeBand = 64;
 
 __global__ __launch_bounds__(256) void k_transpose_bf16(const uint16_t* __restrict__ src, int R, int C, int64_t lds,
@@ -126,6 +475,14 @@ __global__ __launch_bounds__(256) void k_scatter_rows(const u32x4_t* __restrict_
   for (int j = threadIdx.x; j < h_vec; j += 256) dst[t * h_vec + j] = r >= 0 ? src[(int64_t)r * h_vec + j] : zero;
 }
 
+// dst[r, :] = src[rows[r], :] (H % 8 == 0)
+__global__ __launch_bounds__(256) void k_gather_rows(const u32x4_t* __restrict__ src, const int32_t* __restrict__ rows,
+                                                     u32x4_t* __restrict__ dst, int h_vec) {
+  const int64_t r = blockIdx.x;
+  const int64_t t = rows[r];
+  for (int j = threadIdx.x; j < h_vec; j += 256) dst[r * h_vec + j] = src[t * h_vec + j];
+}
+
 __global__ __launch_bounds__(256) void k_zero16(u32x4_t* __restrict__ p, int64_t n_vec) {
   const u32x4_t zero = {0u, 0u, 0u, 0u};
   const int64_t step = (int64_t)gridDim.x * 256;
@@ -155,64 +512,133 @@ __global__ __launch_bounds__(256) void k_f32_to_bf16(const f32x4_t* __restrict__
   __builtin_nontemporal_store(o, dst + i);
 }
 
+// ---- workspace ---------------------------------------------------------------------------------------------------
 struct Workspace {
-  int64_t off_ds, off_lt;           // the [chunk, V] panel, scratch of the GEMM library
-  int64_t off_dst, off_wt, off_ht;  // transposed copies: panel [V, chunk], weight [H, V], hidden chunk [H, chunk]
-  int64_t off_dw;                   // fp32 accumulator of a bf16 d_weight when there is more than one chunk
-  int64_t off_rows, off_dhc;        // row maps of k_compact_map (2 x chunk int32), d_hidden of the kept tokens
-  int64_t chunk;
+  int64_t chunk, blocks;                // tokens per chunk, 128-row vocabulary blocks
+  int64_t off_pk, off_ps, off_pu;       // block partials [blocks][chunk]
+  int64_t off_xy, off_g, off_lse;       // per token of the chunk: label logit, g, logsumexp
+  int64_t fwd_bytes;                    // what the forward alone needs
+  int64_t off_rowc;                     // RowCoef per panel row
+  int64_t off_rows;                     // out_rows, act_rows (2 x chunk int32)
+  int64_t off_panel, off_panel_t;       // d(logits) rows [chunk, V] and their transpose [V, chunk]
+  int64_t off_wt, off_ht;               // weight^T [H, V], hidden rows^T [H, chunk]
+  int64_t off_dhc, off_hc;              // d_hidden of the rows with gradient [chunk, H]; those rows of hidden
+  int64_t off_dw;                       // fp32 accumulator of a bf16 d_weight when there is more than one chunk
   int64_t bytes;
 };
 
 static Workspace plan(int64_t T, int64_t H, int64_t V) {
   Workspace w{};
   auto up = [](int64_t x) { return (x + 255) / 256 * 256; };
-  int64_t off = 0;
   w.chunk = T < kChunkTokens ? round_up(T, 256) : kChunkTokens;
-  w.off_ds = off;  off += up(w.chunk * V * 2);
-  w.off_lt = off;  off += lt::kWorkspaceBytes;
-  w.off_dst = off; off += up(w.chunk * V * 2);
-  w.off_wt = off;  off += up(H * V * 2);
-  w.off_ht = off;  off += up(w.chunk * H * 2);
-  w.off_dw = off;  off += T > w.chunk ? up(V * H * 4) : 0;
-  w.off_rows = off; off += up(2 * w.chunk * 4);
-  w.off_dhc = off;  off += up(w.chunk * H * 2);
+  w.blocks = 2 * ((V + BM - 1) / BM);
+  int64_t off = 0;
+  w.off_pk = off;  off += up(w.blocks * w.chunk * 4);
+  w.off_ps = off;  off += up(w.blocks * w.chunk * 4);
+  w.off_pu = off;  off += up(w.blocks * w.chunk * 4);
+  w.off_xy = off;  off += up(w.chunk * 4);
+  w.off_g = off;   off += up(w.chunk * 4);
+  w.off_lse = off; off += up(w.chunk * 4);
+  w.fwd_bytes = off;
+  w.off_rowc = off;    off += up(w.chunk * (int64_t)sizeof(RowCoef));
+  w.off_rows = off;    off += up(2 * w.chunk * 4);
+  w.off_panel = off;   off += up(w.chunk * V * 2);
+  w.off_panel_t = off; off += up(w.chunk * V * 2);
+  w.off_wt = off;      off += up(H * V * 2);
+  w.off_ht = off;      off += up(w.chunk * H * 2);
+  w.off_dhc = off;     off += up(w.chunk * H * 2);
+  w.off_hc = off;      off += up(w.chunk * H * 2);
+  w.off_dw = off;      off += T > w.chunk ? up(V * H * 4) : 0;
   w.bytes = off;
   return w;
 }
 
-// logits[t0 : t0 + n_tok, :] = hidden . W^T, rounded to bf16.  Row-major [n_tok, V] is column-major [V, n_tok]:
-// W'^T [V, H] . hidden' [H, n_tok].
-static bool panel_logits(hipStream_t st, const Workspace& w, char* ws, const uint16_t* hid, const void* weight,
-                         int64_t n_tok, int64_t H, int64_t V) {
-  return lt::gemm(st, true, false, V, n_tok, H, weight, H, hid, H, ws + w.off_ds, V, false, 0.f, ws + w.off_lt,
-                  lt::kWorkspaceBytes);
+static bool shapes_ok(int64_t T, int64_t H, int64_t V) {
+  // 256 rows of any operand must stay below 2^30 elements (32-bit byte offsets inside a tile)
+  return T > 0 && H > 0 && V > 0 && (H % 8) == 0 && (V % 8) == 0 && T < (1 << 30) && V < (1 << 22) && H < (1 << 22) &&
+         (V / 64 + 1) * ((H > kChunkTokens ? H : kChunkTokens) / 64 + 1) < (1LL << 31);  // transpose grids
 }
 
-// The two GEMMs that contract the d(logits) rows ds [n_rows, V] of one token chunk:
+// The tile kernels use all 160 KiB of LDS: allow it once per kernel and device.
+template <typename Kern>
+static bool allow_big_lds(Kern k) {
+  return hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, wide::kLdsBytes) == hipSuccess;
+}
+
+static bool prepare_kernels() {
+  constexpr int kMaxDevices = 64;
+  static bool done[kMaxDevices] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return false;
+  if (done[dev]) return true;
+  const bool ok = allow_big_lds(k_lmhead_tiles<kModeStats>) && allow_big_lds(k_lmhead_tiles<kModeStatsCarry>) &&
+                  allow_big_lds(k_lmhead_tiles<kModeRecompute>) && allow_big_lds(k_gemm_store<uint16_t, false>) &&
+                  allow_big_lds(k_gemm_store<float, false>) && allow_big_lds(k_gemm_store<float, true>);
+  done[dev] = ok;
+  return ok;
+}
+
+template <int MODE>
+static void launch_tiles(hipStream_t st, const void* weight, const uint16_t* hid, int64_t n_tok, int64_t H, int64_t V,
+                         const TileArgs& a) {
+  const int tiles_m = (int)((V + BM - 1) / BM), tiles_n = (int)((n_tok + BN - 1) / BN);
+  Operand W{(const uint16_t*)weight, H, (int)V};
+  Operand Hd{hid, H, (int)n_tok};
+  hipLaunchKernelGGL(k_lmhead_tiles<MODE>, dim3((unsigned)(tiles_m * tiles_n)), dim3(wide::kThreads), wide::kLdsBytes, st,
+                     W, Hd, (int)H, tiles_m, tiles_n, a);
+}
+
+// D [M, N] = A [M, K] . B [N, K]^T
+template <typename OutT, bool ACCUM>
+static void launch_gemm(hipStream_t st, const uint16_t* A, int64_t lda, int64_t M, const uint16_t* B, int64_t ldb, int64_t N,
+                        int64_t K, OutT* D, int64_t ldd) {
+  const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
+  Operand a{A, lda, (int)M}, b{B, ldb, (int)N};
+  hipLaunchKernelGGL((k_gemm_store<OutT, ACCUM>), dim3((unsigned)(tiles_m * tiles_n)), dim3(wide::kThreads),
+                     wide::kLdsBytes, st, a, b, (int)K, tiles_m, tiles_n, D, ldd);
+}
+
+// The two GEMMs that contract the d(logits) rows ds [n_rows, V] (in the panel) of one token chunk:
 //   d_hidden rows = ds . W          (bf16)          d_weight (+)= ds^T . hidden rows   (fp32, or bf16 when first)
-// with transposed copies of ds and of the hidden rows (made here) and of the weight (made once per call, by the
-// caller, at ws + off_wt).  ds sits in one of the two panel buffers (byte offset ds_off), its transpose goes to the
-// other (dst_off).  hid_rows, when given, lists the rows of the hidden chunk that the n_rows rows of ds belong to
-// (tokens without gradient were left out).  The GEMMs run on n_gemm >= n_rows rows (the library is much faster on
-// round sizes): the transposed copies carry zeros there.  d_hidden_rows receives n_dh rows (n_rows, or n_gemm when
-// it is a scratch buffer with room for them).
-static bool panel_gradients(hipStream_t st, const Workspace& w, char* ws, int64_t ds_off, int64_t dst_off,
-                            const uint16_t* hid, const int32_t* hid_rows, int64_t n_rows, int64_t n_gemm, int64_t n_dh,
-                            int64_t H, int64_t V, uint16_t* d_hidden_rows, void* d_weight, bool dw_f32, bool first) {
-  const uint16_t* ds = (const uint16_t*)(ws + ds_off);
-  uint16_t* ds_t = (uint16_t*)(ws + dst_off);
+// with transposed copies of ds and of the hidden rows (made here; their token count is padded to a multiple of 8 with
+// zeros) and of the weight (made once per call, by the caller, at ws + off_wt).  hid_rows, when given, lists the rows
+// of the hidden chunk that the n_rows rows of ds belong to (tokens without gradient were left out).
+static void panel_gradients(hipStream_t st, const Workspace& w, char* ws, const uint16_t* hid, const int32_t* hid_rows,
+                            int64_t n_rows, int64_t H, int64_t V, uint16_t* d_hidden_rows, void* d_weight, bool dw_f32,
+                            bool first) {
+  const uint16_t* ds = (const uint16_t*)(ws + w.off_panel);
+  uint16_t* ds_t = (uint16_t*)(ws + w.off_panel_t);
   const uint16_t* w_t = (const uint16_t*)(ws + w.off_wt);
   uint16_t* hid_t = (uint16_t*)(ws + w.off_ht);
-  void* lt_ws = ws + w.off_lt;
-  // column-major [H, n_dh] = (W^T)'^T [H, V] . ds' [V, n_dh]
-  if (!lt::gemm(st, true, false, H, n_dh, V, w_t, V, ds, V, d_hidden_rows, H, false, 0.f, lt_ws, lt::kWorkspaceBytes))
-    return false;
-  launch_transpose(st, ds, n_rows, V, V, ds_t, n_gemm);
-  launch_transpose(st, hid, n_rows, H, H, hid_t, n_gemm, hid_rows);
-  // column-major [H, V] = (hidden^T)'^T [H, n_gemm] . (ds^T)' [n_gemm, V], fp32, accumulated over the chunks
-  return lt::gemm(st, true, false, H, V, n_gemm, hid_t, n_gemm, ds_t, n_gemm, d_weight, H, dw_f32, first ? 0.f : 1.f,
-                  lt_ws, lt::kWorkspaceBytes);
+  const int64_t kp = round_up(n_rows, 8);
+  launch_gemm<uint16_t, false>(st, ds, V, n_rows, w_t, V, H, V, d_hidden_rows, H);
+  launch_transpose(st, ds, n_rows, V, V, ds_t, kp);
+  launch_transpose(st, hid, n_rows, H, H, hid_t, kp, hid_rows);
+  if (!dw_f32)
+    launch_gemm<uint16_t, false>(st, ds_t, kp, V, hid_t, kp, H, kp, (uint16_t*)d_weight, H);
+  else if (first)
+    launch_gemm<float, false>(st, ds_t, kp, V, hid_t, kp, H, kp, (float*)d_weight, H);
+  else
+    launch_gemm<float, true>(st, ds_t, kp, V, hid_t, kp, H, kp, (float*)d_weight, H);
+}
+
+// Recompute: d(logits) of the panel rows from the logits tiles formed again.  With a row map only the hidden rows that
+// have a panel row are multiplied (gathered first); `a` carries the per-token inputs of the chunk.
+static void recompute_panel(hipStream_t st, const Workspace& w, char* ws, const void* weight, const uint16_t* hid,
+                            int64_t n_tok, const int32_t* token_of_row, int64_t rows, int64_t H, int64_t V, TileArgs a) {
+  a.panel = (uint16_t*)(ws + w.off_panel);
+  a.panel_ld = V;
+  a.out_rows = nullptr;
+  if (!token_of_row) {
+    a.col_tokens = nullptr;
+    launch_tiles<kModeRecompute>(st, weight, hid, n_tok, H, V, a);
+    return;
+  }
+  uint16_t* hc = (uint16_t*)(ws + w.off_hc);
+  hipLaunchKernelGGL(k_gather_rows, dim3((unsigned)rows), dim3(256), 0, st, (const u32x4_t*)hid, token_of_row, (u32x4_t*)hc,
+                     (int)(H / 8));
+  a.col_tokens = token_of_row;
+  launch_tiles<kModeRecompute>(st, weight, hc, rows, H, V, a);
 }
 
 // d_weight of dtype AA_F32 is accumulated in place.  A bf16 d_weight is written by the GEMM itself when there is one
@@ -236,31 +662,17 @@ static void finish_weight_grad(hipStream_t st, const WeightGrad& g, void* d_weig
                      (u32x4_t*)d_weight, n8);
 }
 
-// Row count of the d_hidden GEMM for `kept` rows with a gradient (its output is a scratch buffer with room for a whole
-// chunk, the extra rows are never read).  The library's kernels for a small output with a very long contraction
-// split the contraction over the compute units, and at H = 4096 (16 tiles of 256 across) they run 20 % slower when
-// the 256 x 256 output tiles do not come to a multiple of half the unit count (n = 11520: 720 tiles, 11.9 ms;
-// n = 12288: 768 tiles, 9.9 ms).  Where H allows such a multiple within 2048 rows the count is rounded up to it;
-// otherwise (H = 5376: 21 tiles across, no gain measured) to the tile size.  The d_weight GEMM, where the rows are
-// the contraction, always takes the count rounded up to 256.
-static int64_t d_hidden_gemm_rows(int64_t kept, int64_t chunk, int64_t H) {
-  static const int64_t half_units = [] {
-    int dev = 0, cus = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 2)
-      cus = 256;
-    return (int64_t)cus / 2;
-  }();
-  const int64_t tiles_across = (H + 255) / 256;
-  int64_t step = 256;
-  if (half_units % tiles_across == 0 && half_units / tiles_across <= 8) step = 256 * (half_units / tiles_across);
-  const int64_t n = round_up(kept, step);
-  return n < chunk ? n : chunk;
-}
-
-static bool shapes_ok(int64_t T, int64_t H, int64_t V) {
-  return T > 0 && H > 0 && V > 0 && (H % 8) == 0 && (V % 8) == 0 && T < (1 << 30) && V < (1 << 30) && H < (1 << 30) &&
-         (V / 64 + 1) * ((H > kChunkTokens ? H : kChunkTokens) / 64 + 1) < (1LL << 31);  // transpose grids
+static TileArgs stats_args(const Workspace& w, char* ws, const int64_t* labels, float inv_t) {
+  TileArgs a{};
+  a.pk = (float*)(ws + w.off_pk);
+  a.ps = (float*)(ws + w.off_ps);
+  a.pu = (float*)(ws + w.off_pu);
+  a.xy = (float*)(ws + w.off_xy);
+  a.labels = labels;
+  a.pitch_t = w.chunk;
+  a.c = kLog2e * inv_t;
+  a.inv_t = inv_t;
+  return a;
 }
 
 }  // namespace lmhead
@@ -274,6 +686,13 @@ extern "C" int64_t aa_lmhead_workspace_bytes(int64_t T, int64_t H, int64_t V) {
   return plan(T, H, V).bytes;
 }
 
+extern "C" int64_t aa_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
+  if (!shapes_ok(T, H, V)) return -1;
+  return plan(T, H, V).fwd_bytes;
+}
+
+extern "C" int64_t aa_lmhead_chunk_tokens(void) { return kChunkTokens; }
+
 extern "C" int aa_lmhead_fwd(const void* hidden, const void* weight, int64_t T, int64_t H, int64_t V,
                              const int64_t* labels, float inv_temperature, float* logp, float* entropy,
                              float* row_lse, float* row_ez, void* workspace, int64_t workspace_bytes, void* stream) {
@@ -281,16 +700,19 @@ extern "C" int aa_lmhead_fwd(const void* hidden, const void* weight, int64_t T, 
   if (!shapes_ok(T, H, V)) return AA_ERR_UNSUPPORTED;
   if ((((uintptr_t)hidden | (uintptr_t)weight | (uintptr_t)workspace) & 15) != 0) return AA_ERR_INVALID_ARGUMENT;
   const Workspace w = plan(T, H, V);
-  if (workspace_bytes < w.bytes) return AA_ERR_INVALID_ARGUMENT;
+  if (workspace_bytes < w.fwd_bytes) return AA_ERR_INVALID_ARGUMENT;
+  if (!prepare_kernels()) return AA_ERR_LAUNCH;
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
   auto at = [](float* p, int64_t t0) { return p ? p + t0 : nullptr; };
   for (int64_t t0 = 0; t0 < T; t0 += w.chunk) {
     const int64_t n_tok = (T - t0) < w.chunk ? (T - t0) : w.chunk;
-    if (!panel_logits(st, w, ws, (const uint16_t*)hidden + t0 * H, weight, n_tok, H, V)) return AA_ERR_LAUNCH;
-    const int rc = aa_logits_fwd(ws + w.off_ds, AA_BF16, n_tok, V, V, labels + t0, inv_temperature, logp + t0,
-                                 at(entropy, t0), at(row_lse, t0), at(row_ez, t0), nullptr, nullptr, stream);
-    if (rc != AA_OK) return rc;
+    const TileArgs a = stats_args(w, ws, labels + t0, inv_temperature);
+    hipLaunchKernelGGL(k_fill_f32, dim3((unsigned)((n_tok + 255) / 256)), dim3(256), 0, st, a.xy, n_tok, __builtin_nanf(""));
+    launch_tiles<kModeStats>(st, weight, (const uint16_t*)hidden + t0 * H, n_tok, H, V, a);
+    hipLaunchKernelGGL(k_combine, dim3((unsigned)((n_tok + 255) / 256)), dim3(256), 0, st, a.pk, a.ps, a.pu, a.xy,
+                       (int)w.blocks, a.pitch_t, (int)n_tok, a.c, logp + t0, at(entropy, t0), at(row_lse, t0),
+                       at(row_ez, t0));
   }
   return launch_status();
 }
@@ -309,6 +731,7 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
     return AA_ERR_INVALID_ARGUMENT;
   const Workspace w = plan(T, H, V);
   if (workspace_bytes < w.bytes) return AA_ERR_INVALID_ARGUMENT;
+  if (!prepare_kernels()) return AA_ERR_LAUNCH;
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
   launch_transpose(st, (const uint16_t*)weight, V, H, H, (uint16_t*)(ws + w.off_wt), V);
@@ -321,17 +744,17 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
     const int64_t n_tok = (T - t0) < w.chunk ? (T - t0) : w.chunk;
     const uint16_t* hid = (const uint16_t*)hidden + t0 * H;
     uint16_t* dh = (uint16_t*)d_hidden + t0 * H;
-    const float* ez = row_ez ? row_ez + t0 : nullptr;
-    const float* gh = g_entropy ? g_entropy + t0 : nullptr;
+    TileArgs a{};
+    a.labels = labels + t0;
+    a.c = kLog2e * inv_temperature;
+    a.inv_t = inv_temperature;
+    a.row_lse = row_lse + t0;
+    a.row_ez = row_ez ? row_ez + t0 : nullptr;
+    a.g_logp = g_logp + t0;
+    a.g_entropy = g_entropy ? g_entropy + t0 : nullptr;
     if (!kept_per_chunk) {
-      void* ds = ws + w.off_ds;  // [chunk, V]: logits of the chunk, then their gradient in place
-      if (!panel_logits(st, w, ws, hid, weight, n_tok, H, V)) return AA_ERR_LAUNCH;
-      const int rc = aa_logits_bwd(ds, AA_BF16, n_tok, V, V, labels + t0, inv_temperature, row_lse + t0, ez, g_logp + t0,
-                                   gh, n_tok, ds, stream);
-      if (rc != AA_OK) return rc;
-      if (!panel_gradients(st, w, ws, w.off_ds, w.off_dst, hid, nullptr, n_tok, round_up(n_tok, 8), n_tok, H, V, dh,
-                           dw.acc, dw.acc_f32, first))
-        return AA_ERR_LAUNCH;
+      recompute_panel(st, w, ws, weight, hid, n_tok, nullptr, n_tok, H, V, a);
+      panel_gradients(st, w, ws, hid, nullptr, n_tok, H, V, dh, dw.acc, dw.acc_f32, first);
       first = false;
       continue;
     }
@@ -344,15 +767,9 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
     }
     hipLaunchKernelGGL(k_compact_map, dim3(1), dim3(1024), 0, st, row_has_gradient + t0, (int)n_tok, (int)n_tok, (int)kept,
                        out_rows, act_rows);
-    if (!panel_logits(st, w, ws, hid, weight, n_tok, H, V)) return AA_ERR_LAUNCH;
-    const int rc = logits_bwd_rows(ws + w.off_ds, AA_BF16, n_tok, V, V, labels + t0, inv_temperature, row_lse + t0, ez,
-                                   g_logp + t0, gh, n_tok, ws + w.off_dst, out_rows, stream);
-    if (rc != AA_OK) return rc;
+    recompute_panel(st, w, ws, weight, hid, n_tok, act_rows, kept, H, V, a);
     uint16_t* dh_kept = (uint16_t*)(ws + w.off_dhc);
-    if (!panel_gradients(st, w, ws, w.off_dst, w.off_ds, hid, act_rows, kept, round_up(kept, 256),
-                         d_hidden_gemm_rows(kept, w.chunk, H), H, V, dh_kept, dw.acc,
-                         dw.acc_f32, first))
-      return AA_ERR_LAUNCH;
+    panel_gradients(st, w, ws, hid, act_rows, kept, H, V, dh_kept, dw.acc, dw.acc_f32, first);
     first = false;
     hipLaunchKernelGGL(k_scatter_rows, dim3((unsigned)n_tok), dim3(256), 0, st, (const u32x4_t*)dh_kept, out_rows,
                        (u32x4_t*)dh, (int)(H / 8));
@@ -362,19 +779,19 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
   return launch_status();
 }
 
-extern "C" int64_t aa_lmhead_chunk_tokens(void) { return kChunkTokens; }
-
 extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64_t T, int64_t H, int64_t V,
                                    const int64_t* labels, float inv_temperature, int64_t T_active,
                                    const float* prox_logp, const float* adv, const uint8_t* mask_eff,
                                    const float* behave_w, const aa_ppo_params* params, const int32_t* n_valid,
-                                   const float* grad_scale, const int64_t* kept_per_chunk, float* logp, float* entropy,
-                                   float* stat_loss, float* ratio, uint8_t* flags, void* d_hidden, void* d_weight,
-                                   int d_weight_dtype, int32_t* work, void* workspace, int64_t workspace_bytes,
-                                   void* stream) {
+                                   const float* grad_scale, const int64_t* kept_per_chunk, int backward_mode,
+                                   float* logp, float* entropy, float* stat_loss, float* ratio, uint8_t* flags,
+                                   void* d_hidden, void* d_weight, int d_weight_dtype, void* workspace,
+                                   int64_t workspace_bytes, void* stream) {
   if (!hidden || !weight || !labels || !d_hidden || !d_weight || !workspace) return AA_ERR_INVALID_ARGUMENT;
   if (!params || !n_valid || !logp) return AA_ERR_INVALID_ARGUMENT;
   if (T_active < 0 || T_active > T || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
+  if (backward_mode != AA_LMHEAD_RECOMPUTE && backward_mode != AA_LMHEAD_CARRY) return AA_ERR_INVALID_ARGUMENT;
+  if (params->loss_kind != AA_LOSS_PPO && params->loss_kind != AA_LOSS_NLL) return AA_ERR_INVALID_ARGUMENT;
   const bool nll = params->loss_kind == AA_LOSS_NLL;  // prox_logp and adv are not used by that loss
   if (T_active > 0 && (!mask_eff || !stat_loss || !ratio || !flags)) return AA_ERR_INVALID_ARGUMENT;
   if (T_active > 0 && !nll && (!prox_logp || !adv)) return AA_ERR_INVALID_ARGUMENT;
@@ -384,12 +801,18 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
     return AA_ERR_INVALID_ARGUMENT;
   const Workspace w = plan(T, H, V);
   if (workspace_bytes < w.bytes) return AA_ERR_INVALID_ARGUMENT;
+  if (!prepare_kernels()) return AA_ERR_LAUNCH;
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
+  const bool carry = backward_mode == AA_LMHEAD_CARRY;
   launch_transpose(st, (const uint16_t*)weight, V, H, H, (uint16_t*)(ws + w.off_wt), V);
   const WeightGrad dw = weight_grad(w, ws, d_weight, d_weight_dtype, T);
   int32_t* out_rows = (int32_t*)(ws + w.off_rows);
   int32_t* act_rows = out_rows + w.chunk;
+  float* g_tok = (float*)(ws + w.off_g);
+  float* lse_tok = (float*)(ws + w.off_lse);
+  RowCoef* rowc = (RowCoef*)(ws + w.off_rowc);
+  uint16_t* panel = (uint16_t*)(ws + w.off_panel);
   bool first = true;  // no GEMM has written d_weight yet
   int64_t chunk_index = 0;
   for (int64_t t0 = 0; t0 < T; t0 += w.chunk, ++chunk_index) {
@@ -399,44 +822,55 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
     const uint16_t* hid = (const uint16_t*)hidden + t0 * H;
     uint16_t* dh = (uint16_t*)d_hidden + t0 * H;
     auto at = [t0](auto* p) { return p ? p + t0 : nullptr; };
-    if (!panel_logits(st, w, ws, hid, weight, n_tok, H, V)) return AA_ERR_LAUNCH;
-    if (!kept_per_chunk) {
-      // log-prob, entropy, PPO loss and d(loss)/d(logits) in place: one streaming pass over the panel
-      void* ds = ws + w.off_ds;
-      const int rc = aa_logits_ppo_fused(ds, AA_BF16, n_tok, V, V, labels + t0, inv_temperature, act, at(prox_logp),
-                                         at(adv), at(mask_eff), at(behave_w), params, n_valid, grad_scale, logp + t0,
-                                         at(entropy), nullptr, nullptr, at(stat_loss), at(ratio), at(flags), ds, work,
-                                         stream);
-      if (rc != AA_OK) return rc;
-      if (!panel_gradients(st, w, ws, w.off_ds, w.off_dst, hid, nullptr, n_tok, round_up(n_tok, 8), n_tok, H, V, dh,
-                           dw.acc, dw.acc_f32, first))
-        return AA_ERR_LAUNCH;
-      first = false;
-      continue;
+    // which tokens get a panel row: those with a mask when the host gave their count, every token otherwise
+    int64_t rows = n_tok;
+    const int32_t* row_of_token = nullptr;
+    const int32_t* token_of_row = nullptr;
+    if (kept_per_chunk) {
+      rows = kept_per_chunk[chunk_index];
+      rows = rows < 0 ? 0 : (rows > act ? act : rows);
+      hipLaunchKernelGGL(k_compact_map, dim3(1), dim3(1024), 0, st, at(mask_eff), (int)act, (int)n_tok, (int)rows, out_rows,
+                         act_rows);
+      row_of_token = out_rows;
+      token_of_row = act_rows;
     }
-    // Tokens whose mask is zero have no gradient: the streaming pass writes the gradient rows of the other tokens,
-    // closed up, into the second panel buffer, and the backward GEMMs run on those rows only.
-    int64_t kept = kept_per_chunk[chunk_index];
-    kept = kept < 0 ? 0 : (kept > act ? act : kept);
-    hipLaunchKernelGGL(k_compact_map, dim3(1), dim3(1024), 0, st, at(mask_eff), (int)act, (int)n_tok, (int)kept, out_rows,
-                       act_rows);
-    const int rc = logits_ppo_fused_rows(ws + w.off_ds, AA_BF16, n_tok, V, V, labels + t0, inv_temperature, act,
-                                         at(prox_logp), at(adv), at(mask_eff), at(behave_w), params, n_valid, grad_scale,
-                                         logp + t0, at(entropy), nullptr, nullptr, at(stat_loss), at(ratio), at(flags),
-                                         ws + w.off_dst, out_rows, work, stream);
-    if (rc != AA_OK) return rc;
-    if (kept == 0) {
+    // forward tiles: block partials (and, in carry mode, the unnormalised probabilities of the panel rows)
+    TileArgs a = stats_args(w, ws, labels + t0, inv_temperature);
+    a.panel = panel;
+    a.panel_ld = V;
+    a.out_rows = row_of_token;
+    hipLaunchKernelGGL(k_fill_f32, dim3((unsigned)((n_tok + 255) / 256)), dim3(256), 0, st, a.xy, n_tok, __builtin_nanf(""));
+    if (carry && rows > 0)
+      launch_tiles<kModeStatsCarry>(st, weight, hid, n_tok, H, V, a);
+    else
+      launch_tiles<kModeStats>(st, weight, hid, n_tok, H, V, a);
+    // row statistics, per-token outputs, g
+    TokenLossArgs la{at(prox_logp), at(adv), at(mask_eff), at(behave_w), n_valid, grad_scale, logp + t0, at(entropy),
+                     at(stat_loss), at(ratio), at(flags), *params, act};
+    hipLaunchKernelGGL(k_token_loss, dim3((unsigned)((n_tok + 255) / 256)), dim3(256), 0, st, a.pk, a.ps, a.pu, a.xy,
+                       (int)w.blocks, a.pitch_t, (int)n_tok, (int)V, a.c, inv_temperature, labels + t0, la, row_of_token,
+                       g_tok, lse_tok, carry ? rowc : nullptr);
+    if (rows == 0) {
       launch_zero(st, dh, n_tok * H * 2);
       continue;
     }
-    uint16_t* dh_kept = (uint16_t*)(ws + w.off_dhc);
-    if (!panel_gradients(st, w, ws, w.off_dst, w.off_ds, hid, act_rows, kept, round_up(kept, 256),
-                         d_hidden_gemm_rows(kept, w.chunk, H), H, V, dh_kept, dw.acc,
-                         dw.acc_f32, first))
-      return AA_ERR_LAUNCH;
+    if (carry) {
+      hipLaunchKernelGGL(k_panel_scale, dim3((unsigned)rows), dim3(256), 0, st, panel, V, (int)V, rowc, token_of_row, a.pk,
+                         a.pitch_t);
+    } else {
+      a.row_lse = lse_tok;
+      a.g_logp = g_tok;
+      recompute_panel(st, w, ws, weight, hid, n_tok, token_of_row, rows, H, V, a);
+    }
+    if (!kept_per_chunk) {
+      panel_gradients(st, w, ws, hid, nullptr, n_tok, H, V, dh, dw.acc, dw.acc_f32, first);
+    } else {
+      uint16_t* dh_kept = (uint16_t*)(ws + w.off_dhc);
+      panel_gradients(st, w, ws, hid, act_rows, rows, H, V, dh_kept, dw.acc, dw.acc_f32, first);
+      hipLaunchKernelGGL(k_scatter_rows, dim3((unsigned)n_tok), dim3(256), 0, st, (const u32x4_t*)dh_kept, out_rows,
+                         (u32x4_t*)dh, (int)(H / 8));
+    }
     first = false;
-    hipLaunchKernelGGL(k_scatter_rows, dim3((unsigned)n_tok), dim3(256), 0, st, (const u32x4_t*)dh_kept, out_rows,
-                       (u32x4_t*)dh, (int)(H / 8));
   }
   if (first) launch_zero(st, dw.acc, V * H * (dw.acc_f32 ? 4 : 2));  // no token of the batch has a gradient
   finish_weight_grad(st, dw, d_weight, V, H);

@@ -667,8 +667,12 @@ def fused_logprobs_ppo_loss(
 # ----------------------------------------------------------------------------
 # fused lm_head: hidden @ weight.T -> logp / entropy without the [T, V] logits
 # ----------------------------------------------------------------------------
-def _lmhead_workspace(T: int, H: int, V: int, dev) -> torch.Tensor:
-    n = N.load().aa_lmhead_workspace_bytes(T, H, V)
+_LMHEAD_BACKWARD = {"recompute": 0, "carry": 1}  # aa_lmhead_backward_mode
+
+
+def _lmhead_workspace(T: int, H: int, V: int, dev, forward_only: bool = False) -> torch.Tensor:
+    lib = N.load()
+    n = lib.aa_lmhead_fwd_workspace_bytes(T, H, V) if forward_only else lib.aa_lmhead_workspace_bytes(T, H, V)
     if n < 0:
         raise N.NativeLibraryError(
             f"the lm_head path needs hidden size and vocabulary to be multiples of 8 (got H={H}, V={V})"
@@ -685,7 +689,7 @@ class _LmHeadLogprobsEntropy(torch.autograd.Function):
         dev = hidden.device
         f32 = dict(dtype=torch.float32, device=dev)
         logp, entropy, row_lse, row_ez = (torch.empty(T, **f32) for _ in range(4))
-        ws = _lmhead_workspace(T, H, V, dev)
+        ws = _lmhead_workspace(T, H, V, dev, forward_only=True)  # softmax partials only: nothing of size T x V
         with torch.cuda.device(dev):
             N.check(
                 lib.aa_lmhead_fwd(
@@ -734,14 +738,18 @@ def lm_head_logprobs_entropy(
     hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0,
     token_mask: torch.Tensor | None = None,
 ) -> tuple[torch.Tensor, torch.Tensor]:
-    """``gather_logprobs_entropy(hidden @ weight.T, labels, temperature)`` without materialising the ``[T, V]`` logits.
+    """``gather_logprobs_entropy(hidden @ weight.T, labels, temperature)`` without writing the ``[T, V]`` logits.
 
-    ``hidden`` is ``[T, H]`` and ``weight`` ``[V, H]`` (the lm_head), both bf16.  Tokens go through in chunks of at
-    most 16384: the chunk's logits are formed on the matrix cores (fp32 accumulation, rounded to bf16 as the model's
-    lm_head output is) and reduced to log-prob and entropy by the streaming kernel of ``gather_logprobs_entropy``.
-    Differentiable in ``hidden`` and ``weight`` (the backward forms each chunk's logits again, turns them in place
-    into their gradient and contracts that with the weight and the hidden states; fp32 accumulation, the weight
-    gradient is returned in the dtype of ``weight``).
+    ``hidden`` is ``[T, H]`` and ``weight`` ``[V, H]`` (the lm_head), both bf16.  The forward forms 256 x 256 tiles of
+    the logits in the accumulator registers of the library's bf16 MFMA tile GEMM (fp32 accumulation, not rounded to
+    bf16 in between) and reduces each tile to softmax partials per token in the GEMM's epilogue; its only scratch
+    memory is those partials (about ``24 * V / 256`` bytes per token of a 16384-token chunk, 0.3 GB at
+    ``V = 151936``).  Differentiable in ``hidden`` and ``weight``: the backward goes through the tokens in chunks of at
+    most 16384, forms the chunk's logits tiles again, writes their gradient as bf16 rows (of the tokens whose upstream
+    gradient is not zero) into a workspace panel ``[chunk, V]`` and contracts that panel with the weight and with the
+    hidden states on the same tile GEMM (fp32 accumulation, the weight gradient is returned in the dtype of
+    ``weight``).  The backward's workspace is the panel and its transposed copy (``4 * chunk * V`` bytes) plus a
+    transposed copy of the weight.
     The reference has no such op: it is the drop-in for its lm_head matmul followed by
     ``gather_logprobs_entropy`` (vocab_parallel.py:434-469).
 
@@ -767,11 +775,9 @@ def lm_head_logprobs_entropy(
         if n_kept == 0:
             zero = (hidden[:1].float().sum() + weight[:1].float().sum()) * 0.0
             return zero.expand(T), zero.expand(T)
-        pad = (n_kept + 255) // 256 * 256 - n_kept  # round sizes keep the GEMM library on its fast kernels
-        lp, ent = _LmHeadLogprobsEntropy.apply(
-            torch.nn.functional.pad(hidden.index_select(0, idx), (0, 0, 0, pad)), weight.contiguous(),
-            torch.nn.functional.pad(y.index_select(0, idx), (0, pad)), float(temperature))
-        full = lambda v: torch.zeros(T, dtype=torch.float32, device=dev).index_copy(0, idx, v[:n_kept])
+        lp, ent = _LmHeadLogprobsEntropy.apply(hidden.index_select(0, idx), weight.contiguous(), y.index_select(0, idx),
+                                               float(temperature))
+        full = lambda v: torch.zeros(T, dtype=torch.float32, device=dev).index_copy(0, idx, v)
         return full(lp), full(ent)
     return _LmHeadLogprobsEntropy.apply(hidden.contiguous(), weight.contiguous(), y, float(temperature))
 
@@ -779,7 +785,7 @@ def lm_head_logprobs_entropy(
 class _FusedLmHeadPpo(torch.autograd.Function):
     @staticmethod
     def forward(ctx, hidden, weight, labels, temperature, T_active, prox, adv, mask_eff, behave_w, params, n_valid,
-                grad_scale, kept_per_chunk):
+                grad_scale, kept_per_chunk, backward_mode):
         lib = N.load()
         kept = None if kept_per_chunk is None else (C.c_int64 * len(kept_per_chunk))(*kept_per_chunk)
         T, H = hidden.shape
@@ -801,8 +807,8 @@ class _FusedLmHeadPpo(torch.autograd.Function):
                 lib.aa_lmhead_ppo_fused(
                     _ptr(hidden), _ptr(weight), T, H, V, _ptr(labels), 1.0 / float(temperature), T_active, _ptr(prox),
                     _ptr(adv), _ptr(mask_eff), _ptr(behave_w), C.byref(params), _ptr(n_valid), _ptr(grad_scale), kept,
-                    _ptr(logp), _ptr(entropy), _ptr(stat_loss), _ptr(ratio), _ptr(flags), _ptr(d_hidden),
-                    _ptr(d_weight), _DTYPES[d_weight.dtype], _ptr(_work_words(dev)), _ptr(ws), ws.numel(), st,
+                    int(backward_mode), _ptr(logp), _ptr(entropy), _ptr(stat_loss), _ptr(ratio), _ptr(flags),
+                    _ptr(d_hidden), _ptr(d_weight), _DTYPES[d_weight.dtype], _ptr(ws), ws.numel(), st,
                 ),
                 "aa_lmhead_ppo_fused",
             )
@@ -822,7 +828,7 @@ class _FusedLmHeadPpo(torch.autograd.Function):
             for t in (d_hidden, d_weight):
                 N.check(lib.aa_scale_inplace(_ptr(t), _DTYPES[t.dtype], t.numel(), _ptr(g), _stream(dev)),
                         "aa_scale_inplace")
-        return (d_hidden, d_weight) + (None,) * 11
+        return (d_hidden, d_weight) + (None,) * 12
 
 
 def fused_lm_head_ppo_loss(
@@ -844,15 +850,25 @@ def fused_lm_head_ppo_loss(
     skip_masked_tokens: bool = True,
     forward_masked_tokens: bool = True,
     kept_per_chunk: list[int] | None = None,
+    backward: str = "carry",
 ) -> tuple[torch.Tensor, dict]:
     """lm_head + ``gather_logprobs_entropy`` + ``ppo_actor_loss_fn`` (+ backward) for one micro-batch.
 
     ``hidden`` is ``[T_pad, H]`` (the final hidden states of the batch-padded micro-batch), ``weight`` the ``[V, H]``
-    lm_head, both bf16; the other arguments are those of ``fused_logprobs_ppo_loss``.  Tokens are processed in chunks
-    of at most 16384: a chunk's logits are rounded to bf16 into a workspace, exactly as the reference's lm_head
-    output is, and turned in place into their gradient, so the full ``[T, V]`` logits never exist and nothing is
-    recomputed.  ``loss.backward()`` hands back ``d(hidden)`` and ``d(weight)`` written during the forward pass.
-    With ``importance_sampling_level="sequence"`` the call runs ``lm_head_logprobs_entropy`` and the unfused loss.
+    lm_head, both bf16; the other arguments are those of ``fused_logprobs_ppo_loss``.  The logits are formed as
+    256 x 256 tiles in the accumulator registers of the library's bf16 MFMA tile GEMM and reduced to softmax partials
+    in its epilogue; they are never written to memory.  Tokens are processed in chunks of at most 16384;
+    ``loss.backward()`` hands back ``d(hidden)`` and ``d(weight)`` written during the forward pass (the loss is
+    known by then).  With ``importance_sampling_level="sequence"`` the call runs ``lm_head_logprobs_entropy`` and the
+    unfused loss.
+
+    ``backward`` chooses how the bf16 ``d(loss)/d(logits)`` rows of a chunk (``[tokens with gradient, V]`` in the
+    workspace, which the two gradient GEMMs contract) are obtained.  ``"recompute"``: the logits tiles of those tokens
+    are formed a second time once the loss is known, as ``lm_head_logprobs_entropy``'s backward does (a third more
+    matrix work).  ``"carry"`` (default, the faster of the two by measurement): the forward tiles also write the
+    unnormalised probabilities ``2^(x c - k_block)`` that their softmax partials are made of into those rows, and a
+    streaming pass scales them into the gradient afterwards; no second GEMM.  Both write the same bytes into the
+    same workspace (``4 * chunk * V`` bytes with the transposed copy; carry writes the rows twice).
 
     ``skip_masked_tokens``: a token whose (effective) loss mask is zero has a zero gradient row, so the two gradient
     GEMMs run on the other tokens only; the results are those of the dense computation.  The per-chunk token counts
@@ -872,6 +888,8 @@ def fused_lm_head_ppo_loss(
         raise ValueError(
             f"Invalid importance_sampling_level: {importance_sampling_level}. Must be 'token' or 'sequence'."
         )
+    if backward not in _LMHEAD_BACKWARD:
+        raise ValueError(f"backward must be one of {sorted(_LMHEAD_BACKWARD)}, got {backward!r}")
     _require_gpu(hidden, "hidden")
     if hidden.ndim != 2 or weight.ndim != 2 or hidden.shape[1] != weight.shape[1]:
         raise ValueError(f"expected hidden [T, H] and weight [V, H], got {tuple(hidden.shape)} and {tuple(weight.shape)}")
@@ -934,18 +952,13 @@ def fused_lm_head_ppo_loss(
             stat = dict(loss=z, importance_weight=z.clone(), approx_kl=z.clone(), clip_mask=zb, dual_clip_mask=zb.clone(),
                         logprobs=z.clone(), entropy=z.clone())
         else:
-            # the closed-up batch is padded to a multiple of 256 rows (batch padding: no outputs, no gradient), which
-            # keeps the GEMM library on its fast kernels
             ones = torch.ones(n_kept, dtype=torch.uint8, device=dev)
             chunk = int(N.load().aa_lmhead_chunk_tokens())
-            n_rows = (n_kept + 255) // 256 * 256
-            pad = n_rows - n_kept
-            kept = [max(0, min(chunk, n_kept - c)) for c in range(0, n_rows, chunk)]
+            kept = [max(0, min(chunk, n_kept - c)) for c in range(0, n_kept, chunk)]
             loss, logp, entropy, stat_loss, ratio, flags = _FusedLmHeadPpo.apply(
-                torch.nn.functional.pad(hidden.index_select(0, idx), (0, 0, 0, pad)), weight.contiguous(),
-                torch.nn.functional.pad(y.index_select(0, idx), (0, pad)), float(temperature), n_kept,
+                hidden.index_select(0, idx), weight.contiguous(), y.index_select(0, idx), float(temperature), n_kept,
                 prox.index_select(0, idx), adv.index_select(0, idx), ones,
-                None if w is None else w.index_select(0, idx), params, n_valid, scale_t, kept,
+                None if w is None else w.index_select(0, idx), params, n_valid, scale_t, kept, _LMHEAD_BACKWARD[backward],
             )
             logp, entropy = logp[:n_kept], entropy[:n_kept]
             stat = dict(
@@ -971,7 +984,7 @@ def fused_lm_head_ppo_loss(
         kept = _HostCounts(on.view(n_chunks, chunk).sum(1)).tolist()
     loss, logp, entropy, stat_loss, ratio, flags = _FusedLmHeadPpo.apply(
         hidden.contiguous(), weight.contiguous(), y, float(temperature), T_active, prox, adv, mask_eff, w, params,
-        n_valid, scale_t, kept,
+        n_valid, scale_t, kept, _LMHEAD_BACKWARD[backward],
     )
     logp_a = logp[:T_active]
     stat = dict(

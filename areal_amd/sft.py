@@ -196,7 +196,7 @@ def fused_lm_head_sft_loss(hidden: torch.Tensor, weight: torch.Tensor, labels: t
             kept = _HostCounts(on.view(n_chunks, chunk).sum(1)).tolist()
     loss, logp, entropy, stat_loss, _ratio, _flags = _FusedLmHeadPpo.apply(
         hidden.contiguous(), weight.contiguous(), y, float(temperature), T_active, None, None, m8, None, _nll_params(),
-        n_valid, scale_t, kept,
+        n_valid, scale_t, kept, 1,  # aa_lmhead_backward_mode: carry
     )
     logp_a = logp[:T_active]
     _, _, _, seq_logp, seq_count, seq_ppl = _launch(logp_a, m8, cu, n_seqs, n_valid, None, False, False)

@@ -6,11 +6,6 @@
  * the HIP stream it is given (hipStream_t passed as void*; NULL = the default
  * stream), allocates nothing, and never synchronises the device.  The return
  * value is an aa_status; a non-zero value means nothing was enqueued.
- * One exception, for the aa_lmhead_* entry points only: the first time they
- * meet a GEMM shape they time a few candidate algorithms of the GEMM library
- * on the given stream (the host waits for those runs; the GEMM library keeps a
- * handle and its kernels per device).  AREAL_AMD_GEMM_TUNE=0 in the environment
- * turns the timing off; a stream that is being captured is never timed.
  *
  * Layout conventions (the reference's "packed 1-D" layout):
  *   logits      [T, V]  row-major, element (t, j) at logits[t * row_stride + j]
@@ -585,23 +580,31 @@ int aa_masked_moments(const float* const* values, int n_tensors,
 /* logits = hidden @ weight.T followed by the logits path above)           */
 /* ------------------------------------------------------------------ */
 
-/* Bytes of workspace aa_lmhead_fwd / aa_lmhead_bwd / aa_lmhead_ppo_fused need
- * for these sizes: about 4 * min(T, 16384) * V + 2 * H * V bytes (one chunk of
- * bf16 logits and its transposed copy, a transposed copy of the weight) plus
- * 128 MiB for the GEMM library, plus 4 * H * V (an fp32 accumulator for a bf16
- * d_weight) when T > 16384. */
+/* Bytes of workspace aa_lmhead_bwd / aa_lmhead_ppo_fused need for these sizes:
+ * about 4 * min(T, 16384) * V bytes (the bf16 d(logits) rows of one token chunk
+ * and their transposed copy), 2 * H * V (a transposed copy of the weight),
+ * 24 * (V / 256) * min(T, 16384) (softmax partials per 128 vocabulary rows and
+ * token), plus 4 * H * V (an fp32 accumulator for a bf16 d_weight) when
+ * T > 16384.  Returns -1 for sizes the path does not take. */
 int64_t aa_lmhead_workspace_bytes(int64_t T, int64_t H, int64_t V);
+
+/* Bytes of workspace aa_lmhead_fwd alone needs: the softmax partials only,
+ * about 24 * (V / 256) * min(T, 16384) bytes (0.3 GB at V = 151936). */
+int64_t aa_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);
 
 /* Tokens per chunk of the lm_head entry points (16384). */
 int64_t aa_lmhead_chunk_tokens(void);
 
 /*
- * logp / entropy of softmax(hidden @ weight.T / temperature), holding at most
- * one chunk of 16384 tokens of logits (bf16, as the reference's lm_head output
- * is) in the workspace: a GEMM per chunk, then the kernel of aa_logits_fwd.
+ * logp / entropy of softmax(hidden @ weight.T / temperature) without writing
+ * the logits anywhere: 256 x 256 tiles of them are formed in the accumulator
+ * registers of this library's bf16 MFMA tile GEMM (fp32 accumulation, no
+ * rounding to bf16 in between), each tile is reduced to softmax partials per
+ * token in the GEMM's epilogue, and a small kernel merges the partials.
  * hidden [T, H] bf16 row-major, weight [V, H] bf16 row-major; H and V
- * multiples of 8.  entropy, row_lse, row_ez may be NULL; row_lse / row_ez as
- * in aa_logits_fwd (needed by aa_lmhead_bwd).
+ * multiples of 8 (below 2^22).  entropy, row_lse, row_ez may be NULL; row_lse /
+ * row_ez as in aa_logits_fwd (needed by aa_lmhead_bwd).
+ * workspace: aa_lmhead_fwd_workspace_bytes(T, H, V) bytes.
  */
 int aa_lmhead_fwd(const void* hidden, const void* weight, int64_t T, int64_t H,
                   int64_t V, const int64_t* labels, float inv_temperature,
@@ -613,13 +616,16 @@ int aa_lmhead_fwd(const void* hidden, const void* weight, int64_t T, int64_t H,
  * (overwritten), given g_logp and optional g_entropy.  d_weight_dtype is
  * AA_F32 or AA_BF16; either way the sum over tokens is accumulated in fp32
  * (bf16: rounded once at the end).
- * Per chunk: the logits GEMM again, the kernel of aa_logits_bwd in place, and
- * the two gradient GEMMs (6 T V H flops for the 4 T V H of the backward).
+ * Per chunk of 16384 tokens: the logits tiles are formed again and turned into
+ * bf16 d(logits) rows in the GEMM's epilogue (a panel [rows, V] in the
+ * workspace), which two more tile GEMMs contract with the weight and with the
+ * hidden states (6 T V H flops for the 4 T V H of the backward).
  * row_has_gradient [T] (device, one byte per token) with kept_per_chunk (HOST,
  * its non-zero count per chunk of aa_lmhead_chunk_tokens() tokens), both or
  * neither: rows whose byte is zero must have g_logp == 0 and g_entropy == 0;
- * they are left out of the gradient GEMMs (see aa_lmhead_ppo_fused), and a
- * chunk without any such row skips its logits GEMM as well.
+ * they are left out of all three GEMMs, and a chunk without any other row is
+ * skipped altogether.
+ * workspace: aa_lmhead_workspace_bytes(T, H, V) bytes.
  */
 int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, int64_t H,
                   int64_t V, const int64_t* labels, float inv_temperature,
@@ -630,20 +636,34 @@ int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, int64_t H,
                   void* d_weight, int d_weight_dtype, void* workspace,
                   int64_t workspace_bytes, void* stream);
 
+/* How aa_lmhead_ppo_fused fills the d(logits) rows that its backward GEMMs
+ * contract. */
+typedef enum {
+  /* the logits tiles of the tokens with gradient are formed a second time,
+   * once the loss is known (2 T_grad V H extra flops; the forward half writes
+   * nothing of size T x V) */
+  AA_LMHEAD_RECOMPUTE = 0,
+  /* the forward tiles also write 2^(x c - k_block), the unnormalised
+   * probabilities their statistics are made of, as bf16 into the rows of the
+   * tokens with gradient; a streaming pass scales them to d(logits) once the
+   * loss is known (no second GEMM; the same rows are written twice) */
+  AA_LMHEAD_CARRY = 1
+} aa_lmhead_backward_mode;
+
 /*
  * Whole training step of the lm_head + PPO actor loss for one micro-batch,
  * token-level importance sampling: what the reference runs as lm_head matmul
- * (bf16 logits) -> gather_logprobs_entropy (vocab_parallel.py:434-469) ->
+ * -> gather_logprobs_entropy (vocab_parallel.py:434-469) ->
  * ppo_actor_loss_fn (functional.py:429-559) -> autograd back to the hidden
  * states and the lm_head weight.  Tokens are processed in chunks of at most
- * 16384: the chunk's logits are formed on the matrix cores and rounded to
- * bf16 into the workspace (as the reference's lm_head output is), one
- * streaming pass turns them in place into d(loss)/d(logits) while emitting
- * the per-token outputs (the kernel of aa_logits_ppo_fused), and two GEMMs
- * accumulate the gradients.  No recompute: 6 T V H flops in all, and never
- * more than one chunk of logits in memory.
+ * 16384.  Per chunk: the forward tiles of aa_lmhead_fwd; one kernel that
+ * merges the softmax partials into log-prob and entropy and evaluates the
+ * per-token loss and its derivative; the bf16 d(logits) rows of the tokens
+ * with gradient (backward_mode says how they are obtained); and the two tile
+ * GEMMs that contract those rows with the weight and the hidden states.  The
+ * logits themselves are never written to memory.
  *
- * Per-token arguments, params, n_valid, grad_scale, work: as in
+ * Per-token arguments, params, n_valid, grad_scale: as in
  * aa_logits_ppo_fused.  d_hidden [T, H] bf16 and d_weight [V, H] (AA_F32 or
  * AA_BF16, fp32 accumulation either way, as in aa_lmhead_bwd) are
  * overwritten.  workspace: aa_lmhead_workspace_bytes(T, H, V) bytes.
@@ -652,10 +672,10 @@ int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, int64_t H,
  * a zero gradient row, so it adds nothing to d_weight and its d_hidden row is
  * zero.  Given, for every chunk of aa_lmhead_chunk_tokens() tokens, the number
  * of non-zero mask_eff bytes among the chunk's first min(T_active - t0, chunk)
- * tokens, the two gradient GEMMs of the chunk run on those tokens only (the
- * reference's autograd multiplies the zero rows through).  The counts size the
- * GEMMs, which is why they come from the host; tokens beyond a count that is
- * too small are treated as masked.  NULL: every row goes through the GEMMs.
+ * tokens, only those tokens get a d(logits) row and go through the backward
+ * GEMMs (the reference's autograd multiplies the zero rows through).  The
+ * counts size the GEMMs, which is why they come from the host; tokens beyond a
+ * count that is too small are treated as masked.  NULL: every token has a row.
  */
 int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64_t T,
                         int64_t H, int64_t V, const int64_t* labels,
@@ -664,10 +684,10 @@ int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64_t T,
                         const uint8_t* mask_eff, const float* behave_w,
                         const aa_ppo_params* params, const int32_t* n_valid,
                         const float* grad_scale, const int64_t* kept_per_chunk,
-                        float* logp, float* entropy,
+                        int backward_mode, float* logp, float* entropy,
                         float* stat_loss, float* ratio, uint8_t* flags,
                         void* d_hidden, void* d_weight, int d_weight_dtype,
-                        int32_t* work, void* workspace, int64_t workspace_bytes,
+                        void* workspace, int64_t workspace_bytes,
                         void* stream);
 
 /* ------------------------------------------------------------------ */

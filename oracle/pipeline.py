@@ -15,11 +15,15 @@ from .logprobs import logprobs_entropy
 from .ppo import ppo_actor_loss
 
 
-def lmhead_logits(hidden: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-    """Logits as the reference's bf16 lm_head hands them to ``gather_logprobs_entropy``: ``hidden @ weight.T`` with
-    fp32 accumulation, rounded to bf16.  Differentiable (the rounding passes gradients through, as autograd's
-    ``.to(torch.bfloat16)`` does)."""
-    return (hidden.float() @ weight.float().t()).to(torch.bfloat16)
+def lmhead_logits(hidden: torch.Tensor, weight: torch.Tensor, round_to_bf16: bool = False) -> torch.Tensor:
+    """``hidden @ weight.T`` in fp32: the logits of the fp32 reference that the lm_head path is held to.
+
+    With ``round_to_bf16`` the product is rounded to bf16, as the reference's bf16 lm_head hands it to
+    ``gather_logprobs_entropy`` (differentiable: the rounding passes gradients through, as autograd's
+    ``.to(torch.bfloat16)`` does).  That rounding moves a logit by up to 2^-9 of its magnitude, and a token's
+    log-prob with it, so the bf16 pipeline itself sits that far from the fp32 reference."""
+    logits = hidden.float() @ weight.float().t()
+    return logits.to(torch.bfloat16) if round_to_bf16 else logits
 
 
 def logits_ppo_step(

@@ -7,11 +7,6 @@ from pathlib import Path
 import pytest
 import torch
 
-# The GEMM front end of the lm_head path picks, by timing, among library kernels that may sum in different orders;
-# the tests pin it to the library's first choice so that every run computes the same bits (one test turns the timing
-# on in a process of its own).
-os.environ.setdefault("AREAL_AMD_GEMM_TUNE", "0")
-
 ROOT = Path(__file__).resolve().parents[1]
 if str(ROOT) not in sys.path:
     sys.path.insert(0, str(ROOT))

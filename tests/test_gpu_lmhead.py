@@ -1,6 +1,7 @@
-"""GPU parity of the lm_head path.  The reference has no such path, so the oracle is its equivalent: bf16 logits
-= hidden @ weight.T (fp32 accumulation, rounded as the model's lm_head output is), then the log-prob / entropy
-oracle, with autograd for the gradients."""
+"""GPU parity of the lm_head path.  The reference has no such path, so the oracle is its equivalent in fp32:
+logits = hidden @ weight.T, then the log-prob / entropy oracle, with autograd for the gradients.  Stated tolerance:
+log-probs within 2e-3 of that fp32 reference, for every token.  The reference's own pipeline rounds the lm_head output
+to bf16 first; one test ties the two together."""
 import math
 
 import pytest
@@ -8,7 +9,7 @@ import torch
 
 import areal_amd
 import oracle
-from helpers import assert_close_up_to_logit_rounding, cosine
+from helpers import assert_same_magnitude, assert_within, assert_within_one_bf16_logit_step, cosine
 
 pytestmark = pytest.mark.gpu
 
@@ -37,11 +38,12 @@ def test_forward_matches_oracle(device, T, H, V, temperature):
     logits = oracle.lmhead_logits(hidden, weight)
     r_lp, r_ent = oracle.logprobs_entropy_f64(logits, labels, temperature)
     assert lp.dtype == torch.float32 and lp.shape == (T,)
-    # stated tolerance; a logit whose fp32 sum lies next to a bf16 rounding boundary may round the other way than the
-    # oracle's (different summation order), which moves a row by up to one bf16 step of that logit, hence the medians
-    assert_close_up_to_logit_rounding(lp, r_lp, 2e-3, "log-prob")
-    assert_close_up_to_logit_rounding(ent, r_ent, 2e-3, "entropy")
-    assert float((lp.cpu().double() - r_lp).abs().median()) < 2e-5
+    assert_within(lp, r_lp, 2e-3, "log-prob")  # stated tolerance, every token
+    assert_within(ent, r_ent, 2e-3, "entropy")
+    assert float((lp.cpu().double() - r_lp).abs().max()) < 1e-4  # what the kernel actually achieves
+    # the reference's pipeline hands bf16 logits to gather_logprobs_entropy: no token further from it than that rounding
+    b_lp, b_ent = oracle.logprobs_entropy_f64(oracle.lmhead_logits(hidden, weight, round_to_bf16=True), labels, temperature)
+    assert_within_one_bf16_logit_step(lp, b_lp, float(logits.abs().max()) / temperature, "log-prob vs bf16 pipeline")
     # deterministic
     lp2, ent2 = areal_amd.lm_head_logprobs_entropy(hidden.to(device), weight.to(device), labels.to(device), temperature)
     assert torch.equal(lp, lp2) and torch.equal(ent, ent2)
@@ -86,8 +88,8 @@ def test_backward_matches_autograd_of_oracle(device, T, H, V, temperature, with_
     assert h_d.grad.dtype == torch.bfloat16 and w_d.grad.dtype == torch.bfloat16
     assert cosine(h_d.grad.cpu(), h_o.grad) > 0.9999
     assert cosine(w_d.grad.cpu(), w_o.grad) > 0.9999
-    assert float((h_d.grad.cpu().float() - h_o.grad).abs().max()) < 0.02 * float(h_o.grad.abs().max()) + 1e-6
-    assert float((w_d.grad.cpu().float() - w_o.grad).abs().max()) < 0.02 * float(w_o.grad.abs().max()) + 1e-6
+    assert_same_magnitude(h_d.grad, h_o.grad, what="d(hidden)")
+    assert_same_magnitude(w_d.grad, w_o.grad, what="d(W)")
 
 
 def test_lm_head_into_ppo_loss_end_to_end(device):
@@ -111,8 +113,10 @@ def test_lm_head_into_ppo_loss_end_to_end(device):
     o_lp, _ = oracle.logprobs_entropy(oracle.lmhead_logits(h_o, w_o), labels)
     o_loss, _ = oracle.ppo_actor_loss(o_lp, prox, old, adv, 0.2, mask, 0.28, 3.0)
     o_loss.backward()
-    assert float(loss.detach()) == pytest.approx(float(o_loss.detach()), rel=1e-3, abs=3e-4)  # abs: one logit step
+    assert float(loss.detach()) == pytest.approx(float(o_loss.detach()), rel=1e-3)
     assert cosine(h_d.grad.cpu(), h_o.grad) > 0.9999 and cosine(w_d.grad.cpu(), w_o.grad) > 0.9999
+    assert_same_magnitude(h_d.grad, h_o.grad, what="d(hidden)")
+    assert_same_magnitude(w_d.grad, w_o.grad, what="d(W)")
 
 
 # ---------------------------------------------------------------------------------------------------------------
@@ -161,12 +165,14 @@ def test_full_size_configuration(device, name):
     lp, ent, dh_only, dw_only = run(g_only)
     assert bool((lp <= 1e-6).all()) and bool((ent >= -1e-4).all()) and bool((ent <= math.log(V) + 1e-4).all())
     o_lp, o_ent, o_dh, o_dw = _oracle_slice(case, idx, g_slice)
-    assert_close_up_to_logit_rounding(lp[idx], o_lp, 2e-3, "log-prob")  # stated tolerance
-    assert_close_up_to_logit_rounding(ent[idx], o_ent, 2e-3, "entropy")
+    assert_within(lp[idx], o_lp, 2e-3, "log-prob")  # stated tolerance
+    assert_within(ent[idx], o_ent, 2e-3, "entropy")
     assert cosine(dh_only[idx].cpu().float(), o_dh) > 0.9999
+    assert_same_magnitude(dh_only[idx], o_dh, what="d(hidden)")
     assert float(dh_only.float().abs().sum()) == pytest.approx(float(dh_only[idx].float().abs().sum()), rel=1e-6)
     # the full-size weight gradient with only the slice's tokens switched on is the oracle's slice gradient
     assert _cos_dev(dw_only, o_dw, device) > 0.9999
+    assert abs(float(dw_only.float().norm()) / float(o_dw.norm()) - 1.0) < 1e-2
     del o_dw
     # determinism and linearity of d(W), d(hidden) in the upstream gradient
     lp2, ent2, dh_rest, dw_rest = run(g_rest)
@@ -333,36 +339,30 @@ def test_row_counts_that_disagree_with_the_mask_stay_in_bounds(device):
     assert bool(torch.isfinite(dh_ok).all()) and float(dh_ok[~has].abs().sum()) == 0.0
 
 
-def test_gemm_candidate_timing_in_its_own_process(device):
-    """The test session pins the GEMM front end to the library's first choice; here a fresh process runs one lm_head
-    step with the timing of candidates switched on (the default outside the tests) and checks it against autograd of
-    plain torch matmuls."""
-    import os
-    import subprocess
-    import sys
-    import textwrap
+def test_forward_needs_no_panel(device):
+    """The forward writes nothing of size T x V: its workspace is the softmax partials only, and it runs with exactly
+    that much."""
+    import ctypes as C
 
-    code = textwrap.dedent("""
-        import torch, areal_amd
-        torch.manual_seed(0)
-        dev = torch.device("cuda:0")
-        T, H, V = 1024, 256, 4096
-        h = torch.randn(T, H, device=dev).bfloat16().requires_grad_(True)
-        w = (0.2 * torch.randn(V, H, device=dev)).bfloat16().requires_grad_(True)
-        y = torch.randint(0, V, (T,), device=dev)
-        g = torch.randn(T, device=dev)
-        lp, ent = areal_amd.lm_head_logprobs_entropy(h, w, y)
-        (lp * g).sum().backward()
-        h2, w2 = h.detach().clone().requires_grad_(True), w.detach().clone().requires_grad_(True)
-        lp2 = areal_amd.gather_logprobs(h2 @ w2.t(), y)
-        (lp2 * g).sum().backward()
-        cos = lambda a, b: float(torch.nn.functional.cosine_similarity(a.double().reshape(-1), b.double().reshape(-1), dim=0))
-        assert float((lp - lp2).abs().median()) < 1e-4 and float((lp - lp2).abs().max()) < 0.06
-        assert cos(h.grad, h2.grad) > 0.9999 and cos(w.grad, w2.grad) > 0.9999
-        print("tuned ok")
-    """)
-    env = dict(os.environ, AREAL_AMD_GEMM_TUNE="1", AREAL_AMD_GEMM_TUNE_LOG="1")
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    out = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True, text=True, timeout=300)
-    assert out.returncode == 0 and "tuned ok" in out.stdout, out.stderr[-2000:]
-    assert "candidate 1" in out.stderr            # more than one kernel was timed
+    from areal_amd import _native as N
+    from areal_amd import functional as F
+
+    lib = N.load()
+    T, H, V = 16384, 4096, 151936
+    assert lib.aa_lmhead_fwd_workspace_bytes(T, H, V) < 0.05 * (2 * T * V)          # bf16 logits would be 2 T V bytes
+    assert lib.aa_lmhead_fwd_workspace_bytes(T, H, V) < lib.aa_lmhead_workspace_bytes(T, H, V) / 20
+    T, H, V = 600, 128, 1088
+    hidden, weight, labels = _case(T, H, V, seed=3, w_std=0.3)
+    hd, wd, ld = hidden.to(device), weight.to(device), labels.to(device)
+    n = lib.aa_lmhead_fwd_workspace_bytes(T, H, V)
+    ws = torch.empty(n, dtype=torch.uint8, device=device)
+    f32 = dict(dtype=torch.float32, device=device)
+    logp, ent = torch.empty(T, **f32), torch.empty(T, **f32)
+    st = C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    N.check(lib.aa_lmhead_fwd(F._ptr(hd), F._ptr(wd), T, H, V, F._ptr(ld), 1.0, F._ptr(logp), F._ptr(ent), None, None,
+                              F._ptr(ws), n, st), "aa_lmhead_fwd")
+    r_lp, r_ent = oracle.logprobs_entropy_f64(oracle.lmhead_logits(hidden, weight), labels, 1.0)
+    assert_within(logp, r_lp, 2e-3, "log-prob")
+    assert_within(ent, r_ent, 2e-3, "entropy")
+    assert lib.aa_lmhead_fwd(F._ptr(hd), F._ptr(wd), T, H, V, F._ptr(ld), 1.0, F._ptr(logp), F._ptr(ent), None, None,
+                             F._ptr(ws), n - 1, st) == 1                                # AA_ERR_INVALID_ARGUMENT

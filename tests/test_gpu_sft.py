@@ -6,7 +6,7 @@ import torch
 import areal_amd
 import oracle
 from areal_amd import engine_glue as G
-from helpers import assert_close_up_to_logit_rounding, cosine
+from helpers import assert_same_magnitude, assert_within, cosine
 from oracle.sft import packed_sft_loss
 
 pytestmark = pytest.mark.gpu
@@ -117,10 +117,12 @@ def test_fused_lm_head_sft_matches_oracle(device, skip):
                                                   skip_masked_tokens=skip)
     loss.backward()
     assert float(loss.detach()) == pytest.approx(float(w_loss.detach()), rel=1e-3)
-    assert_close_up_to_logit_rounding(stat["logprobs"].cpu(), w_logp.detach(), 2e-3)
+    assert_within(stat["logprobs"].cpu(), w_logp.detach(), 2e-3, "log-prob")
     _check_stat(stat, w_stat, len(lens))
     assert cosine(hd.grad.float().cpu(), h.grad.float()) > 0.9999
     assert cosine(wd.grad.float().cpu(), w.grad.float()) > 0.9999
+    assert_same_magnitude(hd.grad.float(), h.grad.float(), what="d(hidden)")
+    assert_same_magnitude(wd.grad.float(), w.grad.float(), what="d(W)")
     assert not hd.grad[~mask.to(device)].any()
     with torch.no_grad():
         loss_f, _ = areal_amd.fused_lm_head_sft_loss(hidden.to(device), weight.to(device), labels.to(device),
