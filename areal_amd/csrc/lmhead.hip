@@ -10,7 +10,8 @@
 // log-prob and entropy.  Nothing of size T x V is written.
 //
 // Backward needs d(logits) twice (for d_hidden and for d_weight), so a bf16 panel [tokens with gradient, V] of it is
-// written once per token chunk and contracted by two plain tile GEMMs.  Two ways to fill the panel:
+// written once per token chunk and contracted by two plain tile GEMMs (which read the panel, the weight and the
+// hidden states as they lie: no transposed copies).  Two ways to fill the panel:
 //   recompute   the logits tiles are formed again and turned into d(logits) in registers (2 T_grad V H extra flops);
 //               what aa_lmhead_bwd does, where the upstream gradients only exist after the forward has returned.
 //   carry       (training step only) the forward tiles also write 2^(x c - k_block), the unnormalised probabilities
@@ -27,10 +28,12 @@ namespace lmhead {
 
 using namespace gemm;
 
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
 constexpr int kChunkTokens = 16384;        // token chunk of the panel
 constexpr int kPanelPitch = BM + 8;        // pitch (elements) of the tile staged in LDS as [token][vocab]
 constexpr int kStageBytes = 256 * kPanelPitch * 2;  // 135168 B, inside the 160 KiB the main loop uses
-static_assert(kStageBytes <= wide::kLdsBytes, "the staged tile must fit the main loop's LDS");
+static_assert(kStageBytes <= kLdsBytes, "the staged tile must fit the main loop's LDS");
 
 __host__ __device__ __forceinline__ int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
@@ -58,91 +61,94 @@ struct TileArgs {
   float inv_t;
 };
 
+// Statistics (and, with CARRY, the staged unnormalised probabilities) of one wave's 128 x 128 block.  RAGGED: the
+// block may reach past the vocabulary (last tile row only), rows at or past V are left out.
+template <bool CARRY, bool RAGGED>
+__device__ __forceinline__ void block_stats(const Acc& acc, const TileArgs& a, int tm, int wm, int wn, int n0, int N,
+                                            int V, int mbase, int lane, uint16_t* Z) {
+  constexpr int PZ = kPanelPitch;
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) {
+    const int nloc = wn * 128 + acc_col(nt, lane);
+    const int n = n0 + nloc;
+    float mx = -FLT_MAX;
+    if constexpr (!RAGGED) {
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) mx = fmaxf(fmaxf(mx, acc.v[mt][nt][i]), acc.v[mt][nt][i + 1]);  // one v_max3 per pair
+    } else {
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mx = (mbase + acc_row(mt, i, lane) < V) ? fmaxf(mx, acc.v[mt][nt][i]) : mx;
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));  // both halves of the wave hold the same token
+    const float k = fmaxf(mx * a.c, kNegBig);   // kNegBig: no valid row in this block
+    float s = 0.f, u = 0.f;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        float e[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float t = fmaf(acc.v[mt][nt][g4 * 4 + q], a.c, -k);
+          e[q] = fast_exp2(t);
+          if constexpr (RAGGED) e[q] = (mbase + acc_row(mt, g4 * 4 + q, lane) < V) ? e[q] : 0.f;
+          s += e[q];
+          u = fmaf(t, e[q], u);
+        }
+        if constexpr (CARRY) {
+          uint2 pk;
+          pk.x = Elem<AA_BF16>::pack(e[0], e[1]);
+          pk.y = Elem<AA_BF16>::pack(e[2], e[3]);
+          *(uint2*)(Z + nloc * PZ + wm * 128 + mt * 32 + 8 * g4 + 4 * (lane >> 5)) = pk;
+        }
+      }
+    s += __shfl_xor(s, 32, kWave);
+    u += __shfl_xor(u, 32, kWave);
+    if (lane < 32 && n < N) {
+      const int64_t at = (int64_t)(tm * 2 + wm) * a.pitch_t + n;
+      a.pk[at] = k;
+      a.ps[at] = s;
+      a.pu[at] = u;
+    }
+  }
+}
+
 // One 256 x 256 tile: rows m = vocabulary (operand A = weight), columns n = tokens (operand B = hidden states), so
 // that everything a token needs from the tile sits in one lane and its partner lane ^ 32.
 template <int MODE>
-__global__ __launch_bounds__(wide::kThreads) void k_lmhead_tiles(Operand W, Operand Hd, int K, int tiles_m, int tiles_n,
+__global__ __launch_bounds__(kThreads) void k_lmhead_tiles(Operand W, Operand Hd, int K, int tiles_m, int tiles_n,
                                                                  TileArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   int tm, tn;
   tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
-  Acc<wide::S> acc;
-  wide::mainloop<0>(W, Hd, K, m0, n0, acc, lds);  // ends with a barrier: LDS is free
+  Acc acc;
+  mainloop<false, false>(W, Hd, K, m0, n0, acc, lds);  // ends with a barrier: LDS is free
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int V = W.rows, N = Hd.rows;
-  const int mbase = m0 + wm * 128;    // first vocabulary row of this wave's block
-  const bool ragged = m0 + BM > V;    // rows past the vocabulary: last tile row only
-  uint16_t* Z = (uint16_t*)lds;       // [256 tokens][kPanelPitch] bf16
+  const int mbase = m0 + wm * 128;  // first vocabulary row of this wave's block
+  uint16_t* Z = (uint16_t*)lds;     // [256 tokens][kPanelPitch] bf16
   constexpr int PZ = kPanelPitch;
 
+  if constexpr (MODE != kModeRecompute) {
+    if (m0 + BM > V)  // rows past the vocabulary: last tile row only
+      block_stats<MODE == kModeStatsCarry, true>(acc, a, tm, wm, wn, n0, N, V, mbase, lane, Z);
+    else
+      block_stats<MODE == kModeStatsCarry, false>(acc, a, tm, wm, wn, n0, N, V, mbase, lane, Z);
+  } else {
 #pragma unroll
-  for (int nt = 0; nt < 4; ++nt) {
-    const int nloc = wn * 128 + acc_col(nt, lane);
-    const int n = n0 + nloc;
-    const bool live = n < N;
-    if constexpr (MODE != kModeRecompute) {
-      float mx = -FLT_MAX;
-#pragma unroll
-      for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const bool in = !ragged || (mbase + acc_row(mt, i, lane) < V);
-          mx = in ? fmaxf(mx, acc.v[mt][nt][i]) : mx;
-        }
-      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));  // both halves of the wave hold the same token
-      const float k = fmaxf(mx * a.c, kNegBig);   // kNegBig: no valid row in this block
-      float s = 0.f, u = 0.f;
-#pragma unroll
-      for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-          float e[4];
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const bool in = !ragged || (mbase + acc_row(mt, g4 * 4 + q, lane) < V);
-            const float t = in ? fmaf(acc.v[mt][nt][g4 * 4 + q], a.c, -k) : 0.f;
-            e[q] = in ? fast_exp2(t) : 0.f;
-            s += e[q];
-            u = fmaf(t, e[q], u);
-          }
-          if constexpr (MODE == kModeStatsCarry) {
-            uint2 pk;
-            pk.x = Elem<AA_BF16>::pack(e[0], e[1]);
-            pk.y = Elem<AA_BF16>::pack(e[2], e[3]);
-            *(uint2*)(Z + nloc * PZ + wm * 128 + mt * 32 + 8 * g4 + 4 * (lane >> 5)) = pk;
-          }
-        }
-      s += __shfl_xor(s, 32, kWave);
-      u += __shfl_xor(u, 32, kWave);
-      if (lane < 32 && live) {
-        const int64_t at = (int64_t)(tm * 2 + wm) * a.pitch_t + n;
-        a.pk[at] = k;
-        a.ps[at] = s;
-        a.pu[at] = u;
-      }
-      // label logit, if the label falls into this wave's 128 vocabulary rows (one of the two partner lanes owns it)
-      if (live) {
-        const int64_t y = a.labels[n];
-        const int64_t rel = y - mbase;
-        if (rel >= 0 && rel < 128 && y < V && (int)((rel >> 2) & 1) == (lane >> 5)) {
-          const int mt_y = (int)(rel >> 5), r5 = (int)(rel & 31);
-          const int i_y = ((r5 >> 3) << 2) | (r5 & 3);
-          float val = 0.f;
-#pragma unroll
-          for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i)
-              if (mt == mt_y && i == i_y) val = acc.v[mt][nt][i];
-          a.xy[n] = val;
-        }
-      }
-    } else {
+    for (int nt = 0; nt < 4; ++nt) {
+      const int nloc = wn * 128 + acc_col(nt, lane);
+      const int n = n0 + nloc;
       float A = 0.f, B = 0.f, lab_add = 0.f, lse2 = 0.f;
       int64_t y = -1;
-      if (live) {
+      if (n < N) {
         const int t = a.col_tokens ? a.col_tokens[n] : n;
         const float gl = a.g_logp[t];
         const float gh = a.g_entropy ? a.g_entropy[t] : 0.f;
@@ -153,7 +159,7 @@ __global__ __launch_bounds__(wide::kThreads) void k_lmhead_tiles(Operand W, Oper
         lab_add = gl * a.inv_t;
         y = a.labels[t];
       }
-      const int64_t rel = y - mbase;
+      const int rel = (int)(y - mbase < -1 ? -1 : (y - mbase > 128 ? 128 : y - mbase));  // outside [0, 128): not here
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
@@ -162,7 +168,7 @@ __global__ __launch_bounds__(wide::kThreads) void k_lmhead_tiles(Operand W, Oper
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             const float x = acc.v[mt][nt][g4 * 4 + q];
-            o[q] = live ? fast_exp2(fmaf(x, a.c, -lse2)) * fmaf(B, x, A) : 0.f;
+            o[q] = fast_exp2(fmaf(x, a.c, -lse2)) * fmaf(B, x, A);  // columns past the tokens: never written out
           }
           const int r0 = mt * 32 + 8 * g4 + 4 * (lane >> 5);  // row of o[0] inside the wave's block
           if (rel >= r0 && rel < r0 + 4) {
@@ -180,7 +186,7 @@ __global__ __launch_bounds__(wide::kThreads) void k_lmhead_tiles(Operand W, Oper
   if constexpr (MODE != kModeStats) {
     __syncthreads();
     // panel rows: 16-byte pieces along the vocabulary (V % 8 == 0: a piece never straddles the end)
-    for (int p = tid; p < 256 * 32; p += wide::kThreads) {
+    for (int p = tid; p < 256 * 32; p += kThreads) {
       const int nloc = p >> 5, mc = (p & 31) * 8;
       const int n = n0 + nloc, m = m0 + mc;
       if (n < N && m < V) {
@@ -191,43 +197,86 @@ __global__ __launch_bounds__(wide::kThreads) void k_lmhead_tiles(Operand W, Oper
   }
 }
 
-// Merge of the block partials of one token, in block order (fixed order: deterministic)
+// Raw label logit of every token: xy[t] = hidden[t] . weight[label[t]] in fp32 (NaN for a label outside [0, V)).  One
+// wave per token.
+__global__ __launch_bounds__(256) void k_label_logit(const uint16_t* __restrict__ hidden, const uint16_t* __restrict__ weight,
+                                                     const int64_t* __restrict__ labels, int n_tok, int H, int V,
+                                                     float* __restrict__ xy) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (t >= n_tok) return;
+  const int64_t y = labels[t];
+  if (y < 0 || y >= V) {
+    if (lane == 0) xy[t] = __builtin_nanf("");
+    return;
+  }
+  const uint16_t* h = hidden + (int64_t)t * H;
+  const uint16_t* w = weight + y * H;
+  float acc = 0.f;
+  for (int j = lane * 8; j < H; j += 64 * 8) {
+    float a[8], b[8];
+    load8<AA_BF16>(h, j, a);
+    load8<AA_BF16>(w, j, b);
+#pragma unroll
+    for (int q = 0; q < 8; ++q) acc = fmaf(a[q], b[q], acc);
+  }
+  acc = wave_sum(acc);
+  if (lane == 0) xy[t] = acc;
+}
+
+// Merge of the block partials of 64 tokens by a workgroup of 1024 threads: lane = token, wave w folds blocks
+// w, w + 16, ... in order, then the 16 wave results are folded in wave order by every wave alike.  Fixed order:
+// deterministic.
 struct Merged {
   float k, s, u;
 };
+constexpr int kMergeWaves = 16;
+
+__device__ __forceinline__ void merge_into(Merged& m, float bk, float bs, float bu) {
+  const float nk = fmaxf(m.k, bk);
+  const float da = m.k - nk, db = bk - nk;
+  const float fa = fast_exp2(da), fb = fast_exp2(db);
+  m.u = fa * fmaf(da, m.s, m.u) + fb * fmaf(db, bs, bu);
+  m.s = m.s * fa + bs * fb;
+  m.k = nk;
+}
+
+// t: the token of this lane (may be past the end: then the result is meaningless and the caller drops it)
 __device__ __forceinline__ Merged merge_blocks(const float* __restrict__ pk, const float* __restrict__ ps,
-                                               const float* __restrict__ pu, int blocks, int64_t pitch_t, int64_t t) {
-  float k = kNegBig, s = 0.f, u = 0.f;
-  for (int b = 0; b < blocks; ++b) {
-    const int64_t at = (int64_t)b * pitch_t + t;
-    const float bk = pk[at], bs = ps[at], bu = pu[at];
-    const float nk = fmaxf(k, bk);
-    const float da = k - nk, db = bk - nk;
-    const float fa = fast_exp2(da), fb = fast_exp2(db);
-    u = fa * fmaf(da, s, u) + fb * fmaf(db, bs, bu);
-    s = s * fa + bs * fb;
-    k = nk;
-  }
-  return {k, s, u};
+                                               const float* __restrict__ pu, int blocks, int64_t pitch_t, int64_t t,
+                                               bool live, float* smem /* [3][16][64] */) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  Merged m{kNegBig, 0.f, 0.f};
+  if (live)
+    for (int b = wave; b < blocks; b += kMergeWaves) {
+      const int64_t at = (int64_t)b * pitch_t + t;
+      merge_into(m, pk[at], ps[at], pu[at]);
+    }
+  smem[(0 * kMergeWaves + wave) * 64 + lane] = m.k;
+  smem[(1 * kMergeWaves + wave) * 64 + lane] = m.s;
+  smem[(2 * kMergeWaves + wave) * 64 + lane] = m.u;
+  __syncthreads();
+  Merged r{kNegBig, 0.f, 0.f};
+#pragma unroll
+  for (int w = 0; w < kMergeWaves; ++w)
+    merge_into(r, smem[(0 * kMergeWaves + w) * 64 + lane], smem[(1 * kMergeWaves + w) * 64 + lane],
+               smem[(2 * kMergeWaves + w) * 64 + lane]);
+  return r;
 }
 
-__global__ __launch_bounds__(256) void k_fill_f32(float* p, int64_t n, float v) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < n) p[i] = v;
-}
-
-// forward of the stand-alone op: one thread per token
-__global__ __launch_bounds__(256) void k_combine(const float* __restrict__ pk, const float* __restrict__ ps,
-                                                 const float* __restrict__ pu, const float* __restrict__ xy, int blocks,
-                                                 int64_t pitch_t, int n_tok, float c, float* __restrict__ logp,
-                                                 float* __restrict__ entropy, float* __restrict__ row_lse,
-                                                 float* __restrict__ row_ez) {
-  const int t = blockIdx.x * 256 + threadIdx.x;
-  if (t >= n_tok) return;
-  const Merged m = merge_blocks(pk, ps, pu, blocks, pitch_t, t);
+// forward of the stand-alone op: 64 tokens per workgroup
+__global__ __launch_bounds__(1024) void k_combine(const float* __restrict__ pk, const float* __restrict__ ps,
+                                                  const float* __restrict__ pu, const float* __restrict__ xy, int blocks,
+                                                  int64_t pitch_t, int n_tok, float c, float* __restrict__ logp,
+                                                  float* __restrict__ entropy, float* __restrict__ row_lse,
+                                                  float* __restrict__ row_ez) {
+  __shared__ float smem[3 * kMergeWaves * 64];
+  const int t = blockIdx.x * 64 + (threadIdx.x & 63);
+  const Merged m = merge_blocks(pk, ps, pu, blocks, pitch_t, t, t < n_tok, smem);
+  if (t >= n_tok || threadIdx.x >= 64) return;
   const float log2s = fast_log2(m.s);
   const float mean_t = m.u / m.s;
-  logp[t] = (fmaf(xy[t], c, -m.k) - log2s) * kLn2;  // xy stays NaN for a label outside [0, V)
+  logp[t] = (fmaf(xy[t], c, -m.k) - log2s) * kLn2;  // xy is NaN for a label outside [0, V)
   if (entropy) entropy[t] = (log2s - mean_t) * kLn2;
   if (row_lse) row_lse[t] = (m.k + log2s) * kLn2;
   if (row_ez) row_ez[t] = (m.k + mean_t) * kLn2;
@@ -260,15 +309,16 @@ struct TokenLossArgs {
 // Training step, after the forward tiles of a chunk: log-prob, entropy, per-token loss outputs (as the fused logits
 // kernel writes them, areal/utils/functional/functional.py:505-558) and g = d(scaled loss) / d(logp); then what the
 // backward needs: g and the row's logsumexp per token (recompute), or the row coefficients per panel row (carry).
-__global__ __launch_bounds__(256) void k_token_loss(const float* __restrict__ pk, const float* __restrict__ ps,
-                                                    const float* __restrict__ pu, const float* __restrict__ xy, int blocks,
-                                                    int64_t pitch_t, int n_tok, int V, float c, float inv_t,
-                                                    const int64_t* __restrict__ labels, TokenLossArgs a,
-                                                    const int32_t* __restrict__ out_rows, float* __restrict__ g_tok,
-                                                    float* __restrict__ lse_tok, RowCoef* __restrict__ rowc) {
-  const int t = blockIdx.x * 256 + threadIdx.x;
-  if (t >= n_tok) return;
-  const Merged m = merge_blocks(pk, ps, pu, blocks, pitch_t, t);
+__global__ __launch_bounds__(1024) void k_token_loss(const float* __restrict__ pk, const float* __restrict__ ps,
+                                                     const float* __restrict__ pu, const float* __restrict__ xy, int blocks,
+                                                     int64_t pitch_t, int n_tok, int V, float c, float inv_t,
+                                                     const int64_t* __restrict__ labels, TokenLossArgs a,
+                                                     const int32_t* __restrict__ out_rows, float* __restrict__ g_tok,
+                                                     float* __restrict__ lse_tok, RowCoef* __restrict__ rowc) {
+  __shared__ float smem[3 * kMergeWaves * 64];
+  const int t = blockIdx.x * 64 + (threadIdx.x & 63);
+  const Merged m = merge_blocks(pk, ps, pu, blocks, pitch_t, t, t < n_tok, smem);
+  if (t >= n_tok || threadIdx.x >= 64) return;
   const float log2s = fast_log2(m.s);
   const float lp = (fmaf(xy[t], c, -m.k) - log2s) * kLn2;
   a.logp[t] = lp;
@@ -335,98 +385,68 @@ __global__ __launch_bounds__(256) void k_panel_scale(uint16_t* __restrict__ pane
   }
 }
 
-// ---- plain product D = A . B^T on the same main loop ---------------------------------------------------------------
-// D [M, N] row-major with leading dimension ldd, bf16 or fp32; ACCUM adds to what D holds (fp32 only).
-template <typename OutT, bool ACCUM>
-__global__ __launch_bounds__(wide::kThreads) void k_gemm_store(Operand A, Operand B, int K, int tiles_m, int tiles_n,
-                                                               OutT* __restrict__ D, int64_t ldd) {
+// ---- plain product C = B . A^T on the same main loop ---------------------------------------------------------------
+// C [N, M] row-major with leading dimension ldc: C[n][m] = sum_k B[n][k] A[m][k]; AKM / BKM: the operand is stored
+// K-major (see gemm_tn.h).  The operand whose rows are the columns of C goes first, because a lane of the accumulator layout owns one n and runs of four consecutive m: four
+// neighbouring outputs of a row of C.  bf16 C: the tile is staged in LDS as [n][m] and leaves in 16-byte pieces,
+// 512 contiguous bytes per row; row n of the product is written to row c_rows[n] of C when a row list is given.
+// fp32 C: 16-byte stores straight from the registers; ACCUM adds to what C holds.
+template <bool AKM, bool BKM, typename OutT, bool ACCUM>
+__global__ __launch_bounds__(kThreads) void k_gemm_store(Operand A, Operand B, int K, int tiles_m, int tiles_n,
+                                                         OutT* __restrict__ C, int64_t ldc,
+                                                         const int32_t* __restrict__ c_rows) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   int tm, tn;
   tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
-  Acc<wide::S> acc;
-  wide::mainloop<0>(A, B, K, m0, n0, acc, lds);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  Acc acc;
+  mainloop<AKM, BKM>(A, B, K, m0, n0, acc, lds);  // ends with a barrier: LDS is free
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int M = A.rows, N = B.rows;
+  if constexpr (sizeof(OutT) == 2) {
+    uint16_t* Z = (uint16_t*)lds;  // [256 n][kPanelPitch] bf16
+    constexpr int PZ = kPanelPitch;
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt)
+    for (int nt = 0; nt < 4; ++nt) {
+      const int nloc = wn * 128 + acc_col(nt, lane);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int m = m0 + wm * 128 + acc_row(mt, i, lane);
-      if (m >= M) continue;
-      OutT* row = D + (int64_t)m * ldd;
+      for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt) {
-        const int n = n0 + wn * 128 + acc_col(nt, lane);
-        if (n >= N) continue;
-        float v = acc.v[mt][nt][i];
-        if constexpr (sizeof(OutT) == 4) {
-          if (ACCUM) v += row[n];
-          row[n] = v;
-        } else {
-          row[n] = (uint16_t)(Elem<AA_BF16>::pack(v, 0.f) & 0xffffu);
+        for (int g4 = 0; g4 < 4; ++g4) {
+          uint2 pk;
+          pk.x = Elem<AA_BF16>::pack(acc.v[mt][nt][g4 * 4], acc.v[mt][nt][g4 * 4 + 1]);
+          pk.y = Elem<AA_BF16>::pack(acc.v[mt][nt][g4 * 4 + 2], acc.v[mt][nt][g4 * 4 + 3]);
+          *(uint2*)(Z + nloc * PZ + wm * 128 + mt * 32 + 8 * g4 + 4 * (lane >> 5)) = pk;
         }
+    }
+    __syncthreads();
+    for (int p = tid; p < 256 * 32; p += kThreads) {  // M % 8 == 0: a piece never straddles the end
+      const int nloc = p >> 5, mc = (p & 31) * 8;
+      const int n = n0 + nloc, m = m0 + mc;
+      if (n < N && m < M) {
+        const int64_t r = c_rows ? c_rows[n] : n;
+        *(u32x4_t*)(C + r * ldc + m) = *(const u32x4_t*)(Z + nloc * PZ + mc);
       }
     }
-}
-
-// ---- bf16 transpose: dst[c, r] = src[r, c] ----------------------------------------------------------------------
-// src is [R, C] with row pitch lds (elements), dst is [C, ldd] with ldd >= R a multiple of 8; columns R .. ldd - 1 of dst
-// are written as zeros; with src_rows, row r of the source is row src_rows[r] of the array.  One workgroup moves a
-// 64 x 64 tile through LDS: each thread loads 8 elements of two adjacent rows (16 B each), pairs them into 32-bit
-// words (two consecutive dst columns) and stores the words transposed; the second half reads 16 B per thread and
-// writes 128 B contiguous per dst row.  The word index is XOR-ed with a key of the row so that both halves run
-// without bank conflicts.  Requires C % 8 == 0, lds % 8 == 0.  Tiles are numbered along r first, in bands of
-// kTransposeBand tile rows, so that the workgroups in flight together write long contiguous pieces of the dst rows
-// (measured: 5.2 TB/s against 3.9 with c first).
-constexpr int kTransposeBand = 64;
-
-__global__ __launch_bounds__(256) void k_transpose_bf16(const uint16_t* __restrict__ src, int R, int C, int64_t lds,
-                                                        uint16_t* __restrict__ dst, int64_t ldd, int tiles_c,
-                                                        int tiles_r, const int32_t* __restrict__ src_rows) {
-  __shared__ uint32_t tile[64 * 32];
-  const int t = threadIdx.x;
-  const int per_band = kTransposeBand * tiles_c;
-  const int band = blockIdx.x / per_band, rem = blockIdx.x % per_band;
-  const int rows_in_band = min(kTransposeBand, tiles_r - band * kTransposeBand);
-  const int c0 = (rem / rows_in_band) * 64, r0 = (band * kTransposeBand + rem % rows_in_band) * 64;
-  {
-    const int rp = t >> 3, c8 = (t & 7) * 8;
-    const int r = r0 + 2 * rp, c = c0 + c8;
-    u32x4_t a = {0u, 0u, 0u, 0u}, b = {0u, 0u, 0u, 0u};
-    if (c < C) {  // logical row r of the source is row src_rows[r] of src when a row list is given
-      if (r < R) a = __builtin_nontemporal_load((const u32x4_t*)(src + (int64_t)(src_rows ? src_rows[r] : r) * lds + c));
-      if (r + 1 < R)
-        b = __builtin_nontemporal_load((const u32x4_t*)(src + (int64_t)(src_rows ? src_rows[r + 1] : r + 1) * lds + c));
-    }
-    const int key = ((t & 7) & 3) << 3;  // = (((c8 + j) >> 3) & 3) << 3 for every j < 8
+  } else {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const uint32_t wa = a[j >> 1], wb = b[j >> 1];
-      const uint32_t lo = (j & 1) ? (wa >> 16) : (wa & 0xffffu);
-      const uint32_t hi = (j & 1) ? (wb & 0xffff0000u) : (wb << 16);
-      tile[(c8 + j) * 32 + (rp ^ key)] = lo | hi;
+    for (int nt = 0; nt < 4; ++nt) {
+      const int n = n0 + wn * 128 + acc_col(nt, lane);
+      if (n >= N) continue;
+      float* row = (float*)C + (c_rows ? c_rows[n] : n) * ldc;
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          const int m = m0 + wm * 128 + mt * 32 + 8 * g4 + 4 * (lane >> 5);  // M % 4 == 0
+          if (m >= M) continue;
+          f32x4_t v = {acc.v[mt][nt][g4 * 4], acc.v[mt][nt][g4 * 4 + 1], acc.v[mt][nt][g4 * 4 + 2], acc.v[mt][nt][g4 * 4 + 3]};
+          if (ACCUM) v += *(const f32x4_t*)(row + m);
+          *(f32x4_t*)(row + m) = v;
+        }
     }
   }
-  __syncthreads();
-#pragma unroll
-  for (int p = 0; p < 2; ++p) {
-    const int cl = (t >> 3) + 32 * p, g = t & 7;
-    const int key = ((cl >> 3) & 3) << 3;
-    const u32x4_t v = *(const u32x4_t*)(tile + cl * 32 + ((4 * g) ^ key));
-    const int c = c0 + cl;
-    const int64_t r = r0 + 8 * g;
-    if (c < C && r < ldd) *(u32x4_t*)(dst + (int64_t)c * ldd + r) = v;
-  }
-}
-
-// dst gets ldd columns (ldd >= R, a multiple of 8): the transposed R rows of src, then zeros
-static void launch_transpose(hipStream_t st, const uint16_t* src, int64_t R, int64_t C, int64_t lds, uint16_t* dst,
-                             int64_t ldd, const int32_t* src_rows = nullptr) {
-  const int64_t tiles_c = (C + 63) / 64, tiles_r = (ldd + 63) / 64;
-  hipLaunchKernelGGL(k_transpose_bf16, dim3((unsigned)(tiles_c * tiles_r)), dim3(256), 0, st, src, (int)R, (int)C, lds, dst,
-                     ldd, (int)tiles_c, (int)tiles_r, src_rows);
 }
 
 // ---- tokens without gradient are left out of the backward GEMMs -------------------------------------------------
@@ -466,15 +486,6 @@ __global__ __launch_bounds__(1024) void k_compact_map(const uint8_t* __restrict_
   for (int p = total + tid; p < limit; p += 1024) act_rows[p] = 0;
 }
 
-// dst[t, :] = out_rows[t] >= 0 ? src[out_rows[t], :] : 0 for the n_tok rows of a chunk (H % 8 == 0)
-__global__ __launch_bounds__(256) void k_scatter_rows(const u32x4_t* __restrict__ src, const int32_t* __restrict__ out_rows,
-                                                      u32x4_t* __restrict__ dst, int h_vec) {
-  const int64_t t = blockIdx.x;
-  const int r = out_rows[t];
-  const u32x4_t zero = {0u, 0u, 0u, 0u};
-  for (int j = threadIdx.x; j < h_vec; j += 256) dst[t * h_vec + j] = r >= 0 ? src[(int64_t)r * h_vec + j] : zero;
-}
-
 // dst[r, :] = src[rows[r], :] (H % 8 == 0)
 __global__ __launch_bounds__(256) void k_gather_rows(const u32x4_t* __restrict__ src, const int32_t* __restrict__ rows,
                                                      u32x4_t* __restrict__ dst, int h_vec) {
@@ -497,7 +508,6 @@ static void launch_zero(hipStream_t st, void* p, int64_t bytes) {  // bytes % 16
 }
 
 // fp32 -> bf16 (round to nearest even), 8 elements per thread; n % 8 == 0
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 __global__ __launch_bounds__(256) void k_f32_to_bf16(const f32x4_t* __restrict__ src, u32x4_t* __restrict__ dst,
                                                      int64_t n8) {
@@ -520,9 +530,8 @@ struct Workspace {
   int64_t fwd_bytes;                    // what the forward alone needs
   int64_t off_rowc;                     // RowCoef per panel row
   int64_t off_rows;                     // out_rows, act_rows (2 x chunk int32)
-  int64_t off_panel, off_panel_t;       // d(logits) rows [chunk, V] and their transpose [V, chunk]
-  int64_t off_wt, off_ht;               // weight^T [H, V], hidden rows^T [H, chunk]
-  int64_t off_dhc, off_hc;              // d_hidden of the rows with gradient [chunk, H]; those rows of hidden
+  int64_t off_panel;                    // d(logits) rows [chunk, V]
+  int64_t off_hc;                       // the hidden rows of the tokens with gradient, closed up [chunk, H]
   int64_t off_dw;                       // fp32 accumulator of a bf16 d_weight when there is more than one chunk
   int64_t bytes;
 };
@@ -543,10 +552,6 @@ static Workspace plan(int64_t T, int64_t H, int64_t V) {
   w.off_rowc = off;    off += up(w.chunk * (int64_t)sizeof(RowCoef));
   w.off_rows = off;    off += up(2 * w.chunk * 4);
   w.off_panel = off;   off += up(w.chunk * V * 2);
-  w.off_panel_t = off; off += up(w.chunk * V * 2);
-  w.off_wt = off;      off += up(H * V * 2);
-  w.off_ht = off;      off += up(w.chunk * H * 2);
-  w.off_dhc = off;     off += up(w.chunk * H * 2);
   w.off_hc = off;      off += up(w.chunk * H * 2);
   w.off_dw = off;      off += T > w.chunk ? up(V * H * 4) : 0;
   w.bytes = off;
@@ -555,14 +560,13 @@ static Workspace plan(int64_t T, int64_t H, int64_t V) {
 
 static bool shapes_ok(int64_t T, int64_t H, int64_t V) {
   // 256 rows of any operand must stay below 2^30 elements (32-bit byte offsets inside a tile)
-  return T > 0 && H > 0 && V > 0 && (H % 8) == 0 && (V % 8) == 0 && T < (1 << 30) && V < (1 << 22) && H < (1 << 22) &&
-         (V / 64 + 1) * ((H > kChunkTokens ? H : kChunkTokens) / 64 + 1) < (1LL << 31);  // transpose grids
+  return T > 0 && H > 0 && V > 0 && (H % 8) == 0 && (V % 8) == 0 && T < (1 << 30) && V < (1 << 22) && H < (1 << 22);
 }
 
 // The tile kernels use all 160 KiB of LDS: allow it once per kernel and device.
 template <typename Kern>
 static bool allow_big_lds(Kern k) {
-  return hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, wide::kLdsBytes) == hipSuccess;
+  return hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) == hipSuccess;
 }
 
 static bool prepare_kernels() {
@@ -572,8 +576,9 @@ static bool prepare_kernels() {
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return false;
   if (done[dev]) return true;
   const bool ok = allow_big_lds(k_lmhead_tiles<kModeStats>) && allow_big_lds(k_lmhead_tiles<kModeStatsCarry>) &&
-                  allow_big_lds(k_lmhead_tiles<kModeRecompute>) && allow_big_lds(k_gemm_store<uint16_t, false>) &&
-                  allow_big_lds(k_gemm_store<float, false>) && allow_big_lds(k_gemm_store<float, true>);
+                  allow_big_lds(k_lmhead_tiles<kModeRecompute>) && allow_big_lds(k_gemm_store<true, false, uint16_t, false>) &&
+                  allow_big_lds(k_gemm_store<true, true, uint16_t, false>) &&
+                  allow_big_lds(k_gemm_store<true, true, float, false>) && allow_big_lds(k_gemm_store<true, true, float, true>);
   done[dev] = ok;
   return ok;
 }
@@ -584,42 +589,45 @@ static void launch_tiles(hipStream_t st, const void* weight, const uint16_t* hid
   const int tiles_m = (int)((V + BM - 1) / BM), tiles_n = (int)((n_tok + BN - 1) / BN);
   Operand W{(const uint16_t*)weight, H, (int)V};
   Operand Hd{hid, H, (int)n_tok};
-  hipLaunchKernelGGL(k_lmhead_tiles<MODE>, dim3((unsigned)(tiles_m * tiles_n)), dim3(wide::kThreads), wide::kLdsBytes, st,
+  hipLaunchKernelGGL(k_lmhead_tiles<MODE>, dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads), kLdsBytes, st,
                      W, Hd, (int)H, tiles_m, tiles_n, a);
 }
 
-// D [M, N] = A [M, K] . B [N, K]^T
-template <typename OutT, bool ACCUM>
+// C [N, M] = B . A^T over K (rows of C through c_rows when given); lda / ldb: leading dimensions of the arrays as stored
+template <bool AKM, bool BKM, typename OutT, bool ACCUM>
 static void launch_gemm(hipStream_t st, const uint16_t* A, int64_t lda, int64_t M, const uint16_t* B, int64_t ldb, int64_t N,
-                        int64_t K, OutT* D, int64_t ldd) {
+                        int64_t K, OutT* C, int64_t ldc, const int32_t* c_rows = nullptr) {
   const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
   Operand a{A, lda, (int)M}, b{B, ldb, (int)N};
-  hipLaunchKernelGGL((k_gemm_store<OutT, ACCUM>), dim3((unsigned)(tiles_m * tiles_n)), dim3(wide::kThreads),
-                     wide::kLdsBytes, st, a, b, (int)K, tiles_m, tiles_n, D, ldd);
+  hipLaunchKernelGGL((k_gemm_store<AKM, BKM, OutT, ACCUM>), dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads), kLdsBytes, st,
+                     a, b, (int)K, tiles_m, tiles_n, C, ldc, c_rows);
 }
 
 // The two GEMMs that contract the d(logits) rows ds [n_rows, V] (in the panel) of one token chunk:
-//   d_hidden rows = ds . W          (bf16)          d_weight (+)= ds^T . hidden rows   (fp32, or bf16 when first)
-// with transposed copies of ds and of the hidden rows (made here; their token count is padded to a multiple of 8 with
-// zeros) and of the weight (made once per call, by the caller, at ws + off_wt).  hid_rows, when given, lists the rows
-// of the hidden chunk that the n_rows rows of ds belong to (tokens without gradient were left out).
-static void panel_gradients(hipStream_t st, const Workspace& w, char* ws, const uint16_t* hid, const int32_t* hid_rows,
-                            int64_t n_rows, int64_t H, int64_t V, uint16_t* d_hidden_rows, void* d_weight, bool dw_f32,
-                            bool first) {
+//   d_hidden rows [n_rows, H] = ds . W                  contraction over V: ds K-contiguous, W [V, H] K-major
+//   d_weight [V, H] (+)= ds^T . hidden rows             contraction over the rows: both arrays K-major
+// No transposed copy of anything is made.  token_of_row, when given, lists the tokens of the chunk that the n_rows
+// rows of ds belong to (tokens without gradient were left out): their hidden rows are closed up first, and the
+// d_hidden rows go to those tokens (the caller has cleared the others).
+static void panel_gradients(hipStream_t st, const Workspace& w, char* ws, const void* weight, const uint16_t* hid,
+                            const int32_t* token_of_row, int64_t n_rows, int64_t H, int64_t V, uint16_t* d_hidden_chunk,
+                            void* d_weight, bool dw_f32, bool first) {
   const uint16_t* ds = (const uint16_t*)(ws + w.off_panel);
-  uint16_t* ds_t = (uint16_t*)(ws + w.off_panel_t);
-  const uint16_t* w_t = (const uint16_t*)(ws + w.off_wt);
-  uint16_t* hid_t = (uint16_t*)(ws + w.off_ht);
-  const int64_t kp = round_up(n_rows, 8);
-  launch_gemm<uint16_t, false>(st, ds, V, n_rows, w_t, V, H, V, d_hidden_rows, H);
-  launch_transpose(st, ds, n_rows, V, V, ds_t, kp);
-  launch_transpose(st, hid, n_rows, H, H, hid_t, kp, hid_rows);
+  const uint16_t* hid_rows = hid;
+  if (token_of_row) {
+    uint16_t* hc = (uint16_t*)(ws + w.off_hc);
+    hipLaunchKernelGGL(k_gather_rows, dim3((unsigned)n_rows), dim3(256), 0, st, (const u32x4_t*)hid, token_of_row,
+                       (u32x4_t*)hc, (int)(H / 8));
+    hid_rows = hc;
+  }
+  launch_gemm<true, false, uint16_t, false>(st, (const uint16_t*)weight, H, H, ds, V, n_rows, V, d_hidden_chunk, H,
+                                            token_of_row);
   if (!dw_f32)
-    launch_gemm<uint16_t, false>(st, ds_t, kp, V, hid_t, kp, H, kp, (uint16_t*)d_weight, H);
+    launch_gemm<true, true, uint16_t, false>(st, hid_rows, H, H, ds, V, V, n_rows, (uint16_t*)d_weight, H);
   else if (first)
-    launch_gemm<float, false>(st, ds_t, kp, V, hid_t, kp, H, kp, (float*)d_weight, H);
+    launch_gemm<true, true, float, false>(st, hid_rows, H, H, ds, V, V, n_rows, (float*)d_weight, H);
   else
-    launch_gemm<float, true>(st, ds_t, kp, V, hid_t, kp, H, kp, (float*)d_weight, H);
+    launch_gemm<true, true, float, true>(st, hid_rows, H, H, ds, V, V, n_rows, (float*)d_weight, H);
 }
 
 // Recompute: d(logits) of the panel rows from the logits tiles formed again.  With a row map only the hidden rows that
@@ -708,9 +716,11 @@ extern "C" int aa_lmhead_fwd(const void* hidden, const void* weight, int64_t T, 
   for (int64_t t0 = 0; t0 < T; t0 += w.chunk) {
     const int64_t n_tok = (T - t0) < w.chunk ? (T - t0) : w.chunk;
     const TileArgs a = stats_args(w, ws, labels + t0, inv_temperature);
-    hipLaunchKernelGGL(k_fill_f32, dim3((unsigned)((n_tok + 255) / 256)), dim3(256), 0, st, a.xy, n_tok, __builtin_nanf(""));
-    launch_tiles<kModeStats>(st, weight, (const uint16_t*)hidden + t0 * H, n_tok, H, V, a);
-    hipLaunchKernelGGL(k_combine, dim3((unsigned)((n_tok + 255) / 256)), dim3(256), 0, st, a.pk, a.ps, a.pu, a.xy,
+    const uint16_t* hid = (const uint16_t*)hidden + t0 * H;
+    hipLaunchKernelGGL(k_label_logit, dim3((unsigned)((n_tok + 3) / 4)), dim3(256), 0, st, hid, (const uint16_t*)weight,
+                       labels + t0, (int)n_tok, (int)H, (int)V, a.xy);
+    launch_tiles<kModeStats>(st, weight, hid, n_tok, H, V, a);
+    hipLaunchKernelGGL(k_combine, dim3((unsigned)((n_tok + 63) / 64)), dim3(1024), 0, st, a.pk, a.ps, a.pu, a.xy,
                        (int)w.blocks, a.pitch_t, (int)n_tok, a.c, logp + t0, at(entropy, t0), at(row_lse, t0),
                        at(row_ez, t0));
   }
@@ -734,7 +744,6 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
   if (!prepare_kernels()) return AA_ERR_LAUNCH;
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
-  launch_transpose(st, (const uint16_t*)weight, V, H, H, (uint16_t*)(ws + w.off_wt), V);
   const WeightGrad dw = weight_grad(w, ws, d_weight, d_weight_dtype, T);
   int32_t* out_rows = (int32_t*)(ws + w.off_rows);
   int32_t* act_rows = out_rows + w.chunk;
@@ -754,7 +763,7 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
     a.g_entropy = g_entropy ? g_entropy + t0 : nullptr;
     if (!kept_per_chunk) {
       recompute_panel(st, w, ws, weight, hid, n_tok, nullptr, n_tok, H, V, a);
-      panel_gradients(st, w, ws, hid, nullptr, n_tok, H, V, dh, dw.acc, dw.acc_f32, first);
+      panel_gradients(st, w, ws, weight, hid, nullptr, n_tok, H, V, dh, dw.acc, dw.acc_f32, first);
       first = false;
       continue;
     }
@@ -768,11 +777,9 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
     hipLaunchKernelGGL(k_compact_map, dim3(1), dim3(1024), 0, st, row_has_gradient + t0, (int)n_tok, (int)n_tok, (int)kept,
                        out_rows, act_rows);
     recompute_panel(st, w, ws, weight, hid, n_tok, act_rows, kept, H, V, a);
-    uint16_t* dh_kept = (uint16_t*)(ws + w.off_dhc);
-    panel_gradients(st, w, ws, hid, act_rows, kept, H, V, dh_kept, dw.acc, dw.acc_f32, first);
+    launch_zero(st, dh, n_tok * H * 2);  // the rows of the other tokens
+    panel_gradients(st, w, ws, weight, hid, act_rows, kept, H, V, dh, dw.acc, dw.acc_f32, first);
     first = false;
-    hipLaunchKernelGGL(k_scatter_rows, dim3((unsigned)n_tok), dim3(256), 0, st, (const u32x4_t*)dh_kept, out_rows,
-                       (u32x4_t*)dh, (int)(H / 8));
   }
   if (first) launch_zero(st, dw.acc, V * H * (dw.acc_f32 ? 4 : 2));  // no row of the batch has a gradient
   finish_weight_grad(st, dw, d_weight, V, H);
@@ -805,7 +812,6 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
   const bool carry = backward_mode == AA_LMHEAD_CARRY;
-  launch_transpose(st, (const uint16_t*)weight, V, H, H, (uint16_t*)(ws + w.off_wt), V);
   const WeightGrad dw = weight_grad(w, ws, d_weight, d_weight_dtype, T);
   int32_t* out_rows = (int32_t*)(ws + w.off_rows);
   int32_t* act_rows = out_rows + w.chunk;
@@ -839,7 +845,8 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
     a.panel = panel;
     a.panel_ld = V;
     a.out_rows = row_of_token;
-    hipLaunchKernelGGL(k_fill_f32, dim3((unsigned)((n_tok + 255) / 256)), dim3(256), 0, st, a.xy, n_tok, __builtin_nanf(""));
+    hipLaunchKernelGGL(k_label_logit, dim3((unsigned)((n_tok + 3) / 4)), dim3(256), 0, st, hid, (const uint16_t*)weight,
+                       labels + t0, (int)n_tok, (int)H, (int)V, a.xy);
     if (carry && rows > 0)
       launch_tiles<kModeStatsCarry>(st, weight, hid, n_tok, H, V, a);
     else
@@ -847,7 +854,7 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
     // row statistics, per-token outputs, g
     TokenLossArgs la{at(prox_logp), at(adv), at(mask_eff), at(behave_w), n_valid, grad_scale, logp + t0, at(entropy),
                      at(stat_loss), at(ratio), at(flags), *params, act};
-    hipLaunchKernelGGL(k_token_loss, dim3((unsigned)((n_tok + 255) / 256)), dim3(256), 0, st, a.pk, a.ps, a.pu, a.xy,
+    hipLaunchKernelGGL(k_token_loss, dim3((unsigned)((n_tok + 63) / 64)), dim3(1024), 0, st, a.pk, a.ps, a.pu, a.xy,
                        (int)w.blocks, a.pitch_t, (int)n_tok, (int)V, a.c, inv_temperature, labels + t0, la, row_of_token,
                        g_tok, lse_tok, carry ? rowc : nullptr);
     if (rows == 0) {
@@ -862,14 +869,8 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
       a.g_logp = g_tok;
       recompute_panel(st, w, ws, weight, hid, n_tok, token_of_row, rows, H, V, a);
     }
-    if (!kept_per_chunk) {
-      panel_gradients(st, w, ws, hid, nullptr, n_tok, H, V, dh, dw.acc, dw.acc_f32, first);
-    } else {
-      uint16_t* dh_kept = (uint16_t*)(ws + w.off_dhc);
-      panel_gradients(st, w, ws, hid, act_rows, rows, H, V, dh_kept, dw.acc, dw.acc_f32, first);
-      hipLaunchKernelGGL(k_scatter_rows, dim3((unsigned)n_tok), dim3(256), 0, st, (const u32x4_t*)dh_kept, out_rows,
-                         (u32x4_t*)dh, (int)(H / 8));
-    }
+    if (token_of_row) launch_zero(st, dh, n_tok * H * 2);  // the rows of the tokens without gradient
+    panel_gradients(st, w, ws, weight, hid, token_of_row, rows, H, V, dh, dw.acc, dw.acc_f32, first);
     first = false;
   }
   if (first) launch_zero(st, dw.acc, V * H * (dw.acc_f32 ? 4 : 2));  // no token of the batch has a gradient

@@ -74,6 +74,9 @@ def parse_args():
     ap.add_argument("--dense-backward", action="store_true",
                     help="lm_head workloads: run masked tokens through the gradient GEMMs too (as the reference's "
                          "autograd does) instead of leaving their zero rows out")
+    ap.add_argument("--lmhead-backward", choices=["carry", "recompute"], default="carry",
+                    help="lm_head workloads: how the d(logits) rows of the backward are obtained (see "
+                         "fused_lm_head_ppo_loss)")
     ap.add_argument("--no-forward-of-masked", action="store_true",
                     help="lm_head workloads, outside the reference's semantics: masked tokens skip the lm_head "
                          "altogether (fused_lm_head_ppo_loss(forward_masked_tokens=False)); only ms_per_step and value "
@@ -364,6 +367,7 @@ def build_fused_case(name: str, seed: int, device):
 
 
 DENSE_BACKWARD = False  # set from --dense-backward
+BACKWARD_MODE = 1  # aa_lmhead_backward_mode: 1 carry, 0 recompute (set from --lmhead-backward)
 NO_FORWARD_OF_MASKED = False  # set from --no-forward-of-masked
 
 
@@ -378,7 +382,8 @@ def run_fused_steps(case, n, kw, cfg):
         loss, _ = areal_amd.fused_lm_head_ppo_loss(
             h, w, case.labels, case.prox_logp, case.old_logp, case.advantages, loss_mask=case.loss_mask,
             rejection_sampling=cfg, cu_seqlens=case.cu_seqlens, temperature=case.temperature,
-            skip_masked_tokens=not DENSE_BACKWARD, forward_masked_tokens=not NO_FORWARD_OF_MASKED, **kw,
+            skip_masked_tokens=not DENSE_BACKWARD, forward_masked_tokens=not NO_FORWARD_OF_MASKED,
+            backward="carry" if BACKWARD_MODE == 1 else "recompute", **kw,
         )
         loss.backward()
     return loss
@@ -423,8 +428,8 @@ def time_lmhead_step(case, kw, cfg, iters: int, skip_masked: bool):
             lib.aa_lmhead_ppo_fused(
                 F._ptr(case.hidden), F._ptr(case.weight), T, H, V, F._ptr(case.labels), 1.0 / case.temperature, T,
                 F._ptr(prox), F._ptr(adv), F._ptr(mask_eff), F._ptr(w), C.byref(params), F._ptr(counts), None, kept,
-                F._ptr(logp), F._ptr(ent), F._ptr(sl), F._ptr(ratio), F._ptr(flags), F._ptr(dh), F._ptr(dw),
-                N.AA_BF16, F._ptr(F._work_words(dev)), F._ptr(ws), ws.numel(), C.c_void_p(stream.cuda_stream),
+                BACKWARD_MODE, F._ptr(logp), F._ptr(ent), F._ptr(sl), F._ptr(ratio), F._ptr(flags), F._ptr(dh), F._ptr(dw),
+                N.AA_BF16, F._ptr(ws), ws.numel(), C.c_void_p(stream.cuda_stream),
             ),
             "aa_lmhead_ppo_fused",
         )
@@ -498,7 +503,7 @@ def fused_cpu_baseline_and_parity(case, kw, cfg, n_tokens: int, iters: int):
     def oracle_step():
         h = hid.clone().requires_grad_(True)
         w = w_cpu.clone().requires_grad_(True)
-        logits = (h @ w.t()).to(torch.bfloat16)  # the lm_head output dtype of the reference
+        logits = oracle.lmhead_logits(h, w)
         lp, _ent = oracle.logprobs_entropy(logits, lab, case.temperature)
         loss, _stat = oracle.ppo_actor_loss(lp, prox, old, adv, loss_mask=mask.bool(), rejection_sampling_cfg=cfg,
                                             cu_seqlens=cu, **kw)
@@ -797,8 +802,9 @@ def synth_lengths(total, seed):
 
 
 def main():
-    global RS_ACTION, DENSE_BACKWARD, NO_FORWARD_OF_MASKED
+    global RS_ACTION, DENSE_BACKWARD, NO_FORWARD_OF_MASKED, BACKWARD_MODE
     args = parse_args()
+    BACKWARD_MODE = 1 if args.lmhead_backward == "carry" else 0
     RS_ACTION = args.rs_action
     DENSE_BACKWARD = args.dense_backward
     NO_FORWARD_OF_MASKED = args.no_forward_of_masked
