@@ -12,6 +12,9 @@ from pathlib import Path
 LIB_PATH = Path(__file__).resolve().parent / "libareal_amd.so"
 
 AA_OK = 0
+AA_ERR_INVALID_ARGUMENT = 1
+AA_ERR_UNSUPPORTED = 2
+AA_ERR_LAUNCH = 3
 AA_BF16, AA_F16, AA_F32 = 0, 1, 2
 
 RS_LEVEL = {"token": 0, "sequence": 1}
@@ -79,6 +82,9 @@ SIGNATURES = {
     "aa_lmhead_fwd_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "aa_lmhead_fwd": (_i, [_p, _p, _i64, _i64, _i64, _p, _f, _p, _p, _p, _p, _p, _i64, _p]),
     "aa_lmhead_chunk_tokens": (_i64, []),
+    "aa_lmhead_fwd_static": (_i, [_p, _p, _i64, _i64, _i64, _p, _f, _p, _p, _p, _p, _p]),
+    "aa_lmhead_fwd_static_scratch_bytes": (_i64, []),
+    "aa_lmhead_fwd_static_max_vocab": (_i64, []),
     "aa_lmhead_bwd": (_i, [_p, _p, _i64, _i64, _i64, _p, _f, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i64, _p]),
     "aa_lmhead_ppo_fused": (
         _i,

@@ -727,6 +727,79 @@ extern "C" int aa_lmhead_fwd(const void* hidden, const void* weight, int64_t T, 
   return launch_status();
 }
 
+// ---- forward for callers that cannot allocate ---------------------------------------------------------------------
+// The softmax partials of aa_lmhead_fwd live in a device array of the library itself instead of a caller's workspace.
+// Host code never uses the array by name (that is a host-side stand-in, not a device address): its address on a device
+// is asked for once, with that device current, and kept.
+constexpr int64_t kStaticScratchBytes = 32ll << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+static char* static_scratch_on_current_device() {
+  constexpr int kMaxDevices = 64;
+  static char* ptr[kMaxDevices] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  if (!ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+    ptr[dev] = (char*)p;
+  }
+  return ptr[dev];
+}
+
+// tokens per pass of aa_lmhead_fwd_static for a vocabulary of V: what fits the array (a multiple of 256), 0 if none do
+static int64_t static_chunk_tokens(int64_t V) {
+  const int64_t blocks = 2 * ((V + BM - 1) / BM);
+  const int64_t per_token = (3 * blocks + 1) * 4;          // three planes of partials and the label logit
+  int64_t c = (kStaticScratchBytes - 4 * 256) / per_token;  // four arrays, each starting on a 256-byte boundary
+  c = c / 256 * 256;
+  return c > kChunkTokens ? kChunkTokens : c;
+}
+
+extern "C" int64_t aa_lmhead_fwd_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int64_t aa_lmhead_fwd_static_max_vocab(void) {
+  // largest V whose partials of 256 tokens fit: (3 * 2 * ceil(V / 256) + 1) * 4 * 256 + 1024 <= kStaticScratchBytes
+  const int64_t blocks = ((kStaticScratchBytes - 1024) / (4 * 256) - 1) / 3;
+  return blocks / 2 * BM;
+}
+
+extern "C" int aa_lmhead_fwd_static(const void* hidden, const void* weight, int64_t T, int64_t H, int64_t V,
+                                    const int64_t* labels, float inv_temperature, float* logp, float* entropy,
+                                    float* row_lse, float* row_ez, void* stream) {
+  if (!hidden || !weight || !labels || !logp || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
+  if (!shapes_ok(T, H, V)) return AA_ERR_UNSUPPORTED;
+  if ((((uintptr_t)hidden | (uintptr_t)weight) & 15) != 0) return AA_ERR_INVALID_ARGUMENT;
+  const int64_t chunk = static_chunk_tokens(V);
+  if (chunk < 256) return AA_ERR_UNSUPPORTED;  // V > aa_lmhead_fwd_static_max_vocab(): not even 256 tokens fit
+  if (!prepare_kernels()) return AA_ERR_LAUNCH;
+  char* ws = static_scratch_on_current_device();
+  if (!ws) return AA_ERR_LAUNCH;
+  hipStream_t st = (hipStream_t)stream;
+  auto up = [](int64_t x) { return (x + 255) / 256 * 256; };
+  const int64_t blocks = 2 * ((V + BM - 1) / BM);
+  TileArgs a{};
+  a.pk = (float*)ws;
+  a.ps = (float*)(ws + up(blocks * chunk * 4));
+  a.pu = (float*)(ws + 2 * up(blocks * chunk * 4));
+  a.xy = (float*)(ws + 3 * up(blocks * chunk * 4));
+  a.pitch_t = chunk;
+  a.c = kLog2e * inv_temperature;
+  a.inv_t = inv_temperature;
+  auto at = [](float* p, int64_t t0) { return p ? p + t0 : nullptr; };
+  for (int64_t t0 = 0; t0 < T; t0 += chunk) {
+    const int64_t n_tok = (T - t0) < chunk ? (T - t0) : chunk;
+    const uint16_t* hid = (const uint16_t*)hidden + t0 * H;
+    a.labels = labels + t0;
+    hipLaunchKernelGGL(k_label_logit, dim3((unsigned)((n_tok + 3) / 4)), dim3(256), 0, st, hid, (const uint16_t*)weight,
+                       labels + t0, (int)n_tok, (int)H, (int)V, a.xy);
+    launch_tiles<kModeStats>(st, weight, hid, n_tok, H, V, a);
+    hipLaunchKernelGGL(k_combine, dim3((unsigned)((n_tok + 63) / 64)), dim3(1024), 0, st, a.pk, a.ps, a.pu, a.xy, (int)blocks,
+                       a.pitch_t, (int)n_tok, a.c, logp + t0, at(entropy, t0), at(row_lse, t0), at(row_ez, t0));
+  }
+  return launch_status();
+}
+
 extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, int64_t H, int64_t V,
                              const int64_t* labels, float inv_temperature, const float* row_lse, const float* row_ez,
                              const float* g_logp, const float* g_entropy, const uint8_t* row_has_gradient,

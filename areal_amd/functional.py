@@ -782,6 +782,46 @@ def lm_head_logprobs_entropy(
     return _LmHeadLogprobsEntropy.apply(hidden.contiguous(), weight.contiguous(), y, float(temperature))
 
 
+def lm_head_logprobs_entropy_static(
+    hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0,
+    out: tuple[torch.Tensor, torch.Tensor] | None = None,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """Forward of ``lm_head_logprobs_entropy`` through ``aa_lmhead_fwd_static``: no workspace, nothing allocated by
+    the library (its softmax partials live in a 32 MiB device array of its own).  For callers that cannot allocate:
+    with ``out = (logp, entropy)`` given (float32 ``[T]``) this function allocates nothing either.  No autograd.
+    Calls that overlap on one GPU share that array and race; a vocabulary above ``aa_lmhead_fwd_static_max_vocab()``
+    is refused.  The reference has no counterpart."""
+    _require_gpu(hidden, "hidden")
+    if hidden.ndim != 2 or weight.ndim != 2 or hidden.shape[1] != weight.shape[1]:
+        raise ValueError(f"expected hidden [T, H] and weight [V, H], got {tuple(hidden.shape)} and {tuple(weight.shape)}")
+    T, H = hidden.shape
+    V = weight.shape[0]
+    if tuple(labels.shape) != (T,) or labels.dtype != torch.int64 or not labels.is_contiguous():
+        raise ValueError("labels must be a contiguous int64 tensor of shape [T]")
+    assert T > 0, "Input must have at least one token"
+    if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise TypeError("fused lm_head expects bf16 hidden states and weights")
+    if not hidden.is_contiguous() or not weight.is_contiguous():
+        raise ValueError("hidden and weight must be contiguous")
+    lib = N.load()
+    if V > lib.aa_lmhead_fwd_static_max_vocab():
+        raise ValueError(f"vocabulary {V} is beyond what aa_lmhead_fwd_static takes ({lib.aa_lmhead_fwd_static_max_vocab()})")
+    dev = hidden.device
+    if out is None:
+        out = (torch.empty(T, dtype=torch.float32, device=dev), torch.empty(T, dtype=torch.float32, device=dev))
+    logp, entropy = out
+    for t in out:
+        if t.dtype != torch.float32 or tuple(t.shape) != (T,) or not t.is_contiguous() or t.device != dev:
+            raise ValueError("out must hold two contiguous float32 tensors of shape [T] on the device of hidden")
+    with torch.cuda.device(dev):
+        N.check(
+            lib.aa_lmhead_fwd_static(_ptr(hidden), _ptr(weight), T, H, V, _ptr(labels), 1.0 / float(temperature), _ptr(logp),
+                                     _ptr(entropy), None, None, _stream(dev)),
+            "aa_lmhead_fwd_static",
+        )
+    return logp, entropy
+
+
 class _FusedLmHeadPpo(torch.autograd.Function):
     @staticmethod
     def forward(ctx, hidden, weight, labels, temperature, T_active, prox, adv, mask_eff, behave_w, params, n_valid,

@@ -612,6 +612,28 @@ int aa_lmhead_fwd(const void* hidden, const void* weight, int64_t T, int64_t H,
                   void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
+ * aa_lmhead_fwd for callers that cannot allocate device memory or bring a
+ * workspace (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc).  No counterpart in the reference.  Same arguments and
+ * results as aa_lmhead_fwd without the workspace: the softmax partials live in
+ * a device array of the library itself, aa_lmhead_fwd_static_scratch_bytes()
+ * = 32 MiB on every GPU the library has been used on, held until the process
+ * ends.  Tokens go through in passes of as many as fit that array (a multiple
+ * of 256; 2304 per pass at V = 151936); a vocabulary above
+ * aa_lmhead_fwd_static_max_vocab() (1 398 016), for which not even 256 tokens
+ * fit, is refused with AA_ERR_UNSUPPORTED.  The call allocates and frees
+ * nothing.  All calls on one GPU share the array: calls that overlap on one GPU
+ * (two streams, two host threads) race and must be serialised by the caller;
+ * nothing in the array needs clearing between calls.
+ */
+int aa_lmhead_fwd_static(const void* hidden, const void* weight, int64_t T,
+                         int64_t H, int64_t V, const int64_t* labels,
+                         float inv_temperature, float* logp, float* entropy,
+                         float* row_lse, float* row_ez, void* stream);
+int64_t aa_lmhead_fwd_static_scratch_bytes(void);
+int64_t aa_lmhead_fwd_static_max_vocab(void);
+
+/*
  * Backward of aa_lmhead_fwd: d_hidden [T, H] bf16 and d_weight [V, H]
  * (overwritten), given g_logp and optional g_entropy.  d_weight_dtype is
  * AA_F32 or AA_BF16; either way the sum over tokens is accumulated in fp32
