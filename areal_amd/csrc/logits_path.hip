@@ -178,13 +178,18 @@ struct GradCoef {
   int label;  // -1 = none
 };
 
+// A + B x.  With B == 0 (no gradient flows through the entropy) the product is left out, so that a logit of -inf
+// (a masked vocabulary entry) gets the gradient 0 that autograd gives it and not 0 * inf.  With B != 0 such a logit
+// has a NaN gradient in the reference as well (the entropy itself is NaN there).
+__device__ __forceinline__ float grad_weight(const GradCoef& g, float x) { return g.B == 0.f ? g.A : fmaf(g.B, x, g.A); }
+
 template <int DT, int NT>
 __device__ __forceinline__ void row_grad_generic(const void* row, void* out, int V, bool vec_ok, const GradCoef& g) {
   const RowSplit sp = split_row<DT>(row, V, vec_ok);
   const int tid = threadIdx.x;
   auto one = [&](int j) {
     const float x = Elem<DT>::load1(row, j);
-    float o = fast_exp2(fmaf(x, g.c, -g.lse2)) * fmaf(g.B, x, g.A);
+    float o = fast_exp2(fmaf(x, g.c, -g.lse2)) * grad_weight(g, x);
     if (j == g.label) o += g.lab_add;
     Elem<DT>::store1(out, j, o);
   };
@@ -194,7 +199,7 @@ __device__ __forceinline__ void row_grad_generic(const void* row, void* out, int
     float x[8], o[8];
     load8<DT>(row, e0, x);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) o[i] = fast_exp2(fmaf(x[i], g.c, -g.lse2)) * fmaf(g.B, x[i], g.A);
+    for (int i = 0; i < 8; ++i) o[i] = fast_exp2(fmaf(x[i], g.c, -g.lse2)) * grad_weight(g, x[i]);
     if ((unsigned)(g.label - e0) < 8u) {
 #pragma unroll
       for (int i = 0; i < 8; ++i)

@@ -132,10 +132,12 @@ def compute_advantages(
         old_logp = torch.roll(data["logprobs"], shifts=-1, dims=-1)          # :188
         if not use_decoupled_loss:
             data["prox_logp"] = old_logp
-    old_logp = old_logp * loss_mask                                           # :195-196
+    # in place, as the reference does (:192-196): data["prox_logp"] (when it is this tensor) and data["ref_logp"]
+    # come out masked as well
+    old_logp.mul_(loss_mask)
     ref_logp = data.get("ref_logp")
     if ref_logp is not None:
-        ref_logp = ref_logp * loss_mask
+        ref_logp.mul_(loss_mask)
     seqlens = data["attention_mask"].sum(-1).long()                           # :199-201
     rewards, kl_rewards = kl_regularized_rewards(old_logp, ref_logp, loss_mask, seqlens, reward_score, kl_ctl,
                                                  kl_estimator, mask_no_eos_with_zero)

@@ -12,11 +12,13 @@ One "step" is one pass of the hot path over one synthetic packed micro-batch tha
   to fp32 first (8 * V per token).  The line also carries ``sft_loss_same_logits``: the supervised loss on the same
   logits, fused in one pass against the log-prob op followed by the loss and a separate backward pass.
 * fused lm_head workloads (cfg2, cfg3, cfg4): ``fused_lm_head_ppo_loss(hidden, W, labels, ...)`` followed by
-  ``loss.backward()``: lm_head, log-prob / entropy, PPO loss and the gradients d(hidden), d(W), token chunk by
-  token chunk, the full [T, V] logits never in memory.  Roofline: bf16 MFMA.  Algorithmic flops: 2 T V H for the
-  logits of every token + 4 T_grad V H for the two gradient GEMMs over the tokens that have a gradient (masked
-  tokens have none and are left out; ``--dense-backward`` multiplies their zero rows through like the reference's
-  autograd, 6 T V H).  ``roofline.dense_equivalent_tflops`` quotes the same time against 6 T V H.
+  ``loss.backward()``: lm_head, log-prob / entropy, PPO loss and the gradients d(hidden), d(W) on this library's own
+  bf16 MFMA tile GEMM; the forward writes no logits.  Roofline: bf16 MFMA, from HIP events around every step of the
+  same timed loop that gives ``ms_per_step``.  ``needed_flops_per_step``: 2 T V H for the logits of every token +
+  4 T_grad V H for the two gradient GEMMs over the tokens that have a gradient (masked tokens have none and are left
+  out; ``--dense-backward`` multiplies their zero rows through like the reference's autograd).  With
+  ``--lmhead-backward recompute`` the backward forms the logits of those tokens a second time (2 T_grad V H more
+  flops are executed; they are not counted as needed).  ``flops_per_step_6TVH`` is the dense figure 6 T V H.
 
 * adv: the advantage pipeline that precedes the loss (not one of the headline configurations): GAE reverse scan plus batch
   normalisation over a padded [512, 4096] batch.  Roofline: HBM, 20 bytes per token for the scan (rewards, values,
@@ -30,9 +32,12 @@ One "step" is one pass of the hot path over one synthetic packed micro-batch tha
 Prints ONE JSON line.  Besides the whole-step throughput it carries
   roofline      of the dominant kernel(s), timed with HIP events on the launch stream;
   cpu_baseline  the CPU oracle (a PyTorch restatement of the reference path) timed on this machine's host cores on a
-                bounded token sample of the same workload;
+                bounded token sample of the same workload (three windows: first, middle and last tokens);
   parity        the GPU result checked against that oracle on the same sample;
-  fused_lm_head (default run only) the same figures for the cfg2 workload, so that one run reports both paths.
+and, in the default run only (every GPU timing is taken before the first CPU baseline starts):
+  configs1_cut_to_32k_tokens  the cfg1 sequences cut at 32 768 tokens;
+  logits_config0              the cfg0 workload with its own roofline, and the plain copy kernel on the same buffers;
+  fused_lm_head               the same figures for the cfg2 workload, so that one run reports both paths.
 """
 from __future__ import annotations
 
@@ -107,6 +112,20 @@ def ppo_kwargs(case):
 def cosine(a, b) -> float:
     a, b = a.double().reshape(-1), b.double().reshape(-1)
     return float(a @ b / (a.norm() * b.norm()))
+
+
+def sample_windows(n_total: int, n_sample: int):
+    """Token indices of the parity / CPU sample: three equal windows, the first, the middle and the last tokens of the
+    workload (sorted, without repeats), and a description of them."""
+    import torch
+
+    n = min(n_sample, n_total)
+    w = n // 3
+    sizes = [w, w, n - 2 * w]
+    starts = [0, (n_total - sizes[1]) // 2, n_total - sizes[2]]
+    idx = torch.unique(torch.cat([torch.arange(a, a + k) for a, k in zip(starts, sizes)]))
+    desc = ", ".join(f"{a}..{a + k - 1}" for a, k in zip(starts, sizes) if k > 0)
+    return idx, desc
 
 
 def time_events(launch, iters: int, stream):
@@ -202,45 +221,63 @@ def time_fused_logits_kernel(case, kw, cfg, iters: int):
     return time_events(launch, iters, stream)
 
 
-def logits_cpu_baseline_and_parity(case, kw, cfg, n_tokens: int, iters: int):
-    """Oracle fwd+bwd on the first ``n_tokens`` tokens (host cores), and the GPU path checked on the same slice."""
+def logits_gpu_sample(case, kw, cfg, n_tokens: int):
+    """The GPU path on the sample tokens (see sample_windows), with everything the CPU phase needs copied to the host:
+    the workload itself can be freed before the CPU baseline runs."""
     import torch
 
     import areal_amd
-    import oracle
 
-    n = min(n_tokens, case.n_tokens)
-    sl = slice(0, n)
-    cpu = lambda t: t[sl].cpu()
-    args = (cpu(case.logits), cpu(case.labels), cpu(case.prox_logp), cpu(case.old_logp), cpu(case.advantages))
+    idx, desc = sample_windows(case.n_tokens, n_tokens)
+    n = int(idx.numel())
+    idx_d = idx.to(case.logits.device)
+    take = lambda t: t[idx_d]
     cu = torch.tensor([0, n], dtype=torch.int32)  # token-level options only: segments do not matter here
-    okw = dict(kw, loss_mask=cpu(case.loss_mask), rejection_sampling_cfg=cfg, cu_seqlens=cu,
-               temperature=case.temperature)
-    threads = torch.get_num_threads()
-    oracle.logits_ppo_step(*args, **okw)  # warm-up
-    t0 = time.perf_counter()
-    for _ in range(iters):
-        w_loss, w_stat, w_grad = oracle.logits_ppo_step(*args, **okw)
-    dt = (time.perf_counter() - t0) / iters
-
-    x = case.logits[sl].detach().clone().requires_grad_(True)
+    x = take(case.logits).detach().clone().requires_grad_(True)
     loss, stat = areal_amd.fused_logprobs_ppo_loss(
-        x, case.labels[sl], case.prox_logp[sl], case.old_logp[sl], case.advantages[sl], loss_mask=case.loss_mask[sl],
-        rejection_sampling=cfg, cu_seqlens=cu.to(x.device), temperature=case.temperature, **kw,
+        x, take(case.labels), take(case.prox_logp), take(case.old_logp), take(case.advantages),
+        loss_mask=take(case.loss_mask), rejection_sampling=cfg, cu_seqlens=cu.to(x.device),
+        temperature=case.temperature, **kw,
     )
     loss.backward()
     torch.cuda.synchronize()
+    cpu = lambda t: take(t).cpu()
+    return dict(
+        n=n, windows=desc, cu=cu, kw=kw, cfg=cfg, temperature=case.temperature,
+        args=(x.detach().cpu(), cpu(case.labels), cpu(case.prox_logp), cpu(case.old_logp), cpu(case.advantages)),
+        loss_mask=cpu(case.loss_mask),
+        gpu=dict(loss=float(loss.detach()), logprobs=stat["logprobs"].cpu(), clip_mask=stat["clip_mask"].cpu(),
+                 grad=x.grad.cpu()),
+    )
+
+
+def logits_cpu_phase(sample, iters: int):
+    """Oracle fwd+bwd on the sample tokens (host cores), and the GPU results of logits_gpu_sample checked against it."""
+    import torch
+
+    import oracle
+
+    n, g = sample["n"], sample["gpu"]
+    okw = dict(sample["kw"], loss_mask=sample["loss_mask"], rejection_sampling_cfg=sample["cfg"], cu_seqlens=sample["cu"],
+               temperature=sample["temperature"])
+    threads = torch.get_num_threads()
+    oracle.logits_ppo_step(*sample["args"], **okw)  # warm-up
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        w_loss, w_stat, w_grad = oracle.logits_ppo_step(*sample["args"], **okw)
+    dt = (time.perf_counter() - t0) / iters
     parity = dict(
-        tokens=n,
-        logp_max_abs_err=float((stat["logprobs"].cpu() - w_stat["logprobs"]).abs().max()),
-        loss_rel_err=abs(float(loss.detach()) - float(w_loss)) / max(abs(float(w_loss)), 1e-12),
-        grad_cosine=cosine(x.grad.cpu(), w_grad),
-        masks_equal=bool(torch.equal(stat["clip_mask"].cpu(), w_stat["clip_mask"])),
+        tokens=n, token_windows=sample["windows"],
+        logp_max_abs_err=float((g["logprobs"] - w_stat["logprobs"]).abs().max()),
+        loss_rel_err=abs(g["loss"] - float(w_loss)) / max(abs(float(w_loss)), 1e-12),
+        grad_cosine=cosine(g["grad"], w_grad),
+        grad_norm_ratio=float(g["grad"].double().norm() / w_grad.double().norm()),
+        masks_equal=bool(torch.equal(g["clip_mask"], w_stat["clip_mask"])),
     )
     baseline = dict(
         value=n / dt, unit="tokens/s", cores=threads, kind="port",
-        sample=f"first {n} tokens of the workload, {iters} timed fwd+bwd passes of the PyTorch CPU oracle "
-               f"(chunked fp32 log_softmax + gather + entropy + PPO loss + autograd to bf16 d(logits))",
+        sample=f"{n} tokens of the workload (tokens {sample['windows']}), {iters} timed fwd+bwd passes of the PyTorch "
+               f"CPU oracle (chunked fp32 log_softmax + gather + entropy + PPO loss + autograd to bf16 d(logits))",
     )
     return baseline, parity
 
@@ -278,10 +315,30 @@ def time_sft_steps(case, iters: int):
     return out
 
 
-def bench_logits(args, dev):
+def time_copy_kernel(src, dst, iters: int):
+    """The plain copy kernel (aa_copy_bytes: 16 bytes per lane, nothing else) from ``src`` to ``dst``: what this chip
+    delivers for a read-once / write-once stream over buffers of this very size."""
     import torch
 
-    case, desc = build_logits_case(args.workload, args.seed, dev)
+    from areal_amd import _native as N
+    from areal_amd import functional as F
+
+    lib = N.load()
+    nbytes = src.numel() * src.element_size()
+    stream = torch.cuda.current_stream(src.device)
+    st = C.c_void_p(stream.cuda_stream)
+    ms, ms_min = time_events(lambda: N.check(lib.aa_copy_bytes(F._ptr(src), F._ptr(dst), nbytes, st), "aa_copy_bytes"),
+                             iters, stream)
+    gbs = 2.0 * nbytes / (ms * 1e-3) / 1e9
+    return dict(kernel="k_copy16 (aa_copy_bytes)", bytes_read=nbytes, bytes_written=nbytes, avg_kernel_ms=ms,
+                min_kernel_ms=ms_min, achieved=gbs, unit="GB/s", frac=gbs / HBM_PEAK_GBS)
+
+
+def bench_logits(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: int, with_sft: bool = True):
+    """GPU part of a logits workload.  Returns the result line and the sample for the CPU phase (None: no CPU phase)."""
+    import torch
+
+    case, desc = build_logits_case(workload, args.seed, dev)
     kw, cfg = ppo_kwargs(case)
     T, V = case.logits.shape
     f32 = args.logits_dtype == "f32"
@@ -289,17 +346,17 @@ def bench_logits(args, dev):
         case.logits = case.logits.float()
         desc += "; logits cast to fp32"
     case.logits.requires_grad_(True)
-    run_logits_steps(case, args.warmup, kw, cfg)
+    run_logits_steps(case, warmup, kw, cfg)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    loss = run_logits_steps(case, args.steps, kw, cfg)
+    loss = run_logits_steps(case, steps, kw, cfg)
     torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    ms_per_step = (time.perf_counter() - t0) / steps * 1e3
     assert bool(torch.isfinite(loss)), "loss is not finite"
 
     case.logits.grad = None
     case.logits.requires_grad_(False)
-    k_ms, k_min_ms = time_fused_logits_kernel(case, kw, cfg, max(args.steps, 10))
+    k_ms, k_min_ms = time_fused_logits_kernel(case, kw, cfg, max(steps, 10))
     alg_bytes = (8.0 if f32 else 4.0) * T * V
     achieved = alg_bytes / (k_ms * 1e-3) / 1e9
     roofline = dict(
@@ -314,7 +371,7 @@ def bench_logits(args, dev):
     )
     out = dict(
         metric=METRIC, value=T / (ms_per_step * 1e-3), unit="tokens/s",
-        n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=ms_per_step, higher_is_better=True,
+        n_gpus=1, steps=steps, warmup=warmup, ms_per_step=ms_per_step, higher_is_better=True,
         scaling="weak", vs_baseline=None, dtype="f32" if f32 else "bf16", data="synthetic",
         config=dict(workload=f"{case.name}: {desc}", tokens=T, vocab=V, sequences=int(case.cu_seqlens.numel() - 1),
                     accumulate="f32", path="logits (fused fwd + PPO loss + bwd, one launch)"),
@@ -322,22 +379,30 @@ def bench_logits(args, dev):
     )
     if cfg is not None:
         out["config"]["importance_weight_cap"] = f"{cfg.level} {cfg.metric} <= {cfg.upper}, action={cfg.action}"
-    out["sft_loss_same_logits"] = time_sft_steps(case, max(args.steps // 2, 3))
+    if with_sft:
+        out["sft_loss_same_logits"] = time_sft_steps(case, max(steps // 2, 3))
+    # the measured ceiling of a read-once / write-once kernel on buffers of this size
+    dst = torch.empty_like(case.logits)
+    out["copy_same_buffers"] = time_copy_kernel(case.logits, dst, max(steps, 10))
+    out["roofline"]["frac_of_copy_kernel"] = achieved / out["copy_same_buffers"]["achieved"]
     if args.copy_launches > 0:
         from areal_amd import _native as N
         from areal_amd import functional as F
 
-        dst = torch.empty_like(case.logits)
         nbytes = case.logits.numel() * case.logits.element_size()
         for _ in range(args.copy_launches):
             N.check(N.load().aa_copy_bytes(F._ptr(case.logits), F._ptr(dst), nbytes, F._stream(dev)), "aa_copy_bytes")
         torch.cuda.synchronize()
         out["copy_calibration"] = dict(kernel="k_copy16 (aa_copy_bytes)", bytes_read=nbytes, bytes_written=nbytes,
                                        launches=args.copy_launches)
-    if args.cpu_tokens > 0:
-        baseline, parity = logits_cpu_baseline_and_parity(case, kw, cfg, args.cpu_tokens, args.cpu_iters)
-        out["cpu_baseline"] = baseline
-        out["parity"] = parity
+    del dst
+    sample = logits_gpu_sample(case, kw, cfg, cpu_tokens) if cpu_tokens > 0 else None
+    return out, sample
+
+
+def finish_with_cpu_phase(out, sample, cpu_phase, iters: int):
+    if sample is not None:
+        out["cpu_baseline"], out["parity"] = cpu_phase(sample, iters)
     return out
 
 
@@ -369,29 +434,67 @@ def build_fused_case(name: str, seed: int, device):
 DENSE_BACKWARD = False  # set from --dense-backward
 BACKWARD_MODE = 1  # aa_lmhead_backward_mode: 1 carry, 0 recompute (set from --lmhead-backward)
 NO_FORWARD_OF_MASKED = False  # set from --no-forward-of-masked
+MODE_NAMES = {1: "carry", 0: "recompute"}
+
+# HBM bytes per step of aa_lmhead_ppo_fused at configs[2], all its kernels together: rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (one run each) summed over the kernels of one step, each scaled by what the same counter reads for the
+# plain copy kernel of known size (profiles/lmhead_step_cfg2_hbm_traffic.md).  Other workloads: not measured.
+LMHEAD_MEASURED_HBM_BYTES = {("cfg2", "carry"): None, ("cfg2", "recompute"): None}
 
 
-def run_fused_steps(case, n, kw, cfg):
+def lmhead_compulsory_bytes(T: int, kept: int, H: int, V: int, mode: str, chunk: int) -> dict:
+    """HBM bytes a step cannot avoid, kernel by kernel: every operand of a kernel read once, every result written
+    once (bf16 = 2 bytes).  ``kept`` = tokens with a gradient.  What the counters read above this is re-fetching."""
+    n_chunks = -(-T // chunk)
+    blocks = 2 * -(-V // 256)
+    w_bytes = 2.0 * V * H
+    partials = 12.0 * blocks * T
+    panel = 2.0 * kept * V
+    out = dict(
+        forward_tiles=n_chunks * w_bytes + 2.0 * T * H + partials + (panel if mode == "carry" else 0.0),
+        merge_partials=partials,
+        panel_scale=2.0 * panel if mode == "carry" else 0.0,
+        recompute_tiles=(n_chunks * w_bytes + 2.0 * kept * H + panel) if mode == "recompute" else 0.0,
+        d_hidden_gemm=panel + n_chunks * w_bytes + 2.0 * kept * H,
+        # d_weight: written once in bf16 when one chunk holds every token, else accumulated in fp32 chunk by chunk
+        d_weight_gemm=panel + 2.0 * kept * H + (w_bytes if n_chunks == 1 else (2 * n_chunks - 1) * 2.0 * w_bytes + 3.0 * w_bytes),
+    )
+    out["total"] = sum(out.values())
+    out["logits_panel_written"] = panel
+    return out
+
+
+def run_fused_steps(case, n, kw, cfg, events=None):
+    """``n`` steps; with ``events`` (a list) a pair of HIP events on the launch stream brackets every step."""
+    import torch
+
     import areal_amd
 
     h, w = case.hidden, case.weight
+    stream = torch.cuda.current_stream(h.device)
     loss = None
     for _ in range(n):
         h.grad = None
         w.grad = None
+        if events is not None:
+            ev = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+            ev[0].record(stream)
         loss, _ = areal_amd.fused_lm_head_ppo_loss(
             h, w, case.labels, case.prox_logp, case.old_logp, case.advantages, loss_mask=case.loss_mask,
             rejection_sampling=cfg, cu_seqlens=case.cu_seqlens, temperature=case.temperature,
             skip_masked_tokens=not DENSE_BACKWARD, forward_masked_tokens=not NO_FORWARD_OF_MASKED,
-            backward="carry" if BACKWARD_MODE == 1 else "recompute", **kw,
+            backward=MODE_NAMES[BACKWARD_MODE], **kw,
         )
         loss.backward()
+        if events is not None:
+            ev[1].record(stream)
+            events.append(ev)
     return loss
 
 
-def time_lmhead_step(case, kw, cfg, iters: int, skip_masked: bool):
-    """Duration of aa_lmhead_ppo_fused (every kernel it enqueues), HIP events on the launch stream, and the number
-    of tokens that go through the gradient GEMMs."""
+def time_lmhead_step(case, kw, cfg, iters: int, skip_masked: bool, mode: int):
+    """Duration of aa_lmhead_ppo_fused (every kernel it enqueues) called through the C ABI with pre-allocated outputs,
+    HIP events on the launch stream, and the number of tokens that go through the gradient GEMMs."""
     import torch
 
     from areal_amd import _native as N
@@ -428,7 +531,7 @@ def time_lmhead_step(case, kw, cfg, iters: int, skip_masked: bool):
             lib.aa_lmhead_ppo_fused(
                 F._ptr(case.hidden), F._ptr(case.weight), T, H, V, F._ptr(case.labels), 1.0 / case.temperature, T,
                 F._ptr(prox), F._ptr(adv), F._ptr(mask_eff), F._ptr(w), C.byref(params), F._ptr(counts), None, kept,
-                BACKWARD_MODE, F._ptr(logp), F._ptr(ent), F._ptr(sl), F._ptr(ratio), F._ptr(flags), F._ptr(dh), F._ptr(dw),
+                mode, F._ptr(logp), F._ptr(ent), F._ptr(sl), F._ptr(ratio), F._ptr(flags), F._ptr(dh), F._ptr(dw),
                 N.AA_BF16, F._ptr(ws), ws.numel(), C.c_void_p(stream.cuda_stream),
             ),
             "aa_lmhead_ppo_fused",
@@ -439,7 +542,7 @@ def time_lmhead_step(case, kw, cfg, iters: int, skip_masked: bool):
 
 def time_lmhead_op(case, iters: int):
     """Durations of aa_lmhead_fwd and aa_lmhead_bwd, the stand-alone differentiable op (its backward forms the
-    logits of each chunk again), HIP events on the launch stream."""
+    logits of the tokens with a gradient again), HIP events on the launch stream."""
     import torch
 
     from areal_amd import _native as N
@@ -464,12 +567,12 @@ def time_lmhead_op(case, iters: int):
                                   F._ptr(logp), F._ptr(ent), F._ptr(lse), F._ptr(ez), F._ptr(ws), ws.numel(), st),
                 "aa_lmhead_fwd")
 
-    has_grad, kept = None, None
+    has_grad, kept, kept_tokens = None, None, T
     if not DENSE_BACKWARD:  # rows with a zero upstream gradient stay out of the gradient GEMMs
         has_grad = (g != 0).view(torch.uint8)
         chunk = int(lib.aa_lmhead_chunk_tokens())
         per_chunk = [int(has_grad[i:i + chunk].ne(0).sum()) for i in range(0, T, chunk)]
-        kept = (C.c_int64 * len(per_chunk))(*per_chunk)
+        kept, kept_tokens = (C.c_int64 * len(per_chunk))(*per_chunk), sum(per_chunk)
 
     def bwd():
         N.check(lib.aa_lmhead_bwd(F._ptr(case.hidden), F._ptr(case.weight), T, H, V, F._ptr(case.labels), inv_t,
@@ -478,35 +581,56 @@ def time_lmhead_op(case, iters: int):
 
     f_ms, _ = time_events(fwd, iters, stream)
     b_ms, _ = time_events(bwd, iters, stream)
-    return f_ms, b_ms
+    return f_ms, b_ms, kept_tokens
 
 
-def fused_cpu_baseline_and_parity(case, kw, cfg, n_tokens: int, iters: int):
-    """Oracle (fp32 matmul + logits path + PPO loss + autograd) on the first ``n_tokens`` tokens against the full
-    weight matrix, and the GPU path checked on the same slice."""
+def fused_gpu_sample(case, kw, cfg, n_tokens: int):
+    """The GPU step on the sample tokens (see sample_windows) against the full weight matrix, with everything the CPU
+    phase needs copied to the host."""
     import torch
 
     import areal_amd
+
+    idx, desc = sample_windows(case.n_tokens, n_tokens)
+    n = int(idx.numel())
+    idx_d = idx.to(case.hidden.device)
+    take = lambda t: t[idx_d]
+    cu = torch.tensor([0, n], dtype=torch.int32)
+    h = take(case.hidden).detach().clone().requires_grad_(True)
+    w = case.weight.detach().clone().requires_grad_(True)
+    loss, stat = areal_amd.fused_lm_head_ppo_loss(
+        h, w, take(case.labels), take(case.prox_logp), take(case.old_logp), take(case.advantages),
+        loss_mask=take(case.loss_mask), rejection_sampling=cfg, cu_seqlens=cu.to(h.device),
+        temperature=case.temperature, backward=MODE_NAMES[BACKWARD_MODE], **kw)
+    loss.backward()
+    torch.cuda.synchronize()
+    cpu = lambda t: take(t).cpu()
+    return dict(
+        n=n, windows=desc, cu=cu, kw=kw, cfg=cfg, temperature=case.temperature,
+        hidden=h.detach().cpu().float(), weight=case.weight.cpu().float(), labels=cpu(case.labels),
+        prox=cpu(case.prox_logp), old=cpu(case.old_logp), adv=cpu(case.advantages), mask=cpu(case.loss_mask),
+        gpu=dict(loss=float(loss.detach()), logprobs=stat["logprobs"].detach().cpu(), d_hidden=h.grad.cpu(),
+                 d_weight=w.grad.cpu()),
+    )
+
+
+def fused_cpu_phase(sample, iters: int):
+    """Oracle (fp32 matmul + logits path + PPO loss + autograd) on the sample tokens against the full weight matrix
+    (host cores), and the GPU results of fused_gpu_sample checked against it."""
+    import torch
+
     import oracle
 
-    n = min(n_tokens, case.n_tokens)
-    first = int(torch.nonzero(case.loss_mask)[0]) if bool(case.loss_mask.any()) else 0
-    start = max(0, min(first - n // 4, case.n_tokens - n))  # a window that holds masked and unmasked tokens
-    sl = slice(start, start + n)
-    cpu = lambda t: t[sl].cpu()
-    hid, lab = cpu(case.hidden).float(), cpu(case.labels)
-    w_cpu = case.weight.cpu().float()
-    prox, old, adv, mask = cpu(case.prox_logp), cpu(case.old_logp), cpu(case.advantages), cpu(case.loss_mask)
-    cu = torch.tensor([0, n], dtype=torch.int32)
+    n, g = sample["n"], sample["gpu"]
     threads = torch.get_num_threads()
 
     def oracle_step():
-        h = hid.clone().requires_grad_(True)
-        w = w_cpu.clone().requires_grad_(True)
+        h = sample["hidden"].clone().requires_grad_(True)
+        w = sample["weight"].clone().requires_grad_(True)
         logits = oracle.lmhead_logits(h, w)
-        lp, _ent = oracle.logprobs_entropy(logits, lab, case.temperature)
-        loss, _stat = oracle.ppo_actor_loss(lp, prox, old, adv, loss_mask=mask.bool(), rejection_sampling_cfg=cfg,
-                                            cu_seqlens=cu, **kw)
+        lp, _ent = oracle.logprobs_entropy(logits, sample["labels"], sample["temperature"])
+        loss, _stat = oracle.ppo_actor_loss(lp, sample["prox"], sample["old"], sample["adv"], loss_mask=sample["mask"].bool(),
+                                            rejection_sampling_cfg=sample["cfg"], cu_seqlens=sample["cu"], **sample["kw"])
         loss.backward()
         return loss.detach(), lp.detach(), h.grad, w.grad
 
@@ -515,34 +639,28 @@ def fused_cpu_baseline_and_parity(case, kw, cfg, n_tokens: int, iters: int):
     for _ in range(iters):
         w_loss, w_lp, w_dh, w_dw = oracle_step()
     dt = (time.perf_counter() - t0) / iters
-
-    h = case.hidden[sl].detach().clone().requires_grad_(True)
-    w = case.weight.detach().clone().requires_grad_(True)
-    loss, stat = areal_amd.fused_lm_head_ppo_loss(
-        h, w, case.labels[sl], case.prox_logp[sl], case.old_logp[sl], case.advantages[sl],
-        loss_mask=case.loss_mask[sl], rejection_sampling=cfg, cu_seqlens=cu.to(h.device),
-        temperature=case.temperature, **kw)
-    lp = stat["logprobs"]
-    loss.backward()
-    torch.cuda.synchronize()
     parity = dict(
-        tokens=n, first_token=start,
-        logp_max_abs_err=float((lp.detach().cpu() - w_lp).abs().max()),
-        loss_rel_err=abs(float(loss.detach()) - float(w_loss)) / max(abs(float(w_loss)), 1e-12),
-        d_hidden_cosine=cosine(h.grad.cpu(), w_dh),
-        d_weight_cosine=cosine(w.grad.cpu(), w_dw),
+        tokens=n, token_windows=sample["windows"], tokens_with_mask=int(sample["mask"].sum()),
+        logp_max_abs_err=float((g["logprobs"] - w_lp).abs().max()),
+        loss_rel_err=abs(g["loss"] - float(w_loss)) / max(abs(float(w_loss)), 1e-12),
+        d_hidden_cosine=cosine(g["d_hidden"], w_dh), d_weight_cosine=cosine(g["d_weight"], w_dw),
+        d_hidden_norm_ratio=float(g["d_hidden"].double().norm() / w_dh.double().norm()),
+        d_weight_norm_ratio=float(g["d_weight"].double().norm() / w_dw.double().norm()),
     )
     baseline = dict(
         value=n / dt, unit="tokens/s", cores=threads, kind="port",
-        sample=f"tokens {start}..{start + n - 1} of the workload against the full weight matrix, {iters} timed fwd+bwd passes of the "
-               f"PyTorch CPU oracle (fp32 hidden @ W.T rounded to bf16, log_softmax + gather + entropy, PPO loss, "
+        sample=f"{n} tokens of the workload (tokens {sample['windows']}) against the full weight matrix, {iters} timed "
+               f"fwd+bwd passes of the PyTorch CPU oracle (fp32 hidden @ W.T, log_softmax + gather + entropy, PPO loss, "
                f"autograd to d(hidden) and d(W))",
     )
     return baseline, parity
 
 
 def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: int):
+    """GPU part of a fused lm_head workload.  Returns the result line and the sample for the CPU phase."""
     import torch
+
+    from areal_amd import _native as N
 
     case, desc = build_fused_case(workload, args.seed, dev)
     kw, cfg = ppo_kwargs(case)
@@ -552,34 +670,54 @@ def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: i
     case.weight.requires_grad_(True)
     run_fused_steps(case, warmup, kw, cfg)
     torch.cuda.synchronize()
+    events = []
     t0 = time.perf_counter()
-    loss = run_fused_steps(case, steps, kw, cfg)
+    loss = run_fused_steps(case, steps, kw, cfg, events)
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) / steps * 1e3
     assert bool(torch.isfinite(loss)), "loss is not finite"
+    ev_ms = sorted(a.elapsed_time(b) for a, b in events)
+    ev_avg = sum(ev_ms) / len(ev_ms)
     case.hidden.grad = None
     case.weight.grad = None
     case.hidden.requires_grad_(False)
     case.weight.requires_grad_(False)
 
-    # at least 10 timed calls: with a handful, one call that meets a clock or power transition moves the mean by 20 %
-    k_ms, k_min_ms, kept_tokens = time_lmhead_step(case, kw, cfg, 10, not args.dense_backward)
-    f_ms, b_ms = time_lmhead_op(case, 3)
+    # the same step through the C ABI alone (outputs pre-allocated, no autograd), in both backward modes
+    mode_name = MODE_NAMES[BACKWARD_MODE]
+    chunk = int(N.load().aa_lmhead_chunk_tokens())
+    modes = {}
+    kept_tokens = T
+    for mode, name in ((1, "carry"), (0, "recompute")):
+        c_ms, c_min, kept_tokens = time_lmhead_step(case, kw, cfg, 10, not args.dense_backward, mode)
+        modes[name] = dict(avg_call_ms=c_ms, min_call_ms=c_min,
+                           executed_flops=(2.0 * T + (4.0 if mode == 1 else 6.0) * kept_tokens) * V * H,
+                           compulsory_hbm_bytes=lmhead_compulsory_bytes(T, kept_tokens, H, V, name, chunk),
+                           measured_hbm_bytes=LMHEAD_MEASURED_HBM_BYTES.get((workload, name)))
+    f_ms, b_ms, op_kept = time_lmhead_op(case, 5)
     # Flops the step needs: logits of every token (2 T V H) and the two gradient GEMMs over the tokens that have a
     # gradient (4 T_kept V H).  The reference's autograd runs them over all T tokens: 6 T V H.
-    dense_flops = 6.0 * T * V * H
-    alg_flops = 2.0 * T * V * H + 4.0 * kept_tokens * V * H
-    achieved = alg_flops / (k_ms * 1e-3) / 1e12
+    needed_flops = 2.0 * T * V * H + 4.0 * kept_tokens * V * H
+    achieved = needed_flops / (ev_avg * 1e-3) / 1e12
     roofline = dict(
-        bound="mfma", kernel="aa_lmhead_ppo_fused (per token chunk: hipBLASLt logits GEMM, k_fused_regs, k_transpose_bf16 copies, hipBLASLt d_hidden and d_weight GEMMs over the tokens with a gradient)",
+        bound="mfma",
+        kernel="every kernel of one fused_lm_head_ppo_loss(...) + backward() step: k_lmhead_tiles (logits tiles on the "
+               "library's bf16 MFMA tile GEMM, softmax partials per tile, " +
+               ("the un-normalised probabilities of the tokens with a gradient kept in bf16" if mode_name == "carry"
+                else "nothing else written") +
+               "), k_label_logit, k_combine / k_token_loss, " +
+               ("k_panel_scale" if mode_name == "carry" else "k_lmhead_tiles again for the tokens with a gradient") +
+               ", k_gemm_store twice (d_hidden, d_weight)",
         achieved=achieved, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s", frac=achieved / MFMA_BF16_PEAK_TFLOPS,
-        traffic=None, avg_call_ms=k_ms, min_call_ms=k_min_ms, algorithmic_flops_per_step=alg_flops,
-        tokens_with_gradient=kept_tokens, dense_flops_per_step=dense_flops,
-        dense_equivalent_tflops=dense_flops / (k_ms * 1e-3) / 1e12,
-        # the stand-alone differentiable op lm_head_logprobs_entropy, whose backward forms the logits again; its
-        # backward rate is quoted on the dense 4 T V H (rows with a zero upstream gradient are left out, as above)
+        traffic=LMHEAD_MEASURED_HBM_BYTES.get((workload, mode_name)),
+        timed="HIP events on the launch stream around each of the steps that ms_per_step is the wall-clock mean of",
+        avg_step_ms=ev_avg, min_step_ms=ev_ms[0], max_step_ms=ev_ms[-1],
+        needed_flops_per_step=needed_flops, flops_per_step_6TVH=6.0 * T * V * H, tokens_with_gradient=kept_tokens,
+        backward_mode=mode_name, backward_modes_through_c_abi=modes,
+        # the stand-alone differentiable op lm_head_logprobs_entropy: its forward writes softmax partials only, its
+        # backward forms the logits of the tokens with a gradient again (6 T_grad V H flops executed)
         standalone_op=dict(fwd_ms=f_ms, bwd_ms=b_ms, fwd_tflops=2.0 * T * V * H / (f_ms * 1e-3) / 1e12,
-                           bwd_dense_equivalent_tflops=4.0 * T * V * H / (b_ms * 1e-3) / 1e12),
+                           bwd_executed_tflops=6.0 * op_kept * V * H / (b_ms * 1e-3) / 1e12),
     )
     out = dict(
         metric=METRIC, value=T / (ms_per_step * 1e-3), unit="tokens/s",
@@ -587,17 +725,13 @@ def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: i
         scaling="weak", vs_baseline=None, dtype="bf16", data="synthetic",
         config=dict(workload=f"{case.name}: {desc}", tokens=T, hidden=H, vocab=V,
                     sequences=int(case.cu_seqlens.numel() - 1), accumulate="f32",
-                    path="lm_head + PPO loss step in token chunks (at most one chunk of logits in memory), fwd + bwd"),
+                    path=f"lm_head + PPO loss step, fwd + bwd (backward={mode_name}); the forward writes no logits"),
         roofline=roofline,
     )
     if NO_FORWARD_OF_MASKED:
-        out["config"]["path"] += "; NOT the reference's semantics: masked tokens skip the lm_head (value and " \
-                                 "ms_per_step only; roofline figures are those of the default call)"
-    if cpu_tokens > 0:
-        baseline, parity = fused_cpu_baseline_and_parity(case, kw, cfg, cpu_tokens, args.cpu_iters)
-        out["cpu_baseline"] = baseline
-        out["parity"] = parity
-    return out
+        out["config"]["path"] += "; NOT the reference's semantics: masked tokens skip the lm_head"
+    sample = fused_gpu_sample(case, kw, cfg, cpu_tokens) if cpu_tokens > 0 else None
+    return out, sample
 
 # ----------------------------------------------------------------------------------------------------------------
 # advantage pipeline
@@ -823,21 +957,31 @@ def main():
     elif args.workload in ADV_WORKLOADS:
         out = bench_adv(args, dev)
     elif args.workload in LOGITS_WORKLOADS:
-        out = bench_logits(args, dev)
+        out, sample = bench_logits(args, dev, args.workload, args.steps, args.warmup, args.cpu_tokens)
+        extra, fused_sample = None, None
         if args.workload == "cfg1" and not args.no_fused_extra and args.copy_launches == 0:
+            # Every GPU timing of the run comes first, the CPU baselines last.
             # configs[1] says "T = 32k" of a length distribution that draws about 130k tokens: the headline figures
             # are on the distribution as stated; the same sequences cut at 32 768 tokens are quoted beside them
             torch.cuda.empty_cache()
-            small = argparse.Namespace(**{**vars(args), "workload": "cfg1-32k", "cpu_tokens": 0})
-            cut = bench_logits(small, dev)
-            out["configs1_cut_to_32k_tokens"] = {k: cut[k] for k in ("value", "unit", "ms_per_step", "config", "roofline")}
+            keys = ("value", "unit", "ms_per_step", "steps", "warmup", "config", "roofline", "copy_same_buffers")
+            cut, _ = bench_logits(args, dev, "cfg1-32k", args.steps, args.warmup, 0, with_sft=False)
+            out["configs1_cut_to_32k_tokens"] = {k: cut[k] for k in keys}
             torch.cuda.empty_cache()
-            extra = bench_fused(args, dev, "cfg2", steps=min(args.steps, 5), warmup=min(args.warmup, 2),
-                                cpu_tokens=min(args.cpu_tokens, 384))
+            small, _ = bench_logits(args, dev, "cfg0", max(args.steps, 50), args.warmup, 0, with_sft=False)
+            out["logits_config0"] = {k: small[k] for k in keys}
+            torch.cuda.empty_cache()
+            extra, fused_sample = bench_fused(args, dev, "cfg2", args.steps, args.warmup, min(args.cpu_tokens, 384))
+            torch.cuda.empty_cache()
+        finish_with_cpu_phase(out, sample, logits_cpu_phase, args.cpu_iters)
+        if extra is not None:
+            finish_with_cpu_phase(extra, fused_sample, fused_cpu_phase, args.cpu_iters)
             keys = ("value", "unit", "ms_per_step", "steps", "warmup", "config", "roofline", "cpu_baseline", "parity")
             out["fused_lm_head"] = {k: extra[k] for k in keys if k in extra}
     else:
-        out = bench_fused(args, dev, args.workload, args.steps, args.warmup, min(args.cpu_tokens, 384))
+        out, sample = bench_fused(args, dev, args.workload, args.steps, args.warmup, min(args.cpu_tokens, 384))
+        torch.cuda.empty_cache()
+        finish_with_cpu_phase(out, sample, fused_cpu_phase, args.cpu_iters)
     # the two fractions the metric names, beside the throughput: of the HBM peak on the logits path, of the bf16 MFMA
     # peak on the fused lm_head path (whichever of the two this run measured)
     fractions = {}

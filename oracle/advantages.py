@@ -179,8 +179,8 @@ def compute_advantages(data, kl_ctl=0.0, kl_estimator="k1", discount=1.0, gae_la
     ref_logp = data.get("ref_logp")
     if ref_logp is None:
         ref_logp = torch.zeros_like(old_logp)
-    ref_logp = ref_logp * loss_mask
-    old_logp = old_logp * loss_mask
+    ref_logp *= loss_mask  # in place (actor.py:194-195): data["ref_logp"] and, where it is this tensor,
+    old_logp *= loss_mask  # data["prox_logp"] come out masked too
     attn_mask = data["attention_mask"]
     seqlens = attn_mask.sum(-1).long()
     seq_no_eos_mask = seqlens == attn_mask.shape[1]

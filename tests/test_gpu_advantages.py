@@ -207,8 +207,16 @@ def test_compute_advantages_matches_oracle(device, case):
     for key in ("advantages", "returns", "kl_rewards", "tot_rewards", "loss_mask", "logprobs"):
         scale = float(want[key].abs().max()) + 1.0
         assert float((got[key].cpu() - want[key]).abs().max()) < 2e-5 * scale, key
+    rolled_mask = torch.roll(lm.float(), shifts=-1, dims=-1)
     if case != "critic_kl":
+        # the reference masks old_logp in place (actor.py:195), and data["prox_logp"] is that very tensor
         assert torch.allclose(got["prox_logp"].cpu(), want["prox_logp"])
+        assert got["prox_logp"] is got["logprobs"]
+        assert float((got["prox_logp"].cpu() * (1 - rolled_mask)).abs().max()) == 0.0
+    else:
+        # ... and data["ref_logp"] likewise (actor.py:194)
+        assert torch.equal(want["ref_logp"], data["ref_logp"] * rolled_mask)
+        assert torch.equal(got["ref_logp"].cpu(), want["ref_logp"])
 
 
 def test_overlong_penalty_matches_oracle_and_updates_in_place(device):

@@ -8,7 +8,7 @@ import torch
 import areal_amd
 import oracle
 from areal_amd import RejectionSamplingConfig, engine_glue, synth
-from helpers import cosine
+from helpers import assert_same_magnitude, cosine
 
 pytestmark = pytest.mark.gpu
 
@@ -57,6 +57,7 @@ def _compare(case, got, want, pad=0):
     assert float(g_loss) == pytest.approx(float(w_loss), rel=1e-3, abs=1e-7)                  # stated
     assert g_grad.dtype == case.logits.dtype and g_grad.shape == case.logits.shape
     assert cosine(g_grad.cpu(), w_grad) > 0.9999                                              # stated
+    assert_same_magnitude(g_grad.cpu(), w_grad, what="d_logits")   # cosine is blind to a wrong scale
     for k in ("clip_mask", "dual_clip_mask"):
         assert torch.equal(g_stat[k].cpu(), w_stat[k]), k
     for k in ("loss", "importance_weight", "approx_kl"):
@@ -177,11 +178,13 @@ def test_fused_equals_unfused_kernels_and_sequence_level_falls_back(device):
     assert float(f_loss) == pytest.approx(float(loss.detach()), rel=1e-6)
     assert float((f_stat["logprobs"] - lp.detach()).abs().max()) < 1e-5
     assert cosine(f_grad, x.grad) > 0.999999
+    assert_same_magnitude(f_grad, x.grad, what="fused vs unfused d_logits")
     # GSPO: per-token loss depends on the whole sequence -> unfused kernels, same API
     s_got = _fused_step(case, importance_sampling_level="sequence")
     s_want = _oracle_step(case, importance_sampling_level="sequence")
     assert float(s_got[0]) == pytest.approx(float(s_want[0]), rel=1e-3, abs=1e-7)
     assert cosine(s_got[2].cpu(), s_want[2]) > 0.9999
+    assert_same_magnitude(s_got[2].cpu(), s_want[2], what="sequence-level d_logits")
 
 
 def test_backward_with_upstream_factor(device):
@@ -237,6 +240,7 @@ def test_engine_contract_roll_pad_and_scale(device):
     for loss, grad, stat in results:
         assert loss == pytest.approx(float(w_loss), rel=1e-3)
         assert cosine(grad.cpu(), w_grad) > 0.9999
+        assert_same_magnitude(grad.cpu(), w_grad, what="d_logits")
         assert float(grad[n:].float().abs().max()) == 0.0
         assert stat["logprobs"].shape == (n,)
     # an all-masked micro-batch keeps the graph alive and contributes nothing
@@ -284,6 +288,68 @@ def test_full_size_properties_config1(device):
         loss_scale=0.5,
     )
     assert float(loss_h.detach()) == pytest.approx(0.5 * float(l1.detach()), rel=1e-6)
+
+
+def test_full_size_config1_properties_and_sampled_parity(device):
+    """The benchmark's own workload, all 64 sequences as drawn (about 122 000 tokens, 37 GB of logits and as much of
+    gradient): what does not depend on size over every row, and the oracle on 64 rows spread over the whole token
+    range (the first, the middle and the last rows)."""
+    case = synth.config1(device, seed=0)
+    T, V = case.logits.shape
+    assert T > 100_000 and V == 151936
+    lp = areal_amd.gather_logprobs(case.logits, case.labels)
+    synth.attach_old_and_prox(case, lp, 0.05, 9)
+    rs = RejectionSamplingConfig(**case.ppo["rejection_sampling"])
+    kw = {k: v for k, v in case.ppo.items() if k != "rejection_sampling"}
+    runs = []
+    for _ in range(2):
+        x = case.logits.detach().requires_grad_(True)
+        loss, stat = areal_amd.fused_logprobs_ppo_loss(
+            x, case.labels, case.prox_logp, case.old_logp, case.advantages, loss_mask=case.loss_mask,
+            rejection_sampling=rs, cu_seqlens=case.cu_seqlens, **kw)
+        loss.backward()
+        runs.append((loss.detach().clone(), stat, x.grad))
+    (l1, s1, g1), (l2, s2, g2) = runs
+    assert torch.equal(l1, l2) and torch.equal(s1["logprobs"], s2["logprobs"]) and torch.equal(s1["entropy"], s2["entropy"])
+    assert torch.equal(g1, g2)                                            # bit-equal from run to run
+    del g2, runs
+    assert float(s1["logprobs"].max()) <= 0.0
+    assert float(s1["entropy"].min()) >= 0.0 and float(s1["entropy"].max()) <= math.log(V) + 1e-4
+    assert float((s1["logprobs"] - lp).abs().max()) < 1e-5               # fused forward == stand-alone forward
+    keep = s1["behave_mask"]
+    assert bool((keep <= case.loss_mask).all()) and 0 < int(keep.sum()) < T
+    worst_off, worst_sum = 0.0, 0.0
+    for a in range(0, T, 4096):                                           # row blocks: no fp32 copy of 37 GB
+        g = g1[a:a + 4096].float()
+        k = keep[a:a + 4096]
+        if bool((~k).any()):
+            worst_off = max(worst_off, float(g[~k].abs().max()))
+        if bool(k.any()):
+            worst_sum = max(worst_sum, float((g[k].sum(-1).abs() / g[k].abs().max(-1).values).max()))
+    assert worst_off == 0.0                                               # rows without a mask: exactly zero
+    assert worst_sum < 0.05                                               # rows of (onehot - p) sum to zero up to bf16 rounding
+    manual = s1["loss"][keep].double().sum() / int(case.loss_mask.sum())
+    assert float(l1) == pytest.approx(float(manual), rel=1e-5)
+    # oracle on 64 rows: 22 first, 21 middle, 21 last
+    idx = torch.cat([torch.arange(0, 22), torch.arange(T // 2 - 10, T // 2 + 11), torch.arange(T - 21, T)])
+    idx_d = idx.to(device)
+    n_s = idx.numel()
+    mask_s = case.loss_mask[idx_d].cpu()
+    assert 0 < int(mask_s.sum()) < n_s                                    # the sample holds rows of both kinds
+    w_loss, w_stat, w_grad = oracle.logits_ppo_step(
+        case.logits[idx_d].cpu(), case.labels[idx_d].cpu(), case.prox_logp[idx_d].cpu(), case.old_logp[idx_d].cpu(),
+        case.advantages[idx_d].cpu(), loss_mask=mask_s, rejection_sampling_cfg=rs,
+        cu_seqlens=torch.tensor([0, n_s], dtype=torch.int32), temperature=case.temperature, **kw)
+    ref_lp, ref_ent = oracle.logprobs_entropy_f64(case.logits[idx_d].cpu(), case.labels[idx_d].cpu(), case.temperature)
+    assert float((s1["logprobs"][idx_d].cpu().double() - ref_lp).abs().max()) < 1e-4      # stated: 2e-3
+    assert float((s1["entropy"][idx_d].cpu().double() - ref_ent).abs().max()) < 1e-4
+    for k in ("clip_mask", "dual_clip_mask", "behave_mask"):
+        assert torch.equal(s1[k][idx_d].cpu(), w_stat[k]), k
+    # the oracle normalised by the masked tokens of its 64 rows, the full step by those of all rows
+    want = w_grad.double() * (int(mask_s.sum()) / int(case.loss_mask.sum()))
+    got = g1[idx_d].cpu()
+    assert cosine(got, want) > 0.9999                                     # stated
+    assert_same_magnitude(got, want, what="d_logits of the sampled rows")
 
 
 def test_fused_step_replays_from_a_hip_graph(device):

@@ -10,7 +10,7 @@ import torch
 
 import areal_amd
 import oracle
-from helpers import cosine
+from helpers import assert_same_magnitude, cosine
 
 pytestmark = pytest.mark.gpu
 
@@ -173,6 +173,50 @@ def test_backward_matches_autograd_of_oracle(device, T, V, dtype, temperature, w
         assert float(got.float().sum(-1).abs().max()) < 5e-2  # each row of (onehot - p) sums to zero
 
 
+@pytest.mark.parametrize(
+    "T,V,dtype",
+    [
+        (6, 4104, torch.bfloat16),     # rows that stay in registers
+        (5, 1031, torch.float32),      # unaligned rows: the generic walk
+        (3, 151936, torch.bfloat16),   # the benchmark vocabulary
+        (2, 300000, torch.float32),    # rows longer than the register file
+    ],
+)
+def test_masked_vocabulary_entries_of_minus_infinity(device, T, V, dtype):
+    """Logits of -inf (vocabulary entries a sampler has masked) take probability 0: the log-probs stay finite and the
+    gradient of the log-probs is exactly 0 there, as autograd of log_softmax gives it (not 0 * inf)."""
+    x, y = _case(T, V, dtype, seed=V + T, std=2.0)
+    g = torch.Generator().manual_seed(2)
+    masked = torch.rand(T, V, generator=g) < 0.3
+    masked[torch.arange(T), y] = False
+    masked[:, -1] = True       # the scalar tail of an unaligned row
+    masked[:, 0] = y != 0      # and its head
+    x[masked] = float("-inf")
+    gl = torch.randn(T, generator=g)
+    xd = x.to(device).requires_grad_(True)
+    lp = areal_amd.gather_logprobs(xd, y.to(device), 0.8)
+    (lp * gl.to(device)).sum().backward()
+    xo = x.double().requires_grad_(True)
+    o_lp = torch.log_softmax(xo / 0.8, dim=-1).gather(-1, y[:, None]).squeeze(-1)
+    (o_lp * gl.double()).sum().backward()
+    assert torch.isfinite(lp).all()
+    assert float((lp.detach().cpu().double() - o_lp.detach()).abs().max()) < LOGP_ATOL
+    got = xd.grad.cpu()
+    assert torch.isfinite(got).all()
+    assert float(got[masked].float().abs().max()) == 0.0
+    assert cosine(got, xo.grad) > 0.9999
+    assert_same_magnitude(got, xo.grad, what="d_logits")
+    # the fused PPO step walks the same rows with its own gradient code.  Importance ratio 1 on every token:
+    # loss = -mean(adv), so d loss / d logits = -(adv / T) d logp / d logits
+    xf = x.to(device).requires_grad_(True)
+    loss, stat = areal_amd.fused_logprobs_ppo_loss(xf, y.to(device), lp.detach(), lp.detach(), gl.to(device), 0.2,
+                                                   torch.ones(T, dtype=torch.bool, device=device), temperature=0.8)
+    loss.backward()
+    assert torch.isfinite(stat["logprobs"]).all() and torch.isfinite(xf.grad).all()
+    assert float(xf.grad.cpu()[masked].float().abs().max()) == 0.0
+    assert_same_magnitude(xf.grad.cpu(), -xo.grad / T, what="fused d_logits")
+
+
 def test_plain_c_consumer_of_the_abi(device):
     """tests/c_abi/consumer.c drives the library from C99 with hipMalloc'ed buffers and checks log-probs, entropy, the
     supervised loss, its gradient and the per-sequence statistics against values it computes itself in double."""
@@ -219,6 +263,7 @@ def test_vocab_shards_equal_the_unsharded_op(device, cuts, dtype, temperature):
     assert float((ent.detach().cpu() - w_ent.detach()).abs().max()) < 2e-3
     grad = torch.cat([sh.grad for sh in shards], dim=1).float().cpu()
     assert cosine(grad, x.grad.float()) > 0.9999
+    assert_same_magnitude(grad, x.grad.float(), what="sharded d_logits")
     # against the unsharded kernels: the same numbers up to the order of the sums
     y = logits.to(device).requires_grad_(True)
     lp1, ent1 = areal_amd.gather_logprobs_entropy(y, labels.to(device), temperature)

@@ -192,8 +192,9 @@ def test_compute_advantages_grpo_shape_by_hand():
     bs, L = 2, 6
     am = torch.tensor([[1, 1, 1, 1, 1, 0], [1, 1, 1, 0, 0, 0]])
     lm = torch.tensor([[0, 0, 1, 1, 1, 0], [0, 1, 1, 0, 0, 0]])
+    logprobs_in = -torch.rand(bs, L)
     data = dict(input_ids=torch.zeros(bs, L, dtype=torch.long), attention_mask=am, loss_mask=lm,
-                logprobs=-torch.rand(bs, L), rewards=torch.tensor([30.0, -0.5]))
+                logprobs=logprobs_in.clone(), rewards=torch.tensor([30.0, -0.5]))
     out = O.compute_advantages(data, reward_scaling=0.5, reward_clip=5.0)
     rolled = torch.roll(lm.float(), -1, -1)
     assert torch.equal(out["loss_mask"], rolled)
@@ -202,7 +203,10 @@ def test_compute_advantages_grpo_shape_by_hand():
     # sequence 1: score -0.25 at position 1; rolled mask = positions 0, 1
     assert out["advantages"][1].tolist() == [-0.25, -0.25, 0.0, 0.0, 0.0, 0.0]
     assert torch.equal(out["returns"], out["advantages"]) and torch.equal(out["tot_rewards"][0, 3], torch.tensor(5.0))
-    assert torch.equal(out["prox_logp"], torch.roll(data["logprobs"], -1, -1))
+    # the reference multiplies old_logp by the rolled mask in place (actor.py:195) after storing that same tensor as
+    # data["prox_logp"] (:191): both come out masked
+    assert torch.equal(out["prox_logp"], torch.roll(logprobs_in, -1, -1) * rolled)
+    assert out["prox_logp"] is out["logprobs"]
 
 
 def test_overlong_penalty_hand_cases():
