@@ -52,11 +52,12 @@ __device__ __forceinline__ int acc_col(int nt, int lane) { return nt * 32 + (lan
 // each XCD gets a contiguous range, and that range then walks the tile grid in bands of `kGroupM` tile rows, so that
 // tiles that run at the same time on one XCD share A and B slices in its L2.
 constexpr int kGroupM = 4;
-// The XCD regrouping above is a bijection only when the tile count is a multiple of 8; otherwise use the plain order.
+// XCD x runs the ids x, x + 8, ...: ceil((total - x) / 8) of them, so its range starts after those of the XCDs before
+// it, at x * (total / 8) + min(x, total % 8): a bijection for every tile count.
 __device__ __forceinline__ void tile_of(int pid, int tiles_m, int tiles_n, int& tm, int& tn, int group_m = kGroupM) {
   const int total = tiles_m * tiles_n;
-  int q = pid;
-  if ((total & 7) == 0) q = (pid & 7) * (total >> 3) + (pid >> 3);
+  const int x = pid & 7, rem = total & 7;
+  const int q = x * (total >> 3) + (x < rem ? x : rem) + (pid >> 3);
   const int in_group = group_m * tiles_n;
   const int g = q / in_group;
   const int first_m = g * group_m;

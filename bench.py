@@ -90,7 +90,7 @@ def parse_args():
                     help="logits workloads: hand the kernels fp32 logits (what a Megatron-style head emits) instead of "
                          "bf16; 8 bytes per element instead of 4")
     ap.add_argument("--copy-launches", type=int, default=0,
-                    help="also launch the plain copy kernel this many times over the logits buffer "
+                    help="also launch the plain copy kernel this many times over the logits buffer (lm_head workloads: the weight matrix) "
                          "(the calibration point for FETCH_SIZE / WRITE_SIZE counters)")
     return ap.parse_args()
 
@@ -730,6 +730,16 @@ def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: i
     )
     if NO_FORWARD_OF_MASKED:
         out["config"]["path"] += "; NOT the reference's semantics: masked tokens skip the lm_head"
+    if args.copy_launches > 0:  # calibration point of the FETCH_SIZE / WRITE_SIZE counters: a copy of the weight matrix
+        from areal_amd import functional as F
+
+        dst = torch.empty_like(case.weight)
+        nbytes = case.weight.numel() * case.weight.element_size()
+        for _ in range(args.copy_launches):
+            N.check(N.load().aa_copy_bytes(F._ptr(case.weight), F._ptr(dst), nbytes, F._stream(dev)), "aa_copy_bytes")
+        torch.cuda.synchronize()
+        out["copy_calibration"] = dict(kernel="k_copy16 (aa_copy_bytes)", bytes_read=nbytes, bytes_written=nbytes,
+                                       launches=args.copy_launches)
     sample = fused_gpu_sample(case, kw, cfg, cpu_tokens) if cpu_tokens > 0 else None
     return out, sample
 
