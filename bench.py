@@ -438,8 +438,9 @@ MODE_NAMES = {1: "carry", 0: "recompute"}
 
 # HBM bytes per step of aa_lmhead_ppo_fused at configs[2], all its kernels together: rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (one run each) summed over the kernels of one step, each scaled by what the same counter reads for the
-# plain copy kernel of known size (profiles/lmhead_step_cfg2_hbm_traffic.md).  Other workloads: not measured.
-LMHEAD_MEASURED_HBM_BYTES = {("cfg2", "carry"): None, ("cfg2", "recompute"): None}
+# plain copy kernel of known size (profiles/lmhead_step_cfg2_hbm_traffic.md).  The counters sit behind the L2 of each
+# XCD: what the memory-side cache serves is in these figures too.  Other workloads: not measured.
+LMHEAD_MEASURED_HBM_BYTES = {("cfg2", "carry"): 90.3e9, ("cfg2", "recompute"): 109.8e9}
 
 
 def lmhead_compulsory_bytes(T: int, kept: int, H: int, V: int, mode: str, chunk: int) -> dict:
