@@ -184,13 +184,21 @@ __global__ __launch_bounds__(kThreads) void k_lmhead_tiles(Operand W, Operand Hd
     }
   }
   if constexpr (MODE != kModeStats) {
+    // panel row of each of the tile's 256 tokens (-1: none), looked up once and shared through LDS behind the staged
+    // tile, so that the store loop below has no dependent global load in it
+    int32_t* rows_lds = (int32_t*)(lds + 256 * PZ * 2);
+    {
+      const int n = n0 + tid;
+      rows_lds[tid] = n < N ? (a.out_rows ? a.out_rows[n] : n) : -1;
+    }
     __syncthreads();
     // panel rows: 16-byte pieces along the vocabulary (V % 8 == 0: a piece never straddles the end)
-    for (int p = tid; p < 256 * 32; p += kThreads) {
-      const int nloc = p >> 5, mc = (p & 31) * 8;
-      const int n = n0 + nloc, m = m0 + mc;
-      if (n < N && m < V) {
-        const int r = a.out_rows ? a.out_rows[n] : n;
+    const int mc = (tid & 31) * 8, m = m0 + mc;
+    if (m < V) {
+#pragma unroll 8
+      for (int i = 0; i < 32; ++i) {
+        const int nloc = (tid >> 5) + 8 * i;
+        const int r = rows_lds[nloc];
         if (r >= 0) *(u32x4_t*)(a.panel + (int64_t)r * a.panel_ld + m) = *(const u32x4_t*)(Z + nloc * PZ + mc);
       }
     }
@@ -420,13 +428,19 @@ __global__ __launch_bounds__(kThreads) void k_gemm_store(Operand A, Operand B, i
           *(uint2*)(Z + nloc * PZ + wm * 128 + mt * 32 + 8 * g4 + 4 * (lane >> 5)) = pk;
         }
     }
+    int32_t* rows_lds = (int32_t*)(lds + 256 * PZ * 2);  // row of C of each of the tile's 256 n (-1: past the end)
+    {
+      const int n = n0 + tid;
+      rows_lds[tid] = n < N ? (c_rows ? c_rows[n] : n) : -1;
+    }
     __syncthreads();
-    for (int p = tid; p < 256 * 32; p += kThreads) {  // M % 8 == 0: a piece never straddles the end
-      const int nloc = p >> 5, mc = (p & 31) * 8;
-      const int n = n0 + nloc, m = m0 + mc;
-      if (n < N && m < M) {
-        const int64_t r = c_rows ? c_rows[n] : n;
-        *(u32x4_t*)(C + r * ldc + m) = *(const u32x4_t*)(Z + nloc * PZ + mc);
+    const int mc = (tid & 31) * 8, m = m0 + mc;  // M % 8 == 0: a piece never straddles the end
+    if (m < M) {
+#pragma unroll 8
+      for (int i = 0; i < 32; ++i) {
+        const int nloc = (tid >> 5) + 8 * i;
+        const int r = rows_lds[nloc];
+        if (r >= 0) *(u32x4_t*)(C + (int64_t)r * ldc + m) = *(const u32x4_t*)(Z + nloc * PZ + mc);
       }
     }
   } else {
