@@ -14,10 +14,12 @@
 // hidden states as they lie: no transposed copies).  Two ways to fill the panel:
 //   recompute   the logits tiles are formed again and turned into d(logits) in registers (2 T_grad V H extra flops);
 //               what aa_lmhead_bwd does, where the upstream gradients only exist after the forward has returned.
-//   carry       (training step only) the forward tiles also write 2^(x c - k_block), the unnormalised probabilities
-//               that their statistics are made of, for the tokens that will have a gradient; once the row statistics
-//               and the loss are known, a streaming pass scales each 128-wide block of a row by
-//               -(g / T) 2^(k_block - k_row) / s_row and adds g / T at the label: the same d(logits), no second GEMM.
+//   carry       (training step only) the forward tiles also write p_v / p_label = 2^((x_v - x_label) c), as bf16, for the
+//               tokens that will have a gradient (the label logit is known before the tiles run).  Once the loss is
+//               known, d(logits) of a row is that row times one factor per token, -(g / T) p_label (the label entry
+//               is patched to 1 - 1 / p_label first), and the factor is applied inside the two GEMMs: no second logits
+//               GEMM and no pass over the panel.  A chunk that holds a token whose label is too unlikely for that
+//               range (log-prob below -80) is redone by the recompute tiles, decided on the device.
 // Tokens whose loss mask is zero have a zero gradient row: they are left out of the panel and of both GEMMs.
 #include "device_utils.h"
 #include "gemm_tn.h"
@@ -59,7 +61,18 @@ struct TileArgs {
   const float* g_logp;
   const float* g_entropy;  // nullable
   float inv_t;
+  const int32_t* run_if;   // recompute tiles only: when given, the kernel does nothing unless *run_if != 0
 };
+
+// Carry mode stores 2^(x c - kref) with kref = c * (label logit of the token): a reference that is known before the
+// first tile runs and is the same in every vocabulary block, so that d(logits) of a panel row is the stored row times
+// ONE factor per token (applied where the gradient GEMMs already touch the token: the d_hidden epilogue and the gather
+// of the hidden rows for d_weight) and no pass over the panel is needed.  The stored value is p_v / p_label, finite
+// in bf16 (which has the exponent range of fp32) as long as the label's log-prob is above about -87; the exponent is
+// clamped so that nothing overflows, and a chunk with such a token (kCarryMinLogp, never seen in training: the label
+// would have to be e^-80 unlikely) is redone by the recompute tiles, decided on the device.
+constexpr float kCarryMaxShift = 126.f;
+constexpr float kCarryMinLogp = -80.f;
 
 // Statistics (and, with CARRY, the staged unnormalised probabilities) of one wave's 128 x 128 block.  RAGGED: the
 // block may reach past the vocabulary (last tile row only), rows at or past V are left out.
@@ -85,6 +98,12 @@ __device__ __forceinline__ void block_stats(const Acc& acc, const TileArgs& a, i
     }
     mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));  // both halves of the wave hold the same token
     const float k = fmaxf(mx * a.c, kNegBig);   // kNegBig: no valid row in this block
+    float to_ref = 1.f;                         // 2^(k - kref): block-relative -> label-relative exponentials
+    if constexpr (CARRY) {
+      const float kref = n < N ? a.xy[n] * a.c : 0.f;
+      // a label outside the vocabulary has no logit (NaN): keep the block-relative values, the row's factor is NaN or 0
+      to_ref = fabsf(kref) < 1e30f ? fast_exp2(fminf(k - kref, kCarryMaxShift)) : 1.f;
+    }
     float s = 0.f, u = 0.f;
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt)
@@ -101,8 +120,8 @@ __device__ __forceinline__ void block_stats(const Acc& acc, const TileArgs& a, i
         }
         if constexpr (CARRY) {
           uint2 pk;
-          pk.x = Elem<AA_BF16>::pack(e[0], e[1]);
-          pk.y = Elem<AA_BF16>::pack(e[2], e[3]);
+          pk.x = Elem<AA_BF16>::pack(e[0] * to_ref, e[1] * to_ref);
+          pk.y = Elem<AA_BF16>::pack(e[2] * to_ref, e[3] * to_ref);
           *(uint2*)(Z + nloc * PZ + wm * 128 + mt * 32 + 8 * g4 + 4 * (lane >> 5)) = pk;
         }
       }
@@ -123,6 +142,9 @@ template <int MODE>
 __global__ __launch_bounds__(kThreads) void k_lmhead_tiles(Operand W, Operand Hd, int K, int tiles_m, int tiles_n,
                                                                  TileArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
+  if constexpr (MODE == kModeRecompute) {
+    if (a.run_if && *a.run_if == 0) return;  // uniform over the grid
+  }
   int tm, tn;
   tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
@@ -209,7 +231,8 @@ __global__ __launch_bounds__(kThreads) void k_lmhead_tiles(Operand W, Operand Hd
 // wave per token.
 __global__ __launch_bounds__(256) void k_label_logit(const uint16_t* __restrict__ hidden, const uint16_t* __restrict__ weight,
                                                      const int64_t* __restrict__ labels, int n_tok, int H, int V,
-                                                     float* __restrict__ xy) {
+                                                     float* __restrict__ xy, int32_t* __restrict__ clear_flag) {
+  if (clear_flag && blockIdx.x == 0 && threadIdx.x == 0) *clear_flag = 0;  // the chunk's "redo by recompute" flag
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (t >= n_tok) return;
@@ -290,12 +313,12 @@ __global__ __launch_bounds__(1024) void k_combine(const float* __restrict__ pk, 
   if (row_ez) row_ez[t] = (m.k + mean_t) * kLn2;
 }
 
-// What the streaming pass of the carry mode needs per panel row
-struct RowCoef {
-  float k_row;    // row maximum of x c
-  float base;     // -(g / T) / s_row
-  float lab_add;  // g / T
-  int32_t label;  // label of the row's token (-1 when it lies outside the vocabulary)
+// What carry mode needs per panel row, written by k_token_loss
+struct CarryOut {
+  float* row_factor;   // [rows] d(logits) of the row = row_factor * stored row (with the label entry patched, below)
+  uint16_t* panel;     // the label entry of each row is overwritten so that the product gives (g / T) (1 - p_label)
+  int64_t panel_ld;
+  int32_t* redo_flag;  // set to 1 when a token with a gradient has a label log-prob below kCarryMinLogp
 };
 
 struct TokenLossArgs {
@@ -322,7 +345,7 @@ __global__ __launch_bounds__(1024) void k_token_loss(const float* __restrict__ p
                                                      int64_t pitch_t, int n_tok, int V, float c, float inv_t,
                                                      const int64_t* __restrict__ labels, TokenLossArgs a,
                                                      const int32_t* __restrict__ out_rows, float* __restrict__ g_tok,
-                                                     float* __restrict__ lse_tok, RowCoef* __restrict__ rowc) {
+                                                     float* __restrict__ lse_tok, CarryOut carry) {
   __shared__ float smem[3 * kMergeWaves * 64];
   const int t = blockIdx.x * 64 + (threadIdx.x & 63);
   const Merged m = merge_blocks(pk, ps, pu, blocks, pitch_t, t, t < n_tok, smem);
@@ -358,39 +381,29 @@ __global__ __launch_bounds__(1024) void k_token_loss(const float* __restrict__ p
   }
   if (g_tok) g_tok[t] = g;
   if (lse_tok) lse_tok[t] = (m.k + log2s) * kLn2;
-  if (rowc) {
+  if (carry.row_factor) {
     const int r = out_rows ? out_rows[t] : t;
     if (r >= 0) {
+      // stored row: q_v = p_v / p_label.  d(logits)_v = (g / T) (onehot_v - p_v) = f q_v with f = -(g / T) p_label for
+      // every v but the label, whose entry is replaced by 1 - 1 / p_label: f (1 - 1 / p_label) = (g / T) (1 - p_label)
+      const float kref = xy[t] * c;                                   // as the tiles formed it
+      const float p_label = fast_exp2(kref - (m.k + log2s));
+      carry.row_factor[r] = g == 0.f ? 0.f : -(g * inv_t) * p_label;  // g == 0: whatever the row holds counts for nothing
       const int64_t y = labels[t];
-      rowc[r] = {m.k, -(g * inv_t) / m.s, g * inv_t, (y >= 0 && y < V) ? (int32_t)y : -1};
+      if (y >= 0 && y < V) {
+        const float patched = -expm1f(-lp);
+        carry.panel[(int64_t)r * carry.panel_ld + y] = (uint16_t)(Elem<AA_BF16>::pack(patched, 0.f) & 0xffffu);
+      }
+      if (g != 0.f && lp < kCarryMinLogp) *carry.redo_flag = 1;
     }
   }
 }
 
-// Carry mode: panel row r holds 2^(x c - k_block) of token act_rows[r] (or r); scale every 128-wide block to
-// d(loss)/d(logits) in place.  One workgroup per row, 16-byte pieces (all 8 elements of a piece lie in one block).
-__global__ __launch_bounds__(256) void k_panel_scale(uint16_t* __restrict__ panel, int64_t panel_ld, int V,
-                                                     const RowCoef* __restrict__ rowc, const int32_t* __restrict__ act_rows,
-                                                     const float* __restrict__ pk, int64_t pitch_t) {
-  const int r = blockIdx.x;
-  const RowCoef rc = rowc[r];
-  const int64_t t = act_rows ? act_rows[r] : r;
-  uint16_t* row = panel + (int64_t)r * panel_ld;
-  const int pieces = V >> 3;
-  for (int p = threadIdx.x; p < pieces; p += 256) {
-    const float f = rc.base * fast_exp2(pk[(int64_t)(p >> 4) * pitch_t + t] - rc.k_row);
-    float x[8];
-    load8<AA_BF16>(row, (int64_t)p * 8, x);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) x[j] *= f;
-    const int rel = rc.label - p * 8;
-    if (rel >= 0 && rel < 8) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j)
-        if (rel == j) x[j] += rc.lab_add;
-    }
-    store8<AA_BF16>(row, (int64_t)p * 8, x);
-  }
+// After the conditional recompute of a flagged chunk the panel holds d(logits) itself: every row factor becomes 1.
+__global__ __launch_bounds__(256) void k_unit_factors(float* __restrict__ row_factor, int rows, const int32_t* __restrict__ flag) {
+  if (*flag == 0) return;
+  const int r = blockIdx.x * 256 + threadIdx.x;
+  if (r < rows) row_factor[r] = 1.f;
 }
 
 // ---- plain product C = B . A^T on the same main loop ---------------------------------------------------------------
@@ -402,7 +415,8 @@ __global__ __launch_bounds__(256) void k_panel_scale(uint16_t* __restrict__ pane
 template <bool AKM, bool BKM, typename OutT, bool ACCUM>
 __global__ __launch_bounds__(kThreads) void k_gemm_store(Operand A, Operand B, int K, int tiles_m, int tiles_n,
                                                          OutT* __restrict__ C, int64_t ldc,
-                                                         const int32_t* __restrict__ c_rows) {
+                                                         const int32_t* __restrict__ c_rows,
+                                                         const float* __restrict__ n_scale) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   int tm, tn;
   tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
@@ -418,13 +432,15 @@ __global__ __launch_bounds__(kThreads) void k_gemm_store(Operand A, Operand B, i
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) {
       const int nloc = wn * 128 + acc_col(nt, lane);
+      // optional factor per row of C (a lane owns one n): applied to the fp32 sums, before the one rounding to bf16
+      const float f = (n_scale && n0 + nloc < N) ? n_scale[n0 + nloc] : 1.f;
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4) {
           uint2 pk;
-          pk.x = Elem<AA_BF16>::pack(acc.v[mt][nt][g4 * 4], acc.v[mt][nt][g4 * 4 + 1]);
-          pk.y = Elem<AA_BF16>::pack(acc.v[mt][nt][g4 * 4 + 2], acc.v[mt][nt][g4 * 4 + 3]);
+          pk.x = Elem<AA_BF16>::pack(acc.v[mt][nt][g4 * 4] * f, acc.v[mt][nt][g4 * 4 + 1] * f);
+          pk.y = Elem<AA_BF16>::pack(acc.v[mt][nt][g4 * 4 + 2] * f, acc.v[mt][nt][g4 * 4 + 3] * f);
           *(uint2*)(Z + nloc * PZ + wm * 128 + mt * 32 + 8 * g4 + 4 * (lane >> 5)) = pk;
         }
     }
@@ -500,12 +516,26 @@ __global__ __launch_bounds__(1024) void k_compact_map(const uint8_t* __restrict_
   for (int p = total + tid; p < limit; p += 1024) act_rows[p] = 0;
 }
 
-// dst[r, :] = src[rows[r], :] (H % 8 == 0)
+// dst[r, :] = scale[r] * src[rows[r], :] (H % 8 == 0); rows == nullptr: row r itself; scale == nullptr: 1;
+// run_if, when given: nothing happens unless *run_if != 0
 __global__ __launch_bounds__(256) void k_gather_rows(const u32x4_t* __restrict__ src, const int32_t* __restrict__ rows,
-                                                     u32x4_t* __restrict__ dst, int h_vec) {
+                                                     u32x4_t* __restrict__ dst, int h_vec,
+                                                     const float* __restrict__ scale, const int32_t* __restrict__ run_if) {
+  if (run_if && *run_if == 0) return;
   const int64_t r = blockIdx.x;
-  const int64_t t = rows[r];
-  for (int j = threadIdx.x; j < h_vec; j += 256) dst[r * h_vec + j] = src[t * h_vec + j];
+  const int64_t t = rows ? rows[r] : r;
+  if (!scale) {
+    for (int j = threadIdx.x; j < h_vec; j += 256) dst[r * h_vec + j] = src[t * h_vec + j];
+    return;
+  }
+  const float f = scale[r];
+  for (int j = threadIdx.x; j < h_vec; j += 256) {
+    float x[8];
+    load8<AA_BF16>((const uint16_t*)(src + t * h_vec), (int64_t)j * 8, x);
+#pragma unroll
+    for (int q = 0; q < 8; ++q) x[q] *= f;
+    store8<AA_BF16>((uint16_t*)(dst + r * h_vec), (int64_t)j * 8, x);
+  }
 }
 
 __global__ __launch_bounds__(256) void k_zero16(u32x4_t* __restrict__ p, int64_t n_vec) {
@@ -542,7 +572,7 @@ struct Workspace {
   int64_t off_pk, off_ps, off_pu;       // block partials [blocks][chunk]
   int64_t off_xy, off_g, off_lse;       // per token of the chunk: label logit, g, logsumexp
   int64_t fwd_bytes;                    // what the forward alone needs
-  int64_t off_rowc;                     // RowCoef per panel row
+  int64_t off_rowf, off_flag;           // carry mode: factor per panel row; the chunk's redo flag
   int64_t off_rows;                     // out_rows, act_rows (2 x chunk int32)
   int64_t off_panel;                    // d(logits) rows [chunk, V]
   int64_t off_hc;                       // the hidden rows of the tokens with gradient, closed up [chunk, H]
@@ -563,7 +593,8 @@ static Workspace plan(int64_t T, int64_t H, int64_t V) {
   w.off_g = off;   off += up(w.chunk * 4);
   w.off_lse = off; off += up(w.chunk * 4);
   w.fwd_bytes = off;
-  w.off_rowc = off;    off += up(w.chunk * (int64_t)sizeof(RowCoef));
+  w.off_rowf = off;    off += up(w.chunk * 4);  // factor per panel row (carry mode)
+  w.off_flag = off;    off += 256;              // the chunk's "redo by recompute" flag
   w.off_rows = off;    off += up(2 * w.chunk * 4);
   w.off_panel = off;   off += up(w.chunk * V * 2);
   w.off_hc = off;      off += up(w.chunk * H * 2);
@@ -610,32 +641,36 @@ static void launch_tiles(hipStream_t st, const void* weight, const uint16_t* hid
 // C [N, M] = B . A^T over K (rows of C through c_rows when given); lda / ldb: leading dimensions of the arrays as stored
 template <bool AKM, bool BKM, typename OutT, bool ACCUM>
 static void launch_gemm(hipStream_t st, const uint16_t* A, int64_t lda, int64_t M, const uint16_t* B, int64_t ldb, int64_t N,
-                        int64_t K, OutT* C, int64_t ldc, const int32_t* c_rows = nullptr) {
+                        int64_t K, OutT* C, int64_t ldc, const int32_t* c_rows = nullptr,
+                        const float* n_scale = nullptr) {
   const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
   Operand a{A, lda, (int)M}, b{B, ldb, (int)N};
   hipLaunchKernelGGL((k_gemm_store<AKM, BKM, OutT, ACCUM>), dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads), kLdsBytes, st,
-                     a, b, (int)K, tiles_m, tiles_n, C, ldc, c_rows);
+                     a, b, (int)K, tiles_m, tiles_n, C, ldc, c_rows, n_scale);
 }
 
-// The two GEMMs that contract the d(logits) rows ds [n_rows, V] (in the panel) of one token chunk:
-//   d_hidden rows [n_rows, H] = ds . W                  contraction over V: ds K-contiguous, W [V, H] K-major
-//   d_weight [V, H] (+)= ds^T . hidden rows             contraction over the rows: both arrays K-major
+// The two GEMMs that contract the d(logits) rows ds [n_rows, V] of one token chunk, ds = row_factor[r] * panel[r, :]
+// (row_factor == nullptr: the panel holds d(logits) itself):
+//   d_hidden rows [n_rows, H] = ds . W                  contraction over V: panel K-contiguous, W [V, H] K-major;
+//                                                       the factor multiplies the fp32 sums in the epilogue
+//   d_weight [V, H] (+)= ds^T . hidden rows             contraction over the rows: both arrays K-major; the factor
+//                                                       goes into the copy of the hidden rows
 // No transposed copy of anything is made.  token_of_row, when given, lists the tokens of the chunk that the n_rows
-// rows of ds belong to (tokens without gradient were left out): their hidden rows are closed up first, and the
-// d_hidden rows go to those tokens (the caller has cleared the others).
+// rows belong to (tokens without gradient were left out): their hidden rows are closed up first, and the d_hidden rows
+// go to those tokens (the caller has cleared the others).
 static void panel_gradients(hipStream_t st, const Workspace& w, char* ws, const void* weight, const uint16_t* hid,
-                            const int32_t* token_of_row, int64_t n_rows, int64_t H, int64_t V, uint16_t* d_hidden_chunk,
-                            void* d_weight, bool dw_f32, bool first) {
+                            const int32_t* token_of_row, const float* row_factor, int64_t n_rows, int64_t H, int64_t V,
+                            uint16_t* d_hidden_chunk, void* d_weight, bool dw_f32, bool first) {
   const uint16_t* ds = (const uint16_t*)(ws + w.off_panel);
   const uint16_t* hid_rows = hid;
-  if (token_of_row) {
+  if (token_of_row || row_factor) {
     uint16_t* hc = (uint16_t*)(ws + w.off_hc);
     hipLaunchKernelGGL(k_gather_rows, dim3((unsigned)n_rows), dim3(256), 0, st, (const u32x4_t*)hid, token_of_row,
-                       (u32x4_t*)hc, (int)(H / 8));
+                       (u32x4_t*)hc, (int)(H / 8), row_factor, (const int32_t*)nullptr);
     hid_rows = hc;
   }
   launch_gemm<true, false, uint16_t, false>(st, (const uint16_t*)weight, H, H, ds, V, n_rows, V, d_hidden_chunk, H,
-                                            token_of_row);
+                                            token_of_row, row_factor);
   if (!dw_f32)
     launch_gemm<true, true, uint16_t, false>(st, hid_rows, H, H, ds, V, V, n_rows, (uint16_t*)d_weight, H);
   else if (first)
@@ -645,12 +680,15 @@ static void panel_gradients(hipStream_t st, const Workspace& w, char* ws, const 
 }
 
 // Recompute: d(logits) of the panel rows from the logits tiles formed again.  With a row map only the hidden rows that
-// have a panel row are multiplied (gathered first); `a` carries the per-token inputs of the chunk.
+// have a panel row are multiplied (gathered first); `a` carries the per-token inputs of the chunk.  With run_if the
+// kernels are enqueued but do nothing unless *run_if != 0 when they start.
 static void recompute_panel(hipStream_t st, const Workspace& w, char* ws, const void* weight, const uint16_t* hid,
-                            int64_t n_tok, const int32_t* token_of_row, int64_t rows, int64_t H, int64_t V, TileArgs a) {
+                            int64_t n_tok, const int32_t* token_of_row, int64_t rows, int64_t H, int64_t V, TileArgs a,
+                            const int32_t* run_if = nullptr) {
   a.panel = (uint16_t*)(ws + w.off_panel);
   a.panel_ld = V;
   a.out_rows = nullptr;
+  a.run_if = run_if;
   if (!token_of_row) {
     a.col_tokens = nullptr;
     launch_tiles<kModeRecompute>(st, weight, hid, n_tok, H, V, a);
@@ -658,7 +696,7 @@ static void recompute_panel(hipStream_t st, const Workspace& w, char* ws, const 
   }
   uint16_t* hc = (uint16_t*)(ws + w.off_hc);
   hipLaunchKernelGGL(k_gather_rows, dim3((unsigned)rows), dim3(256), 0, st, (const u32x4_t*)hid, token_of_row, (u32x4_t*)hc,
-                     (int)(H / 8));
+                     (int)(H / 8), (const float*)nullptr, run_if);
   a.col_tokens = token_of_row;
   launch_tiles<kModeRecompute>(st, weight, hc, rows, H, V, a);
 }
@@ -732,7 +770,7 @@ extern "C" int aa_lmhead_fwd(const void* hidden, const void* weight, int64_t T, 
     const TileArgs a = stats_args(w, ws, labels + t0, inv_temperature);
     const uint16_t* hid = (const uint16_t*)hidden + t0 * H;
     hipLaunchKernelGGL(k_label_logit, dim3((unsigned)((n_tok + 3) / 4)), dim3(256), 0, st, hid, (const uint16_t*)weight,
-                       labels + t0, (int)n_tok, (int)H, (int)V, a.xy);
+                       labels + t0, (int)n_tok, (int)H, (int)V, a.xy, (int32_t*)nullptr);
     launch_tiles<kModeStats>(st, weight, hid, n_tok, H, V, a);
     hipLaunchKernelGGL(k_combine, dim3((unsigned)((n_tok + 63) / 64)), dim3(1024), 0, st, a.pk, a.ps, a.pu, a.xy,
                        (int)w.blocks, a.pitch_t, (int)n_tok, a.c, logp + t0, at(entropy, t0), at(row_lse, t0),
@@ -806,7 +844,7 @@ extern "C" int aa_lmhead_fwd_static(const void* hidden, const void* weight, int6
     const uint16_t* hid = (const uint16_t*)hidden + t0 * H;
     a.labels = labels + t0;
     hipLaunchKernelGGL(k_label_logit, dim3((unsigned)((n_tok + 3) / 4)), dim3(256), 0, st, hid, (const uint16_t*)weight,
-                       labels + t0, (int)n_tok, (int)H, (int)V, a.xy);
+                       labels + t0, (int)n_tok, (int)H, (int)V, a.xy, (int32_t*)nullptr);
     launch_tiles<kModeStats>(st, weight, hid, n_tok, H, V, a);
     hipLaunchKernelGGL(k_combine, dim3((unsigned)((n_tok + 63) / 64)), dim3(1024), 0, st, a.pk, a.ps, a.pu, a.xy, (int)blocks,
                        a.pitch_t, (int)n_tok, a.c, logp + t0, at(entropy, t0), at(row_lse, t0), at(row_ez, t0));
@@ -850,7 +888,7 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
     a.g_entropy = g_entropy ? g_entropy + t0 : nullptr;
     if (!kept_per_chunk) {
       recompute_panel(st, w, ws, weight, hid, n_tok, nullptr, n_tok, H, V, a);
-      panel_gradients(st, w, ws, weight, hid, nullptr, n_tok, H, V, dh, dw.acc, dw.acc_f32, first);
+      panel_gradients(st, w, ws, weight, hid, nullptr, nullptr, n_tok, H, V, dh, dw.acc, dw.acc_f32, first);
       first = false;
       continue;
     }
@@ -865,7 +903,7 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
                        out_rows, act_rows);
     recompute_panel(st, w, ws, weight, hid, n_tok, act_rows, kept, H, V, a);
     launch_zero(st, dh, n_tok * H * 2);  // the rows of the other tokens
-    panel_gradients(st, w, ws, weight, hid, act_rows, kept, H, V, dh, dw.acc, dw.acc_f32, first);
+    panel_gradients(st, w, ws, weight, hid, act_rows, nullptr, kept, H, V, dh, dw.acc, dw.acc_f32, first);
     first = false;
   }
   if (first) launch_zero(st, dw.acc, V * H * (dw.acc_f32 ? 4 : 2));  // no row of the batch has a gradient
@@ -904,7 +942,8 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
   int32_t* act_rows = out_rows + w.chunk;
   float* g_tok = (float*)(ws + w.off_g);
   float* lse_tok = (float*)(ws + w.off_lse);
-  RowCoef* rowc = (RowCoef*)(ws + w.off_rowc);
+  float* row_factor = (float*)(ws + w.off_rowf);
+  int32_t* redo_flag = (int32_t*)(ws + w.off_flag);
   uint16_t* panel = (uint16_t*)(ws + w.off_panel);
   bool first = true;  // no GEMM has written d_weight yet
   int64_t chunk_index = 0;
@@ -933,7 +972,7 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
     a.panel_ld = V;
     a.out_rows = row_of_token;
     hipLaunchKernelGGL(k_label_logit, dim3((unsigned)((n_tok + 3) / 4)), dim3(256), 0, st, hid, (const uint16_t*)weight,
-                       labels + t0, (int)n_tok, (int)H, (int)V, a.xy);
+                       labels + t0, (int)n_tok, (int)H, (int)V, a.xy, redo_flag);
     if (carry && rows > 0)
       launch_tiles<kModeStatsCarry>(st, weight, hid, n_tok, H, V, a);
     else
@@ -943,21 +982,22 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
                      at(stat_loss), at(ratio), at(flags), *params, act};
     hipLaunchKernelGGL(k_token_loss, dim3((unsigned)((n_tok + 63) / 64)), dim3(1024), 0, st, a.pk, a.ps, a.pu, a.xy,
                        (int)w.blocks, a.pitch_t, (int)n_tok, (int)V, a.c, inv_temperature, labels + t0, la, row_of_token,
-                       g_tok, lse_tok, carry ? rowc : nullptr);
+                       g_tok, lse_tok,
+                       (carry && rows > 0) ? CarryOut{row_factor, panel, V, redo_flag} : CarryOut{nullptr, nullptr, 0, nullptr});
     if (rows == 0) {
       launch_zero(st, dh, n_tok * H * 2);
       continue;
     }
-    if (carry) {
-      hipLaunchKernelGGL(k_panel_scale, dim3((unsigned)rows), dim3(256), 0, st, panel, V, (int)V, rowc, token_of_row, a.pk,
-                         a.pitch_t);
-    } else {
-      a.row_lse = lse_tok;
-      a.g_logp = g_tok;
-      recompute_panel(st, w, ws, weight, hid, n_tok, token_of_row, rows, H, V, a);
-    }
+    // d(logits) rows by recompute: always in that mode; in carry mode only if the chunk was flagged (decided on the
+    // device: the kernels start and return at once otherwise), and then the row factors become 1
+    a.row_lse = lse_tok;
+    a.g_logp = g_tok;
+    recompute_panel(st, w, ws, weight, hid, n_tok, token_of_row, rows, H, V, a, carry ? redo_flag : nullptr);
+    if (carry)
+      hipLaunchKernelGGL(k_unit_factors, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, row_factor, (int)rows, redo_flag);
     if (token_of_row) launch_zero(st, dh, n_tok * H * 2);  // the rows of the tokens without gradient
-    panel_gradients(st, w, ws, weight, hid, token_of_row, rows, H, V, dh, dw.acc, dw.acc_f32, first);
+    panel_gradients(st, w, ws, weight, hid, token_of_row, carry ? row_factor : nullptr, rows, H, V, dh, dw.acc, dw.acc_f32,
+                    first);
     first = false;
   }
   if (first) launch_zero(st, dw.acc, V * H * (dw.acc_f32 ? 4 : 2));  // no token of the batch has a gradient

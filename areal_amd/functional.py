@@ -905,10 +905,12 @@ def fused_lm_head_ppo_loss(
     ``backward`` chooses how the bf16 ``d(loss)/d(logits)`` rows of a chunk (``[tokens with gradient, V]`` in the
     workspace, which the two gradient GEMMs contract) are obtained.  ``"recompute"``: the logits tiles of those tokens
     are formed a second time once the loss is known, as ``lm_head_logprobs_entropy``'s backward does (a third more
-    matrix work).  ``"carry"`` (default, the faster of the two by measurement): the forward tiles also write the
-    unnormalised probabilities ``2^(x c - k_block)`` that their softmax partials are made of into those rows, and a
-    streaming pass scales them into the gradient afterwards; no second GEMM.  Both write the same bytes into the
-    same workspace (``4 * chunk * V`` bytes with the transposed copy; carry writes the rows twice).
+    matrix work).  ``"carry"`` (default, the faster of the two by measurement): the forward tiles also write
+    ``p_v / p_label`` of those tokens in bf16 into the rows (the label's logit is known before the tiles run); once
+    the loss is known the gradient row is that row times one factor per token, which the two gradient GEMMs apply
+    themselves, so there is neither a second logits GEMM nor a pass over the rows.  A chunk that holds a token whose
+    label has a log-prob below -80 (outside the stored range) is redone by recompute, decided on the device.  Both
+    modes use the same workspace (``2 * chunk * V`` bytes for the rows).
 
     ``skip_masked_tokens``: a token whose (effective) loss mask is zero has a zero gradient row, so the two gradient
     GEMMs run on the other tokens only; the results are those of the dense computation.  The per-chunk token counts

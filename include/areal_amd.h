@@ -665,10 +665,13 @@ typedef enum {
    * once the loss is known (2 T_grad V H extra flops; the forward half writes
    * nothing of size T x V) */
   AA_LMHEAD_RECOMPUTE = 0,
-  /* the forward tiles also write 2^(x c - k_block), the unnormalised
-   * probabilities their statistics are made of, as bf16 into the rows of the
-   * tokens with gradient; a streaming pass scales them to d(logits) once the
-   * loss is known (no second GEMM; the same rows are written twice) */
+  /* the forward tiles also write p_v / p_label (the label logit is known
+   * before they run) as bf16 into the rows of the tokens with gradient; once
+   * the loss is known, d(logits) of a row is that row times one factor per
+   * token, which the two gradient GEMMs apply themselves (no second logits
+   * GEMM, no pass over the rows).  A chunk with a token whose label has a
+   * log-prob below -80 does not fit the stored range and is redone as in
+   * AA_LMHEAD_RECOMPUTE, decided on the device (same results, slower). */
   AA_LMHEAD_CARRY = 1
 } aa_lmhead_backward_mode;
 

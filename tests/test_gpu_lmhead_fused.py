@@ -104,6 +104,48 @@ def test_carry_and_recompute_give_the_same_step(device):
             assert_same_magnitude(a, b, rel=2e-3)
 
 
+def test_carry_redoes_a_chunk_whose_labels_are_too_unlikely_to_store(device):
+    """Carry mode stores p_v / p_label in bf16; a token with a gradient whose label has a log-prob below -80 does not
+    fit that range, and its chunk is redone by the recompute tiles, decided on the device.  Logits with a spread of
+    about 48 put many labels there; the second chunk of the batch has ordinary logits and stays on the carried rows.
+    Both must match the oracle and the recompute mode."""
+    T, H, V = 16384 + 300, 64, 1088
+    g = torch.Generator().manual_seed(5)
+    hidden = torch.randn(T, H, generator=g)
+    hidden[:16384] *= 12.0                     # first chunk: logits ~ N(0, 48^2)
+    hidden = hidden.bfloat16()
+    weight = (0.5 * torch.randn(V, H, generator=g)).bfloat16()
+    labels = torch.randint(0, V, (T,), generator=g)
+    ref_lp = oracle.logprobs(oracle.lmhead_logits(hidden, weight), labels)
+    assert int((ref_lp[:16384] < -80).sum()) > 100 and float(ref_lp[16384:].min()) > -60
+    prox = ref_lp + 0.05 * torch.randn(T, generator=g)
+    old = ref_lp + 0.3 * torch.randn(T, generator=g)
+    adv = torch.randn(T, generator=g)
+    mask = torch.rand(T, generator=g) < 0.7
+    args = [t.to(device) for t in (labels, prox, old, adv)]
+
+    def run(backward):
+        h = hidden.to(device).requires_grad_(True)
+        w = weight.to(device).requires_grad_(True)
+        loss, stat = areal_amd.fused_lm_head_ppo_loss(h, w, *args, eps_clip=0.2, loss_mask=mask.to(device), backward=backward)
+        loss.backward()
+        return loss.detach(), stat, h.grad.float(), w.grad.float()
+
+    o_loss, _, o_lp, _, o_dh, o_dw = _oracle_step(hidden, weight, labels, prox, old, adv, mask, 1.0, 1.0, eps_clip=0.2)
+    ref = run("recompute")
+    got = run("carry")
+    assert torch.equal(got[0], ref[0]) and torch.equal(got[1]["logprobs"], ref[1]["logprobs"])
+    assert_within(got[1]["logprobs"], o_lp, 2e-3, "log-prob")
+    assert float(got[0]) == pytest.approx(o_loss, rel=1e-3)
+    for name, a, b, o in (("d(hidden)", got[2], ref[2], o_dh), ("d(W)", got[3], ref[3], o_dw)):
+        assert torch.isfinite(a).all(), name
+        assert cosine(a.cpu(), o) > 0.9999, name
+        assert_same_magnitude(a, o, what=name)
+        assert cosine(a.cpu(), b.cpu()) > 0.99999, name
+    # the flagged chunk came out of the recompute tiles: its d(hidden) rows are those of the recompute mode, bit for bit
+    assert torch.equal(got[2][:16384], ref[2][:16384])
+
+
 def test_upstream_gradient_scales_both_gradients(device):
     hidden, weight, labels, prox, old, adv, mask = _inputs(260, 260, 64, 704, seed=3)
     args = [t.to(device) for t in (labels, prox, old, adv)]
