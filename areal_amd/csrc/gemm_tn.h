@@ -53,17 +53,24 @@ __device__ __forceinline__ int acc_col(int nt, int lane) { return nt * 32 + (lan
 // tiles that run at the same time on one XCD share A and B slices in its L2.
 constexpr int kGroupM = 4;
 // XCD x runs the ids x, x + 8, ...: ceil((total - x) / 8) of them, so its range starts after those of the XCDs before
-// it, at x * (total / 8) + min(x, total % 8): a bijection for every tile count.
-__device__ __forceinline__ void tile_of(int pid, int tiles_m, int tiles_n, int& tm, int& tn, int group_m = kGroupM) {
-  const int total = tiles_m * tiles_n;
+// it, at x * (total / 8) + min(x, total % 8): a bijection for every count.
+__device__ __forceinline__ int xcd_contiguous(int pid, int total) {
   const int x = pid & 7, rem = total & 7;
-  const int q = x * (total >> 3) + (x < rem ? x : rem) + (pid >> 3);
+  return x * (total >> 3) + (x < rem ? x : rem) + (pid >> 3);
+}
+
+// tile number q of the band walk: bands of group_m tile rows, inside a band down the rows first
+__device__ __forceinline__ void tile_at(int q, int tiles_m, int tiles_n, int& tm, int& tn, int group_m = kGroupM) {
   const int in_group = group_m * tiles_n;
   const int g = q / in_group;
   const int first_m = g * group_m;
   const int gsz = (tiles_m - first_m) < group_m ? (tiles_m - first_m) : group_m;
   tm = first_m + (q % in_group) % gsz;
   tn = (q % in_group) / gsz;
+}
+
+__device__ __forceinline__ void tile_of(int pid, int tiles_m, int tiles_n, int& tm, int& tn, int group_m = kGroupM) {
+  tile_at(xcd_contiguous(pid, tiles_m * tiles_n), tiles_m, tiles_n, tm, tn, group_m);
 }
 
 // One operand.  K-contiguous: element (x, k) at ptr[x * ld + k], `rows` = number of valid x.  K-major: element (x, k)

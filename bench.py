@@ -440,7 +440,7 @@ MODE_NAMES = {1: "carry", 0: "recompute"}
 # WRITE_SIZE (one run each) summed over the kernels of one step, each scaled by what the same counter reads for the
 # plain copy kernel of known size (profiles/lmhead_step_cfg2_hbm_traffic.md).  The counters sit behind the L2 of each
 # XCD: what the memory-side cache serves is in these figures too.  Other workloads: not measured.
-LMHEAD_MEASURED_HBM_BYTES = {("cfg2", "carry"): 90.3e9, ("cfg2", "recompute"): 109.8e9}
+LMHEAD_MEASURED_HBM_BYTES = {("cfg2", "carry"): 82.0e9, ("cfg2", "recompute"): 105.4e9}
 
 
 def lmhead_compulsory_bytes(T: int, kept: int, H: int, V: int, mode: str, chunk: int) -> dict:
@@ -454,7 +454,6 @@ def lmhead_compulsory_bytes(T: int, kept: int, H: int, V: int, mode: str, chunk:
     out = dict(
         forward_tiles=n_chunks * w_bytes + 2.0 * T * H + partials + (panel if mode == "carry" else 0.0),
         merge_partials=partials,
-        panel_scale=2.0 * panel if mode == "carry" else 0.0,
         recompute_tiles=(n_chunks * w_bytes + 2.0 * kept * H + panel) if mode == "recompute" else 0.0,
         d_hidden_gemm=panel + n_chunks * w_bytes + 2.0 * kept * H,
         # d_weight: written once in bf16 when one chunk holds every token, else accumulated in fp32 chunk by chunk
@@ -704,11 +703,11 @@ def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: i
         bound="mfma",
         kernel="every kernel of one fused_lm_head_ppo_loss(...) + backward() step: k_lmhead_tiles (logits tiles on the "
                "library's bf16 MFMA tile GEMM, softmax partials per tile, " +
-               ("the un-normalised probabilities of the tokens with a gradient kept in bf16" if mode_name == "carry"
+               ("p_v / p_label of the tokens with a gradient kept in bf16" if mode_name == "carry"
                 else "nothing else written") +
-               "), k_label_logit, k_combine / k_token_loss, " +
-               ("k_panel_scale" if mode_name == "carry" else "k_lmhead_tiles again for the tokens with a gradient") +
-               ", k_gemm_store twice (d_hidden, d_weight)",
+               "), k_label_logit, k_token_loss, " +
+               ("" if mode_name == "carry" else "k_lmhead_tiles again for the tokens with a gradient, ") +
+               "k_gemm_store twice (d_hidden, d_weight; in carry mode they apply the per-token gradient factor)",
         achieved=achieved, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s", frac=achieved / MFMA_BF16_PEAK_TFLOPS,
         traffic=LMHEAD_MEASURED_HBM_BYTES.get((workload, mode_name)),
         timed="HIP events on the launch stream around each of the steps that ms_per_step is the wall-clock mean of",

@@ -146,6 +146,36 @@ def test_carry_redoes_a_chunk_whose_labels_are_too_unlikely_to_store(device):
     assert torch.equal(got[2][:16384], ref[2][:16384])
 
 
+@pytest.mark.parametrize("backward", ["carry", "recompute"])
+def test_gradient_products_with_more_tiles_than_compute_units(device, backward):
+    """9 x 30 = 270 tiles of d(hidden) and 5 x 9 tiles of d(W) with 7600 rows to contract: a grid larger than the chip,
+    with a partly filled last round and ragged edges in both products.  Against the oracle row by row, and bit-equal
+    from call to call."""
+    T, H, V = 7600, 2304, 1088
+    hidden, weight, labels, prox, old, adv, mask = _inputs(T, T, H, V, seed=23, w_std=0.05)
+    mask[:] = True
+    args = [t.to(device) for t in (labels, prox, old, adv)]
+
+    def run():
+        h = hidden.to(device).requires_grad_(True)
+        w = weight.to(device).requires_grad_(True)
+        loss, stat = areal_amd.fused_lm_head_ppo_loss(h, w, *args, eps_clip=0.2, loss_mask=mask.to(device), backward=backward)
+        loss.backward()
+        return loss.detach(), h.grad, w.grad
+
+    o_loss, _, _, _, o_dh, o_dw = _oracle_step(hidden, weight, labels, prox, old, adv, mask, 1.0, 1.0, eps_clip=0.2)
+    loss, dh, dw = run()
+    assert float(loss) == pytest.approx(o_loss, rel=1e-3)
+    assert cosine(dh.cpu().float(), o_dh) > 0.9999 and cosine(dw.cpu().float(), o_dw) > 0.9999
+    assert_same_magnitude(dh, o_dh, what="d(hidden)")
+    assert_same_magnitude(dw, o_dw, what="d(W)")
+    # row by row: one wrong tile would spoil 256 tokens x 256 columns and leave the norms nearly intact
+    err = (dh.cpu().float() - o_dh).abs().amax(dim=1)
+    assert float(err.max()) <= float(o_dh.abs().max()) * 2.0 ** -7
+    loss2, dh2, dw2 = run()
+    assert torch.equal(dh, dh2) and torch.equal(dw, dw2) and torch.equal(loss, loss2)
+
+
 def test_upstream_gradient_scales_both_gradients(device):
     hidden, weight, labels, prox, old, adv, mask = _inputs(260, 260, 64, 704, seed=3)
     args = [t.to(device) for t in (labels, prox, old, adv)]
