@@ -13,7 +13,6 @@
 // so that  logp = ln2 (t_label - log2 s)  and  entropy = ln2 (log2 s - u / s)
 // are differences of small numbers whatever the magnitude of the logits.
 #include "device_utils.h"
-#include "logits_path.h"
 #include "ppo_math.h"
 
 namespace aa {
@@ -262,12 +261,10 @@ __global__ __launch_bounds__(NT) void k_logits_bwd(const void* __restrict__ logi
                                                    const float* __restrict__ row_ez,
                                                    const float* __restrict__ g_logp,
                                                    const float* __restrict__ g_entropy, int64_t T_active,
-                                                   void* __restrict__ dlogits, const int32_t* __restrict__ out_rows) {
+                                                   void* __restrict__ dlogits) {
   const int64_t t = blockIdx.x;
-  const int64_t orow = out_rows ? (int64_t)out_rows[t] : t;  // row map of the gradient, as in the fused kernels
-  if (orow < 0) return;
   const void* row = row_ptr(logits, t, stride, Elem<DT>::kBytes);
-  void* out = (void*)row_ptr(dlogits, orow, stride, Elem<DT>::kBytes);
+  void* out = (void*)row_ptr(dlogits, t, stride, Elem<DT>::kBytes);
   const float gl = (t < T_active) ? g_logp[t] : 0.f;
   const float gh = (t < T_active && g_entropy) ? g_entropy[t] : 0.f;
   if (gl == 0.f && gh == 0.f) {
@@ -306,9 +303,6 @@ struct FusedTokenArgs {
   uint8_t* flags;
   aa_ppo_params P;
   int64_t T_active;
-  // Optional row map of the gradient: row t is written to dlogits row out_rows[t]; a negative entry means the row
-  // is not written at all (its token has no gradient).  Null: row t goes to row t.
-  const int32_t* out_rows;
 };
 
 // Per-token inputs of the loss, fetched ahead of the row statistics so that
@@ -422,9 +416,8 @@ __global__ __launch_bounds__(NT) void k_fused_generic(const void* __restrict__ l
   load_loss_scale(a, fn, gscale);
   // one row per trip; with fewer workgroups than rows (T_rows > gridDim.x) a workgroup walks rows t, t + grid, ...
   for (int64_t t = blockIdx.x; t < T_rows; t += gridDim.x) {
-    const int64_t orow = a.out_rows ? (int64_t)a.out_rows[t] : t;
     const void* row = row_ptr(logits, t, stride, Elem<DT>::kBytes);
-    void* out = (void*)row_ptr(dlogits, orow < 0 ? 0 : orow, stride, Elem<DT>::kBytes);
+    void* out = (void*)row_ptr(dlogits, t, stride, Elem<DT>::kBytes);
     const int64_t y = labels[t];
     const bool y_ok = (y >= 0) && (y < V);
     const float xy = y_ok ? Elem<DT>::load1(row, y) : 0.f;
@@ -434,7 +427,7 @@ __global__ __launch_bounds__(NT) void k_fused_generic(const void* __restrict__ l
     const RowOut ro = finish_row(rs);
     const float lp = y_ok ? label_logp(xy, c, rs, ro) : __builtin_nanf("");
     const float g = fused_token_tail(a, t, tin, fn, gscale, lp, rs, ro, threadIdx.x == 0);
-    if (orow >= 0) {  // uniform over the workgroup
+    {
       if (g == 0.f) {
         row_zero_generic<DT, NT>(row, out, V, vec_ok != 0);
       } else {
@@ -470,9 +463,8 @@ __global__ __launch_bounds__(1024) void k_fused_f32_hold(const float* __restrict
   float fn, gscale;
   load_loss_scale(a, fn, gscale);
   for (int64_t t = blockIdx.x; t < T_rows; t += gridDim.x) {
-    const int64_t orow = a.out_rows ? (int64_t)a.out_rows[t] : t;
     const float* row = logits + t * stride;
-    float* out = dlogits + (orow < 0 ? 0 : orow) * stride;
+    float* out = dlogits + t * stride;
     const int64_t y = labels[t];
     const bool y_ok = (y >= 0) && (y < V);
     const float xy = y_ok ? row[y] : 0.f;
@@ -512,7 +504,7 @@ __global__ __launch_bounds__(1024) void k_fused_f32_hold(const float* __restrict
     const float g = fused_token_tail(a, t, tin, fn, gscale, lp, rs, ro, tid == 0);
 
     // pass 2: the gradient row (every thread reads back only what it stored itself: no barrier needed)
-    if (orow >= 0) {  // uniform over the workgroup
+    {
       if (g == 0.f) {
         const float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         for (int e0 = tid * 8; e0 < V; e0 += kHoldChunk) store8<AA_F32>(out, e0, z);
@@ -757,7 +749,6 @@ void k_fused_regs(const uint4* __restrict__ logits, int V, int64_t stride_vec,
   bool y_ok = (y >= 0) && (y < V);
   uint32_t xy_raw = load_u16_uniform(src, y_ok ? y : 0);
   TokenIn tin = load_token_in_ro(in_prox, in_adv, in_mask32, mask_mis, in_bw, has_w, a.T_active, t);
-  int64_t orow = a.out_rows ? (int64_t)a.out_rows[t] : t;  // where the gradient of this row goes; < 0: nowhere
 
   for (;;) {
     // claim the row after this one; the answer is picked up behind the barriers of block_stats
@@ -865,11 +856,8 @@ void k_fused_regs(const uint4* __restrict__ logits, int V, int64_t stride_vec,
     const bool y_ok_n = (y_n >= 0) && (y_n < V);
     const uint32_t xy_raw_n = load_u16_uniform(src_n, y_ok_n ? y_n : 0);
     const TokenIn tin_n = load_token_in_ro(in_prox, in_adv, in_mask32, mask_mis, in_bw, has_w, a.T_active, more ? tn : t);
-    const int64_t orow_n = a.out_rows ? (int64_t)a.out_rows[more ? tn : t] : tn;
 
-    // a row that is not to be written gets an empty descriptor: the hardware drops every store
-    const __amdgpu_buffer_rsrc_t wsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)(dlogits + (orow < 0 ? 0 : orow) * stride_vec), 0, orow < 0 ? 0 : V * 2, kBufferFlags);
+    const __amdgpu_buffer_rsrc_t wsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(dlogits + t * stride_vec), 0, V * 2, kBufferFlags);
     if constexpr (EXT) {
       if (g != 0.f) {
 #pragma unroll
@@ -920,7 +908,7 @@ void k_fused_regs(const uint4* __restrict__ logits, int V, int64_t stride_vec,
         load_lds_chunks(rsrc_n);
       }
     }
-    t = tn; y = y_n; y_ok = y_ok_n; xy_raw = xy_raw_n; tin = tin_n; orow = orow_n;
+    t = tn; y = y_n; y_ok = y_ok_n; xy_raw = xy_raw_n; tin = tin_n;
   }
   if (work && tid == 0) {
     __threadfence();
@@ -1093,13 +1081,6 @@ extern "C" int aa_logits_bwd(const void* logits, int dtype, int64_t T, int64_t V
                              const int64_t* labels, float inv_temperature, const float* row_lse,
                              const float* row_ez, const float* g_logp, const float* g_entropy, int64_t T_active,
                              void* dlogits, void* stream) {
-  return aa::logits_bwd_rows(logits, dtype, T, V, row_stride, labels, inv_temperature, row_lse, row_ez, g_logp, g_entropy,
-                             T_active, dlogits, nullptr, stream);
-}
-
-int aa::logits_bwd_rows(const void* logits, int dtype, int64_t T, int64_t V, int64_t row_stride, const int64_t* labels,
-                        float inv_temperature, const float* row_lse, const float* row_ez, const float* g_logp,
-                        const float* g_entropy, int64_t T_active, void* dlogits, const int32_t* out_rows, void* stream) {
   if (!common_args_ok(logits, dtype, T, V, row_stride, labels)) return AA_ERR_INVALID_ARGUMENT;
   if (!row_lse || !g_logp || !dlogits || (g_entropy && !row_ez)) return AA_ERR_INVALID_ARGUMENT;
   if (T_active < 0 || T_active > T || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
@@ -1108,7 +1089,7 @@ int aa::logits_bwd_rows(const void* logits, int dtype, int64_t T, int64_t V, int
   constexpr int NT = 256;
 #define AA_LAUNCH(DT)                                                                                        \
   hipLaunchKernelGGL((k_logits_bwd<DT, NT>), dim3((unsigned)T), dim3(NT), 0, st, logits, (int)V, row_stride, \
-                     labels, inv_temperature, vec_ok, row_lse, row_ez, g_logp, g_entropy, T_active, dlogits, out_rows)
+                     labels, inv_temperature, vec_ok, row_lse, row_ez, g_logp, g_entropy, T_active, dlogits)
   if (dtype == AA_BF16) AA_LAUNCH(AA_BF16);
   else if (dtype == AA_F16) AA_LAUNCH(AA_F16);
   else AA_LAUNCH(AA_F32);
@@ -1123,17 +1104,6 @@ extern "C" int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int
                                    const float* grad_scale, float* logp, float* entropy, float* vmax, float* vmin,
                                    float* stat_loss, float* ratio, uint8_t* flags, void* dlogits, int32_t* work,
                                    void* stream) {
-  return aa::logits_ppo_fused_rows(logits, dtype, T, V, row_stride, labels, inv_temperature, T_active, prox_logp, adv,
-                                   mask_eff, behave_w, params, n_valid, grad_scale, logp, entropy, vmax, vmin, stat_loss,
-                                   ratio, flags, dlogits, nullptr, work, stream);
-}
-
-int aa::logits_ppo_fused_rows(const void* logits, int dtype, int64_t T, int64_t V, int64_t row_stride,
-                              const int64_t* labels, float inv_temperature, int64_t T_active, const float* prox_logp,
-                              const float* adv, const uint8_t* mask_eff, const float* behave_w,
-                              const aa_ppo_params* params, const int32_t* n_valid, const float* grad_scale, float* logp,
-                              float* entropy, float* vmax, float* vmin, float* stat_loss, float* ratio, uint8_t* flags,
-                              void* dlogits, const int32_t* out_rows, int32_t* work, void* stream) {
   if (!common_args_ok(logits, dtype, T, V, row_stride, labels)) return AA_ERR_INVALID_ARGUMENT;
   if (!params || !n_valid || !logp || !dlogits) return AA_ERR_INVALID_ARGUMENT;
   if (T_active < 0 || T_active > T || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
@@ -1156,7 +1126,6 @@ int aa::logits_ppo_fused_rows(const void* logits, int dtype, int64_t T, int64_t 
   a.logp = logp; a.entropy = entropy; a.vmax = vmax; a.vmin = vmin;
   a.stat_loss = stat_loss; a.ratio = ratio; a.flags = flags;
   a.P = *params; a.T_active = T_active;
-  a.out_rows = out_rows;
 
   const bool fast = (dtype != AA_F32) && (V % 8 == 0) && (row_stride % 8 == 0) && (((uintptr_t)logits & 15) == 0) &&
                     (((uintptr_t)dlogits & 15) == 0) && (V > kTwoPassMaxV) && (V <= kMaxExtChunks * 8192) && (T_active > 0);
