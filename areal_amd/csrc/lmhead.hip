@@ -32,7 +32,9 @@ using namespace gemm;
 
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
-constexpr int kChunkTokens = 16384;        // token chunk of the panel
+// token chunk of the panel.  Measured: with 32768 the forward tiles run 2.4 % slower at H = 4096 (the hidden rows of
+// a chunk, 2 * chunk * H bytes, no longer fit the 256 MB memory-side cache that every band of tiles re-reads them from)
+constexpr int kChunkTokens = 16384;
 constexpr int kPanelPitch = BM + 8;        // pitch (elements) of the tile staged in LDS as [token][vocab]
 constexpr int kStageBytes = 256 * kPanelPitch * 2;  // 135168 B, inside the 160 KiB the main loop uses
 static_assert(kStageBytes <= kLdsBytes, "the staged tile must fit the main loop's LDS");

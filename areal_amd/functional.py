@@ -743,7 +743,7 @@ def lm_head_logprobs_entropy(
     ``hidden`` is ``[T, H]`` and ``weight`` ``[V, H]`` (the lm_head), both bf16.  The forward forms 256 x 256 tiles of
     the logits in the accumulator registers of the library's bf16 MFMA tile GEMM (fp32 accumulation, not rounded to
     bf16 in between) and reduces each tile to softmax partials per token in the GEMM's epilogue; its only scratch
-    memory is those partials (about ``24 * V / 256`` bytes per token of a 16384-token chunk, 0.3 GB at
+    memory is those partials (about ``24 * V / 256`` bytes per token of a chunk of at most 16384 tokens, 0.23 GB at
     ``V = 151936``).  Differentiable in ``hidden`` and ``weight``: the backward goes through the tokens in chunks of at
     most 16384, forms the chunk's logits tiles again, writes their gradient as bf16 rows (of the tokens whose upstream
     gradient is not zero) into a workspace panel ``[chunk, V]`` and contracts that panel with the weight and with the
@@ -917,7 +917,7 @@ def fused_lm_head_ppo_loss(
     size the GEMMs, so the host reads them (one small device-to-host copy that waits for the mask only) before it
     queues the chunk.  ``False`` multiplies the zero rows through, as the reference's autograd does, without that
     read.  A caller that already knows the counts on the host (the number of tokens with a non-zero effective mask
-    in each chunk of 16384 tokens, e.g. from the CPU copy of ``loss_mask`` when there is no rejection sampling) can
+    in each chunk of ``aa_lmhead_chunk_tokens()`` tokens, e.g. from the CPU copy of ``loss_mask`` when there is no rejection sampling) can
     pass them as ``kept_per_chunk``; nothing is read back then.
 
     ``forward_masked_tokens=False`` (token level only) goes one step further than the reference's semantics: tokens

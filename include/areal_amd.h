@@ -580,16 +580,18 @@ int aa_masked_moments(const float* const* values, int n_tensors,
 /* logits = hidden @ weight.T followed by the logits path above)           */
 /* ------------------------------------------------------------------ */
 
-/* Bytes of workspace aa_lmhead_bwd / aa_lmhead_ppo_fused need for these sizes:
- * about 4 * min(T, 16384) * V bytes (the bf16 d(logits) rows of one token chunk
- * and their transposed copy), 2 * H * V (a transposed copy of the weight),
- * 24 * (V / 256) * min(T, 16384) (softmax partials per 128 vocabulary rows and
- * token), plus 4 * H * V (an fp32 accumulator for a bf16 d_weight) when
- * T > 16384.  Returns -1 for sizes the path does not take. */
+/* Bytes of workspace aa_lmhead_bwd / aa_lmhead_ppo_fused need for these sizes.
+ * With C = min(T, aa_lmhead_chunk_tokens()): 2 * C * V (the bf16 d(logits)
+ * rows of one token chunk), 24 * (V / 256) * C (softmax partials per 128
+ * vocabulary rows and token), 2 * C * H (the hidden rows of the tokens with a
+ * gradient, closed up), plus 4 * H * V (an fp32 accumulator for a bf16
+ * d_weight) when there is more than one chunk.  No transposed copy of anything
+ * is made.  Returns -1 for sizes the path does not take. */
 int64_t aa_lmhead_workspace_bytes(int64_t T, int64_t H, int64_t V);
 
 /* Bytes of workspace aa_lmhead_fwd alone needs: the softmax partials only,
- * about 24 * (V / 256) * min(T, 16384) bytes (0.3 GB at V = 151936). */
+ * about 24 * (V / 256) * min(T, aa_lmhead_chunk_tokens()) bytes (0.23 GB at
+ * T = 16384, V = 151936). */
 int64_t aa_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);
 
 /* Tokens per chunk of the lm_head entry points (16384). */
@@ -638,7 +640,7 @@ int64_t aa_lmhead_fwd_static_max_vocab(void);
  * (overwritten), given g_logp and optional g_entropy.  d_weight_dtype is
  * AA_F32 or AA_BF16; either way the sum over tokens is accumulated in fp32
  * (bf16: rounded once at the end).
- * Per chunk of 16384 tokens: the logits tiles are formed again and turned into
+ * Per chunk of tokens: the logits tiles are formed again and turned into
  * bf16 d(logits) rows in the GEMM's epilogue (a panel [rows, V] in the
  * workspace), which two more tile GEMMs contract with the weight and with the
  * hidden states (6 T V H flops for the 4 T V H of the backward).
@@ -681,7 +683,7 @@ typedef enum {
  * -> gather_logprobs_entropy (vocab_parallel.py:434-469) ->
  * ppo_actor_loss_fn (functional.py:429-559) -> autograd back to the hidden
  * states and the lm_head weight.  Tokens are processed in chunks of at most
- * 16384.  Per chunk: the forward tiles of aa_lmhead_fwd; one kernel that
+ * aa_lmhead_chunk_tokens().  Per chunk: the forward tiles of aa_lmhead_fwd; one kernel that
  * merges the softmax partials into log-prob and entropy and evaluates the
  * per-token loss and its derivative; the bf16 d(logits) rows of the tokens
  * with gradient (backward_mode says how they are obtained); and the two tile

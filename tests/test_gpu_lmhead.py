@@ -9,9 +9,12 @@ import torch
 
 import areal_amd
 import oracle
+from areal_amd import _native
 from helpers import assert_same_magnitude, assert_within, assert_within_one_bf16_logit_step, cosine
 
 pytestmark = pytest.mark.gpu
+
+CHUNK = int(_native.load().aa_lmhead_chunk_tokens())  # tokens per chunk of the lm_head entry points
 
 
 def _case(T, H, V, seed, w_std=0.02):
@@ -184,7 +187,7 @@ def test_full_size_configuration(device, name):
     assert torch.equal(dh_all, dh_again) and torch.equal(dw_all, dw_again)
 
 
-@pytest.mark.parametrize("T,H,V", [(300, 128, 1088), (16384 + 72, 64, 640)])  # one chunk; two chunks
+@pytest.mark.parametrize("T,H,V", [(300, 128, 1088), (CHUNK + 72, 64, 640)])  # one chunk; two chunks
 def test_weight_gradient_dtypes_through_the_c_abi(device, T, H, V):
     """aa_lmhead_bwd with d_weight as fp32 and as bf16: the fp32 result against autograd of the oracle, and the bf16
     result equal to it up to one rounding (the sum over tokens is kept in fp32 in both)."""
@@ -237,13 +240,13 @@ def test_backward_leaves_out_rows_without_gradient(device):
     from areal_amd import _native as N
     from areal_amd import functional as F
 
-    T, H, V = 16384 + 520, 64, 1088
+    T, H, V = CHUNK + 520, 64, 1088
     hidden, weight, labels = _case(T, H, V, seed=77, w_std=0.3)
     g = torch.Generator().manual_seed(78)
     gl = torch.randn(T, generator=g) * (torch.rand(T, generator=g) < 0.4)
     gh = 0.2 * torch.randn(T, generator=g) * (torch.rand(T, generator=g) < 0.1)
-    gl[16384:] = 0.0
-    gh[16384:] = 0.0                                   # the second chunk has no gradient at all
+    gl[CHUNK:] = 0.0
+    gh[CHUNK:] = 0.0                                   # the second chunk has no gradient at all
     h_d = hidden.to(device).requires_grad_(True)
     w_d = weight.to(device).requires_grad_(True)
     lp, ent = areal_amd.lm_head_logprobs_entropy(h_d, w_d, labels.to(device))

@@ -8,10 +8,13 @@ import torch
 
 import areal_amd
 import oracle
+from areal_amd import _native
 from areal_amd import RejectionSamplingConfig
 from helpers import assert_same_magnitude, assert_within, cosine
 
 pytestmark = pytest.mark.gpu
+
+CHUNK = int(_native.load().aa_lmhead_chunk_tokens())  # tokens per chunk of the lm_head entry points
 
 
 def _inputs(T_pad, T, H, V, seed, w_std=0.3):
@@ -43,7 +46,7 @@ CASES = [
     # T_pad, T, H, V, temperature, loss_scale, options
     (300, 300, 128, 1088, 1.0, 1.0, dict(eps_clip=0.2)),                                    # ragged last tiles
     (520, 500, 64, 8256, 0.8, 0.37, dict(eps_clip=0.2, eps_clip_higher=0.28, c_clip=3.0)),  # batch padding, dual clip
-    (16384 + 200, 16384 + 130, 64, 640, 1.0, 1.0, dict(eps_clip=0.2, rs=True)),             # two token chunks
+    (CHUNK + 200, CHUNK + 130, 64, 640, 1.0, 1.0, dict(eps_clip=0.2, rs=True)),             # two token chunks
     (203, 203, 200, 1096, 1.3, 1.0, dict(eps_clip=0.2)),                                    # H, V multiples of 8 only
 ]
 
@@ -109,15 +112,15 @@ def test_carry_redoes_a_chunk_whose_labels_are_too_unlikely_to_store(device):
     fit that range, and its chunk is redone by the recompute tiles, decided on the device.  Logits with a spread of
     about 48 put many labels there; the second chunk of the batch has ordinary logits and stays on the carried rows.
     Both must match the oracle and the recompute mode."""
-    T, H, V = 16384 + 300, 64, 1088
+    T, H, V = CHUNK + 300, 64, 1088
     g = torch.Generator().manual_seed(5)
     hidden = torch.randn(T, H, generator=g)
-    hidden[:16384] *= 12.0                     # first chunk: logits ~ N(0, 48^2)
+    hidden[:CHUNK] *= 12.0                     # first chunk: logits ~ N(0, 48^2)
     hidden = hidden.bfloat16()
     weight = (0.5 * torch.randn(V, H, generator=g)).bfloat16()
     labels = torch.randint(0, V, (T,), generator=g)
     ref_lp = oracle.logprobs(oracle.lmhead_logits(hidden, weight), labels)
-    assert int((ref_lp[:16384] < -80).sum()) > 100 and float(ref_lp[16384:].min()) > -60
+    assert int((ref_lp[:CHUNK] < -80).sum()) > 100 and float(ref_lp[CHUNK:].min()) > -60
     prox = ref_lp + 0.05 * torch.randn(T, generator=g)
     old = ref_lp + 0.3 * torch.randn(T, generator=g)
     adv = torch.randn(T, generator=g)
@@ -143,7 +146,7 @@ def test_carry_redoes_a_chunk_whose_labels_are_too_unlikely_to_store(device):
         assert_same_magnitude(a, o, what=name)
         assert cosine(a.cpu(), b.cpu()) > 0.99999, name
     # the flagged chunk came out of the recompute tiles: its d(hidden) rows are those of the recompute mode, bit for bit
-    assert torch.equal(got[2][:16384], ref[2][:16384])
+    assert torch.equal(got[2][:CHUNK], ref[2][:CHUNK])
 
 
 @pytest.mark.parametrize("backward", ["carry", "recompute"])
@@ -258,7 +261,7 @@ def test_full_size_step_agrees_with_unfused_path(device, backward):
 
 def test_padding_only_chunk_and_no_active_token(device):
     g = torch.Generator().manual_seed(0)
-    T_pad, T, H, V = 16384 + 300, 16384, 64, 640           # the second token chunk is batch padding only
+    T_pad, T, H, V = CHUNK + 300, CHUNK, 64, 640           # the second token chunk is batch padding only
     hidden = torch.randn(T_pad, H, generator=g).bfloat16().to(device).requires_grad_(True)
     weight = (0.3 * torch.randn(V, H, generator=g)).bfloat16().to(device).requires_grad_(True)
     labels = torch.randint(0, V, (T_pad,), generator=g).to(device)
@@ -287,7 +290,7 @@ def test_skipping_masked_tokens_equals_the_dense_backward(device, pattern):
     """Tokens with a zero mask are left out of the gradient GEMMs: same loss and statistics, same gradients as when
     their zero rows are multiplied through (two token chunks, batch padding at the end)."""
     g = torch.Generator().manual_seed(5)
-    T_pad, T, H, V = 16384 + 300, 16384 + 200, 64, 8200
+    T_pad, T, H, V = CHUNK + 300, CHUNK + 200, 64, 8200
     if pattern == "random_long_rows":
         V = 180224
     hidden = torch.randn(T_pad, H, generator=g).bfloat16().to(device)
@@ -301,14 +304,14 @@ def test_skipping_masked_tokens_equals_the_dense_backward(device, pattern):
     adv = torch.randn(T, generator=g).to(device)
     mask = (torch.rand(T, generator=g) < 0.5).to(device)
     if pattern == "second_chunk_masked":
-        mask[16384:] = False
+        mask[CHUNK:] = False
     elif pattern == "first_chunk_masked":
-        mask[:16384] = False
+        mask[:CHUNK] = False
     elif pattern == "all_masked":
         mask[:] = False
     elif pattern == "one_token":
         mask[:] = False
-        mask[16384 + 7] = True
+        mask[CHUNK + 7] = True
     rs = RejectionSamplingConfig(level="token", action="mask", metric="ratio", upper=1.3)
 
     def run(skip):
@@ -375,9 +378,9 @@ def test_not_forwarding_masked_tokens_keeps_loss_and_gradients(device, with_rs):
 
 
 def test_counts_from_the_caller_replace_the_read_back(device):
-    hidden, weight, labels, prox, old, adv, mask = _inputs(16384 + 256, 16384 + 200, 64, 640, seed=41)
+    hidden, weight, labels, prox, old, adv, mask = _inputs(CHUNK + 256, CHUNK + 200, 64, 640, seed=41)
     args = [t.to(device) for t in (labels, prox, old, adv)]
-    counts = [int(mask[:16384].sum()), int(mask[16384:].sum())]            # known on the host
+    counts = [int(mask[:CHUNK].sum()), int(mask[CHUNK:].sum())]            # known on the host
 
     def run(**kw):
         h = hidden.to(device).requires_grad_(True)
