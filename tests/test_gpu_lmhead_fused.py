@@ -393,3 +393,89 @@ def test_counts_from_the_caller_replace_the_read_back(device):
     assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]) and torch.equal(a[2], b[2])
     with pytest.raises(ValueError, match="one count per chunk"):
         run(kept_per_chunk=[1])
+
+
+@pytest.mark.parametrize("backward", ["carry", "recompute"])
+@pytest.mark.parametrize("skip", [True, False])
+def test_labels_outside_the_vocabulary_at_masked_tokens(device, backward, skip):
+    """Tokens without a mask may carry any label (prompt positions, batch padding filled with -100): their log-prob is
+    NaN, as on the logits path, and nothing of it reaches the loss or the gradients, with or without their rows in
+    the gradient products."""
+    T, H, V = 700, 64, 1088
+    hidden, weight, labels, prox, old, adv, mask = _inputs(T, T, H, V, seed=77)
+    bad = ~mask
+    labels = labels.clone()
+    labels[bad] = torch.where(torch.arange(T)[bad] % 2 == 0, torch.tensor(-100), torch.tensor(V + 3))
+    prox[bad], old[bad] = 0.0, 0.0
+    h = hidden.to(device).requires_grad_(True)
+    w = weight.to(device).requires_grad_(True)
+    loss, stat = areal_amd.fused_lm_head_ppo_loss(h, w, labels.to(device), prox.to(device), old.to(device), adv.to(device),
+                                                  eps_clip=0.2, loss_mask=mask.to(device), backward=backward,
+                                                  skip_masked_tokens=skip)
+    loss.backward()
+    assert torch.isnan(stat["logprobs"].cpu()[bad]).all() and torch.isfinite(stat["logprobs"].cpu()[mask]).all()
+    ok_labels = torch.where(bad, torch.zeros_like(labels), labels)      # the oracle needs labels it can gather
+    o_loss, _, o_lp, _, o_dh, o_dw = _oracle_step(hidden, weight, ok_labels, prox, old, adv, mask, 1.0, 1.0, eps_clip=0.2)
+    assert float(loss.detach()) == pytest.approx(o_loss, rel=1e-3)
+    assert torch.isfinite(h.grad).all() and torch.isfinite(w.grad).all()
+    assert cosine(h.grad.cpu().float(), o_dh) > 0.9999 and cosine(w.grad.cpu().float(), o_dw) > 0.9999
+    assert_same_magnitude(h.grad, o_dh, what="d(hidden)")
+    assert_same_magnitude(w.grad, o_dw, what="d(W)")
+    assert float(h.grad.cpu()[bad].abs().sum()) == 0.0
+
+
+@pytest.mark.parametrize("backward", ["carry", "recompute"])
+def test_step_replays_from_a_hip_graph(device, backward):
+    """aa_lmhead_ppo_fused allocates nothing, clears memory with kernels only and never waits for the device, so the
+    whole step (every token's row in the gradient products: no count has to reach the host) can be captured into a HIP
+    graph.  Three replays on new inputs, with eager work and synchronisations in between, each equal to the eager
+    result on the same inputs."""
+    T, H, V = 600, 128, 1088
+    g = torch.Generator().manual_seed(3)
+    h = torch.zeros(T, H, dtype=torch.bfloat16, device=device, requires_grad=True)
+    w = torch.zeros(V, H, dtype=torch.bfloat16, device=device, requires_grad=True)
+    labels = torch.randint(0, V, (T,), generator=g).to(device)
+    prox, old, adv = (torch.zeros(T, device=device) for _ in range(3))
+    mask = (torch.rand(T, generator=g) < 0.7).to(device)
+    kw = dict(eps_clip=0.2, loss_mask=mask, eps_clip_higher=0.28, backward=backward, skip_masked_tokens=False)
+
+    def fill(seed):
+        gg = torch.Generator().manual_seed(seed)
+        with torch.no_grad():
+            h.copy_(torch.randn(T, H, generator=gg).bfloat16())
+            w.copy_((0.3 * torch.randn(V, H, generator=gg)).bfloat16())
+            ref, _ = areal_amd.lm_head_logprobs_entropy(h, w, labels)
+            prox.copy_(ref + 0.05 * torch.randn(T, generator=gg).to(device))
+            old.copy_(ref + 0.05 * torch.randn(T, generator=gg).to(device))
+            adv.copy_(torch.randn(T, generator=gg).to(device))
+
+    def step():
+        loss, stat = areal_amd.fused_lm_head_ppo_loss(h, w, labels, prox, old, adv, **kw)
+        loss.backward()
+        return loss, stat["logprobs"]
+
+    fill(0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            h.grad, w.grad = None, None
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    h.grad, w.grad = None, None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        g_loss, g_logp = step()
+    g_dh, g_dw = h.grad, w.grad
+    for seed in (1, 2, 3):
+        fill(seed)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = (g_loss.detach().clone(), g_logp.clone(), g_dh.clone(), g_dw.clone())
+        h2 = h.detach().clone().requires_grad_(True)                    # eager, same inputs
+        w2 = w.detach().clone().requires_grad_(True)
+        e_loss, e_stat = areal_amd.fused_lm_head_ppo_loss(h2, w2, labels, prox, old, adv, **kw)
+        e_loss.backward()
+        torch.cuda.synchronize()
+        assert torch.equal(got[0], e_loss.detach()) and torch.equal(got[1], e_stat["logprobs"])
+        assert torch.equal(got[2], h2.grad) and torch.equal(got[3], w2.grad)
