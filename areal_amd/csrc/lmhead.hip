@@ -6,8 +6,8 @@
 //
 // Forward (aa_lmhead_fwd, and the first half of the training step): 256 (vocabulary) x 256 (tokens) tiles of the
 // logits are formed in accumulator registers; the epilogue reduces every 128-row block of a tile to the softmax
-// partials (k, s, u) per token and captures the label logit; a small kernel merges the partials of all blocks into
-// log-prob and entropy.  Nothing of size T x V is written.
+// partials (k, s, u) per token; the label's logit comes from a dot product per token (k_label_logit), and a small
+// kernel merges the partials of all blocks into log-prob and entropy.  Nothing of size T x V is written.
 //
 // Backward needs d(logits) twice (for d_hidden and for d_weight), so a bf16 panel [tokens with gradient, V] of it is
 // written once per token chunk and contracted by two plain tile GEMMs (which read the panel, the weight and the
@@ -37,7 +37,7 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 constexpr int kChunkTokens = 16384;
 constexpr int kPanelPitch = BM + 8;        // pitch (elements) of the tile staged in LDS as [token][vocab]
 constexpr int kStageBytes = 256 * kPanelPitch * 2;  // 135168 B, inside the 160 KiB the main loop uses
-static_assert(kStageBytes <= kLdsBytes, "the staged tile must fit the main loop's LDS");
+static_assert(kStageBytes + 256 * 4 <= kLdsBytes, "the staged tile and its 256 row numbers must fit the main loop's LDS");
 
 __host__ __device__ __forceinline__ int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
@@ -48,7 +48,7 @@ struct TileArgs {
   float* pk;
   float* ps;
   float* pu;
-  float* xy;              // [tokens of the chunk] raw label logit, written by the block that holds the label
+  float* xy;              // [tokens of the chunk] raw label logit (k_label_logit, before the tiles run)
   const int64_t* labels;  // labels of the chunk
   int64_t pitch_t;
   float c;                // log2(e) / temperature

@@ -1,7 +1,8 @@
 /*
  * A consumer of the C ABI written in plain C, with nothing but the HIP runtime beside it: device buffers from
  * hipMalloc, the library's entry points, and the expected values computed right here in double precision from the
- * definitions (log-softmax, entropy, the supervised loss and its gradient).  Exit status 0 = every check passed.
+ * definitions (log-softmax, entropy, the supervised loss and its gradient; for the lm_head entry points the product
+ * hidden @ weight.T as well).  Exit status 0 = every check passed.
  *
  * Build (done by __graft_entry__.build()):
  *   gcc -std=c99 -D__HIP_PLATFORM_AMD__ -I/opt/rocm/include -Iinclude tests/c_abi/consumer.c \
@@ -18,6 +19,10 @@
 
 #define T 7
 #define V 1003
+/* lm_head part: hidden [LT, LH] and weight [LV, LH] in bf16 */
+#define LT 40
+#define LH 64
+#define LV 520
 
 #define HIP_OK(call)                                                                 \
   do {                                                                               \
@@ -136,6 +141,75 @@ int main(void) {
   /* a bad argument is refused before anything is queued */
   ok &= aa_logits_fwd(d_logits, AA_F32, T, V, V, d_labels, 0.0f, d_logp, NULL, NULL, NULL, NULL, NULL, NULL) ==
         AA_ERR_INVALID_ARGUMENT;
+
+  /* lm_head: log-prob and entropy of softmax(hidden @ weight.T / temperature) without the logits in memory, through
+   * aa_lmhead_fwd (workspace from the caller) and aa_lmhead_fwd_static (no workspace, nothing allocated).  The bf16
+   * inputs are small multiples of 1/64 (hidden) and 1/256 (weight), exact in bf16, so the products are exact. */
+  {
+    static uint16_t hid[LT * LH], wgt[LV * LH];
+    static double hid_d[LT * LH], wgt_d[LV * LH];
+    int64_t llabels[LT];
+    for (int i = 0; i < LT * LH + LV * LH; ++i) {
+      state = state * 1664525u + 1013904223u;
+      const int k = (int)((state >> 8) % 255u) - 127; /* -127 .. 127 */
+      const int is_w = i >= LT * LH;
+      const float f = (float)k / (is_w ? 256.0f : 64.0f); /* weights a quarter of the hidden states' range */
+      uint32_t bits;
+      memcpy(&bits, &f, 4);
+      if (is_w) { wgt[i - LT * LH] = (uint16_t)(bits >> 16); wgt_d[i - LT * LH] = f; }
+      else { hid[i] = (uint16_t)(bits >> 16); hid_d[i] = f; }
+    }
+    double want_lp[LT], want_ent[LT];
+    for (int t = 0; t < LT; ++t) {
+      static double z[LV];
+      double mx = -1e300, sum = 0.0, u = 0.0;
+      llabels[t] = (t * 37 + 11) % LV;
+      for (int v = 0; v < LV; ++v) {
+        double acc = 0.0;
+        for (int h = 0; h < LH; ++h) acc += hid_d[t * LH + h] * wgt_d[v * LH + h];
+        z[v] = acc * inv_temperature;
+        mx = fmax(mx, z[v]);
+      }
+      for (int v = 0; v < LV; ++v) { sum += exp(z[v] - mx); u += exp(z[v] - mx) * z[v]; }
+      want_lp[t] = z[llabels[t]] - (mx + log(sum));
+      want_ent[t] = (mx + log(sum)) - u / sum;
+    }
+    uint16_t *d_hid, *d_wgt;
+    int64_t* d_ll;
+    float *d_lp, *d_ent, *d_lp2, *d_ent2;
+    void* d_ws;
+    const int64_t ws_bytes = aa_lmhead_fwd_workspace_bytes(LT, LH, LV);
+    if (ws_bytes <= 0) return 5;
+    HIP_OK(hipMalloc((void**)&d_hid, sizeof(hid)));
+    HIP_OK(hipMalloc((void**)&d_wgt, sizeof(wgt)));
+    HIP_OK(hipMalloc((void**)&d_ll, sizeof(llabels)));
+    HIP_OK(hipMalloc((void**)&d_lp, LT * sizeof(float)));
+    HIP_OK(hipMalloc((void**)&d_ent, LT * sizeof(float)));
+    HIP_OK(hipMalloc((void**)&d_lp2, LT * sizeof(float)));
+    HIP_OK(hipMalloc((void**)&d_ent2, LT * sizeof(float)));
+    HIP_OK(hipMalloc(&d_ws, (size_t)ws_bytes));
+    HIP_OK(hipMemcpy(d_hid, hid, sizeof(hid), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d_wgt, wgt, sizeof(wgt), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d_ll, llabels, sizeof(llabels), hipMemcpyHostToDevice));
+    AA_CHECK(aa_lmhead_fwd(d_hid, d_wgt, LT, LH, LV, d_ll, inv_temperature, d_lp, d_ent, NULL, NULL, d_ws, ws_bytes, NULL));
+    AA_CHECK(aa_lmhead_fwd_static(d_hid, d_wgt, LT, LH, LV, d_ll, inv_temperature, d_lp2, d_ent2, NULL, NULL, NULL));
+    HIP_OK(hipDeviceSynchronize());
+    float lp[LT], ent[LT], lp2[LT], ent2[LT];
+    HIP_OK(hipMemcpy(lp, d_lp, sizeof(lp), hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(ent, d_ent, sizeof(ent), hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(lp2, d_lp2, sizeof(lp2), hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(ent2, d_ent2, sizeof(ent2), hipMemcpyDeviceToHost));
+    for (int t = 0; t < LT; ++t) {
+      ok &= close_to(lp[t], want_lp[t], 5e-6, "lm_head logp", t);
+      ok &= close_to(ent[t], want_ent[t], 5e-6, "lm_head entropy", t);
+      ok &= lp[t] == lp2[t] && ent[t] == ent2[t]; /* the two entry points run the same kernels */
+    }
+    /* H must be a multiple of 8 */
+    ok &= aa_lmhead_fwd(d_hid, d_wgt, LT, LH - 4, LV, d_ll, inv_temperature, d_lp, d_ent, NULL, NULL, d_ws, ws_bytes, NULL) ==
+          AA_ERR_UNSUPPORTED;
+    hipFree(d_hid); hipFree(d_wgt); hipFree(d_ll); hipFree(d_lp); hipFree(d_ent); hipFree(d_lp2); hipFree(d_ent2);
+    hipFree(d_ws);
+  }
 
   hipFree(d_logits); hipFree(d_labels); hipFree(d_mask); hipFree(d_logp); hipFree(d_entropy); hipFree(d_g);
   hipFree(d_stat); hipFree(d_loss); hipFree(d_ppl); hipFree(d_count); hipFree(d_cu); hipFree(d_seq_count);
