@@ -14,7 +14,8 @@
 // and A(k+2) is in flight; the only wait for memory is a counted vmcnt that leaves the youngest unit outstanding, and
 // the one barrier per slice (before its last 16-wide step) both publishes slice k + 1 and retires A(k), B(k), whose
 // slots the next loads take.  What happens to the accumulators is decided by the caller (an epilogue after
-// mainloop()).
+// mainloop()).  mainloop16(), at the end of this file, is the same loop issued as v_mfma_f32_16x16x32_bf16 for two
+// K-contiguous operands.
 //
 // Register layout of one 32 x 32 x 16 MFMA (checked on the hardware):
 //   A operand, lane l: A[m = l % 32][k = 8 (l / 32) + j], j = 0..7
@@ -307,6 +308,174 @@ __device__ __forceinline__ void mainloop(const Operand& A, const Operand& B, int
     open_b(cx, k + 2, sa);  // unit 2 k + 5 = B(k + 2) takes the slot of A(k)
     __builtin_amdgcn_sched_barrier(0);
     step(1, sa1, sb1, 0, cx, sb_.jstep, 0);
+    sa = sa1;
+  }
+  // the empty loads of the last slices may still deposit zeros: let them finish before the caller reuses LDS
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
+  __builtin_amdgcn_s_barrier();
+}
+
+// ---- the same loop on v_mfma_f32_16x16x32_bf16, for two K-contiguous operands ----------------------------------------
+// The chip is power-limited on random operands, and the 16 x 16 x 32 form draws less power per flop (half the
+// accumulator register traffic): an MFMA-only loop sustains 2.06 PFLOP/s at 2.06 GHz with it against 1.87 at 1.80 GHz
+// with 32 x 32 x 16.  With twice as many MFMAs per slice every direct-to-LDS load falls behind a 16-cycle instead of a
+// 32-cycle MFMA and costs more idle cycles (164 k cycles per 256 x 256 x 4096 tile instead of 151 k), but at
+// 1.9 GHz instead of 1.66: 5 % faster as a bare loop on K-contiguous operands, 2-3 % in the kernels that use it.
+// K-major operands (two transposing reads per fragment) gain nothing, so the products that contract K-major arrays
+// stay on mainloop().
+//
+// Register layout of one 16 x 16 x 32 MFMA (checked on the hardware):
+//   A operand, lane l: A[m = l % 16][k = 8 (l / 16) + j], j = 0..7
+//   B operand, lane l: B[n = l % 16][k = 8 (l / 16) + j]
+//   D, lane l, register i: n = l % 16, m = 4 (l / 16) + i
+// i.e. a lane owns one column n of D and 4 consecutive rows m; the lanes l ^ 16, l ^ 32 own the other rows of that n.
+typedef float f32x4acc_t __attribute__((ext_vector_type(4)));
+constexpr int kAcc16Tiles = 8;  // per direction: a wave's 128 x 128 block is 8 x 8 tiles of 16 x 16
+struct Acc16 {
+  f32x4acc_t v[kAcc16Tiles][kAcc16Tiles];
+};
+__device__ __forceinline__ int acc16_row(int mt, int i, int lane) { return mt * 16 + 4 * (lane >> 4) + i; }
+__device__ __forceinline__ int acc16_col(int nt, int lane) { return nt * 16 + (lane & 15); }
+
+// Per-operand constants of a wave (K-contiguous unit as above: same loads, same swizzle).  A fragment (sub-tile x of 16
+// rows, 32-wide k step kk) of lane l is the 16 bytes of row 16 x + l % 16, chunk 4 kk + l / 16.
+struct Side16 {
+  const uint16_t* base;  // tile origin
+  int bytes;             // valid bytes of the tile
+  int chunk;             // the global chunk (of 8) this lane brings
+  int voffj[8];          // load j of a unit: per-lane byte offset inside the slice (range fix-ups included)
+  int frag[2];           // fragment read: per-lane byte offset inside a unit, per k step
+};
+
+__device__ __forceinline__ Side16 make_side16(const Operand& X, int x0, int wq, int wave, int lane) {
+  Side16 s;
+  const int valid = (X.rows - x0) < 256 ? (X.rows - x0) : 256;
+  const int ld_row = 8 * wave + (lane >> 3);
+  s.chunk = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7);
+  s.base = X.ptr + (int64_t)x0 * X.ld;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) s.voffj[j] = (int)((((int64_t)ld_row + 32 * j) * X.ld + s.chunk * 8) * 2);
+  s.bytes = (int)((int64_t)valid * X.ld * 2);
+  const int kgrp = lane >> 4, r7 = (lane >> 1) & 7;  // row 16 x + lane % 16: (row >> 1) & 7 = (lane >> 1) & 7
+  const int fr = (wq * 128 + (lane & 15)) * 128;
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) s.frag[kk] = fr + (((4 * kk + kgrp) ^ r7) << 4);
+  return s;
+}
+
+// A slice is two 32-wide k steps of 64 MFMAs (A sub-tile mt x B sub-tile nt, 8 x 8); the fragments of both steps live
+// in registers (2 x 16 fragments).  A step is issued as two halves of 32 MFMAs: the first half multiplies A0-3 with
+// B0-3, then with B4-7; the second half A4-7 with B0-7.  So a step can start once A0-3 and B0-3 are there, B4-7 are
+// needed 16 MFMAs later and A4-7 a half later.  Every half carries 8 fragment reads (behind its first 8 MFMAs) and 4
+// global loads (behind MFMAs 7, 15, 23, 31), in exactly the order written here:
+//   half 0 (step 0, first)    reads B4-7, A4-7 of step 0            loads the second half of B(k+1)
+//   half 1 (step 0, second)   reads B0-3, A0-3 of step 1            loads the first half of A(k+2)
+//   half 2 (step 1, first)    reads B4-7, A4-7 of step 1            loads the second half of A(k+2)
+//   wait: own fragment reads done, own loads through B(k+1) landed (A(k+2) may be in flight); barrier
+//   half 3 (step 1, second)   reads B0-3, A0-3 of slice k+1 step 0  loads the first half of B(k+2) into A(k)'s slot
+// The ring of units, the counted waits and the empty descriptors past K are those of mainloop().
+__device__ __forceinline__ void mainloop16(const Operand& A, const Operand& B, int K, int m0, int n0, Acc16& acc, char* lds) {
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const uint32_t lds32 = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
+  Side16 sa_ = make_side16(A, m0, wm, wave, lane);
+  Side16 sb_ = make_side16(B, n0, wn, wave, lane);
+  struct Unit {
+    __amdgpu_buffer_rsrc_t rs;
+    uint32_t dst;
+  };
+  auto open_unit = [&](Unit& c, Side16& s, int slice, int slot) {
+    const int k0 = slice * BK;
+    const bool live = k0 < K;
+    // the descriptor starts at column k0, so row r is in range iff r < rows (the last row may end early, never late)
+    c.rs = __builtin_amdgcn_make_buffer_rsrc((void*)(s.base + (live ? k0 : 0)), 0, live ? s.bytes - k0 * 2 : 0, kBufferFlags);
+    // the one slice that straddles K: chunks at or past K are pushed out of the descriptor's range, for good (the
+    // slices after it are empty anyway)
+    if (live && k0 + BK > K) {
+      const int out = (k0 + s.chunk * 8 >= K) ? (int)0x80000000 : 0;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) s.voffj[j] |= out;
+    }
+    c.dst = lds32 + slot * kUnitBytes + wave * 1024;
+  };
+  auto g_load1 = [&](const Unit& c, const Side16& s, int j) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(c.rs, (lds_ptr_t)(uintptr_t)(c.dst + j * 4096), 16, s.voffj[j], 0, 0, 0);
+  };
+
+#pragma unroll
+  for (int mt = 0; mt < kAcc16Tiles; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < kAcc16Tiles; ++nt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc.v[mt][nt][i] = 0.f;
+
+  bf16x8_t fa[2][8], fb[2][8];
+  // fragment read r (0..7) of a half: group = 0 reads B0-3 then A0-3, group = 1 reads B4-7 then A4-7, of k step kk of
+  // the units in slot_a / slot_b, into fragment buffer buf
+  auto f_load1 = [&](int buf, int slot_a, int slot_b, int kk, int group, int r) {
+    const int x = 4 * group + (r & 3);
+    if (r < 4)
+      fb[buf][x] = __builtin_bit_cast(bf16x8_t, *(const u32x4_t*)(lds + slot_b * kUnitBytes + sb_.frag[kk] + x * 2048));
+    else
+      fa[buf][x] = __builtin_bit_cast(bf16x8_t, *(const u32x4_t*)(lds + slot_a * kUnitBytes + sa_.frag[kk] + x * 2048));
+  };
+  auto mfma1 = [&](int buf, int mt, int nt) {
+    acc.v[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[buf][mt], fb[buf][nt], acc.v[mt][nt], 0, 0, 0);
+  };
+  // one half of a 32-wide k step: 32 MFMAs from fragment buffer `buf` (second = 0: A0-3 x B0-3, then A0-3 x B4-7;
+  // second = 1: A4-7 x B0-7); in their shadow 8 fragment reads (group rgroup of k step rkk of the units in slots ra, rb,
+  // into buffer rbuf) and 4 global loads (blocks j0 .. j0 + 3 of the unit `c` of operand side `cs`)
+  auto half = [&](int buf, int second, int rbuf, int ra, int rb, int rkk, int rgroup, const Unit& c, const Side16& cs, int j0) {
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      if (second)
+        mfma1(buf, 4 + (i >> 3), i & 7);
+      else
+        mfma1(buf, (i >> 2) & 3, (i & 3) + 4 * (i >> 4));
+      if (i < 8) f_load1(rbuf, ra, rb, rkk, rgroup, i);
+      if ((i & 7) == 7) g_load1(c, cs, j0 + (i >> 3));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto next_slot = [](int s, int by) { s += by; return s >= kUnits ? s - kUnits : s; };
+
+  const int nk = (K + BK - 1) / BK;
+  Unit cx, cy;  // cx: the B unit whose first half was issued before the barrier; cy: the A unit issued in halves 1, 2
+  // units 0, 1, 2 (A0, B0, A1) and the first half of unit 3 (B1)
+  open_unit(cy, sa_, 0, 0);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) g_load1(cy, sa_, j);
+  open_unit(cx, sb_, 0, 1);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) g_load1(cx, sb_, j);
+  open_unit(cy, sa_, 1, 2);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) g_load1(cy, sa_, j);
+  open_unit(cx, sb_, 1, 3);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) g_load1(cx, sb_, j);
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(12, 15));  // this wave's parts of units 0 and 1 have landed
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int r = 0; r < 8; ++r) f_load1(0, 0, 1, 0, 0, r);
+  int sa = 0;  // slot of A(k) = (2 k) % 5
+  for (int k = 0; k < nk; ++k) {
+    const int sb = next_slot(sa, 1), sa1 = next_slot(sa, 2), sb1 = next_slot(sa, 3), s4 = next_slot(sa, 4);
+    // cx is unit 2 k + 3 = B(k + 1) in slot sb1, opened when its first half was issued
+    __builtin_amdgcn_sched_barrier(0);
+    half(0, 0, 0, sa, sb, 0, 1, cx, sb_, 4);
+    open_unit(cy, sa_, k + 2, s4);  // unit 2 k + 4 = A(k + 2)
+    __builtin_amdgcn_sched_barrier(0);
+    half(0, 1, 1, sa, sb, 1, 0, cy, sa_, 0);
+    half(1, 0, 1, sa, sb, 1, 1, cy, sa_, 4);
+    // own reads of slice k done; own loads through unit 2 k + 3 landed (unit 2 k + 4 may be in flight)
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(8, 0));
+    __builtin_amdgcn_s_barrier();
+    open_unit(cx, sb_, k + 2, sa);  // unit 2 k + 5 = B(k + 2) takes the slot of A(k)
+    __builtin_amdgcn_sched_barrier(0);
+    half(1, 1, 0, sa1, sb1, 0, 0, cx, sb_, 0);
     sa = sa1;
   }
   // the empty loads of the last slices may still deposit zeros: let them finish before the caller reuses LDS

@@ -76,29 +76,32 @@ struct TileArgs {
 constexpr float kCarryMaxShift = 126.f;
 constexpr float kCarryMinLogp = -80.f;
 
-// Statistics (and, with CARRY, the staged unnormalised probabilities) of one wave's 128 x 128 block.  RAGGED: the
-// block may reach past the vocabulary (last tile row only), rows at or past V are left out.
+// Statistics (and, with CARRY, the staged probability ratios) of one wave's 128 x 128 block, accumulators in the
+// 16 x 16 tile layout: a lane holds, for each of 8 tokens (nt), 8 runs (mt) of 4 consecutive vocabulary rows, and the
+// lanes l ^ 16, l ^ 32 hold the other rows of the same tokens.  RAGGED: the block may reach past the vocabulary (last
+// tile row only), rows at or past V are left out.
 template <bool CARRY, bool RAGGED>
-__device__ __forceinline__ void block_stats(const Acc& acc, const TileArgs& a, int tm, int wm, int wn, int n0, int N,
+__device__ __forceinline__ void block_stats(const Acc16& acc, const TileArgs& a, int tm, int wm, int wn, int n0, int N,
                                             int V, int mbase, int lane, uint16_t* Z) {
   constexpr int PZ = kPanelPitch;
 #pragma unroll
-  for (int nt = 0; nt < 4; ++nt) {
-    const int nloc = wn * 128 + acc_col(nt, lane);
+  for (int nt = 0; nt < kAcc16Tiles; ++nt) {
+    const int nloc = wn * 128 + acc16_col(nt, lane);
     const int n = n0 + nloc;
     float mx = -FLT_MAX;
     if constexpr (!RAGGED) {
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt)
+      for (int mt = 0; mt < kAcc16Tiles; ++mt)
 #pragma unroll
-        for (int i = 0; i < 16; i += 2) mx = fmaxf(fmaxf(mx, acc.v[mt][nt][i]), acc.v[mt][nt][i + 1]);  // one v_max3 per pair
+        for (int i = 0; i < 4; i += 2) mx = fmaxf(fmaxf(mx, acc.v[mt][nt][i]), acc.v[mt][nt][i + 1]);  // one v_max3 per pair
     } else {
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt)
+      for (int mt = 0; mt < kAcc16Tiles; ++mt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) mx = (mbase + acc_row(mt, i, lane) < V) ? fmaxf(mx, acc.v[mt][nt][i]) : mx;
+        for (int i = 0; i < 4; ++i) mx = (mbase + acc16_row(mt, i, lane) < V) ? fmaxf(mx, acc.v[mt][nt][i]) : mx;
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));  // both halves of the wave hold the same token
+    mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));  // four lanes hold the same token
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
     const float k = fmaxf(mx * a.c, kNegBig);   // kNegBig: no valid row in this block
     float to_ref = 1.f;                         // 2^(k - kref): block-relative -> label-relative exponentials
     if constexpr (CARRY) {
@@ -108,28 +111,28 @@ __device__ __forceinline__ void block_stats(const Acc& acc, const TileArgs& a, i
     }
     float s = 0.f, u = 0.f;
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
+    for (int mt = 0; mt < kAcc16Tiles; ++mt) {
+      float e[4];
 #pragma unroll
-      for (int g4 = 0; g4 < 4; ++g4) {
-        float e[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const float t = fmaf(acc.v[mt][nt][g4 * 4 + q], a.c, -k);
-          e[q] = fast_exp2(t);
-          if constexpr (RAGGED) e[q] = (mbase + acc_row(mt, g4 * 4 + q, lane) < V) ? e[q] : 0.f;
-          s += e[q];
-          u = fmaf(t, e[q], u);
-        }
-        if constexpr (CARRY) {
-          uint2 pk;
-          pk.x = Elem<AA_BF16>::pack(e[0] * to_ref, e[1] * to_ref);
-          pk.y = Elem<AA_BF16>::pack(e[2] * to_ref, e[3] * to_ref);
-          *(uint2*)(Z + nloc * PZ + wm * 128 + mt * 32 + 8 * g4 + 4 * (lane >> 5)) = pk;
-        }
+      for (int q = 0; q < 4; ++q) {
+        const float t = fmaf(acc.v[mt][nt][q], a.c, -k);
+        e[q] = fast_exp2(t);
+        if constexpr (RAGGED) e[q] = (mbase + acc16_row(mt, q, lane) < V) ? e[q] : 0.f;
+        s += e[q];
+        u = fmaf(t, e[q], u);
       }
+      if constexpr (CARRY) {
+        uint2 pk;
+        pk.x = Elem<AA_BF16>::pack(e[0] * to_ref, e[1] * to_ref);
+        pk.y = Elem<AA_BF16>::pack(e[2] * to_ref, e[3] * to_ref);
+        *(uint2*)(Z + nloc * PZ + wm * 128 + acc16_row(mt, 0, lane)) = pk;
+      }
+    }
+    s += __shfl_xor(s, 16, kWave);
     s += __shfl_xor(s, 32, kWave);
+    u += __shfl_xor(u, 16, kWave);
     u += __shfl_xor(u, 32, kWave);
-    if (lane < 32 && n < N) {
+    if (lane < 16 && n < N) {
       const int64_t at = (int64_t)(tm * 2 + wm) * a.pitch_t + n;
       a.pk[at] = k;
       a.ps[at] = s;
@@ -139,7 +142,8 @@ __device__ __forceinline__ void block_stats(const Acc& acc, const TileArgs& a, i
 }
 
 // One 256 x 256 tile: rows m = vocabulary (operand A = weight), columns n = tokens (operand B = hidden states), so
-// that everything a token needs from the tile sits in one lane and its partner lane ^ 32.
+// that everything a token needs from the tile sits in one lane and its partner lanes ^ 16, ^ 32.  Both operands are
+// K-contiguous: the 16 x 16 x 32 main loop.
 template <int MODE>
 __global__ __launch_bounds__(kThreads) void k_lmhead_tiles(Operand W, Operand Hd, int K, int tiles_m, int tiles_n,
                                                                  TileArgs a) {
@@ -150,8 +154,8 @@ __global__ __launch_bounds__(kThreads) void k_lmhead_tiles(Operand W, Operand Hd
   int tm, tn;
   tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
-  Acc acc;
-  mainloop<false, false>(W, Hd, K, m0, n0, acc, lds);  // ends with a barrier: LDS is free
+  Acc16 acc;
+  mainloop16(W, Hd, K, m0, n0, acc, lds);  // ends with a barrier: LDS is free
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
@@ -167,8 +171,8 @@ __global__ __launch_bounds__(kThreads) void k_lmhead_tiles(Operand W, Operand Hd
       block_stats<MODE == kModeStatsCarry, false>(acc, a, tm, wm, wn, n0, N, V, mbase, lane, Z);
   } else {
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt) {
-      const int nloc = wn * 128 + acc_col(nt, lane);
+    for (int nt = 0; nt < kAcc16Tiles; ++nt) {
+      const int nloc = wn * 128 + acc16_col(nt, lane);
       const int n = n0 + nloc;
       float A = 0.f, B = 0.f, lab_add = 0.f, lse2 = 0.f;
       int64_t y = -1;
@@ -185,26 +189,24 @@ __global__ __launch_bounds__(kThreads) void k_lmhead_tiles(Operand W, Operand Hd
       }
       const int rel = (int)(y - mbase < -1 ? -1 : (y - mbase > 128 ? 128 : y - mbase));  // outside [0, 128): not here
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt)
+      for (int mt = 0; mt < kAcc16Tiles; ++mt) {
+        float o[4];
 #pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-          float o[4];
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const float x = acc.v[mt][nt][g4 * 4 + q];
-            o[q] = fast_exp2(fmaf(x, a.c, -lse2)) * fmaf(B, x, A);  // columns past the tokens: never written out
-          }
-          const int r0 = mt * 32 + 8 * g4 + 4 * (lane >> 5);  // row of o[0] inside the wave's block
-          if (rel >= r0 && rel < r0 + 4) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-              if (rel - r0 == q) o[q] += lab_add;
-          }
-          uint2 pk;
-          pk.x = Elem<AA_BF16>::pack(o[0], o[1]);
-          pk.y = Elem<AA_BF16>::pack(o[2], o[3]);
-          *(uint2*)(Z + nloc * PZ + wm * 128 + r0) = pk;
+        for (int q = 0; q < 4; ++q) {
+          const float x = acc.v[mt][nt][q];
+          o[q] = fast_exp2(fmaf(x, a.c, -lse2)) * fmaf(B, x, A);  // columns past the tokens: never written out
         }
+        const int r0 = acc16_row(mt, 0, lane);  // row of o[0] inside the wave's block
+        if (rel >= r0 && rel < r0 + 4) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            if (rel - r0 == q) o[q] += lab_add;
+        }
+        uint2 pk;
+        pk.x = Elem<AA_BF16>::pack(o[0], o[1]);
+        pk.y = Elem<AA_BF16>::pack(o[2], o[3]);
+        *(uint2*)(Z + nloc * PZ + wm * 128 + r0) = pk;
+      }
     }
   }
   if constexpr (MODE != kModeStats) {

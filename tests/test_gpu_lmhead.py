@@ -29,7 +29,7 @@ def _case(T, H, V, seed, w_std=0.02):
     "T,H,V,temperature",
     [
         (256, 128, 1024, 1.0),
-        (300, 192, 1088, 1.0),    # token count not a multiple of 8: the transposed copies pad it
+        (300, 192, 1088, 1.0),    # token count not a multiple of 8
         (37, 64, 576, 0.7),
         (700, 256, 4160, 1.3),
         (203, 200, 1096, 1.0),    # H and V multiples of 8 only

@@ -250,8 +250,8 @@ def test_full_size_step_agrees_with_unfused_path(device, backward):
     loss, stat = areal_amd.ppo_actor_loss_fn(lp, case.prox_logp, case.old_logp, case.advantages, 0.2, case.loss_mask)
     loss.backward()
     assert float(l1) == pytest.approx(float(loss.detach()), rel=1e-5)
-    # the same forward tiles, merged by two different kernels
-    assert torch.allclose(s1["logprobs"], lp.detach(), rtol=0, atol=2e-6) and torch.allclose(s1["entropy"], ent.detach(), rtol=0, atol=2e-6)
+    # the same forward tiles, merged by two different kernels: a few ulp of values near 11 (ulp 9.5e-7)
+    assert torch.allclose(s1["logprobs"], lp.detach(), rtol=0, atol=4e-6) and torch.allclose(s1["entropy"], ent.detach(), rtol=0, atol=4e-6)
     for got, want in ((dh1, h.grad), (dw1, w.grad)):
         a, b = got.double().reshape(-1), want.double().reshape(-1)
         assert float(a @ b / (a.norm() * b.norm())) > 0.9999
