@@ -78,6 +78,7 @@ SIGNATURES = {
     "aa_ppo_loss": (_i, [_p, _p, _p, _p, _p, _i64, _p, _i64, _i, C.POINTER(PpoParams), _p, _p, _p, _p, _p, _p]),
     "aa_masked_sum": (_i, [_p, _p, _i64, _p, _p, _p, _p]),
     "aa_scale_inplace": (_i, [_p, _i, _i64, _p, _p]),
+    "aa_scale_rows_inplace": (_i, [_p, _i, _i64, _i64, _i64, _p, _p]),
     "aa_lmhead_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "aa_lmhead_fwd_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "aa_lmhead_fwd": (_i, [_p, _p, _i64, _i64, _i64, _p, _f, _p, _p, _p, _p, _p, _i64, _p]),

@@ -971,6 +971,19 @@ __global__ __launch_bounds__(256) void k_scale(void* __restrict__ data, int64_t 
     Elem<DT>::store1(data, i, Elem<DT>::load1(data, i) * f);
 }
 
+// rows of V elements that start `stride` elements apart: the elements between the rows are left alone
+template <int DT>
+__global__ __launch_bounds__(256) void k_scale_rows(void* __restrict__ data, int64_t T, int64_t V, int64_t stride,
+                                                    const float* __restrict__ factor) {
+  const float f = *factor;
+  if (f == 1.0f) return;
+  const int64_t n = T * V, step = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += step) {
+    const int64_t at = (i / V) * stride + i % V;
+    Elem<DT>::store1(data, at, Elem<DT>::load1(data, at) * f);
+  }
+}
+
 // -----------------------------------------------------------------------------
 // Host-side dispatch
 // -----------------------------------------------------------------------------
@@ -1273,6 +1286,21 @@ extern "C" int aa_scale_inplace(void* data, int dtype, int64_t n, const float* f
   if (dtype == AA_BF16) hipLaunchKernelGGL(k_scale<AA_BF16>, dim3((unsigned)blocks), dim3(256), 0, st, data, n, factor);
   else if (dtype == AA_F16) hipLaunchKernelGGL(k_scale<AA_F16>, dim3((unsigned)blocks), dim3(256), 0, st, data, n, factor);
   else if (dtype == AA_F32) hipLaunchKernelGGL(k_scale<AA_F32>, dim3((unsigned)blocks), dim3(256), 0, st, data, n, factor);
+  else return AA_ERR_INVALID_ARGUMENT;
+  return launch_status();
+}
+
+extern "C" int aa_scale_rows_inplace(void* data, int dtype, int64_t T, int64_t V, int64_t row_stride, const float* factor,
+                                     void* stream) {
+  if (!data || !factor || T < 0 || V < 0 || row_stride < V) return AA_ERR_INVALID_ARGUMENT;
+  if (row_stride == V) return aa_scale_inplace(data, dtype, T * V, factor, stream);
+  if (T == 0 || V == 0) return AA_OK;
+  int64_t blocks = (T * V + 255) / 256;
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == AA_BF16) hipLaunchKernelGGL(k_scale_rows<AA_BF16>, dim3((unsigned)blocks), dim3(256), 0, st, data, T, V, row_stride, factor);
+  else if (dtype == AA_F16) hipLaunchKernelGGL(k_scale_rows<AA_F16>, dim3((unsigned)blocks), dim3(256), 0, st, data, T, V, row_stride, factor);
+  else if (dtype == AA_F32) hipLaunchKernelGGL(k_scale_rows<AA_F32>, dim3((unsigned)blocks), dim3(256), 0, st, data, T, V, row_stride, factor);
   else return AA_ERR_INVALID_ARGUMENT;
   return launch_status();
 }

@@ -124,13 +124,15 @@ def _check_fused_inputs(rows: torch.Tensor, labels: torch.Tensor, loss_mask: tor
 
 def fused_logprobs_sft_loss(logits: torch.Tensor, labels: torch.Tensor, loss_mask: torch.Tensor,
                             cu_seqlens: torch.Tensor | None = None, temperature: float = 1.0,
-                            loss_scale: torch.Tensor | float | None = None) -> tuple[torch.Tensor, dict]:
+                            loss_scale: torch.Tensor | float | None = None,
+                            inplace_backward: bool = False) -> tuple[torch.Tensor, dict]:
     """``gather_logprobs`` + ``compute_packed_sft_loss`` (+ backward) in one pass over the logits.
 
     ``logits`` is ``[T_pad, V]``, ``labels`` ``[T_pad]``, ``loss_mask`` the un-padded ``[T]`` mask with ``T <= T_pad``
     (rows past ``T`` get a zero gradient).  ``loss.backward()`` hands back the gradient written during the forward
     pass.  ``stat`` is that of ``sft_loss_fn`` plus ``logprobs``, ``entropy``, ``vocab_min_logits`` and
-    ``vocab_max_logits`` (``[T]``).  Without a gradient to produce the call is the forward kernel and the loss."""
+    ``vocab_max_logits`` (``[T]``).  Without a gradient to produce the call is the forward kernel and the loss.
+    ``inplace_backward=True`` writes the gradient over the logits, as in ``fused_logprobs_ppo_loss``."""
     _require_gpu(logits, "logits")
     T_active = _check_fused_inputs(logits, labels, loss_mask, "logits")
     dev = logits.device
@@ -146,7 +148,8 @@ def fused_logprobs_sft_loss(logits: torch.Tensor, labels: torch.Tensor, loss_mas
     m8 = _mask_u8(loss_mask.to(dev))
     n_valid = _count_nonzero(m8)
     loss, logp, entropy, vmax, vmin, stat_loss, _ratio, _flags = _FusedLogitsPpo.apply(
-        x, y, stride, float(temperature), T_active, None, None, m8, None, _nll_params(), n_valid, scale_t, True
+        x, y, stride, float(temperature), T_active, None, None, m8, None, _nll_params(), n_valid, scale_t, True,
+        bool(inplace_backward),
     )
     logp_a = logp[:T_active]
     _, _, _, seq_logp, seq_count, seq_ppl = _launch(logp_a, m8, cu, n_seqs, n_valid, None, False, False)

@@ -182,8 +182,9 @@ def run_logits_steps(case, n, kw, cfg):
     return loss
 
 
-def time_fused_logits_kernel(case, kw, cfg, iters: int):
-    """Duration of aa_logits_ppo_fused alone, HIP events on the launch stream, outputs pre-allocated."""
+def time_fused_logits_kernel(case, kw, cfg, iters: int, inplace: bool = False):
+    """Duration of aa_logits_ppo_fused alone, HIP events on the launch stream, outputs pre-allocated.  ``inplace``:
+    the gradient is written over the logits (which are lost: the caller times this variant last)."""
     import torch
 
     from areal_amd import _native as N
@@ -204,7 +205,7 @@ def time_fused_logits_kernel(case, kw, cfg, iters: int):
         mask_eff, w, counts = m8, None, F._count_nonzero(m8)
     logp, ent, sl, ratio = (torch.empty(T, **f32) for _ in range(4))
     flags = torch.empty(T, dtype=torch.uint8, device=dev)
-    dlogits = torch.empty_like(case.logits)
+    dlogits = case.logits if inplace else torch.empty_like(case.logits)
     stream = torch.cuda.current_stream(dev)
 
     def launch():
@@ -397,6 +398,14 @@ def bench_logits(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: 
                                        launches=args.copy_launches)
     del dst
     sample = logits_gpu_sample(case, kw, cfg, cpu_tokens) if cpu_tokens > 0 else None
+    # last, because it overwrites the workload: the same kernel with the gradient written over the logits
+    # (inplace_backward=True: one [T, V] array instead of two)
+    i_ms, i_min_ms = time_fused_logits_kernel(case, kw, cfg, max(steps, 10), inplace=True)
+    out["gradient_over_logits"] = dict(
+        avg_kernel_ms=i_ms, min_kernel_ms=i_min_ms, achieved=alg_bytes / (i_ms * 1e-3) / 1e9, unit="GB/s",
+        frac=alg_bytes / (i_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        bytes_of_logits_and_gradient=case.logits.numel() * case.logits.element_size(),
+        note="inplace_backward=True; after the first launch the rows hold gradients, the traffic is the same")
     return out, sample
 
 

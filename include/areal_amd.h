@@ -128,6 +128,12 @@ int aa_logits_bwd(const void* logits, int dtype, int64_t T, int64_t V,
  *   masking), ratio, flags (bit0 = clip_mask & mask_eff, bit1 =
  *   dual_clip_mask & mask_eff); dlogits [T, V] in the dtype of logits (rows
  *   >= T_active are zeros).  The scalar loss is finished by aa_masked_sum.
+ * dlogits may be the logits array itself (the gradient then takes the place
+ *   of the logits, which halves the memory of the step; no counterpart in the
+ *   reference, whose autograd allocates the gradient): a row belongs to one
+ *   workgroup, and every kernel behind this entry point reads an element for
+ *   the last time before it writes it.  Any other overlap of the two arrays
+ *   is not allowed.
  * work: NULL, or two int32 words of device memory that are zero on entry; the
  *   kernel hands rows to compute units through them (faster than a fixed
  *   assignment) and leaves them zero on exit, so one zeroed buffer serves
@@ -247,6 +253,15 @@ int aa_masked_sum(const float* values, const uint8_t* mask, int64_t n,
 /* data[i] *= *factor for i < n (dtype as aa_dtype); a no-op when *factor == 1. */
 int aa_scale_inplace(void* data, int dtype, int64_t n, const float* factor,
                      void* stream);
+
+/*
+ * The same for T rows of V elements that start row_stride >= V elements apart
+ * (the upstream factor of loss.backward() on a gradient that lies in a slice
+ * of a wider array: what lies between the rows is not touched).
+ */
+int aa_scale_rows_inplace(void* data, int dtype, int64_t T, int64_t V,
+                          int64_t row_stride, const float* factor,
+                          void* stream);
 
 /* ------------------------------------------------------------------ */
 /* Sibling losses and actor-side token filters                            */

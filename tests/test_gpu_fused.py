@@ -443,3 +443,83 @@ def test_second_backward_of_the_fused_step_is_refused(device):
     loss.backward(retain_graph=True)
     with pytest.raises(RuntimeError, match="already handed out"):
         loss.backward()
+
+
+@pytest.mark.parametrize(
+    "V,dtype",
+    [
+        (151936, torch.bfloat16),   # register-resident rows
+        (172040, torch.bfloat16),   # registers + LDS
+        (250008, torch.float16),    # registers + LDS + a tail that is read once per pass
+        (8200, torch.float16),      # two-pass kernel, 16-byte pieces
+        (50257, torch.bfloat16),    # two-pass kernel, element by element
+        (4099, torch.float32),      # the same in fp32
+        (151936, torch.float32),    # fp32 rows held on the chip, the rest read twice
+    ],
+)
+def test_gradient_written_over_the_logits(device, V, dtype):
+    """inplace_backward=True: the gradient takes the place of the logits, with the bits of the separate array, on every
+    kernel behind the entry point; masked rows included (their gradient is zero)."""
+    lengths = synth.lengths_uniform(5, 4, 12, seed=V)
+    case = synth.make_logits_case("t", lengths, V, V, device, synth.per_sequence_normal_advantages(lengths, 3),
+                                  dtype=dtype, ppo=dict(eps_clip=0.2))
+    _finish_case(case)
+    loss, stat, grad = _fused_step(case)
+    x = case.logits.clone().requires_grad_(True)
+    l2, s2 = areal_amd.fused_logprobs_ppo_loss(x, case.labels, case.prox_logp, case.old_logp, case.advantages,
+                                               loss_mask=case.loss_mask, cu_seqlens=case.cu_seqlens,
+                                               temperature=case.temperature, inplace_backward=True, **case.ppo)
+    assert torch.equal(x.detach(), grad)               # already there after the forward call
+    l2.backward()
+    assert torch.equal(x.grad, grad) and torch.equal(x.detach(), grad)
+    assert torch.equal(l2.detach(), loss)
+    for k in ("logprobs", "entropy", "loss", "importance_weight", "clip_mask", "vocab_max_logits", "vocab_min_logits"):
+        assert torch.equal(s2[k], stat[k]), k
+
+
+def test_gradient_written_over_logits_that_another_operation_produced(device):
+    """The usual place of the call: the logits are the output of the lm_head product.  The gradient of the hidden
+    states is that of the separate array; rows with a stride (a slice of a wider array) work the same way; an
+    operation that kept the logits for its own backward is told that they changed."""
+    g = torch.Generator().manual_seed(4)
+    T, H, V = 40, 64, 16384
+    hidden = torch.randn(T, H, generator=g).bfloat16().to(device)
+    weight = (0.3 * torch.randn(V + 8, H, generator=g)).bfloat16().to(device)
+    labels = torch.randint(0, V, (T,), generator=g).to(device)
+    z = torch.zeros(T, device=device) - 9.0
+    adv, mask = torch.randn(T, generator=g).to(device), (torch.rand(T, generator=g) < 0.7).to(device)
+
+    def step(inplace, sliced, through=lambda t: t, factor=1.0):
+        h = hidden.clone().requires_grad_(True)
+        wide = through(h @ weight.T)
+        beside = wide.detach()[:, V:].clone()            # what lies between the rows of the slice
+        if sliced:
+            logits = wide[:, :V]                         # row stride V + 8
+        else:
+            logits = wide[:, :V].contiguous()
+        loss, _ = areal_amd.fused_logprobs_ppo_loss(logits, labels, z, z, adv, 0.2, mask, inplace_backward=inplace)
+        (loss * factor).backward()
+        assert torch.equal(wide.detach()[:, V:], beside)
+        return loss.detach(), h.grad
+
+    for sliced in (False, True):
+        for factor in (1.0, 3.0):
+            l0, g0 = step(False, sliced, factor=factor)
+            l1, g1 = step(True, sliced, factor=factor)
+            assert torch.equal(l0, l1) and torch.equal(g0, g1), (sliced, factor)
+    with pytest.raises(RuntimeError, match="modified by an inplace operation"):
+        step(True, True, through=lambda t: torch.sigmoid(t.float()).bfloat16().sigmoid())
+
+
+def test_supervised_gradient_written_over_the_logits(device):
+    lengths = [9, 14]
+    case = synth.make_logits_case("t", lengths, 16384, 16384, device, synth.per_sequence_normal_advantages(lengths, 3),
+                                  ppo=dict(eps_clip=0.2))
+    x = case.logits.clone().requires_grad_(True)
+    loss, stat = areal_amd.fused_logprobs_sft_loss(x, case.labels, case.loss_mask, case.cu_seqlens)
+    loss.backward()
+    y = case.logits.clone().requires_grad_(True)
+    l2, s2 = areal_amd.fused_logprobs_sft_loss(y, case.labels, case.loss_mask, case.cu_seqlens, inplace_backward=True)
+    l2.backward()
+    assert torch.equal(l2.detach(), loss.detach()) and torch.equal(y.detach(), x.grad) and torch.equal(y.grad, x.grad)
+    assert torch.equal(s2["logprobs"], stat["logprobs"])
