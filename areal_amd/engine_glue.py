@@ -48,13 +48,15 @@ def compute_logprobs_and_loss(
     temperature: float = 1.0,
     loss_multiplier: float = 1.0,
     fused: bool = True,
+    inplace_backward: bool = False,
 ) -> tuple[torch.Tensor, dict]:
     """Scaled PPO loss of one micro-batch and its stat dict (fsdp_engine.py:1977-2046 with
     ``loss_fn = grpo_loss_fn`` and ``loss_weight_fn = loss_mask.count_nonzero``, actor.py:345-364).
 
     ``logits`` is ``[T_pad, V]``; ``mb_input`` holds the un-padded ``[T]`` tensors ``loss_mask``, ``logprobs``
     (behaviour policy), ``prox_logp``, ``advantages`` and ``cu_seqlens``.  An all-masked micro-batch returns
-    ``logits.mean() * 0`` like the reference (fsdp_engine.py:1988-1989).
+    ``logits.mean() * 0`` like the reference (fsdp_engine.py:1988-1989).  ``inplace_backward`` (fused path only):
+    the gradient is written over the logits, see ``fused_logprobs_ppo_loss``.
     """
     loss_mask = mb_input["loss_mask"].bool()
     local_weight = loss_mask.count_nonzero()
@@ -73,7 +75,7 @@ def compute_logprobs_and_loss(
     if fused:
         return fused_logprobs_ppo_loss(
             logits, labels, prox_logp, old_logp, mb_input["advantages"], loss_mask=loss_mask,
-            temperature=temperature, loss_scale=scale, **kw,
+            temperature=temperature, loss_scale=scale, inplace_backward=inplace_backward, **kw,
         )
     logp, entropy, vmin, vmax = gather_logprobs_entropy_stats(logits, labels, temperature)
     if pad_length > 0:

@@ -243,6 +243,12 @@ def test_engine_contract_roll_pad_and_scale(device):
         assert_same_magnitude(grad.cpu(), w_grad, what="d_logits")
         assert float(grad[n:].float().abs().max()) == 0.0
         assert stat["logprobs"].shape == (n,)
+    # the same call with the gradient written over the logits: the bits of the fused result
+    x = logits.to(device).requires_grad_(True)
+    loss, _ = engine_glue.compute_logprobs_and_loss(x, {"input_ids": input_ids.to(device)}, mb_d, pad, total_w,
+                                                    eps_clip=0.2, inplace_backward=True)
+    loss.backward()
+    assert float(loss.detach()) == results[0][0] and torch.equal(x.grad, results[0][1]) and torch.equal(x.detach(), x.grad)
     # an all-masked micro-batch keeps the graph alive and contributes nothing
     mb_d["loss_mask"] = torch.zeros(n, dtype=torch.bool, device=device)
     x = logits.to(device).requires_grad_(True)
