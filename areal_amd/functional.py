@@ -356,6 +356,7 @@ def apply_rejection_sampling(
 class _PpoLoss(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logp, prox, adv, mask_eff, behave_w, cu, B, seq_level, params, n_valid):
+        ctx.set_materialize_grads(False)  # no zero-filled gradients for the outputs that have none
         lib = N.load()
         dev = logp.device
         n = logp.numel()
@@ -384,8 +385,16 @@ class _PpoLoss(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g_loss, *_unused):
+        if g_loss is None:  # the loss was not used (gradients are not materialised, see forward)
+            return (None,) * 10
         (g_logp,) = ctx.saved_tensors
         return (g_logp * g_loss,) + (None,) * 9
+
+
+def _flag_bits(flags: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """(clip_mask, dual_clip_mask) as bool tensors from the kernels' flag bytes (bit 0, bit 1): one launch each, the
+    0 / 1 bytes reinterpreted as bool."""
+    return torch.bitwise_and(flags, 1).view(torch.bool), torch.bitwise_right_shift(flags, 1).view(torch.bool)
 
 
 def _count_nonzero(mask_u8: torch.Tensor) -> torch.Tensor:
@@ -467,12 +476,13 @@ def ppo_actor_loss_fn(
         n_valid = _count_nonzero(m8)
 
     loss, stat_loss, ratio, flags = _PpoLoss.apply(lp, prox, adv, mask_eff, w, cu, B, seq_level, params, n_valid)
+    clip, dual = _flag_bits(flags)
     stat = dict(
         loss=stat_loss.view(shape),
         importance_weight=ratio.view(shape),
         approx_kl=(lp.detach() - prox).view(shape),
-        clip_mask=(flags & 1).bool().view(shape),
-        dual_clip_mask=(flags & 2).bool().view(shape),
+        clip_mask=clip.view(shape),
+        dual_clip_mask=dual.view(shape),
     )
     if rejection_sampling is not None:
         _rs_stats(stat, prox, old, mask_eff, w, host_counts, shape)
@@ -509,6 +519,7 @@ class _FusedLogitsPpo(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits2d, labels1d, stride, temperature, T_active, prox, adv, mask_eff, behave_w, params,
                 n_valid, grad_scale, want_minmax, inplace=False):
+        ctx.set_materialize_grads(False)  # no zero-filled gradients for the outputs that have none
         lib = N.load()
         T, V = logits2d.shape
         dev = logits2d.device
@@ -552,6 +563,8 @@ class _FusedLogitsPpo(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g_loss, *_unused):
+        if g_loss is None:
+            return (None,) * 14
         _hand_out_once(ctx)
         lib = N.load()
         (dlogits,) = ctx.saved_tensors
@@ -668,12 +681,13 @@ def fused_logprobs_ppo_loss(
         bool(inplace_backward),
     )
     logp_a = logp[:T_active]
+    clip, dual = _flag_bits(flags)
     stat = dict(
         loss=stat_loss,
         importance_weight=ratio,
         approx_kl=logp_a - prox,
-        clip_mask=(flags & 1).bool(),
-        dual_clip_mask=(flags & 2).bool(),
+        clip_mask=clip,
+        dual_clip_mask=dual,
         logprobs=logp_a,
         entropy=entropy[:T_active],
         vocab_min_logits=vmin[:T_active],
@@ -846,6 +860,7 @@ class _FusedLmHeadPpo(torch.autograd.Function):
     @staticmethod
     def forward(ctx, hidden, weight, labels, temperature, T_active, prox, adv, mask_eff, behave_w, params, n_valid,
                 grad_scale, kept_per_chunk, backward_mode):
+        ctx.set_materialize_grads(False)  # no zero-filled gradients for the outputs that have none
         lib = N.load()
         kept = None if kept_per_chunk is None else (C.c_int64 * len(kept_per_chunk))(*kept_per_chunk)
         T, H = hidden.shape
@@ -879,6 +894,8 @@ class _FusedLmHeadPpo(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g_loss, *_unused):
+        if g_loss is None:
+            return (None,) * 14
         _hand_out_once(ctx)
         lib = N.load()
         d_hidden, d_weight = ctx.saved_tensors
@@ -1023,9 +1040,10 @@ def fused_lm_head_ppo_loss(
                 None if w is None else w.index_select(0, idx), params, n_valid, scale_t, kept, _LMHEAD_BACKWARD[backward],
             )
             logp, entropy = logp[:n_kept], entropy[:n_kept]
+            clip, dual = _flag_bits(flags)
             stat = dict(
                 loss=full(stat_loss), importance_weight=full(ratio), approx_kl=full(logp - prox.index_select(0, idx)),
-                clip_mask=full((flags & 1).bool(), torch.bool), dual_clip_mask=full((flags & 2).bool(), torch.bool),
+                clip_mask=full(clip, torch.bool), dual_clip_mask=full(dual, torch.bool),
                 logprobs=full(logp), entropy=full(entropy),
             )
         if rejection_sampling is not None:
@@ -1049,12 +1067,13 @@ def fused_lm_head_ppo_loss(
         n_valid, scale_t, kept, _LMHEAD_BACKWARD[backward],
     )
     logp_a = logp[:T_active]
+    clip, dual = _flag_bits(flags)
     stat = dict(
         loss=stat_loss,
         importance_weight=ratio,
         approx_kl=logp_a - prox,
-        clip_mask=(flags & 1).bool(),
-        dual_clip_mask=(flags & 2).bool(),
+        clip_mask=clip,
+        dual_clip_mask=dual,
         logprobs=logp_a,
         entropy=entropy[:T_active],
     )
@@ -1092,6 +1111,8 @@ class _SapoLoss(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g_loss, *_unused):
+        if g_loss is None:  # the loss was not used (gradients are not materialised, see forward)
+            return (None,) * 10
         (g_logp,) = ctx.saved_tensors
         return (g_logp * g_loss,) + (None,) * 9
 
