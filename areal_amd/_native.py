@@ -77,6 +77,7 @@ SIGNATURES = {
     "aa_count_nonzero_u8": (_i, [_p, _i64, _p, _p]),
     "aa_ppo_loss": (_i, [_p, _p, _p, _p, _p, _i64, _p, _i64, _i, C.POINTER(PpoParams), _p, _p, _p, _p, _p, _p]),
     "aa_masked_sum": (_i, [_p, _p, _i64, _p, _p, _p, _p]),
+    "aa_ppo_stat_outputs": (_i, [_p, _p, _p, _p, _p, _p, _i64, _p, _p, _p, _p, _p, _p]),
     "aa_scale_inplace": (_i, [_p, _i, _i64, _p, _p]),
     "aa_scale_rows_inplace": (_i, [_p, _i, _i64, _i64, _i64, _p, _p]),
     "aa_lmhead_workspace_bytes": (_i64, [_i64, _i64, _i64]),

@@ -314,6 +314,29 @@ __global__ __launch_bounds__(1024) void k_masked_sum(const float* __restrict__ v
   }
 }
 
+// ---- the derived entries of the stat dict (functional.py:505-558), one launch instead of one per entry ------------
+__global__ __launch_bounds__(256) void k_ppo_stat_outputs(const float* __restrict__ logp, const float* __restrict__ prox,
+                                                          const float* __restrict__ old, const uint8_t* __restrict__ flags,
+                                                          const float* __restrict__ behave_w,
+                                                          const uint8_t* __restrict__ mask_eff, int64_t n,
+                                                          float* __restrict__ approx_kl, uint8_t* __restrict__ clip,
+                                                          uint8_t* __restrict__ dual, uint8_t* __restrict__ behave_mask,
+                                                          float* __restrict__ behave_kl) {
+  const int64_t step = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += step) {
+    const float p = prox[i];
+    approx_kl[i] = logp[i] - p;
+    const uint8_t f = flags[i];
+    clip[i] = f & 1;
+    dual[i] = (f >> 1) & 1;
+    if (behave_mask) {
+      const bool on = behave_w[i] > 0.f && mask_eff[i] != 0;
+      behave_mask[i] = on ? 1 : 0;
+      behave_kl[i] = on ? p - old[i] : 0.f;
+    }
+  }
+}
+
 // ---- SAPO: soft sigmoid gates instead of clipping (functional.py:562-638) ---------------------------------------
 struct SapoTerm {
   float loss, dloss_dr, soft, gate_pos, gate_neg;
@@ -555,6 +578,20 @@ extern "C" int aa_masked_sum(const float* values, const uint8_t* mask, int64_t n
                              const float* scale, float* out, void* stream) {
   if (!out || n < 0 || (n > 0 && !values)) return AA_ERR_INVALID_ARGUMENT;
   hipLaunchKernelGGL(k_masked_sum, dim3(1), dim3(1024), 0, (hipStream_t)stream, values, mask, n, n_valid, scale, out);
+  return launch_status();
+}
+
+extern "C" int aa_ppo_stat_outputs(const float* logp, const float* prox_logp, const float* old_logp, const uint8_t* flags,
+                                   const float* behave_w, const uint8_t* mask_eff, int64_t n, float* approx_kl,
+                                   uint8_t* clip_mask, uint8_t* dual_clip_mask, uint8_t* behave_mask,
+                                   float* behave_approx_kl, void* stream) {
+  if (n < 0) return AA_ERR_INVALID_ARGUMENT;
+  if (n == 0) return AA_OK;
+  if (!logp || !prox_logp || !flags || !approx_kl || !clip_mask || !dual_clip_mask) return AA_ERR_INVALID_ARGUMENT;
+  if ((behave_mask != nullptr) != (behave_approx_kl != nullptr)) return AA_ERR_INVALID_ARGUMENT;
+  if (behave_mask && (!old_logp || !behave_w || !mask_eff)) return AA_ERR_INVALID_ARGUMENT;
+  hipLaunchKernelGGL(k_ppo_stat_outputs, dim3(grid_for(n)), dim3(256), 0, (hipStream_t)stream, logp, prox_logp, old_logp,
+                     flags, behave_w, mask_eff, n, approx_kl, clip_mask, dual_clip_mask, behave_mask, behave_approx_kl);
   return launch_status();
 }
 

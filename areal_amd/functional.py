@@ -406,11 +406,37 @@ def _count_nonzero(mask_u8: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def _rs_stats(stat, prox, old, mask_eff_u8, w, counts, shape):
-    behave_mask = (w > 0) & mask_eff_u8.bool()
+def _stat_outputs(logp, prox, old, flags, w, mask_eff_u8):
+    """The derived entries of the stat dict (functional.py:505-558) in one launch: ``approx_kl``, ``clip_mask``,
+    ``dual_clip_mask`` and, with rejection sampling (``w`` given), ``behave_mask`` and ``behave_approx_kl``
+    (None otherwise)."""
+    lib = N.load()
+    dev = logp.device
+    n = logp.numel()
+    logp = logp.detach()
+    logp = logp if logp.is_contiguous() else logp.contiguous()
+    approx_kl = torch.empty(n, dtype=torch.float32, device=dev)
+    clip = torch.empty(n, dtype=torch.uint8, device=dev)
+    dual = torch.empty(n, dtype=torch.uint8, device=dev)
+    behave_mask = behave_kl = None
+    if w is not None:
+        behave_mask = torch.empty(n, dtype=torch.uint8, device=dev)
+        behave_kl = torch.empty(n, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        N.check(
+            lib.aa_ppo_stat_outputs(_ptr(logp), _ptr(prox), _ptr(old), _ptr(flags), _ptr(w), _ptr(mask_eff_u8), n,
+                                    _ptr(approx_kl), _ptr(clip), _ptr(dual), _ptr(behave_mask), _ptr(behave_kl),
+                                    _stream(dev)),
+            "aa_ppo_stat_outputs",
+        )
+    as_bool = lambda t: None if t is None else t.view(torch.bool)
+    return approx_kl, as_bool(clip), as_bool(dual), as_bool(behave_mask), behave_kl
+
+
+def _rs_stats(stat, behave_mask, behave_kl, w, counts, shape):
     total, hit, _ = counts.tolist()
     stat.update(
-        behave_approx_kl=torch.where(behave_mask, prox - old, 0.0).view(shape),
+        behave_approx_kl=behave_kl.view(shape),
         behave_imp_weight=w.view(shape),
         behave_mask=behave_mask.view(shape),
         filtered_fraction=hit / max(total, 1),
@@ -476,16 +502,16 @@ def ppo_actor_loss_fn(
         n_valid = _count_nonzero(m8)
 
     loss, stat_loss, ratio, flags = _PpoLoss.apply(lp, prox, adv, mask_eff, w, cu, B, seq_level, params, n_valid)
-    clip, dual = _flag_bits(flags)
+    approx_kl, clip, dual, behave_mask, behave_kl = _stat_outputs(lp, prox, old, flags, w, mask_eff)
     stat = dict(
         loss=stat_loss.view(shape),
         importance_weight=ratio.view(shape),
-        approx_kl=(lp.detach() - prox).view(shape),
+        approx_kl=approx_kl.view(shape),
         clip_mask=clip.view(shape),
         dual_clip_mask=dual.view(shape),
     )
     if rejection_sampling is not None:
-        _rs_stats(stat, prox, old, mask_eff, w, host_counts, shape)
+        _rs_stats(stat, behave_mask, behave_kl, w, host_counts, shape)
     return loss, stat
 
 
@@ -681,11 +707,11 @@ def fused_logprobs_ppo_loss(
         bool(inplace_backward),
     )
     logp_a = logp[:T_active]
-    clip, dual = _flag_bits(flags)
+    approx_kl, clip, dual, behave_mask, behave_kl = _stat_outputs(logp_a, prox, old, flags, w, mask_eff)
     stat = dict(
         loss=stat_loss,
         importance_weight=ratio,
-        approx_kl=logp_a - prox,
+        approx_kl=approx_kl,
         clip_mask=clip,
         dual_clip_mask=dual,
         logprobs=logp_a,
@@ -694,7 +720,7 @@ def fused_logprobs_ppo_loss(
         vocab_max_logits=vmax[:T_active],
     )
     if rejection_sampling is not None:
-        _rs_stats(stat, prox, old, mask_eff, w, host_counts, loss_mask.shape)
+        _rs_stats(stat, behave_mask, behave_kl, w, host_counts, loss_mask.shape)
     return loss, stat
 
 
@@ -1047,7 +1073,8 @@ def fused_lm_head_ppo_loss(
                 logprobs=full(logp), entropy=full(entropy),
             )
         if rejection_sampling is not None:
-            _rs_stats(stat, prox, old, mask_eff, w, host_counts, loss_mask.shape)
+            behave_mask = (w > 0) & mask_eff.bool()
+            _rs_stats(stat, behave_mask, torch.where(behave_mask, prox - old, 0.0), w, host_counts, loss_mask.shape)
         return loss, stat
     kept = None
     if skip_masked_tokens and kept_per_chunk is not None:
@@ -1067,18 +1094,18 @@ def fused_lm_head_ppo_loss(
         n_valid, scale_t, kept, _LMHEAD_BACKWARD[backward],
     )
     logp_a = logp[:T_active]
-    clip, dual = _flag_bits(flags)
+    approx_kl, clip, dual, behave_mask, behave_kl = _stat_outputs(logp_a, prox, old, flags, w, mask_eff)
     stat = dict(
         loss=stat_loss,
         importance_weight=ratio,
-        approx_kl=logp_a - prox,
+        approx_kl=approx_kl,
         clip_mask=clip,
         dual_clip_mask=dual,
         logprobs=logp_a,
         entropy=entropy[:T_active],
     )
     if rejection_sampling is not None:
-        _rs_stats(stat, prox, old, mask_eff, w, host_counts, loss_mask.shape)
+        _rs_stats(stat, behave_mask, behave_kl, w, host_counts, loss_mask.shape)
     return loss, stat
 
 

@@ -241,6 +241,24 @@ int aa_ppo_loss(const float* logp, const float* prox_logp, const float* adv,
                 void* stream);
 
 /*
+ * The derived entries of the stat dict of ppo_actor_loss_fn
+ * (functional.py:505-558), which the reference forms with one small launch
+ * each, in one launch:
+ *   approx_kl = logp - prox_logp;  clip_mask, dual_clip_mask = bit 0 and bit 1
+ *   of flags (bytes 0 / 1);  and, when behave_mask is given (rejection
+ *   sampling), behave_mask = behave_w > 0 && mask_eff != 0 and
+ *   behave_approx_kl = behave_mask ? prox_logp - old_logp : 0.
+ * behave_mask and behave_approx_kl are both NULL or both given (then old_logp,
+ * behave_w and mask_eff are required).
+ */
+int aa_ppo_stat_outputs(const float* logp, const float* prox_logp,
+                        const float* old_logp, const uint8_t* flags,
+                        const float* behave_w, const uint8_t* mask_eff,
+                        int64_t n, float* approx_kl, uint8_t* clip_mask,
+                        uint8_t* dual_clip_mask, uint8_t* behave_mask,
+                        float* behave_approx_kl, void* stream);
+
+/*
  * out[0] = scale * sum_{i<n, mask[i] != 0} values[i] / max(*n_valid, 1)
  * (functional.py:542), accumulated in a fixed order so that repeated calls are
  * bit-identical.  n_valid may be NULL (divide by 1); scale may be NULL (1);
