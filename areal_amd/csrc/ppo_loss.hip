@@ -292,16 +292,29 @@ __global__ __launch_bounds__(1024) void k_masked_sum(const float* __restrict__ v
   // four elements per thread and trip (16-byte value loads when the base allows), always in the same order
   const bool vec = (((uintptr_t)values) & 15) == 0 && (!mask || (((uintptr_t)mask) & 3) == 0);
   const int64_t n4 = vec ? (n >> 2) : 0;
-  for (int64_t q = threadIdx.x; q < n4; q += 1024) {
-    const float4 v = ((const float4*)values)[q];
-    const uint32_t m = mask ? ((const uint32_t*)mask)[q] : 0x01010101u;
+  auto part_of = [](const float4 v, const uint32_t m) {
     double part = 0.0;
     if (m & 0x000000ffu) part += (double)v.x;
     if (m & 0x0000ff00u) part += (double)v.y;
     if (m & 0x00ff0000u) part += (double)v.z;
     if (m & 0xff000000u) part += (double)v.w;
-    acc += part;
+    return part;
+  };
+  // four trips at a time, their loads issued together (one workgroup: the loop is bound by memory latency); the
+  // order of the additions is the one of the plain loop
+  int64_t q = threadIdx.x;
+  for (; q + 3 * 1024 < n4; q += 4 * 1024) {
+    float4 v[4];
+    uint32_t m[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      v[j] = ((const float4*)values)[q + j * 1024];
+      m[j] = mask ? ((const uint32_t*)mask)[q + j * 1024] : 0x01010101u;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc += part_of(v[j], m[j]);
   }
+  for (; q < n4; q += 1024) acc += part_of(((const float4*)values)[q], mask ? ((const uint32_t*)mask)[q] : 0x01010101u);
   for (int64_t i = (n4 << 2) + threadIdx.x; i < n; i += 1024)
     if (!mask || mask[i] != 0) acc += (double)values[i];
   acc = block_sum<double>(acc, smem);
