@@ -117,8 +117,9 @@ class _LogprobsEntropy(torch.autograd.Function):
     """logp, entropy, vocab max, vocab min of each row; differentiable in logits."""
 
     @staticmethod
-    def forward(ctx, logits2d, labels1d, temperature, stride, want_entropy, want_minmax):
+    def forward(ctx, logits2d, labels1d, temperature, stride, want_entropy, want_minmax, inplace=False):
         lib = N.load()
+        ctx.inplace = bool(inplace)
         T, V = logits2d.shape
         dev = logits2d.device
         kw = dict(dtype=torch.float32, device=dev)
@@ -155,7 +156,11 @@ class _LogprobsEntropy(torch.autograd.Function):
             g_logp = torch.zeros(T, dtype=torch.float32, device=dev)
         g_logp = _f32(g_logp)
         g_entropy = _f32(g_entropy) if (g_entropy is not None and row_ez is not None) else None
-        if ctx.stride == V:
+        if ctx.inplace:
+            # the gradient takes the place of the logits (the kernel reads an element before it writes it); the version
+            # bump below makes any other operation that kept the logits for its own backward fail loudly
+            dlogits = logits2d.detach()
+        elif ctx.stride == V:
             dlogits = torch.empty_like(logits2d, memory_format=torch.contiguous_format)
         else:  # keep the row stride of the input so that both buffers are walked alike
             dlogits = torch.empty_strided((T, V), (ctx.stride, 1), dtype=logits2d.dtype, device=dev)
@@ -168,10 +173,12 @@ class _LogprobsEntropy(torch.autograd.Function):
                 ),
                 "aa_logits_bwd",
             )
-        return dlogits, None, None, None, None, None
+        if ctx.inplace:
+            torch.autograd.graph.increment_version(logits2d)
+        return dlogits, None, None, None, None, None, None
 
 
-def _logprobs_impl(logits, labels, temperature, tp_group, want_entropy, want_minmax):
+def _logprobs_impl(logits, labels, temperature, tp_group, want_entropy, want_minmax, inplace_backward=False):
     _check_tp(tp_group)
     _require_gpu(logits, "logits")
     assert logits.shape[0] > 0, "Input logits must have at least one element"
@@ -179,7 +186,8 @@ def _logprobs_impl(logits, labels, temperature, tp_group, want_entropy, want_min
         raise ValueError(f"labels shape {tuple(labels.shape)} != logits shape[:-1] {tuple(logits.shape[:-1])}")
     x, T, V, stride = _rows(logits)
     y = labels.reshape(-1).to(device=x.device, dtype=torch.int64).contiguous()
-    logp, entropy, vmax, vmin = _LogprobsEntropy.apply(x, y, float(temperature), stride, want_entropy, want_minmax)
+    logp, entropy, vmax, vmin = _LogprobsEntropy.apply(x, y, float(temperature), stride, want_entropy, want_minmax,
+                                                       bool(inplace_backward))
     shp = labels.shape
     return (
         logp.view(shp),
@@ -195,15 +203,19 @@ def gather_logprobs(
     temperature: float = 1.0,
     tp_group: Any | None = None,
     chunk_size: int = 1024,
+    inplace_backward: bool = False,
 ) -> torch.Tensor:
     """``log_softmax(logits.float() / temperature)[..., labels]`` as fp32, shaped like ``labels``.
 
     Same contract as vocab_parallel.py:401-431.  ``chunk_size`` is accepted and
     ignored: the kernel never materialises an fp32 copy of the logits, and the
-    result does not depend on chunking.
+    result does not depend on chunking.  ``inplace_backward=True`` (not in the
+    reference): the backward pass writes the gradient over the logits instead
+    of allocating a second ``[T, V]`` array; for callers that need the logits
+    for nothing else after this op.
     """
     del chunk_size
-    return _logprobs_impl(logits, labels, temperature, tp_group, False, False)[0]
+    return _logprobs_impl(logits, labels, temperature, tp_group, False, False, inplace_backward)[0]
 
 
 def gather_logprobs_entropy(
@@ -212,22 +224,24 @@ def gather_logprobs_entropy(
     temperature: float = 1.0,
     tp_group: Any | None = None,
     chunk_size: int = 1024,
+    inplace_backward: bool = False,
 ) -> tuple[torch.Tensor, torch.Tensor]:
-    """(log-probs at ``labels``, entropy of each row); vocab_parallel.py:434-469."""
+    """(log-probs at ``labels``, entropy of each row); vocab_parallel.py:434-469.  ``inplace_backward`` as in
+    ``gather_logprobs``."""
     del chunk_size
-    logp, entropy, _, _ = _logprobs_impl(logits, labels, temperature, tp_group, True, False)
+    logp, entropy, _, _ = _logprobs_impl(logits, labels, temperature, tp_group, True, False, inplace_backward)
     return logp, entropy
 
 
 def gather_logprobs_entropy_stats(
-    logits: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0
+    logits: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0, inplace_backward: bool = False
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """(logp, entropy, vocab_min_logits, vocab_max_logits) from the same single pass.
 
     The last two are what FSDPEngine._get_vocab_min_max_logits
     (fsdp_engine.py:1893-1906) computes with two more passes over the logits.
     """
-    logp, entropy, vmax, vmin = _logprobs_impl(logits, labels, temperature, None, True, True)
+    logp, entropy, vmax, vmin = _logprobs_impl(logits, labels, temperature, None, True, True, inplace_backward)
     return logp, entropy, vmin, vmax
 
 
@@ -657,7 +671,8 @@ def fused_logprobs_ppo_loss(
     call ``logits`` holds its own gradient (for an upstream factor of 1), so it
     is for callers that need the logits for nothing else; an operation that
     saved them for its backward raises autograd's modified-in-place error.
-    Ignored where no gradient is produced and on the sequence-level path.
+    On the sequence-level path the gradient lands there during
+    ``loss.backward()``.  Ignored where no gradient is produced.
     """
     if importance_sampling_level not in ("token", "sequence"):
         raise ValueError(
@@ -682,7 +697,8 @@ def fused_logprobs_ppo_loss(
     # no [T, V] gradient buffer) followed by the loss on log-probs.
     forward_only = not (torch.is_grad_enabled() and logits.requires_grad)
     if importance_sampling_level == "sequence" or forward_only:
-        logp, entropy, vmin, vmax = gather_logprobs_entropy_stats(logits, labels, temperature)
+        logp, entropy, vmin, vmax = gather_logprobs_entropy_stats(logits, labels, temperature,
+                                                                  inplace_backward and not forward_only)
         logp, entropy, vmin, vmax = (t[:T_active] for t in (logp, entropy, vmin, vmax))
         loss, stat = ppo_actor_loss_fn(
             logp, proximal_logprobs, old_logprobs, advantages, eps_clip, loss_mask, eps_clip_higher, c_clip,

@@ -100,6 +100,8 @@ int aa_logits_fwd(const void* logits, int dtype, int64_t T, int64_t V,
  * g_entropy may be NULL (treated as zero).  dlogits has the dtype and row
  * stride of logits.  Rows with t >= T_active (the batch padding the caller
  * trims after the op, fsdp_engine.py:2027-2031) are written as zeros.
+ * dlogits may be the logits array itself (every element is read before it is
+ * written, by the same thread); any other overlap is not allowed.
  */
 int aa_logits_bwd(const void* logits, int dtype, int64_t T, int64_t V,
                   int64_t row_stride, const int64_t* labels,

@@ -275,3 +275,44 @@ def test_vocab_shards_equal_the_unsharded_op(device, cuts, dtype, temperature):
     lse, ez, lpl, _ = VP.shard_statistics(shards[0], torch.full((T,), V + 5), 0, temperature)
     out = VP.combine_shard_statistics(lse[None], ez[None], lpl[None])
     assert bool(torch.isnan(out[0]).all()) and bool(torch.isfinite(out[1]).all())
+
+
+@pytest.mark.parametrize("V,dtype", [(16384, torch.bfloat16), (50257, torch.bfloat16), (4099, torch.float32)])
+def test_backward_written_over_the_logits(device, V, dtype):
+    """inplace_backward=True: the backward pass of the log-prob op writes the gradient over the logits, with the bits
+    of the separate array; through a producer of the logits, and through the sequence-level PPO loss."""
+    g = torch.Generator().manual_seed(V)
+    T = 37
+    logits = (2 * torch.randn(T, V, generator=g)).to(dtype).to(device)
+    labels = torch.randint(0, V, (T,), generator=g).to(device)
+    g_lp, g_ent = torch.randn(T, generator=g).to(device), torch.randn(T, generator=g).to(device)
+
+    def run(inplace):
+        base = logits.clone().requires_grad_(True)
+        x = base * 1.0                                   # a producer: the logits are not a leaf
+        lp, ent = areal_amd.gather_logprobs_entropy(x, labels, 0.8, inplace_backward=inplace)
+        (lp * g_lp + ent * g_ent).sum().backward()
+        return lp.detach(), ent.detach(), base.grad, x.detach()
+
+    lp0, ent0, grad0, x0 = run(False)
+    lp1, ent1, grad1, x1 = run(True)
+    assert torch.equal(lp0, lp1) and torch.equal(ent0, ent1) and torch.equal(grad0, grad1)
+    assert torch.equal(x0, logits) and torch.equal(x1, grad1)   # untouched / holds its own gradient
+
+    # sequence-level importance ratios: the unfused kernels behind fused_logprobs_ppo_loss
+    cu = torch.tensor([0, 20, T], dtype=torch.int32, device=device)
+    ref = areal_amd.gather_logprobs(logits, labels).detach()
+    adv, mask = torch.randn(T, generator=g).to(device), (torch.rand(T, generator=g) < 0.7).to(device)
+
+    def step(inplace):
+        base = logits.clone().requires_grad_(True)
+        x = base * 1.0
+        loss, _ = areal_amd.fused_logprobs_ppo_loss(x, labels, ref - 0.05, ref + 0.03, adv, 0.2, mask,
+                                                    importance_sampling_level="sequence", cu_seqlens=cu,
+                                                    inplace_backward=inplace)
+        loss.backward()
+        return loss.detach(), base.grad
+
+    l0, s0 = step(False)
+    l1, s1 = step(True)
+    assert torch.equal(l0, l1) and torch.equal(s0, s1)
