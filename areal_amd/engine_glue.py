@@ -55,8 +55,8 @@ def compute_logprobs_and_loss(
 
     ``logits`` is ``[T_pad, V]``; ``mb_input`` holds the un-padded ``[T]`` tensors ``loss_mask``, ``logprobs``
     (behaviour policy), ``prox_logp``, ``advantages`` and ``cu_seqlens``.  An all-masked micro-batch returns
-    ``logits.mean() * 0`` like the reference (fsdp_engine.py:1988-1989).  ``inplace_backward`` (fused path only):
-    the gradient is written over the logits, see ``fused_logprobs_ppo_loss``.
+    ``logits.mean() * 0`` like the reference (fsdp_engine.py:1988-1989).  ``inplace_backward``: the gradient is
+    written over the logits, see ``fused_logprobs_ppo_loss``.
     """
     loss_mask = mb_input["loss_mask"].bool()
     local_weight = loss_mask.count_nonzero()
@@ -77,7 +77,7 @@ def compute_logprobs_and_loss(
             logits, labels, prox_logp, old_logp, mb_input["advantages"], loss_mask=loss_mask,
             temperature=temperature, loss_scale=scale, inplace_backward=inplace_backward, **kw,
         )
-    logp, entropy, vmin, vmax = gather_logprobs_entropy_stats(logits, labels, temperature)
+    logp, entropy, vmin, vmax = gather_logprobs_entropy_stats(logits, labels, temperature, inplace_backward)
     if pad_length > 0:
         logp, entropy, vmin, vmax = (t[:-pad_length] for t in (logp, entropy, vmin, vmax))
     loss, stat = ppo_actor_loss_fn(logp, prox_logp, old_logp, mb_input["advantages"], loss_mask=loss_mask, **kw)
