@@ -755,6 +755,11 @@ def fused_logprobs_ppo_loss(
 _LMHEAD_BACKWARD = {"recompute": 0, "carry": 1}  # aa_lmhead_backward_mode
 
 
+def lm_head_chunk_tokens() -> int:
+    """Tokens per chunk of the lm_head entry points (what ``kept_per_chunk`` counts over)."""
+    return int(N.load().aa_lmhead_chunk_tokens())
+
+
 def _lmhead_workspace(T: int, H: int, V: int, dev, forward_only: bool = False) -> torch.Tensor:
     lib = N.load()
     n = lib.aa_lmhead_fwd_workspace_bytes(T, H, V) if forward_only else lib.aa_lmhead_workspace_bytes(T, H, V)
