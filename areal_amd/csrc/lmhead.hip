@@ -483,6 +483,82 @@ __global__ __launch_bounds__(kThreads) void k_gemm_store(Operand A, Operand B, i
   }
 }
 
+// ---- the same product cut along K ------------------------------------------------------------------------------
+// d_hidden has few tiles (16 x rows / 256 at H = 4096): when their number is a little above a multiple of the compute
+// units, the last round of tiles runs on a mostly idle chip and costs almost a whole round all the same (measured:
+// 576 tiles = 2.25 rounds take 9.7 ms where 512 tiles take 6.9 ms).  Cut along K into `splits` parts, the tiles are
+// `splits` times as many and as much shorter, so the last round wastes that much less.  Part s of tile (tm, tn) sums
+// the K slices [s * per, (s + 1) * per) into its own fp32 plane; k_splitk_rows adds the planes in order.  Workgroups
+// are numbered so that an XCD runs a contiguous range of (part, tile): the tiles that share operand slices in its L2
+// are those of one part.
+template <bool AKM, bool BKM>
+__global__ __launch_bounds__(kThreads) void k_gemm_splitk(Operand A, Operand B, int K, int tiles_m, int tiles_n, int splits,
+                                                          float* __restrict__ part, int64_t ldc, int64_t plane) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const int tiles = tiles_m * tiles_n;
+  const int q = xcd_contiguous(blockIdx.x, tiles * splits);
+  const int split = q / tiles;
+  int tm, tn;
+  tile_at(q - split * tiles, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int nk = (K + BK - 1) / BK, per = (nk + splits - 1) / splits;
+  const int k_begin = split * per * BK;
+  int k_len = K - k_begin;
+  k_len = k_len < 0 ? 0 : (k_len > per * BK ? per * BK : k_len);  // 0: this part has nothing, its plane gets zeros
+  const int64_t shift = k_len > 0 ? k_begin : 0;
+  A.ptr += AKM ? shift * A.ld : shift;
+  B.ptr += BKM ? shift * B.ld : shift;
+  Acc acc;
+  mainloop<AKM, BKM>(A, B, k_len, m0, n0, acc, lds);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int M = A.rows, N = B.rows;
+  float* C = part + (int64_t)split * plane;
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) {
+    const int n = n0 + wn * 128 + acc_col(nt, lane);
+    if (n >= N) continue;
+    float* row = C + n * ldc;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const int m = m0 + wm * 128 + mt * 32 + 8 * g4 + 4 * (lane >> 5);  // M % 4 == 0
+        if (m >= M) continue;
+        const f32x4_t v = {acc.v[mt][nt][g4 * 4], acc.v[mt][nt][g4 * 4 + 1], acc.v[mt][nt][g4 * 4 + 2], acc.v[mt][nt][g4 * 4 + 3]};
+        *(f32x4_t*)(row + m) = v;
+      }
+  }
+}
+
+// out[c_rows[r], :] = bf16(n_scale[r] * (plane 0 + plane 1 + ...)[r, :]), the planes added in order; M % 8 == 0.
+// c_rows == nullptr: row r itself (a negative entry: the row is dropped); n_scale == nullptr: 1.
+__global__ __launch_bounds__(256) void k_splitk_rows(const float* __restrict__ part, int splits, int64_t plane, int M,
+                                                     const int32_t* __restrict__ c_rows, const float* __restrict__ n_scale,
+                                                     uint16_t* __restrict__ out, int64_t ldo) {
+  const int64_t r = blockIdx.x;
+  const int64_t dst = c_rows ? c_rows[r] : r;
+  if (dst < 0) return;
+  const float f = n_scale ? n_scale[r] : 1.f;
+  for (int m = threadIdx.x * 8; m < M; m += 256 * 8) {
+    float a[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a[i] = 0.f;
+    for (int sp = 0; sp < splits; ++sp) {
+      const float* src = part + (int64_t)sp * plane + r * M + m;
+      const f32x4_t lo = *(const f32x4_t*)src, hi = *(const f32x4_t*)(src + 4);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        a[i] += lo[i];
+        a[4 + i] += hi[i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a[i] *= f;
+    store8<AA_BF16>(out + dst * ldo, m, a);
+  }
+}
+
 // ---- tokens without gradient are left out of the backward GEMMs -------------------------------------------------
 // A token whose loss mask is zero has d(loss)/d(logits) == 0: its row adds nothing to d_weight and its d_hidden row
 // is zero.  k_compact_map numbers the tokens of a chunk that do have a mask (in order): out_rows[t] = position of
@@ -571,6 +647,8 @@ __global__ __launch_bounds__(256) void k_f32_to_bf16(const f32x4_t* __restrict__
 }
 
 // ---- workspace ---------------------------------------------------------------------------------------------------
+constexpr int kMaxSplits = 4;  // of the d_hidden product along K
+
 struct Workspace {
   int64_t chunk, blocks;                // tokens per chunk, 128-row vocabulary blocks
   int64_t off_pk, off_ps, off_pu;       // block partials [blocks][chunk]
@@ -581,6 +659,7 @@ struct Workspace {
   int64_t off_panel;                    // d(logits) rows [chunk, V]
   int64_t off_hc;                       // the hidden rows of the tokens with gradient, closed up [chunk, H]
   int64_t off_dw;                       // fp32 accumulator of a bf16 d_weight when there is more than one chunk
+  int64_t off_dhp;                      // fp32 planes of a d_hidden product cut along K [kMaxSplits][chunk, H]
   int64_t bytes;
 };
 
@@ -603,6 +682,7 @@ static Workspace plan(int64_t T, int64_t H, int64_t V) {
   w.off_panel = off;   off += up(w.chunk * V * 2);
   w.off_hc = off;      off += up(w.chunk * H * 2);
   w.off_dw = off;      off += T > w.chunk ? up(V * H * 4) : 0;
+  w.off_dhp = off;     off += up(kMaxSplits * w.chunk * H * 4);
   w.bytes = off;
   return w;
 }
@@ -627,9 +707,41 @@ static bool prepare_kernels() {
   const bool ok = allow_big_lds(k_lmhead_tiles<kModeStats>) && allow_big_lds(k_lmhead_tiles<kModeStatsCarry>) &&
                   allow_big_lds(k_lmhead_tiles<kModeRecompute>) && allow_big_lds(k_gemm_store<true, false, uint16_t, false>) &&
                   allow_big_lds(k_gemm_store<true, true, uint16_t, false>) &&
-                  allow_big_lds(k_gemm_store<true, true, float, false>) && allow_big_lds(k_gemm_store<true, true, float, true>);
+                  allow_big_lds(k_gemm_store<true, true, float, false>) && allow_big_lds(k_gemm_store<true, true, float, true>) &&
+                  allow_big_lds(k_gemm_splitk<true, false>);
   done[dev] = ok;
   return ok;
+}
+
+// compute units of the current device (0 if unknown), asked for once per device
+static int compute_units() {
+  constexpr int kMaxDevices = 64;
+  static int units[kMaxDevices] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+  if (units[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
+    units[dev] = n > 0 ? n : -1;
+  }
+  return units[dev] > 0 ? units[dev] : 0;
+}
+
+// Into how many parts along K a product of `tiles` tiles and `slices` K slices is cut (1: not at all): the number of
+// parts, up to kMaxSplits, that shortens the time in rounds of tiles, ceil(tiles * parts / units) / parts, the most,
+// with 0.03 rounds charged per part for writing and adding its fp32 plane; at least 5 % have to be won, and a part
+// keeps at least 64 slices.
+static int choose_splits(int64_t tiles, int64_t slices, int units) {
+  if (units <= 0 || tiles <= 0) return 1;
+  auto rounds = [&](int parts) { return (double)((tiles * parts + units - 1) / units) / parts + 0.03 * parts; };
+  int best = 1;
+  double best_rounds = (rounds(1) - 0.03) * 0.95;
+  for (int parts = 2; parts <= kMaxSplits && slices / parts >= 64; ++parts)
+    if (rounds(parts) < best_rounds) {
+      best = parts;
+      best_rounds = rounds(parts);
+    }
+  return best;
 }
 
 template <int MODE>
@@ -673,8 +785,22 @@ static void panel_gradients(hipStream_t st, const Workspace& w, char* ws, const 
                        (u32x4_t*)hc, (int)(H / 8), row_factor, (const int32_t*)nullptr);
     hid_rows = hc;
   }
-  launch_gemm<true, false, uint16_t, false>(st, (const uint16_t*)weight, H, H, ds, V, n_rows, V, d_hidden_chunk, H,
-                                            token_of_row, row_factor);
+  {
+    const int tiles_m = (int)((H + BM - 1) / BM), tiles_n = (int)((n_rows + BN - 1) / BN);
+    const int splits = choose_splits((int64_t)tiles_m * tiles_n, (V + BK - 1) / BK, compute_units());
+    if (splits == 1) {
+      launch_gemm<true, false, uint16_t, false>(st, (const uint16_t*)weight, H, H, ds, V, n_rows, V, d_hidden_chunk, H,
+                                                token_of_row, row_factor);
+    } else {
+      float* part = (float*)(ws + w.off_dhp);
+      const int64_t plane = n_rows * H;
+      Operand a{(const uint16_t*)weight, H, (int)H}, b{ds, V, (int)n_rows};
+      hipLaunchKernelGGL((k_gemm_splitk<true, false>), dim3((unsigned)(tiles_m * tiles_n * splits)), dim3(kThreads), kLdsBytes,
+                         st, a, b, (int)V, tiles_m, tiles_n, splits, part, H, plane);
+      hipLaunchKernelGGL(k_splitk_rows, dim3((unsigned)n_rows), dim3(256), 0, st, part, splits, plane, (int)H, token_of_row,
+                         row_factor, d_hidden_chunk, H);
+    }
+  }
   if (!dw_f32)
     launch_gemm<true, true, uint16_t, false>(st, hid_rows, H, H, ds, V, V, n_rows, (uint16_t*)d_weight, H);
   else if (first)

@@ -838,8 +838,9 @@ def lm_head_logprobs_entropy(
     most 16384, forms the chunk's logits tiles again, writes their gradient as bf16 rows (of the tokens whose upstream
     gradient is not zero) into a workspace panel ``[chunk, V]`` and contracts that panel with the weight and with the
     hidden states on the same tile GEMM (fp32 accumulation, the weight gradient is returned in the dtype of
-    ``weight``).  The backward's workspace is the panel and its transposed copy (``4 * chunk * V`` bytes) plus a
-    transposed copy of the weight.
+    ``weight``).  The backward's workspace is that panel (``2 * chunk * V`` bytes), the hidden rows of the chunk's
+    tokens with a gradient and a few fp32 planes of ``[chunk, H]``; the arrays are multiplied as they lie, nothing is
+    transposed.
     The reference has no such op: it is the drop-in for its lm_head matmul followed by
     ``gather_logprobs_entropy`` (vocab_parallel.py:434-469).
 

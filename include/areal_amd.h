@@ -619,9 +619,12 @@ int aa_masked_moments(const float* const* values, int n_tensors,
  * With C = min(T, aa_lmhead_chunk_tokens()): 2 * C * V (the bf16 d(logits)
  * rows of one token chunk), 24 * (V / 256) * C (softmax partials per 128
  * vocabulary rows and token), 2 * C * H (the hidden rows of the tokens with a
- * gradient, closed up), plus 4 * H * V (an fp32 accumulator for a bf16
- * d_weight) when there is more than one chunk.  No transposed copy of anything
- * is made.  Returns -1 for sizes the path does not take. */
+ * gradient, closed up), 16 * C * H (four fp32 planes of d_hidden rows: the
+ * product that forms them has few tiles and is cut along the vocabulary into
+ * up to four parts when that fills the chip better), plus 4 * H * V (an fp32
+ * accumulator for a bf16 d_weight) when there is more than one chunk.  No
+ * transposed copy of anything is made.  Returns -1 for sizes the path does
+ * not take. */
 int64_t aa_lmhead_workspace_bytes(int64_t T, int64_t H, int64_t V);
 
 /* Bytes of workspace aa_lmhead_fwd alone needs: the softmax partials only,

@@ -179,6 +179,35 @@ def test_gradient_products_with_more_tiles_than_compute_units(device, backward):
     assert torch.equal(dh, dh2) and torch.equal(dw, dw2) and torch.equal(loss, loss2)
 
 
+@pytest.mark.parametrize("backward", ["carry", "recompute"])
+@pytest.mark.parametrize("T,H,V", [(300, 128, 16640), (700, 320, 20488)])
+def test_hidden_gradient_cut_along_the_vocabulary(device, backward, T, H, V):
+    """Few tiles of d(hidden) and a long vocabulary to contract (260 and 321 slices of 64): the product is cut into
+    parts along the vocabulary, every part sums into its own fp32 plane and the planes are added in a fixed order
+    (the last part is short and ragged).  Against the oracle row by row, bit-equal from call to call, masked tokens
+    with a zero row."""
+    hidden, weight, labels, prox, old, adv, mask = _inputs(T, T, H, V, seed=V, w_std=0.05)
+    args = [t.to(device) for t in (labels, prox, old, adv)]
+
+    def run():
+        h = hidden.to(device).requires_grad_(True)
+        w = weight.to(device).requires_grad_(True)
+        loss, stat = areal_amd.fused_lm_head_ppo_loss(h, w, *args, eps_clip=0.2, loss_mask=mask.to(device), backward=backward)
+        loss.backward()
+        return loss.detach(), h.grad, w.grad
+
+    o_loss, _, _, _, o_dh, o_dw = _oracle_step(hidden, weight, labels, prox, old, adv, mask, 1.0, 1.0, eps_clip=0.2)
+    loss, dh, dw = run()
+    assert float(loss) == pytest.approx(o_loss, rel=1e-3)
+    assert cosine(dh.cpu().float(), o_dh) > 0.9999 and cosine(dw.cpu().float(), o_dw) > 0.9999
+    assert_same_magnitude(dh, o_dh, what="d(hidden)")
+    err = (dh.cpu().float() - o_dh).abs().amax(dim=1)
+    assert float(err.max()) <= float(o_dh.abs().max()) * 2.0 ** -7
+    assert float(dh[~mask.to(device)].float().abs().max()) == 0.0
+    loss2, dh2, dw2 = run()
+    assert torch.equal(dh, dh2) and torch.equal(dw, dw2) and torch.equal(loss, loss2)
+
+
 def test_upstream_gradient_scales_both_gradients(device):
     hidden, weight, labels, prox, old, adv, mask = _inputs(260, 260, 64, 704, seed=3)
     args = [t.to(device) for t in (labels, prox, old, adv)]
