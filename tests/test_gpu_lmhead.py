@@ -69,7 +69,8 @@ def test_closed_form_and_bad_label(device):
 
 
 @pytest.mark.parametrize("T,H,V,temperature,with_entropy",
-                         [(300, 128, 1088, 1.0, False), (520, 192, 832, 0.8, True), (203, 200, 1096, 1.0, True)])
+                         [(300, 128, 1088, 1.0, False), (520, 192, 832, 0.8, True), (203, 200, 1096, 1.0, True),
+                          (300, 128, 16640, 1.0, True)])   # the last: d(hidden) cut into parts along the vocabulary
 def test_backward_matches_autograd_of_oracle(device, T, H, V, temperature, with_entropy):
     hidden, weight, labels = _case(T, H, V, seed=7 * T + V, w_std=0.3)
     g = torch.Generator().manual_seed(3)
