@@ -449,7 +449,7 @@ MODE_NAMES = {1: "carry", 0: "recompute"}
 # WRITE_SIZE (one run each) summed over the kernels of one step, each scaled by what the same counter reads for the
 # plain copy kernel of known size (profiles/lmhead_step_cfg2_hbm_traffic.md).  The counters sit behind the L2 of each
 # XCD: what the memory-side cache serves is in these figures too.  Other workloads: not measured.
-LMHEAD_MEASURED_HBM_BYTES = {("cfg2", "carry"): 83.2e9, ("cfg2", "recompute"): 110.4e9}
+LMHEAD_MEASURED_HBM_BYTES = {("cfg2", "carry"): 82.1e9, ("cfg2", "recompute"): 109.2e9}
 
 
 def lmhead_compulsory_bytes(T: int, kept: int, H: int, V: int, mode: str, chunk: int) -> dict:
