@@ -171,8 +171,7 @@ __device__ __forceinline__ Side make_side(const Operand& X, int x0, int wq, int 
 }
 
 // Main loop.  Leaves the result in `acc`; `lds` is kLdsBytes of dynamic shared memory.  K % 8 == 0.
-// AKM / BKM: the operand is K-major.  ABL (probing only, results are then wrong): bit 0 no global loads, bit 1 no
-// barrier, bit 2 no fragment reads.
+// AKM / BKM: the operand is K-major.
 //
 // Per slice (four 16-wide k steps, fragments double buffered in registers; every step issues its 16 MFMAs with the 8
 // fragment reads of the next step behind MFMAs 0-7 and 4 global loads behind MFMAs 8, 10, 12, 14 (a load blocks the
@@ -182,7 +181,7 @@ __device__ __forceinline__ Side make_side(const Operand& X, int x0, int wq, int 
 //   step 3 (reads the first fragments of slice k + 1)
 // Slices at or past K get an empty descriptor (no memory traffic, zeros in LDS) so that the count of loads per slice,
 // and with it the vmcnt arithmetic, is the same from the first slice to the last.
-template <bool AKM, bool BKM, int ABL = 0>
+template <bool AKM, bool BKM>
 __device__ __forceinline__ void mainloop(const Operand& A, const Operand& B, int K, int m0, int n0, Acc& acc, char* lds) {
   constexpr int MN = 16, NR = 8;
   const int tid = threadIdx.x;
@@ -214,7 +213,6 @@ __device__ __forceinline__ void mainloop(const Operand& A, const Operand& B, int
   auto open_a = [&](Cursor& c, int slice, int slot) { open_unit(c, sa_, AKM, slice, slot); };
   auto open_b = [&](Cursor& c, int slice, int slot) { open_unit(c, sb_, BKM, slice, slot); };
   auto g_load1 = [&](const Cursor& c, int jstep, int j) {
-    if (ABL & 1) return;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(c.rs, (lds_ptr_t)(uintptr_t)(c.dst + j * 4096), 16, c.voff + j * jstep, 0, 0, 0);
   };
 
@@ -226,15 +224,6 @@ __device__ __forceinline__ void mainloop(const Operand& A, const Operand& B, int
       for (int i = 0; i < 16; ++i) acc.v[mt][nt][i] = 0.f;
 
   bf16x8_t fa[2][4], fb[2][4];
-  if (ABL & 4) {
-#pragma unroll
-    for (int bq = 0; bq < 2; ++bq)
-#pragma unroll
-      for (int x = 0; x < 4; ++x) {
-        fa[bq][x] = __builtin_bit_cast(bf16x8_t, *(const u32x4_t*)(lds + (lane & 31) * 128 + x * 4096 + bq * 16));
-        fb[bq][x] = __builtin_bit_cast(bf16x8_t, *(const u32x4_t*)(lds + kUnitBytes + (lane & 31) * 128 + x * 4096 + bq * 16));
-      }
-  }
   // fragment of sub-tile x at k step kk from the unit in `slot`
   auto frag = [&](const Side& s, bool kmajor, int slot, int kk, int x) -> bf16x8_t {
     if (!kmajor) return __builtin_bit_cast(bf16x8_t, *(const u32x4_t*)(lds + slot * kUnitBytes + s.frag[kk] + x * 4096));
@@ -245,7 +234,6 @@ __device__ __forceinline__ void mainloop(const Operand& A, const Operand& B, int
   };
   // fragment r of a step: r < 4 is A sub-tile r, otherwise B sub-tile r - 4; slot_a / slot_b are the units' slots
   auto f_load1 = [&](int buf, int slot_a, int slot_b, int kk, int r) {
-    if (ABL & 4) return;
     if (r < 4)
       fa[buf][r] = frag(sa_, AKM, slot_a, kk, r);
     else
@@ -306,7 +294,7 @@ __device__ __forceinline__ void mainloop(const Operand& A, const Operand& B, int
     step(0, sa, sb, 3, cy, sa_.jstep, 4);
     // own reads of slice k done; own loads through unit 2 k + 3 landed (unit 2 k + 4 may be in flight)
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(8, 0));
-    if (!(ABL & 2)) __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_s_barrier();
     open_b(cx, k + 2, sa);  // unit 2 k + 5 = B(k + 2) takes the slot of A(k)
     __builtin_amdgcn_sched_barrier(0);
     step(1, sa1, sb1, 0, cx, sb_.jstep, 0);
