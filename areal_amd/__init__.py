@@ -29,6 +29,7 @@ from .functional import (
     gather_logprobs_entropy,
     gather_logprobs_entropy_stats,
     lm_head_logprobs_entropy,
+    lm_head_logprobs_entropy_stats,
     lm_head_chunk_tokens,
     lm_head_logprobs_entropy_static,
     ppo_actor_loss_fn,
@@ -82,6 +83,7 @@ __all__ = [
     "gather_packed_tree_logprobs_entropy",
     "kl_regularized_rewards",
     "lm_head_logprobs_entropy",
+    "lm_head_logprobs_entropy_stats",
     "lm_head_chunk_tokens",
     "lm_head_logprobs_entropy_static",
     "masked_moments",

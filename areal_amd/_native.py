@@ -82,7 +82,9 @@ SIGNATURES = {
     "aa_scale_rows_inplace": (_i, [_p, _i, _i64, _i64, _i64, _p, _p]),
     "aa_lmhead_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "aa_lmhead_fwd_workspace_bytes": (_i64, [_i64, _i64, _i64]),
-    "aa_lmhead_fwd": (_i, [_p, _p, _i64, _i64, _i64, _p, _f, _p, _p, _p, _p, _p, _i64, _p]),
+    "aa_lmhead_fwd_stats_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "aa_lmhead_prepare": (_i, []),
+    "aa_lmhead_fwd": (_i, [_p, _p, _i64, _i64, _i64, _p, _f, _p, _p, _p, _p, _p, _p, _p, _i64, _p]),
     "aa_lmhead_chunk_tokens": (_i64, []),
     "aa_lmhead_fwd_static": (_i, [_p, _p, _i64, _i64, _i64, _p, _f, _p, _p, _p, _p, _p]),
     "aa_lmhead_fwd_static_scratch_bytes": (_i64, []),
@@ -91,7 +93,7 @@ SIGNATURES = {
     "aa_lmhead_ppo_fused": (
         _i,
         [_p, _p, _i64, _i64, _i64, _p, _f, _i64, _p, _p, _p, _p, C.POINTER(PpoParams), _p, _p, _p, _i,
-         _p, _p, _p, _p, _p, _p, _p, _i, _p, _i64, _p],
+         _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i64, _p],
     ),
     "aa_sapo_loss": (_i, [_p, _p, _p, _p, _i64, _p, _i64, _i, _f, _f, _p, _p, _p, _p, _p, _p]),
     "aa_critic_loss": (_i, [_p, _p, _p, _p, _i64, _f, _i, _p, _p, _p, _p, _p]),

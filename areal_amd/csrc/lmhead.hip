@@ -48,15 +48,17 @@ struct TileArgs {
   float* pk;
   float* ps;
   float* pu;
+  float* pn;              // nullable: smallest raw logit of the block (for vocab_min_logits), same layout
   float* xy;              // [tokens of the chunk] raw label logit (k_label_logit, before the tiles run)
   const int64_t* labels;  // labels of the chunk
   int64_t pitch_t;
   float c;                // log2(e) / temperature
-  // panel [rows, panel_ld] bf16: row out_rows[token] (or the token itself when out_rows is null); negative: no row
+  // panel [rows, panel_ld] bf16, panel_ld = V rounded up to 8 (the entries past V are written as zeros): row
+  // out_rows[token] (or the token itself when out_rows is null); negative: no row
   uint16_t* panel;
   int64_t panel_ld;
   const int32_t* out_rows;
-  // recompute: per token of the chunk; column n of the tile is token col_tokens[n] (or n when null)
+  // recompute: per token of the chunk; column n of the tile is token col_tokens[n] (or n when null; negative: none)
   const int32_t* col_tokens;
   const float* row_lse;    // natural-log logsumexp of the row
   const float* row_ez;     // sum_j p_j z_j (used with g_entropy)
@@ -75,6 +77,9 @@ struct TileArgs {
 // would have to be e^-80 unlikely) is redone by the recompute tiles, decided on the device.
 constexpr float kCarryMaxShift = 126.f;
 constexpr float kCarryMinLogp = -80.f;
+// d_weight takes the row's factor f = -(g / T) p_label inside the hidden rows, rounded to bf16: |f| times a hidden
+// entry has to stay a normal number (above 2^-126) for entries down to 2^-26 of magnitude, or the chunk is redone
+constexpr float kCarryMinFactor = 0x1p-100f;
 
 // Statistics (and, with CARRY, the staged probability ratios) of one wave's 128 x 128 block, accumulators in the
 // 16 x 16 tile layout: a lane holds, for each of 8 tokens (nt), 8 runs (mt) of 4 consecutive vocabulary rows, and the
@@ -102,6 +107,23 @@ __device__ __forceinline__ void block_stats(const Acc16& acc, const TileArgs& a,
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));  // four lanes hold the same token
     mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    if (a.pn) {  // uniform: the caller wants the smallest logit of every token as well
+      float mn = FLT_MAX;
+      if constexpr (!RAGGED) {
+#pragma unroll
+        for (int mt = 0; mt < kAcc16Tiles; ++mt)
+#pragma unroll
+          for (int i = 0; i < 4; i += 2) mn = fminf(fminf(mn, acc.v[mt][nt][i]), acc.v[mt][nt][i + 1]);
+      } else {
+#pragma unroll
+        for (int mt = 0; mt < kAcc16Tiles; ++mt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) mn = (mbase + acc16_row(mt, i, lane) < V) ? fminf(mn, acc.v[mt][nt][i]) : mn;
+      }
+      mn = fminf(mn, __shfl_xor(mn, 16, kWave));
+      mn = fminf(mn, __shfl_xor(mn, 32, kWave));
+      if (lane < 16 && n < N) a.pn[(int64_t)(tm * 2 + wm) * a.pitch_t + n] = mn;  // FLT_MAX: no valid row in this block
+    }
     const float k = fmaxf(mx * a.c, kNegBig);   // kNegBig: no valid row in this block
     float to_ref = 1.f;                         // 2^(k - kref): block-relative -> label-relative exponentials
     if constexpr (CARRY) {
@@ -170,14 +192,15 @@ __global__ __launch_bounds__(kThreads) void k_lmhead_tiles(Operand W, Operand Hd
     else
       block_stats<MODE == kModeStatsCarry, false>(acc, a, tm, wm, wn, n0, N, V, mbase, lane, Z);
   } else {
+    const bool ragged_rows = m0 + BM > V;
 #pragma unroll
     for (int nt = 0; nt < kAcc16Tiles; ++nt) {
       const int nloc = wn * 128 + acc16_col(nt, lane);
       const int n = n0 + nloc;
       float A = 0.f, B = 0.f, lab_add = 0.f, lse2 = 0.f;
       int64_t y = -1;
-      if (n < N) {
-        const int t = a.col_tokens ? a.col_tokens[n] : n;
+      const int t = n < N ? (a.col_tokens ? a.col_tokens[n] : n) : -1;
+      if (t >= 0) {
         const float gl = a.g_logp[t];
         const float gh = a.g_entropy ? a.g_entropy[t] : 0.f;
         const float ez = a.g_entropy ? a.row_ez[t] : 0.f;
@@ -197,6 +220,10 @@ __global__ __launch_bounds__(kThreads) void k_lmhead_tiles(Operand W, Operand Hd
           o[q] = fast_exp2(fmaf(x, a.c, -lse2)) * fmaf(B, x, A);  // columns past the tokens: never written out
         }
         const int r0 = acc16_row(mt, 0, lane);  // row of o[0] inside the wave's block
+        if (ragged_rows) {  // uniform; rows at or past V: the last piece of a panel row may reach them, they hold zeros
+#pragma unroll
+          for (int q = 0; q < 4; ++q) o[q] = (mbase + r0 + q < V) ? o[q] : 0.f;
+        }
         if (rel >= r0 && rel < r0 + 4) {
 #pragma unroll
           for (int q = 0; q < 4; ++q)
@@ -218,7 +245,8 @@ __global__ __launch_bounds__(kThreads) void k_lmhead_tiles(Operand W, Operand Hd
       rows_lds[tid] = n < N ? (a.out_rows ? a.out_rows[n] : n) : -1;
     }
     __syncthreads();
-    // panel rows: 16-byte pieces along the vocabulary (V % 8 == 0: a piece never straddles the end)
+    // panel rows: 16-byte pieces along the vocabulary (the pitch is a multiple of 8: the piece that straddles V ends in
+    // the row's own padding, whose entries were formed as zeros)
     const int mc = (tid & 31) * 8, m = m0 + mc;
     if (m < V) {
 #pragma unroll 8
@@ -264,8 +292,10 @@ __global__ __launch_bounds__(256) void k_label_logit(const uint16_t* __restrict_
 // deterministic.
 struct Merged {
   float k, s, u;
+  float n;  // smallest raw logit (FLT_MAX when the minimum plane was not asked for)
 };
 constexpr int kMergeWaves = 16;
+constexpr int kMergeSmemFloats = 4 * kMergeWaves * 64;
 
 __device__ __forceinline__ void merge_into(Merged& m, float bk, float bs, float bu) {
   const float nk = fmaxf(m.k, bk);
@@ -278,36 +308,44 @@ __device__ __forceinline__ void merge_into(Merged& m, float bk, float bs, float 
 
 // t: the token of this lane (may be past the end: then the result is meaningless and the caller drops it)
 __device__ __forceinline__ Merged merge_blocks(const float* __restrict__ pk, const float* __restrict__ ps,
-                                               const float* __restrict__ pu, int blocks, int64_t pitch_t, int64_t t,
-                                               bool live, float* smem /* [3][16][64] */) {
+                                               const float* __restrict__ pu, const float* __restrict__ pn, int blocks,
+                                               int64_t pitch_t, int64_t t, bool live, float* smem /* [4][16][64] */) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  Merged m{kNegBig, 0.f, 0.f};
+  Merged m{kNegBig, 0.f, 0.f, FLT_MAX};
   if (live)
     for (int b = wave; b < blocks; b += kMergeWaves) {
       const int64_t at = (int64_t)b * pitch_t + t;
       merge_into(m, pk[at], ps[at], pu[at]);
+      if (pn) m.n = fminf(m.n, pn[at]);
     }
   smem[(0 * kMergeWaves + wave) * 64 + lane] = m.k;
   smem[(1 * kMergeWaves + wave) * 64 + lane] = m.s;
   smem[(2 * kMergeWaves + wave) * 64 + lane] = m.u;
+  smem[(3 * kMergeWaves + wave) * 64 + lane] = m.n;
   __syncthreads();
-  Merged r{kNegBig, 0.f, 0.f};
+  Merged r{kNegBig, 0.f, 0.f, FLT_MAX};
 #pragma unroll
-  for (int w = 0; w < kMergeWaves; ++w)
+  for (int w = 0; w < kMergeWaves; ++w) {
     merge_into(r, smem[(0 * kMergeWaves + w) * 64 + lane], smem[(1 * kMergeWaves + w) * 64 + lane],
                smem[(2 * kMergeWaves + w) * 64 + lane]);
+    r.n = fminf(r.n, smem[(3 * kMergeWaves + w) * 64 + lane]);
+  }
   return r;
 }
 
-// forward of the stand-alone op: 64 tokens per workgroup
+// forward of the stand-alone op: 64 tokens per workgroup.  vmax / vmin (nullable, together): largest and smallest raw
+// logit of the row (what FSDPEngine._get_vocab_min_max_logits takes from materialised logits,
+// areal/engine/fsdp_engine.py:1893-1906); the largest is recovered from the merged exponent k = c * max, i.e. to one
+// rounding, the smallest comes from its own plane.
 __global__ __launch_bounds__(1024) void k_combine(const float* __restrict__ pk, const float* __restrict__ ps,
-                                                  const float* __restrict__ pu, const float* __restrict__ xy, int blocks,
-                                                  int64_t pitch_t, int n_tok, float c, float* __restrict__ logp,
-                                                  float* __restrict__ entropy, float* __restrict__ row_lse,
-                                                  float* __restrict__ row_ez) {
-  __shared__ float smem[3 * kMergeWaves * 64];
+                                                  const float* __restrict__ pu, const float* __restrict__ pn,
+                                                  const float* __restrict__ xy, int blocks, int64_t pitch_t, int n_tok,
+                                                  float c, float* __restrict__ logp, float* __restrict__ entropy,
+                                                  float* __restrict__ row_lse, float* __restrict__ row_ez,
+                                                  float* __restrict__ vmax, float* __restrict__ vmin) {
+  __shared__ float smem[kMergeSmemFloats];
   const int t = blockIdx.x * 64 + (threadIdx.x & 63);
-  const Merged m = merge_blocks(pk, ps, pu, blocks, pitch_t, t, t < n_tok, smem);
+  const Merged m = merge_blocks(pk, ps, pu, pn, blocks, pitch_t, t, t < n_tok, smem);
   if (t >= n_tok || threadIdx.x >= 64) return;
   const float log2s = fast_log2(m.s);
   const float mean_t = m.u / m.s;
@@ -315,6 +353,8 @@ __global__ __launch_bounds__(1024) void k_combine(const float* __restrict__ pk, 
   if (entropy) entropy[t] = (log2s - mean_t) * kLn2;
   if (row_lse) row_lse[t] = (m.k + log2s) * kLn2;
   if (row_ez) row_ez[t] = (m.k + mean_t) * kLn2;
+  if (vmax) vmax[t] = m.k / c;
+  if (vmin) vmin[t] = m.n;
 }
 
 // What carry mode needs per panel row, written by k_token_loss
@@ -337,6 +377,8 @@ struct TokenLossArgs {
   float* stat_loss;
   float* ratio;
   uint8_t* flags;
+  float* vmax;  // nullable (together with vmin): largest / smallest raw logit of the row
+  float* vmin;
   aa_ppo_params P;
   int64_t act;  // tokens of the chunk that are inside T_active
 };
@@ -345,19 +387,22 @@ struct TokenLossArgs {
 // kernel writes them, areal/utils/functional/functional.py:505-558) and g = d(scaled loss) / d(logp); then what the
 // backward needs: g and the row's logsumexp per token (recompute), or the row coefficients per panel row (carry).
 __global__ __launch_bounds__(1024) void k_token_loss(const float* __restrict__ pk, const float* __restrict__ ps,
-                                                     const float* __restrict__ pu, const float* __restrict__ xy, int blocks,
+                                                     const float* __restrict__ pu, const float* __restrict__ pn,
+                                                     const float* __restrict__ xy, int blocks,
                                                      int64_t pitch_t, int n_tok, int V, float c, float inv_t,
                                                      const int64_t* __restrict__ labels, TokenLossArgs a,
                                                      const int32_t* __restrict__ out_rows, float* __restrict__ g_tok,
                                                      float* __restrict__ lse_tok, CarryOut carry) {
-  __shared__ float smem[3 * kMergeWaves * 64];
+  __shared__ float smem[kMergeSmemFloats];
   const int t = blockIdx.x * 64 + (threadIdx.x & 63);
-  const Merged m = merge_blocks(pk, ps, pu, blocks, pitch_t, t, t < n_tok, smem);
+  const Merged m = merge_blocks(pk, ps, pu, pn, blocks, pitch_t, t, t < n_tok, smem);
   if (t >= n_tok || threadIdx.x >= 64) return;
   const float log2s = fast_log2(m.s);
   const float lp = (fmaf(xy[t], c, -m.k) - log2s) * kLn2;
   a.logp[t] = lp;
   if (a.entropy) a.entropy[t] = (log2s - m.u / m.s) * kLn2;
+  if (a.vmax) a.vmax[t] = m.k / c;
+  if (a.vmin) a.vmin[t] = m.n;
   float g = 0.f;
   if (t < a.act) {
     int n = *a.n_valid;
@@ -392,13 +437,18 @@ __global__ __launch_bounds__(1024) void k_token_loss(const float* __restrict__ p
       // every v but the label, whose entry is replaced by 1 - 1 / p_label: f (1 - 1 / p_label) = (g / T) (1 - p_label)
       const float kref = xy[t] * c;                                   // as the tiles formed it
       const float p_label = fast_exp2(kref - (m.k + log2s));
-      carry.row_factor[r] = g == 0.f ? 0.f : -(g * inv_t) * p_label;  // g == 0: whatever the row holds counts for nothing
+      const float f = g == 0.f ? 0.f : -(g * inv_t) * p_label;  // g == 0: whatever the row holds counts for nothing
+      carry.row_factor[r] = f;
       const int64_t y = labels[t];
-      if (y >= 0 && y < V) {
+      // a row without gradient keeps its label entry (1): 1 - 1 / p_label is not finite for a label more than 88 nats
+      // unlikely, and d_weight multiplies every entry of the row, by a zero there
+      if (g != 0.f && y >= 0 && y < V) {
         const float patched = -expm1f(-lp);
         carry.panel[(int64_t)r * carry.panel_ld + y] = (uint16_t)(Elem<AA_BF16>::pack(patched, 0.f) & 0xffffu);
       }
-      if (g != 0.f && lp < kCarryMinLogp) *carry.redo_flag = 1;
+      // redo by recompute when the stored form cannot carry the row: the ratios would overflow (label too unlikely), or
+      // the factor is so small that factor x hidden, which d_weight takes rounded to bf16, leaves the normal range
+      if (g != 0.f && (lp < kCarryMinLogp || fabsf(f) < kCarryMinFactor)) *carry.redo_flag = 1;
     }
   }
 }
@@ -436,15 +486,17 @@ __global__ __launch_bounds__(kThreads) void k_gemm_store(Operand A, Operand B, i
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) {
       const int nloc = wn * 128 + acc_col(nt, lane);
-      // optional factor per row of C (a lane owns one n): applied to the fp32 sums, before the one rounding to bf16
+      // optional factor per row of C (a lane owns one n): applied to the fp32 sums, before the one rounding to bf16.  A
+      // factor of zero gives a zero row whatever the sums hold (a row without gradient may have summed to infinity)
       const float f = (n_scale && n0 + nloc < N) ? n_scale[n0 + nloc] : 1.f;
+      const bool dead = f == 0.f;
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4) {
           uint2 pk;
-          pk.x = Elem<AA_BF16>::pack(acc.v[mt][nt][g4 * 4] * f, acc.v[mt][nt][g4 * 4 + 1] * f);
-          pk.y = Elem<AA_BF16>::pack(acc.v[mt][nt][g4 * 4 + 2] * f, acc.v[mt][nt][g4 * 4 + 3] * f);
+          pk.x = dead ? 0u : Elem<AA_BF16>::pack(acc.v[mt][nt][g4 * 4] * f, acc.v[mt][nt][g4 * 4 + 1] * f);
+          pk.y = dead ? 0u : Elem<AA_BF16>::pack(acc.v[mt][nt][g4 * 4 + 2] * f, acc.v[mt][nt][g4 * 4 + 3] * f);
           *(uint2*)(Z + nloc * PZ + wm * 128 + mt * 32 + 8 * g4 + 4 * (lane >> 5)) = pk;
         }
     }
@@ -454,7 +506,7 @@ __global__ __launch_bounds__(kThreads) void k_gemm_store(Operand A, Operand B, i
       rows_lds[tid] = n < N ? (c_rows ? c_rows[n] : n) : -1;
     }
     __syncthreads();
-    const int mc = (tid & 31) * 8, m = m0 + mc;  // M % 8 == 0: a piece never straddles the end
+    const int mc = (tid & 31) * 8, m = m0 + mc;  // M % 8 == 0 (M is a hidden size): a piece never straddles the end
     if (m < M) {
 #pragma unroll 8
       for (int i = 0; i < 32; ++i) {
@@ -554,7 +606,7 @@ __global__ __launch_bounds__(256) void k_splitk_rows(const float* __restrict__ p
       }
     }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) a[i] *= f;
+    for (int i = 0; i < 8; ++i) a[i] = f == 0.f ? 0.f : a[i] * f;  // a zero factor gives a zero row whatever the sums hold
     store8<AA_BF16>(out + dst * ldo, m, a);
   }
 }
@@ -563,9 +615,14 @@ __global__ __launch_bounds__(256) void k_splitk_rows(const float* __restrict__ p
 // A token whose loss mask is zero has d(loss)/d(logits) == 0: its row adds nothing to d_weight and its d_hidden row
 // is zero.  k_compact_map numbers the tokens of a chunk that do have a mask (in order): out_rows[t] = position of
 // token t among them, or -1; act_rows[position] = t.  `limit` is the count the host sized the GEMMs with; tokens
-// beyond it are dropped.  One workgroup; mask has `act` entries (tokens at and after `act` have no mask).
+// beyond it are dropped.  A host count larger than what the mask holds leaves positions without a token: they get
+// act_rows = -1 (the gathers then produce zero rows and the scatters skip them), a row factor of zero when factors are
+// in use, and the workgroup clears their panel rows, which no tile writes, so that nothing stale (possibly not even
+// finite) enters the d_weight product.  One workgroup; mask has `act` entries (tokens at and after `act` have none).
 __global__ __launch_bounds__(1024) void k_compact_map(const uint8_t* __restrict__ mask, int act, int n_tok, int limit,
-                                                      int32_t* __restrict__ out_rows, int32_t* __restrict__ act_rows) {
+                                                      int32_t* __restrict__ out_rows, int32_t* __restrict__ act_rows,
+                                                      float* __restrict__ row_factor, u32x4_t* __restrict__ panel,
+                                                      int64_t panel_ld) {
   __shared__ int wave_sum[16];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int per = (n_tok + 1023) / 1024;
@@ -589,14 +646,20 @@ __global__ __launch_bounds__(1024) void k_compact_map(const uint8_t* __restrict_
     if (on) act_rows[pos] = t;
     pos += (t < act && mask[t] != 0) ? 1 : 0;
   }
-  // a host count larger than what the mask holds leaves positions without a token: point them at row 0, so that the
-  // gathers that follow stay inside the chunk (their contribution is then meaningless, as the caller's count was)
   int total = 0;
   for (int w = 0; w < 16; ++w) total += wave_sum[w];
-  for (int p = total + tid; p < limit; p += 1024) act_rows[p] = 0;
+  if (total >= limit) return;  // the usual case: every position has its token
+  for (int p = total + tid; p < limit; p += 1024) {
+    act_rows[p] = -1;
+    if (row_factor) row_factor[p] = 0.f;
+  }
+  const u32x4_t zero = {0u, 0u, 0u, 0u};
+  const int64_t vec = panel_ld / 8;
+  for (int64_t i = (int64_t)total * vec + tid; i < (int64_t)limit * vec; i += 1024) panel[i] = zero;
 }
 
-// dst[r, :] = scale[r] * src[rows[r], :] (H % 8 == 0); rows == nullptr: row r itself; scale == nullptr: 1;
+// dst[r, :] = scale[r] * src[rows[r], :] (H % 8 == 0); rows == nullptr: row r itself (a negative entry: a zero row);
+// scale == nullptr: 1;
 // run_if, when given: nothing happens unless *run_if != 0
 __global__ __launch_bounds__(256) void k_gather_rows(const u32x4_t* __restrict__ src, const int32_t* __restrict__ rows,
                                                      u32x4_t* __restrict__ dst, int h_vec,
@@ -604,6 +667,11 @@ __global__ __launch_bounds__(256) void k_gather_rows(const u32x4_t* __restrict__
   if (run_if && *run_if == 0) return;
   const int64_t r = blockIdx.x;
   const int64_t t = rows ? rows[r] : r;
+  if (t < 0) {  // a position without a token
+    const u32x4_t zero = {0u, 0u, 0u, 0u};
+    for (int j = threadIdx.x; j < h_vec; j += 256) dst[r * h_vec + j] = zero;
+    return;
+  }
   if (!scale) {
     for (int j = threadIdx.x; j < h_vec; j += 256) dst[r * h_vec + j] = src[t * h_vec + j];
     return;
@@ -652,8 +720,11 @@ constexpr int kMaxSplits = 4;  // of the d_hidden product along K
 struct Workspace {
   int64_t chunk, blocks;                // tokens per chunk, 128-row vocabulary blocks
   int64_t off_pk, off_ps, off_pu;       // block partials [blocks][chunk]
+  int64_t panel_ld;                     // pitch of the panel: V rounded up to 8 elements
   int64_t off_xy, off_g, off_lse;       // per token of the chunk: label logit, g, logsumexp
   int64_t fwd_bytes;                    // what the forward alone needs
+  int64_t off_pn;                       // smallest logit per block [blocks][chunk] (only when the extrema are asked for)
+  int64_t fwd_stats_bytes;              // what the forward needs when it also returns the extrema of the logits
   int64_t off_rowf, off_flag;           // carry mode: factor per panel row; the chunk's redo flag
   int64_t off_rows;                     // out_rows, act_rows (2 x chunk int32)
   int64_t off_panel;                    // d(logits) rows [chunk, V]
@@ -676,10 +747,13 @@ static Workspace plan(int64_t T, int64_t H, int64_t V) {
   w.off_g = off;   off += up(w.chunk * 4);
   w.off_lse = off; off += up(w.chunk * 4);
   w.fwd_bytes = off;
+  w.off_pn = off;  off += up(w.blocks * w.chunk * 4);
+  w.fwd_stats_bytes = off;
   w.off_rowf = off;    off += up(w.chunk * 4);  // factor per panel row (carry mode)
   w.off_flag = off;    off += 256;              // the chunk's "redo by recompute" flag
   w.off_rows = off;    off += up(2 * w.chunk * 4);
-  w.off_panel = off;   off += up(w.chunk * V * 2);
+  w.panel_ld = round_up(V, 8);
+  w.off_panel = off;   off += up(w.chunk * w.panel_ld * 2);
   w.off_hc = off;      off += up(w.chunk * H * 2);
   w.off_dw = off;      off += T > w.chunk ? up(V * H * 4) : 0;
   w.off_dhp = off;     off += up(kMaxSplits * w.chunk * H * 4);
@@ -689,7 +763,7 @@ static Workspace plan(int64_t T, int64_t H, int64_t V) {
 
 static bool shapes_ok(int64_t T, int64_t H, int64_t V) {
   // 256 rows of any operand must stay below 2^30 elements (32-bit byte offsets inside a tile)
-  return T > 0 && H > 0 && V > 0 && (H % 8) == 0 && (V % 8) == 0 && T < (1 << 30) && V < (1 << 22) && H < (1 << 22);
+  return T > 0 && H > 0 && V > 0 && (H % 8) == 0 && T < (1 << 30) && V < (1 << 22) && H < (1 << 22);
 }
 
 // The tile kernels use all 160 KiB of LDS: allow it once per kernel and device.
@@ -785,16 +859,17 @@ static void panel_gradients(hipStream_t st, const Workspace& w, char* ws, const 
                        (u32x4_t*)hc, (int)(H / 8), row_factor, (const int32_t*)nullptr);
     hid_rows = hc;
   }
+  const int64_t ldp = w.panel_ld;
   {
     const int tiles_m = (int)((H + BM - 1) / BM), tiles_n = (int)((n_rows + BN - 1) / BN);
     const int splits = choose_splits((int64_t)tiles_m * tiles_n, (V + BK - 1) / BK, compute_units());
     if (splits == 1) {
-      launch_gemm<true, false, uint16_t, false>(st, (const uint16_t*)weight, H, H, ds, V, n_rows, V, d_hidden_chunk, H,
+      launch_gemm<true, false, uint16_t, false>(st, (const uint16_t*)weight, H, H, ds, ldp, n_rows, V, d_hidden_chunk, H,
                                                 token_of_row, row_factor);
     } else {
       float* part = (float*)(ws + w.off_dhp);
       const int64_t plane = n_rows * H;
-      Operand a{(const uint16_t*)weight, H, (int)H}, b{ds, V, (int)n_rows};
+      Operand a{(const uint16_t*)weight, H, (int)H}, b{ds, ldp, (int)n_rows};
       hipLaunchKernelGGL((k_gemm_splitk<true, false>), dim3((unsigned)(tiles_m * tiles_n * splits)), dim3(kThreads), kLdsBytes,
                          st, a, b, (int)V, tiles_m, tiles_n, splits, part, H, plane);
       hipLaunchKernelGGL(k_splitk_rows, dim3((unsigned)n_rows), dim3(256), 0, st, part, splits, plane, (int)H, token_of_row,
@@ -802,11 +877,11 @@ static void panel_gradients(hipStream_t st, const Workspace& w, char* ws, const 
     }
   }
   if (!dw_f32)
-    launch_gemm<true, true, uint16_t, false>(st, hid_rows, H, H, ds, V, V, n_rows, (uint16_t*)d_weight, H);
+    launch_gemm<true, true, uint16_t, false>(st, hid_rows, H, H, ds, ldp, V, n_rows, (uint16_t*)d_weight, H);
   else if (first)
-    launch_gemm<true, true, float, false>(st, hid_rows, H, H, ds, V, V, n_rows, (float*)d_weight, H);
+    launch_gemm<true, true, float, false>(st, hid_rows, H, H, ds, ldp, V, n_rows, (float*)d_weight, H);
   else
-    launch_gemm<true, true, float, true>(st, hid_rows, H, H, ds, V, V, n_rows, (float*)d_weight, H);
+    launch_gemm<true, true, float, true>(st, hid_rows, H, H, ds, ldp, V, n_rows, (float*)d_weight, H);
 }
 
 // Recompute: d(logits) of the panel rows from the logits tiles formed again.  With a row map only the hidden rows that
@@ -816,7 +891,7 @@ static void recompute_panel(hipStream_t st, const Workspace& w, char* ws, const 
                             int64_t n_tok, const int32_t* token_of_row, int64_t rows, int64_t H, int64_t V, TileArgs a,
                             const int32_t* run_if = nullptr) {
   a.panel = (uint16_t*)(ws + w.off_panel);
-  a.panel_ld = V;
+  a.panel_ld = w.panel_ld;
   a.out_rows = nullptr;
   a.run_if = run_if;
   if (!token_of_row) {
@@ -852,11 +927,12 @@ static void finish_weight_grad(hipStream_t st, const WeightGrad& g, void* d_weig
                      (u32x4_t*)d_weight, n8);
 }
 
-static TileArgs stats_args(const Workspace& w, char* ws, const int64_t* labels, float inv_t) {
+static TileArgs stats_args(const Workspace& w, char* ws, const int64_t* labels, float inv_t, bool want_min) {
   TileArgs a{};
   a.pk = (float*)(ws + w.off_pk);
   a.ps = (float*)(ws + w.off_ps);
   a.pu = (float*)(ws + w.off_pu);
+  a.pn = want_min ? (float*)(ws + w.off_pn) : nullptr;
   a.xy = (float*)(ws + w.off_xy);
   a.labels = labels;
   a.pitch_t = w.chunk;
@@ -881,30 +957,39 @@ extern "C" int64_t aa_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V
   return plan(T, H, V).fwd_bytes;
 }
 
+extern "C" int64_t aa_lmhead_fwd_stats_workspace_bytes(int64_t T, int64_t H, int64_t V) {
+  if (!shapes_ok(T, H, V)) return -1;
+  return plan(T, H, V).fwd_stats_bytes;
+}
+
 extern "C" int64_t aa_lmhead_chunk_tokens(void) { return kChunkTokens; }
+
+extern "C" int aa_lmhead_prepare(void) { return prepare_kernels() ? AA_OK : AA_ERR_LAUNCH; }
 
 extern "C" int aa_lmhead_fwd(const void* hidden, const void* weight, int64_t T, int64_t H, int64_t V,
                              const int64_t* labels, float inv_temperature, float* logp, float* entropy,
-                             float* row_lse, float* row_ez, void* workspace, int64_t workspace_bytes, void* stream) {
+                             float* row_lse, float* row_ez, float* vocab_max, float* vocab_min, void* workspace,
+                             int64_t workspace_bytes, void* stream) {
   if (!hidden || !weight || !labels || !logp || !workspace || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
+  if ((vocab_max != nullptr) != (vocab_min != nullptr)) return AA_ERR_INVALID_ARGUMENT;
   if (!shapes_ok(T, H, V)) return AA_ERR_UNSUPPORTED;
   if ((((uintptr_t)hidden | (uintptr_t)weight | (uintptr_t)workspace) & 15) != 0) return AA_ERR_INVALID_ARGUMENT;
   const Workspace w = plan(T, H, V);
-  if (workspace_bytes < w.fwd_bytes) return AA_ERR_INVALID_ARGUMENT;
+  if (workspace_bytes < (vocab_min ? w.fwd_stats_bytes : w.fwd_bytes)) return AA_ERR_INVALID_ARGUMENT;
   if (!prepare_kernels()) return AA_ERR_LAUNCH;
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
   auto at = [](float* p, int64_t t0) { return p ? p + t0 : nullptr; };
   for (int64_t t0 = 0; t0 < T; t0 += w.chunk) {
     const int64_t n_tok = (T - t0) < w.chunk ? (T - t0) : w.chunk;
-    const TileArgs a = stats_args(w, ws, labels + t0, inv_temperature);
+    const TileArgs a = stats_args(w, ws, labels + t0, inv_temperature, vocab_min != nullptr);
     const uint16_t* hid = (const uint16_t*)hidden + t0 * H;
     hipLaunchKernelGGL(k_label_logit, dim3((unsigned)((n_tok + 3) / 4)), dim3(256), 0, st, hid, (const uint16_t*)weight,
                        labels + t0, (int)n_tok, (int)H, (int)V, a.xy, (int32_t*)nullptr);
     launch_tiles<kModeStats>(st, weight, hid, n_tok, H, V, a);
-    hipLaunchKernelGGL(k_combine, dim3((unsigned)((n_tok + 63) / 64)), dim3(1024), 0, st, a.pk, a.ps, a.pu, a.xy,
+    hipLaunchKernelGGL(k_combine, dim3((unsigned)((n_tok + 63) / 64)), dim3(1024), 0, st, a.pk, a.ps, a.pu, a.pn, a.xy,
                        (int)w.blocks, a.pitch_t, (int)n_tok, a.c, logp + t0, at(entropy, t0), at(row_lse, t0),
-                       at(row_ez, t0));
+                       at(row_ez, t0), at(vocab_max, t0), at(vocab_min, t0));
   }
   return launch_status();
 }
@@ -976,8 +1061,9 @@ extern "C" int aa_lmhead_fwd_static(const void* hidden, const void* weight, int6
     hipLaunchKernelGGL(k_label_logit, dim3((unsigned)((n_tok + 3) / 4)), dim3(256), 0, st, hid, (const uint16_t*)weight,
                        labels + t0, (int)n_tok, (int)H, (int)V, a.xy, (int32_t*)nullptr);
     launch_tiles<kModeStats>(st, weight, hid, n_tok, H, V, a);
-    hipLaunchKernelGGL(k_combine, dim3((unsigned)((n_tok + 63) / 64)), dim3(1024), 0, st, a.pk, a.ps, a.pu, a.xy, (int)blocks,
-                       a.pitch_t, (int)n_tok, a.c, logp + t0, at(entropy, t0), at(row_lse, t0), at(row_ez, t0));
+    hipLaunchKernelGGL(k_combine, dim3((unsigned)((n_tok + 63) / 64)), dim3(1024), 0, st, a.pk, a.ps, a.pu,
+                       (const float*)nullptr, a.xy, (int)blocks, a.pitch_t, (int)n_tok, a.c, logp + t0, at(entropy, t0),
+                       at(row_lse, t0), at(row_ez, t0), (float*)nullptr, (float*)nullptr);
   }
   return launch_status();
 }
@@ -1030,7 +1116,7 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
       continue;
     }
     hipLaunchKernelGGL(k_compact_map, dim3(1), dim3(1024), 0, st, row_has_gradient + t0, (int)n_tok, (int)n_tok, (int)kept,
-                       out_rows, act_rows);
+                       out_rows, act_rows, (float*)nullptr, (u32x4_t*)(ws + w.off_panel), w.panel_ld);
     recompute_panel(st, w, ws, weight, hid, n_tok, act_rows, kept, H, V, a);
     launch_zero(st, dh, n_tok * H * 2);  // the rows of the other tokens
     panel_gradients(st, w, ws, weight, hid, act_rows, nullptr, kept, H, V, dh, dw.acc, dw.acc_f32, first);
@@ -1047,9 +1133,10 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
                                    const float* behave_w, const aa_ppo_params* params, const int32_t* n_valid,
                                    const float* grad_scale, const int64_t* kept_per_chunk, int backward_mode,
                                    float* logp, float* entropy, float* stat_loss, float* ratio, uint8_t* flags,
-                                   void* d_hidden, void* d_weight, int d_weight_dtype, void* workspace,
-                                   int64_t workspace_bytes, void* stream) {
+                                   float* vocab_max, float* vocab_min, void* d_hidden, void* d_weight,
+                                   int d_weight_dtype, void* workspace, int64_t workspace_bytes, void* stream) {
   if (!hidden || !weight || !labels || !d_hidden || !d_weight || !workspace) return AA_ERR_INVALID_ARGUMENT;
+  if ((vocab_max != nullptr) != (vocab_min != nullptr)) return AA_ERR_INVALID_ARGUMENT;
   if (!params || !n_valid || !logp) return AA_ERR_INVALID_ARGUMENT;
   if (T_active < 0 || T_active > T || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
   if (backward_mode != AA_LMHEAD_RECOMPUTE && backward_mode != AA_LMHEAD_CARRY) return AA_ERR_INVALID_ARGUMENT;
@@ -1092,14 +1179,14 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
       rows = kept_per_chunk[chunk_index];
       rows = rows < 0 ? 0 : (rows > act ? act : rows);
       hipLaunchKernelGGL(k_compact_map, dim3(1), dim3(1024), 0, st, at(mask_eff), (int)act, (int)n_tok, (int)rows, out_rows,
-                         act_rows);
+                         act_rows, carry ? row_factor : (float*)nullptr, (u32x4_t*)panel, w.panel_ld);
       row_of_token = out_rows;
       token_of_row = act_rows;
     }
     // forward tiles: block partials (and, in carry mode, the unnormalised probabilities of the panel rows)
-    TileArgs a = stats_args(w, ws, labels + t0, inv_temperature);
+    TileArgs a = stats_args(w, ws, labels + t0, inv_temperature, vocab_min != nullptr);
     a.panel = panel;
-    a.panel_ld = V;
+    a.panel_ld = w.panel_ld;
     a.out_rows = row_of_token;
     hipLaunchKernelGGL(k_label_logit, dim3((unsigned)((n_tok + 3) / 4)), dim3(256), 0, st, hid, (const uint16_t*)weight,
                        labels + t0, (int)n_tok, (int)H, (int)V, a.xy, redo_flag);
@@ -1109,11 +1196,12 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
       launch_tiles<kModeStats>(st, weight, hid, n_tok, H, V, a);
     // row statistics, per-token outputs, g
     TokenLossArgs la{at(prox_logp), at(adv), at(mask_eff), at(behave_w), n_valid, grad_scale, logp + t0, at(entropy),
-                     at(stat_loss), at(ratio), at(flags), *params, act};
-    hipLaunchKernelGGL(k_token_loss, dim3((unsigned)((n_tok + 63) / 64)), dim3(1024), 0, st, a.pk, a.ps, a.pu, a.xy,
+                     at(stat_loss), at(ratio), at(flags), at(vocab_max), at(vocab_min), *params, act};
+    hipLaunchKernelGGL(k_token_loss, dim3((unsigned)((n_tok + 63) / 64)), dim3(1024), 0, st, a.pk, a.ps, a.pu, a.pn, a.xy,
                        (int)w.blocks, a.pitch_t, (int)n_tok, (int)V, a.c, inv_temperature, labels + t0, la, row_of_token,
                        g_tok, lse_tok,
-                       (carry && rows > 0) ? CarryOut{row_factor, panel, V, redo_flag} : CarryOut{nullptr, nullptr, 0, nullptr});
+                       (carry && rows > 0) ? CarryOut{row_factor, panel, w.panel_ld, redo_flag}
+                                           : CarryOut{nullptr, nullptr, 0, nullptr});
     if (rows == 0) {
       launch_zero(st, dh, n_tok * H * 2);
       continue;

@@ -25,6 +25,7 @@ __all__ = [
     "ppo_actor_loss_fn",
     "fused_logprobs_ppo_loss",
     "lm_head_logprobs_entropy",
+    "lm_head_logprobs_entropy_stats",
 ]
 
 _DTYPES = {torch.bfloat16: N.AA_BF16, torch.float16: N.AA_F16, torch.float32: N.AA_F32}
@@ -760,40 +761,51 @@ def lm_head_chunk_tokens() -> int:
     return int(N.load().aa_lmhead_chunk_tokens())
 
 
-def _lmhead_workspace(T: int, H: int, V: int, dev, forward_only: bool = False) -> torch.Tensor:
+def _lmhead_workspace(T: int, H: int, V: int, dev, forward_only: bool = False, extrema: bool = False) -> torch.Tensor:
     lib = N.load()
-    n = lib.aa_lmhead_fwd_workspace_bytes(T, H, V) if forward_only else lib.aa_lmhead_workspace_bytes(T, H, V)
+    if forward_only:
+        n = lib.aa_lmhead_fwd_stats_workspace_bytes(T, H, V) if extrema else lib.aa_lmhead_fwd_workspace_bytes(T, H, V)
+    else:
+        n = lib.aa_lmhead_workspace_bytes(T, H, V)
     if n < 0:
         raise N.NativeLibraryError(
-            f"the lm_head path needs hidden size and vocabulary to be multiples of 8 (got H={H}, V={V})"
+            f"the lm_head path needs a hidden size that is a multiple of 8, and sizes below 2^22 (got H={H}, V={V})"
         )
     return torch.empty(n, dtype=torch.uint8, device=dev)
 
 
 class _LmHeadLogprobsEntropy(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, hidden, weight, labels, temperature):
+    def forward(ctx, hidden, weight, labels, temperature, want_minmax=False):
+        ctx.set_materialize_grads(False)
         lib = N.load()
         T, H = hidden.shape
         V = weight.shape[0]
         dev = hidden.device
         f32 = dict(dtype=torch.float32, device=dev)
         logp, entropy, row_lse, row_ez = (torch.empty(T, **f32) for _ in range(4))
-        ws = _lmhead_workspace(T, H, V, dev, forward_only=True)  # softmax partials only: nothing of size T x V
+        vmax = torch.empty(T, **f32) if want_minmax else None
+        vmin = torch.empty(T, **f32) if want_minmax else None
+        ws = _lmhead_workspace(T, H, V, dev, forward_only=True, extrema=want_minmax)  # partials only: nothing of size T x V
         with torch.cuda.device(dev):
             N.check(
                 lib.aa_lmhead_fwd(
                     _ptr(hidden), _ptr(weight), T, H, V, _ptr(labels), 1.0 / float(temperature), _ptr(logp),
-                    _ptr(entropy), _ptr(row_lse), _ptr(row_ez), _ptr(ws), ws.numel(), _stream(dev),
+                    _ptr(entropy), _ptr(row_lse), _ptr(row_ez), _ptr(vmax), _ptr(vmin), _ptr(ws), ws.numel(),
+                    _stream(dev),
                 ),
                 "aa_lmhead_fwd",
             )
         ctx.save_for_backward(hidden, weight, labels, row_lse, row_ez)
         ctx.temperature = float(temperature)
-        return logp, entropy
+        if want_minmax:
+            ctx.mark_non_differentiable(vmax, vmin)
+        return logp, entropy, vmax, vmin
 
     @staticmethod
-    def backward(ctx, g_logp, g_entropy):
+    def backward(ctx, g_logp, g_entropy, _g_vmax=None, _g_vmin=None):
+        if g_logp is None and g_entropy is None:
+            return None, None, None, None, None
         lib = N.load()
         hidden, weight, labels, row_lse, row_ez = ctx.saved_tensors
         T, H = hidden.shape
@@ -821,7 +833,7 @@ class _LmHeadLogprobsEntropy(torch.autograd.Function):
                 ),
                 "aa_lmhead_bwd",
             )
-        return d_hidden, d_weight, None, None
+        return d_hidden, d_weight, None, None, None
 
 
 def lm_head_logprobs_entropy(
@@ -829,6 +841,7 @@ def lm_head_logprobs_entropy(
     token_mask: torch.Tensor | None = None,
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """``gather_logprobs_entropy(hidden @ weight.T, labels, temperature)`` without writing the ``[T, V]`` logits.
+    Any vocabulary size; the hidden size has to be a multiple of 8.
 
     ``hidden`` is ``[T, H]`` and ``weight`` ``[V, H]`` (the lm_head), both bf16.  The forward forms 256 x 256 tiles of
     the logits in the accumulator registers of the library's bf16 MFMA tile GEMM (fp32 accumulation, not rounded to
@@ -848,6 +861,24 @@ def lm_head_logprobs_entropy(
     through the lm_head; the others get log-prob 0 and entropy 0 (e.g. the forward-only ``compute_logp`` pass, whose
     results are multiplied by the loss mask anyway).
     """
+    return _lm_head_impl(hidden, weight, labels, temperature, token_mask, False)[:2]
+
+
+def lm_head_logprobs_entropy_stats(
+    hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0,
+    token_mask: torch.Tensor | None = None,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``(logp, entropy, vocab_min_logits, vocab_max_logits)`` of ``hidden @ weight.T`` from the same tiles.
+
+    The last two are what ``FSDPEngine._get_vocab_min_max_logits`` (areal/engine/fsdp_engine.py:1893-1906) reads from
+    materialised logits and hands to the loss function; with no logits in memory the caller could not compute them.
+    They come from the fp32 sums of the tiles, not from logits rounded to bf16 (the smallest exactly, the largest
+    through the softmax exponent, i.e. to one rounding), and carry no gradient.  With ``token_mask`` the tokens left
+    out of the lm_head get 0 for both."""
+    return _lm_head_impl(hidden, weight, labels, temperature, token_mask, True)
+
+
+def _lm_head_impl(hidden, weight, labels, temperature, token_mask, want_minmax):
     _require_gpu(hidden, "hidden")
     if hidden.ndim != 2 or weight.ndim != 2 or hidden.shape[1] != weight.shape[1]:
         raise ValueError(f"expected hidden [T, H] and weight [V, H], got {tuple(hidden.shape)} and {tuple(weight.shape)}")
@@ -865,12 +896,15 @@ def lm_head_logprobs_entropy(
         n_kept = idx.numel()
         if n_kept == 0:
             zero = (hidden[:1].float().sum() + weight[:1].float().sum()) * 0.0
-            return zero.expand(T), zero.expand(T)
-        lp, ent = _LmHeadLogprobsEntropy.apply(hidden.index_select(0, idx), weight.contiguous(), y.index_select(0, idx),
-                                               float(temperature))
+            z = torch.zeros(T, dtype=torch.float32, device=dev) if want_minmax else None
+            return zero.expand(T), zero.expand(T), z, z
+        lp, ent, vmax, vmin = _LmHeadLogprobsEntropy.apply(
+            hidden.index_select(0, idx), weight.contiguous(), y.index_select(0, idx), float(temperature), want_minmax)
         full = lambda v: torch.zeros(T, dtype=torch.float32, device=dev).index_copy(0, idx, v)
-        return full(lp), full(ent)
-    return _LmHeadLogprobsEntropy.apply(hidden.contiguous(), weight.contiguous(), y, float(temperature))
+        return full(lp), full(ent), (full(vmin) if want_minmax else None), (full(vmax) if want_minmax else None)
+    lp, ent, vmax, vmin = _LmHeadLogprobsEntropy.apply(hidden.contiguous(), weight.contiguous(), y, float(temperature),
+                                                       want_minmax)
+    return lp, ent, vmin, vmax
 
 
 def lm_head_logprobs_entropy_static(
@@ -926,6 +960,8 @@ class _FusedLmHeadPpo(torch.autograd.Function):
         f32 = dict(dtype=torch.float32, device=dev)
         logp = torch.empty(T, **f32)
         entropy = torch.empty(T, **f32)
+        vmax = torch.empty(T, **f32)
+        vmin = torch.empty(T, **f32)
         stat_loss = torch.empty(T_active, **f32)
         ratio = torch.empty(T_active, **f32)
         flags = torch.empty(T_active, dtype=torch.uint8, device=dev)
@@ -940,14 +976,15 @@ class _FusedLmHeadPpo(torch.autograd.Function):
                     _ptr(hidden), _ptr(weight), T, H, V, _ptr(labels), 1.0 / float(temperature), T_active, _ptr(prox),
                     _ptr(adv), _ptr(mask_eff), _ptr(behave_w), C.byref(params), _ptr(n_valid), _ptr(grad_scale), kept,
                     int(backward_mode), _ptr(logp), _ptr(entropy), _ptr(stat_loss), _ptr(ratio), _ptr(flags),
-                    _ptr(d_hidden), _ptr(d_weight), _DTYPES[d_weight.dtype], _ptr(ws), ws.numel(), st,
+                    _ptr(vmax), _ptr(vmin), _ptr(d_hidden), _ptr(d_weight), _DTYPES[d_weight.dtype], _ptr(ws),
+                    ws.numel(), st,
                 ),
                 "aa_lmhead_ppo_fused",
             )
             _finish_fused_loss(lib, params, stat_loss, logp, mask_eff, T_active, n_valid, grad_scale, loss, st)
         ctx.save_for_backward(d_hidden, d_weight)
-        ctx.mark_non_differentiable(logp, entropy, stat_loss, ratio, flags)
-        return loss, logp, entropy, stat_loss, ratio, flags
+        ctx.mark_non_differentiable(logp, entropy, stat_loss, ratio, flags, vmax, vmin)
+        return loss, logp, entropy, stat_loss, ratio, flags, vmax, vmin
 
     @staticmethod
     def backward(ctx, g_loss, *_unused):
@@ -1003,7 +1040,8 @@ def fused_lm_head_ppo_loss(
     ``p_v / p_label`` of those tokens in bf16 into the rows (the label's logit is known before the tiles run); once
     the loss is known the gradient row is that row times one factor per token, which the two gradient GEMMs apply
     themselves, so there is neither a second logits GEMM nor a pass over the rows.  A chunk that holds a token whose
-    label has a log-prob below -80 (outside the stored range) is redone by recompute, decided on the device.  Both
+    label has a log-prob below -80, or whose factor is below 2^-100 in magnitude (outside the stored range), is redone
+    by recompute, decided on the device.  Both
     modes use the same workspace (``2 * chunk * V`` bytes for the rows).
 
     ``skip_masked_tokens``: a token whose (effective) loss mask is zero has a zero gradient row, so the two gradient
@@ -1012,7 +1050,12 @@ def fused_lm_head_ppo_loss(
     queues the chunk.  ``False`` multiplies the zero rows through, as the reference's autograd does, without that
     read.  A caller that already knows the counts on the host (the number of tokens with a non-zero effective mask
     in each chunk of ``aa_lmhead_chunk_tokens()`` tokens, e.g. from the CPU copy of ``loss_mask`` when there is no rejection sampling) can
-    pass them as ``kept_per_chunk``; nothing is read back then.
+    pass them as ``kept_per_chunk``; nothing is read back then.  A count that is too small drops the tokens beyond it
+    from the gradient; a count that is too large (e.g. counts of ``loss_mask`` while rejection sampling shrinks the
+    mask on the device) is safe: the surplus rows are cleared on the device and add nothing.
+
+    ``stat`` also holds ``vocab_min_logits`` / ``vocab_max_logits`` (what the engine would read from materialised
+    logits, areal/engine/fsdp_engine.py:1893-1906), from the fp32 sums of the tiles.
 
     ``forward_masked_tokens=False`` (token level only) goes one step further than the reference's semantics: tokens
     whose effective mask is zero are not run through the lm_head at all, so their entries of ``stat["logprobs"]``,
@@ -1048,7 +1091,7 @@ def fused_lm_head_ppo_loss(
 
     forward_only = not (torch.is_grad_enabled() and (hidden.requires_grad or weight.requires_grad))
     if importance_sampling_level == "sequence" or forward_only:  # no gradient to produce: forward GEMM + loss only
-        logp, entropy = lm_head_logprobs_entropy(hidden, weight, y, temperature)
+        logp, entropy, vmin, vmax = lm_head_logprobs_entropy_stats(hidden, weight, y, temperature)
         logp, entropy = logp[:T_active], entropy[:T_active]
         loss, stat = ppo_actor_loss_fn(
             logp, proximal_logprobs, old_logprobs, advantages, eps_clip, loss_mask, eps_clip_higher, c_clip,
@@ -1056,7 +1099,8 @@ def fused_lm_head_ppo_loss(
         )
         if scale_t is not None:
             loss = loss * scale_t.squeeze(0)
-        stat.update(logprobs=logp.detach(), entropy=entropy.detach())
+        stat.update(logprobs=logp.detach(), entropy=entropy.detach(), vocab_min_logits=vmin[:T_active],
+                    vocab_max_logits=vmax[:T_active])
         return loss, stat
 
     prox = _f32(proximal_logprobs.detach())
@@ -1086,12 +1130,12 @@ def fused_lm_head_ppo_loss(
             z = torch.zeros(T_active, dtype=torch.float32, device=dev)
             zb = torch.zeros(T_active, dtype=torch.bool, device=dev)
             stat = dict(loss=z, importance_weight=z.clone(), approx_kl=z.clone(), clip_mask=zb, dual_clip_mask=zb.clone(),
-                        logprobs=z.clone(), entropy=z.clone())
+                        logprobs=z.clone(), entropy=z.clone(), vocab_min_logits=z.clone(), vocab_max_logits=z.clone())
         else:
             ones = torch.ones(n_kept, dtype=torch.uint8, device=dev)
             chunk = int(N.load().aa_lmhead_chunk_tokens())
             kept = [max(0, min(chunk, n_kept - c)) for c in range(0, n_kept, chunk)]
-            loss, logp, entropy, stat_loss, ratio, flags = _FusedLmHeadPpo.apply(
+            loss, logp, entropy, stat_loss, ratio, flags, vmax, vmin = _FusedLmHeadPpo.apply(
                 hidden.index_select(0, idx), weight.contiguous(), y.index_select(0, idx), float(temperature), n_kept,
                 prox.index_select(0, idx), adv.index_select(0, idx), ones,
                 None if w is None else w.index_select(0, idx), params, n_valid, scale_t, kept, _LMHEAD_BACKWARD[backward],
@@ -1102,6 +1146,7 @@ def fused_lm_head_ppo_loss(
                 loss=full(stat_loss), importance_weight=full(ratio), approx_kl=full(logp - prox.index_select(0, idx)),
                 clip_mask=full(clip, torch.bool), dual_clip_mask=full(dual, torch.bool),
                 logprobs=full(logp), entropy=full(entropy),
+                vocab_min_logits=full(vmin[:n_kept]), vocab_max_logits=full(vmax[:n_kept]),
             )
         if rejection_sampling is not None:
             behave_mask = (w > 0) & mask_eff.bool()
@@ -1120,7 +1165,7 @@ def fused_lm_head_ppo_loss(
         if n_chunks * chunk != T_active:
             on = torch.nn.functional.pad(on, (0, n_chunks * chunk - T_active))
         kept = _HostCounts(on.view(n_chunks, chunk).sum(1)).tolist()
-    loss, logp, entropy, stat_loss, ratio, flags = _FusedLmHeadPpo.apply(
+    loss, logp, entropy, stat_loss, ratio, flags, vmax, vmin = _FusedLmHeadPpo.apply(
         hidden.contiguous(), weight.contiguous(), y, float(temperature), T_active, prox, adv, mask_eff, w, params,
         n_valid, scale_t, kept, _LMHEAD_BACKWARD[backward],
     )
@@ -1134,6 +1179,8 @@ def fused_lm_head_ppo_loss(
         dual_clip_mask=dual,
         logprobs=logp_a,
         entropy=entropy[:T_active],
+        vocab_min_logits=vmin[:T_active],
+        vocab_max_logits=vmax[:T_active],
     )
     if rejection_sampling is not None:
         _rs_stats(stat, behave_mask, behave_kl, w, host_counts, loss_mask.shape)

@@ -197,7 +197,7 @@ def fused_lm_head_sft_loss(hidden: torch.Tensor, weight: torch.Tensor, labels: t
             if n_chunks * chunk != T_active:
                 on = torch.nn.functional.pad(on, (0, n_chunks * chunk - T_active))
             kept = _HostCounts(on.view(n_chunks, chunk).sum(1)).tolist()
-    loss, logp, entropy, stat_loss, _ratio, _flags = _FusedLmHeadPpo.apply(
+    loss, logp, entropy, stat_loss, _ratio, _flags, _vmax, _vmin = _FusedLmHeadPpo.apply(
         hidden.contiguous(), weight.contiguous(), y, float(temperature), T_active, None, None, m8, None, _nll_params(),
         n_valid, scale_t, kept, 1,  # aa_lmhead_backward_mode: carry
     )

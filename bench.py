@@ -203,7 +203,7 @@ def time_fused_logits_kernel(case, kw, cfg, iters: int, inplace: bool = False):
             mask_eff = m8
     else:
         mask_eff, w, counts = m8, None, F._count_nonzero(m8)
-    logp, ent, sl, ratio = (torch.empty(T, **f32) for _ in range(4))
+    logp, ent, sl, ratio, vmax, vmin = (torch.empty(T, **f32) for _ in range(6))
     flags = torch.empty(T, dtype=torch.uint8, device=dev)
     dlogits = case.logits if inplace else torch.empty_like(case.logits)
     stream = torch.cuda.current_stream(dev)
@@ -523,7 +523,7 @@ def time_lmhead_step(case, kw, cfg, iters: int, skip_masked: bool, mode: int):
             mask_eff = m8
     else:
         mask_eff, w, counts = m8, None, F._count_nonzero(m8)
-    logp, ent, sl, ratio = (torch.empty(T, **f32) for _ in range(4))
+    logp, ent, sl, ratio, vmax, vmin = (torch.empty(T, **f32) for _ in range(6))
     flags = torch.empty(T, dtype=torch.uint8, device=dev)
     dh = torch.empty_like(case.hidden)
     dw = torch.empty_like(case.weight)  # bf16, as the Python wrapper asks for
@@ -540,8 +540,8 @@ def time_lmhead_step(case, kw, cfg, iters: int, skip_masked: bool, mode: int):
             lib.aa_lmhead_ppo_fused(
                 F._ptr(case.hidden), F._ptr(case.weight), T, H, V, F._ptr(case.labels), 1.0 / case.temperature, T,
                 F._ptr(prox), F._ptr(adv), F._ptr(mask_eff), F._ptr(w), C.byref(params), F._ptr(counts), None, kept,
-                mode, F._ptr(logp), F._ptr(ent), F._ptr(sl), F._ptr(ratio), F._ptr(flags), F._ptr(dh), F._ptr(dw),
-                N.AA_BF16, F._ptr(ws), ws.numel(), C.c_void_p(stream.cuda_stream),
+                mode, F._ptr(logp), F._ptr(ent), F._ptr(sl), F._ptr(ratio), F._ptr(flags), F._ptr(vmax), F._ptr(vmin),
+                F._ptr(dh), F._ptr(dw), N.AA_BF16, F._ptr(ws), ws.numel(), C.c_void_p(stream.cuda_stream),
             ),
             "aa_lmhead_ppo_fused",
         )
@@ -573,7 +573,7 @@ def time_lmhead_op(case, iters: int):
 
     def fwd():
         N.check(lib.aa_lmhead_fwd(F._ptr(case.hidden), F._ptr(case.weight), T, H, V, F._ptr(case.labels), inv_t,
-                                  F._ptr(logp), F._ptr(ent), F._ptr(lse), F._ptr(ez), F._ptr(ws), ws.numel(), st),
+                                  F._ptr(logp), F._ptr(ent), F._ptr(lse), F._ptr(ez), None, None, F._ptr(ws), ws.numel(), st),
                 "aa_lmhead_fwd")
 
     has_grad, kept, kept_tokens = None, None, T

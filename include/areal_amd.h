@@ -617,8 +617,8 @@ int aa_masked_moments(const float* const* values, int n_tensors,
 
 /* Bytes of workspace aa_lmhead_bwd / aa_lmhead_ppo_fused need for these sizes.
  * With C = min(T, aa_lmhead_chunk_tokens()): 2 * C * V (the bf16 d(logits)
- * rows of one token chunk), 24 * (V / 256) * C (softmax partials per 128
- * vocabulary rows and token), 2 * C * H (the hidden rows of the tokens with a
+ * rows of one token chunk; their pitch is V rounded up to 8), 32 * (V / 256) *
+ * C (softmax partials and smallest logit per 128 vocabulary rows and token), 2 * C * H (the hidden rows of the tokens with a
  * gradient, closed up), 16 * C * H (four fp32 planes of d_hidden rows: the
  * product that forms them has few tiles and is cut along the vocabulary into
  * up to four parts when that fills the chip better), plus 4 * H * V (an fp32
@@ -632,8 +632,23 @@ int64_t aa_lmhead_workspace_bytes(int64_t T, int64_t H, int64_t V);
  * T = 16384, V = 151936). */
 int64_t aa_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);
 
+/* The same when aa_lmhead_fwd is also asked for vocab_max / vocab_min: one
+ * more plane, the smallest logit per 128 vocabulary rows and token (a third
+ * more). */
+int64_t aa_lmhead_fwd_stats_workspace_bytes(int64_t T, int64_t H, int64_t V);
+
 /* Tokens per chunk of the lm_head entry points (16384). */
 int64_t aa_lmhead_chunk_tokens(void);
+
+/*
+ * Per-device set-up of the lm_head entry points (the tile kernels are allowed
+ * their 160 KiB of LDS with hipFuncSetAttribute, which is not a stream
+ * operation).  Every aa_lmhead_* entry point does it by itself on its first
+ * call on a device; call this once per device, with that device current,
+ * before capturing any of them into a HIP graph, so that no such call falls
+ * inside the capture.  No counterpart in the reference.
+ */
+int aa_lmhead_prepare(void);
 
 /*
  * logp / entropy of softmax(hidden @ weight.T / temperature) without writing
@@ -641,21 +656,30 @@ int64_t aa_lmhead_chunk_tokens(void);
  * registers of this library's bf16 MFMA tile GEMM (fp32 accumulation, no
  * rounding to bf16 in between), each tile is reduced to softmax partials per
  * token in the GEMM's epilogue, and a small kernel merges the partials.
- * hidden [T, H] bf16 row-major, weight [V, H] bf16 row-major; H and V
- * multiples of 8 (below 2^22).  entropy, row_lse, row_ez may be NULL; row_lse /
- * row_ez as in aa_logits_fwd (needed by aa_lmhead_bwd).
- * workspace: aa_lmhead_fwd_workspace_bytes(T, H, V) bytes.
+ * hidden [T, H] bf16 row-major, weight [V, H] bf16 row-major; H a multiple of
+ * 8, any V (both below 2^22), as the reference's lm_head ->
+ * _gather_logprobs_entropy (areal/utils/functional/vocab_parallel.py:23-29)
+ * takes any vocabulary.  entropy, row_lse, row_ez may be NULL; row_lse / row_ez
+ * as in aa_logits_fwd (needed by aa_lmhead_bwd).
+ * vocab_max / vocab_min [T] (both or neither): largest and smallest logit of
+ * every row, what FSDPEngine._get_vocab_min_max_logits reads from materialised
+ * logits (areal/engine/fsdp_engine.py:1893-1906), here from the fp32 sums of
+ * the tiles (the smallest exactly; the largest through the softmax exponent,
+ * i.e. to one rounding).
+ * workspace: aa_lmhead_fwd_workspace_bytes(T, H, V) bytes, or
+ * aa_lmhead_fwd_stats_workspace_bytes(T, H, V) with the extrema.
  */
 int aa_lmhead_fwd(const void* hidden, const void* weight, int64_t T, int64_t H,
                   int64_t V, const int64_t* labels, float inv_temperature,
                   float* logp, float* entropy, float* row_lse, float* row_ez,
-                  void* workspace, int64_t workspace_bytes, void* stream);
+                  float* vocab_max, float* vocab_min, void* workspace,
+                  int64_t workspace_bytes, void* stream);
 
 /*
  * aa_lmhead_fwd for callers that cannot allocate device memory or bring a
  * workspace (code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc).  No counterpart in the reference.  Same arguments and
- * results as aa_lmhead_fwd without the workspace: the softmax partials live in
+ * results as aa_lmhead_fwd without the workspace and the vocabulary extrema: the softmax partials live in
  * a device array of the library itself, aa_lmhead_fwd_static_scratch_bytes()
  * = 32 MiB on every GPU the library has been used on, held until the process
  * ends.  Tokens go through in passes of as many as fit that array (a multiple
@@ -664,7 +688,10 @@ int aa_lmhead_fwd(const void* hidden, const void* weight, int64_t T, int64_t H,
  * fit, is refused with AA_ERR_UNSUPPORTED.  The call allocates and frees
  * nothing.  All calls on one GPU share the array: calls that overlap on one GPU
  * (two streams, two host threads) race and must be serialised by the caller;
- * nothing in the array needs clearing between calls.
+ * nothing in the array needs clearing between calls.  The first call on a
+ * device also does that device's set-up (aa_lmhead_prepare and the address of
+ * the array, neither a stream operation): make one eager call, or call
+ * aa_lmhead_prepare and then this once, before capturing it into a graph.
  */
 int aa_lmhead_fwd_static(const void* hidden, const void* weight, int64_t T,
                          int64_t H, int64_t V, const int64_t* labels,
@@ -710,8 +737,9 @@ typedef enum {
    * the loss is known, d(logits) of a row is that row times one factor per
    * token, which the two gradient GEMMs apply themselves (no second logits
    * GEMM, no pass over the rows).  A chunk with a token whose label has a
-   * log-prob below -80 does not fit the stored range and is redone as in
-   * AA_LMHEAD_RECOMPUTE, decided on the device (same results, slower). */
+   * log-prob below -80, or whose factor is below 2^-100 in magnitude, does
+   * not fit the stored range and is redone as in AA_LMHEAD_RECOMPUTE, decided
+   * on the device (same results, slower). */
   AA_LMHEAD_CARRY = 1
 } aa_lmhead_backward_mode;
 
@@ -740,7 +768,10 @@ typedef enum {
  * tokens, only those tokens get a d(logits) row and go through the backward
  * GEMMs (the reference's autograd multiplies the zero rows through).  The
  * counts size the GEMMs, which is why they come from the host; tokens beyond a
- * count that is too small are treated as masked.  NULL: every token has a row.
+ * count that is too small are treated as masked, and the surplus rows of a
+ * count that is too large are cleared on the device and add nothing (slower,
+ * same results).  NULL: every token has a row.
+ * vocab_max / vocab_min [T] (nullable, both or neither): as in aa_lmhead_fwd.
  */
 int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64_t T,
                         int64_t H, int64_t V, const int64_t* labels,
@@ -751,9 +782,9 @@ int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64_t T,
                         const float* grad_scale, const int64_t* kept_per_chunk,
                         int backward_mode, float* logp, float* entropy,
                         float* stat_loss, float* ratio, uint8_t* flags,
-                        void* d_hidden, void* d_weight, int d_weight_dtype,
-                        void* workspace, int64_t workspace_bytes,
-                        void* stream);
+                        float* vocab_max, float* vocab_min, void* d_hidden,
+                        void* d_weight, int d_weight_dtype, void* workspace,
+                        int64_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------ */
 /* Packing                                                                 */

@@ -159,7 +159,7 @@ int main(void) {
       if (is_w) { wgt[i - LT * LH] = (uint16_t)(bits >> 16); wgt_d[i - LT * LH] = f; }
       else { hid[i] = (uint16_t)(bits >> 16); hid_d[i] = f; }
     }
-    double want_lp[LT], want_ent[LT];
+    double want_lp[LT], want_ent[LT], want_max[LT], want_min[LT];
     for (int t = 0; t < LT; ++t) {
       static double z[LV];
       double mx = -1e300, sum = 0.0, u = 0.0;
@@ -169,6 +169,8 @@ int main(void) {
         for (int h = 0; h < LH; ++h) acc += hid_d[t * LH + h] * wgt_d[v * LH + h];
         z[v] = acc * inv_temperature;
         mx = fmax(mx, z[v]);
+        want_max[t] = v == 0 ? acc : fmax(want_max[t], acc); /* extrema of the raw logits */
+        want_min[t] = v == 0 ? acc : fmin(want_min[t], acc);
       }
       for (int v = 0; v < LV; ++v) { sum += exp(z[v] - mx); u += exp(z[v] - mx) * z[v]; }
       want_lp[t] = z[llabels[t]] - (mx + log(sum));
@@ -176,9 +178,9 @@ int main(void) {
     }
     uint16_t *d_hid, *d_wgt;
     int64_t* d_ll;
-    float *d_lp, *d_ent, *d_lp2, *d_ent2;
+    float *d_lp, *d_ent, *d_lp2, *d_ent2, *d_vmax, *d_vmin;
     void* d_ws;
-    const int64_t ws_bytes = aa_lmhead_fwd_workspace_bytes(LT, LH, LV);
+    const int64_t ws_bytes = aa_lmhead_fwd_stats_workspace_bytes(LT, LH, LV); /* with the extrema of the logits */
     if (ws_bytes <= 0) return 5;
     HIP_OK(hipMalloc((void**)&d_hid, sizeof(hid)));
     HIP_OK(hipMalloc((void**)&d_wgt, sizeof(wgt)));
@@ -187,14 +189,20 @@ int main(void) {
     HIP_OK(hipMalloc((void**)&d_ent, LT * sizeof(float)));
     HIP_OK(hipMalloc((void**)&d_lp2, LT * sizeof(float)));
     HIP_OK(hipMalloc((void**)&d_ent2, LT * sizeof(float)));
+    HIP_OK(hipMalloc((void**)&d_vmax, LT * sizeof(float)));
+    HIP_OK(hipMalloc((void**)&d_vmin, LT * sizeof(float)));
     HIP_OK(hipMalloc(&d_ws, (size_t)ws_bytes));
     HIP_OK(hipMemcpy(d_hid, hid, sizeof(hid), hipMemcpyHostToDevice));
     HIP_OK(hipMemcpy(d_wgt, wgt, sizeof(wgt), hipMemcpyHostToDevice));
     HIP_OK(hipMemcpy(d_ll, llabels, sizeof(llabels), hipMemcpyHostToDevice));
-    AA_CHECK(aa_lmhead_fwd(d_hid, d_wgt, LT, LH, LV, d_ll, inv_temperature, d_lp, d_ent, NULL, NULL, d_ws, ws_bytes, NULL));
+    AA_CHECK(aa_lmhead_prepare());
+    AA_CHECK(aa_lmhead_fwd(d_hid, d_wgt, LT, LH, LV, d_ll, inv_temperature, d_lp, d_ent, NULL, NULL, d_vmax, d_vmin, d_ws, ws_bytes,
+                           NULL));
     AA_CHECK(aa_lmhead_fwd_static(d_hid, d_wgt, LT, LH, LV, d_ll, inv_temperature, d_lp2, d_ent2, NULL, NULL, NULL));
     HIP_OK(hipDeviceSynchronize());
-    float lp[LT], ent[LT], lp2[LT], ent2[LT];
+    float lp[LT], ent[LT], lp2[LT], ent2[LT], vmax[LT], vmin[LT];
+    HIP_OK(hipMemcpy(vmax, d_vmax, sizeof(vmax), hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(vmin, d_vmin, sizeof(vmin), hipMemcpyDeviceToHost));
     HIP_OK(hipMemcpy(lp, d_lp, sizeof(lp), hipMemcpyDeviceToHost));
     HIP_OK(hipMemcpy(ent, d_ent, sizeof(ent), hipMemcpyDeviceToHost));
     HIP_OK(hipMemcpy(lp2, d_lp2, sizeof(lp2), hipMemcpyDeviceToHost));
@@ -202,13 +210,15 @@ int main(void) {
     for (int t = 0; t < LT; ++t) {
       ok &= close_to(lp[t], want_lp[t], 5e-6, "lm_head logp", t);
       ok &= close_to(ent[t], want_ent[t], 5e-6, "lm_head entropy", t);
+      ok &= close_to(vmax[t], want_max[t], 5e-6, "lm_head vocab max", t);
+      ok &= close_to(vmin[t], want_min[t], 5e-6, "lm_head vocab min", t);
       ok &= lp[t] == lp2[t] && ent[t] == ent2[t]; /* the two entry points run the same kernels */
     }
     /* H must be a multiple of 8 */
-    ok &= aa_lmhead_fwd(d_hid, d_wgt, LT, LH - 4, LV, d_ll, inv_temperature, d_lp, d_ent, NULL, NULL, d_ws, ws_bytes, NULL) ==
+    ok &= aa_lmhead_fwd(d_hid, d_wgt, LT, LH - 4, LV, d_ll, inv_temperature, d_lp, d_ent, NULL, NULL, NULL, NULL, d_ws, ws_bytes, NULL) ==
           AA_ERR_UNSUPPORTED;
     hipFree(d_hid); hipFree(d_wgt); hipFree(d_ll); hipFree(d_lp); hipFree(d_ent); hipFree(d_lp2); hipFree(d_ent2);
-    hipFree(d_ws);
+    hipFree(d_vmax); hipFree(d_vmin); hipFree(d_ws);
   }
 
   hipFree(d_logits); hipFree(d_labels); hipFree(d_mask); hipFree(d_logp); hipFree(d_entropy); hipFree(d_g);

@@ -33,6 +33,10 @@ def _case(T, H, V, seed, w_std=0.02):
         (37, 64, 576, 0.7),
         (700, 256, 4160, 1.3),
         (203, 200, 1096, 1.0),    # H and V multiples of 8 only
+        (37, 64, 577, 0.7),       # vocabularies that are no multiple of 8 (the reference takes any, vocab_parallel.py:15-29)
+        (300, 128, 1001, 1.0),
+        (70, 64, 50257, 1.0),
+        (40, 64, 151643, 1.0),
     ],
 )
 def test_forward_matches_oracle(device, T, H, V, temperature):
@@ -70,7 +74,9 @@ def test_closed_form_and_bad_label(device):
 
 @pytest.mark.parametrize("T,H,V,temperature,with_entropy",
                          [(300, 128, 1088, 1.0, False), (520, 192, 832, 0.8, True), (203, 200, 1096, 1.0, True),
-                          (300, 128, 16640, 1.0, True)])   # the last: d(hidden) cut into parts along the vocabulary
+                          (300, 128, 16640, 1.0, True),    # d(hidden) cut into parts along the vocabulary
+                          (203, 72, 1097, 1.0, True), (70, 64, 50257, 0.9, False),  # any vocabulary size
+                          (300, 128, 16643, 1.0, True)])   # ... with d(hidden) cut into parts
 def test_backward_matches_autograd_of_oracle(device, T, H, V, temperature, with_entropy):
     hidden, weight, labels = _case(T, H, V, seed=7 * T + V, w_std=0.3)
     g = torch.Generator().manual_seed(3)
@@ -212,7 +218,7 @@ def test_weight_gradient_dtypes_through_the_c_abi(device, T, H, V):
     ws = F._lmhead_workspace(T, H, V, device)
     st = C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
     N.check(lib.aa_lmhead_fwd(F._ptr(hd), F._ptr(wd), T, H, V, F._ptr(ld), 1.0, F._ptr(logp), F._ptr(ent), F._ptr(lse),
-                              F._ptr(ez), F._ptr(ws), ws.numel(), st), "aa_lmhead_fwd")
+                              F._ptr(ez), None, None, F._ptr(ws), ws.numel(), st), "aa_lmhead_fwd")
     out = {}
     for dt, code in ((torch.float32, N.AA_F32), (torch.bfloat16, N.AA_BF16)):
         dh = torch.empty_like(hd)
@@ -260,7 +266,7 @@ def test_backward_leaves_out_rows_without_gradient(device):
     ws = F._lmhead_workspace(T, H, V, device)
     st = C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
     N.check(lib.aa_lmhead_fwd(F._ptr(hd), F._ptr(wd), T, H, V, F._ptr(ld), 1.0, F._ptr(logp), F._ptr(e), F._ptr(lse),
-                              F._ptr(ez), F._ptr(ws), ws.numel(), st), "aa_lmhead_fwd")
+                              F._ptr(ez), None, None, F._ptr(ws), ws.numel(), st), "aa_lmhead_fwd")
     dh, dw = torch.empty_like(hd), torch.empty_like(wd)
     gld, ghd = gl.to(device), gh.to(device)
     N.check(lib.aa_lmhead_bwd(F._ptr(hd), F._ptr(wd), T, H, V, F._ptr(ld), 1.0, F._ptr(lse), F._ptr(ez), F._ptr(gld),
@@ -320,7 +326,7 @@ def test_row_counts_that_disagree_with_the_mask_stay_in_bounds(device):
     ws = F._lmhead_workspace(T, H, V, device)
     st = C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
     N.check(lib.aa_lmhead_fwd(F._ptr(hd), F._ptr(wd), T, H, V, F._ptr(ld), 1.0, F._ptr(logp), F._ptr(e), F._ptr(lse),
-                              F._ptr(ez), F._ptr(ws), ws.numel(), st), "aa_lmhead_fwd")
+                              F._ptr(ez), None, None, F._ptr(ws), ws.numel(), st), "aa_lmhead_fwd")
     has = (gl != 0)
     n = int(has.sum())
 
@@ -364,9 +370,26 @@ def test_forward_needs_no_panel(device):
     logp, ent = torch.empty(T, **f32), torch.empty(T, **f32)
     st = C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
     N.check(lib.aa_lmhead_fwd(F._ptr(hd), F._ptr(wd), T, H, V, F._ptr(ld), 1.0, F._ptr(logp), F._ptr(ent), None, None,
-                              F._ptr(ws), n, st), "aa_lmhead_fwd")
+                              None, None, F._ptr(ws), n, st), "aa_lmhead_fwd")
     r_lp, r_ent = oracle.logprobs_entropy_f64(oracle.lmhead_logits(hidden, weight), labels, 1.0)
     assert_within(logp, r_lp, 2e-3, "log-prob")
     assert_within(ent, r_ent, 2e-3, "entropy")
     assert lib.aa_lmhead_fwd(F._ptr(hd), F._ptr(wd), T, H, V, F._ptr(ld), 1.0, F._ptr(logp), F._ptr(ent), None, None,
-                             F._ptr(ws), n - 1, st) == 1                                # AA_ERR_INVALID_ARGUMENT
+                             None, None, F._ptr(ws), n - 1, st) == 1                                # AA_ERR_INVALID_ARGUMENT
+
+
+@pytest.mark.parametrize("T,H,V,temperature", [(300, 128, 1088, 1.0), (203, 72, 1097, 0.7), (CHUNK + 70, 64, 640, 1.3)])
+def test_vocabulary_extrema_of_the_logits(device, T, H, V, temperature):
+    """vocab_min_logits / vocab_max_logits, which the engine reads from materialised logits and hands to the loss
+    function (areal/engine/fsdp_engine.py:1893-1906), here from the tiles: extrema of the raw (not temperature-scaled)
+    fp32 logits.  Tolerance: the order of the fp32 accumulation (1e-5 of the largest logit)."""
+    hidden, weight, labels = _case(T, H, V, seed=3 * T + V, w_std=0.3)
+    lp, ent, vmin, vmax = areal_amd.lm_head_logprobs_entropy_stats(
+        hidden.to(device), weight.to(device), labels.to(device), temperature)
+    logits = oracle.lmhead_logits(hidden, weight)
+    scale = float(logits.abs().max())
+    assert float((vmax.cpu() - logits.max(-1).values).abs().max()) <= 1e-5 * scale
+    assert float((vmin.cpu() - logits.min(-1).values).abs().max()) <= 1e-5 * scale
+    assert not vmin.requires_grad and not vmax.requires_grad
+    lp2, ent2 = areal_amd.lm_head_logprobs_entropy(hidden.to(device), weight.to(device), labels.to(device), temperature)
+    assert torch.equal(lp, lp2) and torch.equal(ent, ent2)  # asking for the extrema changes nothing else

@@ -48,6 +48,9 @@ CASES = [
     (520, 500, 64, 8256, 0.8, 0.37, dict(eps_clip=0.2, eps_clip_higher=0.28, c_clip=3.0)),  # batch padding, dual clip
     (CHUNK + 200, CHUNK + 130, 64, 640, 1.0, 1.0, dict(eps_clip=0.2, rs=True)),             # two token chunks
     (203, 203, 200, 1096, 1.3, 1.0, dict(eps_clip=0.2)),                                    # H, V multiples of 8 only
+    (203, 190, 72, 1097, 0.7, 1.0, dict(eps_clip=0.2, c_clip=3.0)),                         # any vocabulary size
+    (96, 90, 64, 50257, 1.0, 1.0, dict(eps_clip=0.2)),
+    (64, 60, 64, 151643, 1.0, 0.5, dict(eps_clip=0.2, rs=True)),
 ]
 
 
@@ -71,6 +74,9 @@ def test_step_matches_reference_pipeline(device, T_pad, T, H, V, temperature, lo
     assert float(loss.detach()) == pytest.approx(o_loss, rel=1e-3)  # stated tolerances
     assert_within(stat["logprobs"], o_lp[:T], 2e-3, "log-prob")
     assert_within(stat["entropy"], o_ent[:T], 2e-3, "entropy")
+    logits = oracle.lmhead_logits(hidden, weight)[:T]  # what the engine would take the extrema of (fsdp_engine.py:1893-1906)
+    assert float((stat["vocab_max_logits"].cpu() - logits.max(-1).values).abs().max()) <= 1e-5 * float(logits.abs().max())
+    assert float((stat["vocab_min_logits"].cpu() - logits.min(-1).values).abs().max()) <= 1e-5 * float(logits.abs().max())
     for k in ("clip_mask", "dual_clip_mask"):   # a flag can only differ where the ratio sits on a clip boundary
         assert int((stat[k].cpu() != o_stat[k]).sum()) <= 1, k
     assert cosine(h_d.grad.cpu().float(), o_dh) > 0.9999
@@ -422,6 +428,112 @@ def test_counts_from_the_caller_replace_the_read_back(device):
     assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]) and torch.equal(a[2], b[2])
     with pytest.raises(ValueError, match="one count per chunk"):
         run(kept_per_chunk=[1])
+
+
+def _poison_the_allocator_cache(device, nbytes):
+    """The workspace of the step is a fresh ``torch.empty``: fill a block of that size with NaN patterns and hand it
+    back to the caching allocator, so that rows which nothing writes would show."""
+    junk = torch.full((nbytes // 2,), float("nan"), dtype=torch.bfloat16, device=device)
+    del junk
+
+
+@pytest.mark.parametrize("backward", ["carry", "recompute"])
+def test_counts_larger_than_the_mask_holds_add_nothing(device, backward):
+    """Counts taken from ``loss_mask`` on the host while rejection sampling shrinks the mask on the device: the surplus
+    rows have no token.  They are cleared on the device and the results are those of the exact counts."""
+    hidden, weight, labels, prox, old, adv, mask = _inputs(CHUNK + 256, CHUNK + 200, 64, 640, seed=43)
+    args = [t.to(device) for t in (labels, prox, old, adv)]
+    rs = RejectionSamplingConfig(level="token", action="mask", metric="ratio", upper=1.2)
+    cu = torch.tensor([0, CHUNK + 200], dtype=torch.int32, device=device)
+    host_counts = [int(mask[:CHUNK].sum()), int(mask[CHUNK:].sum())]   # before rejection sampling: too large
+
+    def run(**kw):
+        h = hidden.to(device).requires_grad_(True)
+        w = weight.to(device).requires_grad_(True)
+        _poison_the_allocator_cache(device, int(_native.load().aa_lmhead_workspace_bytes(CHUNK + 256, 64, 640)))
+        loss, stat = areal_amd.fused_lm_head_ppo_loss(h, w, *args, eps_clip=0.2, loss_mask=mask.to(device),
+                                                      rejection_sampling=rs, cu_seqlens=cu, backward=backward, **kw)
+        loss.backward()
+        return loss.detach(), stat, h.grad, w.grad
+
+    exact, over = run(), run(kept_per_chunk=host_counts)
+    assert float(exact[1]["filtered_fraction"]) > 0.05              # the mask did shrink
+    assert torch.isfinite(over[2].float()).all() and torch.isfinite(over[3].float()).all()
+    assert torch.equal(exact[0], over[0]) and torch.equal(exact[2], over[2])
+    # d(W): the same rows in the same order, plus rows of zeros at the end of each chunk
+    assert cosine(exact[3].float().cpu(), over[3].float().cpu()) > 0.9999999
+    assert_same_magnitude(over[3].float(), exact[3].float(), rel=1e-4)
+
+
+def test_carry_with_unlikely_labels_at_masked_tokens_of_a_dense_backward(device):
+    """``skip_masked_tokens=False`` puts every token in the panel.  A masked token (a prompt position) whose label is a
+    hundred nats unlikely stores ratios p_v / p_label at the top of the bf16 range; their sum over the vocabulary may be
+    infinite, and its factor is zero: the d(hidden) row has to come out as zero, not as 0 x inf."""
+    T, H, V = 600, 64, 1088
+    g = torch.Generator().manual_seed(9)
+    hidden = torch.randn(T, H, generator=g)
+    hidden[:200] *= 14.0                       # logits ~ N(0, 56^2) at the first 200 tokens
+    hidden = hidden.bfloat16()
+    weight = (0.5 * torch.randn(V, H, generator=g)).bfloat16()
+    labels = torch.randint(0, V, (T,), generator=g)
+    ref_lp = oracle.logprobs(oracle.lmhead_logits(hidden, weight), labels)
+    mask = torch.ones(T, dtype=torch.bool)
+    mask[:200] = False                          # those tokens have no gradient
+    assert int((ref_lp[:200] < -100).sum()) > 20 and float(ref_lp[200:].min()) > -60
+    prox = ref_lp + 0.05 * torch.randn(T, generator=g)
+    old = ref_lp + 0.3 * torch.randn(T, generator=g)
+    adv = torch.randn(T, generator=g)
+    h = hidden.to(device).requires_grad_(True)
+    w = weight.to(device).requires_grad_(True)
+    loss, _ = areal_amd.fused_lm_head_ppo_loss(h, w, labels.to(device), prox.to(device), old.to(device), adv.to(device),
+                                               eps_clip=0.2, loss_mask=mask.to(device), backward="carry",
+                                               skip_masked_tokens=False)
+    loss.backward()
+    o_loss, _, _, _, o_dh, o_dw = _oracle_step(hidden, weight, labels, prox, old, adv, mask, 1.0, 1.0, eps_clip=0.2)
+    assert torch.isfinite(h.grad.float()).all() and torch.isfinite(w.grad.float()).all()
+    assert float(h.grad[:200].abs().sum()) == 0.0
+    assert float(loss.detach()) == pytest.approx(o_loss, rel=1e-3)
+    assert cosine(h.grad.cpu().float(), o_dh) > 0.9999 and cosine(w.grad.cpu().float(), o_dw) > 0.9999
+    assert_same_magnitude(h.grad, o_dh, what="d(hidden)")
+    assert_same_magnitude(w.grad, o_dw, what="d(W)")
+
+
+def test_carry_with_small_factors_keeps_the_weight_gradient(device):
+    """d(W) takes the row factor -(g / T) p_label inside the hidden rows, rounded to bf16.  Labels with a log-prob
+    around -70 and a small loss scale push factor x hidden out of the normal range although d(logits) itself is of
+    ordinary size there: such a chunk is redone by the recompute tiles.  Held to the oracle and to recompute mode."""
+    T, H, V = 700, 64, 1088
+    g = torch.Generator().manual_seed(21)
+    hidden = (9.5 * torch.randn(T, H, generator=g)).bfloat16()     # logits ~ N(0, 38^2)
+    weight = (0.5 * torch.randn(V, H, generator=g)).bfloat16()
+    labels = torch.randint(0, V, (T,), generator=g)
+    ref_lp = oracle.logprobs(oracle.lmhead_logits(hidden, weight), labels)
+    window = (ref_lp < -62) & (ref_lp > -79)
+    assert int(window.sum()) > 30
+    mask = window | (torch.rand(T, generator=g) < 0.3)
+    mask &= ref_lp > -79                        # nothing below the overflow threshold: only the factor can trigger
+    prox = ref_lp + 0.05 * torch.randn(T, generator=g)
+    old = ref_lp + 0.3 * torch.randn(T, generator=g)
+    adv = torch.randn(T, generator=g)
+    scale = 1e-4
+    args = [t.to(device) for t in (labels, prox, old, adv)]
+
+    def run(backward):
+        h = hidden.to(device).requires_grad_(True)
+        w = weight.to(device).requires_grad_(True)
+        loss, _ = areal_amd.fused_lm_head_ppo_loss(h, w, *args, eps_clip=0.2, loss_mask=mask.to(device), backward=backward,
+                                                   loss_scale=scale)
+        loss.backward()
+        return loss.detach(), h.grad.float(), w.grad.float()
+
+    o_loss, _, _, _, o_dh, o_dw = _oracle_step(hidden, weight, labels, prox, old, adv, mask, 1.0, scale, eps_clip=0.2)
+    ref, got = run("recompute"), run("carry")
+    assert float(got[0]) == pytest.approx(o_loss, rel=1e-3)
+    for name, a, b, o in (("d(hidden)", got[1], ref[1], o_dh), ("d(W)", got[2], ref[2], o_dw)):
+        assert torch.isfinite(a).all(), name
+        assert cosine(a.cpu(), o) > 0.9999, name
+        assert_same_magnitude(a, o, what=name)
+        assert cosine(a.cpu(), b.cpu()) > 0.99999, name
 
 
 @pytest.mark.parametrize("backward", ["carry", "recompute"])

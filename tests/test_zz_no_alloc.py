@@ -44,8 +44,8 @@ def _fwd(lib, hidden, weight, labels, inv_t):
     assert n > 0
     ws = torch.empty(n, dtype=torch.uint8, device=dev)
     out = _outputs(T, dev)
-    N.check(lib.aa_lmhead_fwd(_ptr(hidden), _ptr(weight), T, H, V, _ptr(labels), inv_t, *[_ptr(o) for o in out], _ptr(ws),
-                              ws.numel(), _stream(dev)), "aa_lmhead_fwd")
+    N.check(lib.aa_lmhead_fwd(_ptr(hidden), _ptr(weight), T, H, V, _ptr(labels), inv_t, *[_ptr(o) for o in out], None, None,
+                              _ptr(ws), ws.numel(), _stream(dev)), "aa_lmhead_fwd")
     return out
 
 
