@@ -14,7 +14,15 @@ from typing import Any
 import torch
 
 from .advantages import gae_advantages, kl_regularized_rewards
-from .functional import fused_logprobs_ppo_loss, gather_logprobs, gather_logprobs_entropy_stats, ppo_actor_loss_fn
+from .functional import (
+    fused_lm_head_ppo_loss,
+    fused_logprobs_ppo_loss,
+    gather_logprobs,
+    gather_logprobs_entropy_stats,
+    lm_head_chunk_tokens,
+    lm_head_logprobs_entropy,
+    ppo_actor_loss_fn,
+)
 
 
 def rolled_labels(model_inputs: dict[str, Any]) -> torch.Tensor:
@@ -83,6 +91,85 @@ def compute_logprobs_and_loss(
     loss, stat = ppo_actor_loss_fn(logp, prox_logp, old_logp, mb_input["advantages"], loss_mask=loss_mask, **kw)
     stat.update(logprobs=logp.detach(), entropy=entropy.detach(), vocab_min_logits=vmin, vocab_max_logits=vmax)
     return loss * scale, stat
+
+
+def compute_lm_head_logprobs(hidden: torch.Tensor, weight: torch.Tensor, model_inputs: dict[str, Any],
+                             temperature: float = 1.0, token_mask: torch.Tensor | None = None) -> torch.Tensor:
+    """Forward-only log-probs of a micro-batch (fsdp_engine.py:1938-1964) from the final hidden states and the
+    lm_head weight, without the ``[T_pad, V]`` logits.  ``token_mask`` (optional, beyond the reference's semantics):
+    only these tokens go through the lm_head, the others get 0."""
+    if hidden.ndim == 3 and hidden.shape[0] == 1:
+        hidden = hidden.squeeze(0)
+    return lm_head_logprobs_entropy(hidden, weight, rolled_labels(model_inputs), temperature, token_mask)[0]
+
+
+def compute_lm_head_and_loss(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    model_inputs: dict[str, Any],
+    mb_input: dict[str, Any],
+    pad_length: int,
+    total_loss_weight: torch.Tensor | float,
+    eps_clip: float,
+    eps_clip_higher: float | None = None,
+    c_clip: float | None = None,
+    rejection_sampling: Any | None = None,
+    importance_sampling_level: str = "token",
+    temperature: float = 1.0,
+    loss_multiplier: float = 1.0,
+    host_loss_mask: torch.Tensor | None = None,
+    backward: str = "carry",
+) -> tuple[torch.Tensor, dict]:
+    """``compute_logprobs_and_loss`` (fsdp_engine.py:1977-2046) one step earlier in the model: from the final hidden
+    states ``[T_pad, H]`` (a leading batch dimension of 1 is dropped, as ``outputs.logits.squeeze(0)``,
+    fsdp_engine.py:747) and the lm_head weight ``[V, H]``, so that the ``[T_pad, V]`` logits are never written.
+
+    Same contract otherwise: labels are the packed ``input_ids`` rolled by one over the whole tensor
+    (``rolled_labels``), the last ``pad_length`` rows are batch padding (they get no gradient and no outputs), the loss
+    is scaled by ``local_weight / total_loss_weight * loss_multiplier`` with ``local_weight =
+    loss_mask.count_nonzero()`` (actor.py:363), and a micro-batch without any unmasked token returns a zero that keeps
+    the graph to ``hidden`` and ``weight`` alive (fsdp_engine.py:1987-1989).  The stat dict is that of
+    ``fused_logprobs_ppo_loss`` (``logprobs``, ``entropy``, ``vocab_min_logits``, ``vocab_max_logits`` and the entries
+    of ``ppo_actor_loss_fn``), i.e. what ``grpo_loss_fn`` is given and returns.
+
+    ``host_loss_mask``: the host (CPU) copy of ``mb_input["loss_mask"]`` that the data loader still holds.  With it
+    nothing is read back from the device: the weight of the micro-batch and the number of tokens with a gradient per
+    chunk of ``lm_head_chunk_tokens()`` tokens, which size the gradient GEMMs, are counted on the host.  Rejection
+    sampling can only shrink the mask on the device; the counts are then upper bounds, and the rows beyond the true
+    count are cleared on the device.  Without it the call reads them from the device, as the reference's
+    ``local_weight == 0`` does.
+    """
+    if hidden.ndim == 3 and hidden.shape[0] == 1:
+        hidden = hidden.squeeze(0)
+    if hidden.ndim != 2 or hidden.shape[0] - pad_length != mb_input["loss_mask"].shape[0]:
+        raise ValueError(
+            f"hidden {tuple(hidden.shape)} with pad_length {pad_length} does not fit loss_mask "
+            f"{tuple(mb_input['loss_mask'].shape)}"
+        )
+    loss_mask = mb_input["loss_mask"].bool()
+    kept = None
+    if host_loss_mask is not None:
+        host = host_loss_mask.reshape(-1).ne(0)
+        if host.is_cuda or host.shape[0] != loss_mask.shape[0]:
+            raise ValueError("host_loss_mask must be the CPU copy of mb_input['loss_mask']")
+        local_weight: Any = int(host.sum())
+        chunk = lm_head_chunk_tokens()
+        kept = [int(host[i:i + chunk].sum()) for i in range(0, hidden.shape[0], chunk)]
+    else:
+        local_weight = loss_mask.count_nonzero()
+    if local_weight == 0:
+        return hidden.mean() * 0.0 + weight.mean() * 0.0, {}
+    old_logp = mb_input["logprobs"]
+    prox_logp = mb_input.get("prox_logp")
+    if prox_logp is None:
+        raise ValueError("prox_logp is None: only the recomputed proximal log-probs are supported here")
+    scale = local_weight / total_loss_weight * loss_multiplier
+    return fused_lm_head_ppo_loss(
+        hidden, weight, rolled_labels(model_inputs), prox_logp, old_logp, mb_input["advantages"], eps_clip=eps_clip,
+        loss_mask=loss_mask, eps_clip_higher=eps_clip_higher, c_clip=c_clip, rejection_sampling=rejection_sampling,
+        importance_sampling_level=importance_sampling_level, cu_seqlens=mb_input.get("cu_seqlens"),
+        temperature=temperature, loss_scale=scale, kept_per_chunk=kept, backward=backward,
+    )
 
 
 def compute_advantages(

@@ -8,7 +8,7 @@ import torch
 
 import areal_amd
 import oracle
-from areal_amd import _native
+from areal_amd import _native, engine_glue
 from areal_amd import RejectionSamplingConfig
 from helpers import assert_same_magnitude, assert_within, cosine
 
@@ -620,3 +620,66 @@ def test_step_replays_from_a_hip_graph(device, backward):
         torch.cuda.synchronize()
         assert torch.equal(got[0], e_loss.detach()) and torch.equal(got[1], e_stat["logprobs"])
         assert torch.equal(got[2], h2.grad) and torch.equal(got[3], w2.grad)
+
+
+@pytest.mark.parametrize("with_host_mask", [True, False])
+@pytest.mark.parametrize("with_rs", [False, True])
+def test_engine_contract_of_the_lm_head_step(device, with_host_mask, with_rs):
+    """``engine_glue.compute_lm_head_and_loss`` against the reference's engine contract (fsdp_engine.py:1977-2046) on
+    ``hidden @ W.T``: labels rolled over the sequence borders, the pad rows trimmed and without gradient, the loss
+    scaled by local / total weight, the vocabulary extrema handed on, the zero-weight micro-batch."""
+    lengths, pad = [5, 3, 4], 4
+    n = sum(lengths)
+    T, H, V = n + pad, 64, 1097
+    g = torch.Generator().manual_seed(3)
+    input_ids = torch.randint(0, V, (1, T), generator=g)
+    labels = torch.cat([input_ids[0, 1:], input_ids[0, :1]])
+    hidden = torch.randn(1, T, H, generator=g).bfloat16()
+    weight = (0.3 * torch.randn(V, H, generator=g)).bfloat16()
+    logits = oracle.lmhead_logits(hidden[0], weight)
+    ref = oracle.logprobs(logits, labels)[:n]
+    mb = dict(
+        loss_mask=(torch.rand(n, generator=g) < 0.6), logprobs=ref + 0.3 * torch.randn(n, generator=g),
+        prox_logp=ref + 0.05 * torch.randn(n, generator=g), advantages=torch.randn(n, generator=g),
+        cu_seqlens=torch.tensor([0, 5, 8, 12], dtype=torch.int32),
+    )
+    rs = RejectionSamplingConfig(level="token", action="mask", metric="ratio", upper=1.2) if with_rs else None
+    mb_d = {k: v.to(device) for k, v in mb.items()}
+    total_w = torch.tensor(40.0, device=device)
+    scale = float(mb["loss_mask"].sum()) / 40.0 * 0.5
+    h = hidden.to(device).requires_grad_(True)
+    w = weight.to(device).requires_grad_(True)
+    loss, stat = engine_glue.compute_lm_head_and_loss(
+        h, w, {"input_ids": input_ids.to(device)}, mb_d, pad, total_w, eps_clip=0.2, c_clip=3.0, rejection_sampling=rs,
+        loss_multiplier=0.5, host_loss_mask=mb["loss_mask"] if with_host_mask else None)
+    loss.backward()
+    o_loss, o_stat, o_lp, o_ent, o_dh, o_dw = _oracle_step(
+        hidden[0], weight, labels, mb["prox_logp"], mb["logprobs"], mb["advantages"], mb["loss_mask"], 1.0, scale,
+        eps_clip=0.2, c_clip=3.0, rejection_sampling_cfg=rs, cu_seqlens=mb["cu_seqlens"])
+    assert float(loss.detach()) == pytest.approx(o_loss, rel=1e-3)
+    assert stat["logprobs"].shape == (n,) and stat["entropy"].shape == (n,)
+    assert_within(stat["logprobs"], o_lp[:n], 2e-3, "log-prob")
+    assert_within(stat["entropy"], o_ent[:n], 2e-3, "entropy")
+    assert float((stat["vocab_max_logits"].cpu() - logits[:n].max(-1).values).abs().max()) <= 1e-5 * float(logits.abs().max())
+    assert float((stat["vocab_min_logits"].cpu() - logits[:n].min(-1).values).abs().max()) <= 1e-5 * float(logits.abs().max())
+    assert h.grad.shape == hidden.shape
+    assert cosine(h.grad[0].cpu().float(), o_dh) > 0.9999 and cosine(w.grad.cpu().float(), o_dw) > 0.9999
+    assert_same_magnitude(h.grad[0], o_dh, what="d(hidden)")
+    assert_same_magnitude(w.grad, o_dw, what="d(W)")
+    assert float(h.grad[0, n:].float().abs().max()) == 0.0            # batch padding gets no gradient
+    assert torch.equal(stat["clip_mask"].cpu(), o_stat["clip_mask"])
+    if with_rs:
+        assert float(stat["filtered_fraction"]) == pytest.approx(float(o_stat["filtered_fraction"]), abs=1e-6)
+    # a micro-batch without any unmasked token keeps the graph to both inputs alive and contributes nothing
+    mb_d["loss_mask"] = torch.zeros(n, dtype=torch.bool, device=device)
+    h = hidden.to(device).requires_grad_(True)
+    w = weight.to(device).requires_grad_(True)
+    loss, stat = engine_glue.compute_lm_head_and_loss(
+        h, w, {"input_ids": input_ids.to(device)}, mb_d, pad, total_w, eps_clip=0.2,
+        host_loss_mask=torch.zeros(n, dtype=torch.bool) if with_host_mask else None)
+    loss.backward()
+    assert stat == {} and float(loss.detach()) == 0.0
+    assert float(h.grad.float().abs().max()) == 0.0 and float(w.grad.float().abs().max()) == 0.0
+    # forward-only pass of the same micro-batch
+    lp = engine_glue.compute_lm_head_logprobs(hidden.to(device), weight.to(device), {"input_ids": input_ids.to(device)})
+    assert_within(lp[:n], o_lp[:n], 2e-3, "log-prob of the forward-only pass")
