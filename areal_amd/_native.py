@@ -120,6 +120,7 @@ SIGNATURES = {
     "aa_masked_moments": (_i, [C.POINTER(C.c_void_p), _i, _p, _i64, _p, _p]),
     "aa_segment_copy": (_i, [_p, _p, _i64, _p, _p, _p, _i64, _i64, _p]),
     "aa_copy_bytes": (_i, [_p, _p, _i64, _p]),
+    "aa_mfma_only_loop": (_i, [_i, _i, _i, _i, _p, _p]),
 }
 
 _lib = None

@@ -37,7 +37,11 @@ Prints ONE JSON line.  Besides the whole-step throughput it carries
 and, in the default run only (every GPU timing is taken before the first CPU baseline starts):
   configs1_cut_to_32k_tokens  the cfg1 sequences cut at 32 768 tokens;
   logits_config0              the cfg0 workload with its own roofline, and the plain copy kernel on the same buffers;
-  fused_lm_head               the same figures for the cfg2 workload, so that one run reports both paths.
+  fused_lm_head               the same figures for the cfg2 workload, so that one run reports both paths;
+  fused_lm_head_cfg3, _cfg4   the cfg3 and cfg4 workloads (GPU only: three timed steps each, their own roofline).
+
+``--workload mfma`` runs the MFMA-only loop (aa_mfma_only_loop: no LDS, no memory traffic), the measured ceiling that
+the fused lm_head figures are also quoted against (``roofline.frac_of_mfma_only_loop``).
 """
 from __future__ import annotations
 
@@ -59,6 +63,7 @@ METRIC = "tokens/sec for logprob+entropy+PPO loss fwd+bwd; % HBM / % MFMA peak" 
 LOGITS_WORKLOADS = ("cfg0", "cfg1", "cfg1-32k")
 FUSED_WORKLOADS = ("cfg2", "cfg3", "cfg4")
 ADV_WORKLOADS = ("adv", "aux")
+MFMA_WORKLOADS = ("mfma",)
 
 
 def parse_args():
@@ -66,7 +71,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="cfg1", choices=LOGITS_WORKLOADS + FUSED_WORKLOADS + ADV_WORKLOADS)
+    ap.add_argument("--workload", default="cfg1", choices=LOGITS_WORKLOADS + FUSED_WORKLOADS + ADV_WORKLOADS + MFMA_WORKLOADS)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--cpu-tokens", type=int, default=6144,
                     help="token sample of the CPU baseline (0 = skip); fused lm_head workloads use at most 384")
@@ -368,6 +373,10 @@ def bench_logits(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: 
         # fp32 logits: 1.092 x, the part of a row that does not fit on the chip is fetched a second time
         # (profiles/k_fused_f32_hold_cfg1-32k_hbm_traffic.md)
         traffic=alg_bytes * (1.092 if f32 else 1.001), avg_kernel_ms=k_ms, min_kernel_ms=k_min_ms,
+        traffic_source=("profiles/k_fused_f32_hold_cfg1-32k_hbm_traffic.md" if f32 else
+                        "profiles/k_fused_regs_cfg1-32k_hbm_traffic.md") +
+                       ": counter bytes / algorithmic bytes measured on the cfg1-32k workload, applied to this one's "
+                       "algorithmic bytes (not a reading of this run)",
         algorithmic_bytes_per_launch=alg_bytes,
     )
     out = dict(
@@ -445,11 +454,48 @@ BACKWARD_MODE = 1  # aa_lmhead_backward_mode: 1 carry, 0 recompute (set from --l
 NO_FORWARD_OF_MASKED = False  # set from --no-forward-of-masked
 MODE_NAMES = {1: "carry", 0: "recompute"}
 
-# HBM bytes per step of aa_lmhead_ppo_fused at configs[2], all its kernels together: rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE (one run each) summed over the kernels of one step, each scaled by what the same counter reads for the
-# plain copy kernel of known size (profiles/lmhead_step_cfg2_hbm_traffic.md).  The counters sit behind the L2 of each
-# XCD: what the memory-side cache serves is in these figures too.  Other workloads: not measured.
-LMHEAD_MEASURED_HBM_BYTES = {("cfg2", "carry"): 82.1e9, ("cfg2", "recompute"): 109.2e9}
+# HBM bytes per step of aa_lmhead_ppo_fused, all its kernels together: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (one
+# run each) summed over the kernels of one step, each scaled by what the same counter reads for the plain copy kernel of
+# known size.  The counters sit behind the L2 of each XCD: what the memory-side cache serves is in these figures too.
+# Transcribed from the profile summaries named beside them, not read in this run; other workloads: not measured.
+LMHEAD_MEASURED_HBM_BYTES = {
+    ("cfg2", "carry"): (82.1e9, "profiles/lmhead_step_cfg2_hbm_traffic.md"),
+    ("cfg2", "recompute"): (109.2e9, "profiles/lmhead_step_cfg2_hbm_traffic.md"),
+}
+
+
+def lmhead_measured_bytes(workload: str, mode: str):
+    return LMHEAD_MEASURED_HBM_BYTES.get((workload, mode), (None, None))
+
+
+def time_mfma_only_loop(dev, reps: int = 4, target_ms: float = 40.0):
+    """The MFMA-only loop (aa_mfma_only_loop) in both instruction forms, on random and on zero operands: TFLOP/s of
+    launches of about ``target_ms`` each, HIP events on the launch stream, one workgroup per compute unit."""
+    import torch
+
+    from areal_amd import _native as N
+    from areal_amd import functional as F
+
+    lib = N.load()
+    wgs = torch.cuda.get_device_properties(dev).multi_processor_count
+    out = torch.empty(wgs * 256, dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream(dev)
+    st = C.c_void_p(stream.cuda_stream)
+    res = {}
+    for form, name, flops_per_iter in ((0, "v_mfma_f32_32x32x16_bf16", 2097152.0), (1, "v_mfma_f32_16x16x32_bf16", 4194304.0)):
+        for random_operands in (1, 0):
+            # iterations for the target duration at 2 PFLOP/s
+            iters = int(target_ms * 1e-3 * 2.0e15 / (wgs * flops_per_iter))
+
+            def launch():
+                N.check(lib.aa_mfma_only_loop(form, random_operands, wgs, iters, F._ptr(out), st), "aa_mfma_only_loop")
+
+            avg_ms, min_ms = time_events(launch, reps, stream)
+            res[f"{name}, {'random' if random_operands else 'zero'} operands"] = dict(
+                avg_ms=avg_ms, min_ms=min_ms, workgroups=wgs, iterations=iters,
+                tflops=wgs * flops_per_iter * iters / (avg_ms * 1e-3) / 1e12)
+    res["best_on_random_operands_tflops"] = max(v["tflops"] for k, v in res.items() if k.endswith("random operands"))
+    return res
 
 
 def lmhead_compulsory_bytes(T: int, kept: int, H: int, V: int, mode: str, chunk: int) -> dict:
@@ -702,7 +748,8 @@ def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: i
         modes[name] = dict(avg_call_ms=c_ms, min_call_ms=c_min,
                            executed_flops=(2.0 * T + (4.0 if mode == 1 else 6.0) * kept_tokens) * V * H,
                            compulsory_hbm_bytes=lmhead_compulsory_bytes(T, kept_tokens, H, V, name, chunk),
-                           measured_hbm_bytes=LMHEAD_MEASURED_HBM_BYTES.get((workload, name)))
+                           measured_hbm_bytes=lmhead_measured_bytes(workload, name)[0],
+                           measured_hbm_bytes_source=lmhead_measured_bytes(workload, name)[1])
     f_ms, b_ms, op_kept = time_lmhead_op(case, 5)
     # Flops the step needs: logits of every token (2 T V H) and the two gradient GEMMs over the tokens that have a
     # gradient (4 T_kept V H).  The reference's autograd runs them over all T tokens: 6 T V H.
@@ -718,7 +765,8 @@ def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: i
                ("" if mode_name == "carry" else "k_lmhead_tiles again for the tokens with a gradient, ") +
                "k_gemm_store twice (d_hidden, d_weight; in carry mode they apply the per-token gradient factor)",
         achieved=achieved, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s", frac=achieved / MFMA_BF16_PEAK_TFLOPS,
-        traffic=LMHEAD_MEASURED_HBM_BYTES.get((workload, mode_name)),
+        traffic=lmhead_measured_bytes(workload, mode_name)[0],
+        traffic_source=lmhead_measured_bytes(workload, mode_name)[1],
         timed="HIP events on the launch stream around each of the steps that ms_per_step is the wall-clock mean of",
         avg_step_ms=ev_avg, min_step_ms=ev_ms[0], max_step_ms=ev_ms[-1],
         needed_flops_per_step=needed_flops, flops_per_step_6TVH=6.0 * T * V * H, tokens_with_gradient=kept_tokens,
@@ -728,6 +776,10 @@ def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: i
         standalone_op=dict(fwd_ms=f_ms, bwd_ms=b_ms, fwd_tflops=2.0 * T * V * H / (f_ms * 1e-3) / 1e12,
                            bwd_executed_tflops=6.0 * op_kept * V * H / (b_ms * 1e-3) / 1e12),
     )
+    # the measured ceiling of the matrix cores in this process: a loop of MFMAs only (no LDS, no memory traffic)
+    mfma_only = time_mfma_only_loop(dev)
+    roofline["mfma_only_loop"] = mfma_only
+    roofline["frac_of_mfma_only_loop"] = achieved / mfma_only["best_on_random_operands_tflops"]
     out = dict(
         metric=METRIC, value=T / (ms_per_step * 1e-3), unit="tokens/s",
         n_gpus=1, steps=steps, warmup=warmup, ms_per_step=ms_per_step, higher_is_better=True,
@@ -751,6 +803,70 @@ def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: i
                                        launches=args.copy_launches)
     sample = fused_gpu_sample(case, kw, cfg, cpu_tokens) if cpu_tokens > 0 else None
     return out, sample
+
+def bench_fused_leg(args, dev, workload: str, steps: int, warmup: int):
+    """A fused lm_head workload, GPU only: ``warmup`` + ``steps`` steps of fused_lm_head_ppo_loss + backward through the
+    Python API, HIP events on the launch stream around every timed step, roofline on the flops the step needs."""
+    import torch
+
+    case, desc = build_fused_case(workload, args.seed, dev)
+    kw, cfg = ppo_kwargs(case)
+    T, H = case.hidden.shape
+    V = case.weight.shape[0]
+    case.hidden.requires_grad_(True)
+    case.weight.requires_grad_(True)
+    run_fused_steps(case, warmup, kw, cfg)
+    torch.cuda.synchronize()
+    events = []
+    t0 = time.perf_counter()
+    loss = run_fused_steps(case, steps, kw, cfg, events)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / steps * 1e3
+    assert bool(torch.isfinite(loss)), "loss is not finite"
+    assert bool(torch.isfinite(case.hidden.grad.float()).all()) and bool(torch.isfinite(case.weight.grad.float()).all())
+    ev_ms = sorted(a.elapsed_time(b) for a, b in events)
+    ev_avg = sum(ev_ms) / len(ev_ms)
+    with torch.no_grad():
+        from areal_amd import functional as F
+
+        m8 = F._mask_u8(case.loss_mask)
+        if cfg is not None and cfg.action == "mask":
+            prox, old = F._f32(case.prox_logp), F._f32(case.old_logp)
+            m8, _, _ = F._rejection_sampling_device(prox, old, m8, m8.shape, case.cu_seqlens, cfg)
+        kept_tokens = int(m8.ne(0).sum()) if not DENSE_BACKWARD else T
+    needed_flops = 2.0 * T * V * H + 4.0 * kept_tokens * V * H
+    achieved = needed_flops / (ev_avg * 1e-3) / 1e12
+    mode_name = MODE_NAMES[BACKWARD_MODE]
+    return dict(
+        value=T / (ms_per_step * 1e-3), unit="tokens/s", steps=steps, warmup=warmup, ms_per_step=ms_per_step,
+        config=dict(workload=f"{case.name}: {desc}", tokens=T, hidden=H, vocab=V,
+                    sequences=int(case.cu_seqlens.numel() - 1), accumulate="f32",
+                    path=f"lm_head + PPO loss step, fwd + bwd (backward={mode_name}); the forward writes no logits"),
+        roofline=dict(
+            bound="mfma", kernel="every kernel of one fused_lm_head_ppo_loss(...) + backward() step",
+            achieved=achieved, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s", frac=achieved / MFMA_BF16_PEAK_TFLOPS,
+            traffic=lmhead_measured_bytes(workload, mode_name)[0],
+            traffic_source=lmhead_measured_bytes(workload, mode_name)[1],
+            timed="HIP events on the launch stream around each of the timed steps",
+            avg_step_ms=ev_avg, min_step_ms=ev_ms[0], max_step_ms=ev_ms[-1], needed_flops_per_step=needed_flops,
+            flops_per_step_6TVH=6.0 * T * V * H, tokens_with_gradient=kept_tokens, backward_mode=mode_name),
+    )
+
+
+def bench_mfma(args, dev):
+    res = time_mfma_only_loop(dev, reps=max(args.steps, 6), target_ms=50.0)
+    best = res["best_on_random_operands_tflops"]
+    return dict(
+        metric="TFLOP/s of a loop of bf16 MFMAs only (no LDS, no memory traffic): the measured matrix-core ceiling",
+        value=best, unit="TFLOP/s", n_gpus=1, steps=max(args.steps, 6), warmup=2, higher_is_better=True, dtype="bf16",
+        data="synthetic", vs_baseline=None, scaling="weak",
+        config=dict(workload="aa_mfma_only_loop: 4 waves per workgroup, one workgroup per compute unit, operands in "
+                             "registers"),
+        roofline=dict(bound="mfma", kernel="k_mfma_16x16x32 / k_mfma_32x32x16", achieved=best,
+                      peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s", frac=best / MFMA_BF16_PEAK_TFLOPS, traffic=0.0),
+        forms=res,
+    )
+
 
 # ----------------------------------------------------------------------------------------------------------------
 # advantage pipeline
@@ -971,7 +1087,9 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    if args.workload == "aux":
+    if args.workload in MFMA_WORKLOADS:
+        out = bench_mfma(args, dev)
+    elif args.workload == "aux":
         out = bench_aux(args, dev)
     elif args.workload in ADV_WORKLOADS:
         out = bench_adv(args, dev)
@@ -992,6 +1110,10 @@ def main():
             torch.cuda.empty_cache()
             extra, fused_sample = bench_fused(args, dev, "cfg2", args.steps, args.warmup, min(args.cpu_tokens, 384))
             torch.cuda.empty_cache()
+            # the two larger fused configurations, GPU only
+            for wl in ("cfg3", "cfg4"):
+                out[f"fused_lm_head_{wl}"] = bench_fused_leg(args, dev, wl, 3, 1)
+                torch.cuda.empty_cache()
         finish_with_cpu_phase(out, sample, logits_cpu_phase, args.cpu_iters)
         if extra is not None:
             finish_with_cpu_phase(extra, fused_sample, fused_cpu_phase, args.cpu_iters)
@@ -1008,6 +1130,9 @@ def main():
         roof = part.get("roofline")
         if roof:
             fractions["pct_hbm_peak" if roof["bound"] == "hbm" else "pct_mfma_peak"] = 100.0 * roof["frac"]
+    for wl in ("cfg3", "cfg4"):
+        if f"fused_lm_head_{wl}" in out:
+            fractions[f"pct_mfma_peak_{wl}"] = 100.0 * out[f"fused_lm_head_{wl}"]["roofline"]["frac"]
     out["pct_of_peak"] = fractions
     print(json.dumps(out))
 

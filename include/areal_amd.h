@@ -813,6 +813,18 @@ int aa_segment_copy(const void* src, void* dst, int64_t row_bytes,
  * plain copy the HBM counters of the other kernels are calibrated against. */
 int aa_copy_bytes(const void* src, void* dst, int64_t nbytes, void* stream);
 
+/* A loop of nothing but bf16 MFMAs on operands that stay in registers (no LDS,
+ * no memory traffic): what the matrix cores of this chip sustain at its power
+ * limit, the measured ceiling beside the MFMA-bound kernels.  form 0:
+ * v_mfma_f32_32x32x16_bf16, 16 per wave and iteration; form 1:
+ * v_mfma_f32_16x16x32_bf16, 64 per wave and iteration; 4 waves per workgroup,
+ * so an iteration is 2 097 152 (form 0) or 4 194 304 (form 1) flops per
+ * workgroup.  random_operands: random signs and mantissas (as activations
+ * are) or zeros.  out [workgroups * 256] receives a checksum per lane.  No
+ * counterpart in the reference; not on any product path. */
+int aa_mfma_only_loop(int form, int random_operands, int workgroups, int iters,
+                      float* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
