@@ -294,6 +294,94 @@ def test_full_size_step_agrees_with_unfused_path(device, backward):
         assert float((a - b).abs().max()) <= float(b.abs().max()) * 2.0 ** -6
 
 
+def _full_size_case(name, device):
+    """configs[3] / configs[4] as the benchmark builds them, with old / prox log-probs spread widely enough (0.6 nats)
+    that the dual clip and the importance-weight cap both bind on a few percent of the tokens."""
+    from areal_amd import synth
+
+    case = {"cfg3": synth.config3, "cfg4": synth.config4}[name](device, seed=0)
+    with torch.no_grad():
+        ref, _ = areal_amd.lm_head_logprobs_entropy(case.hidden, case.weight, case.labels, case.temperature)
+    synth.attach_old_and_prox(case, ref, 0.6, 9)
+    kw = dict(case.ppo)
+    rs = kw.pop("rejection_sampling", None)
+    kw.setdefault("c_clip", 3.0)                       # configs[4] names no dual clip: switch it on for the test
+    cfg = RejectionSamplingConfig(**(rs or dict(level="token", action="mask", metric="ratio", upper=5.0)))
+    return case, kw, cfg
+
+
+@pytest.mark.parametrize("backward", ["carry", "recompute"])
+@pytest.mark.parametrize("name", ["cfg4", "cfg3"])
+def test_full_size_step_against_oracle_slices(device, name, backward):
+    """The whole step at the size of configs[3] (T = 262144: 16 token chunks, d(W) accumulated in fp32 chunk by chunk)
+    and configs[4] (V = 262144, H = 5376, temperature 0.7, two chunks).  The oracle cannot run these whole.  A token's
+    log-prob, entropy, loss terms and d(hidden) row depend on that token and on the number of unmasked tokens only, so
+    48 tokens (first, middle, last) are held to the oracle; d(W) is held to it with only those tokens switched on, and
+    the full d(W) to the sum of that and of the step on all other tokens (the loss is additive over tokens once the
+    common 1/N is kept)."""
+    case, kw, cfg = _full_size_case(name, device)
+    T, H = case.hidden.shape
+    V = case.weight.shape[0]
+    print(f"full-size step {name} {backward}: T={T} H={H} V={V}", flush=True)
+    idx = torch.cat([torch.arange(0, 16), torch.arange(T // 2 - 8, T // 2 + 8), torch.arange(T - 16, T)])
+    idx_d = idx.to(device)
+    n_full = int(case.loss_mask.sum())
+    in_slice = torch.zeros(T, dtype=torch.bool, device=device)
+    in_slice[idx_d] = True
+    slice_mask = case.loss_mask.bool() & in_slice
+    rest_mask = case.loss_mask.bool() & ~in_slice
+    n_slice = int(slice_mask.sum())
+    assert 8 <= n_slice < 48            # the slice holds masked and unmasked tokens
+
+    def step(mask, scale):
+        h = case.hidden.detach().requires_grad_(True)
+        w = case.weight.detach().requires_grad_(True)
+        loss, stat = areal_amd.fused_lm_head_ppo_loss(
+            h, w, case.labels, case.prox_logp, case.old_logp, case.advantages, loss_mask=mask, rejection_sampling=cfg,
+            cu_seqlens=case.cu_seqlens, temperature=case.temperature, loss_scale=scale, backward=backward, **kw)
+        loss.backward()
+        return loss.detach(), stat, h.grad, w.grad
+
+    loss, stat, dh, dw = step(case.loss_mask, 1.0)
+    assert bool(torch.isfinite(loss)) and bool(torch.isfinite(dw.float()).all())
+    assert int(stat["dual_clip_mask"].sum()) > 100 and float(stat["filtered_fraction"]) > 0.005   # both bind
+    # oracle on the slice, with the full batch's 1/N
+    take = lambda t: t[idx_d].cpu()
+    h_o = case.hidden[idx_d].cpu().float().requires_grad_(True)
+    w_o = case.weight.cpu().float().requires_grad_(True)
+    o_lp, o_ent = oracle.logprobs_entropy(oracle.lmhead_logits(h_o, w_o), take(case.labels), case.temperature)
+    o_loss, o_stat = oracle.ppo_actor_loss(
+        o_lp, take(case.prox_logp), take(case.old_logp), take(case.advantages), loss_mask=take(case.loss_mask).bool(),
+        rejection_sampling_cfg=cfg, cu_seqlens=torch.tensor([0, idx.numel()], dtype=torch.int32), **kw)
+    (o_loss * n_slice / n_full).backward()
+    assert_within(stat["logprobs"][idx_d], o_lp.detach(), 2e-3, "log-prob")       # stated tolerances
+    assert_within(stat["entropy"][idx_d], o_ent.detach(), 2e-3, "entropy")
+    on = take(case.loss_mask).bool()
+    assert_within(stat["loss"][idx_d].cpu()[on], o_stat["loss"][on], 2e-3, "per-token loss")
+    assert int((stat["clip_mask"][idx_d].cpu() != o_stat["clip_mask"]).sum()) <= 1
+    assert cosine(dh[idx_d].cpu().float(), h_o.grad) > 0.9999
+    assert_same_magnitude(dh[idx_d], h_o.grad, what="d(hidden) rows of the slice")
+    # tokens without a mask, and tokens the cap dropped, get a d(hidden) row of exactly zero
+    dead = ~(case.loss_mask.bool() & stat["behave_mask"].bool())
+    assert float(dh[dead].float().abs().sum()) == 0.0
+    # bit-equal repeat
+    loss2, _, dh2, dw2 = step(case.loss_mask, 1.0)
+    assert torch.equal(loss, loss2) and torch.equal(dh, dh2) and torch.equal(dw, dw2)
+    del dh2, dw2
+    # d(W) with only the slice's tokens switched on (every other chunk has no token with a gradient) against the oracle
+    _, _, dh_s, dw_s = step(slice_mask, n_slice / n_full)
+    a, b = dw_s.double().reshape(-1), w_o.grad.to(device).double().reshape(-1)
+    assert float(a @ b / (a.norm() * b.norm())) > 0.9999
+    assert abs(float(a.norm() / b.norm()) - 1.0) < 1e-2
+    assert cosine(dh_s[idx_d].cpu().float(), dh[idx_d].cpu().float()) > 0.99999   # the rows of the full step (1/N rounds differently)
+    del a, b, w_o, h_o
+    # ... and the full d(W) is that plus d(W) of all other tokens
+    _, _, _, dw_r = step(rest_mask, (n_full - n_slice) / n_full)
+    a, b = (dw_s.float() + dw_r.float()).double().reshape(-1), dw.double().reshape(-1)
+    assert float(a @ b / (a.norm() * b.norm())) > 0.99999
+    assert abs(float(a.norm() / b.norm()) - 1.0) < 2e-3
+
+
 def test_padding_only_chunk_and_no_active_token(device):
     g = torch.Generator().manual_seed(0)
     T_pad, T, H, V = CHUNK + 300, CHUNK, 64, 640           # the second token chunk is batch padding only
