@@ -251,17 +251,37 @@ __global__ __launch_bounds__(NT) void k_logits_fwd(const void* __restrict__ logi
   }
 }
 
+// Pointer types of an input / output pair that may be ONE array (the gradient written over the logits, ALIAS): the
+// restrict qualifier, which tells the compiler that the two never overlap, is there only when they are known to be
+// distinct.  The kernels that take such a pair are instantiated both ways and the entry points choose.
+template <bool ALIAS, typename T>
+struct InPtr {
+  typedef const T* __restrict__ type;
+};
+template <typename T>
+struct InPtr<true, T> {
+  typedef const T* type;
+};
+template <bool ALIAS, typename T>
+struct OutPtr {
+  typedef T* __restrict__ type;
+};
+template <typename T>
+struct OutPtr<true, T> {
+  typedef T* type;
+};
+
 // -----------------------------------------------------------------------------
 // Backward: dlogits from g_logp / g_entropy and the saved row statistics.
 // -----------------------------------------------------------------------------
-template <int DT, int NT>
-__global__ __launch_bounds__(NT) void k_logits_bwd(const void* __restrict__ logits, int V, int64_t stride,
+template <int DT, int NT, bool ALIAS>
+__global__ __launch_bounds__(NT) void k_logits_bwd(typename InPtr<ALIAS, void>::type logits, int V, int64_t stride,
                                                    const int64_t* __restrict__ labels, float inv_t, int vec_ok,
                                                    const float* __restrict__ row_lse,
                                                    const float* __restrict__ row_ez,
                                                    const float* __restrict__ g_logp,
                                                    const float* __restrict__ g_entropy, int64_t T_active,
-                                                   void* __restrict__ dlogits) {
+                                                   typename OutPtr<ALIAS, void>::type dlogits) {
   const int64_t t = blockIdx.x;
   const void* row = row_ptr(logits, t, stride, Elem<DT>::kBytes);
   void* out = (void*)row_ptr(dlogits, t, stride, Elem<DT>::kBytes);
@@ -406,10 +426,11 @@ __device__ __forceinline__ float fused_token_tail(const FusedTokenArgs& a, int64
 constexpr int64_t kWalkRowBytes = 256 * 1024;  // rows at least this long are walked by kWalkGroups workgroups
 constexpr int kWalkGroups = 512;               // two per compute unit
 
-template <int DT, int NT>
-__global__ __launch_bounds__(NT) void k_fused_generic(const void* __restrict__ logits, int64_t T_rows, int V,
+template <int DT, int NT, bool ALIAS>
+__global__ __launch_bounds__(NT) void k_fused_generic(typename InPtr<ALIAS, void>::type logits, int64_t T_rows, int V,
                                                       int64_t stride, const int64_t* __restrict__ labels, float inv_t,
-                                                      int vec_ok, FusedTokenArgs a, void* __restrict__ dlogits) {
+                                                      int vec_ok, FusedTokenArgs a,
+                                                      typename OutPtr<ALIAS, void>::type dlogits) {
   __shared__ float smem[(NT / kWave) * 5];
   const float c = kLog2e * inv_t;
   float fn, gscale;
@@ -453,9 +474,11 @@ constexpr int kHoldReg = 10;                        // 10 x 8192 floats in regis
 constexpr int kHoldLds = 4;                         // 4 x 8192 floats in LDS (128 KB)
 constexpr int kHoldChunk = 8 * 1024;                // floats per chunk: 8 per thread
 
-__global__ __launch_bounds__(1024) void k_fused_f32_hold(const float* __restrict__ logits, int64_t T_rows, int V,
+template <bool ALIAS>
+__global__ __launch_bounds__(1024) void k_fused_f32_hold(typename InPtr<ALIAS, float>::type logits, int64_t T_rows, int V,
                                                          int64_t stride, const int64_t* __restrict__ labels,
-                                                         float inv_t, FusedTokenArgs a, float* __restrict__ dlogits) {
+                                                         float inv_t, FusedTokenArgs a,
+                                                         typename OutPtr<ALIAS, float>::type dlogits) {
   __shared__ float smem[16 * 5];
   __shared__ float4 held[kHoldLds * 2 * 1024];      // [chunk][half][thread]: consecutive lanes, consecutive 16 bytes
   const int tid = threadIdx.x;
@@ -702,15 +725,15 @@ constexpr int kTwoPerUnitChunks = 7;  // rows this short run two workgroups per 
 // With EXT the row continues past the NCH register chunks: n_lds chunks in dynamic LDS, then the tail chunks.
 // Up to kTwoPerUnitChunks chunks the kernel is compiled for 8 waves per SIMD, so that two workgroups fit on a
 // compute unit: without that request the scalar registers alone (106 per wave: 7 waves) keep the second one out.
-template <int DT, int NCH, bool EXT = false>
+template <int DT, int NCH, bool EXT, bool ALIAS>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu((!EXT && NCH <= kTwoPerUnitChunks) ? 8 : 1)))
-void k_fused_regs(const uint4* __restrict__ logits, int V, int64_t stride_vec,
+void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stride_vec,
                                                      const int64_t* __restrict__ labels, float inv_t,
                                                      const float* __restrict__ in_prox,
                                                      const float* __restrict__ in_adv,
                                                      const uint32_t* __restrict__ in_mask32, unsigned mask_mis,
                                                      const float* __restrict__ in_bw, FusedTokenArgs a,
-                                                     uint4* __restrict__ dlogits, int64_t T, int32_t* work,
+                                                     typename OutPtr<ALIAS, uint4>::type dlogits, int64_t T, int32_t* work,
                                                      int n_lds) {
   constexpr int NT = 1024;
   constexpr int kChunkBytes = NT * 16;
@@ -1029,9 +1052,14 @@ static void launch_regs(const void* logits, int64_t T, int V, int64_t stride, co
   const int64_t resident = (int64_t)persistent_workgroups() * (NCH <= kTwoPerUnitChunks ? 2 : 1);
   const int64_t wgs = T < resident ? T : resident;
   const uintptr_t mask_addr = (uintptr_t)a.mask_eff;
-  hipLaunchKernelGGL((k_fused_regs<DT, NCH>), dim3((unsigned)wgs), dim3(1024), 0, st, (const uint4*)logits, V,
-                     stride >> 3, labels, inv_t, a.prox_logp, a.adv, (const uint32_t*)(mask_addr & ~(uintptr_t)3),
-                     (unsigned)(mask_addr & 3), a.behave_w, a, (uint4*)dlogits, T, work, 0);
+  if (dlogits == logits)
+    hipLaunchKernelGGL((k_fused_regs<DT, NCH, false, true>), dim3((unsigned)wgs), dim3(1024), 0, st, (const uint4*)logits, V,
+                       stride >> 3, labels, inv_t, a.prox_logp, a.adv, (const uint32_t*)(mask_addr & ~(uintptr_t)3),
+                       (unsigned)(mask_addr & 3), a.behave_w, a, (uint4*)dlogits, T, work, 0);
+  else
+    hipLaunchKernelGGL((k_fused_regs<DT, NCH, false, false>), dim3((unsigned)wgs), dim3(1024), 0, st, (const uint4*)logits, V,
+                       stride >> 3, labels, inv_t, a.prox_logp, a.adv, (const uint32_t*)(mask_addr & ~(uintptr_t)3),
+                       (unsigned)(mask_addr & 3), a.behave_w, a, (uint4*)dlogits, T, work, 0);
 }
 
 // Rows of more than kMaxRegChunks chunks: registers + LDS + streamed tail (see k_fused_regs, EXT).
@@ -1041,16 +1069,24 @@ template <int DT>
 static bool launch_regs_ext(int nch, const void* logits, int64_t T, int V, int64_t stride, const int64_t* labels,
                             float inv_t, const FusedTokenArgs& a, void* dlogits, int32_t* work, hipStream_t st) {
   static const bool ok =
-      hipFuncSetAttribute((const void*)k_fused_regs<DT, kExtRegChunks, true>,
+      hipFuncSetAttribute((const void*)k_fused_regs<DT, kExtRegChunks, true, false>,
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kExtLdsChunks * 16384) == hipSuccess &&
+      hipFuncSetAttribute((const void*)k_fused_regs<DT, kExtRegChunks, true, true>,
                           hipFuncAttributeMaxDynamicSharedMemorySize, kExtLdsChunks * 16384) == hipSuccess;
   if (!ok || nch <= kExtRegChunks || nch > kMaxExtChunks) return false;
   const int n_lds = nch - kExtRegChunks < kExtLdsChunks ? nch - kExtRegChunks : kExtLdsChunks;
   const int64_t wgs = T < persistent_workgroups() ? T : persistent_workgroups();
   const uintptr_t mask_addr = (uintptr_t)a.mask_eff;
-  hipLaunchKernelGGL((k_fused_regs<DT, kExtRegChunks, true>), dim3((unsigned)wgs), dim3(1024), n_lds * 16384, st,
-                     (const uint4*)logits, V, stride >> 3, labels, inv_t, a.prox_logp, a.adv,
-                     (const uint32_t*)(mask_addr & ~(uintptr_t)3), (unsigned)(mask_addr & 3), a.behave_w, a,
-                     (uint4*)dlogits, T, work, n_lds);
+  if (dlogits == logits)
+    hipLaunchKernelGGL((k_fused_regs<DT, kExtRegChunks, true, true>), dim3((unsigned)wgs), dim3(1024), n_lds * 16384, st,
+                       (const uint4*)logits, V, stride >> 3, labels, inv_t, a.prox_logp, a.adv,
+                       (const uint32_t*)(mask_addr & ~(uintptr_t)3), (unsigned)(mask_addr & 3), a.behave_w, a,
+                       (uint4*)dlogits, T, work, n_lds);
+  else
+    hipLaunchKernelGGL((k_fused_regs<DT, kExtRegChunks, true, false>), dim3((unsigned)wgs), dim3(1024), n_lds * 16384, st,
+                       (const uint4*)logits, V, stride >> 3, labels, inv_t, a.prox_logp, a.adv,
+                       (const uint32_t*)(mask_addr & ~(uintptr_t)3), (unsigned)(mask_addr & 3), a.behave_w, a,
+                       (uint4*)dlogits, T, work, n_lds);
   return true;
 }
 
@@ -1100,9 +1136,16 @@ extern "C" int aa_logits_bwd(const void* logits, int dtype, int64_t T, int64_t V
   hipStream_t st = (hipStream_t)stream;
   const int vec_ok = rows_vec_ok(logits, dlogits, dtype) ? 1 : 0;
   constexpr int NT = 256;
-#define AA_LAUNCH(DT)                                                                                        \
-  hipLaunchKernelGGL((k_logits_bwd<DT, NT>), dim3((unsigned)T), dim3(NT), 0, st, logits, (int)V, row_stride, \
-                     labels, inv_temperature, vec_ok, row_lse, row_ez, g_logp, g_entropy, T_active, dlogits)
+#define AA_LAUNCH(DT)                                                                                                 \
+  do {                                                                                                                \
+    if (dlogits == logits)                                                                                            \
+      hipLaunchKernelGGL((k_logits_bwd<DT, NT, true>), dim3((unsigned)T), dim3(NT), 0, st, logits, (int)V, row_stride, \
+                         labels, inv_temperature, vec_ok, row_lse, row_ez, g_logp, g_entropy, T_active, dlogits);     \
+    else                                                                                                              \
+      hipLaunchKernelGGL((k_logits_bwd<DT, NT, false>), dim3((unsigned)T), dim3(NT), 0, st, logits, (int)V,           \
+                         row_stride, labels, inv_temperature, vec_ok, row_lse, row_ez, g_logp, g_entropy, T_active,   \
+                         dlogits);                                                                                    \
+  } while (0)
   if (dtype == AA_BF16) AA_LAUNCH(AA_BF16);
   else if (dtype == AA_F16) AA_LAUNCH(AA_F16);
   else AA_LAUNCH(AA_F32);
@@ -1113,9 +1156,10 @@ extern "C" int aa_logits_bwd(const void* logits, int dtype, int64_t T, int64_t V
 // dlogits may be the logits array itself.  What makes that work in each kernel below: a row belongs to one workgroup;
 // the label's logit and the row statistics are read before the first store of the row; and an element that is read a
 // second time for the gradient (two-pass rows, the tail of a row that does not fit on the chip) is read and then
-// written by the same thread, the store depending on the load.  The kernels keep __restrict__ on both pointers (the
-// register kernel measures 0.7 % slower without it): all it lets the compiler do is move loads of OTHER elements
-// across a store, which the in-place use does not mind.  Tests compare the in-place result bit for bit on every kernel.
+// written by the same thread, the store depending on the load.  The two pointers are restrict-qualified (the
+// register kernel measures 0.7 % slower without that) only in the instantiations that run on two distinct arrays; the
+// in-place call runs the instantiation without the qualifier.  Tests compare the in-place result bit for bit on every
+// kernel.
 extern "C" int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int64_t V, int64_t row_stride,
                                    const int64_t* labels, float inv_temperature, int64_t T_active,
                                    const float* prox_logp, const float* adv, const uint8_t* mask_eff,
@@ -1165,8 +1209,12 @@ extern "C" int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int
       ((((uintptr_t)logits | (uintptr_t)dlogits) & 15) == 0)) {
     const int cus = persistent_workgroups();
     const unsigned grid = (unsigned)(T < cus ? T : cus);
-    hipLaunchKernelGGL(k_fused_f32_hold, dim3(grid), dim3(1024), 0, st, (const float*)logits, T, (int)V, row_stride,
-                       labels, inv_temperature, a, (float*)dlogits);
+    if (dlogits == logits)
+      hipLaunchKernelGGL(k_fused_f32_hold<true>, dim3(grid), dim3(1024), 0, st, (const float*)logits, T, (int)V, row_stride,
+                         labels, inv_temperature, a, (float*)dlogits);
+    else
+      hipLaunchKernelGGL(k_fused_f32_hold<false>, dim3(grid), dim3(1024), 0, st, (const float*)logits, T, (int)V, row_stride,
+                         labels, inv_temperature, a, (float*)dlogits);
     return launch_status();
   }
   const int vec_ok = rows_vec_ok(logits, dlogits, dtype) ? 1 : 0;
@@ -1174,19 +1222,25 @@ extern "C" int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int
   // the rows in flight (one per workgroup) stay small enough for the second read to come from the caches.
   const int64_t row_bytes = V * (dtype == AA_F32 ? 4 : 2);
   const bool walk = row_bytes >= kWalkRowBytes && T > kWalkGroups;
-#define AA_LAUNCH(DT)                                                                                              \
-  do {                                                                                                             \
-    if (walk)                                                                                                      \
-      hipLaunchKernelGGL((k_fused_generic<DT, 1024>), dim3((unsigned)kWalkGroups), dim3(1024), 0, st, logits, T,   \
-                         (int)V, row_stride, labels, inv_temperature, vec_ok, a, dlogits);                         \
-    else                                                                                                           \
-      hipLaunchKernelGGL((k_fused_generic<DT, 256>), dim3((unsigned)T), dim3(256), 0, st, logits, T, (int)V,       \
-                         row_stride, labels, inv_temperature, vec_ok, a, dlogits);                                 \
+#define AA_LAUNCH_AS(DT, ALIAS)                                                                                          \
+  do {                                                                                                                   \
+    if (walk)                                                                                                            \
+      hipLaunchKernelGGL((k_fused_generic<DT, 1024, ALIAS>), dim3((unsigned)kWalkGroups), dim3(1024), 0, st, logits, T,  \
+                         (int)V, row_stride, labels, inv_temperature, vec_ok, a, dlogits);                               \
+    else                                                                                                                 \
+      hipLaunchKernelGGL((k_fused_generic<DT, 256, ALIAS>), dim3((unsigned)T), dim3(256), 0, st, logits, T, (int)V,      \
+                         row_stride, labels, inv_temperature, vec_ok, a, dlogits);                                       \
+  } while (0)
+#define AA_LAUNCH(DT)                                  \
+  do {                                                 \
+    if (dlogits == logits) AA_LAUNCH_AS(DT, true);     \
+    else AA_LAUNCH_AS(DT, false);                      \
   } while (0)
   if (dtype == AA_BF16) AA_LAUNCH(AA_BF16);
   else if (dtype == AA_F16) AA_LAUNCH(AA_F16);
   else AA_LAUNCH(AA_F32);
 #undef AA_LAUNCH
+#undef AA_LAUNCH_AS
   return launch_status();
 }
 
