@@ -90,6 +90,10 @@ SIGNATURES = {
     "aa_lmhead_fwd_static_scratch_bytes": (_i64, []),
     "aa_lmhead_fwd_static_max_vocab": (_i64, []),
     "aa_lmhead_bwd": (_i, [_p, _p, _i64, _i64, _i64, _p, _f, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i64, _p]),
+    "aa_lmhead_carry_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "aa_lmhead_panel_pitch": (_i64, [_i64]),
+    "aa_lmhead_fwd_carry": (_i, [_p, _p, _i64, _i64, _i64, _p, _f, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _p, _i64, _p]),
+    "aa_lmhead_bwd_carry": (_i, [_p, _p, _i64, _i64, _i64, _p, _f, _p, _p, _p, _p, _p, _p, _i64, _p, _p, _i, _p, _i64, _p]),
     "aa_lmhead_ppo_fused": (
         _i,
         [_p, _p, _i64, _i64, _i64, _p, _f, _i64, _p, _p, _p, _p, C.POINTER(PpoParams), _p, _p, _p, _i,

@@ -460,6 +460,27 @@ __global__ __launch_bounds__(256) void k_unit_factors(float* __restrict__ row_fa
   if (r < rows) row_factor[r] = 1.f;
 }
 
+// Backward of the stand-alone op in carry form: what k_token_loss does for the rows of the training step, for upstream
+// gradients that only exist once the forward has returned.  Per token t of the chunk with a panel row r: the row's
+// factor -(g / T) p_label from the saved log-prob, the label entry patched to 1 - 1 / p_label, and the chunk's redo
+// flag when the stored form cannot carry the row.
+__global__ __launch_bounds__(256) void k_carry_factors(const float* __restrict__ logp, const float* __restrict__ g_logp,
+                                                       const int64_t* __restrict__ labels,
+                                                       const int32_t* __restrict__ out_rows, int n_tok, int V, float inv_t,
+                                                       CarryOut carry) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= n_tok) return;
+  const int r = out_rows ? out_rows[t] : t;
+  if (r < 0) return;
+  const float lp = logp[t], g = g_logp[t];
+  const float f = g == 0.f ? 0.f : -(g * inv_t) * fast_exp2(lp * kLog2e);
+  carry.row_factor[r] = f;
+  const int64_t y = labels[t];
+  if (g != 0.f && y >= 0 && y < V)
+    carry.panel[(int64_t)r * carry.panel_ld + y] = (uint16_t)(Elem<AA_BF16>::pack(-expm1f(-lp), 0.f) & 0xffffu);
+  if (g != 0.f && (lp < kCarryMinLogp || fabsf(f) < kCarryMinFactor)) *carry.redo_flag = 1;
+}
+
 // ---- plain product C = B . A^T on the same main loop ---------------------------------------------------------------
 // C [N, M] row-major with leading dimension ldc: C[n][m] = sum_k B[n][k] A[m][k]; AKM / BKM: the operand is stored
 // K-major (see gemm_tn.h).  The operand whose rows are the columns of C goes first, because a lane of the accumulator layout owns one n and runs of four consecutive m: four
@@ -734,7 +755,9 @@ struct Workspace {
   int64_t bytes;
 };
 
-static Workspace plan(int64_t T, int64_t H, int64_t V) {
+// external_panel: the d(logits) rows live in an array of the caller's (the op that keeps them from its forward to its
+// backward), not in the workspace
+static Workspace plan(int64_t T, int64_t H, int64_t V, bool external_panel = false) {
   Workspace w{};
   auto up = [](int64_t x) { return (x + 255) / 256 * 256; };
   w.chunk = T < kChunkTokens ? round_up(T, 256) : kChunkTokens;
@@ -753,7 +776,7 @@ static Workspace plan(int64_t T, int64_t H, int64_t V) {
   w.off_flag = off;    off += 256;              // the chunk's "redo by recompute" flag
   w.off_rows = off;    off += up(2 * w.chunk * 4);
   w.panel_ld = round_up(V, 8);
-  w.off_panel = off;   off += up(w.chunk * w.panel_ld * 2);
+  w.off_panel = off;   off += external_panel ? 0 : up(w.chunk * w.panel_ld * 2);
   w.off_hc = off;      off += up(w.chunk * H * 2);
   w.off_dw = off;      off += T > w.chunk ? up(V * H * 4) : 0;
   w.off_dhp = off;     off += up(kMaxSplits * w.chunk * H * 4);
@@ -848,10 +871,9 @@ static void launch_gemm(hipStream_t st, const uint16_t* A, int64_t lda, int64_t 
 // No transposed copy of anything is made.  token_of_row, when given, lists the tokens of the chunk that the n_rows
 // rows belong to (tokens without gradient were left out): their hidden rows are closed up first, and the d_hidden rows
 // go to those tokens (the caller has cleared the others).
-static void panel_gradients(hipStream_t st, const Workspace& w, char* ws, const void* weight, const uint16_t* hid,
-                            const int32_t* token_of_row, const float* row_factor, int64_t n_rows, int64_t H, int64_t V,
-                            uint16_t* d_hidden_chunk, void* d_weight, bool dw_f32, bool first) {
-  const uint16_t* ds = (const uint16_t*)(ws + w.off_panel);
+static void panel_gradients(hipStream_t st, const Workspace& w, char* ws, const uint16_t* ds, const void* weight,
+                            const uint16_t* hid, const int32_t* token_of_row, const float* row_factor, int64_t n_rows,
+                            int64_t H, int64_t V, uint16_t* d_hidden_chunk, void* d_weight, bool dw_f32, bool first) {
   const uint16_t* hid_rows = hid;
   if (token_of_row || row_factor) {
     uint16_t* hc = (uint16_t*)(ws + w.off_hc);
@@ -887,10 +909,10 @@ static void panel_gradients(hipStream_t st, const Workspace& w, char* ws, const 
 // Recompute: d(logits) of the panel rows from the logits tiles formed again.  With a row map only the hidden rows that
 // have a panel row are multiplied (gathered first); `a` carries the per-token inputs of the chunk.  With run_if the
 // kernels are enqueued but do nothing unless *run_if != 0 when they start.
-static void recompute_panel(hipStream_t st, const Workspace& w, char* ws, const void* weight, const uint16_t* hid,
-                            int64_t n_tok, const int32_t* token_of_row, int64_t rows, int64_t H, int64_t V, TileArgs a,
-                            const int32_t* run_if = nullptr) {
-  a.panel = (uint16_t*)(ws + w.off_panel);
+static void recompute_panel(hipStream_t st, const Workspace& w, char* ws, uint16_t* panel, const void* weight,
+                            const uint16_t* hid, int64_t n_tok, const int32_t* token_of_row, int64_t rows, int64_t H,
+                            int64_t V, TileArgs a, const int32_t* run_if = nullptr) {
+  a.panel = panel;
   a.panel_ld = w.panel_ld;
   a.out_rows = nullptr;
   a.run_if = run_if;
@@ -1088,6 +1110,7 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
   const WeightGrad dw = weight_grad(w, ws, d_weight, d_weight_dtype, T);
   int32_t* out_rows = (int32_t*)(ws + w.off_rows);
   int32_t* act_rows = out_rows + w.chunk;
+  uint16_t* ws_panel = (uint16_t*)(ws + w.off_panel);
   bool first = true;  // no GEMM has written d_weight yet
   int64_t chunk_index = 0;
   for (int64_t t0 = 0; t0 < T; t0 += w.chunk, ++chunk_index) {
@@ -1103,8 +1126,8 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
     a.g_logp = g_logp + t0;
     a.g_entropy = g_entropy ? g_entropy + t0 : nullptr;
     if (!kept_per_chunk) {
-      recompute_panel(st, w, ws, weight, hid, n_tok, nullptr, n_tok, H, V, a);
-      panel_gradients(st, w, ws, weight, hid, nullptr, nullptr, n_tok, H, V, dh, dw.acc, dw.acc_f32, first);
+      recompute_panel(st, w, ws, ws_panel, weight, hid, n_tok, nullptr, n_tok, H, V, a);
+      panel_gradients(st, w, ws, ws_panel, weight, hid, nullptr, nullptr, n_tok, H, V, dh, dw.acc, dw.acc_f32, first);
       first = false;
       continue;
     }
@@ -1117,10 +1140,150 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
     }
     hipLaunchKernelGGL(k_compact_map, dim3(1), dim3(1024), 0, st, row_has_gradient + t0, (int)n_tok, (int)n_tok, (int)kept,
                        out_rows, act_rows, (float*)nullptr, (u32x4_t*)(ws + w.off_panel), w.panel_ld);
-    recompute_panel(st, w, ws, weight, hid, n_tok, act_rows, kept, H, V, a);
+    recompute_panel(st, w, ws, ws_panel, weight, hid, n_tok, act_rows, kept, H, V, a);
     launch_zero(st, dh, n_tok * H * 2);  // the rows of the other tokens
-    panel_gradients(st, w, ws, weight, hid, act_rows, nullptr, kept, H, V, dh, dw.acc, dw.acc_f32, first);
+    panel_gradients(st, w, ws, ws_panel, weight, hid, act_rows, nullptr, kept, H, V, dh, dw.acc, dw.acc_f32, first);
     first = false;
+  }
+  if (first) launch_zero(st, dw.acc, V * H * (dw.acc_f32 ? 4 : 2));  // no row of the batch has a gradient
+  finish_weight_grad(st, dw, d_weight, V, H);
+  return launch_status();
+}
+
+extern "C" int64_t aa_lmhead_carry_workspace_bytes(int64_t T, int64_t H, int64_t V) {
+  if (!shapes_ok(T, H, V)) return -1;
+  return plan(T, H, V, true).bytes;
+}
+
+extern "C" int64_t aa_lmhead_panel_pitch(int64_t V) { return round_up(V, 8); }
+
+// rows of the panel that the chunks before chunk `upto` take: the tokens named by the host's counts, or all of them
+static int64_t panel_rows_before(const int64_t* kept_per_chunk, int64_t chunk, int64_t T, int64_t upto) {
+  int64_t rows = 0;
+  for (int64_t c = 0; c < upto; ++c) {
+    const int64_t n_tok = (T - c * chunk) < chunk ? (T - c * chunk) : chunk;
+    int64_t k = kept_per_chunk ? kept_per_chunk[c] : n_tok;
+    rows += k < 0 ? 0 : (k > n_tok ? n_tok : k);
+  }
+  return rows;
+}
+
+extern "C" int aa_lmhead_fwd_carry(const void* hidden, const void* weight, int64_t T, int64_t H, int64_t V,
+                                   const int64_t* labels, float inv_temperature, const uint8_t* row_has_gradient,
+                                   const int64_t* kept_per_chunk, float* logp, float* entropy, float* row_lse,
+                                   float* row_ez, float* vocab_max, float* vocab_min, void* panel, int64_t panel_rows,
+                                   void* workspace, int64_t workspace_bytes, void* stream) {
+  if (!hidden || !weight || !labels || !logp || !row_lse || !panel || !workspace || !(inv_temperature > 0.f))
+    return AA_ERR_INVALID_ARGUMENT;
+  if ((kept_per_chunk != nullptr) != (row_has_gradient != nullptr)) return AA_ERR_INVALID_ARGUMENT;
+  if ((vocab_max != nullptr) != (vocab_min != nullptr)) return AA_ERR_INVALID_ARGUMENT;
+  if (!shapes_ok(T, H, V)) return AA_ERR_UNSUPPORTED;
+  if ((((uintptr_t)hidden | (uintptr_t)weight | (uintptr_t)workspace | (uintptr_t)panel) & 15)) return AA_ERR_INVALID_ARGUMENT;
+  const Workspace w = plan(T, H, V, true);
+  if (workspace_bytes < w.bytes) return AA_ERR_INVALID_ARGUMENT;
+  const int64_t n_chunks = (T + w.chunk - 1) / w.chunk;
+  if (panel_rows < panel_rows_before(kept_per_chunk, w.chunk, T, n_chunks)) return AA_ERR_INVALID_ARGUMENT;
+  if (!prepare_kernels()) return AA_ERR_LAUNCH;
+  hipStream_t st = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+  int32_t* out_rows = (int32_t*)(ws + w.off_rows);
+  int32_t* act_rows = out_rows + w.chunk;
+  auto at = [](float* p, int64_t t0) { return p ? p + t0 : nullptr; };
+  int64_t chunk_index = 0, row0 = 0;
+  for (int64_t t0 = 0; t0 < T; t0 += w.chunk, ++chunk_index) {
+    const int64_t n_tok = (T - t0) < w.chunk ? (T - t0) : w.chunk;
+    const uint16_t* hid = (const uint16_t*)hidden + t0 * H;
+    uint16_t* chunk_panel = (uint16_t*)panel + row0 * w.panel_ld;
+    int64_t rows = n_tok;
+    if (kept_per_chunk) {
+      rows = kept_per_chunk[chunk_index];
+      rows = rows < 0 ? 0 : (rows > n_tok ? n_tok : rows);
+      hipLaunchKernelGGL(k_compact_map, dim3(1), dim3(1024), 0, st, row_has_gradient + t0, (int)n_tok, (int)n_tok, (int)rows,
+                         out_rows, act_rows, (float*)nullptr, (u32x4_t*)chunk_panel, w.panel_ld);
+    }
+    TileArgs a = stats_args(w, ws, labels + t0, inv_temperature, vocab_min != nullptr);
+    a.panel = chunk_panel;
+    a.panel_ld = w.panel_ld;
+    a.out_rows = kept_per_chunk ? out_rows : nullptr;
+    hipLaunchKernelGGL(k_label_logit, dim3((unsigned)((n_tok + 3) / 4)), dim3(256), 0, st, hid, (const uint16_t*)weight,
+                       labels + t0, (int)n_tok, (int)H, (int)V, a.xy, (int32_t*)nullptr);
+    if (rows > 0)
+      launch_tiles<kModeStatsCarry>(st, weight, hid, n_tok, H, V, a);
+    else
+      launch_tiles<kModeStats>(st, weight, hid, n_tok, H, V, a);
+    hipLaunchKernelGGL(k_combine, dim3((unsigned)((n_tok + 63) / 64)), dim3(1024), 0, st, a.pk, a.ps, a.pu, a.pn, a.xy,
+                       (int)w.blocks, a.pitch_t, (int)n_tok, a.c, logp + t0, at(entropy, t0), row_lse + t0, at(row_ez, t0),
+                       at(vocab_max, t0), at(vocab_min, t0));
+    row0 += rows;
+  }
+  return launch_status();
+}
+
+extern "C" int aa_lmhead_bwd_carry(const void* hidden, const void* weight, int64_t T, int64_t H, int64_t V,
+                                   const int64_t* labels, float inv_temperature, const float* logp, const float* row_lse,
+                                   const float* g_logp, const uint8_t* row_has_gradient, const int64_t* kept_per_chunk,
+                                   void* panel, int64_t panel_rows, void* d_hidden, void* d_weight, int d_weight_dtype,
+                                   void* workspace, int64_t workspace_bytes, void* stream) {
+  if (!hidden || !weight || !labels || !logp || !row_lse || !g_logp || !panel || !d_hidden || !d_weight || !workspace)
+    return AA_ERR_INVALID_ARGUMENT;
+  if (!(inv_temperature > 0.f) || (kept_per_chunk != nullptr) != (row_has_gradient != nullptr)) return AA_ERR_INVALID_ARGUMENT;
+  if (!shapes_ok(T, H, V) || (d_weight_dtype != AA_F32 && d_weight_dtype != AA_BF16)) return AA_ERR_UNSUPPORTED;
+  if ((((uintptr_t)hidden | (uintptr_t)weight | (uintptr_t)workspace | (uintptr_t)d_hidden | (uintptr_t)d_weight |
+        (uintptr_t)panel) & 15))
+    return AA_ERR_INVALID_ARGUMENT;
+  const Workspace w = plan(T, H, V, true);
+  if (workspace_bytes < w.bytes) return AA_ERR_INVALID_ARGUMENT;
+  const int64_t n_chunks = (T + w.chunk - 1) / w.chunk;
+  if (panel_rows < panel_rows_before(kept_per_chunk, w.chunk, T, n_chunks)) return AA_ERR_INVALID_ARGUMENT;
+  if (!prepare_kernels()) return AA_ERR_LAUNCH;
+  hipStream_t st = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+  const WeightGrad dw = weight_grad(w, ws, d_weight, d_weight_dtype, T);
+  int32_t* out_rows = (int32_t*)(ws + w.off_rows);
+  int32_t* act_rows = out_rows + w.chunk;
+  float* row_factor = (float*)(ws + w.off_rowf);
+  int32_t* redo_flag = (int32_t*)(ws + w.off_flag);
+  bool first = true;  // no GEMM has written d_weight yet
+  int64_t chunk_index = 0, row0 = 0;
+  for (int64_t t0 = 0; t0 < T; t0 += w.chunk, ++chunk_index) {
+    const int64_t n_tok = (T - t0) < w.chunk ? (T - t0) : w.chunk;
+    const uint16_t* hid = (const uint16_t*)hidden + t0 * H;
+    uint16_t* dh = (uint16_t*)d_hidden + t0 * H;
+    uint16_t* chunk_panel = (uint16_t*)panel + row0 * w.panel_ld;
+    int64_t rows = n_tok;
+    const int32_t* row_of_token = nullptr;
+    const int32_t* token_of_row = nullptr;
+    if (kept_per_chunk) {
+      rows = kept_per_chunk[chunk_index];
+      rows = rows < 0 ? 0 : (rows > n_tok ? n_tok : rows);
+      if (rows == 0) {
+        launch_zero(st, dh, n_tok * H * 2);
+        continue;
+      }
+      // the same numbering as in the forward (the mask has not changed); surplus rows get a factor of zero
+      hipLaunchKernelGGL(k_compact_map, dim3(1), dim3(1024), 0, st, row_has_gradient + t0, (int)n_tok, (int)n_tok, (int)rows,
+                         out_rows, act_rows, row_factor, (u32x4_t*)chunk_panel, w.panel_ld);
+      row_of_token = out_rows;
+      token_of_row = act_rows;
+    }
+    launch_zero(st, redo_flag, 256);
+    hipLaunchKernelGGL(k_carry_factors, dim3((unsigned)((n_tok + 255) / 256)), dim3(256), 0, st, logp + t0, g_logp + t0,
+                       labels + t0, row_of_token, (int)n_tok, (int)V, inv_temperature,
+                       CarryOut{row_factor, chunk_panel, w.panel_ld, redo_flag});
+    // a chunk whose rows do not fit the stored form is redone from the logits tiles, decided on the device
+    TileArgs a{};
+    a.labels = labels + t0;
+    a.c = kLog2e * inv_temperature;
+    a.inv_t = inv_temperature;
+    a.row_lse = row_lse + t0;
+    a.g_logp = g_logp + t0;
+    a.panel_ld = w.panel_ld;
+    recompute_panel(st, w, ws, chunk_panel, weight, hid, n_tok, token_of_row, rows, H, V, a, redo_flag);
+    hipLaunchKernelGGL(k_unit_factors, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, row_factor, (int)rows, redo_flag);
+    if (token_of_row) launch_zero(st, dh, n_tok * H * 2);  // the rows of the tokens without a panel row
+    panel_gradients(st, w, ws, chunk_panel, weight, hid, token_of_row, row_factor, rows, H, V, dh, dw.acc, dw.acc_f32, first);
+    first = false;
+    row0 += rows;
   }
   if (first) launch_zero(st, dw.acc, V * H * (dw.acc_f32 ? 4 : 2));  // no row of the batch has a gradient
   finish_weight_grad(st, dw, d_weight, V, H);
@@ -1210,12 +1373,12 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
     // device: the kernels start and return at once otherwise), and then the row factors become 1
     a.row_lse = lse_tok;
     a.g_logp = g_tok;
-    recompute_panel(st, w, ws, weight, hid, n_tok, token_of_row, rows, H, V, a, carry ? redo_flag : nullptr);
+    recompute_panel(st, w, ws, panel, weight, hid, n_tok, token_of_row, rows, H, V, a, carry ? redo_flag : nullptr);
     if (carry)
       hipLaunchKernelGGL(k_unit_factors, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, row_factor, (int)rows, redo_flag);
     if (token_of_row) launch_zero(st, dh, n_tok * H * 2);  // the rows of the tokens without gradient
-    panel_gradients(st, w, ws, weight, hid, token_of_row, carry ? row_factor : nullptr, rows, H, V, dh, dw.acc, dw.acc_f32,
-                    first);
+    panel_gradients(st, w, ws, panel, weight, hid, token_of_row, carry ? row_factor : nullptr, rows, H, V, dh, dw.acc,
+                    dw.acc_f32, first);
     first = false;
   }
   if (first) launch_zero(st, dw.acc, V * H * (dw.acc_f32 ? 4 : 2));  // no token of the batch has a gradient

@@ -806,39 +806,123 @@ class _LmHeadLogprobsEntropy(torch.autograd.Function):
     def backward(ctx, g_logp, g_entropy, _g_vmax=None, _g_vmin=None):
         if g_logp is None and g_entropy is None:
             return None, None, None, None, None
-        lib = N.load()
         hidden, weight, labels, row_lse, row_ez = ctx.saved_tensors
+        d_hidden, d_weight = _lmhead_recompute_backward(hidden, weight, labels, ctx.temperature, row_lse, row_ez,
+                                                        g_logp, g_entropy)
+        return d_hidden, d_weight, None, None, None
+
+
+def _lmhead_recompute_backward(hidden, weight, labels, temperature, row_lse, row_ez, g_logp, g_entropy):
+    """``aa_lmhead_bwd``: the logits tiles of the tokens with a gradient are formed again."""
+    lib = N.load()
+    T, H = hidden.shape
+    V = weight.shape[0]
+    dev = hidden.device
+    g_logp = torch.zeros(T, dtype=torch.float32, device=dev) if g_logp is None else _f32(g_logp)
+    g_entropy = None if g_entropy is None else _f32(g_entropy)
+    d_hidden = torch.empty_like(hidden)
+    d_weight = torch.empty_like(weight)  # bf16: rounded once, after fp32 accumulation over the chunks
+    ws = _lmhead_workspace(T, H, V, dev)
+    # Rows whose upstream gradients are all zero (masked tokens) are left out of the gradient GEMMs; their
+    # count per chunk sizes the GEMMs, so the host reads it here.
+    has_grad = g_logp != 0 if g_entropy is None else (g_logp != 0) | (g_entropy != 0)
+    chunk = int(lib.aa_lmhead_chunk_tokens())
+    n_chunks = (T + chunk - 1) // chunk
+    padded = has_grad if n_chunks * chunk == T else torch.nn.functional.pad(has_grad, (0, n_chunks * chunk - T))
+    per_chunk = _HostCounts(padded.view(n_chunks, chunk).sum(1)).tolist()
+    kept = (C.c_int64 * n_chunks)(*per_chunk)
+    with torch.cuda.device(dev):
+        N.check(
+            lib.aa_lmhead_bwd(
+                _ptr(hidden), _ptr(weight), T, H, V, _ptr(labels), 1.0 / temperature, _ptr(row_lse),
+                _ptr(row_ez), _ptr(g_logp), _ptr(g_entropy), _ptr(has_grad.view(torch.uint8)), kept,
+                _ptr(d_hidden), _ptr(d_weight), _DTYPES[d_weight.dtype], _ptr(ws), ws.numel(), _stream(dev),
+            ),
+            "aa_lmhead_bwd",
+        )
+    return d_hidden, d_weight
+
+
+class _LmHeadCarry(torch.autograd.Function):
+    """The lm_head op whose forward also keeps ``p_v / p_label`` of the tokens that may get a gradient (bf16 rows, in a
+    tensor that lives until the backward), so that the backward is two plain GEMMs (``aa_lmhead_fwd_carry`` /
+    ``aa_lmhead_bwd_carry``)."""
+
+    @staticmethod
+    def forward(ctx, hidden, weight, labels, temperature, grad_mask, kept_per_chunk, want_minmax):
+        ctx.set_materialize_grads(False)
+        lib = N.load()
         T, H = hidden.shape
         V = weight.shape[0]
         dev = hidden.device
-        g_logp = torch.zeros(T, dtype=torch.float32, device=dev) if g_logp is None else _f32(g_logp)
-        g_entropy = None if g_entropy is None else _f32(g_entropy)
-        d_hidden = torch.empty_like(hidden)
-        d_weight = torch.empty_like(weight)  # bf16: rounded once, after fp32 accumulation over the chunks
-        ws = _lmhead_workspace(T, H, V, dev)
-        # Rows whose upstream gradients are all zero (masked tokens) are left out of the gradient GEMMs; their
-        # count per chunk sizes the GEMMs, so the host reads it here.
-        has_grad = g_logp != 0 if g_entropy is None else (g_logp != 0) | (g_entropy != 0)
-        chunk = int(lib.aa_lmhead_chunk_tokens())
-        n_chunks = (T + chunk - 1) // chunk
-        padded = has_grad if n_chunks * chunk == T else torch.nn.functional.pad(has_grad, (0, n_chunks * chunk - T))
-        per_chunk = _HostCounts(padded.view(n_chunks, chunk).sum(1)).tolist()
-        kept = (C.c_int64 * n_chunks)(*per_chunk)
+        f32 = dict(dtype=torch.float32, device=dev)
+        logp, entropy, row_lse, row_ez = (torch.empty(T, **f32) for _ in range(4))
+        vmax = torch.empty(T, **f32) if want_minmax else None
+        vmin = torch.empty(T, **f32) if want_minmax else None
+        kept = None if kept_per_chunk is None else (C.c_int64 * len(kept_per_chunk))(*kept_per_chunk)
+        rows = T if kept_per_chunk is None else sum(kept_per_chunk)
+        panel = torch.empty(max(rows, 1), int(lib.aa_lmhead_panel_pitch(V)), dtype=torch.bfloat16, device=dev)
+        n = lib.aa_lmhead_carry_workspace_bytes(T, H, V)
+        if n < 0:
+            raise N.NativeLibraryError(
+                f"the lm_head path needs a hidden size that is a multiple of 8, and sizes below 2^22 (got H={H}, V={V})")
+        ws = torch.empty(n, dtype=torch.uint8, device=dev)
         with torch.cuda.device(dev):
             N.check(
-                lib.aa_lmhead_bwd(
-                    _ptr(hidden), _ptr(weight), T, H, V, _ptr(labels), 1.0 / ctx.temperature, _ptr(row_lse),
-                    _ptr(row_ez), _ptr(g_logp), _ptr(g_entropy), _ptr(has_grad.view(torch.uint8)), kept,
-                    _ptr(d_hidden), _ptr(d_weight), _DTYPES[d_weight.dtype], _ptr(ws), ws.numel(), _stream(dev),
+                lib.aa_lmhead_fwd_carry(
+                    _ptr(hidden), _ptr(weight), T, H, V, _ptr(labels), 1.0 / float(temperature), _ptr(grad_mask), kept,
+                    _ptr(logp), _ptr(entropy), _ptr(row_lse), _ptr(row_ez), _ptr(vmax), _ptr(vmin), _ptr(panel),
+                    panel.shape[0], _ptr(ws), ws.numel(), _stream(dev),
                 ),
-                "aa_lmhead_bwd",
+                "aa_lmhead_fwd_carry",
             )
-        return d_hidden, d_weight, None, None, None
+        ctx.save_for_backward(hidden, weight, labels, logp, row_lse, row_ez, panel, grad_mask)
+        ctx.temperature = float(temperature)
+        ctx.kept_per_chunk = kept_per_chunk
+        if want_minmax:
+            ctx.mark_non_differentiable(vmax, vmin)
+        return logp, entropy, vmax, vmin
+
+    @staticmethod
+    def backward(ctx, g_logp, g_entropy, _g_vmax=None, _g_vmin=None):
+        if g_logp is None and g_entropy is None:
+            return (None,) * 7
+        hidden, weight, labels, logp, row_lse, row_ez, panel, grad_mask = ctx.saved_tensors
+        if g_entropy is not None:  # an entropy gradient is no multiple of the stored rows: form the logits again
+            d_hidden, d_weight = _lmhead_recompute_backward(hidden, weight, labels, ctx.temperature, row_lse, row_ez,
+                                                            g_logp, g_entropy)
+            return (d_hidden, d_weight) + (None,) * 5
+        # the backward patches the stored rows (and may overwrite a chunk of them): they serve one backward
+        if getattr(ctx, "handed_out", False):
+            raise RuntimeError("the stored rows of this lm_head forward were already used by a backward; run the forward "
+                               "pass again instead of a second backward through a retained graph")
+        ctx.handed_out = True
+        lib = N.load()
+        T, H = hidden.shape
+        V = weight.shape[0]
+        dev = hidden.device
+        g_logp = _f32(g_logp)
+        kept_per_chunk = ctx.kept_per_chunk
+        kept = None if kept_per_chunk is None else (C.c_int64 * len(kept_per_chunk))(*kept_per_chunk)
+        d_hidden = torch.empty_like(hidden)
+        d_weight = torch.empty_like(weight)
+        ws = torch.empty(lib.aa_lmhead_carry_workspace_bytes(T, H, V), dtype=torch.uint8, device=dev)
+        with torch.cuda.device(dev):
+            N.check(
+                lib.aa_lmhead_bwd_carry(
+                    _ptr(hidden), _ptr(weight), T, H, V, _ptr(labels), 1.0 / ctx.temperature, _ptr(logp), _ptr(row_lse),
+                    _ptr(g_logp), _ptr(grad_mask), kept, _ptr(panel), panel.shape[0], _ptr(d_hidden), _ptr(d_weight),
+                    _DTYPES[d_weight.dtype], _ptr(ws), ws.numel(), _stream(dev),
+                ),
+                "aa_lmhead_bwd_carry",
+            )
+        return (d_hidden, d_weight) + (None,) * 5
 
 
 def lm_head_logprobs_entropy(
     hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0,
-    token_mask: torch.Tensor | None = None,
+    token_mask: torch.Tensor | None = None, backward: str = "recompute", grad_token_mask: torch.Tensor | None = None,
+    kept_per_chunk: list[int] | None = None,
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """``gather_logprobs_entropy(hidden @ weight.T, labels, temperature)`` without writing the ``[T, V]`` logits.
     Any vocabulary size; the hidden size has to be a multiple of 8.
@@ -860,13 +944,26 @@ def lm_head_logprobs_entropy(
     ``token_mask`` (``[T]``, optional, beyond the reference's semantics): only tokens whose entry is non-zero go
     through the lm_head; the others get log-prob 0 and entropy 0 (e.g. the forward-only ``compute_logp`` pass, whose
     results are multiplied by the loss mask anyway).
+
+    ``backward="carry"`` (default ``"recompute"``): the forward also keeps ``p_v / p_label`` of the tokens that may get
+    a gradient as bf16 rows until the backward, which is then two plain GEMMs instead of three (no second logits GEMM:
+    about a fifth less time for forward + backward at the 8B shape).  For losses that need every log-prob before any
+    gradient exists (sequence-level importance ratios, SAPO, anything custom).  The price is memory between the two
+    passes: 2 bytes x V per such token.  ``grad_token_mask`` (``[T]``, e.g. the loss mask) names those tokens; tokens
+    outside it get NO gradient, whatever the loss says; without it every token is kept.  The number of named tokens per
+    chunk of ``lm_head_chunk_tokens()`` tokens sizes the stored rows: it is read back from the device unless the caller
+    passes it as ``kept_per_chunk`` (counts that are too large are safe, too small ones drop tokens).  A gradient
+    with respect to the entropy cannot use the stored rows: such a backward forms the logits again, as ``"recompute"``
+    does.  The stored rows serve one backward.
     """
-    return _lm_head_impl(hidden, weight, labels, temperature, token_mask, False)[:2]
+    return _lm_head_impl(hidden, weight, labels, temperature, token_mask, False, backward, grad_token_mask,
+                         kept_per_chunk)[:2]
 
 
 def lm_head_logprobs_entropy_stats(
     hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0,
-    token_mask: torch.Tensor | None = None,
+    token_mask: torch.Tensor | None = None, backward: str = "recompute", grad_token_mask: torch.Tensor | None = None,
+    kept_per_chunk: list[int] | None = None,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """``(logp, entropy, vocab_min_logits, vocab_max_logits)`` of ``hidden @ weight.T`` from the same tiles.
 
@@ -874,11 +971,38 @@ def lm_head_logprobs_entropy_stats(
     materialised logits and hands to the loss function; with no logits in memory the caller could not compute them.
     They come from the fp32 sums of the tiles, not from logits rounded to bf16 (the smallest exactly, the largest
     through the softmax exponent, i.e. to one rounding), and carry no gradient.  With ``token_mask`` the tokens left
-    out of the lm_head get 0 for both."""
-    return _lm_head_impl(hidden, weight, labels, temperature, token_mask, True)
+    out of the lm_head get 0 for both.  The other arguments: see ``lm_head_logprobs_entropy``."""
+    return _lm_head_impl(hidden, weight, labels, temperature, token_mask, True, backward, grad_token_mask,
+                         kept_per_chunk)
 
 
-def _lm_head_impl(hidden, weight, labels, temperature, token_mask, want_minmax):
+def _lm_head_apply(hidden, weight, y, temperature, want_minmax, backward, grad_mask, kept_per_chunk):
+    """One of the two autograd functions on a contiguous batch; ``grad_mask``: bool / uint8 ``[T]`` or None."""
+    needs_grad = torch.is_grad_enabled() and (hidden.requires_grad or weight.requires_grad)
+    if backward != "carry" or not needs_grad:
+        return _LmHeadLogprobsEntropy.apply(hidden, weight, y, float(temperature), want_minmax)
+    T = hidden.shape[0]
+    chunk = lm_head_chunk_tokens()
+    n_chunks = (T + chunk - 1) // chunk
+    m8 = kept = None
+    if grad_mask is not None:
+        m8 = _mask_u8(grad_mask)
+        if kept_per_chunk is not None:
+            kept = [max(0, min(int(v), chunk)) for v in kept_per_chunk]
+            if len(kept) != n_chunks:
+                raise ValueError(f"kept_per_chunk needs one count per chunk of {chunk} tokens")
+        else:
+            on = m8.ne(0)
+            if n_chunks * chunk != T:
+                on = torch.nn.functional.pad(on, (0, n_chunks * chunk - T))
+            kept = _HostCounts(on.view(n_chunks, chunk).sum(1)).tolist()
+    return _LmHeadCarry.apply(hidden, weight, y, float(temperature), m8, kept, want_minmax)
+
+
+def _lm_head_impl(hidden, weight, labels, temperature, token_mask, want_minmax, backward="recompute",
+                  grad_token_mask=None, kept_per_chunk=None):
+    if backward not in _LMHEAD_BACKWARD:
+        raise ValueError(f"backward must be one of {sorted(_LMHEAD_BACKWARD)}, got {backward!r}")
     _require_gpu(hidden, "hidden")
     if hidden.ndim != 2 or weight.ndim != 2 or hidden.shape[1] != weight.shape[1]:
         raise ValueError(f"expected hidden [T, H] and weight [V, H], got {tuple(hidden.shape)} and {tuple(weight.shape)}")
@@ -898,12 +1022,17 @@ def _lm_head_impl(hidden, weight, labels, temperature, token_mask, want_minmax):
             zero = (hidden[:1].float().sum() + weight[:1].float().sum()) * 0.0
             z = torch.zeros(T, dtype=torch.float32, device=dev) if want_minmax else None
             return zero.expand(T), zero.expand(T), z, z
-        lp, ent, vmax, vmin = _LmHeadLogprobsEntropy.apply(
-            hidden.index_select(0, idx), weight.contiguous(), y.index_select(0, idx), float(temperature), want_minmax)
+        sub_mask = None if grad_token_mask is None else grad_token_mask.to(dev).reshape(-1).index_select(0, idx)
+        lp, ent, vmax, vmin = _lm_head_apply(
+            hidden.index_select(0, idx), weight.contiguous(), y.index_select(0, idx), temperature, want_minmax, backward,
+            sub_mask, None)   # the counts of the caller are per chunk of the whole batch, not of the selected tokens
         full = lambda v: torch.zeros(T, dtype=torch.float32, device=dev).index_copy(0, idx, v)
         return full(lp), full(ent), (full(vmin) if want_minmax else None), (full(vmax) if want_minmax else None)
-    lp, ent, vmax, vmin = _LmHeadLogprobsEntropy.apply(hidden.contiguous(), weight.contiguous(), y, float(temperature),
-                                                       want_minmax)
+    if grad_token_mask is not None and tuple(grad_token_mask.shape) != (hidden.shape[0],):
+        raise ValueError(f"grad_token_mask shape {tuple(grad_token_mask.shape)} != ({hidden.shape[0]},)")
+    lp, ent, vmax, vmin = _lm_head_apply(hidden.contiguous(), weight.contiguous(), y, temperature, want_minmax, backward,
+                                         None if grad_token_mask is None else grad_token_mask.to(hidden.device),
+                                         kept_per_chunk)
     return lp, ent, vmin, vmax
 
 
@@ -1022,6 +1151,7 @@ def fused_lm_head_ppo_loss(
     forward_masked_tokens: bool = True,
     kept_per_chunk: list[int] | None = None,
     backward: str = "carry",
+    carry_rows_limit_bytes: int = 16 << 30,
 ) -> tuple[torch.Tensor, dict]:
     """lm_head + ``gather_logprobs_entropy`` + ``ppo_actor_loss_fn`` (+ backward) for one micro-batch.
 
@@ -1030,8 +1160,11 @@ def fused_lm_head_ppo_loss(
     256 x 256 tiles in the accumulator registers of the library's bf16 MFMA tile GEMM and reduced to softmax partials
     in its epilogue; they are never written to memory.  Tokens are processed in chunks of at most 16384;
     ``loss.backward()`` hands back ``d(hidden)`` and ``d(weight)`` written during the forward pass (the loss is
-    known by then).  With ``importance_sampling_level="sequence"`` the call runs ``lm_head_logprobs_entropy`` and the
-    unfused loss.
+    known by then).  With ``importance_sampling_level="sequence"`` (GSPO) every log-prob of a sequence is needed before
+    any gradient exists, so the call runs ``lm_head_logprobs_entropy`` and the unfused loss; with ``backward="carry"``
+    that op keeps the bf16 rows of the tokens with a mask from its forward to its backward (two GEMMs instead of
+    three), as long as they take no more than ``carry_rows_limit_bytes`` (2 bytes x V per such token; default 16 GiB),
+    and forms the logits again otherwise.
 
     ``backward`` chooses how the bf16 ``d(loss)/d(logits)`` rows of a chunk (``[tokens with gradient, V]`` in the
     workspace, which the two gradient GEMMs contract) are obtained.  ``"recompute"``: the logits tiles of those tokens
@@ -1090,8 +1223,26 @@ def fused_lm_head_ppo_loss(
     y = labels.to(device=dev, dtype=torch.int64).contiguous()
 
     forward_only = not (torch.is_grad_enabled() and (hidden.requires_grad or weight.requires_grad))
-    if importance_sampling_level == "sequence" or forward_only:  # no gradient to produce: forward GEMM + loss only
-        logp, entropy, vmin, vmax = lm_head_logprobs_entropy_stats(hidden, weight, y, temperature)
+    if importance_sampling_level == "sequence" or forward_only:
+        # forward-only: forward GEMM + loss.  Sequence level: every log-prob of a sequence is needed before any gradient
+        # exists, so the op and the loss run one after the other; in carry mode the op keeps the rows of the tokens with
+        # a mask for its backward (2 bytes x V per such token until then) unless that is more than the caller allows
+        grad_mask = kept_seq = None
+        op_backward = "recompute"
+        if not forward_only and backward == "carry":
+            pad = hidden.shape[0] - T_active
+            grad_mask = loss_mask.to(dev).reshape(-1).ne(0)
+            if pad:
+                grad_mask = torch.nn.functional.pad(grad_mask, (0, pad))
+            if kept_per_chunk is not None:
+                kept_seq = [int(v) for v in kept_per_chunk]
+            rows_bound = sum(kept_seq) if kept_seq is not None else hidden.shape[0]
+            if 2 * rows_bound * weight.shape[0] <= carry_rows_limit_bytes:
+                op_backward = "carry"
+        logp, entropy, vmin, vmax = lm_head_logprobs_entropy_stats(
+            hidden, weight, y, temperature, backward=op_backward,
+            grad_token_mask=grad_mask if op_backward == "carry" else None,
+            kept_per_chunk=kept_seq if op_backward == "carry" else None)
         logp, entropy = logp[:T_active], entropy[:T_active]
         loss, stat = ppo_actor_loss_fn(
             logp, proximal_logprobs, old_logprobs, advantages, eps_clip, loss_mask, eps_clip_higher, c_clip,

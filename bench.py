@@ -637,7 +637,28 @@ def time_lmhead_op(case, iters: int):
 
     f_ms, _ = time_events(fwd, iters, stream)
     b_ms, _ = time_events(bwd, iters, stream)
-    return f_ms, b_ms, kept_tokens
+    # the same op in carry form: the forward keeps p_v / p_label of the tokens with a gradient, the backward is two GEMMs
+    rows = kept_tokens if has_grad is not None else T
+    panel = torch.empty(rows, int(lib.aa_lmhead_panel_pitch(V)), dtype=torch.bfloat16, device=dev)
+    ws_c = torch.empty(lib.aa_lmhead_carry_workspace_bytes(T, H, V), dtype=torch.uint8, device=dev)
+
+    def fwd_carry():
+        N.check(lib.aa_lmhead_fwd_carry(F._ptr(case.hidden), F._ptr(case.weight), T, H, V, F._ptr(case.labels), inv_t,
+                                        F._ptr(has_grad), kept, F._ptr(logp), F._ptr(ent), F._ptr(lse), F._ptr(ez), None, None,
+                                        F._ptr(panel), rows, F._ptr(ws_c), ws_c.numel(), st), "aa_lmhead_fwd_carry")
+
+    def bwd_carry():
+        N.check(lib.aa_lmhead_bwd_carry(F._ptr(case.hidden), F._ptr(case.weight), T, H, V, F._ptr(case.labels), inv_t,
+                                        F._ptr(logp), F._ptr(lse), F._ptr(g), F._ptr(has_grad), kept, F._ptr(panel), rows,
+                                        F._ptr(dh), F._ptr(dw), N.AA_BF16, F._ptr(ws_c), ws_c.numel(), st), "aa_lmhead_bwd_carry")
+
+    def both_carry():  # the backward patches the stored rows: every timed backward follows a forward of its own
+        fwd_carry()
+        bwd_carry()
+
+    fc_ms, _ = time_events(fwd_carry, iters, stream)
+    pair_ms, _ = time_events(both_carry, iters, stream)
+    return f_ms, b_ms, kept_tokens, fc_ms, pair_ms - fc_ms
 
 
 def fused_gpu_sample(case, kw, cfg, n_tokens: int):
@@ -751,7 +772,7 @@ def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: i
                            compulsory_hbm_bytes=lmhead_compulsory_bytes(T, kept_tokens, H, V, name, chunk),
                            measured_hbm_bytes=lmhead_measured_bytes(workload, name)[0],
                            measured_hbm_bytes_source=lmhead_measured_bytes(workload, name)[1])
-    f_ms, b_ms, op_kept = time_lmhead_op(case, 5)
+    f_ms, b_ms, op_kept, fc_ms, bc_ms = time_lmhead_op(case, 5)
     # Flops the step needs: logits of every token (2 T V H) and the two gradient GEMMs over the tokens that have a
     # gradient (4 T_kept V H).  The reference's autograd runs them over all T tokens: 6 T V H.
     needed_flops = 2.0 * T * V * H + 4.0 * kept_tokens * V * H
@@ -775,7 +796,11 @@ def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: i
         # the stand-alone differentiable op lm_head_logprobs_entropy: its forward writes softmax partials only, its
         # backward forms the logits of the tokens with a gradient again (6 T_grad V H flops executed)
         standalone_op=dict(fwd_ms=f_ms, bwd_ms=b_ms, fwd_tflops=2.0 * T * V * H / (f_ms * 1e-3) / 1e12,
-                           bwd_executed_tflops=6.0 * op_kept * V * H / (b_ms * 1e-3) / 1e12),
+                           bwd_executed_tflops=6.0 * op_kept * V * H / (b_ms * 1e-3) / 1e12,
+                           # lm_head_logprobs_entropy(backward="carry"): the forward also keeps the bf16 rows of the
+                           # tokens with a gradient, the backward is the two gradient GEMMs (4 T_grad V H flops)
+                           carry_fwd_ms=fc_ms, carry_bwd_ms=bc_ms,
+                           carry_bwd_tflops=4.0 * op_kept * V * H / (bc_ms * 1e-3) / 1e12),
     )
     # the measured ceiling of the matrix cores in this process: a loop of MFMAs only (no LDS, no memory traffic)
     mfma_only = time_mfma_only_loop(dev)

@@ -725,6 +725,50 @@ int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, int64_t H,
                   void* d_weight, int d_weight_dtype, void* workspace,
                   int64_t workspace_bytes, void* stream);
 
+/*
+ * The stand-alone op with a backward of two plain GEMMs (no counterpart in the
+ * reference, whose autograd keeps the [T, V] logits): aa_lmhead_fwd_carry is
+ * aa_lmhead_fwd that also writes, for the tokens that may get a gradient, the
+ * bf16 rows p_v / p_label into `panel` (see AA_LMHEAD_CARRY below), and
+ * aa_lmhead_bwd_carry turns them into d_hidden and d_weight once g_logp is
+ * known: one factor per row, applied inside the two GEMMs; no second logits
+ * GEMM.  For losses that need the log-probs of the whole batch before any
+ * gradient exists (sequence-level importance ratios, areal/utils/functional/
+ * functional.py:56-149; SAPO, :562-638), at the price of keeping the panel
+ * between the two calls: panel_rows x aa_lmhead_panel_pitch(V) bf16, with
+ * panel_rows >= the sum of kept_per_chunk (or T when that is NULL); the rows of
+ * chunk c start after those of the chunks before it.
+ * row_has_gradient [T] (device) with kept_per_chunk (HOST), both or neither,
+ * as in aa_lmhead_bwd: tokens whose byte is zero get no panel row and no
+ * gradient, whatever g_logp holds for them; the same two arrays must be passed
+ * to both calls.  An entropy gradient cannot be carried: use aa_lmhead_bwd
+ * (row_lse / row_ez of this forward serve it) when there is one.  A chunk with
+ * a row that does not fit the stored form is redone from the logits tiles,
+ * decided on the device.  logp / row_lse: outputs of the forward, inputs of the
+ * backward.  workspace: aa_lmhead_carry_workspace_bytes(T, H, V) bytes for
+ * either call (the workspace of aa_lmhead_bwd without its panel).
+ */
+int64_t aa_lmhead_carry_workspace_bytes(int64_t T, int64_t H, int64_t V);
+int64_t aa_lmhead_panel_pitch(int64_t V);
+int aa_lmhead_fwd_carry(const void* hidden, const void* weight, int64_t T,
+                        int64_t H, int64_t V, const int64_t* labels,
+                        float inv_temperature,
+                        const uint8_t* row_has_gradient,
+                        const int64_t* kept_per_chunk, float* logp,
+                        float* entropy, float* row_lse, float* row_ez,
+                        float* vocab_max, float* vocab_min, void* panel,
+                        int64_t panel_rows, void* workspace,
+                        int64_t workspace_bytes, void* stream);
+int aa_lmhead_bwd_carry(const void* hidden, const void* weight, int64_t T,
+                        int64_t H, int64_t V, const int64_t* labels,
+                        float inv_temperature, const float* logp,
+                        const float* row_lse, const float* g_logp,
+                        const uint8_t* row_has_gradient,
+                        const int64_t* kept_per_chunk, void* panel,
+                        int64_t panel_rows, void* d_hidden, void* d_weight,
+                        int d_weight_dtype, void* workspace,
+                        int64_t workspace_bytes, void* stream);
+
 /* How aa_lmhead_ppo_fused fills the d(logits) rows that its backward GEMMs
  * contract. */
 typedef enum {

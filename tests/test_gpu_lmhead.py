@@ -393,3 +393,118 @@ def test_vocabulary_extrema_of_the_logits(device, T, H, V, temperature):
     assert not vmin.requires_grad and not vmax.requires_grad
     lp2, ent2 = areal_amd.lm_head_logprobs_entropy(hidden.to(device), weight.to(device), labels.to(device), temperature)
     assert torch.equal(lp, lp2) and torch.equal(ent, ent2)  # asking for the extrema changes nothing else
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# backward="carry" of the stand-alone op: the forward keeps p_v / p_label of the tokens that may get a gradient, the
+# backward is two plain GEMMs (aa_lmhead_fwd_carry / aa_lmhead_bwd_carry).  Same oracle, same tolerances.
+# ---------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("T,H,V,temperature,with_mask,counts_from_host", [
+    (300, 128, 1088, 1.0, True, False),
+    (203, 72, 1097, 0.7, True, True),          # vocabulary no multiple of 8
+    (CHUNK + 200, 64, 640, 1.3, True, True),   # two token chunks
+    (CHUNK + 72, 64, 640, 1.0, False, False),  # every token kept
+    (300, 128, 16643, 1.0, True, False),       # d(hidden) cut into parts along the vocabulary
+])
+def test_carried_backward_matches_autograd_of_oracle(device, T, H, V, temperature, with_mask, counts_from_host):
+    hidden, weight, labels = _case(T, H, V, seed=5 * T + V, w_std=0.3)
+    g = torch.Generator().manual_seed(3)
+    mask = (torch.rand(T, generator=g) < 0.6) if with_mask else torch.ones(T, dtype=torch.bool)
+    gl = torch.randn(T, generator=g) * mask.float()
+    gl[::7] = 0.0                                  # a named token may still have no gradient
+    kept = [int(mask[i:i + CHUNK].sum()) for i in range(0, T, CHUNK)] if counts_from_host else None
+
+    def run(backward):
+        h = hidden.to(device).requires_grad_(True)
+        w = weight.to(device).requires_grad_(True)
+        lp, ent = areal_amd.lm_head_logprobs_entropy(
+            h, w, labels.to(device), temperature, backward=backward,
+            grad_token_mask=mask.to(device) if with_mask else None, kept_per_chunk=kept if backward == "carry" else None)
+        (lp * gl.to(device)).sum().backward()
+        return lp.detach(), ent.detach(), h.grad, w.grad
+
+    lp_c, ent_c, dh_c, dw_c = run("carry")
+    lp_r, ent_r, dh_r, dw_r = run("recompute")
+    assert torch.equal(lp_c, lp_r) and torch.equal(ent_c, ent_r)     # the same tiles, the same merge
+    h_o = hidden.float().requires_grad_(True)
+    w_o = weight.float().requires_grad_(True)
+    o_lp, _ = oracle.logprobs_entropy(oracle.lmhead_logits(h_o, w_o), labels, temperature)
+    (o_lp * gl).sum().backward()
+    assert_within(lp_c, o_lp.detach(), 2e-3, "log-prob")
+    for name, got, other, want in (("d(hidden)", dh_c, dh_r, h_o.grad), ("d(W)", dw_c, dw_r, w_o.grad)):
+        assert got.dtype == torch.bfloat16
+        assert cosine(got.cpu(), want) > 0.9999, name
+        assert_same_magnitude(got, want, what=name)
+        assert cosine(got.cpu().float(), other.cpu().float()) > 0.99999, name
+    assert float(dh_c[~mask.to(device)].float().abs().sum()) == 0.0   # tokens outside the mask: no gradient
+
+
+def test_carried_backward_edge_cases(device):
+    T, H, V = 400, 64, 1088
+    hidden, weight, labels = _case(T, H, V, seed=77, w_std=0.3)
+    g = torch.Generator().manual_seed(1)
+    gl, gh = torch.randn(T, generator=g), 0.3 * torch.randn(T, generator=g)
+    args = (hidden.to(device), weight.to(device), labels.to(device))
+
+    def grads(backward, with_entropy, **kw):
+        h, w = args[0].clone().requires_grad_(True), args[1].clone().requires_grad_(True)
+        lp, ent = areal_amd.lm_head_logprobs_entropy(h, w, args[2], 0.9, backward=backward, **kw)
+        obj = (lp * gl.to(device)).sum() + ((ent * gh.to(device)).sum() if with_entropy else 0.0)
+        obj.backward(retain_graph=True)
+        return h, w, obj
+
+    # an entropy gradient is no multiple of the stored rows: the backward forms the logits again, same bits as recompute
+    hc, wc, _ = grads("carry", True)
+    hr, wr, _ = grads("recompute", True)
+    assert torch.equal(hc.grad, hr.grad) and torch.equal(wc.grad, wr.grad)
+    # the stored rows serve one backward
+    _, _, obj = grads("carry", False)
+    with pytest.raises(RuntimeError, match="already used by a backward"):
+        obj.backward()
+    # no gradient asked for: the plain forward, nothing kept
+    with torch.no_grad():
+        lp, _ = areal_amd.lm_head_logprobs_entropy(*args, 0.9, backward="carry")
+    assert not lp.requires_grad
+    # tokens outside grad_token_mask get no gradient even if the loss gives them one
+    mask = torch.zeros(T, dtype=torch.bool)
+    mask[50:200] = True
+    hm, wm, _ = grads("carry", False, grad_token_mask=mask.to(device))
+    assert float(hm.grad[:50].float().abs().sum()) == 0.0 and float(hm.grad[200:].float().abs().sum()) == 0.0
+    assert float(hm.grad[50:200].float().abs().sum()) > 0.0
+    with pytest.raises(ValueError, match="backward must be one of"):
+        areal_amd.lm_head_logprobs_entropy(*args, backward="panel")
+
+
+def test_carried_backward_redoes_a_chunk_that_does_not_fit(device):
+    """Labels with a log-prob below -80 in the first chunk: its rows are redone from the logits tiles (decided on the
+    device); the second chunk stays on the carried rows.  Both against the oracle and against recompute."""
+    T, H, V = CHUNK + 300, 64, 1088
+    g = torch.Generator().manual_seed(5)
+    hidden = torch.randn(T, H, generator=g)
+    hidden[:CHUNK] *= 12.0
+    hidden = hidden.bfloat16()
+    weight = (0.5 * torch.randn(V, H, generator=g)).bfloat16()
+    labels = torch.randint(0, V, (T,), generator=g)
+    ref_lp = oracle.logprobs(oracle.lmhead_logits(hidden, weight), labels)
+    assert int((ref_lp[:CHUNK] < -80).sum()) > 100 and float(ref_lp[CHUNK:].min()) > -60
+    mask = torch.rand(T, generator=g) < 0.7
+    gl = torch.randn(T, generator=g) * mask.float()
+
+    def run(backward):
+        h = hidden.to(device).requires_grad_(True)
+        w = weight.to(device).requires_grad_(True)
+        lp, _ = areal_amd.lm_head_logprobs_entropy(h, w, labels.to(device), backward=backward,
+                                                   grad_token_mask=mask.to(device))
+        (lp * gl.to(device)).sum().backward()
+        return h.grad.float(), w.grad.float()
+
+    got, ref = run("carry"), run("recompute")
+    h_o = hidden.float().requires_grad_(True)
+    w_o = weight.float().requires_grad_(True)
+    o_lp, _ = oracle.logprobs_entropy(oracle.lmhead_logits(h_o, w_o), labels)
+    (o_lp * gl).sum().backward()
+    for name, a, b, o in (("d(hidden)", got[0], ref[0], h_o.grad), ("d(W)", got[1], ref[1], w_o.grad)):
+        assert torch.isfinite(a).all(), name
+        assert cosine(a.cpu(), o) > 0.9999, name
+        assert_same_magnitude(a, o, what=name)
+    assert torch.equal(got[0][:CHUNK], ref[0][:CHUNK])   # the redone chunk: the rows of the recompute mode, bit for bit

@@ -230,23 +230,28 @@ def test_upstream_gradient_scales_both_gradients(device):
     assert torch.allclose(h2, -2.0 * h1, rtol=1e-2, atol=1e-12) and torch.allclose(w2, -2.0 * w1, rtol=1e-2, atol=1e-12)
 
 
-def test_sequence_level_runs_the_unfused_kernels(device):
-    hidden, weight, labels, prox, old, adv, mask = _inputs(300, 300, 64, 704, seed=5)
+@pytest.mark.parametrize("carry_limit", [16 << 30, 0])   # the op keeps its rows for the backward / forms the logits again
+def test_sequence_level_runs_the_unfused_kernels(device, carry_limit):
+    hidden, weight, labels, prox, old, adv, mask = _inputs(320, 300, 64, 704, seed=5)
     cu = torch.tensor([0, 100, 180, 300], dtype=torch.int32)
     h_d = hidden.to(device).requires_grad_(True)
     w_d = weight.to(device).requires_grad_(True)
     loss, stat = areal_amd.fused_lm_head_ppo_loss(
         h_d, w_d, labels.to(device), prox.to(device), old.to(device), adv.to(device), eps_clip=0.2,
-        loss_mask=mask.to(device), importance_sampling_level="sequence", cu_seqlens=cu.to(device))
+        loss_mask=mask.to(device), importance_sampling_level="sequence", cu_seqlens=cu.to(device),
+        carry_rows_limit_bytes=carry_limit)
     loss.backward()
+    hidden, labels = hidden[:300], labels[:300]            # the oracle sees the tokens without the batch padding
+    assert float(h_d.grad[300:].float().abs().sum()) == 0.0
+    dh = h_d.grad[:300]
     h = hidden.float().requires_grad_(True)
     w = weight.float().requires_grad_(True)
     lp, _ = oracle.logprobs_entropy(h @ w.t(), labels)
     o_loss, _ = oracle.ppo_actor_loss(lp, prox, old, adv, 0.2, mask, importance_sampling_level="sequence", cu_seqlens=cu)
     o_loss.backward()
     assert float(loss.detach()) == pytest.approx(float(o_loss.detach()), rel=1e-3)
-    assert cosine(h_d.grad.cpu().float(), h.grad) > 0.9999 and cosine(w_d.grad.cpu().float(), w.grad) > 0.9999
-    assert_same_magnitude(h_d.grad, h.grad, what="d(hidden)")
+    assert cosine(dh.cpu().float(), h.grad) > 0.9999 and cosine(w_d.grad.cpu().float(), w.grad) > 0.9999
+    assert_same_magnitude(dh, h.grad, what="d(hidden)")
     assert_same_magnitude(w_d.grad, w.grad, what="d(W)")
     with pytest.raises(ValueError, match="backward must be one of"):
         areal_amd.fused_lm_head_ppo_loss(h_d, w_d, labels.to(device), prox.to(device), old.to(device), adv.to(device),
