@@ -637,13 +637,13 @@ __global__ __launch_bounds__(256) void k_splitk_rows(const float* __restrict__ p
 // is zero.  k_compact_map numbers the tokens of a chunk that do have a mask (in order): out_rows[t] = position of
 // token t among them, or -1; act_rows[position] = t.  `limit` is the count the host sized the GEMMs with; tokens
 // beyond it are dropped.  A host count larger than what the mask holds leaves positions without a token: they get
-// act_rows = -1 (the gathers then produce zero rows and the scatters skip them), a row factor of zero when factors are
-// in use, and the workgroup clears their panel rows, which no tile writes, so that nothing stale (possibly not even
-// finite) enters the d_weight product.  One workgroup; mask has `act` entries (tokens at and after `act` have none).
+// act_rows = -1 (the gathers then produce zero rows and the scatters skip them) and a row factor of zero when factors
+// are in use; the true count goes to *total_out, and k_clear_surplus_rows, launched behind this kernel, clears their
+// panel rows, which no tile writes, so that nothing stale (possibly not even finite) enters the d_weight product.
+// One workgroup; mask has `act` entries (tokens at and after `act` have none).
 __global__ __launch_bounds__(1024) void k_compact_map(const uint8_t* __restrict__ mask, int act, int n_tok, int limit,
                                                       int32_t* __restrict__ out_rows, int32_t* __restrict__ act_rows,
-                                                      float* __restrict__ row_factor, u32x4_t* __restrict__ panel,
-                                                      int64_t panel_ld) {
+                                                      float* __restrict__ row_factor, int32_t* __restrict__ total_out) {
   __shared__ int wave_sum[16];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int per = (n_tok + 1023) / 1024;
@@ -669,14 +669,33 @@ __global__ __launch_bounds__(1024) void k_compact_map(const uint8_t* __restrict_
   }
   int total = 0;
   for (int w = 0; w < 16; ++w) total += wave_sum[w];
-  if (total >= limit) return;  // the usual case: every position has its token
-  for (int p = total + tid; p < limit; p += 1024) {
+  if (tid == 0) *total_out = total < limit ? total : limit;
+  for (int p = total + tid; p < limit; p += 1024) {  // the usual case: none
     act_rows[p] = -1;
     if (row_factor) row_factor[p] = 0.f;
   }
+}
+
+// Panel rows [*total, limit) are rows without a token (see k_compact_map): cleared, one workgroup per row at a time.
+// In the usual case (*total == limit) every workgroup returns at once.
+__global__ __launch_bounds__(256) void k_clear_surplus_rows(const int32_t* __restrict__ total, int limit,
+                                                            u32x4_t* __restrict__ panel, int64_t panel_ld) {
   const u32x4_t zero = {0u, 0u, 0u, 0u};
   const int64_t vec = panel_ld / 8;
-  for (int64_t i = (int64_t)total * vec + tid; i < (int64_t)limit * vec; i += 1024) panel[i] = zero;
+  for (int64_t r = (int64_t)*total + blockIdx.x; r < limit; r += gridDim.x)
+    for (int64_t i = threadIdx.x; i < vec; i += 256) panel[r * vec + i] = zero;
+}
+
+// numbering of the tokens with a panel row, and the rows without a token cleared (both kernels)
+static void launch_compact_map(hipStream_t st, const uint8_t* mask, int64_t act, int64_t n_tok, int64_t limit,
+                               int32_t* out_rows, int32_t* act_rows, float* row_factor, int32_t* total_word,
+                               uint16_t* panel, int64_t panel_ld) {
+  hipLaunchKernelGGL(k_compact_map, dim3(1), dim3(1024), 0, st, mask, (int)act, (int)n_tok, (int)limit, out_rows, act_rows,
+                     row_factor, total_word);
+  const int64_t blocks = limit < 512 ? limit : 512;
+  if (blocks > 0)
+    hipLaunchKernelGGL(k_clear_surplus_rows, dim3((unsigned)blocks), dim3(256), 0, st, total_word, (int)limit,
+                       (u32x4_t*)panel, panel_ld);
 }
 
 // dst[r, :] = scale[r] * src[rows[r], :] (H % 8 == 0); rows == nullptr: row r itself (a negative entry: a zero row);
@@ -747,6 +766,7 @@ struct Workspace {
   int64_t off_pn;                       // smallest logit per block [blocks][chunk] (only when the extrema are asked for)
   int64_t fwd_stats_bytes;              // what the forward needs when it also returns the extrema of the logits
   int64_t off_rowf, off_flag;           // carry mode: factor per panel row; the chunk's redo flag
+  int64_t off_total;                    // number of tokens the mask of the chunk really holds (k_compact_map)
   int64_t off_rows;                     // out_rows, act_rows (2 x chunk int32)
   int64_t off_panel;                    // d(logits) rows [chunk, V]
   int64_t off_hc;                       // the hidden rows of the tokens with gradient, closed up [chunk, H]
@@ -774,6 +794,7 @@ static Workspace plan(int64_t T, int64_t H, int64_t V, bool external_panel = fal
   w.fwd_stats_bytes = off;
   w.off_rowf = off;    off += up(w.chunk * 4);  // factor per panel row (carry mode)
   w.off_flag = off;    off += 256;              // the chunk's "redo by recompute" flag
+  w.off_total = off;   off += 256;
   w.off_rows = off;    off += up(2 * w.chunk * 4);
   w.panel_ld = round_up(V, 8);
   w.off_panel = off;   off += external_panel ? 0 : up(w.chunk * w.panel_ld * 2);
@@ -1138,8 +1159,8 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
       launch_zero(st, dh, n_tok * H * 2);
       continue;
     }
-    hipLaunchKernelGGL(k_compact_map, dim3(1), dim3(1024), 0, st, row_has_gradient + t0, (int)n_tok, (int)n_tok, (int)kept,
-                       out_rows, act_rows, (float*)nullptr, (u32x4_t*)(ws + w.off_panel), w.panel_ld);
+    launch_compact_map(st, row_has_gradient + t0, n_tok, n_tok, kept, out_rows, act_rows, nullptr,
+                       (int32_t*)(ws + w.off_total), ws_panel, w.panel_ld);
     recompute_panel(st, w, ws, ws_panel, weight, hid, n_tok, act_rows, kept, H, V, a);
     launch_zero(st, dh, n_tok * H * 2);  // the rows of the other tokens
     panel_gradients(st, w, ws, ws_panel, weight, hid, act_rows, nullptr, kept, H, V, dh, dw.acc, dw.acc_f32, first);
@@ -1198,8 +1219,8 @@ extern "C" int aa_lmhead_fwd_carry(const void* hidden, const void* weight, int64
     if (kept_per_chunk) {
       rows = kept_per_chunk[chunk_index];
       rows = rows < 0 ? 0 : (rows > n_tok ? n_tok : rows);
-      hipLaunchKernelGGL(k_compact_map, dim3(1), dim3(1024), 0, st, row_has_gradient + t0, (int)n_tok, (int)n_tok, (int)rows,
-                         out_rows, act_rows, (float*)nullptr, (u32x4_t*)chunk_panel, w.panel_ld);
+      launch_compact_map(st, row_has_gradient + t0, n_tok, n_tok, rows, out_rows, act_rows, nullptr,
+                         (int32_t*)(ws + w.off_total), chunk_panel, w.panel_ld);
     }
     TileArgs a = stats_args(w, ws, labels + t0, inv_temperature, vocab_min != nullptr);
     a.panel = chunk_panel;
@@ -1261,8 +1282,8 @@ extern "C" int aa_lmhead_bwd_carry(const void* hidden, const void* weight, int64
         continue;
       }
       // the same numbering as in the forward (the mask has not changed); surplus rows get a factor of zero
-      hipLaunchKernelGGL(k_compact_map, dim3(1), dim3(1024), 0, st, row_has_gradient + t0, (int)n_tok, (int)n_tok, (int)rows,
-                         out_rows, act_rows, row_factor, (u32x4_t*)chunk_panel, w.panel_ld);
+      launch_compact_map(st, row_has_gradient + t0, n_tok, n_tok, rows, out_rows, act_rows, row_factor,
+                         (int32_t*)(ws + w.off_total), chunk_panel, w.panel_ld);
       row_of_token = out_rows;
       token_of_row = act_rows;
     }
@@ -1341,8 +1362,8 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
     if (kept_per_chunk) {
       rows = kept_per_chunk[chunk_index];
       rows = rows < 0 ? 0 : (rows > act ? act : rows);
-      hipLaunchKernelGGL(k_compact_map, dim3(1), dim3(1024), 0, st, at(mask_eff), (int)act, (int)n_tok, (int)rows, out_rows,
-                         act_rows, carry ? row_factor : (float*)nullptr, (u32x4_t*)panel, w.panel_ld);
+      launch_compact_map(st, at(mask_eff), act, n_tok, rows, out_rows, act_rows, carry ? row_factor : nullptr,
+                         (int32_t*)(ws + w.off_total), panel, w.panel_ld);
       row_of_token = out_rows;
       token_of_row = act_rows;
     }
