@@ -21,6 +21,7 @@ from .functional import (
     gather_logprobs_entropy_stats,
     lm_head_chunk_tokens,
     lm_head_logprobs_entropy,
+    lm_head_logprobs_entropy_stats,
     ppo_actor_loss_fn,
 )
 
@@ -525,6 +526,47 @@ def compute_loss_with(logits: torch.Tensor, model_inputs: dict[str, Any], mb_inp
             if pad_length > 0:
                 logp, entropy, vmin, vmax = (t[:-pad_length] for t in (logp, entropy, vmin, vmax))
         out = loss_fn(logp, entropy, mb_input, vocab_min_logits=vmin, vocab_max_logits=vmax)
+    scale = local_weight / total_loss_weight * loss_multiplier
+    if isinstance(out, tuple):
+        return out[0] * scale, out[1]
+    return out * scale
+
+
+def compute_lm_head_loss_with(hidden: torch.Tensor, weight: torch.Tensor, model_inputs: dict[str, Any],
+                              mb_input: dict[str, Any], pad_length: int, loss_fn, loss_weight_fn,
+                              total_loss_weight: torch.Tensor | float, temperature: float = 1.0,
+                              loss_multiplier: float = 1.0, backward: str = "carry",
+                              grad_token_mask: torch.Tensor | None = None, kept_per_chunk: list[int] | None = None):
+    """``compute_loss_with`` one step earlier in the model: any loss function of the reference's form
+    (``grpo_loss_fn`` with sequence-level ratios, SAPO, M2PO or distillation terms, ``compute_packed_sft_loss``, a custom
+    one) on the final hidden states ``[T_pad, H]`` and the lm_head weight ``[V, H]``, without the ``[T_pad, V]`` logits:
+    log-probs, entropy and the vocabulary extrema come from ``lm_head_logprobs_entropy_stats``, the batch padding is
+    trimmed, ``loss_fn(logprobs, entropy, mb_input, vocab_min_logits=..., vocab_max_logits=...)`` is called as the
+    engine calls it (fsdp_engine.py:2032-2040) and its result scaled by ``local_weight / total_loss_weight *
+    loss_multiplier``.  A micro-batch of weight 0 returns a zero that keeps the graph to ``hidden`` and ``weight``.
+
+    ``backward="carry"`` (default): the op keeps the bf16 probability ratios of the tokens named by ``grad_token_mask``
+    (default: ``mb_input["loss_mask"]``; tokens outside it get no gradient) from its forward to its backward, which is
+    then two GEMMs instead of three; ``kept_per_chunk``: their number per chunk of ``lm_head_chunk_tokens()`` tokens,
+    if the host knows it (else it is read back).  ``"recompute"`` keeps nothing and forms the logits again."""
+    if hidden.ndim == 3 and hidden.shape[0] == 1:
+        hidden = hidden.squeeze(0)
+    local_weight = loss_weight_fn(mb_input)
+    if local_weight == 0:
+        return hidden.mean() * 0.0 + weight.mean() * 0.0
+    if grad_token_mask is None and backward == "carry":
+        grad_token_mask = mb_input.get("loss_mask")
+    if grad_token_mask is not None:
+        grad_token_mask = grad_token_mask.reshape(-1).ne(0)
+        if pad_length > 0:
+            grad_token_mask = torch.nn.functional.pad(grad_token_mask, (0, hidden.shape[0] - grad_token_mask.shape[0]))
+    logp, entropy, vmin, vmax = lm_head_logprobs_entropy_stats(
+        hidden, weight, rolled_labels(model_inputs), temperature, backward=backward,
+        grad_token_mask=grad_token_mask if backward == "carry" else None,
+        kept_per_chunk=kept_per_chunk if backward == "carry" else None)
+    if pad_length > 0:
+        logp, entropy, vmin, vmax = (t[:-pad_length] for t in (logp, entropy, vmin, vmax))
+    out = loss_fn(logp, entropy, mb_input, vocab_min_logits=vmin, vocab_max_logits=vmax)
     scale = local_weight / total_loss_weight * loss_multiplier
     if isinstance(out, tuple):
         return out[0] * scale, out[1]

@@ -776,3 +776,67 @@ def test_engine_contract_of_the_lm_head_step(device, with_host_mask, with_rs):
     # forward-only pass of the same micro-batch
     lp = engine_glue.compute_lm_head_logprobs(hidden.to(device), weight.to(device), {"input_ids": input_ids.to(device)})
     assert_within(lp[:n], o_lp[:n], 2e-3, "log-prob of the forward-only pass")
+
+
+@pytest.mark.parametrize("backward", ["carry", "recompute"])
+@pytest.mark.parametrize("variant", ["sapo", "gspo", "ppo_m2po"])
+def test_any_loss_function_on_the_hidden_states(device, variant, backward):
+    """``engine_glue.compute_lm_head_loss_with``: the actor's loss function in its SAPO, sequence-level (GSPO) and
+    M2PO forms on hidden states and lm_head weight, against ``compute_loss_with`` on fp32 logits ``hidden @ W.T`` formed
+    by torch (that path is held to the oracle in its own tests): same loss, same statistics, same gradients."""
+    import functools
+
+    lengths, pad = [90, 60, 130], 40
+    n = sum(lengths)
+    T, H, V = n + pad, 64, 1097
+    g = torch.Generator().manual_seed(13)
+    input_ids = torch.randint(0, V, (1, T), generator=g)
+    labels = torch.cat([input_ids[0, 1:], input_ids[0, :1]])
+    hidden = torch.randn(T, H, generator=g).bfloat16()
+    weight = (0.3 * torch.randn(V, H, generator=g)).bfloat16()
+    ref = oracle.logprobs(oracle.lmhead_logits(hidden, weight), labels)[:n]
+    mb = dict(
+        input_ids=input_ids[0, :n], loss_mask=(torch.rand(n, generator=g) < 0.6),
+        logprobs=ref + 0.1 * torch.randn(n, generator=g), prox_logp=ref + 0.05 * torch.randn(n, generator=g),
+        advantages=torch.randn(n, generator=g), cu_seqlens=torch.tensor([0, 90, 150, 280], dtype=torch.int32),
+    )
+    mb_d = {k: v.to(device) for k, v in mb.items()}
+    kw = dict(eps_clip=0.2, eps_clip_higher=0.28, c_clip=3.0)
+    if variant == "sapo":
+        kw.update(use_sapo_loss=True, sapo_tau_pos=1.0, sapo_tau_neg=1.05)
+    elif variant == "gspo":
+        kw.update(importance_sampling_level="sequence")
+    else:
+        kw.update(m2_threshold=0.04, use_decoupled_loss=True)
+    loss_fn = functools.partial(engine_glue.grpo_loss_fn, **kw)
+    weight_fn = lambda d: d["loss_mask"].count_nonzero()
+    model_inputs = {"input_ids": input_ids.to(device)}
+    total_w = torch.tensor(500.0, device=device)
+
+    h = hidden.to(device).requires_grad_(True)
+    w = weight.to(device).requires_grad_(True)
+    loss, stat = engine_glue.compute_lm_head_loss_with(h, w, model_inputs, mb_d, pad, loss_fn, weight_fn, total_w,
+                                                       temperature=0.9, backward=backward)
+    loss.backward()
+    h2 = hidden.float().to(device).requires_grad_(True)     # fp32 leaves: the gradients to compare with are not rounded
+    w2 = weight.float().to(device).requires_grad_(True)
+    logits = h2 @ w2.t()
+    loss2, stat2 = engine_glue.compute_loss_with(logits, model_inputs, mb_d, pad, loss_fn, weight_fn, total_w,
+                                                 temperature=0.9)
+    loss2.backward()
+    assert float(loss.detach()) == pytest.approx(float(loss2.detach()), rel=1e-3, abs=1e-7)
+    for k in ("loss", "importance_weight", "approx_kl"):
+        assert_within(stat[k], stat2[k], 2e-3, k)
+    assert torch.equal(stat["clip_mask"], stat2["clip_mask"])
+    assert cosine(h.grad.float().cpu(), h2.grad.float().cpu()) > 0.9999
+    assert cosine(w.grad.float().cpu(), w2.grad.float().cpu()) > 0.9999
+    assert_same_magnitude(h.grad, h2.grad.float(), what="d(hidden)")
+    assert_same_magnitude(w.grad, w2.grad.float(), what="d(W)")
+    assert float(h.grad[n:].float().abs().sum()) == 0.0
+    # a micro-batch of weight zero keeps the graph alive
+    mb_d["loss_mask"] = torch.zeros(n, dtype=torch.bool, device=device)
+    h = hidden.to(device).requires_grad_(True)
+    w = weight.to(device).requires_grad_(True)
+    z = engine_glue.compute_lm_head_loss_with(h, w, model_inputs, mb_d, pad, loss_fn, weight_fn, total_w)
+    z.backward()
+    assert float(z.detach()) == 0.0 and float(h.grad.float().abs().max()) == 0.0
