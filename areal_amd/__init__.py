@@ -45,6 +45,7 @@ from .tree import (
     merge_packed_tree_results,
     tree_sequence_pairs,
 )
+from .sapo import fused_lm_head_sapo_loss, fused_logprobs_sapo_loss
 from .sft import fused_lm_head_sft_loss, fused_logprobs_sft_loss, sft_loss_fn
 from ._native import NativeLibraryError
 
@@ -55,6 +56,8 @@ __all__ = [
     "gather_packed_tree_vocab_stats",
     "merge_packed_tree_results",
     "KLEstimator",
+    "fused_lm_head_sapo_loss",
+    "fused_logprobs_sapo_loss",
     "fused_lm_head_sft_loss",
     "fused_logprobs_sft_loss",
     "sft_loss_fn",

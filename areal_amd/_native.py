@@ -37,6 +37,8 @@ class PpoParams(C.Structure):
         ("has_c_clip", C.c_int32),
         ("has_behave_weight", C.c_int32),
         ("loss_kind", C.c_int32),
+        ("sapo_tau_pos", C.c_float),
+        ("sapo_tau_neg", C.c_float),
     ]
 
 

@@ -420,8 +420,11 @@ __global__ __launch_bounds__(1024) void k_token_loss(const float* __restrict__ p
       a.flags[t] = 0;
       g = on ? (-1.f / fn) * gscale : 0.f;
     } else {
-      const float r = on ? expf(lp - a.prox_logp[t]) : 0.f;
-      const Surrogate sg = surrogate(r, a.adv[t], a.P.has_behave_weight ? a.behave_w[t] : 1.f, a.P);
+      // the clipped surrogate sees a ratio of zero at masked tokens; SAPO's ratio is not masked (functional.py:509, 600)
+      const bool sapo = a.P.loss_kind == AA_LOSS_SAPO;
+      const float r = (on || sapo) ? expf(lp - a.prox_logp[t]) : 0.f;
+      const Surrogate sg = sapo ? sapo_surrogate(r, a.adv[t], a.P)
+                                : surrogate(r, a.adv[t], a.P.has_behave_weight ? a.behave_w[t] : 1.f, a.P);
       a.stat_loss[t] = sg.loss;
       a.ratio[t] = r;
       a.flags[t] = (uint8_t)(((sg.clip && on) ? 1 : 0) | ((sg.dual && on) ? 2 : 0));
@@ -1324,7 +1327,11 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
   if (!params || !n_valid || !logp) return AA_ERR_INVALID_ARGUMENT;
   if (T_active < 0 || T_active > T || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
   if (backward_mode != AA_LMHEAD_RECOMPUTE && backward_mode != AA_LMHEAD_CARRY) return AA_ERR_INVALID_ARGUMENT;
-  if (params->loss_kind != AA_LOSS_PPO && params->loss_kind != AA_LOSS_NLL) return AA_ERR_INVALID_ARGUMENT;
+  if (params->loss_kind != AA_LOSS_PPO && params->loss_kind != AA_LOSS_NLL && params->loss_kind != AA_LOSS_SAPO)
+    return AA_ERR_INVALID_ARGUMENT;
+  if (params->loss_kind == AA_LOSS_SAPO &&
+      (params->has_behave_weight || !(params->sapo_tau_pos > 0.f) || !(params->sapo_tau_neg > 0.f)))
+    return AA_ERR_INVALID_ARGUMENT;
   const bool nll = params->loss_kind == AA_LOSS_NLL;  // prox_logp and adv are not used by that loss
   if (T_active > 0 && (!mask_eff || !stat_loss || !ratio || !flags)) return AA_ERR_INVALID_ARGUMENT;
   if (T_active > 0 && !nll && (!prox_logp || !adv)) return AA_ERR_INVALID_ARGUMENT;

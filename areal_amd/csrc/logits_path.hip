@@ -412,8 +412,10 @@ __device__ __forceinline__ float fused_token_tail(const FusedTokenArgs& a, int64
     }
     return m ? (-1.f / fn) * gscale : 0.f;
   }
-  const float r = m ? expf(lp - in.prox) : 0.f;
-  const Surrogate s = surrogate(r, in.adv, in.w, a.P);
+  // the clipped surrogate sees a ratio of zero at masked tokens (functional.py:509); SAPO's ratio is not masked (:600)
+  const bool sapo = a.P.loss_kind == AA_LOSS_SAPO;
+  const float r = (m || sapo) ? expf(lp - in.prox) : 0.f;
+  const Surrogate s = sapo ? sapo_surrogate(r, in.adv, a.P) : surrogate(r, in.adv, in.w, a.P);
   if (writer) {
     a.stat_loss[t] = s.loss;
     a.ratio[t] = r;
@@ -1171,7 +1173,11 @@ extern "C" int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int
   if (!params || !n_valid || !logp || !dlogits) return AA_ERR_INVALID_ARGUMENT;
   if (T_active < 0 || T_active > T || !(inv_temperature > 0.f)) return AA_ERR_INVALID_ARGUMENT;
   // the per-token arrays have T_active entries: with no active token they may be absent
-  if (params->loss_kind != AA_LOSS_PPO && params->loss_kind != AA_LOSS_NLL) return AA_ERR_INVALID_ARGUMENT;
+  if (params->loss_kind != AA_LOSS_PPO && params->loss_kind != AA_LOSS_NLL && params->loss_kind != AA_LOSS_SAPO)
+    return AA_ERR_INVALID_ARGUMENT;
+  if (params->loss_kind == AA_LOSS_SAPO &&
+      (params->has_behave_weight || !(params->sapo_tau_pos > 0.f) || !(params->sapo_tau_neg > 0.f)))
+    return AA_ERR_INVALID_ARGUMENT;
   if (T_active > 0 && (!mask_eff || !stat_loss || !ratio || !flags)) return AA_ERR_INVALID_ARGUMENT;
   if (params->loss_kind == AA_LOSS_NLL) {
     if (params->has_behave_weight) return AA_ERR_INVALID_ARGUMENT;

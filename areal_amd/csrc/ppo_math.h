@@ -68,4 +68,18 @@ __device__ __forceinline__ Surrogate surrogate(float r, float adv, float behave_
   return o;
 }
 
+// SAPO (areal/utils/functional/functional.py:607-620): the clip is replaced by a sigmoid gate of the ratio, scaled by
+// 4 / tau so that its slope at r = 1 is 1; tau depends on the sign of the advantage (adv > 0, as torch.where(adv > 0)
+// selects: NaN and 0 take the negative branch).  d/dr [4 / tau * sigmoid(tau (r - 1))] = 4 s (1 - s).
+__device__ __forceinline__ Surrogate sapo_surrogate(float r, float adv, const aa_ppo_params& P) {
+  const float tau = adv > 0.f ? P.sapo_tau_pos : P.sapo_tau_neg;
+  const float sg = 1.f / (1.f + expf(-tau * (r - 1.f)));
+  Surrogate o;
+  o.loss = -(sg * (4.f / tau)) * adv;
+  o.dloss_dr = -4.f * sg * (1.f - sg) * adv;
+  o.clip = false;
+  o.dual = false;
+  return o;
+}
+
 }  // namespace aa

@@ -49,8 +49,17 @@ typedef enum { AA_RS_AGG_SUM = 0, AA_RS_AGG_MEAN = 1, AA_RS_AGG_MAX = 2 } aa_rs_
  *                (areal/trainer/sft/lm_engine.py:93-96): -logp on the selected
  *                tokens, divided by (*n_valid + 1e-5).  stat_loss = -logp on
  *                the selected tokens and 0 elsewhere, ratio = 0, flags = 0; prox_logp, adv and behave_w are not
- *                used and may be NULL. */
-typedef enum { AA_LOSS_PPO = 0, AA_LOSS_NLL = 1 } aa_loss_kind;
+ *                used and may be NULL;
+ *   AA_LOSS_SAPO the token-level loss of sapo_loss_fn
+ *                (areal/utils/functional/functional.py:589-622): with r =
+ *                exp(logp - prox_logp) (the caller passes the behaviour
+ *                log-probs there: SAPO has no proximal policy), -adv * 4 / tau *
+ *                sigmoid(tau (r - 1)) with tau = sapo_tau_pos where adv > 0 and
+ *                sapo_tau_neg elsewhere, divided by max(*n_valid, 1).  ratio
+ *                and stat_loss are those of the reference at every token
+ *                (the ratio is not zeroed at masked tokens), flags = 0;
+ *                has_behave_weight must be 0. */
+typedef enum { AA_LOSS_PPO = 0, AA_LOSS_NLL = 1, AA_LOSS_SAPO = 2 } aa_loss_kind;
 
 /* Clipped-surrogate parameters of ppo_actor_loss_fn
  * (areal/utils/functional/functional.py:516-532). */
@@ -61,6 +70,8 @@ typedef struct {
   int32_t has_c_clip;
   int32_t has_behave_weight; /* multiply the loss by behave_w (rejection sampling on) */
   int32_t loss_kind;   /* aa_loss_kind; aa_ppo_loss accepts AA_LOSS_PPO only */
+  float sapo_tau_pos;  /* AA_LOSS_SAPO: gate temperatures, both > 0      */
+  float sapo_tau_neg;
 } aa_ppo_params;
 
 /* Library version (major * 10000 + minor * 100 + patch). */

@@ -97,8 +97,11 @@ def test_argument_validation_of_the_sibling_entry_points_without_gpu():
     assert lib.aa_vocab_partials_combine(p, p, p, 0, 4, p, z, z, z, z) == bad       # no slice
     assert lib.aa_vocab_partials_combine(z, p, p, 2, 4, p, z, z, z, z) == bad
     assert lib.aa_vocab_partials_combine(z, z, z, 2, 0, p, z, z, z, z) == ok
-    params = _native.PpoParams(clip_lo=0.8, clip_hi=1.2, loss_kind=2)
+    params = _native.PpoParams(clip_lo=0.8, clip_hi=1.2, loss_kind=7)
     assert lib.aa_logits_ppo_fused(p, 0, 4, 4096, 4096, p, 1.0, 4, p, p, p, z, ctypes.byref(params), p, z, p, z, z, z,
                                    p, p, p, p, z, z) == bad                             # unknown loss kind
+    params = _native.PpoParams(loss_kind=2, sapo_tau_pos=1.0, sapo_tau_neg=0.0)
+    assert lib.aa_logits_ppo_fused(p, 0, 4, 4096, 4096, p, 1.0, 4, p, p, p, z, ctypes.byref(params), p, z, p, z, z, z,
+                                   p, p, p, p, z, z) == bad                             # SAPO gate temperature of zero
     params = _native.PpoParams(clip_lo=0.8, clip_hi=1.2, loss_kind=1)
     assert lib.aa_ppo_loss(p, p, p, p, z, 4, z, 0, 0, ctypes.byref(params), p, p, p, p, p, z) == 2   # unsupported

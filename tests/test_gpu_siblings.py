@@ -371,3 +371,98 @@ def test_grpo_loss_fn_reports_the_logging_scopes(device):
     data.pop("versions")
     _, st = G.grpo_loss_fn(lp.to(device).requires_grad_(True), ent, data, prox_logp_method="recompute", **kw)
     assert list(st["reduced"]["compute_logp"]) == ["prox_logp_gt"] and st["reduced"]["version_stats"] == {}
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# SAPO fused with the log-prob op (one pass over the logits) and with the lm_head (no logits in memory)
+# ---------------------------------------------------------------------------------------------------------------
+_SAPO_STATS = ("loss", "importance_weight", "approx_kl", "sapo_soft_gate", "sapo_scaled_gate_pos", "sapo_scaled_gate_neg")
+
+
+def _sapo_case(T_pad, T, V, seed):
+    import oracle
+
+    g = torch.Generator().manual_seed(seed)
+    logits = (2.0 * torch.randn(T_pad, V, generator=g)).bfloat16()
+    labels = torch.randint(0, V, (T_pad,), generator=g)
+    ref = oracle.logprobs(logits, labels)[:T]
+    old = ref + 0.3 * torch.randn(T, generator=g)
+    adv = torch.randn(T, generator=g)
+    adv[::9] = 0.0                                   # adv == 0 takes the negative gate, as torch.where(adv > 0) does
+    mask = torch.rand(T, generator=g) < 0.7
+    return logits, labels, old, adv, mask
+
+
+@pytest.mark.parametrize("T_pad,T,V,temperature,scale,inplace", [
+    (40, 40, 9000, 1.0, None, False),       # two-pass rows
+    (300, 280, 32768, 0.8, 0.37, False),    # register-resident rows, batch padding, loss scale
+    (70, 64, 50257, 1.0, None, True),       # generic rows (V % 8 != 0), gradient written over the logits
+])
+def test_fused_logits_sapo_matches_oracle(device, T_pad, T, V, temperature, scale, inplace):
+    import oracle
+    from helpers import assert_same_magnitude, assert_within
+
+    logits, labels, old, adv, mask = _sapo_case(T_pad, T, V, seed=T + V)
+    x = logits.to(device).requires_grad_(True)
+    loss, stat = areal_amd.fused_logprobs_sapo_loss(
+        x, labels.to(device), old.to(device), adv.to(device), 1.0, 1.05, mask.to(device), temperature=temperature,
+        loss_scale=scale, inplace_backward=inplace)
+    loss.backward()
+    z = logits.float().requires_grad_(True)
+    o_lp, o_ent = oracle.logprobs_entropy(z, labels, temperature)
+    w_loss, w_stat = S.sapo_loss(o_lp[:T], old, adv, 1.0, 1.05, mask)
+    (w_loss * (1.0 if scale is None else scale)).backward()
+    assert float(loss.detach()) == pytest.approx(float(w_loss.detach()) * (1.0 if scale is None else scale), rel=1e-3)
+    assert_within(stat["logprobs"], o_lp[:T].detach(), 2e-3, "log-prob")
+    assert_within(stat["entropy"], o_ent[:T].detach(), 2e-3, "entropy")
+    for k in _SAPO_STATS:                                        # at every token, masked ones included
+        assert_within(stat[k], w_stat[k], 2e-3, k)
+    assert not stat["clip_mask"].any() and not stat["dual_clip_mask"].any()
+    assert cosine(x.grad.float().cpu(), z.grad) > 0.9999
+    assert_same_magnitude(x.grad, z.grad, what="d(logits)")
+    assert float(x.grad[T:].float().abs().sum()) == 0.0 and float(x.grad[:T][~mask.to(device)].float().abs().sum()) == 0.0
+    if inplace:
+        assert torch.equal(x.detach(), x.grad)
+    # without a gradient to produce: the forward kernel and the loss on its log-probs
+    with torch.no_grad():
+        l2, s2 = areal_amd.fused_logprobs_sapo_loss(logits.to(device), labels.to(device), old.to(device), adv.to(device),
+                                                    1.0, 1.05, mask.to(device), temperature=temperature, loss_scale=scale)
+    assert float(l2) == pytest.approx(float(loss.detach()), rel=1e-5) and set(s2) == set(stat)
+    with pytest.raises(ValueError, match="must be positive"):
+        areal_amd.fused_logprobs_sapo_loss(x, labels.to(device), old.to(device), adv.to(device), 1.0, 0.0, mask.to(device))
+
+
+@pytest.mark.parametrize("backward", ["carry", "recompute"])
+def test_fused_lm_head_sapo_matches_oracle(device, backward):
+    import oracle
+    from areal_amd import _native
+    from helpers import assert_same_magnitude, assert_within
+
+    chunk = int(_native.load().aa_lmhead_chunk_tokens())
+    T_pad, T, H, V = chunk + 200, chunk + 130, 64, 641           # two token chunks, a vocabulary that is no multiple of 8
+    g = torch.Generator().manual_seed(4)
+    hidden = torch.randn(T_pad, H, generator=g).bfloat16()
+    weight = (0.3 * torch.randn(V, H, generator=g)).bfloat16()
+    labels = torch.randint(0, V, (T_pad,), generator=g)
+    ref = oracle.logprobs(oracle.lmhead_logits(hidden, weight), labels)[:T]
+    old = ref + 0.3 * torch.randn(T, generator=g)
+    adv = torch.randn(T, generator=g)
+    mask = torch.rand(T, generator=g) < 0.7
+    h = hidden.to(device).requires_grad_(True)
+    w = weight.to(device).requires_grad_(True)
+    loss, stat = areal_amd.fused_lm_head_sapo_loss(h, w, labels.to(device), old.to(device), adv.to(device), 1.0, 1.05,
+                                                   mask.to(device), temperature=0.9, loss_scale=0.5, backward=backward)
+    loss.backward()
+    h_o = hidden.float().requires_grad_(True)
+    w_o = weight.float().requires_grad_(True)
+    o_lp, o_ent = oracle.logprobs_entropy(oracle.lmhead_logits(h_o, w_o), labels, 0.9)
+    w_loss, w_stat = S.sapo_loss(o_lp[:T], old, adv, 1.0, 1.05, mask)
+    (w_loss * 0.5).backward()
+    assert float(loss.detach()) == pytest.approx(float(w_loss.detach()) * 0.5, rel=1e-3)
+    assert_within(stat["logprobs"], o_lp[:T].detach(), 2e-3, "log-prob")
+    for k in _SAPO_STATS:
+        assert_within(stat[k], w_stat[k], 2e-3, k)
+    assert cosine(h.grad.float().cpu(), h_o.grad) > 0.9999 and cosine(w.grad.float().cpu(), w_o.grad) > 0.9999
+    assert_same_magnitude(h.grad, h_o.grad, what="d(hidden)")
+    assert_same_magnitude(w.grad, w_o.grad, what="d(W)")
+    assert float(h.grad[T:].float().abs().sum()) == 0.0
