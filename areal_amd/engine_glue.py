@@ -58,6 +58,9 @@ def compute_logprobs_and_loss(
     loss_multiplier: float = 1.0,
     fused: bool = True,
     inplace_backward: bool = False,
+    use_sapo_loss: bool = False,
+    sapo_tau_pos: float = 1.0,
+    sapo_tau_neg: float = 1.05,
 ) -> tuple[torch.Tensor, dict]:
     """Scaled PPO loss of one micro-batch and its stat dict (fsdp_engine.py:1977-2046 with
     ``loss_fn = grpo_loss_fn`` and ``loss_weight_fn = loss_mask.count_nonzero``, actor.py:345-364).
@@ -65,7 +68,8 @@ def compute_logprobs_and_loss(
     ``logits`` is ``[T_pad, V]``; ``mb_input`` holds the un-padded ``[T]`` tensors ``loss_mask``, ``logprobs``
     (behaviour policy), ``prox_logp``, ``advantages`` and ``cu_seqlens``.  An all-masked micro-batch returns
     ``logits.mean() * 0`` like the reference (fsdp_engine.py:1988-1989).  ``inplace_backward``: the gradient is
-    written over the logits, see ``fused_logprobs_ppo_loss``.
+    written over the logits, see ``fused_logprobs_ppo_loss``.  ``use_sapo_loss`` (token level, fused): the SAPO gate in
+    place of the clip, on the behaviour log-probs (actor.py:448-462: SAPO takes ``old_logp``, no proximal policy).
     """
     loss_mask = mb_input["loss_mask"].bool()
     local_weight = loss_mask.count_nonzero()
@@ -74,9 +78,17 @@ def compute_logprobs_and_loss(
     labels = rolled_labels(model_inputs)
     old_logp = mb_input["logprobs"]
     prox_logp = mb_input.get("prox_logp")
-    if prox_logp is None:
+    if prox_logp is None and not use_sapo_loss:
         raise ValueError("prox_logp is None: only the recomputed proximal log-probs are supported here")
     scale = local_weight / total_loss_weight * loss_multiplier
+    if use_sapo_loss and fused and importance_sampling_level == "token":
+        from .sapo import fused_logprobs_sapo_loss
+
+        return fused_logprobs_sapo_loss(logits, labels, old_logp, mb_input["advantages"], sapo_tau_pos, sapo_tau_neg,
+                                        loss_mask, temperature=temperature, loss_scale=scale,
+                                        inplace_backward=inplace_backward)
+    if use_sapo_loss:
+        raise ValueError("use_sapo_loss is built for the fused token-level call; use compute_loss_with(grpo_loss_fn) otherwise")
     kw = dict(
         eps_clip=eps_clip, eps_clip_higher=eps_clip_higher, c_clip=c_clip, rejection_sampling=rejection_sampling,
         importance_sampling_level=importance_sampling_level, cu_seqlens=mb_input.get("cu_seqlens"),

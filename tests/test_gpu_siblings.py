@@ -466,3 +466,24 @@ def test_fused_lm_head_sapo_matches_oracle(device, backward):
     assert_same_magnitude(h.grad, h_o.grad, what="d(hidden)")
     assert_same_magnitude(w.grad, w_o.grad, what="d(W)")
     assert float(h.grad[T:].float().abs().sum()) == 0.0
+
+
+def test_engine_glue_takes_the_fused_sapo_step(device):
+    """``compute_logprobs_and_loss(use_sapo_loss=True)``: label roll, pad rows, loss scale around the fused SAPO pass."""
+    import oracle
+    from areal_amd import engine_glue
+
+    pad, V = 8, 9000
+    logits, labels, old, adv, mask = _sapo_case(64 + pad, 64, V, seed=2)
+    input_ids = torch.cat([labels[-1:], labels[:-1]]).unsqueeze(0)          # rolled by one gives `labels`
+    mb = dict(loss_mask=mask.to(device), logprobs=old.to(device), advantages=adv.to(device), prox_logp=None)
+    x = logits.to(device).requires_grad_(True)
+    loss, stat = engine_glue.compute_logprobs_and_loss(x, {"input_ids": input_ids.to(device)}, mb, pad, 100.0,
+                                                       eps_clip=0.2, use_sapo_loss=True)
+    loss.backward()
+    z = logits.float().requires_grad_(True)
+    w_loss, _ = S.sapo_loss(oracle.logprobs(z, labels)[:64], old, adv, 1.0, 1.05, mask)
+    (w_loss * float(mask.sum()) / 100.0).backward()
+    assert float(loss.detach()) == pytest.approx(float(w_loss.detach()) * float(mask.sum()) / 100.0, rel=1e-3)
+    assert cosine(x.grad.float().cpu(), z.grad) > 0.9999 and float(x.grad[64:].float().abs().sum()) == 0.0
+    assert "sapo_soft_gate" in stat and stat["logprobs"].shape == (64,)
