@@ -573,6 +573,252 @@ __global__ __launch_bounds__(1024) void k_fused_f32_hold(typename InPtr<ALIAS, f
 }
 
 // -----------------------------------------------------------------------------
+// fp32 rows longer than k_fused_f32_hold keeps on the chip (V > 114 688): the statistics (log-prob, entropy, extrema)
+// are taken from the fp32 values as they arrive, and what stays on the chip for the gradient is each value rounded to
+// its upper 24 bits (sign, exponent, 15 bits of mantissa), four values in three words.  kPackReg chunks of 8192 values
+// are held in registers (6 VGPRs per thread and chunk) and kPackLds chunks in LDS (24 KB each): 155 648 values, so a
+// row of V = 151 936 is read once, 8 bytes per element through the fabric.  Longer rows read what is left a second
+// time, as k_fused_f32_hold does.  The rounding moves x_j by at most |x_j| 2^-16, so the probabilities behind the
+// gradient row carry a relative error of at most |x_j| / T * 2^-16 (2e-4 at |x_j| / T = 13): ten times finer than
+// the bf16 rounding of a 16-bit gradient row, cosine to the exact fp32 row 1 - 1e-9.
+// -----------------------------------------------------------------------------
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+constexpr int kBufferFlags = 0x00020000;  // raw buffer, 32-bit data format
+constexpr int kAuxStream = 2;  // cache-policy bit 'nt': data is touched once, do not keep it in the caches
+constexpr int kPackReg = 13;  // 13 x 8192 values in registers (78 VGPRs per thread)
+constexpr int kPackLds = 6;   // 6 x 8192 values in LDS (144 KB)
+
+// upper 24 bits of x, rounded half up in magnitude (bits 7..0 of the result are not part of the value)
+__device__ __forceinline__ uint32_t round24(float x) { return __float_as_uint(x) + 0x80u; }
+
+// words 0..2 keep values 0..2 in their upper three bytes; their low bytes hold bytes 1..3 of value 3
+__device__ __forceinline__ void pack4(const float* x, uint32_t* w) {
+  const uint32_t r3 = round24(x[3]);
+  w[0] = __builtin_amdgcn_perm(round24(x[0]), r3, 0x07060501u);
+  w[1] = __builtin_amdgcn_perm(round24(x[1]), r3, 0x07060502u);
+  w[2] = __builtin_amdgcn_perm(round24(x[2]), r3, 0x07060503u);
+}
+
+__device__ __forceinline__ void unpack4(const uint32_t* w, float* x) {
+  x[0] = __uint_as_float(w[0] & 0xffffff00u);
+  x[1] = __uint_as_float(w[1] & 0xffffff00u);
+  x[2] = __uint_as_float(w[2] & 0xffffff00u);
+  const uint32_t lo = __builtin_amdgcn_perm(w[1], w[0], 0x0c04000cu);    // [0, w0.b0, w1.b0, 0]
+  x[3] = __uint_as_float(__builtin_amdgcn_perm(w[2], lo, 0x04020100u));  // [0, w0.b0, w1.b0, w2.b0]
+}
+
+// Loads of a row run ahead of the arithmetic through buffer descriptors (no branch around a load; lanes past the end
+// of the row read zeros and are left out of the statistics).  The chunks that go to LDS are taken first, while no
+// register holds a packed chunk yet: four chunks are in flight then, fewer as the registers fill, and at least the
+// load of the next chunk is issued before the arithmetic of this one (twelve chunks in flight measured 7 % slower:
+// the registers they need are spilled).  The first loads of the next row are issued right behind the stores of
+// this one, and loads and stores carry the `nt` policy: nothing is read twice.
+constexpr int kPackChunks = kPackReg + kPackLds;
+constexpr int kPackChunkBytes = kHoldChunk * 4;
+constexpr int kPackStageRegs = 32;  // VGPRs for chunks in flight plus packed chunks in registers, while that binds
+
+// step i of a row handles this chunk
+__host__ __device__ constexpr int pack_chunk_of(int i) { return i < kPackLds ? kPackReg + i : i - kPackLds; }
+// number of chunks whose loads have been issued when step i begins
+__host__ __device__ constexpr int pack_issued_at(int i) {
+  const int in_regs = i < kPackLds ? 0 : i - kPackLds;
+  int room = (kPackStageRegs - 6 * in_regs) / 8;
+  if (room < 1) room = 1;
+  const int n = i + room;
+  return n < kPackChunks ? n : kPackChunks;
+}
+
+struct Stage8 {
+  u32x4_t lo, hi;
+};
+
+// statistics of N more values without a branch (the rescaling factor is 1 when the maximum stays)
+template <int N>
+__device__ __forceinline__ void stats_add_flat(ThreadStats& a, const float (&x)[N], float c) {
+  float m = x[0], n = x[0];
+#pragma unroll
+  for (int i = 1; i < N; ++i) {
+    m = fmaxf(m, x[i]);
+    n = fminf(n, x[i]);
+  }
+  const float k_new = fmaxf(a.k, m * c);
+  const float d = a.k - k_new;
+  const float f = fast_exp2(d);
+  a.mx = fmaxf(a.mx, m);
+  a.mn = fminf(a.mn, n);
+  float s = 0.f, u = 0.f;
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    const float t = fmaf(x[i], c, -k_new);
+    const float e = fast_exp2(t);
+    s += e;
+    u = fmaf(t, e, u);
+  }
+  a.u = fmaf(f, fmaf(d, a.s, a.u), u);
+  a.s = fmaf(f, a.s, s);
+  a.k = k_new;
+}
+
+// A thread's eight values of a chunk are two pieces of four, 16 KB apart (values tid * 4 .. + 3 of each half of the
+// chunk), so that every load and store instruction of a wave covers 1 KB of consecutive addresses.
+__global__ __launch_bounds__(1024) void k_fused_f32_pack(const float* logits, int64_t T_rows, int V, int64_t stride,
+                                                         const int64_t* __restrict__ labels, float inv_t,
+                                                         FusedTokenArgs a, float* dlogits, int32_t* work) {
+  constexpr int kHalf = kHoldChunk / 2;          // values per half chunk
+  constexpr int kHalfBytes = kPackChunkBytes / 2;
+  __shared__ float smem[16 * 5];
+  __shared__ uint2 held[kPackLds * 3 * 1024];  // [chunk][word pair][thread]
+  __shared__ int64_t next_row[2];  // written at the top of a row, read behind its barriers: two slots, no reuse race
+  int slot = 0;
+  const int tid = threadIdx.x;
+  const int voff = tid * 16;
+  const float c = kLog2e * inv_t;
+  float fn, gscale;
+  load_loss_scale(a, fn, gscale);
+  Stage8 sg[kPackChunks];
+  auto issue = [&](const __amdgpu_buffer_rsrc_t rsrc, int i) {
+    const int off = pack_chunk_of(i) * kPackChunkBytes;
+    sg[i].lo = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, off, kAuxStream);
+    sg[i].hi = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, off + kHalfBytes, kAuxStream);
+  };
+
+  int64_t t = blockIdx.x;  // the host launches at most T_rows workgroups
+  __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(logits + t * stride), 0, V * 4, kBufferFlags);
+#pragma unroll
+  for (int j = 0; j < pack_issued_at(0); ++j) issue(rsrc, j);
+  for (;;) {
+    // claim the row after this one (through the device counter when there is one, so that compute units that get
+    // through their rows faster take more of them); the answer is picked up behind the barriers of block_stats
+    if (tid == 0) next_row[slot] = work ? (int64_t)atomicAdd(&work[0], 1) + gridDim.x : t + gridDim.x;
+    const float* row = logits + t * stride;
+    float* out = dlogits + t * stride;
+    const int64_t y = labels[t];
+    const bool y_ok = (y >= 0) && (y < V);
+    const float xy = y_ok ? row[y] : 0.f;
+    TokenIn tin{0.f, 0.f, 1.f, 0, false};
+    if (a.T_active > 0) tin = load_token_in(a, t);
+
+    // pass 1: statistics of the whole row from the fp32 values; the row stays on the chip in 24 bits per value
+    ThreadStats st{kNegBig, 0.f, 0.f, -FLT_MAX, FLT_MAX};
+    uint32_t pr[kPackReg][6];
+#pragma unroll
+    for (int i = 0; i < kPackChunks; ++i) {
+#pragma unroll
+      for (int j = pack_issued_at(i); j < pack_issued_at(i + 1); ++j) issue(rsrc, j);
+      if (i < kPackLds) {  // chunks kPackReg ..: the row may end inside or before them
+        float xl[4], xh[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          xl[q] = __uint_as_float(sg[i].lo[q]);
+          xh[q] = __uint_as_float(sg[i].hi[q]);
+        }
+        const int e0 = (kPackReg + i) * kHoldChunk + tid * 4;
+        if (e0 < V) stats_add_flat<4>(st, xl, c);
+        if (e0 + kHalf < V) stats_add_flat<4>(st, xh, c);
+        uint32_t w[6];  // what lies past the row is packed and kept as well (zeros), and never stored
+        pack4(xl, w);
+        pack4(xh, w + 3);
+        held[(i * 3 + 0) * 1024 + tid] = make_uint2(w[0], w[1]);
+        held[(i * 3 + 1) * 1024 + tid] = make_uint2(w[2], w[3]);
+        held[(i * 3 + 2) * 1024 + tid] = make_uint2(w[4], w[5]);
+      } else {  // chunks 0 .. kPackReg - 1 lie inside every row that comes here
+        float x[8];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          x[q] = __uint_as_float(sg[i].lo[q]);
+          x[4 + q] = __uint_as_float(sg[i].hi[q]);
+        }
+        stats_add_flat<8>(st, x, c);
+        pack4(x, pr[i - kPackLds]);
+        pack4(x + 4, pr[i - kPackLds] + 3);
+      }
+    }
+    for (int e0 = kPackChunks * kHoldChunk + tid * 8; e0 < V; e0 += kHoldChunk) {
+      float x[8];
+      load8<AA_F32>(row, e0, x);
+      stats_add8(st, x, c);
+    }
+    const RowStats rs = block_stats<16>(st, smem);
+    const int64_t tn = next_row[slot];
+    slot ^= 1;
+    const RowOut ro = finish_row(rs);
+    const float lp = y_ok ? label_logp(xy, c, rs, ro) : __builtin_nanf("");
+    const float g = fused_token_tail(a, t, tin, fn, gscale, lp, rs, ro, tid == 0);
+
+    // pass 2: the gradient row (every thread reads back only what it stored itself: no barrier needed)
+    const __amdgpu_buffer_rsrc_t wsrc = __builtin_amdgcn_make_buffer_rsrc((void*)out, 0, V * 4, kBufferFlags);
+    // the offsets of the stores are formed here, row by row: computed once for all rows they would occupy 38 registers
+    int so = voff;
+    asm volatile("" : "+v"(so));
+    if (g == 0.f) {
+      const u32x4_t z = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int k = 0; k < 2 * kPackChunks; ++k)  // pieces past the row are dropped by the descriptor
+        __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, so + k * kHalfBytes, 0, kAuxStream);
+      const float z8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      for (int e0 = kPackChunks * kHoldChunk + tid * 8; e0 < V; e0 += kHoldChunk) store8<AA_F32>(out, e0, z8);
+    } else {
+      const float A = -g * inv_t, lab_add = g * inv_t, lse2 = ro.lse2;
+      const int label = y_ok ? (int)y : -1;
+      // four values starting at element e0 of the row, stored at byte `off` past the thread's offset
+      auto emit4 = [&](int e0, int off, const float* x) {
+        float o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = fast_exp2(fmaf(x[i], c, -lse2)) * A;
+        if ((unsigned)(label - e0) < 4u) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (e0 + i == label) o[i] += lab_add;
+        }
+        const u32x4_t v = {__float_as_uint(o[0]), __float_as_uint(o[1]), __float_as_uint(o[2]), __float_as_uint(o[3])};
+        __builtin_amdgcn_raw_buffer_store_b128(v, wsrc, so + off, 0, kAuxStream);
+      };
+      auto emit = [&](int k, const uint32_t* w) {
+        float x[8];
+        unpack4(w, x);
+        unpack4(w + 3, x + 4);
+        emit4(k * kHoldChunk + tid * 4, k * kPackChunkBytes, x);
+        emit4(k * kHoldChunk + kHalf + tid * 4, k * kPackChunkBytes + kHalfBytes, x + 4);
+      };
+#pragma unroll
+      for (int k = 0; k < kPackReg; ++k) emit(k, pr[k]);
+#pragma unroll
+      for (int k = 0; k < kPackLds; ++k) {  // pieces past the row: the descriptor drops the store
+        const uint2 q0 = held[(k * 3 + 0) * 1024 + tid], q1 = held[(k * 3 + 1) * 1024 + tid],
+                    q2 = held[(k * 3 + 2) * 1024 + tid];
+        const uint32_t w[6] = {q0.x, q0.y, q1.x, q1.y, q2.x, q2.y};
+        emit(kPackReg + k, w);
+      }
+      for (int e0 = kPackChunks * kHoldChunk + tid * 8; e0 < V; e0 += kHoldChunk) {
+        float x[8], o[8];
+        load8<AA_F32>(row, e0, x);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = fast_exp2(fmaf(x[i], c, -lse2)) * A;
+        if ((unsigned)(label - e0) < 8u) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+            if (e0 + i == label) o[i] += lab_add;
+        }
+        store8<AA_F32>(out, e0, o);
+      }
+    }
+    t = tn;
+    if (t >= T_rows) break;
+    rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(logits + t * stride), 0, V * 4, kBufferFlags);
+#pragma unroll
+    for (int j = 0; j < pack_issued_at(0); ++j) issue(rsrc, j);
+  }
+  if (work && tid == 0) {  // the last workgroup to finish leaves both words at zero for the next launch
+    __threadfence();
+    if (atomicAdd(&work[1], 1) == (int)gridDim.x - 1) {
+      work[0] = 0;
+      work[1] = 0;
+      __threadfence();
+    }
+  }
+}
+
+// -----------------------------------------------------------------------------
 // Fused kernel, register-resident row: 1024 threads hold one row of 16-bit
 // logits as NCH 16-byte chunks per thread, so HBM sees exactly one read of the
 // row and one write of its gradient.  Requires V % 8 == 0, 16-byte aligned
@@ -587,11 +833,8 @@ __global__ __launch_bounds__(1024) void k_fused_f32_hold(typename InPtr<ALIAS, f
 // the overwritten value in some lanes.  The chunk offset of a store is added to
 // the VGPR offset instead.
 // -----------------------------------------------------------------------------
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef short s16x2_t __attribute__((ext_vector_type(2)));
 typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
-constexpr int kBufferFlags = 0x00020000;  // raw buffer, 32-bit data format
-constexpr int kAuxStream = 2;  // cache-policy bit 'nt': data is touched once, do not keep it in the caches
 
 // Marks the packed row as modified (no instruction is emitted) so that the
 // unpacked floats of one pass are not kept alive for the next: the row stays
@@ -1215,12 +1458,18 @@ extern "C" int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int
       ((((uintptr_t)logits | (uintptr_t)dlogits) & 15) == 0)) {
     const int cus = persistent_workgroups();
     const unsigned grid = (unsigned)(T < cus ? T : cus);
-    if (dlogits == logits)
-      hipLaunchKernelGGL(k_fused_f32_hold<true>, dim3(grid), dim3(1024), 0, st, (const float*)logits, T, (int)V, row_stride,
-                         labels, inv_temperature, a, (float*)dlogits);
-    else
-      hipLaunchKernelGGL(k_fused_f32_hold<false>, dim3(grid), dim3(1024), 0, st, (const float*)logits, T, (int)V, row_stride,
-                         labels, inv_temperature, a, (float*)dlogits);
+    // rows that the exact kernel would read twice in part go to the kernel that keeps 24 bits of each value
+    const bool pack = V > (int64_t)(kHoldReg + kHoldLds) * kHoldChunk && V <= (int64_t)1 << 28;
+#define AA_LAUNCH_F32(KERNEL, ...)                                                                                     \
+  hipLaunchKernelGGL(KERNEL, dim3(grid), dim3(1024), 0, st, (const float*)logits, T, (int)V, row_stride, labels,      \
+                     inv_temperature, a, (float*)dlogits, ##__VA_ARGS__)
+    if (pack) {
+      AA_LAUNCH_F32(k_fused_f32_pack, work);  // no restrict-qualified pointers: the same code serves dlogits == logits
+    } else {
+      if (dlogits == logits) AA_LAUNCH_F32(k_fused_f32_hold<true>);
+      else AA_LAUNCH_F32(k_fused_f32_hold<false>);
+    }
+#undef AA_LAUNCH_F32
     return launch_status();
   }
   const int vec_ok = rows_vec_ok(logits, dlogits, dtype) ? 1 : 0;

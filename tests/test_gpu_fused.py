@@ -82,8 +82,12 @@ def _compare(case, got, want, pad=0):
         (4099, torch.float32, 4, 20),      # generic rows, fp32 logits
         (8192, torch.float32, 4, 12),      # fp32 rows held on the chip: exactly one register chunk
         (81928, torch.float32, 4, 12),     # registers full, one vector in LDS
-        (114696, torch.float32, 4, 12),    # registers and LDS full, one vector read twice
-        (151936, torch.float32, 4, 12),    # benchmark vocabulary in fp32: 22 % of the row read twice
+        (114688, torch.float32, 4, 12),    # registers and LDS full: the longest row that is held exactly
+        (114696, torch.float32, 4, 12),    # one vector more: the row is held in 24 bits per value from here on
+        (151936, torch.float32, 4, 12),    # benchmark vocabulary in fp32: 13 chunks in registers, 5.5 in LDS
+        (155648, torch.float32, 4, 12),    # registers and LDS full of 24-bit values
+        (155656, torch.float32, 4, 12),    # one vector read twice
+        (200000, torch.float32, 4, 12),    # 5.4 chunks read twice
         (172040, torch.bfloat16, 4, 12),   # 22 chunks: 21 in registers, one (a single 16-byte piece of it) in LDS
         (245760, torch.bfloat16, 4, 12),   # 30 chunks: registers and LDS full, no tail
         (250008, torch.float16, 4, 12),    # 31 chunks: a partial streamed tail chunk
@@ -114,17 +118,59 @@ def test_short_rows_with_two_workgroups_per_unit(device, V, dtype):
     assert torch.equal(first[2], again[2]) and float(first[0]) == float(again[0])
 
 
-@pytest.mark.parametrize("V", [70004, 90112])
+@pytest.mark.parametrize("V", [70004, 90112, 122880])
 def test_fp32_long_rows_walked_by_large_workgroups(device, V):
     """More fp32 rows than workgroups, so every workgroup handles several rows: V = 70004 (not a multiple of 8, rows
     of 280 KB) takes the two-pass kernel with 512 walking workgroups, V = 90112 the kernel that holds the row on the
-    chip with one workgroup per compute unit."""
+    chip with one workgroup per compute unit, V = 122880 the one that holds it in 24 bits per value."""
     lengths = synth.lengths_uniform(40, 8, 24, seed=5)            # about 640 tokens
     case = synth.make_logits_case("t", lengths, V, V, device, synth.per_sequence_normal_advantages(lengths, 3),
                                   dtype=torch.float32, ppo=dict(eps_clip=0.2))
     assert case.n_tokens > 512
     _finish_case(case)
     _compare(case, _fused_step(case), _oracle_step(case))
+
+
+@pytest.mark.parametrize("V,temperature", [(151936, 1.0), (180224, 0.6)])
+def test_fp32_rows_held_in_24_bits_entry_by_entry(device, V, temperature):
+    """fp32 rows past 114 688 values stay on the chip rounded to 24 bits: log-probs and entropy come from the fp32
+    values (as exact as for shorter rows), every entry of the gradient row is within |x| / T * 2^-16 (relative,
+    beside the error of the row's logsumexp, which all entries share) of the float64 one, and labels in the
+    register, LDS and re-read parts of the row get their +g / T."""
+    spots = [0, 8191, 13 * 8192 - 1, 13 * 8192, 16 * 8192 + 77, V - 1, 19 * 8192 - 8 if V > 19 * 8192 else 5,
+             min(19 * 8192 + 3, V - 2)]
+    lengths = [len(spots)]
+    case = synth.make_logits_case("t", lengths, V, 11, device, synth.per_sequence_normal_advantages(lengths, 4),
+                                  dtype=torch.float32, ppo=dict(eps_clip=0.2), temperature=temperature)
+    with torch.no_grad():
+        for r, j in enumerate(spots):
+            case.labels[r] = j
+        case.loss_mask[:] = True
+    _finish_case(case)
+    loss, stat, grad = _fused_step(case)
+    x = case.logits.double().cpu().requires_grad_(True)
+    lp = torch.log_softmax(x / temperature, dim=-1).gather(-1, case.labels.cpu()[:, None])[:, 0]
+    assert float((stat["logprobs"].cpu().double() - lp.detach()).abs().max()) < 3e-5
+    # a gradient row is (d loss / d logp_t) / T * (onehot(label) - softmax): fit the one factor, then compare entries
+    probs = torch.softmax(x.detach() / temperature, dim=-1)
+    got = grad.double().cpu()
+    for r, j in enumerate(spots):
+        onehot = torch.zeros(V, dtype=torch.float64)
+        onehot[j] = 1.0
+        want_dir = onehot - probs[r]                 # d logp_label / d x, times T
+        row = got[r]
+        scale = float(row @ want_dir / (want_dir @ want_dir))
+        if scale == 0.0:
+            assert float(row.abs().max()) == 0.0
+            continue
+        resid = row / (scale * want_dir) - 1.0       # relative error, entry by entry
+        resid[j] = 0.0
+        xr = x.detach()[r]
+        common = float(resid[xr.abs() < 0.25].median())   # the row's logsumexp error, shared by every entry
+        assert abs(common) < 1e-4, (r, j, common)
+        bound = xr.abs() / temperature * 2.0 ** -16 + 1e-5
+        assert bool(((resid - common).abs() <= bound).all()), (r, j)
+        assert abs(float(row[j]) - scale * float(want_dir[j])) <= 1e-4 * abs(scale), (r, j)   # the label got its + g / T
 
 
 def test_long_rows_labels_and_extrema_in_every_region(device):
@@ -460,7 +506,9 @@ def test_second_backward_of_the_fused_step_is_refused(device):
         (8200, torch.float16),      # two-pass kernel, 16-byte pieces
         (50257, torch.bfloat16),    # two-pass kernel, element by element
         (4099, torch.float32),      # the same in fp32
-        (151936, torch.float32),    # fp32 rows held on the chip, the rest read twice
+        (90112, torch.float32),     # fp32 rows held on the chip
+        (151936, torch.float32),    # fp32 rows held on the chip in 24 bits per value
+        (200000, torch.float32),    # the same, the rest read twice
     ],
 )
 def test_gradient_written_over_the_logits(device, V, dtype):
