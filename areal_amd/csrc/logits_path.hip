@@ -465,176 +465,91 @@ __global__ __launch_bounds__(NT) void k_fused_generic(typename InPtr<ALIAS, void
 }
 
 // -----------------------------------------------------------------------------
-// Fused kernel for fp32 logits: a row is too long for the register file alone (608 KB at V = 151 936 against
-// 512 KB), so the first kHoldReg chunks of a row (8 floats per thread and chunk) stay in registers, the next
-// kHoldLds chunks in LDS, and only what is left is read a second time for the gradient.  At V = 151 936 that is
-// 24.5 % of the row: at most 9 bytes per element through the fabric instead of the 12 of the two-pass kernel (8 is
-// the floor); rows up to 114 688 elements are read once.  One workgroup of 1024 threads per compute unit (the LDS
-// share allows no second one), walking rows t, t + grid, ...  Needs V % 8 == 0 and 16-byte aligned rows.
-// -----------------------------------------------------------------------------
-constexpr int kHoldReg = 10;                        // 10 x 8192 floats in registers (80 VGPRs per thread)
-constexpr int kHoldLds = 4;                         // 4 x 8192 floats in LDS (128 KB)
-constexpr int kHoldChunk = 8 * 1024;                // floats per chunk: 8 per thread
-
-template <bool ALIAS>
-__global__ __launch_bounds__(1024) void k_fused_f32_hold(typename InPtr<ALIAS, float>::type logits, int64_t T_rows, int V,
-                                                         int64_t stride, const int64_t* __restrict__ labels,
-                                                         float inv_t, FusedTokenArgs a,
-                                                         typename OutPtr<ALIAS, float>::type dlogits) {
-  __shared__ float smem[16 * 5];
-  __shared__ float4 held[kHoldLds * 2 * 1024];      // [chunk][half][thread]: consecutive lanes, consecutive 16 bytes
-  const int tid = threadIdx.x;
-  const float c = kLog2e * inv_t;
-  float fn, gscale;
-  load_loss_scale(a, fn, gscale);
-  for (int64_t t = blockIdx.x; t < T_rows; t += gridDim.x) {
-    const float* row = logits + t * stride;
-    float* out = dlogits + t * stride;
-    const int64_t y = labels[t];
-    const bool y_ok = (y >= 0) && (y < V);
-    const float xy = y_ok ? row[y] : 0.f;
-    TokenIn tin{0.f, 0.f, 1.f, 0, false};
-    if (a.T_active > 0) tin = load_token_in(a, t);
-
-    // pass 1: statistics of the whole row; the head of the row stays on the chip
-    ThreadStats st{kNegBig, 0.f, 0.f, -FLT_MAX, FLT_MAX};
-    float xr[kHoldReg][8];
-#pragma unroll
-    for (int k = 0; k < kHoldReg; ++k) {
-      const int e0 = k * kHoldChunk + tid * 8;
-      if (e0 < V) {
-        load8<AA_F32>(row, e0, xr[k]);
-        stats_add8(st, xr[k], c);
-      }
-    }
-#pragma unroll
-    for (int k = 0; k < kHoldLds; ++k) {
-      const int e0 = (kHoldReg + k) * kHoldChunk + tid * 8;
-      if (e0 < V) {
-        float x[8];
-        load8<AA_F32>(row, e0, x);
-        held[(k * 2 + 0) * 1024 + tid] = make_float4(x[0], x[1], x[2], x[3]);
-        held[(k * 2 + 1) * 1024 + tid] = make_float4(x[4], x[5], x[6], x[7]);
-        stats_add8(st, x, c);
-      }
-    }
-    for (int e0 = (kHoldReg + kHoldLds) * kHoldChunk + tid * 8; e0 < V; e0 += kHoldChunk) {
-      float x[8];
-      load8<AA_F32>(row, e0, x);
-      stats_add8(st, x, c);
-    }
-    const RowStats rs = block_stats<16>(st, smem);
-    const RowOut ro = finish_row(rs);
-    const float lp = y_ok ? label_logp(xy, c, rs, ro) : __builtin_nanf("");
-    const float g = fused_token_tail(a, t, tin, fn, gscale, lp, rs, ro, tid == 0);
-
-    // pass 2: the gradient row (every thread reads back only what it stored itself: no barrier needed)
-    {
-      if (g == 0.f) {
-        const float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        for (int e0 = tid * 8; e0 < V; e0 += kHoldChunk) store8<AA_F32>(out, e0, z);
-      } else {
-        const float A = -g * inv_t, lab_add = g * inv_t, lse2 = ro.lse2;
-        const int label = y_ok ? (int)y : -1;
-        auto emit = [&](int e0, const float (&x)[8]) {
-          float o[8];
-#pragma unroll
-          for (int i = 0; i < 8; ++i) o[i] = fast_exp2(fmaf(x[i], c, -lse2)) * A;
-          if ((unsigned)(label - e0) < 8u) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-              if (e0 + i == label) o[i] += lab_add;
-          }
-          store8<AA_F32>(out, e0, o);
-        };
-#pragma unroll
-        for (int k = 0; k < kHoldReg; ++k) {
-          const int e0 = k * kHoldChunk + tid * 8;
-          if (e0 < V) emit(e0, xr[k]);
-        }
-#pragma unroll
-        for (int k = 0; k < kHoldLds; ++k) {
-          const int e0 = (kHoldReg + k) * kHoldChunk + tid * 8;
-          if (e0 < V) {
-            const float4 lo = held[(k * 2 + 0) * 1024 + tid], hi = held[(k * 2 + 1) * 1024 + tid];
-            const float x[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-            emit(e0, x);
-          }
-        }
-        for (int e0 = (kHoldReg + kHoldLds) * kHoldChunk + tid * 8; e0 < V; e0 += kHoldChunk) {
-          float x[8];
-          load8<AA_F32>(row, e0, x);
-          emit(e0, x);
-        }
-      }
-    }
-    __syncthreads();  // the statistics scratch is reused by the next row
-  }
-}
-
-// -----------------------------------------------------------------------------
-// fp32 rows longer than k_fused_f32_hold keeps on the chip (V > 114 688): the statistics (log-prob, entropy, extrema)
-// are taken from the fp32 values as they arrive, and what stays on the chip for the gradient is each value rounded to
-// its upper 24 bits (sign, exponent, 15 bits of mantissa), four values in three words.  kPackReg chunks of 8192 values
-// are held in registers (6 VGPRs per thread and chunk) and kPackLds chunks in LDS (24 KB each): 155 648 values, so a
-// row of V = 151 936 is read once, 8 bytes per element through the fabric.  Longer rows read what is left a second
-// time, as k_fused_f32_hold does.  The rounding moves x_j by at most |x_j| 2^-16, so the probabilities behind the
-// gradient row carry a relative error of at most |x_j| / T * 2^-16 (2e-4 at |x_j| / T = 13): ten times finer than
-// the bf16 rounding of a 16-bit gradient row, cosine to the exact fp32 row 1 - 1e-9.
+// Fused kernel for fp32 logits, the row held on the chip between its one read and the one write of its gradient.
+// One workgroup of 1024 threads per compute unit (its registers and the LDS belong to one row).  A row is cut into
+// chunks of 8192 values, 8 per thread; the first chunks stay in registers, the next ones in LDS, and only what is
+// left after those is read a second time for the gradient.  Two ways of holding a value:
+//   exact (PACK = false, rows up to 114 688 values): 10 chunks in registers (80 VGPRs), 4 in LDS (128 KB);
+//   24 bits (PACK = true, longer rows; a 608 KB row of V = 151 936 does not fit the 512 KB register file): the
+//     statistics (log-prob, entropy, extrema) are taken from the fp32 values as they arrive, and what stays on the
+//     chip is each value rounded to its upper 24 bits (sign, exponent, 15 bits of mantissa), four values in three
+//     words: 13 chunks in registers (78 VGPRs), 6 in LDS (144 KB), 155 648 values.  The rounding moves x_j by at
+//     most |x_j| 2^-16, so the probabilities behind the gradient row carry a relative error of at most
+//     |x_j| / T * 2^-16 (2e-4 at |x_j| / T = 13): ten times finer than the bf16 rounding of a 16-bit gradient row,
+//     cosine to the exact fp32 row 1 - 1e-9.
+// A thread's eight values of a chunk are two pieces of four, 16 KB apart (values tid * 4 .. + 3 of each half of the
+// chunk), so that every load and store instruction of a wave covers 1 KB of consecutive addresses (with the eight
+// values side by side, every 128-byte line is touched by two instructions: 12 % slower).
+// Loads run ahead of the arithmetic through buffer descriptors (no branch around a load; lanes past the end of the
+// row read zeros and are left out of the statistics).  The chunks that go to LDS are taken first, while no register
+// holds a chunk of the row yet: four chunks are in flight then, fewer as the registers fill, and at least the load
+// of the next chunk is issued before the arithmetic of this one (twelve chunks in flight measured 7 % slower: the
+// registers they need are spilled).  The first loads of the next row are issued right behind the stores of this
+// one; loads and stores carry the `nt` policy.  Rows are handed out through the device counter (work) when there
+// is one.  Needs V % 8 == 0, 16-byte aligned rows and rows below 2 GB.
 // -----------------------------------------------------------------------------
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 constexpr int kBufferFlags = 0x00020000;  // raw buffer, 32-bit data format
 constexpr int kAuxStream = 2;  // cache-policy bit 'nt': data is touched once, do not keep it in the caches
-constexpr int kPackReg = 13;  // 13 x 8192 values in registers (78 VGPRs per thread)
-constexpr int kPackLds = 6;   // 6 x 8192 values in LDS (144 KB)
+constexpr int kHoldChunk = 8 * 1024;  // values per chunk: 8 per thread
+constexpr int kHoldChunkBytes = kHoldChunk * 4;
+constexpr int kHoldStageRegs = 32;  // VGPRs for chunks in flight plus chunks held in registers, while that binds
+
+template <bool PACK, int NREG, int NLDS>
+struct HoldPlan {
+  static constexpr int kReg = NREG;             // chunks in registers
+  static constexpr int kLds = NLDS;             // chunks in LDS
+  static constexpr int kWords = PACK ? 6 : 8;   // words per thread and chunk
+  static constexpr int kChunks = kReg + kLds;
+  static_assert(kReg * kWords <= 80 && kLds * kWords * 4096 <= 147456, "the row does not fit");
+  // step i of a row handles this chunk
+  __host__ __device__ static constexpr int chunk_of(int i) { return i < kLds ? kReg + i : i - kLds; }
+  // number of chunks whose loads have been issued when step i begins
+  __host__ __device__ static constexpr int issued_at(int i) {
+    const int in_regs = i < kLds ? 0 : i - kLds;
+    int room = (kHoldStageRegs - kWords * in_regs) / 8;
+    if (room < 1) room = 1;
+    const int n = i + room;
+    return n < kChunks ? n : kChunks;
+  }
+};
+constexpr int kHoldExactMaxV = 14 * kHoldChunk;  // 10 chunks in registers (80 VGPRs), 4 in LDS (128 KB)
 
 // upper 24 bits of x, rounded half up in magnitude (bits 7..0 of the result are not part of the value)
 __device__ __forceinline__ uint32_t round24(float x) { return __float_as_uint(x) + 0x80u; }
 
-// words 0..2 keep values 0..2 in their upper three bytes; their low bytes hold bytes 1..3 of value 3
-__device__ __forceinline__ void pack4(const float* x, uint32_t* w) {
-  const uint32_t r3 = round24(x[3]);
-  w[0] = __builtin_amdgcn_perm(round24(x[0]), r3, 0x07060501u);
-  w[1] = __builtin_amdgcn_perm(round24(x[1]), r3, 0x07060502u);
-  w[2] = __builtin_amdgcn_perm(round24(x[2]), r3, 0x07060503u);
+// Four values in kWords / 2 words.  PACK: words 0..2 keep values 0..2 in their upper three bytes; their low bytes
+// hold bytes 1..3 of value 3.
+template <bool PACK>
+__device__ __forceinline__ void hold4(const float* x, uint32_t* w) {
+  if constexpr (PACK) {
+    const uint32_t r3 = round24(x[3]);
+    w[0] = __builtin_amdgcn_perm(round24(x[0]), r3, 0x07060501u);
+    w[1] = __builtin_amdgcn_perm(round24(x[1]), r3, 0x07060502u);
+    w[2] = __builtin_amdgcn_perm(round24(x[2]), r3, 0x07060503u);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = __float_as_uint(x[i]);
+  }
 }
 
-__device__ __forceinline__ void unpack4(const uint32_t* w, float* x) {
-  x[0] = __uint_as_float(w[0] & 0xffffff00u);
-  x[1] = __uint_as_float(w[1] & 0xffffff00u);
-  x[2] = __uint_as_float(w[2] & 0xffffff00u);
-  const uint32_t lo = __builtin_amdgcn_perm(w[1], w[0], 0x0c04000cu);    // [0, w0.b0, w1.b0, 0]
-  x[3] = __uint_as_float(__builtin_amdgcn_perm(w[2], lo, 0x04020100u));  // [0, w0.b0, w1.b0, w2.b0]
+template <bool PACK>
+__device__ __forceinline__ void held4(const uint32_t* w, float* x) {
+  if constexpr (PACK) {
+    x[0] = __uint_as_float(w[0] & 0xffffff00u);
+    x[1] = __uint_as_float(w[1] & 0xffffff00u);
+    x[2] = __uint_as_float(w[2] & 0xffffff00u);
+    const uint32_t lo = __builtin_amdgcn_perm(w[1], w[0], 0x0c04000cu);    // [0, w0.b0, w1.b0, 0]
+    x[3] = __uint_as_float(__builtin_amdgcn_perm(w[2], lo, 0x04020100u));  // [0, w0.b0, w1.b0, w2.b0]
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) x[i] = __uint_as_float(w[i]);
+  }
 }
-
-// Loads of a row run ahead of the arithmetic through buffer descriptors (no branch around a load; lanes past the end
-// of the row read zeros and are left out of the statistics).  The chunks that go to LDS are taken first, while no
-// register holds a packed chunk yet: four chunks are in flight then, fewer as the registers fill, and at least the
-// load of the next chunk is issued before the arithmetic of this one (twelve chunks in flight measured 7 % slower:
-// the registers they need are spilled).  The first loads of the next row are issued right behind the stores of
-// this one, and loads and stores carry the `nt` policy: nothing is read twice.
-constexpr int kPackChunks = kPackReg + kPackLds;
-constexpr int kPackChunkBytes = kHoldChunk * 4;
-constexpr int kPackStageRegs = 32;  // VGPRs for chunks in flight plus packed chunks in registers, while that binds
-
-// step i of a row handles this chunk
-__host__ __device__ constexpr int pack_chunk_of(int i) { return i < kPackLds ? kPackReg + i : i - kPackLds; }
-// number of chunks whose loads have been issued when step i begins
-__host__ __device__ constexpr int pack_issued_at(int i) {
-  const int in_regs = i < kPackLds ? 0 : i - kPackLds;
-  int room = (kPackStageRegs - 6 * in_regs) / 8;
-  if (room < 1) room = 1;
-  const int n = i + room;
-  return n < kPackChunks ? n : kPackChunks;
-}
-
-struct Stage8 {
-  u32x4_t lo, hi;
-};
 
 // statistics of N more values without a branch (the rescaling factor is 1 when the maximum stays)
 template <int N>
-__device__ __forceinline__ void stats_add_flat(ThreadStats& a, const float (&x)[N], float c) {
+__device__ __forceinline__ void stats_add_flat(ThreadStats& a, const float* x, float c) {
   float m = x[0], n = x[0];
 #pragma unroll
   for (int i = 1; i < N; ++i) {
@@ -659,25 +574,31 @@ __device__ __forceinline__ void stats_add_flat(ThreadStats& a, const float (&x)[
   a.k = k_new;
 }
 
-// A thread's eight values of a chunk are two pieces of four, 16 KB apart (values tid * 4 .. + 3 of each half of the
-// chunk), so that every load and store instruction of a wave covers 1 KB of consecutive addresses.
-__global__ __launch_bounds__(1024) void k_fused_f32_pack(const float* logits, int64_t T_rows, int V, int64_t stride,
+struct Stage8 {
+  u32x4_t lo, hi;
+};
+
+template <bool PACK, int NREG, int NLDS>
+__global__ __launch_bounds__(1024) void k_fused_f32_hold(const float* logits, int64_t T_rows, int V, int64_t stride,
                                                          const int64_t* __restrict__ labels, float inv_t,
                                                          FusedTokenArgs a, float* dlogits, int32_t* work) {
-  constexpr int kHalf = kHoldChunk / 2;          // values per half chunk
-  constexpr int kHalfBytes = kPackChunkBytes / 2;
+  typedef HoldPlan<PACK, NREG, NLDS> Plan;
+  constexpr int kW = Plan::kWords, kH = kW / 2;
+  constexpr int kHalf = kHoldChunk / 2;  // values per half chunk
+  constexpr int kHalfBytes = kHoldChunkBytes / 2;
   __shared__ float smem[16 * 5];
-  __shared__ uint2 held[kPackLds * 3 * 1024];  // [chunk][word pair][thread]
+  __shared__ uint2 held[(Plan::kLds > 0 ? Plan::kLds : 1) * kH * 1024];  // [chunk][word pair][thread]
   __shared__ int64_t next_row[2];  // written at the top of a row, read behind its barriers: two slots, no reuse race
   int slot = 0;
   const int tid = threadIdx.x;
   const int voff = tid * 16;
+  const int tid4 = tid * 4;
   const float c = kLog2e * inv_t;
   float fn, gscale;
   load_loss_scale(a, fn, gscale);
-  Stage8 sg[kPackChunks];
+  Stage8 sg[Plan::kChunks];
   auto issue = [&](const __amdgpu_buffer_rsrc_t rsrc, int i) {
-    const int off = pack_chunk_of(i) * kPackChunkBytes;
+    const int off = Plan::chunk_of(i) * kHoldChunkBytes;
     sg[i].lo = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, off, kAuxStream);
     sg[i].hi = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, off + kHalfBytes, kAuxStream);
   };
@@ -685,7 +606,7 @@ __global__ __launch_bounds__(1024) void k_fused_f32_pack(const float* logits, in
   int64_t t = blockIdx.x;  // the host launches at most T_rows workgroups
   __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(logits + t * stride), 0, V * 4, kBufferFlags);
 #pragma unroll
-  for (int j = 0; j < pack_issued_at(0); ++j) issue(rsrc, j);
+  for (int j = 0; j < Plan::issued_at(0); ++j) issue(rsrc, j);
   for (;;) {
     // claim the row after this one (through the device counter when there is one, so that compute units that get
     // through their rows faster take more of them); the answer is picked up behind the barriers of block_stats
@@ -698,42 +619,49 @@ __global__ __launch_bounds__(1024) void k_fused_f32_pack(const float* logits, in
     TokenIn tin{0.f, 0.f, 1.f, 0, false};
     if (a.T_active > 0) tin = load_token_in(a, t);
 
-    // pass 1: statistics of the whole row from the fp32 values; the row stays on the chip in 24 bits per value
+    // pass 1: statistics of the whole row from the fp32 values as they arrive; the row stays on the chip
     ThreadStats st{kNegBig, 0.f, 0.f, -FLT_MAX, FLT_MAX};
-    uint32_t pr[kPackReg][6];
+    uint32_t pr[Plan::kReg][kW];
 #pragma unroll
-    for (int i = 0; i < kPackChunks; ++i) {
+    for (int i = 0; i < Plan::kChunks; ++i) {
 #pragma unroll
-      for (int j = pack_issued_at(i); j < pack_issued_at(i + 1); ++j) issue(rsrc, j);
-      if (i < kPackLds) {  // chunks kPackReg ..: the row may end inside or before them
-        float xl[4], xh[4];
+      for (int j = Plan::issued_at(i); j < Plan::issued_at(i + 1); ++j) issue(rsrc, j);
+      __builtin_amdgcn_sched_barrier(0);  // the loads stay where they are issued: no more of them in flight than planned
+      float x[8];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          xl[q] = __uint_as_float(sg[i].lo[q]);
-          xh[q] = __uint_as_float(sg[i].hi[q]);
-        }
-        const int e0 = (kPackReg + i) * kHoldChunk + tid * 4;
-        if (e0 < V) stats_add_flat<4>(st, xl, c);
-        if (e0 + kHalf < V) stats_add_flat<4>(st, xh, c);
-        uint32_t w[6];  // what lies past the row is packed and kept as well (zeros), and never stored
-        pack4(xl, w);
-        pack4(xh, w + 3);
-        held[(i * 3 + 0) * 1024 + tid] = make_uint2(w[0], w[1]);
-        held[(i * 3 + 1) * 1024 + tid] = make_uint2(w[2], w[3]);
-        held[(i * 3 + 2) * 1024 + tid] = make_uint2(w[4], w[5]);
-      } else {  // chunks 0 .. kPackReg - 1 lie inside every row that comes here
-        float x[8];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          x[q] = __uint_as_float(sg[i].lo[q]);
-          x[4 + q] = __uint_as_float(sg[i].hi[q]);
-        }
+      for (int q = 0; q < 4; ++q) {
+        x[q] = __uint_as_float(sg[i].lo[q]);
+        x[4 + q] = __uint_as_float(sg[i].hi[q]);
+      }
+      if (PACK && i >= Plan::kLds) {  // in the 24-bit form the register chunks lie inside every row that comes here
         stats_add_flat<8>(st, x, c);
-        pack4(x, pr[i - kPackLds]);
-        pack4(x + 4, pr[i - kPackLds] + 3);
+      } else {  // the row may end in this chunk or before it: what lies past it read as zeros and is never stored
+        const int left = V - Plan::chunk_of(i) * kHoldChunk;  // values of the row from this chunk on (same in all threads)
+        if (tid4 < left) stats_add_flat<4>(st, x, c);
+        if (tid4 < left - kHalf) stats_add_flat<4>(st, x + 4, c);
+      }
+      if (i < Plan::kLds) {
+        uint32_t w[kW];
+        hold4<PACK>(x, w);
+        hold4<PACK>(x + 4, w + kH);
+        // The LDS addresses are formed here, chunk by chunk, from a copy of the thread index that the compiler
+        // cannot follow: computed once for all rows they end up spilled, and a reload from scratch in the middle
+        // of a row waits for every load (here) or store (in pass 2) that is in flight.
+        int ti = tid;
+        asm volatile("" : "+v"(ti));
+#pragma unroll
+        for (int q = 0; q < kH; ++q) held[(i * kH + q) * 1024 + ti] = make_uint2(w[2 * q], w[2 * q + 1]);
+      } else {
+        uint32_t* w = pr[i - Plan::kLds];
+        hold4<PACK>(x, w);
+        hold4<PACK>(x + 4, w + kH);
+        // the words are formed here (no instruction is emitted): left to the compiler, the rounding and packing move
+        // down to the gradient pass and the registers hold the eight fp32 values until then
+#pragma unroll
+        for (int q = 0; q < kW; ++q) asm volatile("" : "+v"(w[q]));
       }
     }
-    for (int e0 = kPackChunks * kHoldChunk + tid * 8; e0 < V; e0 += kHoldChunk) {
+    for (int e0 = Plan::kChunks * kHoldChunk + tid * 8; e0 < V; e0 += kHoldChunk) {
       float x[8];
       load8<AA_F32>(row, e0, x);
       stats_add8(st, x, c);
@@ -753,43 +681,51 @@ __global__ __launch_bounds__(1024) void k_fused_f32_pack(const float* logits, in
     if (g == 0.f) {
       const u32x4_t z = {0u, 0u, 0u, 0u};
 #pragma unroll
-      for (int k = 0; k < 2 * kPackChunks; ++k)  // pieces past the row are dropped by the descriptor
+      for (int k = 0; k < 2 * Plan::kChunks; ++k)  // pieces past the row are dropped by the descriptor
         __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, so + k * kHalfBytes, 0, kAuxStream);
       const float z8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      for (int e0 = kPackChunks * kHoldChunk + tid * 8; e0 < V; e0 += kHoldChunk) store8<AA_F32>(out, e0, z8);
+      for (int e0 = Plan::kChunks * kHoldChunk + tid * 8; e0 < V; e0 += kHoldChunk) store8<AA_F32>(out, e0, z8);
     } else {
       const float A = -g * inv_t, lab_add = g * inv_t, lse2 = ro.lse2;
       const int label = y_ok ? (int)y : -1;
-      // four values starting at element e0 of the row, stored at byte `off` past the thread's offset
-      auto emit4 = [&](int e0, int off, const float* x) {
+      // the thread's four values of the piece that starts at element `base` of the row and byte `off` of its storage
+      // (the label's place is found from one per-thread value and numbers that are the same in all threads)
+      auto emit4 = [&](int base, int off, const float* x) {
         float o[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) o[i] = fast_exp2(fmaf(x[i], c, -lse2)) * A;
-        if ((unsigned)(label - e0) < 4u) {
+        const int d = (label - base) - tid4;
+        if ((unsigned)d < 4u) {
 #pragma unroll
           for (int i = 0; i < 4; ++i)
-            if (e0 + i == label) o[i] += lab_add;
+            if (d == i) o[i] += lab_add;
         }
         const u32x4_t v = {__float_as_uint(o[0]), __float_as_uint(o[1]), __float_as_uint(o[2]), __float_as_uint(o[3])};
         __builtin_amdgcn_raw_buffer_store_b128(v, wsrc, so + off, 0, kAuxStream);
       };
       auto emit = [&](int k, const uint32_t* w) {
         float x[8];
-        unpack4(w, x);
-        unpack4(w + 3, x + 4);
-        emit4(k * kHoldChunk + tid * 4, k * kPackChunkBytes, x);
-        emit4(k * kHoldChunk + kHalf + tid * 4, k * kPackChunkBytes + kHalfBytes, x + 4);
+        held4<PACK>(w, x);
+        held4<PACK>(w + kH, x + 4);
+        emit4(k * kHoldChunk, k * kHoldChunkBytes, x);
+        emit4(k * kHoldChunk + kHalf, k * kHoldChunkBytes + kHalfBytes, x + 4);
       };
 #pragma unroll
-      for (int k = 0; k < kPackReg; ++k) emit(k, pr[k]);
+      for (int k = 0; k < Plan::kReg; ++k) emit(k, pr[k]);
 #pragma unroll
-      for (int k = 0; k < kPackLds; ++k) {  // pieces past the row: the descriptor drops the store
-        const uint2 q0 = held[(k * 3 + 0) * 1024 + tid], q1 = held[(k * 3 + 1) * 1024 + tid],
-                    q2 = held[(k * 3 + 2) * 1024 + tid];
-        const uint32_t w[6] = {q0.x, q0.y, q1.x, q1.y, q2.x, q2.y};
-        emit(kPackReg + k, w);
+      for (int k = 0; k < Plan::kLds; ++k) {  // pieces past the row: the descriptor drops the store
+        uint32_t w[kW];
+        int ti = tid;
+        asm volatile("" : "+v"(ti));
+#pragma unroll
+        for (int q = 0; q < kH; ++q) {
+          const uint2 v = held[(k * kH + q) * 1024 + ti];
+          w[2 * q] = v.x;
+          w[2 * q + 1] = v.y;
+        }
+        emit(Plan::kReg + k, w);
       }
-      for (int e0 = kPackChunks * kHoldChunk + tid * 8; e0 < V; e0 += kHoldChunk) {
+      for (int e0 = Plan::kChunks * kHoldChunk + tid * 8; e0 < V; e0 += kHoldChunk) {
         float x[8], o[8];
         load8<AA_F32>(row, e0, x);
 #pragma unroll
@@ -806,7 +742,7 @@ __global__ __launch_bounds__(1024) void k_fused_f32_pack(const float* logits, in
     if (t >= T_rows) break;
     rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(logits + t * stride), 0, V * 4, kBufferFlags);
 #pragma unroll
-    for (int j = 0; j < pack_issued_at(0); ++j) issue(rsrc, j);
+    for (int j = 0; j < Plan::issued_at(0); ++j) issue(rsrc, j);
   }
   if (work && tid == 0) {  // the last workgroup to finish leaves both words at zero for the next launch
     __threadfence();
@@ -1454,22 +1390,20 @@ extern "C" int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int
                : launch_regs_ext<AA_F16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st);
     if (ok) return launch_status();
   }
-  if (dtype == AA_F32 && (V % 8 == 0) && (row_stride % 4 == 0) && V >= kHoldChunk &&
+  if (dtype == AA_F32 && (V % 8 == 0) && (row_stride % 4 == 0) && V >= kHoldChunk && V <= ((int64_t)1 << 28) &&
       ((((uintptr_t)logits | (uintptr_t)dlogits) & 15) == 0)) {
     const int cus = persistent_workgroups();
     const unsigned grid = (unsigned)(T < cus ? T : cus);
-    // rows that the exact kernel would read twice in part go to the kernel that keeps 24 bits of each value
-    const bool pack = V > (int64_t)(kHoldReg + kHoldLds) * kHoldChunk && V <= (int64_t)1 << 28;
-#define AA_LAUNCH_F32(KERNEL, ...)                                                                                     \
-  hipLaunchKernelGGL(KERNEL, dim3(grid), dim3(1024), 0, st, (const float*)logits, T, (int)V, row_stride, labels,      \
-                     inv_temperature, a, (float*)dlogits, ##__VA_ARGS__)
-    if (pack) {
-      AA_LAUNCH_F32(k_fused_f32_pack, work);  // no restrict-qualified pointers: the same code serves dlogits == logits
-    } else {
-      if (dlogits == logits) AA_LAUNCH_F32(k_fused_f32_hold<true>);
-      else AA_LAUNCH_F32(k_fused_f32_hold<false>);
-    }
-#undef AA_LAUNCH_F32
+    // rows that the exact form would read twice in part are held in 24 bits per value; the pointers are not
+    // restrict-qualified: the same code serves dlogits == logits
+#define AA_LAUNCH_HOLD(PACK, NREG, NLDS)                                                                              \
+  hipLaunchKernelGGL((k_fused_f32_hold<PACK, NREG, NLDS>), dim3(grid), dim3(1024), 0, st, (const float*)logits, T, (int)V, \
+                     row_stride, labels, inv_temperature, a, (float*)dlogits, work)
+    if (V > kHoldExactMaxV) AA_LAUNCH_HOLD(true, 13, 6);
+    else if (V > 8 * kHoldChunk) AA_LAUNCH_HOLD(false, 10, 4);
+    else if (V > 4 * kHoldChunk) AA_LAUNCH_HOLD(false, 8, 0);  // shorter rows: no arithmetic on chunks that no row has
+    else AA_LAUNCH_HOLD(false, 4, 0);
+#undef AA_LAUNCH_HOLD
     return launch_status();
   }
   const int vec_ok = rows_vec_ok(logits, dlogits, dtype) ? 1 : 0;

@@ -370,9 +370,8 @@ def bench_logits(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: 
         achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
         # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters read
         # for the plain copy kernel: 1.001 x the algorithmic bytes (profiles/k_fused_regs_cfg1-32k_hbm_traffic.md);
-        # fp32 logits: 1.092 x, the part of a row that does not fit on the chip is fetched a second time
-        # (profiles/k_fused_f32_hold_cfg1-32k_hbm_traffic.md)
-        traffic=alg_bytes * (1.092 if f32 else 1.001), avg_kernel_ms=k_ms, min_kernel_ms=k_min_ms,
+        # fp32 logits: 1.001 x as well (profiles/k_fused_f32_hold_cfg1-32k_hbm_traffic.md)
+        traffic=alg_bytes * 1.001, avg_kernel_ms=k_ms, min_kernel_ms=k_min_ms,
         traffic_source=("profiles/k_fused_f32_hold_cfg1-32k_hbm_traffic.md" if f32 else
                         "profiles/k_fused_regs_cfg1-32k_hbm_traffic.md") +
                        ": counter bytes / algorithmic bytes measured on the cfg1-32k workload, applied to this one's "

@@ -152,6 +152,13 @@ int aa_logits_bwd(const void* logits, int dtype, int64_t T, int64_t V,
  *   assignment) and leaves them zero on exit, so one zeroed buffer serves
  *   every launch on a stream.  Launches that may run concurrently need
  *   separate buffers.
+ * AA_F32 logits with V % 8 == 0 and more than 114 688 values per row: the row
+ *   is kept on the chip between its read and the write of its gradient in 24
+ *   bits per value (a 608 KB row of V = 151 936 does not fit the register file
+ *   in fp32).  logp, entropy, vmax and vmin are computed from the fp32 values;
+ *   the softmax probabilities behind dlogits carry a relative error of at
+ *   most |x_j| * inv_temperature * 2^-16 (2e-4 at 13), ten times finer than
+ *   the rounding of a bf16 gradient row.  Shorter fp32 rows are kept exactly.
  */
 int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int64_t V,
                         int64_t row_stride, const int64_t* labels,

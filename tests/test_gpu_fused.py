@@ -118,17 +118,21 @@ def test_short_rows_with_two_workgroups_per_unit(device, V, dtype):
     assert torch.equal(first[2], again[2]) and float(first[0]) == float(again[0])
 
 
-@pytest.mark.parametrize("V", [70004, 90112, 122880])
+@pytest.mark.parametrize("V", [70004, 24576, 49152, 90112, 122880])
 def test_fp32_long_rows_walked_by_large_workgroups(device, V):
     """More fp32 rows than workgroups, so every workgroup handles several rows: V = 70004 (not a multiple of 8, rows
-    of 280 KB) takes the two-pass kernel with 512 walking workgroups, V = 90112 the kernel that holds the row on the
-    chip with one workgroup per compute unit, V = 122880 the one that holds it in 24 bits per value."""
+    of 280 KB) takes the two-pass kernel with 512 walking workgroups, the others the kernel that holds the row on the
+    chip with one workgroup per compute unit: in registers alone (V = 24576: up to 4 chunks, V = 49152: up to 8), in
+    registers and LDS (V = 90112), and in 24 bits per value (V = 122880)."""
     lengths = synth.lengths_uniform(40, 8, 24, seed=5)            # about 640 tokens
     case = synth.make_logits_case("t", lengths, V, V, device, synth.per_sequence_normal_advantages(lengths, 3),
                                   dtype=torch.float32, ppo=dict(eps_clip=0.2))
     assert case.n_tokens > 512
     _finish_case(case)
-    _compare(case, _fused_step(case), _oracle_step(case))
+    first = _fused_step(case)
+    _compare(case, first, _oracle_step(case))
+    again = _fused_step(case)                                     # rows handed out in another order, the same bits
+    assert torch.equal(first[2], again[2]) and float(first[0]) == float(again[0])
 
 
 @pytest.mark.parametrize("V,temperature", [(151936, 1.0), (180224, 0.6)])
