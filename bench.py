@@ -37,6 +37,7 @@ Prints ONE JSON line.  Besides the whole-step throughput it carries
 and, in the default run only (every GPU timing is taken before the first CPU baseline starts):
   configs1_cut_to_32k_tokens  the cfg1 sequences cut at 32 768 tokens;
   logits_config0              the cfg0 workload with its own roofline, and the plain copy kernel on the same buffers;
+  fp32_logits_cut_to_32k_tokens  the 32 768-token cut with the logits cast to fp32 (8 * V bytes per token);
   fused_lm_head               the same figures for the cfg2 workload, so that one run reports both paths;
   fused_lm_head_cfg3, _cfg4   the cfg3 and cfg4 workloads (GPU only: three timed steps each, their own roofline).
 
@@ -1133,6 +1134,15 @@ def main():
             small, _ = bench_logits(args, dev, "cfg0", max(args.steps, 50), args.warmup, 0, with_sft=False)
             out["logits_config0"] = {k: small[k] for k in keys}
             torch.cuda.empty_cache()
+            # the same 32 768 tokens handed over as fp32 logits (what a head that computes in fp32 emits): 8 bytes
+            # per element, its own kernel
+            import copy
+
+            args32 = copy.copy(args)
+            args32.logits_dtype = "f32"
+            wide, _ = bench_logits(args32, dev, "cfg1-32k", args.steps, args.warmup, 0, with_sft=False)
+            out["fp32_logits_cut_to_32k_tokens"] = {k: wide[k] for k in keys}
+            torch.cuda.empty_cache()
             extra, fused_sample = bench_fused(args, dev, "cfg2", args.steps, args.warmup, min(args.cpu_tokens, 384))
             torch.cuda.empty_cache()
             # the two larger fused configurations, GPU only
@@ -1155,6 +1165,8 @@ def main():
         roof = part.get("roofline")
         if roof:
             fractions["pct_hbm_peak" if roof["bound"] == "hbm" else "pct_mfma_peak"] = 100.0 * roof["frac"]
+    if "fp32_logits_cut_to_32k_tokens" in out:
+        fractions["pct_hbm_peak_fp32_logits"] = 100.0 * out["fp32_logits_cut_to_32k_tokens"]["roofline"]["frac"]
     for wl in ("cfg3", "cfg4"):
         if f"fused_lm_head_{wl}" in out:
             fractions[f"pct_mfma_peak_{wl}"] = 100.0 * out[f"fused_lm_head_{wl}"]["roofline"]["frac"]
