@@ -760,7 +760,7 @@ __global__ __launch_bounds__(1024) void k_fused_f32_hold(const float* logits, in
 // row and one write of its gradient.  Requires V % 8 == 0, 16-byte aligned
 // rows and 8192 * (NCH - 1) < V <= 8192 * NCH, so that only the last chunk can
 // be partly out of range (longer rows: the EXT variant below, which adds chunks
-// held in LDS and chunks streamed once per pass).  Rows are addressed through buffer descriptors: one
+// held in LDS and chunks that are read twice).  Rows are addressed through buffer descriptors: one
 // VGPR offset per thread, and the hardware drops out-of-range lanes (loads
 // return 0, stores are ignored).  Loads take the chunk offset in the scalar
 // offset operand.  Stores must NOT: with a register in the scalar-offset operand
@@ -826,7 +826,8 @@ __device__ __forceinline__ void grad_pass(const u32x4_t (&d)[NCH], float g, floa
 // ---- rows longer than the register file --------------------------------------
 // The extended variant of k_fused_regs (EXT) keeps kExtRegChunks chunks of the row in registers, up to
 // kExtLdsChunks more in LDS (brought in by direct-to-LDS loads, each thread reads back only the 16 bytes its own
-// lane deposited) and streams up to kExtTailChunks last chunks from memory once per pass.  These helpers are the
+// lane deposited) and reads up to kExtTailChunks last chunks twice: for the statistics (both passes use the one
+// fetch, left in the cache) and for the gradient.  These helpers are the
 // per-chunk bodies of the three passes for a chunk that is not in registers.
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 constexpr int kExtRegChunks = 21;
@@ -966,7 +967,8 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
     // minimum, otherwise the smallest unsigned pattern is.
     s16x2_t smax = {-32768, -32768}, smin = {32767, 32767};
     u16x2_t umax = {0, 0}, umin = {65535, 65535};
-    // EXT: the tail chunks of this row, fetched again at the top of every pass (lanes past the row read zeros)
+    // EXT: the tail chunks of this row, fetched here for the statistics and once more for the gradient (lanes past
+    // the row read zeros)
     __amdgpu_buffer_rsrc_t rsrc_t;
     u32x4_t tv[kExtTailChunks];
     bool tail_ok[kExtTailChunks];
@@ -974,7 +976,7 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
       rsrc_t = __builtin_amdgcn_make_buffer_rsrc((void*)(logits + t * stride_vec), 0, V * 2, kBufferFlags);
 #pragma unroll
       for (int q = 0; q < kExtTailChunks; ++q) {
-        tv[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_t, voff, (tail0 + q) * kChunkBytes, kAuxStream);
+        tv[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_t, voff, (tail0 + q) * kChunkBytes, 0);  // stays cached for the second read
         tail_ok[q] = (tail0 + q) * NT + tid < nvec;
       }
     }
@@ -1015,10 +1017,10 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
     ts.k = fmaxf(wave_max(mx) * c, kNegBig);
     ts.mx = mx; ts.mn = mn;
     float s = 0.f, u = 0.f;
-    if constexpr (EXT) {
+    if constexpr (EXT) {  // the tail chunks first: they are still in the registers pass 1 read them into
 #pragma unroll
       for (int q = 0; q < kExtTailChunks; ++q)
-        tv[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_t, voff, (tail0 + q) * kChunkBytes, kAuxStream);
+        if (tail_ok[q]) sum_chunk<DT>(tv[q], c, ts.k, s, u);
     }
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
@@ -1039,9 +1041,6 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
     if constexpr (EXT) {
       for (int j = 0; j < n_lds; ++j)
         if ((NCH + j) * NT + tid < nvec) sum_chunk<DT>(my_lds[j * NT], c, ts.k, s, u);
-#pragma unroll
-      for (int q = 0; q < kExtTailChunks; ++q)
-        if (tail_ok[q]) sum_chunk<DT>(tv[q], c, ts.k, s, u);
     }
     ts.s = s; ts.u = u;
     keep_packed(d);

@@ -506,7 +506,7 @@ def test_second_backward_of_the_fused_step_is_refused(device):
     [
         (151936, torch.bfloat16),   # register-resident rows
         (172040, torch.bfloat16),   # registers + LDS
-        (250008, torch.float16),    # registers + LDS + a tail that is read once per pass
+        (250008, torch.float16),    # registers + LDS + a tail that is read twice
         (8200, torch.float16),      # two-pass kernel, 16-byte pieces
         (50257, torch.bfloat16),    # two-pass kernel, element by element
         (4099, torch.float32),      # the same in fp32
