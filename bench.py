@@ -95,6 +95,9 @@ def parse_args():
     ap.add_argument("--logits-dtype", choices=["bf16", "f32"], default="bf16",
                     help="logits workloads: hand the kernels fp32 logits (what a Megatron-style head emits) instead of "
                          "bf16; 8 bytes per element instead of 4")
+    ap.add_argument("--steps-only", action="store_true",
+                    help="fused lm_head workloads: launch the steps of the selected backward mode only (no stand-alone "
+                         "op, no other mode), so that every dispatch a profiler sees belongs to a step")
     ap.add_argument("--copy-launches", type=int, default=0,
                     help="also launch the plain copy kernel this many times over the logits buffer (lm_head workloads: the weight matrix) "
                          "(the calibration point for FETCH_SIZE / WRITE_SIZE counters)")
@@ -459,9 +462,9 @@ MODE_NAMES = {1: "carry", 0: "recompute"}
 # known size.  The counters sit behind the L2 of each XCD: what the memory-side cache serves is in these figures too.
 # Transcribed from the profile summaries named beside them, not read in this run; other workloads: not measured.
 LMHEAD_MEASURED_HBM_BYTES = {
-    ("cfg2", "carry"): (81.6e9, "profiles/lmhead_step_cfg2_hbm_traffic.md"),
-    ("cfg2", "recompute"): (108.8e9, "profiles/lmhead_step_cfg2_hbm_traffic.md"),
-    ("cfg4", "carry"): (432.8e9, "profiles/lmhead_step_cfg4_hbm_traffic.md"),
+    ("cfg2", "carry"): (81.4e9, "profiles/lmhead_step_cfg2_hbm_traffic.md"),
+    ("cfg2", "recompute"): (108.4e9, "profiles/lmhead_step_cfg2_hbm_traffic.md"),
+    ("cfg4", "carry"): (511.7e9, "profiles/lmhead_step_cfg4_hbm_traffic.md"),
 }
 
 
@@ -766,13 +769,26 @@ def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: i
     modes = {}
     kept_tokens = T
     for mode, name in ((1, "carry"), (0, "recompute")):
-        c_ms, c_min, kept_tokens = time_lmhead_step(case, kw, cfg, 10, not args.dense_backward, mode)
+        if args.steps_only and mode != BACKWARD_MODE:
+            continue
+        c_ms, c_min, kept_tokens = time_lmhead_step(case, kw, cfg, 2 if args.steps_only else 10, not args.dense_backward,
+                                                    mode)
         modes[name] = dict(avg_call_ms=c_ms, min_call_ms=c_min,
                            executed_flops=(2.0 * T + (4.0 if mode == 1 else 6.0) * kept_tokens) * V * H,
                            compulsory_hbm_bytes=lmhead_compulsory_bytes(T, kept_tokens, H, V, name, chunk),
                            measured_hbm_bytes=lmhead_measured_bytes(workload, name)[0],
                            measured_hbm_bytes_source=lmhead_measured_bytes(workload, name)[1])
-    f_ms, b_ms, op_kept, fc_ms, bc_ms = time_lmhead_op(case, 5)
+    standalone = None
+    if not args.steps_only:
+        # the stand-alone differentiable op lm_head_logprobs_entropy: its forward writes softmax partials only, its
+        # backward forms the logits of the tokens with a gradient again (6 T_grad V H flops executed)
+        f_ms, b_ms, op_kept, fc_ms, bc_ms = time_lmhead_op(case, 5)
+        standalone = dict(fwd_ms=f_ms, bwd_ms=b_ms, fwd_tflops=2.0 * T * V * H / (f_ms * 1e-3) / 1e12,
+                          bwd_executed_tflops=6.0 * op_kept * V * H / (b_ms * 1e-3) / 1e12,
+                          # lm_head_logprobs_entropy(backward="carry"): the forward also keeps the bf16 rows of the
+                          # tokens with a gradient, the backward is the two gradient GEMMs (4 T_grad V H flops)
+                          carry_fwd_ms=fc_ms, carry_bwd_ms=bc_ms,
+                          carry_bwd_tflops=4.0 * op_kept * V * H / (bc_ms * 1e-3) / 1e12)
     # Flops the step needs: logits of every token (2 T V H) and the two gradient GEMMs over the tokens that have a
     # gradient (4 T_kept V H).  The reference's autograd runs them over all T tokens: 6 T V H.
     needed_flops = 2.0 * T * V * H + 4.0 * kept_tokens * V * H
@@ -793,14 +809,7 @@ def bench_fused(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: i
         avg_step_ms=ev_avg, min_step_ms=ev_ms[0], max_step_ms=ev_ms[-1],
         needed_flops_per_step=needed_flops, flops_per_step_6TVH=6.0 * T * V * H, tokens_with_gradient=kept_tokens,
         backward_mode=mode_name, backward_modes_through_c_abi=modes,
-        # the stand-alone differentiable op lm_head_logprobs_entropy: its forward writes softmax partials only, its
-        # backward forms the logits of the tokens with a gradient again (6 T_grad V H flops executed)
-        standalone_op=dict(fwd_ms=f_ms, bwd_ms=b_ms, fwd_tflops=2.0 * T * V * H / (f_ms * 1e-3) / 1e12,
-                           bwd_executed_tflops=6.0 * op_kept * V * H / (b_ms * 1e-3) / 1e12,
-                           # lm_head_logprobs_entropy(backward="carry"): the forward also keeps the bf16 rows of the
-                           # tokens with a gradient, the backward is the two gradient GEMMs (4 T_grad V H flops)
-                           carry_fwd_ms=fc_ms, carry_bwd_ms=bc_ms,
-                           carry_bwd_tflops=4.0 * op_kept * V * H / (bc_ms * 1e-3) / 1e12),
+        standalone_op=standalone,
     )
     # the measured ceiling of the matrix cores in this process: a loop of MFMAs only (no LDS, no memory traffic)
     mfma_only = time_mfma_only_loop(dev)
