@@ -127,6 +127,7 @@ SIGNATURES = {
     "aa_segment_copy": (_i, [_p, _p, _i64, _p, _p, _p, _i64, _i64, _p]),
     "aa_copy_bytes": (_i, [_p, _p, _i64, _p]),
     "aa_mfma_only_loop": (_i, [_i, _i, _i, _i, _p, _p]),
+    "aa_hbm_stream_probe": (_i, [_i, _i, _p, _p, _i64, _i, _p]),
 }
 
 _lib = None

@@ -93,6 +93,51 @@ __device__ __forceinline__ void load8(const void* base, int64_t i, float (&x)[8]
   }
 }
 
+// The same with the `nt` cache policy: for data that is read once (a read-only pass over a large array sustains
+// 7.1 TB/s with it against 6.3 TB/s without on this part).
+template <int DT>
+__device__ __forceinline__ void load8_stream(const void* base, int64_t i, float (&x)[8]) {
+  typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+  if constexpr (DT == AA_F32) {
+    const u32x4_t* p = (const u32x4_t*)((const float*)base + i);
+    const u32x4_t a = __builtin_nontemporal_load(p), b = __builtin_nontemporal_load(p + 1);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      x[q] = __uint_as_float(a[q]);
+      x[4 + q] = __uint_as_float(b[q]);
+    }
+  } else {
+    const u32x4_t q = __builtin_nontemporal_load((const u32x4_t*)((const uint16_t*)base + i));
+    x[0] = Elem<DT>::lo(q[0]); x[1] = Elem<DT>::hi(q[0]);
+    x[2] = Elem<DT>::lo(q[1]); x[3] = Elem<DT>::hi(q[1]);
+    x[4] = Elem<DT>::lo(q[2]); x[5] = Elem<DT>::hi(q[2]);
+    x[6] = Elem<DT>::lo(q[3]); x[7] = Elem<DT>::hi(q[3]);
+  }
+}
+
+// four consecutive fp32 values at a 16-byte aligned address, `nt` policy
+__device__ __forceinline__ void load4_stream(const float* p, float* x) {
+  typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+  const u32x4_t a = __builtin_nontemporal_load((const u32x4_t*)p);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) x[q] = __uint_as_float(a[q]);
+}
+
+__device__ __forceinline__ void store4_stream(float* p, const float* x) {
+  typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+  const u32x4_t v = {__float_as_uint(x[0]), __float_as_uint(x[1]), __float_as_uint(x[2]), __float_as_uint(x[3])};
+  __builtin_nontemporal_store(v, (u32x4_t*)p);
+}
+
+// eight 16-bit values to consecutive addresses, `nt` policy
+template <int DT>
+__device__ __forceinline__ void store8_stream16(void* base, int64_t i, const float (&x)[8]) {
+  typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+  const u32x4_t q = {Elem<DT>::pack(x[0], x[1]), Elem<DT>::pack(x[2], x[3]), Elem<DT>::pack(x[4], x[5]),
+                     Elem<DT>::pack(x[6], x[7])};
+  __builtin_nontemporal_store(q, (u32x4_t*)((uint16_t*)base + i));
+}
+
 template <int DT>
 __device__ __forceinline__ void store8(void* base, int64_t i, const float (&x)[8]) {
   if constexpr (DT == AA_F32) {

@@ -86,6 +86,31 @@ __device__ __forceinline__ void stats_add8(ThreadStats& a, const float (&x)[8], 
   a.u += u;
 }
 
+// The same with the parts left out that a caller has no use for: the entropy sum u (WANT_U) and the extrema
+// (WANT_MM; the eight-way maximum is needed for the reference exponent either way).  A forward pass for log-probs
+// alone is otherwise bound by these instructions on 16-bit rows, not by the memory.
+template <bool WANT_U, bool WANT_MM>
+__device__ __forceinline__ void stats_add8_sel(ThreadStats& a, const float (&x)[8], float c) {
+  const float m8 = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+  const float kc = m8 * c;
+  if (kc > a.k) rebase(a, kc);
+  if constexpr (WANT_MM) {
+    const float n8 = fminf(fminf(fminf(x[0], x[1]), fminf(x[2], x[3])), fminf(fminf(x[4], x[5]), fminf(x[6], x[7])));
+    a.mx = fmaxf(a.mx, m8);
+    a.mn = fminf(a.mn, n8);
+  }
+  float s = 0.f, u = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float t = fmaf(x[i], c, -a.k);
+    const float e = fast_exp2(t);
+    s += e;
+    if constexpr (WANT_U) u = fmaf(t, e, u);
+  }
+  a.s += s;
+  if constexpr (WANT_U) a.u += u;
+}
+
 struct RowStats {
   float k, s, u, mx, mn;  // merged over the workgroup, same value in every thread
 };
@@ -131,16 +156,38 @@ __device__ __forceinline__ RowStats block_stats(const ThreadStats& t, float* sme
   return r;
 }
 
-template <int DT, int NT>
+template <int DT, int NT, bool STREAM = false, bool WANT_U = true, bool WANT_MM = true>
 __device__ __forceinline__ RowStats row_stats_generic(const void* row, int V, bool vec_ok, float c, float* smem) {
   ThreadStats a{kNegBig, 0.f, 0.f, -FLT_MAX, FLT_MAX};
   const RowSplit sp = split_row<DT>(row, V, vec_ok);
   const int tid = threadIdx.x;
   for (int j = tid; j < sp.head; j += NT) stats_add1(a, Elem<DT>::load1(row, j), c);
-  for (int v = tid; v < sp.nvec; v += NT) {
-    float x[8];
-    load8<DT>(row, sp.head + ((int64_t)v << 3), x);
-    stats_add8(a, x, c);
+  if constexpr (STREAM && DT == AA_F32) {
+    // fp32, read once: a thread's eight values are two 16-byte pieces NT pieces apart, so that every load instruction
+    // of a wave covers 1 KB of consecutive addresses (eight values side by side make two instructions touch every
+    // 128-byte line: slower, and the nt policy then costs instead of gaining); statistics do not depend on the order
+    const int n4 = sp.nvec * 2;  // 16-byte pieces of the vector body
+    const float* body = (const float*)row + sp.head;
+    int v = tid;
+    for (; v + NT < n4; v += 2 * NT) {
+      float x[8];
+      load4_stream(body + ((int64_t)v << 2), x);
+      load4_stream(body + ((int64_t)(v + NT) << 2), x + 4);
+      stats_add8_sel<WANT_U, WANT_MM>(a, x, c);
+    }
+    if (v < n4) {
+      float x[4];
+      load4_stream(body + ((int64_t)v << 2), x);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) stats_add1(a, x[i], c);
+    }
+  } else {
+    for (int v = tid; v < sp.nvec; v += NT) {
+      float x[8];
+      if constexpr (STREAM) load8_stream<DT>(row, sp.head + ((int64_t)v << 3), x);  // the row is not read again
+      else load8<DT>(row, sp.head + ((int64_t)v << 3), x);
+      stats_add8_sel<WANT_U, WANT_MM>(a, x, c);
+    }
   }
   for (int j = sp.tail0 + tid; j < V; j += NT) stats_add1(a, Elem<DT>::load1(row, j), c);
   return block_stats<NT / kWave>(a, smem);
@@ -182,7 +229,9 @@ struct GradCoef {
 // has a NaN gradient in the reference as well (the entropy itself is NaN there).
 __device__ __forceinline__ float grad_weight(const GradCoef& g, float x) { return g.B == 0.f ? g.A : fmaf(g.B, x, g.A); }
 
-template <int DT, int NT>
+// STREAM: the row and its gradient pass through once (`nt` policy on loads and stores); fp32 rows then go in 16-byte
+// pieces, so that every load and store instruction of a wave covers 1 KB of consecutive addresses.
+template <int DT, int NT, bool STREAM = false>
 __device__ __forceinline__ void row_grad_generic(const void* row, void* out, int V, bool vec_ok, const GradCoef& g) {
   const RowSplit sp = split_row<DT>(row, V, vec_ok);
   const int tid = threadIdx.x;
@@ -193,10 +242,29 @@ __device__ __forceinline__ void row_grad_generic(const void* row, void* out, int
     Elem<DT>::store1(out, j, o);
   };
   for (int j = tid; j < sp.head; j += NT) one(j);
+  if constexpr (STREAM && DT == AA_F32) {
+    const int n4 = sp.nvec * 2;
+    for (int v = tid; v < n4; v += NT) {
+      const int e0 = sp.head + (v << 2);
+      float x[4], o[4];
+      load4_stream((const float*)row + e0, x);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] = fast_exp2(fmaf(x[i], g.c, -g.lse2)) * grad_weight(g, x[i]);
+      if ((unsigned)(g.label - e0) < 4u) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (e0 + i == g.label) o[i] += g.lab_add;
+      }
+      store4_stream((float*)out + e0, o);
+    }
+    for (int j = sp.tail0 + tid; j < V; j += NT) one(j);
+    return;
+  }
   for (int v = tid; v < sp.nvec; v += NT) {
     const int e0 = sp.head + (v << 3);
     float x[8], o[8];
-    load8<DT>(row, e0, x);
+    if constexpr (STREAM) load8_stream<DT>(row, e0, x);
+    else load8<DT>(row, e0, x);
 #pragma unroll
     for (int i = 0; i < 8; ++i) o[i] = fast_exp2(fmaf(x[i], g.c, -g.lse2)) * grad_weight(g, x[i]);
     if ((unsigned)(g.label - e0) < 8u) {
@@ -204,18 +272,25 @@ __device__ __forceinline__ void row_grad_generic(const void* row, void* out, int
       for (int i = 0; i < 8; ++i)
         if (e0 + i == g.label) o[i] += g.lab_add;
     }
-    store8<DT>(out, e0, o);
+    if constexpr (STREAM && DT != AA_F32) store8_stream16<DT>(out, e0, o);
+    else store8<DT>(out, e0, o);
   }
   for (int j = sp.tail0 + tid; j < V; j += NT) one(j);
 }
 
-template <int DT, int NT>
+template <int DT, int NT, bool STREAM = false>
 __device__ __forceinline__ void row_zero_generic(const void* row_like, void* out, int V, bool vec_ok) {
   const RowSplit sp = split_row<DT>(row_like, V, vec_ok);
   const int tid = threadIdx.x;
   const float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   for (int j = tid; j < sp.head; j += NT) Elem<DT>::store1(out, j, 0.f);
-  for (int v = tid; v < sp.nvec; v += NT) store8<DT>(out, sp.head + (v << 3), z);
+  if constexpr (STREAM && DT == AA_F32) {
+    for (int v = tid; v < sp.nvec * 2; v += NT) store4_stream((float*)out + sp.head + (v << 2), z);
+  } else if constexpr (STREAM) {
+    for (int v = tid; v < sp.nvec; v += NT) store8_stream16<DT>(out, sp.head + (v << 3), z);
+  } else {
+    for (int v = tid; v < sp.nvec; v += NT) store8<DT>(out, sp.head + (v << 3), z);
+  }
   for (int j = sp.tail0 + tid; j < V; j += NT) Elem<DT>::store1(out, j, 0.f);
 }
 
@@ -226,7 +301,7 @@ __device__ __forceinline__ const void* row_ptr(const void* base, int64_t t, int6
 // -----------------------------------------------------------------------------
 // Forward: logp, entropy, row statistics.  grid = T rows, NT threads.
 // -----------------------------------------------------------------------------
-template <int DT, int NT>
+template <int DT, int NT, bool WANT_U, bool WANT_MM>
 __global__ __launch_bounds__(NT) void k_logits_fwd(const void* __restrict__ logits, int V, int64_t stride,
                                                    const int64_t* __restrict__ labels, float inv_t, int vec_ok,
                                                    float* __restrict__ logp, float* __restrict__ entropy,
@@ -239,7 +314,7 @@ __global__ __launch_bounds__(NT) void k_logits_fwd(const void* __restrict__ logi
   const int64_t y = labels[t];
   const bool y_ok = (y >= 0) && (y < V);
   const float xy = y_ok ? Elem<DT>::load1(row, y) : 0.f;
-  const RowStats rs = row_stats_generic<DT, NT>(row, V, vec_ok != 0, c, smem);
+  const RowStats rs = row_stats_generic<DT, NT, true, WANT_U, WANT_MM>(row, V, vec_ok != 0, c, smem);
   if (threadIdx.x == 0) {
     const RowOut ro = finish_row(rs);
     logp[t] = y_ok ? label_logp(xy, c, rs, ro) : __builtin_nanf("");
@@ -274,7 +349,9 @@ struct OutPtr<true, T> {
 // -----------------------------------------------------------------------------
 // Backward: dlogits from g_logp / g_entropy and the saved row statistics.
 // -----------------------------------------------------------------------------
-template <int DT, int NT, bool ALIAS>
+// STREAM: `nt` loads and stores (the host asks for them when the rows start on 128-byte lines: with rows that do
+// not, the pieces that two waves write into one line are no longer merged in the cache, and the pass is slower).
+template <int DT, int NT, bool ALIAS, bool STREAM>
 __global__ __launch_bounds__(NT) void k_logits_bwd(typename InPtr<ALIAS, void>::type logits, int V, int64_t stride,
                                                    const int64_t* __restrict__ labels, float inv_t, int vec_ok,
                                                    const float* __restrict__ row_lse,
@@ -288,7 +365,7 @@ __global__ __launch_bounds__(NT) void k_logits_bwd(typename InPtr<ALIAS, void>::
   const float gl = (t < T_active) ? g_logp[t] : 0.f;
   const float gh = (t < T_active && g_entropy) ? g_entropy[t] : 0.f;
   if (gl == 0.f && gh == 0.f) {
-    row_zero_generic<DT, NT>(row, out, V, vec_ok != 0);
+    row_zero_generic<DT, NT, STREAM>(row, out, V, vec_ok != 0);
     return;
   }
   const int64_t y = labels[t];
@@ -300,7 +377,7 @@ __global__ __launch_bounds__(NT) void k_logits_bwd(typename InPtr<ALIAS, void>::
   g.B = -gh * inv_t * inv_t;
   g.lab_add = gl * inv_t;
   g.label = (y >= 0 && y < V) ? (int)y : -1;
-  row_grad_generic<DT, NT>(row, out, V, vec_ok != 0, g);
+  row_grad_generic<DT, NT, STREAM>(row, out, V, vec_ok != 0, g);
 }
 
 // -----------------------------------------------------------------------------
@@ -1296,13 +1373,23 @@ extern "C" int aa_logits_fwd(const void* logits, int dtype, int64_t T, int64_t V
   hipStream_t st = (hipStream_t)stream;
   const int vec_ok = rows_vec_ok(logits, nullptr, dtype) ? 1 : 0;
   constexpr int NT = 256;
-#define AA_LAUNCH(DT)                                                                                        \
-  hipLaunchKernelGGL((k_logits_fwd<DT, NT>), dim3((unsigned)T), dim3(NT), 0, st, logits, (int)V, row_stride, \
+  // the entropy sum and the extrema are left out of the pass when no output asks for them
+  const bool want_u = entropy || row_ez, want_mm = vmax || vmin;
+#define AA_LAUNCH_AS(DT, U, MM)                                                                                      \
+  hipLaunchKernelGGL((k_logits_fwd<DT, NT, U, MM>), dim3((unsigned)T), dim3(NT), 0, st, logits, (int)V, row_stride, \
                      labels, inv_temperature, vec_ok, logp, entropy, row_lse, row_ez, vmax, vmin)
+#define AA_LAUNCH(DT)                                        \
+  do {                                                       \
+    if (want_u && want_mm) AA_LAUNCH_AS(DT, true, true);     \
+    else if (want_u) AA_LAUNCH_AS(DT, true, false);          \
+    else if (want_mm) AA_LAUNCH_AS(DT, false, true);         \
+    else AA_LAUNCH_AS(DT, false, false);                     \
+  } while (0)
   if (dtype == AA_BF16) AA_LAUNCH(AA_BF16);
   else if (dtype == AA_F16) AA_LAUNCH(AA_F16);
   else AA_LAUNCH(AA_F32);
 #undef AA_LAUNCH
+#undef AA_LAUNCH_AS
   return launch_status();
 }
 
@@ -1316,20 +1403,27 @@ extern "C" int aa_logits_bwd(const void* logits, int dtype, int64_t T, int64_t V
   hipStream_t st = (hipStream_t)stream;
   const int vec_ok = rows_vec_ok(logits, dlogits, dtype) ? 1 : 0;
   constexpr int NT = 256;
-#define AA_LAUNCH(DT)                                                                                                 \
-  do {                                                                                                                \
-    if (dlogits == logits)                                                                                            \
-      hipLaunchKernelGGL((k_logits_bwd<DT, NT, true>), dim3((unsigned)T), dim3(NT), 0, st, logits, (int)V, row_stride, \
-                         labels, inv_temperature, vec_ok, row_lse, row_ez, g_logp, g_entropy, T_active, dlogits);     \
-    else                                                                                                              \
-      hipLaunchKernelGGL((k_logits_bwd<DT, NT, false>), dim3((unsigned)T), dim3(NT), 0, st, logits, (int)V,           \
-                         row_stride, labels, inv_temperature, vec_ok, row_lse, row_ez, g_logp, g_entropy, T_active,   \
-                         dlogits);                                                                                    \
+  // rows on 128-byte lines take the streaming cache policy
+  const int64_t row_bytes = row_stride * (dtype == AA_F32 ? 4 : 2);
+  const bool streaming = vec_ok && row_bytes % 128 == 0 && ((((uintptr_t)logits | (uintptr_t)dlogits) & 127) == 0);
+#define AA_LAUNCH_AS(DT, ALIAS, STREAM)                                                                               \
+  hipLaunchKernelGGL((k_logits_bwd<DT, NT, ALIAS, STREAM>), dim3((unsigned)T), dim3(NT), 0, st, logits, (int)V,      \
+                     row_stride, labels, inv_temperature, vec_ok, row_lse, row_ez, g_logp, g_entropy, T_active, dlogits)
+#define AA_LAUNCH(DT)                                                \
+  do {                                                               \
+    if (dlogits == logits) {                                         \
+      if (streaming) AA_LAUNCH_AS(DT, true, true);                    \
+      else AA_LAUNCH_AS(DT, true, false);                            \
+    } else {                                                         \
+      if (streaming) AA_LAUNCH_AS(DT, false, true);                    \
+      else AA_LAUNCH_AS(DT, false, false);                           \
+    }                                                                \
   } while (0)
   if (dtype == AA_BF16) AA_LAUNCH(AA_BF16);
   else if (dtype == AA_F16) AA_LAUNCH(AA_F16);
   else AA_LAUNCH(AA_F32);
 #undef AA_LAUNCH
+#undef AA_LAUNCH_AS
   return launch_status();
 }
 

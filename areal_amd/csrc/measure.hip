@@ -1,5 +1,6 @@
-// Measurement helper for the matrix cores: a loop that issues nothing but MFMAs on operands that never leave the
-// registers.  What it sustains is the ceiling that this chip, at its power limit, sets for any bf16 tile GEMM (no LDS,
+// Measurement helpers.  For the HBM-bound kernels: plain streams (read only, write only, copy) with either cache
+// policy, which give the rates that this memory system sustains in each direction.  For the matrix cores: a loop that
+// issues nothing but MFMAs on operands that never leave the registers.  What it sustains is the ceiling that this chip, at its power limit, sets for any bf16 tile GEMM (no LDS,
 // no memory traffic, no epilogue), in the same sense in which k_copy16 is the measured ceiling of the HBM-bound kernels.
 // Not on any product path.
 #include "device_utils.h"
@@ -98,10 +99,91 @@ __global__ __launch_bounds__(256) void k_mfma_16x16x32(float* __restrict__ out, 
   out[id] = s;
 }
 
+// ---- HBM streams: read only, write only, copy ------------------------------------------------------------------------
+// Every workgroup moves pieces of 256 threads x 8 vectors of 16 bytes (32 KB, consecutive addresses per wave
+// instruction), dealt round-robin; NT selects the `nt` cache policy.  The read kernel folds what it reads into a word
+// that is never equal to the magic value, so nothing is written.
+template <bool NT>
+__global__ __launch_bounds__(256) void k_stream_read(const u32x4_t* __restrict__ src, int64_t n_vec, uint32_t* sink) {
+  constexpr int U = 8;
+  u32x4_t acc = {0u, 0u, 0u, 0u};
+  for (int64_t p = blockIdx.x; p * (256 * U) < n_vec; p += gridDim.x) {
+    const u32x4_t* base = src + p * (256 * U) + threadIdx.x;
+    u32x4_t v[U];
+#pragma unroll
+    for (int i = 0; i < U; ++i) {
+      const bool in = p * (256 * U) + i * 256 + threadIdx.x < n_vec;
+      const u32x4_t* q = in ? base + i * 256 : src;
+      v[i] = NT ? __builtin_nontemporal_load(q) : *q;
+    }
+#pragma unroll
+    for (int i = 0; i < U; ++i) acc ^= v[i];
+  }
+  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x5a17c0deu && sink) sink[0] = acc[0];
+}
+
+template <bool NT>
+__global__ __launch_bounds__(256) void k_stream_write(u32x4_t* __restrict__ dst, int64_t n_vec) {
+  constexpr int U = 8;
+  const u32x4_t v = {threadIdx.x, blockIdx.x, 2u, 3u};
+  for (int64_t p = blockIdx.x; p * (256 * U) < n_vec; p += gridDim.x) {
+    u32x4_t* base = dst + p * (256 * U) + threadIdx.x;
+#pragma unroll
+    for (int i = 0; i < U; ++i) {
+      if (p * (256 * U) + i * 256 + threadIdx.x < n_vec) {
+        if (NT) __builtin_nontemporal_store(v, base + i * 256);
+        else base[i * 256] = v;
+      }
+    }
+  }
+}
+
+template <bool NT>
+__global__ __launch_bounds__(256) void k_stream_copy(const u32x4_t* __restrict__ src, u32x4_t* __restrict__ dst, int64_t n_vec) {
+  constexpr int U = 8;
+  for (int64_t p = blockIdx.x; p * (256 * U) < n_vec; p += gridDim.x) {
+    const int64_t at = p * (256 * U) + threadIdx.x;
+    u32x4_t v[U];
+#pragma unroll
+    for (int i = 0; i < U; ++i) {
+      const u32x4_t* q = at + i * 256 < n_vec ? src + at + i * 256 : src;
+      v[i] = NT ? __builtin_nontemporal_load(q) : *q;
+    }
+#pragma unroll
+    for (int i = 0; i < U; ++i) {
+      if (at + i * 256 < n_vec) {
+        if (NT) __builtin_nontemporal_store(v[i], dst + at + i * 256);
+        else dst[at + i * 256] = v[i];
+      }
+    }
+  }
+}
+
 }  // namespace measure
 }  // namespace aa
 
 using namespace aa;
+
+extern "C" int aa_hbm_stream_probe(int kind, int nt_policy, const void* src, void* dst, int64_t bytes, int workgroups,
+                                   void* stream) {
+  if (kind < 0 || kind > 2 || bytes <= 0 || bytes % 16 != 0 || workgroups <= 0 || workgroups > 65536) return AA_ERR_INVALID_ARGUMENT;
+  if ((kind != 1 && (!src || ((uintptr_t)src & 15))) || (kind != 0 && (!dst || ((uintptr_t)dst & 15)))) return AA_ERR_INVALID_ARGUMENT;
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t n_vec = bytes / 16;
+  const dim3 grid((unsigned)workgroups), block(256);
+  typedef measure::u32x4_t vec;
+  if (kind == 0) {
+    if (nt_policy) hipLaunchKernelGGL(measure::k_stream_read<true>, grid, block, 0, st, (const vec*)src, n_vec, (uint32_t*)dst);
+    else hipLaunchKernelGGL(measure::k_stream_read<false>, grid, block, 0, st, (const vec*)src, n_vec, (uint32_t*)dst);
+  } else if (kind == 1) {
+    if (nt_policy) hipLaunchKernelGGL(measure::k_stream_write<true>, grid, block, 0, st, (vec*)dst, n_vec);
+    else hipLaunchKernelGGL(measure::k_stream_write<false>, grid, block, 0, st, (vec*)dst, n_vec);
+  } else {
+    if (nt_policy) hipLaunchKernelGGL(measure::k_stream_copy<true>, grid, block, 0, st, (const vec*)src, (vec*)dst, n_vec);
+    else hipLaunchKernelGGL(measure::k_stream_copy<false>, grid, block, 0, st, (const vec*)src, (vec*)dst, n_vec);
+  }
+  return launch_status();
+}
 
 extern "C" int aa_mfma_only_loop(int form, int random_operands, int workgroups, int iters, float* out, void* stream) {
   if (!out || workgroups <= 0 || workgroups > 65536 || iters <= 0 || (form != 0 && form != 1)) return AA_ERR_INVALID_ARGUMENT;

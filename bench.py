@@ -10,7 +10,8 @@ One "step" is one pass of the hot path over one synthetic packed micro-batch tha
   loss, i.e. ``fused_logprobs_ppo_loss(...)`` followed by ``loss.backward()``.  Roofline: HBM, algorithmic bytes
   4 * V per token (the bf16 logits read once, their gradient written once); ``--logits-dtype f32`` casts the logits
   to fp32 first (8 * V per token).  The line also carries ``sft_loss_same_logits``: the supervised loss on the same
-  logits, fused in one pass against the log-prob op followed by the loss and a separate backward pass.
+  logits, fused in one pass against the log-prob op followed by the loss and a separate backward pass, and
+  ``forward_only_logprobs``: the forward-only op on the same logits (read once: 2 * V bytes per bf16 token).
 * fused lm_head workloads (cfg2, cfg3, cfg4): ``fused_lm_head_ppo_loss(hidden, W, labels, ...)`` followed by
   ``loss.backward()``: lm_head, log-prob / entropy, PPO loss and the gradients d(hidden), d(W) on this library's own
   bf16 MFMA tile GEMM; the forward writes no logits.  Roofline: bf16 MFMA, from HIP events around every step of the
@@ -41,7 +42,8 @@ and, in the default run only (every GPU timing is taken before the first CPU bas
   fused_lm_head               the same figures for the cfg2 workload, so that one run reports both paths;
   fused_lm_head_cfg3, _cfg4   the cfg3 and cfg4 workloads (GPU only: three timed steps each, their own roofline).
 
-``--workload mfma`` runs the MFMA-only loop (aa_mfma_only_loop: no LDS, no memory traffic), the measured ceiling that
+``--workload hbm`` runs plain HBM streams (aa_hbm_stream_probe: read only, write only, copy, either cache policy), the
+measured ceilings of the logits path.  ``--workload mfma`` runs the MFMA-only loop (aa_mfma_only_loop: no LDS, no memory traffic), the measured ceiling that
 the fused lm_head figures are also quoted against (``roofline.frac_of_mfma_only_loop``).
 """
 from __future__ import annotations
@@ -64,7 +66,7 @@ METRIC = "tokens/sec for logprob+entropy+PPO loss fwd+bwd; % HBM / % MFMA peak" 
 LOGITS_WORKLOADS = ("cfg0", "cfg1", "cfg1-32k")
 FUSED_WORKLOADS = ("cfg2", "cfg3", "cfg4")
 ADV_WORKLOADS = ("adv", "aux")
-MFMA_WORKLOADS = ("mfma",)
+MFMA_WORKLOADS = ("mfma", "hbm")
 
 
 def parse_args():
@@ -394,6 +396,8 @@ def bench_logits(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: 
         out["config"]["importance_weight_cap"] = f"{cfg.level} {cfg.metric} <= {cfg.upper}, action={cfg.action}"
     if with_sft:
         out["sft_loss_same_logits"] = time_sft_steps(case, max(steps // 2, 3))
+    # the forward-only op on the same logits (compute_logp: log-probs of a reference or proximal policy): one read
+    out["forward_only_logprobs"] = time_forward_only(case, max(steps, 10))
     # the measured ceiling of a read-once / write-once kernel on buffers of this size
     dst = torch.empty_like(case.logits)
     out["copy_same_buffers"] = time_copy_kernel(case.logits, dst, max(steps, 10))
@@ -419,6 +423,34 @@ def bench_logits(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: 
         bytes_of_logits_and_gradient=case.logits.numel() * case.logits.element_size(),
         note="inplace_backward=True; after the first launch the rows hold gradients, the traffic is the same")
     return out, sample
+
+
+def time_forward_only(case, iters: int):
+    """aa_logits_fwd (k_logits_fwd) on the workload's logits: log-probs alone (what ``gather_logprobs`` asks for), and
+    with entropy and the vocabulary extrema.  Algorithmic bytes: every logit read once."""
+    import torch
+
+    from areal_amd import _native as N
+    from areal_amd import functional as F
+
+    lib = N.load()
+    dev = case.logits.device
+    T, V = case.logits.shape
+    f32 = dict(dtype=torch.float32, device=dev)
+    logp, ent, vmax, vmin = (torch.empty(T, **f32) for _ in range(4))
+    stream = torch.cuda.current_stream(dev)
+    st = C.c_void_p(stream.cuda_stream)
+    nbytes = float(case.logits.numel() * case.logits.element_size())
+    out = dict(kernel="k_logits_fwd (aa_logits_fwd)", algorithmic_bytes_per_launch=nbytes)
+    for name, extra in (("logprobs_only", (None, None, None, None, None)),
+                        ("with_entropy_and_extrema", (F._ptr(ent), None, None, F._ptr(vmax), F._ptr(vmin)))):
+        def launch():
+            N.check(lib.aa_logits_fwd(F._ptr(case.logits), F._DTYPES[case.logits.dtype], T, V, V, F._ptr(case.labels),
+                                      1.0 / case.temperature, F._ptr(logp), *extra, st), "aa_logits_fwd")
+        ms, ms_min = time_events(launch, iters, stream)
+        out[name] = dict(avg_kernel_ms=ms, min_kernel_ms=ms_min, achieved=nbytes / (ms * 1e-3) / 1e9, unit="GB/s",
+                         frac=nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, tokens_per_s=T / (ms * 1e-3))
+    return out
 
 
 def finish_with_cpu_phase(out, sample, cpu_phase, iters: int):
@@ -903,6 +935,46 @@ def bench_mfma(args, dev):
     )
 
 
+def bench_hbm(args, dev):
+    """Plain streams over 20 GB (aa_hbm_stream_probe): read only, write only and copy, with the default and with the
+    streaming cache policy.  The measured ceilings beside the HBM-bound kernels of the logits path."""
+    import torch
+
+    from areal_amd import _native as N
+    from areal_amd import functional as F
+
+    lib = N.load()
+    nbytes = 20 << 30
+    src = torch.full((nbytes,), 1, dtype=torch.uint8, device=dev)
+    dst = torch.full((nbytes,), 2, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev)
+    st = C.c_void_p(stream.cuda_stream)
+    wgs = 8 * torch.cuda.get_device_properties(dev).multi_processor_count
+    res = {}
+    for kind, name, moved in ((0, "read", nbytes), (1, "write", nbytes), (2, "copy", 2 * nbytes)):
+        for nt in (0, 1):
+            def launch():
+                N.check(lib.aa_hbm_stream_probe(kind, nt, F._ptr(src), F._ptr(dst), nbytes, wgs, st), "aa_hbm_stream_probe")
+            ms, ms_min = time_events(launch, max(args.steps, 10), stream)
+            res[f"{name}, {'nt' if nt else 'default'} policy"] = dict(avg_ms=ms, min_ms=ms_min, gb_per_s=moved / (ms * 1e-3) / 1e9,
+                                                                      frac_of_peak=moved / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS)
+    rd = max(res["read, nt policy"]["gb_per_s"], res["read, default policy"]["gb_per_s"])
+    wr = max(res["write, nt policy"]["gb_per_s"], res["write, default policy"]["gb_per_s"])
+    both = 2.0 / (1.0 / rd + 1.0 / wr)
+    return dict(
+        metric="GB/s of plain HBM streams (read only, write only, copy): the measured ceilings of the logits path",
+        value=both, unit="GB/s", n_gpus=1, steps=max(args.steps, 10), warmup=5, higher_is_better=True, dtype="u8",
+        data="synthetic", vs_baseline=None, scaling="weak",
+        config=dict(workload="aa_hbm_stream_probe over 20 GiB buffers, 8 workgroups of 256 threads per compute unit, "
+                             "32 KB pieces"),
+        roofline=dict(bound="hbm", kernel="k_stream_read / k_stream_write", achieved=both, peak=HBM_PEAK_GBS, unit="GB/s",
+                      frac=both / HBM_PEAK_GBS, traffic=None,
+                      note="value = rate of a kernel that reads as many bytes as it writes if its reads ran at the read-only "
+                           "rate and its writes at the write-only rate (harmonic mean of the two)"),
+        streams=res,
+    )
+
+
 # ----------------------------------------------------------------------------------------------------------------
 # advantage pipeline
 # ----------------------------------------------------------------------------------------------------------------
@@ -1122,7 +1194,9 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    if args.workload in MFMA_WORKLOADS:
+    if args.workload == "hbm":
+        out = bench_hbm(args, dev)
+    elif args.workload in MFMA_WORKLOADS:
         out = bench_mfma(args, dev)
     elif args.workload == "aux":
         out = bench_aux(args, dev)
@@ -1136,7 +1210,8 @@ def main():
             # configs[1] says "T = 32k" of a length distribution that draws about 130k tokens: the headline figures
             # are on the distribution as stated; the same sequences cut at 32 768 tokens are quoted beside them
             torch.cuda.empty_cache()
-            keys = ("value", "unit", "ms_per_step", "steps", "warmup", "config", "roofline", "copy_same_buffers")
+            keys = ("value", "unit", "ms_per_step", "steps", "warmup", "config", "roofline", "copy_same_buffers",
+                    "forward_only_logprobs")
             cut, _ = bench_logits(args, dev, "cfg1-32k", args.steps, args.warmup, 0, with_sft=False)
             out["configs1_cut_to_32k_tokens"] = {k: cut[k] for k in keys}
             torch.cuda.empty_cache()

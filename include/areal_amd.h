@@ -887,6 +887,16 @@ int aa_copy_bytes(const void* src, void* dst, int64_t nbytes, void* stream);
 int aa_mfma_only_loop(int form, int random_operands, int workgroups, int iters,
                       float* out, void* stream);
 
+/* Plain streams over `bytes` bytes (a multiple of 16, 16-byte aligned), the
+ * measured ceilings beside the HBM-bound kernels: kind 0 reads src (nothing
+ * is written; dst may be NULL), kind 1 writes dst (src may be NULL), kind 2
+ * copies src to dst.  nt_policy != 0 selects the streaming (`nt`) cache
+ * policy for the loads and stores.  `workgroups` workgroups of 256 threads
+ * deal 32 KB pieces among themselves.  No counterpart in the reference; not on
+ * any product path. */
+int aa_hbm_stream_probe(int kind, int nt_policy, const void* src, void* dst,
+                        int64_t bytes, int workgroups, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

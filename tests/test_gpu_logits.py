@@ -316,3 +316,32 @@ def test_backward_written_over_the_logits(device, V, dtype):
     l0, s0 = step(False)
     l1, s1 = step(True)
     assert torch.equal(l0, l1) and torch.equal(s0, s1)
+
+
+def test_hbm_stream_probe_moves_what_it_says(device):
+    """The measurement kernels behind `bench.py --workload hbm`: the copy copies every byte (ragged last piece
+    included), the write fills exactly the buffer, the read writes nothing, with either cache policy."""
+    import ctypes as C
+
+    from areal_amd import _native as N
+    from areal_amd import functional as F
+
+    lib = N.load()
+    st = C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    n = 16 * (256 * 8 * 5 + 77)                              # five whole 32 KB pieces and a ragged one
+    src = torch.randint(0, 256, (n,), dtype=torch.uint8, device=device)
+    for nt in (0, 1):
+        dst = torch.full((n + 64,), 7, dtype=torch.uint8, device=device)
+        assert lib.aa_hbm_stream_probe(2, nt, F._ptr(src), F._ptr(dst), n, 3, st) == 0
+        assert torch.equal(dst[:n], src) and bool((dst[n:] == 7).all())
+        dst.fill_(7)
+        assert lib.aa_hbm_stream_probe(1, nt, None, F._ptr(dst), n, 3, st) == 0
+        assert bool((dst[n:] == 7).all())
+        words = dst[:n].view(torch.int32).view(-1, 4)
+        assert bool((words[:, 2] == 2).all()) and bool((words[:, 3] == 3).all())
+        before = src.clone()
+        assert lib.aa_hbm_stream_probe(0, nt, F._ptr(src), None, n, 3, st) == 0
+        assert torch.equal(src, before)
+    assert lib.aa_hbm_stream_probe(3, 0, F._ptr(src), None, n, 3, st) == 1      # unknown kind
+    assert lib.aa_hbm_stream_probe(2, 0, F._ptr(src), None, n, 3, st) == 1      # a copy needs a destination
+    assert lib.aa_hbm_stream_probe(0, 0, F._ptr(src), None, n + 8, 3, st) == 1  # not a multiple of 16
