@@ -100,39 +100,47 @@ __global__ __launch_bounds__(256) void k_mfma_16x16x32(float* __restrict__ out, 
 }
 
 // ---- HBM streams: read only, write only, copy ------------------------------------------------------------------------
-// Every workgroup moves pieces of 256 threads x 8 vectors of 16 bytes (32 KB, consecutive addresses per wave
-// instruction), dealt round-robin; NT selects the `nt` cache policy.  The read kernel folds what it reads into a word
-// that is never equal to the magic value, so nothing is written.
+// Every workgroup moves spans of kSpan pieces of 256 threads x 8 vectors of 16 bytes (a span is 512 KB of consecutive
+// addresses, 1 KB per wave instruction, eight instructions in flight per lane), dealt round-robin: the way the
+// row-per-workgroup kernels of the logits path walk memory.  NT selects the `nt` cache policy.  The read kernel folds
+// what it reads into a word that is never equal to the magic value, so nothing is written.
+constexpr int kU = 8;
+constexpr int kSpan = 16;
+constexpr int64_t kPieceVecs = 256 * kU;
+
 template <bool NT>
 __global__ __launch_bounds__(256) void k_stream_read(const u32x4_t* __restrict__ src, int64_t n_vec, uint32_t* sink) {
-  constexpr int U = 8;
   u32x4_t acc = {0u, 0u, 0u, 0u};
-  for (int64_t p = blockIdx.x; p * (256 * U) < n_vec; p += gridDim.x) {
-    const u32x4_t* base = src + p * (256 * U) + threadIdx.x;
-    u32x4_t v[U];
+  for (int64_t sp = blockIdx.x; sp * (kSpan * kPieceVecs) < n_vec; sp += gridDim.x) {
+    for (int j = 0; j < kSpan; ++j) {
+      const int64_t at = (sp * kSpan + j) * kPieceVecs + threadIdx.x;
+      if (at - threadIdx.x >= n_vec) break;
+      u32x4_t v[kU];
 #pragma unroll
-    for (int i = 0; i < U; ++i) {
-      const bool in = p * (256 * U) + i * 256 + threadIdx.x < n_vec;
-      const u32x4_t* q = in ? base + i * 256 : src;
-      v[i] = NT ? __builtin_nontemporal_load(q) : *q;
+      for (int i = 0; i < kU; ++i) {
+        const u32x4_t* q = at + i * 256 < n_vec ? src + at + i * 256 : src;
+        v[i] = NT ? __builtin_nontemporal_load(q) : *q;
+      }
+#pragma unroll
+      for (int i = 0; i < kU; ++i) acc ^= v[i];
     }
-#pragma unroll
-    for (int i = 0; i < U; ++i) acc ^= v[i];
   }
   if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x5a17c0deu && sink) sink[0] = acc[0];
 }
 
 template <bool NT>
 __global__ __launch_bounds__(256) void k_stream_write(u32x4_t* __restrict__ dst, int64_t n_vec) {
-  constexpr int U = 8;
   const u32x4_t v = {threadIdx.x, blockIdx.x, 2u, 3u};
-  for (int64_t p = blockIdx.x; p * (256 * U) < n_vec; p += gridDim.x) {
-    u32x4_t* base = dst + p * (256 * U) + threadIdx.x;
+  for (int64_t sp = blockIdx.x; sp * (kSpan * kPieceVecs) < n_vec; sp += gridDim.x) {
+    for (int j = 0; j < kSpan; ++j) {
+      const int64_t at = (sp * kSpan + j) * kPieceVecs + threadIdx.x;
+      if (at - threadIdx.x >= n_vec) break;
 #pragma unroll
-    for (int i = 0; i < U; ++i) {
-      if (p * (256 * U) + i * 256 + threadIdx.x < n_vec) {
-        if (NT) __builtin_nontemporal_store(v, base + i * 256);
-        else base[i * 256] = v;
+      for (int i = 0; i < kU; ++i) {
+        if (at + i * 256 < n_vec) {
+          if (NT) __builtin_nontemporal_store(v, dst + at + i * 256);
+          else dst[at + i * 256] = v;
+        }
       }
     }
   }
@@ -140,20 +148,22 @@ __global__ __launch_bounds__(256) void k_stream_write(u32x4_t* __restrict__ dst,
 
 template <bool NT>
 __global__ __launch_bounds__(256) void k_stream_copy(const u32x4_t* __restrict__ src, u32x4_t* __restrict__ dst, int64_t n_vec) {
-  constexpr int U = 8;
-  for (int64_t p = blockIdx.x; p * (256 * U) < n_vec; p += gridDim.x) {
-    const int64_t at = p * (256 * U) + threadIdx.x;
-    u32x4_t v[U];
+  for (int64_t sp = blockIdx.x; sp * (kSpan * kPieceVecs) < n_vec; sp += gridDim.x) {
+    for (int j = 0; j < kSpan; ++j) {
+      const int64_t at = (sp * kSpan + j) * kPieceVecs + threadIdx.x;
+      if (at - threadIdx.x >= n_vec) break;
+      u32x4_t v[kU];
 #pragma unroll
-    for (int i = 0; i < U; ++i) {
-      const u32x4_t* q = at + i * 256 < n_vec ? src + at + i * 256 : src;
-      v[i] = NT ? __builtin_nontemporal_load(q) : *q;
-    }
+      for (int i = 0; i < kU; ++i) {
+        const u32x4_t* q = at + i * 256 < n_vec ? src + at + i * 256 : src;
+        v[i] = NT ? __builtin_nontemporal_load(q) : *q;
+      }
 #pragma unroll
-    for (int i = 0; i < U; ++i) {
-      if (at + i * 256 < n_vec) {
-        if (NT) __builtin_nontemporal_store(v[i], dst + at + i * 256);
-        else dst[at + i * 256] = v[i];
+      for (int i = 0; i < kU; ++i) {
+        if (at + i * 256 < n_vec) {
+          if (NT) __builtin_nontemporal_store(v[i], dst + at + i * 256);
+          else dst[at + i * 256] = v[i];
+        }
       }
     }
   }
