@@ -154,6 +154,29 @@ __device__ __forceinline__ void store8(void* base, int64_t i, const float (&x)[8
   }
 }
 
+// ---- extrema of a few values ------------------------------------------------
+// IEEE 754-2019 maximum / minimum (a NaN input gives NaN, as torch.max does) on the three-input instructions of
+// gfx950.  fmaxf / fminf would first pass every value that comes straight out of a load or a shift through a
+// canonicalising v_max_f32 x, x: one more instruction per element in loops that are bound by their instructions.
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  return __builtin_elementwise_maximum(__builtin_elementwise_maximum(a, b), c);
+}
+__device__ __forceinline__ float min3(float a, float b, float c) {
+  return __builtin_elementwise_minimum(__builtin_elementwise_minimum(a, b), c);
+}
+template <int N>
+__device__ __forceinline__ float max_of(const float* x) {
+  static_assert(N == 4 || N == 8, "four or eight values");
+  if constexpr (N == 4) return max3(max3(x[0], x[1], x[2]), x[3], x[3]);
+  else return max3(max3(x[0], x[1], x[2]), max3(x[3], x[4], x[5]), __builtin_elementwise_maximum(x[6], x[7]));
+}
+template <int N>
+__device__ __forceinline__ float min_of(const float* x) {
+  static_assert(N == 4 || N == 8, "four or eight values");
+  if constexpr (N == 4) return min3(min3(x[0], x[1], x[2]), x[3], x[3]);
+  else return min3(min3(x[0], x[1], x[2]), min3(x[3], x[4], x[5]), __builtin_elementwise_minimum(x[6], x[7]));
+}
+
 // ---- wave64 reductions -------------------------------------------------------
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll

@@ -63,17 +63,16 @@ __device__ __forceinline__ void stats_add1(ThreadStats& a, float x, float c) {
   const float e = fast_exp2(t);
   a.s += e;
   a.u = fmaf(t, e, a.u);
-  a.mx = fmaxf(a.mx, x);
-  a.mn = fminf(a.mn, x);
+  a.mx = __builtin_elementwise_maximum(a.mx, x);
+  a.mn = __builtin_elementwise_minimum(a.mn, x);
 }
 
 __device__ __forceinline__ void stats_add8(ThreadStats& a, const float (&x)[8], float c) {
-  float m8 = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
-  float n8 = fminf(fminf(fminf(x[0], x[1]), fminf(x[2], x[3])), fminf(fminf(x[4], x[5]), fminf(x[6], x[7])));
+  const float m8 = max_of<8>(x), n8 = min_of<8>(x);
   const float kc = m8 * c;
   if (kc > a.k) rebase(a, kc);
-  a.mx = fmaxf(a.mx, m8);
-  a.mn = fminf(a.mn, n8);
+  a.mx = __builtin_elementwise_maximum(a.mx, m8);
+  a.mn = __builtin_elementwise_minimum(a.mn, n8);
   float s = 0.f, u = 0.f;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
@@ -91,13 +90,13 @@ __device__ __forceinline__ void stats_add8(ThreadStats& a, const float (&x)[8], 
 // alone is otherwise bound by these instructions on 16-bit rows, not by the memory.
 template <bool WANT_U, bool WANT_MM>
 __device__ __forceinline__ void stats_add8_sel(ThreadStats& a, const float (&x)[8], float c) {
-  const float m8 = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+  const float m8 = max_of<8>(x);
   const float kc = m8 * c;
   if (kc > a.k) rebase(a, kc);
   if constexpr (WANT_MM) {
-    const float n8 = fminf(fminf(fminf(x[0], x[1]), fminf(x[2], x[3])), fminf(fminf(x[4], x[5]), fminf(x[6], x[7])));
-    a.mx = fmaxf(a.mx, m8);
-    a.mn = fminf(a.mn, n8);
+    const float n8 = min_of<8>(x);
+    a.mx = __builtin_elementwise_maximum(a.mx, m8);
+    a.mn = __builtin_elementwise_minimum(a.mn, n8);
   }
   float s = 0.f, u = 0.f;
 #pragma unroll
@@ -627,17 +626,12 @@ __device__ __forceinline__ void held4(const uint32_t* w, float* x) {
 // statistics of N more values without a branch (the rescaling factor is 1 when the maximum stays)
 template <int N>
 __device__ __forceinline__ void stats_add_flat(ThreadStats& a, const float* x, float c) {
-  float m = x[0], n = x[0];
-#pragma unroll
-  for (int i = 1; i < N; ++i) {
-    m = fmaxf(m, x[i]);
-    n = fminf(n, x[i]);
-  }
+  const float m = max_of<N>(x), n = min_of<N>(x);
   const float k_new = fmaxf(a.k, m * c);
   const float d = a.k - k_new;
   const float f = fast_exp2(d);
-  a.mx = fmaxf(a.mx, m);
-  a.mn = fminf(a.mn, n);
+  a.mx = __builtin_elementwise_maximum(a.mx, m);
+  a.mn = __builtin_elementwise_minimum(a.mn, n);
   float s = 0.f, u = 0.f;
 #pragma unroll
   for (int i = 0; i < N; ++i) {
