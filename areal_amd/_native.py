@@ -13,6 +13,7 @@ LIB_PATH = Path(__file__).resolve().parent / "libareal_amd.so"
 
 AA_OK = 0
 AA_ERR_INVALID_ARGUMENT = 1
+AA_LMHEAD_COUNT_ON_DEVICE = -1  # a kept_per_chunk entry: the device counts the rows itself
 AA_ERR_UNSUPPORTED = 2
 AA_ERR_LAUNCH = 3
 AA_BF16, AA_F16, AA_F32 = 0, 1, 2

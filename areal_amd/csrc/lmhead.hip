@@ -66,6 +66,7 @@ struct TileArgs {
   const float* g_entropy;  // nullable
   float inv_t;
   const int32_t* run_if;   // recompute tiles only: when given, the kernel does nothing unless *run_if != 0
+  const int32_t* n_bound;  // recompute tiles only: when given, only the tiles over the first *n_bound token columns run
 };
 
 // Carry mode stores 2^(x c - kref) with kref = c * (label logit of the token): a reference that is known before the
@@ -172,6 +173,15 @@ __global__ __launch_bounds__(kThreads) void k_lmhead_tiles(Operand W, Operand Hd
   extern __shared__ __attribute__((aligned(16))) char lds[];
   if constexpr (MODE == kModeRecompute) {
     if (a.run_if && *a.run_if == 0) return;  // uniform over the grid
+  }
+  if constexpr (MODE == kModeRecompute) {
+    // token columns in use, known to the device alone: the tiles that cover them are numbered as if the host had
+    // launched exactly those (the same walk over the XCDs), the workgroups beyond them return
+    if (a.n_bound) {
+      const int live = (*a.n_bound + BN - 1) / BN;
+      tiles_n = live < tiles_n ? live : tiles_n;
+      if ((int)blockIdx.x >= tiles_m * tiles_n) return;  // the same decision in every thread of the workgroup
+    }
   }
   int tm, tn;
   tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
@@ -491,14 +501,29 @@ __global__ __launch_bounds__(256) void k_carry_factors(const float* __restrict__
 // 512 contiguous bytes per row; row n of the product is written to row c_rows[n] of C when a row list is given.
 // fp32 C: 16-byte stores straight from the registers; ACCUM adds to what C holds.
 template <bool AKM, bool BKM, typename OutT, bool ACCUM>
+// n_bound / k_bound, when given, hold a count that only the device knows (the number of panel rows in use, at most
+// the N or K the host launched with): only the tiles over the first *n_bound rows of B run (numbered as a grid of just
+// those tiles; the other workgroups return at once), and the contraction stops at *k_bound rounded up to a whole K
+// slice (the rows up to there are zero).
 __global__ __launch_bounds__(kThreads) void k_gemm_store(Operand A, Operand B, int K, int tiles_m, int tiles_n,
                                                          OutT* __restrict__ C, int64_t ldc,
                                                          const int32_t* __restrict__ c_rows,
-                                                         const float* __restrict__ n_scale) {
+                                                         const float* __restrict__ n_scale,
+                                                         const int32_t* __restrict__ n_bound,
+                                                         const int32_t* __restrict__ k_bound) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
+  if (n_bound) {  // the tiles over the rows in use are numbered as if the host had launched exactly those
+    const int live = (*n_bound + BN - 1) / BN;
+    tiles_n = live < tiles_n ? live : tiles_n;
+    if ((int)blockIdx.x >= tiles_m * tiles_n) return;  // the same decision in every thread of the workgroup
+  }
   int tm, tn;
   tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
+  if (k_bound) {  // at least one slice: the main loop always starts one
+    const int kb = *k_bound > 0 ? (*k_bound + BK - 1) / BK * BK : BK;
+    K = kb < K ? kb : K;
+  }
   Acc acc;
   mainloop<AKM, BKM>(A, B, K, m0, n0, acc, lds);  // ends with a barrier: LDS is free
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -681,10 +706,16 @@ __global__ __launch_bounds__(1024) void k_compact_map(const uint8_t* __restrict_
 
 // Panel rows [*total, limit) are rows without a token (see k_compact_map): cleared, one workgroup per row at a time.
 // In the usual case (*total == limit) every workgroup returns at once.
-__global__ __launch_bounds__(256) void k_clear_surplus_rows(const int32_t* __restrict__ total, int limit,
+// With `bounded` the kernels that read the panel stop at *total themselves (rounded up to a K slice of the d_weight
+// product), and only the rows up to there are cleared.
+__global__ __launch_bounds__(256) void k_clear_surplus_rows(const int32_t* __restrict__ total, int limit, int bounded,
                                                             u32x4_t* __restrict__ panel, int64_t panel_ld) {
   const u32x4_t zero = {0u, 0u, 0u, 0u};
   const int64_t vec = panel_ld / 8;
+  if (bounded) {
+    const int up = *total > 0 ? (*total + BK - 1) / BK * BK : BK;
+    limit = up < limit ? up : limit;
+  }
   for (int64_t r = (int64_t)*total + blockIdx.x; r < limit; r += gridDim.x)
     for (int64_t i = threadIdx.x; i < vec; i += 256) panel[r * vec + i] = zero;
 }
@@ -692,13 +723,13 @@ __global__ __launch_bounds__(256) void k_clear_surplus_rows(const int32_t* __res
 // numbering of the tokens with a panel row, and the rows without a token cleared (both kernels)
 static void launch_compact_map(hipStream_t st, const uint8_t* mask, int64_t act, int64_t n_tok, int64_t limit,
                                int32_t* out_rows, int32_t* act_rows, float* row_factor, int32_t* total_word,
-                               uint16_t* panel, int64_t panel_ld) {
+                               uint16_t* panel, int64_t panel_ld, bool bounded = false) {
   hipLaunchKernelGGL(k_compact_map, dim3(1), dim3(1024), 0, st, mask, (int)act, (int)n_tok, (int)limit, out_rows, act_rows,
                      row_factor, total_word);
-  const int64_t blocks = limit < 512 ? limit : 512;
+  const int64_t blocks = bounded ? (limit < BK ? limit : BK) : (limit < 512 ? limit : 512);
   if (blocks > 0)
     hipLaunchKernelGGL(k_clear_surplus_rows, dim3((unsigned)blocks), dim3(256), 0, st, total_word, (int)limit,
-                       (u32x4_t*)panel, panel_ld);
+                       bounded ? 1 : 0, (u32x4_t*)panel, panel_ld);
 }
 
 // dst[r, :] = scale[r] * src[rows[r], :] (H % 8 == 0); rows == nullptr: row r itself (a negative entry: a zero row);
@@ -879,11 +910,12 @@ static void launch_tiles(hipStream_t st, const void* weight, const uint16_t* hid
 template <bool AKM, bool BKM, typename OutT, bool ACCUM>
 static void launch_gemm(hipStream_t st, const uint16_t* A, int64_t lda, int64_t M, const uint16_t* B, int64_t ldb, int64_t N,
                         int64_t K, OutT* C, int64_t ldc, const int32_t* c_rows = nullptr,
-                        const float* n_scale = nullptr) {
+                        const float* n_scale = nullptr, const int32_t* n_bound = nullptr,
+                        const int32_t* k_bound = nullptr) {
   const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
   Operand a{A, lda, (int)M}, b{B, ldb, (int)N};
   hipLaunchKernelGGL((k_gemm_store<AKM, BKM, OutT, ACCUM>), dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads), kLdsBytes, st,
-                     a, b, (int)K, tiles_m, tiles_n, C, ldc, c_rows, n_scale);
+                     a, b, (int)K, tiles_m, tiles_n, C, ldc, c_rows, n_scale, n_bound, k_bound);
 }
 
 // The two GEMMs that contract the d(logits) rows ds [n_rows, V] of one token chunk, ds = row_factor[r] * panel[r, :]
@@ -897,7 +929,8 @@ static void launch_gemm(hipStream_t st, const uint16_t* A, int64_t lda, int64_t 
 // go to those tokens (the caller has cleared the others).
 static void panel_gradients(hipStream_t st, const Workspace& w, char* ws, const uint16_t* ds, const void* weight,
                             const uint16_t* hid, const int32_t* token_of_row, const float* row_factor, int64_t n_rows,
-                            int64_t H, int64_t V, uint16_t* d_hidden_chunk, void* d_weight, bool dw_f32, bool first) {
+                            int64_t H, int64_t V, uint16_t* d_hidden_chunk, void* d_weight, bool dw_f32, bool first,
+                            const int32_t* rows_in_use = nullptr) {
   const uint16_t* hid_rows = hid;
   if (token_of_row || row_factor) {
     uint16_t* hc = (uint16_t*)(ws + w.off_hc);
@@ -908,10 +941,11 @@ static void panel_gradients(hipStream_t st, const Workspace& w, char* ws, const 
   const int64_t ldp = w.panel_ld;
   {
     const int tiles_m = (int)((H + BM - 1) / BM), tiles_n = (int)((n_rows + BN - 1) / BN);
-    const int splits = choose_splits((int64_t)tiles_m * tiles_n, (V + BK - 1) / BK, compute_units());
+    // with the row count on the device alone (n_rows is its upper bound) the product is not cut along the vocabulary
+    const int splits = rows_in_use ? 1 : choose_splits((int64_t)tiles_m * tiles_n, (V + BK - 1) / BK, compute_units());
     if (splits == 1) {
       launch_gemm<true, false, uint16_t, false>(st, (const uint16_t*)weight, H, H, ds, ldp, n_rows, V, d_hidden_chunk, H,
-                                                token_of_row, row_factor);
+                                                token_of_row, row_factor, rows_in_use, nullptr);
     } else {
       float* part = (float*)(ws + w.off_dhp);
       const int64_t plane = n_rows * H;
@@ -923,11 +957,14 @@ static void panel_gradients(hipStream_t st, const Workspace& w, char* ws, const 
     }
   }
   if (!dw_f32)
-    launch_gemm<true, true, uint16_t, false>(st, hid_rows, H, H, ds, ldp, V, n_rows, (uint16_t*)d_weight, H);
+    launch_gemm<true, true, uint16_t, false>(st, hid_rows, H, H, ds, ldp, V, n_rows, (uint16_t*)d_weight, H, nullptr, nullptr,
+                                             nullptr, rows_in_use);
   else if (first)
-    launch_gemm<true, true, float, false>(st, hid_rows, H, H, ds, ldp, V, n_rows, (float*)d_weight, H);
+    launch_gemm<true, true, float, false>(st, hid_rows, H, H, ds, ldp, V, n_rows, (float*)d_weight, H, nullptr, nullptr,
+                                          nullptr, rows_in_use);
   else
-    launch_gemm<true, true, float, true>(st, hid_rows, H, H, ds, ldp, V, n_rows, (float*)d_weight, H);
+    launch_gemm<true, true, float, true>(st, hid_rows, H, H, ds, ldp, V, n_rows, (float*)d_weight, H, nullptr, nullptr,
+                                         nullptr, rows_in_use);
 }
 
 // Recompute: d(logits) of the panel rows from the logits tiles formed again.  With a row map only the hidden rows that
@@ -935,11 +972,12 @@ static void panel_gradients(hipStream_t st, const Workspace& w, char* ws, const 
 // kernels are enqueued but do nothing unless *run_if != 0 when they start.
 static void recompute_panel(hipStream_t st, const Workspace& w, char* ws, uint16_t* panel, const void* weight,
                             const uint16_t* hid, int64_t n_tok, const int32_t* token_of_row, int64_t rows, int64_t H,
-                            int64_t V, TileArgs a, const int32_t* run_if = nullptr) {
+                            int64_t V, TileArgs a, const int32_t* run_if = nullptr, const int32_t* rows_in_use = nullptr) {
   a.panel = panel;
   a.panel_ld = w.panel_ld;
   a.out_rows = nullptr;
   a.run_if = run_if;
+  a.n_bound = token_of_row ? rows_in_use : nullptr;
   if (!token_of_row) {
     a.col_tokens = nullptr;
     launch_tiles<kModeRecompute>(st, weight, hid, n_tok, H, V, a);
@@ -1157,16 +1195,20 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
     }
     // rows whose upstream gradients are all zero are left out, as in aa_lmhead_ppo_fused
     int64_t kept = kept_per_chunk[chunk_index];
-    kept = kept < 0 ? 0 : (kept > n_tok ? n_tok : kept);
+    const bool on_device = kept == AA_LMHEAD_COUNT_ON_DEVICE;  // the kernels stop at the count they find themselves
+    kept = on_device ? n_tok : (kept < 0 ? 0 : (kept > n_tok ? n_tok : kept));
     if (kept == 0) {
       launch_zero(st, dh, n_tok * H * 2);
       continue;
     }
-    launch_compact_map(st, row_has_gradient + t0, n_tok, n_tok, kept, out_rows, act_rows, nullptr,
-                       (int32_t*)(ws + w.off_total), ws_panel, w.panel_ld);
-    recompute_panel(st, w, ws, ws_panel, weight, hid, n_tok, act_rows, kept, H, V, a);
+    int32_t* total_word = (int32_t*)(ws + w.off_total);
+    const int32_t* rows_in_use = on_device ? total_word : nullptr;
+    launch_compact_map(st, row_has_gradient + t0, n_tok, n_tok, kept, out_rows, act_rows, nullptr, total_word, ws_panel,
+                       w.panel_ld, on_device);
+    recompute_panel(st, w, ws, ws_panel, weight, hid, n_tok, act_rows, kept, H, V, a, nullptr, rows_in_use);
     launch_zero(st, dh, n_tok * H * 2);  // the rows of the other tokens
-    panel_gradients(st, w, ws, ws_panel, weight, hid, act_rows, nullptr, kept, H, V, dh, dw.acc, dw.acc_f32, first);
+    panel_gradients(st, w, ws, ws_panel, weight, hid, act_rows, nullptr, kept, H, V, dh, dw.acc, dw.acc_f32, first,
+                    rows_in_use);
     first = false;
   }
   if (first) launch_zero(st, dw.acc, V * H * (dw.acc_f32 ? 4 : 2));  // no row of the batch has a gradient
@@ -1366,11 +1408,16 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
     int64_t rows = n_tok;
     const int32_t* row_of_token = nullptr;
     const int32_t* token_of_row = nullptr;
+    const int32_t* rows_in_use = nullptr;
     if (kept_per_chunk) {
       rows = kept_per_chunk[chunk_index];
-      rows = rows < 0 ? 0 : (rows > act ? act : rows);
-      launch_compact_map(st, at(mask_eff), act, n_tok, rows, out_rows, act_rows, carry ? row_factor : nullptr,
-                         (int32_t*)(ws + w.off_total), panel, w.panel_ld);
+      // the count may be left to the device: every active token could have a row, the kernels stop at those in use
+      const bool on_device = rows == AA_LMHEAD_COUNT_ON_DEVICE;
+      rows = on_device ? act : (rows < 0 ? 0 : (rows > act ? act : rows));
+      int32_t* total_word = (int32_t*)(ws + w.off_total);
+      launch_compact_map(st, at(mask_eff), act, n_tok, rows, out_rows, act_rows, carry ? row_factor : nullptr, total_word,
+                         panel, w.panel_ld, on_device);
+      if (on_device) rows_in_use = total_word;
       row_of_token = out_rows;
       token_of_row = act_rows;
     }
@@ -1401,12 +1448,13 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
     // device: the kernels start and return at once otherwise), and then the row factors become 1
     a.row_lse = lse_tok;
     a.g_logp = g_tok;
-    recompute_panel(st, w, ws, panel, weight, hid, n_tok, token_of_row, rows, H, V, a, carry ? redo_flag : nullptr);
+    recompute_panel(st, w, ws, panel, weight, hid, n_tok, token_of_row, rows, H, V, a, carry ? redo_flag : nullptr,
+                    rows_in_use);
     if (carry)
       hipLaunchKernelGGL(k_unit_factors, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, row_factor, (int)rows, redo_flag);
     if (token_of_row) launch_zero(st, dh, n_tok * H * 2);  // the rows of the tokens without gradient
     panel_gradients(st, w, ws, panel, weight, hid, token_of_row, carry ? row_factor : nullptr, rows, H, V, dh, dw.acc,
-                    dw.acc_f32, first);
+                    dw.acc_f32, first, rows_in_use);
     first = false;
   }
   if (first) launch_zero(st, dw.acc, V * H * (dw.acc_f32 ? 4 : 2));  // no token of the batch has a gradient

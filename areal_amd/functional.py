@@ -179,6 +179,20 @@ class _LogprobsEntropy(torch.autograd.Function):
         return dlogits, None, None, None, None, None, None
 
 
+def _device_or_read_back_counts(T: int, T_active: int, mask_u8: torch.Tensor, on_device: bool) -> list[int]:
+    """``kept_per_chunk`` of the lm_head step when the caller gave none: left to the device (the kernels stop at the
+    rows in use, nothing is read back), or read back from the device (exact counts: one small copy that waits for the
+    mask)."""
+    chunk = int(N.load().aa_lmhead_chunk_tokens())
+    n_chunks = (T + chunk - 1) // chunk
+    if on_device:
+        return [N.AA_LMHEAD_COUNT_ON_DEVICE] * n_chunks
+    on = mask_u8.ne(0)
+    if n_chunks * chunk != T_active:
+        on = torch.nn.functional.pad(on, (0, n_chunks * chunk - T_active))
+    return _HostCounts(on.view(n_chunks, chunk).sum(1)).tolist()
+
+
 def _logprobs_impl(logits, labels, temperature, tp_group, want_entropy, want_minmax, inplace_backward=False):
     _check_tp(tp_group)
     _require_gpu(logits, "logits")
@@ -829,14 +843,12 @@ def _lmhead_recompute_backward(hidden, weight, labels, temperature, row_lse, row
     d_hidden = torch.empty_like(hidden)
     d_weight = torch.empty_like(weight)  # bf16: rounded once, after fp32 accumulation over the chunks
     ws = _lmhead_workspace(T, H, V, dev)
-    # Rows whose upstream gradients are all zero (masked tokens) are left out of the gradient GEMMs; their
-    # count per chunk sizes the GEMMs, so the host reads it here.
+    # Rows whose upstream gradients are all zero (masked tokens) are left out of the gradient GEMMs; the device counts
+    # them itself (no read-back: the host does not wait for the gradient to exist).
     has_grad = g_logp != 0 if g_entropy is None else (g_logp != 0) | (g_entropy != 0)
     chunk = int(lib.aa_lmhead_chunk_tokens())
     n_chunks = (T + chunk - 1) // chunk
-    padded = has_grad if n_chunks * chunk == T else torch.nn.functional.pad(has_grad, (0, n_chunks * chunk - T))
-    per_chunk = _HostCounts(padded.view(n_chunks, chunk).sum(1)).tolist()
-    kept = (C.c_int64 * n_chunks)(*per_chunk)
+    kept = (C.c_int64 * n_chunks)(*([N.AA_LMHEAD_COUNT_ON_DEVICE] * n_chunks))
     with torch.cuda.device(dev):
         N.check(
             lib.aa_lmhead_bwd(
@@ -1158,6 +1170,7 @@ def fused_lm_head_ppo_loss(
     kept_per_chunk: list[int] | None = None,
     backward: str = "carry",
     carry_rows_limit_bytes: int = 16 << 30,
+    count_on_device: bool = True,
 ) -> tuple[torch.Tensor, dict]:
     """lm_head + ``gather_logprobs_entropy`` + ``ppo_actor_loss_fn`` (+ backward) for one micro-batch.
 
@@ -1184,14 +1197,18 @@ def fused_lm_head_ppo_loss(
     modes use the same workspace (``2 * chunk * V`` bytes for the rows).
 
     ``skip_masked_tokens``: a token whose (effective) loss mask is zero has a zero gradient row, so the two gradient
-    GEMMs run on the other tokens only; the results are those of the dense computation.  The per-chunk token counts
-    size the GEMMs, so the host reads them (one small device-to-host copy that waits for the mask only) before it
-    queues the chunk.  ``False`` multiplies the zero rows through, as the reference's autograd does, without that
-    read.  A caller that already knows the counts on the host (the number of tokens with a non-zero effective mask
-    in each chunk of ``aa_lmhead_chunk_tokens()`` tokens, e.g. from the CPU copy of ``loss_mask`` when there is no rejection sampling) can
-    pass them as ``kept_per_chunk``; nothing is read back then.  A count that is too small drops the tokens beyond it
-    from the gradient; a count that is too large (e.g. counts of ``loss_mask`` while rejection sampling shrinks the
-    mask on the device) is safe: the surplus rows are cleared on the device and add nothing.
+    GEMMs run on the other tokens only; the results are those of the dense computation.  ``False`` multiplies the
+    zero rows through, as the reference's autograd does.  How many tokens of a chunk take part is counted on the
+    device (``count_on_device=True``, the default): the kernels are queued for every token that could and stop at
+    the rows in use, so the host neither needs the mask nor waits for the device.  With ``count_on_device=False`` the
+    host reads the per-chunk counts back (one small device-to-host copy that waits for the mask only) and sizes the
+    GEMMs exactly, which pays when few tokens of a chunk have a mask (the ``d_hidden`` product can then be cut along
+    the vocabulary to fill the chip).  A caller that already knows the counts on the host (the number of tokens with a
+    non-zero effective mask in each chunk of ``aa_lmhead_chunk_tokens()`` tokens, e.g. from the CPU copy of
+    ``loss_mask`` when there is no rejection sampling) can pass them as ``kept_per_chunk``; nothing is read back then
+    either.  A count that is too small drops the tokens beyond it from the gradient; a count that is too large (e.g.
+    counts of ``loss_mask`` while rejection sampling shrinks the mask on the device) is safe: the surplus rows are
+    cleared on the device and add nothing.
 
     ``stat`` also holds ``vocab_min_logits`` / ``vocab_max_logits`` (what the engine would read from materialised
     logits, areal/engine/fsdp_engine.py:1893-1906), from the fp32 sums of the tiles.
@@ -1316,12 +1333,7 @@ def fused_lm_head_ppo_loss(
         if len(kept) != (hidden.shape[0] + chunk - 1) // chunk:
             raise ValueError(f"kept_per_chunk needs one count per chunk of {chunk} tokens")
     elif skip_masked_tokens:
-        chunk = int(N.load().aa_lmhead_chunk_tokens())
-        n_chunks = (hidden.shape[0] + chunk - 1) // chunk
-        on = mask_eff.ne(0)
-        if n_chunks * chunk != T_active:
-            on = torch.nn.functional.pad(on, (0, n_chunks * chunk - T_active))
-        kept = _HostCounts(on.view(n_chunks, chunk).sum(1)).tolist()
+        kept = _device_or_read_back_counts(hidden.shape[0], T_active, mask_eff, count_on_device)
     loss, logp, entropy, stat_loss, ratio, flags, vmax, vmin = _FusedLmHeadPpo.apply(
         hidden.contiguous(), weight.contiguous(), y, float(temperature), T_active, prox, adv, mask_eff, w, params,
         n_valid, scale_t, kept, _LMHEAD_BACKWARD[backward],

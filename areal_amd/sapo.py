@@ -12,7 +12,6 @@ from . import _native as N
 from .functional import (
     _FusedLmHeadPpo,
     _FusedLogitsPpo,
-    _HostCounts,
     _count_nonzero,
     _f32,
     _mask_u8,
@@ -128,11 +127,8 @@ def fused_lm_head_sapo_loss(hidden: torch.Tensor, weight: torch.Tensor, labels: 
             kept = [int(v) for v in kept_per_chunk]
             if len(kept) != n_chunks:
                 raise ValueError(f"kept_per_chunk needs one count per chunk of {chunk} tokens")
-        else:
-            on = m8.ne(0)
-            if n_chunks * chunk != T_active:
-                on = torch.nn.functional.pad(on, (0, n_chunks * chunk - T_active))
-            kept = _HostCounts(on.view(n_chunks, chunk).sum(1)).tolist()
+        else:  # the device counts the tokens with a mask itself: nothing is read back
+            kept = [N.AA_LMHEAD_COUNT_ON_DEVICE] * n_chunks
     loss, logp, entropy, stat_loss, ratio, _flags, vmax, vmin = _FusedLmHeadPpo.apply(
         hidden.contiguous(), weight.contiguous(), y, float(temperature), T_active, old, adv, m8, None, params,
         _count_nonzero(m8), scale_t, kept, 1 if backward == "carry" else 0,

@@ -14,7 +14,6 @@ from .functional import (
     _DTYPES,
     _FusedLmHeadPpo,
     _FusedLogitsPpo,
-    _HostCounts,
     _count_nonzero,
     _f32,
     _mask_u8,
@@ -192,11 +191,8 @@ def fused_lm_head_sft_loss(hidden: torch.Tensor, weight: torch.Tensor, labels: t
             kept = [int(v) for v in kept_per_chunk]
             if len(kept) != n_chunks:
                 raise ValueError(f"kept_per_chunk needs one count per chunk of {chunk} tokens")
-        else:
-            on = m8.ne(0)
-            if n_chunks * chunk != T_active:
-                on = torch.nn.functional.pad(on, (0, n_chunks * chunk - T_active))
-            kept = _HostCounts(on.view(n_chunks, chunk).sum(1)).tolist()
+        else:  # the device counts the tokens with a mask itself: nothing is read back
+            kept = [N.AA_LMHEAD_COUNT_ON_DEVICE] * n_chunks
     loss, logp, entropy, stat_loss, _ratio, _flags, _vmax, _vmin = _FusedLmHeadPpo.apply(
         hidden.contiguous(), weight.contiguous(), y, float(temperature), T_active, None, None, m8, None, _nll_params(),
         n_valid, scale_t, kept, 1,  # aa_lmhead_backward_mode: carry

@@ -731,7 +731,7 @@ int64_t aa_lmhead_fwd_static_max_vocab(void);
  * its non-zero count per chunk of aa_lmhead_chunk_tokens() tokens), both or
  * neither: rows whose byte is zero must have g_logp == 0 and g_entropy == 0;
  * they are left out of all three GEMMs, and a chunk without any other row is
- * skipped altogether.
+ * skipped altogether.  An entry may be AA_LMHEAD_COUNT_ON_DEVICE.
  * workspace: aa_lmhead_workspace_bytes(T, H, V) bytes.
  */
 int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, int64_t H,
@@ -787,6 +787,15 @@ int aa_lmhead_bwd_carry(const void* hidden, const void* weight, int64_t T,
                         int d_weight_dtype, void* workspace,
                         int64_t workspace_bytes, void* stream);
 
+/* A kept_per_chunk entry that leaves the count to the device (aa_lmhead_bwd,
+ * aa_lmhead_ppo_fused): the kernels of that chunk are launched for every token
+ * that could have a row and stop at the rows in use, which the device counts
+ * itself, so the host needs no copy of the mask and does not wait for the
+ * device.  The price: workgroups that find nothing to do still start, and the
+ * d_hidden product is never cut along the vocabulary (which a host count well
+ * below a chunk can make worthwhile). */
+#define AA_LMHEAD_COUNT_ON_DEVICE (-1)
+
 /* How aa_lmhead_ppo_fused fills the d(logits) rows that its backward GEMMs
  * contract. */
 typedef enum {
@@ -832,7 +841,8 @@ typedef enum {
  * counts size the GEMMs, which is why they come from the host; tokens beyond a
  * count that is too small are treated as masked, and the surplus rows of a
  * count that is too large are cleared on the device and add nothing (slower,
- * same results).  NULL: every token has a row.
+ * same results).  An entry may be AA_LMHEAD_COUNT_ON_DEVICE: no host count
+ * is needed then.  NULL: every token has a row.
  * vocab_max / vocab_min [T] (nullable, both or neither): as in aa_lmhead_fwd.
  */
 int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64_t T,

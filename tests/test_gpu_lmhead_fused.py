@@ -558,6 +558,97 @@ def test_counts_larger_than_the_mask_holds_add_nothing(device, backward):
     assert_same_magnitude(over[3].float(), exact[3].float(), rel=1e-4)
 
 
+@pytest.mark.parametrize("backward", ["carry", "recompute"])
+@pytest.mark.parametrize("mask_kind", ["mixed", "second_chunk_empty", "nothing", "three_tokens"])
+def test_rows_counted_on_the_device_match_host_counts(device, backward, mask_kind):
+    """The default (``count_on_device=True``: the kernels are queued for every token that could have a row and stop at
+    the rows in use, which only the device knows) against counts read back by the host and against counts passed in:
+    the same loss, the same d(hidden) bits, the same d(W) up to the order of the sums; chunks with no token, with a
+    handful and with all but a few."""
+    T_pad, T = CHUNK + 256, CHUNK + 200
+    hidden, weight, labels, prox, old, adv, mask = _inputs(T_pad, T, 64, 640, seed=47)
+    if mask_kind == "second_chunk_empty":
+        mask[CHUNK:] = False
+    elif mask_kind == "nothing":
+        mask[:] = False
+    elif mask_kind == "three_tokens":
+        mask[:] = False
+        mask[[5, CHUNK - 1, CHUNK + 7]] = True
+    args = [t.to(device) for t in (labels, prox, old, adv)]
+    counts = [int(mask[:CHUNK].sum()), int(mask[CHUNK:].sum())]
+
+    def run(**kw):
+        h = hidden.to(device).requires_grad_(True)
+        w = weight.to(device).requires_grad_(True)
+        _poison_the_allocator_cache(device, int(_native.load().aa_lmhead_workspace_bytes(T_pad, 64, 640)))
+        loss, stat = areal_amd.fused_lm_head_ppo_loss(h, w, *args, eps_clip=0.2, loss_mask=mask.to(device),
+                                                      backward=backward, **kw)
+        loss.backward()
+        return loss.detach(), stat, h.grad, w.grad
+
+    on_device, read_back, given = run(), run(count_on_device=False), run(kept_per_chunk=counts)
+    for other in (read_back, given):
+        assert torch.equal(on_device[0], other[0])
+        assert torch.equal(on_device[1]["logprobs"], other[1]["logprobs"])
+        assert torch.isfinite(on_device[3].float()).all()
+        assert torch.equal(on_device[2], other[2])                                   # d(hidden): row by row the same
+        if mask.any():
+            assert cosine(on_device[3].float().cpu(), other[3].float().cpu()) > 0.9999999
+            assert_same_magnitude(on_device[3].float(), other[3].float(), rel=1e-4)
+        else:
+            assert float(on_device[3].float().abs().max()) == 0.0 and float(other[3].float().abs().max()) == 0.0
+    rows_off = torch.ones(T_pad, dtype=torch.bool, device=device)
+    rows_off[:T] = ~mask.to(device)
+    assert float(on_device[2][rows_off].float().abs().max()) == 0.0                  # tokens without a mask: zero rows
+
+
+def test_standalone_backward_counts_its_rows_on_the_device(device):
+    """``lm_head_logprobs_entropy`` (recompute backward): rows with a zero upstream gradient are left out without a
+    read-back, with the results of the dense backward; through the C ABI the same call with host counts and with
+    ``AA_LMHEAD_COUNT_ON_DEVICE`` entries gives the same gradients."""
+    import ctypes as C
+
+    from areal_amd import functional as F
+
+    T, H, V = CHUNK + 300, 64, 1288
+    g = torch.Generator().manual_seed(3)
+    hidden = torch.randn(T, H, generator=g).bfloat16().to(device)
+    weight = (0.3 * torch.randn(V, H, generator=g)).bfloat16().to(device)
+    labels = torch.randint(0, V, (T,), generator=g).to(device)
+    g_lp = (torch.randn(T, generator=g) * (torch.rand(T, generator=g) < 0.4)).to(device)
+    lib = _native.load()
+    f32 = dict(dtype=torch.float32, device=device)
+    logp, ent, lse, ez = (torch.empty(T, **f32) for _ in range(4))
+    ws = torch.empty(int(lib.aa_lmhead_workspace_bytes(T, H, V)), dtype=torch.uint8, device=device)
+    st = C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    assert lib.aa_lmhead_fwd(F._ptr(hidden), F._ptr(weight), T, H, V, F._ptr(labels), 1.0, F._ptr(logp), F._ptr(ent),
+                             F._ptr(lse), F._ptr(ez), None, None, F._ptr(ws), ws.numel(), st) == 0
+    has = (g_lp != 0).view(torch.uint8)
+
+    def bwd(kept):
+        dh, dw = torch.full_like(hidden, float("nan")), torch.full_like(weight, float("nan"))
+        arr = None if kept is None else (C.c_int64 * len(kept))(*kept)
+        assert lib.aa_lmhead_bwd(F._ptr(hidden), F._ptr(weight), T, H, V, F._ptr(labels), 1.0, F._ptr(lse), F._ptr(ez),
+                                 F._ptr(g_lp), None, F._ptr(has) if kept is not None else None, arr, F._ptr(dh), F._ptr(dw),
+                                 _native.AA_BF16, F._ptr(ws), ws.numel(), st) == 0
+        return dh, dw
+
+    dense = bwd(None)
+    host = bwd([int(has[:CHUNK].sum()), int(has[CHUNK:].sum())])
+    dev = bwd([_native.AA_LMHEAD_COUNT_ON_DEVICE] * 2)
+    assert torch.equal(host[0], dev[0]) and torch.equal(dense[0], dev[0])
+    for other in (host, dense):
+        assert cosine(dev[1].float().cpu(), other[1].float().cpu()) > 0.9999999
+        assert_same_magnitude(dev[1].float(), other[1].float(), rel=1e-4)
+    # and through autograd (the wrapper passes the device-count entries)
+    h = hidden.clone().requires_grad_(True)
+    w = weight.clone().requires_grad_(True)
+    lp, _ = areal_amd.lm_head_logprobs_entropy(h, w, labels)
+    (lp * g_lp).sum().backward()
+    assert torch.equal(h.grad, dev[0])
+    assert cosine(w.grad.float().cpu(), dev[1].float().cpu()) > 0.9999999
+
+
 def test_carry_with_unlikely_labels_at_masked_tokens_of_a_dense_backward(device):
     """``skip_masked_tokens=False`` puts every token in the panel.  A masked token (a prompt position) whose label is a
     hundred nats unlikely stores ratios p_v / p_label at the top of the bf16 range; their sum over the vocabulary may be
