@@ -494,6 +494,29 @@ __global__ __launch_bounds__(256) void k_carry_factors(const float* __restrict__
   if (g != 0.f && (lp < kCarryMinLogp || fabsf(f) < kCarryMinFactor)) *carry.redo_flag = 1;
 }
 
+// ---- the d_hidden product cut along K: into how many parts ---------------------------------------------------------
+// Into how many parts along K a product of `tiles` tiles and `slices` K slices is cut (1: not at all): the number of
+// parts, up to kMaxSplits, that shortens the time in rounds of tiles, ceil(tiles * parts / units) / parts, the most,
+// with 0.03 rounds charged per part for writing and adding its fp32 plane; at least 5 % have to be won, and a part
+// keeps at least 64 slices.  In whole numbers (rounds x 1200) so that the host and every workgroup of the kernels that
+// choose for themselves, from a row count that only the device holds, come to the same answer.
+constexpr int kMaxSplits = 4;
+constexpr int kRoundsUnit = 1200;  // divisible by every number of parts
+static_assert(kRoundsUnit % 2 == 0 && kRoundsUnit % 3 == 0 && kRoundsUnit % 4 == 0 && kMaxSplits <= 4, "rounds in whole numbers");
+__host__ __device__ inline int choose_splits(int64_t tiles, int64_t slices, int units) {
+  if (units <= 0 || tiles <= 0) return 1;
+  int best = 1;
+  int64_t best_rounds = (tiles + units - 1) / units * (kRoundsUnit * 95 / 100);  // one part, less the 5 % to be won
+  for (int parts = 2; parts <= kMaxSplits && slices / parts >= 64; ++parts) {
+    const int64_t r = (tiles * parts + units - 1) / units * (kRoundsUnit / parts) + (kRoundsUnit * 3 / 100) * parts;
+    if (r < best_rounds) {
+      best = parts;
+      best_rounds = r;
+    }
+  }
+  return best;
+}
+
 // ---- plain product C = B . A^T on the same main loop ---------------------------------------------------------------
 // C [N, M] row-major with leading dimension ldc: C[n][m] = sum_k B[n][k] A[m][k]; AKM / BKM: the operand is stored
 // K-major (see gemm_tn.h).  The operand whose rows are the columns of C goes first, because a lane of the accumulator layout owns one n and runs of four consecutive m: four
@@ -504,18 +527,20 @@ template <bool AKM, bool BKM, typename OutT, bool ACCUM>
 // n_bound / k_bound, when given, hold a count that only the device knows (the number of panel rows in use, at most
 // the N or K the host launched with): only the tiles over the first *n_bound rows of B run (numbered as a grid of just
 // those tiles; the other workgroups return at once), and the contraction stops at *k_bound rounded up to a whole K
-// slice (the rows up to there are zero).
+// slice (the rows up to there are zero).  With n_bound and split_units > 0 the whole grid returns when the product over
+// *n_bound rows is one that k_gemm_splitk, queued beside it, cuts along K on split_units compute units.
 __global__ __launch_bounds__(kThreads) void k_gemm_store(Operand A, Operand B, int K, int tiles_m, int tiles_n,
                                                          OutT* __restrict__ C, int64_t ldc,
                                                          const int32_t* __restrict__ c_rows,
                                                          const float* __restrict__ n_scale,
                                                          const int32_t* __restrict__ n_bound,
-                                                         const int32_t* __restrict__ k_bound) {
+                                                         const int32_t* __restrict__ k_bound, int split_units) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   if (n_bound) {  // the tiles over the rows in use are numbered as if the host had launched exactly those
     const int live = (*n_bound + BN - 1) / BN;
     tiles_n = live < tiles_n ? live : tiles_n;
     if ((int)blockIdx.x >= tiles_m * tiles_n) return;  // the same decision in every thread of the workgroup
+    if (split_units > 0 && choose_splits((int64_t)tiles_m * tiles_n, (K + BK - 1) / BK, split_units) != 1) return;
   }
   int tm, tn;
   tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
@@ -592,10 +617,20 @@ __global__ __launch_bounds__(kThreads) void k_gemm_store(Operand A, Operand B, i
 // the K slices [s * per, (s + 1) * per) into its own fp32 plane; k_splitk_rows adds the planes in order.  Workgroups
 // are numbered so that an XCD runs a contiguous range of (part, tile): the tiles that share operand slices in its L2
 // are those of one part.
+// With n_bound (the rows of B in use, known to the device alone; `splits` then holds the number of compute units) the
+// kernel numbers the tiles over those rows and chooses the number of parts itself, as the host would have with that
+// count; the workgroups beyond tiles x parts return at once, all of them when the product is not cut.
 template <bool AKM, bool BKM>
 __global__ __launch_bounds__(kThreads) void k_gemm_splitk(Operand A, Operand B, int K, int tiles_m, int tiles_n, int splits,
-                                                          float* __restrict__ part, int64_t ldc, int64_t plane) {
+                                                          float* __restrict__ part, int64_t ldc, int64_t plane,
+                                                          const int32_t* __restrict__ n_bound) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
+  if (n_bound) {
+    const int live = (*n_bound + BN - 1) / BN;
+    tiles_n = live < tiles_n ? live : tiles_n;
+    splits = choose_splits((int64_t)tiles_m * tiles_n, (K + BK - 1) / BK, splits);
+    if (splits == 1 || (int)blockIdx.x >= tiles_m * tiles_n * splits) return;  // the same in every thread
+  }
   const int tiles = tiles_m * tiles_n;
   const int q = xcd_contiguous(blockIdx.x, tiles * splits);
   const int split = q / tiles;
@@ -634,10 +669,19 @@ __global__ __launch_bounds__(kThreads) void k_gemm_splitk(Operand A, Operand B, 
 
 // out[c_rows[r], :] = bf16(n_scale[r] * (plane 0 + plane 1 + ...)[r, :]), the planes added in order; M % 8 == 0.
 // c_rows == nullptr: row r itself (a negative entry: the row is dropped); n_scale == nullptr: 1.
+// With n_bound (see k_gemm_splitk; `splits` then holds the number of compute units, tiles_m and slices describe the
+// product) only the rows below *n_bound are written, from the number of planes that kernel chose; none when it did not
+// cut the product.
 __global__ __launch_bounds__(256) void k_splitk_rows(const float* __restrict__ part, int splits, int64_t plane, int M,
                                                      const int32_t* __restrict__ c_rows, const float* __restrict__ n_scale,
-                                                     uint16_t* __restrict__ out, int64_t ldo) {
+                                                     uint16_t* __restrict__ out, int64_t ldo,
+                                                     const int32_t* __restrict__ n_bound, int tiles_m, int slices) {
   const int64_t r = blockIdx.x;
+  if (n_bound) {
+    if (r >= *n_bound) return;
+    splits = choose_splits((int64_t)tiles_m * ((*n_bound + BN - 1) / BN), slices, splits);
+    if (splits == 1) return;
+  }
   const int64_t dst = c_rows ? c_rows[r] : r;
   if (dst < 0) return;
   const float f = n_scale ? n_scale[r] : 1.f;
@@ -789,7 +833,6 @@ __global__ __launch_bounds__(256) void k_f32_to_bf16(const f32x4_t* __restrict__
 }
 
 // ---- workspace ---------------------------------------------------------------------------------------------------
-constexpr int kMaxSplits = 4;  // of the d_hidden product along K
 
 struct Workspace {
   int64_t chunk, blocks;                // tokens per chunk, 128-row vocabulary blocks
@@ -879,23 +922,6 @@ static int compute_units() {
   return units[dev] > 0 ? units[dev] : 0;
 }
 
-// Into how many parts along K a product of `tiles` tiles and `slices` K slices is cut (1: not at all): the number of
-// parts, up to kMaxSplits, that shortens the time in rounds of tiles, ceil(tiles * parts / units) / parts, the most,
-// with 0.03 rounds charged per part for writing and adding its fp32 plane; at least 5 % have to be won, and a part
-// keeps at least 64 slices.
-static int choose_splits(int64_t tiles, int64_t slices, int units) {
-  if (units <= 0 || tiles <= 0) return 1;
-  auto rounds = [&](int parts) { return (double)((tiles * parts + units - 1) / units) / parts + 0.03 * parts; };
-  int best = 1;
-  double best_rounds = (rounds(1) - 0.03) * 0.95;
-  for (int parts = 2; parts <= kMaxSplits && slices / parts >= 64; ++parts)
-    if (rounds(parts) < best_rounds) {
-      best = parts;
-      best_rounds = rounds(parts);
-    }
-  return best;
-}
-
 template <int MODE>
 static void launch_tiles(hipStream_t st, const void* weight, const uint16_t* hid, int64_t n_tok, int64_t H, int64_t V,
                          const TileArgs& a) {
@@ -911,11 +937,11 @@ template <bool AKM, bool BKM, typename OutT, bool ACCUM>
 static void launch_gemm(hipStream_t st, const uint16_t* A, int64_t lda, int64_t M, const uint16_t* B, int64_t ldb, int64_t N,
                         int64_t K, OutT* C, int64_t ldc, const int32_t* c_rows = nullptr,
                         const float* n_scale = nullptr, const int32_t* n_bound = nullptr,
-                        const int32_t* k_bound = nullptr) {
+                        const int32_t* k_bound = nullptr, int split_units = 0) {
   const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
   Operand a{A, lda, (int)M}, b{B, ldb, (int)N};
   hipLaunchKernelGGL((k_gemm_store<AKM, BKM, OutT, ACCUM>), dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads), kLdsBytes, st,
-                     a, b, (int)K, tiles_m, tiles_n, C, ldc, c_rows, n_scale, n_bound, k_bound);
+                     a, b, (int)K, tiles_m, tiles_n, C, ldc, c_rows, n_scale, n_bound, k_bound, split_units);
 }
 
 // The two GEMMs that contract the d(logits) rows ds [n_rows, V] of one token chunk, ds = row_factor[r] * panel[r, :]
@@ -941,19 +967,39 @@ static void panel_gradients(hipStream_t st, const Workspace& w, char* ws, const 
   const int64_t ldp = w.panel_ld;
   {
     const int tiles_m = (int)((H + BM - 1) / BM), tiles_n = (int)((n_rows + BN - 1) / BN);
-    // with the row count on the device alone (n_rows is its upper bound) the product is not cut along the vocabulary
-    const int splits = rows_in_use ? 1 : choose_splits((int64_t)tiles_m * tiles_n, (V + BK - 1) / BK, compute_units());
-    if (splits == 1) {
+    const int64_t slices = (V + BK - 1) / BK;
+    const int units = compute_units();
+    float* part = (float*)(ws + w.off_dhp);
+    const int64_t plane = n_rows * H;
+    Operand a{(const uint16_t*)weight, H, (int)H}, b{ds, ldp, (int)n_rows};
+    if (rows_in_use) {
+      // the row count is on the device alone (n_rows is its upper bound): both forms of the product are queued, each
+      // kernel works out from the count whether the product is cut along the vocabulary and into how many parts (what
+      // the host would have chosen with that count), and the form that is not in turn returns at once
+      int64_t cut_groups = 0;  // the largest grid the cut product can ask for
+      for (int tn = 1; tn <= tiles_n; ++tn) {
+        const int parts = choose_splits((int64_t)tiles_m * tn, slices, units);
+        if (parts > 1 && (int64_t)tiles_m * tn * parts > cut_groups) cut_groups = (int64_t)tiles_m * tn * parts;
+      }
       launch_gemm<true, false, uint16_t, false>(st, (const uint16_t*)weight, H, H, ds, ldp, n_rows, V, d_hidden_chunk, H,
-                                                token_of_row, row_factor, rows_in_use, nullptr);
+                                                token_of_row, row_factor, rows_in_use, nullptr, cut_groups ? units : 0);
+      if (cut_groups) {
+        hipLaunchKernelGGL((k_gemm_splitk<true, false>), dim3((unsigned)cut_groups), dim3(kThreads), kLdsBytes, st, a, b,
+                           (int)V, tiles_m, tiles_n, units, part, H, plane, rows_in_use);
+        hipLaunchKernelGGL(k_splitk_rows, dim3((unsigned)n_rows), dim3(256), 0, st, part, units, plane, (int)H, token_of_row,
+                           row_factor, d_hidden_chunk, H, rows_in_use, tiles_m, (int)slices);
+      }
     } else {
-      float* part = (float*)(ws + w.off_dhp);
-      const int64_t plane = n_rows * H;
-      Operand a{(const uint16_t*)weight, H, (int)H}, b{ds, ldp, (int)n_rows};
-      hipLaunchKernelGGL((k_gemm_splitk<true, false>), dim3((unsigned)(tiles_m * tiles_n * splits)), dim3(kThreads), kLdsBytes,
-                         st, a, b, (int)V, tiles_m, tiles_n, splits, part, H, plane);
-      hipLaunchKernelGGL(k_splitk_rows, dim3((unsigned)n_rows), dim3(256), 0, st, part, splits, plane, (int)H, token_of_row,
-                         row_factor, d_hidden_chunk, H);
+      const int splits = choose_splits((int64_t)tiles_m * tiles_n, slices, units);
+      if (splits == 1) {
+        launch_gemm<true, false, uint16_t, false>(st, (const uint16_t*)weight, H, H, ds, ldp, n_rows, V, d_hidden_chunk, H,
+                                                  token_of_row, row_factor);
+      } else {
+        hipLaunchKernelGGL((k_gemm_splitk<true, false>), dim3((unsigned)(tiles_m * tiles_n * splits)), dim3(kThreads),
+                           kLdsBytes, st, a, b, (int)V, tiles_m, tiles_n, splits, part, H, plane, (const int32_t*)nullptr);
+        hipLaunchKernelGGL(k_splitk_rows, dim3((unsigned)n_rows), dim3(256), 0, st, part, splits, plane, (int)H,
+                           token_of_row, row_factor, d_hidden_chunk, H, (const int32_t*)nullptr, 0, 0);
+      }
     }
   }
   if (!dw_f32)

@@ -1200,10 +1200,10 @@ def fused_lm_head_ppo_loss(
     GEMMs run on the other tokens only; the results are those of the dense computation.  ``False`` multiplies the
     zero rows through, as the reference's autograd does.  How many tokens of a chunk take part is counted on the
     device (``count_on_device=True``, the default): the kernels are queued for every token that could and stop at
-    the rows in use, so the host neither needs the mask nor waits for the device.  With ``count_on_device=False`` the
+    the rows in use, so the host neither needs the mask nor waits for the device; the results are, bit for bit, those
+    of the same counts given by the host, in the same time.  With ``count_on_device=False`` the
     host reads the per-chunk counts back (one small device-to-host copy that waits for the mask only) and sizes the
-    GEMMs exactly, which pays when few tokens of a chunk have a mask (the ``d_hidden`` product can then be cut along
-    the vocabulary to fill the chip).  A caller that already knows the counts on the host (the number of tokens with a
+    GEMMs itself.  A caller that already knows the counts on the host (the number of tokens with a
     non-zero effective mask in each chunk of ``aa_lmhead_chunk_tokens()`` tokens, e.g. from the CPU copy of
     ``loss_mask`` when there is no rejection sampling) can pass them as ``kept_per_chunk``; nothing is read back then
     either.  A count that is too small drops the tokens beyond it from the gradient; a count that is too large (e.g.

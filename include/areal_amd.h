@@ -791,9 +791,10 @@ int aa_lmhead_bwd_carry(const void* hidden, const void* weight, int64_t T,
  * aa_lmhead_ppo_fused): the kernels of that chunk are launched for every token
  * that could have a row and stop at the rows in use, which the device counts
  * itself, so the host needs no copy of the mask and does not wait for the
- * device.  The price: workgroups that find nothing to do still start, and the
- * d_hidden product is never cut along the vocabulary (which a host count well
- * below a chunk can make worthwhile). */
+ * device.  The tiles over the rows in use are numbered, and the d_hidden
+ * product is cut along the vocabulary or not, exactly as with that count given
+ * by the host: the results are the same bits, and the workgroups that find
+ * nothing to do return at once (no measurable cost). */
 #define AA_LMHEAD_COUNT_ON_DEVICE (-1)
 
 /* How aa_lmhead_ppo_fused fills the d(logits) rows that its backward GEMMs

@@ -559,28 +559,35 @@ def test_counts_larger_than_the_mask_holds_add_nothing(device, backward):
 
 
 @pytest.mark.parametrize("backward", ["carry", "recompute"])
-@pytest.mark.parametrize("mask_kind", ["mixed", "second_chunk_empty", "nothing", "three_tokens"])
+@pytest.mark.parametrize("mask_kind", ["mixed", "second_chunk_empty", "nothing", "three_tokens",
+                                       "three_tokens_long_rows", "a_tile_and_a_bit_long_rows"])
 def test_rows_counted_on_the_device_match_host_counts(device, backward, mask_kind):
     """The default (``count_on_device=True``: the kernels are queued for every token that could have a row and stop at
     the rows in use, which only the device knows) against counts read back by the host and against counts passed in:
     the same loss, the same d(hidden) bits, the same d(W) up to the order of the sums; chunks with no token, with a
-    handful and with all but a few."""
+    handful and with all but a few.  With rows of 8256 entries and few tokens the d(hidden) product is cut along the
+    vocabulary; the device then makes the choice the host makes from the same count (the same bits again)."""
     T_pad, T = CHUNK + 256, CHUNK + 200
-    hidden, weight, labels, prox, old, adv, mask = _inputs(T_pad, T, 64, 640, seed=47)
+    V = 8256 if mask_kind.endswith("long_rows") else 640
+    hidden, weight, labels, prox, old, adv, mask = _inputs(T_pad, T, 64, V, seed=47)
     if mask_kind == "second_chunk_empty":
         mask[CHUNK:] = False
     elif mask_kind == "nothing":
         mask[:] = False
-    elif mask_kind == "three_tokens":
+    elif mask_kind.startswith("three_tokens"):
         mask[:] = False
         mask[[5, CHUNK - 1, CHUNK + 7]] = True
+    elif mask_kind == "a_tile_and_a_bit_long_rows":
+        mask[:] = False
+        mask[torch.arange(0, CHUNK, 60)] = True          # 274 rows: two tiles
+        mask[CHUNK + 3:CHUNK + 120] = True
     args = [t.to(device) for t in (labels, prox, old, adv)]
     counts = [int(mask[:CHUNK].sum()), int(mask[CHUNK:].sum())]
 
     def run(**kw):
         h = hidden.to(device).requires_grad_(True)
         w = weight.to(device).requires_grad_(True)
-        _poison_the_allocator_cache(device, int(_native.load().aa_lmhead_workspace_bytes(T_pad, 64, 640)))
+        _poison_the_allocator_cache(device, int(_native.load().aa_lmhead_workspace_bytes(T_pad, 64, V)))
         loss, stat = areal_amd.fused_lm_head_ppo_loss(h, w, *args, eps_clip=0.2, loss_mask=mask.to(device),
                                                       backward=backward, **kw)
         loss.backward()
