@@ -43,6 +43,15 @@ __host__ __device__ __forceinline__ int64_t round_up(int64_t x, int64_t m) { ret
 
 enum { kModeStats = 0, kModeStatsCarry = 1, kModeRecompute = 2 };
 
+// ---- the row count of a chunk, when only the device knows it -------------------------------------------------------
+// k_compact_map leaves four words per chunk: how many tokens have a panel row, and what the kernels behind it derive
+// from that number, worked out once instead of by every workgroup: the tiles of BN rows that cover them, the count
+// rounded up to a whole K slice (at least one: the main loop always starts one), and the number of parts the d_hidden
+// product over those rows is cut into (choose_splits).  Kernels that are given these words are queued for the
+// largest count possible and stop at the rows in use.
+enum { kRowsTotal = 0, kRowsLive = 1, kRowsSliced = 2, kRowsSplits = 3 };
+enum { kBoundNone = 0, kBoundN = 1, kBoundK = 2 };
+
 struct TileArgs {
   // statistics per (128-row vocabulary block, token): planes [blocks][pitch_t]
   float* pk;
@@ -66,7 +75,8 @@ struct TileArgs {
   const float* g_entropy;  // nullable
   float inv_t;
   const int32_t* run_if;   // recompute tiles only: when given, the kernel does nothing unless *run_if != 0
-  const int32_t* n_bound;  // recompute tiles only: when given, only the tiles over the first *n_bound token columns run
+  const int32_t* n_bound;  // recompute tiles only: when given, the row-count words of the chunk (kRowsLive is used):
+                           // only the tiles over the token columns in use run
 };
 
 // Carry mode stores 2^(x c - kref) with kref = c * (label logit of the token): a reference that is known before the
@@ -178,7 +188,7 @@ __global__ __launch_bounds__(kThreads) void k_lmhead_tiles(Operand W, Operand Hd
     // token columns in use, known to the device alone: the tiles that cover them are numbered as if the host had
     // launched exactly those (the same walk over the XCDs), the workgroups beyond them return
     if (a.n_bound) {
-      const int live = (*a.n_bound + BN - 1) / BN;
+      const int live = a.n_bound[kRowsLive];
       tiles_n = live < tiles_n ? live : tiles_n;
       if ((int)blockIdx.x >= tiles_m * tiles_n) return;  // the same decision in every thread of the workgroup
     }
@@ -498,8 +508,8 @@ __global__ __launch_bounds__(256) void k_carry_factors(const float* __restrict__
 // Into how many parts along K a product of `tiles` tiles and `slices` K slices is cut (1: not at all): the number of
 // parts, up to kMaxSplits, that shortens the time in rounds of tiles, ceil(tiles * parts / units) / parts, the most,
 // with 0.03 rounds charged per part for writing and adding its fp32 plane; at least 5 % have to be won, and a part
-// keeps at least 64 slices.  In whole numbers (rounds x 1200) so that the host and every workgroup of the kernels that
-// choose for themselves, from a row count that only the device holds, come to the same answer.
+// keeps at least 64 slices.  In whole numbers (rounds x 1200) so that the host and the device (k_compact_map, from a
+// row count that only the device holds) come to the same answer.
 constexpr int kMaxSplits = 4;
 constexpr int kRoundsUnit = 1200;  // divisible by every number of parts
 static_assert(kRoundsUnit % 2 == 0 && kRoundsUnit % 3 == 0 && kRoundsUnit % 4 == 0 && kMaxSplits <= 4, "rounds in whole numbers");
@@ -523,30 +533,30 @@ __host__ __device__ inline int choose_splits(int64_t tiles, int64_t slices, int 
 // neighbouring outputs of a row of C.  bf16 C: the tile is staged in LDS as [n][m] and leaves in 16-byte pieces,
 // 512 contiguous bytes per row; row n of the product is written to row c_rows[n] of C when a row list is given.
 // fp32 C: 16-byte stores straight from the registers; ACCUM adds to what C holds.
-template <bool AKM, bool BKM, typename OutT, bool ACCUM>
-// n_bound / k_bound, when given, hold a count that only the device knows (the number of panel rows in use, at most
-// the N or K the host launched with): only the tiles over the first *n_bound rows of B run (numbered as a grid of just
-// those tiles; the other workgroups return at once), and the contraction stops at *k_bound rounded up to a whole K
-// slice (the rows up to there are zero).  With n_bound and split_units > 0 the whole grid returns when the product over
-// *n_bound rows is one that k_gemm_splitk, queued beside it, cuts along K on split_units compute units.
+// BOUND: `bounds` holds the row-count words of the chunk (the number of panel rows in use is known to the device alone
+// and is at most the N or K the host launched with).  kBoundN: only the tiles over the rows of B in use run, numbered
+// as a grid of just those tiles (the walk over the XCDs is the one a grid sized by the host has; the other workgroups
+// return at once), and the whole grid returns when the product over those rows is one that k_gemm_splitk, queued
+// beside it, cuts along K.  kBoundK: the contraction stops at the count rounded up to a whole K slice (the rows up to
+// there are zero).  kBoundNone is the kernel without any of this.
+template <bool AKM, bool BKM, typename OutT, bool ACCUM, int BOUND>
 __global__ __launch_bounds__(kThreads) void k_gemm_store(Operand A, Operand B, int K, int tiles_m, int tiles_n,
                                                          OutT* __restrict__ C, int64_t ldc,
                                                          const int32_t* __restrict__ c_rows,
                                                          const float* __restrict__ n_scale,
-                                                         const int32_t* __restrict__ n_bound,
-                                                         const int32_t* __restrict__ k_bound, int split_units) {
+                                                         const int32_t* __restrict__ bounds) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  if (n_bound) {  // the tiles over the rows in use are numbered as if the host had launched exactly those
-    const int live = (*n_bound + BN - 1) / BN;
+  if constexpr (BOUND == kBoundN) {
+    const int live = bounds[kRowsLive];
     tiles_n = live < tiles_n ? live : tiles_n;
-    if ((int)blockIdx.x >= tiles_m * tiles_n) return;  // the same decision in every thread of the workgroup
-    if (split_units > 0 && choose_splits((int64_t)tiles_m * tiles_n, (K + BK - 1) / BK, split_units) != 1) return;
+    // the same decision in every thread of the workgroup
+    if (bounds[kRowsSplits] != 1 || (int)blockIdx.x >= tiles_m * tiles_n) return;
   }
   int tm, tn;
   tile_of(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
-  if (k_bound) {  // at least one slice: the main loop always starts one
-    const int kb = *k_bound > 0 ? (*k_bound + BK - 1) / BK * BK : BK;
+  if constexpr (BOUND == kBoundK) {
+    const int kb = bounds[kRowsSliced];
     K = kb < K ? kb : K;
   }
   Acc acc;
@@ -617,18 +627,18 @@ __global__ __launch_bounds__(kThreads) void k_gemm_store(Operand A, Operand B, i
 // the K slices [s * per, (s + 1) * per) into its own fp32 plane; k_splitk_rows adds the planes in order.  Workgroups
 // are numbered so that an XCD runs a contiguous range of (part, tile): the tiles that share operand slices in its L2
 // are those of one part.
-// With n_bound (the rows of B in use, known to the device alone; `splits` then holds the number of compute units) the
-// kernel numbers the tiles over those rows and chooses the number of parts itself, as the host would have with that
-// count; the workgroups beyond tiles x parts return at once, all of them when the product is not cut.
-template <bool AKM, bool BKM>
+// BOUNDED (the rows of B in use are known to the device alone; `bounds`: the row-count words of the chunk): the tiles
+// over those rows are numbered as a grid of just those, cut into the number of parts that the host would have chosen
+// with that count; the workgroups beyond tiles x parts return at once, all of them when the product is not cut.
+template <bool AKM, bool BKM, bool BOUNDED>
 __global__ __launch_bounds__(kThreads) void k_gemm_splitk(Operand A, Operand B, int K, int tiles_m, int tiles_n, int splits,
                                                           float* __restrict__ part, int64_t ldc, int64_t plane,
-                                                          const int32_t* __restrict__ n_bound) {
+                                                          const int32_t* __restrict__ bounds) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  if (n_bound) {
-    const int live = (*n_bound + BN - 1) / BN;
+  if constexpr (BOUNDED) {
+    const int live = bounds[kRowsLive];
     tiles_n = live < tiles_n ? live : tiles_n;
-    splits = choose_splits((int64_t)tiles_m * tiles_n, (K + BK - 1) / BK, splits);
+    splits = bounds[kRowsSplits];
     if (splits == 1 || (int)blockIdx.x >= tiles_m * tiles_n * splits) return;  // the same in every thread
   }
   const int tiles = tiles_m * tiles_n;
@@ -669,18 +679,16 @@ __global__ __launch_bounds__(kThreads) void k_gemm_splitk(Operand A, Operand B, 
 
 // out[c_rows[r], :] = bf16(n_scale[r] * (plane 0 + plane 1 + ...)[r, :]), the planes added in order; M % 8 == 0.
 // c_rows == nullptr: row r itself (a negative entry: the row is dropped); n_scale == nullptr: 1.
-// With n_bound (see k_gemm_splitk; `splits` then holds the number of compute units, tiles_m and slices describe the
-// product) only the rows below *n_bound are written, from the number of planes that kernel chose; none when it did not
-// cut the product.
+// With `bounds` (the row-count words of the chunk, see k_gemm_splitk) only the rows in use are written, from the number
+// of planes that kernel was cut into; none when it was not cut.
 __global__ __launch_bounds__(256) void k_splitk_rows(const float* __restrict__ part, int splits, int64_t plane, int M,
                                                      const int32_t* __restrict__ c_rows, const float* __restrict__ n_scale,
                                                      uint16_t* __restrict__ out, int64_t ldo,
-                                                     const int32_t* __restrict__ n_bound, int tiles_m, int slices) {
+                                                     const int32_t* __restrict__ bounds) {
   const int64_t r = blockIdx.x;
-  if (n_bound) {
-    if (r >= *n_bound) return;
-    splits = choose_splits((int64_t)tiles_m * ((*n_bound + BN - 1) / BN), slices, splits);
-    if (splits == 1) return;
+  if (bounds) {
+    splits = bounds[kRowsSplits];
+    if (splits == 1 || r >= bounds[kRowsTotal]) return;
   }
   const int64_t dst = c_rows ? c_rows[r] : r;
   if (dst < 0) return;
@@ -710,12 +718,14 @@ __global__ __launch_bounds__(256) void k_splitk_rows(const float* __restrict__ p
 // token t among them, or -1; act_rows[position] = t.  `limit` is the count the host sized the GEMMs with; tokens
 // beyond it are dropped.  A host count larger than what the mask holds leaves positions without a token: they get
 // act_rows = -1 (the gathers then produce zero rows and the scatters skip them) and a row factor of zero when factors
-// are in use; the true count goes to *total_out, and k_clear_surplus_rows, launched behind this kernel, clears their
+// are in use; the true count goes to total_out (the four row-count words of the chunk; dh_tiles_m, dh_slices and units
+// describe the d_hidden product for choose_splits), and k_clear_surplus_rows, launched behind this kernel, clears their
 // panel rows, which no tile writes, so that nothing stale (possibly not even finite) enters the d_weight product.
 // One workgroup; mask has `act` entries (tokens at and after `act` have none).
 __global__ __launch_bounds__(1024) void k_compact_map(const uint8_t* __restrict__ mask, int act, int n_tok, int limit,
                                                       int32_t* __restrict__ out_rows, int32_t* __restrict__ act_rows,
-                                                      float* __restrict__ row_factor, int32_t* __restrict__ total_out) {
+                                                      float* __restrict__ row_factor, int32_t* __restrict__ total_out,
+                                                      int dh_tiles_m, int dh_slices, int units) {
   __shared__ int wave_sum[16];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int per = (n_tok + 1023) / 1024;
@@ -741,7 +751,14 @@ __global__ __launch_bounds__(1024) void k_compact_map(const uint8_t* __restrict_
   }
   int total = 0;
   for (int w = 0; w < 16; ++w) total += wave_sum[w];
-  if (tid == 0) *total_out = total < limit ? total : limit;
+  if (tid == 0) {
+    const int rows = total < limit ? total : limit;
+    const int live = (rows + BN - 1) / BN;
+    total_out[kRowsTotal] = rows;
+    total_out[kRowsLive] = live;
+    total_out[kRowsSliced] = rows > 0 ? (rows + BK - 1) / BK * BK : BK;
+    total_out[kRowsSplits] = choose_splits((int64_t)dh_tiles_m * live, dh_slices, units);
+  }
   for (int p = total + tid; p < limit; p += 1024) {  // the usual case: none
     act_rows[p] = -1;
     if (row_factor) row_factor[p] = 0.f;
@@ -757,19 +774,22 @@ __global__ __launch_bounds__(256) void k_clear_surplus_rows(const int32_t* __res
   const u32x4_t zero = {0u, 0u, 0u, 0u};
   const int64_t vec = panel_ld / 8;
   if (bounded) {
-    const int up = *total > 0 ? (*total + BK - 1) / BK * BK : BK;
+    const int up = total[kRowsSliced];
     limit = up < limit ? up : limit;
   }
   for (int64_t r = (int64_t)*total + blockIdx.x; r < limit; r += gridDim.x)
     for (int64_t i = threadIdx.x; i < vec; i += 256) panel[r * vec + i] = zero;
 }
 
-// numbering of the tokens with a panel row, and the rows without a token cleared (both kernels)
+static int compute_units();
+
+// numbering of the tokens with a panel row, and the rows without a token cleared (both kernels); H and V are those of
+// the lm_head (they shape the d_hidden product that the row-count words describe)
 static void launch_compact_map(hipStream_t st, const uint8_t* mask, int64_t act, int64_t n_tok, int64_t limit,
                                int32_t* out_rows, int32_t* act_rows, float* row_factor, int32_t* total_word,
-                               uint16_t* panel, int64_t panel_ld, bool bounded = false) {
+                               uint16_t* panel, int64_t panel_ld, int64_t H, int64_t V, bool bounded = false) {
   hipLaunchKernelGGL(k_compact_map, dim3(1), dim3(1024), 0, st, mask, (int)act, (int)n_tok, (int)limit, out_rows, act_rows,
-                     row_factor, total_word);
+                     row_factor, total_word, (int)((H + BM - 1) / BM), (int)((V + BK - 1) / BK), compute_units());
   const int64_t blocks = bounded ? (limit < BK ? limit : BK) : (limit < 512 ? limit : 512);
   if (blocks > 0)
     hipLaunchKernelGGL(k_clear_surplus_rows, dim3((unsigned)blocks), dim3(256), 0, st, total_word, (int)limit,
@@ -900,10 +920,16 @@ static bool prepare_kernels() {
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return false;
   if (done[dev]) return true;
   const bool ok = allow_big_lds(k_lmhead_tiles<kModeStats>) && allow_big_lds(k_lmhead_tiles<kModeStatsCarry>) &&
-                  allow_big_lds(k_lmhead_tiles<kModeRecompute>) && allow_big_lds(k_gemm_store<true, false, uint16_t, false>) &&
-                  allow_big_lds(k_gemm_store<true, true, uint16_t, false>) &&
-                  allow_big_lds(k_gemm_store<true, true, float, false>) && allow_big_lds(k_gemm_store<true, true, float, true>) &&
-                  allow_big_lds(k_gemm_splitk<true, false>);
+                  allow_big_lds(k_lmhead_tiles<kModeRecompute>) &&
+                  allow_big_lds(k_gemm_store<true, false, uint16_t, false, kBoundNone>) &&
+                  allow_big_lds(k_gemm_store<true, false, uint16_t, false, kBoundN>) &&
+                  allow_big_lds(k_gemm_store<true, true, uint16_t, false, kBoundNone>) &&
+                  allow_big_lds(k_gemm_store<true, true, uint16_t, false, kBoundK>) &&
+                  allow_big_lds(k_gemm_store<true, true, float, false, kBoundNone>) &&
+                  allow_big_lds(k_gemm_store<true, true, float, false, kBoundK>) &&
+                  allow_big_lds(k_gemm_store<true, true, float, true, kBoundNone>) &&
+                  allow_big_lds(k_gemm_store<true, true, float, true, kBoundK>) &&
+                  allow_big_lds(k_gemm_splitk<true, false, false>) && allow_big_lds(k_gemm_splitk<true, false, true>);
   done[dev] = ok;
   return ok;
 }
@@ -932,16 +958,31 @@ static void launch_tiles(hipStream_t st, const void* weight, const uint16_t* hid
                      W, Hd, (int)H, tiles_m, tiles_n, a);
 }
 
-// C [N, M] = B . A^T over K (rows of C through c_rows when given); lda / ldb: leading dimensions of the arrays as stored
-template <bool AKM, bool BKM, typename OutT, bool ACCUM>
+// C [N, M] = B . A^T over K (rows of C through c_rows when given); lda / ldb: leading dimensions of the arrays as stored.
+// BOUND / bounds: see k_gemm_store.
+template <bool AKM, bool BKM, typename OutT, bool ACCUM, int BOUND = kBoundNone>
 static void launch_gemm(hipStream_t st, const uint16_t* A, int64_t lda, int64_t M, const uint16_t* B, int64_t ldb, int64_t N,
                         int64_t K, OutT* C, int64_t ldc, const int32_t* c_rows = nullptr,
-                        const float* n_scale = nullptr, const int32_t* n_bound = nullptr,
-                        const int32_t* k_bound = nullptr, int split_units = 0) {
+                        const float* n_scale = nullptr, const int32_t* bounds = nullptr) {
   const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
   Operand a{A, lda, (int)M}, b{B, ldb, (int)N};
-  hipLaunchKernelGGL((k_gemm_store<AKM, BKM, OutT, ACCUM>), dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads), kLdsBytes, st,
-                     a, b, (int)K, tiles_m, tiles_n, C, ldc, c_rows, n_scale, n_bound, k_bound, split_units);
+  hipLaunchKernelGGL((k_gemm_store<AKM, BKM, OutT, ACCUM, BOUND>), dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads),
+                     kLdsBytes, st, a, b, (int)K, tiles_m, tiles_n, C, ldc, c_rows, n_scale, bounds);
+}
+
+// d_weight (+)= ds^T . hidden rows in the dtype and mode asked for; with `bounds` the contraction stops at the rows in use
+template <int BOUND>
+static void launch_d_weight(hipStream_t st, const uint16_t* hid_rows, int64_t H, const uint16_t* ds, int64_t ldp, int64_t V,
+                            int64_t n_rows, void* d_weight, bool dw_f32, bool first, const int32_t* bounds) {
+  if (!dw_f32)
+    launch_gemm<true, true, uint16_t, false, BOUND>(st, hid_rows, H, H, ds, ldp, V, n_rows, (uint16_t*)d_weight, H, nullptr,
+                                                    nullptr, bounds);
+  else if (first)
+    launch_gemm<true, true, float, false, BOUND>(st, hid_rows, H, H, ds, ldp, V, n_rows, (float*)d_weight, H, nullptr,
+                                                 nullptr, bounds);
+  else
+    launch_gemm<true, true, float, true, BOUND>(st, hid_rows, H, H, ds, ldp, V, n_rows, (float*)d_weight, H, nullptr, nullptr,
+                                                bounds);
 }
 
 // The two GEMMs that contract the d(logits) rows ds [n_rows, V] of one token chunk, ds = row_factor[r] * panel[r, :]
@@ -973,21 +1014,23 @@ static void panel_gradients(hipStream_t st, const Workspace& w, char* ws, const 
     const int64_t plane = n_rows * H;
     Operand a{(const uint16_t*)weight, H, (int)H}, b{ds, ldp, (int)n_rows};
     if (rows_in_use) {
-      // the row count is on the device alone (n_rows is its upper bound): both forms of the product are queued, each
-      // kernel works out from the count whether the product is cut along the vocabulary and into how many parts (what
-      // the host would have chosen with that count), and the form that is not in turn returns at once
-      int64_t cut_groups = 0;  // the largest grid the cut product can ask for
+      // the row count is on the device alone (n_rows is its upper bound): both forms of the product are queued, the
+      // row-count words say whether the product is cut along the vocabulary and into how many parts (what the host
+      // would have chosen with that count), and the form that is not in turn returns at once
+      int64_t cut_groups = 0, cut_rows = 0;  // the largest grid, and the most rows, the cut product can come with
       for (int tn = 1; tn <= tiles_n; ++tn) {
         const int parts = choose_splits((int64_t)tiles_m * tn, slices, units);
-        if (parts > 1 && (int64_t)tiles_m * tn * parts > cut_groups) cut_groups = (int64_t)tiles_m * tn * parts;
+        if (parts == 1) continue;
+        if ((int64_t)tiles_m * tn * parts > cut_groups) cut_groups = (int64_t)tiles_m * tn * parts;
+        cut_rows = (int64_t)tn * BN < n_rows ? (int64_t)tn * BN : n_rows;
       }
-      launch_gemm<true, false, uint16_t, false>(st, (const uint16_t*)weight, H, H, ds, ldp, n_rows, V, d_hidden_chunk, H,
-                                                token_of_row, row_factor, rows_in_use, nullptr, cut_groups ? units : 0);
+      launch_gemm<true, false, uint16_t, false, kBoundN>(st, (const uint16_t*)weight, H, H, ds, ldp, n_rows, V,
+                                                         d_hidden_chunk, H, token_of_row, row_factor, rows_in_use);
       if (cut_groups) {
-        hipLaunchKernelGGL((k_gemm_splitk<true, false>), dim3((unsigned)cut_groups), dim3(kThreads), kLdsBytes, st, a, b,
-                           (int)V, tiles_m, tiles_n, units, part, H, plane, rows_in_use);
-        hipLaunchKernelGGL(k_splitk_rows, dim3((unsigned)n_rows), dim3(256), 0, st, part, units, plane, (int)H, token_of_row,
-                           row_factor, d_hidden_chunk, H, rows_in_use, tiles_m, (int)slices);
+        hipLaunchKernelGGL((k_gemm_splitk<true, false, true>), dim3((unsigned)cut_groups), dim3(kThreads), kLdsBytes, st, a,
+                           b, (int)V, tiles_m, tiles_n, 0, part, H, plane, rows_in_use);
+        hipLaunchKernelGGL(k_splitk_rows, dim3((unsigned)cut_rows), dim3(256), 0, st, part, 0, plane, (int)H, token_of_row,
+                           row_factor, d_hidden_chunk, H, rows_in_use);
       }
     } else {
       const int splits = choose_splits((int64_t)tiles_m * tiles_n, slices, units);
@@ -995,22 +1038,17 @@ static void panel_gradients(hipStream_t st, const Workspace& w, char* ws, const 
         launch_gemm<true, false, uint16_t, false>(st, (const uint16_t*)weight, H, H, ds, ldp, n_rows, V, d_hidden_chunk, H,
                                                   token_of_row, row_factor);
       } else {
-        hipLaunchKernelGGL((k_gemm_splitk<true, false>), dim3((unsigned)(tiles_m * tiles_n * splits)), dim3(kThreads),
+        hipLaunchKernelGGL((k_gemm_splitk<true, false, false>), dim3((unsigned)(tiles_m * tiles_n * splits)), dim3(kThreads),
                            kLdsBytes, st, a, b, (int)V, tiles_m, tiles_n, splits, part, H, plane, (const int32_t*)nullptr);
         hipLaunchKernelGGL(k_splitk_rows, dim3((unsigned)n_rows), dim3(256), 0, st, part, splits, plane, (int)H,
-                           token_of_row, row_factor, d_hidden_chunk, H, (const int32_t*)nullptr, 0, 0);
+                           token_of_row, row_factor, d_hidden_chunk, H, (const int32_t*)nullptr);
       }
     }
   }
-  if (!dw_f32)
-    launch_gemm<true, true, uint16_t, false>(st, hid_rows, H, H, ds, ldp, V, n_rows, (uint16_t*)d_weight, H, nullptr, nullptr,
-                                             nullptr, rows_in_use);
-  else if (first)
-    launch_gemm<true, true, float, false>(st, hid_rows, H, H, ds, ldp, V, n_rows, (float*)d_weight, H, nullptr, nullptr,
-                                          nullptr, rows_in_use);
+  if (rows_in_use)
+    launch_d_weight<kBoundK>(st, hid_rows, H, ds, ldp, V, n_rows, d_weight, dw_f32, first, rows_in_use);
   else
-    launch_gemm<true, true, float, true>(st, hid_rows, H, H, ds, ldp, V, n_rows, (float*)d_weight, H, nullptr, nullptr,
-                                         nullptr, rows_in_use);
+    launch_d_weight<kBoundNone>(st, hid_rows, H, ds, ldp, V, n_rows, d_weight, dw_f32, first, nullptr);
 }
 
 // Recompute: d(logits) of the panel rows from the logits tiles formed again.  With a row map only the hidden rows that
@@ -1250,7 +1288,7 @@ extern "C" int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, 
     int32_t* total_word = (int32_t*)(ws + w.off_total);
     const int32_t* rows_in_use = on_device ? total_word : nullptr;
     launch_compact_map(st, row_has_gradient + t0, n_tok, n_tok, kept, out_rows, act_rows, nullptr, total_word, ws_panel,
-                       w.panel_ld, on_device);
+                       w.panel_ld, H, V, on_device);
     recompute_panel(st, w, ws, ws_panel, weight, hid, n_tok, act_rows, kept, H, V, a, nullptr, rows_in_use);
     launch_zero(st, dh, n_tok * H * 2);  // the rows of the other tokens
     panel_gradients(st, w, ws, ws_panel, weight, hid, act_rows, nullptr, kept, H, V, dh, dw.acc, dw.acc_f32, first,
@@ -1311,7 +1349,7 @@ extern "C" int aa_lmhead_fwd_carry(const void* hidden, const void* weight, int64
       rows = kept_per_chunk[chunk_index];
       rows = rows < 0 ? 0 : (rows > n_tok ? n_tok : rows);
       launch_compact_map(st, row_has_gradient + t0, n_tok, n_tok, rows, out_rows, act_rows, nullptr,
-                         (int32_t*)(ws + w.off_total), chunk_panel, w.panel_ld);
+                         (int32_t*)(ws + w.off_total), chunk_panel, w.panel_ld, H, V);
     }
     TileArgs a = stats_args(w, ws, labels + t0, inv_temperature, vocab_min != nullptr);
     a.panel = chunk_panel;
@@ -1374,7 +1412,7 @@ extern "C" int aa_lmhead_bwd_carry(const void* hidden, const void* weight, int64
       }
       // the same numbering as in the forward (the mask has not changed); surplus rows get a factor of zero
       launch_compact_map(st, row_has_gradient + t0, n_tok, n_tok, rows, out_rows, act_rows, row_factor,
-                         (int32_t*)(ws + w.off_total), chunk_panel, w.panel_ld);
+                         (int32_t*)(ws + w.off_total), chunk_panel, w.panel_ld, H, V);
       row_of_token = out_rows;
       token_of_row = act_rows;
     }
@@ -1462,7 +1500,7 @@ extern "C" int aa_lmhead_ppo_fused(const void* hidden, const void* weight, int64
       rows = on_device ? act : (rows < 0 ? 0 : (rows > act ? act : rows));
       int32_t* total_word = (int32_t*)(ws + w.off_total);
       launch_compact_map(st, at(mask_eff), act, n_tok, rows, out_rows, act_rows, carry ? row_factor : nullptr, total_word,
-                         panel, w.panel_ld, on_device);
+                         panel, w.panel_ld, H, V, on_device);
       if (on_device) rows_in_use = total_word;
       row_of_token = out_rows;
       token_of_row = act_rows;
