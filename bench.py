@@ -494,9 +494,9 @@ MODE_NAMES = {1: "carry", 0: "recompute"}
 # known size.  The counters sit behind the L2 of each XCD: what the memory-side cache serves is in these figures too.
 # Transcribed from the profile summaries named beside them, not read in this run; other workloads: not measured.
 LMHEAD_MEASURED_HBM_BYTES = {
-    ("cfg2", "carry"): (82.7e9, "profiles/lmhead_step_cfg2_hbm_traffic.md"),
-    ("cfg2", "recompute"): (111.3e9, "profiles/lmhead_step_cfg2_hbm_traffic.md"),
-    ("cfg4", "carry"): (511.9e9, "profiles/lmhead_step_cfg4_hbm_traffic.md"),
+    ("cfg2", "carry"): (81.3e9, "profiles/lmhead_step_cfg2_hbm_traffic.md"),
+    ("cfg2", "recompute"): (109.0e9, "profiles/lmhead_step_cfg2_hbm_traffic.md"),
+    ("cfg4", "carry"): (512.3e9, "profiles/lmhead_step_cfg4_hbm_traffic.md"),
 }
 
 
