@@ -756,24 +756,31 @@ def test_labels_outside_the_vocabulary_at_masked_tokens(device, backward, skip):
     assert float(h.grad.cpu()[bad].abs().sum()) == 0.0
 
 
+@pytest.mark.parametrize("skip_masked_tokens", [False, True])
 @pytest.mark.parametrize("backward", ["carry", "recompute"])
-def test_step_replays_from_a_hip_graph(device, backward):
+def test_step_replays_from_a_hip_graph(device, backward, skip_masked_tokens):
     """aa_lmhead_ppo_fused allocates nothing, clears memory with kernels only and never waits for the device, so the
-    whole step (every token's row in the gradient products: no count has to reach the host) can be captured into a HIP
-    graph.  Three replays on new inputs, with eager work and synchronisations in between, each equal to the eager
-    result on the same inputs."""
-    T, H, V = 600, 128, 1088
+    whole step can be captured into a HIP graph: with every token's row in the gradient products, or with the tokens
+    without a mask left out (the rows in use are counted on the device, so the graph holds for any mask: the replays
+    below come with masks of 70 %, 10 %, none and all of the tokens; the vocabulary is long enough for the d(hidden)
+    product to be cut along it when few rows are in use).  Four replays on new inputs, with eager work and
+    synchronisations in between, each equal to the eager result on the same inputs."""
+    T, H, V = 600, 128, 8256 if skip_masked_tokens else 1088
     g = torch.Generator().manual_seed(3)
     h = torch.zeros(T, H, dtype=torch.bfloat16, device=device, requires_grad=True)
     w = torch.zeros(V, H, dtype=torch.bfloat16, device=device, requires_grad=True)
     labels = torch.randint(0, V, (T,), generator=g).to(device)
     prox, old, adv = (torch.zeros(T, device=device) for _ in range(3))
     mask = (torch.rand(T, generator=g) < 0.7).to(device)
-    kw = dict(eps_clip=0.2, loss_mask=mask, eps_clip_higher=0.28, backward=backward, skip_masked_tokens=False)
+    kw = dict(eps_clip=0.2, loss_mask=mask, eps_clip_higher=0.28, backward=backward,
+              skip_masked_tokens=skip_masked_tokens)
+    density = {0: 0.7, 1: 0.7, 2: 0.1, 3: 0.0, 4: 1.0}
 
     def fill(seed):
         gg = torch.Generator().manual_seed(seed)
         with torch.no_grad():
+            if skip_masked_tokens:
+                mask.copy_((torch.rand(T, generator=gg) < density[seed]).to(device))
             h.copy_(torch.randn(T, H, generator=gg).bfloat16())
             w.copy_((0.3 * torch.randn(V, H, generator=gg)).bfloat16())
             ref, _ = areal_amd.lm_head_logprobs_entropy(h, w, labels)
@@ -799,7 +806,7 @@ def test_step_replays_from_a_hip_graph(device, backward):
     with torch.cuda.graph(graph):
         g_loss, g_logp = step()
     g_dh, g_dw = h.grad, w.grad
-    for seed in (1, 2, 3):
+    for seed in (1, 2, 3, 4):
         fill(seed)
         graph.replay()
         torch.cuda.synchronize()
