@@ -1313,6 +1313,7 @@ static int64_t panel_rows_before(const int64_t* kept_per_chunk, int64_t chunk, i
   for (int64_t c = 0; c < upto; ++c) {
     const int64_t n_tok = (T - c * chunk) < chunk ? (T - c * chunk) : chunk;
     int64_t k = kept_per_chunk ? kept_per_chunk[c] : n_tok;
+    if (k == AA_LMHEAD_COUNT_ON_DEVICE) k = n_tok;  // the count is on the device alone: room for every token
     rows += k < 0 ? 0 : (k > n_tok ? n_tok : k);
   }
   return rows;
@@ -1347,9 +1348,10 @@ extern "C" int aa_lmhead_fwd_carry(const void* hidden, const void* weight, int64
     int64_t rows = n_tok;
     if (kept_per_chunk) {
       rows = kept_per_chunk[chunk_index];
-      rows = rows < 0 ? 0 : (rows > n_tok ? n_tok : rows);
+      const bool on_device = rows == AA_LMHEAD_COUNT_ON_DEVICE;  // the chunk keeps room for every token
+      rows = on_device ? n_tok : (rows < 0 ? 0 : (rows > n_tok ? n_tok : rows));
       launch_compact_map(st, row_has_gradient + t0, n_tok, n_tok, rows, out_rows, act_rows, nullptr,
-                         (int32_t*)(ws + w.off_total), chunk_panel, w.panel_ld, H, V);
+                         (int32_t*)(ws + w.off_total), chunk_panel, w.panel_ld, H, V, on_device);
     }
     TileArgs a = stats_args(w, ws, labels + t0, inv_temperature, vocab_min != nullptr);
     a.panel = chunk_panel;
@@ -1403,16 +1405,20 @@ extern "C" int aa_lmhead_bwd_carry(const void* hidden, const void* weight, int64
     int64_t rows = n_tok;
     const int32_t* row_of_token = nullptr;
     const int32_t* token_of_row = nullptr;
+    const int32_t* rows_in_use = nullptr;  // the count of the chunk, when only the device has it
     if (kept_per_chunk) {
       rows = kept_per_chunk[chunk_index];
-      rows = rows < 0 ? 0 : (rows > n_tok ? n_tok : rows);
+      const bool on_device = rows == AA_LMHEAD_COUNT_ON_DEVICE;
+      rows = on_device ? n_tok : (rows < 0 ? 0 : (rows > n_tok ? n_tok : rows));
       if (rows == 0) {
         launch_zero(st, dh, n_tok * H * 2);
         continue;
       }
       // the same numbering as in the forward (the mask has not changed); surplus rows get a factor of zero
-      launch_compact_map(st, row_has_gradient + t0, n_tok, n_tok, rows, out_rows, act_rows, row_factor,
-                         (int32_t*)(ws + w.off_total), chunk_panel, w.panel_ld, H, V);
+      int32_t* total_word = (int32_t*)(ws + w.off_total);
+      launch_compact_map(st, row_has_gradient + t0, n_tok, n_tok, rows, out_rows, act_rows, row_factor, total_word,
+                         chunk_panel, w.panel_ld, H, V, on_device);
+      if (on_device) rows_in_use = total_word;
       row_of_token = out_rows;
       token_of_row = act_rows;
     }
@@ -1428,10 +1434,11 @@ extern "C" int aa_lmhead_bwd_carry(const void* hidden, const void* weight, int64
     a.row_lse = row_lse + t0;
     a.g_logp = g_logp + t0;
     a.panel_ld = w.panel_ld;
-    recompute_panel(st, w, ws, chunk_panel, weight, hid, n_tok, token_of_row, rows, H, V, a, redo_flag);
+    recompute_panel(st, w, ws, chunk_panel, weight, hid, n_tok, token_of_row, rows, H, V, a, redo_flag, rows_in_use);
     hipLaunchKernelGGL(k_unit_factors, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, row_factor, (int)rows, redo_flag);
     if (token_of_row) launch_zero(st, dh, n_tok * H * 2);  // the rows of the tokens without a panel row
-    panel_gradients(st, w, ws, chunk_panel, weight, hid, token_of_row, row_factor, rows, H, V, dh, dw.acc, dw.acc_f32, first);
+    panel_gradients(st, w, ws, chunk_panel, weight, hid, token_of_row, row_factor, rows, H, V, dh, dw.acc, dw.acc_f32, first,
+                    rows_in_use);
     first = false;
     row0 += rows;
   }

@@ -878,7 +878,12 @@ class _LmHeadCarry(torch.autograd.Function):
         vmax = torch.empty(T, **f32) if want_minmax else None
         vmin = torch.empty(T, **f32) if want_minmax else None
         kept = None if kept_per_chunk is None else (C.c_int64 * len(kept_per_chunk))(*kept_per_chunk)
-        rows = T if kept_per_chunk is None else sum(kept_per_chunk)
+        if kept_per_chunk is None:
+            rows = T
+        else:  # a chunk whose count stays on the device keeps room for every one of its tokens
+            chunk = lm_head_chunk_tokens()
+            rows = sum(min(chunk, T - i * chunk) if k == N.AA_LMHEAD_COUNT_ON_DEVICE else k
+                       for i, k in enumerate(kept_per_chunk))
         panel = torch.empty(max(rows, 1), int(lib.aa_lmhead_panel_pitch(V)), dtype=torch.bfloat16, device=dev)
         n = lib.aa_lmhead_carry_workspace_bytes(T, H, V)
         if n < 0:
@@ -940,7 +945,7 @@ class _LmHeadCarry(torch.autograd.Function):
 def lm_head_logprobs_entropy(
     hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0,
     token_mask: torch.Tensor | None = None, backward: str = "recompute", grad_token_mask: torch.Tensor | None = None,
-    kept_per_chunk: list[int] | None = None,
+    kept_per_chunk: list[int] | None = None, count_on_device: bool = False,
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """``gather_logprobs_entropy(hidden @ weight.T, labels, temperature)`` without writing the ``[T, V]`` logits.
     Any vocabulary size; the hidden size has to be a multiple of 8.
@@ -970,18 +975,21 @@ def lm_head_logprobs_entropy(
     passes: 2 bytes x V per such token.  ``grad_token_mask`` (``[T]``, e.g. the loss mask) names those tokens; tokens
     outside it get NO gradient, whatever the loss says; without it every token is kept.  The number of named tokens per
     chunk of ``lm_head_chunk_tokens()`` tokens sizes the stored rows: it is read back from the device unless the caller
-    passes it as ``kept_per_chunk`` (counts that are too large are safe, too small ones drop tokens).  A gradient
+    passes it as ``kept_per_chunk`` (counts that are too large are safe, too small ones drop tokens), or leaves it to
+    the device with ``count_on_device=True``: nothing is read back then and the host does not wait, the stored rows
+    take the room of every token (2 bytes x V x T) whatever the mask holds, and the kernels stop at the rows in use
+    (same results, bit for bit).  A gradient
     with respect to the entropy cannot use the stored rows: such a backward forms the logits again, as ``"recompute"``
     does.  The stored rows serve one backward.
     """
     return _lm_head_impl(hidden, weight, labels, temperature, token_mask, False, backward, grad_token_mask,
-                         kept_per_chunk)[:2]
+                         kept_per_chunk, count_on_device)[:2]
 
 
 def lm_head_logprobs_entropy_stats(
     hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0,
     token_mask: torch.Tensor | None = None, backward: str = "recompute", grad_token_mask: torch.Tensor | None = None,
-    kept_per_chunk: list[int] | None = None,
+    kept_per_chunk: list[int] | None = None, count_on_device: bool = False,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """``(logp, entropy, vocab_min_logits, vocab_max_logits)`` of ``hidden @ weight.T`` from the same tiles.
 
@@ -991,10 +999,11 @@ def lm_head_logprobs_entropy_stats(
     through the softmax exponent, i.e. to one rounding), and carry no gradient.  With ``token_mask`` the tokens left
     out of the lm_head get 0 for both.  The other arguments: see ``lm_head_logprobs_entropy``."""
     return _lm_head_impl(hidden, weight, labels, temperature, token_mask, True, backward, grad_token_mask,
-                         kept_per_chunk)
+                         kept_per_chunk, count_on_device)
 
 
-def _lm_head_apply(hidden, weight, y, temperature, want_minmax, backward, grad_mask, kept_per_chunk):
+def _lm_head_apply(hidden, weight, y, temperature, want_minmax, backward, grad_mask, kept_per_chunk,
+                   count_on_device=False):
     """One of the two autograd functions on a contiguous batch; ``grad_mask``: bool / uint8 ``[T]`` or None."""
     needs_grad = torch.is_grad_enabled() and (hidden.requires_grad or weight.requires_grad)
     if backward != "carry" or not needs_grad:
@@ -1009,6 +1018,8 @@ def _lm_head_apply(hidden, weight, y, temperature, want_minmax, backward, grad_m
             kept = [max(0, min(int(v), chunk)) for v in kept_per_chunk]
             if len(kept) != n_chunks:
                 raise ValueError(f"kept_per_chunk needs one count per chunk of {chunk} tokens")
+        elif count_on_device:
+            kept = [N.AA_LMHEAD_COUNT_ON_DEVICE] * n_chunks
         else:
             on = m8.ne(0)
             if n_chunks * chunk != T:
@@ -1018,7 +1029,7 @@ def _lm_head_apply(hidden, weight, y, temperature, want_minmax, backward, grad_m
 
 
 def _lm_head_impl(hidden, weight, labels, temperature, token_mask, want_minmax, backward="recompute",
-                  grad_token_mask=None, kept_per_chunk=None):
+                  grad_token_mask=None, kept_per_chunk=None, count_on_device=False):
     if backward not in _LMHEAD_BACKWARD:
         raise ValueError(f"backward must be one of {sorted(_LMHEAD_BACKWARD)}, got {backward!r}")
     _require_gpu(hidden, "hidden")
@@ -1043,14 +1054,14 @@ def _lm_head_impl(hidden, weight, labels, temperature, token_mask, want_minmax, 
         sub_mask = None if grad_token_mask is None else grad_token_mask.to(dev).reshape(-1).index_select(0, idx)
         lp, ent, vmax, vmin = _lm_head_apply(
             hidden.index_select(0, idx), weight.contiguous(), y.index_select(0, idx), temperature, want_minmax, backward,
-            sub_mask, None)   # the counts of the caller are per chunk of the whole batch, not of the selected tokens
+            sub_mask, None, count_on_device)   # the caller's counts are per chunk of the whole batch, not of these tokens
         full = lambda v: torch.zeros(T, dtype=torch.float32, device=dev).index_copy(0, idx, v)
         return full(lp), full(ent), (full(vmin) if want_minmax else None), (full(vmax) if want_minmax else None)
     if grad_token_mask is not None and tuple(grad_token_mask.shape) != (hidden.shape[0],):
         raise ValueError(f"grad_token_mask shape {tuple(grad_token_mask.shape)} != ({hidden.shape[0]},)")
     lp, ent, vmax, vmin = _lm_head_apply(hidden.contiguous(), weight.contiguous(), y, temperature, want_minmax, backward,
                                          None if grad_token_mask is None else grad_token_mask.to(hidden.device),
-                                         kept_per_chunk)
+                                         kept_per_chunk, count_on_device)
     return lp, ent, vmin, vmax
 
 
@@ -1265,7 +1276,8 @@ def fused_lm_head_ppo_loss(
         logp, entropy, vmin, vmax = lm_head_logprobs_entropy_stats(
             hidden, weight, y, temperature, backward=op_backward,
             grad_token_mask=grad_mask if op_backward == "carry" else None,
-            kept_per_chunk=kept_seq if op_backward == "carry" else None)
+            kept_per_chunk=kept_seq if op_backward == "carry" else None,
+            count_on_device=count_on_device)
         logp, entropy = logp[:T_active], entropy[:T_active]
         loss, stat = ppo_actor_loss_fn(
             logp, proximal_logprobs, old_logprobs, advantages, eps_clip, loss_mask, eps_clip_higher, c_clip,

@@ -759,7 +759,10 @@ int aa_lmhead_bwd(const void* hidden, const void* weight, int64_t T, int64_t H,
  * row_has_gradient [T] (device) with kept_per_chunk (HOST), both or neither,
  * as in aa_lmhead_bwd: tokens whose byte is zero get no panel row and no
  * gradient, whatever g_logp holds for them; the same two arrays must be passed
- * to both calls.  An entropy gradient cannot be carried: use aa_lmhead_bwd
+ * to both calls.  An entry of kept_per_chunk may be AA_LMHEAD_COUNT_ON_DEVICE
+ * (below): that chunk counts as all of its tokens in panel_rows and in where
+ * the next chunk's rows start, and its kernels stop at the rows in use.  An
+ * entropy gradient cannot be carried: use aa_lmhead_bwd
  * (row_lse / row_ez of this forward serve it) when there is one.  A chunk with
  * a row that does not fit the stored form is redone from the logits tiles,
  * decided on the device.  logp / row_lse: outputs of the forward, inputs of the
@@ -788,7 +791,7 @@ int aa_lmhead_bwd_carry(const void* hidden, const void* weight, int64_t T,
                         int64_t workspace_bytes, void* stream);
 
 /* A kept_per_chunk entry that leaves the count to the device (aa_lmhead_bwd,
- * aa_lmhead_ppo_fused): the kernels of that chunk are launched for every token
+ * aa_lmhead_ppo_fused, aa_lmhead_fwd_carry / aa_lmhead_bwd_carry): the kernels of that chunk are launched for every token
  * that could have a row and stop at the rows in use, which the device counts
  * itself, so the host needs no copy of the mask and does not wait for the
  * device.  The tiles over the rows in use are numbered, and the d_hidden

@@ -508,3 +508,98 @@ def test_carried_backward_redoes_a_chunk_that_does_not_fit(device):
         assert cosine(a.cpu(), o) > 0.9999, name
         assert_same_magnitude(a, o, what=name)
     assert torch.equal(got[0][:CHUNK], ref[0][:CHUNK])   # the redone chunk: the rows of the recompute mode, bit for bit
+
+
+@pytest.mark.parametrize("T,H,V,density", [
+    (300, 128, 1088, 0.6),
+    (CHUNK + 200, 64, 640, 0.6),       # two token chunks: the second one's rows start a whole chunk further on
+    (CHUNK + 200, 64, 8256, 0.004),    # a handful of rows: d(hidden) is cut along the vocabulary, chosen on the device
+    (CHUNK + 200, 64, 640, 0.0),       # no token named at all
+])
+def test_carried_backward_with_the_rows_counted_on_the_device(device, T, H, V, density):
+    """``count_on_device=True``: nothing is read back, the stored rows keep room for every token and the kernels stop
+    at the rows in use.  The same log-probs and d(hidden) bits as with the counts read back, d(W) up to the order of
+    the sums (the rows of a chunk are the same, in the same order), and both against the oracle."""
+    hidden, weight, labels = _case(T, H, V, seed=3 * T + V, w_std=0.3)
+    g = torch.Generator().manual_seed(9)
+    mask = torch.rand(T, generator=g) < density
+    gl = torch.randn(T, generator=g) * mask.float()
+
+    def run(**kw):
+        h = hidden.to(device).requires_grad_(True)
+        w = weight.to(device).requires_grad_(True)
+        lp, _ = areal_amd.lm_head_logprobs_entropy(h, w, labels.to(device), 0.9, backward="carry",
+                                                   grad_token_mask=mask.to(device), **kw)
+        (lp * gl.to(device)).sum().backward()
+        return lp.detach(), h.grad, w.grad
+
+    on_device, read_back = run(count_on_device=True), run()
+    assert torch.equal(on_device[0], read_back[0]) and torch.equal(on_device[1], read_back[1])
+    assert torch.isfinite(on_device[2].float()).all()
+    if mask.any():
+        assert cosine(on_device[2].float().cpu(), read_back[2].float().cpu()) > 0.9999999
+        assert_same_magnitude(on_device[2].float(), read_back[2].float(), rel=1e-4)
+        h_o = hidden.float().requires_grad_(True)
+        w_o = weight.float().requires_grad_(True)
+        o_lp, _ = oracle.logprobs_entropy(oracle.lmhead_logits(h_o, w_o), labels, 0.9)
+        (o_lp * gl).sum().backward()
+        assert cosine(on_device[1].cpu(), h_o.grad) > 0.9999 and cosine(on_device[2].cpu(), w_o.grad) > 0.9999
+        assert_same_magnitude(on_device[1], h_o.grad, what="d(hidden)")
+        assert_same_magnitude(on_device[2], w_o.grad, what="d(W)")
+    else:
+        assert float(on_device[1].float().abs().max()) == 0.0 and float(on_device[2].float().abs().max()) == 0.0
+
+
+def test_carried_backward_redoes_a_chunk_with_the_rows_counted_on_the_device(device):
+    """The chunk that does not fit the stored form is redone from the logits tiles over the rows in use only; the
+    rows of the recompute mode, bit for bit."""
+    T, H, V = CHUNK + 300, 64, 1088
+    g = torch.Generator().manual_seed(5)
+    hidden = torch.randn(T, H, generator=g)
+    hidden[:CHUNK] *= 12.0
+    hidden = hidden.bfloat16()
+    weight = (0.5 * torch.randn(V, H, generator=g)).bfloat16()
+    labels = torch.randint(0, V, (T,), generator=g)
+    mask = torch.rand(T, generator=g) < 0.3
+    gl = torch.randn(T, generator=g) * mask.float()
+
+    def run(backward, **kw):
+        h = hidden.to(device).requires_grad_(True)
+        w = weight.to(device).requires_grad_(True)
+        lp, _ = areal_amd.lm_head_logprobs_entropy(h, w, labels.to(device), backward=backward,
+                                                   grad_token_mask=mask.to(device), **kw)
+        (lp * gl.to(device)).sum().backward()
+        return h.grad.float(), w.grad.float()
+
+    got, host, ref = run("carry", count_on_device=True), run("carry"), run("recompute")
+    assert torch.isfinite(got[0]).all() and torch.isfinite(got[1]).all()
+    assert torch.equal(got[0], host[0]) and torch.equal(got[0][:CHUNK], ref[0][:CHUNK])
+    assert cosine(got[1].cpu(), host[1].cpu()) > 0.9999999
+    assert_same_magnitude(got[1], host[1], rel=1e-4)
+
+
+def test_sequence_level_step_reads_nothing_back(device):
+    """GSPO through the lm_head (``fused_lm_head_ppo_loss(importance_sampling_level="sequence")``): the op keeps its
+    rows with the count on the device (default) or read back; same loss, same gradients."""
+    T, H, V = 700, 64, 1088
+    hidden, weight, labels = _case(T, H, V, seed=21, w_std=0.3)
+    g = torch.Generator().manual_seed(2)
+    ref = oracle.logprobs(oracle.lmhead_logits(hidden, weight), labels)
+    prox, old = ref + 0.05 * torch.randn(T, generator=g), ref + 0.05 * torch.randn(T, generator=g)
+    adv = torch.randn(T, generator=g)
+    mask = torch.rand(T, generator=g) < 0.5
+    cu = torch.tensor([0, 130, 400, 700], dtype=torch.int32, device=device)
+
+    def run(**kw):
+        h = hidden.to(device).requires_grad_(True)
+        w = weight.to(device).requires_grad_(True)
+        loss, _ = areal_amd.fused_lm_head_ppo_loss(h, w, labels.to(device), prox.to(device), old.to(device), adv.to(device),
+                                                   eps_clip=0.2, loss_mask=mask.to(device), cu_seqlens=cu,
+                                                   importance_sampling_level="sequence", **kw)
+        loss.backward()
+        return loss.detach(), h.grad, w.grad
+
+    a, b = run(), run(count_on_device=False)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    assert cosine(a[2].float().cpu(), b[2].float().cpu()) > 0.9999999
+    assert float(a[1].float().abs().sum()) > 0.0
