@@ -51,6 +51,22 @@ def test_header_is_plain_c(tmp_path):
     subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", "-fsyntax-only", str(src)], check=True)
 
 
+def test_count_on_device_marker_agrees_with_the_header(tmp_path):
+    """``AA_LMHEAD_COUNT_ON_DEVICE`` of the binding is the header's: a C program prints the macro."""
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    src, exe = tmp_path / "m.c", tmp_path / "m"
+    src.write_text(f'#include <stdio.h>\n#include "{HEADER}"\n'
+                   'int main(void) { printf("%lld\\n", (long long)AA_LMHEAD_COUNT_ON_DEVICE); return 0; }\n')
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    assert int(out) == _native.AA_LMHEAD_COUNT_ON_DEVICE
+
+
 def test_argument_validation_without_gpu():
     """Entry points reject bad arguments before touching the device."""
     lib = _native.load()
