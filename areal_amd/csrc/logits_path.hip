@@ -861,14 +861,32 @@ __device__ __forceinline__ void keep_packed(u32x4_t (&d)[NCH]) {
 // The factor g / T is folded into the exponent, 2^(x_j c - lse2 + log2|g / T|),
 // and its sign is applied in the conversion to 16 bits, so an element costs
 // one fma and one exponential.
-template <int DT, int NCH, bool G_POSITIVE>
+// Rows whose stride is a multiple of 32 KB (whole pairs of chunks) run 3-4 % below the others when every chunk a
+// workgroup asks for starts on a 16 KB boundary of the row; asked for 1 KB off that grid they do not (measured:
+// V = 131 072, 147 456, 180 224, 262 144, with the arrays at any base; padding every row by 1 KB, or moving the base
+// of both arrays by 1 KB, has the same effect).  SHIFT instantiations therefore lay the chunk grid of a row
+// kShiftPieces 16-byte pieces back: slot (chunk c, thread) holds piece c * 1024 + thread - kShiftPieces, and the first
+// kShiftPieces threads of chunk 0, whose piece would lie before the row, hold its last kShiftPieces pieces instead
+// (rows of whole chunks only, so every slot holds a piece).  Only chunk 0, which is always in registers, needs an
+// offset of its own per thread (voff_first); a label's slot moves with the grid (shifted_piece).
+constexpr int kShiftPieces = 64;
+constexpr int kShiftBytes = kShiftPieces * 16;
+__device__ __forceinline__ int shifted_piece(int piece, int row_pieces) {
+  if (piece < 0) return -1;
+  const int q = piece + kShiftPieces;
+  return q < row_pieces ? q : q - row_pieces;
+}
+
+template <int DT, int NCH, bool G_POSITIVE, bool SHIFT = false>
 __device__ __forceinline__ void grad_pass(const u32x4_t (&d)[NCH], float g, float inv_t, float c, float lse2,
-                                          int64_t y, int tid, int voff, __amdgpu_buffer_rsrc_t wsrc) {
+                                          int64_t y, int tid, int voff, __amdgpu_buffer_rsrc_t wsrc, int voff_first = 0,
+                                          int row_pieces = 0) {
   constexpr int NT = 1024;
   constexpr int kChunkBytes = NT * 16;
   const float lab_add = g * inv_t;
   const float kk = fast_log2(fabsf(lab_add)) - lse2;
-  const int yv = y >= 0 ? (int)(y >> 3) : -1;
+  int yv = y >= 0 ? (int)(y >> 3) : -1;
+  if constexpr (SHIFT) yv = shifted_piece(yv, row_pieces);
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     float o[8];
@@ -890,7 +908,10 @@ __device__ __forceinline__ void grad_pass(const u32x4_t (&d)[NCH], float g, floa
     r[1] = Elem<DT>::pack(o[2], o[3]);
     r[2] = Elem<DT>::pack(o[4], o[5]);
     r[3] = Elem<DT>::pack(o[6], o[7]);
-    __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + i * kChunkBytes, 0, kAuxStream);
+    if (SHIFT && i == 0)
+      __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff_first, 0, kAuxStream);
+    else
+      __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + i * kChunkBytes - (SHIFT ? kShiftBytes : 0), 0, kAuxStream);
   }
 }
 
@@ -978,7 +999,8 @@ constexpr int kTwoPerUnitChunks = 7;  // rows this short run two workgroups per 
 // With EXT the row continues past the NCH register chunks: n_lds chunks in dynamic LDS, then the tail chunks.
 // Up to kTwoPerUnitChunks chunks the kernel is compiled for 8 waves per SIMD, so that two workgroups fit on a
 // compute unit: without that request the scalar registers alone (106 per wave: 7 waves) keep the second one out.
-template <int DT, int NCH, bool EXT, bool ALIAS>
+// SHIFT: the chunk grid of a row laid 1 KB back (see grad_pass); for rows of whole chunks only.
+template <int DT, int NCH, bool EXT, bool ALIAS, bool SHIFT = false>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu((!EXT && NCH <= kTwoPerUnitChunks) ? 8 : 1)))
 void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stride_vec,
                                                      const int64_t* __restrict__ labels, float inv_t,
@@ -999,7 +1021,12 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
   const int tid = threadIdx.x;
   const float c = kLog2e * inv_t;
   const int voff = tid * 16;
-  const bool last_ok = EXT || (NCH - 1) * NT + tid < nvec;  // EXT: every register chunk is full
+  constexpr int kSh = SHIFT ? kShiftBytes : 0;  // chunks 1, 2, ... are asked for this many bytes before their place
+  // SHIFT: this thread's byte offset in chunk 0 (the last pieces of the row for the first kShiftPieces threads)
+  const int voff_first = tid < kShiftPieces ? voff + (nvec - kShiftPieces) * 16 : voff - kShiftBytes;
+  // EXT: every register chunk is full; SHIFT: the row is whole chunks (the comparison stays, so that the passes over
+  // the row keep the schedule of the other instantiations)
+  const bool last_ok = EXT || (NCH - 1) * NT + (SHIFT ? (tid & 1) : tid) < nvec;
   float fn, gscale;
   load_loss_scale(a, fn, gscale);
   // EXT: chunk NCH + j goes to LDS for j < n_lds; each wave deposits its 1 KiB piece, lane by lane
@@ -1009,7 +1036,12 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
   auto load_lds_chunks = [&](const __amdgpu_buffer_rsrc_t rsrc) {
     for (int j = 0; j < n_lds; ++j)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(ext_lds + j * kChunkBytes + lds_wave_off), 16, voff,
-                                               (NCH + j) * kChunkBytes, 0, kAuxStream);
+                                               (NCH + j) * kChunkBytes - kSh, 0, kAuxStream);
+  };
+  // load of register chunk i (a compile-time slot)
+  auto load_reg = [&](const __amdgpu_buffer_rsrc_t rsrc, int i) {
+    if (SHIFT && i == 0) return __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff_first, 0, kAuxStream);
+    return __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, i * kChunkBytes - kSh, kAuxStream);
   };
 
   int64_t t = blockIdx.x;  // the host launches at most T workgroups
@@ -1018,7 +1050,7 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
   {
     const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, V * 2, kBufferFlags);
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) d[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, i * kChunkBytes, kAuxStream);
+    for (int i = 0; i < NCH; ++i) d[i] = load_reg(rsrc, i);
     if constexpr (EXT) load_lds_chunks(rsrc);
   }
   int64_t y = labels[t];
@@ -1047,7 +1079,7 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
       rsrc_t = __builtin_amdgcn_make_buffer_rsrc((void*)(logits + t * stride_vec), 0, V * 2, kBufferFlags);
 #pragma unroll
       for (int q = 0; q < kExtTailChunks; ++q) {
-        tv[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_t, voff, (tail0 + q) * kChunkBytes, 0);  // stays cached for the second read
+        tv[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_t, voff, (tail0 + q) * kChunkBytes - kSh, 0);  // stays cached for the second read
         tail_ok[q] = (tail0 + q) * NT + tid < nvec;
       }
     }
@@ -1136,36 +1168,42 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
       if (g != 0.f) {
 #pragma unroll
         for (int q = 0; q < kExtTailChunks; ++q)
-          tv[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_t, voff, (tail0 + q) * kChunkBytes, kAuxStream);
+          tv[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_t, voff, (tail0 + q) * kChunkBytes - kSh, kAuxStream);
       }
     }
     if (g == 0.f) {
       const u32x4_t z = {0u, 0u, 0u, 0u};
 #pragma unroll
-      for (int i = 0; i < NCH; ++i) __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, voff + i * kChunkBytes, 0, kAuxStream);
+      for (int i = 0; i < NCH; ++i)
+        __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, (SHIFT && i == 0) ? voff_first : voff + i * kChunkBytes - kSh, 0,
+                                               kAuxStream);
       if constexpr (EXT) {
-        for (int j = 0; j < n_lds + kExtTailChunks; ++j)  // chunks past the row are dropped by the descriptor
-          __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, voff + (NCH + j) * kChunkBytes, 0, kAuxStream);
+        // chunks past the row are dropped by the descriptor (SHIFT: the first of them would reach back into the row)
+        for (int j = 0; j < n_lds + kExtTailChunks && !(SHIFT && (NCH + j) * NT >= nvec); ++j)
+          __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, voff + (NCH + j) * kChunkBytes - kSh, 0, kAuxStream);
       }
     } else if (g > 0.f) {
-      grad_pass<DT, NCH, true>(d, g, inv_t, c, ro.lse2, y_ok ? y : -1, tid, voff, wsrc);
+      grad_pass<DT, NCH, true, SHIFT>(d, g, inv_t, c, ro.lse2, y_ok ? y : -1, tid, voff, wsrc, voff_first, nvec);
     } else {
-      grad_pass<DT, NCH, false>(d, g, inv_t, c, ro.lse2, y_ok ? y : -1, tid, voff, wsrc);
+      grad_pass<DT, NCH, false, SHIFT>(d, g, inv_t, c, ro.lse2, y_ok ? y : -1, tid, voff, wsrc, voff_first, nvec);
     }
     if constexpr (EXT) {
       if (g != 0.f) {
         const float lab_add = g * inv_t;
         const float kk = fast_log2(fabsf(lab_add)) - ro.lse2;
-        const int yv = y_ok ? (int)(y >> 3) : -1;
+        const int yv_row = y_ok ? (int)(y >> 3) : -1;
+        const int yv = SHIFT ? shifted_piece(yv_row, nvec) : yv_row;
         const int y_elem = (int)(y & 7);
         for (int j = 0; j < n_lds; ++j) {
           const u32x4_t r = grad_chunk<DT>(my_lds[j * NT], c, kk, lab_add, g > 0.f, yv, y_elem, NCH + j, tid);
-          __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + (NCH + j) * kChunkBytes, 0, kAuxStream);
+          __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + (NCH + j) * kChunkBytes - kSh, 0, kAuxStream);
         }
 #pragma unroll
         for (int q = 0; q < kExtTailChunks; ++q) {
+          // SHIFT: a chunk past the row would reach back into it (the descriptor drops it otherwise)
+          if (SHIFT && (tail0 + q) * NT >= nvec) continue;
           const u32x4_t r = grad_chunk<DT>(tv[q], c, kk, lab_add, g > 0.f, yv, y_elem, tail0 + q, tid);
-          __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + (tail0 + q) * kChunkBytes, 0, kAuxStream);
+          __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + (tail0 + q) * kChunkBytes - kSh, 0, kAuxStream);
         }
       }
     }
@@ -1175,8 +1213,7 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
     {
       const __amdgpu_buffer_rsrc_t rsrc_n = __builtin_amdgcn_make_buffer_rsrc((void*)src_n, 0, V * 2, kBufferFlags);
 #pragma unroll
-      for (int i = 0; i < NCH; ++i)
-        d[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_n, voff, i * kChunkBytes, kAuxStream);
+      for (int i = 0; i < NCH; ++i) d[i] = load_reg(rsrc_n, i);
       if constexpr (EXT) {
         asm volatile("" ::: "memory");  // the LDS reads of the gradient pass stay ahead of the next row's deposits
         load_lds_chunks(rsrc_n);
@@ -1295,7 +1332,7 @@ static int persistent_workgroups() {
   return n;
 }
 
-template <int DT, int NCH>
+template <int DT, int NCH, bool SHIFT = false>
 static void launch_regs(const void* logits, int64_t T, int V, int64_t stride, const int64_t* labels, float inv_t,
                         const FusedTokenArgs& a, void* dlogits, int32_t* work, hipStream_t st) {
   // Short rows (up to 6 chunks: at most 64 VGPRs per thread) leave room for a second workgroup on every compute
@@ -1304,11 +1341,11 @@ static void launch_regs(const void* logits, int64_t T, int V, int64_t stride, co
   const int64_t wgs = T < resident ? T : resident;
   const uintptr_t mask_addr = (uintptr_t)a.mask_eff;
   if (dlogits == logits)
-    hipLaunchKernelGGL((k_fused_regs<DT, NCH, false, true>), dim3((unsigned)wgs), dim3(1024), 0, st, (const uint4*)logits, V,
+    hipLaunchKernelGGL((k_fused_regs<DT, NCH, false, true, SHIFT>), dim3((unsigned)wgs), dim3(1024), 0, st, (const uint4*)logits, V,
                        stride >> 3, labels, inv_t, a.prox_logp, a.adv, (const uint32_t*)(mask_addr & ~(uintptr_t)3),
                        (unsigned)(mask_addr & 3), a.behave_w, a, (uint4*)dlogits, T, work, 0);
   else
-    hipLaunchKernelGGL((k_fused_regs<DT, NCH, false, false>), dim3((unsigned)wgs), dim3(1024), 0, st, (const uint4*)logits, V,
+    hipLaunchKernelGGL((k_fused_regs<DT, NCH, false, false, SHIFT>), dim3((unsigned)wgs), dim3(1024), 0, st, (const uint4*)logits, V,
                        stride >> 3, labels, inv_t, a.prox_logp, a.adv, (const uint32_t*)(mask_addr & ~(uintptr_t)3),
                        (unsigned)(mask_addr & 3), a.behave_w, a, (uint4*)dlogits, T, work, 0);
 }
@@ -1316,34 +1353,51 @@ static void launch_regs(const void* logits, int64_t T, int V, int64_t stride, co
 // Rows of more than kMaxRegChunks chunks: registers + LDS + streamed tail (see k_fused_regs, EXT).
 constexpr int kMaxExtChunks = kExtRegChunks + kExtLdsChunks + kExtTailChunks;
 
-template <int DT>
+template <int DT, bool SHIFT>
 static bool launch_regs_ext(int nch, const void* logits, int64_t T, int V, int64_t stride, const int64_t* labels,
                             float inv_t, const FusedTokenArgs& a, void* dlogits, int32_t* work, hipStream_t st) {
   static const bool ok =
-      hipFuncSetAttribute((const void*)k_fused_regs<DT, kExtRegChunks, true, false>,
+      hipFuncSetAttribute((const void*)k_fused_regs<DT, kExtRegChunks, true, false, SHIFT>,
                           hipFuncAttributeMaxDynamicSharedMemorySize, kExtLdsChunks * 16384) == hipSuccess &&
-      hipFuncSetAttribute((const void*)k_fused_regs<DT, kExtRegChunks, true, true>,
+      hipFuncSetAttribute((const void*)k_fused_regs<DT, kExtRegChunks, true, true, SHIFT>,
                           hipFuncAttributeMaxDynamicSharedMemorySize, kExtLdsChunks * 16384) == hipSuccess;
   if (!ok || nch <= kExtRegChunks || nch > kMaxExtChunks) return false;
   const int n_lds = nch - kExtRegChunks < kExtLdsChunks ? nch - kExtRegChunks : kExtLdsChunks;
   const int64_t wgs = T < persistent_workgroups() ? T : persistent_workgroups();
   const uintptr_t mask_addr = (uintptr_t)a.mask_eff;
   if (dlogits == logits)
-    hipLaunchKernelGGL((k_fused_regs<DT, kExtRegChunks, true, true>), dim3((unsigned)wgs), dim3(1024), n_lds * 16384, st,
+    hipLaunchKernelGGL((k_fused_regs<DT, kExtRegChunks, true, true, SHIFT>), dim3((unsigned)wgs), dim3(1024), n_lds * 16384, st,
                        (const uint4*)logits, V, stride >> 3, labels, inv_t, a.prox_logp, a.adv,
                        (const uint32_t*)(mask_addr & ~(uintptr_t)3), (unsigned)(mask_addr & 3), a.behave_w, a,
                        (uint4*)dlogits, T, work, n_lds);
   else
-    hipLaunchKernelGGL((k_fused_regs<DT, kExtRegChunks, true, false>), dim3((unsigned)wgs), dim3(1024), n_lds * 16384, st,
+    hipLaunchKernelGGL((k_fused_regs<DT, kExtRegChunks, true, false, SHIFT>), dim3((unsigned)wgs), dim3(1024), n_lds * 16384, st,
                        (const uint4*)logits, V, stride >> 3, labels, inv_t, a.prox_logp, a.adv,
                        (const uint32_t*)(mask_addr & ~(uintptr_t)3), (unsigned)(mask_addr & 3), a.behave_w, a,
                        (uint4*)dlogits, T, work, n_lds);
   return true;
 }
 
+// Rows of whole chunks at a stride of whole pairs of chunks, from kShiftMinChunks chunks on, take the shifted chunk
+// grid (see grad_pass).
+constexpr int kShiftMinChunks = 10;
+static bool wants_shift(int nch, int V, int64_t stride) {
+  return nch >= kShiftMinChunks && V % 8192 == 0 && stride % 16384 == 0;
+}
+
 template <int DT>
 static bool dispatch_regs(int nch, const void* logits, int64_t T, int V, int64_t stride, const int64_t* labels,
                           float inv_t, const FusedTokenArgs& a, void* dlogits, int32_t* work, hipStream_t st) {
+  if (wants_shift(nch, V, stride)) {
+    switch (nch) {
+#define AA_CASE(N) \
+  case N: launch_regs<DT, N, true>(logits, T, V, stride, labels, inv_t, a, dlogits, work, st); return true;
+      AA_CASE(10) AA_CASE(11) AA_CASE(12) AA_CASE(13) AA_CASE(14) AA_CASE(15)
+      AA_CASE(16) AA_CASE(17) AA_CASE(18) AA_CASE(19) AA_CASE(20) AA_CASE(21)
+#undef AA_CASE
+      default: break;
+    }
+  }
   switch (nch) {
 #define AA_CASE(N) \
   case N: launch_regs<DT, N>(logits, T, V, stride, labels, inv_t, a, dlogits, work, st); return true;
@@ -1472,9 +1526,15 @@ extern "C" int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int
                ? dispatch_regs<AA_BF16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st)
                : dispatch_regs<AA_F16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st);
     else
-      ok = (dtype == AA_BF16)
-               ? launch_regs_ext<AA_BF16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st)
-               : launch_regs_ext<AA_F16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st);
+      ok = wants_shift(nch, (int)V, row_stride)
+               ? ((dtype == AA_BF16) ? launch_regs_ext<AA_BF16, true>(nch, logits, T, (int)V, row_stride, labels,
+                                                                     inv_temperature, a, dlogits, work, st)
+                                     : launch_regs_ext<AA_F16, true>(nch, logits, T, (int)V, row_stride, labels,
+                                                                    inv_temperature, a, dlogits, work, st))
+               : ((dtype == AA_BF16) ? launch_regs_ext<AA_BF16, false>(nch, logits, T, (int)V, row_stride, labels,
+                                                                      inv_temperature, a, dlogits, work, st)
+                                     : launch_regs_ext<AA_F16, false>(nch, logits, T, (int)V, row_stride, labels,
+                                                                     inv_temperature, a, dlogits, work, st));
     if (ok) return launch_status();
   }
   if (dtype == AA_F32 && (V % 8 == 0) && (row_stride % 4 == 0) && V >= kHoldChunk && V <= ((int64_t)1 << 28) &&

@@ -581,3 +581,48 @@ def test_supervised_gradient_written_over_the_logits(device):
     l2.backward()
     assert torch.equal(l2.detach(), loss.detach()) and torch.equal(y.detach(), x.grad) and torch.equal(y.grad, x.grad)
     assert torch.equal(s2["logprobs"], stat["logprobs"])
+
+
+@pytest.mark.parametrize("V,dtype", [
+    (81920, torch.bfloat16),     # 10 chunks: the shortest rows that take the shifted chunk grid
+    (131072, torch.float16),     # 16 chunks
+    (163840, torch.bfloat16),    # 20 chunks
+    (180224, torch.bfloat16),    # 22 chunks: 21 in registers, one in LDS
+    (262144, torch.bfloat16),    # 32 chunks: registers, LDS and the tail that is read twice
+])
+def test_rows_of_whole_chunks_on_the_shifted_grid(device, V, dtype):
+    """Rows of whole 8192-value chunks at a stride of whole chunk pairs are walked on a chunk grid laid 1 KB back (the
+    first 64 threads of chunk 0 hold the last 512 values of the row).  Labels in every place that moves: the first and
+    last 512 values, both sides of the first chunk borders, the last value.  Against the oracle, in place, and against
+    the same rows at a stride that keeps the plain grid."""
+    lengths = synth.lengths_uniform(6, 6, 12, seed=V)
+    case = synth.make_logits_case("t", lengths, V, V, device, synth.per_sequence_normal_advantages(lengths, 3),
+                                  dtype=dtype, ppo=dict(eps_clip=0.2))
+    special = [0, 7, 8, 511, 512, 7679, 7680, 8191, 8192, 8703, 8704, 16383, 16384, V - 8193, V - 8192, V - 513, V - 512,
+               V - 9, V - 8, V - 1]
+    n = min(len(special), case.n_tokens)
+    case.labels[:n] = torch.tensor(special[:n], device=device)
+    case.loss_mask[:n] = True
+    _finish_case(case)
+    got = _fused_step(case)
+    _compare(case, got, _oracle_step(case))
+    # the gradient written over the logits: the same bits
+    x = case.logits.clone().requires_grad_(True)
+    l2, s2 = areal_amd.fused_logprobs_ppo_loss(x, case.labels, case.prox_logp, case.old_logp, case.advantages,
+                                               loss_mask=case.loss_mask, cu_seqlens=case.cu_seqlens,
+                                               temperature=case.temperature, inplace_backward=True, **case.ppo)
+    assert torch.equal(x.detach(), got[2]) and torch.equal(l2.detach(), got[0])
+    assert torch.equal(s2["logprobs"], got[1]["logprobs"]) and torch.equal(s2["entropy"], got[1]["entropy"])
+    # the same rows inside a wider array (stride V + 8: the plain grid): the same results up to the order of the sums
+    wide = torch.zeros(case.n_tokens, V + 8, dtype=dtype, device=device)
+    wide[:, :V] = case.logits
+    y = wide[:, :V].requires_grad_(True)
+    l3, s3 = areal_amd.fused_logprobs_ppo_loss(y, case.labels, case.prox_logp, case.old_logp, case.advantages,
+                                               loss_mask=case.loss_mask, cu_seqlens=case.cu_seqlens,
+                                               temperature=case.temperature, **case.ppo)
+    l3.backward()
+    assert float((s3["logprobs"] - got[1]["logprobs"]).abs().max()) < 1e-5
+    assert float(l3.detach()) == pytest.approx(float(got[0]), rel=1e-5)
+    step = float(got[2].float().abs().max()) * (2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11)
+    assert float((y.grad.float() - got[2].float()).abs().max()) <= step
+    assert float((y.grad == got[2]).float().mean()) > 0.999
