@@ -97,6 +97,9 @@ def parse_args():
     ap.add_argument("--logits-dtype", choices=["bf16", "f32"], default="bf16",
                     help="logits workloads: hand the kernels fp32 logits (what a Megatron-style head emits) instead of "
                          "bf16; 8 bytes per element instead of 4")
+    ap.add_argument("--vocab", type=int, default=None,
+                    help="cfg1-32k only: width of the logits rows instead of 151936 (other vocabulary sizes through the "
+                         "same kernels; the traffic factor quoted is that of 151936)")
     ap.add_argument("--steps-only", action="store_true",
                     help="fused lm_head workloads: launch the steps of the selected backward mode only (no stand-alone "
                          "op, no other mode), so that every dispatch a profiler sees belongs to a step")
@@ -159,7 +162,7 @@ def time_events(launch, iters: int, stream):
 # ----------------------------------------------------------------------------------------------------------------
 # logits path
 # ----------------------------------------------------------------------------------------------------------------
-def build_logits_case(name: str, seed: int, device):
+def build_logits_case(name: str, seed: int, device, vocab: int | None = None):
     import areal_amd
     from areal_amd import synth
 
@@ -170,6 +173,9 @@ def build_logits_case(name: str, seed: int, device):
         case = synth.config1(device, seed)
         desc = ("configs[1]: 64 packed seqs, lengths lognormal(7.5,0.6) clipped to [128,4096], V=151936, GRPO groups "
                 "of 16, decoupled loss, importance-weight cap 5.0 (token/mask/ratio)")
+    elif vocab is not None:
+        case = synth.config1(device, seed, V=vocab, total_tokens=32768)
+        desc = f"configs[1] truncated to the leading sequences that total 32768 tokens, with a vocabulary of {vocab}"
     else:
         case = synth.config1(device, seed, total_tokens=32768)
         desc = "configs[1] truncated to the leading sequences that total 32768 tokens"
@@ -350,7 +356,7 @@ def bench_logits(args, dev, workload: str, steps: int, warmup: int, cpu_tokens: 
     """GPU part of a logits workload.  Returns the result line and the sample for the CPU phase (None: no CPU phase)."""
     import torch
 
-    case, desc = build_logits_case(workload, args.seed, dev)
+    case, desc = build_logits_case(workload, args.seed, dev, getattr(args, "vocab", None) if workload == "cfg1-32k" else None)
     kw, cfg = ppo_kwargs(case)
     T, V = case.logits.shape
     f32 = args.logits_dtype == "f32"
