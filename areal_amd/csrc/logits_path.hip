@@ -861,10 +861,11 @@ __device__ __forceinline__ void keep_packed(u32x4_t (&d)[NCH]) {
 // The factor g / T is folded into the exponent, 2^(x_j c - lse2 + log2|g / T|),
 // and its sign is applied in the conversion to 16 bits, so an element costs
 // one fma and one exponential.
-// Rows whose stride is a multiple of 32 KB (whole pairs of chunks) run 3-4 % below the others when every chunk a
-// workgroup asks for starts on a 16 KB boundary of the row; asked for 1 KB off that grid they do not (measured:
-// V = 131 072, 147 456, 180 224, 262 144, with the arrays at any base; padding every row by 1 KB, or moving the base
-// of both arrays by 1 KB, has the same effect).  SHIFT instantiations therefore lay the chunk grid of a row
+// Rows of whole chunks at a stride of whole chunks run 2-4 % below what they can when every 16 KB request of a
+// workgroup starts on a 4 KB boundary; asked for 1, 2 or 3 KB off that grid they do not (measured on V = 90 112 ...
+// 262 144 with the plain grid and the base of both arrays moved in steps of 128 bytes: multiples of 4 KB read
+// 75.4-76.4 % of the HBM peak, the other multiples of 1 KB 77.6-77.7 %, anything else 75-76.3 %; worst at strides of
+// whole 32 KB, where some layouts of the arrays lose 4 % more).  SHIFT instantiations therefore lay the chunk grid of a row
 // kShiftPieces 16-byte pieces back: slot (chunk c, thread) holds piece c * 1024 + thread - kShiftPieces, and the first
 // kShiftPieces threads of chunk 0, whose piece would lie before the row, hold its last kShiftPieces pieces instead
 // (rows of whole chunks only, so every slot holds a piece).  Only chunk 0, which is always in registers, needs an
@@ -1378,11 +1379,11 @@ static bool launch_regs_ext(int nch, const void* logits, int64_t T, int V, int64
   return true;
 }
 
-// Rows of whole chunks at a stride of whole pairs of chunks, from kShiftMinChunks chunks on, take the shifted chunk
-// grid (see grad_pass).
+// Rows of whole chunks at a stride of whole chunks, from kShiftMinChunks chunks on, take the shifted chunk grid (see
+// grad_pass): their requests would all start on 16 KB boundaries.  (Below 10 chunks the shift does nothing or costs.)
 constexpr int kShiftMinChunks = 10;
 static bool wants_shift(int nch, int V, int64_t stride) {
-  return nch >= kShiftMinChunks && V % 8192 == 0 && stride % 16384 == 0;
+  return nch >= kShiftMinChunks && V % 8192 == 0 && stride % 8192 == 0;
 }
 
 template <int DT>

@@ -585,13 +585,15 @@ def test_supervised_gradient_written_over_the_logits(device):
 
 @pytest.mark.parametrize("V,dtype", [
     (81920, torch.bfloat16),     # 10 chunks: the shortest rows that take the shifted chunk grid
+    (90112, torch.bfloat16),     # 11 chunks: a stride of an odd number of chunks
+    (155648, torch.float16),     # 19 chunks
     (131072, torch.float16),     # 16 chunks
     (163840, torch.bfloat16),    # 20 chunks
     (180224, torch.bfloat16),    # 22 chunks: 21 in registers, one in LDS
     (262144, torch.bfloat16),    # 32 chunks: registers, LDS and the tail that is read twice
 ])
 def test_rows_of_whole_chunks_on_the_shifted_grid(device, V, dtype):
-    """Rows of whole 8192-value chunks at a stride of whole chunk pairs are walked on a chunk grid laid 1 KB back (the
+    """Rows of whole 8192-value chunks at a stride of whole chunks are walked on a chunk grid laid 1 KB back (the
     first 64 threads of chunk 0 hold the last 512 values of the row).  Labels in every place that moves: the first and
     last 512 values, both sides of the first chunk borders, the last value.  Against the oracle, in place, and against
     the same rows at a stride that keeps the plain grid."""
