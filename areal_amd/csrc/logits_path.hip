@@ -878,16 +878,32 @@ __device__ __forceinline__ int shifted_piece(int piece, int row_pieces) {
   return q < row_pieces ? q : q - row_pieces;
 }
 
-template <int DT, int NCH, bool G_POSITIVE, bool SHIFT = false>
+// SHIFT == 2 (rows that are not whole chunks, or not a whole number of chunks apart): the same idea with a shift of
+// the row's own, `sh` bytes (a multiple of 16, below 16 KB), chosen so that the 16 KB requests of the row start
+// kShiftTargetBytes past a 16 KB boundary of the address space.  The buffer descriptor of the row starts `sh` bytes
+// before the row, so slot (chunk c, thread) is asked for at c * 16 KB + thread * 16 as in the plain grid and holds
+// piece c * 1024 + thread - sh / 16; the threads of chunk 0 below sh / 16, whose piece would lie before the row, hold
+// its last pieces, which the plain grid's slots at and past the row's piece count would have held: those slots stay
+// empty (the same test as in the plain grid), but the descriptor no longer drops what they would store, so the last
+// chunk's store is skipped by the threads without a piece.
+constexpr int kShiftTargetBytes = 1024;
+__device__ __forceinline__ int shifted_piece_by(int piece, int shift_pieces, int row_pieces) {
+  if (piece < 0) return -1;
+  const int q = piece + shift_pieces;
+  return q < row_pieces ? q : q - row_pieces;
+}
+
+template <int DT, int NCH, bool G_POSITIVE, int SHIFT = 0>
 __device__ __forceinline__ void grad_pass(const u32x4_t (&d)[NCH], float g, float inv_t, float c, float lse2,
                                           int64_t y, int tid, int voff, __amdgpu_buffer_rsrc_t wsrc, int voff_first = 0,
-                                          int row_pieces = 0) {
+                                          int row_pieces = 0, int sh = 0, bool last_ok = true) {
   constexpr int NT = 1024;
   constexpr int kChunkBytes = NT * 16;
   const float lab_add = g * inv_t;
   const float kk = fast_log2(fabsf(lab_add)) - lse2;
   int yv = y >= 0 ? (int)(y >> 3) : -1;
-  if constexpr (SHIFT) yv = shifted_piece(yv, row_pieces);
+  if constexpr (SHIFT == 1) yv = shifted_piece(yv, row_pieces);
+  if constexpr (SHIFT == 2) yv = shifted_piece_by(yv, sh >> 4, row_pieces);
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     float o[8];
@@ -909,10 +925,16 @@ __device__ __forceinline__ void grad_pass(const u32x4_t (&d)[NCH], float g, floa
     r[1] = Elem<DT>::pack(o[2], o[3]);
     r[2] = Elem<DT>::pack(o[4], o[5]);
     r[3] = Elem<DT>::pack(o[6], o[7]);
-    if (SHIFT && i == 0)
+    if constexpr (SHIFT == 2) {
+      if (i == 0)
+        __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + (voff < sh ? row_pieces * 16 : 0), 0, kAuxStream);
+      else if (i < NCH - 1 || last_ok)
+        __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + i * kChunkBytes, 0, kAuxStream);
+    } else if (SHIFT == 1 && i == 0) {
       __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff_first, 0, kAuxStream);
-    else
-      __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + i * kChunkBytes - (SHIFT ? kShiftBytes : 0), 0, kAuxStream);
+    } else {
+      __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + i * kChunkBytes - (SHIFT == 1 ? kShiftBytes : 0), 0, kAuxStream);
+    }
   }
 }
 
@@ -1000,8 +1022,9 @@ constexpr int kTwoPerUnitChunks = 7;  // rows this short run two workgroups per 
 // With EXT the row continues past the NCH register chunks: n_lds chunks in dynamic LDS, then the tail chunks.
 // Up to kTwoPerUnitChunks chunks the kernel is compiled for 8 waves per SIMD, so that two workgroups fit on a
 // compute unit: without that request the scalar registers alone (106 per wave: 7 waves) keep the second one out.
-// SHIFT: the chunk grid of a row laid 1 KB back (see grad_pass); for rows of whole chunks only.
-template <int DT, int NCH, bool EXT, bool ALIAS, bool SHIFT = false>
+// SHIFT (see grad_pass): 1: the chunk grid of a row laid 1 KB back, for rows of whole chunks a whole number of chunks
+// apart; 2: laid back by an amount of the row's own (not with EXT).
+template <int DT, int NCH, bool EXT, bool ALIAS, int SHIFT = 0>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu((!EXT && NCH <= kTwoPerUnitChunks) ? 8 : 1)))
 void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stride_vec,
                                                      const int64_t* __restrict__ labels, float inv_t,
@@ -1022,12 +1045,28 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
   const int tid = threadIdx.x;
   const float c = kLog2e * inv_t;
   const int voff = tid * 16;
-  constexpr int kSh = SHIFT ? kShiftBytes : 0;  // chunks 1, 2, ... are asked for this many bytes before their place
+  static_assert(SHIFT != 2 || !EXT, "a shift per row is written for rows that fit in registers");
+  constexpr int kSh = SHIFT == 1 ? kShiftBytes : 0;  // chunks 1, 2, ... are asked for this many bytes before their place
   // SHIFT: this thread's byte offset in chunk 0 (the last pieces of the row for the first kShiftPieces threads)
   const int voff_first = tid < kShiftPieces ? voff + (nvec - kShiftPieces) * 16 : voff - kShiftBytes;
   // EXT: every register chunk is full; SHIFT: the row is whole chunks (the comparison stays, so that the passes over
   // the row keep the schedule of the other instantiations)
-  const bool last_ok = EXT || (NCH - 1) * NT + (SHIFT ? (tid & 1) : tid) < nvec;
+  const bool last_ok = EXT || (NCH - 1) * NT + (SHIFT == 1 ? (tid & 1) : tid) < nvec;
+  // SHIFT == 2: the shift of a row in bytes (uniform), and the descriptor of a row that starts that far before it
+  // It is taken from where the row starts inside the array (row index x stride), as if the array started on a 4 KB
+  // boundary, which large allocations do: results then do not depend on where an array lies.  The smallest shift that
+  // puts the requests on a 1 KB boundary other than a 4 KB one.
+  auto row_shift = [&](int64_t row_index) -> int {
+    if constexpr (SHIFT != 2) return 0;
+    else {
+      const int off = (int)(((uint32_t)row_index * (uint32_t)((stride_vec * 16) & 4095)) & 4095);
+      const int a = off & 1023;
+      return __builtin_amdgcn_readfirstlane((off >> 10) == 0 ? a + 1024 : a);
+    }
+  };
+  auto row_rsrc = [&](const void* row, int sh) {
+    return __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)row - sh), 0, V * 2 + sh, kBufferFlags);
+  };
   float fn, gscale;
   load_loss_scale(a, fn, gscale);
   // EXT: chunk NCH + j goes to LDS for j < n_lds; each wave deposits its 1 KiB piece, lane by lane
@@ -1040,18 +1079,21 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
                                                (NCH + j) * kChunkBytes - kSh, 0, kAuxStream);
   };
   // load of register chunk i (a compile-time slot)
-  auto load_reg = [&](const __amdgpu_buffer_rsrc_t rsrc, int i) {
-    if (SHIFT && i == 0) return __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff_first, 0, kAuxStream);
+  auto load_reg = [&](const __amdgpu_buffer_rsrc_t rsrc, int i, int sh) {
+    if (SHIFT == 2 && i == 0)
+      return __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff + (voff < sh ? nvec * 16 : 0), 0, kAuxStream);
+    if (SHIFT == 1 && i == 0) return __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff_first, 0, kAuxStream);
     return __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, i * kChunkBytes - kSh, kAuxStream);
   };
 
   int64_t t = blockIdx.x;  // the host launches at most T workgroups
   const uint4* src = logits + t * stride_vec;
   u32x4_t d[NCH];
+  int sh = row_shift(t);
   {
-    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, V * 2, kBufferFlags);
+    const __amdgpu_buffer_rsrc_t rsrc = row_rsrc(src, sh);
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) d[i] = load_reg(rsrc, i);
+    for (int i = 0; i < NCH; ++i) d[i] = load_reg(rsrc, i, sh);
     if constexpr (EXT) load_lds_chunks(rsrc);
   }
   int64_t y = labels[t];
@@ -1164,7 +1206,7 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
     const uint32_t xy_raw_n = load_u16_uniform(src_n, y_ok_n ? y_n : 0);
     const TokenIn tin_n = load_token_in_ro(in_prox, in_adv, in_mask32, mask_mis, in_bw, has_w, a.T_active, more ? tn : t);
 
-    const __amdgpu_buffer_rsrc_t wsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(dlogits + t * stride_vec), 0, V * 2, kBufferFlags);
+    const __amdgpu_buffer_rsrc_t wsrc = row_rsrc((const void*)(dlogits + t * stride_vec), sh);
     if constexpr (EXT) {
       if (g != 0.f) {
 #pragma unroll
@@ -1175,25 +1217,33 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
     if (g == 0.f) {
       const u32x4_t z = {0u, 0u, 0u, 0u};
 #pragma unroll
-      for (int i = 0; i < NCH; ++i)
-        __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, (SHIFT && i == 0) ? voff_first : voff + i * kChunkBytes - kSh, 0,
-                                               kAuxStream);
+      for (int i = 0; i < NCH; ++i) {
+        if constexpr (SHIFT == 2) {
+          if (i == 0)
+            __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, voff + (voff < sh ? nvec * 16 : 0), 0, kAuxStream);
+          else if (i < NCH - 1 || last_ok)
+            __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, voff + i * kChunkBytes, 0, kAuxStream);
+        } else {
+          __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, (SHIFT == 1 && i == 0) ? voff_first : voff + i * kChunkBytes - kSh,
+                                                 0, kAuxStream);
+        }
+      }
       if constexpr (EXT) {
         // chunks past the row are dropped by the descriptor (SHIFT: the first of them would reach back into the row)
-        for (int j = 0; j < n_lds + kExtTailChunks && !(SHIFT && (NCH + j) * NT >= nvec); ++j)
+        for (int j = 0; j < n_lds + kExtTailChunks && !(SHIFT == 1 && (NCH + j) * NT >= nvec); ++j)
           __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, voff + (NCH + j) * kChunkBytes - kSh, 0, kAuxStream);
       }
     } else if (g > 0.f) {
-      grad_pass<DT, NCH, true, SHIFT>(d, g, inv_t, c, ro.lse2, y_ok ? y : -1, tid, voff, wsrc, voff_first, nvec);
+      grad_pass<DT, NCH, true, SHIFT>(d, g, inv_t, c, ro.lse2, y_ok ? y : -1, tid, voff, wsrc, voff_first, nvec, sh, last_ok);
     } else {
-      grad_pass<DT, NCH, false, SHIFT>(d, g, inv_t, c, ro.lse2, y_ok ? y : -1, tid, voff, wsrc, voff_first, nvec);
+      grad_pass<DT, NCH, false, SHIFT>(d, g, inv_t, c, ro.lse2, y_ok ? y : -1, tid, voff, wsrc, voff_first, nvec, sh, last_ok);
     }
     if constexpr (EXT) {
       if (g != 0.f) {
         const float lab_add = g * inv_t;
         const float kk = fast_log2(fabsf(lab_add)) - ro.lse2;
         const int yv_row = y_ok ? (int)(y >> 3) : -1;
-        const int yv = SHIFT ? shifted_piece(yv_row, nvec) : yv_row;
+        const int yv = SHIFT == 1 ? shifted_piece(yv_row, nvec) : yv_row;
         const int y_elem = (int)(y & 7);
         for (int j = 0; j < n_lds; ++j) {
           const u32x4_t r = grad_chunk<DT>(my_lds[j * NT], c, kk, lab_add, g > 0.f, yv, y_elem, NCH + j, tid);
@@ -1202,7 +1252,7 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
 #pragma unroll
         for (int q = 0; q < kExtTailChunks; ++q) {
           // SHIFT: a chunk past the row would reach back into it (the descriptor drops it otherwise)
-          if (SHIFT && (tail0 + q) * NT >= nvec) continue;
+          if (SHIFT == 1 && (tail0 + q) * NT >= nvec) continue;
           const u32x4_t r = grad_chunk<DT>(tv[q], c, kk, lab_add, g > 0.f, yv, y_elem, tail0 + q, tid);
           __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + (tail0 + q) * kChunkBytes - kSh, 0, kAuxStream);
         }
@@ -1212,9 +1262,10 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
     // All stores of this row are issued before the loads of the next one:
     // alternating them chunk by chunk costs bandwidth on this memory system.
     {
-      const __amdgpu_buffer_rsrc_t rsrc_n = __builtin_amdgcn_make_buffer_rsrc((void*)src_n, 0, V * 2, kBufferFlags);
+      sh = row_shift(more ? tn : t);
+      const __amdgpu_buffer_rsrc_t rsrc_n = row_rsrc(src_n, sh);
 #pragma unroll
-      for (int i = 0; i < NCH; ++i) d[i] = load_reg(rsrc_n, i);
+      for (int i = 0; i < NCH; ++i) d[i] = load_reg(rsrc_n, i, sh);
       if constexpr (EXT) {
         asm volatile("" ::: "memory");  // the LDS reads of the gradient pass stay ahead of the next row's deposits
         load_lds_chunks(rsrc_n);
@@ -1333,7 +1384,7 @@ static int persistent_workgroups() {
   return n;
 }
 
-template <int DT, int NCH, bool SHIFT = false>
+template <int DT, int NCH, int SHIFT = 0>
 static void launch_regs(const void* logits, int64_t T, int V, int64_t stride, const int64_t* labels, float inv_t,
                         const FusedTokenArgs& a, void* dlogits, int32_t* work, hipStream_t st) {
   // Short rows (up to 6 chunks: at most 64 VGPRs per thread) leave room for a second workgroup on every compute
@@ -1354,7 +1405,7 @@ static void launch_regs(const void* logits, int64_t T, int V, int64_t stride, co
 // Rows of more than kMaxRegChunks chunks: registers + LDS + streamed tail (see k_fused_regs, EXT).
 constexpr int kMaxExtChunks = kExtRegChunks + kExtLdsChunks + kExtTailChunks;
 
-template <int DT, bool SHIFT>
+template <int DT, int SHIFT>
 static bool launch_regs_ext(int nch, const void* logits, int64_t T, int V, int64_t stride, const int64_t* labels,
                             float inv_t, const FusedTokenArgs& a, void* dlogits, int32_t* work, hipStream_t st) {
   static const bool ok =
@@ -1386,14 +1437,31 @@ static bool wants_shift(int nch, int V, int64_t stride) {
   return nch >= kShiftMinChunks && V % 8192 == 0 && stride % 8192 == 0;
 }
 
+// A shift of the row's own (SHIFT == 2) for rows that are not a whole number of KB apart (from kShiftMinChunks chunks
+// on: +1 point at V = 151 936, nothing or a loss when the rows already start on 1 KB boundaries), and for any rows
+// that are not a whole number of 128-byte lines apart (+3.5 to +10 points: V = 50 272, 50 280, 65 544, 163 848).
+static bool wants_row_shift(int nch, int64_t stride) {
+  const int64_t step = stride * 2;
+  return (nch >= kShiftMinChunks && step % 1024 != 0) || step % 128 != 0;
+}
+
 template <int DT>
 static bool dispatch_regs(int nch, const void* logits, int64_t T, int V, int64_t stride, const int64_t* labels,
                           float inv_t, const FusedTokenArgs& a, void* dlogits, int32_t* work, hipStream_t st) {
   if (wants_shift(nch, V, stride)) {
     switch (nch) {
 #define AA_CASE(N) \
-  case N: launch_regs<DT, N, true>(logits, T, V, stride, labels, inv_t, a, dlogits, work, st); return true;
+  case N: launch_regs<DT, N, 1>(logits, T, V, stride, labels, inv_t, a, dlogits, work, st); return true;
       AA_CASE(10) AA_CASE(11) AA_CASE(12) AA_CASE(13) AA_CASE(14) AA_CASE(15)
+      AA_CASE(16) AA_CASE(17) AA_CASE(18) AA_CASE(19) AA_CASE(20) AA_CASE(21)
+#undef AA_CASE
+      default: break;
+    }
+  } else if (wants_row_shift(nch, stride)) {
+    switch (nch) {
+#define AA_CASE(N) \
+  case N: launch_regs<DT, N, 2>(logits, T, V, stride, labels, inv_t, a, dlogits, work, st); return true;
+      AA_CASE(3) AA_CASE(4) AA_CASE(5) AA_CASE(6) AA_CASE(7) AA_CASE(8) AA_CASE(9) AA_CASE(10) AA_CASE(11) AA_CASE(12) AA_CASE(13) AA_CASE(14) AA_CASE(15)
       AA_CASE(16) AA_CASE(17) AA_CASE(18) AA_CASE(19) AA_CASE(20) AA_CASE(21)
 #undef AA_CASE
       default: break;
@@ -1528,13 +1596,13 @@ extern "C" int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int
                : dispatch_regs<AA_F16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st);
     else
       ok = wants_shift(nch, (int)V, row_stride)
-               ? ((dtype == AA_BF16) ? launch_regs_ext<AA_BF16, true>(nch, logits, T, (int)V, row_stride, labels,
+               ? ((dtype == AA_BF16) ? launch_regs_ext<AA_BF16, 1>(nch, logits, T, (int)V, row_stride, labels,
                                                                      inv_temperature, a, dlogits, work, st)
-                                     : launch_regs_ext<AA_F16, true>(nch, logits, T, (int)V, row_stride, labels,
+                                     : launch_regs_ext<AA_F16, 1>(nch, logits, T, (int)V, row_stride, labels,
                                                                     inv_temperature, a, dlogits, work, st))
-               : ((dtype == AA_BF16) ? launch_regs_ext<AA_BF16, false>(nch, logits, T, (int)V, row_stride, labels,
+               : ((dtype == AA_BF16) ? launch_regs_ext<AA_BF16, 0>(nch, logits, T, (int)V, row_stride, labels,
                                                                       inv_temperature, a, dlogits, work, st)
-                                     : launch_regs_ext<AA_F16, false>(nch, logits, T, (int)V, row_stride, labels,
+                                     : launch_regs_ext<AA_F16, 0>(nch, logits, T, (int)V, row_stride, labels,
                                                                      inv_temperature, a, dlogits, work, st));
     if (ok) return launch_status();
   }

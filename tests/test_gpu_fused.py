@@ -591,17 +591,22 @@ def test_supervised_gradient_written_over_the_logits(device):
     (163840, torch.bfloat16),    # 20 chunks
     (180224, torch.bfloat16),    # 22 chunks: 21 in registers, one in LDS
     (262144, torch.bfloat16),    # 32 chunks: registers, LDS and the tail that is read twice
+    (151936, torch.bfloat16),    # rows 296.75 KB apart: every row gets a shift of its own (0 to 2 KB)
+    (50280, torch.float16),      # 7 chunks (two workgroups per compute unit), rows not a whole number of lines apart
+    (100360, torch.bfloat16),    # 13 chunks, the same
 ])
-def test_rows_of_whole_chunks_on_the_shifted_grid(device, V, dtype):
+def test_rows_on_a_shifted_chunk_grid(device, V, dtype):
     """Rows of whole 8192-value chunks at a stride of whole chunks are walked on a chunk grid laid 1 KB back (the
-    first 64 threads of chunk 0 hold the last 512 values of the row).  Labels in every place that moves: the first and
-    last 512 values, both sides of the first chunk borders, the last value.  Against the oracle, in place, and against
-    the same rows at a stride that keeps the plain grid."""
-    lengths = synth.lengths_uniform(6, 6, 12, seed=V)
+    first 64 threads of chunk 0 hold the last 512 values of the row); rows that are not a whole number of KB (or of
+    128-byte lines) apart on a grid laid back by an amount of the row's own (up to 2 KB: the first threads of chunk 0
+    hold up to 1016 values from the end of the row).  Labels in every place that moves: the first and last 1024 values,
+    both sides of the first chunk borders, the last value.  Against the oracle, in place, and against the same rows at
+    another stride (another grid)."""
+    lengths = synth.lengths_uniform(6, 8, 14, seed=V)
     case = synth.make_logits_case("t", lengths, V, V, device, synth.per_sequence_normal_advantages(lengths, 3),
                                   dtype=dtype, ppo=dict(eps_clip=0.2))
-    special = [0, 7, 8, 511, 512, 7679, 7680, 8191, 8192, 8703, 8704, 16383, 16384, V - 8193, V - 8192, V - 513, V - 512,
-               V - 9, V - 8, V - 1]
+    special = [0, 7, 8, 511, 512, 1023, 1024, 7679, 7680, 8191, 8192, 8703, 8704, 16383, 16384, V - 8193, V - 8192,
+               V - 1025, V - 1024, V - 1017, V - 1016, V - 513, V - 512, V - 9, V - 8, V - 1]
     n = min(len(special), case.n_tokens)
     case.labels[:n] = torch.tensor(special[:n], device=device)
     case.loss_mask[:n] = True
@@ -615,7 +620,7 @@ def test_rows_of_whole_chunks_on_the_shifted_grid(device, V, dtype):
                                                temperature=case.temperature, inplace_backward=True, **case.ppo)
     assert torch.equal(x.detach(), got[2]) and torch.equal(l2.detach(), got[0])
     assert torch.equal(s2["logprobs"], got[1]["logprobs"]) and torch.equal(s2["entropy"], got[1]["entropy"])
-    # the same rows inside a wider array (stride V + 8: the plain grid): the same results up to the order of the sums
+    # the same rows inside a wider array (stride V + 8: another grid): the same results up to the order of the sums
     wide = torch.zeros(case.n_tokens, V + 8, dtype=dtype, device=device)
     wide[:, :V] = case.logits
     y = wide[:, :V].requires_grad_(True)
