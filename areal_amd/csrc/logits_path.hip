@@ -885,7 +885,8 @@ __device__ __forceinline__ int shifted_piece(int piece, int row_pieces) {
 // piece c * 1024 + thread - sh / 16; the threads of chunk 0 below sh / 16, whose piece would lie before the row, hold
 // its last pieces, which the plain grid's slots at and past the row's piece count would have held: those slots stay
 // empty (the same test as in the plain grid), but the descriptor no longer drops what they would store, so the last
-// chunk's store is skipped by the threads without a piece.
+// chunk's store is skipped by the threads without a piece (longer rows: the store of every chunk in LDS or in the
+// tail is).
 constexpr int kShiftTargetBytes = 1024;
 __device__ __forceinline__ int shifted_piece_by(int piece, int shift_pieces, int row_pieces) {
   if (piece < 0) return -1;
@@ -1023,7 +1024,7 @@ constexpr int kTwoPerUnitChunks = 7;  // rows this short run two workgroups per 
 // Up to kTwoPerUnitChunks chunks the kernel is compiled for 8 waves per SIMD, so that two workgroups fit on a
 // compute unit: without that request the scalar registers alone (106 per wave: 7 waves) keep the second one out.
 // SHIFT (see grad_pass): 1: the chunk grid of a row laid 1 KB back, for rows of whole chunks a whole number of chunks
-// apart; 2: laid back by an amount of the row's own (not with EXT).
+// apart; 2: laid back by an amount of the row's own.
 template <int DT, int NCH, bool EXT, bool ALIAS, int SHIFT = 0>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu((!EXT && NCH <= kTwoPerUnitChunks) ? 8 : 1)))
 void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stride_vec,
@@ -1045,7 +1046,6 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
   const int tid = threadIdx.x;
   const float c = kLog2e * inv_t;
   const int voff = tid * 16;
-  static_assert(SHIFT != 2 || !EXT, "a shift per row is written for rows that fit in registers");
   constexpr int kSh = SHIFT == 1 ? kShiftBytes : 0;  // chunks 1, 2, ... are asked for this many bytes before their place
   // SHIFT: this thread's byte offset in chunk 0 (the last pieces of the row for the first kShiftPieces threads)
   const int voff_first = tid < kShiftPieces ? voff + (nvec - kShiftPieces) * 16 : voff - kShiftBytes;
@@ -1119,7 +1119,7 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
     u32x4_t tv[kExtTailChunks];
     bool tail_ok[kExtTailChunks];
     if constexpr (EXT) {
-      rsrc_t = __builtin_amdgcn_make_buffer_rsrc((void*)(logits + t * stride_vec), 0, V * 2, kBufferFlags);
+      rsrc_t = row_rsrc((const void*)(logits + t * stride_vec), sh);
 #pragma unroll
       for (int q = 0; q < kExtTailChunks; ++q) {
         tv[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_t, voff, (tail0 + q) * kChunkBytes - kSh, 0);  // stays cached for the second read
@@ -1229,9 +1229,11 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
         }
       }
       if constexpr (EXT) {
-        // chunks past the row are dropped by the descriptor (SHIFT: the first of them would reach back into the row)
+        // chunks past the row are dropped by the descriptor (SHIFT == 1: the first of them would reach back into the
+        // row; SHIFT == 2: the descriptor ends behind the pieces that chunk 0 holds, so threads without a piece skip)
         for (int j = 0; j < n_lds + kExtTailChunks && !(SHIFT == 1 && (NCH + j) * NT >= nvec); ++j)
-          __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, voff + (NCH + j) * kChunkBytes - kSh, 0, kAuxStream);
+          if (SHIFT != 2 || (NCH + j) * NT + tid < nvec)
+            __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, voff + (NCH + j) * kChunkBytes - kSh, 0, kAuxStream);
       }
     } else if (g > 0.f) {
       grad_pass<DT, NCH, true, SHIFT>(d, g, inv_t, c, ro.lse2, y_ok ? y : -1, tid, voff, wsrc, voff_first, nvec, sh, last_ok);
@@ -1243,18 +1245,20 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
         const float lab_add = g * inv_t;
         const float kk = fast_log2(fabsf(lab_add)) - ro.lse2;
         const int yv_row = y_ok ? (int)(y >> 3) : -1;
-        const int yv = SHIFT == 1 ? shifted_piece(yv_row, nvec) : yv_row;
+        const int yv = SHIFT == 1 ? shifted_piece(yv_row, nvec) : SHIFT == 2 ? shifted_piece_by(yv_row, sh >> 4, nvec) : yv_row;
         const int y_elem = (int)(y & 7);
         for (int j = 0; j < n_lds; ++j) {
           const u32x4_t r = grad_chunk<DT>(my_lds[j * NT], c, kk, lab_add, g > 0.f, yv, y_elem, NCH + j, tid);
-          __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + (NCH + j) * kChunkBytes - kSh, 0, kAuxStream);
+          if (SHIFT != 2 || (NCH + j) * NT + tid < nvec)
+            __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + (NCH + j) * kChunkBytes - kSh, 0, kAuxStream);
         }
 #pragma unroll
         for (int q = 0; q < kExtTailChunks; ++q) {
           // SHIFT: a chunk past the row would reach back into it (the descriptor drops it otherwise)
           if (SHIFT == 1 && (tail0 + q) * NT >= nvec) continue;
           const u32x4_t r = grad_chunk<DT>(tv[q], c, kk, lab_add, g > 0.f, yv, y_elem, tail0 + q, tid);
-          __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + (tail0 + q) * kChunkBytes - kSh, 0, kAuxStream);
+          if (SHIFT != 2 || tail_ok[q])
+            __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + (tail0 + q) * kChunkBytes - kSh, 0, kAuxStream);
         }
       }
     }
@@ -1440,6 +1444,8 @@ static bool wants_shift(int nch, int V, int64_t stride) {
 // A shift of the row's own (SHIFT == 2) for rows that are not a whole number of KB apart (from kShiftMinChunks chunks
 // on: +1 point at V = 151 936, nothing or a loss when the rows already start on 1 KB boundaries), and for any rows
 // that are not a whole number of 128-byte lines apart (+3.5 to +10 points: V = 50 272, 50 280, 65 544, 163 848).
+// Rows longer than the registers hold gain the same way (V = 200 064: +0.6, 229 376 at a stride of 229 440: +1.2,
+// 180 232: +8.9, 256 000 at a stride of 256 008: +7.8).
 static bool wants_row_shift(int nch, int64_t stride) {
   const int64_t step = stride * 2;
   return (nch >= kShiftMinChunks && step % 1024 != 0) || step % 128 != 0;
@@ -1448,7 +1454,8 @@ static bool wants_row_shift(int nch, int64_t stride) {
 template <int DT>
 static bool dispatch_regs(int nch, const void* logits, int64_t T, int V, int64_t stride, const int64_t* labels,
                           float inv_t, const FusedTokenArgs& a, void* dlogits, int32_t* work, hipStream_t st) {
-  if (wants_shift(nch, V, stride)) {
+  const int mode = wants_shift(nch, V, stride) ? 1 : wants_row_shift(nch, stride) ? 2 : 0;
+  if (mode == 1) {
     switch (nch) {
 #define AA_CASE(N) \
   case N: launch_regs<DT, N, 1>(logits, T, V, stride, labels, inv_t, a, dlogits, work, st); return true;
@@ -1457,7 +1464,7 @@ static bool dispatch_regs(int nch, const void* logits, int64_t T, int V, int64_t
 #undef AA_CASE
       default: break;
     }
-  } else if (wants_row_shift(nch, stride)) {
+  } else if (mode == 2) {
     switch (nch) {
 #define AA_CASE(N) \
   case N: launch_regs<DT, N, 2>(logits, T, V, stride, labels, inv_t, a, dlogits, work, st); return true;
@@ -1594,16 +1601,13 @@ extern "C" int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int
       ok = (dtype == AA_BF16)
                ? dispatch_regs<AA_BF16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st)
                : dispatch_regs<AA_F16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st);
-    else
-      ok = wants_shift(nch, (int)V, row_stride)
-               ? ((dtype == AA_BF16) ? launch_regs_ext<AA_BF16, 1>(nch, logits, T, (int)V, row_stride, labels,
-                                                                     inv_temperature, a, dlogits, work, st)
-                                     : launch_regs_ext<AA_F16, 1>(nch, logits, T, (int)V, row_stride, labels,
-                                                                    inv_temperature, a, dlogits, work, st))
-               : ((dtype == AA_BF16) ? launch_regs_ext<AA_BF16, 0>(nch, logits, T, (int)V, row_stride, labels,
-                                                                      inv_temperature, a, dlogits, work, st)
-                                     : launch_regs_ext<AA_F16, 0>(nch, logits, T, (int)V, row_stride, labels,
-                                                                     inv_temperature, a, dlogits, work, st));
+    else {
+      const int mode = wants_shift(nch, (int)V, row_stride) ? 1 : wants_row_shift(nch, row_stride) ? 2 : 0;
+#define AA_EXT(DT, S) launch_regs_ext<DT, S>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st)
+      if (dtype == AA_BF16) ok = mode == 1 ? AA_EXT(AA_BF16, 1) : mode == 2 ? AA_EXT(AA_BF16, 2) : AA_EXT(AA_BF16, 0);
+      else ok = mode == 1 ? AA_EXT(AA_F16, 1) : mode == 2 ? AA_EXT(AA_F16, 2) : AA_EXT(AA_F16, 0);
+#undef AA_EXT
+    }
     if (ok) return launch_status();
   }
   if (dtype == AA_F32 && (V % 8 == 0) && (row_stride % 4 == 0) && V >= kHoldChunk && V <= ((int64_t)1 << 28) &&

@@ -594,6 +594,9 @@ def test_supervised_gradient_written_over_the_logits(device):
     (151936, torch.bfloat16),    # rows 296.75 KB apart: every row gets a shift of its own (0 to 2 KB)
     (50280, torch.float16),      # 7 chunks (two workgroups per compute unit), rows not a whole number of lines apart
     (100360, torch.bfloat16),    # 13 chunks, the same
+    (200064, torch.bfloat16),    # 25 chunks (registers, LDS), rows 390.75 KB apart: a shift per row
+    (180232, torch.float16),     # 23 chunks, rows not a whole number of lines apart
+    (250888, torch.bfloat16),    # 31 chunks (registers, LDS and the tail that is read twice), the same
 ])
 def test_rows_on_a_shifted_chunk_grid(device, V, dtype):
     """Rows of whole 8192-value chunks at a stride of whole chunks are walked on a chunk grid laid 1 KB back (the
@@ -633,3 +636,42 @@ def test_rows_on_a_shifted_chunk_grid(device, V, dtype):
     step = float(got[2].float().abs().max()) * (2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11)
     assert float((y.grad.float() - got[2].float()).abs().max()) <= step
     assert float((y.grad == got[2]).float().mean()) > 0.999
+
+
+@pytest.mark.parametrize("V,wide_V,dtype", [
+    (100360, 100864, torch.bfloat16),   # 13 chunks in registers
+    (180232, 180736, torch.float16),    # 23 chunks: registers and LDS
+    (250888, 251392, torch.bfloat16),   # 31 chunks: registers, LDS and the tail that is read twice
+])
+def test_shift_changes_from_row_to_row_of_a_workgroup(device, V, wide_V, dtype):
+    """More rows than workgroups: a workgroup goes from row to row, each with a shift of its own.  Against the same
+    rows a whole number of KB apart (inside a wider array), which are walked on the plain grid: the same results up
+    to the order of the sums.  Masked rows (zero gradient rows) among them."""
+    T = 700
+    lengths = [T]
+    case = synth.make_logits_case("t", lengths, V, V, device, synth.per_sequence_normal_advantages(lengths, 5),
+                                  dtype=dtype, ppo=dict(eps_clip=0.2))
+    case.labels[:4] = torch.tensor([0, V - 1, V - 1017, 8192], device=device)
+    case.labels[-4:] = torch.tensor([V - 8, 1023, V - 513, 7], device=device)
+    case.loss_mask[:4] = True
+    case.loss_mask[-4:] = True
+    _finish_case(case)
+    got = _fused_step(case)
+    assert (wide_V * case.logits.element_size()) % 1024 == 0
+    wide = torch.zeros(T, wide_V, dtype=dtype, device=device)
+    wide[:, :V] = case.logits
+    y = wide[:, :V].requires_grad_(True)
+    l3, s3 = areal_amd.fused_logprobs_ppo_loss(y, case.labels, case.prox_logp, case.old_logp, case.advantages,
+                                               loss_mask=case.loss_mask, cu_seqlens=case.cu_seqlens,
+                                               temperature=case.temperature, **case.ppo)
+    l3.backward()
+    assert float((s3["logprobs"] - got[1]["logprobs"]).abs().max()) < 1e-5
+    assert float((s3["entropy"] - got[1]["entropy"]).abs().max()) < 1e-5
+    assert float(l3.detach()) == pytest.approx(float(got[0]), rel=1e-5)
+    step = float(got[2].float().abs().max()) * (2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11)
+    assert float((y.grad.float() - got[2].float()).abs().max()) <= step
+    assert float((y.grad == got[2]).float().mean()) > 0.999
+    assert bool((wide[:, V:] == 0).all())
+    masked = ~case.loss_mask
+    assert bool(masked.any()) and bool((got[2][masked] == 0).all())
+
