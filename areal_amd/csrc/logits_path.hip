@@ -894,17 +894,48 @@ __device__ __forceinline__ int shifted_piece_by(int piece, int shift_pieces, int
   return q < row_pieces ? q : q - row_pieces;
 }
 
+// SHIFT == 3 (rows that start at any even address: V or the stride not a multiple of 8 values, or arrays that do not
+// start on a 16-byte boundary): the grid of SHIFT == 2 laid over the 16-byte pieces of memory that hold the row.  The
+// first of them may hold values of the row before (`head` values), the last one values of the row after; both are
+// pieces of chunk 0 (the grid is always laid back by at least one piece: the last piece goes to the thread before the
+// one that holds the first).  What does not belong to the row is replaced by a value of the row when the piece
+// arrives (the extrema keep, the sums are corrected by the thread), and these two threads store their values of the
+// gradient one by one.
+struct RowEdge {
+  int lo, hi;  // this thread's piece of chunk 0 holds values lo .. hi - 1 of the row's (0, 8 for every thread but two)
+};
+__device__ __forceinline__ uint32_t patch_edge(u32x4_t& v, RowEdge e) {
+  const uint32_t fill = e.lo > 0 ? (v[3] >> 16) : (v[0] & 0xffffu);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    uint32_t w = v[q];
+    if (2 * q < e.lo || 2 * q >= e.hi) w = (w & 0xffff0000u) | fill;
+    if (2 * q + 1 < e.lo || 2 * q + 1 >= e.hi) w = (w & 0xffffu) | (fill << 16);
+    v[q] = w;
+  }
+  return fill;
+}
+__device__ __forceinline__ void store_edge(u32x4_t r, __amdgpu_buffer_rsrc_t wsrc, int off, RowEdge e) {
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    const uint32_t w = r[q >> 1];
+    if (q >= e.lo && q < e.hi)
+      __builtin_amdgcn_raw_buffer_store_b16((short)((q & 1) ? (w >> 16) : (w & 0xffffu)), wsrc, off + 2 * q, 0, kAuxStream);
+  }
+}
+
 template <int DT, int NCH, bool G_POSITIVE, int SHIFT = 0>
 __device__ __forceinline__ void grad_pass(const u32x4_t (&d)[NCH], float g, float inv_t, float c, float lse2,
                                           int64_t y, int tid, int voff, __amdgpu_buffer_rsrc_t wsrc, int voff_first = 0,
-                                          int row_pieces = 0, int sh = 0, bool last_ok = true) {
+                                          int row_pieces = 0, int sh = 0, bool last_ok = true, int head = 0,
+                                          RowEdge edge = RowEdge{0, 8}) {
   constexpr int NT = 1024;
   constexpr int kChunkBytes = NT * 16;
   const float lab_add = g * inv_t;
   const float kk = fast_log2(fabsf(lab_add)) - lse2;
-  int yv = y >= 0 ? (int)(y >> 3) : -1;
+  int yv = y >= 0 ? (int)((y + head) >> 3) : -1;
   if constexpr (SHIFT == 1) yv = shifted_piece(yv, row_pieces);
-  if constexpr (SHIFT == 2) yv = shifted_piece_by(yv, sh >> 4, row_pieces);
+  if constexpr (SHIFT == 2 || SHIFT == 3) yv = shifted_piece_by(yv, sh >> 4, row_pieces);
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     float o[8];
@@ -916,7 +947,7 @@ __device__ __forceinline__ void grad_pass(const u32x4_t (&d)[NCH], float g, floa
       o[2 * q + 1] = G_POSITIVE ? -e1 : e1;
     }
     if (yv - i * NT == tid) {  // uniform left side: no per-chunk index registers
-      const int e = (int)(y & 7);
+      const int e = (int)((y + head) & 7);
 #pragma unroll
       for (int q = 0; q < 8; ++q)
         if (q == e) o[q] += lab_add;
@@ -926,10 +957,12 @@ __device__ __forceinline__ void grad_pass(const u32x4_t (&d)[NCH], float g, floa
     r[1] = Elem<DT>::pack(o[2], o[3]);
     r[2] = Elem<DT>::pack(o[4], o[5]);
     r[3] = Elem<DT>::pack(o[6], o[7]);
-    if constexpr (SHIFT == 2) {
-      if (i == 0)
-        __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + (voff < sh ? row_pieces * 16 : 0), 0, kAuxStream);
-      else if (i < NCH - 1 || last_ok)
+    if constexpr (SHIFT == 2 || SHIFT == 3) {
+      if (i == 0) {
+        const int off = voff + (voff < sh ? row_pieces * 16 : 0);
+        if (SHIFT == 3 && edge.hi - edge.lo != 8) store_edge(r, wsrc, off, edge);
+        else __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, off, 0, kAuxStream);
+      } else if (i < NCH - 1 || last_ok)
         __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + i * kChunkBytes, 0, kAuxStream);
     } else if (SHIFT == 1 && i == 0) {
       __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff_first, 0, kAuxStream);
@@ -1042,7 +1075,8 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
   __shared__ float smem[(NT / kWave) * 5];
   __shared__ int64_t next_row[2];  // written at the top of a row, read behind its barriers: two slots, no reuse race
   int slot = 0;
-  const int nvec = V >> 3;
+  constexpr bool kRowShift = SHIFT == 2 || SHIFT == 3;
+  int nvec = V >> 3;  // 16-byte pieces of a row (SHIFT == 3: of the memory that holds it, set row by row)
   const int tid = threadIdx.x;
   const float c = kLog2e * inv_t;
   const int voff = tid * 16;
@@ -1051,7 +1085,7 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
   const int voff_first = tid < kShiftPieces ? voff + (nvec - kShiftPieces) * 16 : voff - kShiftBytes;
   // EXT: every register chunk is full; SHIFT: the row is whole chunks (the comparison stays, so that the passes over
   // the row keep the schedule of the other instantiations)
-  const bool last_ok = EXT || (NCH - 1) * NT + (SHIFT == 1 ? (tid & 1) : tid) < nvec;
+  bool last_ok = EXT || (NCH - 1) * NT + (SHIFT == 1 ? (tid & 1) : tid) < nvec;
   // SHIFT == 2: the shift of a row in bytes (uniform), and the descriptor of a row that starts that far before it
   // It is taken from where the row starts inside the array (row index x stride), as if the array started on a 4 KB
   // boundary, which large allocations do: results then do not depend on where an array lies.  The smallest shift that
@@ -1064,8 +1098,46 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
       return __builtin_amdgcn_readfirstlane((off >> 10) == 0 ? a + 1024 : a);
     }
   };
+  // SHIFT == 3: stride_vec is the stride in values; a row starts `head` values into its first piece.  The place of a
+  // row is taken from its index and from where the arrays start inside a 16-byte piece (both arrays the same).
+  int head = 0;
+  RowEdge edge{0, 8};
+  const uint32_t base_mis = SHIFT == 3 ? (uint32_t)((uintptr_t)logits & 15) : 0u;
+  auto set_row = [&](int64_t row_index) -> int {  // returns the shift in bytes (a multiple of 16); sets head, nvec, ...
+    if constexpr (SHIFT != 3) return row_shift(row_index);
+    else {
+      const uint32_t off = ((uint32_t)row_index * (uint32_t)((stride_vec * 2) & 4095) + base_mis) & 4095u;
+      const int h = (int)(off & 15u), off16 = (int)(off & ~15u);
+      const int a = off16 & 1023, k = off16 >> 10;
+      int s16 = k == 0 ? a + 1024 : a;
+      if (s16 == 0) s16 = k == 1 ? 2048 : 1024;
+      s16 = __builtin_amdgcn_readfirstlane(s16);
+      head = __builtin_amdgcn_readfirstlane(h >> 1);
+      nvec = __builtin_amdgcn_readfirstlane((h + V * 2 + 15) >> 4);
+      last_ok = EXT || (NCH - 1) * NT + tid < nvec;
+      const int p0 = s16 >> 4;
+      edge.lo = tid == p0 ? head : 0;
+      edge.hi = tid == p0 - 1 ? ((h + V * 2 - (nvec - 1) * 16) >> 1) : 8;
+      return s16;
+    }
+  };
+  auto row_in = [&](int64_t row_index) -> const char* {
+    return (const char*)logits + row_index * stride_vec * (SHIFT == 3 ? 2 : 16);
+  };
+  auto row_out = [&](int64_t row_index) -> const char* {
+    return (const char*)dlogits + row_index * stride_vec * (SHIFT == 3 ? 2 : 16);
+  };
+  // the descriptor of a row on a grid laid back by sh bytes (SHIFT == 3: and by the row's place in its first piece; it
+  // ends with the last piece that holds values of the row)
   auto row_rsrc = [&](const void* row, int sh) {
-    return __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)row - sh), 0, V * 2 + sh, kBufferFlags);
+    if constexpr (SHIFT == 3)
+      return __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)row - sh - head * 2), 0, sh + nvec * 16, kBufferFlags);
+    else
+      return __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)row - sh), 0, V * 2 + sh, kBufferFlags);
+  };
+  auto label_bits = [&](const void* row, int64_t i) -> uint32_t {
+    if constexpr (SHIFT == 3) return ((const uint16_t*)row)[i];
+    else return load_u16_uniform(row, i);
   };
   float fn, gscale;
   load_loss_scale(a, fn, gscale);
@@ -1080,16 +1152,16 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
   };
   // load of register chunk i (a compile-time slot)
   auto load_reg = [&](const __amdgpu_buffer_rsrc_t rsrc, int i, int sh) {
-    if (SHIFT == 2 && i == 0)
+    if (kRowShift && i == 0)
       return __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff + (voff < sh ? nvec * 16 : 0), 0, kAuxStream);
     if (SHIFT == 1 && i == 0) return __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff_first, 0, kAuxStream);
     return __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, i * kChunkBytes - kSh, kAuxStream);
   };
 
   int64_t t = blockIdx.x;  // the host launches at most T workgroups
-  const uint4* src = logits + t * stride_vec;
+  const char* src = row_in(t);
   u32x4_t d[NCH];
-  int sh = row_shift(t);
+  int sh = set_row(t);
   {
     const __amdgpu_buffer_rsrc_t rsrc = row_rsrc(src, sh);
 #pragma unroll
@@ -1098,7 +1170,7 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
   }
   int64_t y = labels[t];
   bool y_ok = (y >= 0) && (y < V);
-  uint32_t xy_raw = load_u16_uniform(src, y_ok ? y : 0);
+  uint32_t xy_raw = label_bits(src, y_ok ? y : 0);
   TokenIn tin = load_token_in_ro(in_prox, in_adv, in_mask32, mask_mis, in_bw, has_w, a.T_active, t);
 
   for (;;) {
@@ -1113,13 +1185,18 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
     // minimum, otherwise the smallest unsigned pattern is.
     s16x2_t smax = {-32768, -32768}, smin = {32767, 32767};
     u16x2_t umax = {0, 0}, umin = {65535, 65535};
+    // SHIFT == 3: what the first and the last piece hold of other rows is replaced by a value of this row
+    uint32_t edge_fill = 0;
+    if constexpr (SHIFT == 3) {
+      if (edge.hi - edge.lo != 8) edge_fill = patch_edge(d[0], edge);
+    }
     // EXT: the tail chunks of this row, fetched here for the statistics and once more for the gradient (lanes past
     // the row read zeros)
     __amdgpu_buffer_rsrc_t rsrc_t;
     u32x4_t tv[kExtTailChunks];
     bool tail_ok[kExtTailChunks];
     if constexpr (EXT) {
-      rsrc_t = row_rsrc((const void*)(logits + t * stride_vec), sh);
+      rsrc_t = row_rsrc((const void*)row_in(t), sh);
 #pragma unroll
       for (int q = 0; q < kExtTailChunks; ++q) {
         tv[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_t, voff, (tail0 + q) * kChunkBytes - kSh, 0);  // stays cached for the second read
@@ -1188,6 +1265,15 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
       for (int j = 0; j < n_lds; ++j)
         if ((NCH + j) * NT + tid < nvec) sum_chunk<DT>(my_lds[j * NT], c, ts.k, s, u);
     }
+    if constexpr (SHIFT == 3) {  // the values that stand in for other rows' leave the sums again
+      if (edge.hi - edge.lo != 8) {
+        const float m = (float)(8 - (edge.hi - edge.lo));
+        const float t0 = fmaf(Elem<DT>::lo(edge_fill), c, -ts.k);
+        const float e0 = fast_exp2(t0);
+        s = fmaf(-m, e0, s);
+        u = fmaf(-m, t0 * e0, u);
+      }
+    }
     ts.s = s; ts.u = u;
     keep_packed(d);
     const RowStats rs = block_stats<NT / kWave>(ts, smem);
@@ -1200,13 +1286,13 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
 
     // scalars of the next row, fetched ahead of the gradient pass
     const bool more = tn < T;
-    const uint4* src_n = logits + (more ? tn : t) * stride_vec;
+    const char* src_n = row_in(more ? tn : t);
     const int64_t y_n = more ? labels[tn] : -1;
     const bool y_ok_n = (y_n >= 0) && (y_n < V);
-    const uint32_t xy_raw_n = load_u16_uniform(src_n, y_ok_n ? y_n : 0);
+    const uint32_t xy_raw_n = label_bits(src_n, y_ok_n ? y_n : 0);
     const TokenIn tin_n = load_token_in_ro(in_prox, in_adv, in_mask32, mask_mis, in_bw, has_w, a.T_active, more ? tn : t);
 
-    const __amdgpu_buffer_rsrc_t wsrc = row_rsrc((const void*)(dlogits + t * stride_vec), sh);
+    const __amdgpu_buffer_rsrc_t wsrc = row_rsrc((const void*)row_out(t), sh);
     if constexpr (EXT) {
       if (g != 0.f) {
 #pragma unroll
@@ -1218,10 +1304,12 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
       const u32x4_t z = {0u, 0u, 0u, 0u};
 #pragma unroll
       for (int i = 0; i < NCH; ++i) {
-        if constexpr (SHIFT == 2) {
-          if (i == 0)
-            __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, voff + (voff < sh ? nvec * 16 : 0), 0, kAuxStream);
-          else if (i < NCH - 1 || last_ok)
+        if constexpr (kRowShift) {
+          if (i == 0) {
+            const int off = voff + (voff < sh ? nvec * 16 : 0);
+            if (SHIFT == 3 && edge.hi - edge.lo != 8) store_edge(z, wsrc, off, edge);
+            else __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, off, 0, kAuxStream);
+          } else if (i < NCH - 1 || last_ok)
             __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, voff + i * kChunkBytes, 0, kAuxStream);
         } else {
           __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, (SHIFT == 1 && i == 0) ? voff_first : voff + i * kChunkBytes - kSh,
@@ -1230,26 +1318,26 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
       }
       if constexpr (EXT) {
         // chunks past the row are dropped by the descriptor (SHIFT == 1: the first of them would reach back into the
-        // row; SHIFT == 2: the descriptor ends behind the pieces that chunk 0 holds, so threads without a piece skip)
+        // row; a shift per row: the descriptor ends behind the pieces that chunk 0 holds, so threads without a piece skip)
         for (int j = 0; j < n_lds + kExtTailChunks && !(SHIFT == 1 && (NCH + j) * NT >= nvec); ++j)
-          if (SHIFT != 2 || (NCH + j) * NT + tid < nvec)
+          if (!kRowShift || (NCH + j) * NT + tid < nvec)
             __builtin_amdgcn_raw_buffer_store_b128(z, wsrc, voff + (NCH + j) * kChunkBytes - kSh, 0, kAuxStream);
       }
     } else if (g > 0.f) {
-      grad_pass<DT, NCH, true, SHIFT>(d, g, inv_t, c, ro.lse2, y_ok ? y : -1, tid, voff, wsrc, voff_first, nvec, sh, last_ok);
+      grad_pass<DT, NCH, true, SHIFT>(d, g, inv_t, c, ro.lse2, y_ok ? y : -1, tid, voff, wsrc, voff_first, nvec, sh, last_ok, head, edge);
     } else {
-      grad_pass<DT, NCH, false, SHIFT>(d, g, inv_t, c, ro.lse2, y_ok ? y : -1, tid, voff, wsrc, voff_first, nvec, sh, last_ok);
+      grad_pass<DT, NCH, false, SHIFT>(d, g, inv_t, c, ro.lse2, y_ok ? y : -1, tid, voff, wsrc, voff_first, nvec, sh, last_ok, head, edge);
     }
     if constexpr (EXT) {
       if (g != 0.f) {
         const float lab_add = g * inv_t;
         const float kk = fast_log2(fabsf(lab_add)) - ro.lse2;
-        const int yv_row = y_ok ? (int)(y >> 3) : -1;
-        const int yv = SHIFT == 1 ? shifted_piece(yv_row, nvec) : SHIFT == 2 ? shifted_piece_by(yv_row, sh >> 4, nvec) : yv_row;
-        const int y_elem = (int)(y & 7);
+        const int yv_row = y_ok ? (int)((y + head) >> 3) : -1;
+        const int yv = SHIFT == 1 ? shifted_piece(yv_row, nvec) : kRowShift ? shifted_piece_by(yv_row, sh >> 4, nvec) : yv_row;
+        const int y_elem = (int)((y + head) & 7);
         for (int j = 0; j < n_lds; ++j) {
           const u32x4_t r = grad_chunk<DT>(my_lds[j * NT], c, kk, lab_add, g > 0.f, yv, y_elem, NCH + j, tid);
-          if (SHIFT != 2 || (NCH + j) * NT + tid < nvec)
+          if (!kRowShift || (NCH + j) * NT + tid < nvec)
             __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + (NCH + j) * kChunkBytes - kSh, 0, kAuxStream);
         }
 #pragma unroll
@@ -1257,7 +1345,7 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
           // SHIFT: a chunk past the row would reach back into it (the descriptor drops it otherwise)
           if (SHIFT == 1 && (tail0 + q) * NT >= nvec) continue;
           const u32x4_t r = grad_chunk<DT>(tv[q], c, kk, lab_add, g > 0.f, yv, y_elem, tail0 + q, tid);
-          if (SHIFT != 2 || tail_ok[q])
+          if (!kRowShift || tail_ok[q])
             __builtin_amdgcn_raw_buffer_store_b128(r, wsrc, voff + (tail0 + q) * kChunkBytes - kSh, 0, kAuxStream);
         }
       }
@@ -1266,7 +1354,7 @@ void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stri
     // All stores of this row are issued before the loads of the next one:
     // alternating them chunk by chunk costs bandwidth on this memory system.
     {
-      sh = row_shift(more ? tn : t);
+      sh = set_row(more ? tn : t);
       const __amdgpu_buffer_rsrc_t rsrc_n = row_rsrc(src_n, sh);
 #pragma unroll
       for (int i = 0; i < NCH; ++i) d[i] = load_reg(rsrc_n, i, sh);
@@ -1398,11 +1486,11 @@ static void launch_regs(const void* logits, int64_t T, int V, int64_t stride, co
   const uintptr_t mask_addr = (uintptr_t)a.mask_eff;
   if (dlogits == logits)
     hipLaunchKernelGGL((k_fused_regs<DT, NCH, false, true, SHIFT>), dim3((unsigned)wgs), dim3(1024), 0, st, (const uint4*)logits, V,
-                       stride >> 3, labels, inv_t, a.prox_logp, a.adv, (const uint32_t*)(mask_addr & ~(uintptr_t)3),
+                       SHIFT == 3 ? stride : stride >> 3, labels, inv_t, a.prox_logp, a.adv, (const uint32_t*)(mask_addr & ~(uintptr_t)3),
                        (unsigned)(mask_addr & 3), a.behave_w, a, (uint4*)dlogits, T, work, 0);
   else
     hipLaunchKernelGGL((k_fused_regs<DT, NCH, false, false, SHIFT>), dim3((unsigned)wgs), dim3(1024), 0, st, (const uint4*)logits, V,
-                       stride >> 3, labels, inv_t, a.prox_logp, a.adv, (const uint32_t*)(mask_addr & ~(uintptr_t)3),
+                       SHIFT == 3 ? stride : stride >> 3, labels, inv_t, a.prox_logp, a.adv, (const uint32_t*)(mask_addr & ~(uintptr_t)3),
                        (unsigned)(mask_addr & 3), a.behave_w, a, (uint4*)dlogits, T, work, 0);
 }
 
@@ -1423,12 +1511,12 @@ static bool launch_regs_ext(int nch, const void* logits, int64_t T, int V, int64
   const uintptr_t mask_addr = (uintptr_t)a.mask_eff;
   if (dlogits == logits)
     hipLaunchKernelGGL((k_fused_regs<DT, kExtRegChunks, true, true, SHIFT>), dim3((unsigned)wgs), dim3(1024), n_lds * 16384, st,
-                       (const uint4*)logits, V, stride >> 3, labels, inv_t, a.prox_logp, a.adv,
+                       (const uint4*)logits, V, SHIFT == 3 ? stride : stride >> 3, labels, inv_t, a.prox_logp, a.adv,
                        (const uint32_t*)(mask_addr & ~(uintptr_t)3), (unsigned)(mask_addr & 3), a.behave_w, a,
                        (uint4*)dlogits, T, work, n_lds);
   else
     hipLaunchKernelGGL((k_fused_regs<DT, kExtRegChunks, true, false, SHIFT>), dim3((unsigned)wgs), dim3(1024), n_lds * 16384, st,
-                       (const uint4*)logits, V, stride >> 3, labels, inv_t, a.prox_logp, a.adv,
+                       (const uint4*)logits, V, SHIFT == 3 ? stride : stride >> 3, labels, inv_t, a.prox_logp, a.adv,
                        (const uint32_t*)(mask_addr & ~(uintptr_t)3), (unsigned)(mask_addr & 3), a.behave_w, a,
                        (uint4*)dlogits, T, work, n_lds);
   return true;
@@ -1451,10 +1539,29 @@ static bool wants_row_shift(int nch, int64_t stride) {
   return (nch >= kShiftMinChunks && step % 1024 != 0) || step % 128 != 0;
 }
 
+// Rows that do not start on 16-byte boundaries (V or the stride not a multiple of 8 values, arrays that start inside a
+// 16-byte piece, both at the same place in it): SHIFT == 3.  The chunks are counted over the 16-byte pieces of memory
+// that hold a row: one more than the row has when it starts and ends inside a piece.
+static int any_alignment_chunks(int64_t V) { return (int)((((14 + V * 2 + 15) >> 4) + 1023) / 1024); }
+static bool wants_any_alignment(const void* logits, const void* dlogits, int64_t V, int64_t stride) {
+  const uintptr_t a = (uintptr_t)logits, b = (uintptr_t)dlogits;
+  if (V % 8 == 0 && stride % 8 == 0 && ((a | b) & 15) == 0) return false;
+  return ((a | b) & 1) == 0 && ((a ^ b) & 15) == 0;
+}
+
 template <int DT>
-static bool dispatch_regs(int nch, const void* logits, int64_t T, int V, int64_t stride, const int64_t* labels,
+static bool dispatch_regs(int mode, int nch, const void* logits, int64_t T, int V, int64_t stride, const int64_t* labels,
                           float inv_t, const FusedTokenArgs& a, void* dlogits, int32_t* work, hipStream_t st) {
-  const int mode = wants_shift(nch, V, stride) ? 1 : wants_row_shift(nch, stride) ? 2 : 0;
+  if (mode == 3) {
+    switch (nch) {
+#define AA_CASE(N) \
+  case N: launch_regs<DT, N, 3>(logits, T, V, stride, labels, inv_t, a, dlogits, work, st); return true;
+      AA_CASE(3) AA_CASE(4) AA_CASE(5) AA_CASE(6) AA_CASE(7) AA_CASE(8) AA_CASE(9) AA_CASE(10) AA_CASE(11) AA_CASE(12) AA_CASE(13) AA_CASE(14) AA_CASE(15)
+      AA_CASE(16) AA_CASE(17) AA_CASE(18) AA_CASE(19) AA_CASE(20) AA_CASE(21)
+#undef AA_CASE
+      default: return false;
+    }
+  }
   if (mode == 1) {
     switch (nch) {
 #define AA_CASE(N) \
@@ -1592,20 +1699,25 @@ extern "C" int aa_logits_ppo_fused(const void* logits, int dtype, int64_t T, int
   a.stat_loss = stat_loss; a.ratio = ratio; a.flags = flags;
   a.P = *params; a.T_active = T_active;
 
-  const bool fast = (dtype != AA_F32) && (V % 8 == 0) && (row_stride % 8 == 0) && (((uintptr_t)logits & 15) == 0) &&
-                    (((uintptr_t)dlogits & 15) == 0) && (V > kTwoPassMaxV) && (V <= kMaxExtChunks * 8192) && (T_active > 0);
+  const bool any_alignment = wants_any_alignment(logits, dlogits, V, row_stride);
+  const bool fast = (dtype != AA_F32) && (V > kTwoPassMaxV) && (T_active > 0) &&
+                    (any_alignment ? any_alignment_chunks(V) <= kMaxExtChunks
+                                   : (V % 8 == 0) && (row_stride % 8 == 0) && (((uintptr_t)logits & 15) == 0) &&
+                                         (((uintptr_t)dlogits & 15) == 0) && (V <= kMaxExtChunks * 8192));
   if (fast) {
-    const int nch = (int)((V / 8 + 1023) / 1024);
+    const int nch = any_alignment ? any_alignment_chunks(V) : (int)((V / 8 + 1023) / 1024);
+    const int mode = any_alignment ? 3 : wants_shift(nch, (int)V, row_stride) ? 1 : wants_row_shift(nch, row_stride) ? 2 : 0;
     bool ok;
-    if (nch <= kMaxRegChunks)
-      ok = (dtype == AA_BF16)
-               ? dispatch_regs<AA_BF16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st)
-               : dispatch_regs<AA_F16>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st);
-    else {
-      const int mode = wants_shift(nch, (int)V, row_stride) ? 1 : wants_row_shift(nch, row_stride) ? 2 : 0;
+    if (nch <= kMaxRegChunks) {
+      ok = (dtype == AA_BF16) ? dispatch_regs<AA_BF16>(mode, nch, logits, T, (int)V, row_stride, labels, inv_temperature, a,
+                                                       dlogits, work, st)
+                              : dispatch_regs<AA_F16>(mode, nch, logits, T, (int)V, row_stride, labels, inv_temperature, a,
+                                                      dlogits, work, st);
+    } else {
 #define AA_EXT(DT, S) launch_regs_ext<DT, S>(nch, logits, T, (int)V, row_stride, labels, inv_temperature, a, dlogits, work, st)
-      if (dtype == AA_BF16) ok = mode == 1 ? AA_EXT(AA_BF16, 1) : mode == 2 ? AA_EXT(AA_BF16, 2) : AA_EXT(AA_BF16, 0);
-      else ok = mode == 1 ? AA_EXT(AA_F16, 1) : mode == 2 ? AA_EXT(AA_F16, 2) : AA_EXT(AA_F16, 0);
+#define AA_EXT_MODES(DT) (mode == 3 ? AA_EXT(DT, 3) : mode == 2 ? AA_EXT(DT, 2) : mode == 1 ? AA_EXT(DT, 1) : AA_EXT(DT, 0))
+      ok = (dtype == AA_BF16) ? AA_EXT_MODES(AA_BF16) : AA_EXT_MODES(AA_F16);
+#undef AA_EXT_MODES
 #undef AA_EXT
     }
     if (ok) return launch_status();

@@ -74,6 +74,18 @@ def _rows(logits: torch.Tensor) -> tuple[torch.Tensor, int, int, int]:
     return x, T, V, stride
 
 
+def _empty_rows_like(logits2d: torch.Tensor, stride: int) -> torch.Tensor:
+    """An uninitialised [T, V] array for the gradient of ``logits2d``: the same row stride, and the same place inside
+    a 16-byte piece of memory, so that the kernels walk both arrays alike (the fused kernel's fast path for rows that
+    do not start on 16-byte boundaries asks for that)."""
+    T, V = logits2d.shape
+    lead = (logits2d.data_ptr() % 16) // logits2d.element_size()
+    if stride == V and lead == 0:
+        return torch.empty_like(logits2d, memory_format=torch.contiguous_format)
+    flat = torch.empty(lead + (T - 1) * stride + V, dtype=logits2d.dtype, device=logits2d.device)
+    return flat.as_strided((T, V), (stride, 1), lead)
+
+
 def _check_tp(tp_group: Any) -> None:
     if tp_group is not None:
         import torch.distributed as dist
@@ -161,10 +173,8 @@ class _LogprobsEntropy(torch.autograd.Function):
             # the gradient takes the place of the logits (the kernel reads an element before it writes it); the version
             # bump below makes any other operation that kept the logits for its own backward fail loudly
             dlogits = logits2d.detach()
-        elif ctx.stride == V:
-            dlogits = torch.empty_like(logits2d, memory_format=torch.contiguous_format)
-        else:  # keep the row stride of the input so that both buffers are walked alike
-            dlogits = torch.empty_strided((T, V), (ctx.stride, 1), dtype=logits2d.dtype, device=dev)
+        else:  # the row stride of the input, so that both buffers are walked alike
+            dlogits = _empty_rows_like(logits2d, ctx.stride)
         with torch.cuda.device(dev):
             N.check(
                 lib.aa_logits_bwd(
@@ -600,10 +610,8 @@ class _FusedLogitsPpo(torch.autograd.Function):
             # the gradient takes the place of the logits: every kernel reads an element for the last time before it
             # writes it, so the two arrays of the C entry point may be one
             dlogits = logits2d.detach()
-        elif stride == V:
-            dlogits = torch.empty_like(logits2d, memory_format=torch.contiguous_format)
         else:
-            dlogits = torch.empty_strided((T, V), (stride, 1), dtype=logits2d.dtype, device=dev)
+            dlogits = _empty_rows_like(logits2d, stride)
         with torch.cuda.device(dev):
             st = _stream(dev)
             N.check(

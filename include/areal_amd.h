@@ -152,6 +152,13 @@ int aa_logits_bwd(const void* logits, int dtype, int64_t T, int64_t V,
  *   assignment) and leaves them zero on exit, so one zeroed buffer serves
  *   every launch on a stream.  Launches that may run concurrently need
  *   separate buffers.
+ * Layout: any V, any row_stride >= V, logits and dlogits at any address that
+ *   their element size divides.  16-bit rows of 16 385 to 262 136 values are
+ *   read once and held in registers whatever their alignment, provided that
+ *   logits and dlogits start at the same offset inside a 16-byte piece of
+ *   memory (both on a 16-byte boundary, the usual case, or both k bytes past
+ *   one); otherwise the rows that are not on 16-byte boundaries are read
+ *   twice.
  * AA_F32 logits with V % 8 == 0 and more than 114 688 values per row: the row
  *   is kept on the chip between its read and the write of its gradient in 24
  *   bits per value (a 608 KB row of V = 151 936 does not fit the register file

@@ -675,3 +675,62 @@ def test_shift_changes_from_row_to_row_of_a_workgroup(device, V, wide_V, dtype):
     masked = ~case.loss_mask
     assert bool(masked.any()) and bool((got[2][masked] == 0).all())
 
+
+
+def _rows_in_a_flat_array(rows, stride, lead):
+    """The rows copied into a flat array filled with 7, `lead` values in and `stride` values apart."""
+    T, V = rows.shape
+    flat = torch.full((lead + T * stride + 16,), 7.0, dtype=rows.dtype, device=rows.device)
+    view = flat.as_strided((T, V), (stride, 1), lead)
+    view.copy_(rows)
+    return flat, view
+
+
+def _untouched_outside_the_rows(flat, T, V, stride, lead):
+    seen = flat.clone()
+    seen.as_strided((T, V), (stride, 1), lead).fill_(7.0)
+    return bool((seen == 7.0).all())
+
+
+@pytest.mark.parametrize("V,stride,lead,dtype,n_seq", [
+    (50257, 50257, 0, torch.bfloat16, 6),     # 7 chunks (two workgroups per compute unit), rows 2 bytes off and more
+    (32001, 32001, 3, torch.float16, 6),      # 4 chunks, the array itself 6 bytes into a 16-byte piece
+    (151643, 151643, 0, torch.bfloat16, 6),   # 19 chunks
+    (151936, 151937, 0, torch.bfloat16, 6),   # rows of whole pieces at a stride that is not
+    (151936, 151936, 1, torch.bfloat16, 6),   # an array that starts 2 bytes into a piece: every row split the same way
+    (40957, 40957, 0, torch.bfloat16, 60),    # the last chunk holds a piece only in rows that start late in theirs
+    (172031, 172031, 5, torch.float16, 40),   # registers + LDS: the chunk in LDS holds one piece, in some rows
+    (250002, 250003, 0, torch.bfloat16, 40),  # registers, LDS and the tail that is read twice; more rows than workgroups
+])
+def test_rows_at_any_alignment(device, V, stride, lead, dtype, n_seq):
+    """16-bit rows that do not start on 16-byte boundaries (V or the stride not a multiple of 8, or the array itself
+    inside a 16-byte piece) are held in registers like the others: the first and the last 16-byte piece of the memory
+    that holds a row are shared with its neighbours.  Labels at both ends of the row; against the oracle; nothing
+    outside the rows is written; and the same bits when the gradient is written over the logits."""
+    lengths = synth.lengths_uniform(n_seq, 8, 14, seed=V)
+    case = synth.make_logits_case("t", lengths, V, V, device, synth.per_sequence_normal_advantages(lengths, 3),
+                                  dtype=dtype, ppo=dict(eps_clip=0.2))
+    T = case.n_tokens
+    special = [0, 1, 6, 7, 8, 9, 1023, 1024, 8191, 8192, 16383, 16384, V - 8193, V - 8192, V - 1025, V - 1024, V - 17,
+               V - 16, V - 9, V - 8, V - 7, V - 2, V - 1]
+    n = min(len(special), T)
+    case.labels[:n] = torch.tensor(special[:n], device=device)
+    case.loss_mask[:n] = True
+    _finish_case(case)
+    flat, view = _rows_in_a_flat_array(case.logits, stride, lead)
+    x = view.detach().requires_grad_(True)
+    kw = dict(loss_mask=case.loss_mask, cu_seqlens=case.cu_seqlens, temperature=case.temperature, **case.ppo)
+    loss, stat = areal_amd.fused_logprobs_ppo_loss(x, case.labels, case.prox_logp, case.old_logp, case.advantages, **kw)
+    loss.backward()
+    assert x.grad.data_ptr() % 16 == x.data_ptr() % 16
+    got = (loss.detach(), stat, x.grad)
+    _compare(case, got, _oracle_step(case))
+    assert torch.equal(view, case.logits) and _untouched_outside_the_rows(flat, T, V, stride, lead)
+    # the gradient written over the logits: the same bits, and nothing but the rows is written
+    flat2, view2 = _rows_in_a_flat_array(case.logits, stride, lead)
+    y = view2.detach().requires_grad_(True)
+    l2, s2 = areal_amd.fused_logprobs_ppo_loss(y, case.labels, case.prox_logp, case.old_logp, case.advantages,
+                                               inplace_backward=True, **kw)
+    assert torch.equal(y.detach(), got[2]) and torch.equal(l2.detach(), got[0])
+    assert torch.equal(s2["logprobs"], stat["logprobs"]) and torch.equal(s2["entropy"], stat["entropy"])
+    assert _untouched_outside_the_rows(flat2, T, V, stride, lead)
