@@ -118,12 +118,14 @@ def test_short_rows_with_two_workgroups_per_unit(device, V, dtype):
     assert torch.equal(first[2], again[2]) and float(first[0]) == float(again[0])
 
 
-@pytest.mark.parametrize("V", [70004, 24576, 49152, 90112, 122880])
+@pytest.mark.parametrize("V", [70004, 24576, 49152, 90112, 122880, 32776, 90120, 122888, 200008])
 def test_fp32_long_rows_walked_by_large_workgroups(device, V):
     """More fp32 rows than workgroups, so every workgroup handles several rows: V = 70004 (not a multiple of 8, rows
     of 280 KB) takes the two-pass kernel with 512 walking workgroups, the others the kernel that holds the row on the
     chip with one workgroup per compute unit: in registers alone (V = 24576: up to 4 chunks, V = 49152: up to 8), in
-    registers and LDS (V = 90112), and in 24 bits per value (V = 122880)."""
+    registers and LDS (V = 90112), and in 24 bits per value (V = 122880).  The last four widths put the rows 32 bytes
+    off the 128-byte lines: their requests go out on a grid shifted per row (V = 200008: with a part of the row that is
+    read twice)."""
     lengths = synth.lengths_uniform(40, 8, 24, seed=5)            # about 640 tokens
     case = synth.make_logits_case("t", lengths, V, V, device, synth.per_sequence_normal_advantages(lengths, 3),
                                   dtype=torch.float32, ppo=dict(eps_clip=0.2))
