@@ -115,3 +115,25 @@ def test_infer_token_denominator_cases_of_the_reference():
     for data, fallback, shape in cases:
         n_tokens = infer_token_denominator(data, fallback)
         assert tuple(n_tokens.shape) == shape and n_tokens.dtype == torch.bool and bool(n_tokens.all())
+
+
+@pytest.mark.parametrize("V,stride,lead", [(50257, 50257, 0), (151936, 151936, 1), (32001, 32004, 5), (64, 64, 0),
+                                           (64, 72, 0)])
+def test_gradient_array_is_laid_out_like_the_logits(V, stride, lead):
+    """The array the fused step writes the gradient into has the row stride of the logits and starts at the same
+    offset inside a 16-byte piece of memory (the register kernel's condition for rows that are not on 16-byte
+    boundaries); rows do not overlap and nothing is shared with the logits."""
+    from areal_amd import functional as F
+
+    T = 5
+    flat = torch.zeros(lead + T * stride + 8, dtype=torch.bfloat16)
+    while flat.data_ptr() % 16:                      # a base on a 16-byte boundary, whatever the allocator gave
+        flat = flat[1:]
+    logits = flat.as_strided((T, V), (stride, 1), lead)
+    out = F._empty_rows_like(logits, stride)
+    assert out.shape == logits.shape and out.dtype == logits.dtype
+    assert out.stride(1) == 1 and (out.stride(0) == stride or T == 1)
+    assert out.data_ptr() % 16 == logits.data_ptr() % 16 == (2 * lead) % 16
+    out.fill_(1.0)
+    assert float(flat.abs().sum()) == 0.0
+    assert float(out.float().sum()) == T * V
