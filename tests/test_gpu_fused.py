@@ -78,7 +78,7 @@ def _compare(case, got, want, pad=0):
         (32768, torch.bfloat16, 8, 40),    # register-resident rows, exact multiple of the chunk size
         (8200, torch.float16, 8, 40),      # up to two chunks: the two-pass kernel
         (16392, torch.float16, 8, 40),     # 3 chunks in registers, the third almost empty
-        (50257, torch.bfloat16, 4, 20),    # generic rows (V % 8 != 0)
+        (50257, torch.bfloat16, 4, 20),    # V % 8 != 0: rows at every even address, held in registers all the same
         (4099, torch.float32, 4, 20),      # generic rows, fp32 logits
         (8192, torch.float32, 4, 12),      # fp32 rows held on the chip: exactly one register chunk
         (81928, torch.float32, 4, 12),     # registers full, one vector in LDS
@@ -736,3 +736,51 @@ def test_rows_at_any_alignment(device, V, stride, lead, dtype, n_seq):
     assert torch.equal(y.detach(), got[2]) and torch.equal(l2.detach(), got[0])
     assert torch.equal(s2["logprobs"], stat["logprobs"]) and torch.equal(s2["entropy"], stat["entropy"])
     assert _untouched_outside_the_rows(flat2, T, V, stride, lead)
+
+
+@pytest.mark.parametrize("V,dtype", [(50257, torch.bfloat16), (151643, torch.float16), (250002, torch.bfloat16)])
+def test_register_kernel_and_twice_read_kernel_agree_on_unaligned_rows(device, V, dtype):
+    """Through the C ABI: the same unaligned rows with the gradient array at the same offset inside a 16-byte piece as
+    the logits (rows held in registers) and at another offset (the kernel that reads a row twice).  The same results up
+    to the order of the sums, and neither writes outside its rows."""
+    import ctypes as C
+    from areal_amd import _native as N, functional as F
+
+    lib = N.load()
+    T = 300
+    g = torch.Generator(device=device).manual_seed(V)
+    logits = (torch.randn(T, V, device=device, generator=g) * 3).to(dtype)
+    labels = torch.randint(0, V, (T,), device=device, generator=g)
+    labels[:4] = torch.tensor([0, V - 1, 7, V - 8], device=device)
+    prox = torch.full((T,), -12.0, device=device)
+    adv = torch.randn(T, device=device, generator=g)
+    mask = (torch.rand(T, device=device, generator=g) < 0.7).to(torch.uint8)
+    mask[:4] = 1
+    counts = F._count_nonzero(mask)
+    params = F._ppo_params(0.2, None, None, False)
+    work = torch.zeros(2, dtype=torch.int32, device=device)
+    stream = torch.cuda.current_stream(device)
+    results = []
+    for lead in (0, 3):                  # values between a 16-byte boundary and the gradient array
+        flat = torch.full((lead + T * V + 16,), 7.0, dtype=dtype, device=device)
+        assert flat.data_ptr() % 16 == 0 and logits.data_ptr() % 16 == 0
+        dlogits = flat.as_strided((T, V), (V, 1), lead)
+        f32 = dict(dtype=torch.float32, device=device)
+        logp, ent, stat_loss, ratio = (torch.empty(T, **f32) for _ in range(4))
+        flags = torch.empty(T, dtype=torch.uint8, device=device)
+        N.check(lib.aa_logits_ppo_fused(
+            F._ptr(logits), F._DTYPES[dtype], T, V, V, F._ptr(labels), 1.0, T, F._ptr(prox), F._ptr(adv), F._ptr(mask),
+            None, C.byref(params), F._ptr(counts), None, F._ptr(logp), F._ptr(ent), None, None, F._ptr(stat_loss),
+            F._ptr(ratio), F._ptr(flags), F._ptr(dlogits), F._ptr(work), C.c_void_p(stream.cuda_stream)),
+            "aa_logits_ppo_fused")
+        torch.cuda.synchronize()
+        assert _untouched_outside_the_rows(flat, T, V, V, lead)
+        results.append((dlogits.clone(), logp, ent, stat_loss, flags))
+    (g0, lp0, e0, sl0, f0), (g1, lp1, e1, sl1, f1) = results
+    assert float((lp0 - lp1).abs().max()) < 1e-5 and float((e0 - e1).abs().max()) < 1e-5
+    assert torch.equal(f0, f1) and torch.allclose(sl0, sl1, rtol=1e-4, atol=1e-6)
+    step = float(g1.float().abs().max()) * (2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11)
+    assert float((g0.float() - g1.float()).abs().max()) <= step
+    assert float((g0 == g1).float().mean()) > 0.999
+    assert bool((g0[mask == 0] == 0).all()) and bool((g1[mask == 0] == 0).all())
+

@@ -396,7 +396,7 @@ def _sapo_case(T_pad, T, V, seed):
 @pytest.mark.parametrize("T_pad,T,V,temperature,scale,inplace", [
     (40, 40, 9000, 1.0, None, False),       # two-pass rows
     (300, 280, 32768, 0.8, 0.37, False),    # register-resident rows, batch padding, loss scale
-    (70, 64, 50257, 1.0, None, True),       # generic rows (V % 8 != 0), gradient written over the logits
+    (70, 64, 50257, 1.0, None, True),       # rows at every even address (V % 8 != 0), gradient written over the logits
 ])
 def test_fused_logits_sapo_matches_oracle(device, T_pad, T, V, temperature, scale, inplace):
     import oracle
