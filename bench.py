@@ -67,6 +67,7 @@ LOGITS_WORKLOADS = ("cfg0", "cfg1", "cfg1-32k")
 FUSED_WORKLOADS = ("cfg2", "cfg3", "cfg4")
 ADV_WORKLOADS = ("adv", "aux")
 MFMA_WORKLOADS = ("mfma", "hbm")
+TORCH_WORKLOADS = ("torch-ops",)
 
 
 def parse_args():
@@ -74,7 +75,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="cfg1", choices=LOGITS_WORKLOADS + FUSED_WORKLOADS + ADV_WORKLOADS + MFMA_WORKLOADS)
+    ap.add_argument("--workload", default="cfg1", choices=LOGITS_WORKLOADS + FUSED_WORKLOADS + ADV_WORKLOADS + MFMA_WORKLOADS + TORCH_WORKLOADS)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--cpu-tokens", type=int, default=6144,
                     help="token sample of the CPU baseline (0 = skip); fused lm_head workloads use at most 384")
@@ -103,6 +104,9 @@ def parse_args():
     ap.add_argument("--steps-only", action="store_true",
                     help="fused lm_head workloads: launch the steps of the selected backward mode only (no stand-alone "
                          "op, no other mode), so that every dispatch a profiler sees belongs to a step")
+    ap.add_argument("--torch-compile", action="store_true",
+                    help="torch-ops only: also time the reference's two vocabulary functions under torch.compile, as "
+                         "the reference wraps them on GPUs (compilation takes a minute or two)")
     ap.add_argument("--copy-launches", type=int, default=0,
                     help="also launch the plain copy kernel this many times over the logits buffer (lm_head workloads: the weight matrix) "
                          "(the calibration point for FETCH_SIZE / WRITE_SIZE counters)")
@@ -1183,6 +1187,122 @@ def synth_lengths(total, seed):
     return synth.truncate_to_total(synth.lengths_lognormal(64, 7.5, 0.6, 128, 4096, seed), total)
 
 
+def bench_torch_ops(args, dev):
+    """What the reference itself would execute on this GPU for the two paths, restated in plain torch ops (no kernel
+    of this library runs in the timed regions): the vocabulary-sized functions exactly as
+    areal/utils/functional/vocab_parallel.py:15-81 has them (log_softmax of the fp32 cast, gather, entropy, applied in
+    chunks of 1024 rows; optionally under torch.compile, as the reference wraps them on GPUs), a token-level clipped
+    surrogate on the [T] vectors after areal/utils/functional/functional.py:429-559 (a dozen elementwise ops, well under
+    1 % of the time), autograd for the backward, and for the lm_head path the logits as torch.nn.functional.linear of
+    hidden and weight (the library GEMM) with its two backward GEMMs over all tokens.  A reported baseline beside the
+    figures of this library's paths on the same workloads; not a parity check."""
+    import torch
+
+    import areal_amd
+
+    def logp_entropy(logits, labels, temperature):
+        log_probs = torch.nn.functional.log_softmax(logits.float() / temperature, dim=-1)
+        entropy = -torch.sum(log_probs.exp() * log_probs, dim=-1)
+        return log_probs.gather(dim=-1, index=labels.unsqueeze(-1)).squeeze(-1), entropy
+
+    def chunked(fn, logits, labels, temperature, chunk=1024):
+        parts = [fn(logits[i:i + chunk], labels[i:i + chunk], temperature) for i in range(0, logits.shape[0], chunk)]
+        return torch.cat([p[0] for p in parts]), torch.cat([p[1] for p in parts])
+
+    def surrogate(logp, case, kw, cfg):
+        mask = case.loss_mask.bool()
+        behave = torch.exp(case.prox_logp - case.old_logp)
+        if cfg is not None:
+            mask = mask & (behave <= cfg.upper)
+        ratio = torch.exp(logp - case.prox_logp)
+        hi = kw.get("eps_clip_higher") or kw["eps_clip"]
+        pg = torch.max(-case.advantages * ratio, -case.advantages * ratio.clamp(1.0 - kw["eps_clip"], 1.0 + hi))
+        if kw.get("c_clip"):
+            pg = torch.where(case.advantages < 0, torch.min(pg, -case.advantages * kw["c_clip"]), pg)
+        return torch.where(mask, pg * behave, 0.0).sum() / mask.count_nonzero().clamp(min=1)
+
+    def timed(step, iters):
+        step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / iters * 1e3
+
+    variants = [("eager", logp_entropy)]
+    if args.torch_compile:
+        variants.append(("torch.compile", torch.compile(logp_entropy)))
+    out = dict(metric=METRIC, unit="tokens/s", n_gpus=1, data="synthetic", higher_is_better=True,
+               config=dict(workload="the reference's torch ops on this GPU, beside this library's paths on the same inputs"))
+    iters = max(args.steps // 4, 3)
+
+    # logits path: configs[1] cut to 32 768 tokens
+    case, desc = build_logits_case("cfg1-32k", args.seed, dev)
+    kw, cfg = ppo_kwargs(case)
+    T = case.logits.shape[0]
+    leg = dict(workload=f"{case.name}: {desc}", tokens=T)
+    for name, fn in variants:
+        def step():
+            x = case.logits.detach().requires_grad_(True)
+            logp, _ = chunked(fn, x, case.labels, case.temperature)
+            surrogate(logp, case, kw, cfg).backward()
+        try:
+            ms = timed(step, iters)
+            leg[name] = dict(ms_per_step=ms, tokens_per_s=T / (ms * 1e-3))
+        except Exception as e:  # a compiler that is not there or fails is reported, not fatal
+            leg[name] = dict(error=f"{type(e).__name__}: {str(e)[:200]}")
+    def ours():
+        x = case.logits.detach().requires_grad_(True)
+        loss, _ = areal_amd.fused_logprobs_ppo_loss(x, case.labels, case.prox_logp, case.old_logp, case.advantages,
+                                                    loss_mask=case.loss_mask, rejection_sampling=cfg,
+                                                    cu_seqlens=case.cu_seqlens, temperature=case.temperature, **kw)
+        loss.backward()
+    ms = timed(ours, max(args.steps, 10))
+    leg["this_library"] = dict(ms_per_step=ms, tokens_per_s=T / (ms * 1e-3))
+    out["logits_path"] = leg
+    del case
+    torch.cuda.empty_cache()
+
+    # lm_head path: configs[2]
+    case, desc = build_fused_case("cfg2", args.seed, dev)
+    kw, cfg = ppo_kwargs(case)
+    T = case.hidden.shape[0]
+    leg = dict(workload=f"{case.name}: {desc}", tokens=T)
+    for name, fn in variants:
+        def step():
+            h = case.hidden.detach().requires_grad_(True)
+            w = case.weight.detach().requires_grad_(True)
+            logp, _ = chunked(fn, torch.nn.functional.linear(h, w), case.labels, case.temperature)
+            surrogate(logp, case, kw, cfg).backward()
+        try:
+            ms = timed(step, iters)
+            leg[name] = dict(ms_per_step=ms, tokens_per_s=T / (ms * 1e-3))
+        except Exception as e:
+            leg[name] = dict(error=f"{type(e).__name__}: {str(e)[:200]}")
+    def gemm():
+        return torch.nn.functional.linear(case.hidden, case.weight)
+    ms = timed(gemm, max(args.steps, 10))
+    leg["library_gemm_logits_only"] = dict(ms=ms, tflops=2.0 * T * case.weight.shape[0] * case.hidden.shape[1] / (ms * 1e-3) / 1e12,
+                                           note="torch.nn.functional.linear(hidden, weight) alone: the forward product, "
+                                                "5 GB of bf16 logits written")
+    def ours2():
+        h = case.hidden.detach().requires_grad_(True)
+        w = case.weight.detach().requires_grad_(True)
+        loss, _ = areal_amd.fused_lm_head_ppo_loss(h, w, case.labels, case.prox_logp, case.old_logp, case.advantages,
+                                                   loss_mask=case.loss_mask, rejection_sampling=cfg,
+                                                   cu_seqlens=case.cu_seqlens, temperature=case.temperature, **kw)
+        loss.backward()
+    ms = timed(ours2, max(args.steps, 10))
+    leg["this_library"] = dict(ms_per_step=ms, tokens_per_s=T / (ms * 1e-3))
+    out["lm_head_path"] = leg
+    best = min(v["ms_per_step"] for k, v in out["logits_path"].items() if isinstance(v, dict) and "ms_per_step" in v and k != "this_library")
+    out["value"] = out["logits_path"]["tokens"] / (best * 1e-3)
+    out["ms_per_step"] = best
+    out["dtype"] = "bf16"
+    return out
+
+
 def main():
     global RS_ACTION, DENSE_BACKWARD, NO_FORWARD_OF_MASKED, BACKWARD_MODE
     args = parse_args()
@@ -1204,6 +1324,10 @@ def main():
         out = bench_hbm(args, dev)
     elif args.workload in MFMA_WORKLOADS:
         out = bench_mfma(args, dev)
+    elif args.workload in TORCH_WORKLOADS:
+        out = bench_torch_ops(args, dev)
+        print(json.dumps(out))
+        return
     elif args.workload == "aux":
         out = bench_aux(args, dev)
     elif args.workload in ADV_WORKLOADS:
