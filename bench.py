@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the PPO/GRPO log-prob + entropy + actor-loss path (forward and backward) on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg1|cfg1-32k|cfg0|cfg2|cfg3|cfg4|adv|aux]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg1|cfg1-32k|cfg0|cfg2|cfg3|cfg4|adv|aux|hbm|mfma|torch-ops]
 
 One "step" is one pass of the hot path over one synthetic packed micro-batch that is already resident in HBM.
 
@@ -44,7 +44,9 @@ and, in the default run only (every GPU timing is taken before the first CPU bas
 
 ``--workload hbm`` runs plain HBM streams (aa_hbm_stream_probe: read only, write only, copy, either cache policy), the
 measured ceilings of the logits path.  ``--workload mfma`` runs the MFMA-only loop (aa_mfma_only_loop: no LDS, no memory traffic), the measured ceiling that
-the fused lm_head figures are also quoted against (``roofline.frac_of_mfma_only_loop``).
+the fused lm_head figures are also quoted against (``roofline.frac_of_mfma_only_loop``).  ``--workload torch-ops``
+times what the reference itself executes for the two paths, restated in plain torch ops, on this GPU (cfg1-32k and
+cfg2; ``--torch-compile`` adds the compiled form), beside this library's step on the same inputs.
 """
 from __future__ import annotations
 
