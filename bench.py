@@ -1288,6 +1288,17 @@ def bench_torch_ops(args, dev):
     leg["library_gemm_logits_only"] = dict(ms=ms, tflops=2.0 * T * case.weight.shape[0] * case.hidden.shape[1] / (ms * 1e-3) / 1e12,
                                            note="torch.nn.functional.linear(hidden, weight) alone: the forward product, "
                                                 "5 GB of bf16 logits written")
+    # the two backward products at the step's shapes (rows of the tokens that have a gradient), library GEMM alone
+    n_grad = int(case.loss_mask.count_nonzero())
+    V_, H_ = case.weight.shape
+    panel = (1e-3 * torch.randn(n_grad, V_, device=dev)).to(torch.bfloat16)
+    rows = case.hidden[:n_grad].contiguous()
+    for key, fn in (("library_gemm_d_hidden_only", lambda: panel @ case.weight),
+                    ("library_gemm_d_weight_only", lambda: panel.t() @ rows)):
+        ms = timed(fn, max(args.steps, 10))
+        leg[key] = dict(ms=ms, tflops=2.0 * n_grad * V_ * H_ / (ms * 1e-3) / 1e12, rows=n_grad)
+    del panel, rows
+
     def ours2():
         h = case.hidden.detach().requires_grad_(True)
         w = case.weight.detach().requires_grad_(True)
