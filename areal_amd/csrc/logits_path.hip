@@ -1101,7 +1101,8 @@ constexpr int kTwoPerUnitChunks = 7;  // rows this short run two workgroups per 
 // Up to kTwoPerUnitChunks chunks the kernel is compiled for 8 waves per SIMD, so that two workgroups fit on a
 // compute unit: without that request the scalar registers alone (106 per wave: 7 waves) keep the second one out.
 // SHIFT (see grad_pass): 1: the chunk grid of a row laid 1 KB back, for rows of whole chunks a whole number of chunks
-// apart; 2: laid back by an amount of the row's own.
+// apart; 2: laid back by an amount of the row's own; 3: the same over the 16-byte pieces of memory that hold a row which
+// starts at any even address (stride_vec is then the stride in values, and NCH counts the chunks of those pieces).
 template <int DT, int NCH, bool EXT, bool ALIAS, int SHIFT = 0>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu((!EXT && NCH <= kTwoPerUnitChunks) ? 8 : 1)))
 void k_fused_regs(typename InPtr<ALIAS, uint4>::type logits, int V, int64_t stride_vec,
