@@ -506,9 +506,9 @@ MODE_NAMES = {1: "carry", 0: "recompute"}
 # known size.  The counters sit behind the L2 of each XCD: what the memory-side cache serves is in these figures too.
 # Transcribed from the profile summaries named beside them, not read in this run; other workloads: not measured.
 LMHEAD_MEASURED_HBM_BYTES = {
-    ("cfg2", "carry"): (81.4e9, "profiles/lmhead_step_cfg2_hbm_traffic.md"),
-    ("cfg2", "recompute"): (110.6e9, "profiles/lmhead_step_cfg2_hbm_traffic.md"),
-    ("cfg4", "carry"): (508.0e9, "profiles/lmhead_step_cfg4_hbm_traffic.md"),
+    ("cfg2", "carry"): (81.7e9, "profiles/lmhead_step_cfg2_hbm_traffic.md"),
+    ("cfg2", "recompute"): (111.1e9, "profiles/lmhead_step_cfg2_hbm_traffic.md"),
+    ("cfg4", "carry"): (515.3e9, "profiles/lmhead_step_cfg4_hbm_traffic.md"),
 }
 
 
